@@ -1,0 +1,27 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def port():
+    from oracle import binding
+    return binding.load_port()
+
+
+@pytest.fixture(scope="session")
+def ref():
+    from oracle import binding
+    lib = binding.load_ref()
+    if lib is None:
+        pytest.skip("oracle/_ref/libcnet_ref.so not built (upstream tree absent)")
+    return lib
