@@ -1,0 +1,116 @@
+// FourierTrans as a dense complex GEMM against a twiddle matrix generated on the device.
+//   F[p][q] = exp(-2 pi i (p*q mod n) / n) / sqrt(n)        (sign and scaling of impl/utils.h:218-221, impl/ft.h:44-47 upstream)
+// p*q is reduced mod n in 64-bit integers before the angle is formed, and sin/cos are evaluated in double, so every
+// entry is the correctly rounded fp32 value of the exact root of unity; F is symmetric, so y = x * F.
+#include "common.hpp"
+
+#include <map>
+
+namespace cnet {
+
+int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
+		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
+		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate);
+
+struct Twiddle {
+	float *re = nullptr;
+	float *im = nullptr;
+	long ld = 0;
+};
+static std::map<int, Twiddle> g_twiddles;
+
+void release_twiddles() {
+	for (auto &kv : g_twiddles) hipFree(kv.second.re);  // one allocation holds both planes
+	g_twiddles.clear();
+}
+
+__global__ void twiddle_kernel(float *__restrict__ fre, float *__restrict__ fim, int n, long ld) {
+	const long idx = (long) blockIdx.x * blockDim.x + threadIdx.x;
+	if (idx >= (long) n * n) return;
+	const int p = (int) (idx / n), q = (int) (idx % n);
+	const long e = ((long) p * q) % n;
+	double s, c;
+	sincospi(-2.0 * (double) e / (double) n, &s, &c);
+	const double scale = 1.0 / sqrt((double) n);
+	fre[(long) p * ld + q] = (float) (c * scale);
+	fim[(long) p * ld + q] = (float) (s * scale);
+}
+
+static int get_plan(int n, Twiddle *out, bool create) {
+	auto it = g_twiddles.find(n);
+	if (it != g_twiddles.end()) {
+		*out = it->second;
+		return CNET_OK;
+	}
+	if (!create) return fail(CNET_ERR_INVALID_ARGUMENT, "no twiddle plan for n=%d: call cnet_cdft_plan first", n);
+	Twiddle t;
+	t.ld = (n + 3) / 4 * 4;  // rows start 16-byte aligned
+	size_t plane = (size_t) n * t.ld;
+	CNET_HIP(hipMalloc((void **) &t.re, 2 * plane * sizeof(float)));
+	t.im = t.re + plane;
+	if (t.ld != n) CNET_HIP(hipMemsetAsync(t.re, 0, 2 * plane * sizeof(float), rt().stream));
+	const long total = (long) n * n;
+	hipLaunchKernelGGL(twiddle_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, rt().stream, t.re, t.im, n, t.ld);
+	CNET_LAUNCH_CHECK();
+	g_twiddles[n] = t;
+	*out = t;
+	return CNET_OK;
+}
+
+}  // namespace cnet
+
+using namespace cnet;
+
+extern "C" {
+
+int cnet_cdft_plan(int n) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(n > 0 && n <= 46340);  // p*q must fit the upstream int exponent as well (impl/ft.h:66)
+	Twiddle t;
+	return get_plan(n, &t, true);
+}
+
+int cnet_cdft_twiddle(int n, const float **f_re, const float **f_im) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(f_re && f_im);
+	Twiddle t;
+	int rc = get_plan(n, &t, false);
+	if (rc) return rc;
+	*f_re = t.re;
+	*f_im = t.im;
+	return CNET_OK;
+}
+
+int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy, int B, int n,
+		int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && n > 0);
+	if (B == 0) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= n && ldy >= n);
+	Twiddle t;
+	int rc = get_plan(n, &t, true);
+	if (rc) return rc;
+	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {t.re, t.re}, *bi[2] = {t.im, t.im};
+	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
+	bool cj[2] = {false, false};
+	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate);
+}
+
+int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+		float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int B, int n, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && n > 0);
+	if (B == 0) return CNET_OK;
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && g_dzs_re && g_dzs_im && dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
+	CNET_CHECK_ARG(ldg >= n && lddx >= n);
+	Twiddle t;
+	int rc = get_plan(n, &t, true);
+	if (rc) return rc;
+	// impl/ft.h:57-79 upstream: dz_q += sum_p G_p w^{pq}/sqrt n ; dzs_q += sum_p Gs_p conj(w^{pq})/sqrt n
+	const float *ar[2] = {g_dz_re, g_dzs_re}, *ai[2] = {g_dz_im, g_dzs_im}, *br[2] = {t.re, t.re}, *bi[2] = {t.im, t.im};
+	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
+	bool cj[2] = {false, true};
+	return cgemm_pair(false, true, 2, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate);
+}
+
+}  // extern "C"

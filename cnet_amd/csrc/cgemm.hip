@@ -1,0 +1,439 @@
+// Split-plane complex GEMM on gfx950 fp32 MFMA, and the Linear entry points built on it.
+//
+//   C[M x N] (+)= A[M x K] * B[K x N]      (complex; optionally conj(B))
+//   Cr += Ar*Br - Ai*Bi ,  Ci += Ar*Bi + Ai*Br      -> four v_mfma_f32_32x32x2_f32 per (A tile, B tile, k pair)
+//
+// Work decomposition
+//   workgroup = 256 threads = 4 wavefronts (one per SIMD) computing a BM x BN block of C;
+//   wavefront = WM x WN sub-block = (WM/32) x (WN/32) MFMA tiles, with a real and an imaginary accumulator
+//   (16 VGPR each) per tile kept in registers for the whole K loop.
+// Data movement
+//   K is walked in chunks of KC = 16.  Each chunk of the four operand planes is fetched from global memory into
+//   registers (float4, coalesced along the contiguous dimension of the source), then written to LDS in
+//   [k][row] order, whatever the source layout: an MFMA operand fragment (lane l -> row l%32, k = l/32) is
+//   then 32 consecutive floats per half-wave, free of bank conflicts.  Sources that are contiguous along k are
+//   transposed by the LDS write; the row pitch (rows + 4) spreads those writes over all banks.
+//   LDS is double buffered: the global loads of chunk c+1 are issued before the MFMAs of chunk c and are written
+//   to the other buffer late in that chunk, so there is one barrier per chunk and it is covered by MFMA work.
+//   conj(B) costs nothing: the sign goes onto B's imaginary plane on its way into LDS.  The minus sign of
+//   Ai*Bi is one v_xor on the Ai fragment per k pair.
+// Launch
+//   one workgroup per C block and per problem (blockIdx.y: the dz and the dzs product of a backward pass are
+//   one launch).  Workgroup ids are dealt round-robin to the 8 XCDs by the hardware; the id is remapped so that
+//   each XCD works on a contiguous strip of C blocks and re-uses operand tiles through its own L2.
+#include "common.hpp"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int KC = 16;         // k extent of one LDS stage
+constexpr int NTHREADS = 256;  // 4 wavefronts
+constexpr int NUM_XCD = 8;
+
+struct CgemmProblem {
+	const float *a_re, *a_im, *b_re, *b_im;
+	float *c_re, *c_im;
+	float b_im_sign;  // -1: multiply by conj(B)
+};
+
+struct CgemmArgs {
+	CgemmProblem p[2];
+	int M, N, K;
+	long lda, ldb, ldc;
+	int accumulate;
+	int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ float keep(float v, unsigned mask) { return __uint_as_float(__float_as_uint(v) & mask); }
+
+// One operand (both planes) of one K chunk: ROWS rows of the block by KC values of k.
+// MCONTIG: the source is stored [k][row] (row contiguous); otherwise [row][k] (k contiguous).
+template <int ROWS, bool MCONTIG, int VEC>
+struct Stage;
+
+template <int ROWS, bool MCONTIG>
+struct Stage<ROWS, MCONTIG, 4> {
+	static constexpr int UNITS = ROWS * KC / 4 / NTHREADS;  // float4 per thread and plane
+	float4 re[UNITS], im[UNITS];
+	bool ok[UNITS];
+
+	__device__ __forceinline__ void load(const float *__restrict__ pre, const float *__restrict__ pim, int row0, int k0,
+			int rows_total, int K, long ld) {
+#pragma unroll
+		for (int u = 0; u < UNITS; ++u) {
+			int unit = threadIdx.x + u * NTHREADS;
+			int row, k;
+			if (MCONTIG) {
+				k = unit / (ROWS / 4);
+				row = (unit % (ROWS / 4)) * 4;
+			} else {
+				row = unit / (KC / 4);
+				k = (unit % (KC / 4)) * 4;
+			}
+			// branch-free edge handling: an out-of-range unit reads element 0 and is replaced by zeros when it is
+			// written to LDS, so nothing consumes the loaded registers before the MFMAs of the current chunk
+			ok[u] = (row0 + row < rows_total) && (k0 + k < K);
+			long off = MCONTIG ? (long) (k0 + k) * ld + row0 + row : (long) (row0 + row) * ld + k0 + k;
+			off = ok[u] ? off : 0;
+			re[u] = *reinterpret_cast<const float4 *>(pre + off);
+			im[u] = *reinterpret_cast<const float4 *>(pim + off);
+		}
+	}
+
+	template <int LDS_PITCH>
+	__device__ __forceinline__ void store(float *sre, float *sim, float im_sign) const {
+#pragma unroll
+		for (int u = 0; u < UNITS; ++u) {
+			int unit = threadIdx.x + u * NTHREADS;
+			const unsigned m = ok[u] ? 0xffffffffu : 0u;  // bitwise zeroing: no branch, no NaN * 0
+			float4 a = make_float4(keep(re[u].x, m), keep(re[u].y, m), keep(re[u].z, m), keep(re[u].w, m));
+			float4 b = make_float4(keep(im[u].x * im_sign, m), keep(im[u].y * im_sign, m), keep(im[u].z * im_sign, m),
+					keep(im[u].w * im_sign, m));
+			if (MCONTIG) {
+				int k = unit / (ROWS / 4);
+				int row = (unit % (ROWS / 4)) * 4;
+				*reinterpret_cast<float4 *>(sre + k * LDS_PITCH + row) = a;
+				*reinterpret_cast<float4 *>(sim + k * LDS_PITCH + row) = b;
+			} else {
+				int row = unit / (KC / 4);
+				int k = (unit % (KC / 4)) * 4;
+				sre[(k + 0) * LDS_PITCH + row] = a.x;
+				sre[(k + 1) * LDS_PITCH + row] = a.y;
+				sre[(k + 2) * LDS_PITCH + row] = a.z;
+				sre[(k + 3) * LDS_PITCH + row] = a.w;
+				sim[(k + 0) * LDS_PITCH + row] = b.x;
+				sim[(k + 1) * LDS_PITCH + row] = b.y;
+				sim[(k + 2) * LDS_PITCH + row] = b.z;
+				sim[(k + 3) * LDS_PITCH + row] = b.w;
+			}
+		}
+	}
+};
+
+// Scalar variant for shapes whose contiguous extent or leading dimension is not a multiple of 4.
+template <int ROWS, bool MCONTIG>
+struct Stage<ROWS, MCONTIG, 1> {
+	static constexpr int UNITS = ROWS * KC / NTHREADS;
+	float re[UNITS], im[UNITS];
+	bool ok[UNITS];
+
+	__device__ __forceinline__ void load(const float *__restrict__ pre, const float *__restrict__ pim, int row0, int k0,
+			int rows_total, int K, long ld) {
+#pragma unroll
+		for (int u = 0; u < UNITS; ++u) {
+			int unit = threadIdx.x + u * NTHREADS;
+			int row = MCONTIG ? unit % ROWS : unit / KC;
+			int k = MCONTIG ? unit / ROWS : unit % KC;
+			ok[u] = (row0 + row < rows_total) && (k0 + k < K);
+			long off = MCONTIG ? (long) (k0 + k) * ld + row0 + row : (long) (row0 + row) * ld + k0 + k;
+			off = ok[u] ? off : 0;
+			re[u] = pre[off];
+			im[u] = pim[off];
+		}
+	}
+
+	template <int LDS_PITCH>
+	__device__ __forceinline__ void store(float *sre, float *sim, float im_sign) const {
+#pragma unroll
+		for (int u = 0; u < UNITS; ++u) {
+			int unit = threadIdx.x + u * NTHREADS;
+			int row = MCONTIG ? unit % ROWS : unit / KC;
+			int k = MCONTIG ? unit / ROWS : unit % KC;
+			const unsigned m = ok[u] ? 0xffffffffu : 0u;
+			sre[k * LDS_PITCH + row] = keep(re[u], m);
+			sim[k * LDS_PITCH + row] = keep(im[u] * im_sign, m);
+		}
+	}
+};
+
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
+__global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args) {
+	static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per workgroup");
+	constexpr int TM = WM / 32, TN = WN / 32;
+	constexpr int PA = BM + 4, PB = BN + 4;  // LDS row pitch in floats
+	constexpr int A_PLANE = KC * PA, B_PLANE = KC * PB;
+	constexpr int STAGE_FLOATS = 2 * A_PLANE + 2 * B_PLANE;
+	extern __shared__ float smem[];
+
+	const CgemmProblem pb = args.p[blockIdx.y];
+	const int M = args.M, N = args.N, K = args.K;
+
+	// ---- which block of C
+	int pid = blockIdx.x;
+	const int total = args.tiles_m * args.tiles_n;
+	if (total % NUM_XCD == 0) pid = (pid % NUM_XCD) * (total / NUM_XCD) + pid / NUM_XCD;
+	constexpr int GROUP = 8;
+	const int width = GROUP * args.tiles_n;
+	const int first_m = (pid / width) * GROUP;
+	const int gsize = min(args.tiles_m - first_m, GROUP);
+	const int tile_m = first_m + (pid % width) % gsize;
+	const int tile_n = (pid % width) / gsize;
+	const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int wm0 = (wave / (BN / WN)) * WM;
+	const int wn0 = (wave % (BN / WN)) * WN;
+	const int r = lane & 31, h = lane >> 5;
+
+	floatx16 acc_re[TM][TN], acc_im[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+#pragma unroll
+			for (int e = 0; e < 16; ++e) {
+				acc_re[i][j][e] = 0.f;
+				acc_im[i][j][e] = 0.f;
+			}
+
+	Stage<BM, A_MCONTIG, VEC> sa;
+	Stage<BN, B_NCONTIG, VEC> sb;
+
+	const int nchunks = (K + KC - 1) / KC;
+	sa.load(pb.a_re, pb.a_im, m0, 0, M, K, args.lda);
+	sb.load(pb.b_re, pb.b_im, n0, 0, N, K, args.ldb);
+	sa.template store<PA>(smem, smem + A_PLANE, 1.0f);
+	sb.template store<PB>(smem + 2 * A_PLANE, smem + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
+	__syncthreads();
+
+	// Operand fragments are double buffered in registers: those of k pair ks+1 are read from LDS while the MFMAs
+	// of k pair ks run.  Per chunk there is ONE barrier, placed two k pairs before the end: by then every wave has
+	// issued its last read of the current stage and has written the next stage, so the 32 MFMAs that follow cover
+	// the barrier skew and the LDS latency of the first fragment of the next chunk.
+	float are[2][TM], aim[2][TM], anim[2][TM], bre[2][TN], bim[2][TN];
+	auto fetch = [&](const float *stage, int ks, int slot) {
+		const int k = ks * 2 + h;
+		const float *s_are = stage + wm0 + r, *s_aim = stage + A_PLANE + wm0 + r;
+		const float *s_bre = stage + 2 * A_PLANE + wn0 + r, *s_bim = stage + 2 * A_PLANE + B_PLANE + wn0 + r;
+#pragma unroll
+		for (int i = 0; i < TM; ++i) {
+			are[slot][i] = s_are[k * PA + i * 32];
+			aim[slot][i] = s_aim[k * PA + i * 32];
+		}
+#pragma unroll
+		for (int j = 0; j < TN; ++j) {
+			bre[slot][j] = s_bre[k * PB + j * 32];
+			bim[slot][j] = s_bim[k * PB + j * 32];
+		}
+	};
+	fetch(smem, 0, 0);
+
+	for (int c = 0; c < nchunks; ++c) {
+		const float *cur = smem + (c & 1) * STAGE_FLOATS;
+		float *nxt = smem + ((c + 1) & 1) * STAGE_FLOATS;
+		const bool more = (c + 1 < nchunks);
+		if (more) {
+			sa.load(pb.a_re, pb.a_im, m0, (c + 1) * KC, M, K, args.lda);
+			sb.load(pb.b_re, pb.b_im, n0, (c + 1) * KC, N, K, args.ldb);
+		}
+#pragma unroll
+		for (int ks = 0; ks < KC / 2; ++ks) {
+			const int cs = ks & 1;
+			if (ks + 1 < KC / 2) fetch(cur, ks + 1, cs ^ 1);
+			if (ks == KC / 2 - 2) {
+				if (more) {
+					sa.template store<PA>(nxt, nxt + A_PLANE, 1.0f);
+					sb.template store<PB>(nxt + 2 * A_PLANE, nxt + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
+				}
+				__syncthreads();
+			}
+			if (ks == KC / 2 - 1 && more) fetch(nxt, 0, cs ^ 1);
+#pragma unroll
+			for (int i = 0; i < TM; ++i) anim[cs][i] = -aim[cs][i];
+			__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+			for (int i = 0; i < TM; ++i)
+#pragma unroll
+				for (int j = 0; j < TN; ++j) {
+					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[cs][i], bre[cs][j], acc_re[i][j], 0, 0, 0);
+					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[cs][i], bim[cs][j], acc_im[i][j], 0, 0, 0);
+				}
+#pragma unroll
+			for (int i = 0; i < TM; ++i)
+#pragma unroll
+				for (int j = 0; j < TN; ++j) {
+					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(anim[cs][i], bim[cs][j], acc_re[i][j], 0, 0, 0);
+					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aim[cs][i], bre[cs][j], acc_im[i][j], 0, 0, 0);
+				}
+			__builtin_amdgcn_sched_barrier(0);
+		}
+	}
+
+	// ---- epilogue: accumulator element e of lane (r, h) is C[(e/4)*8 + h*4 + e%4][r] of its 32x32 tile
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+#pragma unroll
+		for (int j = 0; j < TN; ++j) {
+			const int col = n0 + wn0 + j * 32 + r;
+			if (col >= N) continue;
+#pragma unroll
+			for (int e = 0; e < 16; ++e) {
+				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
+				if (row < M) {
+					const long off = (long) row * args.ldc + col;
+					float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
+					if (args.accumulate) {
+						vr += pb.c_re[off];
+						vi += pb.c_im[off];
+					}
+					pb.c_re[off] = vr;
+					pb.c_im[off] = vi;
+				}
+			}
+		}
+}
+
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
+int launch(const CgemmArgs &proto, int nprob) {
+	CgemmArgs args = proto;
+	args.tiles_m = (args.M + BM - 1) / BM;
+	args.tiles_n = (args.N + BN - 1) / BN;
+	constexpr size_t smem = 2 * (size_t) (2 * KC * (BM + 4) + 2 * KC * (BN + 4)) * sizeof(float);
+	auto kern = cgemm_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, VEC>;
+	static bool attr_set = false;  // per instantiation
+	if (!attr_set) {
+		CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+				(int) smem));
+		attr_set = true;
+	}
+	dim3 grid(args.tiles_m * args.tiles_n, nprob);
+	hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, cnet::rt().stream, args);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+template <bool A_MCONTIG, bool B_NCONTIG, int VEC>
+int pick_tile(const CgemmArgs &a, int nprob) {
+	const long cus = cnet::rt().prop.multiProcessorCount;
+	auto blocks = [&](int bm, int bn) { return (long) ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * nprob; };
+	// the scalar-load fallback (odd shapes) keeps to the small block: its address arithmetic would spill otherwise
+	if constexpr (VEC == 1) {
+		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+	} else {
+		// the largest block that still gives every compute unit a workgroup
+		if (blocks(128, 128) >= cus) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		if (a.N >= a.M) {
+			if (blocks(64, 128) >= cus) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		} else {
+			if (blocks(128, 64) >= cus) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		}
+		if (blocks(64, 128) >= cus) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		if (blocks(128, 64) >= cus) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+	}
+}
+
+}  // namespace
+
+namespace cnet {
+
+// nprob = 1 or 2 problems of identical shape.
+static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int nprob) {
+	if (a.M <= 0 || a.N <= 0) return CNET_OK;
+	if (a.K <= 0) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: K must be positive");
+	// float4 path: every contiguous run starts 16-byte aligned and has a length that is a multiple of 4
+	bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0);
+	vec = vec && (a_mcontig ? a.M % 4 == 0 : a.K % 4 == 0) && (b_ncontig ? a.N % 4 == 0 : a.K % 4 == 0);
+	for (int q = 0; q < nprob; ++q)
+		vec = vec && aligned16(a.p[q].a_re) && aligned16(a.p[q].a_im) && aligned16(a.p[q].b_re) && aligned16(a.p[q].b_im);
+	if (vec) {
+		if (!a_mcontig && !b_ncontig) return pick_tile<false, false, 4>(a, nprob);
+		if (!a_mcontig && b_ncontig) return pick_tile<false, true, 4>(a, nprob);
+		if (a_mcontig && b_ncontig) return pick_tile<true, true, 4>(a, nprob);
+		return pick_tile<true, false, 4>(a, nprob);
+	}
+	if (!a_mcontig && !b_ncontig) return pick_tile<false, false, 1>(a, nprob);
+	if (!a_mcontig && b_ncontig) return pick_tile<false, true, 1>(a, nprob);
+	if (a_mcontig && b_ncontig) return pick_tile<true, true, 1>(a, nprob);
+	return pick_tile<true, false, 1>(a, nprob);
+}
+
+// Used by cdft.hip
+int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
+		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
+		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate) {
+	CgemmArgs a;
+	for (int q = 0; q < nprob; ++q) {
+		a.p[q].a_re = a_re[q];
+		a.p[q].a_im = a_im[q];
+		a.p[q].b_re = b_re[q];
+		a.p[q].b_im = b_im[q];
+		a.p[q].c_re = c_re[q];
+		a.p[q].c_im = c_im[q];
+		a.p[q].b_im_sign = conj_b[q] ? -1.0f : 1.0f;
+	}
+	if (nprob == 1) a.p[1] = a.p[0];
+	a.M = M;
+	a.N = N;
+	a.K = K;
+	a.lda = lda;
+	a.ldb = ldb;
+	a.ldc = ldc;
+	a.accumulate = accumulate;
+	a.tiles_m = a.tiles_n = 0;
+	return cgemm_dispatch(a_mcontig, b_ncontig, a, nprob);
+}
+
+}  // namespace cnet
+
+using namespace cnet;
+
+extern "C" {
+
+int cnet_cgemm(int a_kmajor, int b_kmajor, int conj_b, int M, int N, int K, const float *a_re, const float *a_im,
+		int64_t lda, const float *b_re, const float *b_im, int64_t ldb, float *c_re, float *c_im, int64_t ldc,
+		int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(M >= 0 && N >= 0 && K > 0);
+	if (M == 0 || N == 0) return CNET_OK;
+	CNET_CHECK_ARG(a_re && a_im && b_re && b_im && c_re && c_im);
+	CNET_CHECK_ARG(lda >= (a_kmajor ? M : K) && ldb >= (b_kmajor ? N : K) && ldc >= N);
+	const float *ar[2] = {a_re, a_re}, *ai[2] = {a_im, a_im}, *br[2] = {b_re, b_re}, *bi[2] = {b_im, b_im};
+	float *cr[2] = {c_re, c_re}, *ci[2] = {c_im, c_im};
+	bool cj[2] = {conj_b != 0, conj_b != 0};
+	return cgemm_pair(a_kmajor != 0, b_kmajor != 0, 1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, accumulate);
+}
+
+int cnet_clinear_fwd(const float *x_re, const float *x_im, int64_t ldx, const float *w_re, const float *w_im,
+		int64_t ldw, float *y_re, float *y_im, int64_t ldy, int B, int K, int N, int accumulate) {
+	// y[B][N] = x[B][K] * w[N][K]^T : both operands contiguous along the reduction index
+	return cnet_cgemm(0, 0, 0, B, N, K, x_re, x_im, ldx, w_re, w_im, ldw, y_re, y_im, ldy, accumulate);
+}
+
+int cnet_clinear_bwd_input(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,
+		int64_t ldg, const float *w_re, const float *w_im, int64_t ldw, float *dx_dz_re, float *dx_dz_im,
+		float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int B, int K, int N, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && K >= 0 && N > 0);
+	if (B == 0 || K == 0) return CNET_OK;
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && g_dzs_re && g_dzs_im && w_re && w_im);
+	CNET_CHECK_ARG(dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
+	CNET_CHECK_ARG(ldg >= N && ldw >= K && lddx >= K);
+	// dx[B][K] = g[B][N] * w[N][K] : reduction over N; w is stored [k=N][n=K]
+	const float *ar[2] = {g_dz_re, g_dzs_re}, *ai[2] = {g_dz_im, g_dzs_im};
+	const float *br[2] = {w_re, w_re}, *bi[2] = {w_im, w_im};
+	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
+	bool cj[2] = {false, true};
+	return cgemm_pair(false, true, 2, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate);
+}
+
+int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,
+		int64_t ldg, const float *x_re, const float *x_im, int64_t ldx, float *dw_dz_re, float *dw_dz_im,
+		float *dw_dzs_re, float *dw_dzs_im, int64_t lddw, int B, int K, int N, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B > 0 && K >= 0 && N >= 0);
+	if (N == 0 || K == 0) return CNET_OK;
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && g_dzs_re && g_dzs_im && x_re && x_im);
+	CNET_CHECK_ARG(dw_dz_re && dw_dz_im && dw_dzs_re && dw_dzs_im);
+	CNET_CHECK_ARG(ldg >= N && ldx >= K && lddw >= K);
+	// dw[N][K] = g[B][N]^T * x[B][K] : reduction over the batch; both operands stored [k=B][row]
+	const float *ar[2] = {g_dz_re, g_dzs_re}, *ai[2] = {g_dz_im, g_dzs_im};
+	const float *br[2] = {x_re, x_re}, *bi[2] = {x_im, x_im};
+	float *cr[2] = {dw_dz_re, dw_dzs_re}, *ci[2] = {dw_dz_im, dw_dzs_im};
+	bool cj[2] = {false, true};
+	return cgemm_pair(true, true, 2, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate);
+}
+
+}  // extern "C"

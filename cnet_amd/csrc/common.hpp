@@ -1,0 +1,59 @@
+// Internal declarations shared by the translation units of libcnet_hip.so.
+#ifndef CNET_CSRC_COMMON_HPP_
+#define CNET_CSRC_COMMON_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "cnet_hip.h"
+
+namespace cnet {
+
+struct Runtime {
+	bool ready = false;
+	int device = -1;
+	hipStream_t own_stream = nullptr;
+	hipStream_t stream = nullptr;   // the stream in use (own_stream unless the caller supplied one)
+	hipDeviceProp_t prop;
+	// grow-only scratch for two-stage deterministic reductions (never allocated inside a hot loop twice
+	// for the same size)
+	void *workspace = nullptr;
+	size_t workspace_bytes = 0;
+};
+
+Runtime &rt();
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char *what);
+// returns nullptr (and records the error) when the allocation fails
+void *workspace(size_t bytes);
+
+#define CNET_REQUIRE_INIT()                                                              \
+	do {                                                                                 \
+		if (!cnet::rt().ready) return cnet::fail(CNET_ERR_NOT_INITIALIZED, "%s: cnet_init() has not been called", __func__); \
+	} while (0)
+
+#define CNET_HIP(call)                                             \
+	do {                                                           \
+		hipError_t e__ = (call);                                   \
+		if (e__ != hipSuccess) return cnet::hip_fail(e__, #call);  \
+	} while (0)
+
+#define CNET_CHECK_ARG(cond)                                                                   \
+	do {                                                                                       \
+		if (!(cond)) return cnet::fail(CNET_ERR_INVALID_ARGUMENT, "%s: requirement failed: %s", __func__, #cond); \
+	} while (0)
+
+#define CNET_LAUNCH_CHECK()                                            \
+	do {                                                               \
+		hipError_t e__ = hipGetLastError();                            \
+		if (e__ != hipSuccess) return cnet::hip_fail(e__, __func__);   \
+	} while (0)
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace cnet
+
+#endif

@@ -1,0 +1,628 @@
+// HBM-bound elementwise kernels on split complex planes: Hadamard, CGelu, Residual, the loss backward passes,
+// CInput copies, SGD update, zero fill.
+//
+// All of them walk a [rows x cols] region of row-major planes with per-operand leading dimensions.  One thread
+// handles one group of V consecutive columns (V = 4 -> 128-bit loads and stores; V = 1 for odd shapes), so a
+// wavefront touches 1 KiB of each plane per access and every byte is read and written exactly once.
+#include "common.hpp"
+
+namespace {
+
+constexpr int TPB = 256;
+
+template <int V>
+__device__ __forceinline__ void ldv(float (&d)[V], const float *__restrict__ p) {
+	if (V == 4) {
+		float4 t = *reinterpret_cast<const float4 *>(p);
+		d[0] = t.x;
+		d[1 % V] = t.y;
+		d[2 % V] = t.z;
+		d[3 % V] = t.w;
+	} else {
+		d[0] = *p;
+	}
+}
+
+template <int V>
+__device__ __forceinline__ void stv(float *__restrict__ p, const float (&d)[V]) {
+	if (V == 4)
+		*reinterpret_cast<float4 *>(p) = make_float4(d[0], d[1 % V], d[2 % V], d[3 % V]);
+	else
+		*p = d[0];
+}
+
+// store or accumulate
+template <int V>
+__device__ __forceinline__ void outv(float *__restrict__ p, const float (&d)[V], int accumulate) {
+	if (accumulate) {
+		float o[V];
+		ldv<V>(o, p);
+		float s[V];
+#pragma unroll
+		for (int k = 0; k < V; ++k) s[k] = o[k] + d[k];
+		stv<V>(p, s);
+	} else {
+		stv<V>(p, d);
+	}
+}
+
+struct Grad4 {
+	float *dz_re, *dz_im, *dzs_re, *dzs_im;
+};
+struct CGrad4 {
+	const float *dz_re, *dz_im, *dzs_re, *dzs_im;
+};
+
+#define CNET_ELEM_INDEX()                                                        \
+	const long cv = cols / V;                                                    \
+	const long idx = (long) blockIdx.x * TPB + threadIdx.x;                      \
+	if (idx >= (long) rows * cv) return;                                         \
+	const long row = idx / cv;                                                   \
+	const long col = (idx - row * cv) * V;
+
+// ------------------------------------------------------------------------------------------------ Hadamard
+template <int V>
+__global__ __launch_bounds__(TPB) void hadamard_fwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
+		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, float *__restrict__ yr,
+		float *__restrict__ yi, long ldy, int rows, int cols) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], c[V], d[V], pr[V], pi[V];
+	ldv<V>(a, ur + row * ldu + col);
+	ldv<V>(b, ui + row * ldu + col);
+	ldv<V>(c, vr + row * ldv_ + col);
+	ldv<V>(d, vi + row * ldv_ + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		pr[k] = a[k] * c[k] - b[k] * d[k];
+		pi[k] = a[k] * d[k] + b[k] * c[k];
+	}
+	stv<V>(yr + row * ldy + col, pr);
+	stv<V>(yi + row * ldy + col, pi);
+}
+
+// Both operands per-row: du = (G v, Gs conj v), dv = (G u, Gs conj u).
+template <int V>
+__global__ __launch_bounds__(TPB) void hadamard_bwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
+		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, CGrad4 g, long ldg, Grad4 du, long lddu,
+		Grad4 dv, long lddv, int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], c[V], d[V], gr[V], gi[V], sr[V], si[V], o[V];
+	ldv<V>(a, ur + row * ldu + col);
+	ldv<V>(b, ui + row * ldu + col);
+	ldv<V>(c, vr + row * ldv_ + col);
+	ldv<V>(d, vi + row * ldv_ + col);
+	ldv<V>(gr, g.dz_re + row * ldg + col);
+	ldv<V>(gi, g.dz_im + row * ldg + col);
+	ldv<V>(sr, g.dzs_re + row * ldg + col);
+	ldv<V>(si, g.dzs_im + row * ldg + col);
+	const long ou = row * lddu + col, ov = row * lddv + col;
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = gr[k] * c[k] - gi[k] * d[k];
+	outv<V>(du.dz_re + ou, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = gr[k] * d[k] + gi[k] * c[k];
+	outv<V>(du.dz_im + ou, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = sr[k] * c[k] + si[k] * d[k];
+	outv<V>(du.dzs_re + ou, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = si[k] * c[k] - sr[k] * d[k];
+	outv<V>(du.dzs_im + ou, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = gr[k] * a[k] - gi[k] * b[k];
+	outv<V>(dv.dz_re + ov, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = gr[k] * b[k] + gi[k] * a[k];
+	outv<V>(dv.dz_im + ov, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = sr[k] * a[k] + si[k] * b[k];
+	outv<V>(dv.dzs_re + ov, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = si[k] * a[k] - sr[k] * b[k];
+	outv<V>(dv.dzs_im + ov, o, accumulate);
+}
+
+// v is one shared parameter row.  blockIdx.y selects a slab of rows; each thread owns V columns, writes du for its
+// rows and keeps the four dv sums of its slab in registers; partial[slab][plane][cols] goes to the workspace and a
+// second kernel adds the slabs in slab order (deterministic, no atomics).
+template <int V>
+__global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *__restrict__ ur, const float *__restrict__ ui,
+		long ldu, const float *__restrict__ vr, const float *__restrict__ vi, CGrad4 g, long ldg, Grad4 du, long lddu,
+		float *__restrict__ partial, int rows, int cols, int rows_per_slab, int accumulate) {
+	const long col = ((long) blockIdx.x * TPB + threadIdx.x) * V;
+	if (col >= cols) return;
+	const int slab = blockIdx.y;
+	const int r0 = slab * rows_per_slab;
+	const int r1 = min(rows, r0 + rows_per_slab);
+	float c[V], d[V];
+	ldv<V>(c, vr + col);
+	ldv<V>(d, vi + col);
+	float acc[4][V];
+#pragma unroll
+	for (int p = 0; p < 4; ++p)
+#pragma unroll
+		for (int k = 0; k < V; ++k) acc[p][k] = 0.f;
+	for (int row = r0; row < r1; ++row) {
+		float a[V], b[V], gr[V], gi[V], sr[V], si[V], o[V];
+		ldv<V>(a, ur + (long) row * ldu + col);
+		ldv<V>(b, ui + (long) row * ldu + col);
+		ldv<V>(gr, g.dz_re + (long) row * ldg + col);
+		ldv<V>(gi, g.dz_im + (long) row * ldg + col);
+		ldv<V>(sr, g.dzs_re + (long) row * ldg + col);
+		ldv<V>(si, g.dzs_im + (long) row * ldg + col);
+		const long ou = (long) row * lddu + col;
+#pragma unroll
+		for (int k = 0; k < V; ++k) o[k] = gr[k] * c[k] - gi[k] * d[k];
+		outv<V>(du.dz_re + ou, o, accumulate);
+#pragma unroll
+		for (int k = 0; k < V; ++k) o[k] = gr[k] * d[k] + gi[k] * c[k];
+		outv<V>(du.dz_im + ou, o, accumulate);
+#pragma unroll
+		for (int k = 0; k < V; ++k) o[k] = sr[k] * c[k] + si[k] * d[k];
+		outv<V>(du.dzs_re + ou, o, accumulate);
+#pragma unroll
+		for (int k = 0; k < V; ++k) o[k] = si[k] * c[k] - sr[k] * d[k];
+		outv<V>(du.dzs_im + ou, o, accumulate);
+#pragma unroll
+		for (int k = 0; k < V; ++k) {
+			acc[0][k] += gr[k] * a[k] - gi[k] * b[k];
+			acc[1][k] += gr[k] * b[k] + gi[k] * a[k];
+			acc[2][k] += sr[k] * a[k] + si[k] * b[k];
+			acc[3][k] += si[k] * a[k] - sr[k] * b[k];
+		}
+	}
+#pragma unroll
+	for (int p = 0; p < 4; ++p) stv<V>(partial + ((long) slab * 4 + p) * cols + col, acc[p]);
+}
+
+// dst[p][c] (+)= sum over slabs of partial[slab][p][c], slabs added in index order.
+__global__ __launch_bounds__(TPB) void slab_sum_kernel(const float *__restrict__ partial, int nslabs, int nplanes, int cols,
+		Grad4 dst, int accumulate) {
+	const long idx = (long) blockIdx.x * TPB + threadIdx.x;
+	if (idx >= (long) nplanes * cols) return;
+	const int p = (int) (idx / cols);
+	const int c = (int) (idx - (long) p * cols);
+	float s = 0.f;
+	for (int k = 0; k < nslabs; ++k) s += partial[((long) k * nplanes + p) * cols + c];
+	float *out = p == 0 ? dst.dz_re : (p == 1 ? dst.dz_im : (p == 2 ? dst.dzs_re : dst.dzs_im));
+	out[c] = accumulate ? out[c] + s : s;
+}
+
+// ------------------------------------------------------------------------------------------------ CGelu
+// tanh-GELU on each real plane (impl/relu.h:119-131 upstream).
+__device__ __forceinline__ float gelu_value(float t) {
+	const float c = 0.7978845608028654f;  // sqrt(2/pi)
+	float arg = c * (t + 0.044715f * t * t * t);
+	return 0.5f * t * (1.0f + tanhf(arg));
+}
+
+__device__ __forceinline__ float gelu_slope(float t) {
+	const float c = 0.7978845608028654f;
+	float arg = c * (t + 0.044715f * t * t * t);
+	float th = tanhf(arg);
+	float sech2 = 1.0f - th * th;  // = 1/cosh^2
+	return 0.5f * (1.0f + th) + t * 0.5f * sech2 * c * (1.0f + 3.0f * 0.044715f * t * t);
+}
+
+template <int V>
+__global__ __launch_bounds__(TPB) void gelu_fwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
+		float *__restrict__ yr, float *__restrict__ yi, long ldy, int rows, int cols) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V];
+	ldv<V>(a, xr + row * ldx + col);
+	ldv<V>(b, xi + row * ldx + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		a[k] = gelu_value(a[k]);
+		b[k] = gelu_value(b[k]);
+	}
+	stv<V>(yr + row * ldy + col, a);
+	stv<V>(yi + row * ldy + col, b);
+}
+
+// dz = G s + Gs d ; dzs = G d + Gs s ; s = (g'(x)+g'(y))/2, d = (g'(x)-g'(y))/2   (impl/relu.h:144-166 upstream)
+template <int V>
+__global__ __launch_bounds__(TPB) void gelu_bwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
+		CGrad4 g, long ldg, Grad4 dx, long lddx, int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], gr[V], gi[V], sr[V], si[V], s[V], d[V], o[V];
+	ldv<V>(a, xr + row * ldx + col);
+	ldv<V>(b, xi + row * ldx + col);
+	ldv<V>(gr, g.dz_re + row * ldg + col);
+	ldv<V>(gi, g.dz_im + row * ldg + col);
+	ldv<V>(sr, g.dzs_re + row * ldg + col);
+	ldv<V>(si, g.dzs_im + row * ldg + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		float px = 0.5f * gelu_slope(a[k]), py = 0.5f * gelu_slope(b[k]);
+		s[k] = px + py;
+		d[k] = px - py;
+	}
+	const long off = row * lddx + col;
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = gr[k] * s[k] + sr[k] * d[k];
+	outv<V>(dx.dz_re + off, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = gi[k] * s[k] + si[k] * d[k];
+	outv<V>(dx.dz_im + off, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = gr[k] * d[k] + sr[k] * s[k];
+	outv<V>(dx.dzs_re + off, o, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) o[k] = gi[k] * d[k] + si[k] * s[k];
+	outv<V>(dx.dzs_im + off, o, accumulate);
+}
+
+// ------------------------------------------------------------------------------------------------ Residual
+template <int V>
+__global__ __launch_bounds__(TPB) void residual_fwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
+		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, float *__restrict__ yr,
+		float *__restrict__ yi, long ldy, int rows, int cols) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], c[V], d[V];
+	ldv<V>(a, ur + row * ldu + col);
+	ldv<V>(b, ui + row * ldu + col);
+	ldv<V>(c, vr + row * ldv_ + col);
+	ldv<V>(d, vi + row * ldv_ + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		a[k] += c[k];
+		b[k] += d[k];
+	}
+	stv<V>(yr + row * ldy + col, a);
+	stv<V>(yi + row * ldy + col, b);
+}
+
+template <int V>
+__global__ __launch_bounds__(TPB) void residual_bwd_kernel(CGrad4 g, long ldg, Grad4 du, long lddu, Grad4 dv, long lddv,
+		int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float t[V];
+	const long og = row * ldg + col, ou = row * lddu + col, ov = row * lddv + col;
+	ldv<V>(t, g.dz_re + og);
+	outv<V>(du.dz_re + ou, t, accumulate);
+	outv<V>(dv.dz_re + ov, t, accumulate);
+	ldv<V>(t, g.dz_im + og);
+	outv<V>(du.dz_im + ou, t, accumulate);
+	outv<V>(dv.dz_im + ov, t, accumulate);
+	ldv<V>(t, g.dzs_re + og);
+	outv<V>(du.dzs_re + ou, t, accumulate);
+	outv<V>(dv.dzs_re + ov, t, accumulate);
+	ldv<V>(t, g.dzs_im + og);
+	outv<V>(du.dzs_im + ou, t, accumulate);
+	outv<V>(dv.dzs_im + ov, t, accumulate);
+}
+
+// ------------------------------------------------------------------------------------------------ loss backward
+// L2Out: dz = conj z, dzs = z  (impl/l2out.h:44-58 upstream)
+template <int V>
+__global__ __launch_bounds__(TPB) void l2out_bwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		Grad4 dz, long lddz, int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], nb[V];
+	ldv<V>(a, zr + row * ldz + col);
+	ldv<V>(b, zi + row * ldz + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) nb[k] = -b[k];
+	const long off = row * lddz + col;
+	outv<V>(dz.dz_re + off, a, accumulate);
+	outv<V>(dz.dz_im + off, nb, accumulate);
+	outv<V>(dz.dzs_re + off, a, accumulate);
+	outv<V>(dz.dzs_im + off, b, accumulate);
+}
+
+// CrossEntropy (impl/crossent.h:82-104 upstream): assigns.  label: dzs = -z (S-m)/(m S), m = max(|z_l|^2, 1e-15);
+// other entries: dzs = z/S; dz = conj(dzs).
+template <int V>
+__global__ __launch_bounds__(TPB) void crossent_bwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		const float *__restrict__ s, const int *__restrict__ labels, Grad4 dz, long lddz, int rows, int cols) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], o_r[V], o_i[V], n_i[V];
+	ldv<V>(a, zr + row * ldz + col);
+	ldv<V>(b, zi + row * ldz + col);
+	const float S = s[row];
+	const int label = labels[row];
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		if (col + k == label) {
+			float m = (float) ((double) a[k] * (double) a[k] + (double) b[k] * (double) b[k]);
+			m = (m < 1e-15f ? 1e-15f : m);
+			o_r[k] = -a[k] * (S - m) / (m * S);
+			o_i[k] = -b[k] * (S - m) / (m * S);
+		} else {
+			o_r[k] = a[k] / S;
+			o_i[k] = b[k] / S;
+		}
+		n_i[k] = -o_i[k];
+	}
+	const long off = row * lddz + col;
+	stv<V>(dz.dzs_re + off, o_r);
+	stv<V>(dz.dzs_im + off, o_i);
+	stv<V>(dz.dz_re + off, o_r);
+	stv<V>(dz.dz_im + off, n_i);
+}
+
+// ------------------------------------------------------------------------------------------------ plumbing
+template <int V>
+__global__ __launch_bounds__(TPB) void copy2d_kernel(const float *__restrict__ src, long lds, float *__restrict__ dst, long ldd,
+		int rows, int cols, int add) {
+	CNET_ELEM_INDEX();
+	float t[V];
+	ldv<V>(t, src + row * lds + col);
+	outv<V>(dst + row * ldd + col, t, add);
+}
+
+// z -= lr * dzs ; dzs = 0   (impl/cfunc.h:147-152, impl/cnet.h:413-421 upstream)
+template <int V>
+__global__ __launch_bounds__(TPB) void sgd_kernel(float *__restrict__ zr, float *__restrict__ zi, float *__restrict__ dr,
+		float *__restrict__ di, long n, float lr, int zero_grad) {
+	const long i = ((long) blockIdx.x * TPB + threadIdx.x) * V;
+	if (i >= n) return;
+	float a[V], b[V], c[V], d[V], z[V];
+	ldv<V>(a, zr + i);
+	ldv<V>(b, zi + i);
+	ldv<V>(c, dr + i);
+	ldv<V>(d, di + i);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		a[k] -= lr * c[k];
+		b[k] -= lr * d[k];
+		z[k] = 0.f;
+	}
+	stv<V>(zr + i, a);
+	stv<V>(zi + i, b);
+	if (zero_grad) {
+		stv<V>(dr + i, z);
+		stv<V>(di + i, z);
+	}
+}
+
+__global__ __launch_bounds__(TPB) void zero_kernel(uint4 *__restrict__ p16, long n16, unsigned char *__restrict__ tail, int ntail) {
+	const long i = (long) blockIdx.x * TPB + threadIdx.x;
+	if (i < n16) p16[i] = make_uint4(0, 0, 0, 0);
+	if (i < ntail) tail[i] = 0;
+}
+
+inline unsigned nblocks(long work) { return (unsigned) ((work + TPB - 1) / TPB); }
+
+inline bool all_aligned(std::initializer_list<const void *> ptrs) {
+	for (const void *p : ptrs)
+		if (p && !cnet::aligned16(p)) return false;
+	return true;
+}
+inline bool all_mult4(std::initializer_list<long> v) {
+	for (long x : v)
+		if (x % 4) return false;
+	return true;
+}
+
+}  // namespace
+
+using namespace cnet;
+
+#define CNET_GRID_2D(V) dim3(nblocks((long) rows * (cols / (V)))), dim3(TPB), 0, rt().stream
+
+extern "C" {
+
+int cnet_memset_zero(void *dst, size_t bytes) {
+	CNET_REQUIRE_INIT();
+	if (!bytes) return CNET_OK;
+	CNET_CHECK_ARG(dst != nullptr);
+	// a fill kernel rather than hipMemsetAsync, so the call can be captured into a HIP graph
+	unsigned char *p = (unsigned char *) dst;
+	size_t head = (16 - ((uintptr_t) p & 15)) & 15;
+	if (head > bytes) head = bytes;
+	if (head) {
+		hipLaunchKernelGGL(zero_kernel, dim3(1), dim3(TPB), 0, rt().stream, (uint4 *) nullptr, 0L, p, (int) head);
+		CNET_LAUNCH_CHECK();
+	}
+	p += head;
+	bytes -= head;
+	long n16 = (long) (bytes / 16);
+	int ntail = (int) (bytes % 16);
+	if (n16 || ntail) {
+		hipLaunchKernelGGL(zero_kernel, dim3(nblocks(n16 > ntail ? n16 : ntail)), dim3(TPB), 0, rt().stream, (uint4 *) p, n16,
+				p + n16 * 16, ntail);
+		CNET_LAUNCH_CHECK();
+	}
+	return CNET_OK;
+}
+
+int cnet_hadamard_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+		float *y_re, float *y_im, int64_t ldy, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && y_re && y_im);
+	CNET_CHECK_ARG(ldu >= cols && ldy >= cols && (ldv == 0 || ldv >= cols));
+	if (all_mult4({cols, ldu, ldv, ldy}) && all_aligned({u_re, u_im, v_re, v_im, y_re, y_im}))
+		hipLaunchKernelGGL(hadamard_fwd_kernel<4>, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+	else
+		hipLaunchKernelGGL(hadamard_fwd_kernel<1>, CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+		const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+		float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu, float *dv_dz_re,
+		float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && g_dz_re && g_dz_im && g_dzs_re && g_dzs_im);
+	CNET_CHECK_ARG(du_dz_re && du_dz_im && du_dzs_re && du_dzs_im && dv_dz_re && dv_dz_im && dv_dzs_re && dv_dzs_im);
+	CNET_CHECK_ARG(ldu >= cols && ldg >= cols && lddu >= cols && (ldv == 0 || (ldv >= cols && lddv >= cols)));
+	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
+	Grad4 du = {du_dz_re, du_dz_im, du_dzs_re, du_dzs_im};
+	Grad4 dv = {dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im};
+	bool vec = all_mult4({cols, ldu, ldv, ldg, lddu, ldv ? lddv : 0}) &&
+			all_aligned({u_re, u_im, v_re, v_im, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, du_dz_re, du_dz_im, du_dzs_re,
+					du_dzs_im, dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im});
+	if (ldv != 0) {
+		if (vec)
+			hipLaunchKernelGGL(hadamard_bwd_kernel<4>, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, g, ldg, du, lddu, dv, lddv,
+					rows, cols, accumulate);
+		else
+			hipLaunchKernelGGL(hadamard_bwd_kernel<1>, CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, g, ldg, du, lddu, dv, lddv,
+					rows, cols, accumulate);
+		CNET_LAUNCH_CHECK();
+		return CNET_OK;
+	}
+	// shared parameter row: slabs of rows sized so that the grid covers the chip a few times over
+	const int V = vec ? 4 : 1;
+	const long col_blocks = ((long) cols / V + TPB - 1) / TPB;
+	const long want_blocks = 8L * rt().prop.multiProcessorCount;
+	int nslabs = (int) ((want_blocks + col_blocks - 1) / col_blocks);
+	if (nslabs > rows) nslabs = rows;
+	if (nslabs < 1) nslabs = 1;
+	const int rows_per_slab = (rows + nslabs - 1) / nslabs;
+	nslabs = (rows + rows_per_slab - 1) / rows_per_slab;
+	float *partial = (float *) workspace((size_t) nslabs * 4 * cols * sizeof(float));
+	if (!partial) return CNET_ERR_OUT_OF_MEMORY;
+	dim3 grid((unsigned) col_blocks, (unsigned) nslabs);
+	if (vec)
+		hipLaunchKernelGGL(hadamard_bwd_shared_kernel<4>, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
+				lddu, partial, rows, cols, rows_per_slab, accumulate);
+	else
+		hipLaunchKernelGGL(hadamard_bwd_shared_kernel<1>, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
+				lddu, partial, rows, cols, rows_per_slab, accumulate);
+	CNET_LAUNCH_CHECK();
+	hipLaunchKernelGGL(slab_sum_kernel, dim3(nblocks(4L * cols)), dim3(TPB), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= cols && ldy >= cols);
+	if (all_mult4({cols, ldx, ldy}) && all_aligned({x_re, x_im, y_re, y_im}))
+		hipLaunchKernelGGL(gelu_fwd_kernel<4>, CNET_GRID_2D(4), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+	else
+		hipLaunchKernelGGL(gelu_fwd_kernel<1>, CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_cgelu_bwd(const float *x_re, const float *x_im, int64_t ldx, const float *g_dz_re, const float *g_dz_im,
+		const float *g_dzs_re, const float *g_dzs_im, int64_t ldg, float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re,
+		float *dx_dzs_im, int64_t lddx, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && g_dz_re && g_dz_im && g_dzs_re && g_dzs_im && dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
+	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
+	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
+	Grad4 dx = {dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im};
+	if (all_mult4({cols, ldx, ldg, lddx}) &&
+			all_aligned({x_re, x_im, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
+		hipLaunchKernelGGL(gelu_bwd_kernel<4>, CNET_GRID_2D(4), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+	else
+		hipLaunchKernelGGL(gelu_bwd_kernel<1>, CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_residual_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+		float *y_re, float *y_im, int64_t ldy, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && y_re && y_im && ldu >= cols && ldv >= cols && ldy >= cols);
+	if (all_mult4({cols, ldu, ldv, ldy}) && all_aligned({u_re, u_im, v_re, v_im, y_re, y_im}))
+		hipLaunchKernelGGL(residual_fwd_kernel<4>, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+	else
+		hipLaunchKernelGGL(residual_fwd_kernel<1>, CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_residual_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+		float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu, float *dv_dz_re,
+		float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && g_dzs_re && g_dzs_im);
+	CNET_CHECK_ARG(du_dz_re && du_dz_im && du_dzs_re && du_dzs_im && dv_dz_re && dv_dz_im && dv_dzs_re && dv_dzs_im);
+	CNET_CHECK_ARG(ldg >= cols && lddu >= cols && lddv >= cols);
+	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
+	Grad4 du = {du_dz_re, du_dz_im, du_dzs_re, du_dzs_im};
+	Grad4 dv = {dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im};
+	if (all_mult4({cols, ldg, lddu, lddv}) &&
+			all_aligned({g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, du_dz_re, du_dz_im, du_dzs_re, du_dzs_im, dv_dz_re, dv_dz_im,
+					dv_dzs_re, dv_dzs_im}))
+		hipLaunchKernelGGL(residual_bwd_kernel<4>, CNET_GRID_2D(4), g, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
+	else
+		hipLaunchKernelGGL(residual_bwd_kernel<1>, CNET_GRID_2D(1), g, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_l2out_bwd(const float *z_re, const float *z_im, int64_t ldz, float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re,
+		float *dz_dzs_im, int64_t lddz, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && dz_dz_re && dz_dz_im && dz_dzs_re && dz_dzs_im && ldz >= cols && lddz >= cols);
+	Grad4 dz = {dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im};
+	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
+		hipLaunchKernelGGL(l2out_bwd_kernel<4>, CNET_GRID_2D(4), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
+	else
+		hipLaunchKernelGGL(l2out_bwd_kernel<1>, CNET_GRID_2D(1), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_cross_entropy_bwd(const float *z_re, const float *z_im, int64_t ldz, const float *s, const int32_t *labels,
+		float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && s && labels && dz_dz_re && dz_dz_im && dz_dzs_re && dz_dzs_im && ldz >= cols && lddz >= cols);
+	Grad4 dz = {dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im};
+	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
+		hipLaunchKernelGGL(crossent_bwd_kernel<4>, CNET_GRID_2D(4), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
+	else
+		hipLaunchKernelGGL(crossent_bwd_kernel<1>, CNET_GRID_2D(1), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+static int copy_or_add(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols, int add) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(src && dst && lds >= cols && ldd >= cols);
+	if (all_mult4({cols, lds, ldd}) && all_aligned({src, dst}))
+		hipLaunchKernelGGL(copy2d_kernel<4>, CNET_GRID_2D(4), src, lds, dst, ldd, rows, cols, add);
+	else
+		hipLaunchKernelGGL(copy2d_kernel<1>, CNET_GRID_2D(1), src, lds, dst, ldd, rows, cols, add);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_copy2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols) {
+	return copy_or_add(src, lds, dst, ldd, rows, cols, 0);
+}
+
+int cnet_add2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols) {
+	return copy_or_add(src, lds, dst, ldd, rows, cols, 1);
+}
+
+int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int64_t n, float lr, int zero_grad) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(n >= 0);
+	if (!n) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && dzs_re && dzs_im);
+	if (n % 4 == 0 && all_aligned({z_re, z_im, dzs_re, dzs_im}))
+		hipLaunchKernelGGL(sgd_kernel<4>, dim3(nblocks(n / 4)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
+	else
+		hipLaunchKernelGGL(sgd_kernel<1>, dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,430 @@
+// Reductions on split complex planes: the row reductions of L2Out / CrossEntropy / SoftMax (sum |z|^2, argmax,
+// the two inner products of the SoftMax backward) and the column reduction that sums per-sample parameter
+// gradients over the batch.
+//
+// Row reductions: one row is owned by G wavefronts of one workgroup (G = 1 for short rows, 4 for long ones).
+// Each lane strides over the row with 128-bit loads, then the 64 lanes are combined with DPP row operations
+// (quad_perm, row_ror) plus one ds_swizzle and one cross-half exchange, always in the same order, and the G
+// wavefront results are added through LDS in wavefront order.  No atomics anywhere: results do not depend on
+// scheduling.
+#include "common.hpp"
+
+namespace {
+
+constexpr int TPB = 256;
+
+// ---------------------------------------------------------------------------------------------- lane exchange
+// value of the lane selected by a DPP control word, for 32-bit payloads
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) {
+	return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+constexpr int DPP_QUAD_XOR1 = 0xB1;  // quad_perm:[1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;  // quad_perm:[2,3,0,1]
+constexpr int DPP_ROW_ROR4 = 0x124;
+constexpr int DPP_ROW_ROR8 = 0x128;
+constexpr int SWIZZLE_XOR16 = 0x401F;  // bit mode: and 0x1f, or 0, xor 0x10
+
+template <class T, int STEP>
+__device__ __forceinline__ T exchange(T v) {
+	static_assert(sizeof(T) % 4 == 0, "32-bit words");
+	constexpr int W = sizeof(T) / 4;
+	union {
+		T t;
+		int w[W];
+	} a, b;
+	a.t = v;
+#pragma unroll
+	for (int k = 0; k < W; ++k) {
+		if (STEP == 0) b.w[k] = dpp_i<DPP_QUAD_XOR1>(a.w[k]);
+		if (STEP == 1) b.w[k] = dpp_i<DPP_QUAD_XOR2>(a.w[k]);
+		if (STEP == 2) b.w[k] = dpp_i<DPP_ROW_ROR4>(a.w[k]);
+		if (STEP == 3) b.w[k] = dpp_i<DPP_ROW_ROR8>(a.w[k]);
+		if (STEP == 4) b.w[k] = __builtin_amdgcn_ds_swizzle(a.w[k], SWIZZLE_XOR16);
+		if (STEP == 5) b.w[k] = __shfl_xor(a.w[k], 32, 64);
+	}
+	return b.t;
+}
+
+// After the six steps lane 0 (in fact every lane) holds op over all 64 lanes, combined in a fixed order.
+template <class T, class Op>
+__device__ __forceinline__ T wave_reduce(T v, Op op) {
+	v = op(v, exchange<T, 0>(v));
+	v = op(v, exchange<T, 1>(v));
+	v = op(v, exchange<T, 2>(v));
+	v = op(v, exchange<T, 3>(v));
+	v = op(v, exchange<T, 4>(v));
+	v = op(v, exchange<T, 5>(v));
+	return v;
+}
+
+// G wavefronts of a workgroup share one row: combine their results in wavefront order through LDS.
+// `slot` is this row's position within the workgroup.  Returns the total to every thread of the group.
+template <class T, int G, class Op>
+__device__ __forceinline__ T group_reduce(T v, Op op, T *lds, int slot, int wave_in_group, int lane) {
+	v = wave_reduce(v, op);
+	if (G == 1) return v;
+	if (lane == 0) lds[slot * G + wave_in_group] = v;
+	__syncthreads();
+	T total = lds[slot * G];
+#pragma unroll
+	for (int k = 1; k < G; ++k) total = op(total, lds[slot * G + k]);
+	__syncthreads();
+	return total;
+}
+
+struct SumF {
+	__device__ float operator()(float a, float b) const { return a + b; }
+};
+struct SumD {
+	__device__ double operator()(double a, double b) const { return a + b; }
+};
+struct ArgMax {
+	float v;
+	int i;
+};
+// larger value wins; equal values keep the smaller index (the first maximum of a serial strict-> scan)
+struct ArgMaxOp {
+	__device__ ArgMax operator()(ArgMax a, ArgMax b) const {
+		if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+		return a;
+	}
+};
+struct Cplx4 {
+	float a, b, c, d;
+};
+struct SumC4 {
+	__device__ Cplx4 operator()(Cplx4 x, Cplx4 y) const { return Cplx4{x.a + y.a, x.b + y.b, x.c + y.c, x.d + y.d}; }
+};
+
+// Row geometry shared by the row kernels: TPB/(64*G) rows per workgroup.
+#define CNET_ROW_SETUP()                                        \
+	constexpr int ROWS_PER_BLOCK = TPB / (64 * G);              \
+	const int lane = threadIdx.x & 63;                          \
+	const int wave = threadIdx.x >> 6;                          \
+	const int slot = wave / G;                                  \
+	const int wig = wave % G;                                   \
+	const int row_raw = blockIdx.x * ROWS_PER_BLOCK + slot;     \
+	const bool live = row_raw < rows;                           \
+	const int row = live ? row_raw : rows - 1;                  \
+	const int t = wig * 64 + lane;                              \
+	constexpr int STRIDE = 64 * G;
+
+// sum over one row of f(re, im), 128-bit loads when V == 4
+template <int V, int G, class T, class F>
+__device__ __forceinline__ T row_accumulate(const float *__restrict__ pr, const float *__restrict__ pi, int cols, int t, F f) {
+	T acc = T();
+	constexpr int STRIDE = 64 * G;
+	if (V == 4) {
+		for (int c = t * 4; c < cols; c += STRIDE * 4) {
+			float4 a = *reinterpret_cast<const float4 *>(pr + c);
+			float4 b = *reinterpret_cast<const float4 *>(pi + c);
+			acc += f(a.x, b.x);
+			acc += f(a.y, b.y);
+			acc += f(a.z, b.z);
+			acc += f(a.w, b.w);
+		}
+	} else {
+		for (int c = t; c < cols; c += STRIDE) acc += f(pr[c], pi[c]);
+	}
+	return acc;
+}
+
+// ---------------------------------------------------------------------------------------------- L2Out forward
+template <int V, int G>
+__global__ __launch_bounds__(TPB) void l2out_fwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		float *__restrict__ loss, int rows, int cols) {
+	__shared__ float lds[TPB / 64];
+	CNET_ROW_SETUP();
+	(void) STRIDE;
+	float acc = row_accumulate<V, G, float>(zr + (long) row * ldz, zi + (long) row * ldz, cols, t,
+			[](float a, float b) { return a * a + b * b; });
+	acc = group_reduce<float, G>(acc, SumF(), lds, slot, wig, lane);
+	if (live && t == 0) loss[row] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------- CrossEntropy forward
+// impl/crossent.h:50-80, 117-130 upstream: S in double, clamped; out = z / sqrt(S); p_k = out_r^2 + out_i^2 evaluated
+// in double and rounded to float; argmax = first strict maximum of p; loss = -log(max(p_label, 1e-15)).
+template <int V, int G>
+__global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		const int *__restrict__ labels, float *__restrict__ outr, float *__restrict__ outi, long ldo, float *__restrict__ s,
+		float *__restrict__ loss, int *__restrict__ argmax, int rows, int cols) {
+	__shared__ double lds_d[TPB / 64];
+	__shared__ ArgMax lds_a[TPB / 64];
+	CNET_ROW_SETUP();
+	const float *pr = zr + (long) row * ldz, *pi = zi + (long) row * ldz;
+	double sum = row_accumulate<V, G, double>(pr, pi, cols, t,
+			[](float a, float b) { return (double) a * (double) a + (double) b * (double) b; });
+	sum = group_reduce<double, G>(sum, SumD(), lds_d, slot, wig, lane);
+	float S = (float) sum;
+	if (S <= 1.0e-15f) S = 1.0e-15f;
+	double nrm = sqrt((double) S);
+	if (nrm <= 1.0e-15) nrm = 1.0e-15;
+	const double inv = 1.0 / nrm;
+
+	ArgMax best = {-1.0f, 0x7fffffff};
+	const bool want_out = (outr != nullptr);
+	float *qr = want_out ? outr + (long) row * ldo : nullptr;
+	float *qi = want_out ? outi + (long) row * ldo : nullptr;
+	if (V == 4) {
+		for (int c = t * 4; c < cols; c += STRIDE * 4) {
+			float4 a = *reinterpret_cast<const float4 *>(pr + c);
+			float4 b = *reinterpret_cast<const float4 *>(pi + c);
+			float o_r[4] = {(float) (a.x * inv), (float) (a.y * inv), (float) (a.z * inv), (float) (a.w * inv)};
+			float o_i[4] = {(float) (b.x * inv), (float) (b.y * inv), (float) (b.z * inv), (float) (b.w * inv)};
+#pragma unroll
+			for (int k = 0; k < 4; ++k) {
+				float p = (float) ((double) o_r[k] * o_r[k] + (double) o_i[k] * o_i[k]);
+				if (p > best.v) best = ArgMax{p, c + k};
+			}
+			if (want_out && live) {
+				*reinterpret_cast<float4 *>(qr + c) = make_float4(o_r[0], o_r[1], o_r[2], o_r[3]);
+				*reinterpret_cast<float4 *>(qi + c) = make_float4(o_i[0], o_i[1], o_i[2], o_i[3]);
+			}
+		}
+	} else {
+		for (int c = t; c < cols; c += STRIDE) {
+			float o_r = (float) (pr[c] * inv), o_i = (float) (pi[c] * inv);
+			float p = (float) ((double) o_r * o_r + (double) o_i * o_i);
+			if (p > best.v) best = ArgMax{p, c};
+			if (want_out && live) {
+				qr[c] = o_r;
+				qi[c] = o_i;
+			}
+		}
+	}
+	best = group_reduce<ArgMax, G>(best, ArgMaxOp(), lds_a, slot, wig, lane);
+	if (live && t == 0) {
+		const int label = labels[row];
+		float o_r = (float) (pr[label] * inv), o_i = (float) (pi[label] * inv);
+		float p = (float) ((double) o_r * o_r + (double) o_i * o_i);
+		p = (p < 1e-15f ? 1e-15f : p);
+		s[row] = S;
+		loss[row] = -logf(p);
+		argmax[row] = best.i;
+	}
+}
+
+// ---------------------------------------------------------------------------------------------- SoftMax (L2 normalise)
+// impl/softmax.h:33-60 upstream
+template <int V, int G>
+__global__ __launch_bounds__(TPB) void l2norm_fwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		float *__restrict__ yr, float *__restrict__ yi, long ldy, float *__restrict__ s, int rows, int cols) {
+	__shared__ double lds_d[TPB / 64];
+	CNET_ROW_SETUP();
+	const float *pr = zr + (long) row * ldz, *pi = zi + (long) row * ldz;
+	double sum = row_accumulate<V, G, double>(pr, pi, cols, t,
+			[](float a, float b) { return (double) a * (double) a + (double) b * (double) b; });
+	sum = group_reduce<double, G>(sum, SumD(), lds_d, slot, wig, lane);
+	double nrm = sqrt(sum);
+	if (nrm <= 1.0e-15) nrm = 1.0e-15;
+	if ((float) (nrm * nrm * nrm) < 1.0e-15f) nrm = 1.0e-15;
+	const double inv = 1.0 / nrm;
+	if (!live) return;
+	float *qr = yr + (long) row * ldy, *qi = yi + (long) row * ldy;
+	if (V == 4) {
+		for (int c = t * 4; c < cols; c += STRIDE * 4) {
+			float4 a = *reinterpret_cast<const float4 *>(pr + c);
+			float4 b = *reinterpret_cast<const float4 *>(pi + c);
+			*reinterpret_cast<float4 *>(qr + c) =
+					make_float4((float) (a.x * inv), (float) (a.y * inv), (float) (a.z * inv), (float) (a.w * inv));
+			*reinterpret_cast<float4 *>(qi + c) =
+					make_float4((float) (b.x * inv), (float) (b.y * inv), (float) (b.z * inv), (float) (b.w * inv));
+		}
+	} else {
+		for (int c = t; c < cols; c += STRIDE) {
+			qr[c] = (float) (pr[c] * inv);
+			qi[c] = (float) (pi[c] * inv);
+		}
+	}
+	if (t == 0 && s) s[row] = (float) sum;
+}
+
+// Closed form of the chain rule of impl/cfunc.h:290-325 with the Jacobians of impl/softmax.h:62-73 upstream:
+//   A = sum_j G_j z_j + sum_j Gs_j conj(z_j)
+//   dz_i  = G_i /sqrt(S) - conj(z_i) A / (2 S^1.5)
+//   dzs_i = Gs_i/sqrt(S) - z_i       A / (2 S^1.5)
+template <int V, int G>
+__global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		const float *__restrict__ s, const float *__restrict__ g_re, const float *__restrict__ g_im,
+		const float *__restrict__ gs_re, const float *__restrict__ gs_im, long ldg, float *__restrict__ d_re,
+		float *__restrict__ d_im, float *__restrict__ ds_re, float *__restrict__ ds_im, long ldd, int rows, int cols,
+		int accumulate) {
+	__shared__ Cplx4 lds_c[TPB / 64];
+	CNET_ROW_SETUP();
+	const long oz = (long) row * ldz, og = (long) row * ldg, od = (long) row * ldd;
+	Cplx4 acc = {0.f, 0.f, 0.f, 0.f};  // a,b: G z   c,d: Gs conj z
+	for (int c = t; c < cols; c += STRIDE) {
+		float a = zr[oz + c], b = zi[oz + c];
+		float gr = g_re[og + c], gi = g_im[og + c], sr = gs_re[og + c], si = gs_im[og + c];
+		acc.a += gr * a - gi * b;
+		acc.b += gr * b + gi * a;
+		acc.c += sr * a + si * b;
+		acc.d += si * a - sr * b;
+	}
+	acc = group_reduce<Cplx4, G>(acc, SumC4(), lds_c, slot, wig, lane);
+	if (!live) return;
+	const float S = s[row];
+	double nrm = sqrt((double) S);
+	if (nrm <= 1.0e-15) nrm = 1.0e-15;
+	float cube = (float) (nrm * nrm * nrm);
+	const float inv = (float) (1.0 / nrm);
+	const float Ar = 0.5f * (acc.a + acc.c) / cube, Ai = 0.5f * (acc.b + acc.d) / cube;
+	for (int c = t; c < cols; c += STRIDE) {
+		float a = zr[oz + c], b = zi[oz + c];
+		float gr = g_re[og + c], gi = g_im[og + c], sr = gs_re[og + c], si = gs_im[og + c];
+		// conj(z) A = (a Ar + b Ai) + i (a Ai - b Ar) ;  z A = (a Ar - b Ai) + i (a Ai + b Ar)
+		float o0 = gr * inv - (a * Ar + b * Ai);
+		float o1 = gi * inv - (a * Ai - b * Ar);
+		float o2 = sr * inv - (a * Ar - b * Ai);
+		float o3 = si * inv - (a * Ai + b * Ar);
+		if (accumulate) {
+			o0 += d_re[od + c];
+			o1 += d_im[od + c];
+			o2 += ds_re[od + c];
+			o3 += ds_im[od + c];
+		}
+		d_re[od + c] = o0;
+		d_im[od + c] = o1;
+		ds_re[od + c] = o2;
+		ds_im[od + c] = o3;
+	}
+}
+
+// ---------------------------------------------------------------------------------------------- batch (column) sum
+// stage 1: blockIdx.y = slab of rows; thread = V columns; partial[slab][cols]
+template <int V>
+__global__ __launch_bounds__(TPB) void colsum_partial_kernel(const float *__restrict__ src, long ld, float *__restrict__ partial,
+		int rows, int cols, int rows_per_slab) {
+	const long col = ((long) blockIdx.x * TPB + threadIdx.x) * V;
+	if (col >= cols) return;
+	const int r0 = blockIdx.y * rows_per_slab, r1 = min(rows, r0 + rows_per_slab);
+	float acc[V];
+#pragma unroll
+	for (int k = 0; k < V; ++k) acc[k] = 0.f;
+	for (int r = r0; r < r1; ++r) {
+		if (V == 4) {
+			float4 v = *reinterpret_cast<const float4 *>(src + (long) r * ld + col);
+			acc[0] += v.x;
+			acc[1 % V] += v.y;
+			acc[2 % V] += v.z;
+			acc[3 % V] += v.w;
+		} else {
+			acc[0] += src[(long) r * ld + col];
+		}
+	}
+#pragma unroll
+	for (int k = 0; k < V; ++k) partial[(long) blockIdx.y * cols + col + k] = acc[k];
+}
+
+__global__ __launch_bounds__(TPB) void colsum_final_kernel(const float *__restrict__ partial, int nslabs, int cols,
+		float *__restrict__ dst, int accumulate) {
+	const int c = blockIdx.x * TPB + threadIdx.x;
+	if (c >= cols) return;
+	float s = 0.f;
+	for (int k = 0; k < nslabs; ++k) s += partial[(long) k * cols + c];
+	dst[c] = accumulate ? dst[c] + s : s;
+}
+
+inline bool mult4(long a, long b = 0, long c = 0, long d = 0) { return !(a % 4) && !(b % 4) && !(c % 4) && !(d % 4); }
+
+}  // namespace
+
+using namespace cnet;
+
+// rows short enough for one wavefront each get four rows per workgroup; long rows get the whole workgroup
+#define CNET_ROW_LAUNCH(KERNEL, VEC_OK, ...)                                                                          \
+	do {                                                                                                              \
+		const bool wide = cols > 2048;                                                                                \
+		const int rpb = wide ? 1 : TPB / 64;                                                                          \
+		dim3 grid((unsigned) ((rows + rpb - 1) / rpb));                                                               \
+		if (VEC_OK) {                                                                                                 \
+			if (wide) hipLaunchKernelGGL((KERNEL<4, 4>), grid, dim3(TPB), 0, rt().stream, __VA_ARGS__);               \
+			else hipLaunchKernelGGL((KERNEL<4, 1>), grid, dim3(TPB), 0, rt().stream, __VA_ARGS__);                    \
+		} else {                                                                                                      \
+			if (wide) hipLaunchKernelGGL((KERNEL<1, 4>), grid, dim3(TPB), 0, rt().stream, __VA_ARGS__);               \
+			else hipLaunchKernelGGL((KERNEL<1, 1>), grid, dim3(TPB), 0, rt().stream, __VA_ARGS__);                    \
+		}                                                                                                             \
+		CNET_LAUNCH_CHECK();                                                                                          \
+	} while (0)
+
+extern "C" {
+
+int cnet_l2out_fwd(const float *z_re, const float *z_im, int64_t ldz, float *loss, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols > 0);
+	if (!rows) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && loss && ldz >= cols);
+	const bool vec = mult4(cols, ldz) && aligned16(z_re) && aligned16(z_im);
+	CNET_ROW_LAUNCH(l2out_fwd_kernel, vec, z_re, z_im, (long) ldz, loss, rows, cols);
+	return CNET_OK;
+}
+
+int cnet_cross_entropy_fwd(const float *z_re, const float *z_im, int64_t ldz, const int32_t *labels, float *out_re,
+		float *out_im, int64_t ldo, float *s, float *loss, int32_t *argmax, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols > 0);
+	if (!rows) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && labels && s && loss && argmax && ldz >= cols);
+	CNET_CHECK_ARG((out_re == nullptr) == (out_im == nullptr));
+	CNET_CHECK_ARG(out_re == nullptr || ldo >= cols);
+	const bool vec = mult4(cols, ldz, out_re ? ldo : 0) && aligned16(z_re) && aligned16(z_im) && aligned16(out_re) &&
+			aligned16(out_im);
+	CNET_ROW_LAUNCH(crossent_fwd_kernel, vec, z_re, z_im, (long) ldz, labels, out_re, out_im, (long) ldo, s, loss, argmax, rows,
+			cols);
+	return CNET_OK;
+}
+
+int cnet_l2norm_fwd(const float *z_re, const float *z_im, int64_t ldz, float *y_re, float *y_im, int64_t ldy, float *s,
+		int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols > 0);
+	if (!rows) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && y_re && y_im && ldz >= cols && ldy >= cols);
+	const bool vec = mult4(cols, ldz, ldy) && aligned16(z_re) && aligned16(z_im) && aligned16(y_re) && aligned16(y_im);
+	CNET_ROW_LAUNCH(l2norm_fwd_kernel, vec, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols);
+	return CNET_OK;
+}
+
+int cnet_l2norm_bwd(const float *z_re, const float *z_im, int64_t ldz, const float *s, const float *g_dz_re,
+		const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg, float *dz_dz_re, float *dz_dz_im,
+		float *dz_dzs_re, float *dz_dzs_im, int64_t lddz, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols > 0);
+	if (!rows) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && s && g_dz_re && g_dz_im && g_dzs_re && g_dzs_im);
+	CNET_CHECK_ARG(dz_dz_re && dz_dz_im && dz_dzs_re && dz_dzs_im && ldz >= cols && ldg >= cols && lddz >= cols);
+	CNET_ROW_LAUNCH(l2norm_bwd_kernel, false, z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg, dz_dz_re,
+			dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate);
+	return CNET_OK;
+}
+
+int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows > 0 && cols >= 0);
+	if (!cols) return CNET_OK;
+	CNET_CHECK_ARG(src && dst && lds >= cols);
+	const bool vec = mult4(cols, lds) && aligned16(src);
+	const int V = vec ? 4 : 1;
+	const long col_blocks = ((long) cols / V + TPB - 1) / TPB;
+	const long want_blocks = 8L * rt().prop.multiProcessorCount;
+	int nslabs = (int) ((want_blocks + col_blocks - 1) / col_blocks);
+	if (nslabs > rows) nslabs = rows;
+	const int rows_per_slab = (rows + nslabs - 1) / nslabs;
+	nslabs = (rows + rows_per_slab - 1) / rows_per_slab;
+	float *partial = (float *) workspace((size_t) nslabs * cols * sizeof(float));
+	if (!partial) return CNET_ERR_OUT_OF_MEMORY;
+	dim3 grid((unsigned) col_blocks, (unsigned) nslabs);
+	if (vec)
+		hipLaunchKernelGGL(colsum_partial_kernel<4>, grid, dim3(TPB), 0, rt().stream, src, (long) lds, partial, rows, cols, rows_per_slab);
+	else
+		hipLaunchKernelGGL(colsum_partial_kernel<1>, grid, dim3(TPB), 0, rt().stream, src, (long) lds, partial, rows, cols, rows_per_slab);
+	CNET_LAUNCH_CHECK();
+	hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned) ((cols + TPB - 1) / TPB)), dim3(TPB), 0, rt().stream, partial, nslabs, cols, dst,
+			accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,170 @@
+// Lifetime, memory and stream entry points of libcnet_hip.so.
+#include "common.hpp"
+
+#include <cstring>
+#include <map>
+#include <string>
+
+namespace cnet {
+
+static thread_local char g_error[1024] = "";
+static Runtime g_rt;
+
+Runtime &rt() { return g_rt; }
+
+int fail(int code, const char *fmt, ...) {
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(g_error, sizeof(g_error), fmt, ap);
+	va_end(ap);
+	return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+	snprintf(g_error, sizeof(g_error), "HIP error %d (%s) in %s", (int) e, hipGetErrorString(e), what);
+	return e == hipErrorOutOfMemory ? CNET_ERR_OUT_OF_MEMORY : CNET_ERR_HIP;
+}
+
+void *workspace(size_t bytes) {
+	Runtime &r = rt();
+	if (bytes <= r.workspace_bytes) return r.workspace;
+	if (r.workspace) {
+		// queued kernels may still read the old buffer
+		hipStreamSynchronize(r.stream);
+		hipFree(r.workspace);
+		r.workspace = nullptr;
+		r.workspace_bytes = 0;
+	}
+	size_t want = bytes + bytes / 2;
+	hipError_t e = hipMalloc(&r.workspace, want);
+	if (e != hipSuccess) {
+		hip_fail(e, "workspace hipMalloc");
+		r.workspace = nullptr;
+		return nullptr;
+	}
+	r.workspace_bytes = want;
+	return r.workspace;
+}
+
+void release_twiddles();  // cdft.hip
+
+}  // namespace cnet
+
+using namespace cnet;
+
+extern "C" {
+
+int cnet_init(int device) {
+	Runtime &r = rt();
+	if (r.ready) {
+		if (r.device == device) return CNET_OK;
+		return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_init: already initialised on device %d", r.device);
+	}
+	int count = 0;
+	CNET_HIP(hipGetDeviceCount(&count));
+	if (device < 0 || device >= count) return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_init: device %d of %d", device, count);
+	CNET_HIP(hipSetDevice(device));
+	CNET_HIP(hipGetDeviceProperties(&r.prop, device));
+	if (strncmp(r.prop.gcnArchName, "gfx950", 6) != 0)
+		return fail(CNET_ERR_UNSUPPORTED, "cnet_init: kernels are built for gfx950 only, device is %s", r.prop.gcnArchName);
+	CNET_HIP(hipStreamCreateWithFlags(&r.own_stream, hipStreamNonBlocking));
+	r.stream = r.own_stream;
+	r.device = device;
+	r.ready = true;
+	return CNET_OK;
+}
+
+int cnet_shutdown(void) {
+	Runtime &r = rt();
+	if (!r.ready) return CNET_OK;
+	hipStreamSynchronize(r.stream);
+	release_twiddles();
+	if (r.workspace) hipFree(r.workspace);
+	r.workspace = nullptr;
+	r.workspace_bytes = 0;
+	if (r.own_stream) hipStreamDestroy(r.own_stream);
+	r.own_stream = r.stream = nullptr;
+	r.ready = false;
+	r.device = -1;
+	return CNET_OK;
+}
+
+int cnet_get_device_info(cnet_device_info *out) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(out != nullptr);
+	Runtime &r = rt();
+	memset(out, 0, sizeof(*out));
+	snprintf(out->name, sizeof(out->name), "%s", r.prop.name);
+	snprintf(out->arch, sizeof(out->arch), "%s", r.prop.gcnArchName);
+	out->compute_units = r.prop.multiProcessorCount;
+	out->clock_khz = r.prop.clockRate;
+	out->wavefront_size = r.prop.warpSize;
+	out->lds_bytes_per_block = (int) r.prop.maxSharedMemoryPerMultiProcessor;
+	out->hbm_bytes = (int64_t) r.prop.totalGlobalMem;
+	out->fp32_matrix_peak_tflops = 256.0 * r.prop.multiProcessorCount * (r.prop.clockRate * 1e3) / 1e12;
+	return CNET_OK;
+}
+
+const char *cnet_last_error(void) { return g_error; }
+
+void *cnet_stream(void) { return rt().ready ? (void *) rt().stream : nullptr; }
+
+int cnet_set_stream(void *hip_stream) {
+	CNET_REQUIRE_INIT();
+	Runtime &r = rt();
+	CNET_HIP(hipStreamSynchronize(r.stream));
+	r.stream = hip_stream ? (hipStream_t) hip_stream : r.own_stream;
+	return CNET_OK;
+}
+
+int cnet_sync(void) {
+	CNET_REQUIRE_INIT();
+	CNET_HIP(hipStreamSynchronize(rt().stream));
+	return CNET_OK;
+}
+
+int cnet_alloc(size_t bytes, void **out) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(out != nullptr);
+	*out = nullptr;
+	if (bytes == 0) return CNET_OK;
+	CNET_HIP(hipMalloc(out, bytes));
+	return CNET_OK;
+}
+
+int cnet_free(void *ptr) {
+	CNET_REQUIRE_INIT();
+	if (!ptr) return CNET_OK;
+	CNET_HIP(hipStreamSynchronize(rt().stream));
+	CNET_HIP(hipFree(ptr));
+	return CNET_OK;
+}
+
+int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes) {
+	CNET_REQUIRE_INIT();
+	if (!bytes) return CNET_OK;
+	CNET_CHECK_ARG(dst && host_src);
+	// pageable source: hipMemcpyAsync stages and returns after the copy was consumed from the host buffer
+	CNET_HIP(hipMemcpyAsync(dst, host_src, bytes, hipMemcpyHostToDevice, rt().stream));
+	CNET_HIP(hipStreamSynchronize(rt().stream));
+	return CNET_OK;
+}
+
+int cnet_memcpy_d2h(void *host_dst, const void *src, size_t bytes) {
+	CNET_REQUIRE_INIT();
+	if (!bytes) return CNET_OK;
+	CNET_CHECK_ARG(host_dst && src);
+	CNET_HIP(hipMemcpyAsync(host_dst, src, bytes, hipMemcpyDeviceToHost, rt().stream));
+	CNET_HIP(hipStreamSynchronize(rt().stream));
+	return CNET_OK;
+}
+
+int cnet_memcpy_d2d(void *dst, const void *src, size_t bytes) {
+	CNET_REQUIRE_INIT();
+	if (!bytes) return CNET_OK;
+	CNET_CHECK_ARG(dst && src);
+	CNET_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, rt().stream));
+	return CNET_OK;
+}
+
+}  // extern "C"

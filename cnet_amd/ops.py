@@ -1,0 +1,195 @@
+"""Thin Python call wrappers over the C-ABI layer entry points (argument marshalling only; used by tests and bench).
+
+A complex matrix on the device is a `CMat`: two planes (re, im) of one DevArray pair with a leading dimension.
+A gradient carrier is a `Grad`: four planes.  `sub(col0, cols)` selects a column window without copying, which is
+how a producer writes into its slot of a consumer's concatenated input block.
+"""
+import numpy as np
+
+from . import capi
+from .capi import call
+
+
+class Plane:
+    """One fp32 plane: device pointer, logical shape, leading dimension (elements)."""
+
+    def __init__(self, ptr, rows, cols, ld, owner=None):
+        self.ptr, self.rows, self.cols, self.ld, self.owner = ptr, rows, cols, ld, owner
+
+    @staticmethod
+    def from_host(a):
+        a = np.ascontiguousarray(a, np.float32)
+        if a.ndim == 1:
+            a = a.reshape(1, -1)
+        d = capi.to_device(a)
+        return Plane(d.ptr, a.shape[0], a.shape[1], a.shape[1], d)
+
+    @staticmethod
+    def empty(rows, cols, ld=None, zero=False):
+        ld = ld or cols
+        d = capi.DevArray((rows, ld))
+        if zero:
+            d.zero()
+        return Plane(d.ptr, rows, cols, ld, d)
+
+    def sub(self, col0, cols):
+        return Plane(self.ptr + 4 * col0, self.rows, cols, self.ld, self.owner)
+
+    def host(self):
+        full = self.owner.download().reshape(-1)
+        base = (self.ptr - self.owner.ptr) // 4
+        idx = base + np.arange(self.rows)[:, None] * self.ld + np.arange(self.cols)[None, :]
+        return full[idx]
+
+
+class CMat:
+    def __init__(self, re, im):
+        self.re, self.im = re, im
+        self.rows, self.cols, self.ld = re.rows, re.cols, re.ld
+        assert im.ld == re.ld and im.cols == re.cols
+
+    @staticmethod
+    def from_host(re, im):
+        return CMat(Plane.from_host(re), Plane.from_host(im))
+
+    @staticmethod
+    def empty(rows, cols, ld=None, zero=False):
+        return CMat(Plane.empty(rows, cols, ld, zero), Plane.empty(rows, cols, ld, zero))
+
+    def sub(self, col0, cols):
+        return CMat(self.re.sub(col0, cols), self.im.sub(col0, cols))
+
+    def host(self):
+        return self.re.host(), self.im.host()
+
+    def p(self):
+        return (self.re.ptr, self.im.ptr)
+
+
+class Grad:
+    def __init__(self, planes):
+        self.planes = list(planes)
+        self.rows, self.cols, self.ld = planes[0].rows, planes[0].cols, planes[0].ld
+
+    @staticmethod
+    def from_host(four):
+        return Grad([Plane.from_host(a) for a in four])
+
+    @staticmethod
+    def empty(rows, cols, ld=None, zero=False):
+        return Grad([Plane.empty(rows, cols, ld, zero) for _ in range(4)])
+
+    def sub(self, col0, cols):
+        return Grad([p.sub(col0, cols) for p in self.planes])
+
+    def host(self):
+        return [p.host() for p in self.planes]
+
+    def p(self):
+        return tuple(p.ptr for p in self.planes)
+
+
+def ints(a):
+    return capi.to_device(np.ascontiguousarray(a, np.int32))
+
+
+# ------------------------------------------------------------------------------------------------- GEMM family
+def cgemm(A, Bm, Cm, M, N, K, a_kmajor=0, b_kmajor=0, conj_b=0, accumulate=0):
+    call("cnet_cgemm", a_kmajor, b_kmajor, conj_b, M, N, K, *A.p(), A.ld, *Bm.p(), Bm.ld, *Cm.p(), Cm.ld, accumulate)
+
+
+def linear_fwd(x, w, y, accumulate=0):
+    call("cnet_clinear_fwd", *x.p(), x.ld, *w.p(), w.ld, *y.p(), y.ld, x.rows, x.cols, w.rows, accumulate)
+
+
+def linear_bwd_input(g, w, dx, accumulate=0):
+    call("cnet_clinear_bwd_input", *g.p(), g.ld, *w.p(), w.ld, *dx.p(), dx.ld, g.rows, w.cols, w.rows, accumulate)
+
+
+def linear_bwd_weight(g, x, dw, accumulate=0):
+    call("cnet_clinear_bwd_weight", *g.p(), g.ld, *x.p(), x.ld, *dw.p(), dw.ld, g.rows, x.cols, g.cols, accumulate)
+
+
+def dft_fwd(x, y, accumulate=0):
+    call("cnet_cdft_fwd", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols, accumulate)
+
+
+def dft_bwd(g, dx, accumulate=0):
+    call("cnet_cdft_bwd", *g.p(), g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
+
+
+# ------------------------------------------------------------------------------------------------- elementwise
+def hadamard_fwd(u, v, y, shared=False):
+    call("cnet_hadamard_fwd", *u.p(), u.ld, *v.p(), 0 if shared else v.ld, *y.p(), y.ld, u.rows, u.cols)
+
+
+def hadamard_bwd(u, v, g, du, dv, shared=False, accumulate=0):
+    call("cnet_hadamard_bwd", *u.p(), u.ld, *v.p(), 0 if shared else v.ld, *g.p(), g.ld, *du.p(), du.ld, *dv.p(),
+         dv.ld, u.rows, u.cols, accumulate)
+
+
+def gelu_fwd(x, y):
+    call("cnet_cgelu_fwd", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols)
+
+
+def gelu_bwd(x, g, dx, accumulate=0):
+    call("cnet_cgelu_bwd", *x.p(), x.ld, *g.p(), g.ld, *dx.p(), dx.ld, x.rows, x.cols, accumulate)
+
+
+def residual_fwd(u, v, y):
+    call("cnet_residual_fwd", *u.p(), u.ld, *v.p(), v.ld, *y.p(), y.ld, u.rows, u.cols)
+
+
+def residual_bwd(g, du, dv, accumulate=0):
+    call("cnet_residual_bwd", *g.p(), g.ld, *du.p(), du.ld, *dv.p(), dv.ld, g.rows, g.cols, accumulate)
+
+
+def l2norm_fwd(z, y, s):
+    call("cnet_l2norm_fwd", *z.p(), z.ld, *y.p(), y.ld, s.ptr, z.rows, z.cols)
+
+
+def l2norm_bwd(z, s, g, dz, accumulate=0):
+    call("cnet_l2norm_bwd", *z.p(), z.ld, s.ptr, *g.p(), g.ld, *dz.p(), dz.ld, z.rows, z.cols, accumulate)
+
+
+def cross_entropy_fwd(z, labels, s, loss, argmax, out=None):
+    o = out.p() if out is not None else (None, None)
+    call("cnet_cross_entropy_fwd", *z.p(), z.ld, labels.ptr, o[0], o[1], out.ld if out is not None else 0, s.ptr,
+         loss.ptr, argmax.ptr, z.rows, z.cols)
+
+
+def cross_entropy_bwd(z, s, labels, dz):
+    call("cnet_cross_entropy_bwd", *z.p(), z.ld, s.ptr, labels.ptr, *dz.p(), dz.ld, z.rows, z.cols)
+
+
+def l2out_fwd(z, loss):
+    call("cnet_l2out_fwd", *z.p(), z.ld, loss.ptr, z.rows, z.cols)
+
+
+def l2out_bwd(z, dz, accumulate=0):
+    call("cnet_l2out_bwd", *z.p(), z.ld, *dz.p(), dz.ld, z.rows, z.cols, accumulate)
+
+
+def copy2d(src, dst):
+    call("cnet_copy2d", src.ptr, src.ld, dst.ptr, dst.ld, src.rows, src.cols)
+
+
+def add2d(src, dst):
+    call("cnet_add2d", src.ptr, src.ld, dst.ptr, dst.ld, src.rows, src.cols)
+
+
+def batch_sum(src, dst, accumulate=0):
+    call("cnet_batch_sum", src.ptr, src.ld, dst.ptr, src.rows, src.cols, accumulate)
+
+
+def sgd_update(z, dzs_re, dzs_im, lr, zero_grad=1):
+    call("cnet_sgd_update", z.re.ptr, z.im.ptr, dzs_re.ptr, dzs_im.ptr, z.rows * z.cols, lr, zero_grad)
+
+
+def embedding_fwd(table, tokens, y, slots):
+    call("cnet_embedding_fwd", *table.p(), table.cols, table.rows, tokens.ptr, *y.p(), y.ld, y.rows, slots)
+
+
+def embedding_bwd(tokens, gs_re, gs_im, dtab_re, dtab_im, dim, vocab, rows, slots, accumulate=0):
+    call("cnet_embedding_bwd", tokens.ptr, gs_re.ptr, gs_im.ptr, gs_re.ld, dtab_re.ptr, dtab_im.ptr, dim, vocab, rows,
+         slots, accumulate)

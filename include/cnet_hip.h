@@ -1,0 +1,185 @@
+/*
+ * cnet_hip.h - C ABI of the MI355X (gfx950) device layer for CNet's dense complex-valued hot path.
+ *
+ * This library takes the place of the device layer of upstream CNet: the CUDA kernels and host launchers in
+ * gpu/kernels.cpp, gpu/reduce.cpp, gpu/reducegrad.cpp and the allocator in gpu/allocator.h / gpu/allocator.cu.
+ * Each entry point names the upstream interface it replaces (paths under the upstream tree).
+ *
+ * Conventions
+ *  - A complex matrix is two fp32 planes (re, im), row-major, with a leading dimension in ELEMENTS (ld >= cols).
+ *    One row = one sample of the batch (one upstream "clone").  Parameters are stored once (no per-sample copy).
+ *  - A gradient carrier is four planes: dz_re, dz_im (dL/dz) and dzs_re, dzs_im (dL/d conj z), as in
+ *    impl/vars.h:40-46 upstream.
+ *  - `accumulate` != 0 adds into the destination (the upstream `+=` into zeroed planes); 0 overwrites, which saves
+ *    the zero-fill and the read.
+ *  - Every function returns 0 on success and a negative cnet_status otherwise; it never exits the process
+ *    (upstream gpuErrchk prints and exits, gpu/kernels.h:18-28).  cnet_last_error() describes the last failure
+ *    of the calling thread.
+ *  - All work is queued on one HIP stream (cnet_stream()); nothing synchronises except cnet_sync(), the
+ *    device-to-host copies and cnet_shutdown().  One host thread per process drives the library.
+ *  - Pointers are device pointers unless the parameter name starts with host_.
+ */
+#ifndef CNET_HIP_H_
+#define CNET_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+	CNET_OK = 0,
+	CNET_ERR_NOT_INITIALIZED = -1,
+	CNET_ERR_INVALID_ARGUMENT = -2,
+	CNET_ERR_HIP = -3,          /* a HIP runtime call failed; text in cnet_last_error() */
+	CNET_ERR_OUT_OF_MEMORY = -4,
+	CNET_ERR_UNSUPPORTED = -5
+} cnet_status;
+
+typedef struct {
+	char name[256];
+	char arch[64];
+	int compute_units;
+	int clock_khz;            /* maximum engine clock */
+	int wavefront_size;
+	int lds_bytes_per_block;  /* largest LDS allocation one workgroup may request */
+	int64_t hbm_bytes;
+	double fp32_matrix_peak_tflops; /* 256 flop/clk/CU x compute_units x clock */
+} cnet_device_info;
+
+/* ---- lifetime, memory, stream: replaces GpuHelper (gpu/allocator.h:97-408, gpu/allocator.cu:4-31) ---------- */
+int cnet_init(int device);                 /* select device, create the stream; idempotent */
+int cnet_shutdown(void);                   /* sync, free library-owned buffers (twiddles, workspace), destroy stream */
+int cnet_get_device_info(cnet_device_info *out);   /* getTotalGlobalMem / getMaxThreadsPerBlock / PrintInfo */
+const char *cnet_last_error(void);
+void *cnet_stream(void);                   /* the hipStream_t all launches use */
+int cnet_set_stream(void *hip_stream);     /* adopt a caller-owned stream (NULL restores the library's own) */
+int cnet_sync(void);
+int cnet_alloc(size_t bytes, void **out);  /* float_allocate_on_gpu & friends (gpu/allocator.h:121-180) */
+int cnet_free(void *ptr);
+int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes);   /* *_copy_to_gpu   (gpu/allocator.h:182-260) */
+int cnet_memcpy_d2h(void *host_dst, const void *src, size_t bytes);   /* *_copy_from_gpu (gpu/allocator.h:262-328); synchronises */
+int cnet_memcpy_d2d(void *dst, const void *src, size_t bytes);
+int cnet_memset_zero(void *dst, size_t bytes);  /* GpuMapping::zeroGradients (gpu/kernels.cpp:444-469) */
+
+/* ---- complex GEMM core -------------------------------------------------------------------------------------
+ * C[M x N] (+)= op(A)[M x K] * op(B)[K x N], complex, fp32 MFMA, four real products per complex product.
+ *   a_kmajor = 0: A stored [M][lda] (k contiguous)      1: A stored [K][lda] (m contiguous, i.e. A^T in memory)
+ *   b_kmajor = 0: B stored [N][ldb] (k contiguous)      1: B stored [K][ldb] (n contiguous)
+ *   conj_b  != 0: use conj(B).
+ * The layer entry points below are thin shape adapters over this one.  No upstream counterpart (upstream has
+ * no GEMM: one thread per multiply and a shared-memory tree, gpu/reduce.cpp:100-158). */
+int cnet_cgemm(int a_kmajor, int b_kmajor, int conj_b, int M, int N, int K,
+               const float *a_re, const float *a_im, int64_t lda,
+               const float *b_re, const float *b_im, int64_t ldb,
+               float *c_re, float *c_im, int64_t ldc, int accumulate);
+
+/* ---- Linear: replaces LinearGpu::gpu_linear_forward / gpu_linear_backward
+ *      (gpu/reduce.cpp:56-77,532-604; gpu/reducegrad.cpp:20-44,288-322), CPU twin impl/linear.h:51-110.
+ * x[B][K], w[N][K] (stored once), y[B][N].   y = x * w^T */
+int cnet_clinear_fwd(const float *x_re, const float *x_im, int64_t ldx,
+                     const float *w_re, const float *w_im, int64_t ldw,
+                     float *y_re, float *y_im, int64_t ldy, int B, int K, int N, int accumulate);
+/* dx.dz = g.dz * w ; dx.dzs = g.dzs * conj(w)            (both products in one launch) */
+int cnet_clinear_bwd_input(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,
+                           int64_t ldg, const float *w_re, const float *w_im, int64_t ldw,
+                           float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
+                           int B, int K, int N, int accumulate);
+/* dw.dz = g.dz^T * x ; dw.dzs = g.dzs^T * conj(x), summed over the B rows (the upstream sum over clones,
+ * gpu/kernels.cpp:566-598, is part of the product here; deterministic, no atomics). */
+int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,
+                            int64_t ldg, const float *x_re, const float *x_im, int64_t ldx,
+                            float *dw_dz_re, float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im, int64_t lddw,
+                            int B, int K, int N, int accumulate);
+
+/* ---- FourierTrans as dense complex GEMM: replaces FourierGpu::gpu_fft_forward / gpu_fft_backward
+ *      (gpu/reduce.cpp:25-35,160-187,382-393; gpu/reducegrad.cpp:45-48,324-336) and the root-table upload
+ *      u_roots_allocate_and_copy_on_gpu (gpu/allocator.h:389-407).  CPU twin impl/ft.h:37-80.
+ * F[p][q] = exp(-2 pi i p q / n) / sqrt(n), generated on the device with exact integer reduction of p*q mod n. */
+int cnet_cdft_plan(int n);      /* build (once) and keep the n x n twiddle planes; called at net allocation time */
+int cnet_cdft_twiddle(int n, const float **f_re, const float **f_im);  /* the planes of an existing plan */
+int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
+                  int B, int n, int accumulate);      /* y = x * F */
+int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+                  float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
+                  int B, int n, int accumulate);      /* dx.dz = g.dz * F ; dx.dzs = g.dzs * conj(F) */
+
+/* ---- Hadamard: replaces gpu_hadamard_forward / _backward (gpu/kernels.cpp:204-274), CPU twin impl/hadamard.h:34-68.
+ * y = u .* v.  ldv == 0: v is one parameter row shared by all rows and dv is the sum over rows. */
+int cnet_hadamard_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+                      float *y_re, float *y_im, int64_t ldy, int rows, int cols);
+int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+                      const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+                      float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
+                      float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
+                      int rows, int cols, int accumulate);
+
+/* ---- CGelu: replaces gpu_gelu_forward / _backward (gpu/kernels.cpp:276-360), CPU twin impl/relu.h:119-168. */
+int cnet_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
+                   int rows, int cols);
+int cnet_cgelu_bwd(const float *x_re, const float *x_im, int64_t ldx,
+                   const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+                   float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
+                   int rows, int cols, int accumulate);
+
+/* ---- Residual: replaces gpu_residual_forward / _backward (gpu/kernels.cpp:145-202), CPU twin impl/residual.h:40-77. */
+int cnet_residual_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+                      float *y_re, float *y_im, int64_t ldy, int rows, int cols);
+int cnet_residual_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+                      float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
+                      float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
+                      int rows, int cols, int accumulate);
+
+/* ---- SoftMax (L2 normalisation y = z/|z|): replaces SoftMaxGpu::gpu_soft_max_forward / _backward
+ *      (gpu/reduce.cpp:189-230,449-466; gpu/reducegrad.cpp:10-19,60-66,268-286), CPU twin impl/softmax.h:33-73 with
+ *      the chain rule of impl/cfunc.h:290-325 in closed O(n) form.  s[rows] receives sum |z|^2 per row. */
+int cnet_l2norm_fwd(const float *z_re, const float *z_im, int64_t ldz, float *y_re, float *y_im, int64_t ldy,
+                    float *s, int rows, int cols);
+int cnet_l2norm_bwd(const float *z_re, const float *z_im, int64_t ldz, const float *s,
+                    const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+                    float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,
+                    int rows, int cols, int accumulate);
+
+/* ---- CrossEntropy: replaces CrossEntropyGpu::gpu_cross_ent_forward / _backward (gpu/reduce.cpp:469-530,609-655)
+ *      and the loss read-back of CNet::getLoss (gpu/gpu_func.h:906-926).  CPU twin impl/crossent.h:50-130.
+ * labels[rows] int32.  s = clamped sum |z|^2, loss = -log(max(|z_label|^2/s, 1e-15)), argmax = first index of the
+ * strict maximum of |z_k/sqrt(s)|^2.  out_re/out_im (normalised z) may be NULL. */
+int cnet_cross_entropy_fwd(const float *z_re, const float *z_im, int64_t ldz, const int32_t *labels,
+                           float *out_re, float *out_im, int64_t ldo, float *s, float *loss, int32_t *argmax,
+                           int rows, int cols);
+/* assigns (never accumulates), as impl/crossent.h:82-104 */
+int cnet_cross_entropy_bwd(const float *z_re, const float *z_im, int64_t ldz, const float *s, const int32_t *labels,
+                           float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,
+                           int rows, int cols);
+
+/* ---- L2Out: replaces L2Gpu::gpu_norm_forward / gpu_norm_backward (gpu/reduce.cpp:232-251,408-446),
+ *      CPU twin impl/l2out.h:33-58.  loss[rows] = sum |z|^2 ; dz = conj z, dzs = z. */
+int cnet_l2out_fwd(const float *z_re, const float *z_im, int64_t ldz, float *loss, int rows, int cols);
+int cnet_l2out_bwd(const float *z_re, const float *z_im, int64_t ldz,
+                   float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,
+                   int rows, int cols, int accumulate);
+
+/* ---- CInput and parameter plumbing: replaces gpu_input_forward / _backward (gpu/kernels.cpp:89-143),
+ *      gpu_update_input (gpu/kernels.cpp:471-492) and gpu_copy_to_clones / gpu_grad_from_clones
+ *      (gpu/kernels.cpp:528-598; with parameters stored once there is nothing to broadcast, and the sum over
+ *      clones becomes cnet_batch_sum or is fused into the producing kernel). */
+int cnet_copy2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols);       /* one plane */
+int cnet_add2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols);        /* dst += src */
+int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate); /* dst[c] (+)= sum_r src[r][c] */
+/* z -= lr * dzs ; then dzs = 0 when zero_grad != 0   (impl/cfunc.h:147-152 + impl/cnet.h:413-421) */
+int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int64_t n, float lr, int zero_grad);
+
+/* ---- CEmbedding: replaces gpu_embedding_forward / _backward (gpu/kernels.cpp:362-442), CPU twin impl/embed.h:109-148.
+ * tokens[rows][slots] int32, -1 = padding (zero row).  y[rows][slots*dim].  The backward adds the dzs rows of equal
+ * tokens in (row, slot) order - deterministic, no atomics. */
+int cnet_embedding_fwd(const float *table_re, const float *table_im, int dim, int vocab, const int32_t *tokens,
+                       float *y_re, float *y_im, int64_t ldy, int rows, int slots);
+int cnet_embedding_bwd(const int32_t *tokens, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+                       float *table_dzs_re, float *table_dzs_im, int dim, int vocab, int rows, int slots, int accumulate);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CNET_HIP_H_ */

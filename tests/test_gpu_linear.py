@@ -1,0 +1,124 @@
+"""Complex Linear (forward and the four Wirtinger backward products) on the GPU against the CPU oracle.
+
+Mirrors upstream testLinear / testLinearMaxGradient (tests/gputests.h:317, 756): same layer, CPU result as the
+reference, but seeded inputs and a relative Frobenius bound (1e-4; observed ~1e-6) instead of a loose absolute one.
+"""
+import numpy as np
+import pytest
+
+from cnet_amd import capi, ops
+from tests.gpu_util import gpu, rel_c, seeded, TOL  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [  # B, K, N
+    (1, 4, 4), (3, 8, 5), (64, 784, 10), (37, 100, 19), (130, 68, 132), (256, 256, 256), (96, 1024, 64), (257, 33, 7),
+]
+
+
+def _case(port, B, K, N, seed):
+    xr, xi = seeded(port, seed, (B, K)), seeded(port, seed + 1, (B, K))
+    wr, wi = seeded(port, seed + 2, (N, K), 1 / np.sqrt(K)), seeded(port, seed + 3, (N, K), 1 / np.sqrt(K))
+    g4 = [seeded(port, seed + 4 + p, (B, N)) for p in range(4)]
+    return xr, xi, wr, wi, g4
+
+
+@pytest.mark.parametrize("B,K,N", SHAPES)
+def test_linear_forward_and_backward(gpu, port, B, K, N):
+    xr, xi, wr, wi, g4 = _case(port, B, K, N, seed=B + K + N)
+    yr, yi = port.linear_fwd(xr, xi, wr, wi)
+    dx_o, dw_o = port.linear_bwd(xr, xi, wr, wi, g4)
+
+    x, w, g = ops.CMat.from_host(xr, xi), ops.CMat.from_host(wr, wi), ops.Grad.from_host(g4)
+    y = ops.CMat.empty(B, N)
+    ops.linear_fwd(x, w, y)
+    assert rel_c(y.host(), (yr, yi)) < TOL / 5
+    dx, dw = ops.Grad.empty(B, K), ops.Grad.empty(N, K)
+    ops.linear_bwd_input(g, w, dx)
+    ops.linear_bwd_weight(g, x, dw)
+    hx, hw = dx.host(), dw.host()
+    assert rel_c(hx[0:2], dx_o[0:2]) < TOL / 5 and rel_c(hx[2:4], dx_o[2:4]) < TOL / 5
+    assert rel_c(hw[0:2], dw_o[0:2]) < TOL / 5 and rel_c(hw[2:4], dw_o[2:4]) < TOL / 5
+
+
+def test_linear_accumulate_and_leading_dimensions(gpu, port):
+    """Outputs land in a column window of a wider buffer (a consumer's concatenated input block) and add to what is there."""
+    B, K, N = 48, 40, 24
+    xr, xi, wr, wi, g4 = _case(port, B, K, N, seed=9)
+    yr, yi = port.linear_fwd(xr, xi, wr, wi)
+    dx_o, dw_o = port.linear_bwd(xr, xi, wr, wi, g4)
+    base = seeded(port, 77, (B, 100))
+    wide = ops.CMat(ops.Plane.from_host(base), ops.Plane.from_host(base))
+    x, w, g = ops.CMat.from_host(xr, xi), ops.CMat.from_host(wr, wi), ops.Grad.from_host(g4)
+    ops.linear_fwd(x, w, wide.sub(12, N), accumulate=1)
+    hr, hi = wide.re.owner.download(), wide.im.owner.download()
+    assert rel_c((hr[:, 12:12 + N] - base[:, 12:12 + N], hi[:, 12:12 + N] - base[:, 12:12 + N]), (yr, yi)) < 1e-5
+    mask = np.ones(100, bool); mask[12:12 + N] = False
+    assert np.array_equal(hr[:, mask], base[:, mask]) and np.array_equal(hi[:, mask], base[:, mask])
+    # x read from a window of a wider buffer, gradients accumulated twice
+    xw = ops.CMat(ops.Plane.from_host(np.concatenate([base[:, :8], xr, base[:, :4]], 1)),
+                  ops.Plane.from_host(np.concatenate([base[:, :8], xi, base[:, :4]], 1))).sub(8, K)
+    dw = ops.Grad.empty(N, K, zero=True)
+    ops.linear_bwd_weight(g, xw, dw, accumulate=1)
+    ops.linear_bwd_weight(g, xw, dw, accumulate=1)
+    h = dw.host()
+    assert rel_c((h[2] / 2, h[3] / 2), dw_o[2:4]) < 1e-5
+    dx = ops.Grad.empty(B, K, ld=K + 4, zero=True)
+    ops.linear_bwd_input(g, w, dx, accumulate=1)
+    assert rel_c(dx.host()[0:2], dx_o[0:2]) < 1e-5
+
+
+def test_cgemm_all_layouts(gpu, port):
+    """C = op(A) op(B) for the four storage combinations, with and without conj(B), against numpy complex128."""
+    M, N, K = 72, 40, 52
+    A = seeded(port, 1, (M, K)) + 1j * seeded(port, 2, (M, K))
+    Bm = seeded(port, 3, (K, N)) + 1j * seeded(port, 4, (K, N))
+    for a_km in (0, 1):
+        for b_km in (0, 1):
+            for cj in (0, 1):
+                a_h = A.T if a_km else A
+                b_h = Bm if b_km else Bm.T
+                a = ops.CMat.from_host(np.ascontiguousarray(a_h.real), np.ascontiguousarray(a_h.imag))
+                b = ops.CMat.from_host(np.ascontiguousarray(b_h.real), np.ascontiguousarray(b_h.imag))
+                c = ops.CMat.empty(M, N)
+                ops.cgemm(a, b, c, M, N, K, a_km, b_km, cj)
+                want = A @ (Bm.conj() if cj else Bm)
+                cr, ci = c.host()
+                err = np.linalg.norm(cr + 1j * ci - want) / np.linalg.norm(want)
+                assert err < 1e-5, (a_km, b_km, cj, err)
+
+
+def test_linear_headline_shape_rows_against_oracle(gpu, port):
+    """B=4096, 1024->1024 (the benchmark shape).  The oracle computes a 24-row subsample; dW/dW* are compared on a
+    batch equal to that subsample, and the full-size run is checked through linearity in the batch:
+    dW(all rows) = dW(first half) + dW(second half)."""
+    B, K, N, sub = 4096, 1024, 1024, 24
+    xr, xi, wr, wi, g4 = _case(port, B, K, N, seed=2024)
+    x, w, g = ops.CMat.from_host(xr, xi), ops.CMat.from_host(wr, wi), ops.Grad.from_host(g4)
+    y, dx, dw = ops.CMat.empty(B, N), ops.Grad.empty(B, K), ops.Grad.empty(N, K)
+    ops.linear_fwd(x, w, y)
+    ops.linear_bwd_input(g, w, dx)
+    ops.linear_bwd_weight(g, x, dw)
+    rows = np.linspace(0, B - 1, sub).astype(int)
+    sx = (np.ascontiguousarray(xr[rows]), np.ascontiguousarray(xi[rows]))
+    sg = [np.ascontiguousarray(p[rows]) for p in g4]
+    yr, yi = port.linear_fwd(sx[0], sx[1], wr, wi)
+    dx_o, dw_o = port.linear_bwd(sx[0], sx[1], wr, wi, sg)
+    hy, hdx = y.host(), dx.host()
+    assert rel_c((hy[0][rows], hy[1][rows]), (yr, yi)) < TOL / 5
+    assert rel_c((hdx[0][rows], hdx[1][rows]), dx_o[0:2]) < TOL / 5
+    assert rel_c((hdx[2][rows], hdx[3][rows]), dx_o[2:4]) < TOL / 5
+    # weight gradients on the subsample batch
+    dws = ops.Grad.empty(N, K)
+    ops.linear_bwd_weight(ops.Grad.from_host(sg), ops.CMat.from_host(*sx), dws)
+    h = dws.host()
+    assert rel_c(h[0:2], dw_o[0:2]) < TOL / 5 and rel_c(h[2:4], dw_o[2:4]) < TOL / 5
+    # full batch: additivity over a split of the batch
+    half = B // 2
+    acc = ops.Grad.empty(N, K)
+    for k, sl in enumerate((slice(0, half), slice(half, B))):
+        gs = ops.Grad.from_host([np.ascontiguousarray(p[sl]) for p in g4])
+        xs = ops.CMat.from_host(np.ascontiguousarray(xr[sl]), np.ascontiguousarray(xi[sl]))
+        ops.linear_bwd_weight(gs, xs, acc, accumulate=k)
+    full, parts = dw.host(), acc.host()
+    assert rel_c(full[0:2], parts[0:2]) < 1e-5 and rel_c(full[2:4], parts[2:4]) < 1e-5
