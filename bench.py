@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X: isolated complex Linear, forward + Wirtinger backward.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = y = x W^T, then (dx, dx*) = (g W, g* conj W), then (dW, dW*) = (g^T x, g*^T conj x): 3 launches, 5 complex
+GEMMs, 40*B*N*K real flops (8 per complex multiply-add, the 4-real-GEMM count).  Inputs are synthetic, seeded, and
+resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X published dense fp32 matrix peak
+B, K, N = 4096, 1024, 1024      # BASELINE.json configs[1]
+
+
+class HipEvents:
+    """hipEvent timing on the stream the library launches on."""
+
+    def __init__(self, stream):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.stream = C.c_void_p(stream)
+
+    def event(self):
+        e = C.c_void_p()
+        rc = self.hip.hipEventCreate(C.byref(e))
+        assert rc == 0, rc
+        return e
+
+    def record(self, e):
+        rc = self.hip.hipEventRecord(e, self.stream)
+        assert rc == 0, rc
+
+    def elapsed_ms(self, a, b):
+        rc = self.hip.hipEventSynchronize(b)
+        assert rc == 0, rc
+        ms = C.c_float()
+        rc = self.hip.hipEventElapsedTime(C.byref(ms), a, b)
+        assert rc == 0, rc
+        return float(ms.value)
+
+
+def cpu_baseline(budget_s=15.0):
+    """Upstream CPU path (oracle/_ref, "reference") or the restatement ("port") timed on this host: per-sample
+    forward + backward of the same Linear on a bounded number of batch rows (per-sample cost is constant: the CPU path
+    processes one sample at a time), reported in the metric's unit."""
+    from oracle import binding as ob
+    lib = ob.load_ref() or ob.load_port()
+    port = ob.load_port()
+    net = lib.net()
+    x = net.add(ob.INPUT, K)
+    w = net.add(ob.INPUT, N * K)
+    lin = net.add(ob.LINEAR, K, N * K, inputs=[x, w])
+    sink = net.add(ob.L2OUT, N, inputs=[lin])
+    net.plane(w, ob.RE)[:] = port.normal(3, N * K, 0, K ** -0.5)
+    net.plane(w, ob.IM)[:] = port.normal(4, N * K, 0, K ** -0.5)
+    rows_max = 256
+    xs = port.normal(1, (2, rows_max, K))
+    gs = port.normal(5, (4, rows_max, N))
+
+    def one(r):
+        net.plane(x, ob.RE)[:] = xs[0, r % rows_max]
+        net.plane(x, ob.IM)[:] = xs[1, r % rows_max]
+        net.forward()                    # zero non-input gradients, x and W into the layer, y = x W^T
+        for p in range(4):
+            net.plane(sink, ob.DZ_RE + p)[:] = gs[p, r % rows_max]
+        net.node_backward(lin)           # dx, dx*, dW, dW* of this sample
+        net.node_backward(w)             # parameter node gathers dW* across samples
+        net.node_backward(x)
+
+    one(0)
+    t0 = time.perf_counter()
+    for r in range(4):
+        one(r)
+    per_row = (time.perf_counter() - t0) / 4
+    rows = int(max(16, min(4096, budget_s / per_row)))
+    t0 = time.perf_counter()
+    for r in range(rows):
+        one(r)
+    dt = time.perf_counter() - t0
+    return {"value": round(40.0 * rows * N * K / dt / 1e12, 5), "unit": "TFLOP/s", "cores": lib.threads,
+            "kind": lib.backend,
+            "sample": "%d of %d batch rows, per-sample forward+backward as the upstream CPU loop, %.1f s, "
+                      "%.2f ms/row (%.1f samples/s)" % (rows, B, dt, 1e3 * dt / rows, rows / dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (one process, one device, no collectives); --gpus %d is not "
+                 "supported. Run with --gpus 1." % args.gpus)
+
+    from cnet_amd import capi, ops
+    capi.init(0)
+    info = capi.device_info()
+    ev = HipEvents(capi.load().cnet_stream())
+    try:
+        import torch
+        tsync = torch.cuda.synchronize if torch.cuda.is_available() else (lambda: None)
+    except Exception:  # torch is only used for the contract's device-wide synchronize
+        tsync = lambda: None
+
+    from oracle import binding as ob   # seeded generator only (identical arrays for every backend)
+    gen = ob.load_port()
+    x = ops.CMat.from_host(gen.normal(1, (B, K)), gen.normal(2, (B, K)))
+    w = ops.CMat.from_host(gen.normal(3, (N, K), 0, K ** -0.5), gen.normal(4, (N, K), 0, K ** -0.5))
+    g = ops.Grad.from_host([gen.normal(5 + p, (B, N)) for p in range(4)])
+    y, dx, dw = ops.CMat.empty(B, N), ops.Grad.empty(B, K), ops.Grad.empty(N, K)
+
+    launches = {
+        "linear_fwd": (lambda: ops.linear_fwd(x, w, y), 1),
+        "linear_bwd_input": (lambda: ops.linear_bwd_input(g, w, dx), 2),
+        "linear_bwd_weight": (lambda: ops.linear_bwd_weight(g, x, dw), 2),
+    }
+
+    def step():
+        for fn, _ in launches.values():
+            fn()
+
+    for _ in range(args.warmup):
+        step()
+    capi.sync(); tsync()
+    e0, e1 = ev.event(), ev.event()
+    t0 = time.perf_counter()
+    ev.record(e0)
+    for _ in range(args.steps):
+        step()
+    ev.record(e1)
+    capi.sync(); tsync()
+    wall = time.perf_counter() - t0
+    gpu_ms = ev.elapsed_ms(e0, e1)
+    ms_per_step = 1e3 * wall / args.steps
+    flops_step = 40.0 * B * N * K
+    tflops = flops_step / (wall / args.steps) / 1e12
+
+    # per-launch durations (HIP events around back-to-back launches of one kernel on the library's stream)
+    kern = {}
+    for name, (fn, ngemm) in launches.items():
+        a, b = ev.event(), ev.event()
+        fn(); capi.sync()
+        ev.record(a)
+        for _ in range(args.steps):
+            fn()
+        ev.record(b)
+        ms = ev.elapsed_ms(a, b) / args.steps
+        fl = 8.0 * B * N * K * ngemm
+        kern[name] = {"ms": round(ms, 4), "flops": fl, "tflops": round(fl / ms / 1e9, 2)}
+    dom = max(kern, key=lambda k: kern[k]["ms"])
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "cgemm_traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(dom)
+    roofline = {"bound": "mfma", "kernel": "cgemm_kernel (%s)" % dom, "achieved": kern[dom]["tflops"],
+                "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(kern[dom]["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": traffic,
+                "flops_per_launch": kern[dom]["flops"], "avg_launch_ms": kern[dom]["ms"],
+                "all_launches": kern, "device_clock_khz": info.clock_khz, "compute_units": info.compute_units}
+
+    out = {
+        "metric": "complex-Linear fwd+bwd TFLOP/s (% fp32 MFMA peak); train samples/sec",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: isolated complex Linear fwd + Wirtinger bwd (dx, dx*, dW, dW*), "
+                               "complex64 split-plane", "batch": B, "in": K, "out": N,
+                   "flops_per_step": flops_step, "launches_per_step": 3},
+        "pct_fp32_mfma_peak": round(100 * tflops / PEAK_FP32_MFMA_TFLOPS, 2),
+        "samples_per_sec": round(B / (wall / args.steps), 1),
+        "gpu_ms_per_step_events": round(gpu_ms / args.steps, 4),
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -19,6 +19,9 @@ LIB = os.path.join(HERE, "lib", "libcnet_hip.so")
 SOURCES = ["runtime.hip", "cgemm.hip", "cdft.hip", "elementwise.hip", "reduce.hip", "embedding.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+         # no fused multiply-add contraction: the elementwise kernels then round like the CPU path
+         # (mul, then add), e.g. the SGD step is bit-identical to it; the GEMMs use MFMA either way
+         "-ffp-contract=off",
          # packed-fp32 VALU forms are kept out of every kernel
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-result", "-Wno-unused-value", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
