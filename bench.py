@@ -99,6 +99,9 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--counter-pass", action="store_true",
+                    help="short run for `rocprofv3 --pmc`: 3 launches of each GEMM kernel plus a plain copy kernel of "
+                         "known size (256 MiB read, 256 MiB written) that calibrates FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (one process, one device, no collectives); --gpus %d is not "
@@ -130,6 +133,16 @@ def main():
     def step():
         for fn, _ in launches.values():
             fn()
+
+    if args.counter_pass:
+        rows, cols = 8192, 8192   # 256 MiB per plane
+        src, dst = ops.Plane.empty(rows, cols, zero=True), ops.Plane.empty(rows, cols, zero=True)
+        for _ in range(3):
+            ops.copy2d(src, dst)
+            step()
+        capi.sync()
+        print(json.dumps({"counter_pass": True, "copy_bytes_read": rows * cols * 4, "copy_bytes_written": rows * cols * 4}))
+        return
 
     for _ in range(args.warmup):
         step()

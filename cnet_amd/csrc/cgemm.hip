@@ -23,6 +23,9 @@
 //   each XCD works on a contiguous strip of C blocks and re-uses operand tiles through its own L2.
 #include "common.hpp"
 
+#include <cstdlib>
+#include <type_traits>
+
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -285,12 +288,252 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 		}
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// Fast path: M % BM == 0, N % BN == 0, K % KC == 0, 128-bit aligned operands.  Same decomposition as cgemm_kernel,
+// with the per-chunk overhead taken out of the vector ALU:
+//   * global addresses are "uniform tile base (SGPR, advanced with scalar adds) + per-thread 32-bit offset that never
+//     changes", so a chunk costs no address arithmetic in VGPRs and needs no edge masks;
+//   * LDS addresses are "per-thread base + stage toggle (one add per chunk) + immediate";
+//   * the LDS writes of the next chunk are spread over the second half of the current chunk's MFMAs and the scheduler
+//     is told to interleave them (one MFMA, then a few VALU / DS instructions) so they issue in the shadow of the
+//     matrix pipe instead of stalling it.
+template <int ROWS, bool MCONTIG>
+struct FastStage {
+	static constexpr int UNITS = ROWS * KC / 4 / NTHREADS;
+	unsigned goff[UNITS];  // byte offset of this thread's float4 inside the operand tile of a chunk
+	int soff[UNITS];       // float offset of its LDS destination inside a plane
+	float4 re[UNITS], im[UNITS];
+
+	__device__ __forceinline__ void init(long ld, int pitch) {
+#pragma unroll
+		for (int u = 0; u < UNITS; ++u) {
+			const int unit = threadIdx.x + u * NTHREADS;
+			int row, k;
+			if (MCONTIG) {
+				k = unit / (ROWS / 4);
+				row = (unit % (ROWS / 4)) * 4;
+				goff[u] = (unsigned) (((long) k * ld + row) * 4);
+			} else {
+				row = unit / (KC / 4);
+				k = (unit % (KC / 4)) * 4;
+				goff[u] = (unsigned) (((long) row * ld + k) * 4);
+			}
+			soff[u] = k * pitch + row;
+		}
+	}
+	// tile_re / tile_im: uniform pointers to element (first row of the block, first k of the chunk)
+	__device__ __forceinline__ void load_unit(int u, const float *tile_re, const float *tile_im) {
+		re[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(tile_re) + goff[u]);
+		im[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(tile_im) + goff[u]);
+	}
+	template <int PITCH>
+	__device__ __forceinline__ void store_unit(int u, float *sre, float *sim, float im_sign) const {
+		const float4 a = re[u];
+		const float4 b = make_float4(im[u].x * im_sign, im[u].y * im_sign, im[u].z * im_sign, im[u].w * im_sign);
+		if (MCONTIG) {
+			*reinterpret_cast<float4 *>(sre + soff[u]) = a;
+			*reinterpret_cast<float4 *>(sim + soff[u]) = b;
+		} else {
+			sre[soff[u] + 0 * PITCH] = a.x;
+			sre[soff[u] + 1 * PITCH] = a.y;
+			sre[soff[u] + 2 * PITCH] = a.z;
+			sre[soff[u] + 3 * PITCH] = a.w;
+			sim[soff[u] + 0 * PITCH] = b.x;
+			sim[soff[u] + 1 * PITCH] = b.y;
+			sim[soff[u] + 2 * PITCH] = b.z;
+			sim[soff[u] + 3 * PITCH] = b.w;
+		}
+	}
+};
+
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG>
+__global__ __launch_bounds__(NTHREADS, 2) void cgemm_fast_kernel(const CgemmArgs args) {
+	static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per workgroup");
+	constexpr int TM = WM / 32, TN = WN / 32;
+	constexpr int PA = BM + 4, PB = BN + 4;
+	constexpr int A_PLANE = KC * PA, B_PLANE = KC * PB;
+	constexpr int STAGE_FLOATS = 2 * A_PLANE + 2 * B_PLANE;
+	constexpr int KS = KC / 2;  // k pairs (MFMA k extent = 2) per chunk
+#ifndef CNET_SCHED_RECIPE
+#define CNET_SCHED_RECIPE 1
+#endif
+	constexpr bool SCHED_RECIPE = CNET_SCHED_RECIPE;
+	extern __shared__ float smem[];
+
+	const CgemmProblem pb = args.p[blockIdx.y];
+	const int K = args.K;
+
+	int pid = blockIdx.x;
+	const int total = args.tiles_m * args.tiles_n;
+	if (total % NUM_XCD == 0) pid = (pid % NUM_XCD) * (total / NUM_XCD) + pid / NUM_XCD;
+	constexpr int GROUP = 8;
+	const int width = GROUP * args.tiles_n;
+	const int first_m = (pid / width) * GROUP;
+	const int gsize = min(args.tiles_m - first_m, GROUP);
+	const int tile_m = first_m + (pid % width) % gsize;
+	const int tile_n = (pid % width) / gsize;
+	const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int wm0 = (wave / (BN / WN)) * WM;
+	const int wn0 = (wave % (BN / WN)) * WN;
+	const int r = lane & 31, h = lane >> 5;
+
+	floatx16 acc_re[TM][TN], acc_im[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+#pragma unroll
+			for (int e = 0; e < 16; ++e) {
+				acc_re[i][j][e] = 0.f;
+				acc_im[i][j][e] = 0.f;
+			}
+
+	FastStage<BM, A_MCONTIG> sa;
+	FastStage<BN, B_NCONTIG> sb;
+	sa.init(args.lda, PA);
+	sb.init(args.ldb, PB);
+	constexpr int UA = FastStage<BM, A_MCONTIG>::UNITS, UB = FastStage<BN, B_NCONTIG>::UNITS, NU = UA + UB;
+
+	// uniform tile bases of chunk 0 and the per-chunk advance (elements)
+	const long a_tile0 = A_MCONTIG ? (long) m0 : (long) m0 * args.lda;
+	const long b_tile0 = B_NCONTIG ? (long) n0 : (long) n0 * args.ldb;
+	const long a_step = A_MCONTIG ? (long) KC * args.lda : (long) KC;
+	const long b_step = B_NCONTIG ? (long) KC * args.ldb : (long) KC;
+	const int nchunks = K / KC;
+
+	auto load_unit = [&](int idx, int chunk) {
+		if (idx < UA)
+			sa.load_unit(idx, pb.a_re + a_tile0 + chunk * a_step, pb.a_im + a_tile0 + chunk * a_step);
+		else
+			sb.load_unit(idx - UA, pb.b_re + b_tile0 + chunk * b_step, pb.b_im + b_tile0 + chunk * b_step);
+	};
+	auto store_unit = [&](int idx, float *stage) {
+		if (idx < UA)
+			sa.template store_unit<PA>(idx, stage, stage + A_PLANE, 1.0f);
+		else
+			sb.template store_unit<PB>(idx - UA, stage + 2 * A_PLANE, stage + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
+	};
+
+#pragma unroll
+	for (int u = 0; u < NU; ++u) load_unit(u, 0);
+#pragma unroll
+	for (int u = 0; u < NU; ++u) store_unit(u, smem);
+	__syncthreads();
+
+	float are[2][TM], aim[2][TM], anim[2][TM], bre[2][TN], bim[2][TN];
+	const float *frag_a = smem + wm0 + r + h * PA;                  // + stage + plane + k pair * 2 * PA + tile * 32
+	const float *frag_b = smem + 2 * A_PLANE + wn0 + r + h * PB;
+	auto fetch = [&](int stage_off, int ks, int slot) {
+		const float *fa = frag_a + stage_off, *fb = frag_b + stage_off;  // one add each; the rest are immediates
+#pragma unroll
+		for (int i = 0; i < TM; ++i) {
+			are[slot][i] = fa[ks * 2 * PA + i * 32];
+			aim[slot][i] = fa[A_PLANE + ks * 2 * PA + i * 32];
+		}
+#pragma unroll
+		for (int j = 0; j < TN; ++j) {
+			bre[slot][j] = fb[ks * 2 * PB + j * 32];
+			bim[slot][j] = fb[B_PLANE + ks * 2 * PB + j * 32];
+		}
+	};
+	fetch(0, 0, 0);
+
+	for (int c = 0; c < nchunks; ++c) {
+		const int CUR = (c & 1) * STAGE_FLOATS, NXT = STAGE_FLOATS - CUR;
+		const bool more = (c + 1 < nchunks);
+		const int next_chunk = more ? c + 1 : 0;  // the last chunk re-reads chunk 0 (in bounds, never used)
+#pragma unroll
+		for (int u = 0; u < NU; ++u) load_unit(u, next_chunk);
+#pragma unroll
+		for (int ks = 0; ks < KS; ++ks) {
+			const int cs = ks & 1;
+			if (ks + 1 < KS) fetch(CUR, ks + 1, cs ^ 1);
+			// the LDS writes of the next chunk ride on the MFMAs of the second half of this chunk
+			if (ks >= KS / 2) {
+#pragma unroll
+				for (int u = 0; u < NU; ++u)
+					if (KS / 2 + (u * (KS / 2)) / NU == ks) store_unit(u, smem + NXT);
+			}
+			if (ks == KS - 1) {
+				__syncthreads();
+				fetch(NXT, 0, cs ^ 1);
+			}
+#pragma unroll
+			for (int i = 0; i < TM; ++i) anim[cs][i] = -aim[cs][i];
+#pragma unroll
+			for (int i = 0; i < TM; ++i)
+#pragma unroll
+				for (int j = 0; j < TN; ++j) {
+					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[cs][i], bre[cs][j], acc_re[i][j], 0, 0, 0);
+					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[cs][i], bim[cs][j], acc_im[i][j], 0, 0, 0);
+				}
+#pragma unroll
+			for (int i = 0; i < TM; ++i)
+#pragma unroll
+				for (int j = 0; j < TN; ++j) {
+					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(anim[cs][i], bim[cs][j], acc_re[i][j], 0, 0, 0);
+					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aim[cs][i], bre[cs][j], acc_im[i][j], 0, 0, 0);
+				}
+			if (SCHED_RECIPE && ks < KS - 1) {
+				// scheduling recipe for this k pair: after each MFMA let a few of the pending VALU / LDS / global
+				// instructions issue, so they run in the shadow of the matrix pipe
+#pragma unroll
+				for (int q = 0; q < 4 * TM * TN; ++q) {
+					__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+					__builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // <= 2 VALU
+					__builtin_amdgcn_sched_group_barrier(0x080, 1, 0);  // <= 1 LDS
+					__builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // <= 1 global load
+				}
+			}
+			__builtin_amdgcn_sched_barrier(0);
+		}
+	}
+
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+#pragma unroll
+		for (int j = 0; j < TN; ++j) {
+			const int col = n0 + wn0 + j * 32 + r;
+#pragma unroll
+			for (int e = 0; e < 16; ++e) {
+				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
+				const long off = (long) row * args.ldc + col;
+				float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
+				if (args.accumulate) {
+					vr += pb.c_re[off];
+					vi += pb.c_im[off];
+				}
+				pb.c_re[off] = vr;
+				pb.c_im[off] = vi;
+			}
+		}
+}
+
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
 int launch(const CgemmArgs &proto, int nprob) {
 	CgemmArgs args = proto;
 	args.tiles_m = (args.M + BM - 1) / BM;
 	args.tiles_n = (args.N + BN - 1) / BN;
 	constexpr size_t smem = 2 * (size_t) (2 * KC * (BM + 4) + 2 * KC * (BN + 4)) * sizeof(float);
+	dim3 grid(args.tiles_m * args.tiles_n, nprob);
+	if constexpr (VEC == 4) {
+		if (args.M % BM == 0 && args.N % BN == 0 && args.K % KC == 0) {
+			auto fast = cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG>;
+			static bool fast_attr_set = false;
+			if (!fast_attr_set) {
+				CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fast), hipFuncAttributeMaxDynamicSharedMemorySize,
+						(int) smem));
+				fast_attr_set = true;
+			}
+			hipLaunchKernelGGL(fast, grid, dim3(NTHREADS), smem, cnet::rt().stream, args);
+			CNET_LAUNCH_CHECK();
+			return CNET_OK;
+		}
+	}
 	auto kern = cgemm_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, VEC>;
 	static bool attr_set = false;  // per instantiation
 	if (!attr_set) {
@@ -298,7 +541,6 @@ int launch(const CgemmArgs &proto, int nprob) {
 				(int) smem));
 		attr_set = true;
 	}
-	dim3 grid(args.tiles_m * args.tiles_n, nprob);
 	hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, cnet::rt().stream, args);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
@@ -312,15 +554,23 @@ int pick_tile(const CgemmArgs &a, int nprob) {
 	if constexpr (VEC == 1) {
 		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
 	} else {
-		// the largest block that still gives every compute unit a workgroup
-		if (blocks(128, 128) >= cus) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
-		if (a.N >= a.M) {
-			if (blocks(64, 128) >= cus) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
-		} else {
-			if (blocks(128, 64) >= cus) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		// tuning override: CNET_CGEMM_TILE = 0 (128x128), 1 (64x128), 2 (128x64), 3 (64x64)
+		static const int forced = [] {
+			const char *e = getenv("CNET_CGEMM_TILE");
+			return e ? atoi(e) : -1;
+		}();
+		if (forced == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		if (forced == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		if (forced == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		if (forced == 3) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		// The largest block that still gives every compute unit TWO workgroups (two wavefronts per SIMD: one issues
+		// MFMAs while the other waits at its barrier or moves data); failing that, one workgroup per compute unit.
+		for (long want = 2 * cus; want >= cus; want -= cus) {
+			if (blocks(128, 128) >= want) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+			if (blocks(64, 128) >= want) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+			if (blocks(128, 64) >= want) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+			if (blocks(64, 64) >= want) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
 		}
-		if (blocks(64, 128) >= cus) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
-		if (blocks(128, 64) >= cus) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
 		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
 	}
 }
