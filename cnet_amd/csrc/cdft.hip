@@ -5,6 +5,7 @@
 #include "common.hpp"
 
 #include <map>
+#include <vector>
 
 namespace cnet {
 
@@ -16,11 +17,18 @@ struct Twiddle {
 	float *re = nullptr;
 	float *im = nullptr;
 	long ld = 0;
+	// optional caller-supplied forward operator, stored transposed ([q][p]) so that y = x * B; the backward pass
+	// always uses the exact twiddles above, as the CPU path does (impl/ft.h:57-79 upstream)
+	float *fwd_re = nullptr;
+	float *fwd_im = nullptr;
 };
 static std::map<int, Twiddle> g_twiddles;
 
 void release_twiddles() {
-	for (auto &kv : g_twiddles) hipFree(kv.second.re);  // one allocation holds both planes
+	for (auto &kv : g_twiddles) {
+		(void) hipFree(kv.second.re);  // one allocation holds both planes
+		if (kv.second.fwd_re) (void) hipFree(kv.second.fwd_re);
+	}
 	g_twiddles.clear();
 }
 
@@ -81,6 +89,36 @@ int cnet_cdft_twiddle(int n, const float **f_re, const float **f_im) {
 	return CNET_OK;
 }
 
+int cnet_cdft_set_forward_matrix(int n, const float *host_f_re, const float *host_f_im) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(n > 0 && n <= 46340);
+	Twiddle t;
+	int rc = get_plan(n, &t, true);
+	if (rc) return rc;
+	Twiddle &slot = g_twiddles[n];
+	if (!host_f_re && !host_f_im) {  // back to the exact transform
+		if (slot.fwd_re) {
+			CNET_HIP(hipStreamSynchronize(rt().stream));
+			CNET_HIP(hipFree(slot.fwd_re));
+		}
+		slot.fwd_re = slot.fwd_im = nullptr;
+		return CNET_OK;
+	}
+	CNET_CHECK_ARG(host_f_re && host_f_im);
+	const size_t plane = (size_t) n * t.ld;
+	std::vector<float> tr(2 * plane, 0.0f);
+	for (int p = 0; p < n; ++p)
+		for (int q = 0; q < n; ++q) {
+			tr[(size_t) q * t.ld + p] = host_f_re[(size_t) p * n + q];
+			tr[plane + (size_t) q * t.ld + p] = host_f_im[(size_t) p * n + q];
+		}
+	if (!slot.fwd_re) CNET_HIP(hipMalloc((void **) &slot.fwd_re, 2 * plane * sizeof(float)));
+	slot.fwd_im = slot.fwd_re + plane;
+	CNET_HIP(hipMemcpyAsync(slot.fwd_re, tr.data(), 2 * plane * sizeof(float), hipMemcpyHostToDevice, rt().stream));
+	CNET_HIP(hipStreamSynchronize(rt().stream));
+	return CNET_OK;
+}
+
 int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy, int B, int n,
 		int accumulate) {
 	CNET_REQUIRE_INIT();
@@ -90,7 +128,8 @@ int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re
 	Twiddle t;
 	int rc = get_plan(n, &t, true);
 	if (rc) return rc;
-	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {t.re, t.re}, *bi[2] = {t.im, t.im};
+	const float *f_re = t.fwd_re ? t.fwd_re : t.re, *f_im = t.fwd_re ? t.fwd_im : t.im;
+	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {f_re, f_re}, *bi[2] = {f_im, f_im};
 	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
 	bool cj[2] = {false, false};
 	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate);

@@ -1,0 +1,1105 @@
+// Host-side mirror of CNet's public C++ API over the MI355X device library (include/cnet_hip.h).
+//
+// Same class names, constructor arguments, method names and error behaviour as upstream CNet for the dense complex
+// path (upstream gpu/gpu_func.h:41-1113, impl/cfunc.h, impl/cnet.h, impl/vars.h, impl/batch.h and the layer
+// headers), so a program written against upstream -- net.add(new Linear(...), {x, w}); allocateOnGpu(B);
+// gpuForward(inp, out, batch); getLoss(...); gpuBackward(); gpuUpdateInputs(lr / B) -- compiles against this header.
+// What is underneath is different by design:
+//   * no per-sample graph clones: one node = one set of batched device planes [rows x len]; parameter nodes
+//     (every CInput that is not the data input, and the embedding table) are stored ONCE (rows = 1);
+//   * a producer owns its output planes and each consumer reads them in place (no copies into consumer blocks; fan-out
+//     costs nothing); every consumer slot owns its four gradient planes;
+//   * every layer step is a call into the C ABI (batched GEMMs / fused elementwise / wavefront reductions) queued on
+//     one stream; nothing synchronises until a result is read back.
+// There is NO CPU execution path here: forward()/backward()/updateInputs() of the per-sample API also run on the
+// device (batch of one), and every method fails loudly (std::runtime_error) when the device layer reports an error.
+//
+// Host views: net[uid]->input() is the per-sample six-plane block of upstream (impl/vars.h:40-46).  The batched calls
+// leave results on the device; CNet::fetch(node, batch_index) fills a node's host view for one sample
+// (upstream: testDataFromGpu / printMappingFromGpu copy a mapping back, gpu/gpu_func.h:700-862).
+#ifndef CNET_AMD_HOST_CNET_HPP_
+#define CNET_AMD_HOST_CNET_HPP_
+
+#include <algorithm>
+#include <cassert>
+#include <cmath>
+#include <complex>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <ctime>
+#include <initializer_list>
+#include <iostream>
+#include <map>
+#include <memory>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "cnet_hip.h"
+
+// ---------------------------------------------------------------------------------------------------------------
+// impl/sizes.h
+// ---------------------------------------------------------------------------------------------------------------
+class Size {
+	int value_;
+public:
+	Size(int value) : value_(value) {}
+	unsigned int value() { return value_; }
+};
+class InSize {
+	unsigned int value_;
+public:
+	InSize(int value) : value_(value) {}
+	unsigned int value() { return value_; }
+};
+class OutSize {
+	unsigned int value_;
+public:
+	OutSize(int value) : value_(value) {}
+	unsigned int value() { return value_; }
+};
+class Uid {
+	int value_;
+public:
+	Uid(int value) : value_(value) {}
+	int value() { return value_; }
+};
+
+// ---------------------------------------------------------------------------------------------------------------
+// utils/myrand.h: xorshift64* and the polar normal, for reproducible parameter initialisation
+// ---------------------------------------------------------------------------------------------------------------
+class SimpleRand {
+	uint64_t state_;
+	double lastVal_;
+public:
+	SimpleRand(uint64_t seed = 88172645463325252ULL) : state_(0x2545F4914F6CDD1DULL ^ seed), lastVal_(0.0) {}
+	uint64_t randUint64() {
+		uint64_t x = state_;
+		x ^= x >> 12;
+		x ^= x << 25;
+		x ^= x >> 27;
+		state_ = x;
+		return x * 0x2545F4914F6CDD1DULL;
+	}
+	double randDouble() { return 5.42101086242752217E-20 * randUint64(); }
+	double normal(double mu, double sig) {
+		if (lastVal_ == 0.) {
+			double v1, v2, rsq;
+			do {
+				v1 = 2.0 * randDouble() - 1.0;
+				v2 = 2.0 * randDouble() - 1.0;
+				rsq = v1 * v1 + v2 * v2;
+			} while (rsq >= 1.0 || rsq == 0.0);
+			double fac = sqrt(-2.0 * log(rsq) / rsq);
+			lastVal_ = v1 * fac;
+			return mu + sig * v2 * fac;
+		}
+		double fac = lastVal_;
+		lastVal_ = 0.;
+		return mu + sig * fac;
+	}
+};
+
+// ---------------------------------------------------------------------------------------------------------------
+// impl/vars.h: six contiguous planes on the host (the per-sample view)
+// ---------------------------------------------------------------------------------------------------------------
+class Vars {
+public:
+	int length_ = 0;
+	float *real_ = NULL, *imag_ = NULL, *dz_real_ = NULL, *dz_imag_ = NULL, *dz_star_real_ = NULL, *dz_star_imag_ = NULL;
+
+	Vars() {}
+	explicit Vars(int length) : length_(length) {
+		assert(length > 0);
+		real_ = new float[(size_t) length_ * 6];
+		bind();
+		std::fill(real_, real_ + (size_t) length_ * 6, 0.0f);
+	}
+	Vars(const Vars &o) : length_(o.length_) {
+		if (!o.real_) return;
+		real_ = new float[(size_t) length_ * 6];
+		bind();
+		std::copy(o.real_, o.real_ + (size_t) length_ * 6, real_);
+	}
+	Vars &operator=(const Vars &) = delete;
+	virtual ~Vars() { delete[] real_; }
+
+	void zero_gradients() { std::fill(dz_real_, dz_real_ + (size_t) length_ * 4, 0.0f); }
+	void zero_input() { std::fill(real_, real_ + (size_t) length_ * 2, 0.0f); }
+	std::complex<float> z(int i) const { return std::complex<float>(real_[i], imag_[i]); }
+	std::complex<float> dz(int i) const { return std::complex<float>(dz_real_[i], dz_imag_[i]); }
+	std::complex<float> dz_star(int i) const { return std::complex<float>(dz_star_real_[i], dz_star_imag_[i]); }
+	void zSetValue(int i, std::complex<float> v) { real_[i] = v.real(); imag_[i] = v.imag(); }
+	unsigned long long size_in_bytes() const { return 6ULL * length_ * sizeof(float); }
+	float *plane(int p) { return real_ + (size_t) p * length_; }
+private:
+	void bind() {
+		imag_ = real_ + length_;
+		dz_real_ = imag_ + length_;
+		dz_imag_ = dz_real_ + length_;
+		dz_star_real_ = dz_imag_ + length_;
+		dz_star_imag_ = dz_star_real_ + length_;
+	}
+};
+
+// ---------------------------------------------------------------------------------------------------------------
+// impl/batch.h
+// ---------------------------------------------------------------------------------------------------------------
+const int NO_TOKEN = -1;
+
+class Batch {
+	friend class CNet;
+protected:
+	std::vector<float> losses_;
+	std::vector<int> labels_;
+	std::vector<int> sizes_;
+	int current_pos_ = 0, batch_size_ = 0, sample_dim_ = 0;
+	void addLoss(float loss) { losses_.push_back(loss); }
+public:
+	Batch() {}
+	Batch(int batch_size, int sample_dim) : batch_size_(batch_size), sample_dim_(sample_dim) {}
+	virtual ~Batch() {}
+	int size() { return batch_size_; }
+	int sampleDim() { return sample_dim_; }
+	float loss(int i) { return losses_[i]; }
+	int noOfLabels() const { return (int) labels_.size(); }
+	const int *labelsPtr() const { return &labels_[0]; }
+	int label(int i) { return labels_[i]; }
+};
+
+class InputBatch : public Batch {
+	std::vector<float> real_data_, imag_data_;
+public:
+	InputBatch() : Batch() {}
+	InputBatch(int batch_size, int sample_dim) : Batch(batch_size, sample_dim) {}
+	void add(const std::vector<std::complex<float> > &sample, int label) {
+		assert(current_pos_ < batch_size_);
+		for (auto c : sample) {
+			real_data_.push_back(c.real());
+			imag_data_.push_back(c.imag());
+		}
+		while (real_data_.size() < (size_t) (1 + current_pos_) * sample_dim_) {  // padding with 0s
+			real_data_.push_back(0.f);
+			imag_data_.push_back(0.f);
+		}
+		labels_.push_back(label);
+		sizes_.push_back((int) sample.size());
+		current_pos_++;
+	}
+	void add(std::initializer_list<std::complex<float> > list, int label) {
+		add(std::vector<std::complex<float> >(list), label);
+	}
+	// bulk variant for callers that already hold the two planes of one sample
+	void add(const float *re, const float *im, int n, int label) {
+		assert(current_pos_ < batch_size_ && n <= sample_dim_);
+		real_data_.insert(real_data_.end(), re, re + n);
+		imag_data_.insert(imag_data_.end(), im, im + n);
+		real_data_.resize((size_t) (1 + current_pos_) * sample_dim_, 0.f);
+		imag_data_.resize((size_t) (1 + current_pos_) * sample_dim_, 0.f);
+		labels_.push_back(label);
+		sizes_.push_back(n);
+		current_pos_++;
+	}
+	const float *realDataPtr() const { return &real_data_[0]; }
+	const float *imagDataPtr() const { return &imag_data_[0]; }
+	const float *realDataPtr(int b) const { return &real_data_[0] + (size_t) b * sample_dim_; }
+	const float *imagDataPtr(int b) const { return &imag_data_[0] + (size_t) b * sample_dim_; }
+};
+
+class EmbeddingBatch : public Batch {
+	friend class CNet;
+	std::vector<int> token_;
+	int counter_ = 0;
+public:
+	EmbeddingBatch() : Batch() {}
+	EmbeddingBatch(int batch_size, int sample_dim) : Batch(batch_size, sample_dim) {}
+	void add(const std::vector<int> &sample, int label) {
+		assert(current_pos_ < batch_size_);
+		token_.insert(token_.end(), sample.begin(), sample.end());
+		while (token_.size() < (size_t) (1 + current_pos_) * sample_dim_) token_.push_back(NO_TOKEN);  // padding with -1s
+		labels_.push_back(label);
+		sizes_.push_back((int) sample.size());
+		current_pos_++;
+		counter_ += (int) sample.size();
+	}
+	int noOfTokens() const { return (int) token_.size(); }
+	const int *tokensPtr() const { return &token_[0]; }
+	int tokenCount() { return counter_; }
+};
+
+// ---------------------------------------------------------------------------------------------------------------
+// impl/cfunc.h: graph node.  The layer arithmetic lives in the device library; a node here carries the wiring, the
+// per-sample host view and its device planes.
+// ---------------------------------------------------------------------------------------------------------------
+class OutputFunc {
+	bool isMainOutput_ = false;
+public:
+	virtual ~OutputFunc() {}
+	virtual int outputLength() = 0;
+	virtual float loss(int label) = 0;
+	virtual Vars *mutableOutput() = 0;
+	bool isMainOutput() { return isMainOutput_; }
+	void setIsMainOutput(bool v) { isMainOutput_ = v; }
+};
+
+class InputFunc {
+	bool isMainInput_ = false;
+public:
+	virtual ~InputFunc() {}
+	bool isMainInput() { return isMainInput_; }
+	void setIsMainInput(bool v) { isMainInput_ = v; }
+};
+
+// node type ids of impl/cnet.h:31-44
+const int isHadamard = 1, isEmbedding = 2, isLinear = 3, isFourier = 4, isCrossEntropy = 5, isResidual = 6, isSoftMax = 7,
+		isInput = 8, isCrelu = 9, isGelu = 10, isL2Out = 11, isTrianFourier = 12;
+
+class CFunc {
+	friend class CNet;
+	Vars input_;
+protected:
+	int uid_ = 0;
+	int out_size_;
+	std::vector<CFunc *> prev_func_, next_func_;  // not owned
+	std::vector<int> offset_;
+	int depth_ = 0;
+	bool is_input_ = false, is_output_ = false;
+	int type_ = 0;
+	SimpleRand rand_;
+
+	// ---- device side (owned by CNet's plan) ----
+	struct Slot {            // one producer feeding this node
+		CFunc *producer = NULL;
+		int offset = 0, len = 0, rows = 0;
+		float *grad = NULL;  // 4 planes [rows][len]
+		float *g(int plane) const { return grad + (size_t) plane * rows * len; }
+	};
+	std::vector<Slot> slots_;
+	int rows_ = 0;           // batch rows of this node's output (1 for parameter nodes)
+	float *out_ = NULL;      // 2 planes [rows][out_size]: what consumers read
+	float *out_re() const { return out_; }
+	float *out_im() const { return out_ + (size_t) rows_ * out_size_; }
+
+public:
+	CFunc(Uid uid, InSize in_size, OutSize out_size) : input_(in_size.value()), uid_(uid.value()), out_size_(out_size.value()) {}
+	CFunc(InSize in_size, OutSize out_size) : input_(in_size.value()), out_size_(out_size.value()) {}
+	virtual ~CFunc() {}
+	void setRandSeed(uint64_t seed) { rand_ = SimpleRand(seed); }
+	bool isInput() { return is_input_; }
+	bool isOutput() { return is_output_; }
+	int getType() const { return type_; }
+	int outSize() { return out_size_; }
+	const Vars &input() const { return input_; }
+	Vars *mutable_input() { return &input_; }
+	const Vars &output() { assert(next_func_.size()); return next_func_[0]->input(); }
+	const Vars &output(int i) { return next_func_[i]->input(); }
+	int uid() { return uid_; }
+	int depth() { return depth_; }
+	CFunc *next(int i) const { return next_func_[i]; }
+	int offset(int i) { return offset_[i]; }
+	int no_outputs() const { return (int) next_func_.size(); }
+	int no_previous_func() const { return (int) prev_func_.size(); }
+	CFunc *previous(int i) { return prev_func_[i]; }
+	virtual int sizeInBytes() const { return (int) input_.size_in_bytes(); }
+	virtual std::string getName() = 0;
+	virtual int typeId() const = 0;
+
+	// impl/cfunc.h:195-201
+	virtual void init_inputs() {
+		for (int i = 0; i < input_.length_; ++i) {
+			float re = (float) rand_.randDouble() - 0.5;
+			input_.real_[i] = re / input_.length_;
+			input_.imag_[i] = sqrt(1 - re * re) / input_.length_;
+		}
+	}
+	// impl/cfunc.h:211-224
+	void addOutput(CFunc *next, int offset) {
+		assert(next && offset >= 0);
+		if (next->input().length_ < offset + out_size_)
+			throw std::invalid_argument("add: " + next->getName() + " input is shorter than offset + output of " + getName());
+		next_func_.push_back(next);
+		offset_.push_back(offset);
+		if (next->depth_ <= depth_) next->depth_ = depth_ + 1;
+	}
+};
+
+class CInput : public CFunc, public InputFunc {
+	bool batched_ = false;
+public:
+	// A second per-sample data input (e.g. regression targets).  Upstream's GPU path knows exactly one data input
+	// ("Only one main input supported", impl/cnet.h:541-544); flagging a CInput before allocateOnGpu() gives it batch
+	// rows as well, filled with CNet::gpuSetInput().
+	void setIsBatched(bool v) { batched_ = v; }
+	bool isBatched() const { return batched_; }
+	CInput(Uid uid, OutSize out) : CFunc(uid, InSize(out.value()), out) { is_input_ = true; }
+	CInput(OutSize out) : CFunc(InSize(out.value()), out) { is_input_ = true; }
+	std::string getName() override { return "Input_" + std::to_string(uid_); }
+	int typeId() const override { return ::isInput; }
+	void setInput(InputBatch &batch, int b) {
+		assert(batch.sampleDim() == input().length_);
+		std::copy(batch.realDataPtr(b), batch.realDataPtr(b) + input().length_, mutable_input()->real_);
+		std::copy(batch.imagDataPtr(b), batch.imagDataPtr(b) + input().length_, mutable_input()->imag_);
+	}
+};
+
+class Linear : public CFunc {
+	int in1_len, in2_len;
+public:
+	Linear(Uid uid, InSize in1, InSize in2) : CFunc(uid, InSize(in1.value() + in2.value()), OutSize(in2.value() / in1.value())),
+			in1_len(in1.value()), in2_len(in2.value()) { assert(in2.value() % in1.value() == 0); }
+	Linear(InSize in1, InSize in2) : CFunc(InSize(in1.value() + in2.value()), OutSize(in2.value() / in1.value())),
+			in1_len(in1.value()), in2_len(in2.value()) { assert(in2.value() % in1.value() == 0); }
+	int firstInputLength() { return in1_len; }
+	int secondInputLength() { return in2_len; }
+	std::string getName() override { return "Linear_" + std::to_string(uid_); }
+	int typeId() const override { return isLinear; }
+};
+
+class FourierTrans : public CFunc {
+public:
+	FourierTrans(Uid uid, InSize n) : CFunc(uid, n, OutSize(n.value())) {}
+	FourierTrans(InSize n) : CFunc(n, OutSize(n.value())) {}
+	std::string getName() override { return "FourierTrans_" + std::to_string(uid_); }
+	int typeId() const override { return isFourier; }
+};
+
+class Hadamard : public CFunc {
+public:
+	Hadamard(Uid uid, InSize a, InSize b) : CFunc(uid, InSize(a.value() + b.value()), OutSize(a.value())) { assert(a.value() == b.value()); }
+	Hadamard(InSize a, InSize b) : CFunc(InSize(a.value() + b.value()), OutSize(a.value())) { assert(a.value() == b.value()); }
+	std::string getName() override { return "Hadamard_" + std::to_string(uid_); }
+	int typeId() const override { return isHadamard; }
+};
+
+class CGelu : public CFunc {
+public:
+	CGelu(Uid uid, InSize n) : CFunc(uid, n, OutSize(n.value())) {}
+	CGelu(InSize n) : CFunc(n, OutSize(n.value())) {}
+	std::string getName() override { return "CGelu_" + std::to_string(uid_); }
+	int typeId() const override { return isGelu; }
+};
+
+class Residual : public CFunc {
+public:
+	Residual(Uid uid, InSize n) : CFunc(uid, InSize(2 * n.value()), OutSize(n.value())) {}
+	Residual(Uid uid, InSize a, InSize b) : CFunc(uid, InSize(2 * a.value()), OutSize(a.value())) { assert(a.value() == b.value()); }
+	Residual(InSize n) : CFunc(InSize(2 * n.value()), OutSize(n.value())) {}
+	Residual(InSize a, InSize b) : CFunc(InSize(2 * a.value()), OutSize(a.value())) { assert(a.value() == b.value()); }
+	std::string getName() override { return "Res_" + std::to_string(uid_); }
+	int typeId() const override { return isResidual; }
+};
+
+class SoftMax : public CFunc {
+	friend class CNet;
+	float *d_s_ = NULL;  // device: sum |z|^2 per row
+public:
+	SoftMax(Uid uid, InSize n) : CFunc(uid, n, OutSize(n.value())) {}
+	SoftMax(InSize n) : CFunc(n, OutSize(n.value())) {}
+	std::string getName() override { return "SoftMax_" + std::to_string(uid_); }
+	int typeId() const override { return isSoftMax; }
+};
+
+class CrossEntropy : public CFunc, public OutputFunc {
+	friend class CNet;
+	Vars output_;
+	int prediction_ = 0;                    // argmax of the fetched sample, computed on the device
+	float *d_s_ = NULL, *d_loss_ = NULL;    // device: [rows]
+	int32_t *d_argmax_ = NULL;
+	float *d_norm_ = NULL;                  // device: normalised z, 2 planes [rows][n]
+public:
+	CrossEntropy(Uid uid, InSize n) : CFunc(uid, n, OutSize(1)), output_(n.value()) { is_output_ = true; }
+	CrossEntropy(InSize n) : CFunc(n, OutSize(1)), output_(n.value()) { is_output_ = true; }
+	std::string getName() override { return "CrossEntropy_" + std::to_string(uid_); }
+	int typeId() const override { return isCrossEntropy; }
+	// impl/crossent.h:38-59: accessors over the normalised output of the last fetched sample
+	float getProbability(int label) { return std::pow(output_.real_[label], 2) + std::pow(output_.imag_[label], 2); }
+	float loss(int label) override {
+		assert(label >= 0 && label < input().length_);
+		float v = getProbability(label);
+		v = (v < 1e-15 ? 1e-15 : v);
+		return -std::log(v);
+	}
+	int get_prediction() { return prediction_; }
+	int sizeInBytes() const override { return (int) (input().size_in_bytes() + output_.size_in_bytes()); }
+	int outputLength() override { return output_.length_; }
+	Vars *mutableOutput() override { return &output_; }
+};
+
+class L2Out : public CFunc, public OutputFunc {
+	friend class CNet;
+	Vars output_;
+	float *d_loss_ = NULL;  // device: [rows]
+public:
+	L2Out(Uid uid, InSize n) : CFunc(uid, n, OutSize(1)), output_(1) { is_output_ = true; }
+	L2Out(InSize n) : CFunc(n, OutSize(1)), output_(1) { is_output_ = true; }
+	std::string getName() override { return "L2Out_" + std::to_string(uid_); }
+	int typeId() const override { return isL2Out; }
+	float loss() { return output_.real_[0]; }
+	float loss(int) override { return output_.real_[0]; }
+	int sizeInBytes() const override { return (int) (input().size_in_bytes() + output_.size_in_bytes()); }
+	int outputLength() override { return output_.length_; }
+	Vars *mutableOutput() override { return &output_; }
+};
+
+class CEmbedding : public CFunc, public InputFunc {
+	friend class CNet;
+	int embedding_dim_, no_embeddings_, no_out_tokens_;
+	std::vector<int> tokens_;
+	int32_t *d_tokens_ = NULL;  // device: [rows][no_out_tokens]
+public:
+	CEmbedding(Uid uid, int dim, int max_out_tokens, int no_embeddings)
+			: CFunc(uid, InSize(no_embeddings * dim), OutSize(max_out_tokens * dim)), embedding_dim_(dim),
+			  no_embeddings_(no_embeddings), no_out_tokens_(max_out_tokens) { is_input_ = true; }
+	CEmbedding(int dim, int max_out_tokens, int no_embeddings)
+			: CFunc(InSize(no_embeddings * dim), OutSize(max_out_tokens * dim)), embedding_dim_(dim),
+			  no_embeddings_(no_embeddings), no_out_tokens_(max_out_tokens) { is_input_ = true; }
+	int embeddingDim() { return embedding_dim_; }
+	int noEmbeddings() { return no_embeddings_; }
+	int noOutTokens() { return no_out_tokens_; }
+	std::string getName() override { return "Embedding " + std::to_string(uid_); }
+	int typeId() const override { return isEmbedding; }
+	void setInput(const std::vector<int> &list) {
+		tokens_.clear();
+		for (auto id : list) {
+			assert(id < no_embeddings_);
+			tokens_.push_back(id);
+		}
+		assert(tokens_.size() && (int) tokens_.size() <= no_out_tokens_);
+	}
+	void setInput(std::initializer_list<int> list) { setInput(std::vector<int>(list)); }
+	void init_inputs() override {  // impl/embed.h:101-107
+		for (int i = 0; i < input().length_; ++i) {
+			float re = (float) rand_.randDouble() - 0.5;
+			mutable_input()->real_[i] = re / sqrt(embedding_dim_);
+			mutable_input()->imag_[i] = sqrt(1 - re * re) / sqrt(embedding_dim_);
+		}
+	}
+};
+
+// ---------------------------------------------------------------------------------------------------------------
+// gpu/gpu_func.h: CNet
+// ---------------------------------------------------------------------------------------------------------------
+class CNet {
+	std::vector<CFunc *> func_list_;  // owned
+	std::map<int, CFunc *> map_;
+	std::vector<CFunc *> inputs_, outputs_;
+	int next_uid_ = 0;
+	bool graph_ready_ = false;
+
+	// device plan
+	int batch_ = 0;                   // 0: nothing allocated
+	std::vector<void *> allocations_;
+	CFunc *main_input_ = NULL;
+	int32_t *d_labels_ = NULL;
+	std::vector<int> labels_;
+
+	static void ck(int rc, const char *what) {
+		if (rc != CNET_OK)
+			throw std::runtime_error(std::string(what) + " failed (" + std::to_string(rc) + "): " + cnet_last_error());
+	}
+	template <class T>
+	T *dalloc(size_t count) {
+		void *p = NULL;
+		ck(cnet_alloc(count * sizeof(T), &p), "cnet_alloc");
+		allocations_.push_back(p);
+		return (T *) p;
+	}
+	static bool isParameter(CFunc *f) {  // stored once: every CInput that carries no per-sample data
+		if (f->typeId() != isInput) return false;
+		CInput *c = (CInput *) f;
+		return !c->isMainInput() && !c->isBatched();
+	}
+	CFunc::Slot *slotOf(CFunc *consumer, CFunc *producer, int offset) {
+		for (auto &s : consumer->slots_)
+			if (s.producer == producer && s.offset == offset) return &s;
+		return NULL;
+	}
+
+public:
+	CNet() {}
+	~CNet() {
+		try {
+			releaseGpu();
+		} catch (...) {
+		}
+		for (auto f : func_list_) delete f;
+	}
+	CNet(const CNet &) = delete;
+	CNet &operator=(const CNet &) = delete;
+
+	bool hasGPU() { return cnet_init(0) == CNET_OK; }
+
+	std::string PrintInfo(bool &was_failure) {
+		cnet_device_info info;
+		if (cnet_init(0) != CNET_OK || cnet_get_device_info(&info) != CNET_OK) {
+			was_failure = true;
+			return std::string("PrintInfo: ") + cnet_last_error();
+		}
+		was_failure = false;
+		std::ostringstream oss;
+		oss << "Device Number: 0\n  Device name: " << info.name << " (" << info.arch << ")\n  TotalGlobalMem: "
+			<< info.hbm_bytes / (1024 * 1024) << "\n  WarpSize: " << info.wavefront_size << "\n  MultiProcessorCount: "
+			<< info.compute_units << "\n  Clock (KHz): " << info.clock_khz << "\n  fp32 matrix peak (TFLOP/s): "
+			<< info.fp32_matrix_peak_tflops << "\n";
+		return oss.str();
+	}
+
+	// ---- graph construction (impl/cnet.h:228-289) ----
+	int add(CFunc *func) {
+		assert(func);
+		if (batch_) throw std::logic_error("add: the net is already allocated on the GPU");
+		if (func->uid_ == 0) func->uid_ = ++next_uid_;
+		else next_uid_ = std::max(next_uid_, func->uid_);
+		func->type_ = func->typeId();
+		if (map_.find(func->uid_) != map_.end()) throw std::invalid_argument("add: duplicate uid " + std::to_string(func->uid_));
+		func_list_.push_back(func);
+		map_[func->uid_] = func;
+		if (func->is_input_) inputs_.push_back(func);
+		if (func->is_output_) outputs_.push_back(func);
+		return func->uid_;
+	}
+	int add(CFunc *func, const std::vector<int> &in_uids) {
+		int uid = add(func);
+		int offset = 0;
+		for (auto in_uid : in_uids) {
+			auto it = map_.find(in_uid);
+			if (it == map_.end()) throw std::invalid_argument("add: unknown input uid " + std::to_string(in_uid));
+			it->second->addOutput(func, offset);
+			offset += it->second->out_size_;
+			func->prev_func_.push_back(it->second);
+		}
+		if (offset > func->input().length_) throw std::invalid_argument("add: inputs longer than " + func->getName());
+		return uid;
+	}
+	int add(CFunc *func, std::initializer_list<int> in_uids) { return add(func, std::vector<int>(in_uids)); }
+	CFunc *&operator[](int uid) { return map_[uid]; }
+	std::vector<CFunc *> &functionList() { return func_list_; }
+	const std::vector<CFunc *> &inputs() const { return inputs_; }
+
+	void init_inputs() { init_inputs((uint64_t) clock()); }
+	void init_inputs(uint64_t seed) {  // impl/cnet.h:301-311
+		int indx = 1;
+		for (auto f : inputs_) {
+			f->setRandSeed(seed + indx++);
+			f->init_inputs();
+		}
+	}
+	void init_exec_graph(bool print_status = false) {
+		graph_ready_ = true;
+		if (print_status) std::cout << toString();
+	}
+	std::string toString() {
+		std::ostringstream oss;
+		for (auto f : func_list_) {
+			oss << "depth: " << f->depth() << ": " << f->getName() << ": from C^" << f->input().length_ << " to C^" << f->out_size_;
+			for (int i = 0; i < f->no_outputs(); ++i) oss << " into " << f->next(i)->getName() << " at offset " << f->offset(i);
+			oss << "\n";
+		}
+		return oss.str();
+	}
+	CFunc *findFirstInput() {
+		for (auto f : func_list_)
+			if (dynamic_cast<InputFunc *>(f)) return f;
+		return NULL;
+	}
+	CFunc *findFirstOutput() {
+		for (auto f : func_list_)
+			if (dynamic_cast<OutputFunc *>(f)) return f;
+		return NULL;
+	}
+
+	// ---- device plan (upstream allocateOnGpu / AllocateNet, gpu/gpu_func.h:576-643, 1071-1086) ----
+	bool allocateOnGpu(int batch_size) {
+		if (batch_size < 1) throw std::invalid_argument("allocateOnGpu: batch size must be positive");
+		if (batch_) throw std::logic_error("Net already initialised on GPU.");
+		if (func_list_.empty()) throw std::logic_error("AllocateNet error: 0 depth net.");
+		ck(cnet_init(0), "cnet_init");
+		CFunc *inp = findFirstInput(), *outp = findFirstOutput();
+		if (!inp || !outp) throw std::logic_error("allocateOnGpu: the net needs an input and an output function");
+		dynamic_cast<InputFunc *>(inp)->setIsMainInput(true);
+		dynamic_cast<OutputFunc *>(outp)->setIsMainOutput(true);
+		main_input_ = inp;
+		batch_ = batch_size;
+		try {
+			plan();
+		} catch (...) {
+			releaseGpu();
+			throw;
+		}
+		return true;
+	}
+
+	void releaseGpu() {
+		if (!batch_ && allocations_.empty()) return;
+		for (void *p : allocations_) cnet_free(p);
+		allocations_.clear();
+		for (auto f : func_list_) {
+			f->slots_.clear();
+			f->out_ = NULL;
+			f->rows_ = 0;
+		}
+		batch_ = 0;
+		d_labels_ = NULL;
+	}
+
+	int batchSize() const { return batch_; }
+
+private:
+	void plan() {
+		// rows: data inputs and everything downstream of them are batched; parameter nodes have one row
+		for (auto f : func_list_) {
+			if (f->typeId() == isInput) {
+				f->rows_ = isParameter(f) ? 1 : batch_;
+			} else if (f->typeId() == isEmbedding) {
+				f->rows_ = batch_;
+			} else {
+				f->rows_ = 1;
+				for (auto p : f->prev_func_) f->rows_ = std::max(f->rows_, p->rows_);
+			}
+		}
+		for (auto f : func_list_) {
+			const int t = f->typeId();
+			const size_t rows = f->rows_;
+			if (t == isInput) {
+				// the node's own six planes are the parameter / the data; consumers read its z planes in place
+				float *six = dalloc<float>(6 * rows * f->input().length_);
+				f->out_ = six;
+				CFunc::Slot s;
+				s.producer = NULL;
+				s.len = f->input().length_;
+				s.rows = (int) rows;
+				s.grad = six + 2 * rows * s.len;
+				f->slots_.push_back(s);
+				ck(cnet_memset_zero(six, 6 * rows * s.len * sizeof(float)), "zero");
+			} else if (t == isEmbedding) {
+				CEmbedding *e = (CEmbedding *) f;
+				float *six = dalloc<float>(6 * (size_t) f->input().length_);  // the table, stored once
+				CFunc::Slot s;
+				s.len = f->input().length_;
+				s.rows = 1;
+				s.grad = six + 2 * (size_t) s.len;
+				f->slots_.push_back(s);
+				ck(cnet_memset_zero(six, 6 * (size_t) s.len * sizeof(float)), "zero");
+				e->d_tokens_ = dalloc<int32_t>(rows * e->no_out_tokens_);
+				f->out_ = dalloc<float>(2 * rows * f->out_size_);
+			} else {
+				int k = 0;
+				for (auto p : f->prev_func_) {
+					CFunc::Slot s;
+					s.producer = p;
+					// offset of this producer inside the concatenated per-sample input block (impl/cnet.h:259-268)
+					s.offset = 0;
+					for (int j = 0; j < k; ++j) s.offset += f->prev_func_[j]->out_size_;
+					s.len = p->out_size_;
+					s.rows = p->rows_;
+					s.grad = dalloc<float>(4 * (size_t) s.rows * s.len);
+					ck(cnet_memset_zero(s.grad, 4 * (size_t) s.rows * s.len * sizeof(float)), "zero");
+					f->slots_.push_back(s);
+					++k;
+				}
+				if (!f->is_output_) f->out_ = dalloc<float>(2 * rows * f->out_size_);
+			}
+			switch (t) {
+			case isLinear:
+				if (f->slots_.size() != 2 || f->slots_[1].rows != 1)
+					throw std::invalid_argument(f->getName() + ": the weight operand must be a parameter CInput (stored once)");
+				break;
+			case isHadamard:
+			case isResidual:
+				if (f->slots_.size() != 2) throw std::invalid_argument(f->getName() + ": needs two inputs");
+				if (t == isResidual && f->slots_[0].rows != f->slots_[1].rows)
+					throw std::invalid_argument(f->getName() + ": mixing a parameter and a batched operand is not supported");
+				if (t == isHadamard && f->slots_[0].rows < f->slots_[1].rows)
+					throw std::invalid_argument(f->getName() + ": put the batched operand first, the parameter second");
+				break;
+			case isFourier:
+				ck(cnet_cdft_plan(f->out_size_), "cnet_cdft_plan");
+				break;
+			case isSoftMax:
+				((SoftMax *) f)->d_s_ = dalloc<float>(rows);
+				break;
+			case isCrossEntropy: {
+				CrossEntropy *c = (CrossEntropy *) f;
+				c->d_s_ = dalloc<float>(rows);
+				c->d_loss_ = dalloc<float>(rows);
+				c->d_argmax_ = dalloc<int32_t>(rows);
+				c->d_norm_ = dalloc<float>(2 * rows * f->input().length_);
+				break;
+			}
+			case isL2Out:
+				((L2Out *) f)->d_loss_ = dalloc<float>(rows);
+				break;
+			default: break;
+			}
+			if (t != isInput && t != isEmbedding && f->slots_.empty())
+				throw std::invalid_argument(f->getName() + ": has no inputs");
+		}
+		d_labels_ = dalloc<int32_t>(batch_);
+		ck(cnet_memset_zero(d_labels_, batch_ * sizeof(int32_t)), "zero");
+		copyInputsToGpu();
+	}
+
+	// z planes of slot k of node f (read in place from the producer)
+	static const float *zre(CFunc *f, int k) { return f->slots_[k].producer->out_re(); }
+	static const float *zim(CFunc *f, int k) { return f->slots_[k].producer->out_im(); }
+	// the slot of consumer c that is fed by f (its gradient planes are f's upstream gradient)
+	static CFunc::Slot &upstream(CFunc *f, int c) {
+		CFunc *n = f->next_func_[c];
+		for (auto &s : n->slots_)
+			if (s.producer == f && s.offset == f->offset_[c]) return s;
+		throw std::logic_error("broken wiring at " + f->getName());
+	}
+
+	void nodeForward(CFunc *f) {
+		const int rows = f->rows_;
+		switch (f->typeId()) {
+		case isInput: break;  // consumers read the node's z planes in place
+		case isEmbedding: {
+			CEmbedding *e = (CEmbedding *) f;
+			const float *tab = f->slots_[0].grad - 2 * (size_t) f->slots_[0].len;
+			ck(cnet_embedding_fwd(tab, tab + f->slots_[0].len, e->embedding_dim_, e->no_embeddings_, e->d_tokens_, f->out_re(),
+					f->out_im(), f->out_size_, rows, e->no_out_tokens_), "cnet_embedding_fwd");
+			break;
+		}
+		case isLinear: {
+			const int K = f->slots_[0].len, N = f->out_size_;
+			ck(cnet_clinear_fwd(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), N, rows, K, N, 0),
+					"cnet_clinear_fwd");
+			break;
+		}
+		case isFourier:
+			ck(cnet_cdft_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_, 0),
+					"cnet_cdft_fwd");
+			break;
+		case isHadamard: {
+			const int n = f->out_size_;
+			ck(cnet_hadamard_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), f->slots_[1].rows == rows ? n : 0, f->out_re(),
+					f->out_im(), n, rows, n), "cnet_hadamard_fwd");
+			break;
+		}
+		case isGelu:
+			ck(cnet_cgelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_),
+					"cnet_cgelu_fwd");
+			break;
+		case isResidual: {
+			const int n = f->out_size_;
+			ck(cnet_residual_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), n, f->out_re(), f->out_im(), n, rows, n),
+					"cnet_residual_fwd");
+			break;
+		}
+		case isSoftMax:
+			ck(cnet_l2norm_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, ((SoftMax *) f)->d_s_, rows,
+					f->out_size_), "cnet_l2norm_fwd");
+			break;
+		case isCrossEntropy: {
+			CrossEntropy *c = (CrossEntropy *) f;
+			const int n = f->input().length_;
+			ck(cnet_cross_entropy_fwd(zre(f, 0), zim(f, 0), n, d_labels_, c->d_norm_, c->d_norm_ + (size_t) rows * n, n, c->d_s_,
+					c->d_loss_, c->d_argmax_, rows, n), "cnet_cross_entropy_fwd");
+			break;
+		}
+		case isL2Out:
+			ck(cnet_l2out_fwd(zre(f, 0), zim(f, 0), f->input().length_, ((L2Out *) f)->d_loss_, rows, f->input().length_),
+					"cnet_l2out_fwd");
+			break;
+		default: throw std::logic_error(f->getName() + ": no device implementation");
+		}
+	}
+
+	// Each consumer's contribution is added in turn (the per-consumer loops of the upstream layers); the first one
+	// overwrites, so the planes never need zeroing between steps.  Nodes without consumers get zeros.
+	void nodeBackward(CFunc *f, bool with_labels) {
+		const int rows = f->rows_;
+		const int t = f->typeId();
+		if (t == isCrossEntropy) {
+			if (!with_labels) return;  // upstream: CrossEntropy::backward() without a label does nothing
+			CrossEntropy *c = (CrossEntropy *) f;
+			CFunc::Slot &s = f->slots_[0];
+			ck(cnet_cross_entropy_bwd(zre(f, 0), zim(f, 0), s.len, c->d_s_, d_labels_, s.g(0), s.g(1), s.g(2), s.g(3), s.len, rows, s.len),
+					"cnet_cross_entropy_bwd");
+			return;
+		}
+		if (t == isL2Out) {
+			CFunc::Slot &s = f->slots_[0];
+			ck(cnet_l2out_bwd(zre(f, 0), zim(f, 0), s.len, s.g(0), s.g(1), s.g(2), s.g(3), s.len, rows, s.len, 0), "cnet_l2out_bwd");
+			return;
+		}
+		if (t == isInput) {  // impl/cinput.h:54-65: gathers dzs only, and keeps adding until the next update
+			CFunc::Slot &own = f->slots_[0];
+			for (int c = 0; c < f->no_outputs(); ++c) {
+				CFunc::Slot &u = upstream(f, c);
+				ck(cnet_add2d(u.g(2), u.len, own.g(2), own.len, own.rows, own.len), "cnet_add2d");
+				ck(cnet_add2d(u.g(3), u.len, own.g(3), own.len, own.rows, own.len), "cnet_add2d");
+			}
+			return;
+		}
+		if (t == isEmbedding) {
+			CEmbedding *e = (CEmbedding *) f;
+			CFunc::Slot &own = f->slots_[0];
+			for (int c = 0; c < f->no_outputs(); ++c) {
+				CFunc::Slot &u = upstream(f, c);
+				ck(cnet_embedding_bwd(e->d_tokens_, u.g(2), u.g(3), u.len, own.g(2), own.g(3), e->embedding_dim_, e->no_embeddings_,
+						rows, e->no_out_tokens_, 1), "cnet_embedding_bwd");
+			}
+			return;
+		}
+		if (f->no_outputs() == 0) {
+			for (auto &s : f->slots_) ck(cnet_memset_zero(s.grad, 4 * (size_t) s.rows * s.len * sizeof(float)), "zero");
+			return;
+		}
+		for (int c = 0; c < f->no_outputs(); ++c) {
+			CFunc::Slot &u = upstream(f, c);
+			const int acc = c > 0;
+			CFunc::Slot &a = f->slots_[0];
+			switch (t) {
+			case isLinear: {
+				CFunc::Slot &w = f->slots_[1];
+				const int K = a.len, N = f->out_size_;
+				ck(cnet_clinear_bwd_input(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K,
+						rows, K, N, acc), "cnet_clinear_bwd_input");
+				ck(cnet_clinear_bwd_weight(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K,
+						rows, K, N, acc), "cnet_clinear_bwd_weight");
+				break;
+			}
+			case isFourier:
+				ck(cnet_cdft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
+						"cnet_cdft_bwd");
+				break;
+			case isHadamard: {
+				CFunc::Slot &v = f->slots_[1];
+				const int n = f->out_size_;
+				ck(cnet_hadamard_bwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, u.g(0), u.g(1), u.g(2), u.g(3),
+						u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3), n, rows, n, acc), "cnet_hadamard_bwd");
+				break;
+			}
+			case isGelu:
+				ck(cnet_cgelu_bwd(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len,
+						rows, a.len, acc), "cnet_cgelu_bwd");
+				break;
+			case isResidual: {
+				CFunc::Slot &v = f->slots_[1];
+				const int n = f->out_size_;
+				ck(cnet_residual_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3),
+						n, rows, n, acc), "cnet_residual_bwd");
+				break;
+			}
+			case isSoftMax:
+				ck(cnet_l2norm_bwd(zre(f, 0), zim(f, 0), a.len, ((SoftMax *) f)->d_s_, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1),
+						a.g(2), a.g(3), a.len, rows, a.len, acc), "cnet_l2norm_bwd");
+				break;
+			default: throw std::logic_error(f->getName() + ": no device implementation");
+			}
+		}
+	}
+
+	void requireAllocated(const char *who) const {
+		if (!batch_) throw std::logic_error(std::string(who) + ": call allocateOnGpu(batch_size) first");
+	}
+
+public:
+	// ---- host <-> device (upstream copyInputsToGpu / getInputsFromGpu, gpu/gpu_func.h:512-527, 543-574) ----
+	bool copyInputsToGpu() {
+		requireAllocated("copyInputsToGpu");
+		for (auto f : inputs_) {
+			CFunc::Slot &s = f->slots_[0];
+			float *z = s.grad - 2 * (size_t) s.rows * s.len;
+			if (s.rows == 1) {
+				ck(cnet_memcpy_h2d(z, f->mutable_input()->real_, 2 * (size_t) s.len * sizeof(float)), "cnet_memcpy_h2d");
+			} else {  // the data input: the host view holds one sample, replicate it to every row
+				for (int b = 0; b < s.rows; ++b) {
+					ck(cnet_memcpy_h2d(z + (size_t) b * s.len, f->mutable_input()->real_, s.len * sizeof(float)), "cnet_memcpy_h2d");
+					ck(cnet_memcpy_h2d(z + (size_t) (s.rows + b) * s.len, f->mutable_input()->imag_, s.len * sizeof(float)), "cnet_memcpy_h2d");
+				}
+			}
+			if (f->typeId() == isEmbedding) uploadTokens((CEmbedding *) f, NULL);
+		}
+		return true;
+	}
+
+	bool getInputsFromGpu() {
+		requireAllocated("getInputsFromGpu");
+		for (auto f : inputs_) fetch(f, 0);
+		return true;
+	}
+
+	// Fill the per-sample host view of `f` (all six planes of its input block; for output functions also the output
+	// block) from row `b` of the device planes.  Parameter operands always come from their single row.
+	void fetch(CFunc *f, int b) {
+		requireAllocated("fetch");
+		if (b < 0 || b >= batch_) throw std::out_of_range("fetch: batch index");
+		ck(cnet_sync(), "cnet_sync");
+		Vars *v = f->mutable_input();
+		for (auto &s : f->slots_) {
+			const int row = s.rows == 1 ? 0 : b;
+			const float *z_re, *z_im;
+			if (s.producer) {
+				z_re = s.producer->out_re() + (size_t) (s.producer->rows_ == 1 ? 0 : b) * s.len;
+				z_im = s.producer->out_im() + (size_t) (s.producer->rows_ == 1 ? 0 : b) * s.len;
+			} else {
+				const float *z = s.grad - 2 * (size_t) s.rows * s.len;
+				z_re = z + (size_t) row * s.len;
+				z_im = z + (size_t) (s.rows + row) * s.len;
+			}
+			ck(cnet_memcpy_d2h(v->real_ + s.offset, z_re, s.len * sizeof(float)), "cnet_memcpy_d2h");
+			ck(cnet_memcpy_d2h(v->imag_ + s.offset, z_im, s.len * sizeof(float)), "cnet_memcpy_d2h");
+			for (int p = 0; p < 4; ++p)
+				ck(cnet_memcpy_d2h(v->plane(2 + p) + s.offset, s.g(p) + (size_t) row * s.len, s.len * sizeof(float)), "cnet_memcpy_d2h");
+		}
+		if (f->typeId() == isCrossEntropy) {
+			CrossEntropy *c = (CrossEntropy *) f;
+			const int n = f->input().length_;
+			ck(cnet_memcpy_d2h(c->output_.real_, c->d_norm_ + (size_t) b * n, n * sizeof(float)), "cnet_memcpy_d2h");
+			ck(cnet_memcpy_d2h(c->output_.imag_, c->d_norm_ + (size_t) (f->rows_ + b) * n, n * sizeof(float)), "cnet_memcpy_d2h");
+			int32_t am = 0;
+			ck(cnet_memcpy_d2h(&am, c->d_argmax_ + b, sizeof(am)), "cnet_memcpy_d2h");
+			c->prediction_ = am;
+		} else if (f->typeId() == isL2Out) {
+			ck(cnet_memcpy_d2h(((L2Out *) f)->output_.real_, ((L2Out *) f)->d_loss_ + b, sizeof(float)), "cnet_memcpy_d2h");
+		}
+	}
+	void fetchAll(int b) {
+		for (auto f : func_list_) fetch(f, b);
+	}
+
+	// ---- batched step (upstream gpuForward / gpuBackward / gpuUpdateInputs / getLoss,
+	//      gpu/gpu_func.h:1088-1101, 491-495, 906-926; step semantics of cnet.cpp:104-150) ----
+	bool gpuForward(InputFunc *inp, OutputFunc *outp, InputBatch &batch) {
+		requireAllocated("gpuForward");
+		CInput *cin = dynamic_cast<CInput *>(inp);
+		if (!cin) throw std::invalid_argument("gpuForward: this type of input is not supported with an InputBatch");
+		if (cin != main_input_) throw std::invalid_argument("gpuForward: not the main input of the allocated net");
+		if (batch.size() != batch_ || batch.noOfLabels() != batch_) throw std::invalid_argument("gpuForward: batch size differs from allocateOnGpu");
+		if (batch.sampleDim() != cin->input().length_) throw std::invalid_argument("gpuForward: sample dimension differs from the input length");
+		(void) outp;
+		CFunc::Slot &s = cin->slots_[0];
+		float *z = s.grad - 2 * (size_t) s.rows * s.len;
+		// one copy per plane (upstream: two small copies per sample, gpu/gpu_func.h:403-419)
+		ck(cnet_memcpy_h2d(z, batch.realDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
+		ck(cnet_memcpy_h2d(z + (size_t) batch_ * s.len, batch.imagDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
+		setLabels(batch.labelsPtr(), batch_);
+		return GpuForward();
+	}
+	// upload a batch into a CInput flagged with setIsBatched(true); labels of that batch are ignored
+	void gpuSetInput(CInput *cin, InputBatch &batch) {
+		requireAllocated("gpuSetInput");
+		if (cin->rows_ != batch_ || batch.size() != batch_ || batch.sampleDim() != cin->input().length_)
+			throw std::invalid_argument("gpuSetInput: " + cin->getName() + " is not a data input of this batch shape");
+		CFunc::Slot &s = cin->slots_[0];
+		float *z = s.grad - 2 * (size_t) s.rows * s.len;
+		ck(cnet_memcpy_h2d(z, batch.realDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
+		ck(cnet_memcpy_h2d(z + (size_t) batch_ * s.len, batch.imagDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
+	}
+	bool gpuForward(InputFunc *inp, OutputFunc *outp, EmbeddingBatch &batch) {
+		requireAllocated("gpuForward");
+		CEmbedding *emb = dynamic_cast<CEmbedding *>(inp);
+		if (!emb || emb != main_input_) throw std::invalid_argument("gpuForward: the EmbeddingBatch needs the main CEmbedding input");
+		if (batch.size() != batch_ || batch.noOfLabels() != batch_ || batch.sampleDim() != emb->no_out_tokens_)
+			throw std::invalid_argument("gpuForward: batch shape differs from the allocated net");
+		(void) outp;
+		uploadTokens(emb, batch.tokensPtr());
+		setLabels(batch.labelsPtr(), batch_);
+		return GpuForward();
+	}
+	bool GpuForward() {
+		requireAllocated("GpuForward");
+		for (auto f : func_list_) nodeForward(f);
+		return true;
+	}
+	bool gpuBackward() {
+		requireAllocated("gpuBackward");
+		for (int k = (int) func_list_.size() - 1; k >= 0; --k) nodeBackward(func_list_[k], true);
+		return true;
+	}
+	// z -= l_rate * dzs on every input function (the data input too, impl/cnet.h:413-421), then its gradients are cleared
+	void gpuUpdateInputs(float l_rate) {
+		requireAllocated("gpuUpdateInputs");
+		for (auto f : inputs_) {
+			CFunc::Slot &s = f->slots_[0];
+			const size_t n = (size_t) s.rows * s.len;
+			float *z = s.grad - 2 * n;
+			ck(cnet_sgd_update(z, z + n, s.g(2), s.g(3), (int64_t) n, l_rate, 1), "cnet_sgd_update");
+			ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
+		}
+	}
+	float getLoss(OutputFunc *outp, Batch *batch) {
+		requireAllocated("getLoss");
+		CFunc *f = dynamic_cast<CFunc *>(outp);
+		float *d = NULL;
+		if (CrossEntropy *c = dynamic_cast<CrossEntropy *>(f)) d = c->d_loss_;
+		else if (L2Out *l = dynamic_cast<L2Out *>(f)) d = l->d_loss_;
+		else throw std::invalid_argument("getLoss: not supported for this output");
+		std::vector<float> tmp(f->rows_);
+		ck(cnet_memcpy_d2h(tmp.data(), d, tmp.size() * sizeof(float)), "cnet_memcpy_d2h");
+		float loss = 0.f;
+		for (float v : tmp) {
+			loss += v;
+			if (batch) batch->addLoss(v);
+		}
+		return loss / tmp.size();
+	}
+	std::vector<int> getPredictions(OutputFunc *outp) {
+		requireAllocated("getPredictions");
+		CrossEntropy *c = dynamic_cast<CrossEntropy *>(outp);
+		if (!c) throw std::invalid_argument("getPredictions: needs a CrossEntropy output");
+		std::vector<int32_t> tmp(c->rows_);
+		ck(cnet_memcpy_d2h(tmp.data(), c->d_argmax_, tmp.size() * sizeof(int32_t)), "cnet_memcpy_d2h");
+		return std::vector<int>(tmp.begin(), tmp.end());
+	}
+	void setLabels(const int *labels, int count) {
+		requireAllocated("setLabels");
+		if (count != batch_) throw std::invalid_argument("setLabels: one label per batch row");
+		for (auto f : outputs_)
+			if (f->typeId() == isCrossEntropy)
+				for (int k = 0; k < count; ++k)
+					if (labels[k] < 0 || labels[k] >= f->input().length_) throw std::out_of_range("setLabels: label outside the CrossEntropy input");
+		labels_.assign(labels, labels + count);
+		ck(cnet_memcpy_h2d(d_labels_, labels, count * sizeof(int32_t)), "cnet_memcpy_h2d");
+	}
+	void sync() { ck(cnet_sync(), "cnet_sync"); }
+
+	// ---- per-sample API of upstream (CNet::forward / backward / updateInputs, gpu/gpu_func.h:1046-1056, 497-501):
+	//      host views are the state, the arithmetic runs on the device with a batch of one ----
+	void forward() {
+		if (!batch_) allocateOnGpu(1);
+		if (batch_ != 1) throw std::logic_error("forward(): the per-sample API needs allocateOnGpu(1); use gpuForward for batches");
+		copyInputsToGpu();
+		// upstream forward() clears the gradients of every non-input function (impl/cnet.h:372-374); the batched path
+		// never needs that (first contribution overwrites), the per-sample views do
+		for (auto f : func_list_)
+			if (!f->is_input_)
+				for (auto &s : f->slots_) ck(cnet_memset_zero(s.grad, 4 * (size_t) s.rows * s.len * sizeof(float)), "zero");
+		GpuForward();
+		fetchAll(0);
+	}
+	void backward(int label) {
+		if (batch_ != 1) throw std::logic_error("backward(): call forward() first");
+		if (label >= 0) setLabels(&label, 1);
+		// the label only enters the backward pass of CrossEntropy; its forward outputs do not depend on it except
+		// the device-side loss, which is refreshed here so getLoss() matches the label in use
+		for (auto f : outputs_)
+			if (f->typeId() == isCrossEntropy) nodeForward(f);
+		for (int k = (int) func_list_.size() - 1; k >= 0; --k) nodeBackward(func_list_[k], label >= 0);
+		fetchAll(0);
+	}
+	void backward() { backward(-1); }
+	void updateInputs(float l_rate) {
+		if (batch_ != 1) throw std::logic_error("updateInputs(): call forward() first");
+		gpuUpdateInputs(l_rate);
+		for (auto f : inputs_) fetch(f, 0);
+	}
+
+private:
+	void uploadTokens(CEmbedding *e, const int *batch_tokens) {
+		std::vector<int32_t> buf((size_t) e->rows_ * e->no_out_tokens_, NO_TOKEN);
+		if (batch_tokens) {
+			std::copy(batch_tokens, batch_tokens + buf.size(), buf.begin());
+		} else {  // the per-sample token list of setInput(), in every row
+			for (int b = 0; b < e->rows_; ++b) std::copy(e->tokens_.begin(), e->tokens_.end(), buf.begin() + (size_t) b * e->no_out_tokens_);
+		}
+		ck(cnet_memcpy_h2d(e->d_tokens_, buf.data(), buf.size() * sizeof(int32_t)), "cnet_memcpy_h2d");
+	}
+};
+
+#endif  // CNET_AMD_HOST_CNET_HPP_

@@ -100,6 +100,12 @@ int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const fl
  * F[p][q] = exp(-2 pi i p q / n) / sqrt(n), generated on the device with exact integer reduction of p*q mod n. */
 int cnet_cdft_plan(int n);      /* build (once) and keep the n x n twiddle planes; called at net allocation time */
 int cnet_cdft_twiddle(int n, const float **f_re, const float **f_im);  /* the planes of an existing plan */
+/* Diagnostic: replace the FORWARD operator of length n by a caller-supplied matrix f[p][q] (host, row-major, y_p =
+ * sum_q f[p][q] x_q); NULL, NULL restores the exact transform.  The upstream CPU forward is a float FFT whose twiddle
+ * recurrence (impl/utils.h:204-211, 242-249) makes it a fixed operator up to 9e-5 away from the exact DFT; feeding that
+ * operator here reproduces the CPU path to ~1e-6 and so separates its rounding from everything else.  The backward pass
+ * keeps the exact twiddles, as upstream's does (impl/ft.h:57-79). */
+int cnet_cdft_set_forward_matrix(int n, const float *host_f_re, const float *host_f_im);
 int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
                   int B, int n, int accumulate);      /* y = x * F */
 int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,

@@ -1,0 +1,545 @@
+// GPU test driver for the C++ host facade (cnet_amd/host/cnet.hpp): builds nets through the upstream-shaped API,
+// runs them on the device, and compares every plane with the CPU oracle (oracle/cnet_oracle.hpp) run sample by sample
+// with the upstream step semantics.  Run by tests/test_gpu_facade.py; prints one line per check and exits non-zero on
+// the first failure.
+//
+//   facade_test mnist              README net at config-1 shape: batch 64, 784 -> ... -> 10, one full training step
+//   facade_test resblock           residual stack with a second data input (L2 target), several SGD steps
+//   facade_test persample          the per-sample API (forward / backward(label) / updateInputs) on the device
+//   facade_test embedding          CEmbedding -> Linear -> CrossEntropy with an EmbeddingBatch
+//   facade_test errors             error behaviour
+//   facade_test c4 n blocks B steps lr   throughput of the residual stack (no oracle), JSON line
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <string>
+
+#include "cnet_amd/host/cnet.hpp"
+#include "oracle/cnet_oracle.hpp"
+
+static int g_fail = 0;
+static const double TOL = 1e-4;  // relative Frobenius bound of this build
+
+struct ErrAcc {  // accumulates |got - want|^2 and |want|^2 over many calls
+	double d = 0, r = 0;
+	void add(const float *got, const float *want, int n) {
+		for (int k = 0; k < n; ++k) {
+			double e = (double) got[k] - want[k];
+			d += e * e;
+			r += (double) want[k] * want[k];
+		}
+	}
+	double value() const { return std::sqrt(d) / std::max(std::sqrt(r), 1e-30); }
+};
+
+static void report(const std::string &what, double err, double tol = TOL) {
+	bool ok = err <= tol && std::isfinite(err);
+	printf("%s %-46s rel.err %.3e (bound %.1e)\n", ok ? "PASS" : "FAIL", what.c_str(), err, tol);
+	if (!ok) g_fail++;
+}
+static void expect(const std::string &what, bool ok) {
+	printf("%s %s\n", ok ? "PASS" : "FAIL", what.c_str());
+	if (!ok) g_fail++;
+}
+
+static void fill_normal(orc::Rng &r, float *p, size_t n, double sig) {
+	for (size_t k = 0; k < n; ++k) p[k] = (float) r.normal(0.0, sig);
+}
+
+// compare the six planes of a facade node's host view with an oracle node's block
+static void cmp_node(CFunc *f, orc::Node *o, ErrAcc *z, ErrAcc *g) {
+	const Vars &v = f->input();
+	z->add(v.real_, o->in.re, 2 * v.length_);
+	g->add(v.dz_real_, o->in.dz_re, 4 * v.length_);
+}
+
+// ------------------------------------------------------------------------------------------------- README net
+// exact = true : the device transform is the exact DFT.  The CPU forward differs from it by its own float-FFT rounding
+//                (6.7e-5 at n = 784), so one forward + backward is held to the 1e-4 bar and the step after an SGD update,
+//                where that difference has been fed back through the weights, to 3e-4.
+// exact = false: the CPU path's forward operator (its FFT applied to unit vectors) is installed on the device; everything
+//                must then agree to 1e-5 on both steps.
+static void test_mnist(bool exact) {
+	const int n = 784, classes = 10, B = 64;
+	const float lr = 0.05f;
+	orc::Rng rng(0);
+	std::vector<float> xs((size_t) B * n), hw(2 * n), lw((size_t) 2 * n * classes);
+	for (auto &v : xs) v = (float) rng.uniform();
+	fill_normal(rng, hw.data(), hw.size(), 0.05);
+	fill_normal(rng, lw.data(), lw.size(), 1.0 / std::sqrt((double) n));
+	std::vector<int> labels(B);
+	for (auto &l : labels) l = (int) (rng.next() % classes);
+
+	// facade: upstream README.md:19-30
+	CNet cnet;
+	auto inp = cnet.add(new CInput(OutSize(n)));
+	auto fft = cnet.add(new FourierTrans(InSize(n)), {inp});
+	auto h_data = cnet.add(new CInput(OutSize(n)));
+	auto hdm = cnet.add(new Hadamard(InSize(n), InSize(n)), {fft, h_data});
+	auto gelu = cnet.add(new CGelu(InSize(n)), {hdm});
+	auto l_data = cnet.add(new CInput(OutSize(n * classes)));
+	auto lin = cnet.add(new Linear(InSize(n), InSize(n * classes)), {gelu, l_data});
+	auto outp = cnet.add(new CrossEntropy(InSize(classes)), {lin});
+	std::copy(hw.begin(), hw.end(), cnet[h_data]->mutable_input()->real_);
+	std::copy(lw.begin(), lw.end(), cnet[l_data]->mutable_input()->real_);
+	cnet.init_exec_graph();
+	expect("allocateOnGpu(64)", cnet.allocateOnGpu(B));
+	if (!exact) {
+		std::vector<float> fr((size_t) n * n), fi((size_t) n * n), er(n), ei(n, 0.f), yr(n), yi(n);
+		for (int q = 0; q < n; ++q) {
+			std::fill(er.begin(), er.end(), 0.f);
+			er[q] = 1.f;
+			orc::dft_forward(n, er.data(), ei.data(), yr.data(), yi.data());
+			for (int p = 0; p < n; ++p) {
+				fr[(size_t) p * n + q] = yr[p];
+				fi[(size_t) p * n + q] = yi[p];
+			}
+		}
+		expect("install the CPU path's forward operator", cnet_cdft_set_forward_matrix(n, fr.data(), fi.data()) == CNET_OK);
+	}
+	const double tol0 = exact ? TOL : 1e-5, tol1 = exact ? 3e-4 : 1e-5;
+	CInput *cin = (CInput *) cnet[inp];
+	CrossEntropy *cen = (CrossEntropy *) cnet[outp];
+
+	// oracle: same net, one sample at a time
+	orc::Net on;
+	int ids[1];
+	int o_inp = on.add(orc::kInput, n, 0, 0, NULL, 0);
+	ids[0] = o_inp;
+	int o_fft = on.add(orc::kFourier, n, 0, 0, ids, 1);
+	int o_hw = on.add(orc::kInput, n, 0, 0, NULL, 0);
+	int two[2] = {o_fft, o_hw};
+	int o_hdm = on.add(orc::kHadamard, n, 0, 0, two, 2);
+	ids[0] = o_hdm;
+	int o_gelu = on.add(orc::kGelu, n, 0, 0, ids, 1);
+	int o_lw = on.add(orc::kInput, n * classes, 0, 0, NULL, 0);
+	two[0] = o_gelu;
+	two[1] = o_lw;
+	int o_lin = on.add(orc::kLinear, n, n * classes, 0, two, 2);
+	ids[0] = o_lin;
+	int o_out = on.add(orc::kCrossEntropy, classes, 0, 0, ids, 1);
+	std::copy(hw.begin(), hw.end(), on.at(o_hw)->in.re);
+	std::copy(lw.begin(), lw.end(), on.at(o_lw)->in.re);
+
+	std::vector<float> zeros(n, 0.f);
+	for (int step = 0; step < 2; ++step) {
+		InputBatch batch(B, n);
+		for (int b = 0; b < B; ++b) batch.add(xs.data() + (size_t) b * n, zeros.data(), n, labels[b]);
+		expect("gpuForward", cnet.gpuForward(cin, cen, batch));
+		float mean_loss = cnet.getLoss(cen, &batch);
+		expect("gpuBackward", cnet.gpuBackward());
+		std::vector<int> pred = cnet.getPredictions(cen);
+
+		ErrAcc z_fft, g_fft, z_hdm, g_hdm, z_gelu, g_gelu, z_lin, g_lin, z_out, g_out, e_norm, g_inp;
+		double loss_sum = 0, loss_err = 0;
+		int pred_mismatch = 0;
+		for (int b = 0; b < B; ++b) {
+			std::copy(xs.begin() + (size_t) b * n, xs.begin() + (size_t) (b + 1) * n, on.at(o_inp)->in.re);
+			std::fill(on.at(o_inp)->in.im, on.at(o_inp)->in.im + n, 0.f);
+			on.forward();
+			float l = on.loss(o_out, labels[b]);
+			loss_sum += l;
+			loss_err = std::max(loss_err, (double) std::fabs(l - batch.loss(b)) / std::max(1.0, (double) std::fabs(l)));
+			pred_mismatch += on.prediction(o_out) != pred[b];
+			on.backward(labels[b]);
+			cnet.fetchAll(b);
+			cmp_node(cnet[fft], on.at(o_fft), &z_fft, &g_fft);
+			// Hadamard: the u part per sample (the host view of the shared v part holds the batch sum, checked below)
+			z_hdm.add(cnet[hdm]->input().real_, on.at(o_hdm)->in.re, n);
+			z_hdm.add(cnet[hdm]->input().imag_, on.at(o_hdm)->in.im, n);
+			for (int p = 0; p < 4; ++p) g_hdm.add(cnet[hdm]->mutable_input()->plane(2 + p), on.at(o_hdm)->in.re + (size_t) (2 + p) * on.at(o_hdm)->in.n, n);
+			cmp_node(cnet[gelu], on.at(o_gelu), &z_gelu, &g_gelu);
+			cmp_node(cnet[outp], on.at(o_out), &z_out, &g_out);
+			// Linear: the x part per sample (the W part of the host view holds the batch sum, checked below)
+			z_lin.add(cnet[lin]->input().real_, on.at(o_lin)->in.re, n);
+			z_lin.add(cnet[lin]->input().imag_, on.at(o_lin)->in.im, n);
+			for (int p = 0; p < 4; ++p) g_lin.add(cnet[lin]->mutable_input()->plane(2 + p), on.at(o_lin)->in.re + (size_t) (2 + p) * on.at(o_lin)->in.n, n);
+			e_norm.add(cen->mutableOutput()->real_, on.at(o_out)->out.re, 2 * classes);
+			if (step == 0) {  // the data input accumulates dzs per row
+				g_inp.add(cnet[inp]->input().dz_star_real_, on.at(o_inp)->in.dzs_re, 2 * n);
+				// undo what the oracle's accumulation will not see again: each row is its own sample
+				on.at(o_inp)->in.zero_gradients();
+			}
+		}
+		std::string s = std::string(exact ? " [exact DFT]" : " [CPU forward operator]") + " step " + std::to_string(step);
+		const double tol = step == 0 ? tol0 : tol1;
+		report("FourierTrans input z" + s, z_fft.value(), tol);
+		report("FourierTrans dz, dz*" + s, g_fft.value(), tol);
+		report("Hadamard input u" + s, z_hdm.value(), tol);
+		report("Hadamard du, du*" + s, g_hdm.value(), tol);
+		report("CGelu input z" + s, z_gelu.value(), tol);
+		report("CGelu dz, dz*" + s, g_gelu.value(), tol);
+		report("Linear x" + s, z_lin.value(), tol);
+		report("Linear dx, dx*" + s, g_lin.value(), tol);
+		report("CrossEntropy input z" + s, z_out.value(), tol);
+		report("CrossEntropy dz, dz*" + s, g_out.value(), tol);
+		report("CrossEntropy normalised output" + s, e_norm.value(), tol);
+		if (step == 0) report("data input dz* per row" + s, g_inp.value(), tol);
+		report("per-sample loss" + s, loss_err, tol);
+		report("mean loss" + s, std::fabs(mean_loss - loss_sum / B) / std::fabs(loss_sum / B), tol);
+		expect("argmax bit-exact on all " + std::to_string(B) + " rows" + s, pred_mismatch == 0);
+
+		// parameter gradients: the sum over the batch, gathered by the parameter nodes
+		cnet.fetch(cnet[h_data], 0);
+		cnet.fetch(cnet[l_data], 0);
+		ErrAcc g_hw, g_lw;
+		g_hw.add(cnet[h_data]->input().dz_star_real_, on.at(o_hw)->in.dzs_re, 2 * n);
+		g_lw.add(cnet[l_data]->input().dz_star_real_, on.at(o_lw)->in.dzs_re, 2 * n * classes);
+		report("Hadamard weights dz* (batch sum)" + s, g_hw.value(), tol);
+		report("Linear weights dz* (batch sum)" + s, g_lw.value(), tol);
+		bool dz_zero = true;
+		for (int k = 0; k < 2 * n; ++k) dz_zero = dz_zero && cnet[h_data]->input().dz_real_[k] == 0.f;
+		expect("parameter dz stays zero" + s, dz_zero);
+
+		// SGD with lr / B as the upstream GPU loop (cnet.cpp:147 upstream)
+		cnet.gpuUpdateInputs(lr / B);
+		on.update(lr, B);
+		expect("getInputsFromGpu", cnet.getInputsFromGpu());
+		ErrAcc w1, w2, gz;
+		w1.add(cnet[h_data]->input().real_, on.at(o_hw)->in.re, 2 * n);
+		w2.add(cnet[l_data]->input().real_, on.at(o_lw)->in.re, 2 * n * classes);
+		report("Hadamard weights after update" + s, w1.value(), tol / 5);
+		report("Linear weights after update" + s, w2.value(), tol / 5);
+		bool cleared = true;
+		for (int k = 0; k < 4 * n * classes; ++k) cleared = cleared && cnet[l_data]->input().dz_real_[k] == 0.f;
+		expect("gradients cleared by the update" + s, cleared);
+	}
+	if (!exact) expect("restore the exact transform", cnet_cdft_set_forward_matrix(n, NULL, NULL) == CNET_OK);
+}
+
+// ------------------------------------------------------------------------------------------------- residual stack
+struct ResStack {
+	CNet net;
+	int x, t, l2;
+	std::vector<int> w;
+};
+
+static void build_stack(ResStack &r, int n, int blocks) {
+	r.x = r.net.add(new CInput(OutSize(n)));
+	int cur = r.x;
+	for (int b = 0; b < blocks; ++b) {
+		int w = r.net.add(new CInput(OutSize(n * n)));
+		r.w.push_back(w);
+		int lin = r.net.add(new Linear(InSize(n), InSize(n * n)), {cur, w});
+		int ge = r.net.add(new CGelu(InSize(n)), {lin});
+		cur = r.net.add(new Residual(InSize(n)), {cur, ge});
+	}
+	CInput *t = new CInput(OutSize(n));
+	t->setIsBatched(true);  // the (negated) L2 target: a second per-sample data input
+	r.t = r.net.add(t);
+	int diff = r.net.add(new Residual(InSize(n)), {cur, r.t});
+	r.l2 = r.net.add(new L2Out(InSize(n)), {diff});
+}
+
+static void test_resblock() {
+	const int n = 64, blocks = 3, B = 24, steps = 4;
+	const float lr = 0.01f;
+	orc::Rng rng(4);
+	std::vector<float> xs((size_t) 2 * B * n), ts((size_t) 2 * B * n);
+	fill_normal(rng, xs.data(), xs.size(), 1.0);
+	fill_normal(rng, ts.data(), ts.size(), 1.0);
+	std::vector<std::vector<float> > w0(blocks, std::vector<float>((size_t) 2 * n * n));
+	for (auto &w : w0) fill_normal(rng, w.data(), w.size(), 1.0 / std::sqrt((double) n));
+
+	ResStack r;
+	build_stack(r, n, blocks);
+	for (int b = 0; b < blocks; ++b) std::copy(w0[b].begin(), w0[b].end(), r.net[r.w[b]]->mutable_input()->real_);
+	r.net.allocateOnGpu(B);
+
+	orc::Net on;
+	int ox = on.add(orc::kInput, n, 0, 0, NULL, 0), cur = ox;
+	std::vector<int> ow;
+	for (int b = 0; b < blocks; ++b) {
+		int w = on.add(orc::kInput, n * n, 0, 0, NULL, 0);
+		ow.push_back(w);
+		int two[2] = {cur, w};
+		int lin = on.add(orc::kLinear, n, n * n, 0, two, 2);
+		int ge = on.add(orc::kGelu, n, 0, 0, &lin, 1);
+		int two2[2] = {cur, ge};
+		cur = on.add(orc::kResidual, n, 0, 0, two2, 2);
+		std::copy(w0[b].begin(), w0[b].end(), on.at(w)->in.re);
+	}
+	int ot = on.add(orc::kInput, n, 0, 0, NULL, 0);
+	int two[2] = {cur, ot};
+	int odiff = on.add(orc::kResidual, n, 0, 0, two, 2);
+	int ol2 = on.add(orc::kL2Out, n, 0, 0, &odiff, 1);
+
+	CInput *cx = (CInput *) r.net[r.x], *ct = (CInput *) r.net[r.t];
+	L2Out *l2 = (L2Out *) r.net[r.l2];
+	for (int step = 0; step < steps; ++step) {
+		InputBatch bx(B, n), bt(B, n);
+		for (int b = 0; b < B; ++b) {
+			bx.add(xs.data() + (size_t) b * n, xs.data() + (size_t) (B + b) * n, n, 0);
+			bt.add(ts.data() + (size_t) b * n, ts.data() + (size_t) (B + b) * n, n, 0);
+		}
+		r.net.gpuSetInput(ct, bt);  // inputs are re-set every step: the update steps the data inputs too
+		r.net.gpuForward(cx, l2, bx);
+		float mean = r.net.getLoss(l2, &bx);
+		r.net.gpuBackward();
+		double loss_sum = 0, loss_err = 0;
+		ErrAcc gx;
+		for (int b = 0; b < B; ++b) {
+			orc::Planes &px = on.at(ox)->in, &pt = on.at(ot)->in;
+			std::copy(xs.data() + (size_t) b * n, xs.data() + (size_t) (b + 1) * n, px.re);
+			std::copy(xs.data() + (size_t) (B + b) * n, xs.data() + (size_t) (B + b + 1) * n, px.im);
+			std::copy(ts.data() + (size_t) b * n, ts.data() + (size_t) (b + 1) * n, pt.re);
+			std::copy(ts.data() + (size_t) (B + b) * n, ts.data() + (size_t) (B + b + 1) * n, pt.im);
+			px.zero_gradients();
+			pt.zero_gradients();
+			on.forward();
+			float l = on.loss(ol2, 0);
+			loss_sum += l;
+			loss_err = std::max(loss_err, (double) std::fabs(l - bx.loss(b)) / l);
+			on.backward(-1);
+			r.net.fetch(cx, b);
+			gx.add(cx->input().dz_star_real_, px.dzs_re, 2 * n);  // fan-out 2: Linear and Residual
+		}
+		std::string s = " step " + std::to_string(step);
+		report("L2 loss per sample" + s, loss_err, 2e-5);
+		report("mean loss" + s, std::fabs(mean - loss_sum / B) / (loss_sum / B), 2e-5);
+		report("data input dz* (two consumers)" + s, gx.value());
+		ErrAcc gw;
+		for (int b = 0; b < blocks; ++b) {
+			r.net.fetch(r.net[r.w[b]], 0);
+			gw.add(r.net[r.w[b]]->input().dz_star_real_, on.at(ow[b])->in.dzs_re, 2 * n * n);
+		}
+		report("weight dz* of all blocks (batch sum)" + s, gw.value());
+		r.net.gpuUpdateInputs(lr / B);
+		on.update(lr, B);
+		ErrAcc ww;
+		for (int b = 0; b < blocks; ++b) {
+			r.net.fetch(r.net[r.w[b]], 0);
+			ww.add(r.net[r.w[b]]->input().real_, on.at(ow[b])->in.re, 2 * n * n);
+		}
+		report("weights after update" + s, ww.value(), 1e-5);
+		printf("     step %d mean loss %.6f\n", step, mean);
+	}
+}
+
+// ------------------------------------------------------------------------------------------------- per-sample API
+static void test_persample() {
+	// upstream README.md:103-117 pattern: forward / loss / backward / updateInputs in a loop, on a small net
+	const int n = 48, classes = 6;
+	orc::Rng rng(9);
+	std::vector<float> x(2 * n), w((size_t) 2 * n * classes);
+	fill_normal(rng, x.data(), x.size(), 1.0);
+	fill_normal(rng, w.data(), w.size(), 0.2);
+
+	CNet net;
+	auto inp = net.add(new CInput(OutSize(n)));
+	auto sm = net.add(new SoftMax(InSize(n)), {inp});
+	auto wd = net.add(new CInput(OutSize(n * classes)));
+	auto lin = net.add(new Linear(InSize(n), InSize(n * classes)), {sm, wd});
+	auto ge = net.add(new CGelu(InSize(classes)), {lin});
+	auto ce = net.add(new CrossEntropy(InSize(classes)), {ge});
+	std::copy(x.begin(), x.end(), net[inp]->mutable_input()->real_);
+	std::copy(w.begin(), w.end(), net[wd]->mutable_input()->real_);
+	net.init_exec_graph(false);
+
+	orc::Net on;
+	int oi = on.add(orc::kInput, n, 0, 0, NULL, 0);
+	int osm = on.add(orc::kSoftMax, n, 0, 0, &oi, 1);
+	int owd = on.add(orc::kInput, n * classes, 0, 0, NULL, 0);
+	int two[2] = {osm, owd};
+	int olin = on.add(orc::kLinear, n, n * classes, 0, two, 2);
+	int oge = on.add(orc::kGelu, classes, 0, 0, &olin, 1);
+	int oce = on.add(orc::kCrossEntropy, classes, 0, 0, &oge, 1);
+	std::copy(x.begin(), x.end(), on.at(oi)->in.re);
+	std::copy(w.begin(), w.end(), on.at(owd)->in.re);
+
+	CrossEntropy *cen = (CrossEntropy *) net[ce];
+	float first = 0, last = 0;
+	for (int it = 0; it < 12; ++it) {
+		const int label = 2;
+		net.forward();
+		on.forward();
+		float l = cen->loss(label), lo = on.loss(oce, label);
+		if (it == 0) first = l;
+		last = l;
+		net.backward(label);
+		on.backward(label);
+		ErrAcc z, g;
+		int ids[6][2] = {{inp, oi}, {sm, osm}, {wd, owd}, {lin, olin}, {ge, oge}, {ce, oce}};
+		for (auto &p : ids) cmp_node(net[p[0]], on.at(p[1]), &z, &g);
+		if (it == 0 || it == 11) {
+			report("iteration " + std::to_string(it) + " all node values", z.value());
+			report("iteration " + std::to_string(it) + " all node gradients", g.value());
+			report("iteration " + std::to_string(it) + " loss", std::fabs(l - lo) / std::fabs(lo), 1e-5);
+			expect("iteration " + std::to_string(it) + " prediction", cen->get_prediction() == on.prediction(oce));
+		}
+		net.updateInputs(0.3f);
+		on.update(0.3f, 1);
+	}
+	expect("loss decreases under Wirtinger gradient descent (" + std::to_string(first) + " -> " + std::to_string(last) + ")", last < first);
+}
+
+// ------------------------------------------------------------------------------------------------- embedding
+static void test_embedding() {
+	const int dim = 8, slots = 5, vocab = 23, classes = 7, B = 6;
+	orc::Rng rng(21);
+	std::vector<float> table((size_t) 2 * vocab * dim), w((size_t) 2 * slots * dim * classes);
+	fill_normal(rng, table.data(), table.size(), 1.0);
+	fill_normal(rng, w.data(), w.size(), 0.3);
+	std::vector<std::vector<int> > toks(B);
+	std::vector<int> labels(B);
+	for (int b = 0; b < B; ++b) {
+		int count = 1 + (int) (rng.next() % slots);
+		for (int k = 0; k < count; ++k) toks[b].push_back((int) (rng.next() % vocab));
+		labels[b] = (int) (rng.next() % classes);
+	}
+	toks[1] = toks[0];  // repeated tokens across rows
+
+	CNet net;
+	auto emb = net.add(new CEmbedding(dim, slots, vocab));
+	auto wd = net.add(new CInput(OutSize(slots * dim * classes)));
+	auto lin = net.add(new Linear(InSize(slots * dim), InSize(slots * dim * classes)), {emb, wd});
+	auto ce = net.add(new CrossEntropy(InSize(classes)), {lin});
+	std::copy(table.begin(), table.end(), net[emb]->mutable_input()->real_);
+	std::copy(w.begin(), w.end(), net[wd]->mutable_input()->real_);
+	((CEmbedding *) net[emb])->setInput({0});
+	net.allocateOnGpu(B);
+
+	orc::Net on;
+	int oe = on.add(orc::kEmbedding, dim, slots, vocab, NULL, 0);
+	int ow = on.add(orc::kInput, slots * dim * classes, 0, 0, NULL, 0);
+	int two[2] = {oe, ow};
+	int ol = on.add(orc::kLinear, slots * dim, slots * dim * classes, 0, two, 2);
+	int oc = on.add(orc::kCrossEntropy, classes, 0, 0, &ol, 1);
+	std::copy(table.begin(), table.end(), on.at(oe)->in.re);
+	std::copy(w.begin(), w.end(), on.at(ow)->in.re);
+
+	EmbeddingBatch batch(B, slots);
+	for (int b = 0; b < B; ++b) batch.add(toks[b], labels[b]);
+	CrossEntropy *cen = (CrossEntropy *) net[ce];
+	net.gpuForward((CEmbedding *) net[emb], cen, batch);
+	net.getLoss(cen, &batch);
+	net.gpuBackward();
+	ErrAcc zl;
+	double loss_err = 0;
+	for (int b = 0; b < B; ++b) {
+		on.at(oe)->tokens = toks[b];
+		on.forward();
+		loss_err = std::max(loss_err, (double) std::fabs(on.loss(oc, labels[b]) - batch.loss(b)));
+		on.backward(labels[b]);
+		net.fetch(net[lin], b);
+		zl.add(net[lin]->input().real_, on.at(ol)->in.re, slots * dim);  // gathered rows incl. zero padding
+		zl.add(net[lin]->input().imag_, on.at(ol)->in.im, slots * dim);
+	}
+	report("gathered embedding rows", zl.value(), 0.0);
+	report("loss per sample", loss_err, 1e-5);
+	net.fetch(net[emb], 0);
+	ErrAcc gt;
+	gt.add(net[emb]->input().dz_star_real_, on.at(oe)->in.dzs_re, 2 * vocab * dim);
+	report("embedding table dz* (scatter-add over the batch)", gt.value());
+}
+
+// ------------------------------------------------------------------------------------------------- error behaviour
+template <class E, class F>
+static bool throws(F f) {
+	try {
+		f();
+	} catch (const E &) {
+		return true;
+	} catch (...) {
+		return false;
+	}
+	return false;
+}
+
+static void test_errors() {
+	CNet net;
+	auto x = net.add(new CInput(OutSize(8)));
+	auto l2 = net.add(new L2Out(InSize(8)), {x});
+	expect("gpuBackward before allocateOnGpu throws", throws<std::logic_error>([&] { net.gpuBackward(); }));
+	expect("unknown input uid throws", throws<std::invalid_argument>([&] { net.add(new CGelu(InSize(8)), {77}); }));
+	expect("producer longer than consumer throws", throws<std::invalid_argument>([&] { net.add(new L2Out(InSize(4)), {x}); }));
+	CNet net2;
+	auto x2 = net2.add(new CInput(OutSize(8)));
+	auto o2 = net2.add(new L2Out(InSize(8)), {x2});
+	net2.allocateOnGpu(4);
+	expect("second allocateOnGpu throws", throws<std::logic_error>([&] { net2.allocateOnGpu(4); }));
+	expect("add after allocation throws", throws<std::logic_error>([&] { net2.add(new CInput(OutSize(2))); }));
+	InputBatch wrong(3, 8);
+	for (int b = 0; b < 3; ++b) wrong.add({{1.f, 2.f}}, 0);
+	expect("batch of the wrong size throws", throws<std::invalid_argument>([&] {
+		net2.gpuForward((CInput *) net2[x2], (L2Out *) net2[o2], wrong);
+	}));
+	expect("per-sample forward on a batched plan throws", throws<std::logic_error>([&] { net2.forward(); }));
+	CNet net3;  // a Linear whose weight operand is per-sample data is refused
+	auto a = net3.add(new CInput(OutSize(4)));
+	CInput *wb = new CInput(OutSize(8));
+	wb->setIsBatched(true);
+	auto b = net3.add(wb);
+	auto lin = net3.add(new Linear(InSize(4), InSize(8)), {a, b});
+	net3.add(new L2Out(InSize(2)), {lin});
+	expect("batched weight operand is refused", throws<std::invalid_argument>([&] { net3.allocateOnGpu(2); }));
+	(void) l2;
+	// device layer status codes
+	expect("invalid argument gives a status, not an exit", cnet_cgemm(0, 0, 0, 4, 4, 0, NULL, NULL, 0, NULL, NULL, 0, NULL, NULL, 0, 0) == CNET_ERR_INVALID_ARGUMENT);
+	expect("error text names the call", std::string(cnet_last_error()).find("cnet_cgemm") != std::string::npos);
+}
+
+// ------------------------------------------------------------------------------------------------- throughput
+static void run_c4(int n, int blocks, int B, int steps, float lr) {
+	orc::Rng rng(4);
+	ResStack r;
+	build_stack(r, n, blocks);
+	for (int b = 0; b < blocks; ++b) fill_normal(rng, r.net[r.w[b]]->mutable_input()->real_, (size_t) 2 * n * n, 1.0 / std::sqrt((double) n));
+	r.net.allocateOnGpu(B);
+	std::vector<float> xs((size_t) 2 * B * n), ts((size_t) 2 * B * n);
+	fill_normal(rng, xs.data(), xs.size(), 1.0);
+	fill_normal(rng, ts.data(), ts.size(), 1.0);
+	InputBatch bx(B, n), bt(B, n);
+	for (int b = 0; b < B; ++b) {
+		bx.add(xs.data() + (size_t) b * n, xs.data() + (size_t) (B + b) * n, n, 0);
+		bt.add(ts.data() + (size_t) b * n, ts.data() + (size_t) (B + b) * n, n, 0);
+	}
+	CInput *cx = (CInput *) r.net[r.x], *ct = (CInput *) r.net[r.t];
+	L2Out *l2 = (L2Out *) r.net[r.l2];
+	std::vector<float> losses;
+	auto one = [&]() {
+		r.net.gpuSetInput(ct, bt);
+		r.net.gpuForward(cx, l2, bx);
+		losses.push_back(r.net.getLoss(l2, NULL));
+		r.net.gpuBackward();
+		r.net.gpuUpdateInputs(lr / B);  // upstream GPU loop: l_rate / batch.size() (cnet.cpp:147 upstream)
+	};
+	// timed region = the `steps` training steps from the initial weights (the first call also pays the one-off
+	// workspace growth; it is part of the job)
+	r.net.sync();
+	auto t0 = std::chrono::steady_clock::now();
+	for (int s = 0; s < steps; ++s) one();
+	r.net.sync();
+	double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+	printf("losses:");
+	for (float l : losses) printf(" %.4f", l);
+	printf("\n");
+	double flops = 40.0 * B * (double) n * n * blocks;  // GEMM flops per step
+	printf("{\"workload\": \"residual stack: %d x (Linear %d->%d, CGelu, Residual), L2Out, SGD\", \"batch\": %d, \"steps\": %d, "
+		   "\"ms_per_step\": %.3f, \"samples_per_sec\": %.1f, \"gemm_tflops\": %.2f, \"first_loss\": %.4f, \"last_loss\": %.4f}\n",
+			blocks, n, n, B, steps, 1e3 * sec / steps, B * steps / sec, flops * steps / sec / 1e12, losses.front(), losses.back());
+	if (!(losses.back() < losses.front())) {
+		printf("FAIL loss did not decrease\n");
+		g_fail++;
+	}
+}
+
+int main(int argc, char **argv) {
+	std::string what = argc > 1 ? argv[1] : "all";
+	try {
+		if (what == "mnist" || what == "all") test_mnist(true);
+		if (what == "mnist_cpu_operator" || what == "all") test_mnist(false);
+		if (what == "resblock" || what == "all") test_resblock();
+		if (what == "persample" || what == "all") test_persample();
+		if (what == "embedding" || what == "all") test_embedding();
+		if (what == "errors" || what == "all") test_errors();
+		if (what == "c4")
+			run_c4(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048, argc > 5 ? atoi(argv[5]) : 10,
+					argc > 6 ? (float) atof(argv[6]) : 0.01f);
+	} catch (const std::exception &e) {
+		printf("FAIL uncaught exception: %s\n", e.what());
+		return 2;
+	}
+	printf("%s: %d failure(s)\n", what.c_str(), g_fail);
+	return g_fail ? 1 : 0;
+}

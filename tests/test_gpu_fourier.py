@@ -81,3 +81,31 @@ def test_twiddle_matrix_entries(gpu):
         assert np.max(np.abs(host[0, :, :n] - want.real)) < 1e-8 + 6e-8 / np.sqrt(n)
         assert np.max(np.abs(host[1, :, :n] - want.imag)) < 1e-8 + 6e-8 / np.sqrt(n)
         assert np.array_equal(host[0, :, :n], host[0, :, :n].T)
+
+
+def test_cpu_forward_operator_can_be_installed(gpu, port):
+    """With the CPU path's own forward operator (its FFT applied to unit vectors) on the device, the forward pass matches
+    the CPU path to summation-order rounding; this isolates the CPU FFT's twiddle rounding as the source of the ~1e-4
+    forward difference.  The backward pass keeps the exact twiddles on both sides."""
+    B, n = 8, 784
+    xr, xi = seeded(port, 5, (B, n)), seeded(port, 6, (B, n))
+    yr, yi = port.dft_fwd(xr, xi)
+    fr, fi = port.dft_matrix(n)
+    x, y = ops.CMat.from_host(xr, xi), ops.CMat.empty(B, n)
+    ops.dft_fwd(x, y)
+    exact_err = rel_c(y.host(), (yr, yi))
+    capi.call("cnet_cdft_set_forward_matrix", n, fr.ctypes.data, fi.ctypes.data)
+    try:
+        ops.dft_fwd(x, y)
+        installed_err = rel_c(y.host(), (yr, yi))
+        g4 = [seeded(port, 7 + p, (B, n)) for p in range(4)]
+        dx = ops.Grad.empty(B, n)
+        ops.dft_bwd(ops.Grad.from_host(g4), dx)
+        dxo = port.dft_bwd(g4)
+        assert rel_c(dx.host()[0:2], dxo[0:2]) < 2e-6
+    finally:
+        capi.call("cnet_cdft_set_forward_matrix", n, None, None)
+    ops.dft_fwd(x, y)
+    assert installed_err < 2e-6, installed_err
+    assert 2e-5 < exact_err < TOL, exact_err
+    assert abs(rel_c(y.host(), (yr, yi)) - exact_err) < 1e-9
