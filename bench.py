@@ -93,6 +93,95 @@ def cpu_baseline(budget_s=15.0):
                       "%.2f ms/row (%.1f samples/s)" % (rows, B, dt, 1e3 * dt / rows, rows / dt)}
 
 
+def kernel_suite(steps):
+    """Per-kernel lines for the other rows of the hot path: the DFT-as-GEMM at config-3 shape (MFMA bound) and the
+    elementwise / reduction kernels at config-4/5 shapes (HBM bound).  Bytes are the algorithmic (compulsory) traffic
+    per complex element: every operand read once, every result written once, parameters amortised over the batch."""
+    from cnet_amd import capi, ops
+    capi.init(0)
+    ev = HipEvents(capi.load().cnet_stream())
+    rs = np.random.RandomState(0)
+
+    def cmat(r, c):
+        return ops.CMat.from_host(rs.randn(r, c).astype(np.float32), rs.randn(r, c).astype(np.float32))
+
+    def grad(r, c):
+        return ops.Grad.from_host([rs.randn(r, c).astype(np.float32) for _ in range(4)])
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        capi.sync()
+        a, b = ev.event(), ev.event()
+        ev.record(a)
+        for _ in range(steps):
+            fn()
+        ev.record(b)
+        return ev.elapsed_ms(a, b) / steps
+
+    lines = []
+
+    def hbm(name, shape, bytes_per_elem, elems, fn, extra_bytes=0):
+        ms = timed(fn)
+        gbs = (bytes_per_elem * elems + extra_bytes) / ms / 1e6
+        lines.append({"kernel": name, "shape": shape, "ms": round(ms, 4), "roofline": {
+            "bound": "hbm", "achieved": round(gbs, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(gbs / 8000.0, 4),
+            "bytes_per_complex_element": bytes_per_elem}})
+
+    def mfma(name, shape, flops, fn):
+        ms = timed(fn)
+        tf = flops / ms / 1e9
+        lines.append({"kernel": name, "shape": shape, "ms": round(ms, 4), "roofline": {
+            "bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}})
+
+    # config 3: FourierTrans n = 4096, batch 1024 (3 complex GEMMs against the twiddle matrix)
+    Bf, nf = 1024, 4096
+    x, y, g, dx = cmat(Bf, nf), ops.CMat.empty(Bf, nf), grad(Bf, nf), ops.Grad.empty(Bf, nf)
+    mfma("cdft_fwd", [Bf, nf], 8.0 * Bf * nf * nf, lambda: ops.dft_fwd(x, y))
+    mfma("cdft_bwd", [Bf, nf], 16.0 * Bf * nf * nf, lambda: ops.dft_bwd(g, dx))
+    del x, y, g, dx
+
+    # config 5 activation shape [8192 x 4096]: 256 MiB per complex matrix, so every operand streams from HBM
+    # (config 4's [2048 x 2048] planes would sit in the 256 MB memory-side cache and overstate the rate)
+    R, Cc = 8192, 4096
+    n = R * Cc
+    u, v, w1 = cmat(R, Cc), cmat(R, Cc), cmat(1, Cc)
+    yy, g, du, dv, dw1 = ops.CMat.empty(R, Cc), grad(R, Cc), ops.Grad.empty(R, Cc), ops.Grad.empty(R, Cc), ops.Grad.empty(1, Cc)
+    hbm("plain copy of one plane (practical HBM ceiling)", [R, Cc], 8, n, lambda: ops.copy2d(u.re, yy.re))
+    hbm("cgelu_fwd", [R, Cc], 16, n, lambda: ops.gelu_fwd(u, yy))
+    hbm("cgelu_bwd", [R, Cc], 40, n, lambda: ops.gelu_bwd(u, g, du))
+    hbm("residual_fwd", [R, Cc], 24, n, lambda: ops.residual_fwd(u, v, yy))
+    hbm("residual_bwd", [R, Cc], 48, n, lambda: ops.residual_bwd(g, du, dv))
+    hbm("hadamard_fwd (shared weights)", [R, Cc], 16, n, lambda: ops.hadamard_fwd(u, w1, yy, True))
+    hbm("hadamard_bwd (shared weights, batch-summed dW)", [R, Cc], 40, n, lambda: ops.hadamard_bwd(u, w1, g, du, dw1, True),
+        extra_bytes=16 * Cc)
+    loss = capi.empty(R)
+    hbm("l2out_fwd", [R, Cc], 8, n, lambda: ops.l2out_fwd(u, loss))
+    hbm("l2out_bwd", [R, Cc], 24, n, lambda: ops.l2out_bwd(u, du))
+    s_ = capi.empty(R)
+    hbm("l2norm_fwd (SoftMax)", [R, Cc], 16, n, lambda: ops.l2norm_fwd(u, yy, s_))
+    hbm("l2norm_bwd (SoftMax)", [R, Cc], 40, n, lambda: ops.l2norm_bwd(u, s_, g, du))
+    hbm("sgd_update", [n], 32, n, lambda: ops.sgd_update(u, du.planes[2], du.planes[3], 1e-9))
+    hbm("zero 4 gradient planes", [R, Cc], 16, n, lambda: [p.owner.zero() for p in du.planes])
+    out1 = ops.Plane.empty(1, Cc)
+    hbm("batch_sum (one plane)", [R, Cc], 4, n, lambda: ops.batch_sum(u.re, out1))
+    del u, v, yy, g, du, dv
+
+    # config 5: CrossEntropy over 32768 logits (rows reduced from 8192 to 2048 to keep the suite short)
+    R, Cc = 2048, 32768
+    n = R * Cc
+    z = cmat(R, Cc)
+    labels = ops.ints(rs.randint(0, Cc, R))
+    s_, l_, am = capi.empty(R), capi.empty(R), capi.empty(R, np.int32)
+    dz = ops.Grad.empty(R, Cc)
+    hbm("cross_entropy_fwd (loss, argmax; no normalised output)", [R, Cc], 8, n,
+        lambda: ops.cross_entropy_fwd(z, labels, s_, l_, am, None), extra_bytes=4 * R)
+    hbm("cross_entropy_bwd", [R, Cc], 24, n, lambda: ops.cross_entropy_bwd(z, s_, labels, dz))
+    for ln in lines:
+        print(json.dumps(ln))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -102,10 +191,16 @@ def main():
     ap.add_argument("--counter-pass", action="store_true",
                     help="short run for `rocprofv3 --pmc`: 3 launches of each GEMM kernel plus a plain copy kernel of "
                          "known size (256 MiB read, 256 MiB written) that calibrates FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--suite", choices=["linear", "kernels"], default="linear",
+                    help="linear (default): the headline line.  kernels: one line per other kernel of the hot path")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (one process, one device, no collectives); --gpus %d is not "
                  "supported. Run with --gpus 1." % args.gpus)
+
+    if args.suite == "kernels":
+        kernel_suite(max(args.steps // 5, 10))
+        return
 
     from cnet_amd import capi, ops
     capi.init(0)

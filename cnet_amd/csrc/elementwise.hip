@@ -6,6 +6,8 @@
 // wavefront touches 1 KiB of each plane per access and every byte is read and written exactly once.
 #include "common.hpp"
 
+#include <algorithm>
+
 namespace {
 
 constexpr int TPB = 256;
@@ -122,57 +124,76 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_kernel(const float *__restri
 	outv<V>(dv.dzs_im + ov, o, accumulate);
 }
 
-// v is one shared parameter row.  blockIdx.y selects a slab of rows; each thread owns V columns, writes du for its
-// rows and keeps the four dv sums of its slab in registers; partial[slab][plane][cols] goes to the workspace and a
-// second kernel adds the slabs in slab order (deterministic, no atomics).
+// v is one shared parameter row.  Workgroup = 64 column groups (V columns each) x 4 row lanes; blockIdx.y selects a slab
+// of rows.  Each thread writes du for its rows and keeps the four dv sums of those rows in registers; the four row
+// lanes are added through LDS in lane order and partial[slab][plane][cols] goes to the workspace; a second kernel adds
+// the slabs in slab order.  Deterministic: no atomics, fixed summation tree.
+constexpr int CS_X = 64, CS_Y = 4;
+
 template <int V>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *__restrict__ ur, const float *__restrict__ ui,
 		long ldu, const float *__restrict__ vr, const float *__restrict__ vi, CGrad4 g, long ldg, Grad4 du, long lddu,
 		float *__restrict__ partial, int rows, int cols, int rows_per_slab, int accumulate) {
-	const long col = ((long) blockIdx.x * TPB + threadIdx.x) * V;
-	if (col >= cols) return;
+	__shared__ float red[CS_Y][4][CS_X * V];
+	const int tx = threadIdx.x % CS_X, ty = threadIdx.x / CS_X;
+	const long col = ((long) blockIdx.x * CS_X + tx) * V;
+	const bool live = col < cols;
 	const int slab = blockIdx.y;
 	const int r0 = slab * rows_per_slab;
 	const int r1 = min(rows, r0 + rows_per_slab);
-	float c[V], d[V];
-	ldv<V>(c, vr + col);
-	ldv<V>(d, vi + col);
 	float acc[4][V];
 #pragma unroll
 	for (int p = 0; p < 4; ++p)
 #pragma unroll
 		for (int k = 0; k < V; ++k) acc[p][k] = 0.f;
-	for (int row = r0; row < r1; ++row) {
-		float a[V], b[V], gr[V], gi[V], sr[V], si[V], o[V];
-		ldv<V>(a, ur + (long) row * ldu + col);
-		ldv<V>(b, ui + (long) row * ldu + col);
-		ldv<V>(gr, g.dz_re + (long) row * ldg + col);
-		ldv<V>(gi, g.dz_im + (long) row * ldg + col);
-		ldv<V>(sr, g.dzs_re + (long) row * ldg + col);
-		ldv<V>(si, g.dzs_im + (long) row * ldg + col);
-		const long ou = (long) row * lddu + col;
+	if (live) {
+		float c[V], d[V];
+		ldv<V>(c, vr + col);
+		ldv<V>(d, vi + col);
+		for (int row = r0 + ty; row < r1; row += CS_Y) {
+			float a[V], b[V], gr[V], gi[V], sr[V], si[V], o[V];
+			ldv<V>(a, ur + (long) row * ldu + col);
+			ldv<V>(b, ui + (long) row * ldu + col);
+			ldv<V>(gr, g.dz_re + (long) row * ldg + col);
+			ldv<V>(gi, g.dz_im + (long) row * ldg + col);
+			ldv<V>(sr, g.dzs_re + (long) row * ldg + col);
+			ldv<V>(si, g.dzs_im + (long) row * ldg + col);
+			const long ou = (long) row * lddu + col;
 #pragma unroll
-		for (int k = 0; k < V; ++k) o[k] = gr[k] * c[k] - gi[k] * d[k];
-		outv<V>(du.dz_re + ou, o, accumulate);
+			for (int k = 0; k < V; ++k) o[k] = gr[k] * c[k] - gi[k] * d[k];
+			outv<V>(du.dz_re + ou, o, accumulate);
 #pragma unroll
-		for (int k = 0; k < V; ++k) o[k] = gr[k] * d[k] + gi[k] * c[k];
-		outv<V>(du.dz_im + ou, o, accumulate);
+			for (int k = 0; k < V; ++k) o[k] = gr[k] * d[k] + gi[k] * c[k];
+			outv<V>(du.dz_im + ou, o, accumulate);
 #pragma unroll
-		for (int k = 0; k < V; ++k) o[k] = sr[k] * c[k] + si[k] * d[k];
-		outv<V>(du.dzs_re + ou, o, accumulate);
+			for (int k = 0; k < V; ++k) o[k] = sr[k] * c[k] + si[k] * d[k];
+			outv<V>(du.dzs_re + ou, o, accumulate);
 #pragma unroll
-		for (int k = 0; k < V; ++k) o[k] = si[k] * c[k] - sr[k] * d[k];
-		outv<V>(du.dzs_im + ou, o, accumulate);
+			for (int k = 0; k < V; ++k) o[k] = si[k] * c[k] - sr[k] * d[k];
+			outv<V>(du.dzs_im + ou, o, accumulate);
 #pragma unroll
-		for (int k = 0; k < V; ++k) {
-			acc[0][k] += gr[k] * a[k] - gi[k] * b[k];
-			acc[1][k] += gr[k] * b[k] + gi[k] * a[k];
-			acc[2][k] += sr[k] * a[k] + si[k] * b[k];
-			acc[3][k] += si[k] * a[k] - sr[k] * b[k];
+			for (int k = 0; k < V; ++k) {
+				acc[0][k] += gr[k] * a[k] - gi[k] * b[k];
+				acc[1][k] += gr[k] * b[k] + gi[k] * a[k];
+				acc[2][k] += sr[k] * a[k] + si[k] * b[k];
+				acc[3][k] += si[k] * a[k] - sr[k] * b[k];
+			}
 		}
 	}
 #pragma unroll
-	for (int p = 0; p < 4; ++p) stv<V>(partial + ((long) slab * 4 + p) * cols + col, acc[p]);
+	for (int p = 0; p < 4; ++p)
+#pragma unroll
+		for (int k = 0; k < V; ++k) red[ty][p][tx * V + k] = acc[p][k];
+	__syncthreads();
+	if (ty == 0 && live) {
+#pragma unroll
+		for (int p = 0; p < 4; ++p) {
+			float t[V];
+#pragma unroll
+			for (int k = 0; k < V; ++k) t[k] = ((red[0][p][tx * V + k] + red[1][p][tx * V + k]) + red[2][p][tx * V + k]) + red[3][p][tx * V + k];
+			stv<V>(partial + ((long) slab * 4 + p) * cols + col, t);
+		}
+	}
 }
 
 // dst[p][c] (+)= sum over slabs of partial[slab][p][c], slabs added in index order.
@@ -469,13 +490,11 @@ int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const f
 		CNET_LAUNCH_CHECK();
 		return CNET_OK;
 	}
-	// shared parameter row: slabs of rows sized so that the grid covers the chip a few times over
+	// shared parameter row: slabs of rows sized so that the grid covers the chip about four times
 	const int V = vec ? 4 : 1;
-	const long col_blocks = ((long) cols / V + TPB - 1) / TPB;
-	const long want_blocks = 8L * rt().prop.multiProcessorCount;
-	int nslabs = (int) ((want_blocks + col_blocks - 1) / col_blocks);
-	if (nslabs > rows) nslabs = rows;
-	if (nslabs < 1) nslabs = 1;
+	const long col_blocks = ((long) cols / V + CS_X - 1) / CS_X;
+	int nslabs = (int) std::max(1L, std::min(256L, 4L * rt().prop.multiProcessorCount / col_blocks));
+	nslabs = std::min(nslabs, (rows + CS_Y - 1) / CS_Y);
 	const int rows_per_slab = (rows + nslabs - 1) / nslabs;
 	nslabs = (rows + rows_per_slab - 1) / rows_per_slab;
 	float *partial = (float *) workspace((size_t) nslabs * 4 * cols * sizeof(float));

@@ -9,6 +9,8 @@
 // scheduling.
 #include "common.hpp"
 
+#include <algorithm>
+
 namespace {
 
 constexpr int TPB = 256;
@@ -90,6 +92,23 @@ struct ArgMaxOp {
 		return a;
 	}
 };
+// the largest |z|^2 of a row with its first index, and the runner-up value (to detect near ties)
+struct Top2 {
+	double q1, q2;
+	int i1, pad;
+};
+struct Top2Op {
+	__device__ Top2 operator()(Top2 a, Top2 b) const {
+		Top2 r;
+		const bool b_wins = b.q1 > a.q1 || (b.q1 == a.q1 && b.i1 < a.i1);
+		const Top2 &w = b_wins ? b : a, &l = b_wins ? a : b;
+		r.q1 = w.q1;
+		r.i1 = w.i1;
+		r.q2 = fmax(w.q2, l.q1);
+		r.pad = 0;
+		return r;
+	}
+};
 struct Cplx4 {
 	float a, b, c, d;
 };
@@ -152,19 +171,61 @@ __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restri
 		float *__restrict__ loss, int *__restrict__ argmax, int rows, int cols) {
 	__shared__ double lds_d[TPB / 64];
 	__shared__ ArgMax lds_a[TPB / 64];
+	__shared__ Top2 lds_t[TPB / 64];
 	CNET_ROW_SETUP();
 	const float *pr = zr + (long) row * ldz, *pi = zi + (long) row * ldz;
-	double sum = row_accumulate<V, G, double>(pr, pi, cols, t,
-			[](float a, float b) { return (double) a * (double) a + (double) b * (double) b; });
+	// pass 1 (the only pass in the common case): sum |z|^2 in double, and the two largest |z_k|^2 of the row
+	double sum = 0.0;
+	Top2 top = {-1.0, -1.0, 0x7fffffff, 0};
+	auto visit = [&](float a, float b, int k) {
+		const double q = (double) a * (double) a + (double) b * (double) b;
+		sum += q;
+		if (q > top.q1) {
+			top.q2 = top.q1;
+			top.q1 = q;
+			top.i1 = k;
+		} else if (q > top.q2) {
+			top.q2 = q;
+		}
+	};
+	if (V == 4) {
+		for (int c = t * 4; c < cols; c += STRIDE * 4) {
+			float4 a = *reinterpret_cast<const float4 *>(pr + c);
+			float4 b = *reinterpret_cast<const float4 *>(pi + c);
+			visit(a.x, b.x, c);
+			visit(a.y, b.y, c + 1);
+			visit(a.z, b.z, c + 2);
+			visit(a.w, b.w, c + 3);
+		}
+	} else {
+		for (int c = t; c < cols; c += STRIDE) visit(pr[c], pi[c], c);
+	}
 	sum = group_reduce<double, G>(sum, SumD(), lds_d, slot, wig, lane);
+	top = group_reduce<Top2, G>(top, Top2Op(), lds_t, slot, wig, lane);
 	float S = (float) sum;
 	if (S <= 1.0e-15f) S = 1.0e-15f;
 	double nrm = sqrt((double) S);
 	if (nrm <= 1.0e-15) nrm = 1.0e-15;
 	const double inv = 1.0 / nrm;
+	const bool want_out = (outr != nullptr);
+	// The reference argmax is taken over p_k = fl(|fl(z_k / sqrt S)|^2), which orders like |z_k|^2 except within a few
+	// ulp.  When the runner-up is more than 1e-5 (relative) below the maximum the winner is already decided; otherwise,
+	// or when the normalised planes are wanted, a second pass evaluates p_k exactly as the reference does.
+	const bool clear_cut = top.q2 < top.q1 * (1.0 - 1.0e-5);
+	if (!want_out && clear_cut) {
+		if (live && t == 0) {
+			const int label = labels[row];
+			float o_r = (float) (pr[label] * inv), o_i = (float) (pi[label] * inv);
+			float p = (float) ((double) o_r * o_r + (double) o_i * o_i);
+			p = (p < 1e-15f ? 1e-15f : p);
+			s[row] = S;
+			loss[row] = -logf(p);
+			argmax[row] = top.i1;
+		}
+		return;
+	}
 
 	ArgMax best = {-1.0f, 0x7fffffff};
-	const bool want_out = (outr != nullptr);
 	float *qr = want_out ? outr + (long) row * ldo : nullptr;
 	float *qi = want_out ? outi + (long) row * ldo : nullptr;
 	if (V == 4) {
@@ -253,15 +314,31 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict
 		int accumulate) {
 	__shared__ Cplx4 lds_c[TPB / 64];
 	CNET_ROW_SETUP();
-	const long oz = (long) row * ldz, og = (long) row * ldg, od = (long) row * ldd;
+	const float *pzr = zr + (long) row * ldz, *pzi = zi + (long) row * ldz;
+	const float *pgr = g_re + (long) row * ldg, *pgi = g_im + (long) row * ldg;
+	const float *psr = gs_re + (long) row * ldg, *psi = gs_im + (long) row * ldg;
+	float *q0 = d_re + (long) row * ldd, *q1 = d_im + (long) row * ldd, *q2 = ds_re + (long) row * ldd, *q3 = ds_im + (long) row * ldd;
+	constexpr int W = V;  // columns per thread and step
 	Cplx4 acc = {0.f, 0.f, 0.f, 0.f};  // a,b: G z   c,d: Gs conj z
-	for (int c = t; c < cols; c += STRIDE) {
-		float a = zr[oz + c], b = zi[oz + c];
-		float gr = g_re[og + c], gi = g_im[og + c], sr = gs_re[og + c], si = gs_im[og + c];
-		acc.a += gr * a - gi * b;
-		acc.b += gr * b + gi * a;
-		acc.c += sr * a + si * b;
-		acc.d += si * a - sr * b;
+	for (int c = t * W; c < cols; c += STRIDE * W) {
+		float a[W], b[W], gr[W], gi[W], sr[W], si[W];
+		if (W == 4) {
+			*reinterpret_cast<float4 *>(a) = *reinterpret_cast<const float4 *>(pzr + c);
+			*reinterpret_cast<float4 *>(b) = *reinterpret_cast<const float4 *>(pzi + c);
+			*reinterpret_cast<float4 *>(gr) = *reinterpret_cast<const float4 *>(pgr + c);
+			*reinterpret_cast<float4 *>(gi) = *reinterpret_cast<const float4 *>(pgi + c);
+			*reinterpret_cast<float4 *>(sr) = *reinterpret_cast<const float4 *>(psr + c);
+			*reinterpret_cast<float4 *>(si) = *reinterpret_cast<const float4 *>(psi + c);
+		} else {
+			a[0] = pzr[c]; b[0] = pzi[c]; gr[0] = pgr[c]; gi[0] = pgi[c]; sr[0] = psr[c]; si[0] = psi[c];
+		}
+#pragma unroll
+		for (int k = 0; k < W; ++k) {
+			acc.a += gr[k] * a[k] - gi[k] * b[k];
+			acc.b += gr[k] * b[k] + gi[k] * a[k];
+			acc.c += sr[k] * a[k] + si[k] * b[k];
+			acc.d += si[k] * a[k] - sr[k] * b[k];
+		}
 	}
 	acc = group_reduce<Cplx4, G>(acc, SumC4(), lds_c, slot, wig, lane);
 	if (!live) return;
@@ -271,51 +348,80 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict
 	float cube = (float) (nrm * nrm * nrm);
 	const float inv = (float) (1.0 / nrm);
 	const float Ar = 0.5f * (acc.a + acc.c) / cube, Ai = 0.5f * (acc.b + acc.d) / cube;
-	for (int c = t; c < cols; c += STRIDE) {
-		float a = zr[oz + c], b = zi[oz + c];
-		float gr = g_re[og + c], gi = g_im[og + c], sr = gs_re[og + c], si = gs_im[og + c];
-		// conj(z) A = (a Ar + b Ai) + i (a Ai - b Ar) ;  z A = (a Ar - b Ai) + i (a Ai + b Ar)
-		float o0 = gr * inv - (a * Ar + b * Ai);
-		float o1 = gi * inv - (a * Ai - b * Ar);
-		float o2 = sr * inv - (a * Ar - b * Ai);
-		float o3 = si * inv - (a * Ai + b * Ar);
-		if (accumulate) {
-			o0 += d_re[od + c];
-			o1 += d_im[od + c];
-			o2 += ds_re[od + c];
-			o3 += ds_im[od + c];
+	for (int c = t * W; c < cols; c += STRIDE * W) {
+		float a[W], b[W], gr[W], gi[W], sr[W], si[W], o0[W], o1[W], o2[W], o3[W];
+		if (W == 4) {
+			*reinterpret_cast<float4 *>(a) = *reinterpret_cast<const float4 *>(pzr + c);
+			*reinterpret_cast<float4 *>(b) = *reinterpret_cast<const float4 *>(pzi + c);
+			*reinterpret_cast<float4 *>(gr) = *reinterpret_cast<const float4 *>(pgr + c);
+			*reinterpret_cast<float4 *>(gi) = *reinterpret_cast<const float4 *>(pgi + c);
+			*reinterpret_cast<float4 *>(sr) = *reinterpret_cast<const float4 *>(psr + c);
+			*reinterpret_cast<float4 *>(si) = *reinterpret_cast<const float4 *>(psi + c);
+		} else {
+			a[0] = pzr[c]; b[0] = pzi[c]; gr[0] = pgr[c]; gi[0] = pgi[c]; sr[0] = psr[c]; si[0] = psi[c];
 		}
-		d_re[od + c] = o0;
-		d_im[od + c] = o1;
-		ds_re[od + c] = o2;
-		ds_im[od + c] = o3;
+#pragma unroll
+		for (int k = 0; k < W; ++k) {
+			// conj(z) A = (a Ar + b Ai) + i (a Ai - b Ar) ;  z A = (a Ar - b Ai) + i (a Ai + b Ar)
+			o0[k] = gr[k] * inv - (a[k] * Ar + b[k] * Ai);
+			o1[k] = gi[k] * inv - (a[k] * Ai - b[k] * Ar);
+			o2[k] = sr[k] * inv - (a[k] * Ar - b[k] * Ai);
+			o3[k] = si[k] * inv - (a[k] * Ai + b[k] * Ar);
+			if (accumulate) {
+				o0[k] += q0[c + k];
+				o1[k] += q1[c + k];
+				o2[k] += q2[c + k];
+				o3[k] += q3[c + k];
+			}
+		}
+		if (W == 4) {
+			*reinterpret_cast<float4 *>(q0 + c) = *reinterpret_cast<float4 *>(o0);
+			*reinterpret_cast<float4 *>(q1 + c) = *reinterpret_cast<float4 *>(o1);
+			*reinterpret_cast<float4 *>(q2 + c) = *reinterpret_cast<float4 *>(o2);
+			*reinterpret_cast<float4 *>(q3 + c) = *reinterpret_cast<float4 *>(o3);
+		} else {
+			q0[c] = o0[0]; q1[c] = o1[0]; q2[c] = o2[0]; q3[c] = o3[0];
+		}
 	}
 }
 
 // ---------------------------------------------------------------------------------------------- batch (column) sum
-// stage 1: blockIdx.y = slab of rows; thread = V columns; partial[slab][cols]
+// stage 1: workgroup = 64 column groups (V columns each) x 4 row lanes, blockIdx.y = slab of rows; the four row lanes
+// are added through LDS in lane order; partial[slab][cols]
+constexpr int CS_X = 64, CS_Y = 4;
+
 template <int V>
 __global__ __launch_bounds__(TPB) void colsum_partial_kernel(const float *__restrict__ src, long ld, float *__restrict__ partial,
 		int rows, int cols, int rows_per_slab) {
-	const long col = ((long) blockIdx.x * TPB + threadIdx.x) * V;
-	if (col >= cols) return;
+	__shared__ float red[CS_Y][CS_X * V];
+	const int tx = threadIdx.x % CS_X, ty = threadIdx.x / CS_X;
+	const long col = ((long) blockIdx.x * CS_X + tx) * V;
+	const bool live = col < cols;
 	const int r0 = blockIdx.y * rows_per_slab, r1 = min(rows, r0 + rows_per_slab);
 	float acc[V];
 #pragma unroll
 	for (int k = 0; k < V; ++k) acc[k] = 0.f;
-	for (int r = r0; r < r1; ++r) {
-		if (V == 4) {
-			float4 v = *reinterpret_cast<const float4 *>(src + (long) r * ld + col);
-			acc[0] += v.x;
-			acc[1 % V] += v.y;
-			acc[2 % V] += v.z;
-			acc[3 % V] += v.w;
-		} else {
-			acc[0] += src[(long) r * ld + col];
+	if (live) {
+		for (int r = r0 + ty; r < r1; r += CS_Y) {
+			if (V == 4) {
+				float4 v = *reinterpret_cast<const float4 *>(src + (long) r * ld + col);
+				acc[0] += v.x;
+				acc[1 % V] += v.y;
+				acc[2 % V] += v.z;
+				acc[3 % V] += v.w;
+			} else {
+				acc[0] += src[(long) r * ld + col];
+			}
 		}
 	}
 #pragma unroll
-	for (int k = 0; k < V; ++k) partial[(long) blockIdx.y * cols + col + k] = acc[k];
+	for (int k = 0; k < V; ++k) red[ty][tx * V + k] = acc[k];
+	__syncthreads();
+	if (ty == 0 && live) {
+#pragma unroll
+		for (int k = 0; k < V; ++k)
+			partial[(long) blockIdx.y * cols + col + k] = ((red[0][tx * V + k] + red[1][tx * V + k]) + red[2][tx * V + k]) + red[3][tx * V + k];
+	}
 }
 
 __global__ __launch_bounds__(TPB) void colsum_final_kernel(const float *__restrict__ partial, int nslabs, int cols,
@@ -395,7 +501,10 @@ int cnet_l2norm_bwd(const float *z_re, const float *z_im, int64_t ldz, const flo
 	if (!rows) return CNET_OK;
 	CNET_CHECK_ARG(z_re && z_im && s && g_dz_re && g_dz_im && g_dzs_re && g_dzs_im);
 	CNET_CHECK_ARG(dz_dz_re && dz_dz_im && dz_dzs_re && dz_dzs_im && ldz >= cols && ldg >= cols && lddz >= cols);
-	CNET_ROW_LAUNCH(l2norm_bwd_kernel, false, z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg, dz_dz_re,
+	const bool vec = mult4(cols, ldz, ldg, lddz) && aligned16(z_re) && aligned16(z_im) && aligned16(g_dz_re) && aligned16(g_dz_im) &&
+			aligned16(g_dzs_re) && aligned16(g_dzs_im) && aligned16(dz_dz_re) && aligned16(dz_dz_im) && aligned16(dz_dzs_re) &&
+			aligned16(dz_dzs_im);
+	CNET_ROW_LAUNCH(l2norm_bwd_kernel, vec, z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg, dz_dz_re,
 			dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate);
 	return CNET_OK;
 }
@@ -407,10 +516,9 @@ int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols
 	CNET_CHECK_ARG(src && dst && lds >= cols);
 	const bool vec = mult4(cols, lds) && aligned16(src);
 	const int V = vec ? 4 : 1;
-	const long col_blocks = ((long) cols / V + TPB - 1) / TPB;
-	const long want_blocks = 8L * rt().prop.multiProcessorCount;
-	int nslabs = (int) ((want_blocks + col_blocks - 1) / col_blocks);
-	if (nslabs > rows) nslabs = rows;
+	const long col_blocks = ((long) cols / V + CS_X - 1) / CS_X;
+	int nslabs = (int) std::max(1L, std::min(256L, 4L * rt().prop.multiProcessorCount / col_blocks));
+	nslabs = std::min(nslabs, (rows + CS_Y - 1) / CS_Y);
 	const int rows_per_slab = (rows + nslabs - 1) / nslabs;
 	nslabs = (rows + rows_per_slab - 1) / rows_per_slab;
 	float *partial = (float *) workspace((size_t) nslabs * cols * sizeof(float));
