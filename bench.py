@@ -20,6 +20,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X published dense fp32 matrix peak
+# Bytes the eight L2s exchanged with the fabric per launch (FETCH_SIZE + WRITE_SIZE of `rocprofv3 --pmc`, each scaled by
+# what the same counter reads for a 256 MiB copy kernel: x2.000 and x1.000); an upper bound on HBM traffic, since hits
+# in the memory-side cache are included.  Source: profiles/cgemm_linear_b4096_1024x1024_counters.md.
+MEASURED_TRAFFIC_BYTES = {"linear_fwd": 139261607, "linear_bwd_input": 242998234, "linear_bwd_weight": 386294002}
 B, K, N = 4096, 1024, 1024      # BASELINE.json configs[1]
 
 
@@ -268,11 +272,8 @@ def main():
         fl = 8.0 * B * N * K * ngemm
         kern[name] = {"ms": round(ms, 4), "flops": fl, "tflops": round(fl / ms / 1e9, 2)}
     dom = max(kern, key=lambda k: kern[k]["ms"])
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "cgemm_traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(dom)
-    roofline = {"bound": "mfma", "kernel": "cgemm_kernel (%s)" % dom, "achieved": kern[dom]["tflops"],
+    traffic = MEASURED_TRAFFIC_BYTES.get(dom)
+    roofline = {"bound": "mfma", "kernel": "cgemm_fast_kernel (%s)" % dom, "achieved": kern[dom]["tflops"],
                 "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(kern[dom]["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": traffic,
                 "flops_per_launch": kern[dom]["flops"], "avg_launch_ms": kern[dom]["ms"],
