@@ -186,6 +186,35 @@ def kernel_suite(steps):
         print(json.dumps(ln))
 
 
+def token_model_suite(steps):
+    """Fifth configuration at full size: batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096; forward + backward."""
+    from cnet_amd import capi
+    from cnet_amd.workloads import TokenModel
+    from oracle import binding as ob
+    capi.init(0)
+    gen = ob.load_port()
+    Bq, S, D, H, V = 16, 512, 1024, 4096, 32768
+    P = {"table": gen.normal(1, (2, V, D)), "gate": gen.normal(2, (2, D), 0, 0.05),
+         "w1": gen.normal(3, (2, H, D), 0, D ** -0.5), "w2": gen.normal(4, (2, D, H), 0, H ** -0.5),
+         "w3": gen.normal(5, (2, V, D), 0, D ** -0.5)}
+    model = TokenModel(Bq, S, D, H, V, P).set_tokens(gen.randint(6, (Bq, S), V))
+    ev = HipEvents(capi.load().cnet_stream())
+    for _ in range(2):
+        model.forward(); model.backward()
+    capi.sync()
+    a, b = ev.event(), ev.event()
+    ev.record(a)
+    for _ in range(steps):
+        model.forward(); model.backward()
+    ev.record(b)
+    ms = ev.elapsed_ms(a, b) / steps
+    loss = float(model.loss.download().mean())
+    print(json.dumps({"workload": "configs[4]: complex token model fwd+bwd, batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096",
+                      "ms_per_step": round(ms, 3), "tokens_per_sec": round(Bq * S / ms * 1e3, 1),
+                      "gemm_tflops": round(model.gemm_flops() / ms / 1e9, 2), "mean_loss": round(loss, 4),
+                      "loss_of_uniform_guess": round(float(np.log(V)), 4)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -195,7 +224,7 @@ def main():
     ap.add_argument("--counter-pass", action="store_true",
                     help="short run for `rocprofv3 --pmc`: 3 launches of each GEMM kernel plus a plain copy kernel of "
                          "known size (256 MiB read, 256 MiB written) that calibrates FETCH_SIZE / WRITE_SIZE")
-    ap.add_argument("--suite", choices=["linear", "kernels"], default="linear",
+    ap.add_argument("--suite", choices=["linear", "kernels", "token_model"], default="linear",
                     help="linear (default): the headline line.  kernels: one line per other kernel of the hot path")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -204,6 +233,9 @@ def main():
 
     if args.suite == "kernels":
         kernel_suite(max(args.steps // 5, 10))
+        return
+    if args.suite == "token_model":
+        token_model_suite(max(args.steps // 20, 3))
         return
 
     from cnet_amd import capi, ops

@@ -31,6 +31,7 @@ SIGNATURES = {
     "cnet_memcpy_d2d": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_memset_zero": [C.c_void_p, C.c_size_t],
     "cnet_cgemm": [_i, _i, _i, _i, _i, _i, c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, _i],
+    "cnet_cgemm_batched": [_i, _i, _i, _i, _i, _i, _i, c_fp, c_fp, _l, _l, c_fp, c_fp, _l, _l, c_fp, c_fp, _l, _l, _i, _i],
     "cnet_clinear_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i, _i, _i],
     "cnet_clinear_bwd_input": [c_fp] * 4 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
     "cnet_clinear_bwd_weight": [c_fp] * 4 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],

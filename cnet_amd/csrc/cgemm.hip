@@ -37,6 +37,7 @@ constexpr int NUM_XCD = 8;
 struct CgemmProblem {
 	const float *a_re, *a_im, *b_re, *b_im;
 	float *c_re, *c_im;
+	float a_im_sign;  // -1: multiply by conj(A)
 	float b_im_sign;  // -1: multiply by conj(B)
 };
 
@@ -46,7 +47,18 @@ struct CgemmArgs {
 	long lda, ldb, ldc;
 	int accumulate;
 	int tiles_m, tiles_n;
+	long stride_a, stride_b, stride_c;  // element strides between the matrices of a strided batch (blockIdx.z)
 };
+
+__device__ __forceinline__ void batch_offset(CgemmProblem &pb, const CgemmArgs &args) {
+	const long z = blockIdx.z;
+	pb.a_re += z * args.stride_a;
+	pb.a_im += z * args.stride_a;
+	pb.b_re += z * args.stride_b;
+	pb.b_im += z * args.stride_b;
+	pb.c_re += z * args.stride_c;
+	pb.c_im += z * args.stride_c;
+}
 
 __device__ __forceinline__ float keep(float v, unsigned mask) { return __uint_as_float(__float_as_uint(v) & mask); }
 
@@ -159,7 +171,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 	constexpr int STAGE_FLOATS = 2 * A_PLANE + 2 * B_PLANE;
 	extern __shared__ float smem[];
 
-	const CgemmProblem pb = args.p[blockIdx.y];
+	CgemmProblem pb = args.p[blockIdx.y];
+	batch_offset(pb, args);
 	const int M = args.M, N = args.N, K = args.K;
 
 	// ---- which block of C
@@ -197,7 +210,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 	const int nchunks = (K + KC - 1) / KC;
 	sa.load(pb.a_re, pb.a_im, m0, 0, M, K, args.lda);
 	sb.load(pb.b_re, pb.b_im, n0, 0, N, K, args.ldb);
-	sa.template store<PA>(smem, smem + A_PLANE, 1.0f);
+	sa.template store<PA>(smem, smem + A_PLANE, pb.a_im_sign);
 	sb.template store<PB>(smem + 2 * A_PLANE, smem + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
 	__syncthreads();
 
@@ -237,7 +250,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 			if (ks + 1 < KC / 2) fetch(cur, ks + 1, cs ^ 1);
 			if (ks == KC / 2 - 2) {
 				if (more) {
-					sa.template store<PA>(nxt, nxt + A_PLANE, 1.0f);
+					sa.template store<PA>(nxt, nxt + A_PLANE, pb.a_im_sign);
 					sb.template store<PB>(nxt + 2 * A_PLANE, nxt + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
 				}
 				__syncthreads();
@@ -361,7 +374,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_fast_kernel(const CgemmArgs
 	constexpr bool SCHED_RECIPE = CNET_SCHED_RECIPE;
 	extern __shared__ float smem[];
 
-	const CgemmProblem pb = args.p[blockIdx.y];
+	CgemmProblem pb = args.p[blockIdx.y];
+	batch_offset(pb, args);
 	const int K = args.K;
 
 	int pid = blockIdx.x;
@@ -413,7 +427,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_fast_kernel(const CgemmArgs
 	};
 	auto store_unit = [&](int idx, float *stage) {
 		if (idx < UA)
-			sa.template store_unit<PA>(idx, stage, stage + A_PLANE, 1.0f);
+			sa.template store_unit<PA>(idx, stage, stage + A_PLANE, pb.a_im_sign);
 		else
 			sb.template store_unit<PB>(idx - UA, stage + 2 * A_PLANE, stage + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
 	};
@@ -514,12 +528,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_fast_kernel(const CgemmArgs
 }
 
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
-int launch(const CgemmArgs &proto, int nprob) {
+int launch(const CgemmArgs &proto, int nprob, int batch) {
 	CgemmArgs args = proto;
 	args.tiles_m = (args.M + BM - 1) / BM;
 	args.tiles_n = (args.N + BN - 1) / BN;
 	constexpr size_t smem = 2 * (size_t) (2 * KC * (BM + 4) + 2 * KC * (BN + 4)) * sizeof(float);
-	dim3 grid(args.tiles_m * args.tiles_n, nprob);
+	dim3 grid(args.tiles_m * args.tiles_n, nprob, batch);
 	if constexpr (VEC == 4) {
 		if (args.M % BM == 0 && args.N % BN == 0 && args.K % KC == 0) {
 			auto fast = cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG>;
@@ -547,31 +561,31 @@ int launch(const CgemmArgs &proto, int nprob) {
 }
 
 template <bool A_MCONTIG, bool B_NCONTIG, int VEC>
-int pick_tile(const CgemmArgs &a, int nprob) {
+int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 	const long cus = cnet::rt().prop.multiProcessorCount;
-	auto blocks = [&](int bm, int bn) { return (long) ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * nprob; };
+	auto blocks = [&](int bm, int bn) { return (long) ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * nprob * batch; };
 	// the scalar-load fallback (odd shapes) keeps to the small block: its address arithmetic would spill otherwise
 	if constexpr (VEC == 1) {
-		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 	} else {
 		// tuning override: CNET_CGEMM_TILE = 0 (128x128), 1 (64x128), 2 (128x64), 3 (64x64)
 		static const int forced = [] {
 			const char *e = getenv("CNET_CGEMM_TILE");
 			return e ? atoi(e) : -1;
 		}();
-		if (forced == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
-		if (forced == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
-		if (forced == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
-		if (forced == 3) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		if (forced == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+		if (forced == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+		if (forced == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+		if (forced == 3) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 		// The largest block that still gives every compute unit TWO workgroups (two wavefronts per SIMD: one issues
 		// MFMAs while the other waits at its barrier or moves data); failing that, one workgroup per compute unit.
 		for (long want = 2 * cus; want >= cus; want -= cus) {
-			if (blocks(128, 128) >= want) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
-			if (blocks(64, 128) >= want) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
-			if (blocks(128, 64) >= want) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
-			if (blocks(64, 64) >= want) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+			if (blocks(128, 128) >= want) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+			if (blocks(64, 128) >= want) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+			if (blocks(128, 64) >= want) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+			if (blocks(64, 64) >= want) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 		}
-		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob);
+		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 	}
 }
 
@@ -580,24 +594,24 @@ int pick_tile(const CgemmArgs &a, int nprob) {
 namespace cnet {
 
 // nprob = 1 or 2 problems of identical shape.
-static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int nprob) {
+static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int nprob, int batch) {
 	if (a.M <= 0 || a.N <= 0) return CNET_OK;
 	if (a.K <= 0) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: K must be positive");
 	// float4 path: every contiguous run starts 16-byte aligned and has a length that is a multiple of 4
-	bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0);
+	bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (a.stride_a % 4 == 0) && (a.stride_b % 4 == 0);
 	vec = vec && (a_mcontig ? a.M % 4 == 0 : a.K % 4 == 0) && (b_ncontig ? a.N % 4 == 0 : a.K % 4 == 0);
 	for (int q = 0; q < nprob; ++q)
 		vec = vec && aligned16(a.p[q].a_re) && aligned16(a.p[q].a_im) && aligned16(a.p[q].b_re) && aligned16(a.p[q].b_im);
 	if (vec) {
-		if (!a_mcontig && !b_ncontig) return pick_tile<false, false, 4>(a, nprob);
-		if (!a_mcontig && b_ncontig) return pick_tile<false, true, 4>(a, nprob);
-		if (a_mcontig && b_ncontig) return pick_tile<true, true, 4>(a, nprob);
-		return pick_tile<true, false, 4>(a, nprob);
+		if (!a_mcontig && !b_ncontig) return pick_tile<false, false, 4>(a, nprob, batch);
+		if (!a_mcontig && b_ncontig) return pick_tile<false, true, 4>(a, nprob, batch);
+		if (a_mcontig && b_ncontig) return pick_tile<true, true, 4>(a, nprob, batch);
+		return pick_tile<true, false, 4>(a, nprob, batch);
 	}
-	if (!a_mcontig && !b_ncontig) return pick_tile<false, false, 1>(a, nprob);
-	if (!a_mcontig && b_ncontig) return pick_tile<false, true, 1>(a, nprob);
-	if (a_mcontig && b_ncontig) return pick_tile<true, true, 1>(a, nprob);
-	return pick_tile<true, false, 1>(a, nprob);
+	if (!a_mcontig && !b_ncontig) return pick_tile<false, false, 1>(a, nprob, batch);
+	if (!a_mcontig && b_ncontig) return pick_tile<false, true, 1>(a, nprob, batch);
+	if (a_mcontig && b_ncontig) return pick_tile<true, true, 1>(a, nprob, batch);
+	return pick_tile<true, false, 1>(a, nprob, batch);
 }
 
 // Used by cdft.hip
@@ -612,6 +626,7 @@ int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, c
 		a.p[q].b_im = b_im[q];
 		a.p[q].c_re = c_re[q];
 		a.p[q].c_im = c_im[q];
+		a.p[q].a_im_sign = 1.0f;
 		a.p[q].b_im_sign = conj_b[q] ? -1.0f : 1.0f;
 	}
 	if (nprob == 1) a.p[1] = a.p[0];
@@ -623,7 +638,8 @@ int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, c
 	a.ldc = ldc;
 	a.accumulate = accumulate;
 	a.tiles_m = a.tiles_n = 0;
-	return cgemm_dispatch(a_mcontig, b_ncontig, a, nprob);
+	a.stride_a = a.stride_b = a.stride_c = 0;
+	return cgemm_dispatch(a_mcontig, b_ncontig, a, nprob, 1);
 }
 
 }  // namespace cnet
@@ -644,6 +660,39 @@ int cnet_cgemm(int a_kmajor, int b_kmajor, int conj_b, int M, int N, int K, cons
 	float *cr[2] = {c_re, c_re}, *ci[2] = {c_im, c_im};
 	bool cj[2] = {conj_b != 0, conj_b != 0};
 	return cgemm_pair(a_kmajor != 0, b_kmajor != 0, 1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, accumulate);
+}
+
+int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M, int N, int K, const float *a_re,
+		const float *a_im, int64_t lda, int64_t stride_a, const float *b_re, const float *b_im, int64_t ldb, int64_t stride_b,
+		float *c_re, float *c_im, int64_t ldc, int64_t stride_c, int batch, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(M >= 0 && N >= 0 && K > 0 && batch >= 0 && batch <= 65535);
+	if (M == 0 || N == 0 || batch == 0) return CNET_OK;
+	CNET_CHECK_ARG(a_re && a_im && b_re && b_im && c_re && c_im);
+	CNET_CHECK_ARG(lda >= (a_kmajor ? M : K) && ldb >= (b_kmajor ? N : K) && ldc >= N);
+	CNET_CHECK_ARG(stride_a >= 0 && stride_b >= 0 && (batch == 1 || stride_c >= (int64_t) M * ldc - (ldc - N)));
+	CgemmArgs a;
+	a.p[0].a_re = a_re;
+	a.p[0].a_im = a_im;
+	a.p[0].b_re = b_re;
+	a.p[0].b_im = b_im;
+	a.p[0].c_re = c_re;
+	a.p[0].c_im = c_im;
+	a.p[0].a_im_sign = conj_a ? -1.0f : 1.0f;
+	a.p[0].b_im_sign = conj_b ? -1.0f : 1.0f;
+	a.p[1] = a.p[0];
+	a.M = M;
+	a.N = N;
+	a.K = K;
+	a.lda = lda;
+	a.ldb = ldb;
+	a.ldc = ldc;
+	a.accumulate = accumulate;
+	a.tiles_m = a.tiles_n = 0;
+	a.stride_a = stride_a;
+	a.stride_b = stride_b;
+	a.stride_c = stride_c;
+	return cgemm_dispatch(a_kmajor != 0, b_kmajor != 0, a, 1, batch);
 }
 
 int cnet_clinear_fwd(const float *x_re, const float *x_im, int64_t ldx, const float *w_re, const float *w_im,

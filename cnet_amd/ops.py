@@ -98,6 +98,12 @@ def cgemm(A, Bm, Cm, M, N, K, a_kmajor=0, b_kmajor=0, conj_b=0, accumulate=0):
     call("cnet_cgemm", a_kmajor, b_kmajor, conj_b, M, N, K, *A.p(), A.ld, *Bm.p(), Bm.ld, *Cm.p(), Cm.ld, accumulate)
 
 
+def cgemm_batched(A, stride_a, Bm, stride_b, Cm, stride_c, M, N, K, batch, a_kmajor=0, b_kmajor=0, conj_a=0, conj_b=0,
+                  accumulate=0):
+    call("cnet_cgemm_batched", a_kmajor, b_kmajor, conj_a, conj_b, M, N, K, *A.p(), A.ld, stride_a, *Bm.p(), Bm.ld, stride_b,
+         *Cm.p(), Cm.ld, stride_c, batch, accumulate)
+
+
 def linear_fwd(x, w, y, accumulate=0):
     call("cnet_clinear_fwd", *x.p(), x.ld, *w.p(), w.ld, *y.p(), y.ld, x.rows, x.cols, w.rows, accumulate)
 

@@ -76,6 +76,14 @@ int cnet_cgemm(int a_kmajor, int b_kmajor, int conj_b, int M, int N, int K,
                const float *b_re, const float *b_im, int64_t ldb,
                float *c_re, float *c_im, int64_t ldc, int accumulate);
 
+/* Strided batch of the same product: matrix z of the batch starts z * stride_x elements after matrix 0 (stride 0 = the
+ * operand is shared by the whole batch); conj_a != 0 uses conj(A).  Used for a transform applied along an inner axis,
+ * e.g. a DFT along the sequence axis of [batch][seq][dim] activations: C_z = F * X_z and, backwards, conj(F) * G*_z. */
+int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M, int N, int K,
+                       const float *a_re, const float *a_im, int64_t lda, int64_t stride_a,
+                       const float *b_re, const float *b_im, int64_t ldb, int64_t stride_b,
+                       float *c_re, float *c_im, int64_t ldc, int64_t stride_c, int batch, int accumulate);
+
 /* ---- Linear: replaces LinearGpu::gpu_linear_forward / gpu_linear_backward
  *      (gpu/reduce.cpp:56-77,532-604; gpu/reducegrad.cpp:20-44,288-322), CPU twin impl/linear.h:51-110.
  * x[B][K], w[N][K] (stored once), y[B][N].   y = x * w^T */
