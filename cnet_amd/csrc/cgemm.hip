@@ -304,35 +304,45 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 
 // ---------------------------------------------------------------------------------------------------------------
 // Fast path: M % BM == 0, N % BN == 0, K % KC == 0, 128-bit aligned operands.  Same decomposition as cgemm_kernel,
-// with the per-chunk overhead taken out of the vector ALU:
-//   * global addresses are "uniform tile base (SGPR, advanced with scalar adds) + per-thread 32-bit offset that never
+// with the per-chunk overhead taken out of the vector ALU and out of LDS:
+//   * global addresses are "uniform tile base (advanced with scalar adds) + per-thread 32-bit offset that never
 //     changes", so a chunk costs no address arithmetic in VGPRs and needs no edge masks;
 //   * LDS addresses are "per-thread base + stage toggle (one add per chunk) + immediate";
+//   * every operand goes to LDS with 128-bit writes and no transposition:
+//       - a source contiguous along its rows lands as [k][row] (pitch rows + 4) and is read one float per k pair;
+//       - a source contiguous along k lands as [row][16 k values], the four 16-byte groups of a row XOR-swizzled with
+//         bits 2..3 of the row, and is read back with 128-bit reads: lane (row r, half h) takes k group h for k steps
+//         0..3 and k group h + 2 for k steps 4..7.  Both the write (4 lanes cover one row) and the read (16 consecutive
+//         rows cover all 64 banks) are free of bank conflicts.
+//     The k order inside a chunk is therefore permuted: MFMA step s of half h multiplies k = 4h + s (s < 4) or
+//     k = 8 + 4h + (s - 4); the [k][row] operands are addressed with the same map, so the products pair up correctly.
 //   * the LDS writes of the next chunk are spread over the second half of the current chunk's MFMAs and the scheduler
 //     is told to interleave them (one MFMA, then a few VALU / DS instructions) so they issue in the shadow of the
 //     matrix pipe instead of stalling it.
 template <int ROWS, bool MCONTIG>
 struct FastStage {
 	static constexpr int UNITS = ROWS * KC / 4 / NTHREADS;
+	static constexpr int PITCH = MCONTIG ? ROWS + 4 : KC;      // floats per LDS line
+	static constexpr int PLANE = MCONTIG ? KC * PITCH : ROWS * KC;
 	unsigned goff[UNITS];  // byte offset of this thread's float4 inside the operand tile of a chunk
 	int soff[UNITS];       // float offset of its LDS destination inside a plane
 	float4 re[UNITS], im[UNITS];
 
-	__device__ __forceinline__ void init(long ld, int pitch) {
+	__device__ __forceinline__ void init(long ld) {
 #pragma unroll
 		for (int u = 0; u < UNITS; ++u) {
 			const int unit = threadIdx.x + u * NTHREADS;
-			int row, k;
 			if (MCONTIG) {
-				k = unit / (ROWS / 4);
-				row = (unit % (ROWS / 4)) * 4;
+				const int k = unit / (ROWS / 4);
+				const int row = (unit % (ROWS / 4)) * 4;
 				goff[u] = (unsigned) (((long) k * ld + row) * 4);
+				soff[u] = k * PITCH + row;
 			} else {
-				row = unit / (KC / 4);
-				k = (unit % (KC / 4)) * 4;
-				goff[u] = (unsigned) (((long) row * ld + k) * 4);
+				const int row = unit / (KC / 4);
+				const int kq = unit % (KC / 4);
+				goff[u] = (unsigned) (((long) row * ld + kq * 4) * 4);
+				soff[u] = row * KC + ((kq ^ ((row >> 2) & 3)) * 4);
 			}
-			soff[u] = k * pitch + row;
 		}
 	}
 	// tile_re / tile_im: uniform pointers to element (first row of the block, first k of the chunk)
@@ -340,32 +350,73 @@ struct FastStage {
 		re[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(tile_re) + goff[u]);
 		im[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(tile_im) + goff[u]);
 	}
-	template <int PITCH>
 	__device__ __forceinline__ void store_unit(int u, float *sre, float *sim, float im_sign) const {
-		const float4 a = re[u];
-		const float4 b = make_float4(im[u].x * im_sign, im[u].y * im_sign, im[u].z * im_sign, im[u].w * im_sign);
-		if (MCONTIG) {
-			*reinterpret_cast<float4 *>(sre + soff[u]) = a;
-			*reinterpret_cast<float4 *>(sim + soff[u]) = b;
-		} else {
-			sre[soff[u] + 0 * PITCH] = a.x;
-			sre[soff[u] + 1 * PITCH] = a.y;
-			sre[soff[u] + 2 * PITCH] = a.z;
-			sre[soff[u] + 3 * PITCH] = a.w;
-			sim[soff[u] + 0 * PITCH] = b.x;
-			sim[soff[u] + 1 * PITCH] = b.y;
-			sim[soff[u] + 2 * PITCH] = b.z;
-			sim[soff[u] + 3 * PITCH] = b.w;
-		}
+		// component-wise on purpose: an aggregate copy of re[u] keeps the array in scratch memory
+		*reinterpret_cast<float4 *>(sre + soff[u]) = make_float4(re[u].x, re[u].y, re[u].z, re[u].w);
+		*reinterpret_cast<float4 *>(sim + soff[u]) =
+				make_float4(im[u].x * im_sign, im[u].y * im_sign, im[u].z * im_sign, im[u].w * im_sign);
 	}
 };
 
+// Operand fragments of one wavefront: T tiles of 32 rows, both planes.
+//   MCONTIG ([k][row] in LDS): one float per tile, plane and k step, double buffered per step.
+//   otherwise ([row][k] swizzled): one float4 per tile, plane and half chunk (set 0: steps 0..3, set 1: steps 4..7).
+template <int T, bool MCONTIG, int PITCH, int PLANE>
+struct Frag {
+	float s_re[2][T], s_im[2][T];
+	float4 q_re[2][T], q_im[2][T];
+	const float *base0, *base1;  // per-lane LDS addresses inside stage 0, plane re
+
+	// w0: first row of the wavefront's sub-block; r = lane % 32, h = lane / 32
+	__device__ __forceinline__ void init(const float *plane_re, int w0, int r, int h) {
+		if (MCONTIG) {
+			base0 = plane_re + w0 + r + h * 4 * PITCH;
+			base1 = base0;
+		} else {
+			const int row = w0 + r;
+			const int sw = (row >> 2) & 3;
+			base0 = plane_re + row * KC + ((h ^ sw) * 4);
+			base1 = plane_re + row * KC + (((h + 2) ^ sw) * 4);
+		}
+	}
+	// [k][row] operands: values of k step s into slot s & 1
+	__device__ __forceinline__ void fetch_step(int stage_off, int s) {
+		if (MCONTIG) {
+			const float *b = base0 + stage_off;
+			const int line = (s < 4 ? s : s + 4) * PITCH;
+#pragma unroll
+			for (int i = 0; i < T; ++i) {
+				s_re[s & 1][i] = b[line + i * 32];
+				s_im[s & 1][i] = b[PLANE + line + i * 32];
+			}
+		}
+	}
+	// [row][k] operands: the four k values of half chunk `set`
+	__device__ __forceinline__ void fetch_set(int stage_off, int set) {
+		if (!MCONTIG) {
+			const float *b = (set ? base1 : base0) + stage_off;
+#pragma unroll
+			for (int i = 0; i < T; ++i) {
+				q_re[set][i] = *reinterpret_cast<const float4 *>(b + i * 32 * KC);
+				q_im[set][i] = *reinterpret_cast<const float4 *>(b + PLANE + i * 32 * KC);
+			}
+		}
+	}
+	static __device__ __forceinline__ float comp(const float4 &v, int c) { return c == 0 ? v.x : (c == 1 ? v.y : (c == 2 ? v.z : v.w)); }
+	__device__ __forceinline__ float re(int s, int i) const { return MCONTIG ? s_re[s & 1][i] : comp(q_re[s >> 2][i], s & 3); }
+	__device__ __forceinline__ float im(int s, int i) const { return MCONTIG ? s_im[s & 1][i] : comp(q_im[s >> 2][i], s & 3); }
+};
+
+// waves_per_eu(2, 4): LDS allows at most four workgroups per compute unit anyway, so the register allocator may use up to
+// 128 VGPRs for the small blocks instead of squeezing them (and spilling global loads to scratch) for an occupancy that
+// cannot materialise.
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG>
-__global__ __launch_bounds__(NTHREADS, 2) void cgemm_fast_kernel(const CgemmArgs args) {
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))) void cgemm_fast_kernel(const CgemmArgs args) {
 	static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per workgroup");
 	constexpr int TM = WM / 32, TN = WN / 32;
-	constexpr int PA = BM + 4, PB = BN + 4;
-	constexpr int A_PLANE = KC * PA, B_PLANE = KC * PB;
+	typedef FastStage<BM, A_MCONTIG> StageA;
+	typedef FastStage<BN, B_NCONTIG> StageB;
+	constexpr int A_PLANE = StageA::PLANE, B_PLANE = StageB::PLANE;
 	constexpr int STAGE_FLOATS = 2 * A_PLANE + 2 * B_PLANE;
 	constexpr int KS = KC / 2;  // k pairs (MFMA k extent = 2) per chunk
 #ifndef CNET_SCHED_RECIPE
@@ -406,11 +457,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_fast_kernel(const CgemmArgs
 				acc_im[i][j][e] = 0.f;
 			}
 
-	FastStage<BM, A_MCONTIG> sa;
-	FastStage<BN, B_NCONTIG> sb;
-	sa.init(args.lda, PA);
-	sb.init(args.ldb, PB);
-	constexpr int UA = FastStage<BM, A_MCONTIG>::UNITS, UB = FastStage<BN, B_NCONTIG>::UNITS, NU = UA + UB;
+	StageA sa;
+	StageB sb;
+	sa.init(args.lda);
+	sb.init(args.ldb);
+	constexpr int UA = StageA::UNITS, UB = StageB::UNITS, NU = UA + UB;
 
 	// uniform tile bases of chunk 0 and the per-chunk advance (elements)
 	const long a_tile0 = A_MCONTIG ? (long) m0 : (long) m0 * args.lda;
@@ -420,16 +471,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_fast_kernel(const CgemmArgs
 	const int nchunks = K / KC;
 
 	auto load_unit = [&](int idx, int chunk) {
+		// indices are clamped so that the branch not taken still addresses inside the register arrays (an out-of-range
+		// constant index would push them to scratch memory)
 		if (idx < UA)
-			sa.load_unit(idx, pb.a_re + a_tile0 + chunk * a_step, pb.a_im + a_tile0 + chunk * a_step);
+			sa.load_unit(idx < UA ? idx : 0, pb.a_re + a_tile0 + chunk * a_step, pb.a_im + a_tile0 + chunk * a_step);
 		else
-			sb.load_unit(idx - UA, pb.b_re + b_tile0 + chunk * b_step, pb.b_im + b_tile0 + chunk * b_step);
+			sb.load_unit(idx >= UA ? idx - UA : 0, pb.b_re + b_tile0 + chunk * b_step, pb.b_im + b_tile0 + chunk * b_step);
 	};
 	auto store_unit = [&](int idx, float *stage) {
 		if (idx < UA)
-			sa.template store_unit<PA>(idx, stage, stage + A_PLANE, pb.a_im_sign);
+			sa.store_unit(idx < UA ? idx : 0, stage, stage + A_PLANE, pb.a_im_sign);
 		else
-			sb.template store_unit<PB>(idx - UA, stage + 2 * A_PLANE, stage + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
+			sb.store_unit(idx >= UA ? idx - UA : 0, stage + 2 * A_PLANE, stage + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
 	};
 
 #pragma unroll
@@ -438,23 +491,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_fast_kernel(const CgemmArgs
 	for (int u = 0; u < NU; ++u) store_unit(u, smem);
 	__syncthreads();
 
-	float are[2][TM], aim[2][TM], anim[2][TM], bre[2][TN], bim[2][TN];
-	const float *frag_a = smem + wm0 + r + h * PA;                  // + stage + plane + k pair * 2 * PA + tile * 32
-	const float *frag_b = smem + 2 * A_PLANE + wn0 + r + h * PB;
-	auto fetch = [&](int stage_off, int ks, int slot) {
-		const float *fa = frag_a + stage_off, *fb = frag_b + stage_off;  // one add each; the rest are immediates
-#pragma unroll
-		for (int i = 0; i < TM; ++i) {
-			are[slot][i] = fa[ks * 2 * PA + i * 32];
-			aim[slot][i] = fa[A_PLANE + ks * 2 * PA + i * 32];
-		}
-#pragma unroll
-		for (int j = 0; j < TN; ++j) {
-			bre[slot][j] = fb[ks * 2 * PB + j * 32];
-			bim[slot][j] = fb[B_PLANE + ks * 2 * PB + j * 32];
-		}
-	};
-	fetch(0, 0, 0);
+	Frag<TM, A_MCONTIG, StageA::PITCH, A_PLANE> fa;
+	Frag<TN, B_NCONTIG, StageB::PITCH, B_PLANE> fb;
+	fa.init(smem, wm0, r, h);
+	fb.init(smem + 2 * A_PLANE, wn0, r, h);
+	fa.fetch_step(0, 0);
+	fb.fetch_step(0, 0);
+	fa.fetch_set(0, 0);
+	fb.fetch_set(0, 0);
 
 	for (int c = 0; c < nchunks; ++c) {
 		const int CUR = (c & 1) * STAGE_FLOATS, NXT = STAGE_FLOATS - CUR;
@@ -464,33 +508,53 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_fast_kernel(const CgemmArgs
 		for (int u = 0; u < NU; ++u) load_unit(u, next_chunk);
 #pragma unroll
 		for (int ks = 0; ks < KS; ++ks) {
-			const int cs = ks & 1;
-			if (ks + 1 < KS) fetch(CUR, ks + 1, cs ^ 1);
+			if (ks + 1 < KS) {
+				fa.fetch_step(CUR, ks + 1);
+				fb.fetch_step(CUR, ks + 1);
+			}
+			if (ks == 0) {  // second half of this chunk for the [row][k] operands
+				fa.fetch_set(CUR, 1);
+				fb.fetch_set(CUR, 1);
+			}
 			// the LDS writes of the next chunk ride on the MFMAs of the second half of this chunk
-			if (ks >= KS / 2) {
+			constexpr int SF = KS / 2;  // first k pair that carries LDS writes of the next chunk
+			if (ks >= SF) {
 #pragma unroll
 				for (int u = 0; u < NU; ++u)
-					if (KS / 2 + (u * (KS / 2)) / NU == ks) store_unit(u, smem + NXT);
+					if (SF + (u * (KS - SF)) / NU == ks) store_unit(u, smem + NXT);
 			}
 			if (ks == KS - 1) {
 				__syncthreads();
-				fetch(NXT, 0, cs ^ 1);
+				fa.fetch_step(NXT, 0);
+				fb.fetch_step(NXT, 0);
+				fa.fetch_set(NXT, 0);
+				fb.fetch_set(NXT, 0);
+			}
+			float are[TM], aim[TM], anim[TM], bre[TN], bim[TN];
+#pragma unroll
+			for (int i = 0; i < TM; ++i) {
+				are[i] = fa.re(ks, i);
+				aim[i] = fa.im(ks, i);
+				anim[i] = -aim[i];
 			}
 #pragma unroll
-			for (int i = 0; i < TM; ++i) anim[cs][i] = -aim[cs][i];
+			for (int j = 0; j < TN; ++j) {
+				bre[j] = fb.re(ks, j);
+				bim[j] = fb.im(ks, j);
+			}
 #pragma unroll
 			for (int i = 0; i < TM; ++i)
 #pragma unroll
 				for (int j = 0; j < TN; ++j) {
-					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[cs][i], bre[cs][j], acc_re[i][j], 0, 0, 0);
-					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[cs][i], bim[cs][j], acc_im[i][j], 0, 0, 0);
+					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bre[j], acc_re[i][j], 0, 0, 0);
+					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bim[j], acc_im[i][j], 0, 0, 0);
 				}
 #pragma unroll
 			for (int i = 0; i < TM; ++i)
 #pragma unroll
 				for (int j = 0; j < TN; ++j) {
-					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(anim[cs][i], bim[cs][j], acc_re[i][j], 0, 0, 0);
-					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aim[cs][i], bre[cs][j], acc_im[i][j], 0, 0, 0);
+					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(anim[i], bim[j], acc_re[i][j], 0, 0, 0);
+					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aim[i], bre[j], acc_im[i][j], 0, 0, 0);
 				}
 			if (SCHED_RECIPE && ks < KS - 1) {
 				// scheduling recipe for this k pair: after each MFMA let a few of the pending VALU / LDS / global
