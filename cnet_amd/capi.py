@@ -40,10 +40,15 @@ SIGNATURES = {
     "cnet_cdft_set_forward_matrix": [_i, C.c_void_p, C.c_void_p],
     "cnet_cdft_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i, _i],
     "cnet_cdft_bwd": [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_ctriang_dft_plan": [_i],
+    "cnet_ctriang_dft_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i, _i],
+    "cnet_ctriang_dft_bwd": [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_hadamard_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i],
     "cnet_hadamard_bwd": [c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_cgelu_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i],
     "cnet_cgelu_bwd": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_crelu_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i],
+    "cnet_crelu_bwd": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_residual_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i],
     "cnet_residual_bwd": [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_l2norm_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, _i, _i],
@@ -56,6 +61,7 @@ SIGNATURES = {
     "cnet_add2d": [c_fp, _l, c_fp, _l, _i, _i],
     "cnet_batch_sum": [c_fp, _l, c_fp, _i, _i, _i],
     "cnet_sgd_update": [c_fp, c_fp, c_fp, c_fp, _l, C.c_float, _i],
+    "cnet_adam_update": [c_fp] * 6 + [_l, C.c_float, C.c_float, _i, _i],
     "cnet_embedding_fwd": [c_fp, c_fp, _i, _i, c_fp, c_fp, c_fp, _l, _i, _i],
     "cnet_embedding_bwd": [c_fp, c_fp, c_fp, _l, c_fp, c_fp, _i, _i, _i, _i, _i],
     "cnet_last_error": [],

@@ -11,7 +11,7 @@ namespace cnet {
 
 int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
 		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
-		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate);
+		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri);
 
 struct Twiddle {
 	float *re = nullptr;
@@ -21,6 +21,10 @@ struct Twiddle {
 	// always uses the exact twiddles above, as the CPU path does (impl/ft.h:57-79 upstream)
 	float *fwd_re = nullptr;
 	float *fwd_im = nullptr;
+	// TriangFourier operator: T[i][o] = F[i][o] for i <= o, zero below the diagonal (impl/ft.h:151-156 upstream);
+	// built on first use
+	float *tri_re = nullptr;
+	float *tri_im = nullptr;
 };
 static std::map<int, Twiddle> g_twiddles;
 
@@ -28,18 +32,20 @@ void release_twiddles() {
 	for (auto &kv : g_twiddles) {
 		(void) hipFree(kv.second.re);  // one allocation holds both planes
 		if (kv.second.fwd_re) (void) hipFree(kv.second.fwd_re);
+		if (kv.second.tri_re) (void) hipFree(kv.second.tri_re);
 	}
 	g_twiddles.clear();
 }
 
-__global__ void twiddle_kernel(float *__restrict__ fre, float *__restrict__ fim, int n, long ld) {
+// upper_only: entries with p > q are written as zeros
+__global__ void twiddle_kernel(float *__restrict__ fre, float *__restrict__ fim, int n, long ld, int upper_only) {
 	const long idx = (long) blockIdx.x * blockDim.x + threadIdx.x;
 	if (idx >= (long) n * n) return;
 	const int p = (int) (idx / n), q = (int) (idx % n);
 	const long e = ((long) p * q) % n;
 	double s, c;
 	sincospi(-2.0 * (double) e / (double) n, &s, &c);
-	const double scale = 1.0 / sqrt((double) n);
+	const double scale = (upper_only && p > q) ? 0.0 : 1.0 / sqrt((double) n);
 	fre[(long) p * ld + q] = (float) (c * scale);
 	fim[(long) p * ld + q] = (float) (s * scale);
 }
@@ -58,10 +64,26 @@ static int get_plan(int n, Twiddle *out, bool create) {
 	t.im = t.re + plane;
 	if (t.ld != n) CNET_HIP(hipMemsetAsync(t.re, 0, 2 * plane * sizeof(float), rt().stream));
 	const long total = (long) n * n;
-	hipLaunchKernelGGL(twiddle_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, rt().stream, t.re, t.im, n, t.ld);
+	hipLaunchKernelGGL(twiddle_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, rt().stream, t.re, t.im, n, t.ld, 0);
 	CNET_LAUNCH_CHECK();
 	g_twiddles[n] = t;
 	*out = t;
+	return CNET_OK;
+}
+
+static int get_triangular(int n, Twiddle *out) {
+	int rc = get_plan(n, out, true);
+	if (rc || out->tri_re) return rc;
+	Twiddle &slot = g_twiddles[n];
+	const size_t plane = (size_t) n * slot.ld;
+	CNET_HIP(hipMalloc((void **) &slot.tri_re, 2 * plane * sizeof(float)));
+	slot.tri_im = slot.tri_re + plane;
+	if (slot.ld != n) CNET_HIP(hipMemsetAsync(slot.tri_re, 0, 2 * plane * sizeof(float), rt().stream));
+	const long total = (long) n * n;
+	hipLaunchKernelGGL(twiddle_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, rt().stream, slot.tri_re, slot.tri_im, n,
+			slot.ld, 1);
+	CNET_LAUNCH_CHECK();
+	*out = slot;
 	return CNET_OK;
 }
 
@@ -132,7 +154,7 @@ int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re
 	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {f_re, f_re}, *bi[2] = {f_im, f_im};
 	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate);
+	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate, 0);
 }
 
 int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
@@ -149,7 +171,48 @@ int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs
 	const float *ar[2] = {g_dz_re, g_dzs_re}, *ai[2] = {g_dz_im, g_dzs_im}, *br[2] = {t.re, t.re}, *bi[2] = {t.im, t.im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, true};
-	return cgemm_pair(false, true, 2, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate);
+	return cgemm_pair(false, true, 2, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 0);
+}
+
+int cnet_ctriang_dft_plan(int n) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(n > 0 && n <= 46340);
+	Twiddle t;
+	return get_triangular(n, &t);
+}
+
+// y_o = sum_{i <= o} x_i T[i][o] : T is stored [k = i][n = o]; the column block [n0, n0 + BN) needs k < n0 + BN only
+int cnet_ctriang_dft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy, int B, int n,
+		int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && n > 0 && n <= 46340);
+	if (B == 0) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= n && ldy >= n);
+	Twiddle t;
+	int rc = get_triangular(n, &t);
+	if (rc) return rc;
+	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {t.tri_re, t.tri_re}, *bi[2] = {t.tri_im, t.tri_im};
+	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
+	bool cj[2] = {false, false};
+	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate, 1);
+}
+
+// dz_i = sum_{o >= i} G_o T[i][o], dzs_i = sum_{o >= i} Gs_o conj(T[i][o])  (impl/ft.h:163-189 upstream): the same
+// planes read as [n = i][k = o], i.e. contiguous along the reduction index; the block of rows i >= n0 needs k >= n0 only
+int cnet_ctriang_dft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+		float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int B, int n, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && n > 0 && n <= 46340);
+	if (B == 0) return CNET_OK;
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && g_dzs_re && g_dzs_im && dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
+	CNET_CHECK_ARG(ldg >= n && lddx >= n);
+	Twiddle t;
+	int rc = get_triangular(n, &t);
+	if (rc) return rc;
+	const float *ar[2] = {g_dz_re, g_dzs_re}, *ai[2] = {g_dz_im, g_dzs_im}, *br[2] = {t.tri_re, t.tri_re}, *bi[2] = {t.tri_im, t.tri_im};
+	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
+	bool cj[2] = {false, true};
+	return cgemm_pair(false, false, 2, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 2);
 }
 
 }  // extern "C"

@@ -48,7 +48,19 @@ struct CgemmArgs {
 	int accumulate;
 	int tiles_m, tiles_n;
 	long stride_a, stride_b, stride_c;  // element strides between the matrices of a strided batch (blockIdx.z)
+	// Triangular B (square, zeros stored outside the triangle): 1 = B[k][n] is zero for k > n, 2 = zero for k < n.
+	// A block of columns [n0, n0 + BN) then only walks the K chunks that can hold non-zeros.
+	int tri;
 };
+
+// first chunk and one-past-last chunk of K for the block of columns starting at n0
+template <int BN>
+__device__ __forceinline__ void chunk_range(const CgemmArgs &args, int n0, int &c_lo, int &c_hi) {
+	c_lo = 0;
+	c_hi = (args.K + KC - 1) / KC;
+	if (args.tri == 1) c_hi = min(c_hi, (n0 + BN + KC - 1) / KC);
+	if (args.tri == 2) c_lo = n0 / KC;
+}
 
 __device__ __forceinline__ void batch_offset(CgemmProblem &pb, const CgemmArgs &args) {
 	const long z = blockIdx.z;
@@ -207,9 +219,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 	Stage<BM, A_MCONTIG, VEC> sa;
 	Stage<BN, B_NCONTIG, VEC> sb;
 
-	const int nchunks = (K + KC - 1) / KC;
-	sa.load(pb.a_re, pb.a_im, m0, 0, M, K, args.lda);
-	sb.load(pb.b_re, pb.b_im, n0, 0, N, K, args.ldb);
+	int c_lo, c_hi;
+	chunk_range<BN>(args, n0, c_lo, c_hi);
+	sa.load(pb.a_re, pb.a_im, m0, c_lo * KC, M, K, args.lda);
+	sb.load(pb.b_re, pb.b_im, n0, c_lo * KC, N, K, args.ldb);
 	sa.template store<PA>(smem, smem + A_PLANE, pb.a_im_sign);
 	sb.template store<PB>(smem + 2 * A_PLANE, smem + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
 	__syncthreads();
@@ -236,10 +249,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 	};
 	fetch(smem, 0, 0);
 
-	for (int c = 0; c < nchunks; ++c) {
-		const float *cur = smem + (c & 1) * STAGE_FLOATS;
-		float *nxt = smem + ((c + 1) & 1) * STAGE_FLOATS;
-		const bool more = (c + 1 < nchunks);
+	for (int c = c_lo; c < c_hi; ++c) {
+		const float *cur = smem + ((c - c_lo) & 1) * STAGE_FLOATS;
+		float *nxt = smem + ((c - c_lo + 1) & 1) * STAGE_FLOATS;
+		const bool more = (c + 1 < c_hi);
 		if (more) {
 			sa.load(pb.a_re, pb.a_im, m0, (c + 1) * KC, M, K, args.lda);
 			sb.load(pb.b_re, pb.b_im, n0, (c + 1) * KC, N, K, args.ldb);
@@ -468,7 +481,8 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	const long b_tile0 = B_NCONTIG ? (long) n0 : (long) n0 * args.ldb;
 	const long a_step = A_MCONTIG ? (long) KC * args.lda : (long) KC;
 	const long b_step = B_NCONTIG ? (long) KC * args.ldb : (long) KC;
-	const int nchunks = K / KC;
+	int c_lo, c_hi;
+	chunk_range<BN>(args, n0, c_lo, c_hi);
 
 	auto load_unit = [&](int idx, int chunk) {
 		// indices are clamped so that the branch not taken still addresses inside the register arrays (an out-of-range
@@ -486,7 +500,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	};
 
 #pragma unroll
-	for (int u = 0; u < NU; ++u) load_unit(u, 0);
+	for (int u = 0; u < NU; ++u) load_unit(u, c_lo);
 #pragma unroll
 	for (int u = 0; u < NU; ++u) store_unit(u, smem);
 	__syncthreads();
@@ -500,10 +514,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	fa.fetch_set(0, 0);
 	fb.fetch_set(0, 0);
 
-	for (int c = 0; c < nchunks; ++c) {
-		const int CUR = (c & 1) * STAGE_FLOATS, NXT = STAGE_FLOATS - CUR;
-		const bool more = (c + 1 < nchunks);
-		const int next_chunk = more ? c + 1 : 0;  // the last chunk re-reads chunk 0 (in bounds, never used)
+	for (int c = c_lo; c < c_hi; ++c) {
+		const int CUR = ((c - c_lo) & 1) * STAGE_FLOATS, NXT = STAGE_FLOATS - CUR;
+		const bool more = (c + 1 < c_hi);
+		const int next_chunk = more ? c + 1 : c_lo;  // the last chunk re-reads the first one (in bounds, never used)
 #pragma unroll
 		for (int u = 0; u < NU; ++u) load_unit(u, next_chunk);
 #pragma unroll
@@ -681,8 +695,10 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 // Used by cdft.hip
 int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
 		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
-		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate) {
+		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri) {
+	if (tri && N != K) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: a triangular operand must be square");
 	CgemmArgs a;
+	a.tri = tri;
 	for (int q = 0; q < nprob; ++q) {
 		a.p[q].a_re = a_re[q];
 		a.p[q].a_im = a_im[q];
@@ -723,7 +739,7 @@ int cnet_cgemm(int a_kmajor, int b_kmajor, int conj_b, int M, int N, int K, cons
 	const float *ar[2] = {a_re, a_re}, *ai[2] = {a_im, a_im}, *br[2] = {b_re, b_re}, *bi[2] = {b_im, b_im};
 	float *cr[2] = {c_re, c_re}, *ci[2] = {c_im, c_im};
 	bool cj[2] = {conj_b != 0, conj_b != 0};
-	return cgemm_pair(a_kmajor != 0, b_kmajor != 0, 1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, accumulate);
+	return cgemm_pair(a_kmajor != 0, b_kmajor != 0, 1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, accumulate, 0);
 }
 
 int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M, int N, int K, const float *a_re,
@@ -736,6 +752,7 @@ int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M
 	CNET_CHECK_ARG(lda >= (a_kmajor ? M : K) && ldb >= (b_kmajor ? N : K) && ldc >= N);
 	CNET_CHECK_ARG(stride_a >= 0 && stride_b >= 0 && (batch == 1 || stride_c >= (int64_t) M * ldc - (ldc - N)));
 	CgemmArgs a;
+	a.tri = 0;
 	a.p[0].a_re = a_re;
 	a.p[0].a_im = a_im;
 	a.p[0].b_re = b_re;
@@ -779,7 +796,7 @@ int cnet_clinear_bwd_input(const float *g_dz_re, const float *g_dz_im, const flo
 	const float *br[2] = {w_re, w_re}, *bi[2] = {w_im, w_im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, true};
-	return cgemm_pair(false, true, 2, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate);
+	return cgemm_pair(false, true, 2, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0);
 }
 
 int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,
@@ -796,7 +813,7 @@ int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const fl
 	const float *br[2] = {x_re, x_re}, *bi[2] = {x_im, x_im};
 	float *cr[2] = {dw_dz_re, dw_dzs_re}, *ci[2] = {dw_dz_im, dw_dzs_im};
 	bool cj[2] = {false, true};
-	return cgemm_pair(true, true, 2, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate);
+	return cgemm_pair(true, true, 2, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0);
 }
 
 }  // extern "C"

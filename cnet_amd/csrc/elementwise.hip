@@ -7,6 +7,7 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <cmath>
 
 namespace {
 
@@ -274,6 +275,44 @@ __global__ __launch_bounds__(TPB) void gelu_bwd_kernel(const float *__restrict__
 	outv<V>(dx.dzs_im + off, o, accumulate);
 }
 
+// ------------------------------------------------------------------------------------------------ CRelu
+// y = z where Re z > 0 and Im z > 0, else 0 (impl/relu.h:32-46 upstream); the gradients pass under the same test
+// (impl/relu.h:48-63).
+template <int V>
+__global__ __launch_bounds__(TPB) void crelu_fwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
+		float *__restrict__ yr, float *__restrict__ yi, long ldy, int rows, int cols) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V];
+	ldv<V>(a, xr + row * ldx + col);
+	ldv<V>(b, xi + row * ldx + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		const bool on = a[k] > 0.f && b[k] > 0.f;
+		a[k] = on ? a[k] : 0.f;
+		b[k] = on ? b[k] : 0.f;
+	}
+	stv<V>(yr + row * ldy + col, a);
+	stv<V>(yi + row * ldy + col, b);
+}
+
+template <int V>
+__global__ __launch_bounds__(TPB) void crelu_bwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
+		CGrad4 g, long ldg, Grad4 dx, long lddx, int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], o[V];
+	ldv<V>(a, xr + row * ldx + col);
+	ldv<V>(b, xi + row * ldx + col);
+	const float *src[4] = {g.dz_re, g.dz_im, g.dzs_re, g.dzs_im};
+	float *dst[4] = {dx.dz_re, dx.dz_im, dx.dzs_re, dx.dzs_im};
+#pragma unroll
+	for (int p = 0; p < 4; ++p) {
+		ldv<V>(o, src[p] + row * ldg + col);
+#pragma unroll
+		for (int k = 0; k < V; ++k) o[k] = (a[k] > 0.f && b[k] > 0.f) ? o[k] : 0.f;
+		outv<V>(dst[p] + row * lddx + col, o, accumulate);
+	}
+}
+
 // ------------------------------------------------------------------------------------------------ Residual
 template <int V>
 __global__ __launch_bounds__(TPB) void residual_fwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
@@ -392,6 +431,41 @@ __global__ __launch_bounds__(TPB) void sgd_kernel(float *__restrict__ zr, float 
 	}
 	stv<V>(zr + i, a);
 	stv<V>(zi + i, b);
+	if (zero_grad) {
+		stv<V>(dr + i, z);
+		stv<V>(di + i, z);
+	}
+}
+
+// m = beta m + (1 - beta) dzs ; z -= lr m / denom ; dzs = 0   (impl/cfunc.h:273-287, gpu/kernels.cpp:494-514 upstream).
+// denom = 1 - beta^(t+1) arrives as a double and the quotient is formed in double, as the CPU loop does
+// (pow(float, int) promotes), so the parameter gets one rounding per step.
+template <int V>
+__global__ __launch_bounds__(TPB) void adam_kernel(float *__restrict__ zr, float *__restrict__ zi, float *__restrict__ mr,
+		float *__restrict__ mi, float *__restrict__ dr, float *__restrict__ di, long n, float lr, float beta, double denom,
+		int zero_grad) {
+	const long i = ((long) blockIdx.x * TPB + threadIdx.x) * V;
+	if (i >= n) return;
+	float a[V], b[V], c[V], d[V], e[V], f[V], z[V];
+	ldv<V>(a, zr + i);
+	ldv<V>(b, zi + i);
+	ldv<V>(c, mr + i);
+	ldv<V>(d, mi + i);
+	ldv<V>(e, dr + i);
+	ldv<V>(f, di + i);
+	const float one_minus_beta = 1 - beta;
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		c[k] = c[k] * beta + one_minus_beta * e[k];
+		d[k] = d[k] * beta + one_minus_beta * f[k];
+		a[k] = (float) ((double) a[k] - (double) (lr * c[k]) / denom);
+		b[k] = (float) ((double) b[k] - (double) (lr * d[k]) / denom);
+		z[k] = 0.f;
+	}
+	stv<V>(zr + i, a);
+	stv<V>(zi + i, b);
+	stv<V>(mr + i, c);
+	stv<V>(mi + i, d);
 	if (zero_grad) {
 		stv<V>(dr + i, z);
 		stv<V>(di + i, z);
@@ -544,6 +618,38 @@ int cnet_cgelu_bwd(const float *x_re, const float *x_im, int64_t ldx, const floa
 	return CNET_OK;
 }
 
+int cnet_crelu_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= cols && ldy >= cols);
+	if (all_mult4({cols, ldx, ldy}) && all_aligned({x_re, x_im, y_re, y_im}))
+		hipLaunchKernelGGL(crelu_fwd_kernel<4>, CNET_GRID_2D(4), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+	else
+		hipLaunchKernelGGL(crelu_fwd_kernel<1>, CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_crelu_bwd(const float *x_re, const float *x_im, int64_t ldx, const float *g_dz_re, const float *g_dz_im,
+		const float *g_dzs_re, const float *g_dzs_im, int64_t ldg, float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re,
+		float *dx_dzs_im, int64_t lddx, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && g_dz_re && g_dz_im && g_dzs_re && g_dzs_im && dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
+	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
+	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
+	Grad4 dx = {dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im};
+	if (all_mult4({cols, ldx, ldg, lddx}) &&
+			all_aligned({x_re, x_im, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
+		hipLaunchKernelGGL(crelu_bwd_kernel<4>, CNET_GRID_2D(4), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+	else
+		hipLaunchKernelGGL(crelu_bwd_kernel<1>, CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
 int cnet_residual_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
 		float *y_re, float *y_im, int64_t ldy, int rows, int cols) {
 	CNET_REQUIRE_INIT();
@@ -640,6 +746,24 @@ int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int6
 		hipLaunchKernelGGL(sgd_kernel<4>, dim3(nblocks(n / 4)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
 	else
 		hipLaunchKernelGGL(sgd_kernel<1>, dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_adam_update(float *z_re, float *z_im, float *m_re, float *m_im, float *dzs_re, float *dzs_im, int64_t n, float lr,
+		float beta, int t, int zero_grad) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(n >= 0 && t >= 0);
+	if (!n) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && m_re && m_im && dzs_re && dzs_im);
+	const double denom = 1 - std::pow((double) beta, (double) (t + 1));
+	CNET_CHECK_ARG(denom != 0.0);
+	if (n % 4 == 0 && all_aligned({z_re, z_im, m_re, m_im, dzs_re, dzs_im}))
+		hipLaunchKernelGGL(adam_kernel<4>, dim3(nblocks(n / 4)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
+				(long) n, lr, beta, denom, zero_grad);
+	else
+		hipLaunchKernelGGL(adam_kernel<1>, dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
+				(long) n, lr, beta, denom, zero_grad);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }

@@ -381,6 +381,24 @@ public:
 	int typeId() const override { return isGelu; }
 };
 
+// impl/relu.h:12-30
+class CRelu : public CFunc {
+public:
+	CRelu(Uid uid, InSize n) : CFunc(uid, n, OutSize(n.value())) {}
+	CRelu(InSize n) : CFunc(n, OutSize(n.value())) {}
+	std::string getName() override { return "CRelu_" + std::to_string(uid_); }
+	int typeId() const override { return isCrelu; }
+};
+
+// impl/ft.h:115-137
+class TriangFourier : public CFunc {
+public:
+	TriangFourier(Uid uid, InSize n) : CFunc(uid, n, OutSize(n.value())) {}
+	TriangFourier(InSize n) : CFunc(n, OutSize(n.value())) {}
+	std::string getName() override { return "TriangFourier_" + std::to_string(uid_); }
+	int typeId() const override { return isTrianFourier; }
+};
+
 class Residual : public CFunc {
 public:
 	Residual(Uid uid, InSize n) : CFunc(uid, InSize(2 * n.value()), OutSize(n.value())) {}
@@ -717,6 +735,9 @@ private:
 			case isFourier:
 				ck(cnet_cdft_plan(f->out_size_), "cnet_cdft_plan");
 				break;
+			case isTrianFourier:
+				ck(cnet_ctriang_dft_plan(f->out_size_), "cnet_ctriang_dft_plan");
+				break;
 			case isSoftMax:
 				((SoftMax *) f)->d_s_ = dalloc<float>(rows);
 				break;
@@ -772,6 +793,14 @@ private:
 		case isFourier:
 			ck(cnet_cdft_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_, 0),
 					"cnet_cdft_fwd");
+			break;
+		case isTrianFourier:
+			ck(cnet_ctriang_dft_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_, 0),
+					"cnet_ctriang_dft_fwd");
+			break;
+		case isCrelu:
+			ck(cnet_crelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_),
+					"cnet_crelu_fwd");
 			break;
 		case isHadamard: {
 			const int n = f->out_size_;
@@ -866,6 +895,14 @@ private:
 			case isFourier:
 				ck(cnet_cdft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
 						"cnet_cdft_bwd");
+				break;
+			case isTrianFourier:
+				ck(cnet_ctriang_dft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
+						"cnet_ctriang_dft_bwd");
+				break;
+			case isCrelu:
+				ck(cnet_crelu_bwd(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len,
+						rows, a.len, acc), "cnet_crelu_bwd");
 				break;
 			case isHadamard: {
 				CFunc::Slot &v = f->slots_[1];
@@ -1023,6 +1060,17 @@ public:
 			ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
 		}
 	}
+	// The Adam-style step of upstream GpuNet::adamUpdate (gpu/gpu_func.h:503-510, gpu/kernels.cpp:494-514) on every input
+	// function: the first moment lives in the node's dz planes, dz* is cleared, dz is kept.
+	void gpuAdamUpdate(float l_rate, float beta, int t) {
+		requireAllocated("gpuAdamUpdate");
+		for (auto f : inputs_) {
+			CFunc::Slot &s = f->slots_[0];
+			const size_t n = (size_t) s.rows * s.len;
+			float *z = s.grad - 2 * n;
+			ck(cnet_adam_update(z, z + n, s.g(0), s.g(1), s.g(2), s.g(3), (int64_t) n, l_rate, beta, t, 1), "cnet_adam_update");
+		}
+	}
 	float getLoss(OutputFunc *outp, Batch *batch) {
 		requireAllocated("getLoss");
 		CFunc *f = dynamic_cast<CFunc *>(outp);
@@ -1087,6 +1135,13 @@ public:
 	void updateInputs(float l_rate) {
 		if (batch_ != 1) throw std::logic_error("updateInputs(): call forward() first");
 		gpuUpdateInputs(l_rate);
+		for (auto f : inputs_) fetch(f, 0);
+	}
+
+	// per-sample twin of ComplexNet::adamUpdate (impl/cnet.h:423-431)
+	void adamUpdate(float learning_rate, int batch_size, float beta, int t) {
+		if (batch_ != 1) throw std::logic_error("adamUpdate(): call forward() first");
+		gpuAdamUpdate(learning_rate / batch_size, beta, t);
 		for (auto f : inputs_) fetch(f, 0);
 	}
 

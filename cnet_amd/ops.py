@@ -124,6 +124,14 @@ def dft_bwd(g, dx, accumulate=0):
     call("cnet_cdft_bwd", *g.p(), g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
 
 
+def triang_dft_fwd(x, y, accumulate=0):
+    call("cnet_ctriang_dft_fwd", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols, accumulate)
+
+
+def triang_dft_bwd(g, dx, accumulate=0):
+    call("cnet_ctriang_dft_bwd", *g.p(), g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
+
+
 # ------------------------------------------------------------------------------------------------- elementwise
 def hadamard_fwd(u, v, y, shared=False):
     call("cnet_hadamard_fwd", *u.p(), u.ld, *v.p(), 0 if shared else v.ld, *y.p(), y.ld, u.rows, u.cols)
@@ -140,6 +148,14 @@ def gelu_fwd(x, y):
 
 def gelu_bwd(x, g, dx, accumulate=0):
     call("cnet_cgelu_bwd", *x.p(), x.ld, *g.p(), g.ld, *dx.p(), dx.ld, x.rows, x.cols, accumulate)
+
+
+def crelu_fwd(x, y):
+    call("cnet_crelu_fwd", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols)
+
+
+def crelu_bwd(x, g, dx, accumulate=0):
+    call("cnet_crelu_bwd", *x.p(), x.ld, *g.p(), g.ld, *dx.p(), dx.ld, x.rows, x.cols, accumulate)
 
 
 def residual_fwd(u, v, y):
@@ -190,6 +206,10 @@ def batch_sum(src, dst, accumulate=0):
 
 def sgd_update(z, dzs_re, dzs_im, lr, zero_grad=1):
     call("cnet_sgd_update", z.re.ptr, z.im.ptr, dzs_re.ptr, dzs_im.ptr, z.rows * z.cols, lr, zero_grad)
+
+
+def adam_update(z, m_re, m_im, dzs_re, dzs_im, lr, beta, t, zero_grad=1):
+    call("cnet_adam_update", z.re.ptr, z.im.ptr, m_re.ptr, m_im.ptr, dzs_re.ptr, dzs_im.ptr, z.rows * z.cols, lr, beta, t, zero_grad)
 
 
 def embedding_fwd(table, tokens, y, slots):

@@ -120,6 +120,17 @@ int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs
                   float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
                   int B, int n, int accumulate);      /* dx.dz = g.dz * F ; dx.dzs = g.dzs * conj(F) */
 
+/* ---- TriangFourier: the DFT sums restricted to in <= out, y_o = (1/sqrt n) sum_{i <= o} x_i w^{i o}; CPU twin
+ *      impl/ft.h:139-189 (upstream has no device kernel for it: its GPU tests expect "not supported",
+ *      tests/gputests.h:1319-1330).  Runs as the same complex GEMM against an upper-triangular twiddle matrix; blocks of
+ *      the matrix that lie wholly below the diagonal are skipped, so it costs about half of cnet_cdft_*. */
+int cnet_ctriang_dft_plan(int n);
+int cnet_ctriang_dft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
+                         int B, int n, int accumulate);
+int cnet_ctriang_dft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+                         float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
+                         int B, int n, int accumulate);
+
 /* ---- Hadamard: replaces gpu_hadamard_forward / _backward (gpu/kernels.cpp:204-274), CPU twin impl/hadamard.h:34-68.
  * y = u .* v.  ldv == 0: v is one parameter row shared by all rows and dv is the sum over rows. */
 int cnet_hadamard_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
@@ -134,6 +145,15 @@ int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const f
 int cnet_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
                    int rows, int cols);
 int cnet_cgelu_bwd(const float *x_re, const float *x_im, int64_t ldx,
+                   const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
+                   float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
+                   int rows, int cols, int accumulate);
+
+/* ---- CRelu: y = z where Re z > 0 and Im z > 0, else 0; gradients pass under the same test.  CPU twin
+ *      impl/relu.h:32-63 (no upstream device kernel either). */
+int cnet_crelu_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
+                   int rows, int cols);
+int cnet_crelu_bwd(const float *x_re, const float *x_im, int64_t ldx,
                    const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
                    float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
                    int rows, int cols, int accumulate);
@@ -184,6 +204,12 @@ int cnet_add2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows,
 int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate); /* dst[c] (+)= sum_r src[r][c] */
 /* z -= lr * dzs ; then dzs = 0 when zero_grad != 0   (impl/cfunc.h:147-152 + impl/cnet.h:413-421) */
 int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int64_t n, float lr, int zero_grad);
+
+/* Adam-style step: replaces gpu_update_adam_input (gpu/kernels.cpp:494-525), CPU twin impl/cfunc.h:273-287 +
+ * impl/cnet.h:423-431.  m = beta m + (1 - beta) dzs ; z -= lr m / (1 - beta^(t+1)) ; then dzs = 0 when zero_grad != 0.
+ * m_re / m_im are the first-moment planes (upstream keeps them in the node's dz planes, impl/cfunc.h:341-349). */
+int cnet_adam_update(float *z_re, float *z_im, float *m_re, float *m_im, float *dzs_re, float *dzs_im, int64_t n,
+                     float lr, float beta, int t, int zero_grad);
 
 /* ---- CEmbedding: replaces gpu_embedding_forward / _backward (gpu/kernels.cpp:362-442), CPU twin impl/embed.h:109-148.
  * tokens[rows][slots] int32, -1 = padding (zero row).  y[rows][slots*dim].  The backward adds the dzs rows of equal

@@ -19,6 +19,7 @@ REF_SO = os.path.join(HERE, "_ref", "libcnet_ref.so")
 
 # node kinds (numeric ids of impl/cnet.h:31-42 upstream)
 HADAMARD, EMBEDDING, LINEAR, FOURIER, CROSSENT, RESIDUAL, SOFTMAX, INPUT, GELU, L2OUT = 1, 2, 3, 4, 5, 6, 7, 8, 10, 11
+CRELU, TRIANG_FOURIER = 9, 12
 # plane ids of a node's input block
 RE, IM, DZ_RE, DZ_IM, DZS_RE, DZS_IM, OUT_RE, OUT_IM = range(8)
 
@@ -62,6 +63,7 @@ class OracleLib:
         L.cno_net_forward.argtypes = [C.c_void_p]
         L.cno_net_backward.argtypes = [C.c_void_p, C.c_int]
         L.cno_net_update.argtypes = [C.c_void_p, C.c_float, C.c_int]
+        L.cno_net_adam_update.argtypes = [C.c_void_p, C.c_float, C.c_int, C.c_float, C.c_int]
         L.cno_net_loss.argtypes = [C.c_void_p, C.c_int, C.c_int]
         L.cno_net_loss.restype = C.c_float
         L.cno_net_prediction.argtypes = [C.c_void_p, C.c_int]
@@ -154,6 +156,28 @@ class OracleLib:
         self.lib.cno_gelu_bwd(C.c_long(xr.size), _fp(xr), _fp(xi), _p4(g4), _p4(dx))
         return dx
 
+    def crelu_fwd(self, xr, xi):
+        yr, yi = np.empty_like(xr), np.empty_like(xi)
+        self.lib.cno_crelu_fwd(C.c_long(xr.size), _fp(xr), _fp(xi), _fp(yr), _fp(yi))
+        return yr, yi
+
+    def crelu_bwd(self, xr, xi, g4):
+        dx = [np.empty_like(xr) for _ in range(4)]
+        self.lib.cno_crelu_bwd(C.c_long(xr.size), _fp(xr), _fp(xi), _p4(g4), _p4(dx))
+        return dx
+
+    def triang_fwd(self, xr, xi):
+        B, n = xr.shape
+        yr, yi = np.empty_like(xr), np.empty_like(xi)
+        self.lib.cno_triang_fwd(B, n, _fp(xr), _fp(xi), _fp(yr), _fp(yi))
+        return yr, yi
+
+    def triang_bwd(self, g4):
+        B, n = g4[0].shape
+        dx = [np.empty((B, n), np.float32) for _ in range(4)]
+        self.lib.cno_triang_bwd(B, n, _p4(g4), _p4(dx))
+        return dx
+
     def residual_fwd(self, ur, ui, vr, vi):
         yr, yi = np.empty_like(ur), np.empty_like(ui)
         self.lib.cno_residual_fwd(C.c_long(ur.size), _fp(ur), _fp(ui), _fp(vr), _fp(vi), _fp(yr), _fp(yi))
@@ -224,6 +248,11 @@ class OracleLib:
     def sgd_update(self, zr, zi, dsr, dsi, lr):
         self.lib.cno_sgd_update(C.c_long(zr.size), _fp(zr), _fp(zi), _fp(dsr), _fp(dsi), C.c_float(lr))
 
+    def adam_update(self, zr, zi, mr, mi, dsr, dsi, lr, beta, t):
+        """In place on z and m (first moment); dsr/dsi are left as they are."""
+        self.lib.cno_adam_update(C.c_long(zr.size), _fp(zr), _fp(zi), _fp(mr), _fp(mi), _fp(dsr), _fp(dsi), C.c_float(lr),
+                                 C.c_float(beta), C.c_int(t))
+
 
 class Net:
     """Per-sample graph with the upstream step semantics; mirrors ComplexNet's add/forward/backward/update."""
@@ -267,6 +296,9 @@ class Net:
 
     def update(self, lr, batch=1):
         self.o.lib.cno_net_update(self.h, C.c_float(lr), batch)
+
+    def adam_update(self, lr, batch, beta, t):
+        self.o.lib.cno_net_adam_update(self.h, C.c_float(lr), batch, C.c_float(beta), t)
 
     def loss(self, uid, label=0):
         return self.o.lib.cno_net_loss(self.h, uid, label)

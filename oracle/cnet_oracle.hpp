@@ -317,6 +317,43 @@ inline void dft_backward(int n, const std::vector<cf> &root, GradIn g, GradOut d
 }
 
 // ------------------------------------------------------------------------------------
+// TriangFourier  (impl/ft.h:139-189): the O(n^2) DFT sums restricted to in <= out,
+// y[o] = (1/sqrt n) sum_{i <= o} x[i] root(i o), float accumulation in index order.
+// ------------------------------------------------------------------------------------
+inline void triang_forward(int n, const std::vector<cf> &root, const float *xr, const float *xi, float *yr, float *yi) {
+	float scaling = sqrt(n);
+	for (int o = 0; o < n; ++o) {
+		cf sum = 0;
+		for (int i = 0; i < n; ++i) {
+			if (o < i) continue;
+			int e = i * o;
+			sum += cf(xr[i], xi[i]) * root[e % n];
+		}
+		sum /= scaling;
+		yr[o] = sum.real();
+		yi[o] = sum.imag();
+	}
+}
+
+inline void triang_backward(int n, const std::vector<cf> &root, GradIn g, GradOut dx) {
+	float scaling = sqrt(n);
+	for (int i = 0; i < n; ++i) {
+		cf a = 0, b = 0;
+		for (int o = 0; o < n; ++o) {
+			if (o < i) continue;
+			int e = i * o;
+			cf w = root[e % n];
+			a += g.dz(o) * w;
+			b += g.dzs(o) * std::conj(w);
+		}
+		dx.dz_re[i] += a.real() / scaling;
+		dx.dz_im[i] += a.imag() / scaling;
+		dx.dzs_re[i] += b.real() / scaling;
+		dx.dzs_im[i] += b.imag() / scaling;
+	}
+}
+
+// ------------------------------------------------------------------------------------
 // Hadamard  (impl/hadamard.h:34-68).  Input block = [u (n) | v (n)], y = u .* v.
 // ------------------------------------------------------------------------------------
 inline void hadamard_forward(int n, const float *ur, const float *ui, const float *vr, const float *vi,
@@ -389,6 +426,29 @@ inline void gelu_backward(int n, const float *xr, const float *xi, GradIn g, Gra
 		dx.dz_im[k] += a.imag();
 		dx.dzs_re[k] += b.real();
 		dx.dzs_im[k] += b.imag();
+	}
+}
+
+// ------------------------------------------------------------------------------------
+// CRelu  (impl/relu.h:32-63): passes z where both Re z > 0 and Im z > 0, else 0; the
+// backward pass hands both gradients through under the same test.
+// ------------------------------------------------------------------------------------
+inline void crelu_forward(int n, const float *xr, const float *xi, float *yr, float *yi) {
+	for (int k = 0; k < n; ++k) {
+		bool on = xr[k] > 0 && xi[k] > 0;
+		yr[k] = on ? xr[k] : 0;
+		yi[k] = on ? xi[k] : 0;
+	}
+}
+
+inline void crelu_backward(int n, const float *xr, const float *xi, GradIn g, GradOut dx) {
+	for (int k = 0; k < n; ++k) {
+		if (xr[k] > 0 && xi[k] > 0) {
+			dx.dz_re[k] += g.dz_re[k];
+			dx.dz_im[k] += g.dz_im[k];
+			dx.dzs_re[k] += g.dzs_re[k];
+			dx.dzs_im[k] += g.dzs_im[k];
+		}
 	}
 }
 
@@ -599,13 +659,29 @@ inline void sgd_update(int n, float *zr, float *zi, const float *dsr, const floa
 	}
 }
 
+// ------------------------------------------------------------------------------------
+// Adam-style step  (impl/cfunc.h:273-287; device twin gpu/kernels.cpp:494-514).  The first
+// moment lives in the node's own dz planes (impl/cfunc.h:341-349); there is no second
+// moment.  pow(float, int) promotes to double, so the step is evaluated in double and
+// rounded once when it is subtracted from the float parameter.
+// ------------------------------------------------------------------------------------
+inline void adam_update(int n, float *zr, float *zi, float *mr, float *mi, const float *dsr, const float *dsi,
+		float lr, float beta1, int t) {
+	for (int k = 0; k < n; ++k) {
+		mr[k] = mr[k] * beta1 + (1 - beta1) * dsr[k];
+		mi[k] = mi[k] * beta1 + (1 - beta1) * dsi[k];
+		zr[k] -= lr * mr[k] / (1 - pow(beta1, t + 1));
+		zi[k] -= lr * mi[k] / (1 - pow(beta1, t + 1));
+	}
+}
+
 // ====================================================================================
 // Graph runtime: the per-sample semantics of ComplexNet (impl/cnet.h:228-289, 366-421)
 // and of the producer-writes-into-consumer wiring of CFunc (impl/cfunc.h:211-224).
 // ====================================================================================
 enum Kind {  // numeric values as impl/cnet.h:31-42
 	kHadamard = 1, kEmbedding = 2, kLinear = 3, kFourier = 4, kCrossEntropy = 5, kResidual = 6,
-	kSoftMax = 7, kInput = 8, kGelu = 10, kL2Out = 11
+	kSoftMax = 7, kInput = 8, kCrelu = 9, kGelu = 10, kL2Out = 11, kTriangFourier = 12
 };
 
 struct Node {
@@ -679,6 +755,8 @@ public:
 		case kFourier: in_len = p0; nd->out_size = p0; nd->roots = unity_roots(p0); break;
 		case kHadamard: in_len = 2 * p0; nd->out_size = p0; break;
 		case kGelu: in_len = p0; nd->out_size = p0; break;
+		case kCrelu: in_len = p0; nd->out_size = p0; break;
+		case kTriangFourier: in_len = p0; nd->out_size = p0; nd->roots = unity_roots(p0); break;
 		case kResidual: in_len = 2 * p0; nd->out_size = p0; break;
 		case kSoftMax: in_len = p0; nd->out_size = p0; break;
 		case kCrossEntropy: in_len = p0; nd->out_size = 1; nd->is_output = true; nd->out.resize(p0); break;
@@ -727,6 +805,8 @@ public:
 			hadamard_forward(nd->p0, x.re, x.im, x.re + nd->p0, x.im + nd->p0, yr.data(), yi.data());
 			break;
 		case kGelu: gelu_forward(nd->p0, x.re, x.im, yr.data(), yi.data()); break;
+		case kCrelu: crelu_forward(nd->p0, x.re, x.im, yr.data(), yi.data()); break;
+		case kTriangFourier: triang_forward(nd->p0, nd->roots, x.re, x.im, yr.data(), yi.data()); break;
 		case kResidual:
 			residual_forward(nd->p0, x.re, x.im, x.re + nd->p0, x.im + nd->p0, yr.data(), yi.data());
 			break;
@@ -782,6 +862,12 @@ public:
 		case kGelu:
 			for (int c = 0; c < nc; ++c) gelu_backward(nd->p0, x.re, x.im, nd->upstream(c), nd->own(0));
 			break;
+		case kCrelu:
+			for (int c = 0; c < nc; ++c) crelu_backward(nd->p0, x.re, x.im, nd->upstream(c), nd->own(0));
+			break;
+		case kTriangFourier:
+			for (int c = 0; c < nc; ++c) triang_backward(nd->p0, nd->roots, nd->upstream(c), nd->own(0));
+			break;
 		case kResidual:
 			for (int c = 0; c < nc; ++c) residual_backward(nd->p0, nd->upstream(c), nd->own(0), nd->own(nd->p0));
 			break;
@@ -814,6 +900,16 @@ public:
 			Planes &x = inputs_[k]->in;
 			sgd_update(x.n, x.re, x.im, x.dzs_re, x.dzs_im, lr / batch);
 			x.zero_gradients();
+		}
+	}
+	// impl/cnet.h:423-431: every input node takes the Adam-style step, then only dz* is cleared
+	// (dz keeps the first moment).
+	void adam_update_inputs(float lr, int batch, float beta, int t) {
+		for (size_t k = 0; k < inputs_.size(); ++k) {
+			Planes &x = inputs_[k]->in;
+			adam_update(x.n, x.re, x.im, x.dz_re, x.dz_im, x.dzs_re, x.dzs_im, lr / batch, beta, t);
+			std::fill(x.dzs_re, x.dzs_re + x.n, 0.0f);
+			std::fill(x.dzs_im, x.dzs_im + x.n, 0.0f);
 		}
 	}
 	float loss(int uid, int label) {

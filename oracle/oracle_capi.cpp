@@ -79,6 +79,7 @@ void cno_net_set_tokens(void *h, int uid, const int *tok, int count) {
 void cno_net_forward(void *h) { ((Net *) h)->forward(); }
 void cno_net_backward(void *h, int label) { ((Net *) h)->backward(label); }
 void cno_net_update(void *h, float lr, int batch) { ((Net *) h)->update(lr, batch); }
+void cno_net_adam_update(void *h, float lr, int batch, float beta, int t) { ((Net *) h)->adam_update_inputs(lr, batch, beta, t); }
 float cno_net_loss(void *h, int uid, int label) { return ((Net *) h)->loss(uid, label); }
 int cno_net_prediction(void *h, int uid) { return ((Net *) h)->prediction(uid); }
 void cno_node_forward(void *h, int uid) { ((Net *) h)->node_forward(((Net *) h)->at(uid)); }
@@ -180,6 +181,29 @@ void cno_gelu_bwd(long total, const float *xr, const float *xi, const float *con
 	gelu_backward((int) total, xr, xi, gin(g, 0), gout(dx, 0));
 }
 
+void cno_crelu_fwd(long total, const float *xr, const float *xi, float *yr, float *yi) {
+	crelu_forward((int) total, xr, xi, yr, yi);
+}
+
+void cno_crelu_bwd(long total, const float *xr, const float *xi, const float *const *g, float *const *dx) {
+	zero4(dx, (size_t) total);
+	crelu_backward((int) total, xr, xi, gin(g, 0), gout(dx, 0));
+}
+
+void cno_triang_fwd(int B, int n, const float *xr, const float *xi, float *yr, float *yi) {
+	std::vector<cf> roots = unity_roots(n);
+#pragma omp parallel for
+	for (int b = 0; b < B; ++b)
+		triang_forward(n, roots, xr + (size_t) b * n, xi + (size_t) b * n, yr + (size_t) b * n, yi + (size_t) b * n);
+}
+
+void cno_triang_bwd(int B, int n, const float *const *g, float *const *dx) {
+	zero4(dx, (size_t) B * n);
+	std::vector<cf> roots = unity_roots(n);
+#pragma omp parallel for
+	for (int b = 0; b < B; ++b) triang_backward(n, roots, gin(g, (size_t) b * n), gout(dx, (size_t) b * n));
+}
+
 void cno_residual_fwd(long total, const float *ur, const float *ui, const float *vr, const float *vi, float *yr,
 		float *yi) {
 	residual_forward((int) total, ur, ui, vr, vi, yr, yi);
@@ -261,6 +285,11 @@ void cno_embedding_bwd(int B, int T, int D, int V, const int *tokens, const floa
 
 void cno_sgd_update(long n, float *zr, float *zi, const float *dsr, const float *dsi, float lr) {
 	sgd_update((int) n, zr, zi, dsr, dsi, lr);
+}
+
+void cno_adam_update(long n, float *zr, float *zi, float *mr, float *mi, const float *dsr, const float *dsi, float lr,
+		float beta, int t) {
+	adam_update((int) n, zr, zi, mr, mi, dsr, dsi, lr, beta, t);
 }
 
 // Dense matrix of the CPU forward transform: column q = forward(unit vector e_q).

@@ -53,6 +53,8 @@ int cno_net_add(void *h, int kind, int p0, int p1, int p2, const int *in_uids, i
 	case isFourier: f = new FourierTrans(InSize(p0)); break;
 	case isHadamard: f = new Hadamard(InSize(p0), InSize(p0)); break;
 	case isGelu: f = new CGelu(InSize(p0)); break;
+	case isCrelu: f = new CRelu(InSize(p0)); break;
+	case isTrianFourier: f = new TriangFourier(InSize(p0)); break;
 	case isResidual: f = new Residual(InSize(p0)); break;
 	case isSoftMax: f = new SoftMax(InSize(p0)); break;
 	case isCrossEntropy: f = new CrossEntropy(InSize(p0)); break;
@@ -96,6 +98,8 @@ void cno_net_backward(void *h, int label) {
 }
 
 void cno_net_update(void *h, float lr, int batch) { ((RefNet *) h)->net.update(lr, batch); }
+
+void cno_net_adam_update(void *h, float lr, int batch, float beta, int t) { ((RefNet *) h)->net.adamUpdate(lr, batch, beta, t); }
 
 float cno_net_loss(void *h, int uid, int label) {
 	OutputFunc *o = dynamic_cast<OutputFunc *>(((RefNet *) h)->net[uid]);

@@ -7,6 +7,7 @@
 //   facade_test resblock           residual stack with a second data input (L2 target), several SGD steps
 //   facade_test persample          the per-sample API (forward / backward(label) / updateInputs) on the device
 //   facade_test embedding          CEmbedding -> Linear -> CrossEntropy with an EmbeddingBatch
+//   facade_test adam               TriangFourier / CRelu net trained with the Adam-style step, batched and per sample
 //   facade_test errors             error behaviour
 //   facade_test c4 n blocks B steps lr   throughput of the residual stack (no oracle), JSON line
 #include <chrono>
@@ -433,6 +434,151 @@ static void test_embedding() {
 	report("embedding table dz* (scatter-add over the batch)", gt.value());
 }
 
+// ------------------------------------------------------------------------------------------------- Adam, TriangFourier, CRelu
+// x -> TriangFourier -> Hadamard(w) -> CRelu -> Linear(W) -> CrossEntropy, Adam-style steps t = 0..3 with the first
+// moment in the parameters' dz planes (upstream testAdam pattern, tests/gputests.h:1377-1378).
+static void test_adam() {
+	const int n = 96, classes = 12, B = 16, steps = 4;
+	const float lr = 0.05f, beta = 0.9f;
+	orc::Rng rng(33);
+	std::vector<float> hw(2 * n), lw((size_t) 2 * n * classes);
+	for (int k = 0; k < 2 * n; ++k) hw[k] = (float) rng.normal(0.5, 0.3);
+	fill_normal(rng, lw.data(), lw.size(), 1.0 / std::sqrt((double) n));
+
+	CNet cnet;
+	auto inp = cnet.add(new CInput(OutSize(n)));
+	auto tf = cnet.add(new TriangFourier(InSize(n)), {inp});
+	auto h_data = cnet.add(new CInput(OutSize(n)));
+	auto hdm = cnet.add(new Hadamard(InSize(n), InSize(n)), {tf, h_data});
+	auto relu = cnet.add(new CRelu(InSize(n)), {hdm});
+	auto l_data = cnet.add(new CInput(OutSize(n * classes)));
+	auto lin = cnet.add(new Linear(InSize(n), InSize(n * classes)), {relu, l_data});
+	auto outp = cnet.add(new CrossEntropy(InSize(classes)), {lin});
+	std::copy(hw.begin(), hw.end(), cnet[h_data]->mutable_input()->real_);
+	std::copy(lw.begin(), lw.end(), cnet[l_data]->mutable_input()->real_);
+	expect("allocateOnGpu", cnet.allocateOnGpu(B));
+	CInput *cin = (CInput *) cnet[inp];
+	CrossEntropy *cen = (CrossEntropy *) cnet[outp];
+
+	orc::Net on;
+	int ids[1], two[2];
+	int o_inp = on.add(orc::kInput, n, 0, 0, NULL, 0);
+	ids[0] = o_inp;
+	int o_tf = on.add(orc::kTriangFourier, n, 0, 0, ids, 1);
+	int o_hw = on.add(orc::kInput, n, 0, 0, NULL, 0);
+	two[0] = o_tf;
+	two[1] = o_hw;
+	int o_hdm = on.add(orc::kHadamard, n, 0, 0, two, 2);
+	ids[0] = o_hdm;
+	int o_relu = on.add(orc::kCrelu, n, 0, 0, ids, 1);
+	int o_lw = on.add(orc::kInput, n * classes, 0, 0, NULL, 0);
+	two[0] = o_relu;
+	two[1] = o_lw;
+	int o_lin = on.add(orc::kLinear, n, n * classes, 0, two, 2);
+	ids[0] = o_lin;
+	int o_out = on.add(orc::kCrossEntropy, classes, 0, 0, ids, 1);
+	std::copy(hw.begin(), hw.end(), on.at(o_hw)->in.re);
+	std::copy(lw.begin(), lw.end(), on.at(o_lw)->in.re);
+
+	for (int t = 0; t < steps; ++t) {
+		std::vector<float> xr((size_t) B * n), xi((size_t) B * n);
+		fill_normal(rng, xr.data(), xr.size(), 1.0);
+		fill_normal(rng, xi.data(), xi.size(), 1.0);
+		std::vector<int> labels(B);
+		for (auto &l : labels) l = (int) (rng.next() % classes);
+		InputBatch batch(B, n);
+		for (int b = 0; b < B; ++b) batch.add(xr.data() + (size_t) b * n, xi.data() + (size_t) b * n, n, labels[b]);
+		cnet.gpuForward(cin, cen, batch);
+		cnet.getLoss(cen, &batch);
+		cnet.gpuBackward();
+		ErrAcc z_tf, g_tf, z_relu, g_relu, z_out;
+		double loss_err = 0;
+		int active = 0;
+		for (int b = 0; b < B; ++b) {
+			std::copy(xr.begin() + (size_t) b * n, xr.begin() + (size_t) (b + 1) * n, on.at(o_inp)->in.re);
+			std::copy(xi.begin() + (size_t) b * n, xi.begin() + (size_t) (b + 1) * n, on.at(o_inp)->in.im);
+			on.forward();
+			float l = on.loss(o_out, labels[b]);
+			loss_err = std::max(loss_err, (double) std::fabs(l - batch.loss(b)) / std::max(1.0, (double) std::fabs(l)));
+			on.backward(labels[b]);
+			cnet.fetchAll(b);
+			cmp_node(cnet[tf], on.at(o_tf), &z_tf, &g_tf);
+			cmp_node(cnet[relu], on.at(o_relu), &z_relu, &g_relu);
+			z_out.add(cnet[outp]->input().real_, on.at(o_out)->in.re, 2 * classes);
+			for (int k = 0; k < n; ++k) active += on.at(o_lin)->in.re[k] != 0.f;
+			// each row is its own sample of the data input: drop what the oracle gathered for it
+			std::fill(on.at(o_inp)->in.dzs_re, on.at(o_inp)->in.dzs_re + 2 * n, 0.f);
+		}
+		std::string s = " step " + std::to_string(t);
+		report("TriangFourier input z" + s, z_tf.value());
+		report("TriangFourier dz, dz*" + s, g_tf.value());
+		report("CRelu input z" + s, z_relu.value());
+		report("CRelu dz, dz*" + s, g_relu.value());
+		report("CrossEntropy input z" + s, z_out.value());
+		report("per-sample loss" + s, loss_err);
+		if (t == 0) expect("CRelu passes some and blocks some entries", active > B * n / 10 && active < B * n * 9 / 10);
+
+		cnet.gpuAdamUpdate(lr / B, beta, t);
+		on.adam_update_inputs(lr, B, beta, t);
+		cnet.getInputsFromGpu();
+		ErrAcc w1, w2, m1, m2;
+		w1.add(cnet[h_data]->input().real_, on.at(o_hw)->in.re, 2 * n);
+		w2.add(cnet[l_data]->input().real_, on.at(o_lw)->in.re, 2 * n * classes);
+		m1.add(cnet[h_data]->input().dz_real_, on.at(o_hw)->in.dz_re, 2 * n);
+		m2.add(cnet[l_data]->input().dz_real_, on.at(o_lw)->in.dz_re, 2 * n * classes);
+		report("Hadamard weights after Adam step" + s, w1.value(), TOL / 5);
+		report("Linear weights after Adam step" + s, w2.value(), TOL / 5);
+		report("Hadamard first moment (dz planes)" + s, m1.value());
+		report("Linear first moment (dz planes)" + s, m2.value());
+		bool cleared = true;
+		for (int k = 0; k < 2 * n * classes; ++k) cleared = cleared && cnet[l_data]->input().dz_star_real_[k] == 0.f;
+		expect("dz* cleared by the Adam step" + s, cleared);
+	}
+
+	// per-sample API: forward / backward(label) / adamUpdate on a fresh small net
+	{
+		const int m = 20, cls = 4;
+		CNet net;
+		auto x = net.add(new CInput(OutSize(m)));
+		auto f = net.add(new TriangFourier(InSize(m)), {x});
+		auto r = net.add(new CRelu(InSize(m)), {f});
+		auto w = net.add(new CInput(OutSize(m * cls)));
+		auto l = net.add(new Linear(InSize(m), InSize(m * cls)), {r, w});
+		auto o = net.add(new CrossEntropy(InSize(cls)), {l});
+		net.init_inputs(5);
+		orc::Net pn;
+		int px = pn.add(orc::kInput, m, 0, 0, NULL, 0);
+		ids[0] = px;
+		int pf = pn.add(orc::kTriangFourier, m, 0, 0, ids, 1);
+		ids[0] = pf;
+		int pr = pn.add(orc::kCrelu, m, 0, 0, ids, 1);
+		int pw = pn.add(orc::kInput, m * cls, 0, 0, NULL, 0);
+		two[0] = pr;
+		two[1] = pw;
+		int pl = pn.add(orc::kLinear, m, m * cls, 0, two, 2);
+		ids[0] = pl;
+		int po = pn.add(orc::kCrossEntropy, cls, 0, 0, ids, 1);
+		std::copy(net[x]->input().real_, net[x]->input().real_ + 2 * m, pn.at(px)->in.re);
+		std::copy(net[w]->input().real_, net[w]->input().real_ + 2 * m * cls, pn.at(pw)->in.re);
+		ErrAcc zw, zx, lo;
+		for (int t = 0; t < 3; ++t) {
+			net.forward();
+			pn.forward();
+			float got = ((CrossEntropy *) net[o])->loss(t % cls), want = pn.loss(po, t % cls);
+			lo.add(&got, &want, 1);
+			net.backward(t % cls);
+			pn.backward(t % cls);
+			net.adamUpdate(0.1f, 1, 0.9f, t);
+			pn.adam_update_inputs(0.1f, 1, 0.9f, t);
+			zw.add(net[w]->input().real_, pn.at(pw)->in.re, 4 * m * cls);  // z and the first moment
+			zx.add(net[x]->input().real_, pn.at(px)->in.re, 4 * m);
+		}
+		report("per-sample API: loss", lo.value());
+		report("per-sample API: weights and first moment after adamUpdate", zw.value());
+		report("per-sample API: data input and its first moment", zx.value());
+	}
+}
+
 // ------------------------------------------------------------------------------------------------- error behaviour
 template <class E, class F>
 static bool throws(F f) {
@@ -532,6 +678,7 @@ int main(int argc, char **argv) {
 		if (what == "resblock" || what == "all") test_resblock();
 		if (what == "persample" || what == "all") test_persample();
 		if (what == "embedding" || what == "all") test_embedding();
+		if (what == "adam" || what == "all") test_adam();
 		if (what == "errors" || what == "all") test_errors();
 		if (what == "c4")
 			run_c4(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048, argc > 5 ? atoi(argv[5]) : 10,

@@ -72,6 +72,41 @@ def residual(lib):
     return _layer(lib, ob.RESIDUAL, (9,), [9, 9], 9, seed=8, consumers=2)
 
 
+def crelu(lib):
+    return _layer(lib, ob.CRELU, (129,), [129], 129, seed=21, consumers=2)
+
+
+def triang_fourier(lib):
+    return _layer(lib, ob.TRIANG_FOURIER, (50,), [50], 50, seed=22)
+
+
+def adam_training(lib, n=20, classes=4, steps=4):
+    """TriangFourier -> Hadamard(w) -> CRelu -> Linear(W) -> CrossEntropy with the Adam-style step, t = 0..steps-1."""
+    net = lib.net()
+    x = net.add(ob.INPUT, n)
+    f = net.add(ob.TRIANG_FOURIER, n, inputs=[x])
+    hw = net.add(ob.INPUT, n)
+    h = net.add(ob.HADAMARD, n, inputs=[f, hw])
+    r = net.add(ob.CRELU, n, inputs=[h])
+    lw = net.add(ob.INPUT, n * classes)
+    lin = net.add(ob.LINEAR, n, n * classes, inputs=[r, lw])
+    ce = net.add(ob.CROSSENT, classes, inputs=[lin])
+    rec = dict(hw0=_rand(31, 2, n) * 0.3 + 0.5, lw0=_rand(32, 2, n * classes) / np.float32(np.sqrt(n)), xs=_rand(33, steps, 2, n),
+               labels=np.arange(steps, dtype=np.int32) % classes)
+    rec["hw0"] = rec["hw0"].astype(np.float32)
+    net.plane(hw, ob.RE)[:] = rec["hw0"][0]; net.plane(hw, ob.IM)[:] = rec["hw0"][1]
+    net.plane(lw, ob.RE)[:] = rec["lw0"][0]; net.plane(lw, ob.IM)[:] = rec["lw0"][1]
+    for t in range(steps):
+        net.plane(x, ob.RE)[:] = rec["xs"][t, 0]; net.plane(x, ob.IM)[:] = rec["xs"][t, 1]
+        net.forward()
+        rec["loss%d" % t] = np.float32(net.loss(ce, int(rec["labels"][t])))
+        net.backward(int(rec["labels"][t]))
+        net.adam_update(0.05, 1, 0.9, t)
+        for name, uid in (("hw", hw), ("lw", lw)):
+            rec["%s_step%d" % (name, t)] = np.stack([net.plane(uid, p).copy() for p in range(4)])
+    return rec
+
+
 def softmax(lib):
     return _layer(lib, ob.SOFTMAX, (31,), [31], 31, seed=9)
 
@@ -227,5 +262,6 @@ def generators(lib):
     return dict(normal=lib.normal(2024, 257, 0.0, 1.0), uniform=lib.uniform(2024, 257, 0.0, 1.0))
 
 
-SCENARIOS = [linear, linear_fanout, fourier_pow2, fourier_784, fourier_12, hadamard, gelu, residual, softmax,
+SCENARIOS = [linear, linear_fanout, fourier_pow2, fourier_784, fourier_12, hadamard, gelu, residual, softmax, crelu,
+             triang_fourier, adam_training,
              fourier_rows_4096, losses, readme_net_training, residual_block_training, embedding, generators]

@@ -52,6 +52,11 @@ def test_embedding_batch():
     assert "FAIL" not in out
 
 
+def test_triang_fourier_crelu_net_with_adam_steps():
+    out = _run("adam")
+    assert "FAIL" not in out and out.count("PASS") > 30
+
+
 def test_error_behaviour():
     out = _run("errors")
     assert "FAIL" not in out

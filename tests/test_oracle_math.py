@@ -237,6 +237,56 @@ def test_sgd_update(port):
     assert np.array_equal(a, zr - np.float32(0.25) * dr) and np.array_equal(b, zi - np.float32(0.25) * di)
 
 
+def test_adam_update_closed_forms(port):
+    """beta = 0 is plain SGD (m = g, bias correction 1); from m = 0 the first step at any beta is also lr * g,
+    because (1 - beta) g / (1 - beta^1) = g; later steps follow the textbook recursion in float64."""
+    z, g = rnd(5, 2, 64), rnd(6, 2, 64)
+    zr, zi, mr, mi = z[0].copy(), z[1].copy(), rnd(7, 64), rnd(8, 64)
+    port.adam_update(zr, zi, mr, mi, g[0], g[1], 0.25, 0.0, 3)
+    assert np.array_equal(mr, g[0]) and np.array_equal(mi, g[1])
+    assert np.array_equal(zr, z[0] - np.float32(0.25) * g[0]) and np.array_equal(zi, z[1] - np.float32(0.25) * g[1])
+    zr, zi, mr, mi = z[0].copy(), z[1].copy(), np.zeros(64, np.float32), np.zeros(64, np.float32)
+    z64, m64 = z.astype(np.float64), np.zeros((2, 64))
+    for t in range(5):
+        gt = rnd(20 + t, 2, 64)
+        port.adam_update(zr, zi, mr, mi, gt[0], gt[1], 0.1, 0.9, t)
+        m64 = 0.9 * m64 + (1 - 0.9) * gt
+        z64 = z64 - 0.1 * m64 / (1 - 0.9 ** (t + 1))
+        if t == 0:
+            assert np.allclose(zr, z[0] - 0.1 * gt[0], rtol=0, atol=1e-6)
+        assert np.allclose(np.stack([mr, mi]), m64, atol=1e-6)
+        assert np.allclose(np.stack([zr, zi]), z64, atol=2e-6)
+
+
+def test_crelu_closed_form(port):
+    x = rnd(9, 2, 500)
+    x[:, :4] = [[0.0, 1.0, -0.0, 1.0], [1.0, 0.0, 1.0, -1.0]]  # zero parts do not pass (strict >)
+    on = (x[0] > 0) & (x[1] > 0)
+    yr, yi = port.crelu_fwd(x[0], x[1])
+    assert np.array_equal(yr, np.where(on, x[0], 0)) and np.array_equal(yi, np.where(on, x[1], 0))
+    assert not on[:4].any() and 50 < on.sum() < 200
+    g4 = [rnd(10 + p, 500) for p in range(4)]
+    for got, g in zip(port.crelu_bwd(x[0], x[1], g4), g4):
+        assert np.array_equal(got, np.where(on, g, 0))
+
+
+@pytest.mark.parametrize("n", [1, 2, 9, 64, 100])
+def test_triang_fourier_is_masked_dft_matrix(port, n):
+    """y = x T with T[i][o] = exp(-2 pi i (i o) / n) / sqrt n for i <= o, 0 below; backward is g T^T and g* conj(T)^T."""
+    i, o = np.meshgrid(np.arange(n), np.arange(n), indexing="ij")
+    T = np.where(i <= o, np.exp(-2j * np.pi * ((i * o) % n) / n) / np.sqrt(n), 0)
+    x = rnd(n, 3, n) + 1j * rnd(n + 1, 3, n)
+    yr, yi = port.triang_fwd(np.ascontiguousarray(x.real, np.float32), np.ascontiguousarray(x.imag, np.float32))
+    assert rel(cplx(yr, yi), x @ T) < 2e-6
+    if n > 2:  # the mask is one-sided: the full DFT differs
+        F = np.exp(-2j * np.pi * ((i * o) % n) / n) / np.sqrt(n)
+        assert rel(cplx(yr, yi), x @ F) > 0.1
+    g4 = [rnd(40 + p, 3, n) for p in range(4)]
+    dx = port.triang_bwd(g4)
+    assert rel(cplx(dx[0], dx[1]), cplx(g4[0], g4[1]) @ T.T) < 2e-6
+    assert rel(cplx(dx[2], dx[3]), cplx(g4[2], g4[3]) @ np.conj(T).T) < 2e-6
+
+
 # ---------------------------------------------------------------- finite differences through whole nets
 def _fd_check(port, build, in_len, seed, tol=3e-2, label=-1):
     """d(real loss)/d Re x = 2 Re dz*, d/d Im x = 2 Im dz*; dz = conj(dz*) for a real loss."""
@@ -290,6 +340,7 @@ def _chain(kinds):
     [ob.L2OUT], [ob.LINEAR, ob.L2OUT], [ob.FOURIER, ob.GELU, ob.L2OUT], [ob.HADAMARD, ob.GELU, ob.L2OUT],
     [ob.GELU, ob.L2OUT], [ob.LINEAR, ob.GELU, ob.RESIDUAL, ob.L2OUT], [ob.SOFTMAX, ob.GELU, ob.L2OUT],
     [ob.FOURIER, ob.HADAMARD, ob.GELU, ob.LINEAR, ob.SOFTMAX, ob.GELU, ob.L2OUT],
+    [ob.TRIANG_FOURIER, ob.L2OUT], [ob.LINEAR, ob.TRIANG_FOURIER, ob.GELU, ob.L2OUT],
 ])
 def test_wirtinger_gradients_by_finite_differences(port, kinds):
     _fd_check(port, _chain(kinds), 6, seed=len(kinds))

@@ -94,6 +94,16 @@ def test_gelu(port, ref, n):
     _layer_case(port, ref, ob.GELU, (n,), [n], seed=n)
 
 
+@pytest.mark.parametrize("n", [1, 6, 1000])
+def test_crelu(port, ref, n):
+    _layer_case(port, ref, ob.CRELU, (n,), [n], seed=n, consumers=2)
+
+
+@pytest.mark.parametrize("n", [1, 2, 7, 64, 100])
+def test_triang_fourier(port, ref, n):
+    _layer_case(port, ref, ob.TRIANG_FOURIER, (n,), [n], seed=n, consumers=2)
+
+
 @pytest.mark.parametrize("n", [1, 6, 300])
 def test_residual(port, ref, n):
     _layer_case(port, ref, ob.RESIDUAL, (n,), [n, n], seed=n, consumers=2)
@@ -245,6 +255,43 @@ def test_residual_block_with_fanout(port, ref):
                 rec += [net.plane(uid, p).copy() for p in range(6)]
             net.update(0.01, 1)
         out.append(rec)
+    for k, (a, b) in enumerate(zip(*out)):
+        _same(np.atleast_1d(a), np.atleast_1d(b), "record %d" % k)
+
+
+def test_adam_steps_triang_crelu_net(port, ref):
+    """x -> TriangFourier -> Hadamard(w) -> CRelu -> Linear(W) -> CrossEntropy, four Adam-style steps (t = 0..3) with
+    the first moment carried in the inputs' dz planes (upstream tests/gputests.h:1377-1378 drives the same call)."""
+    n, classes = 24, 5
+    xs = port.uniform(17, (4, n))
+    hw = port.normal(18, (2, n), 0.5, 0.3)
+    lw = port.normal(19, (2, n * classes), 0.0, 1.0 / np.sqrt(n))
+    labels = [3, 0, 4, 1]
+    out = []
+    for lib in (port, ref):
+        net = lib.net()
+        x = net.add(ob.INPUT, n)
+        f = net.add(ob.TRIANG_FOURIER, n, inputs=[x])
+        hwi = net.add(ob.INPUT, n)
+        h = net.add(ob.HADAMARD, n, inputs=[f, hwi])
+        r = net.add(ob.CRELU, n, inputs=[h])
+        lwi = net.add(ob.INPUT, n * classes)
+        lin = net.add(ob.LINEAR, n, n * classes, inputs=[r, lwi])
+        ce = net.add(ob.CROSSENT, classes, inputs=[lin])
+        _fill(net, hwi, ob.RE, hw[0]); _fill(net, hwi, ob.IM, hw[1])
+        _fill(net, lwi, ob.RE, lw[0]); _fill(net, lwi, ob.IM, lw[1])
+        rec = []
+        for t in range(4):
+            _fill(net, x, ob.RE, xs[t]); _fill(net, x, ob.IM, xs[(t + 1) % 4])
+            net.forward()
+            rec.append(np.float32(net.loss(ce, labels[t])))
+            net.backward(labels[t])
+            for uid in (f, h, r, lin):
+                rec += [net.plane(uid, p).copy() for p in range(6)]
+            net.adam_update(0.1, 2, 0.9, t)
+            rec += [net.plane(uid, p).copy() for uid in (hwi, lwi, x) for p in range(6)]
+        out.append(rec)
+    assert any(np.any(a != 0) for a in out[0][-18:])
     for k, (a, b) in enumerate(zip(*out)):
         _same(np.atleast_1d(a), np.atleast_1d(b), "record %d" % k)
 
