@@ -655,7 +655,8 @@ int cnet_residual_fwd(const float *u_re, const float *u_im, int64_t ldu, const f
 	CNET_REQUIRE_INIT();
 	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
 	if (!rows || !cols) return CNET_OK;
-	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && y_re && y_im && ldu >= cols && ldv >= cols && ldy >= cols);
+	// a leading dimension of 0 makes that operand one row shared by all rows (a parameter added to every sample)
+	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && y_re && y_im && (ldu >= cols || ldu == 0) && (ldv >= cols || ldv == 0) && ldy >= cols);
 	if (all_mult4({cols, ldu, ldv, ldy}) && all_aligned({u_re, u_im, v_re, v_im, y_re, y_im}))
 		hipLaunchKernelGGL(residual_fwd_kernel<4>, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
 	else

@@ -571,7 +571,11 @@ public:
 		if (func->uid_ == 0) func->uid_ = ++next_uid_;
 		else next_uid_ = std::max(next_uid_, func->uid_);
 		func->type_ = func->typeId();
-		if (map_.find(func->uid_) != map_.end()) throw std::invalid_argument("add: duplicate uid " + std::to_string(func->uid_));
+		if (map_.find(func->uid_) != map_.end()) {
+			const std::string msg = "add: duplicate uid " + std::to_string(func->uid_);
+			delete func;  // the net owns what it is given, also when it refuses it
+			throw std::invalid_argument(msg);
+		}
 		func_list_.push_back(func);
 		map_[func->uid_] = func;
 		if (func->is_input_) inputs_.push_back(func);
@@ -727,8 +731,6 @@ private:
 			case isHadamard:
 			case isResidual:
 				if (f->slots_.size() != 2) throw std::invalid_argument(f->getName() + ": needs two inputs");
-				if (t == isResidual && f->slots_[0].rows != f->slots_[1].rows)
-					throw std::invalid_argument(f->getName() + ": mixing a parameter and a batched operand is not supported");
 				if (t == isHadamard && f->slots_[0].rows < f->slots_[1].rows)
 					throw std::invalid_argument(f->getName() + ": put the batched operand first, the parameter second");
 				break;
@@ -814,8 +816,9 @@ private:
 			break;
 		case isResidual: {
 			const int n = f->out_size_;
-			ck(cnet_residual_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), n, f->out_re(), f->out_im(), n, rows, n),
-					"cnet_residual_fwd");
+			// an operand that is a parameter (one row, e.g. a positional table) is added to every row
+			ck(cnet_residual_fwd(zre(f, 0), zim(f, 0), f->slots_[0].rows == rows ? n : 0, zre(f, 1), zim(f, 1),
+					f->slots_[1].rows == rows ? n : 0, f->out_re(), f->out_im(), n, rows, n), "cnet_residual_fwd");
 			break;
 		}
 		case isSoftMax:
@@ -918,8 +921,21 @@ private:
 			case isResidual: {
 				CFunc::Slot &v = f->slots_[1];
 				const int n = f->out_size_;
-				ck(cnet_residual_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3),
-						n, rows, n, acc), "cnet_residual_bwd");
+				if (a.rows == rows && v.rows == rows) {
+					ck(cnet_residual_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3),
+							n, rows, n, acc), "cnet_residual_bwd");
+					break;
+				}
+				// a parameter operand receives the sum over the batch rows, a batched one a copy
+				for (CFunc::Slot *s : {&a, &v})
+					for (int p = 0; p < 4; ++p) {
+						if (s->rows == 1 && rows > 1)
+							ck(cnet_batch_sum(u.g(p), u.len, s->g(p), rows, n, acc), "cnet_batch_sum");
+						else if (acc)
+							ck(cnet_add2d(u.g(p), u.len, s->g(p), n, s->rows, n), "cnet_add2d");
+						else
+							ck(cnet_copy2d(u.g(p), u.len, s->g(p), n, s->rows, n), "cnet_copy2d");
+					}
 				break;
 			}
 			case isSoftMax:
@@ -1107,6 +1123,10 @@ public:
 	}
 	void sync() { ck(cnet_sync(), "cnet_sync"); }
 
+	// upstream CNet::save / restore (gpu/gpu_func.h:1103-1111); defined in model_saver.hpp
+	bool save(std::string file);
+	bool restore(std::string file);
+
 	// ---- per-sample API of upstream (CNet::forward / backward / updateInputs, gpu/gpu_func.h:1046-1056, 497-501):
 	//      host views are the state, the arithmetic runs on the device with a batch of one ----
 	void forward() {
@@ -1156,5 +1176,7 @@ private:
 		ck(cnet_memcpy_h2d(e->d_tokens_, buf.data(), buf.size() * sizeof(int32_t)), "cnet_memcpy_h2d");
 	}
 };
+
+#include "model_saver.hpp"
 
 #endif  // CNET_AMD_HOST_CNET_HPP_

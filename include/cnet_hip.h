@@ -158,7 +158,9 @@ int cnet_crelu_bwd(const float *x_re, const float *x_im, int64_t ldx,
                    float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
                    int rows, int cols, int accumulate);
 
-/* ---- Residual: replaces gpu_residual_forward / _backward (gpu/kernels.cpp:145-202), CPU twin impl/residual.h:40-77. */
+/* ---- Residual: replaces gpu_residual_forward / _backward (gpu/kernels.cpp:145-202), CPU twin impl/residual.h:40-77.
+ * Forward: ldu == 0 or ldv == 0 makes that operand one parameter row added to every row (its gradient is then the
+ * column sum of g: cnet_batch_sum). */
 int cnet_residual_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
                       float *y_re, float *y_im, int64_t ldy, int rows, int cols);
 int cnet_residual_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,

@@ -63,6 +63,12 @@ class OracleLib:
         L.cno_net_forward.argtypes = [C.c_void_p]
         L.cno_net_backward.argtypes = [C.c_void_p, C.c_int]
         L.cno_net_update.argtypes = [C.c_void_p, C.c_float, C.c_int]
+        L.cno_net_save.argtypes = [C.c_void_p, C.c_char_p, C.c_long]
+        L.cno_net_save.restype = C.c_long
+        L.cno_net_restore.argtypes = [C.c_void_p, C.c_char_p, C.c_long]
+        L.cno_net_count.argtypes = [C.c_void_p]
+        L.cno_net_uid_at.argtypes = [C.c_void_p, C.c_int]
+        L.cno_net_kind.argtypes = [C.c_void_p, C.c_int]
         L.cno_net_adam_update.argtypes = [C.c_void_p, C.c_float, C.c_int, C.c_float, C.c_int]
         L.cno_net_loss.argtypes = [C.c_void_p, C.c_int, C.c_int]
         L.cno_net_loss.restype = C.c_float
@@ -296,6 +302,24 @@ class Net:
 
     def update(self, lr, batch=1):
         self.o.lib.cno_net_update(self.h, C.c_float(lr), batch)
+
+    def save(self):
+        """The .mod record stream of this net (bytes)."""
+        n = self.o.lib.cno_net_save(self.h, None, 0)
+        buf = C.create_string_buffer(n)
+        assert self.o.lib.cno_net_save(self.h, buf, n) == n
+        return buf.raw
+
+    def restore(self, blob):
+        """Append the functions stored in a .mod stream; returns False when the stream is refused."""
+        ok = bool(self.o.lib.cno_net_restore(self.h, blob, len(blob)))
+        if ok:
+            for uid in self.uids():
+                self.kind[uid] = self.o.lib.cno_net_kind(self.h, uid)
+        return ok
+
+    def uids(self):
+        return [self.o.lib.cno_net_uid_at(self.h, k) for k in range(self.o.lib.cno_net_count(self.h))]
 
     def adam_update(self, lr, batch, beta, t):
         self.o.lib.cno_net_adam_update(self.h, C.c_float(lr), batch, C.c_float(beta), t)

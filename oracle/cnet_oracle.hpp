@@ -742,7 +742,7 @@ public:
 	// CGelu(n) impl/relu.h:102; Residual(n) impl/residual.h:15; SoftMax(n) impl/softmax.h:14-16;
 	// CrossEntropy(n) impl/crossent.h:14-17; L2Out(n) impl/l2out.h:14-16;
 	// CEmbedding(dim, slots, vocab) impl/embed.h:41-45.
-	int add(int kind, int p0, int p1, int p2, const int *in_uids, int n_in) {
+	int add(int kind, int p0, int p1, int p2, const int *in_uids, int n_in, int uid = 0) {
 		Node *nd = new Node();
 		nd->kind = kind;
 		nd->p0 = p0;
@@ -765,7 +765,13 @@ public:
 		default: delete nd; return -1;
 		}
 		nd->in.resize(in_len);
-		nd->uid = ++next_uid_;
+		if (uid > 0) {  // impl/cnet.h:228-246: an explicit uid is kept and moves the counter past it
+			assert(!by_uid_.count(uid));
+			nd->uid = uid;
+			next_uid_ = std::max(next_uid_, uid);
+		} else {
+			nd->uid = ++next_uid_;
+		}
 		list_.push_back(nd);
 		by_uid_[nd->uid] = nd;
 		if (nd->is_input) inputs_.push_back(nd);
@@ -911,6 +917,98 @@ public:
 			std::fill(x.dzs_re, x.dzs_re + x.n, 0.0f);
 			std::fill(x.dzs_im, x.dzs_im + x.n, 0.0f);
 		}
+	}
+	// ---- the .mod record stream of impl/model_saver.h:483-967: big-endian int32 / float32 throughout.
+	//   magic 0xABCDE0EE, then per function in insertion order:
+	//   type id, uid, input length, output size, number of producers, producer uids,
+	//   then CInput: re[len], im[len]; CEmbedding: dim, slots, vocab, re[len], im[len]; Linear: in1, in2.
+	static void put32(std::string &o, uint32_t v) {
+		for (int k = 3; k >= 0; --k) o.push_back((char) ((v >> (8 * k)) & 0xff));
+	}
+	static void putf(std::string &o, const float *p, int n) {
+		for (int k = 0; k < n; ++k) {
+			uint32_t u;
+			memcpy(&u, p + k, 4);
+			put32(o, u);
+		}
+	}
+	std::string save() const {
+		std::string o;
+		put32(o, 0xABCDE0EEu);
+		for (size_t k = 0; k < list_.size(); ++k) {
+			const Node *nd = list_[k];
+			put32(o, (uint32_t) nd->kind);
+			put32(o, (uint32_t) nd->uid);
+			put32(o, (uint32_t) nd->in.n);
+			put32(o, (uint32_t) nd->out_size);
+			put32(o, (uint32_t) nd->prev.size());
+			for (size_t q = 0; q < nd->prev.size(); ++q) put32(o, (uint32_t) nd->prev[q]->uid);
+			if (nd->kind == kEmbedding) {
+				put32(o, (uint32_t) nd->p0);
+				put32(o, (uint32_t) nd->p1);
+				put32(o, (uint32_t) nd->p2);
+			}
+			if (nd->kind == kInput || nd->kind == kEmbedding) {
+				putf(o, nd->in.re, nd->in.n);
+				putf(o, nd->in.im, nd->in.n);
+			}
+			if (nd->kind == kLinear) {
+				put32(o, (uint32_t) nd->p0);
+				put32(o, (uint32_t) nd->p1);
+			}
+		}
+		return o;
+	}
+	// Appends the stored functions to this net (upstream restores into an empty net); false on a bad magic number,
+	// an unknown type id or a truncated record.
+	bool restore(const std::string &blob) {
+		size_t pos = 0;
+		auto get32 = [&](int *v) {
+			if (pos + 4 > blob.size()) return false;
+			uint32_t u = 0;
+			for (int k = 0; k < 4; ++k) u = (u << 8) | (unsigned char) blob[pos + k];
+			pos += 4;
+			*v = (int) u;
+			return true;
+		};
+		auto getf = [&](float *p, int n) {
+			for (int k = 0; k < n; ++k) {
+				int v;
+				if (!get32(&v)) return false;
+				memcpy(p + k, &v, 4);
+			}
+			return true;
+		};
+		int magic;
+		if (!get32(&magic) || (uint32_t) magic != 0xABCDE0EEu) return false;
+		int kind;
+		while (get32(&kind)) {
+			int uid, in_len, out_size, nprev;
+			if (!get32(&uid) || !get32(&in_len) || !get32(&out_size) || !get32(&nprev)) return false;
+			std::vector<int> prev(nprev);
+			for (int q = 0; q < nprev; ++q)
+				if (!get32(&prev[q])) return false;
+			int p0 = 0, p1 = 0, p2 = 0;
+			switch (kind) {  // constructor arguments as the Restore* members choose them (impl/model_saver.h:557-800)
+			case kInput: case kFourier: case kTriangFourier: case kCrossEntropy: case kL2Out: case kSoftMax: p0 = in_len; break;
+			case kCrelu: case kGelu: case kHadamard: case kResidual: p0 = out_size; break;
+			case kEmbedding:
+				if (!get32(&p0) || !get32(&p1) || !get32(&p2)) return false;
+				break;
+			case kLinear: break;
+			default: return false;
+			}
+			if (kind == kLinear && (!get32(&p0) || !get32(&p1))) return false;
+			if (kind == kInput || kind == kEmbedding) {
+				int got = add(kind, p0, p1, p2, prev.data(), nprev, uid);
+				if (got != uid) return false;
+				Node *nd = at(uid);
+				if (!getf(nd->in.re, nd->in.n) || !getf(nd->in.im, nd->in.n)) return false;
+			} else if (add(kind, p0, p1, p2, prev.data(), nprev, uid) != uid) {
+				return false;
+			}
+		}
+		return true;
 	}
 	float loss(int uid, int label) {
 		Node *nd = at(uid);

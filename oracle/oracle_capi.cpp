@@ -79,6 +79,16 @@ void cno_net_set_tokens(void *h, int uid, const int *tok, int count) {
 void cno_net_forward(void *h) { ((Net *) h)->forward(); }
 void cno_net_backward(void *h, int label) { ((Net *) h)->backward(label); }
 void cno_net_update(void *h, float lr, int batch) { ((Net *) h)->update(lr, batch); }
+// .mod stream: returns the stream length; copies it when it fits into cap bytes
+long cno_net_save(void *h, char *buf, long cap) {
+	std::string blob = ((Net *) h)->save();
+	if ((long) blob.size() <= cap) memcpy(buf, blob.data(), blob.size());
+	return (long) blob.size();
+}
+int cno_net_restore(void *h, const char *buf, long len) { return ((Net *) h)->restore(std::string(buf, (size_t) len)) ? 1 : 0; }
+int cno_net_count(void *h) { return (int) ((Net *) h)->nodes().size(); }
+int cno_net_uid_at(void *h, int index) { return ((Net *) h)->nodes()[index]->uid; }
+int cno_net_kind(void *h, int uid) { return ((Net *) h)->at(uid)->kind; }
 void cno_net_adam_update(void *h, float lr, int batch, float beta, int t) { ((Net *) h)->adam_update_inputs(lr, batch, beta, t); }
 float cno_net_loss(void *h, int uid, int label) { return ((Net *) h)->loss(uid, label); }
 int cno_net_prediction(void *h, int uid) { return ((Net *) h)->prediction(uid); }

@@ -10,6 +10,7 @@
 
 #include "impl/cnet.h"
 #include "impl/batch.h"
+#include "impl/model_saver.h"
 
 #ifdef _OPENMP
 #include <omp.h>
@@ -99,6 +100,22 @@ void cno_net_backward(void *h, int label) {
 
 void cno_net_update(void *h, float lr, int batch) { ((RefNet *) h)->net.update(lr, batch); }
 
+long cno_net_save(void *h, char *buf, long cap) {
+	ModelSaver saver;
+	std::string blob = saver.SaveToString(((RefNet *) h)->net);
+	if ((long) blob.size() <= cap) memcpy(buf, blob.data(), blob.size());
+	return (long) blob.size();
+}
+int cno_net_restore(void *h, const char *buf, long len) {
+	ModelSaver saver;
+	RefNet *r = (RefNet *) h;
+	if (!saver.RestoreFromString(r->net, std::string(buf, (size_t) len))) return 0;
+	for (auto f : r->net.functionList()) r->kind_of[f->uid()] = f->getType();
+	return 1;
+}
+int cno_net_count(void *h) { return (int) ((RefNet *) h)->net.functionList().size(); }
+int cno_net_uid_at(void *h, int index) { return ((RefNet *) h)->net.functionList()[index]->uid(); }
+int cno_net_kind(void *h, int uid) { return ((RefNet *) h)->net[uid]->getType(); }
 void cno_net_adam_update(void *h, float lr, int batch, float beta, int t) { ((RefNet *) h)->net.adamUpdate(lr, batch, beta, t); }
 
 float cno_net_loss(void *h, int uid, int label) {

@@ -8,11 +8,14 @@
 //   facade_test persample          the per-sample API (forward / backward(label) / updateInputs) on the device
 //   facade_test embedding          CEmbedding -> Linear -> CrossEntropy with an EmbeddingBatch
 //   facade_test adam               TriangFourier / CRelu net trained with the Adam-style step, batched and per sample
+//   facade_test saved_model <golden dir> <scratch dir>   upstream-written .mod files restored and run on the device
 //   facade_test errors             error behaviour
 //   facade_test c4 n blocks B steps lr   throughput of the residual stack (no oracle), JSON line
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
+#include <fstream>
+#include <sstream>
 #include <string>
 
 #include "cnet_amd/host/cnet.hpp"
@@ -579,6 +582,128 @@ static void test_adam() {
 	}
 }
 
+// ------------------------------------------------------------------------------------------------- saved models
+// .mod files written by upstream's ModelSaver (tests/golden/*.mod): restore, run batched on the device, compare with the
+// oracle restored from the same bytes; then train one step on the device, save, and read the file back into the oracle.
+static std::string slurp(const std::string &path) {
+	std::ifstream in(path, std::ifstream::binary);
+	std::ostringstream all;
+	all << in.rdbuf();
+	return all.str();
+}
+
+static void test_saved_model(const std::string &dir, const std::string &tmp) {
+	ModelSaver saver;
+	{  // README net, 100 -> 10, batch of 5
+		const int n = 100, classes = 10, B = 5;
+		CNet net;
+		expect("restore readme_net.mod", net.restore(dir + "/readme_net.mod"));
+		orc::Net on;
+		expect("oracle restores the same file", on.restore(slurp(dir + "/readme_net.mod")));
+		CInput *cin = dynamic_cast<CInput *>(net.findFirstInput());
+		CrossEntropy *cen = dynamic_cast<CrossEntropy *>(net.findFirstOutput());
+		expect("restored net has its input and output", cin && cen && cin->input().length_ == n && cen->input().length_ == classes);
+		net.allocateOnGpu(B);
+		orc::Rng rng(77);
+		std::vector<float> xs((size_t) B * n), zeros(n, 0.f);
+		for (auto &v : xs) v = (float) rng.uniform();
+		InputBatch batch(B, n);
+		std::vector<int> labels(B);
+		for (int b = 0; b < B; ++b) {
+			labels[b] = (int) (rng.next() % classes);
+			batch.add(xs.data() + (size_t) b * n, zeros.data(), n, labels[b]);
+		}
+		net.gpuForward(cin, cen, batch);
+		net.getLoss(cen, &batch);
+		net.gpuBackward();
+		std::vector<int> pred = net.getPredictions(cen);
+		ErrAcc e_out;
+		double loss_err = 0;
+		int mism = 0;
+		const int o_in = cin->uid(), o_out = cen->uid();
+		for (int b = 0; b < B; ++b) {
+			std::copy(xs.begin() + (size_t) b * n, xs.begin() + (size_t) (b + 1) * n, on.at(o_in)->in.re);
+			on.forward();
+			loss_err = std::max(loss_err, (double) std::fabs(on.loss(o_out, labels[b]) - batch.loss(b)));
+			mism += on.prediction(o_out) != pred[b];
+			on.backward(labels[b]);
+			net.fetch(cen, b);
+			e_out.add(cen->mutableOutput()->real_, on.at(o_out)->out.re, 2 * classes);
+			on.at(o_in)->in.zero_gradients();
+		}
+		report("restored README net: normalised output", e_out.value());
+		report("restored README net: loss per sample", loss_err);
+		expect("restored README net: argmax bit-exact", mism == 0);
+		// one SGD step on the device, written to disk, read back by the oracle's reader
+		net.gpuUpdateInputs(0.05f / B);
+		on.update(0.05f, B);
+		net.getInputsFromGpu();
+		expect("save the device-trained net", net.save(tmp + "/trained.mod"));
+		orc::Net back;
+		expect("oracle reads the saved file", back.restore(slurp(tmp + "/trained.mod")));
+		ErrAcc w;
+		for (auto nd : on.nodes())
+			if (nd->kind == orc::kInput && nd->uid != o_in) w.add(back.at(nd->uid)->in.re, nd->in.re, 2 * nd->in.n);
+		report("weights in the saved file after the step", w.value(), TOL / 5);
+	}
+	{  // token net: embedding + positional parameter, every other function kind, two outputs
+		CNet net;
+		expect("restore token_net.mod", net.restore(dir + "/token_net.mod"));
+		orc::Net on;
+		on.restore(slurp(dir + "/token_net.mod"));
+		CEmbedding *emb = dynamic_cast<CEmbedding *>(net.findFirstInput());
+		CrossEntropy *cen = dynamic_cast<CrossEntropy *>(net.findFirstOutput());
+		L2Out *side = NULL;
+		for (auto f : net.functionList())
+			if (dynamic_cast<L2Out *>(f)) side = (L2Out *) f;
+		expect("restored token net has embedding, CrossEntropy and the L2Out branch", emb && cen && side);
+		const int slots = emb->noOutTokens(), vocab = emb->noEmbeddings(), dim = emb->embeddingDim(), B = 4;
+		emb->setInput({0});
+		net.allocateOnGpu(B);
+		std::vector<std::vector<int> > toks = {{3, 18, 0, 7, 7, 2}, {5, 1, 4}, {7}, {18, 18, 18, 18, 18}};
+		std::vector<int> labels = {3, 5, 0, 18};
+		EmbeddingBatch batch(B, slots);
+		for (int b = 0; b < B; ++b) batch.add(toks[b], labels[b]);
+		net.gpuForward(emb, cen, batch);
+		net.getLoss(cen, &batch);
+		std::vector<float> l2(B);
+		{
+			Batch tmpb;
+			net.getLoss(side, NULL);
+			for (int b = 0; b < B; ++b) {
+				net.fetch(side, b);
+				l2[b] = side->loss();
+			}
+		}
+		net.gpuBackward();
+		ErrAcc e_out, e_l2;
+		double loss_err = 0;
+		for (int b = 0; b < B; ++b) {
+			on.at(emb->uid())->tokens = toks[b];
+			on.forward();
+			loss_err = std::max(loss_err, (double) std::fabs(on.loss(cen->uid(), labels[b]) - batch.loss(b)));
+			float want = on.loss(side->uid(), 0);
+			e_l2.add(&l2[b], &want, 1);
+			on.backward(labels[b]);
+			net.fetch(cen, b);
+			e_out.add(cen->mutableOutput()->real_, on.at(cen->uid())->out.re, 2 * vocab);
+		}
+		report("restored token net: normalised output", e_out.value());
+		report("restored token net: CrossEntropy loss per sample", loss_err);
+		report("restored token net: L2Out branch loss", e_l2.value());
+		ErrAcc g_tab, g_par;
+		net.fetch(emb, 0);
+		g_tab.add(emb->input().dz_star_real_, on.at(emb->uid())->in.dzs_re, 2 * vocab * dim);
+		report("restored token net: embedding table dz* over the batch", g_tab.value());
+		for (auto f : net.inputs()) {
+			if (f == emb) continue;
+			net.fetch(f, 0);
+			g_par.add(f->input().dz_star_real_, on.at(f->uid())->in.dzs_re, 2 * f->input().length_);
+		}
+		report("restored token net: parameter dz* (positional input summed over rows, weights)", g_par.value());
+	}
+}
+
 // ------------------------------------------------------------------------------------------------- error behaviour
 template <class E, class F>
 static bool throws(F f) {
@@ -679,6 +804,7 @@ int main(int argc, char **argv) {
 		if (what == "persample" || what == "all") test_persample();
 		if (what == "embedding" || what == "all") test_embedding();
 		if (what == "adam" || what == "all") test_adam();
+		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
 		if (what == "errors" || what == "all") test_errors();
 		if (what == "c4")
 			run_c4(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048, argc > 5 ? atoi(argv[5]) : 10,

@@ -24,6 +24,10 @@ def main():
     for fn in recipes.SCENARIOS:
         for key, val in fn(ref).items():
             blob["%s/%s" % (fn.__name__, key)] = np.asarray(val)
+    # the two model streams also as files, for the readers that take a path
+    for name in ("readme", "token"):
+        with open(os.path.join(HERE, "%s_net.mod" % name), "wb") as f:
+            f.write(blob["model_files/%s_mod" % name].tobytes())
     path = os.path.join(HERE, "golden.npz")
     np.savez_compressed(path, **blob)
     print("wrote %s: %d arrays, %.1f KB" % (path, len(blob), os.path.getsize(path) / 1024))

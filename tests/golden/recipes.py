@@ -258,10 +258,86 @@ def embedding(lib):
     return rec
 
 
+def _mod_readme_net(lib, n=100, classes=10):
+    net = lib.net()
+    x = net.add(ob.INPUT, n)
+    f = net.add(ob.FOURIER, n, inputs=[x])
+    hw = net.add(ob.INPUT, n)
+    h = net.add(ob.HADAMARD, n, inputs=[f, hw])
+    g = net.add(ob.GELU, n, inputs=[h])
+    lw = net.add(ob.INPUT, n * classes)
+    lin = net.add(ob.LINEAR, n, n * classes, inputs=[g, lw])
+    ce = net.add(ob.CROSSENT, classes, inputs=[lin])
+    net.plane(hw, ob.RE)[:] = _rand(41, n) * 0.3 + 1; net.plane(hw, ob.IM)[:] = _rand(42, n) * 0.3
+    net.plane(lw, ob.RE)[:] = _rand(43, n * classes) * 0.1; net.plane(lw, ob.IM)[:] = _rand(44, n * classes) * 0.1
+    return net, x, ce
+
+
+def _mod_token_net(lib, dim=4, slots=6, vocab=19):
+    """Every remaining function kind in one graph: embedding + positional input -> Residual -> TriangFourier -> Linear ->
+    Residual -> SoftMax -> CRelu -> Hadamard -> logits Linear -> CrossEntropy, with an L2Out side branch."""
+    size = dim * slots
+    net = lib.net()
+    emb = net.add(ob.EMBEDDING, dim, slots, vocab)
+    pos = net.add(ob.INPUT, size)
+    r0 = net.add(ob.RESIDUAL, size, inputs=[emb, pos])
+    tf = net.add(ob.TRIANG_FOURIER, size, inputs=[r0])
+    w1 = net.add(ob.INPUT, size * size)
+    l1 = net.add(ob.LINEAR, size, size * size, inputs=[tf, w1])
+    r1 = net.add(ob.RESIDUAL, size, inputs=[tf, l1])
+    sm = net.add(ob.SOFTMAX, size, inputs=[r1])
+    cr = net.add(ob.CRELU, size, inputs=[sm])
+    hd = net.add(ob.INPUT, size)
+    h = net.add(ob.HADAMARD, size, inputs=[cr, hd])
+    w2 = net.add(ob.INPUT, size * vocab)
+    l2 = net.add(ob.LINEAR, size, size * vocab, inputs=[h, w2])
+    ce = net.add(ob.CROSSENT, vocab, inputs=[l2])
+    side = net.add(ob.L2OUT, size, inputs=[sm])
+    for k, uid in enumerate((emb, pos, w1, hd, w2)):
+        n = net.plane(uid, ob.RE).size
+        net.plane(uid, ob.RE)[:] = _rand(50 + 2 * k, n) * 0.5 + 0.3
+        net.plane(uid, ob.IM)[:] = _rand(51 + 2 * k, n) * 0.5 + 0.3
+    return net, emb, ce, side
+
+
+def model_files(lib):
+    """.mod streams as the backend writes them, and what a net restored from each computes on seeded inputs."""
+    rec = {}
+    net, x, ce = _mod_readme_net(lib)
+    blob = net.save()
+    rec["readme_mod"] = np.frombuffer(blob, np.uint8).copy()
+    back = lib.net()
+    assert back.restore(blob)
+    rec["readme_uids"] = np.asarray(back.uids(), np.int32)
+    rec["readme_x"] = np.abs(_rand(45, 3, 100))
+    for k in range(3):
+        back.plane(x, ob.RE)[:] = rec["readme_x"][k]; back.plane(x, ob.IM)[:] = 0
+        back.forward()
+        rec["readme_out%d" % k] = np.stack([back.plane(ce, ob.OUT_RE).copy(), back.plane(ce, ob.OUT_IM).copy()])
+        rec["readme_loss%d" % k] = np.float32(back.loss(ce, k))
+        rec["readme_pred%d" % k] = np.int32(back.prediction(ce))
+    net, emb, ce, side = _mod_token_net(lib)
+    blob = net.save()
+    rec["token_mod"] = np.frombuffer(blob, np.uint8).copy()
+    back = lib.net()
+    assert back.restore(blob)
+    rec["token_uids"] = np.asarray(back.uids(), np.int32)
+    rec["token_tokens"] = np.asarray([[3, 18, 0, 7, 7, 2], [5, 1, 4, -1, -1, -1]], np.int32)
+    for k in range(2):
+        row = rec["token_tokens"][k]
+        back.set_tokens(emb, row[row >= 0])
+        back.forward()
+        rec["token_out%d" % k] = np.stack([back.plane(ce, ob.OUT_RE).copy(), back.plane(ce, ob.OUT_IM).copy()])
+        rec["token_l2_%d" % k] = np.float32(back.loss(side, 0))
+        back.backward(int(row[0]))
+        rec["token_table_dzs%d" % k] = np.stack([back.plane(emb, ob.DZS_RE).copy(), back.plane(emb, ob.DZS_IM).copy()])
+    return rec
+
+
 def generators(lib):
     return dict(normal=lib.normal(2024, 257, 0.0, 1.0), uniform=lib.uniform(2024, 257, 0.0, 1.0))
 
 
 SCENARIOS = [linear, linear_fanout, fourier_pow2, fourier_784, fourier_12, hadamard, gelu, residual, softmax, crelu,
-             triang_fourier, adam_training,
+             triang_fourier, adam_training, model_files,
              fourier_rows_4096, losses, readme_net_training, residual_block_training, embedding, generators]

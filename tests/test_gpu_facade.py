@@ -57,6 +57,11 @@ def test_triang_fourier_crelu_net_with_adam_steps():
     assert "FAIL" not in out and out.count("PASS") > 30
 
 
+def test_upstream_model_files_restore_and_run_on_the_device(tmp_path):
+    out = _run("saved_model", os.path.join(ROOT, "tests", "golden"), str(tmp_path))
+    assert "FAIL" not in out and out.count("PASS") >= 16
+
+
 def test_error_behaviour():
     out = _run("errors")
     assert "FAIL" not in out
