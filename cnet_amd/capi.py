@@ -27,6 +27,15 @@ SIGNATURES = {
     "cnet_alloc": [C.c_size_t, C.POINTER(C.c_void_p)],
     "cnet_free": [C.c_void_p],
     "cnet_memcpy_h2d": [C.c_void_p, C.c_void_p, C.c_size_t],
+    "cnet_host_alloc": [C.c_size_t, C.POINTER(C.c_void_p)],
+    "cnet_host_free": [C.c_void_p],
+    "cnet_memcpy_h2d_async": [C.c_void_p, C.c_void_p, C.c_size_t],
+    "cnet_upload_async": [C.c_void_p, C.c_void_p, C.c_size_t],
+    "cnet_upload_wait_compute": [],
+    "cnet_mark_compute": [_i],
+    "cnet_upload_wait_marker": [_i],
+    "cnet_compute_wait_upload": [],
+    "cnet_upload_sync": [],
     "cnet_memcpy_d2h": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_memcpy_d2d": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_memset_zero": [C.c_void_p, C.c_size_t],

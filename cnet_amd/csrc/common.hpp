@@ -17,6 +17,12 @@ struct Runtime {
 	int device = -1;
 	hipStream_t own_stream = nullptr;
 	hipStream_t stream = nullptr;   // the stream in use (own_stream unless the caller supplied one)
+	// host -> device uploads that overlap compute run on their own stream (default priority, like the compute stream);
+	// the two events order the streams against each other
+	hipStream_t upload_stream = nullptr;
+	hipEvent_t upload_done = nullptr, compute_done = nullptr;
+	static constexpr int kMarkers = 8;
+	hipEvent_t marker[kMarkers] = {};  // caller-numbered points of the compute stream
 	hipDeviceProp_t prop;
 	// grow-only scratch for two-stage deterministic reductions (never allocated inside a hot loop twice
 	// for the same size)

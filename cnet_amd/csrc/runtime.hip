@@ -69,6 +69,10 @@ int cnet_init(int device) {
 		return fail(CNET_ERR_UNSUPPORTED, "cnet_init: kernels are built for gfx950 only, device is %s", r.prop.gcnArchName);
 	CNET_HIP(hipStreamCreateWithFlags(&r.own_stream, hipStreamNonBlocking));
 	r.stream = r.own_stream;
+	CNET_HIP(hipStreamCreateWithFlags(&r.upload_stream, hipStreamNonBlocking));
+	CNET_HIP(hipEventCreateWithFlags(&r.upload_done, hipEventDisableTiming));
+	CNET_HIP(hipEventCreateWithFlags(&r.compute_done, hipEventDisableTiming));
+	for (auto &m : r.marker) CNET_HIP(hipEventCreateWithFlags(&m, hipEventDisableTiming));
 	r.device = device;
 	r.ready = true;
 	return CNET_OK;
@@ -82,6 +86,17 @@ int cnet_shutdown(void) {
 	if (r.workspace) hipFree(r.workspace);
 	r.workspace = nullptr;
 	r.workspace_bytes = 0;
+	if (r.upload_stream) {
+		hipStreamSynchronize(r.upload_stream);
+		hipStreamDestroy(r.upload_stream);
+		hipEventDestroy(r.upload_done);
+		hipEventDestroy(r.compute_done);
+		for (auto &m : r.marker) {
+			hipEventDestroy(m);
+			m = nullptr;
+		}
+		r.upload_stream = nullptr;
+	}
 	if (r.own_stream) hipStreamDestroy(r.own_stream);
 	r.own_stream = r.stream = nullptr;
 	r.ready = false;
@@ -147,6 +162,76 @@ int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes) {
 	// pageable source: hipMemcpyAsync stages and returns after the copy was consumed from the host buffer
 	CNET_HIP(hipMemcpyAsync(dst, host_src, bytes, hipMemcpyHostToDevice, rt().stream));
 	CNET_HIP(hipStreamSynchronize(rt().stream));
+	return CNET_OK;
+}
+
+int cnet_host_alloc(size_t bytes, void **out) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(out != nullptr);
+	*out = nullptr;
+	if (bytes == 0) return CNET_OK;
+	CNET_HIP(hipHostMalloc(out, bytes, hipHostMallocDefault));
+	return CNET_OK;
+}
+
+int cnet_host_free(void *ptr) {
+	CNET_REQUIRE_INIT();
+	if (!ptr) return CNET_OK;
+	// copies queued from this buffer must have left it
+	CNET_HIP(hipStreamSynchronize(rt().stream));
+	CNET_HIP(hipStreamSynchronize(rt().upload_stream));
+	CNET_HIP(hipHostFree(ptr));
+	return CNET_OK;
+}
+
+int cnet_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes) {
+	CNET_REQUIRE_INIT();
+	if (!bytes) return CNET_OK;
+	CNET_CHECK_ARG(dst && pinned_src);
+	CNET_HIP(hipMemcpyAsync(dst, pinned_src, bytes, hipMemcpyHostToDevice, rt().stream));
+	return CNET_OK;
+}
+
+int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes) {
+	CNET_REQUIRE_INIT();
+	if (!bytes) return CNET_OK;
+	CNET_CHECK_ARG(dst && pinned_src);
+	CNET_HIP(hipMemcpyAsync(dst, pinned_src, bytes, hipMemcpyHostToDevice, rt().upload_stream));
+	return CNET_OK;
+}
+
+int cnet_upload_wait_compute(void) {
+	CNET_REQUIRE_INIT();
+	CNET_HIP(hipEventRecord(rt().compute_done, rt().stream));
+	CNET_HIP(hipStreamWaitEvent(rt().upload_stream, rt().compute_done, 0));
+	return CNET_OK;
+}
+
+int cnet_mark_compute(int marker) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(marker >= 0 && marker < Runtime::kMarkers);
+	CNET_HIP(hipEventRecord(rt().marker[marker], rt().stream));
+	return CNET_OK;
+}
+
+int cnet_upload_wait_marker(int marker) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(marker >= 0 && marker < Runtime::kMarkers);
+	// a marker that was never set does not hold anything back
+	CNET_HIP(hipStreamWaitEvent(rt().upload_stream, rt().marker[marker], 0));
+	return CNET_OK;
+}
+
+int cnet_compute_wait_upload(void) {
+	CNET_REQUIRE_INIT();
+	CNET_HIP(hipEventRecord(rt().upload_done, rt().upload_stream));
+	CNET_HIP(hipStreamWaitEvent(rt().stream, rt().upload_done, 0));
+	return CNET_OK;
+}
+
+int cnet_upload_sync(void) {
+	CNET_REQUIRE_INIT();
+	CNET_HIP(hipStreamSynchronize(rt().upload_stream));
 	return CNET_OK;
 }
 

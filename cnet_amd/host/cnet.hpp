@@ -169,24 +169,95 @@ public:
 	int label(int i) { return labels_[i]; }
 };
 
+// Two [batch x dim] planes in page-locked host memory when the device library is initialised (pageable otherwise), so
+// a batch goes to the device as one asynchronous copy per plane (upstream: two pageable copies per sample,
+// gpu/gpu_func.h:403-419).  Movable and reusable: clear() empties it for the next fill without giving the memory back.
 class InputBatch : public Batch {
-	std::vector<float> real_data_, imag_data_;
+	friend class CNet;
+	float *real_data_ = NULL, *imag_data_ = NULL;  // [batch][dim] each, one allocation
+	bool pinned_ = false;
+	bool in_flight_ = false;  // an upload queued from these planes may not have finished
+
+	void allocate() {
+		const size_t bytes = 2 * (size_t) batch_size_ * sample_dim_ * sizeof(float);
+		if (!bytes) return;
+		void *p = NULL;
+		if (cnet_host_alloc(bytes, &p) == CNET_OK && p) {
+			pinned_ = true;
+		} else {
+			p = ::operator new(bytes);
+			pinned_ = false;
+		}
+		real_data_ = (float *) p;
+		imag_data_ = real_data_ + (size_t) batch_size_ * sample_dim_;
+	}
+	void release() {
+		if (!real_data_) return;
+		if (pinned_) cnet_host_free(real_data_);  // waits for copies still reading it
+		else ::operator delete(real_data_);
+		real_data_ = imag_data_ = NULL;
+	}
+	void settle() {  // before the host writes the planes again
+		if (in_flight_) {
+			cnet_upload_sync();
+			cnet_sync();
+			in_flight_ = false;
+		}
+	}
+	float *rowRe() { return real_data_ + (size_t) current_pos_ * sample_dim_; }
+	float *rowIm() { return imag_data_ + (size_t) current_pos_ * sample_dim_; }
+	void finishRow(int filled, int label) {
+		std::fill(rowRe() + filled, rowRe() + sample_dim_, 0.f);  // padding with 0s
+		std::fill(rowIm() + filled, rowIm() + sample_dim_, 0.f);
+		labels_.push_back(label);
+		sizes_.push_back(filled);
+		current_pos_++;
+	}
+
 public:
 	InputBatch() : Batch() {}
-	InputBatch(int batch_size, int sample_dim) : Batch(batch_size, sample_dim) {}
+	InputBatch(int batch_size, int sample_dim) : Batch(batch_size, sample_dim) { allocate(); }
+	InputBatch(const InputBatch &o) : Batch(o) {
+		allocate();
+		if (o.real_data_) std::copy(o.real_data_, o.real_data_ + 2 * (size_t) batch_size_ * sample_dim_, real_data_);
+	}
+	InputBatch(InputBatch &&o) noexcept : Batch(std::move(o)), real_data_(o.real_data_), imag_data_(o.imag_data_), pinned_(o.pinned_),
+			in_flight_(o.in_flight_) {
+		o.real_data_ = o.imag_data_ = NULL;
+	}
+	InputBatch &operator=(InputBatch &&o) noexcept {
+		if (this != &o) {
+			release();
+			Batch::operator=(std::move(o));
+			real_data_ = o.real_data_;
+			imag_data_ = o.imag_data_;
+			pinned_ = o.pinned_;
+			in_flight_ = o.in_flight_;
+			o.real_data_ = o.imag_data_ = NULL;
+		}
+		return *this;
+	}
+	InputBatch &operator=(const InputBatch &) = delete;
+	~InputBatch() override { release(); }
+
+	bool isPinned() const { return pinned_; }
+	// empty the batch for refilling; the planes are kept
+	void clear() {
+		settle();
+		losses_.clear();
+		labels_.clear();
+		sizes_.clear();
+		current_pos_ = 0;
+	}
 	void add(const std::vector<std::complex<float> > &sample, int label) {
-		assert(current_pos_ < batch_size_);
-		for (auto c : sample) {
-			real_data_.push_back(c.real());
-			imag_data_.push_back(c.imag());
+		assert(current_pos_ < batch_size_ && (int) sample.size() <= sample_dim_);
+		settle();
+		float *re = rowRe(), *im = rowIm();
+		for (size_t k = 0; k < sample.size(); ++k) {
+			re[k] = sample[k].real();
+			im[k] = sample[k].imag();
 		}
-		while (real_data_.size() < (size_t) (1 + current_pos_) * sample_dim_) {  // padding with 0s
-			real_data_.push_back(0.f);
-			imag_data_.push_back(0.f);
-		}
-		labels_.push_back(label);
-		sizes_.push_back((int) sample.size());
-		current_pos_++;
+		finishRow((int) sample.size(), label);
 	}
 	void add(std::initializer_list<std::complex<float> > list, int label) {
 		add(std::vector<std::complex<float> >(list), label);
@@ -194,18 +265,15 @@ public:
 	// bulk variant for callers that already hold the two planes of one sample
 	void add(const float *re, const float *im, int n, int label) {
 		assert(current_pos_ < batch_size_ && n <= sample_dim_);
-		real_data_.insert(real_data_.end(), re, re + n);
-		imag_data_.insert(imag_data_.end(), im, im + n);
-		real_data_.resize((size_t) (1 + current_pos_) * sample_dim_, 0.f);
-		imag_data_.resize((size_t) (1 + current_pos_) * sample_dim_, 0.f);
-		labels_.push_back(label);
-		sizes_.push_back(n);
-		current_pos_++;
+		settle();
+		std::copy(re, re + n, rowRe());
+		std::copy(im, im + n, rowIm());
+		finishRow(n, label);
 	}
-	const float *realDataPtr() const { return &real_data_[0]; }
-	const float *imagDataPtr() const { return &imag_data_[0]; }
-	const float *realDataPtr(int b) const { return &real_data_[0] + (size_t) b * sample_dim_; }
-	const float *imagDataPtr(int b) const { return &imag_data_[0] + (size_t) b * sample_dim_; }
+	const float *realDataPtr() const { return real_data_; }
+	const float *imagDataPtr() const { return imag_data_; }
+	const float *realDataPtr(int b) const { return real_data_ + (size_t) b * sample_dim_; }
+	const float *imagDataPtr(int b) const { return imag_data_ + (size_t) b * sample_dim_; }
 };
 
 class EmbeddingBatch : public Batch {
@@ -274,6 +342,7 @@ protected:
 		CFunc *producer = NULL;
 		int offset = 0, len = 0, rows = 0;
 		float *grad = NULL;  // 4 planes [rows][len]
+		float *z = NULL;     // input functions only: their own 2 value planes [rows][len] (the parameter, the data batch, the table)
 		float *g(int plane) const { return grad + (size_t) plane * rows * len; }
 	};
 	std::vector<Slot> slots_;
@@ -512,6 +581,16 @@ class CNet {
 	CFunc *main_input_ = NULL;
 	int32_t *d_labels_ = NULL;
 	std::vector<int> labels_;
+	// device double buffer of the data input: stage_[active_] is what the kernels read, the other one can be filled by
+	// gpuPrefetch() meanwhile
+	struct Stage {
+		float *z = NULL;            // 2 planes [batch][len]
+		int32_t *labels = NULL;     // [batch]
+		int32_t *host_labels = NULL;  // page-locked staging of the labels
+		const InputBatch *holds = NULL;
+	};
+	Stage stage_[2];
+	int active_ = 0;
 
 	static void ck(int rc, const char *what) {
 		if (rc != CNET_OK)
@@ -567,7 +646,10 @@ public:
 	// ---- graph construction (impl/cnet.h:228-289) ----
 	int add(CFunc *func) {
 		assert(func);
-		if (batch_) throw std::logic_error("add: the net is already allocated on the GPU");
+		if (batch_) {
+			delete func;  // the net owns what it is given, also when it refuses it
+			throw std::logic_error("add: the net is already allocated on the GPU");
+		}
 		if (func->uid_ == 0) func->uid_ = ++next_uid_;
 		else next_uid_ = std::max(next_uid_, func->uid_);
 		func->type_ = func->typeId();
@@ -664,6 +746,11 @@ public:
 		}
 		batch_ = 0;
 		d_labels_ = NULL;
+		for (auto &st : stage_) {
+			if (st.host_labels) cnet_host_free(st.host_labels);
+			st = Stage();
+		}
+		active_ = 0;
 	}
 
 	int batchSize() const { return batch_; }
@@ -693,6 +780,7 @@ private:
 				s.len = f->input().length_;
 				s.rows = (int) rows;
 				s.grad = six + 2 * rows * s.len;
+				s.z = six;
 				f->slots_.push_back(s);
 				ck(cnet_memset_zero(six, 6 * rows * s.len * sizeof(float)), "zero");
 			} else if (t == isEmbedding) {
@@ -702,6 +790,7 @@ private:
 				s.len = f->input().length_;
 				s.rows = 1;
 				s.grad = six + 2 * (size_t) s.len;
+				s.z = six;
 				f->slots_.push_back(s);
 				ck(cnet_memset_zero(six, 6 * (size_t) s.len * sizeof(float)), "zero");
 				e->d_tokens_ = dalloc<int32_t>(rows * e->no_out_tokens_);
@@ -761,6 +850,10 @@ private:
 		}
 		d_labels_ = dalloc<int32_t>(batch_);
 		ck(cnet_memset_zero(d_labels_, batch_ * sizeof(int32_t)), "zero");
+		if (main_input_->typeId() == isInput) {
+			stage_[0].z = main_input_->slots_[0].z;
+			stage_[0].labels = d_labels_;
+		}
 		copyInputsToGpu();
 	}
 
@@ -781,7 +874,7 @@ private:
 		case isInput: break;  // consumers read the node's z planes in place
 		case isEmbedding: {
 			CEmbedding *e = (CEmbedding *) f;
-			const float *tab = f->slots_[0].grad - 2 * (size_t) f->slots_[0].len;
+			const float *tab = f->slots_[0].z;
 			ck(cnet_embedding_fwd(tab, tab + f->slots_[0].len, e->embedding_dim_, e->no_embeddings_, e->d_tokens_, f->out_re(),
 					f->out_im(), f->out_size_, rows, e->no_out_tokens_), "cnet_embedding_fwd");
 			break;
@@ -957,7 +1050,7 @@ public:
 		requireAllocated("copyInputsToGpu");
 		for (auto f : inputs_) {
 			CFunc::Slot &s = f->slots_[0];
-			float *z = s.grad - 2 * (size_t) s.rows * s.len;
+			float *z = s.z;
 			if (s.rows == 1) {
 				ck(cnet_memcpy_h2d(z, f->mutable_input()->real_, 2 * (size_t) s.len * sizeof(float)), "cnet_memcpy_h2d");
 			} else {  // the data input: the host view holds one sample, replicate it to every row
@@ -991,7 +1084,7 @@ public:
 				z_re = s.producer->out_re() + (size_t) (s.producer->rows_ == 1 ? 0 : b) * s.len;
 				z_im = s.producer->out_im() + (size_t) (s.producer->rows_ == 1 ? 0 : b) * s.len;
 			} else {
-				const float *z = s.grad - 2 * (size_t) s.rows * s.len;
+				const float *z = s.z;
 				z_re = z + (size_t) row * s.len;
 				z_im = z + (size_t) (s.rows + row) * s.len;
 			}
@@ -1027,12 +1120,69 @@ public:
 		if (batch.sampleDim() != cin->input().length_) throw std::invalid_argument("gpuForward: sample dimension differs from the input length");
 		(void) outp;
 		CFunc::Slot &s = cin->slots_[0];
-		float *z = s.grad - 2 * (size_t) s.rows * s.len;
+		Stage &staged = stage_[1 - active_];
+		if (staged.holds == &batch) {
+			// the batch was sent ahead by gpuPrefetch(): switch the data input to the buffer it landed in.  Everything
+			// queued so far may still read the buffer in use, so its retirement point is remembered for the next refill.
+			checkLabels(batch.labelsPtr(), batch_);
+			ck(cnet_compute_wait_upload(), "cnet_compute_wait_upload");
+			ck(cnet_mark_compute(active_), "cnet_mark_compute");
+			active_ = 1 - active_;
+			staged.holds = NULL;
+			cin->out_ = staged.z;
+			s.z = staged.z;
+			d_labels_ = staged.labels;
+			labels_.assign(batch.labelsPtr(), batch.labelsPtr() + batch_);
+			return GpuForward();
+		}
+		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
 		// one copy per plane (upstream: two small copies per sample, gpu/gpu_func.h:403-419)
-		ck(cnet_memcpy_h2d(z, batch.realDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
-		ck(cnet_memcpy_h2d(z + (size_t) batch_ * s.len, batch.imagDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
+		if (batch.isPinned()) {
+			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d_async");
+			ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
+			batch.in_flight_ = true;
+		} else {
+			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d");
+			ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
+		}
 		setLabels(batch.labelsPtr(), batch_);
 		return GpuForward();
+	}
+	// Send the NEXT batch to the device on the upload stream while the kernels of the current step run; the later
+	// gpuForward(inp, outp, batch) with the same batch object then only switches buffers.  The data input is double
+	// buffered on the device (the second buffer is allocated on the first call); at most one batch can be staged.  The
+	// batch must be page-locked (built after the device library was initialised) and must not be refilled before its
+	// gpuForward; clear() / add() on it wait for the copy.
+	void gpuPrefetch(InputFunc *inp, InputBatch &batch) {
+		requireAllocated("gpuPrefetch");
+		CInput *cin = dynamic_cast<CInput *>(inp);
+		if (!cin || cin != main_input_) throw std::invalid_argument("gpuPrefetch: not the main input of the allocated net");
+		if (batch.size() != batch_ || batch.noOfLabels() != batch_ || batch.sampleDim() != cin->input().length_)
+			throw std::invalid_argument("gpuPrefetch: batch shape differs from the allocated net");
+		if (!batch.isPinned()) throw std::invalid_argument("gpuPrefetch: the batch is not in page-locked memory");
+		checkLabels(batch.labelsPtr(), batch_);
+		const int other = 1 - active_;
+		Stage &st = stage_[other];
+		if (st.holds) throw std::logic_error("gpuPrefetch: a staged batch is still waiting for its gpuForward");
+		CFunc::Slot &s = cin->slots_[0];
+		const size_t plane = (size_t) batch_ * s.len;
+		if (!st.z) {
+			st.z = dalloc<float>(2 * plane);
+			st.labels = dalloc<int32_t>(batch_);
+		}
+		if (!st.host_labels) {
+			void *h = NULL;
+			ck(cnet_host_alloc(batch_ * sizeof(int32_t), &h), "cnet_host_alloc");
+			st.host_labels = (int32_t *) h;
+		}
+		ck(cnet_upload_sync(), "cnet_upload_sync");  // the previous upload has left host_labels
+		std::copy(batch.labelsPtr(), batch.labelsPtr() + batch_, st.host_labels);
+		ck(cnet_upload_wait_marker(other), "cnet_upload_wait_marker");  // kernels of the step that last used this buffer
+		ck(cnet_upload_async(st.z, batch.realDataPtr(), plane * sizeof(float)), "cnet_upload_async");
+		ck(cnet_upload_async(st.z + plane, batch.imagDataPtr(), plane * sizeof(float)), "cnet_upload_async");
+		ck(cnet_upload_async(st.labels, st.host_labels, batch_ * sizeof(int32_t)), "cnet_upload_async");
+		batch.in_flight_ = true;
+		st.holds = &batch;
 	}
 	// upload a batch into a CInput flagged with setIsBatched(true); labels of that batch are ignored
 	void gpuSetInput(CInput *cin, InputBatch &batch) {
@@ -1040,9 +1190,8 @@ public:
 		if (cin->rows_ != batch_ || batch.size() != batch_ || batch.sampleDim() != cin->input().length_)
 			throw std::invalid_argument("gpuSetInput: " + cin->getName() + " is not a data input of this batch shape");
 		CFunc::Slot &s = cin->slots_[0];
-		float *z = s.grad - 2 * (size_t) s.rows * s.len;
-		ck(cnet_memcpy_h2d(z, batch.realDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
-		ck(cnet_memcpy_h2d(z + (size_t) batch_ * s.len, batch.imagDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
+		ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
+		ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
 	}
 	bool gpuForward(InputFunc *inp, OutputFunc *outp, EmbeddingBatch &batch) {
 		requireAllocated("gpuForward");
@@ -1071,7 +1220,7 @@ public:
 		for (auto f : inputs_) {
 			CFunc::Slot &s = f->slots_[0];
 			const size_t n = (size_t) s.rows * s.len;
-			float *z = s.grad - 2 * n;
+			float *z = s.z;
 			ck(cnet_sgd_update(z, z + n, s.g(2), s.g(3), (int64_t) n, l_rate, 1), "cnet_sgd_update");
 			ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
 		}
@@ -1083,7 +1232,7 @@ public:
 		for (auto f : inputs_) {
 			CFunc::Slot &s = f->slots_[0];
 			const size_t n = (size_t) s.rows * s.len;
-			float *z = s.grad - 2 * n;
+			float *z = s.z;
 			ck(cnet_adam_update(z, z + n, s.g(0), s.g(1), s.g(2), s.g(3), (int64_t) n, l_rate, beta, t, 1), "cnet_adam_update");
 		}
 	}
@@ -1111,13 +1260,16 @@ public:
 		ck(cnet_memcpy_d2h(tmp.data(), c->d_argmax_, tmp.size() * sizeof(int32_t)), "cnet_memcpy_d2h");
 		return std::vector<int>(tmp.begin(), tmp.end());
 	}
-	void setLabels(const int *labels, int count) {
-		requireAllocated("setLabels");
+	void checkLabels(const int *labels, int count) {
 		if (count != batch_) throw std::invalid_argument("setLabels: one label per batch row");
 		for (auto f : outputs_)
 			if (f->typeId() == isCrossEntropy)
 				for (int k = 0; k < count; ++k)
 					if (labels[k] < 0 || labels[k] >= f->input().length_) throw std::out_of_range("setLabels: label outside the CrossEntropy input");
+	}
+	void setLabels(const int *labels, int count) {
+		requireAllocated("setLabels");
+		checkLabels(labels, count);
 		labels_.assign(labels, labels + count);
 		ck(cnet_memcpy_h2d(d_labels_, labels, count * sizeof(int32_t)), "cnet_memcpy_h2d");
 	}

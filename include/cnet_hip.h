@@ -60,6 +60,29 @@ int cnet_sync(void);
 int cnet_alloc(size_t bytes, void **out);  /* float_allocate_on_gpu & friends (gpu/allocator.h:121-180) */
 int cnet_free(void *ptr);
 int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes);   /* *_copy_to_gpu   (gpu/allocator.h:182-260) */
+/* ---- Host batch pipeline: replaces the per-sample copies of GpuNet::batchToGpu (gpu/gpu_func.h:368-427: two pageable
+ *      cudaMemcpy per sample) with page-locked [B x dim] planes, one asynchronous copy per plane, and an upload stream
+ *      that runs ahead of the compute stream.
+ * cnet_host_alloc / cnet_host_free: page-locked host memory (hipHostMalloc).
+ * cnet_memcpy_h2d_async: copy on the compute stream, returns at once; the source must be page-locked and stay
+ *      untouched until the stream reaches the copy (cnet_sync, or any later blocking call).
+ * cnet_upload_async: the same on the library's upload stream, so it overlaps kernels of the compute stream.
+ * cnet_upload_wait_compute: uploads queued after this call start only when everything queued on the compute stream so
+ *      far has finished (call before overwriting a device buffer that kernels may still read).
+ * cnet_mark_compute(m) / cnet_upload_wait_marker(m), m = 0..7: the same in two halves - remember the current tail of the
+ *      compute stream under number m now, make later uploads wait for that point when a buffer is about to be refilled
+ *      (double buffering: the marker is set when a buffer is retired, the wait is issued when it is reused).
+ * cnet_compute_wait_upload: kernels queued after this call start only when every upload queued so far has landed.
+ * cnet_upload_sync: host waits for the upload stream (before reusing a page-locked source buffer). */
+int cnet_host_alloc(size_t bytes, void **host_ptr);
+int cnet_host_free(void *host_ptr);
+int cnet_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
+int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes);
+int cnet_upload_wait_compute(void);
+int cnet_mark_compute(int marker);
+int cnet_upload_wait_marker(int marker);
+int cnet_compute_wait_upload(void);
+int cnet_upload_sync(void);
 int cnet_memcpy_d2h(void *host_dst, const void *src, size_t bytes);   /* *_copy_from_gpu (gpu/allocator.h:262-328); synchronises */
 int cnet_memcpy_d2d(void *dst, const void *src, size_t bytes);
 int cnet_memset_zero(void *dst, size_t bytes);  /* GpuMapping::zeroGradients (gpu/kernels.cpp:444-469) */

@@ -9,6 +9,8 @@
 //   facade_test embedding          CEmbedding -> Linear -> CrossEntropy with an EmbeddingBatch
 //   facade_test adam               TriangFourier / CRelu net trained with the Adam-style step, batched and per sample
 //   facade_test saved_model <golden dir> <scratch dir>   upstream-written .mod files restored and run on the device
+//   facade_test pipeline [B steps]  reader -> page-locked batches -> device, with and without gpuPrefetch (same bits)
+//   facade_test pipeline_timing B steps   the same, timing only (JSON line)
 //   facade_test errors             error behaviour
 //   facade_test c4 n blocks B steps lr   throughput of the residual stack (no oracle), JSON line
 #include <chrono>
@@ -19,6 +21,7 @@
 #include <string>
 
 #include "cnet_amd/host/cnet.hpp"
+#include "cnet_amd/host/data.hpp"
 #include "oracle/cnet_oracle.hpp"
 
 static int g_fail = 0;
@@ -704,6 +707,123 @@ static void test_saved_model(const std::string &dir, const std::string &tmp) {
 	}
 }
 
+// ------------------------------------------------------------------------------------------------- host batch pipeline
+// README net fed from a BatchedDataReader: (a) every batch copied inside gpuForward, (b) batches sent ahead with
+// gpuPrefetch() into the device double buffer while the previous step computes.  Both must give the same bits.
+static void build_readme(CNet &net, int n, int classes, int *inp, int *outp) {
+	*inp = net.add(new CInput(OutSize(n)));
+	auto fft = net.add(new FourierTrans(InSize(n)), {*inp});
+	auto h_data = net.add(new CInput(OutSize(n)));
+	auto hdm = net.add(new Hadamard(InSize(n), InSize(n)), {fft, h_data});
+	auto gelu = net.add(new CGelu(InSize(n)), {hdm});
+	auto l_data = net.add(new CInput(OutSize(n * classes)));
+	auto lin = net.add(new Linear(InSize(n), InSize(n * classes)), {gelu, l_data});
+	*outp = net.add(new CrossEntropy(InSize(classes)), {lin});
+	net.init_inputs(11);
+}
+
+struct SyntheticReader : public BatchedDataReader {
+	SyntheticReader(int dim, int count, int classes) : BatchedDataReader(dim) {
+		orc::Rng rng(123);
+		std::vector<float> re(dim), im(dim);
+		reserve(count);
+		for (int s = 0; s < count; ++s) {
+			for (int k = 0; k < dim; ++k) {
+				re[k] = (float) rng.uniform();
+				im[k] = (float) rng.uniform();
+			}
+			addPlanes(re.data(), im.data(), (int) (rng.next() % classes));
+		}
+	}
+	bool readData() override { return true; }
+};
+
+static void test_pipeline(int B, int steps, bool timing_only) {
+	const int n = 784, classes = 10;
+	const float lr = 0.01f;
+	if (cnet_init(0) != CNET_OK) {
+		expect("cnet_init", false);
+		return;
+	}
+	SyntheticReader data(n, 3 * B + 7, classes);
+	std::vector<float> losses[2];
+	std::vector<float> weights[2];
+	double ms[2] = {0, 0};
+	for (int mode = 0; mode < 2; ++mode) {
+		CNet net;
+		int inp, outp;
+		build_readme(net, n, classes, &inp, &outp);
+		net.allocateOnGpu(B);
+		CInput *cin = (CInput *) net[inp];
+		CrossEntropy *cen = (CrossEntropy *) net[outp];
+		SyntheticReader reader = data;  // same order for both modes
+		InputBatch ring[3] = {InputBatch(B, n), InputBatch(B, n), InputBatch(B, n)};
+		if (mode == 0 && !timing_only) expect("batches built after cnet_init are page-locked", ring[0].isPinned());
+		net.sync();
+		auto t0 = std::chrono::steady_clock::now();
+		if (mode == 1) {
+			reader.nextBatch(ring[0]);
+			net.gpuPrefetch(cin, ring[0]);
+		}
+		for (int s = 0; s < steps; ++s) {
+			InputBatch &cur = ring[s % 3];
+			if (mode == 0) reader.nextBatch(cur);
+			net.gpuForward(cin, cen, cur);
+			if (mode == 1 && s + 1 < steps) {  // the next batch travels while this step computes
+				InputBatch &next = ring[(s + 1) % 3];
+				reader.nextBatch(next);
+				net.gpuPrefetch(cin, next);
+			}
+			losses[mode].push_back(net.getLoss(cen, &cur));
+			net.gpuBackward();
+			net.gpuUpdateInputs(lr / B);
+		}
+		net.sync();
+		ms[mode] = 1e3 * std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / steps;
+		net.getInputsFromGpu();
+		for (auto f : net.inputs()) {
+			if (f == cin) continue;
+			weights[mode].insert(weights[mode].end(), f->input().real_, f->input().real_ + 2 * f->input().length_);
+		}
+		if (mode == 1 && !timing_only) {
+			// error behaviour of the staging
+			InputBatch a(B, n), b(B, n);
+			reader.nextBatch(a);
+			reader.nextBatch(b);
+			net.gpuPrefetch(cin, a);
+			bool threw = false;
+			try {
+				net.gpuPrefetch(cin, b);
+			} catch (const std::logic_error &) {
+				threw = true;
+			}
+			expect("a second staged batch is refused until the first was consumed", threw);
+			net.gpuForward(cin, cen, b);  // a batch that was not staged takes the direct path; the staged one stays
+			net.gpuForward(cin, cen, a);
+			float la = net.getLoss(cen, NULL);
+			net.gpuForward(cin, cen, a);  // again, now through the direct path
+			expect("staged and direct upload of the same batch give the same loss", la == net.getLoss(cen, NULL));
+			InputBatch wrong(B, n - 1);
+			threw = false;
+			try {
+				net.gpuPrefetch(cin, wrong);
+			} catch (const std::invalid_argument &) {
+				threw = true;
+			}
+			expect("a batch of the wrong shape is refused", threw);
+		}
+	}
+	if (!timing_only) {
+		expect("losses identical with and without prefetch (" + std::to_string(steps) + " steps)", losses[0] == losses[1]);
+		expect("weights identical after training with and without prefetch", weights[0] == weights[1] && !weights[0].empty());
+		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
+	}
+	printf("{\"workload\": \"README net 784 -> 10, SGD, batches from a BatchedDataReader\", \"batch\": %d, \"steps\": %d, "
+		   "\"ms_per_step_copy_in_forward\": %.3f, \"ms_per_step_prefetch\": %.3f, \"samples_per_sec_copy_in_forward\": %.1f, "
+		   "\"samples_per_sec_prefetch\": %.1f, \"upload_bytes_per_step\": %zu}\n",
+			B, steps, ms[0], ms[1], B / ms[0] * 1e3, B / ms[1] * 1e3, (size_t) 2 * B * n * sizeof(float));
+}
+
 // ------------------------------------------------------------------------------------------------- error behaviour
 template <class E, class F>
 static bool throws(F f) {
@@ -797,6 +917,7 @@ static void run_c4(int n, int blocks, int B, int steps, float lr) {
 
 int main(int argc, char **argv) {
 	std::string what = argc > 1 ? argv[1] : "all";
+	setvbuf(stdout, NULL, _IOLBF, 0);  // keep the log complete if a scenario dies
 	try {
 		if (what == "mnist" || what == "all") test_mnist(true);
 		if (what == "mnist_cpu_operator" || what == "all") test_mnist(false);
@@ -805,6 +926,8 @@ int main(int argc, char **argv) {
 		if (what == "embedding" || what == "all") test_embedding();
 		if (what == "adam" || what == "all") test_adam();
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
+		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 7, false);
+		if (what == "pipeline_timing") test_pipeline(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, true);
 		if (what == "errors" || what == "all") test_errors();
 		if (what == "c4")
 			run_c4(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048, argc > 5 ? atoi(argv[5]) : 10,

@@ -6,6 +6,7 @@
 #include <sstream>
 
 #include "cnet_amd/host/cnet.hpp"
+#include "cnet_amd/host/data.hpp"
 #include "oracle/cnet_oracle.hpp"
 
 static int g_fail = 0;
@@ -91,6 +92,64 @@ int main(int argc, char **argv) {
 		expect("unknown type id is refused", !saver.RestoreFromString(n3, bad));
 		expect("missing file is refused", !saver.Restore(n4, tmp + "/does_not_exist.mod"));
 		expect("empty string is refused", !saver.RestoreFromString(n4, ""));
+	}
+	{  // MNIST idx reader and batching (upstream data/data.h:28-165), host only: the batch planes are pageable here
+		const int count = 10;
+		std::string img = tmp + "/images.idx3-ubyte", lab = tmp + "/labels.idx1-ubyte";
+		{
+			std::ofstream fi(img, std::ofstream::binary), fl(lab, std::ofstream::binary);
+			const unsigned char hi[16] = {0, 0, 8, 3, 0, 0, 0, 10, 0, 0, 0, 28, 0, 0, 0, 28}, hl[8] = {0, 0, 8, 1, 0, 0, 0, 10};
+			fi.write((const char *) hi, 16);
+			fl.write((const char *) hl, 8);
+			for (int s = 0; s < count; ++s) {
+				for (int k = 0; k < 784; ++k) fi.put((char) (unsigned char) ((s * 31 + k * 7) & 255));
+				fl.put((char) (s % 10));
+			}
+		}
+		MnistDataReader reader;
+		expect("MNIST reader: missing file is refused", !reader.Open(tmp + "/nope", lab, count));
+		expect("MNIST reader: asking for more samples than the file holds is refused", !reader.Open(img, lab, count + 1));
+		expect("MNIST reader: Open + readData", reader.Open(img, lab, count) && reader.readData() && reader.size() == count);
+		bool ok = true;
+		for (int s = 0; s < count; ++s)
+			for (int k = 0; k < 784; ++k) {
+				// a pixel byte read through a signed char becomes the real AND the imaginary part (data/data.h:129-132)
+				float want = (float) (signed char) (unsigned char) ((s * 31 + k * 7) & 255);
+				ok = ok && reader.realOf(s)[k] == want && reader.imagOf(s)[k] == want;
+			}
+		expect("MNIST reader: pixel conversion, labels", ok && reader.labelOf(3) == 3 && reader.labelOf(9) == 9);
+		expect("hasNextBatch", reader.hasNextBatch(10) && !reader.hasNextBatch(11));
+		InputBatch b = reader.nextBatch(4);
+		expect("nextBatch(4): shape, labels, first rows", b.size() == 4 && b.sampleDim() == 784 && b.noOfLabels() == 4 && b.label(2) == 2 &&
+				std::equal(b.realDataPtr(1), b.realDataPtr(1) + 784, reader.realOf(1)) && !b.isPinned());
+		reader.nextBatch(b);
+		expect("refill continues with samples 4..7", b.label(0) == 4 && b.label(3) == 7 && std::equal(b.imagDataPtr(3), b.imagDataPtr(3) + 784, reader.imagOf(7)));
+		reader.nextBatch(b);
+		expect("wrap-around at the end of the data (8, 9, 0, 1)", b.label(0) == 8 && b.label(1) == 9 && b.label(2) == 0 && b.label(3) == 1);
+		reader.shuffle(5);
+		std::vector<int> seen(10, 0);
+		InputBatch all(10, 784);
+		// two positions were consumed after the wrap: the next ten positions still cover every sample once
+		reader.nextBatch(all);
+		bool rows_match = true;
+		for (int r = 0; r < 10; ++r) {
+			seen[all.label(r)]++;
+			rows_match = rows_match && std::equal(all.realDataPtr(r), all.realDataPtr(r) + 784, reader.realOf(all.label(r)));
+		}
+		bool perm = true, moved = false;
+		for (int r = 0; r < 10; ++r) {
+			perm = perm && seen[r] == 1;
+			moved = moved || all.label(r) != (r + 2) % 10;
+		}
+		expect("shuffle(seed) is a permutation that keeps rows and labels together", perm && moved && rows_match);
+		// short samples are zero padded, as InputBatch::add upstream (impl/batch.h)
+		InputBatch pad(2, 5);
+		pad.add({{1.f, 2.f}, {3.f, 4.f}}, 7);
+		pad.add({{5.f, 6.f}}, 1);
+		expect("InputBatch pads short samples with zeros", pad.realDataPtr(0)[1] == 3.f && pad.imagDataPtr(0)[1] == 4.f && pad.realDataPtr(0)[2] == 0.f &&
+				pad.realDataPtr(1)[0] == 5.f && pad.imagDataPtr(1)[4] == 0.f && pad.label(0) == 7);
+		InputBatch moved_to = std::move(pad);
+		expect("InputBatch moves", moved_to.realDataPtr(1)[0] == 5.f && moved_to.size() == 2);
 	}
 	printf("saver: %d failure(s)\n", g_fail);
 	return g_fail ? 1 : 0;

@@ -62,6 +62,11 @@ def test_upstream_model_files_restore_and_run_on_the_device(tmp_path):
     assert "FAIL" not in out and out.count("PASS") >= 16
 
 
+def test_host_batch_pipeline_prefetch_gives_the_same_bits():
+    out = _run("pipeline")
+    assert "FAIL" not in out and out.count("PASS") >= 7 and "samples_per_sec_prefetch" in out
+
+
 def test_error_behaviour():
     out = _run("errors")
     assert "FAIL" not in out
