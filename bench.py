@@ -144,6 +144,10 @@ def kernel_suite(steps):
     x, y, g, dx = cmat(Bf, nf), ops.CMat.empty(Bf, nf), grad(Bf, nf), ops.Grad.empty(Bf, nf)
     mfma("cdft_fwd", [Bf, nf], 8.0 * Bf * nf * nf, lambda: ops.dft_fwd(x, y))
     mfma("cdft_bwd", [Bf, nf], 16.0 * Bf * nf * nf, lambda: ops.dft_bwd(g, dx))
+    # TriangFourier: only the pairs in <= out contribute, n (n + 1) / 2 complex multiply-adds per row
+    tri = nf * (nf + 1) / 2.0
+    mfma("ctriang_dft_fwd (useful flops: upper triangle only)", [Bf, nf], 8.0 * Bf * tri, lambda: ops.triang_dft_fwd(x, y))
+    mfma("ctriang_dft_bwd (useful flops: upper triangle only)", [Bf, nf], 16.0 * Bf * tri, lambda: ops.triang_dft_bwd(g, dx))
     del x, y, g, dx
 
     # config 5 activation shape [8192 x 4096]: 256 MiB per complex matrix, so every operand streams from HBM
@@ -155,6 +159,8 @@ def kernel_suite(steps):
     hbm("plain copy of one plane (practical HBM ceiling)", [R, Cc], 8, n, lambda: ops.copy2d(u.re, yy.re))
     hbm("cgelu_fwd", [R, Cc], 16, n, lambda: ops.gelu_fwd(u, yy))
     hbm("cgelu_bwd", [R, Cc], 40, n, lambda: ops.gelu_bwd(u, g, du))
+    hbm("crelu_fwd", [R, Cc], 16, n, lambda: ops.crelu_fwd(u, yy))
+    hbm("crelu_bwd", [R, Cc], 40, n, lambda: ops.crelu_bwd(u, g, du))
     hbm("residual_fwd", [R, Cc], 24, n, lambda: ops.residual_fwd(u, v, yy))
     hbm("residual_bwd", [R, Cc], 48, n, lambda: ops.residual_bwd(g, du, dv))
     hbm("hadamard_fwd (shared weights)", [R, Cc], 16, n, lambda: ops.hadamard_fwd(u, w1, yy, True))
@@ -167,6 +173,7 @@ def kernel_suite(steps):
     hbm("l2norm_fwd (SoftMax)", [R, Cc], 16, n, lambda: ops.l2norm_fwd(u, yy, s_))
     hbm("l2norm_bwd (SoftMax)", [R, Cc], 40, n, lambda: ops.l2norm_bwd(u, s_, g, du))
     hbm("sgd_update", [n], 32, n, lambda: ops.sgd_update(u, du.planes[2], du.planes[3], 1e-9))
+    hbm("adam_update", [n], 48, n, lambda: ops.adam_update(u, du.planes[0], du.planes[1], du.planes[2], du.planes[3], 1e-9, 0.9, 3))
     hbm("zero 4 gradient planes", [R, Cc], 16, n, lambda: [p.owner.zero() for p in du.planes])
     out1 = ops.Plane.empty(1, Cc)
     hbm("batch_sum (one plane)", [R, Cc], 4, n, lambda: ops.batch_sum(u.re, out1))

@@ -53,6 +53,9 @@ struct CgemmArgs {
 	int tri;
 };
 
+// column blocks per grid row: with a triangular operand each workgroup handles a block and its mirror image
+__device__ __host__ __forceinline__ int grid_tiles_n(const CgemmArgs &args) { return args.tri ? (args.tiles_n + 1) / 2 : args.tiles_n; }
+
 // first chunk and one-past-last chunk of K for the block of columns starting at n0
 template <int BN>
 __device__ __forceinline__ void chunk_range(const CgemmArgs &args, int n0, int &c_lo, int &c_hi) {
@@ -189,15 +192,19 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 
 	// ---- which block of C
 	int pid = blockIdx.x;
-	const int total = args.tiles_m * args.tiles_n;
+	const int grid_n = grid_tiles_n(args);
+	const int total = args.tiles_m * grid_n;
 	if (total % NUM_XCD == 0) pid = (pid % NUM_XCD) * (total / NUM_XCD) + pid / NUM_XCD;
 	constexpr int GROUP = 8;
-	const int width = GROUP * args.tiles_n;
+	const int width = GROUP * grid_n;
 	const int first_m = (pid / width) * GROUP;
 	const int gsize = min(args.tiles_m - first_m, GROUP);
 	const int tile_m = first_m + (pid % width) % gsize;
-	const int tile_n = (pid % width) / gsize;
-	const int m0 = tile_m * BM, n0 = tile_n * BN;
+	const int tile_n_first = (pid % width) / gsize;
+	const int m0 = tile_m * BM;
+	// a triangular operand: this workgroup takes column block j and then its mirror tiles_n - 1 - j, so that every
+	// workgroup walks the same number of K chunks in total
+	const int npass = (args.tri && tile_n_first != args.tiles_n - 1 - tile_n_first) ? 2 : 1;
 
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
@@ -206,6 +213,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 	const int r = lane & 31, h = lane >> 5;
 
 	floatx16 acc_re[TM][TN], acc_im[TM][TN];
+	for (int pass = 0; pass < npass; ++pass) {
+	const int tile_n = pass ? args.tiles_n - 1 - tile_n_first : tile_n_first;
+	const int n0 = tile_n * BN;
+	if (pass) __syncthreads();  // every wave has finished reading the last stage of the previous block
 #pragma unroll
 	for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -312,6 +323,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 				}
 			}
 		}
+	}  // pass
 }
 
 
@@ -443,15 +455,19 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	const int K = args.K;
 
 	int pid = blockIdx.x;
-	const int total = args.tiles_m * args.tiles_n;
+	const int grid_n = grid_tiles_n(args);
+	const int total = args.tiles_m * grid_n;
 	if (total % NUM_XCD == 0) pid = (pid % NUM_XCD) * (total / NUM_XCD) + pid / NUM_XCD;
 	constexpr int GROUP = 8;
-	const int width = GROUP * args.tiles_n;
+	const int width = GROUP * grid_n;
 	const int first_m = (pid / width) * GROUP;
 	const int gsize = min(args.tiles_m - first_m, GROUP);
 	const int tile_m = first_m + (pid % width) % gsize;
-	const int tile_n = (pid % width) / gsize;
-	const int m0 = tile_m * BM, n0 = tile_n * BN;
+	const int tile_n_first = (pid % width) / gsize;
+	const int m0 = tile_m * BM;
+	// a triangular operand: this workgroup takes column block j and then its mirror tiles_n - 1 - j, so that every
+	// workgroup walks the same number of K chunks in total
+	const int npass = (args.tri && tile_n_first != args.tiles_n - 1 - tile_n_first) ? 2 : 1;
 
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
@@ -460,6 +476,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	const int r = lane & 31, h = lane >> 5;
 
 	floatx16 acc_re[TM][TN], acc_im[TM][TN];
+	for (int pass = 0; pass < npass; ++pass) {
+	const int tile_n = pass ? args.tiles_n - 1 - tile_n_first : tile_n_first;
+	const int n0 = tile_n * BN;
+	if (pass) __syncthreads();  // every wave has finished reading the last stage of the previous block
 #pragma unroll
 	for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -603,6 +623,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				pb.c_im[off] = vi;
 			}
 		}
+	}  // pass
 }
 
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
@@ -611,7 +632,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch) {
 	args.tiles_m = (args.M + BM - 1) / BM;
 	args.tiles_n = (args.N + BN - 1) / BN;
 	constexpr size_t smem = 2 * (size_t) (2 * KC * (BM + 4) + 2 * KC * (BN + 4)) * sizeof(float);
-	dim3 grid(args.tiles_m * args.tiles_n, nprob, batch);
+	dim3 grid(args.tiles_m * grid_tiles_n(args), nprob, batch);
 	if constexpr (VEC == 4) {
 		if (args.M % BM == 0 && args.N % BN == 0 && args.K % KC == 0) {
 			auto fast = cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG>;
@@ -641,7 +662,11 @@ int launch(const CgemmArgs &proto, int nprob, int batch) {
 template <bool A_MCONTIG, bool B_NCONTIG, int VEC>
 int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 	const long cus = cnet::rt().prop.multiProcessorCount;
-	auto blocks = [&](int bm, int bn) { return (long) ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * nprob * batch; };
+	auto blocks = [&](int bm, int bn) {
+		long tn = (a.N + bn - 1) / bn;
+		if (a.tri) tn = (tn + 1) / 2;  // one workgroup per mirrored pair of column blocks
+		return (long) ((a.M + bm - 1) / bm) * tn * nprob * batch;
+	};
 	// the scalar-load fallback (odd shapes) keeps to the small block: its address arithmetic would spill otherwise
 	if constexpr (VEC == 1) {
 		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
