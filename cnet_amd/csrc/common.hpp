@@ -58,6 +58,22 @@ void *workspace(size_t bytes);
 		if (e__ != hipSuccess) return cnet::hip_fail(e__, __func__);   \
 	} while (0)
 
+// Second stage of the deterministic column sums: adds `count` partial values that lie `stride` floats apart, in index
+// order, requesting eight of them before the first is added (the additions stay sequential, the loads overlap).
+__device__ __forceinline__ float ordered_sum(const float *__restrict__ first, long stride, int count) {
+	float s = 0.f;
+	int k = 0;
+	for (; k + 8 <= count; k += 8) {
+		float v[8];
+#pragma unroll
+		for (int u = 0; u < 8; ++u) v[u] = first[(long) (k + u) * stride];
+#pragma unroll
+		for (int u = 0; u < 8; ++u) s += v[u];
+	}
+	for (; k < count; ++k) s += first[(long) k * stride];
+	return s;
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace cnet

@@ -13,10 +13,17 @@ namespace {
 
 constexpr int TPB = 256;
 
-template <int V>
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// NT: the access carries the streaming (non-temporal) hint.  Launches whose operands together exceed the 256 MB
+// memory-side cache set it: nothing they touch can be found there again, and without the hint the lines they leave
+// behind cost ~8 % of the achievable rate; smaller launches keep normal accesses, because the next kernel does find
+// their results in that cache.
+template <int V, bool NT>
 __device__ __forceinline__ void ldv(float (&d)[V], const float *__restrict__ p) {
 	if (V == 4) {
-		float4 t = *reinterpret_cast<const float4 *>(p);
+		const f32x4 *q = reinterpret_cast<const f32x4 *>(p);
+		f32x4 t = NT ? __builtin_nontemporal_load(q) : *q;
 		d[0] = t.x;
 		d[1 % V] = t.y;
 		d[2 % V] = t.z;
@@ -26,26 +33,31 @@ __device__ __forceinline__ void ldv(float (&d)[V], const float *__restrict__ p) 
 	}
 }
 
-template <int V>
+template <int V, bool NT>
 __device__ __forceinline__ void stv(float *__restrict__ p, const float (&d)[V]) {
-	if (V == 4)
-		*reinterpret_cast<float4 *>(p) = make_float4(d[0], d[1 % V], d[2 % V], d[3 % V]);
-	else
+	if (V == 4) {
+		f32x4 t = {d[0], d[1 % V], d[2 % V], d[3 % V]};
+		if (NT)
+			__builtin_nontemporal_store(t, reinterpret_cast<f32x4 *>(p));
+		else
+			*reinterpret_cast<f32x4 *>(p) = t;
+	} else {
 		*p = d[0];
+	}
 }
 
 // store or accumulate
-template <int V>
+template <int V, bool NT>
 __device__ __forceinline__ void outv(float *__restrict__ p, const float (&d)[V], int accumulate) {
 	if (accumulate) {
 		float o[V];
-		ldv<V>(o, p);
+		ldv<V, NT>(o, p);
 		float s[V];
 #pragma unroll
 		for (int k = 0; k < V; ++k) s[k] = o[k] + d[k];
-		stv<V>(p, s);
+		stv<V, NT>(p, s);
 	} else {
-		stv<V>(p, d);
+		stv<V, NT>(p, d);
 	}
 }
 
@@ -64,65 +76,65 @@ struct CGrad4 {
 	const long col = (idx - row * cv) * V;
 
 // ------------------------------------------------------------------------------------------------ Hadamard
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void hadamard_fwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
 		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, float *__restrict__ yr,
 		float *__restrict__ yi, long ldy, int rows, int cols) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V], c[V], d[V], pr[V], pi[V];
-	ldv<V>(a, ur + row * ldu + col);
-	ldv<V>(b, ui + row * ldu + col);
-	ldv<V>(c, vr + row * ldv_ + col);
-	ldv<V>(d, vi + row * ldv_ + col);
+	ldv<V, NT>(a, ur + row * ldu + col);
+	ldv<V, NT>(b, ui + row * ldu + col);
+	ldv<V, false>(c, vr + row * ldv_ + col);  // may be one row shared by all rows: keep it cached
+	ldv<V, false>(d, vi + row * ldv_ + col);
 #pragma unroll
 	for (int k = 0; k < V; ++k) {
 		pr[k] = a[k] * c[k] - b[k] * d[k];
 		pi[k] = a[k] * d[k] + b[k] * c[k];
 	}
-	stv<V>(yr + row * ldy + col, pr);
-	stv<V>(yi + row * ldy + col, pi);
+	stv<V, NT>(yr + row * ldy + col, pr);
+	stv<V, NT>(yi + row * ldy + col, pi);
 }
 
 // Both operands per-row: du = (G v, Gs conj v), dv = (G u, Gs conj u).
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
 		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, CGrad4 g, long ldg, Grad4 du, long lddu,
 		Grad4 dv, long lddv, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V], c[V], d[V], gr[V], gi[V], sr[V], si[V], o[V];
-	ldv<V>(a, ur + row * ldu + col);
-	ldv<V>(b, ui + row * ldu + col);
-	ldv<V>(c, vr + row * ldv_ + col);
-	ldv<V>(d, vi + row * ldv_ + col);
-	ldv<V>(gr, g.dz_re + row * ldg + col);
-	ldv<V>(gi, g.dz_im + row * ldg + col);
-	ldv<V>(sr, g.dzs_re + row * ldg + col);
-	ldv<V>(si, g.dzs_im + row * ldg + col);
+	ldv<V, NT>(a, ur + row * ldu + col);
+	ldv<V, NT>(b, ui + row * ldu + col);
+	ldv<V, NT>(c, vr + row * ldv_ + col);
+	ldv<V, NT>(d, vi + row * ldv_ + col);
+	ldv<V, NT>(gr, g.dz_re + row * ldg + col);
+	ldv<V, NT>(gi, g.dz_im + row * ldg + col);
+	ldv<V, NT>(sr, g.dzs_re + row * ldg + col);
+	ldv<V, NT>(si, g.dzs_im + row * ldg + col);
 	const long ou = row * lddu + col, ov = row * lddv + col;
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = gr[k] * c[k] - gi[k] * d[k];
-	outv<V>(du.dz_re + ou, o, accumulate);
+	outv<V, NT>(du.dz_re + ou, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = gr[k] * d[k] + gi[k] * c[k];
-	outv<V>(du.dz_im + ou, o, accumulate);
+	outv<V, NT>(du.dz_im + ou, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = sr[k] * c[k] + si[k] * d[k];
-	outv<V>(du.dzs_re + ou, o, accumulate);
+	outv<V, NT>(du.dzs_re + ou, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = si[k] * c[k] - sr[k] * d[k];
-	outv<V>(du.dzs_im + ou, o, accumulate);
+	outv<V, NT>(du.dzs_im + ou, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = gr[k] * a[k] - gi[k] * b[k];
-	outv<V>(dv.dz_re + ov, o, accumulate);
+	outv<V, NT>(dv.dz_re + ov, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = gr[k] * b[k] + gi[k] * a[k];
-	outv<V>(dv.dz_im + ov, o, accumulate);
+	outv<V, NT>(dv.dz_im + ov, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = sr[k] * a[k] + si[k] * b[k];
-	outv<V>(dv.dzs_re + ov, o, accumulate);
+	outv<V, NT>(dv.dzs_re + ov, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = si[k] * a[k] - sr[k] * b[k];
-	outv<V>(dv.dzs_im + ov, o, accumulate);
+	outv<V, NT>(dv.dzs_im + ov, o, accumulate);
 }
 
 // v is one shared parameter row.  Workgroup = 64 column groups (V columns each) x 4 row lanes; blockIdx.y selects a slab
@@ -131,7 +143,7 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_kernel(const float *__restri
 // the slabs in slab order.  Deterministic: no atomics, fixed summation tree.
 constexpr int CS_X = 64, CS_Y = 4;
 
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *__restrict__ ur, const float *__restrict__ ui,
 		long ldu, const float *__restrict__ vr, const float *__restrict__ vi, CGrad4 g, long ldg, Grad4 du, long lddu,
 		float *__restrict__ partial, int rows, int cols, int rows_per_slab, int accumulate) {
@@ -149,29 +161,29 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *_
 		for (int k = 0; k < V; ++k) acc[p][k] = 0.f;
 	if (live) {
 		float c[V], d[V];
-		ldv<V>(c, vr + col);
-		ldv<V>(d, vi + col);
+		ldv<V, false>(c, vr + col);
+		ldv<V, false>(d, vi + col);
 		for (int row = r0 + ty; row < r1; row += CS_Y) {
 			float a[V], b[V], gr[V], gi[V], sr[V], si[V], o[V];
-			ldv<V>(a, ur + (long) row * ldu + col);
-			ldv<V>(b, ui + (long) row * ldu + col);
-			ldv<V>(gr, g.dz_re + (long) row * ldg + col);
-			ldv<V>(gi, g.dz_im + (long) row * ldg + col);
-			ldv<V>(sr, g.dzs_re + (long) row * ldg + col);
-			ldv<V>(si, g.dzs_im + (long) row * ldg + col);
+			ldv<V, NT>(a, ur + (long) row * ldu + col);
+			ldv<V, NT>(b, ui + (long) row * ldu + col);
+			ldv<V, NT>(gr, g.dz_re + (long) row * ldg + col);
+			ldv<V, NT>(gi, g.dz_im + (long) row * ldg + col);
+			ldv<V, NT>(sr, g.dzs_re + (long) row * ldg + col);
+			ldv<V, NT>(si, g.dzs_im + (long) row * ldg + col);
 			const long ou = (long) row * lddu + col;
 #pragma unroll
 			for (int k = 0; k < V; ++k) o[k] = gr[k] * c[k] - gi[k] * d[k];
-			outv<V>(du.dz_re + ou, o, accumulate);
+			outv<V, NT>(du.dz_re + ou, o, accumulate);
 #pragma unroll
 			for (int k = 0; k < V; ++k) o[k] = gr[k] * d[k] + gi[k] * c[k];
-			outv<V>(du.dz_im + ou, o, accumulate);
+			outv<V, NT>(du.dz_im + ou, o, accumulate);
 #pragma unroll
 			for (int k = 0; k < V; ++k) o[k] = sr[k] * c[k] + si[k] * d[k];
-			outv<V>(du.dzs_re + ou, o, accumulate);
+			outv<V, NT>(du.dzs_re + ou, o, accumulate);
 #pragma unroll
 			for (int k = 0; k < V; ++k) o[k] = si[k] * c[k] - sr[k] * d[k];
-			outv<V>(du.dzs_im + ou, o, accumulate);
+			outv<V, NT>(du.dzs_im + ou, o, accumulate);
 #pragma unroll
 			for (int k = 0; k < V; ++k) {
 				acc[0][k] += gr[k] * a[k] - gi[k] * b[k];
@@ -192,7 +204,7 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *_
 			float t[V];
 #pragma unroll
 			for (int k = 0; k < V; ++k) t[k] = ((red[0][p][tx * V + k] + red[1][p][tx * V + k]) + red[2][p][tx * V + k]) + red[3][p][tx * V + k];
-			stv<V>(partial + ((long) slab * 4 + p) * cols + col, t);
+			stv<V, NT>(partial + ((long) slab * 4 + p) * cols + col, t);
 		}
 	}
 }
@@ -200,14 +212,22 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *_
 // dst[p][c] (+)= sum over slabs of partial[slab][p][c], slabs added in index order.
 __global__ __launch_bounds__(TPB) void slab_sum_kernel(const float *__restrict__ partial, int nslabs, int nplanes, int cols,
 		Grad4 dst, int accumulate) {
-	const long idx = (long) blockIdx.x * TPB + threadIdx.x;
-	if (idx >= (long) nplanes * cols) return;
-	const int p = (int) (idx / cols);
-	const int c = (int) (idx - (long) p * cols);
-	float s = 0.f;
-	for (int k = 0; k < nslabs; ++k) s += partial[((long) k * nplanes + p) * cols + c];
-	float *out = p == 0 ? dst.dz_re : (p == 1 ? dst.dz_im : (p == 2 ? dst.dzs_re : dst.dzs_im));
-	out[c] = accumulate ? out[c] + s : s;
+	// 64 (plane, column) pairs per workgroup x 4 lanes that each add one contiguous quarter of the slabs in order; the
+	// four quarter sums are then added in lane order
+	__shared__ float red[4][64];
+	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+	const long idx = (long) blockIdx.x * 64 + tx;
+	const bool live = idx < (long) nplanes * cols;
+	const int p = live ? (int) (idx / cols) : 0;
+	const int c = live ? (int) (idx - (long) p * cols) : 0;
+	const int per = (nslabs + 3) / 4, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
+	red[ty][tx] = live ? cnet::ordered_sum(partial + ((long) k0 * nplanes + p) * cols + c, (long) nplanes * cols, k1 - k0) : 0.f;
+	__syncthreads();
+	if (ty == 0 && live) {
+		const float s = ((red[0][tx] + red[1][tx]) + red[2][tx]) + red[3][tx];
+		float *out = p == 0 ? dst.dz_re : (p == 1 ? dst.dz_im : (p == 2 ? dst.dzs_re : dst.dzs_im));
+		out[c] = accumulate ? out[c] + s : s;
+	}
 }
 
 // ------------------------------------------------------------------------------------------------ CGelu
@@ -226,34 +246,34 @@ __device__ __forceinline__ float gelu_slope(float t) {
 	return 0.5f * (1.0f + th) + t * 0.5f * sech2 * c * (1.0f + 3.0f * 0.044715f * t * t);
 }
 
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void gelu_fwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		float *__restrict__ yr, float *__restrict__ yi, long ldy, int rows, int cols) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V];
-	ldv<V>(a, xr + row * ldx + col);
-	ldv<V>(b, xi + row * ldx + col);
+	ldv<V, NT>(a, xr + row * ldx + col);
+	ldv<V, NT>(b, xi + row * ldx + col);
 #pragma unroll
 	for (int k = 0; k < V; ++k) {
 		a[k] = gelu_value(a[k]);
 		b[k] = gelu_value(b[k]);
 	}
-	stv<V>(yr + row * ldy + col, a);
-	stv<V>(yi + row * ldy + col, b);
+	stv<V, NT>(yr + row * ldy + col, a);
+	stv<V, NT>(yi + row * ldy + col, b);
 }
 
 // dz = G s + Gs d ; dzs = G d + Gs s ; s = (g'(x)+g'(y))/2, d = (g'(x)-g'(y))/2   (impl/relu.h:144-166 upstream)
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void gelu_bwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		CGrad4 g, long ldg, Grad4 dx, long lddx, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V], gr[V], gi[V], sr[V], si[V], s[V], d[V], o[V];
-	ldv<V>(a, xr + row * ldx + col);
-	ldv<V>(b, xi + row * ldx + col);
-	ldv<V>(gr, g.dz_re + row * ldg + col);
-	ldv<V>(gi, g.dz_im + row * ldg + col);
-	ldv<V>(sr, g.dzs_re + row * ldg + col);
-	ldv<V>(si, g.dzs_im + row * ldg + col);
+	ldv<V, NT>(a, xr + row * ldx + col);
+	ldv<V, NT>(b, xi + row * ldx + col);
+	ldv<V, NT>(gr, g.dz_re + row * ldg + col);
+	ldv<V, NT>(gi, g.dz_im + row * ldg + col);
+	ldv<V, NT>(sr, g.dzs_re + row * ldg + col);
+	ldv<V, NT>(si, g.dzs_im + row * ldg + col);
 #pragma unroll
 	for (int k = 0; k < V; ++k) {
 		float px = 0.5f * gelu_slope(a[k]), py = 0.5f * gelu_slope(b[k]);
@@ -263,123 +283,123 @@ __global__ __launch_bounds__(TPB) void gelu_bwd_kernel(const float *__restrict__
 	const long off = row * lddx + col;
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = gr[k] * s[k] + sr[k] * d[k];
-	outv<V>(dx.dz_re + off, o, accumulate);
+	outv<V, NT>(dx.dz_re + off, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = gi[k] * s[k] + si[k] * d[k];
-	outv<V>(dx.dz_im + off, o, accumulate);
+	outv<V, NT>(dx.dz_im + off, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = gr[k] * d[k] + sr[k] * s[k];
-	outv<V>(dx.dzs_re + off, o, accumulate);
+	outv<V, NT>(dx.dzs_re + off, o, accumulate);
 #pragma unroll
 	for (int k = 0; k < V; ++k) o[k] = gi[k] * d[k] + si[k] * s[k];
-	outv<V>(dx.dzs_im + off, o, accumulate);
+	outv<V, NT>(dx.dzs_im + off, o, accumulate);
 }
 
 // ------------------------------------------------------------------------------------------------ CRelu
 // y = z where Re z > 0 and Im z > 0, else 0 (impl/relu.h:32-46 upstream); the gradients pass under the same test
 // (impl/relu.h:48-63).
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void crelu_fwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		float *__restrict__ yr, float *__restrict__ yi, long ldy, int rows, int cols) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V];
-	ldv<V>(a, xr + row * ldx + col);
-	ldv<V>(b, xi + row * ldx + col);
+	ldv<V, NT>(a, xr + row * ldx + col);
+	ldv<V, NT>(b, xi + row * ldx + col);
 #pragma unroll
 	for (int k = 0; k < V; ++k) {
 		const bool on = a[k] > 0.f && b[k] > 0.f;
 		a[k] = on ? a[k] : 0.f;
 		b[k] = on ? b[k] : 0.f;
 	}
-	stv<V>(yr + row * ldy + col, a);
-	stv<V>(yi + row * ldy + col, b);
+	stv<V, NT>(yr + row * ldy + col, a);
+	stv<V, NT>(yi + row * ldy + col, b);
 }
 
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void crelu_bwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		CGrad4 g, long ldg, Grad4 dx, long lddx, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V], o[V];
-	ldv<V>(a, xr + row * ldx + col);
-	ldv<V>(b, xi + row * ldx + col);
+	ldv<V, NT>(a, xr + row * ldx + col);
+	ldv<V, NT>(b, xi + row * ldx + col);
 	const float *src[4] = {g.dz_re, g.dz_im, g.dzs_re, g.dzs_im};
 	float *dst[4] = {dx.dz_re, dx.dz_im, dx.dzs_re, dx.dzs_im};
 #pragma unroll
 	for (int p = 0; p < 4; ++p) {
-		ldv<V>(o, src[p] + row * ldg + col);
+		ldv<V, NT>(o, src[p] + row * ldg + col);
 #pragma unroll
 		for (int k = 0; k < V; ++k) o[k] = (a[k] > 0.f && b[k] > 0.f) ? o[k] : 0.f;
-		outv<V>(dst[p] + row * lddx + col, o, accumulate);
+		outv<V, NT>(dst[p] + row * lddx + col, o, accumulate);
 	}
 }
 
 // ------------------------------------------------------------------------------------------------ Residual
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void residual_fwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
 		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, float *__restrict__ yr,
 		float *__restrict__ yi, long ldy, int rows, int cols) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V], c[V], d[V];
-	ldv<V>(a, ur + row * ldu + col);
-	ldv<V>(b, ui + row * ldu + col);
-	ldv<V>(c, vr + row * ldv_ + col);
-	ldv<V>(d, vi + row * ldv_ + col);
+	ldv<V, NT>(a, ur + row * ldu + col);
+	ldv<V, NT>(b, ui + row * ldu + col);
+	ldv<V, false>(c, vr + row * ldv_ + col);
+	ldv<V, false>(d, vi + row * ldv_ + col);
 #pragma unroll
 	for (int k = 0; k < V; ++k) {
 		a[k] += c[k];
 		b[k] += d[k];
 	}
-	stv<V>(yr + row * ldy + col, a);
-	stv<V>(yi + row * ldy + col, b);
+	stv<V, NT>(yr + row * ldy + col, a);
+	stv<V, NT>(yi + row * ldy + col, b);
 }
 
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void residual_bwd_kernel(CGrad4 g, long ldg, Grad4 du, long lddu, Grad4 dv, long lddv,
 		int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
 	float t[V];
 	const long og = row * ldg + col, ou = row * lddu + col, ov = row * lddv + col;
-	ldv<V>(t, g.dz_re + og);
-	outv<V>(du.dz_re + ou, t, accumulate);
-	outv<V>(dv.dz_re + ov, t, accumulate);
-	ldv<V>(t, g.dz_im + og);
-	outv<V>(du.dz_im + ou, t, accumulate);
-	outv<V>(dv.dz_im + ov, t, accumulate);
-	ldv<V>(t, g.dzs_re + og);
-	outv<V>(du.dzs_re + ou, t, accumulate);
-	outv<V>(dv.dzs_re + ov, t, accumulate);
-	ldv<V>(t, g.dzs_im + og);
-	outv<V>(du.dzs_im + ou, t, accumulate);
-	outv<V>(dv.dzs_im + ov, t, accumulate);
+	ldv<V, NT>(t, g.dz_re + og);
+	outv<V, NT>(du.dz_re + ou, t, accumulate);
+	outv<V, NT>(dv.dz_re + ov, t, accumulate);
+	ldv<V, NT>(t, g.dz_im + og);
+	outv<V, NT>(du.dz_im + ou, t, accumulate);
+	outv<V, NT>(dv.dz_im + ov, t, accumulate);
+	ldv<V, NT>(t, g.dzs_re + og);
+	outv<V, NT>(du.dzs_re + ou, t, accumulate);
+	outv<V, NT>(dv.dzs_re + ov, t, accumulate);
+	ldv<V, NT>(t, g.dzs_im + og);
+	outv<V, NT>(du.dzs_im + ou, t, accumulate);
+	outv<V, NT>(dv.dzs_im + ov, t, accumulate);
 }
 
 // ------------------------------------------------------------------------------------------------ loss backward
 // L2Out: dz = conj z, dzs = z  (impl/l2out.h:44-58 upstream)
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void l2out_bwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		Grad4 dz, long lddz, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V], nb[V];
-	ldv<V>(a, zr + row * ldz + col);
-	ldv<V>(b, zi + row * ldz + col);
+	ldv<V, NT>(a, zr + row * ldz + col);
+	ldv<V, NT>(b, zi + row * ldz + col);
 #pragma unroll
 	for (int k = 0; k < V; ++k) nb[k] = -b[k];
 	const long off = row * lddz + col;
-	outv<V>(dz.dz_re + off, a, accumulate);
-	outv<V>(dz.dz_im + off, nb, accumulate);
-	outv<V>(dz.dzs_re + off, a, accumulate);
-	outv<V>(dz.dzs_im + off, b, accumulate);
+	outv<V, NT>(dz.dz_re + off, a, accumulate);
+	outv<V, NT>(dz.dz_im + off, nb, accumulate);
+	outv<V, NT>(dz.dzs_re + off, a, accumulate);
+	outv<V, NT>(dz.dzs_im + off, b, accumulate);
 }
 
 // CrossEntropy (impl/crossent.h:82-104 upstream): assigns.  label: dzs = -z (S-m)/(m S), m = max(|z_l|^2, 1e-15);
 // other entries: dzs = z/S; dz = conj(dzs).
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void crossent_bwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		const float *__restrict__ s, const int *__restrict__ labels, Grad4 dz, long lddz, int rows, int cols) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V], o_r[V], o_i[V], n_i[V];
-	ldv<V>(a, zr + row * ldz + col);
-	ldv<V>(b, zi + row * ldz + col);
+	ldv<V, NT>(a, zr + row * ldz + col);
+	ldv<V, NT>(b, zi + row * ldz + col);
 	const float S = s[row];
 	const int label = labels[row];
 #pragma unroll
@@ -396,63 +416,63 @@ __global__ __launch_bounds__(TPB) void crossent_bwd_kernel(const float *__restri
 		n_i[k] = -o_i[k];
 	}
 	const long off = row * lddz + col;
-	stv<V>(dz.dzs_re + off, o_r);
-	stv<V>(dz.dzs_im + off, o_i);
-	stv<V>(dz.dz_re + off, o_r);
-	stv<V>(dz.dz_im + off, n_i);
+	stv<V, NT>(dz.dzs_re + off, o_r);
+	stv<V, NT>(dz.dzs_im + off, o_i);
+	stv<V, NT>(dz.dz_re + off, o_r);
+	stv<V, NT>(dz.dz_im + off, n_i);
 }
 
 // ------------------------------------------------------------------------------------------------ plumbing
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void copy2d_kernel(const float *__restrict__ src, long lds, float *__restrict__ dst, long ldd,
 		int rows, int cols, int add) {
 	CNET_ELEM_INDEX();
 	float t[V];
-	ldv<V>(t, src + row * lds + col);
-	outv<V>(dst + row * ldd + col, t, add);
+	ldv<V, NT>(t, src + row * lds + col);
+	outv<V, NT>(dst + row * ldd + col, t, add);
 }
 
 // z -= lr * dzs ; dzs = 0   (impl/cfunc.h:147-152, impl/cnet.h:413-421 upstream)
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void sgd_kernel(float *__restrict__ zr, float *__restrict__ zi, float *__restrict__ dr,
 		float *__restrict__ di, long n, float lr, int zero_grad) {
 	const long i = ((long) blockIdx.x * TPB + threadIdx.x) * V;
 	if (i >= n) return;
 	float a[V], b[V], c[V], d[V], z[V];
-	ldv<V>(a, zr + i);
-	ldv<V>(b, zi + i);
-	ldv<V>(c, dr + i);
-	ldv<V>(d, di + i);
+	ldv<V, NT>(a, zr + i);
+	ldv<V, NT>(b, zi + i);
+	ldv<V, NT>(c, dr + i);
+	ldv<V, NT>(d, di + i);
 #pragma unroll
 	for (int k = 0; k < V; ++k) {
 		a[k] -= lr * c[k];
 		b[k] -= lr * d[k];
 		z[k] = 0.f;
 	}
-	stv<V>(zr + i, a);
-	stv<V>(zi + i, b);
+	stv<V, NT>(zr + i, a);
+	stv<V, NT>(zi + i, b);
 	if (zero_grad) {
-		stv<V>(dr + i, z);
-		stv<V>(di + i, z);
+		stv<V, NT>(dr + i, z);
+		stv<V, NT>(di + i, z);
 	}
 }
 
 // m = beta m + (1 - beta) dzs ; z -= lr m / denom ; dzs = 0   (impl/cfunc.h:273-287, gpu/kernels.cpp:494-514 upstream).
 // denom = 1 - beta^(t+1) arrives as a double and the quotient is formed in double, as the CPU loop does
 // (pow(float, int) promotes), so the parameter gets one rounding per step.
-template <int V>
+template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void adam_kernel(float *__restrict__ zr, float *__restrict__ zi, float *__restrict__ mr,
 		float *__restrict__ mi, float *__restrict__ dr, float *__restrict__ di, long n, float lr, float beta, double denom,
 		int zero_grad) {
 	const long i = ((long) blockIdx.x * TPB + threadIdx.x) * V;
 	if (i >= n) return;
 	float a[V], b[V], c[V], d[V], e[V], f[V], z[V];
-	ldv<V>(a, zr + i);
-	ldv<V>(b, zi + i);
-	ldv<V>(c, mr + i);
-	ldv<V>(d, mi + i);
-	ldv<V>(e, dr + i);
-	ldv<V>(f, di + i);
+	ldv<V, NT>(a, zr + i);
+	ldv<V, NT>(b, zi + i);
+	ldv<V, NT>(c, mr + i);
+	ldv<V, NT>(d, mi + i);
+	ldv<V, NT>(e, dr + i);
+	ldv<V, NT>(f, di + i);
 	const float one_minus_beta = 1 - beta;
 #pragma unroll
 	for (int k = 0; k < V; ++k) {
@@ -462,13 +482,13 @@ __global__ __launch_bounds__(TPB) void adam_kernel(float *__restrict__ zr, float
 		b[k] = (float) ((double) b[k] - (double) (lr * d[k]) / denom);
 		z[k] = 0.f;
 	}
-	stv<V>(zr + i, a);
-	stv<V>(zi + i, b);
-	stv<V>(mr + i, c);
-	stv<V>(mi + i, d);
+	stv<V, NT>(zr + i, a);
+	stv<V, NT>(zi + i, b);
+	stv<V, NT>(mr + i, c);
+	stv<V, NT>(mi + i, d);
 	if (zero_grad) {
-		stv<V>(dr + i, z);
-		stv<V>(di + i, z);
+		stv<V, NT>(dr + i, z);
+		stv<V, NT>(di + i, z);
 	}
 }
 
@@ -494,6 +514,18 @@ inline bool all_mult4(std::initializer_list<long> v) {
 }  // namespace
 
 using namespace cnet;
+
+// the 128-bit variant of a kernel, with or without the streaming hint
+#define CNET_LAUNCH_V4(kernel, nt, ...)                          \
+	do {                                                         \
+		if (nt)                                                  \
+			hipLaunchKernelGGL((kernel<4, true>), __VA_ARGS__);  \
+		else                                                     \
+			hipLaunchKernelGGL((kernel<4, false>), __VA_ARGS__); \
+	} while (0)
+
+// planes: fp32 planes of [rows x cols] the launch reads or writes
+static inline bool streaming(int planes, long elems) { return (long) planes * elems * 4 > (256L << 20); }
 
 #define CNET_GRID_2D(V) dim3(nblocks((long) rows * (cols / (V)))), dim3(TPB), 0, rt().stream
 
@@ -530,10 +562,11 @@ int cnet_hadamard_fwd(const float *u_re, const float *u_im, int64_t ldu, const f
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && y_re && y_im);
 	CNET_CHECK_ARG(ldu >= cols && ldy >= cols && (ldv == 0 || ldv >= cols));
+	const bool nt = streaming(4, (long) rows * cols);
 	if (all_mult4({cols, ldu, ldv, ldy}) && all_aligned({u_re, u_im, v_re, v_im, y_re, y_im}))
-		hipLaunchKernelGGL(hadamard_fwd_kernel<4>, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+		CNET_LAUNCH_V4(hadamard_fwd_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
 	else
-		hipLaunchKernelGGL(hadamard_fwd_kernel<1>, CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+		hipLaunchKernelGGL((hadamard_fwd_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -554,12 +587,13 @@ int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const f
 	bool vec = all_mult4({cols, ldu, ldv, ldg, lddu, ldv ? lddv : 0}) &&
 			all_aligned({u_re, u_im, v_re, v_im, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, du_dz_re, du_dz_im, du_dzs_re,
 					du_dzs_im, dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im});
+	const bool nt = streaming(10, (long) rows * cols);
 	if (ldv != 0) {
 		if (vec)
-			hipLaunchKernelGGL(hadamard_bwd_kernel<4>, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, g, ldg, du, lddu, dv, lddv,
+			CNET_LAUNCH_V4(hadamard_bwd_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, g, ldg, du, lddu, dv, lddv,
 					rows, cols, accumulate);
 		else
-			hipLaunchKernelGGL(hadamard_bwd_kernel<1>, CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, g, ldg, du, lddu, dv, lddv,
+			hipLaunchKernelGGL((hadamard_bwd_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, g, ldg, du, lddu, dv, lddv,
 					rows, cols, accumulate);
 		CNET_LAUNCH_CHECK();
 		return CNET_OK;
@@ -575,13 +609,13 @@ int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const f
 	if (!partial) return CNET_ERR_OUT_OF_MEMORY;
 	dim3 grid((unsigned) col_blocks, (unsigned) nslabs);
 	if (vec)
-		hipLaunchKernelGGL(hadamard_bwd_shared_kernel<4>, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
+		CNET_LAUNCH_V4(hadamard_bwd_shared_kernel, nt, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
 				lddu, partial, rows, cols, rows_per_slab, accumulate);
 	else
-		hipLaunchKernelGGL(hadamard_bwd_shared_kernel<1>, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
+		hipLaunchKernelGGL((hadamard_bwd_shared_kernel<1, false>), grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
 				lddu, partial, rows, cols, rows_per_slab, accumulate);
 	CNET_LAUNCH_CHECK();
-	hipLaunchKernelGGL(slab_sum_kernel, dim3(nblocks(4L * cols)), dim3(TPB), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
+	hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned) ((4L * cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -591,10 +625,11 @@ int cnet_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_r
 	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= cols && ldy >= cols);
+	const bool nt = streaming(4, (long) rows * cols);
 	if (all_mult4({cols, ldx, ldy}) && all_aligned({x_re, x_im, y_re, y_im}))
-		hipLaunchKernelGGL(gelu_fwd_kernel<4>, CNET_GRID_2D(4), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+		CNET_LAUNCH_V4(gelu_fwd_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
 	else
-		hipLaunchKernelGGL(gelu_fwd_kernel<1>, CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+		hipLaunchKernelGGL((gelu_fwd_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -609,11 +644,12 @@ int cnet_cgelu_bwd(const float *x_re, const float *x_im, int64_t ldx, const floa
 	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
 	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
 	Grad4 dx = {dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im};
+	const bool nt = streaming(10, (long) rows * cols);
 	if (all_mult4({cols, ldx, ldg, lddx}) &&
 			all_aligned({x_re, x_im, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
-		hipLaunchKernelGGL(gelu_bwd_kernel<4>, CNET_GRID_2D(4), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+		CNET_LAUNCH_V4(gelu_bwd_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL(gelu_bwd_kernel<1>, CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+		hipLaunchKernelGGL((gelu_bwd_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -623,10 +659,11 @@ int cnet_crelu_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_r
 	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= cols && ldy >= cols);
+	const bool nt = streaming(4, (long) rows * cols);
 	if (all_mult4({cols, ldx, ldy}) && all_aligned({x_re, x_im, y_re, y_im}))
-		hipLaunchKernelGGL(crelu_fwd_kernel<4>, CNET_GRID_2D(4), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+		CNET_LAUNCH_V4(crelu_fwd_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
 	else
-		hipLaunchKernelGGL(crelu_fwd_kernel<1>, CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+		hipLaunchKernelGGL((crelu_fwd_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -641,11 +678,12 @@ int cnet_crelu_bwd(const float *x_re, const float *x_im, int64_t ldx, const floa
 	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
 	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
 	Grad4 dx = {dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im};
+	const bool nt = streaming(10, (long) rows * cols);
 	if (all_mult4({cols, ldx, ldg, lddx}) &&
 			all_aligned({x_re, x_im, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
-		hipLaunchKernelGGL(crelu_bwd_kernel<4>, CNET_GRID_2D(4), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+		CNET_LAUNCH_V4(crelu_bwd_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL(crelu_bwd_kernel<1>, CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+		hipLaunchKernelGGL((crelu_bwd_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -657,10 +695,11 @@ int cnet_residual_fwd(const float *u_re, const float *u_im, int64_t ldu, const f
 	if (!rows || !cols) return CNET_OK;
 	// a leading dimension of 0 makes that operand one row shared by all rows (a parameter added to every sample)
 	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && y_re && y_im && (ldu >= cols || ldu == 0) && (ldv >= cols || ldv == 0) && ldy >= cols);
+	const bool nt = streaming(6, (long) rows * cols);
 	if (all_mult4({cols, ldu, ldv, ldy}) && all_aligned({u_re, u_im, v_re, v_im, y_re, y_im}))
-		hipLaunchKernelGGL(residual_fwd_kernel<4>, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+		CNET_LAUNCH_V4(residual_fwd_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
 	else
-		hipLaunchKernelGGL(residual_fwd_kernel<1>, CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+		hipLaunchKernelGGL((residual_fwd_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -677,12 +716,13 @@ int cnet_residual_bwd(const float *g_dz_re, const float *g_dz_im, const float *g
 	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
 	Grad4 du = {du_dz_re, du_dz_im, du_dzs_re, du_dzs_im};
 	Grad4 dv = {dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im};
+	const bool nt = streaming(12, (long) rows * cols);
 	if (all_mult4({cols, ldg, lddu, lddv}) &&
 			all_aligned({g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, du_dz_re, du_dz_im, du_dzs_re, du_dzs_im, dv_dz_re, dv_dz_im,
 					dv_dzs_re, dv_dzs_im}))
-		hipLaunchKernelGGL(residual_bwd_kernel<4>, CNET_GRID_2D(4), g, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
+		CNET_LAUNCH_V4(residual_bwd_kernel, nt, CNET_GRID_2D(4), g, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL(residual_bwd_kernel<1>, CNET_GRID_2D(1), g, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
+		hipLaunchKernelGGL((residual_bwd_kernel<1, false>), CNET_GRID_2D(1), g, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -694,10 +734,11 @@ int cnet_l2out_bwd(const float *z_re, const float *z_im, int64_t ldz, float *dz_
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(z_re && z_im && dz_dz_re && dz_dz_im && dz_dzs_re && dz_dzs_im && ldz >= cols && lddz >= cols);
 	Grad4 dz = {dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im};
+	const bool nt = streaming(6, (long) rows * cols);
 	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
-		hipLaunchKernelGGL(l2out_bwd_kernel<4>, CNET_GRID_2D(4), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
+		CNET_LAUNCH_V4(l2out_bwd_kernel, nt, CNET_GRID_2D(4), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL(l2out_bwd_kernel<1>, CNET_GRID_2D(1), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
+		hipLaunchKernelGGL((l2out_bwd_kernel<1, false>), CNET_GRID_2D(1), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -709,10 +750,11 @@ int cnet_cross_entropy_bwd(const float *z_re, const float *z_im, int64_t ldz, co
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(z_re && z_im && s && labels && dz_dz_re && dz_dz_im && dz_dzs_re && dz_dzs_im && ldz >= cols && lddz >= cols);
 	Grad4 dz = {dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im};
+	const bool nt = streaming(6, (long) rows * cols);
 	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
-		hipLaunchKernelGGL(crossent_bwd_kernel<4>, CNET_GRID_2D(4), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
+		CNET_LAUNCH_V4(crossent_bwd_kernel, nt, CNET_GRID_2D(4), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
 	else
-		hipLaunchKernelGGL(crossent_bwd_kernel<1>, CNET_GRID_2D(1), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
+		hipLaunchKernelGGL((crossent_bwd_kernel<1, false>), CNET_GRID_2D(1), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -722,10 +764,11 @@ static int copy_or_add(const float *src, int64_t lds, float *dst, int64_t ldd, i
 	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(src && dst && lds >= cols && ldd >= cols);
+	const bool nt = streaming(2, (long) rows * cols);
 	if (all_mult4({cols, lds, ldd}) && all_aligned({src, dst}))
-		hipLaunchKernelGGL(copy2d_kernel<4>, CNET_GRID_2D(4), src, lds, dst, ldd, rows, cols, add);
+		CNET_LAUNCH_V4(copy2d_kernel, nt, CNET_GRID_2D(4), src, lds, dst, ldd, rows, cols, add);
 	else
-		hipLaunchKernelGGL(copy2d_kernel<1>, CNET_GRID_2D(1), src, lds, dst, ldd, rows, cols, add);
+		hipLaunchKernelGGL((copy2d_kernel<1, false>), CNET_GRID_2D(1), src, lds, dst, ldd, rows, cols, add);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -743,10 +786,11 @@ int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int6
 	CNET_CHECK_ARG(n >= 0);
 	if (!n) return CNET_OK;
 	CNET_CHECK_ARG(z_re && z_im && dzs_re && dzs_im);
+	const bool nt = streaming(4, (long) n);
 	if (n % 4 == 0 && all_aligned({z_re, z_im, dzs_re, dzs_im}))
-		hipLaunchKernelGGL(sgd_kernel<4>, dim3(nblocks(n / 4)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
+		CNET_LAUNCH_V4(sgd_kernel, nt, dim3(nblocks(n / 4)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
 	else
-		hipLaunchKernelGGL(sgd_kernel<1>, dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
+		hipLaunchKernelGGL((sgd_kernel<1, false>), dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -759,11 +803,12 @@ int cnet_adam_update(float *z_re, float *z_im, float *m_re, float *m_im, float *
 	CNET_CHECK_ARG(z_re && z_im && m_re && m_im && dzs_re && dzs_im);
 	const double denom = 1 - std::pow((double) beta, (double) (t + 1));
 	CNET_CHECK_ARG(denom != 0.0);
+	const bool nt = streaming(6, (long) n);
 	if (n % 4 == 0 && all_aligned({z_re, z_im, m_re, m_im, dzs_re, dzs_im}))
-		hipLaunchKernelGGL(adam_kernel<4>, dim3(nblocks(n / 4)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
+		CNET_LAUNCH_V4(adam_kernel, nt, dim3(nblocks(n / 4)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
 				(long) n, lr, beta, denom, zero_grad);
 	else
-		hipLaunchKernelGGL(adam_kernel<1>, dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
+		hipLaunchKernelGGL((adam_kernel<1, false>), dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
 				(long) n, lr, beta, denom, zero_grad);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;

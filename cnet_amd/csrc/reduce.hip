@@ -385,6 +385,132 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict
 	}
 }
 
+// Register-resident variants for rows of at most 64 * G * 4 * NIT columns (128-bit path): the row is read from memory
+// once, held in registers across the reduction and written back normalised, so the traffic is the algorithmic one
+// (the two-pass kernels above read every operand twice).  Same per-thread summation order as the two-pass kernels.
+template <int G, int NIT>
+__global__ __launch_bounds__(TPB) void l2norm_fwd_reg_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		float *__restrict__ yr, float *__restrict__ yi, long ldy, float *__restrict__ s, int rows, int cols) {
+	__shared__ double lds_d[TPB / 64];
+	CNET_ROW_SETUP();
+	const float *pr = zr + (long) row * ldz, *pi = zi + (long) row * ldz;
+	float4 a[NIT], b[NIT];
+#pragma unroll
+	for (int k = 0; k < NIT; ++k) {
+		const int c = (t + k * STRIDE) * 4;
+		a[k] = b[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+		if (c < cols) {
+			a[k] = *reinterpret_cast<const float4 *>(pr + c);
+			b[k] = *reinterpret_cast<const float4 *>(pi + c);
+		}
+	}
+	double sum = 0.0;
+	auto sq = [](float x, float y) { return (double) x * (double) x + (double) y * (double) y; };
+#pragma unroll
+	for (int k = 0; k < NIT; ++k) {
+		if ((t + k * STRIDE) * 4 < cols) {
+			sum += sq(a[k].x, b[k].x);
+			sum += sq(a[k].y, b[k].y);
+			sum += sq(a[k].z, b[k].z);
+			sum += sq(a[k].w, b[k].w);
+		}
+	}
+	sum = group_reduce<double, G>(sum, SumD(), lds_d, slot, wig, lane);
+	double nrm = sqrt(sum);
+	if (nrm <= 1.0e-15) nrm = 1.0e-15;
+	if ((float) (nrm * nrm * nrm) < 1.0e-15f) nrm = 1.0e-15;
+	const double inv = 1.0 / nrm;
+	if (!live) return;
+	float *qr = yr + (long) row * ldy, *qi = yi + (long) row * ldy;
+#pragma unroll
+	for (int k = 0; k < NIT; ++k) {
+		const int c = (t + k * STRIDE) * 4;
+		if (c < cols) {
+			*reinterpret_cast<float4 *>(qr + c) =
+					make_float4((float) (a[k].x * inv), (float) (a[k].y * inv), (float) (a[k].z * inv), (float) (a[k].w * inv));
+			*reinterpret_cast<float4 *>(qi + c) =
+					make_float4((float) (b[k].x * inv), (float) (b[k].y * inv), (float) (b[k].z * inv), (float) (b[k].w * inv));
+		}
+	}
+	if (t == 0 && s) s[row] = (float) sum;
+}
+
+template <int G, int NIT>
+__global__ __launch_bounds__(TPB) void l2norm_bwd_reg_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		const float *__restrict__ s, const float *__restrict__ g_re, const float *__restrict__ g_im,
+		const float *__restrict__ gs_re, const float *__restrict__ gs_im, long ldg, float *__restrict__ d_re,
+		float *__restrict__ d_im, float *__restrict__ ds_re, float *__restrict__ ds_im, long ldd, int rows, int cols,
+		int accumulate) {
+	__shared__ Cplx4 lds_c[TPB / 64];
+	CNET_ROW_SETUP();
+	const float *src[6] = {zr + (long) row * ldz, zi + (long) row * ldz, g_re + (long) row * ldg, g_im + (long) row * ldg,
+			gs_re + (long) row * ldg, gs_im + (long) row * ldg};
+	float *dst[4] = {d_re + (long) row * ldd, d_im + (long) row * ldd, ds_re + (long) row * ldd, ds_im + (long) row * ldd};
+	float v[NIT][6][4];  // [chunk][z_re, z_im, g_re, g_im, gs_re, gs_im][column]
+#pragma unroll
+	for (int k = 0; k < NIT; ++k) {
+		const int c = (t + k * STRIDE) * 4;
+#pragma unroll
+		for (int p = 0; p < 6; ++p) {
+			float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+			if (c < cols) x = *reinterpret_cast<const float4 *>(src[p] + c);
+			v[k][p][0] = x.x;
+			v[k][p][1] = x.y;
+			v[k][p][2] = x.z;
+			v[k][p][3] = x.w;
+		}
+	}
+	Cplx4 acc = {0.f, 0.f, 0.f, 0.f};  // a,b: G z   c,d: Gs conj z
+#pragma unroll
+	for (int k = 0; k < NIT; ++k) {
+		if ((t + k * STRIDE) * 4 < cols) {
+#pragma unroll
+			for (int q = 0; q < 4; ++q) {
+				const float a = v[k][0][q], b = v[k][1][q], gr = v[k][2][q], gi = v[k][3][q], sr = v[k][4][q], si = v[k][5][q];
+				acc.a += gr * a - gi * b;
+				acc.b += gr * b + gi * a;
+				acc.c += sr * a + si * b;
+				acc.d += si * a - sr * b;
+			}
+		}
+	}
+	acc = group_reduce<Cplx4, G>(acc, SumC4(), lds_c, slot, wig, lane);
+	if (!live) return;
+	const float S = s[row];
+	double nrm = sqrt((double) S);
+	if (nrm <= 1.0e-15) nrm = 1.0e-15;
+	float cube = (float) (nrm * nrm * nrm);
+	const float inv = (float) (1.0 / nrm);
+	const float Ar = 0.5f * (acc.a + acc.c) / cube, Ai = 0.5f * (acc.b + acc.d) / cube;
+#pragma unroll
+	for (int k = 0; k < NIT; ++k) {
+		const int c = (t + k * STRIDE) * 4;
+		if (c < cols) {
+			float o[4][4];
+#pragma unroll
+			for (int q = 0; q < 4; ++q) {
+				const float a = v[k][0][q], b = v[k][1][q], gr = v[k][2][q], gi = v[k][3][q], sr = v[k][4][q], si = v[k][5][q];
+				o[0][q] = gr * inv - (a * Ar + b * Ai);
+				o[1][q] = gi * inv - (a * Ai - b * Ar);
+				o[2][q] = sr * inv - (a * Ar - b * Ai);
+				o[3][q] = si * inv - (a * Ai + b * Ar);
+			}
+#pragma unroll
+			for (int p = 0; p < 4; ++p) {
+				float4 w = make_float4(o[p][0], o[p][1], o[p][2], o[p][3]);
+				if (accumulate) {
+					const float4 old = *reinterpret_cast<const float4 *>(dst[p] + c);
+					w.x += old.x;
+					w.y += old.y;
+					w.z += old.z;
+					w.w += old.w;
+				}
+				*reinterpret_cast<float4 *>(dst[p] + c) = w;
+			}
+		}
+	}
+}
+
 // ---------------------------------------------------------------------------------------------- batch (column) sum
 // stage 1: workgroup = 64 column groups (V columns each) x 4 row lanes, blockIdx.y = slab of rows; the four row lanes
 // are added through LDS in lane order; partial[slab][cols]
@@ -402,7 +528,23 @@ __global__ __launch_bounds__(TPB) void colsum_partial_kernel(const float *__rest
 #pragma unroll
 	for (int k = 0; k < V; ++k) acc[k] = 0.f;
 	if (live) {
-		for (int r = r0 + ty; r < r1; r += CS_Y) {
+		int r = r0 + ty;
+		if (V == 4) {
+			// four rows are requested before the first is added (same order of additions, more loads in flight)
+			for (; r + 3 * CS_Y < r1; r += 4 * CS_Y) {
+				float4 v[4];
+#pragma unroll
+				for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const float4 *>(src + (long) (r + u * CS_Y) * ld + col);
+#pragma unroll
+				for (int u = 0; u < 4; ++u) {
+					acc[0] += v[u].x;
+					acc[1 % V] += v[u].y;
+					acc[2 % V] += v[u].z;
+					acc[3 % V] += v[u].w;
+				}
+			}
+		}
+		for (; r < r1; r += CS_Y) {
 			if (V == 4) {
 				float4 v = *reinterpret_cast<const float4 *>(src + (long) r * ld + col);
 				acc[0] += v.x;
@@ -426,11 +568,19 @@ __global__ __launch_bounds__(TPB) void colsum_partial_kernel(const float *__rest
 
 __global__ __launch_bounds__(TPB) void colsum_final_kernel(const float *__restrict__ partial, int nslabs, int cols,
 		float *__restrict__ dst, int accumulate) {
-	const int c = blockIdx.x * TPB + threadIdx.x;
-	if (c >= cols) return;
-	float s = 0.f;
-	for (int k = 0; k < nslabs; ++k) s += partial[(long) k * cols + c];
-	dst[c] = accumulate ? dst[c] + s : s;
+	// 64 columns per workgroup x 4 lanes that each add one contiguous quarter of the slabs in order; the four quarter
+	// sums are then added in lane order
+	__shared__ float red[4][64];
+	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+	const int c = blockIdx.x * 64 + tx;
+	const bool live = c < cols;
+	const int per = (nslabs + 3) / 4, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
+	red[ty][tx] = live ? cnet::ordered_sum(partial + (long) k0 * cols + c, cols, k1 - k0) : 0.f;
+	__syncthreads();
+	if (ty == 0 && live) {
+		const float s = ((red[0][tx] + red[1][tx]) + red[2][tx]) + red[3][tx];
+		dst[c] = accumulate ? dst[c] + s : s;
+	}
 }
 
 inline bool mult4(long a, long b = 0, long c = 0, long d = 0) { return !(a % 4) && !(b % 4) && !(c % 4) && !(d % 4); }
@@ -454,6 +604,20 @@ using namespace cnet;
 		}                                                                                                             \
 		CNET_LAUNCH_CHECK();                                                                                          \
 	} while (0)
+
+// register-resident row kernels: NIT 128-bit chunks per thread and plane cover the row
+#define CNET_ROW_LAUNCH_REG(KERNEL, NIT_, ...)                                                                       \
+	do {                                                                                                              \
+		const bool wide = cols > 2048;                                                                                \
+		const int rpb = wide ? 1 : TPB / 64;                                                                          \
+		dim3 grid((unsigned) ((rows + rpb - 1) / rpb));                                                               \
+		if (wide) hipLaunchKernelGGL((KERNEL<4, NIT_>), grid, dim3(TPB), 0, rt().stream, __VA_ARGS__);                \
+		else hipLaunchKernelGGL((KERNEL<1, NIT_>), grid, dim3(TPB), 0, rt().stream, __VA_ARGS__);                     \
+		CNET_LAUNCH_CHECK();                                                                                          \
+	} while (0)
+
+// chunks of 4 columns each thread must hold so that its group (64 lanes, x4 wavefronts for wide rows) covers a row
+static inline int chunks_per_thread(int cols) { return (cols + (cols > 2048 ? 1024 : 256) - 1) / (cols > 2048 ? 1024 : 256); }
 
 extern "C" {
 
@@ -489,6 +653,13 @@ int cnet_l2norm_fwd(const float *z_re, const float *z_im, int64_t ldz, float *y_
 	if (!rows) return CNET_OK;
 	CNET_CHECK_ARG(z_re && z_im && y_re && y_im && ldz >= cols && ldy >= cols);
 	const bool vec = mult4(cols, ldz, ldy) && aligned16(z_re) && aligned16(z_im) && aligned16(y_re) && aligned16(y_im);
+	const int nit = chunks_per_thread(cols);
+	if (vec && nit <= 8) {
+		if (nit <= 2) CNET_ROW_LAUNCH_REG(l2norm_fwd_reg_kernel, 2, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols);
+		else if (nit <= 4) CNET_ROW_LAUNCH_REG(l2norm_fwd_reg_kernel, 4, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols);
+		else CNET_ROW_LAUNCH_REG(l2norm_fwd_reg_kernel, 8, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols);
+		return CNET_OK;
+	}
 	CNET_ROW_LAUNCH(l2norm_fwd_kernel, vec, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols);
 	return CNET_OK;
 }
@@ -504,6 +675,16 @@ int cnet_l2norm_bwd(const float *z_re, const float *z_im, int64_t ldz, const flo
 	const bool vec = mult4(cols, ldz, ldg, lddz) && aligned16(z_re) && aligned16(z_im) && aligned16(g_dz_re) && aligned16(g_dz_im) &&
 			aligned16(g_dzs_re) && aligned16(g_dzs_im) && aligned16(dz_dz_re) && aligned16(dz_dz_im) && aligned16(dz_dzs_re) &&
 			aligned16(dz_dzs_im);
+	const int nit = chunks_per_thread(cols);
+	if (vec && nit <= 4) {
+		if (nit <= 2)
+			CNET_ROW_LAUNCH_REG(l2norm_bwd_reg_kernel, 2, z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg,
+					dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate);
+		else
+			CNET_ROW_LAUNCH_REG(l2norm_bwd_reg_kernel, 4, z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg,
+					dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate);
+		return CNET_OK;
+	}
 	CNET_ROW_LAUNCH(l2norm_bwd_kernel, vec, z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg, dz_dz_re,
 			dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate);
 	return CNET_OK;
@@ -529,7 +710,7 @@ int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols
 	else
 		hipLaunchKernelGGL(colsum_partial_kernel<1>, grid, dim3(TPB), 0, rt().stream, src, (long) lds, partial, rows, cols, rows_per_slab);
 	CNET_LAUNCH_CHECK();
-	hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned) ((cols + TPB - 1) / TPB)), dim3(TPB), 0, rt().stream, partial, nslabs, cols, dst,
+	hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned) ((cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, nslabs, cols, dst,
 			accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
