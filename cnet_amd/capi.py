@@ -36,6 +36,10 @@ SIGNATURES = {
     "cnet_upload_wait_marker": [_i],
     "cnet_compute_wait_upload": [],
     "cnet_upload_sync": [],
+    "cnet_graph_begin": [],
+    "cnet_graph_end": [C.POINTER(C.c_void_p)],
+    "cnet_graph_launch": [C.c_void_p],
+    "cnet_graph_destroy": [C.c_void_p],
     "cnet_memcpy_d2h": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_memcpy_d2d": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_memset_zero": [C.c_void_p, C.c_size_t],

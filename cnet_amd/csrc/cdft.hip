@@ -57,6 +57,8 @@ static int get_plan(int n, Twiddle *out, bool create) {
 		return CNET_OK;
 	}
 	if (!create) return fail(CNET_ERR_INVALID_ARGUMENT, "no twiddle plan for n=%d: call cnet_cdft_plan first", n);
+	if (rt().capturing)
+		return fail(CNET_ERR_UNSUPPORTED, "the twiddle planes for n=%d would have to be built while a graph is being recorded: call cnet_cdft_plan first", n);
 	Twiddle t;
 	t.ld = (n + 3) / 4 * 4;  // rows start 16-byte aligned
 	size_t plane = (size_t) n * t.ld;
@@ -74,6 +76,8 @@ static int get_plan(int n, Twiddle *out, bool create) {
 static int get_triangular(int n, Twiddle *out) {
 	int rc = get_plan(n, out, true);
 	if (rc || out->tri_re) return rc;
+	if (rt().capturing)
+		return fail(CNET_ERR_UNSUPPORTED, "the triangular twiddle planes for n=%d would have to be built while a graph is being recorded: call cnet_ctriang_dft_plan first", n);
 	Twiddle &slot = g_twiddles[n];
 	const size_t plane = (size_t) n * slot.ld;
 	CNET_HIP(hipMalloc((void **) &slot.tri_re, 2 * plane * sizeof(float)));
@@ -113,6 +117,7 @@ int cnet_cdft_twiddle(int n, const float **f_re, const float **f_im) {
 
 int cnet_cdft_set_forward_matrix(int n, const float *host_f_re, const float *host_f_im) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	CNET_CHECK_ARG(n > 0 && n <= 46340);
 	Twiddle t;
 	int rc = get_plan(n, &t, true);

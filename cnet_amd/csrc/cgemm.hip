@@ -23,6 +23,7 @@
 //   each XCD works on a contiguous strip of C blocks and re-uses operand tiles through its own L2.
 #include "common.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 #include <type_traits>
 
@@ -51,6 +52,11 @@ struct CgemmArgs {
 	// Triangular B (square, zeros stored outside the triangle): 1 = B[k][n] is zero for k > n, 2 = zero for k < n.
 	// A block of columns [n0, n0 + BN) then only walks the K chunks that can hold non-zeros.
 	int tri;
+	// Split K: short grids (a small batch against a long reduction) run `splits` workgroups per block of C, each over
+	// `chunks_per_split` chunks of K, writing partial blocks to `partial`; splitk_reduce_kernel adds them in split order.
+	// blockIdx.z = batch index * splits + split.
+	int splits, chunks_per_split;
+	float *partial;  // [split][problem][batch][re, im][M][N]
 };
 
 // column blocks per grid row: with a triangular operand each workgroup handles a block and its mirror image
@@ -63,10 +69,28 @@ __device__ __forceinline__ void chunk_range(const CgemmArgs &args, int n0, int &
 	c_hi = (args.K + KC - 1) / KC;
 	if (args.tri == 1) c_hi = min(c_hi, (n0 + BN + KC - 1) / KC);
 	if (args.tri == 2) c_lo = n0 / KC;
+	if (args.splits > 1) {
+		c_lo = (blockIdx.z % args.splits) * args.chunks_per_split;
+		c_hi = min(c_hi, c_lo + args.chunks_per_split);
+	}
+}
+
+// where this workgroup writes its block: C itself, or its slice of the partial planes when K is split
+__device__ __forceinline__ void output_planes(const CgemmArgs &args, CgemmProblem &pb, long &ldc, int &accumulate) {
+	ldc = args.ldc;
+	accumulate = args.accumulate;
+	if (args.splits > 1) {
+		const long plane = (long) args.M * args.N;
+		const long nbatch = gridDim.z / args.splits, split = blockIdx.z % args.splits, b = blockIdx.z / args.splits;
+		pb.c_re = args.partial + (((split * gridDim.y + blockIdx.y) * nbatch + b) * 2) * plane;
+		pb.c_im = pb.c_re + plane;
+		ldc = args.N;
+		accumulate = 0;
+	}
 }
 
 __device__ __forceinline__ void batch_offset(CgemmProblem &pb, const CgemmArgs &args) {
-	const long z = blockIdx.z;
+	const long z = blockIdx.z / args.splits;
 	pb.a_re += z * args.stride_a;
 	pb.a_im += z * args.stride_a;
 	pb.b_re += z * args.stride_b;
@@ -188,6 +212,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 
 	CgemmProblem pb = args.p[blockIdx.y];
 	batch_offset(pb, args);
+	long ldc;
+	int accumulate;
+	output_planes(args, pb, ldc, accumulate);
 	const int M = args.M, N = args.N, K = args.K;
 
 	// ---- which block of C
@@ -312,9 +339,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 			for (int e = 0; e < 16; ++e) {
 				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
 				if (row < M) {
-					const long off = (long) row * args.ldc + col;
+					const long off = (long) row * ldc + col;
 					float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
-					if (args.accumulate) {
+					if (accumulate) {
 						vr += pb.c_re[off];
 						vi += pb.c_im[off];
 					}
@@ -452,6 +479,9 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 
 	CgemmProblem pb = args.p[blockIdx.y];
 	batch_offset(pb, args);
+	long ldc;
+	int accumulate;
+	output_planes(args, pb, ldc, accumulate);
 	const int K = args.K;
 
 	int pid = blockIdx.x;
@@ -613,9 +643,9 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 #pragma unroll
 			for (int e = 0; e < 16; ++e) {
 				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-				const long off = (long) row * args.ldc + col;
+				const long off = (long) row * ldc + col;
 				float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
-				if (args.accumulate) {
+				if (accumulate) {
 					vr += pb.c_re[off];
 					vi += pb.c_im[off];
 				}
@@ -626,13 +656,56 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	}  // pass
 }
 
+// C (+)= sum over splits of the partial blocks, added in split order (deterministic).  One thread per element of one plane.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(CgemmArgs args, int nprob, int nbatch) {
+	const long plane = (long) args.M * args.N;
+	const long idx = (long) blockIdx.x * 256 + threadIdx.x;
+	if (idx >= 2 * plane) return;
+	const int prob = blockIdx.y, b = blockIdx.z;
+	const int part = idx >= plane;  // 0: re, 1: im
+	const long e = idx - part * plane;
+	const long row = e / args.N, col = e - row * args.N;
+	const float *first = args.partial + (((long) prob * nbatch + b) * 2 + part) * plane + e;
+	float v = cnet::ordered_sum(first, (long) nprob * nbatch * 2 * plane, args.splits);
+	float *c = (part ? args.p[prob].c_im : args.p[prob].c_re) + (long) b * args.stride_c + row * args.ldc + col;
+	*c = args.accumulate ? *c + v : v;
+}
+
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
 int launch(const CgemmArgs &proto, int nprob, int batch) {
 	CgemmArgs args = proto;
 	args.tiles_m = (args.M + BM - 1) / BM;
 	args.tiles_n = (args.N + BN - 1) / BN;
 	constexpr size_t smem = 2 * (size_t) (2 * KC * (BM + 4) + 2 * KC * (BN + 4)) * sizeof(float);
-	dim3 grid(args.tiles_m * grid_tiles_n(args), nprob, batch);
+	// A grid that leaves most compute units idle while each workgroup walks a long K (a small batch against a long
+	// reduction: every chunk then waits a full memory latency) is cut along K.
+	args.splits = 1;
+	args.chunks_per_split = 0;
+	args.partial = nullptr;
+	{
+		const long blocks = (long) args.tiles_m * args.tiles_n * nprob * batch;
+		const long cus = cnet::rt().prop.multiProcessorCount;
+		const int nchunks = (args.K + KC - 1) / KC;
+		if (!args.tri && blocks * 2 <= cus && nchunks >= 8 && (long) batch * (cus / blocks) <= 65535) {
+			int splits = (int) std::min<long>(cus / blocks, nchunks / 4);
+			if (splits >= 2) {
+				args.chunks_per_split = (nchunks + splits - 1) / splits;
+				args.splits = (nchunks + args.chunks_per_split - 1) / args.chunks_per_split;  // no empty split
+				const size_t bytes = (size_t) args.splits * nprob * batch * 2 * args.M * args.N * sizeof(float);
+				args.partial = (float *) cnet::workspace(bytes);
+				if (!args.partial) return CNET_ERR_OUT_OF_MEMORY;
+			}
+		}
+	}
+	dim3 grid(args.tiles_m * grid_tiles_n(args), nprob, batch * args.splits);
+	auto finish = [&]() -> int {
+		if (args.splits > 1) {
+			dim3 rgrid((unsigned) ((2L * args.M * args.N + 255) / 256), nprob, batch);
+			hipLaunchKernelGGL(splitk_reduce_kernel, rgrid, dim3(256), 0, cnet::rt().stream, args, nprob, batch);
+			CNET_LAUNCH_CHECK();
+		}
+		return CNET_OK;
+	};
 	if constexpr (VEC == 4) {
 		if (args.M % BM == 0 && args.N % BN == 0 && args.K % KC == 0) {
 			auto fast = cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG>;
@@ -644,7 +717,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch) {
 			}
 			hipLaunchKernelGGL(fast, grid, dim3(NTHREADS), smem, cnet::rt().stream, args);
 			CNET_LAUNCH_CHECK();
-			return CNET_OK;
+			return finish();
 		}
 	}
 	auto kern = cgemm_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, VEC>;
@@ -656,7 +729,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch) {
 	}
 	hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, cnet::rt().stream, args);
 	CNET_LAUNCH_CHECK();
-	return CNET_OK;
+	return finish();
 }
 
 template <bool A_MCONTIG, bool B_NCONTIG, int VEC>

@@ -23,6 +23,7 @@ struct Runtime {
 	hipEvent_t upload_done = nullptr, compute_done = nullptr;
 	static constexpr int kMarkers = 8;
 	hipEvent_t marker[kMarkers] = {};  // caller-numbered points of the compute stream
+	bool capturing = false;  // between cnet_graph_begin and cnet_graph_end: nothing may allocate or wait
 	hipDeviceProp_t prop;
 	// grow-only scratch for two-stage deterministic reductions (never allocated inside a hot loop twice
 	// for the same size)
@@ -39,6 +40,12 @@ void *workspace(size_t bytes);
 #define CNET_REQUIRE_INIT()                                                              \
 	do {                                                                                 \
 		if (!cnet::rt().ready) return cnet::fail(CNET_ERR_NOT_INITIALIZED, "%s: cnet_init() has not been called", __func__); \
+	} while (0)
+
+// entry points that wait for the device or allocate cannot be recorded into a graph
+#define CNET_NOT_IN_CAPTURE()                                                                                                \
+	do {                                                                                                                     \
+		if (cnet::rt().capturing) return cnet::fail(CNET_ERR_UNSUPPORTED, "%s: not allowed between cnet_graph_begin and cnet_graph_end", __func__); \
 	} while (0)
 
 #define CNET_HIP(call)                                             \

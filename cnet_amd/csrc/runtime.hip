@@ -28,6 +28,10 @@ int hip_fail(hipError_t e, const char *what) {
 void *workspace(size_t bytes) {
 	Runtime &r = rt();
 	if (bytes <= r.workspace_bytes) return r.workspace;
+	if (r.capturing) {
+		fail(CNET_ERR_UNSUPPORTED, "the workspace would have to grow while a graph is being recorded: run the same calls once before recording");
+		return nullptr;
+	}
 	if (r.workspace) {
 		// queued kernels may still read the old buffer
 		hipStreamSynchronize(r.stream);
@@ -126,6 +130,7 @@ void *cnet_stream(void) { return rt().ready ? (void *) rt().stream : nullptr; }
 
 int cnet_set_stream(void *hip_stream) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	Runtime &r = rt();
 	CNET_HIP(hipStreamSynchronize(r.stream));
 	r.stream = hip_stream ? (hipStream_t) hip_stream : r.own_stream;
@@ -134,12 +139,14 @@ int cnet_set_stream(void *hip_stream) {
 
 int cnet_sync(void) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	CNET_HIP(hipStreamSynchronize(rt().stream));
 	return CNET_OK;
 }
 
 int cnet_alloc(size_t bytes, void **out) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	CNET_CHECK_ARG(out != nullptr);
 	*out = nullptr;
 	if (bytes == 0) return CNET_OK;
@@ -149,6 +156,7 @@ int cnet_alloc(size_t bytes, void **out) {
 
 int cnet_free(void *ptr) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	if (!ptr) return CNET_OK;
 	CNET_HIP(hipStreamSynchronize(rt().stream));
 	CNET_HIP(hipFree(ptr));
@@ -157,6 +165,7 @@ int cnet_free(void *ptr) {
 
 int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	if (!bytes) return CNET_OK;
 	CNET_CHECK_ARG(dst && host_src);
 	// pageable source: hipMemcpyAsync stages and returns after the copy was consumed from the host buffer
@@ -167,6 +176,7 @@ int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes) {
 
 int cnet_host_alloc(size_t bytes, void **out) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	CNET_CHECK_ARG(out != nullptr);
 	*out = nullptr;
 	if (bytes == 0) return CNET_OK;
@@ -176,6 +186,7 @@ int cnet_host_alloc(size_t bytes, void **out) {
 
 int cnet_host_free(void *ptr) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	if (!ptr) return CNET_OK;
 	// copies queued from this buffer must have left it
 	CNET_HIP(hipStreamSynchronize(rt().stream));
@@ -231,16 +242,67 @@ int cnet_compute_wait_upload(void) {
 
 int cnet_upload_sync(void) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	CNET_HIP(hipStreamSynchronize(rt().upload_stream));
 	return CNET_OK;
 }
 
 int cnet_memcpy_d2h(void *host_dst, const void *src, size_t bytes) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	if (!bytes) return CNET_OK;
 	CNET_CHECK_ARG(host_dst && src);
 	CNET_HIP(hipMemcpyAsync(host_dst, src, bytes, hipMemcpyDeviceToHost, rt().stream));
 	CNET_HIP(hipStreamSynchronize(rt().stream));
+	return CNET_OK;
+}
+
+// ---- graphs: record the launches of a repeated sequence once, replay them with one call
+int cnet_graph_begin(void) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
+	CNET_HIP(hipStreamBeginCapture(rt().stream, hipStreamCaptureModeThreadLocal));
+	rt().capturing = true;
+	return CNET_OK;
+}
+
+int cnet_graph_end(void **graph_exec) {
+	CNET_REQUIRE_INIT();
+	Runtime &r = rt();
+	if (!r.capturing) return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_graph_end without cnet_graph_begin");
+	r.capturing = false;
+	hipGraph_t graph = nullptr;
+	hipError_t e = hipStreamEndCapture(r.stream, &graph);
+	if (e != hipSuccess || !graph) {
+		(void) hipGetLastError();
+		if (graph_exec) *graph_exec = nullptr;
+		return hip_fail(e != hipSuccess ? e : hipErrorUnknown, "hipStreamEndCapture (a call inside the recording failed)");
+	}
+	if (!graph_exec) {  // the caller abandons the recording
+		(void) hipGraphDestroy(graph);
+		return CNET_OK;
+	}
+	hipGraphExec_t exec = nullptr;
+	e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+	(void) hipGraphDestroy(graph);
+	if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+	*graph_exec = exec;
+	return CNET_OK;
+}
+
+int cnet_graph_launch(void *graph_exec) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
+	CNET_CHECK_ARG(graph_exec != nullptr);
+	CNET_HIP(hipGraphLaunch((hipGraphExec_t) graph_exec, rt().stream));
+	return CNET_OK;
+}
+
+int cnet_graph_destroy(void *graph_exec) {
+	CNET_REQUIRE_INIT();
+	if (!graph_exec) return CNET_OK;
+	CNET_HIP(hipStreamSynchronize(rt().stream));
+	CNET_HIP(hipGraphExecDestroy((hipGraphExec_t) graph_exec));
 	return CNET_OK;
 }
 

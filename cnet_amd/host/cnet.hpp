@@ -591,6 +591,46 @@ class CNet {
 	};
 	Stage stage_[2];
 	int active_ = 0;
+	// recorded phases of a step, one set per buffer of the data input (device pointers are frozen into a recording)
+	struct StepGraphs {
+		void *fwd = NULL, *bwd = NULL, *upd = NULL;
+		float upd_lr = 0.f;
+	};
+	StepGraphs graphs_[2];
+	bool use_graphs_ = false;
+	bool warmed_[3] = {false, false, false};  // phase has run once since useGraphs(true)
+
+	void dropGraphs() {
+		for (auto &g : graphs_) {
+			for (void *e : {g.fwd, g.bwd, g.upd})
+				if (e) cnet_graph_destroy(e);
+			g = StepGraphs();
+		}
+		warmed_[0] = warmed_[1] = warmed_[2] = false;
+	}
+	template <class Body>
+	void runPhase(int phase, void *&exec, Body body) {
+		if (!use_graphs_) {
+			body();
+			return;
+		}
+		if (!exec) {
+			if (!warmed_[phase]) {  // first time: run as usual, so that every buffer the library needs exists
+				body();
+				warmed_[phase] = true;
+				return;
+			}
+			ck(cnet_graph_begin(), "cnet_graph_begin");
+			try {
+				body();
+			} catch (...) {
+				cnet_graph_end(NULL);
+				throw;
+			}
+			ck(cnet_graph_end(&exec), "cnet_graph_end");
+		}
+		ck(cnet_graph_launch(exec), "cnet_graph_launch");
+	}
 
 	static void ck(int rc, const char *what) {
 		if (rc != CNET_OK)
@@ -746,6 +786,8 @@ public:
 		}
 		batch_ = 0;
 		d_labels_ = NULL;
+		dropGraphs();
+		use_graphs_ = false;
 		for (auto &st : stage_) {
 			if (st.host_labels) cnet_host_free(st.host_labels);
 			st = Stage();
@@ -955,8 +997,14 @@ private:
 			CFunc::Slot &own = f->slots_[0];
 			for (int c = 0; c < f->no_outputs(); ++c) {
 				CFunc::Slot &u = upstream(f, c);
-				ck(cnet_add2d(u.g(2), u.len, own.g(2), own.len, own.rows, own.len), "cnet_add2d");
-				ck(cnet_add2d(u.g(3), u.len, own.g(3), own.len, own.rows, own.len), "cnet_add2d");
+				// both dz* planes in one launch: they are adjacent and dense in the consumer's slot and in the node's own block
+				const int64_t both = 2 * (int64_t) own.rows * own.len;
+				if (both <= INT32_MAX) {
+					ck(cnet_add2d(u.g(2), both, own.g(2), both, 1, (int) both), "cnet_add2d");
+				} else {
+					ck(cnet_add2d(u.g(2), u.len, own.g(2), own.len, own.rows, own.len), "cnet_add2d");
+					ck(cnet_add2d(u.g(3), u.len, own.g(3), own.len, own.rows, own.len), "cnet_add2d");
+				}
 			}
 			return;
 		}
@@ -1206,25 +1254,47 @@ public:
 	}
 	bool GpuForward() {
 		requireAllocated("GpuForward");
-		for (auto f : func_list_) nodeForward(f);
+		runPhase(0, graphs_[active_].fwd, [&] {
+			for (auto f : func_list_) nodeForward(f);
+		});
 		return true;
 	}
 	bool gpuBackward() {
 		requireAllocated("gpuBackward");
-		for (int k = (int) func_list_.size() - 1; k >= 0; --k) nodeBackward(func_list_[k], true);
+		runPhase(1, graphs_[active_].bwd, [&] {
+			for (int k = (int) func_list_.size() - 1; k >= 0; --k) nodeBackward(func_list_[k], true);
+		});
 		return true;
 	}
 	// z -= l_rate * dzs on every input function (the data input too, impl/cnet.h:413-421), then its gradients are cleared
 	void gpuUpdateInputs(float l_rate) {
 		requireAllocated("gpuUpdateInputs");
-		for (auto f : inputs_) {
-			CFunc::Slot &s = f->slots_[0];
-			const size_t n = (size_t) s.rows * s.len;
-			float *z = s.z;
-			ck(cnet_sgd_update(z, z + n, s.g(2), s.g(3), (int64_t) n, l_rate, 1), "cnet_sgd_update");
-			ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
+		StepGraphs &g = graphs_[active_];
+		if (g.upd && g.upd_lr != l_rate) {  // the rate is frozen into a recording
+			ck(cnet_graph_destroy(g.upd), "cnet_graph_destroy");
+			g.upd = NULL;
 		}
+		g.upd_lr = l_rate;
+		runPhase(2, g.upd, [&] {
+			for (auto f : inputs_) {
+				CFunc::Slot &s = f->slots_[0];
+				const size_t n = (size_t) s.rows * s.len;
+				float *z = s.z;
+				ck(cnet_sgd_update(z, z + n, s.g(2), s.g(3), (int64_t) n, l_rate, 1), "cnet_sgd_update");
+				ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
+			}
+		});
 	}
+	// Replay the kernels of GpuForward / gpuBackward / gpuUpdateInputs from recorded graphs instead of launching them
+	// one by one (a step at small batch sizes is bound by launch overhead).  Each phase runs once as usual after this
+	// call (which also sizes the library's workspace), is recorded on its next call and replayed from then on; there is
+	// one recording per phase and per buffer of the data input.  Same kernels, same arguments, same results.
+	void useGraphs(bool on) {
+		requireAllocated("useGraphs");
+		if (!on) dropGraphs();
+		use_graphs_ = on;
+	}
+	bool usingGraphs() const { return use_graphs_; }
 	// The Adam-style step of upstream GpuNet::adamUpdate (gpu/gpu_func.h:503-510, gpu/kernels.cpp:494-514) on every input
 	// function: the first moment lives in the node's dz planes, dz* is cleared, dz is kept.
 	void gpuAdamUpdate(float l_rate, float beta, int t) {

@@ -83,6 +83,19 @@ int cnet_mark_compute(int marker);
 int cnet_upload_wait_marker(int marker);
 int cnet_compute_wait_upload(void);
 int cnet_upload_sync(void);
+
+/* ---- Graphs: a training step at small batch sizes is bound by launch overhead (upstream pays a cudaDeviceSynchronize
+ *      per layer on top, gpu/kernels.cpp:104-105).  Between cnet_graph_begin and cnet_graph_end the layer entry points
+ *      record their kernels on the library's stream instead of running them; cnet_graph_launch replays the recording
+ *      with one call.  Pointers, shapes and scalars (learning rate, accumulate flags) are frozen into the recording.
+ *      Entry points that allocate or wait (cnet_alloc, cnet_free, cnet_sync, the blocking copies, the first use of a DFT
+ *      length or of a larger workspace) return CNET_ERR_UNSUPPORTED while recording, and cnet_graph_end then fails:
+ *      run the sequence once before recording it.  Clearing memory inside a recording uses a fill kernel
+ *      (cnet_memset_zero), never a memset node. */
+int cnet_graph_begin(void);
+int cnet_graph_end(void **graph_exec);      /* NULL: drop the recording */
+int cnet_graph_launch(void *graph_exec);
+int cnet_graph_destroy(void *graph_exec);
 int cnet_memcpy_d2h(void *host_dst, const void *src, size_t bytes);   /* *_copy_from_gpu (gpu/allocator.h:262-328); synchronises */
 int cnet_memcpy_d2d(void *dst, const void *src, size_t bytes);
 int cnet_memset_zero(void *dst, size_t bytes);  /* GpuMapping::zeroGradients (gpu/kernels.cpp:444-469) */

@@ -709,7 +709,9 @@ static void test_saved_model(const std::string &dir, const std::string &tmp) {
 
 // ------------------------------------------------------------------------------------------------- host batch pipeline
 // README net fed from a BatchedDataReader: (a) every batch copied inside gpuForward, (b) batches sent ahead with
-// gpuPrefetch() into the device double buffer while the previous step computes.  Both must give the same bits.
+// gpuPrefetch() into the device double buffer while the previous step computes, (c) as (b) with the three phases of a
+// step replayed from recorded graphs, (d) graphs without prefetch.  All must give the same bits; the learning rate
+// changes half way, which forces the update phase to be recorded again.
 static void build_readme(CNet &net, int n, int classes, int *inp, int *outp) {
 	*inp = net.add(new CInput(OutSize(n)));
 	auto fft = net.add(new FourierTrans(InSize(n)), {*inp});
@@ -746,10 +748,12 @@ static void test_pipeline(int B, int steps, bool timing_only) {
 		return;
 	}
 	SyntheticReader data(n, 3 * B + 7, classes);
-	std::vector<float> losses[2];
-	std::vector<float> weights[2];
-	double ms[2] = {0, 0};
-	for (int mode = 0; mode < 2; ++mode) {
+	constexpr int MODES = 4;
+	std::vector<float> losses[MODES];
+	std::vector<float> weights[MODES];
+	double ms[MODES] = {0, 0, 0, 0};
+	for (int mode = 0; mode < MODES; ++mode) {
+		const bool prefetch = mode == 1 || mode == 2, graphs = mode >= 2;
 		CNet net;
 		int inp, outp;
 		build_readme(net, n, classes, &inp, &outp);
@@ -759,24 +763,25 @@ static void test_pipeline(int B, int steps, bool timing_only) {
 		SyntheticReader reader = data;  // same order for both modes
 		InputBatch ring[3] = {InputBatch(B, n), InputBatch(B, n), InputBatch(B, n)};
 		if (mode == 0 && !timing_only) expect("batches built after cnet_init are page-locked", ring[0].isPinned());
+		if (graphs) net.useGraphs(true);
 		net.sync();
 		auto t0 = std::chrono::steady_clock::now();
-		if (mode == 1) {
+		if (prefetch) {
 			reader.nextBatch(ring[0]);
 			net.gpuPrefetch(cin, ring[0]);
 		}
 		for (int s = 0; s < steps; ++s) {
 			InputBatch &cur = ring[s % 3];
-			if (mode == 0) reader.nextBatch(cur);
+			if (!prefetch) reader.nextBatch(cur);
 			net.gpuForward(cin, cen, cur);
-			if (mode == 1 && s + 1 < steps) {  // the next batch travels while this step computes
+			if (prefetch && s + 1 < steps) {  // the next batch travels while this step computes
 				InputBatch &next = ring[(s + 1) % 3];
 				reader.nextBatch(next);
 				net.gpuPrefetch(cin, next);
 			}
 			losses[mode].push_back(net.getLoss(cen, &cur));
 			net.gpuBackward();
-			net.gpuUpdateInputs(lr / B);
+			net.gpuUpdateInputs((s < steps / 2 ? lr : 0.5f * lr) / B);
 		}
 		net.sync();
 		ms[mode] = 1e3 * std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / steps;
@@ -816,12 +821,17 @@ static void test_pipeline(int B, int steps, bool timing_only) {
 	if (!timing_only) {
 		expect("losses identical with and without prefetch (" + std::to_string(steps) + " steps)", losses[0] == losses[1]);
 		expect("weights identical after training with and without prefetch", weights[0] == weights[1] && !weights[0].empty());
+		expect("losses identical with graph replay (prefetch)", losses[0] == losses[2]);
+		expect("weights identical with graph replay (prefetch)", weights[0] == weights[2]);
+		expect("losses identical with graph replay (copy in forward)", losses[0] == losses[3]);
+		expect("weights identical with graph replay (copy in forward)", weights[0] == weights[3]);
 		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
 	}
 	printf("{\"workload\": \"README net 784 -> 10, SGD, batches from a BatchedDataReader\", \"batch\": %d, \"steps\": %d, "
-		   "\"ms_per_step_copy_in_forward\": %.3f, \"ms_per_step_prefetch\": %.3f, \"samples_per_sec_copy_in_forward\": %.1f, "
-		   "\"samples_per_sec_prefetch\": %.1f, \"upload_bytes_per_step\": %zu}\n",
-			B, steps, ms[0], ms[1], B / ms[0] * 1e3, B / ms[1] * 1e3, (size_t) 2 * B * n * sizeof(float));
+		   "\"ms_per_step_copy_in_forward\": %.3f, \"ms_per_step_prefetch\": %.3f, \"ms_per_step_prefetch_graphs\": %.3f, "
+		   "\"ms_per_step_graphs\": %.3f, \"samples_per_sec_copy_in_forward\": %.1f, \"samples_per_sec_prefetch\": %.1f, "
+		   "\"samples_per_sec_prefetch_graphs\": %.1f, \"upload_bytes_per_step\": %zu}\n",
+			B, steps, ms[0], ms[1], ms[2], ms[3], B / ms[0] * 1e3, B / ms[1] * 1e3, B / ms[2] * 1e3, (size_t) 2 * B * n * sizeof(float));
 }
 
 // ------------------------------------------------------------------------------------------------- error behaviour
@@ -926,7 +936,7 @@ int main(int argc, char **argv) {
 		if (what == "embedding" || what == "all") test_embedding();
 		if (what == "adam" || what == "all") test_adam();
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
-		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 7, false);
+		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12, false);
 		if (what == "pipeline_timing") test_pipeline(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, true);
 		if (what == "errors" || what == "all") test_errors();
 		if (what == "c4")

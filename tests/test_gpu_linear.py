@@ -88,6 +88,53 @@ def test_cgemm_all_layouts(gpu, port):
                 assert err < 1e-5, (a_km, b_km, cj, err)
 
 
+@pytest.mark.parametrize("M,N,K", [(8, 24, 1000), (64, 64, 4096), (40, 100, 333), (64, 784, 784), (3, 5, 2049)])
+def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
+    """Few blocks of C against a long K: the launch is cut along K and the partial blocks are added in a fixed order.
+    All four layouts, conj(B), accumulation into a window of a wider buffer, and run-to-run identical bits."""
+    A = seeded(port, 1, (M, K)) + 1j * seeded(port, 2, (M, K))
+    Bm = seeded(port, 3, (K, N)) + 1j * seeded(port, 4, (K, N))
+    base = seeded(port, 5, (M, N + 9))
+    for a_km in (0, 1):
+        for b_km in (0, 1):
+            a_h = A.T if a_km else A
+            b_h = Bm if b_km else Bm.T
+            a = ops.CMat.from_host(np.ascontiguousarray(a_h.real), np.ascontiguousarray(a_h.imag))
+            b = ops.CMat.from_host(np.ascontiguousarray(b_h.real), np.ascontiguousarray(b_h.imag))
+            cj = (a_km + b_km) % 2
+            want = A @ (Bm.conj() if cj else Bm)
+            c = ops.CMat.empty(M, N)
+            ops.cgemm(a, b, c, M, N, K, a_km, b_km, cj)
+            first = c.host()
+            err = np.linalg.norm(first[0] + 1j * first[1] - want) / np.linalg.norm(want)
+            assert err < 1e-5, (a_km, b_km, err)
+            ops.cgemm(a, b, c, M, N, K, a_km, b_km, cj)
+            again = c.host()
+            assert np.array_equal(first[0], again[0]) and np.array_equal(first[1], again[1])
+            wide = ops.CMat(ops.Plane.from_host(base), ops.Plane.from_host(base))
+            ops.cgemm(a, b, wide.sub(4, N), M, N, K, a_km, b_km, cj, accumulate=1)
+            hr, hi = wide.re.owner.download(), wide.im.owner.download()
+            got = (hr[:, 4:4 + N] - base[:, 4:4 + N]) + 1j * (hi[:, 4:4 + N] - base[:, 4:4 + N])
+            assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-5
+            keep = np.ones(N + 9, bool); keep[4:4 + N] = False
+            assert np.array_equal(hr[:, keep], base[:, keep]) and np.array_equal(hi[:, keep], base[:, keep])
+
+
+def test_cgemm_batched_short_grid(gpu, port):
+    """Strided batch of small products with a long K: the batch index and the K split share one grid dimension."""
+    nb, M, N, K = 3, 16, 32, 640
+    A = seeded(port, 11, (nb, M, K)) + 1j * seeded(port, 12, (nb, M, K))
+    Bm = seeded(port, 13, (K, N)) + 1j * seeded(port, 14, (K, N))
+    a = ops.CMat.from_host(np.ascontiguousarray(A.real).reshape(nb * M, K), np.ascontiguousarray(A.imag).reshape(nb * M, K))
+    b = ops.CMat.from_host(np.ascontiguousarray(Bm.real), np.ascontiguousarray(Bm.imag))
+    c = ops.CMat.empty(nb * M, N)
+    ops.cgemm_batched(a, M * K, b, 0, c, M * N, M, N, K, nb, a_kmajor=0, b_kmajor=1, conj_a=1)
+    cr, ci = c.host()
+    want = np.conj(A) @ Bm
+    got = (cr + 1j * ci).reshape(nb, M, N)
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-5
+
+
 def test_linear_headline_shape_rows_against_oracle(gpu, port):
     """B=4096, 1024->1024 (the benchmark shape).  The oracle computes a 24-row subsample; dW/dW* are compared on a
     batch equal to that subsample, and the full-size run is checked through linearity in the batch:
