@@ -1144,13 +1144,14 @@ public:
 		if (f->typeId() == isCrossEntropy) {
 			CrossEntropy *c = (CrossEntropy *) f;
 			const int n = f->input().length_;
-			ck(cnet_memcpy_d2h(c->output_.real_, c->d_norm_ + (size_t) b * n, n * sizeof(float)), "cnet_memcpy_d2h");
-			ck(cnet_memcpy_d2h(c->output_.imag_, c->d_norm_ + (size_t) (f->rows_ + b) * n, n * sizeof(float)), "cnet_memcpy_d2h");
+			const int rb = f->rows_ == 1 ? 0 : b;  // an output that hangs off parameters only has one row
+			ck(cnet_memcpy_d2h(c->output_.real_, c->d_norm_ + (size_t) rb * n, n * sizeof(float)), "cnet_memcpy_d2h");
+			ck(cnet_memcpy_d2h(c->output_.imag_, c->d_norm_ + (size_t) (f->rows_ + rb) * n, n * sizeof(float)), "cnet_memcpy_d2h");
 			int32_t am = 0;
-			ck(cnet_memcpy_d2h(&am, c->d_argmax_ + b, sizeof(am)), "cnet_memcpy_d2h");
+			ck(cnet_memcpy_d2h(&am, c->d_argmax_ + rb, sizeof(am)), "cnet_memcpy_d2h");
 			c->prediction_ = am;
 		} else if (f->typeId() == isL2Out) {
-			ck(cnet_memcpy_d2h(((L2Out *) f)->output_.real_, ((L2Out *) f)->d_loss_ + b, sizeof(float)), "cnet_memcpy_d2h");
+			ck(cnet_memcpy_d2h(((L2Out *) f)->output_.real_, ((L2Out *) f)->d_loss_ + (f->rows_ == 1 ? 0 : b), sizeof(float)), "cnet_memcpy_d2h");
 		}
 	}
 	void fetchAll(int b) {

@@ -11,6 +11,7 @@
 //   facade_test saved_model <golden dir> <scratch dir>   upstream-written .mod files restored and run on the device
 //   facade_test pipeline [B steps]  reader -> page-locked batches -> device, with and without gpuPrefetch (same bits)
 //   facade_test pipeline_timing B steps   the same, timing only (JSON line)
+//   facade_test upstream_nets      the nets of upstream's own GPU tests (E2E chain, fan-out into one consumer, ...)
 //   facade_test errors             error behaviour
 //   facade_test c4 n blocks B steps lr   throughput of the residual stack (no oracle), JSON line
 #include <chrono>
@@ -834,6 +835,156 @@ static void test_pipeline(int B, int steps, bool timing_only) {
 			B, steps, ms[0], ms[1], ms[2], ms[3], B / ms[0] * 1e3, B / ms[1] * 1e3, B / ms[2] * 1e3, (size_t) 2 * B * n * sizeof(float));
 }
 
+// ------------------------------------------------------------------------------------------------- upstream's test nets
+// The nets of upstream's own GPU tests (tests/gputests.h: testE2E :378, testTwoOutputs :560, testZeroGradient :641,
+// testInputGradient :1143, testRelu :30), built from one description for the facade and for the oracle.  Upstream
+// doubles every net into two identical branches to get two samples; here the batch rows play that part.
+struct SpecNode {
+	int kind, a, b;        // kind-specific sizes (Linear: in1, in2; others: n)
+	std::vector<int> in;   // uids of the producers (uid = position + 1)
+};
+
+static CFunc *make_func(const SpecNode &n) {
+	switch (n.kind) {
+	case orc::kInput: return new CInput(OutSize(n.a));
+	case orc::kLinear: return new Linear(InSize(n.a), InSize(n.b));
+	case orc::kFourier: return new FourierTrans(InSize(n.a));
+	case orc::kTriangFourier: return new TriangFourier(InSize(n.a));
+	case orc::kHadamard: return new Hadamard(InSize(n.a), InSize(n.a));
+	case orc::kGelu: return new CGelu(InSize(n.a));
+	case orc::kCrelu: return new CRelu(InSize(n.a));
+	case orc::kResidual: return new Residual(InSize(n.a));
+	case orc::kSoftMax: return new SoftMax(InSize(n.a));
+	case orc::kCrossEntropy: return new CrossEntropy(InSize(n.a));
+	case orc::kL2Out: return new L2Out(InSize(n.a));
+	}
+	return NULL;
+}
+
+// Runs `steps` rounds of forward / backward(label) / SGD on a batch of B rows and compares, per row, every node's input
+// block and gradients (ranges fed by batched producers), every output's loss, and at the end of each round the
+// parameter gradients (summed over the rows) and the updated parameters.
+static void run_spec(const std::string &name, const std::vector<SpecNode> &spec, int B, int steps) {
+	CNet net;
+	orc::Net on;
+	orc::Rng rng(1234 + spec.size());
+	for (auto &n : spec) {
+		net.add(make_func(n), n.in);
+		on.add(n.kind, n.a, n.b, 0, n.in.empty() ? NULL : n.in.data(), (int) n.in.size());
+	}
+	const int main_in = 1;  // the first function of every net here is the data input
+	for (size_t k = 0; k < spec.size(); ++k) {
+		if (spec[k].kind != orc::kInput) continue;
+		Vars *v = net[(int) k + 1]->mutable_input();
+		fill_normal(rng, v->real_, 2 * (size_t) v->length_, 0.7);
+		std::copy(v->real_, v->real_ + 2 * v->length_, on.at((int) k + 1)->in.re);
+	}
+	net.allocateOnGpu(B);
+	CInput *cin = (CInput *) net[main_in];
+	OutputFunc *outp = dynamic_cast<OutputFunc *>(net.findFirstOutput());
+	const int n_in = cin->input().length_;
+	auto is_param = [&](int uid) { return spec[uid - 1].kind == orc::kInput && uid != main_in; };
+	// nodes that only depend on parameters have a single row
+	std::vector<int> batched(spec.size() + 1, 0);
+	batched[main_in] = 1;
+	for (size_t k = 0; k < spec.size(); ++k)
+		for (int p : spec[k].in) batched[k + 1] |= batched[p];
+
+	for (int step = 0; step < steps; ++step) {
+		std::vector<float> xr((size_t) B * n_in), xi((size_t) B * n_in);
+		fill_normal(rng, xr.data(), xr.size(), 1.0);
+		fill_normal(rng, xi.data(), xi.size(), 1.0);
+		std::vector<int> labels(B);
+		InputBatch batch(B, n_in);
+		for (int b = 0; b < B; ++b) {
+			labels[b] = (int) (rng.next() % 3);
+			batch.add(xr.data() + (size_t) b * n_in, xi.data() + (size_t) b * n_in, n_in, labels[b]);
+		}
+		net.gpuForward(cin, outp, batch);
+		net.gpuBackward();
+		ErrAcc z, g, loss;
+		for (int b = 0; b < B; ++b) {
+			std::copy(xr.begin() + (size_t) b * n_in, xr.begin() + (size_t) (b + 1) * n_in, on.at(main_in)->in.re);
+			std::copy(xi.begin() + (size_t) b * n_in, xi.begin() + (size_t) (b + 1) * n_in, on.at(main_in)->in.im);
+			on.forward();
+			on.backward(labels[b]);
+			net.fetchAll(b);
+			for (size_t k = 0; k < spec.size(); ++k) {
+				const int uid = (int) k + 1;
+				if (spec[k].kind == orc::kInput) continue;
+				if (!batched[uid] && b > 0) continue;  // a chain that hangs off parameters only: one row
+				CFunc *f = net[uid];
+				orc::Node *o = on.at(uid);
+				const int len = f->input().length_;
+				z.add(f->input().real_, o->in.re, 2 * len);
+				int off = 0;
+				for (int p : spec[k].in) {
+					const int plen = net[p]->outSize();
+					// gradient ranges fed by a parameter hold the sum over the rows on the device side
+					if (!is_param(p) || !batched[uid])
+						for (int q = 0; q < 4; ++q) g.add(f->mutable_input()->plane(2 + q) + off, o->in.re + (size_t) (2 + q) * len + off, plen);
+					off += plen;
+				}
+				if (OutputFunc *of = dynamic_cast<OutputFunc *>(f)) {
+					const int lab = batched[uid] ? labels[b] : labels[0];
+					(void) lab;
+					float got = of->loss(labels[b]), want = on.loss(uid, labels[b]);
+					if (batched[uid]) loss.add(&got, &want, 1);
+				}
+			}
+			// each row is its own sample of the data input
+			std::fill(on.at(main_in)->in.dzs_re, on.at(main_in)->in.dzs_re + 2 * n_in, 0.f);
+		}
+		const std::string s = name + " step " + std::to_string(step);
+		report(s + ": node inputs", z.value());
+		report(s + ": node gradients", g.value());
+		report(s + ": losses", loss.value());
+		ErrAcc pg, pw;
+		for (size_t k = 0; k < spec.size(); ++k) {
+			const int uid = (int) k + 1;
+			if (!is_param(uid)) continue;
+			net.fetch(net[uid], 0);
+			bool feeds_batched = false;
+			for (size_t c = 0; c < spec.size(); ++c)
+				for (int p : spec[c].in) feeds_batched |= (p == uid && batched[c + 1]);
+			// a parameter that only feeds a single-row chain saw one backward pass on the device, B on the oracle
+			if (feeds_batched) pg.add(net[uid]->input().dz_star_real_, on.at(uid)->in.dzs_re, 2 * net[uid]->input().length_);
+		}
+		if (pg.r > 0) report(s + ": parameter dz* summed over the rows", pg.value());
+		net.gpuUpdateInputs(0.01f / B);
+		on.update(0.01f, B);
+		net.getInputsFromGpu();
+		for (size_t k = 0; k < spec.size(); ++k) {
+			const int uid = (int) k + 1;
+			if (!is_param(uid)) continue;
+			bool feeds_batched = false;
+			for (size_t c = 0; c < spec.size(); ++c)
+				for (int p : spec[c].in) feeds_batched |= (p == uid && batched[c + 1]);
+			if (feeds_batched) pw.add(net[uid]->input().real_, on.at(uid)->in.re, 2 * net[uid]->input().length_);
+			else std::copy(net[uid]->input().real_, net[uid]->input().real_ + 2 * net[uid]->input().length_, on.at(uid)->in.re);
+		}
+		if (pw.r > 0) report(s + ": parameters after the update", pw.value(), TOL / 5);
+	}
+}
+
+static void test_upstream_nets() {
+	using namespace orc;
+	const int n = 6;  // upstream's segment_len default (tests/gputests.h:27)
+	// testE2E: input -> FourierTrans -> SoftMax -> CRelu -> Residual(with the input) -> Linear -> CGelu -> CrossEntropy
+	run_spec("E2E chain", {{kInput, n, 0, {}}, {kFourier, n, 0, {1}}, {kSoftMax, n, 0, {2}}, {kCrelu, n, 0, {3}}, {kResidual, n, 0, {4, 1}},
+			{kInput, n * n / 2, 0, {}}, {kLinear, n, n * n / 2, {5, 6}}, {kGelu, n / 2, 0, {7}}, {kCrossEntropy, n / 2, 0, {8}}}, 3, 2);
+	// testTwoOutputs: one producer feeds both operands of a Residual
+	run_spec("one producer, two slots", {{kInput, n, 0, {}}, {kResidual, n, 0, {1, 1}}, {kCrossEntropy, n, 0, {2}}}, 3, 2);
+	// testZeroGradient / testInputGradient: a second, disconnected chain with its own input and output
+	run_spec("two disconnected chains", {{kInput, n, 0, {}}, {kGelu, n, 0, {1}}, {kCrossEntropy, n, 0, {2}}, {kInput, n, 0, {}}, {kGelu, n, 0, {4}},
+			{kCrossEntropy, n, 0, {5}}}, 3, 2);
+	// testRelu: two CRelu in a row
+	run_spec("CRelu twice", {{kInput, n, 0, {}}, {kCrelu, n, 0, {1}}, {kCrelu, n, 0, {2}}, {kL2Out, n, 0, {3}}}, 4, 1);
+	// testT_FFTGradient: TriangFourier between Linear layers with a fan-out
+	run_spec("TriangFourier with fan-out", {{kInput, n, 0, {}}, {kTriangFourier, n, 0, {1}}, {kInput, n * n, 0, {}}, {kLinear, n, n * n, {2, 3}},
+			{kResidual, n, 0, {2, 4}}, {kSoftMax, n, 0, {5}}, {kInput, n, 0, {}}, {kHadamard, n, 0, {6, 7}}, {kL2Out, n, 0, {8}}}, 5, 2);
+}
+
 // ------------------------------------------------------------------------------------------------- error behaviour
 template <class E, class F>
 static bool throws(F f) {
@@ -938,6 +1089,7 @@ int main(int argc, char **argv) {
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
 		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12, false);
 		if (what == "pipeline_timing") test_pipeline(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, true);
+		if (what == "upstream_nets" || what == "all") test_upstream_nets();
 		if (what == "errors" || what == "all") test_errors();
 		if (what == "c4")
 			run_c4(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048, argc > 5 ? atoi(argv[5]) : 10,

@@ -67,6 +67,11 @@ def test_host_batch_pipeline_prefetch_and_graph_replay_give_the_same_bits():
     assert "FAIL" not in out and out.count("PASS") >= 11 and "samples_per_sec_prefetch" in out
 
 
+def test_nets_of_the_upstream_gpu_tests():
+    out = _run("upstream_nets")
+    assert "FAIL" not in out and out.count("PASS") >= 25
+
+
 def test_error_behaviour():
     out = _run("errors")
     assert "FAIL" not in out
