@@ -7,7 +7,7 @@
 //   workgroup = 256 threads = 4 wavefronts (one per SIMD) computing a BM x BN block of C;
 //   wavefront = WM x WN sub-block = (WM/32) x (WN/32) MFMA tiles, with a real and an imaginary accumulator
 //   (16 VGPR each) per tile kept in registers for the whole K loop.
-// Data movement
+// Data movement (cgemm_kernel, any shape; the fast path further down moves tiles from global memory straight into LDS)
 //   K is walked in chunks of KC = 16.  Each chunk of the four operand planes is fetched from global memory into
 //   registers (float4, coalesced along the contiguous dimension of the source), then written to LDS in
 //   [k][row] order, whatever the source layout: an MFMA operand fragment (lane l -> row l%32, k = l/32) is
@@ -356,60 +356,22 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 
 // ---------------------------------------------------------------------------------------------------------------
 // Fast path: M % BM == 0, N % BN == 0, K % KC == 0, 128-bit aligned operands.  Same decomposition as cgemm_kernel,
-// with the per-chunk overhead taken out of the vector ALU and out of LDS:
-//   * global addresses are "uniform tile base (advanced with scalar adds) + per-thread 32-bit offset that never
-//     changes", so a chunk costs no address arithmetic in VGPRs and needs no edge masks;
-//   * LDS addresses are "per-thread base + stage toggle (one add per chunk) + immediate";
-//   * every operand goes to LDS with 128-bit writes and no transposition:
-//       - a source contiguous along its rows lands as [k][row] (pitch rows + 4) and is read one float per k pair;
-//       - a source contiguous along k lands as [row][16 k values], the four 16-byte groups of a row XOR-swizzled with
-//         bits 2..3 of the row, and is read back with 128-bit reads: lane (row r, half h) takes k group h for k steps
-//         0..3 and k group h + 2 for k steps 4..7.  Both the write (4 lanes cover one row) and the read (16 consecutive
-//         rows cover all 64 banks) are free of bank conflicts.
+// with the per-chunk overhead taken out of the vector ALU, the registers and the LDS write port:
+//   * operand tiles go from global memory straight into LDS (global_load_lds_dwordx4), 1 KiB per wave-wide
+//     instruction, so a chunk needs no staging registers and no LDS write instructions; global addresses are
+//     "uniform tile base (advanced with scalar adds) + per-lane 32-bit offset that never changes";
+//   * LDS layouts follow from that (a transfer fills consecutive LDS bytes in lane order):
+//       - a source contiguous along its rows lands as [k][row] (pitch = rows) and is read one float per k pair;
+//       - a source contiguous along k lands as [row][16 k values]; the four 16-byte groups of a row are XOR-swizzled
+//         with bits 2..3 of the row (applied to the global address each lane fetches), and the fragments come back with
+//         128-bit reads: lane (row r, half h) takes k group h for k steps 0..3 and k group h + 2 for k steps 4..7;
+//         16 consecutive rows cover all 64 banks.
 //     The k order inside a chunk is therefore permuted: MFMA step s of half h multiplies k = 4h + s (s < 4) or
 //     k = 8 + 4h + (s - 4); the [k][row] operands are addressed with the same map, so the products pair up correctly.
-//   * the LDS writes of the next chunk are spread over the second half of the current chunk's MFMAs and the scheduler
-//     is told to interleave them (one MFMA, then a few VALU / DS instructions) so they issue in the shadow of the
-//     matrix pipe instead of stalling it.
-template <int ROWS, bool MCONTIG>
-struct FastStage {
-	static constexpr int UNITS = ROWS * KC / 4 / NTHREADS;
-	static constexpr int PITCH = MCONTIG ? ROWS + 4 : KC;      // floats per LDS line
-	static constexpr int PLANE = MCONTIG ? KC * PITCH : ROWS * KC;
-	unsigned goff[UNITS];  // byte offset of this thread's float4 inside the operand tile of a chunk
-	int soff[UNITS];       // float offset of its LDS destination inside a plane
-	float4 re[UNITS], im[UNITS];
-
-	__device__ __forceinline__ void init(long ld) {
-#pragma unroll
-		for (int u = 0; u < UNITS; ++u) {
-			const int unit = threadIdx.x + u * NTHREADS;
-			if (MCONTIG) {
-				const int k = unit / (ROWS / 4);
-				const int row = (unit % (ROWS / 4)) * 4;
-				goff[u] = (unsigned) (((long) k * ld + row) * 4);
-				soff[u] = k * PITCH + row;
-			} else {
-				const int row = unit / (KC / 4);
-				const int kq = unit % (KC / 4);
-				goff[u] = (unsigned) (((long) row * ld + kq * 4) * 4);
-				soff[u] = row * KC + ((kq ^ ((row >> 2) & 3)) * 4);
-			}
-		}
-	}
-	// tile_re / tile_im: uniform pointers to element (first row of the block, first k of the chunk)
-	__device__ __forceinline__ void load_unit(int u, const float *tile_re, const float *tile_im) {
-		re[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(tile_re) + goff[u]);
-		im[u] = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(tile_im) + goff[u]);
-	}
-	__device__ __forceinline__ void store_unit(int u, float *sre, float *sim, float im_sign) const {
-		// component-wise on purpose: an aggregate copy of re[u] keeps the array in scratch memory
-		*reinterpret_cast<float4 *>(sre + soff[u]) = make_float4(re[u].x, re[u].y, re[u].z, re[u].w);
-		*reinterpret_cast<float4 *>(sim + soff[u]) =
-				make_float4(im[u].x * im_sign, im[u].y * im_sign, im[u].z * im_sign, im[u].w * im_sign);
-	}
-};
-
+//   * LDS holds two (128 x 128) or three (smaller blocks) stages; the transfers of chunk c + stages - 1 are issued
+//     before the MFMAs of chunk c, one vmcnt wait and one barrier per chunk publish the next stage;
+//   * the scheduler is told to interleave (one MFMA, then a few VALU / DS / memory instructions) so everything else
+//     issues in the shadow of the matrix pipe.
 // Operand fragments of one wavefront: T tiles of 32 rows, both planes.
 //   MCONTIG ([k][row] in LDS): one float per tile, plane and k step, double buffered per step.
 //   otherwise ([row][k] swizzled): one float4 per tile, plane and half chunk (set 0: steps 0..3, set 1: steps 4..7).
@@ -459,15 +421,60 @@ struct Frag {
 	__device__ __forceinline__ float im(int s, int i) const { return MCONTIG ? s_im[s & 1][i] : comp(q_im[s >> 2][i], s & 3); }
 };
 
-// waves_per_eu(2, 4): LDS allows at most four workgroups per compute unit anyway, so the register allocator may use up to
-// 128 VGPRs for the small blocks instead of squeezing them (and spilling global loads to scratch) for an occupancy that
-// cannot materialise.
-template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG>
+// One operand (both planes) of one K chunk, loaded straight into LDS.  A unit is one wave-wide instruction: lane l
+// delivers 16 bytes to LDS float offset (unit * 64 + l) * 4 of the plane, unit = u * 4 + wavefront.
+//   MCONTIG: the plane is [k][ROWS] (pitch ROWS): the unit covers 256 / ROWS lines of k.
+//   otherwise: the plane is [row][KC] with the 16-byte groups of a row XOR-swizzled by bits 2..3 of the row; LDS
+//   position (row, q) receives global group q ^ swizzle(row).
+template <int ROWS, bool MCONTIG>
+struct DlStage {
+	static constexpr int UNITS = ROWS * KC / 256 / 4;
+	static constexpr int PITCH = MCONTIG ? ROWS : KC;
+	static constexpr int PLANE = ROWS * KC;
+	unsigned goff[UNITS];  // byte offset of this lane's 16 bytes inside the operand tile of a chunk
+	int wave;
+
+	__device__ __forceinline__ void init(long ld) {
+		wave = threadIdx.x >> 6;
+		const int lane = threadIdx.x & 63;
+#pragma unroll
+		for (int u = 0; u < UNITS; ++u) {
+			const int pos = ((u * 4 + wave) * 64 + lane) * 4;  // float offset inside the LDS plane
+			if (MCONTIG) {
+				const int k = pos / ROWS, row = pos % ROWS;
+				goff[u] = (unsigned) (((long) k * ld + row) * 4);
+			} else {
+				const int row = pos / KC, q = (pos % KC) / 4;
+				goff[u] = (unsigned) (((long) row * ld + ((q ^ ((row >> 2) & 3)) * 4)) * 4);
+			}
+		}
+	}
+	__device__ __forceinline__ void issue(int u, const float *tile_re, const float *tile_im, float *sre, float *sim) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+		// Written as assembly on purpose: for the builtin the compiler cannot tell which LDS reads the transfer may
+		// alias and puts a vmcnt(0) wait in front of the first fragment read of the current chunk, which exposes the
+		// whole memory latency once per chunk.  The wait that is needed (before the barrier that publishes the stage)
+		// is in the kernel.  m0 = LDS byte address of the KiB this wavefront fills; one wait state before its use.
+		const unsigned dst = (unsigned) ((u * 4 + wave) * 1024);
+		const unsigned lre = __builtin_amdgcn_readfirstlane((unsigned) (size_t) sre + dst);
+		const unsigned lim = __builtin_amdgcn_readfirstlane((unsigned) (size_t) sim + dst);
+		asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(goff[u]), "s"(tile_re), "s"(lre) : "memory", "m0");
+		asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(goff[u]), "s"(tile_im), "s"(lim) : "memory", "m0");
+#endif
+	}
+};
+
+// Signs (conj) are applied to the fragments.  NST stages of LDS: chunk c + NST - 1 is requested while chunk c is
+// multiplied, so with three stages a transfer has two chunks of MFMA time to arrive (the small blocks, whose chunk is
+// shorter than a memory round trip, use three; 128 x 128 has room for two).
+// waves_per_eu(2, 4): LDS allows at most four workgroups per compute unit anyway, so the register allocator need not
+// squeeze the small blocks for an occupancy that cannot materialise.
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int NST>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))) void cgemm_fast_kernel(const CgemmArgs args) {
 	static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per workgroup");
 	constexpr int TM = WM / 32, TN = WN / 32;
-	typedef FastStage<BM, A_MCONTIG> StageA;
-	typedef FastStage<BN, B_NCONTIG> StageB;
+	typedef DlStage<BM, A_MCONTIG> StageA;
+	typedef DlStage<BN, B_NCONTIG> StageB;
 	constexpr int A_PLANE = StageA::PLANE, B_PLANE = StageB::PLANE;
 	constexpr int STAGE_FLOATS = 2 * A_PLANE + 2 * B_PLANE;
 	constexpr int KS = KC / 2;  // k pairs (MFMA k extent = 2) per chunk
@@ -524,7 +531,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	StageB sb;
 	sa.init(args.lda);
 	sb.init(args.ldb);
-	constexpr int UA = StageA::UNITS, UB = StageB::UNITS, NU = UA + UB;
+	constexpr int UA = StageA::UNITS, UB = StageB::UNITS;
 
 	// uniform tile bases of chunk 0 and the per-chunk advance (elements)
 	const long a_tile0 = A_MCONTIG ? (long) m0 : (long) m0 * args.lda;
@@ -534,25 +541,25 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	int c_lo, c_hi;
 	chunk_range<BN>(args, n0, c_lo, c_hi);
 
-	auto load_unit = [&](int idx, int chunk) {
-		// indices are clamped so that the branch not taken still addresses inside the register arrays (an out-of-range
-		// constant index would push them to scratch memory)
-		if (idx < UA)
-			sa.load_unit(idx < UA ? idx : 0, pb.a_re + a_tile0 + chunk * a_step, pb.a_im + a_tile0 + chunk * a_step);
-		else
-			sb.load_unit(idx >= UA ? idx - UA : 0, pb.b_re + b_tile0 + chunk * b_step, pb.b_im + b_tile0 + chunk * b_step);
+	// all units of one chunk of both operands into the stage at `stage`
+	auto issue_chunk = [&](int chunk, float *stage) {
+#pragma unroll
+		for (int u = 0; u < UA; ++u)
+			sa.issue(u, pb.a_re + a_tile0 + chunk * a_step, pb.a_im + a_tile0 + chunk * a_step, stage, stage + A_PLANE);
+#pragma unroll
+		for (int u = 0; u < UB; ++u)
+			sb.issue(u, pb.b_re + b_tile0 + chunk * b_step, pb.b_im + b_tile0 + chunk * b_step, stage + 2 * A_PLANE,
+					stage + 2 * A_PLANE + B_PLANE);
 	};
-	auto store_unit = [&](int idx, float *stage) {
-		if (idx < UA)
-			sa.store_unit(idx < UA ? idx : 0, stage, stage + A_PLANE, pb.a_im_sign);
-		else
-			sb.store_unit(idx >= UA ? idx - UA : 0, stage + 2 * A_PLANE, stage + 2 * A_PLANE + B_PLANE, pb.b_im_sign);
-	};
+	const unsigned a_neg = pb.a_im_sign < 0.f ? 0x80000000u : 0u, b_neg = pb.b_im_sign < 0.f ? 0x80000000u : 0u;
 
+	constexpr int LOADS_PER_CHUNK = 2 * (UA + UB);  // transfers one wavefront issues per chunk
+	static_assert(NST == 2 || NST == 3, "two or three stages");
+	static_assert(LOADS_PER_CHUNK < 16, "fits the low bits of the vmcnt field");
 #pragma unroll
-	for (int u = 0; u < NU; ++u) load_unit(u, c_lo);
-#pragma unroll
-	for (int u = 0; u < NU; ++u) store_unit(u, smem);
+	for (int d = 0; d < NST - 1; ++d)
+		if (c_lo + d < c_hi) issue_chunk(c_lo + d, smem + d * STAGE_FLOATS);
+	__builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tiles have landed in LDS
 	__syncthreads();
 
 	Frag<TM, A_MCONTIG, StageA::PITCH, A_PLANE> fa;
@@ -564,12 +571,13 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	fa.fetch_set(0, 0);
 	fb.fetch_set(0, 0);
 
+	int cur = 0;  // stage that holds chunk c
 	for (int c = c_lo; c < c_hi; ++c) {
-		const int CUR = ((c - c_lo) & 1) * STAGE_FLOATS, NXT = STAGE_FLOATS - CUR;
-		const bool more = (c + 1 < c_hi);
-		const int next_chunk = more ? c + 1 : c_lo;  // the last chunk re-reads the first one (in bounds, never used)
-#pragma unroll
-		for (int u = 0; u < NU; ++u) load_unit(u, next_chunk);
+		const int nxt = cur + 1 == NST ? 0 : cur + 1, far = cur == 0 ? NST - 1 : cur - 1;
+		const int CUR = cur * STAGE_FLOATS, NXT = nxt * STAGE_FLOATS;
+		const bool ahead = (c + NST - 1 < c_hi);
+		if (ahead) issue_chunk(c + NST - 1, smem + far * STAGE_FLOATS);
+		cur = nxt;
 #pragma unroll
 		for (int ks = 0; ks < KS; ++ks) {
 			if (ks + 1 < KS) {
@@ -580,14 +588,13 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				fa.fetch_set(CUR, 1);
 				fb.fetch_set(CUR, 1);
 			}
-			// the LDS writes of the next chunk ride on the MFMAs of the second half of this chunk
-			constexpr int SF = KS / 2;  // first k pair that carries LDS writes of the next chunk
-			if (ks >= SF) {
-#pragma unroll
-				for (int u = 0; u < NU; ++u)
-					if (SF + (u * (KS - SF)) / NU == ks) store_unit(u, smem + NXT);
-			}
 			if (ks == KS - 1) {
+				// this wavefront's part of the next chunk is in LDS (transfers complete in order: with three stages the
+				// ones just issued for the chunk after it may still be in flight)
+				if (NST == 3 && ahead)
+					__builtin_amdgcn_s_waitcnt(0x0F70 | LOADS_PER_CHUNK);
+				else
+					__builtin_amdgcn_s_waitcnt(0x0F70);
 				__syncthreads();
 				fa.fetch_step(NXT, 0);
 				fb.fetch_step(NXT, 0);
@@ -598,13 +605,13 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 #pragma unroll
 			for (int i = 0; i < TM; ++i) {
 				are[i] = fa.re(ks, i);
-				aim[i] = fa.im(ks, i);
+				aim[i] = __uint_as_float(__float_as_uint(fa.im(ks, i)) ^ a_neg);
 				anim[i] = -aim[i];
 			}
 #pragma unroll
 			for (int j = 0; j < TN; ++j) {
 				bre[j] = fb.re(ks, j);
-				bim[j] = fb.im(ks, j);
+				bim[j] = __uint_as_float(__float_as_uint(fb.im(ks, j)) ^ b_neg);
 			}
 #pragma unroll
 			for (int i = 0; i < TM; ++i)
@@ -708,14 +715,16 @@ int launch(const CgemmArgs &proto, int nprob, int batch) {
 	};
 	if constexpr (VEC == 4) {
 		if (args.M % BM == 0 && args.N % BN == 0 && args.K % KC == 0) {
-			auto fast = cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG>;
+			constexpr int NST = (BM == 128 && BN == 128) ? 2 : 3;
+			constexpr size_t fast_smem = (size_t) NST * 2 * KC * (BM + BN) * sizeof(float);
 			static bool fast_attr_set = false;
 			if (!fast_attr_set) {
-				CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(fast), hipFuncAttributeMaxDynamicSharedMemorySize,
-						(int) smem));
+				CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST>),
+						hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem));
 				fast_attr_set = true;
 			}
-			hipLaunchKernelGGL(fast, grid, dim3(NTHREADS), smem, cnet::rt().stream, args);
+			hipLaunchKernelGGL((cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST>), grid, dim3(NTHREADS), fast_smem,
+					cnet::rt().stream, args);
 			CNET_LAUNCH_CHECK();
 			return finish();
 		}
