@@ -112,8 +112,8 @@ def kernel_suite(steps):
     def grad(r, c):
         return ops.Grad.from_host([rs.randn(r, c).astype(np.float32) for _ in range(4)])
 
-    def timed(fn):
-        for _ in range(3):
+    def timed(fn, warm=3):
+        for _ in range(warm):
             fn()
         capi.sync()
         a, b = ev.event(), ev.event()
@@ -133,7 +133,7 @@ def kernel_suite(steps):
             "bytes_per_complex_element": bytes_per_elem}})
 
     def mfma(name, shape, flops, fn):
-        ms = timed(fn)
+        ms = timed(fn, warm=20)  # millisecond launches: the clocks settle within a few of them
         tf = flops / ms / 1e9
         lines.append({"kernel": name, "shape": shape, "ms": round(ms, 4), "roofline": {
             "bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
