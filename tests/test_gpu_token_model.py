@@ -89,3 +89,57 @@ def test_token_model_reduced(gpu, port):
     chk(model.d_m, d_m, "d seq-DFT output")
     chk(model.d_x, d_x, "d embedding rows")
     assert rel_c((model.d_table_re.host(), model.d_table_im.host()), (dt_r, dt_i)) < TOL
+
+
+def test_token_model_full_size_properties(gpu, port):
+    """The fifth configuration at its full size (16 x 512 tokens, vocab 32768, dim 1024, hidden 4096), checked through
+    what does not need the CPU path on all of it: the oracle on a subsample of logit rows, bit-identical repetition,
+    and a directional finite difference of the total loss along the gradient of the shared gate weights."""
+    B, S, D, H, V = 16, 512, 1024, 4096, 32768
+    rs = np.random.RandomState(5)
+
+    def nrm(shape, sig):
+        return (rs.standard_normal(shape) * sig).astype(np.float32)
+
+    P = {"table": nrm((2, V, D), 1.0), "gate": nrm((2, D), 0.05), "w1": nrm((2, H, D), D ** -0.5),
+         "w2": nrm((2, D, H), H ** -0.5), "w3": nrm((2, V, D), D ** -0.5)}
+    ids = rs.randint(0, V, (B, S)).astype(np.int32)
+    model = TokenModel(B, S, D, H, V, P).set_tokens(ids)
+    model.forward()
+    model.backward()
+    loss0 = model.loss.download().copy()
+    gate_grad = [p.copy() for p in model.d_gate.host()]
+    assert np.all(np.isfinite(loss0)) and abs(loss0.mean() - np.log(V)) < 1.5
+
+    # rows of the logits layer and of the loss against the oracle
+    rows = [0, 511, 4097, 8191]
+    o = model.o.host()
+    labels = np.roll(ids, -1, axis=1).reshape(-1)[rows].astype(np.int32)
+    lr_, li_ = port.linear_fwd(np.ascontiguousarray(o[0][rows]), np.ascontiguousarray(o[1][rows]), P["w3"][0], P["w3"][1])
+    _, _, _, loss_o, pred_o = port.crossent_fwd(lr_, li_, labels)
+    lg = model.logits.host()
+    assert rel_c((lg[0][rows], lg[1][rows]), (lr_, li_)) < TOL / 5
+    assert np.allclose(loss0[rows], loss_o, rtol=2e-4, atol=2e-5)
+    assert np.array_equal(model.argmax.download()[rows], pred_o)
+    del lg, o
+
+    # same bits on repetition
+    model.forward()
+    model.backward()
+    assert np.array_equal(model.loss.download(), loss0)
+    for a, b in zip(model.d_gate.host(), gate_grad):
+        assert np.array_equal(a, b)
+
+    # d(total loss) along the normalised dz* of the gate: 2 |dz*| (d/dRe = 2 Re dz*, d/dIm = 2 Im dz*)
+    gs = gate_grad[2].astype(np.float64) + 1j * gate_grad[3].astype(np.float64)
+    norm = np.linalg.norm(gs)
+    direction = gs / norm
+    eps = 5e-4  # the loss is strongly curved along this direction: 2e-3 already loses 6 %, 2e-2 loses 40 %
+    totals = []
+    for sign in (+1, -1):
+        w = (P["gate"][0] + 1j * P["gate"][1]) + sign * eps * direction.reshape(-1)
+        model.gate = ops.CMat.from_host(np.ascontiguousarray(w.real, np.float32), np.ascontiguousarray(w.imag, np.float32))
+        model.forward()
+        totals.append(model.loss.download().astype(np.float64).sum())
+    numeric = (totals[0] - totals[1]) / (2 * eps)
+    assert abs(numeric - 2 * norm) / (2 * norm) < 4e-2, (numeric, 2 * norm)
