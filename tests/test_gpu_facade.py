@@ -80,3 +80,11 @@ def test_error_behaviour():
 def test_config4_residual_stack_reduced_runs_and_learns():
     out = _run("c4", "512", "4", "256", "5", "0.001")
     assert "samples_per_sec" in out and "FAIL" not in out
+
+
+def test_config4_residual_stack_full_size_runs_and_learns():
+    """8 x (Linear 2048 -> 2048, CGelu, Residual), batch 2048, L2Out: three SGD steps at the full size.  With the
+    configured rate 0.01 this net overflows after one step in exact arithmetic as well (its initial loss is 8e6 per
+    sample), so the run uses 1e-6; the driver fails unless the loss falls."""
+    out = _run("c4", "2048", "8", "2048", "3", "0.000001", timeout=300)
+    assert "samples_per_sec" in out and "FAIL" not in out
