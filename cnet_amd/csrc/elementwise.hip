@@ -492,6 +492,48 @@ __global__ __launch_bounds__(TPB) void adam_kernel(float *__restrict__ zr, float
 	}
 }
 
+// Several parameter tensors in one launch (a net has many small ones; a launch per tensor costs more than the update).
+// blockIdx.y selects the tensor, blocks past its end leave at once.  Same arithmetic as sgd_kernel.
+constexpr int SGD_MULTI_MAX = 8;
+struct SgdMulti {
+	float *z_re[SGD_MULTI_MAX], *z_im[SGD_MULTI_MAX], *d_re[SGD_MULTI_MAX], *d_im[SGD_MULTI_MAX];
+	long n[SGD_MULTI_MAX];
+	int vec[SGD_MULTI_MAX];  // tensor can take the 128-bit path
+};
+__global__ __launch_bounds__(TPB) void sgd_multi_kernel(SgdMulti t, float lr, int zero_grad) {
+	const int k = blockIdx.y;
+	const long n = t.n[k];
+	float *zr = t.z_re[k], *zi = t.z_im[k], *dr = t.d_re[k], *di = t.d_im[k];
+	if (t.vec[k]) {
+		const long i = ((long) blockIdx.x * TPB + threadIdx.x) * 4;
+		if (i >= n) return;
+		float a[4], b[4], c[4], d[4], z[4] = {0.f, 0.f, 0.f, 0.f};
+		ldv<4, false>(a, zr + i);
+		ldv<4, false>(b, zi + i);
+		ldv<4, false>(c, dr + i);
+		ldv<4, false>(d, di + i);
+#pragma unroll
+		for (int q = 0; q < 4; ++q) {
+			a[q] -= lr * c[q];
+			b[q] -= lr * d[q];
+		}
+		stv<4, false>(zr + i, a);
+		stv<4, false>(zi + i, b);
+		if (zero_grad) {
+			stv<4, false>(dr + i, z);
+			stv<4, false>(di + i, z);
+		}
+	} else {
+		// scalar path: four consecutive elements per thread keep the grid shape of the vector path
+		const long i0 = ((long) blockIdx.x * TPB + threadIdx.x) * 4;
+		for (long i = i0; i < i0 + 4 && i < n; ++i) {
+			zr[i] -= lr * dr[i];
+			zi[i] -= lr * di[i];
+			if (zero_grad) dr[i] = di[i] = 0.f;
+		}
+	}
+}
+
 __global__ __launch_bounds__(TPB) void zero_kernel(uint4 *__restrict__ p16, long n16, unsigned char *__restrict__ tail, int ntail) {
 	const long i = (long) blockIdx.x * TPB + threadIdx.x;
 	if (i < n16) p16[i] = make_uint4(0, 0, 0, 0);
@@ -792,6 +834,35 @@ int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int6
 	else
 		hipLaunchKernelGGL((sgd_kernel<1, false>), dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
 	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_sgd_update_multi(int count, float *const *z_re, float *const *z_im, float *const *dzs_re, float *const *dzs_im,
+		const int64_t *n, float lr, int zero_grad) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(count >= 0);
+	if (!count) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && dzs_re && dzs_im && n);
+	for (int k = 0; k < count; ++k) CNET_CHECK_ARG(n[k] >= 0 && (n[k] == 0 || (z_re[k] && z_im[k] && dzs_re[k] && dzs_im[k])));
+	for (int first = 0; first < count; first += SGD_MULTI_MAX) {
+		SgdMulti t;
+		int used = 0;
+		long longest = 0;
+		for (int k = first; k < count && used < SGD_MULTI_MAX; ++k) {
+			if (!n[k]) continue;
+			t.z_re[used] = z_re[k];
+			t.z_im[used] = z_im[k];
+			t.d_re[used] = dzs_re[k];
+			t.d_im[used] = dzs_im[k];
+			t.n[used] = (long) n[k];
+			t.vec[used] = n[k] % 4 == 0 && all_aligned({z_re[k], z_im[k], dzs_re[k], dzs_im[k]});
+			longest = std::max(longest, (long) n[k]);
+			++used;
+		}
+		if (!used) continue;
+		hipLaunchKernelGGL(sgd_multi_kernel, dim3(nblocks((longest + 3) / 4), used), dim3(TPB), 0, rt().stream, t, lr, zero_grad);
+		CNET_LAUNCH_CHECK();
+	}
 	return CNET_OK;
 }
 

@@ -598,6 +598,7 @@ class CNet {
 	};
 	StepGraphs graphs_[2];
 	bool use_graphs_ = false;
+	bool input_dz_dirty_ = false;  // the dz planes of the input functions hold a first moment
 	bool warmed_[3] = {false, false, false};  // phase has run once since useGraphs(true)
 
 	void dropGraphs() {
@@ -788,6 +789,7 @@ public:
 		d_labels_ = NULL;
 		dropGraphs();
 		use_graphs_ = false;
+		input_dz_dirty_ = false;
 		for (auto &st : stage_) {
 			if (st.host_labels) cnet_host_free(st.host_labels);
 			st = Stage();
@@ -1276,15 +1278,31 @@ public:
 			g.upd = NULL;
 		}
 		g.upd_lr = l_rate;
+		if (input_dz_dirty_)  // this update also clears the first moment: not what a recording made without it does
+			for (auto &sg : graphs_)
+				if (sg.upd) {
+					ck(cnet_graph_destroy(sg.upd), "cnet_graph_destroy");
+					sg.upd = NULL;
+				}
 		runPhase(2, g.upd, [&] {
+			// every input function in one launch; their dz planes only hold something after an Adam-style step (its
+			// first moment), so they are cleared only then
+			std::vector<float *> zr, zi, dr, di;
+			std::vector<int64_t> len;
 			for (auto f : inputs_) {
 				CFunc::Slot &s = f->slots_[0];
 				const size_t n = (size_t) s.rows * s.len;
-				float *z = s.z;
-				ck(cnet_sgd_update(z, z + n, s.g(2), s.g(3), (int64_t) n, l_rate, 1), "cnet_sgd_update");
-				ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
+				zr.push_back(s.z);
+				zi.push_back(s.z + n);
+				dr.push_back(s.g(2));
+				di.push_back(s.g(3));
+				len.push_back((int64_t) n);
+				if (input_dz_dirty_) ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
 			}
+			ck(cnet_sgd_update_multi((int) zr.size(), zr.data(), zi.data(), dr.data(), di.data(), len.data(), l_rate, 1),
+					"cnet_sgd_update_multi");
 		});
+		input_dz_dirty_ = false;
 	}
 	// Replay the kernels of GpuForward / gpuBackward / gpuUpdateInputs from recorded graphs instead of launching them
 	// one by one (a step at small batch sizes is bound by launch overhead).  Each phase runs once as usual after this
@@ -1306,6 +1324,7 @@ public:
 			float *z = s.z;
 			ck(cnet_adam_update(z, z + n, s.g(0), s.g(1), s.g(2), s.g(3), (int64_t) n, l_rate, beta, t, 1), "cnet_adam_update");
 		}
+		input_dz_dirty_ = true;
 	}
 	float getLoss(OutputFunc *outp, Batch *batch) {
 		requireAllocated("getLoss");

@@ -243,6 +243,10 @@ int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols
 /* z -= lr * dzs ; then dzs = 0 when zero_grad != 0   (impl/cfunc.h:147-152 + impl/cnet.h:413-421) */
 int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int64_t n, float lr, int zero_grad);
 
+/* The same step for `count` tensors in one launch (host arrays of device pointers and lengths): a net with many small
+ * parameter tensors is otherwise bound by launches. */
+int cnet_sgd_update_multi(int count, float *const *z_re, float *const *z_im, float *const *dzs_re, float *const *dzs_im,
+                          const int64_t *n, float lr, int zero_grad);
 /* Adam-style step: replaces gpu_update_adam_input (gpu/kernels.cpp:494-525), CPU twin impl/cfunc.h:273-287 +
  * impl/cnet.h:423-431.  m = beta m + (1 - beta) dzs ; z -= lr m / (1 - beta^(t+1)) ; then dzs = 0 when zero_grad != 0.
  * m_re / m_im are the first-moment planes (upstream keeps them in the node's dz planes, impl/cfunc.h:341-349). */

@@ -118,3 +118,30 @@ def test_sgd_update_zero_copy_add(gpu, port):
     assert rel(first, m.astype(np.float64).sum(0, keepdims=True)) < 1e-6
     ops.batch_sum(ops.Plane.from_host(m), out)
     assert np.array_equal(out.host(), first)
+
+
+def test_sgd_update_of_several_tensors_in_one_launch(gpu, port):
+    """cnet_sgd_update_multi against the single-tensor entry point: same bits, odd lengths and empty tensors included."""
+    import ctypes as C
+    sizes = [7840, 784, 1, 0, 100003, 64, 4096, 12, 999, 50000, 8]  # more than one launch's worth of tensors
+    zs, ds, ref = [], [], []
+    for k, n in enumerate(sizes):
+        m = max(n, 1)
+        zr, zi, dr, di = [seeded(port, 10 * k + j, (1, m)) for j in range(4)]
+        z = ops.CMat.from_host(zr, zi)
+        d = (ops.Plane.from_host(dr), ops.Plane.from_host(di))
+        z2 = ops.CMat.from_host(zr, zi)
+        d2 = (ops.Plane.from_host(dr), ops.Plane.from_host(di))
+        if n:
+            capi.call("cnet_sgd_update", z2.re.ptr, z2.im.ptr, d2[0].ptr, d2[1].ptr, n, 0.03, 1)
+        zs.append(z); ds.append(d); ref.append((z2, d2))
+    arr = lambda ptrs: (C.c_void_p * len(ptrs))(*ptrs)
+    lens = (C.c_int64 * len(sizes))(*sizes)
+    capi.call("cnet_sgd_update_multi", len(sizes), arr([z.re.ptr for z in zs]), arr([z.im.ptr for z in zs]),
+              arr([d[0].ptr for d in ds]), arr([d[1].ptr for d in ds]), lens, 0.03, 1)
+    for n, z, d, (z2, d2) in zip(sizes, zs, ds, ref):
+        a, b = z.host(), z2.host()
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1]), n
+        assert np.array_equal(d[0].host(), d2[0].host()) and np.array_equal(d[1].host(), d2[1].host()), n
+        if n:
+            assert not d[0].host()[0, :n].any()
