@@ -25,7 +25,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
          # packed-fp32 VALU forms are kept out of every kernel
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-DCNET_SCHED_RECIPE=" + os.environ.get("CNET_SCHED_RECIPE", "1"),
-         "-Wno-unused-result", "-Wno-unused-value", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+         "-Wno-unused-result", "-Wno-inline-asm", "-Wno-unused-value", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
 
 
 def _stale(src, obj):
