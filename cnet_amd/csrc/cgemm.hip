@@ -355,7 +355,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 
 
 // ---------------------------------------------------------------------------------------------------------------
-// Fast path: M % BM == 0, N % BN == 0, K % KC == 0, 128-bit aligned operands.  Same decomposition as cgemm_kernel,
+// Fast path: K % KC == 0, 128-bit aligned operands with shapes that are multiples of 4 (any number of blocks).  Same decomposition as cgemm_kernel,
 // with the per-chunk overhead taken out of the vector ALU, the registers and the LDS write port:
 //   * operand tiles go from global memory straight into LDS (global_load_lds_dwordx4), 1 KiB per wave-wide
 //     instruction, so a chunk needs no staging registers and no LDS write instructions; global addresses are
@@ -434,18 +434,21 @@ struct DlStage {
 	unsigned goff[UNITS];  // byte offset of this lane's 16 bytes inside the operand tile of a chunk
 	int wave;
 
-	__device__ __forceinline__ void init(long ld) {
+	// rows_valid: rows of the operand that exist from the first row of this block on (>= ROWS inside the matrix; a
+	// multiple of 4 when MCONTIG).  Rows past the end are fetched from the last valid ones instead: what they produce
+	// lies outside C and is never stored.
+	__device__ __forceinline__ void init(long ld, int rows_valid) {
 		wave = threadIdx.x >> 6;
 		const int lane = threadIdx.x & 63;
 #pragma unroll
 		for (int u = 0; u < UNITS; ++u) {
 			const int pos = ((u * 4 + wave) * 64 + lane) * 4;  // float offset inside the LDS plane
 			if (MCONTIG) {
-				const int k = pos / ROWS, row = pos % ROWS;
+				const int k = pos / ROWS, row = min(pos % ROWS, rows_valid - 4);
 				goff[u] = (unsigned) (((long) k * ld + row) * 4);
 			} else {
 				const int row = pos / KC, q = (pos % KC) / 4;
-				goff[u] = (unsigned) (((long) row * ld + ((q ^ ((row >> 2) & 3)) * 4)) * 4);
+				goff[u] = (unsigned) (((long) min(row, rows_valid - 1) * ld + ((q ^ ((row >> 2) & 3)) * 4)) * 4);
 			}
 		}
 	}
@@ -529,8 +532,8 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 
 	StageA sa;
 	StageB sb;
-	sa.init(args.lda);
-	sb.init(args.ldb);
+	sa.init(args.lda, args.M - m0);
+	sb.init(args.ldb, args.N - n0);
 	constexpr int UA = StageA::UNITS, UB = StageB::UNITS;
 
 	// uniform tile bases of chunk 0 and the per-chunk advance (elements)
@@ -647,17 +650,20 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 #pragma unroll
 		for (int j = 0; j < TN; ++j) {
 			const int col = n0 + wn0 + j * 32 + r;
+			if (col >= args.N) continue;  // blocks on the right and bottom edge of C are partly outside
 #pragma unroll
 			for (int e = 0; e < 16; ++e) {
 				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-				const long off = (long) row * ldc + col;
-				float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
-				if (accumulate) {
-					vr += pb.c_re[off];
-					vi += pb.c_im[off];
+				if (row < args.M) {
+					const long off = (long) row * ldc + col;
+					float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
+					if (accumulate) {
+						vr += pb.c_re[off];
+						vi += pb.c_im[off];
+					}
+					pb.c_re[off] = vr;
+					pb.c_im[off] = vi;
 				}
-				pb.c_re[off] = vr;
-				pb.c_im[off] = vi;
 			}
 		}
 	}  // pass
@@ -714,7 +720,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch) {
 		return CNET_OK;
 	};
 	if constexpr (VEC == 4) {
-		if (args.M % BM == 0 && args.N % BN == 0 && args.K % KC == 0) {
+		if (args.K % KC == 0) {  // any M and N: edge blocks re-read the last valid rows and store only what is inside C
 			constexpr int NST = (BM == 128 && BN == 128) ? 2 : 3;
 			constexpr size_t fast_smem = (size_t) NST * 2 * KC * (BM + BN) * sizeof(float);
 			static bool fast_attr_set = false;
@@ -762,14 +768,32 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 		if (forced == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 		if (forced == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 		if (forced == 3) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-		// The largest block that still gives every compute unit TWO workgroups (two wavefronts per SIMD: one issues
-		// MFMAs while the other waits at its barrier or moves data); failing that, one workgroup per compute unit.
-		for (long want = 2 * cus; want >= cus; want -= cus) {
-			if (blocks(128, 128) >= want) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-			if (blocks(64, 128) >= want) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-			if (blocks(128, 64) >= want) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-			if (blocks(64, 64) >= want) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+		// Expected matrix-pipe efficiency of each block shape for this problem.  The busiest compute unit works through
+		// ceil(blocks / units) blocks, so the launch costs that many block-times on every unit, whether or not all units have
+		// that many and whether or not a block on the edge of C is full: efficiency = real elements of C / elements paid for
+		// x the efficiency measured for the shape on full blocks with at least two workgroups per unit (two wavefronts per
+		// SIMD: one issues MFMAs while the other waits at its barrier), less a penalty where a unit gets a single block.
+		struct Shape {
+			int bm, bn;
+			double eff;
+		};
+		static const Shape shapes[4] = {{128, 128, 0.885}, {64, 128, 0.865}, {128, 64, 0.860}, {64, 64, 0.843}};
+		int best = 3;
+		double best_score = -1.0;
+		for (int k = 0; k < 4; ++k) {
+			const long nb = blocks(shapes[k].bm, shapes[k].bn);
+			const long per_unit = (nb + cus - 1) / cus;
+			const double paid = (double) per_unit * cus * shapes[k].bm * shapes[k].bn;
+			const double real = (double) nb / ((double) ((a.M + shapes[k].bm - 1) / shapes[k].bm) * ((a.N + shapes[k].bn - 1) / shapes[k].bn)) * a.M * a.N;
+			const double score = shapes[k].eff * real / paid * (per_unit >= 2 ? 1.0 : 0.9);
+			if (score > best_score) {
+				best_score = score;
+				best = k;
+			}
 		}
+		if (best == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+		if (best == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+		if (best == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 	}
 }
