@@ -88,13 +88,12 @@ def test_cgemm_all_layouts(gpu, port):
                 assert err < 1e-5, (a_km, b_km, cj, err)
 
 
-@pytest.mark.parametrize("M,N,K", [(8, 24, 1000), (64, 64, 4096), (40, 100, 333), (64, 784, 784), (3, 5, 2049)])
-def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
-    """Few blocks of C against a long K: the launch is cut along K and the partial blocks are added in a fixed order.
-    All four layouts, conj(B), accumulation into a window of a wider buffer, and run-to-run identical bits."""
+def _check_all_layouts(port, M, N, K):
+    """All four layouts, conj(B), accumulation into a window of a wider and taller buffer whose other elements must keep
+    their bits, and run-to-run identical results; the expected product is numpy's in complex128."""
     A = seeded(port, 1, (M, K)) + 1j * seeded(port, 2, (M, K))
     Bm = seeded(port, 3, (K, N)) + 1j * seeded(port, 4, (K, N))
-    base = seeded(port, 5, (M, N + 9))
+    base = seeded(port, 5, (M + 2, N + 9))
     for a_km in (0, 1):
         for b_km in (0, 1):
             a_h = A.T if a_km else A
@@ -114,10 +113,24 @@ def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
             wide = ops.CMat(ops.Plane.from_host(base), ops.Plane.from_host(base))
             ops.cgemm(a, b, wide.sub(4, N), M, N, K, a_km, b_km, cj, accumulate=1)
             hr, hi = wide.re.owner.download(), wide.im.owner.download()
-            got = (hr[:, 4:4 + N] - base[:, 4:4 + N]) + 1j * (hi[:, 4:4 + N] - base[:, 4:4 + N])
+            got = (hr[:M, 4:4 + N] - base[:M, 4:4 + N]) + 1j * (hi[:M, 4:4 + N] - base[:M, 4:4 + N])
             assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-5
-            keep = np.ones(N + 9, bool); keep[4:4 + N] = False
-            assert np.array_equal(hr[:, keep], base[:, keep]) and np.array_equal(hi[:, keep], base[:, keep])
+            hr[:M, 4:4 + N] = hi[:M, 4:4 + N] = base[:M, 4:4 + N]  # what is left is the frame around the window
+            assert np.array_equal(hr, base) and np.array_equal(hi, base)
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 24, 1000), (64, 64, 4096), (40, 100, 333), (64, 784, 784), (3, 5, 2049)])
+def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
+    """Few blocks of C against a long K: the launch is cut along K and the partial blocks are added in a fixed order."""
+    _check_all_layouts(port, M, N, K)
+
+
+@pytest.mark.parametrize("M,N,K", [(4, 4, 16), (132, 200, 64), (260, 68, 48), (700, 388, 32), (1028, 516, 80), (68, 1300, 160),
+                                   (4100, 1028, 16), (61, 67, 64)])
+def test_cgemm_blocks_on_the_edge_of_c(gpu, port, M, N, K):
+    """K a multiple of 16 with M and N that are not multiples of any block shape: blocks that hang over the edge of C
+    read the last valid rows again and must store nothing outside C."""
+    _check_all_layouts(port, M, N, K)
 
 
 def test_cgemm_batched_short_grid(gpu, port):
