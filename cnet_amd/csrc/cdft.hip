@@ -67,8 +67,8 @@ static int get_plan(int n, Twiddle *out, bool create) {
 	if (t.ld != n) CNET_HIP(hipMemsetAsync(t.re, 0, 2 * plane * sizeof(float), rt().stream));
 	const long total = (long) n * n;
 	hipLaunchKernelGGL(twiddle_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, rt().stream, t.re, t.im, n, t.ld, 0);
+	g_twiddles[n] = t;  // owned by the table from here on, whatever the launch reports
 	CNET_LAUNCH_CHECK();
-	g_twiddles[n] = t;
 	*out = t;
 	return CNET_OK;
 }
@@ -149,7 +149,7 @@ int cnet_cdft_set_forward_matrix(int n, const float *host_f_re, const float *hos
 int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy, int B, int n,
 		int accumulate) {
 	CNET_REQUIRE_INIT();
-	CNET_CHECK_ARG(B >= 0 && n > 0);
+	CNET_CHECK_ARG(B >= 0 && n > 0 && n <= 46340);
 	if (B == 0) return CNET_OK;
 	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= n && ldy >= n);
 	Twiddle t;
@@ -165,7 +165,7 @@ int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re
 int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
 		float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int B, int n, int accumulate) {
 	CNET_REQUIRE_INIT();
-	CNET_CHECK_ARG(B >= 0 && n > 0);
+	CNET_CHECK_ARG(B >= 0 && n > 0 && n <= 46340);
 	if (B == 0) return CNET_OK;
 	CNET_CHECK_ARG(g_dz_re && g_dz_im && g_dzs_re && g_dzs_im && dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
 	CNET_CHECK_ARG(ldg >= n && lddx >= n);

@@ -7,16 +7,18 @@ namespace {
 
 constexpr int TPB = 256;
 
-// y[row][slot*dim + d] = table[token][d], zeros for token < 0   (impl/embed.h:109-131 upstream)
+// y[row][slot*dim + d] = table[token][d], zeros for token < 0   (impl/embed.h:109-131 upstream).  An id >= vocab, which
+// upstream rejects with an assert on the host, is treated as padding here: a wrong id must not become a wild access.
 template <int V>
 __global__ __launch_bounds__(TPB) void embedding_fwd_kernel(const float *__restrict__ tr, const float *__restrict__ ti, int dim,
-		const int *__restrict__ tokens, float *__restrict__ yr, float *__restrict__ yi, long ldy, long positions, int slots) {
+		const int *__restrict__ tokens, float *__restrict__ yr, float *__restrict__ yi, long ldy, long positions, int slots, int vocab) {
 	const long dv = dim / V;
 	const long idx = (long) blockIdx.x * TPB + threadIdx.x;
 	if (idx >= positions * dv) return;
 	const long pos = idx / dv;
 	const int d = (int) (idx - pos * dv) * V;
-	const int tok = tokens[pos];
+	int tok = tokens[pos];
+	if (tok >= vocab) tok = -1;
 	const long row = pos / slots, slot = pos - row * slots;
 	const long dst = row * ldy + slot * dim + d;
 	if (V == 4) {
@@ -41,11 +43,11 @@ __global__ __launch_bounds__(TPB) void iota_kernel(int *__restrict__ p, long n) 
 // keys/pos: token ids sorted ascending (stable), pos = original (row, slot) position.  One workgroup per sorted
 // index; only the head of a run of equal tokens works: it adds the run's dzs rows in position order.
 __global__ __launch_bounds__(TPB) void embedding_bwd_kernel(const int *__restrict__ keys, const int *__restrict__ pos, long n,
-		const float *__restrict__ gr, const float *__restrict__ gi, long ldg, int slots, int dim, float *__restrict__ dr,
+		const float *__restrict__ gr, const float *__restrict__ gi, long ldg, int slots, int dim, int vocab, float *__restrict__ dr,
 		float *__restrict__ di) {
 	const long i = blockIdx.x;
 	const int tok = keys[i];
-	if (tok < 0) return;
+	if (tok < 0 || tok >= vocab) return;
 	if (i > 0 && keys[i - 1] == tok) return;
 	for (int d = threadIdx.x; d < dim; d += TPB) {
 		float ar = dr[(long) tok * dim + d], ai = di[(long) tok * dim + d];
@@ -80,10 +82,10 @@ int cnet_embedding_fwd(const float *table_re, const float *table_im, int dim, in
 	dim3 grid((unsigned) ((work + TPB - 1) / TPB));
 	if (vec)
 		hipLaunchKernelGGL(embedding_fwd_kernel<4>, grid, dim3(TPB), 0, rt().stream, table_re, table_im, dim, tokens, y_re, y_im, (long) ldy,
-				positions, slots);
+				positions, slots, vocab);
 	else
 		hipLaunchKernelGGL(embedding_fwd_kernel<1>, grid, dim3(TPB), 0, rt().stream, table_re, table_im, dim, tokens, y_re, y_im, (long) ldy,
-				positions, slots);
+				positions, slots, vocab);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -116,7 +118,7 @@ int cnet_embedding_bwd(const int32_t *tokens, const float *g_dzs_re, const float
 	CNET_HIP(hipcub::DeviceRadixSort::SortPairs(sort_ws, sort_bytes, (const int *) tokens, keys_out, (const int *) pos_in, pos_out, (int) n, 0,
 			32, rt().stream));
 	hipLaunchKernelGGL(embedding_bwd_kernel, dim3((unsigned) n), dim3(TPB), 0, rt().stream, keys_out, pos_out, n, g_dzs_re, g_dzs_im,
-			(long) ldg, slots, dim, table_dzs_re, table_dzs_im);
+			(long) ldg, slots, dim, vocab, table_dzs_re, table_dzs_im);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }

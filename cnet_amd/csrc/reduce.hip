@@ -163,6 +163,16 @@ __global__ __launch_bounds__(TPB) void l2out_fwd_kernel(const float *__restrict_
 }
 
 // ---------------------------------------------------------------------------------------------- CrossEntropy forward
+// loss of one row: -log(max(|z_label / sqrt S|^2, 1e-15)) (impl/crossent.h:62-72 upstream).  A label outside the row, which
+// upstream would read out of bounds, gives NaN here instead of a wild access.
+__device__ __forceinline__ float label_loss(const float *__restrict__ pr, const float *__restrict__ pi, int label, int cols, double inv) {
+	if ((unsigned) label >= (unsigned) cols) return __builtin_nanf("");
+	const float o_r = (float) (pr[label] * inv), o_i = (float) (pi[label] * inv);
+	float p = (float) ((double) o_r * o_r + (double) o_i * o_i);
+	p = (p < 1e-15f ? 1e-15f : p);
+	return -logf(p);
+}
+
 // impl/crossent.h:50-80, 117-130 upstream: S in double, clamped; out = z / sqrt(S); p_k = out_r^2 + out_i^2 evaluated
 // in double and rounded to float; argmax = first strict maximum of p; loss = -log(max(p_label, 1e-15)).
 template <int V, int G>
@@ -214,12 +224,8 @@ __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restri
 	const bool clear_cut = top.q2 < top.q1 * (1.0 - 1.0e-5);
 	if (!want_out && clear_cut) {
 		if (live && t == 0) {
-			const int label = labels[row];
-			float o_r = (float) (pr[label] * inv), o_i = (float) (pi[label] * inv);
-			float p = (float) ((double) o_r * o_r + (double) o_i * o_i);
-			p = (p < 1e-15f ? 1e-15f : p);
 			s[row] = S;
-			loss[row] = -logf(p);
+			loss[row] = label_loss(pr, pi, labels[row], cols, inv);
 			argmax[row] = top.i1;
 		}
 		return;
@@ -257,12 +263,8 @@ __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restri
 	}
 	best = group_reduce<ArgMax, G>(best, ArgMaxOp(), lds_a, slot, wig, lane);
 	if (live && t == 0) {
-		const int label = labels[row];
-		float o_r = (float) (pr[label] * inv), o_i = (float) (pi[label] * inv);
-		float p = (float) ((double) o_r * o_r + (double) o_i * o_i);
-		p = (p < 1e-15f ? 1e-15f : p);
 		s[row] = S;
-		loss[row] = -logf(p);
+		loss[row] = label_loss(pr, pi, labels[row], cols, inv);
 		argmax[row] = best.i;
 	}
 }

@@ -52,6 +52,33 @@ void *workspace(size_t bytes) {
 
 void release_twiddles();  // cdft.hip
 
+// destroys whatever streams and events exist (also the leftovers of an initialisation that failed half-way)
+static void destroy_streams(Runtime &r) {
+	if (r.upload_stream) {
+		hipStreamSynchronize(r.upload_stream);
+		hipStreamDestroy(r.upload_stream);
+	}
+	if (r.upload_done) hipEventDestroy(r.upload_done);
+	if (r.compute_done) hipEventDestroy(r.compute_done);
+	for (auto &m : r.marker) {
+		if (m) hipEventDestroy(m);
+		m = nullptr;
+	}
+	if (r.own_stream) hipStreamDestroy(r.own_stream);
+	r.upload_stream = r.own_stream = r.stream = nullptr;
+	r.upload_done = r.compute_done = nullptr;
+}
+
+static int create_streams(Runtime &r) {
+	CNET_HIP(hipStreamCreateWithFlags(&r.own_stream, hipStreamNonBlocking));
+	r.stream = r.own_stream;
+	CNET_HIP(hipStreamCreateWithFlags(&r.upload_stream, hipStreamNonBlocking));
+	CNET_HIP(hipEventCreateWithFlags(&r.upload_done, hipEventDisableTiming));
+	CNET_HIP(hipEventCreateWithFlags(&r.compute_done, hipEventDisableTiming));
+	for (auto &m : r.marker) CNET_HIP(hipEventCreateWithFlags(&m, hipEventDisableTiming));
+	return CNET_OK;
+}
+
 }  // namespace cnet
 
 using namespace cnet;
@@ -71,12 +98,11 @@ int cnet_init(int device) {
 	CNET_HIP(hipGetDeviceProperties(&r.prop, device));
 	if (strncmp(r.prop.gcnArchName, "gfx950", 6) != 0)
 		return fail(CNET_ERR_UNSUPPORTED, "cnet_init: kernels are built for gfx950 only, device is %s", r.prop.gcnArchName);
-	CNET_HIP(hipStreamCreateWithFlags(&r.own_stream, hipStreamNonBlocking));
-	r.stream = r.own_stream;
-	CNET_HIP(hipStreamCreateWithFlags(&r.upload_stream, hipStreamNonBlocking));
-	CNET_HIP(hipEventCreateWithFlags(&r.upload_done, hipEventDisableTiming));
-	CNET_HIP(hipEventCreateWithFlags(&r.compute_done, hipEventDisableTiming));
-	for (auto &m : r.marker) CNET_HIP(hipEventCreateWithFlags(&m, hipEventDisableTiming));
+	const int rc = create_streams(r);
+	if (rc != CNET_OK) {
+		destroy_streams(r);
+		return rc;
+	}
 	r.device = device;
 	r.ready = true;
 	return CNET_OK;
@@ -90,19 +116,8 @@ int cnet_shutdown(void) {
 	if (r.workspace) hipFree(r.workspace);
 	r.workspace = nullptr;
 	r.workspace_bytes = 0;
-	if (r.upload_stream) {
-		hipStreamSynchronize(r.upload_stream);
-		hipStreamDestroy(r.upload_stream);
-		hipEventDestroy(r.upload_done);
-		hipEventDestroy(r.compute_done);
-		for (auto &m : r.marker) {
-			hipEventDestroy(m);
-			m = nullptr;
-		}
-		r.upload_stream = nullptr;
-	}
-	if (r.own_stream) hipStreamDestroy(r.own_stream);
-	r.own_stream = r.stream = nullptr;
+	destroy_streams(r);
+	r.capturing = false;
 	r.ready = false;
 	r.device = -1;
 	return CNET_OK;
@@ -213,6 +228,7 @@ int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes) {
 
 int cnet_upload_wait_compute(void) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // would pull the upload stream into the recording
 	CNET_HIP(hipEventRecord(rt().compute_done, rt().stream));
 	CNET_HIP(hipStreamWaitEvent(rt().upload_stream, rt().compute_done, 0));
 	return CNET_OK;
@@ -220,6 +236,7 @@ int cnet_upload_wait_compute(void) {
 
 int cnet_mark_compute(int marker) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	CNET_CHECK_ARG(marker >= 0 && marker < Runtime::kMarkers);
 	CNET_HIP(hipEventRecord(rt().marker[marker], rt().stream));
 	return CNET_OK;
@@ -227,6 +244,7 @@ int cnet_mark_compute(int marker) {
 
 int cnet_upload_wait_marker(int marker) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
 	CNET_CHECK_ARG(marker >= 0 && marker < Runtime::kMarkers);
 	// a marker that was never set does not hold anything back
 	CNET_HIP(hipStreamWaitEvent(rt().upload_stream, rt().marker[marker], 0));
@@ -235,6 +253,7 @@ int cnet_upload_wait_marker(int marker) {
 
 int cnet_compute_wait_upload(void) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // would pull the upload stream into the recording
 	CNET_HIP(hipEventRecord(rt().upload_done, rt().upload_stream));
 	CNET_HIP(hipStreamWaitEvent(rt().stream, rt().upload_done, 0));
 	return CNET_OK;

@@ -1241,8 +1241,15 @@ public:
 		if (cin->rows_ != batch_ || batch.size() != batch_ || batch.sampleDim() != cin->input().length_)
 			throw std::invalid_argument("gpuSetInput: " + cin->getName() + " is not a data input of this batch shape");
 		CFunc::Slot &s = cin->slots_[0];
-		ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
-		ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), (size_t) batch_ * s.len * sizeof(float)), "cnet_memcpy_h2d");
+		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
+		if (batch.isPinned()) {  // queued behind the kernels that still read the previous contents; the host does not wait
+			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d_async");
+			ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
+			batch.in_flight_ = true;
+		} else {
+			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d");
+			ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
+		}
 	}
 	bool gpuForward(InputFunc *inp, OutputFunc *outp, EmbeddingBatch &batch) {
 		requireAllocated("gpuForward");
@@ -1415,6 +1422,9 @@ private:
 		} else {  // the per-sample token list of setInput(), in every row
 			for (int b = 0; b < e->rows_; ++b) std::copy(e->tokens_.begin(), e->tokens_.end(), buf.begin() + (size_t) b * e->no_out_tokens_);
 		}
+		// upstream asserts id < no_embeddings in setInput (impl/embed.h:84-100); anything below zero is padding
+		for (int32_t id : buf)
+			if (id >= e->no_embeddings_) throw std::out_of_range("token id " + std::to_string(id) + " outside the embedding table of " + e->getName());
 		ck(cnet_memcpy_h2d(e->d_tokens_, buf.data(), buf.size() * sizeof(int32_t)), "cnet_memcpy_h2d");
 	}
 };

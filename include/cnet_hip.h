@@ -88,8 +88,8 @@ int cnet_upload_sync(void);
  *      per layer on top, gpu/kernels.cpp:104-105).  Between cnet_graph_begin and cnet_graph_end the layer entry points
  *      record their kernels on the library's stream instead of running them; cnet_graph_launch replays the recording
  *      with one call.  Pointers, shapes and scalars (learning rate, accumulate flags) are frozen into the recording.
- *      Entry points that allocate or wait (cnet_alloc, cnet_free, cnet_sync, the blocking copies, the first use of a DFT
- *      length or of a larger workspace) return CNET_ERR_UNSUPPORTED while recording, and cnet_graph_end then fails:
+ *      Entry points that allocate, wait or order the two streams (cnet_alloc, cnet_free, cnet_sync, the blocking copies,
+ *      the marker / wait calls of the upload stream, the first use of a DFT length or of a larger workspace) return CNET_ERR_UNSUPPORTED while recording, and cnet_graph_end then fails:
  *      run the sequence once before recording it.  Clearing memory inside a recording uses a fill kernel
  *      (cnet_memset_zero), never a memset node. */
 int cnet_graph_begin(void);
@@ -217,7 +217,8 @@ int cnet_l2norm_bwd(const float *z_re, const float *z_im, int64_t ldz, const flo
 /* ---- CrossEntropy: replaces CrossEntropyGpu::gpu_cross_ent_forward / _backward (gpu/reduce.cpp:469-530,609-655)
  *      and the loss read-back of CNet::getLoss (gpu/gpu_func.h:906-926).  CPU twin impl/crossent.h:50-130.
  * labels[rows] int32.  s = clamped sum |z|^2, loss = -log(max(|z_label|^2/s, 1e-15)), argmax = first index of the
- * strict maximum of |z_k/sqrt(s)|^2.  out_re/out_im (normalised z) may be NULL. */
+ * strict maximum of |z_k/sqrt(s)|^2.  out_re/out_im (normalised z) may be NULL.  A label outside [0, cols) gives a NaN
+ * loss for its row (upstream reads out of bounds); the backward pass then treats every entry as a non-label entry. */
 int cnet_cross_entropy_fwd(const float *z_re, const float *z_im, int64_t ldz, const int32_t *labels,
                            float *out_re, float *out_im, int64_t ldo, float *s, float *loss, int32_t *argmax,
                            int rows, int cols);
@@ -254,7 +255,8 @@ int cnet_adam_update(float *z_re, float *z_im, float *m_re, float *m_im, float *
                      float lr, float beta, int t, int zero_grad);
 
 /* ---- CEmbedding: replaces gpu_embedding_forward / _backward (gpu/kernels.cpp:362-442), CPU twin impl/embed.h:109-148.
- * tokens[rows][slots] int32, -1 = padding (zero row).  y[rows][slots*dim].  The backward adds the dzs rows of equal
+ * tokens[rows][slots] int32, -1 = padding (zero row); an id >= vocab is treated as padding too (upstream asserts on
+ * the host; the host side above this ABI rejects it).  y[rows][slots*dim].  The backward adds the dzs rows of equal
  * tokens in (row, slot) order - deterministic, no atomics. */
 int cnet_embedding_fwd(const float *table_re, const float *table_im, int dim, int vocab, const int32_t *tokens,
                        float *y_re, float *y_im, int64_t ldy, int rows, int slots);

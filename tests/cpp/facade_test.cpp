@@ -1026,6 +1026,16 @@ static void test_errors() {
 	net3.add(new L2Out(InSize(2)), {lin});
 	expect("batched weight operand is refused", throws<std::invalid_argument>([&] { net3.allocateOnGpu(2); }));
 	(void) l2;
+	CNet net4;  // a token id outside the table is refused on the host before it reaches the device
+	auto emb = net4.add(new CEmbedding(2, 3, 5));
+	auto out4 = net4.add(new L2Out(InSize(6)), {emb});
+	net4.allocateOnGpu(2);
+	EmbeddingBatch ids(2, 3);
+	ids.add({1, 4, 0}, 0);
+	ids.add({2, 5}, 0);
+	expect("token id outside the table throws", throws<std::out_of_range>([&] {
+		net4.gpuForward((CEmbedding *) net4[emb], (L2Out *) net4[out4], ids);
+	}));
 	// device layer status codes
 	expect("invalid argument gives a status, not an exit", cnet_cgemm(0, 0, 0, 4, 4, 0, NULL, NULL, 0, NULL, NULL, 0, NULL, NULL, 0, 0) == CNET_ERR_INVALID_ARGUMENT);
 	expect("error text names the call", std::string(cnet_last_error()).find("cnet_cgemm") != std::string::npos);

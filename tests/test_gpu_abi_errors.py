@@ -92,3 +92,39 @@ def test_graph_recording_rules_and_replay(gpu, port):
         capi.sync()
     capi.call("cnet_graph_destroy", exe)
     capi.call("cnet_graph_destroy", None)
+
+
+def test_out_of_range_labels_and_token_ids_touch_nothing_outside_their_operands(gpu, port):
+    """Upstream indexes with a label or a token id unchecked (impl/crossent.h:62-72, impl/embed.h:113-118; its host side
+    asserts).  On the device a wrong index must not become a wild access: the loss of such a row is NaN, such a token
+    is padding, and the rows with valid indices are unaffected."""
+    B, n = 4, 24
+    zr, zi = seeded(port, 7, (B, n)), seeded(port, 8, (B, n))
+    good = np.array([3, 0, 23, 5], np.int32)
+    bad = good.copy(); bad[1], bad[3] = n, -7
+    _, _, S, loss, pred = port.crossent_fwd(zr, zi, good)
+    z = ops.CMat.from_host(zr, zi)
+    s, l, am = capi.empty(B), capi.empty(B), capi.empty(B, np.int32)
+    ops.cross_entropy_fwd(z, ops.ints(bad), s, l, am, None)
+    got = l.download()
+    assert np.isnan(got[[1, 3]]).all() and np.allclose(got[[0, 2]], loss[[0, 2]], rtol=2e-6)
+    assert np.array_equal(am.download(), pred)
+    dz = ops.Grad.empty(B, n)
+    ops.cross_entropy_bwd(z, s, ops.ints(bad), dz)    # rows 1 and 3: every entry is a non-label entry, z / S
+    h = dz.host()
+    assert np.allclose(h[2][1], zr[1] / S[1], rtol=1e-6) and np.isfinite(h[2]).all()
+
+    V, D, T = 6, 4, 3
+    tr, ti = seeded(port, 9, (V, D)), seeded(port, 10, (V, D))
+    tok = np.array([[1, 2, V], [5, V + 100, -1]], np.int32)   # padding only at the tail of a row, as upstream has it
+    as_padding = np.where(tok >= V, -1, tok).astype(np.int32)
+    yr, yi = port.embedding_fwd(tr, ti, as_padding)
+    y = ops.CMat.empty(2, T * D)
+    ops.embedding_fwd(ops.CMat.from_host(tr, ti), ops.ints(tok), y, T)
+    hy = y.host()
+    assert np.array_equal(hy[0], yr) and np.array_equal(hy[1], yi)
+    gs = [seeded(port, 11 + p, (2, T * D)) for p in range(2)]
+    dsr, dsi = port.embedding_bwd(V, D, as_padding, gs[0], gs[1])
+    d_re, d_im = ops.Plane.empty(V, D), ops.Plane.empty(V, D)
+    ops.embedding_bwd(ops.ints(tok), ops.Plane.from_host(gs[0]), ops.Plane.from_host(gs[1]), d_re, d_im, D, V, 2, T)
+    assert np.array_equal(d_re.host(), dsr) and np.array_equal(d_im.host(), dsi)
