@@ -581,6 +581,7 @@ class CNet {
 	CFunc *main_input_ = NULL;
 	int32_t *d_labels_ = NULL;
 	std::vector<int> labels_;
+	bool batch_labels_ = false;       // labels_ came with a batch (they then win over a label argument, as upstream)
 	// device double buffer of the data input: stage_[active_] is what the kernels read, the other one can be filled by
 	// gpuPrefetch() meanwhile
 	struct Stage {
@@ -598,6 +599,7 @@ class CNet {
 	};
 	StepGraphs graphs_[2];
 	bool use_graphs_ = false;
+	SimpleRand rand_{(uint64_t) clock()};  // upstream ComplexNet::rand_ (impl/cnet.h:56): the coin of sample()
 	bool input_dz_dirty_ = false;  // the dz planes of the input functions hold a first moment
 	bool warmed_[3] = {false, false, false};  // phase has run once since useGraphs(true)
 
@@ -1184,6 +1186,7 @@ public:
 			s.z = staged.z;
 			d_labels_ = staged.labels;
 			labels_.assign(batch.labelsPtr(), batch.labelsPtr() + batch_);
+			batch_labels_ = true;
 			return GpuForward();
 		}
 		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
@@ -1269,6 +1272,25 @@ public:
 		});
 		return true;
 	}
+	// spellings of upstream GpuNet (gpu/gpu_func.h:645-681).  GpuInfer is upstream's forward pass without the clearing of
+	// gradients; no forward pass clears gradients here (the first contribution of a backward pass overwrites), so it is
+	// the same pass.  GpuBackward's label applies when no batch has supplied labels, as upstream's does.
+	std::string GpuForward(bool &was_failure) {
+		was_failure = !GpuForward();
+		return "";
+	}
+	std::string GpuInfer(bool &was_failure) { return GpuForward(was_failure); }
+	std::string GpuBackward(int label, bool &was_failure) {
+		requireAllocated("GpuBackward");
+		if (!batch_labels_) {
+			std::vector<int> all(batch_, label);
+			setLabels(all.data(), batch_, false);
+			for (auto f : outputs_)  // the loss on the device follows the label in use
+				if (f->typeId() == isCrossEntropy) nodeForward(f);
+		}
+		was_failure = !gpuBackward();
+		return "";
+	}
 	bool gpuBackward() {
 		requireAllocated("gpuBackward");
 		runPhase(1, graphs_[active_].bwd, [&] {
@@ -1349,6 +1371,60 @@ public:
 		}
 		return loss / tmp.size();
 	}
+	// upstream GpuNet::getLoss(int label) (gpu/gpu_func.h:928-969): the loss of every output function, keyed by uid.
+	// Upstream has one entry per clone, i.e. per batch row, each clone under a uid of its own; there are no clones here,
+	// so an output's entry is the loss of batch row 0, which is the entry upstream's tests read (tests/gputests.h:64,
+	// 416, 456).  Per-row losses come from getLoss(outp, &batch).  As upstream, the label of the batch wins over the
+	// argument, and the CrossEntropy loss is formed on the host from z_label and S: -log(max(|z_label|^2 / S, 1e-15)).
+	std::map<int, float> getLoss(int label) {
+		requireAllocated("getLoss");
+		std::map<int, float> ret;
+		for (auto f : outputs_) {
+			if (f->typeId() == isL2Out) {
+				float v = 0.f;
+				ck(cnet_memcpy_d2h(&v, ((L2Out *) f)->d_loss_, sizeof(float)), "cnet_memcpy_d2h");
+				ret[f->uid()] = v;
+			} else if (f->typeId() == isCrossEntropy) {
+				const int lab = batch_labels_ ? labels_[0] : label;
+				if (lab < 0 || lab >= f->input().length_) throw std::out_of_range("getLoss: label outside the CrossEntropy input");
+				const float S = rowZeroOfCrossEntropy((CrossEntropy *) f);
+				float prob = std::norm(f->input().z(lab)) / S;
+				prob = (prob < 1e-15 ? 1e-15 : prob);
+				ret[f->uid()] = -std::log(prob);
+			}
+		}
+		return ret;
+	}
+	// upstream GpuNet::sample (gpu/gpu_func.h:971-1011): draws an index from the probabilities p_k = |z_k|^2 / S of the
+	// first CrossEntropy output (batch row 0): the first k whose running sum of p reaches a uniform coin; if rounding
+	// leaves the total below the coin, the most probable index.  0 for a net without a CrossEntropy output.
+	int sample() {
+		requireAllocated("sample");
+		for (auto f : outputs_) {
+			if (f->typeId() != isCrossEntropy) continue;
+			const float S = rowZeroOfCrossEntropy((CrossEntropy *) f);
+			const float coin = (float) rand_.randDouble();
+			float c_val = 0.f, max = 0.f;
+			int var_max = 0;
+			for (int var = 0; var < f->input().length_; ++var) {
+				const float p = std::norm(f->input().z(var)) / S;
+				c_val += p;
+				if (coin <= c_val) return var;
+				if (max < p) {
+					max = p;
+					var_max = var;
+				}
+			}
+			return var_max;
+		}
+		return 0;
+	}
+	void setRandSeed(uint64_t seed) { rand_ = SimpleRand(seed); }  // repeatable sample(); upstream seeds from clock()
+	CFunc *findFirstOfType(int type_id) {  // impl/cnet.h:85-92
+		for (auto f : func_list_)
+			if (f->typeId() == type_id) return f;
+		return NULL;
+	}
 	std::vector<int> getPredictions(OutputFunc *outp) {
 		requireAllocated("getPredictions");
 		CrossEntropy *c = dynamic_cast<CrossEntropy *>(outp);
@@ -1364,10 +1440,11 @@ public:
 				for (int k = 0; k < count; ++k)
 					if (labels[k] < 0 || labels[k] >= f->input().length_) throw std::out_of_range("setLabels: label outside the CrossEntropy input");
 	}
-	void setLabels(const int *labels, int count) {
+	void setLabels(const int *labels, int count, bool from_batch = true) {
 		requireAllocated("setLabels");
 		checkLabels(labels, count);
 		labels_.assign(labels, labels + count);
+		batch_labels_ = from_batch;
 		ck(cnet_memcpy_h2d(d_labels_, labels, count * sizeof(int32_t)), "cnet_memcpy_h2d");
 	}
 	void sync() { ck(cnet_sync(), "cnet_sync"); }
@@ -1392,7 +1469,7 @@ public:
 	}
 	void backward(int label) {
 		if (batch_ != 1) throw std::logic_error("backward(): call forward() first");
-		if (label >= 0) setLabels(&label, 1);
+		if (label >= 0) setLabels(&label, 1, false);
 		// the label only enters the backward pass of CrossEntropy; its forward outputs do not depend on it except
 		// the device-side loss, which is refreshed here so getLoss() matches the label in use
 		for (auto f : outputs_)
@@ -1415,6 +1492,13 @@ public:
 	}
 
 private:
+	// brings row 0 of a CrossEntropy node's input to its host view and returns that row's clamped S = sum |z|^2
+	float rowZeroOfCrossEntropy(CrossEntropy *c) {
+		fetch(c, 0);
+		float S = 0.f;
+		ck(cnet_memcpy_d2h(&S, c->d_s_, sizeof(float)), "cnet_memcpy_d2h");
+		return S < 1e-15 ? 1e-15 : S;
+	}
 	void uploadTokens(CEmbedding *e, const int *batch_tokens) {
 		std::vector<int32_t> buf((size_t) e->rows_ * e->no_out_tokens_, NO_TOKEN);
 		if (batch_tokens) {

@@ -50,6 +50,18 @@ static void expect(const std::string &what, bool ok) {
 	if (!ok) g_fail++;
 }
 
+template <class E, class F>
+static bool throws(F f) {
+	try {
+		f();
+	} catch (const E &) {
+		return true;
+	} catch (...) {
+		return false;
+	}
+	return false;
+}
+
 static void fill_normal(orc::Rng &r, float *p, size_t n, double sig) {
 	for (size_t k = 0; k < n; ++k) p[k] = (float) r.normal(0.0, sig);
 }
@@ -379,6 +391,108 @@ static void test_persample() {
 		on.update(0.3f, 1);
 	}
 	expect("loss decreases under Wirtinger gradient descent (" + std::to_string(first) + " -> " + std::to_string(last) + ")", last < first);
+}
+
+// ------------------------------------------------------------------------------------------------- loss map, sampling
+// Members of upstream's GpuNet / CNet that its own GPU tests and its generation loop use: getLoss(label)[uid]
+// (tests/gputests.h:64, 227, 416), GpuForward / GpuInfer / GpuBackward(label, was_failure) (tests/gputests.h:50, 71),
+// findFirstOfType (cnet.cpp:163-164), sample() (gpu/gpu_func.h:971-1011).
+static void test_loss_map_and_sampling() {
+	const int n = 6, classes = 5, B = 3;
+	orc::Rng rng(77);
+	std::vector<float> x((size_t) 2 * B * n), w((size_t) 2 * n * classes);
+	fill_normal(rng, x.data(), x.size(), 1.0);
+	fill_normal(rng, w.data(), w.size(), 0.6);
+	auto build = [&](CNet &net, int ids[5]) {
+		ids[0] = net.add(new CInput(OutSize(n)));
+		ids[1] = net.add(new CInput(OutSize(n * classes)));
+		ids[2] = net.add(new Linear(InSize(n), InSize(n * classes)), {ids[0], ids[1]});
+		ids[3] = net.add(new CrossEntropy(InSize(classes)), {ids[2]});
+		ids[4] = net.add(new L2Out(InSize(classes)), {ids[2]});
+		std::copy(w.begin(), w.end(), net[ids[1]]->mutable_input()->real_);
+	};
+	// the same net in the oracle, fed with sample 0
+	orc::Net on;
+	int oi = on.add(orc::kInput, n, 0, 0, NULL, 0), ow = on.add(orc::kInput, n * classes, 0, 0, NULL, 0);
+	int two[2] = {oi, ow};
+	int olin = on.add(orc::kLinear, n, n * classes, 0, two, 2);
+	int oce = on.add(orc::kCrossEntropy, classes, 0, 0, &olin, 1), ol2 = on.add(orc::kL2Out, classes, 0, 0, &olin, 1);
+	std::copy(w.begin(), w.end(), on.at(ow)->in.re);
+	std::copy(x.begin(), x.begin() + n, on.at(oi)->in.re);
+	std::copy(x.begin() + (size_t) B * n, x.begin() + (size_t) B * n + n, on.at(oi)->in.im);
+	on.forward();
+
+	CNet net;
+	int id[5];
+	build(net, id);
+	net.allocateOnGpu(B);
+	InputBatch batch(B, n);
+	const int labels[B] = {2, 0, 4};
+	for (int b = 0; b < B; ++b) batch.add(x.data() + (size_t) b * n, x.data() + (size_t) (B + b) * n, n, labels[b]);
+	net.gpuForward((CInput *) net[id[0]], (CrossEntropy *) net[id[3]], batch);
+	std::map<int, float> loss = net.getLoss(1);  // the label of the batch (2 for row 0) wins over the argument
+	expect("getLoss(label) has one entry per output function", loss.size() == 2 && loss.count(id[3]) && loss.count(id[4]));
+	report("getLoss(label)[CrossEntropy] = loss of row 0 under the batch label", std::fabs(loss[id[3]] - on.loss(oce, 2)) / on.loss(oce, 2), 1e-5);
+	report("getLoss(label)[L2Out] = loss of row 0", std::fabs(loss[id[4]] - on.loss(ol2, 0)) / on.loss(ol2, 0), 1e-5);
+	expect("findFirstOfType", net.findFirstOfType(isCrossEntropy) == net[id[3]] && net.findFirstOfType(isLinear) == net[id[2]] &&
+			net.findFirstOfType(isFourier) == NULL);
+
+	// sample(): frequencies follow p_k = |z_k|^2 / S of row 0; a seed repeats the draws
+	std::vector<double> p(classes);
+	{
+		const orc::Planes &z = on.at(oce)->in;
+		double S = 0;
+		for (int k = 0; k < classes; ++k) S += (double) z.re[k] * z.re[k] + (double) z.im[k] * z.im[k];
+		for (int k = 0; k < classes; ++k) p[k] = ((double) z.re[k] * z.re[k] + (double) z.im[k] * z.im[k]) / S;
+	}
+	const int draws = 6000;
+	std::vector<int> count(classes, 0), first;
+	net.setRandSeed(12345);
+	for (int d = 0; d < draws; ++d) {
+		int k = net.sample();
+		if (k < 0 || k >= classes) {
+			expect("sample() stays inside the distribution", false);
+			return;
+		}
+		count[k]++;
+		if (d < 32) first.push_back(k);
+	}
+	double worst = 0;
+	for (int k = 0; k < classes; ++k) worst = std::max(worst, std::fabs(count[k] / (double) draws - p[k]));
+	report("sample() frequencies against |z_k|^2 / S (6000 draws)", worst, 0.025);
+	net.setRandSeed(12345);
+	bool same = true;
+	for (int d = 0; d < 32; ++d) same = same && net.sample() == first[d];
+	expect("sample() repeats under the same seed", same);
+
+	// batch of one without batch labels: the label argument is the label (upstream AllocateNet(1) + GpuForward +
+	// getLoss(label) + GpuBackward(label), tests/gputests.h:44-71)
+	CNet one;
+	int jd[5];
+	build(one, jd);
+	std::copy(x.begin(), x.begin() + n, one[jd[0]]->mutable_input()->real_);
+	std::copy(x.begin() + (size_t) B * n, x.begin() + (size_t) B * n + n, one[jd[0]]->mutable_input()->imag_);
+	one.allocateOnGpu(1);
+	one.copyInputsToGpu();
+	bool was_failure = true;
+	one.GpuForward(was_failure);
+	expect("GpuForward(was_failure) reports success", !was_failure);
+	for (int label : {3, 1})
+		report("getLoss(" + std::to_string(label) + ")[CrossEntropy] without batch labels",
+				std::fabs(one.getLoss(label)[jd[3]] - on.loss(oce, label)) / on.loss(oce, label), 1e-5);
+	was_failure = true;
+	one.GpuInfer(was_failure);
+	expect("GpuInfer(was_failure) reports success", !was_failure);
+	one.GpuBackward(3, was_failure);
+	expect("GpuBackward(label, was_failure) reports success", !was_failure);
+	on.backward(3);
+	one.fetchAll(0);
+	ErrAcc z, g;
+	int pairs[5][2] = {{jd[0], oi}, {jd[1], ow}, {jd[2], olin}, {jd[3], oce}, {jd[4], ol2}};
+	for (auto &pr : pairs) cmp_node(one[pr[0]], on.at(pr[1]), &z, &g);
+	report("GpuBackward(3): all node values", z.value());
+	report("GpuBackward(3): all node gradients", g.value());
+	expect("a label outside the output throws", throws<std::out_of_range>([&] { one.getLoss(classes); }));
 }
 
 // ------------------------------------------------------------------------------------------------- embedding
@@ -986,17 +1100,6 @@ static void test_upstream_nets() {
 }
 
 // ------------------------------------------------------------------------------------------------- error behaviour
-template <class E, class F>
-static bool throws(F f) {
-	try {
-		f();
-	} catch (const E &) {
-		return true;
-	} catch (...) {
-		return false;
-	}
-	return false;
-}
 
 static void test_errors() {
 	CNet net;
@@ -1096,6 +1199,7 @@ int main(int argc, char **argv) {
 		if (what == "persample" || what == "all") test_persample();
 		if (what == "embedding" || what == "all") test_embedding();
 		if (what == "adam" || what == "all") test_adam();
+		if (what == "loss_map" || what == "all") test_loss_map_and_sampling();
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
 		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12, false);
 		if (what == "pipeline_timing") test_pipeline(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, true);

@@ -57,6 +57,12 @@ def test_triang_fourier_crelu_net_with_adam_steps():
     assert "FAIL" not in out and out.count("PASS") > 30
 
 
+def test_loss_map_sampling_and_the_gpunet_spellings():
+    """getLoss(label)[uid], sample(), findFirstOfType, GpuForward / GpuInfer / GpuBackward(label, was_failure)."""
+    out = _run("loss_map")
+    assert "FAIL" not in out and out.count("PASS") >= 14
+
+
 def test_upstream_model_files_restore_and_run_on_the_device(tmp_path):
     out = _run("saved_model", os.path.join(ROOT, "tests", "golden"), str(tmp_path))
     assert "FAIL" not in out and out.count("PASS") >= 16
