@@ -222,6 +222,22 @@ def token_model_suite(steps):
                       "loss_of_uniform_guess": round(float(np.log(V)), 4)}))
 
 
+def train_suite(steps):
+    """Training steps (upload of the batch, forward, loss read-back, backward, SGD) of the FourierTrans -> Hadamard ->
+    CGelu -> Linear -> CrossEntropy net on 784-long samples, run by the C++ facade's own driver; one JSON line per
+    batch size with the time per step of each input mode (copy inside forward / prefetch / recorded graphs)."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "bin", "facade_test")
+    if not os.path.exists(exe):
+        sys.exit("bench.py: %s is missing; run __graft_entry__.build() first" % exe)
+    for batch in (64, 4096):
+        r = subprocess.run([exe, "pipeline_timing", str(batch), str(steps)], capture_output=True, text=True, timeout=600)
+        lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
+        if r.returncode != 0 or not lines:
+            sys.exit("bench.py: facade_test pipeline_timing failed:\n" + r.stdout[-2000:] + r.stderr[-2000:])
+        print(lines[-1])
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -231,8 +247,10 @@ def main():
     ap.add_argument("--counter-pass", action="store_true",
                     help="short run for `rocprofv3 --pmc`: 3 launches of each GEMM kernel plus a plain copy kernel of "
                          "known size (256 MiB read, 256 MiB written) that calibrates FETCH_SIZE / WRITE_SIZE")
-    ap.add_argument("--suite", choices=["linear", "kernels", "token_model"], default="linear",
-                    help="linear (default): the headline line.  kernels: one line per other kernel of the hot path")
+    ap.add_argument("--suite", choices=["linear", "kernels", "token_model", "train"], default="linear",
+                    help="linear (default): the headline line.  kernels: one line per other kernel of the hot path.  "
+                         "token_model: configs[4] fwd+bwd.  train: training steps of the 784 -> 10 net of configs[0] "
+                         "through the C++ facade, input pipeline included, at batch 64 and 4096")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (one process, one device, no collectives); --gpus %d is not "
@@ -243,6 +261,9 @@ def main():
         return
     if args.suite == "token_model":
         token_model_suite(max(args.steps // 20, 3))
+        return
+    if args.suite == "train":
+        train_suite(max(args.steps, 30))
         return
 
     from cnet_amd import capi, ops

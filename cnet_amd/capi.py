@@ -36,6 +36,8 @@ SIGNATURES = {
     "cnet_upload_wait_marker": [_i],
     "cnet_compute_wait_upload": [],
     "cnet_upload_sync": [],
+    "cnet_copy_ticket": [_i, C.POINTER(C.c_int64)],
+    "cnet_copy_wait": [C.c_int64],
     "cnet_graph_begin": [],
     "cnet_graph_end": [C.POINTER(C.c_void_p)],
     "cnet_graph_launch": [C.c_void_p],

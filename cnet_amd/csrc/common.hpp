@@ -23,6 +23,12 @@ struct Runtime {
 	hipEvent_t upload_done = nullptr, compute_done = nullptr;
 	static constexpr int kMarkers = 8;
 	hipEvent_t marker[kMarkers] = {};  // caller-numbered points of the compute stream
+	// tickets: points of either stream the HOST can wait for one by one (has this copy left its page-locked source?).
+	// A ring of events per stream; a slot that was reused stands for a later point of the same stream, so waiting on it
+	// can only wait longer, never too short.
+	static constexpr int kTickets = 32;
+	hipEvent_t ticket_event[2][kTickets] = {};
+	int64_t tickets_issued[2] = {0, 0};
 	bool capturing = false;  // between cnet_graph_begin and cnet_graph_end: nothing may allocate or wait
 	hipDeviceProp_t prop;
 	// grow-only scratch for two-stage deterministic reductions (never allocated inside a hot loop twice

@@ -64,6 +64,12 @@ static void destroy_streams(Runtime &r) {
 		if (m) hipEventDestroy(m);
 		m = nullptr;
 	}
+	for (auto &ring : r.ticket_event)
+		for (auto &e : ring) {
+			if (e) hipEventDestroy(e);
+			e = nullptr;
+		}
+	r.tickets_issued[0] = r.tickets_issued[1] = 0;
 	if (r.own_stream) hipStreamDestroy(r.own_stream);
 	r.upload_stream = r.own_stream = r.stream = nullptr;
 	r.upload_done = r.compute_done = nullptr;
@@ -76,6 +82,8 @@ static int create_streams(Runtime &r) {
 	CNET_HIP(hipEventCreateWithFlags(&r.upload_done, hipEventDisableTiming));
 	CNET_HIP(hipEventCreateWithFlags(&r.compute_done, hipEventDisableTiming));
 	for (auto &m : r.marker) CNET_HIP(hipEventCreateWithFlags(&m, hipEventDisableTiming));
+	for (auto &ring : r.ticket_event)
+		for (auto &e : ring) CNET_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
 	return CNET_OK;
 }
 
@@ -256,6 +264,30 @@ int cnet_compute_wait_upload(void) {
 	CNET_NOT_IN_CAPTURE();  // would pull the upload stream into the recording
 	CNET_HIP(hipEventRecord(rt().upload_done, rt().upload_stream));
 	CNET_HIP(hipStreamWaitEvent(rt().stream, rt().upload_done, 0));
+	return CNET_OK;
+}
+
+int cnet_copy_ticket(int upload_stream, int64_t *ticket) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
+	CNET_CHECK_ARG(ticket != nullptr);
+	Runtime &r = rt();
+	const int which = upload_stream ? 1 : 0;
+	const int64_t n = r.tickets_issued[which];
+	CNET_HIP(hipEventRecord(r.ticket_event[which][n % Runtime::kTickets], which ? r.upload_stream : r.stream));
+	r.tickets_issued[which] = n + 1;
+	*ticket = 2 * n + which;
+	return CNET_OK;
+}
+
+int cnet_copy_wait(int64_t ticket) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
+	Runtime &r = rt();
+	const int which = (int) (ticket & 1);
+	const int64_t n = ticket >> 1;
+	CNET_CHECK_ARG(ticket >= 0 && n < r.tickets_issued[which]);
+	CNET_HIP(hipEventSynchronize(r.ticket_event[which][n % Runtime::kTickets]));
 	return CNET_OK;
 }
 

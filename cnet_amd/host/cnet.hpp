@@ -176,7 +176,7 @@ class InputBatch : public Batch {
 	friend class CNet;
 	float *real_data_ = NULL, *imag_data_ = NULL;  // [batch][dim] each, one allocation
 	bool pinned_ = false;
-	bool in_flight_ = false;  // an upload queued from these planes may not have finished
+	int64_t ticket_ = -1;     // >= 0: a copy queued from these planes may not have finished; what the host waits for
 
 	void allocate() {
 		const size_t bytes = 2 * (size_t) batch_size_ * sample_dim_ * sizeof(float);
@@ -198,10 +198,12 @@ class InputBatch : public Batch {
 		real_data_ = imag_data_ = NULL;
 	}
 	void settle() {  // before the host writes the planes again
-		if (in_flight_) {
-			cnet_upload_sync();
-			cnet_sync();
-			in_flight_ = false;
+		if (ticket_ >= 0) {  // waits for that copy only: a copy out of another batch may still be running
+			if (cnet_copy_wait(ticket_) != CNET_OK) {
+				cnet_upload_sync();
+				cnet_sync();
+			}
+			ticket_ = -1;
 		}
 	}
 	float *rowRe() { return real_data_ + (size_t) current_pos_ * sample_dim_; }
@@ -222,7 +224,7 @@ public:
 		if (o.real_data_) std::copy(o.real_data_, o.real_data_ + 2 * (size_t) batch_size_ * sample_dim_, real_data_);
 	}
 	InputBatch(InputBatch &&o) noexcept : Batch(std::move(o)), real_data_(o.real_data_), imag_data_(o.imag_data_), pinned_(o.pinned_),
-			in_flight_(o.in_flight_) {
+			ticket_(o.ticket_) {
 		o.real_data_ = o.imag_data_ = NULL;
 	}
 	InputBatch &operator=(InputBatch &&o) noexcept {
@@ -232,7 +234,7 @@ public:
 			real_data_ = o.real_data_;
 			imag_data_ = o.imag_data_;
 			pinned_ = o.pinned_;
-			in_flight_ = o.in_flight_;
+			ticket_ = o.ticket_;
 			o.real_data_ = o.imag_data_ = NULL;
 		}
 		return *this;
@@ -269,6 +271,25 @@ public:
 		std::copy(re, re + n, rowRe());
 		std::copy(im, im + n, rowIm());
 		finishRow(n, label);
+	}
+	// Fill the next `count` rows from planar sample storage ([sample][dim] re and im): row k takes sample index[k] and
+	// label labels[index[k]].  The rows are independent copies, spread over the host threads when built with OpenMP (a
+	// batch of 4096 x 784 is 25 MB; one thread assembles it no faster than the device trains on it).
+	void gather(const float *re, const float *im, const int *labels, const int *index, int count) {
+		assert(current_pos_ + count <= batch_size_);
+		settle();
+		const size_t dim = (size_t) sample_dim_;
+		float *dst_re = rowRe(), *dst_im = rowIm();
+#pragma omp parallel for schedule(static) if ((size_t) count * dim >= (1u << 18))
+		for (int k = 0; k < count; ++k) {
+			std::memcpy(dst_re + k * dim, re + index[k] * dim, dim * sizeof(float));
+			std::memcpy(dst_im + k * dim, im + index[k] * dim, dim * sizeof(float));
+		}
+		for (int k = 0; k < count; ++k) {
+			labels_.push_back(labels[index[k]]);
+			sizes_.push_back(sample_dim_);
+		}
+		current_pos_ += count;
 	}
 	const float *realDataPtr() const { return real_data_; }
 	const float *imagDataPtr() const { return imag_data_; }
@@ -588,6 +609,7 @@ class CNet {
 		float *z = NULL;            // 2 planes [batch][len]
 		int32_t *labels = NULL;     // [batch]
 		int32_t *host_labels = NULL;  // page-locked staging of the labels
+		int64_t labels_ticket = -1;   // the last copy out of host_labels
 		const InputBatch *holds = NULL;
 	};
 	Stage stage_[2];
@@ -1105,11 +1127,13 @@ public:
 			float *z = s.z;
 			if (s.rows == 1) {
 				ck(cnet_memcpy_h2d(z, f->mutable_input()->real_, 2 * (size_t) s.len * sizeof(float)), "cnet_memcpy_h2d");
-			} else {  // the data input: the host view holds one sample, replicate it to every row
+			} else {  // the data input: the host view holds one sample, replicate it to every row (one copy for both planes)
+				std::vector<float> rows(2 * (size_t) s.rows * s.len);
 				for (int b = 0; b < s.rows; ++b) {
-					ck(cnet_memcpy_h2d(z + (size_t) b * s.len, f->mutable_input()->real_, s.len * sizeof(float)), "cnet_memcpy_h2d");
-					ck(cnet_memcpy_h2d(z + (size_t) (s.rows + b) * s.len, f->mutable_input()->imag_, s.len * sizeof(float)), "cnet_memcpy_h2d");
+					std::copy(f->input().real_, f->input().real_ + s.len, rows.begin() + (size_t) b * s.len);
+					std::copy(f->input().imag_, f->input().imag_ + s.len, rows.begin() + (size_t) (s.rows + b) * s.len);
 				}
+				ck(cnet_memcpy_h2d(z, rows.data(), rows.size() * sizeof(float)), "cnet_memcpy_h2d");
 			}
 			if (f->typeId() == isEmbedding) uploadTokens((CEmbedding *) f, NULL);
 		}
@@ -1194,7 +1218,7 @@ public:
 		if (batch.isPinned()) {
 			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d_async");
 			ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
-			batch.in_flight_ = true;
+			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
 		} else {
 			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d");
 			ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
@@ -1229,13 +1253,14 @@ public:
 			ck(cnet_host_alloc(batch_ * sizeof(int32_t), &h), "cnet_host_alloc");
 			st.host_labels = (int32_t *) h;
 		}
-		ck(cnet_upload_sync(), "cnet_upload_sync");  // the previous upload has left host_labels
+		if (st.labels_ticket >= 0) ck(cnet_copy_wait(st.labels_ticket), "cnet_copy_wait");  // the previous copy has left host_labels
 		std::copy(batch.labelsPtr(), batch.labelsPtr() + batch_, st.host_labels);
 		ck(cnet_upload_wait_marker(other), "cnet_upload_wait_marker");  // kernels of the step that last used this buffer
 		ck(cnet_upload_async(st.z, batch.realDataPtr(), plane * sizeof(float)), "cnet_upload_async");
 		ck(cnet_upload_async(st.z + plane, batch.imagDataPtr(), plane * sizeof(float)), "cnet_upload_async");
 		ck(cnet_upload_async(st.labels, st.host_labels, batch_ * sizeof(int32_t)), "cnet_upload_async");
-		batch.in_flight_ = true;
+		ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
+		st.labels_ticket = batch.ticket_;
 		st.holds = &batch;
 	}
 	// upload a batch into a CInput flagged with setIsBatched(true); labels of that batch are ignored
@@ -1248,7 +1273,7 @@ public:
 		if (batch.isPinned()) {  // queued behind the kernels that still read the previous contents; the host does not wait
 			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d_async");
 			ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
-			batch.in_flight_ = true;
+			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
 		} else {
 			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d");
 			ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");

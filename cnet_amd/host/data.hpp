@@ -21,6 +21,7 @@ class BatchedDataReader {
 	std::vector<float> re_, im_;  // [count][dim]
 	std::vector<int> labels_;
 	std::vector<int> order_;      // position -> sample
+	std::vector<int> pick_;       // samples of the batch being assembled
 
 protected:
 	int sample_dim_ = 0;
@@ -53,11 +54,12 @@ public:
 	void nextBatch(InputBatch &batch) {
 		assert(labels_.size() && batch.sampleDim() == sample_dim_);
 		batch.clear();
+		pick_.resize(batch.size());
 		for (int i = 0; i < batch.size(); ++i) {
-			const size_t at = (size_t) order_[current_] * sample_dim_;
-			batch.add(&re_[at], &im_[at], sample_dim_, labels_[order_[current_]]);
+			pick_[i] = order_[current_];
 			current_ = (current_ + 1) % (int) labels_.size();
 		}
+		batch.gather(re_.data(), im_.data(), labels_.data(), pick_.data(), batch.size());
 	}
 
 	void add(const std::vector<std::complex<float> > &data, int label) {

@@ -73,7 +73,11 @@ int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes);   /* *_copy_
  *      compute stream under number m now, make later uploads wait for that point when a buffer is about to be refilled
  *      (double buffering: the marker is set when a buffer is retired, the wait is issued when it is reused).
  * cnet_compute_wait_upload: kernels queued after this call start only when every upload queued so far has landed.
- * cnet_upload_sync: host waits for the upload stream (before reusing a page-locked source buffer). */
+ * cnet_upload_sync: host waits for the upload stream (before reusing a page-locked source buffer).
+ * cnet_copy_ticket(upload_stream, &t) / cnet_copy_wait(t): the host-side twin of the markers - t names the current tail of
+ *      the compute stream (upload_stream = 0) or of the upload stream (1); cnet_copy_wait(t) blocks the host until that
+ *      point has been reached and nothing later, so one page-locked buffer can be refilled while the copy out of the
+ *      next one is still running.  May wait for a somewhat later point of the same stream once 32 newer tickets exist. */
 int cnet_host_alloc(size_t bytes, void **host_ptr);
 int cnet_host_free(void *host_ptr);
 int cnet_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
@@ -83,6 +87,8 @@ int cnet_mark_compute(int marker);
 int cnet_upload_wait_marker(int marker);
 int cnet_compute_wait_upload(void);
 int cnet_upload_sync(void);
+int cnet_copy_ticket(int upload_stream, int64_t *ticket);
+int cnet_copy_wait(int64_t ticket);
 
 /* ---- Graphs: a training step at small batch sizes is bound by launch overhead (upstream pays a cudaDeviceSynchronize
  *      per layer on top, gpu/kernels.cpp:104-105).  Between cnet_graph_begin and cnet_graph_end the layer entry points

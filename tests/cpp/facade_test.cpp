@@ -881,22 +881,26 @@ static void test_pipeline(int B, int steps, bool timing_only) {
 		if (graphs) net.useGraphs(true);
 		net.sync();
 		auto t0 = std::chrono::steady_clock::now();
+		// With prefetch the host runs two batches ahead: while the device computes step s, batch s+1 (assembled during
+		// step s-1) travels on the upload stream and batch s+2 is assembled into the third buffer of the ring.
 		if (prefetch) {
 			reader.nextBatch(ring[0]);
 			net.gpuPrefetch(cin, ring[0]);
+			if (steps > 1) reader.nextBatch(ring[1]);
 		}
 		for (int s = 0; s < steps; ++s) {
 			InputBatch &cur = ring[s % 3];
 			if (!prefetch) reader.nextBatch(cur);
+			// the whole step is queued first; only then does the host turn to the next batches, and last of all it waits
+			// for this step's losses (backward and update do not touch them)
 			net.gpuForward(cin, cen, cur);
-			if (prefetch && s + 1 < steps) {  // the next batch travels while this step computes
-				InputBatch &next = ring[(s + 1) % 3];
-				reader.nextBatch(next);
-				net.gpuPrefetch(cin, next);
-			}
-			losses[mode].push_back(net.getLoss(cen, &cur));
 			net.gpuBackward();
 			net.gpuUpdateInputs((s < steps / 2 ? lr : 0.5f * lr) / B);
+			if (prefetch) {
+				if (s + 1 < steps) net.gpuPrefetch(cin, ring[(s + 1) % 3]);
+				if (s + 2 < steps) reader.nextBatch(ring[(s + 2) % 3]);
+			}
+			losses[mode].push_back(net.getLoss(cen, &cur));
 		}
 		net.sync();
 		ms[mode] = 1e3 * std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / steps;
