@@ -43,6 +43,13 @@ def test_invalid_arguments_are_reported_not_fatal(gpu, port):
     assert _status("cnet_cdft_plan", 50000) == INVALID
     assert _status("cnet_adam_update", x.re.ptr, x.im.ptr, y.re.ptr, y.im.ptr, y.re.ptr, y.im.ptr, 32, 0.1, 0.9, -1, 1) == INVALID
     assert _status("cnet_mark_compute", 8) == INVALID and _status("cnet_upload_wait_marker", -1) == INVALID
+    # copy tickets: one per stream, waited for one by one; a ticket that was never issued is refused
+    t0, t1 = C.c_int64(-1), C.c_int64(-1)
+    assert _status("cnet_copy_ticket", 0, C.byref(t0)) == 0 and _status("cnet_copy_ticket", 1, C.byref(t1)) == 0
+    assert t0.value >= 0 and t1.value >= 0 and t0.value % 2 == 0 and t1.value % 2 == 1
+    assert _status("cnet_copy_wait", t1.value) == 0 and _status("cnet_copy_wait", t0.value) == 0
+    assert _status("cnet_copy_wait", t1.value + 2) == INVALID and _status("cnet_copy_wait", -1) == INVALID
+    assert _status("cnet_copy_ticket", 0, None) == INVALID
     # a second init on the same device is idempotent, on another device it is refused
     assert _status("cnet_init", 0) == 0
     assert _status("cnet_init", 3) == INVALID
@@ -69,6 +76,9 @@ def test_graph_recording_rules_and_replay(gpu, port):
     assert _status("cnet_sync") == UNSUPPORTED
     assert _status("cnet_cdft_plan", 96) == UNSUPPORTED  # a new transform length needs memory
     assert _status("cnet_graph_begin") == UNSUPPORTED
+    assert _status("cnet_mark_compute", 0) == UNSUPPORTED and _status("cnet_compute_wait_upload") == UNSUPPORTED
+    t = C.c_int64(-1)
+    assert _status("cnet_copy_ticket", 0, C.byref(t)) == UNSUPPORTED
     capi.call("cnet_graph_end", None)
     capi.sync()
     # record forward + activation + clearing of a buffer, replay three times with eager work and syncs in between
