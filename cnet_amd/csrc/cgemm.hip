@@ -380,12 +380,15 @@ struct Frag {
 	float s_re[2][T], s_im[2][T];
 	float4 q_re[2][T], q_im[2][T];
 	const float *base0, *base1;  // per-lane LDS addresses inside stage 0, plane re
+	const float *row_base[T];    // [k][row] operands: base0 of each tile; everything else in an address is a multiple of 256 bytes
 
 	// w0: first row of the wavefront's sub-block; r = lane % 32, h = lane / 32
 	__device__ __forceinline__ void init(const float *plane_re, int w0, int r, int h) {
 		if (MCONTIG) {
 			base0 = plane_re + w0 + r + h * 4 * PITCH;
 			base1 = base0;
+#pragma unroll
+			for (int i = 0; i < T; ++i) row_base[i] = base0 + i * 32;
 		} else {
 			const int row = w0 + r;
 			const int sw = (row >> 2) & 3;
@@ -396,12 +399,11 @@ struct Frag {
 	// [k][row] operands: values of k step s into slot s & 1
 	__device__ __forceinline__ void fetch_step(int stage_off, int s) {
 		if (MCONTIG) {
-			const float *b = base0 + stage_off;
 			const int line = (s < 4 ? s : s + 4) * PITCH;
 #pragma unroll
 			for (int i = 0; i < T; ++i) {
-				s_re[s & 1][i] = b[line + i * 32];
-				s_im[s & 1][i] = b[PLANE + line + i * 32];
+				s_re[s & 1][i] = row_base[i][stage_off + line];
+				s_im[s & 1][i] = row_base[i][stage_off + PLANE + line];
 			}
 		}
 	}
@@ -432,13 +434,14 @@ struct DlStage {
 	static constexpr int PITCH = MCONTIG ? ROWS : KC;
 	static constexpr int PLANE = ROWS * KC;
 	unsigned goff[UNITS];  // byte offset of this lane's 16 bytes inside the operand tile of a chunk
-	int wave;
+	int wave_s;            // wavefront number, held in a scalar register
 
 	// rows_valid: rows of the operand that exist from the first row of this block on (>= ROWS inside the matrix; a
 	// multiple of 4 when MCONTIG).  Rows past the end are fetched from the last valid ones instead: what they produce
 	// lies outside C and is never stored.
 	__device__ __forceinline__ void init(long ld, int rows_valid) {
-		wave = threadIdx.x >> 6;
+		const int wave = threadIdx.x >> 6;
+		wave_s = __builtin_amdgcn_readfirstlane(wave);
 		const int lane = threadIdx.x & 63;
 #pragma unroll
 		for (int u = 0; u < UNITS; ++u) {
@@ -458,9 +461,9 @@ struct DlStage {
 		// alias and puts a vmcnt(0) wait in front of the first fragment read of the current chunk, which exposes the
 		// whole memory latency once per chunk.  The wait that is needed (before the barrier that publishes the stage)
 		// is in the kernel.  m0 = LDS byte address of the KiB this wavefront fills; one wait state before its use.
-		const unsigned dst = (unsigned) ((u * 4 + wave) * 1024);
-		const unsigned lre = __builtin_amdgcn_readfirstlane((unsigned) (size_t) sre + dst);
-		const unsigned lim = __builtin_amdgcn_readfirstlane((unsigned) (size_t) sim + dst);
+		const unsigned dst = (unsigned) ((u * 4 + wave_s) * 1024);  // scalar arithmetic: nothing for the vector ALU
+		const unsigned lre = (unsigned) (size_t) sre + dst;
+		const unsigned lim = (unsigned) (size_t) sim + dst;
 		asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(goff[u]), "s"(tile_re), "s"(lre) : "memory", "m0");
 		asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(goff[u]), "s"(tile_im), "s"(lim) : "memory", "m0");
 #endif
@@ -515,7 +518,12 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	const int wn0 = (wave % (BN / WN)) * WN;
 	const int r = lane & 31, h = lane >> 5;
 
-	floatx16 acc_re[TM][TN], acc_im[TM][TN];
+	// Accumulators.  A wavefront with one or two tiles keeps the four real products apart (P = Ar Br, R = Ar Bi, Q = Ai Bi,
+	// S = Ai Br) and combines them with their signs when it stores, so its K loop has no vector-ALU instruction for signs at
+	// all; with four tiles there are only registers for two sets, re = P -+ Q and im = +-R +- S, and one operand of the
+	// second product is negated per k pair (see the modes below).
+	constexpr bool ACC4 = TM * TN <= 2;
+	floatx16 acc_re[TM][TN], acc_im[TM][TN], acc_q[ACC4 ? TM : 1][ACC4 ? TN : 1], acc_s[ACC4 ? TM : 1][ACC4 ? TN : 1];
 	for (int pass = 0; pass < npass; ++pass) {
 	const int tile_n = pass ? args.tiles_n - 1 - tile_n_first : tile_n_first;
 	const int n0 = tile_n * BN;
@@ -528,6 +536,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			for (int e = 0; e < 16; ++e) {
 				acc_re[i][j][e] = 0.f;
 				acc_im[i][j][e] = 0.f;
+				if (ACC4) {
+					acc_q[i][j][e] = 0.f;
+					acc_s[i][j][e] = 0.f;
+				}
 			}
 
 	StageA sa;
@@ -554,7 +566,14 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			sb.issue(u, pb.b_re + b_tile0 + chunk * b_step, pb.b_im + b_tile0 + chunk * b_step, stage + 2 * A_PLANE,
 					stage + 2 * A_PLANE + B_PLANE);
 	};
-	const unsigned a_neg = pb.a_im_sign < 0.f ? 0x80000000u : 0u, b_neg = pb.b_im_sign < 0.f ? 0x80000000u : 0u;
+	// Signs of the imaginary parts (conj): (Ar + i sa Ai)(Br + i sb Bi) = (Ar Br - sa sb Ai Bi) + i (sb Ar Bi + sa Ai Br).
+	// Which operand is negated is a compile-time property of the loop below, so the only vector-ALU work per k pair is one
+	// negation per A fragment (every VALU instruction costs the matrix pipe a few cycles: it shares its issue port):
+	//   mode 0 (no conj):  re += Ar Br + (-Ai) Bi   im += Ar Bi + Ai Br
+	//   mode 1 (conj B):   re += Ar Br + Ai Bi      im += (-Ar) Bi + Ai Br
+	//   mode 2 (conj A):   re += Ar Br + Ai Bi      im += Ar Bi + (-Ai) Br
+	//   mode 3 (both):     re += Ar Br + (-Ai) Bi   im += Ar Bi + Ai Br, negated when it is stored
+	const int mode = (pb.a_im_sign < 0.f ? 2 : 0) | (pb.b_im_sign < 0.f ? 1 : 0);
 
 	constexpr int LOADS_PER_CHUNK = 2 * (UA + UB);  // transfers one wavefront issues per chunk
 	static_assert(NST == 2 || NST == 3, "two or three stages");
@@ -574,13 +593,13 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	fa.fetch_set(0, 0);
 	fb.fetch_set(0, 0);
 
-	int cur = 0;  // stage that holds chunk c
-	for (int c = c_lo; c < c_hi; ++c) {
+	// One chunk, held in stage `cur`.
+	auto chunk = [&](int cur, auto mode_c, int c) {
+		constexpr int MODE = decltype(mode_c)::value;
 		const int nxt = cur + 1 == NST ? 0 : cur + 1, far = cur == 0 ? NST - 1 : cur - 1;
-		const int CUR = cur * STAGE_FLOATS, NXT = nxt * STAGE_FLOATS;
+		const int CUR = cur * STAGE_FLOATS, NXT = nxt * STAGE_FLOATS, FAR = far * STAGE_FLOATS;
 		const bool ahead = (c + NST - 1 < c_hi);
-		if (ahead) issue_chunk(c + NST - 1, smem + far * STAGE_FLOATS);
-		cur = nxt;
+		if (ahead) issue_chunk(c + NST - 1, smem + FAR);
 #pragma unroll
 		for (int ks = 0; ks < KS; ++ks) {
 			if (ks + 1 < KS) {
@@ -604,32 +623,49 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				fa.fetch_set(NXT, 0);
 				fb.fetch_set(NXT, 0);
 			}
-			float are[TM], aim[TM], anim[TM], bre[TN], bim[TN];
+			float are[TM], aim[TM], neg[TM], bre[TN], bim[TN];
 #pragma unroll
 			for (int i = 0; i < TM; ++i) {
 				are[i] = fa.re(ks, i);
-				aim[i] = __uint_as_float(__float_as_uint(fa.im(ks, i)) ^ a_neg);
-				anim[i] = -aim[i];
+				aim[i] = fa.im(ks, i);
+				if (!ACC4) neg[i] = MODE == 1 ? -are[i] : -aim[i];
 			}
 #pragma unroll
 			for (int j = 0; j < TN; ++j) {
 				bre[j] = fb.re(ks, j);
-				bim[j] = __uint_as_float(__float_as_uint(fb.im(ks, j)) ^ b_neg);
+				bim[j] = fb.im(ks, j);
 			}
+			if constexpr (ACC4) {
 #pragma unroll
-			for (int i = 0; i < TM; ++i)
+				for (int i = 0; i < TM; ++i)
 #pragma unroll
-				for (int j = 0; j < TN; ++j) {
-					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bre[j], acc_re[i][j], 0, 0, 0);
-					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bim[j], acc_im[i][j], 0, 0, 0);
-				}
+					for (int j = 0; j < TN; ++j) {
+						acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bre[j], acc_re[i][j], 0, 0, 0);  // P
+						acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bim[j], acc_im[i][j], 0, 0, 0);  // R
+					}
 #pragma unroll
-			for (int i = 0; i < TM; ++i)
+				for (int i = 0; i < TM; ++i)
 #pragma unroll
-				for (int j = 0; j < TN; ++j) {
-					acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(anim[i], bim[j], acc_re[i][j], 0, 0, 0);
-					acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aim[i], bre[j], acc_im[i][j], 0, 0, 0);
-				}
+					for (int j = 0; j < TN; ++j) {
+						acc_q[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aim[i], bim[j], acc_q[i][j], 0, 0, 0);  // Q
+						acc_s[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aim[i], bre[j], acc_s[i][j], 0, 0, 0);  // S
+					}
+			} else {
+#pragma unroll
+				for (int i = 0; i < TM; ++i)
+#pragma unroll
+					for (int j = 0; j < TN; ++j) {
+						acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bre[j], acc_re[i][j], 0, 0, 0);
+						acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(MODE == 1 ? neg[i] : are[i], bim[j], acc_im[i][j], 0, 0, 0);
+					}
+#pragma unroll
+				for (int i = 0; i < TM; ++i)
+#pragma unroll
+					for (int j = 0; j < TN; ++j) {
+						acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32((MODE == 0 || MODE == 3) ? neg[i] : aim[i], bim[j], acc_re[i][j], 0, 0, 0);
+						acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(MODE == 2 ? neg[i] : aim[i], bre[j], acc_im[i][j], 0, 0, 0);
+					}
+			}
 			if (SCHED_RECIPE && ks < KS - 1) {
 				// scheduling recipe for this k pair: after each MFMA let a few of the pending VALU / LDS / global
 				// instructions issue, so they run in the shadow of the matrix pipe
@@ -643,7 +679,26 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			}
 			__builtin_amdgcn_sched_barrier(0);
 		}
+	};
+	// the chunks of this block: chunk c_lo + n sits in stage n % NST
+	auto kloop = [&](auto mode_c) {
+		int cur = 0;
+		for (int c = c_lo; c < c_hi; ++c) {
+			chunk(cur, mode_c, c);
+			cur = cur + 1 == NST ? 0 : cur + 1;
+		}
+	};
+	if constexpr (ACC4) {
+		kloop(std::integral_constant<int, 0>());  // the signs wait for the store
+	} else {
+		switch (mode) {
+		case 0: kloop(std::integral_constant<int, 0>()); break;
+		case 1: kloop(std::integral_constant<int, 1>()); break;
+		case 2: kloop(std::integral_constant<int, 2>()); break;
+		default: kloop(std::integral_constant<int, 3>()); break;
+		}
 	}
+	const bool q_minus = mode == 0 || mode == 3, r_minus = (mode & 1) != 0, s_minus = (mode & 2) != 0;
 
 #pragma unroll
 	for (int i = 0; i < TM; ++i)
@@ -656,7 +711,15 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
 				if (row < args.M) {
 					const long off = (long) row * ldc + col;
-					float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
+					float vr, vi;
+					if constexpr (ACC4) {
+						const float q = acc_q[i][j][e], rr = acc_im[i][j][e], ss = acc_s[i][j][e];
+						vr = q_minus ? acc_re[i][j][e] - q : acc_re[i][j][e] + q;
+						vi = (r_minus ? -rr : rr) + (s_minus ? -ss : ss);
+					} else {
+						vr = acc_re[i][j][e];
+						vi = mode == 3 ? -acc_im[i][j][e] : acc_im[i][j][e];
+					}
 					if (accumulate) {
 						vr += pb.c_re[off];
 						vi += pb.c_im[off];
@@ -769,15 +832,21 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 		if (forced == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 		if (forced == 3) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 		// Expected matrix-pipe efficiency of each block shape for this problem.  The busiest compute unit works through
-		// ceil(blocks / units) blocks, so the launch costs that many block-times on every unit, whether or not all units have
-		// that many and whether or not a block on the edge of C is full: efficiency = real elements of C / elements paid for
-		// x the efficiency measured for the shape on full blocks with at least two workgroups per unit (two wavefronts per
-		// SIMD: one issues MFMAs while the other waits at its barrier), less a penalty where a unit gets a single block.
+		// p = ceil(blocks / units) blocks, so the launch costs p block-times on every unit, whether or not all units have that
+		// many and whether or not a block on the edge of C is full: efficiency = real elements of C / elements paid for x
+		// the efficiency measured for the shape at p blocks per unit on full blocks (fraction of the fp32 MFMA peak, lowest
+		// of three operand layouts, K = 2048).  The table carries what a formula would miss: a unit holds two workgroups
+		// of the larger shapes and three of 64 x 64, a lone workgroup cannot keep the matrix pipe busy, and with 3 or 5
+		// blocks of 128 x 128 per unit the hardware dispatcher leaves some units with one block more than the others.
 		struct Shape {
 			int bm, bn;
-			double eff;
+			float eff[8];  // p = 1 .. 8 (8 stands for everything above)
 		};
-		static const Shape shapes[4] = {{128, 128, 0.885}, {64, 128, 0.865}, {128, 64, 0.860}, {64, 64, 0.843}};
+		static const Shape shapes[4] = {
+				{128, 128, {0.858f, 0.934f, 0.707f, 0.936f, 0.784f, 0.938f, 0.800f, 0.939f}},
+				{64, 128, {0.853f, 0.920f, 0.909f, 0.926f, 0.923f, 0.930f, 0.931f, 0.932f}},
+				{128, 64, {0.862f, 0.932f, 0.917f, 0.939f, 0.928f, 0.941f, 0.942f, 0.943f}},
+				{64, 64, {0.825f, 0.910f, 0.929f, 0.926f, 0.936f, 0.940f, 0.941f, 0.943f}}};
 		int best = 3;
 		double best_score = -1.0;
 		for (int k = 0; k < 4; ++k) {
@@ -785,7 +854,7 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 			const long per_unit = (nb + cus - 1) / cus;
 			const double paid = (double) per_unit * cus * shapes[k].bm * shapes[k].bn;
 			const double real = (double) nb / ((double) ((a.M + shapes[k].bm - 1) / shapes[k].bm) * ((a.N + shapes[k].bn - 1) / shapes[k].bn)) * a.M * a.N;
-			const double score = shapes[k].eff * real / paid * (per_unit >= 2 ? 1.0 : 0.9);
+			const double score = shapes[k].eff[per_unit < 8 ? per_unit - 1 : 7] * real / paid;
 			if (score > best_score) {
 				best_score = score;
 				best = k;
