@@ -328,16 +328,19 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 		}
 	}
 
-	// ---- epilogue: accumulator element e of lane (r, h) is C[(e/4)*8 + h*4 + e%4][r] of its 32x32 tile
+	// ---- epilogue: accumulator element e of lane (r, h) is C[(e/4)*8 + h*4 + e%4][r] of its 32x32 tile.  The empty
+	// asm keeps the address arithmetic below the loop (hoisted above it, it is spilled).
+	int r_st = r, h_st = h;
+	asm volatile("" : "+v"(r_st), "+v"(h_st));
 #pragma unroll
 	for (int i = 0; i < TM; ++i)
 #pragma unroll
 		for (int j = 0; j < TN; ++j) {
-			const int col = n0 + wn0 + j * 32 + r;
+			const int col = n0 + wn0 + j * 32 + r_st;
 			if (col >= N) continue;
 #pragma unroll
 			for (int e = 0; e < 16; ++e) {
-				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
+				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h_st * 4 + (e & 3);
 				if (row < M) {
 					const long off = (long) row * ldc + col;
 					float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
@@ -699,16 +702,20 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 		}
 	}
 	const bool q_minus = mode == 0 || mode == 3, r_minus = (mode & 1) != 0, s_minus = (mode & 2) != 0;
+	// The addresses of the stores are formed here, after the loop: left to itself the compiler computes them before the
+	// loop, where the registers are full, and spills them.
+	int r_st = r, h_st = h;
+	asm volatile("" : "+v"(r_st), "+v"(h_st));
 
 #pragma unroll
 	for (int i = 0; i < TM; ++i)
 #pragma unroll
 		for (int j = 0; j < TN; ++j) {
-			const int col = n0 + wn0 + j * 32 + r;
+			const int col = n0 + wn0 + j * 32 + r_st;
 			if (col >= args.N) continue;  // blocks on the right and bottom edge of C are partly outside
 #pragma unroll
 			for (int e = 0; e < 16; ++e) {
-				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
+				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h_st * 4 + (e & 3);
 				if (row < args.M) {
 					const long off = (long) row * ldc + col;
 					float vr, vi;
@@ -854,7 +861,8 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 			const long per_unit = (nb + cus - 1) / cus;
 			const double paid = (double) per_unit * cus * shapes[k].bm * shapes[k].bn;
 			const double real = (double) nb / ((double) ((a.M + shapes[k].bm - 1) / shapes[k].bm) * ((a.N + shapes[k].bn - 1) / shapes[k].bn)) * a.M * a.N;
-			const double score = shapes[k].eff[per_unit < 8 ? per_unit - 1 : 7] * real / paid;
+			// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
+			const double score = shapes[k].eff[per_unit < 8 ? per_unit - 1 : 7] * real / paid * (1.0 + 0.000001 * shapes[k].bm * shapes[k].bn);
 			if (score > best_score) {
 				best_score = score;
 				best = k;
