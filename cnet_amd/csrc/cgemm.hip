@@ -597,7 +597,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	fb.fetch_set(0, 0);
 
 	// One chunk, held in stage `cur`.
-	auto chunk = [&](int cur, auto mode_c, int c) {
+	auto chunk = [&](int cur, auto mode_c, int c) __attribute__((always_inline)) {
 		constexpr int MODE = decltype(mode_c)::value;
 		const int nxt = cur + 1 == NST ? 0 : cur + 1, far = cur == 0 ? NST - 1 : cur - 1;
 		const int CUR = cur * STAGE_FLOATS, NXT = nxt * STAGE_FLOATS, FAR = far * STAGE_FLOATS;
@@ -683,12 +683,25 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			__builtin_amdgcn_sched_barrier(0);
 		}
 	};
-	// the chunks of this block: chunk c_lo + n sits in stage n % NST
-	auto kloop = [&](auto mode_c) {
-		int cur = 0;
-		for (int c = c_lo; c < c_hi; ++c) {
-			chunk(cur, mode_c, c);
-			cur = cur + 1 == NST ? 0 : cur + 1;
+	// the chunks of this block: chunk c_lo + n sits in stage n % NST.  The loop body is one round over the stages, so the
+	// stage part of every LDS address is an immediate (no address additions in the loop); what is left over after the
+	// last full round follows the loop.
+	auto kloop = [&](auto mode_c) __attribute__((always_inline)) {
+		int c = c_lo;
+		if constexpr (NST == 2) {
+			for (; c + 1 < c_hi; c += 2) {
+				chunk(0, mode_c, c);
+				chunk(1, mode_c, c + 1);
+			}
+			if (c < c_hi) chunk(0, mode_c, c);
+		} else {
+			for (; c + 2 < c_hi; c += 3) {
+				chunk(0, mode_c, c);
+				chunk(1, mode_c, c + 1);
+				chunk(2, mode_c, c + 2);
+			}
+			if (c < c_hi) chunk(0, mode_c, c);
+			if (c + 1 < c_hi) chunk(1, mode_c, c + 1);
 		}
 	};
 	if constexpr (ACC4) {
@@ -844,16 +857,17 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 		// the efficiency measured for the shape at p blocks per unit on full blocks (fraction of the fp32 MFMA peak, lowest
 		// of three operand layouts, K = 2048).  The table carries what a formula would miss: a unit holds two workgroups
 		// of the larger shapes and three of 64 x 64, a lone workgroup cannot keep the matrix pipe busy, and with 3 or 5
-		// blocks of 128 x 128 per unit the hardware dispatcher leaves some units with one block more than the others.
+		// blocks of 128 x 128 per unit, or 4 of 64 x 64, the hardware dispatcher leaves some units with one block more than
+		// the others.
 		struct Shape {
 			int bm, bn;
 			float eff[8];  // p = 1 .. 8 (8 stands for everything above)
 		};
 		static const Shape shapes[4] = {
-				{128, 128, {0.858f, 0.934f, 0.707f, 0.936f, 0.784f, 0.938f, 0.800f, 0.939f}},
-				{64, 128, {0.853f, 0.920f, 0.909f, 0.926f, 0.923f, 0.930f, 0.931f, 0.932f}},
-				{128, 64, {0.862f, 0.932f, 0.917f, 0.939f, 0.928f, 0.941f, 0.942f, 0.943f}},
-				{64, 64, {0.825f, 0.910f, 0.929f, 0.926f, 0.936f, 0.940f, 0.941f, 0.943f}}};
+				{128, 128, {0.887f, 0.946f, 0.713f, 0.941f, 0.794f, 0.946f, 0.800f, 0.948f}},
+				{64, 128, {0.883f, 0.935f, 0.931f, 0.943f, 0.938f, 0.943f, 0.943f, 0.944f}},
+				{128, 64, {0.892f, 0.940f, 0.936f, 0.945f, 0.945f, 0.948f, 0.949f, 0.950f}},
+				{64, 64, {0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}}};
 		int best = 3;
 		double best_score = -1.0;
 		for (int k = 0; k < 4; ++k) {
