@@ -182,3 +182,22 @@ def test_linear_headline_shape_rows_against_oracle(gpu, port):
         ops.linear_bwd_weight(gs, xs, acc, accumulate=k)
     full, parts = dw.host(), acc.host()
     assert rel_c(full[0:2], parts[0:2]) < 1e-5 and rel_c(full[2:4], parts[2:4]) < 1e-5
+
+
+@pytest.mark.parametrize("M,N,K,nb", [(8192, 1024, 64, 1), (192, 256, 48, 2), (4096, 512, 32, 1), (1024, 2048, 32, 1)])
+def test_cgemm_conjugate_combinations(gpu, port, M, N, K, nb):
+    """conj(A) and conj(B) in all four combinations, on shapes that take each block shape of the fast path: the signs are
+    applied when the block is stored (one- and two-tile wavefronts) or by the choice of the negated operand (four
+    tiles), and conj(A) conj(B) negates the imaginary plane on its way out."""
+    A = seeded(port, 21, (nb, M, K)) + 1j * seeded(port, 22, (nb, M, K))
+    Bm = seeded(port, 23, (K, N)) + 1j * seeded(port, 24, (K, N))
+    a = ops.CMat.from_host(np.ascontiguousarray(A.real).reshape(nb * M, K), np.ascontiguousarray(A.imag).reshape(nb * M, K))
+    b = ops.CMat.from_host(np.ascontiguousarray(Bm.real), np.ascontiguousarray(Bm.imag))
+    for conj_a in (0, 1):
+        for conj_b in (0, 1):
+            c = ops.CMat.empty(nb * M, N)
+            ops.cgemm_batched(a, M * K, b, 0, c, M * N, M, N, K, nb, a_kmajor=0, b_kmajor=1, conj_a=conj_a, conj_b=conj_b)
+            cr, ci = c.host()
+            want = (np.conj(A) if conj_a else A) @ (np.conj(Bm) if conj_b else Bm)
+            got = (cr + 1j * ci).reshape(nb, M, N)
+            assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-5, (conj_a, conj_b)
