@@ -201,3 +201,36 @@ def test_cgemm_conjugate_combinations(gpu, port, M, N, K, nb):
             want = (np.conj(A) if conj_a else A) @ (np.conj(Bm) if conj_b else Bm)
             got = (cr + 1j * ci).reshape(nb, M, N)
             assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-5, (conj_a, conj_b)
+
+
+def test_cgemm_random_shapes(gpu, port):
+    """Eighty seeded random problems across the paths of the GEMM: aligned and odd shapes, K with and without a whole
+    number of chunks, every layout, conj(B), accumulation, leading dimensions wider than the matrix, against numpy in
+    complex128."""
+    rs = np.random.RandomState(20240)
+    for case in range(80):
+        M = int(rs.choice([1, 3, 4, 7, 16, 60, 64, 68, 100, 128, 132, 200, 257, 384, 520]))
+        N = int(rs.choice([1, 2, 4, 10, 16, 36, 64, 72, 128, 196, 260, 512, 784]))
+        K = int(rs.choice([1, 2, 5, 16, 32, 48, 33, 64, 100, 128, 160, 784, 1024]))
+        a_km, b_km, cj, acc = int(rs.randint(2)), int(rs.randint(2)), int(rs.randint(2)), int(rs.randint(2))
+        pad_a, pad_b, pad_c = (int(rs.choice([0, 4, 8, 3])) for _ in range(3))
+        A = rs.randn(M, K) + 1j * rs.randn(M, K)
+        Bm = rs.randn(K, N) + 1j * rs.randn(K, N)
+        a_h = A.T if a_km else A
+        b_h = Bm if b_km else Bm.T
+        def wide(h, pad):  # the matrix sits in the first columns of a wider buffer
+            buf = np.zeros((h.shape[0], h.shape[1] + pad), np.complex64)
+            buf[:, :h.shape[1]] = h
+            full = ops.CMat.from_host(np.ascontiguousarray(buf.real), np.ascontiguousarray(buf.imag))
+            return full.sub(0, h.shape[1])
+        a, b = wide(a_h, pad_a), wide(b_h, pad_b)
+        c0 = (rs.randn(M, N + pad_c) + 1j * rs.randn(M, N + pad_c)).astype(np.complex64)
+        cfull = ops.CMat.from_host(np.ascontiguousarray(c0.real), np.ascontiguousarray(c0.imag))
+        ops.cgemm(a, b, cfull.sub(0, N), M, N, K, a_km, b_km, cj, accumulate=acc)
+        cr, ci = cfull.re.owner.download(), cfull.im.owner.download()
+        got = cr + 1j * ci
+        a32, b32 = A.astype(np.complex64).astype(np.complex128), Bm.astype(np.complex64).astype(np.complex128)
+        want = a32 @ (b32.conj() if cj else b32) + (c0[:, :N] if acc else 0)
+        err = np.linalg.norm(got[:, :N] - want) / max(np.linalg.norm(want), 1e-30)
+        assert err < 2e-5, (case, M, N, K, a_km, b_km, cj, acc, pad_a, pad_b, pad_c, err)
+        assert np.array_equal(got[:, N:], c0[:, N:]), (case, "columns beside C were touched")
