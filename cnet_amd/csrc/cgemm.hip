@@ -57,7 +57,27 @@ struct CgemmArgs {
 	// blockIdx.z = batch index * splits + split.
 	int splits, chunks_per_split;
 	float *partial;  // [split][problem][batch][re, im][M][N]
+	// Tail: when the blocks of C do not fill a whole number of rounds over the compute units, the blocks of the last,
+	// partly filled round ("tail blocks": the last tail_tiles of the nprob x tiles_m x tiles_n blocks) are cut into
+	// tail_splits pieces along K, tail_chunks chunks each.  The launch has one workgroup per block of the full rounds
+	// (problems share blockIdx.x); workgroup i < tail_tiles x tail_splits computes piece i as well, after its block, so
+	// every compute unit gets the same share of the tail wherever the hardware places the workgroups.  A piece writes its
+	// whole block to partial[tail block][piece][re, im][BM][BN]; tail_reduce_kernel adds the pieces in order.
+	int tail_tiles, tail_splits, tail_chunks, nprob;
 };
+
+// Which block of C (per problem) a linear block number stands for: walks groups of 8 block rows column by column, after
+// spreading consecutive workgroup numbers (which the hardware deals round-robin to the XCDs) over contiguous strips.
+__device__ __forceinline__ void map_block(const CgemmArgs &args, int pid, int grid_n, int &tile_m, int &tile_n) {
+	const int total = args.tiles_m * grid_n;
+	if (total % NUM_XCD == 0) pid = (pid % NUM_XCD) * (total / NUM_XCD) + pid / NUM_XCD;
+	constexpr int GROUP = 8;
+	const int width = GROUP * grid_n;
+	const int first_m = (pid / width) * GROUP;
+	const int gsize = min(args.tiles_m - first_m, GROUP);
+	tile_m = first_m + (pid % width) % gsize;
+	tile_n = (pid % width) / gsize;
+}
 
 // column blocks per grid row: with a triangular operand each workgroup handles a block and its mirror image
 __device__ __host__ __forceinline__ int grid_tiles_n(const CgemmArgs &args) { return args.tri ? (args.tiles_n + 1) / 2 : args.tiles_n; }
@@ -218,16 +238,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 	const int M = args.M, N = args.N, K = args.K;
 
 	// ---- which block of C
-	int pid = blockIdx.x;
 	const int grid_n = grid_tiles_n(args);
-	const int total = args.tiles_m * grid_n;
-	if (total % NUM_XCD == 0) pid = (pid % NUM_XCD) * (total / NUM_XCD) + pid / NUM_XCD;
-	constexpr int GROUP = 8;
-	const int width = GROUP * grid_n;
-	const int first_m = (pid / width) * GROUP;
-	const int gsize = min(args.tiles_m - first_m, GROUP);
-	const int tile_m = first_m + (pid % width) % gsize;
-	const int tile_n_first = (pid % width) / gsize;
+	int tile_m, tile_n_first;
+	map_block(args, blockIdx.x, grid_n, tile_m, tile_n_first);
 	const int m0 = tile_m * BM;
 	// a triangular operand: this workgroup takes column block j and then its mirror tiles_n - 1 - j, so that every
 	// workgroup walks the same number of K chunks in total
@@ -493,33 +506,24 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	constexpr bool SCHED_RECIPE = CNET_SCHED_RECIPE;
 	extern __shared__ float smem[];
 
-	CgemmProblem pb = args.p[blockIdx.y];
-	batch_offset(pb, args);
-	long ldc;
-	int accumulate;
-	output_planes(args, pb, ldc, accumulate);
-	const int K = args.K;
-
-	int pid = blockIdx.x;
 	const int grid_n = grid_tiles_n(args);
-	const int total = args.tiles_m * grid_n;
-	if (total % NUM_XCD == 0) pid = (pid % NUM_XCD) * (total / NUM_XCD) + pid / NUM_XCD;
-	constexpr int GROUP = 8;
-	const int width = GROUP * grid_n;
-	const int first_m = (pid / width) * GROUP;
-	const int gsize = min(args.tiles_m - first_m, GROUP);
-	const int tile_m = first_m + (pid % width) % gsize;
-	const int tile_n_first = (pid % width) / gsize;
-	const int m0 = tile_m * BM;
-	// a triangular operand: this workgroup takes column block j and then its mirror tiles_n - 1 - j, so that every
-	// workgroup walks the same number of K chunks in total
-	const int npass = (args.tri && tile_n_first != args.tiles_n - 1 - tile_n_first) ? 2 : 1;
-
+	const int total = args.tiles_m * grid_n;  // blocks of C per problem
+	const int K = args.K;
 	const int lane = threadIdx.x & 63;
 	const int wave = threadIdx.x >> 6;
 	const int wm0 = (wave / (BN / WN)) * WM;
 	const int wn0 = (wave % (BN / WN)) * WN;
 	const int r = lane & 31, h = lane >> 5;
+
+	// Work of this workgroup: one block of C; with a triangular operand the mirrored column block j -> tiles_n - 1 - j
+	// as a second pass (every workgroup then walks the same number of K chunks in total); with tail blocks (see
+	// CgemmArgs) the first tail_tiles x tail_splits workgroups also compute one K piece of a tail block as a second
+	// pass: every workgroup of the launch has the same amount of work, wherever the hardware places it.
+	int tile_m_first = 0, tile_n_first = 0;
+	if (!args.tail_tiles) map_block(args, blockIdx.x, grid_n, tile_m_first, tile_n_first);
+	int npass = 1;
+	if (args.tri && tile_n_first != args.tiles_n - 1 - tile_n_first) npass = 2;
+	if (args.tail_tiles && (int) blockIdx.x < args.tail_tiles * args.tail_splits) npass = 2;
 
 	// Accumulators.  A wavefront with one or two tiles keeps the four real products apart (P = Ar Br, R = Ar Bi, Q = Ai Bi,
 	// S = Ai Br) and combines them with their signs when it stores, so its K loop has no vector-ALU instruction for signs at
@@ -528,8 +532,24 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	constexpr bool ACC4 = TM * TN <= 2;
 	floatx16 acc_re[TM][TN], acc_im[TM][TN], acc_q[ACC4 ? TM : 1][ACC4 ? TN : 1], acc_s[ACC4 ? TM : 1][ACC4 ? TN : 1];
 	for (int pass = 0; pass < npass; ++pass) {
-	const int tile_n = pass ? args.tiles_n - 1 - tile_n_first : tile_n_first;
-	const int n0 = tile_n * BN;
+	int prob = blockIdx.y, tile_m = tile_m_first, tile_n = pass ? args.tiles_n - 1 - tile_n_first : tile_n_first;
+	int piece = -1, tail_block = 0;  // piece >= 0: this pass computes one K piece of a tail block
+	if (args.tail_tiles) {
+		int w = blockIdx.x;
+		if (pass) {
+			tail_block = blockIdx.x / args.tail_splits;
+			piece = blockIdx.x - tail_block * args.tail_splits;
+			w = total * args.nprob - args.tail_tiles + tail_block;
+		}
+		prob = w / total;
+		map_block(args, w - prob * total, grid_n, tile_m, tile_n);
+	}
+	CgemmProblem pb = args.p[prob];
+	batch_offset(pb, args);
+	long ldc;
+	int accumulate;
+	output_planes(args, pb, ldc, accumulate);
+	const int m0 = tile_m * BM, n0 = tile_n * BN;
 	if (pass) __syncthreads();  // every wave has finished reading the last stage of the previous block
 #pragma unroll
 	for (int i = 0; i < TM; ++i)
@@ -558,6 +578,17 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	const long b_step = B_NCONTIG ? (long) KC * args.ldb : (long) KC;
 	int c_lo, c_hi;
 	chunk_range<BN>(args, n0, c_lo, c_hi);
+	int row_org = 0, col_org = 0;  // what the stores subtract from (row, col): a piece writes block-local coordinates
+	if (piece >= 0) {
+		c_lo = piece * args.tail_chunks;
+		c_hi = min(c_hi, c_lo + args.tail_chunks);
+		pb.c_re = args.partial + ((long) (tail_block * args.tail_splits + piece) * 2) * (BM * BN);
+		pb.c_im = pb.c_re + BM * BN;
+		ldc = BN;
+		accumulate = 0;
+		row_org = m0;
+		col_org = n0;
+	}
 
 	// all units of one chunk of both operands into the stage at `stage`
 	auto issue_chunk = [&](int chunk, float *stage) {
@@ -730,7 +761,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			for (int e = 0; e < 16; ++e) {
 				const int row = m0 + wm0 + i * 32 + (e >> 2) * 8 + h_st * 4 + (e & 3);
 				if (row < args.M) {
-					const long off = (long) row * ldc + col;
+					const long off = (long) (row - row_org) * ldc + (col - col_org);
 					float vr, vi;
 					if constexpr (ACC4) {
 						const float q = acc_q[i][j][e], rr = acc_im[i][j][e], ss = acc_s[i][j][e];
@@ -767,11 +798,37 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(CgemmArgs args, int 
 	*c = args.accumulate ? *c + v : v;
 }
 
+// C (+)= sum over the K pieces of each tail block, added in piece order.  blockIdx.x = tail block, blockIdx.y = a slice
+// of its two planes.
+template <int BM, int BN>
+__global__ __launch_bounds__(256) void tail_reduce_kernel(CgemmArgs args) {
+	const int grid_n = grid_tiles_n(args);
+	const int total = args.tiles_m * grid_n;
+	const int w = total * args.nprob - args.tail_tiles + blockIdx.x;
+	const int prob = w / total;
+	int tile_m, tile_n;
+	map_block(args, w - prob * total, grid_n, tile_m, tile_n);
+	const int m0 = tile_m * BM, n0 = tile_n * BN;
+	const float *first = args.partial + ((long) blockIdx.x * args.tail_splits * 2) * (BM * BN);
+	// blockIdx.y = which 1024 of the 2 x BM x BN values of the block
+	for (int idx = blockIdx.y * 1024 + threadIdx.x; idx < (int) (blockIdx.y + 1) * 1024; idx += 256) {
+		const int part = idx / (BM * BN), e = idx - part * (BM * BN);
+		const int row = m0 + e / BN, col = n0 + e % BN;
+		if (row >= args.M || col >= args.N) continue;
+		const float v = cnet::ordered_sum(first + idx, 2L * BM * BN, args.tail_splits);
+		float *c = (part ? args.p[prob].c_im : args.p[prob].c_re) + (long) row * args.ldc + col;
+		*c = args.accumulate ? *c + v : v;
+	}
+}
+
+// tail_splits >= 2: cut the blocks of the last, partly filled round into that many pieces along K (see CgemmArgs)
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
-int launch(const CgemmArgs &proto, int nprob, int batch) {
+int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0) {
 	CgemmArgs args = proto;
 	args.tiles_m = (args.M + BM - 1) / BM;
 	args.tiles_n = (args.N + BN - 1) / BN;
+	args.nprob = nprob;
+	args.tail_tiles = args.tail_splits = args.tail_chunks = 0;
 	constexpr size_t smem = 2 * (size_t) (2 * KC * (BM + 4) + 2 * KC * (BN + 4)) * sizeof(float);
 	// A grid that leaves most compute units idle while each workgroup walks a long K (a small batch against a long
 	// reduction: every chunk then waits a full memory latency) is cut along K.
@@ -794,7 +851,25 @@ int launch(const CgemmArgs &proto, int nprob, int batch) {
 		}
 	}
 	dim3 grid(args.tiles_m * grid_tiles_n(args), nprob, batch * args.splits);
+	if (tail_splits >= 2 && VEC == 4 && args.K % KC == 0 && !args.tri && batch == 1 && args.splits == 1) {
+		const long cus = cnet::rt().prop.multiProcessorCount;
+		const long all = (long) args.tiles_m * args.tiles_n * nprob;
+		const int nchunks = args.K / KC;
+		const int r = (int) (all % cus);
+		if (all > cus && r > 0 && (long) r * tail_splits <= all - r) {
+			args.tail_chunks = (nchunks + tail_splits - 1) / tail_splits;
+			args.tail_splits = (nchunks + args.tail_chunks - 1) / args.tail_chunks;  // no empty piece
+			args.tail_tiles = r;
+			args.partial = (float *) cnet::workspace((size_t) r * args.tail_splits * 2 * BM * BN * sizeof(float));
+			if (!args.partial) return CNET_ERR_OUT_OF_MEMORY;
+			grid = dim3((unsigned) (all - r), 1, 1);  // one workgroup per full block; the first r x s also do a piece
+		}
+	}
 	auto finish = [&]() -> int {
+		if (args.tail_tiles) {
+			hipLaunchKernelGGL((tail_reduce_kernel<BM, BN>), dim3(args.tail_tiles, 2 * BM * BN / 1024), dim3(256), 0, cnet::rt().stream, args);
+			CNET_LAUNCH_CHECK();
+		}
 		if (args.splits > 1) {
 			dim3 rgrid((unsigned) ((2L * args.M * args.N + 255) / 256), nprob, batch);
 			hipLaunchKernelGGL(splitk_reduce_kernel, rgrid, dim3(256), 0, cnet::rt().stream, args, nprob, batch);
@@ -847,18 +922,21 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 			const char *e = getenv("CNET_CGEMM_TILE");
 			return e ? atoi(e) : -1;
 		}();
-		if (forced == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-		if (forced == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-		if (forced == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-		if (forced == 3) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-		// Expected matrix-pipe efficiency of each block shape for this problem.  The busiest compute unit works through
-		// p = ceil(blocks / units) blocks, so the launch costs p block-times on every unit, whether or not all units have that
-		// many and whether or not a block on the edge of C is full: efficiency = real elements of C / elements paid for x
-		// the efficiency measured for the shape at p blocks per unit on full blocks (fraction of the fp32 MFMA peak, lowest
-		// of three operand layouts, K = 2048).  The table carries what a formula would miss: a unit holds two workgroups
-		// of the larger shapes and three of 64 x 64, a lone workgroup cannot keep the matrix pipe busy, and with 3 or 5
-		// blocks of 128 x 128 per unit, or 4 of 64 x 64, the hardware dispatcher leaves some units with one block more than
-		// the others.
+		// CNET_CGEMM_TAIL = 0 / 1: never / whenever possible cut the blocks of a partly filled last round along K
+		static const int forced_tail = [] {
+			const char *e = getenv("CNET_CGEMM_TAIL");
+			return e ? atoi(e) : -1;
+		}();
+		// Expected duration of the launch with each block shape.  The busiest compute unit works through p = ceil(blocks /
+		// units) blocks, so the launch takes p block-times, whether or not all units have that many and whether or not a
+		// block on the edge of C is full, divided by the efficiency measured for the shape at p blocks per unit on full
+		// blocks (fraction of the fp32 MFMA peak, lowest of three operand layouts, K = 2048).  The table carries what a
+		// formula would miss: a unit holds two workgroups of the larger shapes and three of 64 x 64, a lone workgroup
+		// cannot keep the matrix pipe busy, and with 3 or 5 blocks of 128 x 128 per unit, or 4 of 64 x 64, the hardware
+		// dispatcher leaves some units with one block more than the others.
+		// Alternative for a partly filled last round (q full rounds, r blocks left over): cut those r blocks into s pieces
+		// along K, one piece for each workgroup of the full rounds.  Then the launch takes q block-times plus 1/s of one,
+		// plus the fixed cost of a short piece and of the kernel that adds the pieces.
 		struct Shape {
 			int bm, bn;
 			float eff[8];  // p = 1 .. 8 (8 stands for everything above)
@@ -868,24 +946,43 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 				{64, 128, {0.883f, 0.935f, 0.931f, 0.943f, 0.938f, 0.943f, 0.943f, 0.944f}},
 				{128, 64, {0.892f, 0.940f, 0.936f, 0.945f, 0.945f, 0.948f, 0.949f, 0.950f}},
 				{64, 64, {0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}}};
-		int best = 3;
-		double best_score = -1.0;
+		const double flop_per_us_per_unit = 256.0 * 2.4e3;  // 256 flop per clock at 2.4 GHz
+		const int nchunks = (a.K + KC - 1) / KC;
+		const bool tail_possible = forced_tail != 0 && a.K % KC == 0 && !a.tri && batch == 1;
+		int best = 3, best_tail = 0;
+		double best_us = 1e30;
 		for (int k = 0; k < 4; ++k) {
+			if (forced >= 0 && forced != k) continue;
 			const long nb = blocks(shapes[k].bm, shapes[k].bn);
 			const long per_unit = (nb + cus - 1) / cus;
-			const double paid = (double) per_unit * cus * shapes[k].bm * shapes[k].bn;
-			const double real = (double) nb / ((double) ((a.M + shapes[k].bm - 1) / shapes[k].bm) * ((a.N + shapes[k].bn - 1) / shapes[k].bn)) * a.M * a.N;
+			const double block_us = 8.0 * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
 			// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
-			const double score = shapes[k].eff[per_unit < 8 ? per_unit - 1 : 7] * real / paid * (1.0 + 0.000001 * shapes[k].bm * shapes[k].bn);
-			if (score > best_score) {
-				best_score = score;
+			const double bonus = 1.0 - 0.000001 * shapes[k].bm * shapes[k].bn;
+			double us = per_unit * block_us / shapes[k].eff[per_unit < 8 ? per_unit - 1 : 7] * bonus;
+			int tail = 0;
+			const long q = nb / cus, r = nb % cus;
+			if (tail_possible && q >= 1 && r > 0) {
+				// as many pieces as there are workgroups in the full rounds, so that each of them gets one; a piece is at
+				// least three chunks long
+				const int s = (int) std::min<long>(q * cus / r, nchunks / 3);
+				if (s >= 2) {
+					const double tail_us = (q * block_us / shapes[k].eff[q < 8 ? q - 1 : 7] + block_us / s / 0.8 + 20.0) * bonus;
+					if (tail_us < us || forced_tail == 1) {
+						us = tail_us;
+						tail = s;
+					}
+				}
+			}
+			if (us < best_us) {
+				best_us = us;
 				best = k;
+				best_tail = tail;
 			}
 		}
-		if (best == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-		if (best == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-		if (best == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
-		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
+		if (best == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
+		if (best == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
+		if (best == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
+		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
 	}
 }
 

@@ -234,3 +234,18 @@ def test_cgemm_random_shapes(gpu, port):
         err = np.linalg.norm(got[:, :N] - want) / max(np.linalg.norm(want), 1e-30)
         assert err < 2e-5, (case, M, N, K, a_km, b_km, cj, acc, pad_a, pad_b, pad_c, err)
         assert np.array_equal(got[:, N:], c0[:, N:]), (case, "columns beside C were touched")
+
+
+@pytest.mark.parametrize("tile", ["0", "1", "2", "3", ""])
+def test_cgemm_tail_blocks_cut_along_k(gpu, tile):
+    """Products whose blocks do not fill a whole number of rounds over the compute units, with the cut of the last round's
+    blocks along K switched on for every such launch and each block shape in turn (and the library's own choice)."""
+    import os
+    import subprocess
+    import sys
+    env = dict(os.environ, CNET_CGEMM_TAIL="1")
+    if tile:
+        env["CNET_CGEMM_TILE"] = tile
+    script = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gpu_tail_blocks_check.py")
+    r = subprocess.run([sys.executable, script], env=env, capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0 and "OK" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
