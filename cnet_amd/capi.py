@@ -74,6 +74,7 @@ SIGNATURES = {
     "cnet_l2out_bwd": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_copy2d": [c_fp, _l, c_fp, _l, _i, _i],
     "cnet_add2d": [c_fp, _l, c_fp, _l, _i, _i],
+    "cnet_add_multi": [_i, C.c_void_p, C.c_void_p, C.c_void_p],
     "cnet_batch_sum": [c_fp, _l, c_fp, _i, _i, _i],
     "cnet_sgd_update": [c_fp, c_fp, c_fp, c_fp, _l, C.c_float, _i],
     "cnet_sgd_update_multi": [_i, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, _i],

@@ -534,6 +534,32 @@ __global__ __launch_bounds__(TPB) void sgd_multi_kernel(SgdMulti t, float lr, in
 	}
 }
 
+// dst[k][i] += src[k][i] for up to SGD_MULTI_MAX dense arrays in one launch (blockIdx.y selects the array).
+struct AddMulti {
+	const float *src[SGD_MULTI_MAX];
+	float *dst[SGD_MULTI_MAX];
+	long n[SGD_MULTI_MAX];
+	int vec[SGD_MULTI_MAX];
+};
+__global__ __launch_bounds__(TPB) void add_multi_kernel(AddMulti t) {
+	const int k = blockIdx.y;
+	const long n = t.n[k];
+	const float *src = t.src[k];
+	float *dst = t.dst[k];
+	const long i0 = ((long) blockIdx.x * TPB + threadIdx.x) * 4;
+	if (i0 >= n) return;
+	if (t.vec[k]) {
+		float a[4], b[4];
+		ldv<4, false>(a, src + i0);
+		ldv<4, false>(b, dst + i0);
+#pragma unroll
+		for (int q = 0; q < 4; ++q) b[q] += a[q];
+		stv<4, false>(dst + i0, b);
+	} else {
+		for (long i = i0; i < i0 + 4 && i < n; ++i) dst[i] += src[i];
+	}
+}
+
 __global__ __launch_bounds__(TPB) void zero_kernel(uint4 *__restrict__ p16, long n16, unsigned char *__restrict__ tail, int ntail) {
 	const long i = (long) blockIdx.x * TPB + threadIdx.x;
 	if (i < n16) p16[i] = make_uint4(0, 0, 0, 0);
@@ -821,6 +847,32 @@ int cnet_copy2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows
 
 int cnet_add2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols) {
 	return copy_or_add(src, lds, dst, ldd, rows, cols, 1);
+}
+
+int cnet_add_multi(int count, const float *const *src, float *const *dst, const int64_t *n) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(count >= 0);
+	if (!count) return CNET_OK;
+	CNET_CHECK_ARG(src && dst && n);
+	for (int k = 0; k < count; ++k) CNET_CHECK_ARG(n[k] >= 0 && (n[k] == 0 || (src[k] && dst[k])));
+	for (int first = 0; first < count; first += SGD_MULTI_MAX) {
+		AddMulti t;
+		int used = 0;
+		long longest = 0;
+		for (int k = first; k < count && k < first + SGD_MULTI_MAX; ++k) {
+			if (!n[k]) continue;
+			t.src[used] = src[k];
+			t.dst[used] = dst[k];
+			t.n[used] = (long) n[k];
+			t.vec[used] = n[k] % 4 == 0 && all_aligned({src[k], dst[k]});
+			longest = std::max(longest, (long) n[k]);
+			++used;
+		}
+		if (!used) continue;
+		hipLaunchKernelGGL(add_multi_kernel, dim3(nblocks((longest + 3) / 4), used), dim3(TPB), 0, rt().stream, t);
+		CNET_LAUNCH_CHECK();
+	}
+	return CNET_OK;
 }
 
 int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int64_t n, float lr, int zero_grad) {

@@ -621,6 +621,17 @@ class CNet {
 	};
 	StepGraphs graphs_[2];
 	bool use_graphs_ = false;
+	std::vector<const float *> gather_src_;  // pending dz* gathers of the input functions (see nodeBackward)
+	std::vector<float *> gather_dst_;
+	std::vector<int64_t> gather_len_;
+	void flushGathers() {
+		if (gather_src_.empty()) return;
+		const int rc = cnet_add_multi((int) gather_src_.size(), gather_src_.data(), gather_dst_.data(), gather_len_.data());
+		gather_src_.clear();
+		gather_dst_.clear();
+		gather_len_.clear();
+		ck(rc, "cnet_add_multi");
+	}
 	SimpleRand rand_{(uint64_t) clock()};  // upstream ComplexNet::rand_ (impl/cnet.h:56): the coin of sample()
 	bool input_dz_dirty_ = false;  // the dz planes of the input functions hold a first moment
 	bool warmed_[3] = {false, false, false};  // phase has run once since useGraphs(true)
@@ -1020,17 +1031,16 @@ private:
 			return;
 		}
 		if (t == isInput) {  // impl/cinput.h:54-65: gathers dzs only, and keeps adding until the next update
+			// Both dz* planes of a consumer's slot are adjacent and dense, as they are in the node's own block: one array per
+			// consumer.  Nothing in the backward pass reads what an input function gathers, so the gathers of all of them
+			// wait for the end of the pass and go out as one launch (flushGathers).
 			CFunc::Slot &own = f->slots_[0];
 			for (int c = 0; c < f->no_outputs(); ++c) {
 				CFunc::Slot &u = upstream(f, c);
-				// both dz* planes in one launch: they are adjacent and dense in the consumer's slot and in the node's own block
-				const int64_t both = 2 * (int64_t) own.rows * own.len;
-				if (both <= INT32_MAX) {
-					ck(cnet_add2d(u.g(2), both, own.g(2), both, 1, (int) both), "cnet_add2d");
-				} else {
-					ck(cnet_add2d(u.g(2), u.len, own.g(2), own.len, own.rows, own.len), "cnet_add2d");
-					ck(cnet_add2d(u.g(3), u.len, own.g(3), own.len, own.rows, own.len), "cnet_add2d");
-				}
+				if (c) flushGathers();  // one launch must not hold two additions into the same planes
+				gather_src_.push_back(u.g(2));
+				gather_dst_.push_back(own.g(2));
+				gather_len_.push_back(2 * (int64_t) own.rows * own.len);
 			}
 			return;
 		}
@@ -1319,7 +1329,11 @@ public:
 	bool gpuBackward() {
 		requireAllocated("gpuBackward");
 		runPhase(1, graphs_[active_].bwd, [&] {
+			gather_src_.clear();  // nothing is left over from a pass that threw
+			gather_dst_.clear();
+			gather_len_.clear();
 			for (int k = (int) func_list_.size() - 1; k >= 0; --k) nodeBackward(func_list_[k], true);
+			flushGathers();
 		});
 		return true;
 	}
@@ -1499,7 +1513,11 @@ public:
 		// the device-side loss, which is refreshed here so getLoss() matches the label in use
 		for (auto f : outputs_)
 			if (f->typeId() == isCrossEntropy) nodeForward(f);
+		gather_src_.clear();
+		gather_dst_.clear();
+		gather_len_.clear();
 		for (int k = (int) func_list_.size() - 1; k >= 0; --k) nodeBackward(func_list_[k], label >= 0);
+		flushGathers();
 		fetchAll(0);
 	}
 	void backward() { backward(-1); }

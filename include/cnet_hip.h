@@ -247,6 +247,10 @@ int cnet_l2out_bwd(const float *z_re, const float *z_im, int64_t ldz,
 int cnet_copy2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols);       /* one plane */
 int cnet_add2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols);        /* dst += src */
 int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate); /* dst[c] (+)= sum_r src[r][c] */
+/* dst[k][0..n[k]) += src[k][0..n[k]) for `count` dense arrays in one launch: what the loop over the input functions in
+ * GpuNet::GpuBackward becomes (each CInput gathers the dz* of its consumer, impl/cinput.h:54-65, gpu/kernels.cpp:118-143).
+ * The destinations of one call must not overlap (the additions of a call run concurrently). */
+int cnet_add_multi(int count, const float *const *src, float *const *dst, const int64_t *n);
 /* z -= lr * dzs ; then dzs = 0 when zero_grad != 0   (impl/cfunc.h:147-152 + impl/cnet.h:413-421) */
 int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int64_t n, float lr, int zero_grad);
 

@@ -145,3 +145,22 @@ def test_sgd_update_of_several_tensors_in_one_launch(gpu, port):
         assert np.array_equal(d[0].host(), d2[0].host()) and np.array_equal(d[1].host(), d2[1].host()), n
         if n:
             assert not d[0].host()[0, :n].any()
+
+
+def test_add_of_several_arrays_in_one_launch(gpu, port):
+    """cnet_add_multi: dst += src for a list of dense arrays (the gathers of all input functions of a net), odd lengths,
+    empty entries and more entries than one launch takes included."""
+    import ctypes as C
+    sizes = [15680, 1568, 1, 0, 100003, 64, 4096, 12, 999, 50000, 8]
+    srcs, dsts, want = [], [], []
+    for k, n in enumerate(sizes):
+        m = max(n, 1)
+        a, b = seeded(port, 30 + 2 * k, (1, m)), seeded(port, 31 + 2 * k, (1, m))
+        srcs.append(ops.Plane.from_host(a)); dsts.append(ops.Plane.from_host(b))
+        w = b.copy(); w[0, :n] += a[0, :n]
+        want.append(w)
+    arr = lambda ptrs: (C.c_void_p * len(ptrs))(*ptrs)
+    lens = (C.c_int64 * len(sizes))(*sizes)
+    capi.call("cnet_add_multi", len(sizes), arr([p.ptr for p in srcs]), arr([p.ptr for p in dsts]), lens)
+    for n, d, w in zip(sizes, dsts, want):
+        assert np.array_equal(d.host(), w), n
