@@ -23,7 +23,7 @@ PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X published dense fp32 matrix peak
 # Bytes the eight L2s exchanged with the fabric per launch (FETCH_SIZE + WRITE_SIZE of `rocprofv3 --pmc`, each scaled by
 # what the same counter reads for a 256 MiB copy kernel: x2.000 and x1.000); an upper bound on HBM traffic, since hits
 # in the memory-side cache are included.  Source: profiles/cgemm_linear_b4096_1024x1024_counters.md.
-MEASURED_TRAFFIC_BYTES = {"linear_fwd": 197392749, "linear_bwd_input": 235260279, "linear_bwd_weight": 417968754}
+MEASURED_TRAFFIC_BYTES = {"linear_fwd": 197399783, "linear_bwd_input": 235300390, "linear_bwd_weight": 417957585}
 B, K, N = 4096, 1024, 1024      # BASELINE.json configs[1]
 
 
