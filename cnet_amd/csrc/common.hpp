@@ -35,6 +35,12 @@ struct Runtime {
 	// for the same size)
 	void *workspace = nullptr;
 	size_t workspace_bytes = 0;
+	// A recorded graph holds the workspace address it was recorded with: while any recording exists, a workspace that
+	// has to grow is retired (kept until shutdown) instead of freed.
+	int graphs_alive = 0;
+	static constexpr int kRetired = 16;
+	void *retired[kRetired] = {};
+	int retired_count = 0;
 };
 
 Runtime &rt();

@@ -33,9 +33,17 @@ void *workspace(size_t bytes) {
 		return nullptr;
 	}
 	if (r.workspace) {
-		// queued kernels may still read the old buffer
-		hipStreamSynchronize(r.stream);
-		hipFree(r.workspace);
+		if (r.graphs_alive > 0) {  // a recording may replay kernels that use the old buffer
+			if (r.retired_count == Runtime::kRetired) {
+				fail(CNET_ERR_UNSUPPORTED, "the workspace had to grow %d times while recorded graphs exist: destroy the graphs first", Runtime::kRetired);
+				return nullptr;
+			}
+			r.retired[r.retired_count++] = r.workspace;
+		} else {
+			// queued kernels may still read the old buffer
+			hipStreamSynchronize(r.stream);
+			hipFree(r.workspace);
+		}
 		r.workspace = nullptr;
 		r.workspace_bytes = 0;
 	}
@@ -124,6 +132,9 @@ int cnet_shutdown(void) {
 	if (r.workspace) hipFree(r.workspace);
 	r.workspace = nullptr;
 	r.workspace_bytes = 0;
+	for (int k = 0; k < r.retired_count; ++k) hipFree(r.retired[k]);
+	r.retired_count = 0;
+	r.graphs_alive = 0;
 	destroy_streams(r);
 	r.capturing = false;
 	r.ready = false;
@@ -338,6 +349,7 @@ int cnet_graph_end(void **graph_exec) {
 	(void) hipGraphDestroy(graph);
 	if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
 	*graph_exec = exec;
+	r.graphs_alive++;
 	return CNET_OK;
 }
 
@@ -354,6 +366,7 @@ int cnet_graph_destroy(void *graph_exec) {
 	if (!graph_exec) return CNET_OK;
 	CNET_HIP(hipStreamSynchronize(rt().stream));
 	CNET_HIP(hipGraphExecDestroy((hipGraphExec_t) graph_exec));
+	if (rt().graphs_alive > 0) rt().graphs_alive--;
 	return CNET_OK;
 }
 

@@ -97,7 +97,8 @@ int cnet_copy_wait(int64_t ticket);
  *      Entry points that allocate, wait or order the two streams (cnet_alloc, cnet_free, cnet_sync, the blocking copies,
  *      the marker / wait calls of the upload stream, the first use of a DFT length or of a larger workspace) return CNET_ERR_UNSUPPORTED while recording, and cnet_graph_end then fails:
  *      run the sequence once before recording it.  Clearing memory inside a recording uses a fill kernel
- *      (cnet_memset_zero), never a memset node. */
+ *      (cnet_memset_zero), never a memset node.  While a recording exists, a library workspace that has to grow for a
+ *      later call is kept instead of freed, so the recording stays valid. */
 int cnet_graph_begin(void);
 int cnet_graph_end(void **graph_exec);      /* NULL: drop the recording */
 int cnet_graph_launch(void *graph_exec);

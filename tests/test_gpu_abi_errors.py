@@ -138,3 +138,33 @@ def test_out_of_range_labels_and_token_ids_touch_nothing_outside_their_operands(
     d_re, d_im = ops.Plane.empty(V, D), ops.Plane.empty(V, D)
     ops.embedding_bwd(ops.ints(tok), ops.Plane.from_host(gs[0]), ops.Plane.from_host(gs[1]), d_re, d_im, D, V, 2, T)
     assert np.array_equal(d_re.host(), dsr) and np.array_equal(d_im.host(), dsi)
+
+
+def test_recorded_graph_survives_growth_of_the_workspace(gpu, port):
+    """A recording holds the address of the library workspace it was made with (here: the partial blocks of a product
+    that is cut along K).  A later, larger request makes the workspace grow; the old one must stay alive for the replay."""
+    M, N, K = 8, 24, 2048
+    A = seeded(port, 41, (M, K)) + 1j * seeded(port, 42, (M, K))
+    Bm = seeded(port, 43, (K, N)) + 1j * seeded(port, 44, (K, N))
+    a = ops.CMat.from_host(np.ascontiguousarray(A.real), np.ascontiguousarray(A.imag))
+    b = ops.CMat.from_host(np.ascontiguousarray(Bm.real), np.ascontiguousarray(Bm.imag))
+    c = ops.CMat.empty(M, N)
+    ops.cgemm(a, b, c, M, N, K, 0, 1)      # eager: sizes the workspace for this product
+    eager = c.host()
+    capi.call("cnet_graph_begin")
+    ops.cgemm(a, b, c, M, N, K, 0, 1)
+    exe = C.c_void_p()
+    capi.call("cnet_graph_end", C.byref(exe))
+    # a much larger cut product: the workspace has to grow
+    M2, N2, K2 = 128, 512, 8192
+    a2, b2, c2 = ops.CMat.empty(M2, K2, zero=True), ops.CMat.empty(K2, N2, zero=True), ops.CMat.empty(M2, N2)
+    ops.cgemm(a2, b2, c2, M2, N2, K2, 0, 1)
+    capi.sync()
+    for _ in range(2):
+        c.re.owner.zero(); c.im.owner.zero()
+        capi.call("cnet_graph_launch", exe)
+        got = c.host()
+        assert np.array_equal(got[0], eager[0]) and np.array_equal(got[1], eager[1])
+        ops.cgemm(a2, b2, c2, M2, N2, K2, 0, 1)   # eager work on the new workspace in between
+        capi.sync()
+    capi.call("cnet_graph_destroy", exe)
