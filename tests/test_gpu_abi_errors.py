@@ -168,3 +168,14 @@ def test_recorded_graph_survives_growth_of_the_workspace(gpu, port):
         ops.cgemm(a2, b2, c2, M2, N2, K2, 0, 1)   # eager work on the new workspace in between
         capi.sync()
     capi.call("cnet_graph_destroy", exe)
+
+
+def test_init_shutdown_init(gpu):
+    """Lifetime of the library in a process of its own: nothing works before cnet_init or after cnet_shutdown (a status,
+    not a crash), shutdown is idempotent, and a second initialisation gives the same results as the first."""
+    import os
+    import subprocess
+    import sys
+    script = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gpu_lifecycle_check.py")
+    r = subprocess.run([sys.executable, script], capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0 and "OK" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
