@@ -179,3 +179,51 @@ def test_init_shutdown_init(gpu):
     script = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gpu_lifecycle_check.py")
     r = subprocess.run([sys.executable, script], capture_output=True, text=True, timeout=280)
     assert r.returncode == 0 and "OK" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
+def test_device_copy_caller_stream_and_upload_ordering(gpu, port):
+    """cnet_memcpy_d2d, cnet_set_stream (the library launches on a stream the caller owns, here one made with
+    hipStreamCreate through the HIP runtime the library itself is linked against) and cnet_upload_wait_compute (an upload
+    that must not overtake the kernels queued before it)."""
+    hip = C.CDLL("libamdhip64.so")
+    src = capi.to_device(seeded(port, 51, (33, 17)))
+    dst = capi.zeros((33, 17))
+    capi.call("cnet_memcpy_d2d", dst.ptr, src.ptr, src.nbytes)
+    capi.sync()
+    assert np.array_equal(dst.download(), src.download())
+
+    xr, xi = seeded(port, 52, (40, 64)), seeded(port, 53, (40, 64))
+    x, y = ops.CMat.from_host(xr, xi), ops.CMat.empty(40, 64)
+    ops.gelu_fwd(x, y)
+    want = y.host()
+    own = capi.load().cnet_stream()
+    ts = C.c_void_p()
+    assert hip.hipStreamCreate(C.byref(ts)) == 0
+    capi.call("cnet_set_stream", ts)
+    assert capi.load().cnet_stream() == ts.value
+    y2 = ops.CMat.empty(40, 64)
+    ops.gelu_fwd(x, y2)
+    assert hip.hipStreamSynchronize(ts) == 0   # the caller's own wait is enough: the kernel ran on its stream
+    got = y2.host()
+    capi.call("cnet_set_stream", None)     # back to the library's stream
+    assert capi.load().cnet_stream() == own
+    assert hip.hipStreamDestroy(ts) == 0
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+
+    # upload stream held back behind the compute stream: the kernel reads the old contents, then the upload lands
+    n = 1 << 20
+    host = C.c_void_p()
+    capi.call("cnet_host_alloc", 4 * n, C.byref(host))
+    pinned = np.ctypeslib.as_array((C.c_float * n).from_address(host.value))
+    pinned[:] = 7.0
+    a = capi.to_device(np.ones(n, np.float32))
+    b = capi.zeros((n,))
+    for _ in range(20):                    # some queued work in front
+        capi.call("cnet_copy2d", a.ptr, n, b.ptr, n, 1, n)
+    capi.call("cnet_upload_wait_compute")
+    capi.call("cnet_upload_async", a.ptr, host, 4 * n)
+    capi.call("cnet_upload_sync")
+    capi.sync()
+    assert (b.download() == 1.0).all() and (a.download() == 7.0).all()
+    del pinned
+    capi.call("cnet_host_free", host)
