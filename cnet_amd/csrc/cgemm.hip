@@ -371,7 +371,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 
 
 // ---------------------------------------------------------------------------------------------------------------
-// Fast path: K % KC == 0, 128-bit aligned operands with shapes that are multiples of 4 (any number of blocks).  Same decomposition as cgemm_kernel,
+// Fast path: K % KC == 0, 128-bit aligned operands whose contiguous extents and leading dimensions are multiples of 4 (any
+// M and N).  Same decomposition as cgemm_kernel,
 // with the per-chunk overhead taken out of the vector ALU, the registers and the LDS write port:
 //   * operand tiles go from global memory straight into LDS (global_load_lds_dwordx4), 1 KiB per wave-wide
 //     instruction, so a chunk needs no staging registers and no LDS write instructions; global addresses are
@@ -386,8 +387,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 //     k = 8 + 4h + (s - 4); the [k][row] operands are addressed with the same map, so the products pair up correctly.
 //   * LDS holds two (128 x 128) or three (smaller blocks) stages; the transfers of chunk c + stages - 1 are issued
 //     before the MFMAs of chunk c, one vmcnt wait and one barrier per chunk publish the next stage;
-//   * the scheduler is told to interleave (one MFMA, then a few VALU / DS / memory instructions) so everything else
-//     issues in the shadow of the matrix pipe.
+//   * the scheduler is told to interleave (one MFMA, then a few DS / memory instructions) so everything else
+//     issues in the shadow of the matrix pipe;
+//   * the K loop holds (almost) no vector-ALU instruction, because each one costs the matrix pipe a few cycles (shared
+//     issue port): signs are applied to the accumulators when they are stored (or compiled into the choice of the
+//     negated operand, for the 128 x 128 block), and the chunk loop is unrolled over the LDS stages so that addresses
+//     are "lane base + immediate".
 // Operand fragments of one wavefront: T tiles of 32 rows, both planes.
 //   MCONTIG ([k][row] in LDS): one float per tile, plane and k step, double buffered per step.
 //   otherwise ([row][k] swizzled): one float4 per tile, plane and half chunk (set 0: steps 0..3, set 1: steps 4..7).
