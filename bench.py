@@ -222,20 +222,32 @@ def token_model_suite(steps):
                       "loss_of_uniform_guess": round(float(np.log(V)), 4)}))
 
 
-def train_suite(steps):
+def train_lines(steps):
     """Training steps (upload of the batch, forward, loss read-back, backward, SGD) of the FourierTrans -> Hadamard ->
-    CGelu -> Linear -> CrossEntropy net on 784-long samples, run by the C++ facade's own driver; one JSON line per
-    batch size with the time per step of each input mode (copy inside forward / prefetch / recorded graphs)."""
+    CGelu -> Linear -> CrossEntropy net on 784-long samples, run by the C++ facade's own driver in a process of its own;
+    one dict per batch size with the time per step of each input mode (copy inside forward / prefetch / recorded
+    graphs).  None when the driver is not built or fails."""
     import subprocess
     exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "bin", "facade_test")
     if not os.path.exists(exe):
-        sys.exit("bench.py: %s is missing; run __graft_entry__.build() first" % exe)
+        return None
+    out = []
     for batch in (64, 4096):
         r = subprocess.run([exe, "pipeline_timing", str(batch), str(steps)], capture_output=True, text=True, timeout=600)
         lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
         if r.returncode != 0 or not lines:
-            sys.exit("bench.py: facade_test pipeline_timing failed:\n" + r.stdout[-2000:] + r.stderr[-2000:])
-        print(lines[-1])
+            sys.stderr.write("bench.py: facade_test pipeline_timing failed:\n" + r.stdout[-2000:] + r.stderr[-2000:])
+            return None
+        out.append(json.loads(lines[-1]))
+    return out
+
+
+def train_suite(steps):
+    lines = train_lines(steps)
+    if lines is None:
+        sys.exit("bench.py: tests/bin/facade_test is missing or failed; run __graft_entry__.build() first")
+    for l in lines:
+        print(json.dumps(l))
 
 
 def main():
@@ -354,6 +366,11 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+        train = train_lines(100)
+        if train:   # the other half of the metric: training steps of the configs[0] net through the C++ facade
+            out["train"] = [{"workload": t["workload"], "batch": t["batch"], "ms_per_step": t["ms_per_step_prefetch"],
+                             "samples_per_sec": t["samples_per_sec_prefetch"],
+                             "samples_per_sec_copy_inside_forward": t["samples_per_sec_copy_in_forward"]} for t in train]
     print(json.dumps(out))
 
 
