@@ -618,6 +618,9 @@ class CNet {
 	struct StepGraphs {
 		void *fwd = NULL, *bwd = NULL, *upd = NULL;
 		float upd_lr = 0.f;
+		void *step = NULL;      // forward + backward + update in one recording (gpuTrainStep)
+		float step_lr = 0.f;
+		bool step_warm = false;  // the three phases have run once with this buffer since the last change of the plan
 	};
 	StepGraphs graphs_[2];
 	bool use_graphs_ = false;
@@ -638,7 +641,7 @@ class CNet {
 
 	void dropGraphs() {
 		for (auto &g : graphs_) {
-			for (void *e : {g.fwd, g.bwd, g.upd})
+			for (void *e : {g.fwd, g.bwd, g.upd, g.step})
 				if (e) cnet_graph_destroy(e);
 			g = StepGraphs();
 		}
@@ -1199,6 +1202,58 @@ public:
 	// ---- batched step (upstream gpuForward / gpuBackward / gpuUpdateInputs / getLoss,
 	//      gpu/gpu_func.h:1088-1101, 491-495, 906-926; step semantics of cnet.cpp:104-150) ----
 	bool gpuForward(InputFunc *inp, OutputFunc *outp, InputBatch &batch) {
+		feedBatch(inp, outp, batch);
+		return GpuForward();
+	}
+	// forward + backward + update of one batch, replayed from ONE recorded graph: a step at small batch sizes is bound by
+	// the cost of launching ~20 kernels one by one, not by the kernels.  The first call with each buffer of the data input
+	// runs the three phases as usual (which also sizes the library's workspace), the second records them, later ones
+	// replay; a change of the learning rate records again.  Same kernels, same arguments, same results as
+	// gpuForward / gpuBackward / gpuUpdateInputs; the losses of the step are read with getLoss() whenever they are wanted
+	// (every call of it waits for the device).
+	void gpuTrainStep(InputFunc *inp, OutputFunc *outp, InputBatch &batch, float l_rate) {
+		if (use_graphs_) throw std::logic_error("gpuTrainStep records the whole step itself: call useGraphs(false) first");
+		feedBatch(inp, outp, batch);
+		StepGraphs &g = graphs_[active_];
+		auto eager = [&] {
+			const bool was = use_graphs_;
+			use_graphs_ = false;  // the phases launch (or record) their kernels themselves
+			try {
+				GpuForward();
+				gpuBackward();
+				gpuUpdateInputs(l_rate);
+			} catch (...) {
+				use_graphs_ = was;
+				throw;
+			}
+			use_graphs_ = was;
+		};
+		if (input_dz_dirty_ || !g.step_warm) {  // an update that also clears a first moment is not what a recording replays
+			eager();
+			g.step_warm = true;
+			return;
+		}
+		if (g.step && g.step_lr != l_rate) {
+			ck(cnet_graph_destroy(g.step), "cnet_graph_destroy");
+			g.step = NULL;
+		}
+		if (!g.step) {
+			ck(cnet_graph_begin(), "cnet_graph_begin");
+			try {
+				eager();
+			} catch (...) {
+				cnet_graph_end(NULL);
+				throw;
+			}
+			ck(cnet_graph_end(&g.step), "cnet_graph_end");
+			g.step_lr = l_rate;
+		}
+		ck(cnet_graph_launch(g.step), "cnet_graph_launch");
+	}
+
+private:
+	// a batch for the main data input: switch to the buffer it was sent ahead to (gpuPrefetch), or copy it now
+	void feedBatch(InputFunc *inp, OutputFunc *outp, InputBatch &batch) {
 		requireAllocated("gpuForward");
 		CInput *cin = dynamic_cast<CInput *>(inp);
 		if (!cin) throw std::invalid_argument("gpuForward: this type of input is not supported with an InputBatch");
@@ -1221,7 +1276,7 @@ public:
 			d_labels_ = staged.labels;
 			labels_.assign(batch.labelsPtr(), batch.labelsPtr() + batch_);
 			batch_labels_ = true;
-			return GpuForward();
+			return;
 		}
 		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
 		// one copy per plane (upstream: two small copies per sample, gpu/gpu_func.h:403-419)
@@ -1234,8 +1289,9 @@ public:
 			ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
 		}
 		setLabels(batch.labelsPtr(), batch_);
-		return GpuForward();
 	}
+
+public:
 	// Send the NEXT batch to the device on the upload stream while the kernels of the current step run; the later
 	// gpuForward(inp, outp, batch) with the same batch object then only switches buffers.  The data input is double
 	// buffered on the device (the second buffer is allocated on the first call); at most one batch can be staged.  The

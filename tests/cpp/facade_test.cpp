@@ -865,12 +865,12 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs) 
 		return;
 	}
 	SyntheticReader data(n, 3 * B + 7, classes);
-	constexpr int MODES = 4;
+	constexpr int MODES = 5;  // 4: prefetch + gpuTrainStep (the whole step as one recorded graph)
 	std::vector<float> losses[MODES];
 	std::vector<float> weights[MODES];
-	double ms[MODES] = {0, 0, 0, 0};
+	double ms[MODES] = {0, 0, 0, 0, 0};
 	for (int mode = 0; mode < (with_graphs ? MODES : 2); ++mode) {
-		const bool prefetch = mode == 1 || mode == 2, graphs = mode >= 2;
+		const bool prefetch = mode == 1 || mode == 2 || mode == 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4;
 		CNet net;
 		int inp, outp;
 		build_readme(net, n, classes, &inp, &outp);
@@ -895,9 +895,14 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs) 
 			if (!prefetch) reader.nextBatch(cur);
 			// the whole step is queued first; only then does the host turn to the next batches, and last of all it waits
 			// for this step's losses (backward and update do not touch them)
-			net.gpuForward(cin, cen, cur);
-			net.gpuBackward();
-			net.gpuUpdateInputs((s < steps / 2 ? lr : 0.5f * lr) / B);
+			const float rate = (s < steps / 2 ? lr : 0.5f * lr) / B;
+			if (one_graph) {
+				net.gpuTrainStep(cin, cen, cur, rate);
+			} else {
+				net.gpuForward(cin, cen, cur);
+				net.gpuBackward();
+				net.gpuUpdateInputs(rate);
+			}
 			if (prefetch) {
 				if (s + 1 < steps) net.gpuPrefetch(cin, ring[(s + 1) % 3]);
 				if (s + 2 < steps) reader.nextBatch(ring[(s + 2) % 3]);
@@ -946,13 +951,17 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs) 
 		expect("weights identical with graph replay (prefetch)", weights[0] == weights[2]);
 		expect("losses identical with graph replay (copy in forward)", losses[0] == losses[3]);
 		expect("weights identical with graph replay (copy in forward)", weights[0] == weights[3]);
+		expect("losses identical with gpuTrainStep (one recorded graph per step)", losses[0] == losses[4]);
+		expect("weights identical with gpuTrainStep", weights[0] == weights[4]);
 		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
 	}
 	printf("{\"workload\": \"README net 784 -> 10, SGD, batches from a BatchedDataReader\", \"batch\": %d, \"steps\": %d, "
 		   "\"ms_per_step_copy_in_forward\": %.3f, \"ms_per_step_prefetch\": %.3f, \"ms_per_step_prefetch_graphs\": %.3f, "
 		   "\"ms_per_step_graphs\": %.3f, \"samples_per_sec_copy_in_forward\": %.1f, \"samples_per_sec_prefetch\": %.1f, "
-		   "\"samples_per_sec_prefetch_graphs\": %.1f, \"upload_bytes_per_step\": %zu}\n",
-			B, steps, ms[0], ms[1], ms[2], ms[3], B / ms[0] * 1e3, B / ms[1] * 1e3, ms[2] > 0 ? B / ms[2] * 1e3 : 0.0, (size_t) 2 * B * n * sizeof(float));
+		   "\"samples_per_sec_prefetch_graphs\": %.1f, \"ms_per_step_train_step_graph\": %.3f, \"samples_per_sec_train_step_graph\": %.1f, "
+		   "\"upload_bytes_per_step\": %zu}\n",
+			B, steps, ms[0], ms[1], ms[2], ms[3], B / ms[0] * 1e3, B / ms[1] * 1e3, ms[2] > 0 ? B / ms[2] * 1e3 : 0.0, ms[4],
+			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, (size_t) 2 * B * n * sizeof(float));
 }
 
 // ------------------------------------------------------------------------------------------------- upstream's test nets
