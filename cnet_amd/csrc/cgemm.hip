@@ -826,6 +826,170 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(CgemmArgs args) {
 	}
 }
 
+// ---- small C: one 16 x 16 tile per workgroup, K shared out among its wavefronts ---------------------------------------
+//
+// A product with a small C (a batch of 64 rows against a 784-long reduction) has too few blocks for the kernels above
+// and is bound by latency, not by arithmetic.  Here a workgroup of W wavefronts owns one 16 x 16 tile of C (small, so
+// that even a 64 x 784 result spreads over 196 compute units); wavefront w walks the w-th part of K with its operands
+// loaded straight from global memory into the MFMA operand registers (no LDS staging: nothing is shared between
+// wavefronts but the tile of C), three groups of 16 k values in flight (more in flight was slower: the vector memory
+// pipeline of the compute unit, not latency, sets the pace).  The W partial tiles meet in LDS and are added
+// in wavefront order, so the result does not depend on timing, and C is written once: no second kernel.  Lane (r, q) of
+// a wavefront, r = lane % 16, feeds row / column r of the tile; step s of a group (v_mfma_f32_16x16x4_f32) takes k =
+// 16 g + 4 q + s from lane quarter q, which lets an operand that is contiguous along K arrive as one float4 per plane.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// Four k values of one plane for this lane.  Every load is unconditional (addresses past the end of K are pulled back
+// inside; the caller zeroes what they return), so the loads of several groups stay in flight together.
+template <bool V4>
+__device__ __forceinline__ void load_k4(const float *__restrict__ base, long kstride, int k, int K, float v[4]) {
+	if constexpr (V4) {
+		const float4 t = *reinterpret_cast<const float4 *>(base + min(k, K - 4));
+		v[0] = t.x;
+		v[1] = t.y;
+		v[2] = t.z;
+		v[3] = t.w;
+	} else {
+#pragma unroll
+		for (int s = 0; s < 4; ++s) v[s] = base[(long) min(k + s, K - 1) * kstride];
+	}
+}
+
+template <int W, bool A_V4, bool B_V4>
+__global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs args, long a_kstride, long a_mstride, long b_kstride,
+		long b_nstride) {
+	__shared__ float red[W * 2 * 4 * 64];  // [W][re, im][4][64]
+	constexpr int DEPTH = 3;
+	const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+	CgemmProblem pb = args.p[blockIdx.y];
+	batch_offset(pb, args);
+	// Consecutive workgroup numbers go round-robin to the XCDs: give each XCD a contiguous run of tiles, row tiles
+	// fastest, so that the tiles sharing columns of B meet in one L2 and each XCD reads its own part of B only.
+	const int total = args.tiles_m * args.tiles_n, xcd = blockIdx.x % NUM_XCD, share = total / NUM_XCD, extra = total % NUM_XCD;
+	const int tile = xcd * share + min(xcd, extra) + blockIdx.x / NUM_XCD;
+	const int tile_n = tile / args.tiles_m, tile_m = tile - tile_n * args.tiles_m;
+	const int m0 = tile_m * 16, n0 = tile_n * 16;
+	// lanes beyond the edge of C read the last valid row / column again; their results are not stored
+	const long a_off = (long) min(m0 + r, args.M - 1) * a_mstride, b_off = (long) min(n0 + r, args.N - 1) * b_nstride;
+	const float *a_re = pb.a_re + a_off, *a_im = pb.a_im + a_off, *b_re = pb.b_re + b_off, *b_im = pb.b_im + b_off;
+	const int groups = (args.K + 15) / 16, per = (groups + W - 1) / W;
+	const int g_lo = wave * per, g_hi = min(groups, g_lo + per);
+	const float sa = pb.a_im_sign, sb = pb.b_im_sign, sq = -sa * sb;
+
+	struct Group {
+		float ar[4], ai[4], br[4], bi[4];
+	};
+	auto fetch = [&](Group &t, int g) __attribute__((always_inline)) {
+		const int k = g * 16 + 4 * q;
+		load_k4<A_V4>(a_re, a_kstride, k, args.K, t.ar);
+		load_k4<A_V4>(a_im, a_kstride, k, args.K, t.ai);
+		load_k4<B_V4>(b_re, b_kstride, k, args.K, t.br);
+		load_k4<B_V4>(b_im, b_kstride, k, args.K, t.bi);
+	};
+	floatx4 acc_re = {0.f, 0.f, 0.f, 0.f}, acc_im = {0.f, 0.f, 0.f, 0.f};
+	Group buf[DEPTH];
+#pragma unroll
+	for (int d = 0; d < DEPTH; ++d) fetch(buf[d], g_lo + d);
+	for (int g = g_lo; g < g_hi; g += DEPTH) {
+#pragma unroll
+		for (int d = 0; d < DEPTH; ++d) {
+			Group cur = buf[d];
+			fetch(buf[d], g + d + DEPTH);
+			if (g + d < g_hi) {
+				// the last group of K may reach past its end (selects, no branches: the loads above stay countable)
+				const int left = args.K - ((g + d) * 16 + 4 * q);
+#pragma unroll
+				for (int s = 0; s < 4; ++s) {
+					const bool in = s < left;
+					cur.ar[s] = in ? cur.ar[s] : 0.f;
+					cur.ai[s] = in ? cur.ai[s] : 0.f;
+					cur.br[s] = in ? cur.br[s] : 0.f;
+					cur.bi[s] = in ? cur.bi[s] : 0.f;
+				}
+#pragma unroll
+				for (int s = 0; s < 4; ++s) {
+					// re = Ar Br - (sa Ai)(sb Bi), im = Ar (sb Bi) + (sa Ai) Br
+					acc_re = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.ar[s], cur.br[s], acc_re, 0, 0, 0);
+					acc_im = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.ar[s], sb * cur.bi[s], acc_im, 0, 0, 0);
+					acc_re = __builtin_amdgcn_mfma_f32_16x16x4f32(sq * cur.ai[s], cur.bi[s], acc_re, 0, 0, 0);
+					acc_im = __builtin_amdgcn_mfma_f32_16x16x4f32(sa * cur.ai[s], cur.br[s], acc_im, 0, 0, 0);
+				}
+			}
+		}
+	}
+#pragma unroll
+	for (int e = 0; e < 4; ++e) {
+		red[((wave * 2 + 0) * 4 + e) * 64 + lane] = acc_re[e];
+		red[((wave * 2 + 1) * 4 + e) * 64 + lane] = acc_im[e];
+	}
+	__syncthreads();
+	// the 8 (plane, accumulator register) pairs are added and stored by the first wavefronts, one or two pairs each
+	const int col = n0 + r;
+	for (int c = wave; c < 8; c += W) {
+		const int part = c >> 2, e = c & 3;
+		float v = 0.f;
+#pragma unroll
+		for (int w = 0; w < W; ++w) v += red[((w * 2 + part) * 4 + e) * 64 + lane];
+		const int row = m0 + 4 * q + e;
+		if (row < args.M && col < args.N) {
+			float *dst = (part ? pb.c_im : pb.c_re) + (long) row * args.ldc + col;
+			*dst = args.accumulate ? *dst + v : v;
+		}
+	}
+}
+
+template <int W, bool A_V4, bool B_V4>
+int launch_skinny(const CgemmArgs &args, bool a_mcontig, bool b_ncontig, int nprob, int batch) {
+	auto kern = cgemm_skinny_kernel<W, A_V4, B_V4>;
+	hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, nprob, batch), dim3(64 * W), 0, cnet::rt().stream, args,
+			a_mcontig ? args.lda : 1L, a_mcontig ? 1L : args.lda, b_ncontig ? args.ldb : 1L, b_ncontig ? 1L : args.ldb);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+// true and *rc set when the product was small enough for cgemm_skinny_kernel
+bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int nprob, int batch, int *rc) {
+	static const bool enabled = [] {
+		const char *e = getenv("CNET_CGEMM_SKINNY");  // tuning override: 0 sends every product to the block kernels
+		return !e || atoi(e) != 0;
+	}();
+	if (!enabled || proto.tri || batch > 65535) return false;
+	CgemmArgs args = proto;
+	args.tiles_m = (args.M + 15) / 16;
+	args.tiles_n = (args.N + 15) / 16;
+	const long tiles = (long) args.tiles_m * args.tiles_n * nprob * batch;
+	// Measured against the block kernels with K cut (64 x 784 x 784: 10 against 15 us; 64 x 10 x 784: 9 against 12 us;
+	// 10 x 784 x 64: 4 against 9 us); beyond two tiles per compute unit, or with a long K, those win again (256 x 784 x
+	// 784: 27 against 23 us; 10 x 784 x 4096: 36 against 29 us).
+	static const long tile_limit = [] {
+		const char *e = getenv("CNET_CGEMM_SKINNY_TILES");  // tuning override of the largest number of tiles
+		return e ? atol(e) : 0L;
+	}();
+	if (tiles > (tile_limit ? tile_limit : 2L * cnet::rt().prop.multiProcessorCount) || args.K > 1024) return false;
+	args.splits = 1;
+	args.chunks_per_split = 0;
+	args.partial = nullptr;
+	args.nprob = nprob;
+	args.tail_tiles = args.tail_splits = args.tail_chunks = 0;
+	bool a_v4 = !a_mcontig && args.lda % 4 == 0 && args.stride_a % 4 == 0 && args.K % 4 == 0;
+	bool b_v4 = !b_ncontig && args.ldb % 4 == 0 && args.stride_b % 4 == 0 && args.K % 4 == 0;
+	for (int q = 0; q < nprob; ++q) {
+		a_v4 = a_v4 && cnet::aligned16(args.p[q].a_re) && cnet::aligned16(args.p[q].a_im);
+		b_v4 = b_v4 && cnet::aligned16(args.p[q].b_re) && cnet::aligned16(args.p[q].b_im);
+	}
+#define CNET_SKINNY(W)                                                                                         \
+	(a_v4 ? (b_v4 ? launch_skinny<W, true, true>(args, a_mcontig, b_ncontig, nprob, batch)                     \
+				  : launch_skinny<W, true, false>(args, a_mcontig, b_ncontig, nprob, batch))                   \
+		  : (b_v4 ? launch_skinny<W, false, true>(args, a_mcontig, b_ncontig, nprob, batch)                    \
+				  : launch_skinny<W, false, false>(args, a_mcontig, b_ncontig, nprob, batch)))
+	// Four wavefronts per tile: the time of a tile is set by the compute unit's vector memory pipeline (each load
+	// instruction touches 4 to 16 cache lines), not by how many wavefronts share the work, and small workgroups leave
+	// room for a second tile on the same unit.
+	*rc = CNET_SKINNY(4);
+#undef CNET_SKINNY
+	return true;
+}
+
 // tail_splits >= 2: cut the blocks of the last, partly filled round into that many pieces along K (see CgemmArgs)
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
 int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0) {
@@ -999,6 +1163,8 @@ namespace cnet {
 static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int nprob, int batch) {
 	if (a.M <= 0 || a.N <= 0) return CNET_OK;
 	if (a.K <= 0) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: K must be positive");
+	int rc = CNET_OK;
+	if (try_skinny(a_mcontig, b_ncontig, a, nprob, batch, &rc)) return rc;
 	// float4 path: every contiguous run starts 16-byte aligned and has a length that is a multiple of 4
 	bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (a.stride_a % 4 == 0) && (a.stride_b % 4 == 0);
 	vec = vec && (a_mcontig ? a.M % 4 == 0 : a.K % 4 == 0) && (b_ncontig ? a.N % 4 == 0 : a.K % 4 == 0);

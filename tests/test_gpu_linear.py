@@ -121,7 +121,8 @@ def _check_all_layouts(port, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(8, 24, 1000), (64, 64, 4096), (40, 100, 333), (64, 784, 784), (3, 5, 2049)])
 def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
-    """Few blocks of C against a long K: the launch is cut along K and the partial blocks are added in a fixed order."""
+    """Few blocks of C against a long K.  Up to K = 1024 each 16 x 16 tile of C has a workgroup of its own whose wavefronts
+    share K; beyond, the launch of the block kernel is cut along K and the partial blocks are added in a fixed order."""
     _check_all_layouts(port, M, N, K)
 
 
@@ -184,11 +185,13 @@ def test_linear_headline_shape_rows_against_oracle(gpu, port):
     assert rel_c(full[0:2], parts[0:2]) < 1e-5 and rel_c(full[2:4], parts[2:4]) < 1e-5
 
 
-@pytest.mark.parametrize("M,N,K,nb", [(8192, 1024, 64, 1), (192, 256, 48, 2), (4096, 512, 32, 1), (1024, 2048, 32, 1)])
+@pytest.mark.parametrize("M,N,K,nb", [(8192, 1024, 64, 1), (192, 256, 48, 2), (4096, 512, 32, 1), (1024, 2048, 32, 1),
+                                      (40, 52, 200, 2), (64, 10, 784, 1)])
 def test_cgemm_conjugate_combinations(gpu, port, M, N, K, nb):
     """conj(A) and conj(B) in all four combinations, on shapes that take each block shape of the fast path: the signs are
     applied when the block is stored (one- and two-tile wavefronts) or by the choice of the negated operand (four
-    tiles), and conj(A) conj(B) negates the imaginary plane on its way out."""
+    tiles), and conj(A) conj(B) negates the imaginary plane on its way out.  The last two shapes have a small C and go
+    to the kernel with one 16 x 16 tile per workgroup, which scales the imaginary operands by the signs."""
     A = seeded(port, 21, (nb, M, K)) + 1j * seeded(port, 22, (nb, M, K))
     Bm = seeded(port, 23, (K, N)) + 1j * seeded(port, 24, (K, N))
     a = ops.CMat.from_host(np.ascontiguousarray(A.real).reshape(nb * M, K), np.ascontiguousarray(A.imag).reshape(nb * M, K))
