@@ -872,8 +872,17 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 	// lanes beyond the edge of C read the last valid row / column again; their results are not stored
 	const long a_off = (long) min(m0 + r, args.M - 1) * a_mstride, b_off = (long) min(n0 + r, args.N - 1) * b_nstride;
 	const float *a_re = pb.a_re + a_off, *a_im = pb.a_im + a_off, *b_re = pb.b_re + b_off, *b_im = pb.b_im + b_off;
-	const int groups = (args.K + 15) / 16, per = (groups + W - 1) / W;
-	const int g_lo = wave * per, g_hi = min(groups, g_lo + per);
+	// this workgroup's groups of K (all of them, or one slice when a long K is cut across workgroups), then this wavefront's
+	int first = 0, last = (args.K + 15) / 16;
+	if (args.splits > 1) {
+		first = (blockIdx.z % args.splits) * args.chunks_per_split;
+		last = min(last, first + args.chunks_per_split);
+	}
+	const int per = (last - first + W - 1) / W;
+	const int g_lo = first + wave * per, g_hi = min(last, g_lo + per);
+	long ldc;
+	int accumulate;
+	output_planes(args, pb, ldc, accumulate);  // C, or the slice of the partial planes that splitk_reduce_kernel adds up
 	const float sa = pb.a_im_sign, sb = pb.b_im_sign, sq = -sa * sb;
 
 	struct Group {
@@ -932,8 +941,8 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 		for (int w = 0; w < W; ++w) v += red[((w * 2 + part) * 4 + e) * 64 + lane];
 		const int row = m0 + 4 * q + e;
 		if (row < args.M && col < args.N) {
-			float *dst = (part ? pb.c_im : pb.c_re) + (long) row * args.ldc + col;
-			*dst = args.accumulate ? *dst + v : v;
+			float *dst = (part ? pb.c_im : pb.c_re) + (long) row * ldc + col;
+			*dst = accumulate ? *dst + v : v;
 		}
 	}
 }
@@ -941,9 +950,14 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 template <int W, bool A_V4, bool B_V4>
 int launch_skinny(const CgemmArgs &args, bool a_mcontig, bool b_ncontig, int nprob, int batch) {
 	auto kern = cgemm_skinny_kernel<W, A_V4, B_V4>;
-	hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, nprob, batch), dim3(64 * W), 0, cnet::rt().stream, args,
+	hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, nprob, batch * args.splits), dim3(64 * W), 0, cnet::rt().stream, args,
 			a_mcontig ? args.lda : 1L, a_mcontig ? 1L : args.lda, b_ncontig ? args.ldb : 1L, b_ncontig ? 1L : args.ldb);
 	CNET_LAUNCH_CHECK();
+	if (args.splits > 1) {
+		dim3 rgrid((unsigned) ((2L * args.M * args.N + 255) / 256), nprob, batch);
+		hipLaunchKernelGGL(splitk_reduce_kernel, rgrid, dim3(256), 0, cnet::rt().stream, args, nprob, batch);
+		CNET_LAUNCH_CHECK();
+	}
 	return CNET_OK;
 }
 
@@ -959,18 +973,35 @@ bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int npro
 	args.tiles_n = (args.N + 15) / 16;
 	const long tiles = (long) args.tiles_m * args.tiles_n * nprob * batch;
 	// Measured against the block kernels with K cut (64 x 784 x 784: 10 against 15 us; 64 x 10 x 784: 9 against 12 us;
-	// 10 x 784 x 64: 4 against 9 us); beyond two tiles per compute unit, or with a long K, those win again (256 x 784 x
-	// 784: 27 against 23 us; 10 x 784 x 4096: 36 against 29 us).
+	// 10 x 784 x 64: 4 against 9 us); beyond two tiles per compute unit those win again (256 x 784 x 784: 27 against
+	// 23 us).
 	static const long tile_limit = [] {
 		const char *e = getenv("CNET_CGEMM_SKINNY_TILES");  // tuning override of the largest number of tiles
 		return e ? atol(e) : 0L;
 	}();
-	if (tiles > (tile_limit ? tile_limit : 2L * cnet::rt().prop.multiProcessorCount) || args.K > 1024) return false;
+	const long most = tile_limit ? tile_limit : 2L * cnet::rt().prop.multiProcessorCount;
+	if (tiles > most) return false;
 	args.splits = 1;
 	args.chunks_per_split = 0;
 	args.partial = nullptr;
 	args.nprob = nprob;
 	args.tail_tiles = args.tail_splits = args.tail_chunks = 0;
+	if (args.K > 1024) {
+		// A long K against a C of few tiles (the weight gradient of a narrow layer over a large batch): slices of K go to
+		// workgroups of their own, at least 256 long and no more slices than keep the launch within the tile limit; the
+		// slices are added in order by splitk_reduce_kernel.
+		const int groups = (args.K + 15) / 16;
+		const long splits = std::min<long>(most / tiles, groups / 16);
+		if (splits < 2 || (long) batch * splits > 65535) return false;
+		args.chunks_per_split = (int) ((groups + splits - 1) / splits);
+		if (args.chunks_per_split > 64) return false;  // still longer than 1024 per slice: the block kernels do better
+		args.splits = (groups + args.chunks_per_split - 1) / args.chunks_per_split;  // no empty slice
+		args.partial = (float *) cnet::workspace((size_t) args.splits * nprob * batch * 2 * args.M * args.N * sizeof(float));
+		if (!args.partial) {
+			*rc = CNET_ERR_OUT_OF_MEMORY;
+			return true;
+		}
+	}
 	bool a_v4 = !a_mcontig && args.lda % 4 == 0 && args.stride_a % 4 == 0 && args.K % 4 == 0;
 	bool b_v4 = !b_ncontig && args.ldb % 4 == 0 && args.stride_b % 4 == 0 && args.K % 4 == 0;
 	for (int q = 0; q < nprob; ++q) {
