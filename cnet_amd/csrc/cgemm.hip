@@ -832,35 +832,47 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(CgemmArgs args) {
 // and is bound by latency, not by arithmetic.  Here a workgroup of W wavefronts owns one 16 x 16 tile of C (small, so
 // that even a 64 x 784 result spreads over 196 compute units); wavefront w walks the w-th part of K with its operands
 // loaded straight from global memory into the MFMA operand registers (no LDS staging: nothing is shared between
-// wavefronts but the tile of C), three groups of 16 k values in flight (more in flight was slower: the vector memory
-// pipeline of the compute unit, not latency, sets the pace).  The W partial tiles meet in LDS and are added
+// wavefronts but the tile of C), three groups of 16 k values in flight.  The W partial tiles meet in LDS and are added
 // in wavefront order, so the result does not depend on timing, and C is written once: no second kernel.  Lane (r, q) of
 // a wavefront, r = lane % 16, feeds row / column r of the tile; step s of a group (v_mfma_f32_16x16x4_f32) takes k =
 // 16 g + 4 q + s from lane quarter q, which lets an operand that is contiguous along K arrive as one float4 per plane.
+// What makes the loop run at the pace of its 16 MFMAs per group: the loop body has no branch (otherwise the compiler
+// waits for every load in flight at the top of each round), the ring slots are refilled after use, in place (no register
+// copies), the wavefront number is a scalar, and addresses are 32-bit offsets into buffer descriptors.
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-// Four k values of one plane for this lane.  Every load is unconditional (addresses past the end of K are pulled back
-// inside; the caller zeroes what they return), so the loads of several groups stay in flight together.
+// Four k values of one plane for this lane, through a buffer descriptor of the plane: the lane's part of the address
+// is a 32-bit byte offset shared by the re and im planes (one integer add per load instead of 64-bit address
+// arithmetic, which would cost this kernel more issue cycles than its MFMAs), every load is unconditional, so the loads
+// of several groups stay in flight together, and a load past the end of the plane returns zero instead of faulting.
 template <bool V4>
-__device__ __forceinline__ void load_k4(const float *__restrict__ base, long kstride, int k, int K, float v[4]) {
+__device__ __forceinline__ void load_k4(__amdgpu_buffer_rsrc_t plane, unsigned lane_bytes, unsigned kstride_bytes, int k, float v[4]) {
 	if constexpr (V4) {
-		const float4 t = *reinterpret_cast<const float4 *>(base + min(k, K - 4));
-		v[0] = t.x;
-		v[1] = t.y;
-		v[2] = t.z;
-		v[3] = t.w;
+		const floatx4 t = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(plane, lane_bytes + 4u * k, 0, 0));
+		v[0] = t[0];
+		v[1] = t[1];
+		v[2] = t[2];
+		v[3] = t[3];
 	} else {
 #pragma unroll
-		for (int s = 0; s < 4; ++s) v[s] = base[(long) min(k + s, K - 1) * kstride];
+		for (int s = 0; s < 4; ++s)
+			v[s] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(plane, lane_bytes + (unsigned) (k + s) * kstride_bytes, 0, 0));
 	}
 }
 
+// descriptor of `bytes` bytes at p: raw 32-bit data, no swizzle, loads checked against `bytes`
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t plane_rsrc(const float *p, unsigned bytes) {
+	return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p), 0, bytes, 0x00020000);
+}
+
 template <int W, bool A_V4, bool B_V4>
-__global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs args, long a_kstride, long a_mstride, long b_kstride,
-		long b_nstride) {
+__global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs args, unsigned a_kstride, unsigned a_mstride,
+		unsigned b_kstride, unsigned b_nstride, unsigned a_bytes, unsigned b_bytes) {
 	__shared__ float red[W * 2 * 4 * 64];  // [W][re, im][4][64]
 	constexpr int DEPTH = 3;
-	const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+	// the wavefront number as a scalar: the K range, the loop over it and its branches then run on the scalar unit
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
 	CgemmProblem pb = args.p[blockIdx.y];
 	batch_offset(pb, args);
 	// Consecutive workgroup numbers go round-robin to the XCDs: give each XCD a contiguous run of tiles, row tiles
@@ -870,10 +882,12 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 	const int tile_n = tile / args.tiles_m, tile_m = tile - tile_n * args.tiles_m;
 	const int m0 = tile_m * 16, n0 = tile_n * 16;
 	// lanes beyond the edge of C read the last valid row / column again; their results are not stored
-	const long a_off = (long) min(m0 + r, args.M - 1) * a_mstride, b_off = (long) min(n0 + r, args.N - 1) * b_nstride;
-	const float *a_re = pb.a_re + a_off, *a_im = pb.a_im + a_off, *b_re = pb.b_re + b_off, *b_im = pb.b_im + b_off;
+	const unsigned a_off = 4u * min(m0 + r, args.M - 1) * a_mstride, b_off = 4u * min(n0 + r, args.N - 1) * b_nstride;  // bytes
+	const __amdgpu_buffer_rsrc_t a_re = plane_rsrc(pb.a_re, a_bytes), a_im = plane_rsrc(pb.a_im, a_bytes);
+	const __amdgpu_buffer_rsrc_t b_re = plane_rsrc(pb.b_re, b_bytes), b_im = plane_rsrc(pb.b_im, b_bytes);
 	// this workgroup's groups of K (all of them, or one slice when a long K is cut across workgroups), then this wavefront's
-	int first = 0, last = (args.K + 15) / 16;
+	const int all_groups = (args.K + 15) / 16;
+	int first = 0, last = all_groups;
 	if (args.splits > 1) {
 		first = (blockIdx.z % args.splits) * args.chunks_per_split;
 		last = min(last, first + args.chunks_per_split);
@@ -883,53 +897,65 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 	long ldc;
 	int accumulate;
 	output_planes(args, pb, ldc, accumulate);  // C, or the slice of the partial planes that splitk_reduce_kernel adds up
-	const float sa = pb.a_im_sign, sb = pb.b_im_sign, sq = -sa * sb;
 
 	struct Group {
 		float ar[4], ai[4], br[4], bi[4];
 	};
 	auto fetch = [&](Group &t, int g) __attribute__((always_inline)) {
 		const int k = g * 16 + 4 * q;
-		load_k4<A_V4>(a_re, a_kstride, k, args.K, t.ar);
-		load_k4<A_V4>(a_im, a_kstride, k, args.K, t.ai);
-		load_k4<B_V4>(b_re, b_kstride, k, args.K, t.br);
-		load_k4<B_V4>(b_im, b_kstride, k, args.K, t.bi);
+		load_k4<A_V4>(a_re, a_off, 4u * a_kstride, k, t.ar);
+		load_k4<A_V4>(a_im, a_off, 4u * a_kstride, k, t.ai);
+		load_k4<B_V4>(b_re, b_off, 4u * b_kstride, k, t.br);
+		load_k4<B_V4>(b_im, b_off, 4u * b_kstride, k, t.bi);
 	};
-	floatx4 acc_re = {0.f, 0.f, 0.f, 0.f}, acc_im = {0.f, 0.f, 0.f, 0.f};
+	// four independent accumulator chains, P = Ar Br, R = Ar Bi, Q = Ai Bi, S = Ai Br: no MFMA waits for the one before
+	// it, and the conjugation signs wait until the sums are complete
+	const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+	floatx4 acc_p = zero, acc_r = zero, acc_q = zero, acc_s = zero;
 	Group buf[DEPTH];
 #pragma unroll
 	for (int d = 0; d < DEPTH; ++d) fetch(buf[d], g_lo + d);
-	for (int g = g_lo; g < g_hi; g += DEPTH) {
+	// One group: what lies past the end of K is zeroed first (an operand stored along K has its next row or padding
+	// there; four selects per plane, nothing next to 16 MFMAs), then P, R, Q, S advance by four k values per step.
+	auto use = [&](Group &t, int g) __attribute__((always_inline)) {
+		const int left = args.K - (g * 16 + 4 * q);
+#pragma unroll
+		for (int s = 0; s < 4; ++s) {
+			const bool in = s < left;
+			t.ar[s] = in ? t.ar[s] : 0.f;
+			t.ai[s] = in ? t.ai[s] : 0.f;
+			t.br[s] = in ? t.br[s] : 0.f;
+			t.bi[s] = in ? t.bi[s] : 0.f;
+		}
+#pragma unroll
+		for (int s = 0; s < 4; ++s) {
+			acc_p = __builtin_amdgcn_mfma_f32_16x16x4f32(t.ar[s], t.br[s], acc_p, 0, 0, 0);
+			acc_r = __builtin_amdgcn_mfma_f32_16x16x4f32(t.ar[s], t.bi[s], acc_r, 0, 0, 0);
+			acc_q = __builtin_amdgcn_mfma_f32_16x16x4f32(t.ai[s], t.bi[s], acc_q, 0, 0, 0);
+			acc_s = __builtin_amdgcn_mfma_f32_16x16x4f32(t.ai[s], t.br[s], acc_s, 0, 0, 0);
+		}
+	};
+	// Slot d of the ring is used, then refilled with the group DEPTH further on (in this order, so that the loaded values
+	// stay in the registers they arrived in).  The loop body is one round over the slots without a branch, which lets
+	// the compiler count the loads in flight instead of waiting for all of them; the refill is unconditional (beyond
+	// this wavefront's range it is not used), and what is left after the last full round follows the loop.
+	int g = g_lo;
+	for (; g + DEPTH <= g_hi; g += DEPTH) {
 #pragma unroll
 		for (int d = 0; d < DEPTH; ++d) {
-			Group cur = buf[d];
+			use(buf[d], g + d);
 			fetch(buf[d], g + d + DEPTH);
-			if (g + d < g_hi) {
-				// the last group of K may reach past its end (selects, no branches: the loads above stay countable)
-				const int left = args.K - ((g + d) * 16 + 4 * q);
-#pragma unroll
-				for (int s = 0; s < 4; ++s) {
-					const bool in = s < left;
-					cur.ar[s] = in ? cur.ar[s] : 0.f;
-					cur.ai[s] = in ? cur.ai[s] : 0.f;
-					cur.br[s] = in ? cur.br[s] : 0.f;
-					cur.bi[s] = in ? cur.bi[s] : 0.f;
-				}
-#pragma unroll
-				for (int s = 0; s < 4; ++s) {
-					// re = Ar Br - (sa Ai)(sb Bi), im = Ar (sb Bi) + (sa Ai) Br
-					acc_re = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.ar[s], cur.br[s], acc_re, 0, 0, 0);
-					acc_im = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.ar[s], sb * cur.bi[s], acc_im, 0, 0, 0);
-					acc_re = __builtin_amdgcn_mfma_f32_16x16x4f32(sq * cur.ai[s], cur.bi[s], acc_re, 0, 0, 0);
-					acc_im = __builtin_amdgcn_mfma_f32_16x16x4f32(sa * cur.ai[s], cur.br[s], acc_im, 0, 0, 0);
-				}
-			}
 		}
 	}
 #pragma unroll
+	for (int d = 0; d < DEPTH - 1; ++d)
+		if (g + d < g_hi) use(buf[d], g + d);
+	// re = Ar Br - (sa Ai)(sb Bi), im = Ar (sb Bi) + (sa Ai) Br
+	const float sa = pb.a_im_sign, sb = pb.b_im_sign, sq = -sa * sb;
+#pragma unroll
 	for (int e = 0; e < 4; ++e) {
-		red[((wave * 2 + 0) * 4 + e) * 64 + lane] = acc_re[e];
-		red[((wave * 2 + 1) * 4 + e) * 64 + lane] = acc_im[e];
+		red[((wave * 2 + 0) * 4 + e) * 64 + lane] = acc_p[e] + sq * acc_q[e];
+		red[((wave * 2 + 1) * 4 + e) * 64 + lane] = sb * acc_r[e] + sa * acc_s[e];
 	}
 	__syncthreads();
 	// the 8 (plane, accumulator register) pairs are added and stored by the first wavefronts, one or two pairs each
@@ -949,9 +975,13 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 
 template <int W, bool A_V4, bool B_V4>
 int launch_skinny(const CgemmArgs &args, bool a_mcontig, bool b_ncontig, int nprob, int batch) {
+	// elements from the first to one past the last of an operand plane
+	const long span_a = a_mcontig ? (args.K - 1) * args.lda + args.M : (args.M - 1) * args.lda + args.K;
+	const long span_b = b_ncontig ? (args.K - 1) * args.ldb + args.N : (args.N - 1) * args.ldb + args.K;
 	auto kern = cgemm_skinny_kernel<W, A_V4, B_V4>;
 	hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, nprob, batch * args.splits), dim3(64 * W), 0, cnet::rt().stream, args,
-			a_mcontig ? args.lda : 1L, a_mcontig ? 1L : args.lda, b_ncontig ? args.ldb : 1L, b_ncontig ? 1L : args.ldb);
+			a_mcontig ? (unsigned) args.lda : 1u, a_mcontig ? 1u : (unsigned) args.lda, b_ncontig ? (unsigned) args.ldb : 1u,
+			b_ncontig ? 1u : (unsigned) args.ldb, (unsigned) (4 * span_a), (unsigned) (4 * span_b));
 	CNET_LAUNCH_CHECK();
 	if (args.splits > 1) {
 		dim3 rgrid((unsigned) ((2L * args.M * args.N + 255) / 256), nprob, batch);
@@ -972,15 +1002,20 @@ bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int npro
 	args.tiles_m = (args.M + 15) / 16;
 	args.tiles_n = (args.N + 15) / 16;
 	const long tiles = (long) args.tiles_m * args.tiles_n * nprob * batch;
-	// Measured against the block kernels with K cut (64 x 784 x 784: 10 against 15 us; 64 x 10 x 784: 9 against 12 us;
-	// 10 x 784 x 64: 4 against 9 us); beyond two tiles per compute unit those win again (256 x 784 x 784: 27 against
-	// 23 us).
+	// Measured against the block kernels with K cut (64 x 784 x 784: 9 against 15 us; 64 x 10 x 784: 8 against 12 us;
+	// 10 x 784 x 64: 4 against 9 us; 256 x 784 x 784, 784 tiles: 19.5 against 23 us); with more than four tiles per
+	// compute unit the block kernels have enough blocks of their own.
 	static const long tile_limit = [] {
 		const char *e = getenv("CNET_CGEMM_SKINNY_TILES");  // tuning override of the largest number of tiles
 		return e ? atol(e) : 0L;
 	}();
-	const long most = tile_limit ? tile_limit : 2L * cnet::rt().prop.multiProcessorCount;
+	const long cus = cnet::rt().prop.multiProcessorCount;
+	const long most = tile_limit ? tile_limit : 4 * cus;
 	if (tiles > most) return false;
+	// the kernel addresses each operand plane with 32-bit byte offsets
+	const long span_a = a_mcontig ? (args.K - 1) * args.lda + args.M : (args.M - 1) * args.lda + args.K;
+	const long span_b = b_ncontig ? (args.K - 1) * args.ldb + args.N : (args.N - 1) * args.ldb + args.K;
+	if (span_a >= (1L << 30) || span_b >= (1L << 30)) return false;
 	args.splits = 1;
 	args.chunks_per_split = 0;
 	args.partial = nullptr;
@@ -988,10 +1023,10 @@ bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int npro
 	args.tail_tiles = args.tail_splits = args.tail_chunks = 0;
 	if (args.K > 1024) {
 		// A long K against a C of few tiles (the weight gradient of a narrow layer over a large batch): slices of K go to
-		// workgroups of their own, at least 256 long and no more slices than keep the launch within the tile limit; the
-		// slices are added in order by splitk_reduce_kernel.
+		// workgroups of their own, at least 256 long and no more slices than give two workgroups to every compute unit;
+		// the slices are added in order by splitk_reduce_kernel.
 		const int groups = (args.K + 15) / 16;
-		const long splits = std::min<long>(most / tiles, groups / 16);
+		const long splits = std::min<long>(2 * cus / tiles, groups / 16);
 		if (splits < 2 || (long) batch * splits > 65535) return false;
 		args.chunks_per_split = (int) ((groups + splits - 1) / splits);
 		if (args.chunks_per_split > 64) return false;  // still longer than 1024 per slice: the block kernels do better
