@@ -21,6 +21,10 @@
 //   one workgroup per C block and per problem (blockIdx.y: the dz and the dzs product of a backward pass are
 //   one launch).  Workgroup ids are dealt round-robin to the 8 XCDs by the hardware; the id is remapped so that
 //   each XCD works on a contiguous strip of C blocks and re-uses operand tiles through its own L2.
+// Three kernels share this file: cgemm_kernel (above; any shape and alignment), cgemm_fast_kernel (16-byte aligned
+// operands and K a multiple of 16: tiles go from global memory straight into LDS; the one the large products run on),
+// and cgemm_skinny_kernel (a C of few 16 x 16 tiles: one tile per workgroup, K shared among its wavefronts).
+// cgemm_dispatch picks among them and pick_tile picks the block shape.
 #include "common.hpp"
 
 #include <algorithm>
