@@ -995,14 +995,15 @@ int launch_skinny(const CgemmArgs &args, bool a_mcontig, bool b_ncontig, int npr
 	return CNET_OK;
 }
 
-// true and *rc set when the product was small enough for cgemm_skinny_kernel
-bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int nprob, int batch, int *rc) {
+// Whether the product is small enough for cgemm_skinny_kernel; if so, `args` gets the tile counts and, for a long K,
+// the number and length of the slices of K (the partial planes are allocated by try_skinny).
+bool plan_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int nprob, int batch, CgemmArgs &args) {
 	static const bool enabled = [] {
 		const char *e = getenv("CNET_CGEMM_SKINNY");  // tuning override: 0 sends every product to the block kernels
 		return !e || atoi(e) != 0;
 	}();
 	if (!enabled || proto.tri || batch > 65535) return false;
-	CgemmArgs args = proto;
+	args = proto;
 	args.tiles_m = (args.M + 15) / 16;
 	args.tiles_n = (args.N + 15) / 16;
 	const long tiles = (long) args.tiles_m * args.tiles_n * nprob * batch;
@@ -1035,6 +1036,24 @@ bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int npro
 		args.chunks_per_split = (int) ((groups + splits - 1) / splits);
 		if (args.chunks_per_split > 64) return false;  // still longer than 1024 per slice: the block kernels do better
 		args.splits = (groups + args.chunks_per_split - 1) / args.chunks_per_split;  // no empty slice
+	}
+	return true;
+}
+
+// expected duration in us of the launch planned by plan_skinny: about 3 us plus 7.5 ns per k of a slice (measured at up
+// to two tiles per compute unit), plus the kernel that adds the slices
+double skinny_us(const CgemmArgs &args, int nprob, int batch) {
+	const long cus = cnet::rt().prop.multiProcessorCount;
+	const long wgs = (long) args.tiles_m * args.tiles_n * nprob * batch * args.splits;
+	const int k_slice = args.splits > 1 ? args.chunks_per_split * 16 : args.K;
+	return (3.0 + 0.0075 * k_slice) * std::max(1.0, wgs / (2.0 * cus)) + (args.splits > 1 ? 6.0 : 0.0);
+}
+
+// true and *rc set when the product was small enough for cgemm_skinny_kernel
+bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int nprob, int batch, int *rc) {
+	CgemmArgs args;
+	if (!plan_skinny(a_mcontig, b_ncontig, proto, nprob, batch, args)) return false;
+	if (args.splits > 1) {
 		args.partial = (float *) cnet::workspace((size_t) args.splits * nprob * batch * 2 * args.M * args.N * sizeof(float));
 		if (!args.partial) {
 			*rc = CNET_ERR_OUT_OF_MEMORY;
@@ -1144,80 +1163,90 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0) {
 	return finish();
 }
 
-template <bool A_MCONTIG, bool B_NCONTIG, int VEC>
-int pick_tile(const CgemmArgs &a, int nprob, int batch) {
+// Block shape for the fast kernel (0: 128 x 128, 1: 64 x 128, 2: 128 x 64, 3: 64 x 64), whether the blocks of a partly
+// filled last round are cut along K (*tail = number of pieces, 0 = no), and the expected duration of the launch in us.
+double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *tail_pieces) {
 	const long cus = cnet::rt().prop.multiProcessorCount;
 	auto blocks = [&](int bm, int bn) {
 		long tn = (a.N + bn - 1) / bn;
 		if (a.tri) tn = (tn + 1) / 2;  // one workgroup per mirrored pair of column blocks
 		return (long) ((a.M + bm - 1) / bm) * tn * nprob * batch;
 	};
+	// tuning override: CNET_CGEMM_TILE = 0 (128x128), 1 (64x128), 2 (128x64), 3 (64x64)
+	static const int forced = [] {
+		const char *e = getenv("CNET_CGEMM_TILE");
+		return e ? atoi(e) : -1;
+	}();
+	// CNET_CGEMM_TAIL = 0 / 1: never / whenever possible cut the blocks of a partly filled last round along K
+	static const int forced_tail = [] {
+		const char *e = getenv("CNET_CGEMM_TAIL");
+		return e ? atoi(e) : -1;
+	}();
+	// Expected duration of the launch with each block shape.  The busiest compute unit works through p = ceil(blocks /
+	// units) blocks, so the launch takes p block-times, whether or not all units have that many and whether or not a
+	// block on the edge of C is full, divided by the efficiency measured for the shape at p blocks per unit on full
+	// blocks (fraction of the fp32 MFMA peak, lowest of three operand layouts, K = 2048).  The table carries what a
+	// formula would miss: a unit holds two workgroups of the larger shapes and three of 64 x 64, a lone workgroup
+	// cannot keep the matrix pipe busy, and with 3 or 5 blocks of 128 x 128 per unit, or 4 of 64 x 64, the hardware
+	// dispatcher leaves some units with one block more than the others.
+	// Alternative for a partly filled last round (q full rounds, r blocks left over): cut those r blocks into s pieces
+	// along K, one piece for each workgroup of the full rounds.  Then the launch takes q block-times plus 1/s of one,
+	// plus the fixed cost of a short piece and of the kernel that adds the pieces.
+	struct Shape {
+		int bm, bn;
+		float eff[8];  // p = 1 .. 8 (8 stands for everything above)
+	};
+	static const Shape shapes[4] = {
+			{128, 128, {0.887f, 0.946f, 0.713f, 0.941f, 0.794f, 0.946f, 0.800f, 0.948f}},
+			{64, 128, {0.883f, 0.935f, 0.931f, 0.943f, 0.938f, 0.943f, 0.943f, 0.944f}},
+			{128, 64, {0.892f, 0.940f, 0.936f, 0.945f, 0.945f, 0.948f, 0.949f, 0.950f}},
+			{64, 64, {0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}}};
+	const double flop_per_us_per_unit = 256.0 * 2.4e3;  // 256 flop per clock at 2.4 GHz
+	const int nchunks = (a.K + KC - 1) / KC;
+	const bool tail_possible = forced_tail != 0 && a.K % KC == 0 && !a.tri && batch == 1;
+	int best = 3, best_tail = 0;
+	double best_us = 1e30;
+	for (int k = 0; k < 4; ++k) {
+		if (forced >= 0 && forced != k) continue;
+		const long nb = blocks(shapes[k].bm, shapes[k].bn);
+		const long per_unit = (nb + cus - 1) / cus;
+		const double block_us = 8.0 * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
+		// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
+		const double bonus = 1.0 - 0.000001 * shapes[k].bm * shapes[k].bn;
+		double us = per_unit * block_us / shapes[k].eff[per_unit < 8 ? per_unit - 1 : 7] * bonus;
+		int tail = 0;
+		const long q = nb / cus, r = nb % cus;
+		if (tail_possible && q >= 1 && r > 0) {
+			// as many pieces as there are workgroups in the full rounds, so that each of them gets one; a piece is at
+			// least three chunks long
+			const int s = (int) std::min<long>(q * cus / r, nchunks / 3);
+			if (s >= 2) {
+				const double tail_us = (q * block_us / shapes[k].eff[q < 8 ? q - 1 : 7] + block_us / s / 0.8 + 20.0) * bonus;
+				if (tail_us < us || forced_tail == 1) {
+					us = tail_us;
+					tail = s;
+				}
+			}
+		}
+		if (us < best_us) {
+			best_us = us;
+			best = k;
+			best_tail = tail;
+		}
+	}
+	*shape = best;
+	*tail_pieces = best_tail;
+	return best_us + 12.0;  // launch, first loads and the write-out of C
+}
+
+template <bool A_MCONTIG, bool B_NCONTIG, int VEC>
+int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 	// the scalar-load fallback (odd shapes) keeps to the small block: its address arithmetic would spill otherwise
 	if constexpr (VEC == 1) {
 		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 	} else {
-		// tuning override: CNET_CGEMM_TILE = 0 (128x128), 1 (64x128), 2 (128x64), 3 (64x64)
-		static const int forced = [] {
-			const char *e = getenv("CNET_CGEMM_TILE");
-			return e ? atoi(e) : -1;
-		}();
-		// CNET_CGEMM_TAIL = 0 / 1: never / whenever possible cut the blocks of a partly filled last round along K
-		static const int forced_tail = [] {
-			const char *e = getenv("CNET_CGEMM_TAIL");
-			return e ? atoi(e) : -1;
-		}();
-		// Expected duration of the launch with each block shape.  The busiest compute unit works through p = ceil(blocks /
-		// units) blocks, so the launch takes p block-times, whether or not all units have that many and whether or not a
-		// block on the edge of C is full, divided by the efficiency measured for the shape at p blocks per unit on full
-		// blocks (fraction of the fp32 MFMA peak, lowest of three operand layouts, K = 2048).  The table carries what a
-		// formula would miss: a unit holds two workgroups of the larger shapes and three of 64 x 64, a lone workgroup
-		// cannot keep the matrix pipe busy, and with 3 or 5 blocks of 128 x 128 per unit, or 4 of 64 x 64, the hardware
-		// dispatcher leaves some units with one block more than the others.
-		// Alternative for a partly filled last round (q full rounds, r blocks left over): cut those r blocks into s pieces
-		// along K, one piece for each workgroup of the full rounds.  Then the launch takes q block-times plus 1/s of one,
-		// plus the fixed cost of a short piece and of the kernel that adds the pieces.
-		struct Shape {
-			int bm, bn;
-			float eff[8];  // p = 1 .. 8 (8 stands for everything above)
-		};
-		static const Shape shapes[4] = {
-				{128, 128, {0.887f, 0.946f, 0.713f, 0.941f, 0.794f, 0.946f, 0.800f, 0.948f}},
-				{64, 128, {0.883f, 0.935f, 0.931f, 0.943f, 0.938f, 0.943f, 0.943f, 0.944f}},
-				{128, 64, {0.892f, 0.940f, 0.936f, 0.945f, 0.945f, 0.948f, 0.949f, 0.950f}},
-				{64, 64, {0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}}};
-		const double flop_per_us_per_unit = 256.0 * 2.4e3;  // 256 flop per clock at 2.4 GHz
-		const int nchunks = (a.K + KC - 1) / KC;
-		const bool tail_possible = forced_tail != 0 && a.K % KC == 0 && !a.tri && batch == 1;
-		int best = 3, best_tail = 0;
-		double best_us = 1e30;
-		for (int k = 0; k < 4; ++k) {
-			if (forced >= 0 && forced != k) continue;
-			const long nb = blocks(shapes[k].bm, shapes[k].bn);
-			const long per_unit = (nb + cus - 1) / cus;
-			const double block_us = 8.0 * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
-			// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
-			const double bonus = 1.0 - 0.000001 * shapes[k].bm * shapes[k].bn;
-			double us = per_unit * block_us / shapes[k].eff[per_unit < 8 ? per_unit - 1 : 7] * bonus;
-			int tail = 0;
-			const long q = nb / cus, r = nb % cus;
-			if (tail_possible && q >= 1 && r > 0) {
-				// as many pieces as there are workgroups in the full rounds, so that each of them gets one; a piece is at
-				// least three chunks long
-				const int s = (int) std::min<long>(q * cus / r, nchunks / 3);
-				if (s >= 2) {
-					const double tail_us = (q * block_us / shapes[k].eff[q < 8 ? q - 1 : 7] + block_us / s / 0.8 + 20.0) * bonus;
-					if (tail_us < us || forced_tail == 1) {
-						us = tail_us;
-						tail = s;
-					}
-				}
-			}
-			if (us < best_us) {
-				best_us = us;
-				best = k;
-				best_tail = tail;
-			}
-		}
+		int best, best_tail;
+		plan_blocks(a, nprob, batch, &best, &best_tail);
 		if (best == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
 		if (best == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
 		if (best == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
@@ -1235,6 +1264,38 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 	if (a.K <= 0) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: K must be positive");
 	int rc = CNET_OK;
 	if (try_skinny(a_mcontig, b_ncontig, a, nprob, batch, &rc)) return rc;
+	// A C that is a few columns wider than a multiple of the block width (784 = 12 x 64 + 16) costs a whole extra column
+	// of blocks.  If the cost model says so, the product is done as two: the columns up to that multiple by the block
+	// kernels, the narrow rest by the small-C kernel.  The two write disjoint columns of C.
+	static const bool split_cols = [] {
+		const char *e = getenv("CNET_CGEMM_COLSPLIT");  // tuning override: 0 never splits
+		return !e || atoi(e) != 0;
+	}();
+	const int rest = a.N % 64;
+	if (split_cols && !a.tri && batch == 1 && a.N > 64 && rest != 0 && rest <= 32 && a.K % KC == 0) {
+		CgemmArgs left = a, right = a, planned;
+		left.N = a.N - rest;
+		right.N = rest;
+		for (int q = 0; q < nprob; ++q) {
+			const long shift = b_ncontig ? left.N : (long) left.N * a.ldb;
+			right.p[q].b_re += shift;
+			right.p[q].b_im += shift;
+			right.p[q].c_re += left.N;
+			right.p[q].c_im += left.N;
+		}
+		if (plan_skinny(a_mcontig, b_ncontig, right, nprob, batch, planned)) {
+			int shape, tail;
+			const double whole = plan_blocks(a, nprob, batch, &shape, &tail);
+			const double parts = plan_blocks(left, nprob, batch, &shape, &tail) + skinny_us(planned, nprob, batch);
+			if (parts < whole) {
+				// one after the other on the compute stream: run side by side on two streams the narrow part's
+				// workgroups took slots from the first round of the block kernel and the pair got slower (842 against
+				// 773 us per step of the 784 -> 10 net at batch 4096)
+				rc = cgemm_dispatch(a_mcontig, b_ncontig, left, nprob, batch);
+				return rc != CNET_OK ? rc : cgemm_dispatch(a_mcontig, b_ncontig, right, nprob, batch);
+			}
+		}
+	}
 	// float4 path: every contiguous run starts 16-byte aligned and has a length that is a multiple of 4
 	bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (a.stride_a % 4 == 0) && (a.stride_b % 4 == 0);
 	vec = vec && (a_mcontig ? a.M % 4 == 0 : a.K % 4 == 0) && (b_ncontig ? a.N % 4 == 0 : a.K % 4 == 0);

@@ -127,10 +127,11 @@ def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(4, 4, 16), (132, 200, 64), (260, 68, 48), (700, 388, 32), (1028, 516, 80), (68, 1300, 160),
-                                   (4100, 1028, 16), (61, 67, 64)])
+                                   (4100, 1028, 16), (61, 67, 64), (4096, 784, 256)])
 def test_cgemm_blocks_on_the_edge_of_c(gpu, port, M, N, K):
     """K a multiple of 16 with M and N that are not multiples of any block shape: blocks that hang over the edge of C
-    read the last valid rows again and must store nothing outside C."""
+    read the last valid rows again and must store nothing outside C.  The last shape (784 = 12 x 64 + 16 columns) is one
+    the library computes as two products, columns 0..767 by the block kernel and the 16 left over by the small-C kernel."""
     _check_all_layouts(port, M, N, K)
 
 
