@@ -1185,22 +1185,34 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 	// Expected duration of the launch with each block shape.  The busiest compute unit works through p = ceil(blocks /
 	// units) blocks, so the launch takes p block-times, whether or not all units have that many and whether or not a
 	// block on the edge of C is full, divided by the efficiency measured for the shape at p blocks per unit on full
-	// blocks (fraction of the fp32 MFMA peak, lowest of three operand layouts, K = 2048).  The table carries what a
-	// formula would miss: a unit holds two workgroups of the larger shapes and three of 64 x 64, a lone workgroup
-	// cannot keep the matrix pipe busy, and with 3 or 5 blocks of 128 x 128 per unit, or 4 of 64 x 64, the hardware
-	// dispatcher leaves some units with one block more than the others.
+	// blocks (fraction of the fp32 MFMA peak, lowest of three operand layouts), at K = 512 and at K = 2048; in between
+	// and beyond, 1 / efficiency is taken as linear in 1 / K (a loop part and a fixed part per block: first loads and
+	// the write-out of C weigh more on a short K, and more on the small shapes).  The tables carry what a formula would
+	// miss: a unit holds two workgroups of the larger shapes and three of 64 x 64, a lone workgroup cannot keep the
+	// matrix pipe busy, and with 3 or 5 blocks of 128 x 128 per unit, or 4 of 64 x 64, the hardware dispatcher leaves
+	// some units with one block more than the others.
 	// Alternative for a partly filled last round (q full rounds, r blocks left over): cut those r blocks into s pieces
 	// along K, one piece for each workgroup of the full rounds.  Then the launch takes q block-times plus 1/s of one,
 	// plus the fixed cost of a short piece and of the kernel that adds the pieces.
 	struct Shape {
 		int bm, bn;
-		float eff[8];  // p = 1 .. 8 (8 stands for everything above)
+		float eff_k512[8], eff_k2048[8];  // p = 1 .. 8 (8 stands for everything above)
 	};
 	static const Shape shapes[4] = {
-			{128, 128, {0.887f, 0.946f, 0.713f, 0.941f, 0.794f, 0.946f, 0.800f, 0.948f}},
-			{64, 128, {0.883f, 0.935f, 0.931f, 0.943f, 0.938f, 0.943f, 0.943f, 0.944f}},
-			{128, 64, {0.892f, 0.940f, 0.936f, 0.945f, 0.945f, 0.948f, 0.949f, 0.950f}},
-			{64, 64, {0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}}};
+			{128, 128, {0.834f, 0.911f, 0.743f, 0.918f, 0.777f, 0.917f, 0.785f, 0.918f},
+					{0.887f, 0.946f, 0.713f, 0.941f, 0.794f, 0.946f, 0.800f, 0.948f}},
+			{64, 128, {0.786f, 0.868f, 0.876f, 0.890f, 0.894f, 0.899f, 0.901f, 0.903f},
+					{0.883f, 0.935f, 0.931f, 0.943f, 0.938f, 0.943f, 0.943f, 0.944f}},
+			{128, 64, {0.786f, 0.861f, 0.883f, 0.888f, 0.898f, 0.900f, 0.902f, 0.905f},
+					{0.892f, 0.940f, 0.936f, 0.945f, 0.945f, 0.948f, 0.949f, 0.950f}},
+			{64, 64, {0.768f, 0.840f, 0.873f, 0.723f, 0.884f, 0.866f, 0.870f, 0.874f},
+					{0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}}};
+	auto eff = [&](int k, long p) {
+		const int i = p < 8 ? (int) p - 1 : 7;
+		const double inv512 = 1.0 / shapes[k].eff_k512[i], inv2048 = 1.0 / shapes[k].eff_k2048[i];
+		const double slope = (inv512 - inv2048) / (1.0 / 512 - 1.0 / 2048);  // per 1 / K
+		return 1.0 / std::max(1.0, inv2048 + slope * (1.0 / a.K - 1.0 / 2048));
+	};
 	const double flop_per_us_per_unit = 256.0 * 2.4e3;  // 256 flop per clock at 2.4 GHz
 	const int nchunks = (a.K + KC - 1) / KC;
 	const bool tail_possible = forced_tail != 0 && a.K % KC == 0 && !a.tri && batch == 1;
@@ -1213,7 +1225,7 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 		const double block_us = 8.0 * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
 		// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
 		const double bonus = 1.0 - 0.000001 * shapes[k].bm * shapes[k].bn;
-		double us = per_unit * block_us / shapes[k].eff[per_unit < 8 ? per_unit - 1 : 7] * bonus;
+		double us = per_unit * block_us / eff(k, per_unit) * bonus;
 		int tail = 0;
 		const long q = nb / cus, r = nb % cus;
 		if (tail_possible && q >= 1 && r > 0) {
@@ -1221,7 +1233,7 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 			// least three chunks long
 			const int s = (int) std::min<long>(q * cus / r, nchunks / 3);
 			if (s >= 2) {
-				const double tail_us = (q * block_us / shapes[k].eff[q < 8 ? q - 1 : 7] + block_us / s / 0.8 + 20.0) * bonus;
+				const double tail_us = (q * block_us / eff(k, q) + block_us / s / 0.8 + 20.0) * bonus;
 				if (tail_us < us || forced_tail == 1) {
 					us = tail_us;
 					tail = s;
