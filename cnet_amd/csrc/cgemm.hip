@@ -1186,7 +1186,7 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 	// units) blocks, so the launch takes p block-times, whether or not all units have that many and whether or not a
 	// block on the edge of C is full, divided by the efficiency measured for the shape at p blocks per unit on full
 	// blocks (fraction of the fp32 MFMA peak, lowest of three operand layouts), at K = 512 and at K = 2048; in between
-	// and beyond, 1 / efficiency is taken as linear in 1 / K (a loop part and a fixed part per block: first loads and
+	// and below, 1 / efficiency is taken as linear in 1 / K (a loop part and a fixed part per block: first loads and
 	// the write-out of C weigh more on a short K, and more on the small shapes).  The tables carry what a formula would
 	// miss: a unit holds two workgroups of the larger shapes and three of 64 x 64, a lone workgroup cannot keep the
 	// matrix pipe busy, and with 3 or 5 blocks of 128 x 128 per unit, or 4 of 64 x 64, the hardware dispatcher leaves
@@ -1207,11 +1207,18 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 					{0.892f, 0.940f, 0.936f, 0.945f, 0.945f, 0.948f, 0.949f, 0.950f}},
 			{64, 64, {0.768f, 0.840f, 0.873f, 0.723f, 0.884f, 0.866f, 0.870f, 0.874f},
 					{0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}}};
+	static const bool k_dependent = [] {
+		const char *e = getenv("CNET_CGEMM_KMODEL");  // tuning override: 0 uses the K = 2048 table for every K
+		return !e || atoi(e) != 0;
+	}();
 	auto eff = [&](int k, long p) {
 		const int i = p < 8 ? (int) p - 1 : 7;
+		if (!k_dependent) return (double) shapes[k].eff_k2048[i];
 		const double inv512 = 1.0 / shapes[k].eff_k512[i], inv2048 = 1.0 / shapes[k].eff_k2048[i];
 		const double slope = (inv512 - inv2048) / (1.0 / 512 - 1.0 / 2048);  // per 1 / K
-		return 1.0 / std::max(1.0, inv2048 + slope * (1.0 / a.K - 1.0 / 2048));
+		// beyond K = 2048 the K = 2048 table stands: the straight line would credit the small shapes with a loop
+		// efficiency above that of the large ones
+		return 1.0 / (inv2048 + slope * std::max(0.0, 1.0 / a.K - 1.0 / 2048));
 	};
 	const double flop_per_us_per_unit = 256.0 * 2.4e3;  // 256 flop per clock at 2.4 GHz
 	const int nchunks = (a.K + KC - 1) / KC;
