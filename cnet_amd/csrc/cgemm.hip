@@ -68,7 +68,23 @@ struct CgemmArgs {
 	// every compute unit gets the same share of the tail wherever the hardware places the workgroups.  A piece writes its
 	// whole block to partial[tail block][piece][re, im][BM][BN]; tail_reduce_kernel adds the pieces in order.
 	int tail_tiles, tail_splits, tail_chunks, nprob;
+	// Mirror: one problem is computed and its result also written, conjugated, to the C planes of p[1] (honouring
+	// `accumulate` there as well).  The backward passes use it when the incoming dz* gradient is the conjugate of the dz
+	// gradient, as it is under every real-valued loss: the dz* product is then the conjugate of the dz product (the same
+	// sums with signs applied exactly) and need not be computed.  Not combined with a strided batch.
+	int mirror;
 };
+
+// the conjugate of (vr, vi) into element `off` of the mirror planes
+__device__ __forceinline__ void mirror_store(const CgemmArgs &args, long off, float vr, float vi) {
+	float mr = vr, mi = -vi;
+	if (args.accumulate) {
+		mr += args.p[1].c_re[off];
+		mi += args.p[1].c_im[off];
+	}
+	args.p[1].c_re[off] = mr;
+	args.p[1].c_im[off] = mi;
+}
 
 // Which block of C (per problem) a linear block number stands for: walks groups of 8 block rows column by column, after
 // spreading consecutive workgroup numbers (which the hardware deals round-robin to the XCDs) over contiguous strips.
@@ -361,6 +377,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 				if (row < M) {
 					const long off = (long) row * ldc + col;
 					float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
+					if (args.mirror && args.splits == 1) mirror_store(args, (long) row * args.ldc + col, vr, vi);
 					if (accumulate) {
 						vr += pb.c_re[off];
 						vi += pb.c_im[off];
@@ -759,6 +776,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	// loop, where the registers are full, and spills them.
 	int r_st = r, h_st = h;
 	asm volatile("" : "+v"(r_st), "+v"(h_st));
+	const bool mirror_now = args.mirror && piece < 0 && args.splits == 1;  // partial blocks are mirrored when they are added up
 
 #pragma unroll
 	for (int i = 0; i < TM; ++i)
@@ -780,6 +798,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 						vr = acc_re[i][j][e];
 						vi = mode == 3 ? -acc_im[i][j][e] : acc_im[i][j][e];
 					}
+					if (mirror_now) mirror_store(args, (long) row * args.ldc + col, vr, vi);
 					if (accumulate) {
 						vr += pb.c_re[off];
 						vi += pb.c_im[off];
@@ -805,6 +824,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(CgemmArgs args, int 
 	float v = cnet::ordered_sum(first, (long) nprob * nbatch * 2 * plane, args.splits);
 	float *c = (part ? args.p[prob].c_im : args.p[prob].c_re) + (long) b * args.stride_c + row * args.ldc + col;
 	*c = args.accumulate ? *c + v : v;
+	if (args.mirror) {
+		float *m = (part ? args.p[1].c_im : args.p[1].c_re) + row * args.ldc + col;
+		const float mv = part ? -v : v;
+		*m = args.accumulate ? *m + mv : mv;
+	}
 }
 
 // C (+)= sum over the K pieces of each tail block, added in piece order.  blockIdx.x = tail block, blockIdx.y = a slice
@@ -827,6 +851,11 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(CgemmArgs args) {
 		const float v = cnet::ordered_sum(first + idx, 2L * BM * BN, args.tail_splits);
 		float *c = (part ? args.p[prob].c_im : args.p[prob].c_re) + (long) row * args.ldc + col;
 		*c = args.accumulate ? *c + v : v;
+		if (args.mirror) {
+			float *m = (part ? args.p[1].c_im : args.p[1].c_re) + (long) row * args.ldc + col;
+			const float mv = part ? -v : v;
+			*m = args.accumulate ? *m + mv : mv;
+		}
 	}
 }
 
@@ -973,6 +1002,11 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 		if (row < args.M && col < args.N) {
 			float *dst = (part ? pb.c_im : pb.c_re) + (long) row * ldc + col;
 			*dst = accumulate ? *dst + v : v;
+			if (args.mirror && args.splits == 1) {
+				float *m = (part ? args.p[1].c_im : args.p[1].c_re) + (long) row * args.ldc + col;
+				const float mv = part ? -v : v;
+				*m = args.accumulate ? *m + mv : mv;
+			}
 		}
 	}
 }
@@ -1295,12 +1329,16 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 		CgemmArgs left = a, right = a, planned;
 		left.N = a.N - rest;
 		right.N = rest;
-		for (int q = 0; q < nprob; ++q) {
+		for (int q = 0; q < 2; ++q) {
 			const long shift = b_ncontig ? left.N : (long) left.N * a.ldb;
-			right.p[q].b_re += shift;
-			right.p[q].b_im += shift;
-			right.p[q].c_re += left.N;
-			right.p[q].c_im += left.N;
+			if (q < nprob) {
+				right.p[q].b_re += shift;
+				right.p[q].b_im += shift;
+			}
+			if (q < nprob || a.mirror) {  // the planes of p[1] are written by a mirrored product as well
+				right.p[q].c_re += left.N;
+				right.p[q].c_im += left.N;
+			}
 		}
 		if (plan_skinny(a_mcontig, b_ncontig, right, nprob, batch, planned)) {
 			int shape, tail;
@@ -1335,10 +1373,12 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 // Used by cdft.hip
 int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
 		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
-		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri) {
+		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri, bool mirror) {
 	if (tri && N != K) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: a triangular operand must be square");
+	if (mirror && nprob != 1) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: a mirrored product is one problem");
 	CgemmArgs a;
 	a.tri = tri;
+	a.mirror = mirror ? 1 : 0;
 	for (int q = 0; q < nprob; ++q) {
 		a.p[q].a_re = a_re[q];
 		a.p[q].a_im = a_im[q];
@@ -1349,7 +1389,13 @@ int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, c
 		a.p[q].a_im_sign = 1.0f;
 		a.p[q].b_im_sign = conj_b[q] ? -1.0f : 1.0f;
 	}
-	if (nprob == 1) a.p[1] = a.p[0];
+	if (nprob == 1) {
+		a.p[1] = a.p[0];
+		if (mirror) {  // the planes that receive the conjugate of the product
+			a.p[1].c_re = c_re[1];
+			a.p[1].c_im = c_im[1];
+		}
+	}
 	a.M = M;
 	a.N = N;
 	a.K = K;
@@ -1379,7 +1425,7 @@ int cnet_cgemm(int a_kmajor, int b_kmajor, int conj_b, int M, int N, int K, cons
 	const float *ar[2] = {a_re, a_re}, *ai[2] = {a_im, a_im}, *br[2] = {b_re, b_re}, *bi[2] = {b_im, b_im};
 	float *cr[2] = {c_re, c_re}, *ci[2] = {c_im, c_im};
 	bool cj[2] = {conj_b != 0, conj_b != 0};
-	return cgemm_pair(a_kmajor != 0, b_kmajor != 0, 1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, accumulate, 0);
+	return cgemm_pair(a_kmajor != 0, b_kmajor != 0, 1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, accumulate, 0, false);
 }
 
 int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M, int N, int K, const float *a_re,
@@ -1393,6 +1439,7 @@ int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M
 	CNET_CHECK_ARG(stride_a >= 0 && stride_b >= 0 && (batch == 1 || stride_c >= (int64_t) M * ldc - (ldc - N)));
 	CgemmArgs a;
 	a.tri = 0;
+	a.mirror = 0;
 	a.p[0].a_re = a_re;
 	a.p[0].a_im = a_im;
 	a.p[0].b_re = b_re;
@@ -1436,7 +1483,7 @@ int cnet_clinear_bwd_input(const float *g_dz_re, const float *g_dz_im, const flo
 	const float *br[2] = {w_re, w_re}, *bi[2] = {w_im, w_im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, true};
-	return cgemm_pair(false, true, 2, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0);
+	return cgemm_pair(false, true, 2, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0, false);
 }
 
 int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,
@@ -1453,7 +1500,38 @@ int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const fl
 	const float *br[2] = {x_re, x_re}, *bi[2] = {x_im, x_im};
 	float *cr[2] = {dw_dz_re, dw_dzs_re}, *ci[2] = {dw_dz_im, dw_dzs_im};
 	bool cj[2] = {false, true};
-	return cgemm_pair(true, true, 2, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0);
+	return cgemm_pair(true, true, 2, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0, false);
+}
+
+int cnet_clinear_bwd_input_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *w_re, const float *w_im,
+		int64_t ldw, float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int B, int K, int N,
+		int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && K >= 0 && N > 0);
+	if (B == 0 || K == 0) return CNET_OK;
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && w_re && w_im && dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
+	CNET_CHECK_ARG(ldg >= N && ldw >= K && lddx >= K);
+	// dx = g * w as in cnet_clinear_bwd_input; dx* = conj(g) * conj(w) is its conjugate and is written, not computed
+	const float *ar[2] = {g_dz_re, g_dz_re}, *ai[2] = {g_dz_im, g_dz_im};
+	const float *br[2] = {w_re, w_re}, *bi[2] = {w_im, w_im};
+	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
+	bool cj[2] = {false, false};
+	return cgemm_pair(false, true, 1, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0, true);
+}
+
+int cnet_clinear_bwd_weight_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *x_re, const float *x_im,
+		int64_t ldx, float *dw_dz_re, float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im, int64_t lddw, int B, int K, int N,
+		int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B > 0 && K >= 0 && N >= 0);
+	if (N == 0 || K == 0) return CNET_OK;
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && x_re && x_im && dw_dz_re && dw_dz_im && dw_dzs_re && dw_dzs_im);
+	CNET_CHECK_ARG(ldg >= N && ldx >= K && lddw >= K);
+	const float *ar[2] = {g_dz_re, g_dz_re}, *ai[2] = {g_dz_im, g_dz_im};
+	const float *br[2] = {x_re, x_re}, *bi[2] = {x_im, x_im};
+	float *cr[2] = {dw_dz_re, dw_dzs_re}, *ci[2] = {dw_dz_im, dw_dzs_im};
+	bool cj[2] = {false, false};
+	return cgemm_pair(true, true, 1, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0, true);
 }
 
 }  // extern "C"

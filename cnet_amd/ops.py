@@ -116,12 +116,29 @@ def linear_bwd_weight(g, x, dw, accumulate=0):
     call("cnet_clinear_bwd_weight", *g.p(), g.ld, *x.p(), x.ld, *dw.p(), dw.ld, g.rows, x.cols, g.cols, accumulate)
 
 
+def linear_bwd_input_sym(g, w, dx, accumulate=0):
+    """g is a Grad whose dz* planes are the conjugate of its dz planes; only the dz planes are read."""
+    call("cnet_clinear_bwd_input_sym", *g.p()[:2], g.ld, *w.p(), w.ld, *dx.p(), dx.ld, g.rows, w.cols, w.rows, accumulate)
+
+
+def linear_bwd_weight_sym(g, x, dw, accumulate=0):
+    call("cnet_clinear_bwd_weight_sym", *g.p()[:2], g.ld, *x.p(), x.ld, *dw.p(), dw.ld, g.rows, x.cols, g.cols, accumulate)
+
+
 def dft_fwd(x, y, accumulate=0):
     call("cnet_cdft_fwd", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols, accumulate)
 
 
 def dft_bwd(g, dx, accumulate=0):
     call("cnet_cdft_bwd", *g.p(), g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
+
+
+def dft_bwd_sym(g, dx, accumulate=0):
+    call("cnet_cdft_bwd_sym", *g.p()[:2], g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
+
+
+def triang_dft_bwd_sym(g, dx, accumulate=0):
+    call("cnet_ctriang_dft_bwd_sym", *g.p()[:2], g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
 
 
 def triang_dft_fwd(x, y, accumulate=0):

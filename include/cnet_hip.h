@@ -145,6 +145,19 @@ int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const fl
                             float *dw_dz_re, float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im, int64_t lddw,
                             int B, int K, int N, int accumulate);
 
+/* The same two backward passes for a gradient pair that is conjugate, g.dzs == conj(g.dz), as the loss layers produce it
+ * (CrossEntropy impl/crossent.h, L2Out impl/l2out.h: the loss is real) and every layer's backward pass hands it on: then
+ * g.dzs * conj(w) == conj(g.dz * w), in floating point as well (same sums, signs applied exactly), so one product is
+ * computed and written twice, once conjugated.  Same results as cnet_clinear_bwd_input / _bwd_weight on such a pair (to
+ * rounding: half as many blocks may take another block shape) at half the matrix work.  Replace the same upstream
+ * functions (gpu/reduce.cpp:532-604, gpu/reducegrad.cpp:288-322); the caller vouches for the pair. */
+int cnet_clinear_bwd_input_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *w_re, const float *w_im,
+                               int64_t ldw, float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im,
+                               int64_t lddx, int B, int K, int N, int accumulate);
+int cnet_clinear_bwd_weight_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *x_re, const float *x_im,
+                                int64_t ldx, float *dw_dz_re, float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im,
+                                int64_t lddw, int B, int K, int N, int accumulate);
+
 /* ---- FourierTrans as dense complex GEMM: replaces FourierGpu::gpu_fft_forward / gpu_fft_backward
  *      (gpu/reduce.cpp:25-35,160-187,382-393; gpu/reducegrad.cpp:45-48,324-336) and the root-table upload
  *      u_roots_allocate_and_copy_on_gpu (gpu/allocator.h:389-407).  CPU twin impl/ft.h:37-80.
@@ -162,6 +175,10 @@ int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re
 int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
                   float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
                   int B, int n, int accumulate);      /* dx.dz = g.dz * F ; dx.dzs = g.dzs * conj(F) */
+/* for a conjugate gradient pair (see cnet_clinear_bwd_input_sym): dx.dz = g.dz * F, dx.dzs = its conjugate
+ * (gpu/reducegrad.cpp:324-336 upstream) */
+int cnet_cdft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, float *dx_dz_re, float *dx_dz_im,
+                      float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int B, int n, int accumulate);
 
 /* ---- TriangFourier: the DFT sums restricted to in <= out, y_o = (1/sqrt n) sum_{i <= o} x_i w^{i o}; CPU twin
  *      impl/ft.h:139-189 (upstream has no device kernel for it: its GPU tests expect "not supported",
@@ -173,6 +190,9 @@ int cnet_ctriang_dft_fwd(const float *x_re, const float *x_im, int64_t ldx, floa
 int cnet_ctriang_dft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
                          float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
                          int B, int n, int accumulate);
+/* for a conjugate gradient pair (see cnet_clinear_bwd_input_sym); CPU twin impl/ft.h:164-189 */
+int cnet_ctriang_dft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, float *dx_dz_re, float *dx_dz_im,
+                             float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int B, int n, int accumulate);
 
 /* ---- Hadamard: replaces gpu_hadamard_forward / _backward (gpu/kernels.cpp:204-274), CPU twin impl/hadamard.h:34-68.
  * y = u .* v.  ldv == 0: v is one parameter row shared by all rows and dv is the sum over rows. */

@@ -349,3 +349,35 @@ def test_wirtinger_gradients_by_finite_differences(port, kinds):
 @pytest.mark.parametrize("kinds", [[ob.CROSSENT], [ob.LINEAR, ob.GELU, ob.CROSSENT], [ob.FOURIER, ob.HADAMARD, ob.CROSSENT]])
 def test_cross_entropy_gradient_by_finite_differences(port, kinds):
     _fd_check(port, _chain(kinds), 6, seed=11, label=2)
+
+
+def _conj_gap(g4):
+    a, b = g4[0] + 1j * g4[1], g4[2] + 1j * g4[3]
+    return float(np.abs(b - np.conj(a)).max() / max(np.abs(a).max(), 1e-30))
+
+
+def test_gradient_pairs_are_conjugate_under_a_real_loss(port):
+    """The loss of CrossEntropy and L2Out is real, so dL/dz* = conj(dL/dz): the loss layers write such a pair exactly, and
+    every backward pass maps a conjugate pair to a conjugate pair (exactly where the dz and dz* formulas mirror each other
+    operation by operation, to rounding otherwise).  The *_sym entry points of the device library rest on this."""
+    rs = np.random.RandomState(5)
+    B, n = 6, 12
+    f32 = lambda *s: rs.randn(*s).astype(np.float32)  # noqa: E731
+    zr, zi, xr, xi = f32(B, n), f32(B, n), f32(B, n), f32(B, n)
+    labels = rs.randint(0, n, B).astype(np.int32)
+    sources = {"crossent": port.crossent_bwd(zr, zi, labels), "l2out": port.l2out_bwd(zr, zi)}
+    for name, g in sources.items():
+        assert _conj_gap(g) == 0.0, name
+        g = [np.ascontiguousarray(p) for p in g]
+        wr, wi = f32(n, n), f32(n, n)
+        dx, dw = port.linear_bwd(xr, xi, wr, wi, g)
+        assert _conj_gap(dx) == 0.0 and _conj_gap(dw) == 0.0, name
+        assert _conj_gap(port.dft_bwd(g)) < 1e-6, name
+        assert _conj_gap(port.triang_bwd(g)) < 1e-6, name
+        du, dv = port.hadamard_bwd(xr, xi, zr, zi, g)
+        assert _conj_gap(du) < 1e-6 and _conj_gap(dv) < 1e-6, name
+        assert _conj_gap(port.gelu_bwd(xr, xi, g)) < 1e-6, name
+        assert _conj_gap(port.crelu_bwd(xr, xi, g)) == 0.0, name
+        assert _conj_gap(port.softmax_bwd(xr, xi, g)) < 1e-6, name
+        for part in port.residual_bwd(g):
+            assert _conj_gap(part) == 0.0, name
