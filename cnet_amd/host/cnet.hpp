@@ -624,6 +624,7 @@ class CNet {
 	};
 	StepGraphs graphs_[2];
 	bool use_graphs_ = false;
+	bool conjugate_gradients_ = true;
 	std::vector<const float *> gather_src_;  // pending dz* gathers of the input functions (see nodeBackward)
 	std::vector<float *> gather_dst_;
 	std::vector<int64_t> gather_len_;
@@ -1069,6 +1070,13 @@ private:
 			case isLinear: {
 				CFunc::Slot &w = f->slots_[1];
 				const int K = a.len, N = f->out_size_;
+				if (conjugate_gradients_) {  // dz* = conj(dz): one product each, written to both pairs of planes
+					ck(cnet_clinear_bwd_input_sym(u.g(0), u.g(1), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K, rows, K, N,
+							acc), "cnet_clinear_bwd_input_sym");
+					ck(cnet_clinear_bwd_weight_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K, rows, K, N,
+							acc), "cnet_clinear_bwd_weight_sym");
+					break;
+				}
 				ck(cnet_clinear_bwd_input(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K,
 						rows, K, N, acc), "cnet_clinear_bwd_input");
 				ck(cnet_clinear_bwd_weight(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K,
@@ -1076,12 +1084,19 @@ private:
 				break;
 			}
 			case isFourier:
-				ck(cnet_cdft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
-						"cnet_cdft_bwd");
+				if (conjugate_gradients_)
+					ck(cnet_cdft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc), "cnet_cdft_bwd_sym");
+				else
+					ck(cnet_cdft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
+							"cnet_cdft_bwd");
 				break;
 			case isTrianFourier:
-				ck(cnet_ctriang_dft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
-						"cnet_ctriang_dft_bwd");
+				if (conjugate_gradients_)
+					ck(cnet_ctriang_dft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
+							"cnet_ctriang_dft_bwd_sym");
+				else
+					ck(cnet_ctriang_dft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
+							"cnet_ctriang_dft_bwd");
 				break;
 			case isCrelu:
 				ck(cnet_crelu_bwd(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len,
@@ -1438,6 +1453,16 @@ public:
 		use_graphs_ = on;
 	}
 	bool usingGraphs() const { return use_graphs_; }
+	// Every backward pass starts at a CrossEntropy or an L2Out, whose loss is real: the gradient with respect to z* is then
+	// the conjugate of the gradient with respect to z at every node, and the matrix products of Linear, FourierTrans and
+	// TriangFourier compute the dz half only and write its conjugate to the dz* planes (half the matrix work of a backward
+	// pass; same results to rounding).  Off: both halves are computed, as upstream does.  Recordings are dropped, since
+	// they hold the kernels of the other setting.
+	void conjugateGradients(bool on) {
+		if (on != conjugate_gradients_ && batch_) dropGraphs();
+		conjugate_gradients_ = on;
+	}
+	bool conjugateGradients() const { return conjugate_gradients_; }
 	// The Adam-style step of upstream GpuNet::adamUpdate (gpu/gpu_func.h:503-510, gpu/kernels.cpp:494-514) on every input
 	// function: the first moment lives in the node's dz planes, dz* is cleared, dz is kept.
 	void gpuAdamUpdate(float l_rate, float beta, int t) {

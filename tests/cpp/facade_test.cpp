@@ -865,12 +865,15 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs) 
 		return;
 	}
 	SyntheticReader data(n, 3 * B + 7, classes);
-	constexpr int MODES = 5;  // 4: prefetch + gpuTrainStep (the whole step as one recorded graph)
+	// 4: prefetch + gpuTrainStep (the whole step as one recorded graph); 5: prefetch with both halves of every gradient
+	// pair computed by matrix products (conjugateGradients(false), what upstream does)
+	constexpr int MODES = 6;
 	std::vector<float> losses[MODES];
 	std::vector<float> weights[MODES];
-	double ms[MODES] = {0, 0, 0, 0, 0};
-	for (int mode = 0; mode < (with_graphs ? MODES : 2); ++mode) {
-		const bool prefetch = mode == 1 || mode == 2 || mode == 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4;
+	double ms[MODES] = {0, 0, 0, 0, 0, 0};
+	for (int mode = 0; mode < MODES; ++mode) {
+		if (!with_graphs && mode >= 2 && mode <= 4) continue;
+		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4;
 		CNet net;
 		int inp, outp;
 		build_readme(net, n, classes, &inp, &outp);
@@ -881,6 +884,7 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs) 
 		InputBatch ring[3] = {InputBatch(B, n), InputBatch(B, n), InputBatch(B, n)};
 		if (mode == 0 && !timing_only) expect("batches built after cnet_init are page-locked", ring[0].isPinned());
 		if (graphs) net.useGraphs(true);
+		if (mode == 5) net.conjugateGradients(false);
 		net.sync();
 		auto t0 = std::chrono::steady_clock::now();
 		// With prefetch the host runs two batches ahead: while the device computes step s, batch s+1 (assembled during
@@ -954,14 +958,25 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs) 
 		expect("losses identical with gpuTrainStep (one recorded graph per step)", losses[0] == losses[4]);
 		expect("weights identical with gpuTrainStep", weights[0] == weights[4]);
 		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
+		// dz* planes written as the conjugate of the dz product against dz* planes computed by a product of their own
+		double worst = 0, num = 0, den = 0;
+		for (size_t k = 0; k < losses[1].size(); ++k)
+			worst = std::max(worst, (double) std::fabs(losses[1][k] - losses[5][k]) / std::fabs(losses[5][k]));
+		for (size_t k = 0; k < weights[1].size(); ++k) {
+			num += ((double) weights[1][k] - weights[5][k]) * ((double) weights[1][k] - weights[5][k]);
+			den += (double) weights[5][k] * weights[5][k];
+		}
+		report("losses with conjugate gradient pairs written, not computed (relative, worst step)", worst, 1e-5);
+		report("weights after training with conjugate gradient pairs written, not computed (relative Frobenius)", std::sqrt(num / den), 1e-5);
+		expect("both settings trained the same number of weights", weights[1].size() == weights[5].size() && !weights[5].empty());
 	}
 	printf("{\"workload\": \"README net 784 -> 10, SGD, batches from a BatchedDataReader\", \"batch\": %d, \"steps\": %d, "
 		   "\"ms_per_step_copy_in_forward\": %.3f, \"ms_per_step_prefetch\": %.3f, \"ms_per_step_prefetch_graphs\": %.3f, "
 		   "\"ms_per_step_graphs\": %.3f, \"samples_per_sec_copy_in_forward\": %.1f, \"samples_per_sec_prefetch\": %.1f, "
 		   "\"samples_per_sec_prefetch_graphs\": %.1f, \"ms_per_step_train_step_graph\": %.3f, \"samples_per_sec_train_step_graph\": %.1f, "
-		   "\"upload_bytes_per_step\": %zu}\n",
+		   "\"ms_per_step_prefetch_two_products_per_gradient_pair\": %.3f, \"upload_bytes_per_step\": %zu}\n",
 			B, steps, ms[0], ms[1], ms[2], ms[3], B / ms[0] * 1e3, B / ms[1] * 1e3, ms[2] > 0 ? B / ms[2] * 1e3 : 0.0, ms[4],
-			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, (size_t) 2 * B * n * sizeof(float));
+			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, ms[5], (size_t) 2 * B * n * sizeof(float));
 }
 
 // ------------------------------------------------------------------------------------------------- upstream's test nets
@@ -1160,10 +1175,11 @@ static void test_errors() {
 }
 
 // ------------------------------------------------------------------------------------------------- throughput
-static void run_c4(int n, int blocks, int B, int steps, float lr) {
+static void run_c4(int n, int blocks, int B, int steps, float lr, bool both_halves) {
 	orc::Rng rng(4);
 	ResStack r;
 	build_stack(r, n, blocks);
+	if (both_halves) r.net.conjugateGradients(false);  // dz* products computed as upstream does, not written as conjugates
 	for (int b = 0; b < blocks; ++b) fill_normal(rng, r.net[r.w[b]]->mutable_input()->real_, (size_t) 2 * n * n, 1.0 / std::sqrt((double) n));
 	r.net.allocateOnGpu(B);
 	std::vector<float> xs((size_t) 2 * B * n), ts((size_t) 2 * B * n);
@@ -1204,11 +1220,14 @@ static void run_c4(int n, int blocks, int B, int steps, float lr) {
 	printf("losses:");
 	for (float l : losses) printf(" %.4f", l);
 	printf("\n");
-	double flops = 40.0 * B * (double) n * n * blocks;  // GEMM flops per step
+	// matrix products executed per Linear and step: forward, and per gradient pair one product (the other half written as
+	// its conjugate) or two (both computed), for the input and for the weight
+	const int products = both_halves ? 5 : 3;
+	double flops = 8.0 * products * B * (double) n * n * blocks;
 	printf("{\"workload\": \"residual stack: %d x (Linear %d->%d, CGelu, Residual), L2Out, SGD\", \"batch\": %d, \"steps\": %d, "
-		   "\"ms_per_step\": %.3f, \"ms_per_step_after_the_first\": %.3f, \"samples_per_sec\": %.1f, \"gemm_tflops\": %.2f, "
-		   "\"first_loss\": %.4f, \"last_loss\": %.4f}\n",
-			blocks, n, n, B, steps, 1e3 * sec / steps, steps > 1 ? 1e3 * sec_later / (steps - 1) : 0.0, B * steps / sec,
+		   "\"ms_per_step\": %.3f, \"ms_per_step_after_the_first\": %.3f, \"samples_per_sec\": %.1f, "
+		   "\"complex_products_per_linear\": %d, \"gemm_tflops_executed\": %.2f, \"first_loss\": %.4f, \"last_loss\": %.4f}\n",
+			blocks, n, n, B, steps, 1e3 * sec / steps, steps > 1 ? 1e3 * sec_later / (steps - 1) : 0.0, B * steps / sec, products,
 			flops * steps / sec / 1e12, losses.front(), losses.back());
 	if (!(losses.back() < losses.front())) {
 		printf("FAIL loss did not decrease\n");
@@ -1235,7 +1254,7 @@ int main(int argc, char **argv) {
 		if (what == "errors" || what == "all") test_errors();
 		if (what == "c4")
 			run_c4(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048, argc > 5 ? atoi(argv[5]) : 10,
-					argc > 6 ? (float) atof(argv[6]) : 0.01f);
+					argc > 6 ? (float) atof(argv[6]) : 0.01f, argc > 7 && std::string(argv[7]) == "both_halves");
 	} catch (const std::exception &e) {
 		printf("FAIL uncaught exception: %s\n", e.what());
 		return 2;
