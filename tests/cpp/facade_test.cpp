@@ -857,7 +857,7 @@ struct SyntheticReader : public BatchedDataReader {
 
 // with_graphs: also run the two modes that replay recorded graphs (left out of plain timing runs: they are not faster, and
 // the profiler's kernel trace has been seen to crash inside hipGraphLaunch on them)
-static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs) {
+static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, bool both_halves = false) {
 	const int n = 784, classes = 10;
 	const float lr = 0.01f;
 	if (cnet_init(0) != CNET_OK) {
@@ -873,6 +873,7 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs) 
 	double ms[MODES] = {0, 0, 0, 0, 0, 0};
 	for (int mode = 0; mode < MODES; ++mode) {
 		if (!with_graphs && mode >= 2 && mode <= 4) continue;
+		if (mode == 5 && timing_only && !both_halves) continue;
 		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4;
 		CNet net;
 		int inp, outp;
@@ -1249,7 +1250,8 @@ int main(int argc, char **argv) {
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
 		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12, false, true);
 		if (what == "pipeline_timing")
-			test_pipeline(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, true, argc > 4 && std::string(argv[4]) == "graphs");
+			test_pipeline(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, true, argc > 4 && std::string(argv[4]) == "graphs",
+					argc > 4 && std::string(argv[4]) == "both_halves");
 		if (what == "upstream_nets" || what == "all") test_upstream_nets();
 		if (what == "errors" || what == "all") test_errors();
 		if (what == "c4")
