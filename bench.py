@@ -204,22 +204,28 @@ def token_model_suite(steps):
     P = {"table": gen.normal(1, (2, V, D)), "gate": gen.normal(2, (2, D), 0, 0.05),
          "w1": gen.normal(3, (2, H, D), 0, D ** -0.5), "w2": gen.normal(4, (2, D, H), 0, H ** -0.5),
          "w3": gen.normal(5, (2, V, D), 0, D ** -0.5)}
-    model = TokenModel(Bq, S, D, H, V, P).set_tokens(gen.randint(6, (Bq, S), V))
+    ids = gen.randint(6, (Bq, S), V)
     ev = HipEvents(capi.load().cnet_stream())
-    for _ in range(2):
-        model.forward(); model.backward()
-    capi.sync()
-    a, b = ev.event(), ev.event()
-    ev.record(a)
-    for _ in range(steps):
-        model.forward(); model.backward()
-    ev.record(b)
-    ms = ev.elapsed_ms(a, b) / steps
-    loss = float(model.loss.download().mean())
-    print(json.dumps({"workload": "configs[4]: complex token model fwd+bwd, batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096",
-                      "ms_per_step": round(ms, 3), "tokens_per_sec": round(Bq * S / ms * 1e3, 1),
-                      "gemm_tflops": round(model.gemm_flops() / ms / 1e9, 2), "mean_loss": round(loss, 4),
-                      "loss_of_uniform_guess": round(float(np.log(V)), 4)}))
+    # first with every product computed (what upstream's backward pass does), then with the dz* halves of the gradient
+    # pairs written as conjugates of the dz products (the loss is real); one model at a time on the device
+    for conjugate_pairs in (False, True):
+        model = TokenModel(Bq, S, D, H, V, P, conjugate_pairs=conjugate_pairs).set_tokens(ids)
+        for _ in range(2):
+            model.forward(); model.backward()
+        capi.sync()
+        a, b = ev.event(), ev.event()
+        ev.record(a)
+        for _ in range(steps):
+            model.forward(); model.backward()
+        ev.record(b)
+        ms = ev.elapsed_ms(a, b) / steps
+        loss = float(model.loss.download().mean())
+        print(json.dumps({"workload": "configs[4]: complex token model fwd+bwd, batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096",
+                          "gradient_pairs": "dz* written as conj(dz)" if conjugate_pairs else "both halves computed",
+                          "ms_per_step": round(ms, 3), "tokens_per_sec": round(Bq * S / ms * 1e3, 1),
+                          "gemm_tflops_executed": round(model.gemm_flops() / ms / 1e9, 2), "mean_loss": round(loss, 4),
+                          "loss_of_uniform_guess": round(float(np.log(V)), 4)}), flush=True)
+        del model
 
 
 def train_lines(steps):

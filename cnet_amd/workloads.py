@@ -13,8 +13,12 @@ from . import capi, ops
 
 
 class TokenModel:
-    def __init__(self, batch, seq, dim, hidden, vocab, params):
-        """params: dict of host arrays: table (2,V,D), gate (2,D), w1 (2,H,D), w2 (2,D,H), w3 (2,V,D)."""
+    def __init__(self, batch, seq, dim, hidden, vocab, params, conjugate_pairs=False):
+        """params: dict of host arrays: table (2,V,D), gate (2,D), w1 (2,H,D), w2 (2,D,H), w3 (2,V,D).
+        conjugate_pairs: the loss is real, so every dz* gradient is the conjugate of the dz gradient; the Linear backward
+        passes then compute the dz products only and write the dz* halves as their conjugates, and of the sequence-axis
+        transform only the dz* product is formed (its one consumer, the embedding table, gathers dz* alone)."""
+        self.conjugate_pairs = conjugate_pairs
         self.B, self.S, self.D, self.H, self.V = batch, seq, dim, hidden, vocab
         self.rows = batch * seq
         p = {k: ops.CMat.from_host(v[0], v[1]) for k, v in params.items()}
@@ -57,21 +61,24 @@ class TokenModel:
 
     def backward(self):
         B, S, D = self.B, self.S, self.D
+        bwd_input = ops.linear_bwd_input_sym if self.conjugate_pairs else ops.linear_bwd_input
+        bwd_weight = ops.linear_bwd_weight_sym if self.conjugate_pairs else ops.linear_bwd_weight
         ops.cross_entropy_bwd(self.logits, self.s, self.labels, self.d_logits)
-        ops.linear_bwd_input(self.d_logits, self.w3, self.d_o)
-        ops.linear_bwd_weight(self.d_logits, self.o, self.d_w3)
-        ops.linear_bwd_input(self.d_o, self.w2, self.d_a)
-        ops.linear_bwd_weight(self.d_o, self.a, self.d_w2)
+        bwd_input(self.d_logits, self.w3, self.d_o)
+        bwd_weight(self.d_logits, self.o, self.d_w3)
+        bwd_input(self.d_o, self.w2, self.d_a)
+        bwd_weight(self.d_o, self.a, self.d_w2)
         ops.gelu_bwd(self.u, self.d_a, self.d_u)
-        ops.linear_bwd_input(self.d_u, self.w1, self.d_h)
-        ops.linear_bwd_weight(self.d_u, self.h, self.d_w1)
+        bwd_input(self.d_u, self.w1, self.d_h)
+        bwd_weight(self.d_u, self.h, self.d_w1)
         ops.hadamard_bwd(self.m, self.gate, self.d_h, self.d_m, self.d_gate, shared=True)
         # dz_b = F dM_b.dz ; dz*_b = conj(F) dM_b.dz*   (F symmetric)
         gdz = ops.CMat(self.d_m.planes[0], self.d_m.planes[1])
         gds = ops.CMat(self.d_m.planes[2], self.d_m.planes[3])
         xdz = ops.CMat(self.d_x.planes[0], self.d_x.planes[1])
         xds = ops.CMat(self.d_x.planes[2], self.d_x.planes[3])
-        ops.cgemm_batched(self.F, 0, gdz, S * D, xdz, S * D, S, D, S, B, b_kmajor=1)
+        if not self.conjugate_pairs:
+            ops.cgemm_batched(self.F, 0, gdz, S * D, xdz, S * D, S, D, S, B, b_kmajor=1)
         ops.cgemm_batched(self.F, 0, gds, S * D, xds, S * D, S, D, S, B, b_kmajor=1, conj_a=1)
         gs_re = ops.Plane(self.d_x.planes[2].ptr, B, S * D, S * D)
         gs_im = ops.Plane(self.d_x.planes[3].ptr, B, S * D, S * D)
@@ -81,4 +88,4 @@ class TokenModel:
         R, S, D, H, V, B = self.rows, self.S, self.D, self.H, self.V, self.B
         lin = 8.0 * R * (D * H + H * D + D * V)
         dft = 8.0 * B * S * S * D
-        return 5 * lin + 3 * dft
+        return 3 * lin + 2 * dft if self.conjugate_pairs else 5 * lin + 3 * dft  # the products that are executed

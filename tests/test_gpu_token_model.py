@@ -39,7 +39,10 @@ def test_strided_batched_gemm_with_conj_a(gpu, port):
         assert np.linalg.norm(cr + 1j * ci - want) / np.linalg.norm(want) < 1e-5
 
 
-def test_token_model_reduced(gpu, port):
+@pytest.mark.parametrize("conjugate_pairs", [False, True])
+def test_token_model_reduced(gpu, port, conjugate_pairs):
+    """conjugate_pairs: the Linear backward passes write the dz* halves as conjugates of the dz products, and of the
+    sequence-axis transform only the dz* product is formed (the embedding table gathers dz* alone)."""
     B, S, D, H, V = 3, 32, 64, 128, 512
     R = B * S
     P = {"table": seeded(port, 1, (2, V, D)), "gate": seeded(port, 2, (2, D), 0.5),
@@ -47,7 +50,7 @@ def test_token_model_reduced(gpu, port):
          "w3": seeded(port, 5, (2, V, D), D ** -0.5)}
     ids = port.randint(6, (B, S), V)
     ids[1, 5] = ids[1, 9] = ids[0, 3]      # repeated tokens
-    model = TokenModel(B, S, D, H, V, P).set_tokens(ids)
+    model = TokenModel(B, S, D, H, V, P, conjugate_pairs=conjugate_pairs).set_tokens(ids)
     model.forward()
     model.backward()
 
@@ -75,9 +78,9 @@ def test_token_model_reduced(gpu, port):
     d_x = _seq_dft(port, None, None, B, S, D, backward_g4=d_m)
     dt_r, dt_i = port.embedding_bwd(V, D, ids, d_x[2].reshape(B, S * D), d_x[3].reshape(B, S * D))
 
-    def chk(got, want, what):
+    def chk(got, want, what, halves=(0, 2)):
         h = got.host()
-        for k in (0, 2):
+        for k in halves:
             e = rel_c(h[k:k + 2], [w.reshape(h[k].shape) for w in want[k:k + 2]])
             assert e < TOL, (what, k, e)
 
@@ -87,7 +90,7 @@ def test_token_model_reduced(gpu, port):
     chk(model.d_w1, d_w1, "dW1")
     chk(model.d_gate, d_gate, "d gate")
     chk(model.d_m, d_m, "d seq-DFT output")
-    chk(model.d_x, d_x, "d embedding rows")
+    chk(model.d_x, d_x, "d embedding rows", halves=(2,) if conjugate_pairs else (0, 2))
     assert rel_c((model.d_table_re.host(), model.d_table_im.host()), (dt_r, dt_i)) < TOL
 
 
