@@ -1115,7 +1115,7 @@ bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int npro
 
 // tail_splits >= 2: cut the blocks of the last, partly filled round into that many pieces along K (see CgemmArgs)
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
-int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0) {
+int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, int k_cuts = -1) {
 	CgemmArgs args = proto;
 	args.tiles_m = (args.M + BM - 1) / BM;
 	args.tiles_n = (args.N + BN - 1) / BN;
@@ -1131,15 +1131,18 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0) {
 		const long blocks = (long) args.tiles_m * args.tiles_n * nprob * batch;
 		const long cus = cnet::rt().prop.multiProcessorCount;
 		const int nchunks = (args.K + KC - 1) / KC;
-		if (!args.tri && blocks * 2 <= cus && nchunks >= 8 && (long) batch * (cus / blocks) <= 65535) {
-			int splits = (int) std::min<long>(cus / blocks, nchunks / 4);
-			if (splits >= 2) {
-				args.chunks_per_split = (nchunks + splits - 1) / splits;
-				args.splits = (nchunks + args.chunks_per_split - 1) / args.chunks_per_split;  // no empty split
-				const size_t bytes = (size_t) args.splits * nprob * batch * 2 * args.M * args.N * sizeof(float);
-				args.partial = (float *) cnet::workspace(bytes);
-				if (!args.partial) return CNET_ERR_OUT_OF_MEMORY;
-			}
+		int splits = k_cuts;  // from the cost model; -1: the rule for the kernels it does not cover
+		if (k_cuts < 0) {
+			splits = 1;
+			if (!args.tri && blocks * 2 <= cus && nchunks >= 8 && (long) batch * (cus / blocks) <= 65535)
+				splits = (int) std::min<long>(cus / blocks, nchunks / 4);
+		}
+		if (splits >= 2) {
+			args.chunks_per_split = (nchunks + splits - 1) / splits;
+			args.splits = (nchunks + args.chunks_per_split - 1) / args.chunks_per_split;  // no empty split
+			const size_t bytes = (size_t) args.splits * nprob * batch * 2 * args.M * args.N * sizeof(float);
+			args.partial = (float *) cnet::workspace(bytes);
+			if (!args.partial) return CNET_ERR_OUT_OF_MEMORY;
 		}
 	}
 	dim3 grid(args.tiles_m * grid_tiles_n(args), nprob, batch * args.splits);
@@ -1199,7 +1202,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0) {
 
 // Block shape for the fast kernel (0: 128 x 128, 1: 64 x 128, 2: 128 x 64, 3: 64 x 64), whether the blocks of a partly
 // filled last round are cut along K (*tail = number of pieces, 0 = no), and the expected duration of the launch in us.
-double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *tail_pieces) {
+double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *tail_pieces, int *k_cuts) {
 	const long cus = cnet::rt().prop.multiProcessorCount;
 	auto blocks = [&](int bm, int bn) {
 		long tn = (a.N + bn - 1) / bn;
@@ -1245,19 +1248,19 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 		const char *e = getenv("CNET_CGEMM_KMODEL");  // tuning override: 0 uses the K = 2048 table for every K
 		return !e || atoi(e) != 0;
 	}();
-	auto eff = [&](int k, long p) {
+	auto eff = [&](int k, long p, int K) {
 		const int i = p < 8 ? (int) p - 1 : 7;
 		if (!k_dependent) return (double) shapes[k].eff_k2048[i];
 		const double inv512 = 1.0 / shapes[k].eff_k512[i], inv2048 = 1.0 / shapes[k].eff_k2048[i];
 		const double slope = (inv512 - inv2048) / (1.0 / 512 - 1.0 / 2048);  // per 1 / K
 		// beyond K = 2048 the K = 2048 table stands: the straight line would credit the small shapes with a loop
 		// efficiency above that of the large ones
-		return 1.0 / (inv2048 + slope * std::max(0.0, 1.0 / a.K - 1.0 / 2048));
+		return 1.0 / (inv2048 + slope * std::max(0.0, 1.0 / K - 1.0 / 2048));
 	};
 	const double flop_per_us_per_unit = 256.0 * 2.4e3;  // 256 flop per clock at 2.4 GHz
 	const int nchunks = (a.K + KC - 1) / KC;
 	const bool tail_possible = forced_tail != 0 && a.K % KC == 0 && !a.tri && batch == 1;
-	int best = 3, best_tail = 0;
+	int best = 3, best_tail = 0, best_cuts = 1;
 	double best_us = 1e30;
 	for (int k = 0; k < 4; ++k) {
 		if (forced >= 0 && forced != k) continue;
@@ -1266,18 +1269,42 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 		const double block_us = 8.0 * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
 		// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
 		const double bonus = 1.0 - 0.000001 * shapes[k].bm * shapes[k].bn;
-		double us = per_unit * block_us / eff(k, per_unit) * bonus;
-		int tail = 0;
+		double us = per_unit * block_us / eff(k, per_unit, a.K) * bonus;
+		int tail = 0, cuts = 1;
 		const long q = nb / cus, r = nb % cus;
 		if (tail_possible && q >= 1 && r > 0) {
 			// as many pieces as there are workgroups in the full rounds, so that each of them gets one; a piece is at
 			// least three chunks long
 			const int s = (int) std::min<long>(q * cus / r, nchunks / 3);
 			if (s >= 2) {
-				const double tail_us = (q * block_us / eff(k, q) + block_us / s / 0.8 + 20.0) * bonus;
+				const double tail_us = (q * block_us / eff(k, q, a.K) + block_us / s / 0.8 + 20.0) * bonus;
 				if (tail_us < us || forced_tail == 1) {
 					us = tail_us;
 					tail = s;
+				}
+			}
+		}
+		// A short grid (fewer than two blocks per unit: idle units, or lone workgroups that cannot fill the matrix pipe)
+		// against a long K: every block is cut into s slices along K that run as workgroups of their own and are added
+		// in order by splitk_reduce_kernel.  Costs the shorter K per slice (lower efficiency) and the pass over the
+		// partial planes (written and read once, C written, at about 4 TB/s).
+		static const bool plan_cuts = [] {
+			const char *e = getenv("CNET_CGEMM_KCUT");  // tuning override: 0 cuts K only when half of the units would idle
+			return !e || atoi(e) != 0;
+		}();
+		if (!a.tri && nb < 2 * cus && nchunks >= 8 && (plan_cuts || nb * 2 <= cus)) {
+			const long few = nb * 2 <= cus ? std::min<long>(cus / nb, nchunks / 4) : 0;  // one slice-workgroup per unit
+			for (long s : {2L, 3L, 4L, 6L, 8L, few}) {
+				if (s < 2 || nchunks / s < 4 || (long) batch * s > 65535) continue;
+				const int k_slice = (int) ((nchunks + s - 1) / s) * KC;
+				const long p = (nb * s + cus - 1) / cus;
+				const double slice_us = 8.0 * shapes[k].bm * shapes[k].bn * k_slice / flop_per_us_per_unit;
+				const double pass_us = 6.0 + (s + 1.0 + (a.accumulate ? 1.0 : 0.0)) * 8.0 * a.M * a.N * nprob * batch / 4.0e6;
+				const double cut_us = p * slice_us / eff(k, p, k_slice) * bonus + pass_us;
+				if (cut_us < us) {
+					us = cut_us;
+					cuts = (int) s;
+					tail = 0;
 				}
 			}
 		}
@@ -1285,10 +1312,12 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 			best_us = us;
 			best = k;
 			best_tail = tail;
+			best_cuts = cuts;
 		}
 	}
 	*shape = best;
 	*tail_pieces = best_tail;
+	*k_cuts = best_cuts;
 	return best_us + 12.0;  // launch, first loads and the write-out of C
 }
 
@@ -1298,12 +1327,12 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 	if constexpr (VEC == 1) {
 		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 	} else {
-		int best, best_tail;
-		plan_blocks(a, nprob, batch, &best, &best_tail);
-		if (best == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
-		if (best == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
-		if (best == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
-		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail);
+		int best, best_tail, cuts;
+		plan_blocks(a, nprob, batch, &best, &best_tail, &cuts);
+		if (best == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
+		if (best == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
+		if (best == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
+		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
 	}
 }
 
@@ -1341,9 +1370,9 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 			}
 		}
 		if (plan_skinny(a_mcontig, b_ncontig, right, nprob, batch, planned)) {
-			int shape, tail;
-			const double whole = plan_blocks(a, nprob, batch, &shape, &tail);
-			const double parts = plan_blocks(left, nprob, batch, &shape, &tail) + skinny_us(planned, nprob, batch);
+			int shape, tail, cuts;
+			const double whole = plan_blocks(a, nprob, batch, &shape, &tail, &cuts);
+			const double parts = plan_blocks(left, nprob, batch, &shape, &tail, &cuts) + skinny_us(planned, nprob, batch);
 			if (parts < whole) {
 				// one after the other on the compute stream: run side by side on two streams the narrow part's
 				// workgroups took slots from the first round of the block kernel and the pair got slower (842 against

@@ -119,10 +119,13 @@ def _check_all_layouts(port, M, N, K):
             assert np.array_equal(hr, base) and np.array_equal(hi, base)
 
 
-@pytest.mark.parametrize("M,N,K", [(8, 24, 1000), (64, 64, 4096), (40, 100, 333), (64, 784, 784), (3, 5, 2049)])
+@pytest.mark.parametrize("M,N,K", [(8, 24, 1000), (64, 64, 4096), (40, 100, 333), (64, 784, 784), (3, 5, 2049), (784, 784, 4096),
+                                   (64, 64, 100000), (520, 516, 2048)])
 def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
     """Few blocks of C against a long K.  Up to K = 1024 each 16 x 16 tile of C has a workgroup of its own whose wavefronts
-    share K; beyond, the launch of the block kernel is cut along K and the partial blocks are added in a fixed order."""
+    share K; beyond, the launch of the block kernel is cut along K and the partial blocks are added in a fixed order (also
+    when the blocks of C are fewer than two per compute unit, 784 x 784: 169 blocks, and the cost model finds the cut
+    cheaper than idle units)."""
     _check_all_layouts(port, M, N, K)
 
 
