@@ -81,15 +81,12 @@ def cpu_baseline(budget_s=15.0):
         net.node_backward(w)             # parameter node gathers dW* across samples
         net.node_backward(x)
 
-    one(0)
-    t0 = time.perf_counter()
-    for r in range(4):
+    for r in range(4):   # warm-up: page in the weight planes, start the thread pool
         one(r)
-    per_row = (time.perf_counter() - t0) / 4
-    rows = int(max(16, min(4096, budget_s / per_row)))
-    t0 = time.perf_counter()
-    for r in range(rows):
-        one(r)
+    rows, t0 = 0, time.perf_counter()
+    while rows < B and (rows < 16 or time.perf_counter() - t0 < budget_s):   # a bounded sample of the batch, by time
+        one(rows)
+        rows += 1
     dt = time.perf_counter() - t0
     return {"value": round(40.0 * rows * N * K / dt / 1e12, 5), "unit": "TFLOP/s", "cores": lib.threads,
             "kind": lib.backend,
