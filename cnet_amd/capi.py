@@ -30,6 +30,7 @@ SIGNATURES = {
     "cnet_host_alloc": [C.c_size_t, C.POINTER(C.c_void_p)],
     "cnet_host_free": [C.c_void_p],
     "cnet_memcpy_h2d_async": [C.c_void_p, C.c_void_p, C.c_size_t],
+    "cnet_memcpy_d2h_async": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_upload_async": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_upload_wait_compute": [],
     "cnet_mark_compute": [_i],

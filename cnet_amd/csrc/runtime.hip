@@ -237,6 +237,15 @@ int cnet_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes) {
 	return CNET_OK;
 }
 
+int cnet_memcpy_d2h_async(void *pinned_dst, const void *src, size_t bytes) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // a recording would replay the copy into the same host address
+	if (!bytes) return CNET_OK;
+	CNET_CHECK_ARG(pinned_dst && src);
+	CNET_HIP(hipMemcpyAsync(pinned_dst, src, bytes, hipMemcpyDeviceToHost, rt().stream));
+	return CNET_OK;
+}
+
 int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes) {
 	CNET_REQUIRE_INIT();
 	if (!bytes) return CNET_OK;

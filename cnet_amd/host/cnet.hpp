@@ -625,6 +625,8 @@ class CNet {
 	StepGraphs graphs_[2];
 	bool use_graphs_ = false;
 	bool conjugate_gradients_ = true;
+	float *loss_ring_ = NULL;  // page-locked [kLossSlots][batch]: losses on their way to the host (gpuQueueLoss)
+	int64_t loss_queued_ = 0;
 	std::vector<const float *> gather_src_;  // pending dz* gathers of the input functions (see nodeBackward)
 	std::vector<float *> gather_dst_;
 	std::vector<int64_t> gather_len_;
@@ -834,6 +836,9 @@ public:
 			st = Stage();
 		}
 		active_ = 0;
+		if (loss_ring_) cnet_host_free(loss_ring_);
+		loss_ring_ = NULL;
+		loss_queued_ = 0;
 	}
 
 	int batchSize() const { return batch_; }
@@ -1490,6 +1495,48 @@ public:
 			if (batch) batch->addLoss(v);
 		}
 		return loss / tmp.size();
+	}
+	// The same read in two halves, so that a training loop never waits for the step it has just queued: gpuQueueLoss sends
+	// the per-row losses of the forward pass that was queued last to page-locked memory without waiting; getLoss(pending)
+	// waits for that copy alone, typically one step later, when it has long arrived.  The host can then queue step k+1
+	// before it looks at the loss of step k, and the device never runs dry between steps.  Up to kLossSlots reads may be
+	// pending; an older one is overwritten.
+	static constexpr int kLossSlots = 4;
+	struct PendingLoss {
+		int64_t ticket = -1, serial = -1;
+		int rows = 0;
+	};
+	PendingLoss gpuQueueLoss(OutputFunc *outp) {
+		requireAllocated("gpuQueueLoss");
+		CFunc *f = dynamic_cast<CFunc *>(outp);
+		float *d = NULL;
+		if (CrossEntropy *c = dynamic_cast<CrossEntropy *>(f)) d = c->d_loss_;
+		else if (L2Out *l = dynamic_cast<L2Out *>(f)) d = l->d_loss_;
+		else throw std::invalid_argument("gpuQueueLoss: not supported for this output");
+		if (!loss_ring_) {
+			void *h = NULL;
+			ck(cnet_host_alloc((size_t) kLossSlots * batch_ * sizeof(float), &h), "cnet_host_alloc");
+			loss_ring_ = (float *) h;
+		}
+		PendingLoss p;
+		p.serial = loss_queued_++;
+		p.rows = f->rows_;
+		ck(cnet_memcpy_d2h_async(loss_ring_ + (size_t) (p.serial % kLossSlots) * batch_, d, (size_t) p.rows * sizeof(float)),
+				"cnet_memcpy_d2h_async");
+		ck(cnet_copy_ticket(0, &p.ticket), "cnet_copy_ticket");
+		return p;
+	}
+	float getLoss(const PendingLoss &p, Batch *batch) {
+		if (p.serial < 0 || !loss_ring_) throw std::logic_error("getLoss: nothing was queued under this handle");
+		if (loss_queued_ - p.serial > kLossSlots) throw std::logic_error("getLoss: the queued losses were overwritten by later ones");
+		ck(cnet_copy_wait(p.ticket), "cnet_copy_wait");
+		const float *v = loss_ring_ + (size_t) (p.serial % kLossSlots) * batch_;
+		float loss = 0.f;
+		for (int b = 0; b < p.rows; ++b) {
+			loss += v[b];
+			if (batch) batch->addLoss(v[b]);
+		}
+		return loss / p.rows;
 	}
 	// upstream GpuNet::getLoss(int label) (gpu/gpu_func.h:928-969): the loss of every output function, keyed by uid.
 	// Upstream has one entry per clone, i.e. per batch row, each clone under a uid of its own; there are no clones here,

@@ -66,6 +66,9 @@ int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes);   /* *_copy_
  * cnet_host_alloc / cnet_host_free: page-locked host memory (hipHostMalloc).
  * cnet_memcpy_h2d_async: copy on the compute stream, returns at once; the source must be page-locked and stay
  *      untouched until the stream reaches the copy (cnet_sync, or any later blocking call).
+ * cnet_memcpy_d2h_async: the other direction on the compute stream (the per-row losses of a step, replacing the blocking
+ *      read of CNet::getLoss, impl/cnet.h / gpu/gpu_func.h:928-969 upstream); the page-locked destination is valid once a
+ *      ticket taken after the call has been waited for.
  * cnet_upload_async: the same on the library's upload stream, so it overlaps kernels of the compute stream.
  * cnet_upload_wait_compute: uploads queued after this call start only when everything queued on the compute stream so
  *      far has finished (call before overwriting a device buffer that kernels may still read).
@@ -81,6 +84,7 @@ int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes);   /* *_copy_
 int cnet_host_alloc(size_t bytes, void **host_ptr);
 int cnet_host_free(void *host_ptr);
 int cnet_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
+int cnet_memcpy_d2h_async(void *pinned_dst, const void *src, size_t bytes);
 int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes);
 int cnet_upload_wait_compute(void);
 int cnet_mark_compute(int marker);

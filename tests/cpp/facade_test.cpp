@@ -867,14 +867,17 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 	SyntheticReader data(n, 3 * B + 7, classes);
 	// 4: prefetch + gpuTrainStep (the whole step as one recorded graph); 5: prefetch with both halves of every gradient
 	// pair computed by matrix products (conjugateGradients(false), what upstream does)
-	constexpr int MODES = 6;
+	// 6: prefetch, the loss of a step read one step later (gpuQueueLoss / getLoss(pending)); 7: the same with gpuTrainStep
+	constexpr int MODES = 8;
 	std::vector<float> losses[MODES];
 	std::vector<float> weights[MODES];
-	double ms[MODES] = {0, 0, 0, 0, 0, 0};
+	double ms[MODES] = {0, 0, 0, 0, 0, 0, 0, 0};
 	for (int mode = 0; mode < MODES; ++mode) {
-		if (!with_graphs && mode >= 2 && mode <= 4) continue;
+		if (!with_graphs && ((mode >= 2 && mode <= 4) || mode == 7)) continue;
 		if (mode == 5 && timing_only && !both_halves) continue;
-		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4;
+		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4 || mode == 7;
+		const bool late_loss = mode == 6 || mode == 7;
+		CNet::PendingLoss pending;
 		CNet net;
 		int inp, outp;
 		build_readme(net, n, classes, &inp, &outp);
@@ -908,12 +911,23 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 				net.gpuBackward();
 				net.gpuUpdateInputs(rate);
 			}
+			if (late_loss) {
+				// the loss of this step starts its way to the host; the one of the step before is read (into its batch,
+				// which is the buffer of the ring that is refilled next)
+				CNet::PendingLoss now = net.gpuQueueLoss(cen);
+				if (s + 1 < steps) net.gpuPrefetch(cin, ring[(s + 1) % 3]);
+				if (s > 0) losses[mode].push_back(net.getLoss(pending, &ring[(s + 2) % 3]));
+				if (s + 2 < steps) reader.nextBatch(ring[(s + 2) % 3]);
+				pending = now;
+				continue;
+			}
 			if (prefetch) {
 				if (s + 1 < steps) net.gpuPrefetch(cin, ring[(s + 1) % 3]);
 				if (s + 2 < steps) reader.nextBatch(ring[(s + 2) % 3]);
 			}
 			losses[mode].push_back(net.getLoss(cen, &cur));
 		}
+		if (late_loss) losses[mode].push_back(net.getLoss(pending, NULL));
 		net.sync();
 		ms[mode] = 1e3 * std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / steps;
 		net.getInputsFromGpu();
@@ -958,6 +972,9 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 		expect("weights identical with graph replay (copy in forward)", weights[0] == weights[3]);
 		expect("losses identical with gpuTrainStep (one recorded graph per step)", losses[0] == losses[4]);
 		expect("weights identical with gpuTrainStep", weights[0] == weights[4]);
+		expect("losses identical when each is read one step late (gpuQueueLoss)", losses[0] == losses[6]);
+		expect("weights identical when each loss is read one step late", weights[0] == weights[6]);
+		expect("losses and weights identical with gpuTrainStep and the late read together", losses[0] == losses[7] && weights[0] == weights[7]);
 		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
 		// dz* planes written as the conjugate of the dz product against dz* planes computed by a product of their own
 		double worst = 0, num = 0, den = 0;
@@ -975,9 +992,11 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 		   "\"ms_per_step_copy_in_forward\": %.3f, \"ms_per_step_prefetch\": %.3f, \"ms_per_step_prefetch_graphs\": %.3f, "
 		   "\"ms_per_step_graphs\": %.3f, \"samples_per_sec_copy_in_forward\": %.1f, \"samples_per_sec_prefetch\": %.1f, "
 		   "\"samples_per_sec_prefetch_graphs\": %.1f, \"ms_per_step_train_step_graph\": %.3f, \"samples_per_sec_train_step_graph\": %.1f, "
-		   "\"ms_per_step_prefetch_two_products_per_gradient_pair\": %.3f, \"upload_bytes_per_step\": %zu}\n",
+		   "\"ms_per_step_prefetch_two_products_per_gradient_pair\": %.3f, \"ms_per_step_prefetch_loss_read_one_step_late\": %.3f, "
+		   "\"samples_per_sec_prefetch_loss_read_one_step_late\": %.1f, \"ms_per_step_train_step_graph_loss_read_one_step_late\": %.3f, "
+		   "\"upload_bytes_per_step\": %zu}\n",
 			B, steps, ms[0], ms[1], ms[2], ms[3], B / ms[0] * 1e3, B / ms[1] * 1e3, ms[2] > 0 ? B / ms[2] * 1e3 : 0.0, ms[4],
-			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, ms[5], (size_t) 2 * B * n * sizeof(float));
+			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, ms[5], ms[6], B / ms[6] * 1e3, ms[7], (size_t) 2 * B * n * sizeof(float));
 }
 
 // ------------------------------------------------------------------------------------------------- upstream's test nets

@@ -225,5 +225,19 @@ def test_device_copy_caller_stream_and_upload_ordering(gpu, port):
     capi.call("cnet_upload_sync")
     capi.sync()
     assert (b.download() == 1.0).all() and (a.download() == 7.0).all()
+
+    # the way back without a blocking call: copy to page-locked memory on the compute stream, valid once a ticket taken
+    # after the copy has been waited for (what reading the loss of a step one step later is built on)
+    pinned[:] = -1.0
+    capi.call("cnet_copy2d", a.ptr, n, b.ptr, n, 1, n)          # b <- 7 on the compute stream, in front of the copy
+    capi.call("cnet_memcpy_d2h_async", host, b.ptr, 4 * n)
+    t = C.c_int64(-1)
+    capi.call("cnet_copy_ticket", 0, C.byref(t))
+    capi.call("cnet_copy_wait", t)
+    assert (pinned == 7.0).all()
+    assert _status("cnet_memcpy_d2h_async", None, b.ptr, 16) == INVALID
+    capi.call("cnet_graph_begin")
+    assert _status("cnet_memcpy_d2h_async", host, b.ptr, 4 * n) == UNSUPPORTED
+    capi.call("cnet_graph_end", None)
     del pinned
     capi.call("cnet_host_free", host)
