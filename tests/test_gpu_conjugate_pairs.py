@@ -79,3 +79,22 @@ def test_triangular_dft_backward_of_a_conjugate_pair(gpu, port, B, n):
         ops.triang_dft_bwd(g, full, accumulate=accumulate)
         ops.triang_dft_bwd_sym(g, sym, accumulate=accumulate)
         _same(full, sym, ("triangular dft", accumulate))
+
+
+@pytest.mark.parametrize("overrides", [
+    {"CNET_CGEMM_SKINNY": "0"},                            # small products on the block kernels (cut along K)
+    {"CNET_CGEMM_TILE": "0", "CNET_CGEMM_COLSPLIT": "0"},  # 128 x 128 blocks (two accumulator sets, negated operand)
+    {"CNET_CGEMM_TILE": "3", "CNET_CGEMM_TAIL": "1"},      # 64 x 64 blocks, tail blocks cut along K whenever possible
+])
+def test_conjugate_pairs_under_other_kernel_choices(gpu, overrides):
+    """The tests of this file again, in a process whose tuning overrides (read once per process) send the same shapes to
+    other kernels and block shapes: every epilogue and both partial-sum kernels write the conjugate half."""
+    import os
+    import subprocess
+    import sys
+    if os.environ.get("CNET_TEST_INNER"):
+        pytest.skip("already the inner run")
+    env = dict(os.environ, CNET_TEST_INNER="1", **overrides)
+    r = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-m", "gpu"], env=env,
+                       capture_output=True, text=True, timeout=280, cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-2000:]
