@@ -1105,10 +1105,16 @@ bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int npro
 				  : launch_skinny<W, true, false>(args, a_mcontig, b_ncontig, nprob, batch))                   \
 		  : (b_v4 ? launch_skinny<W, false, true>(args, a_mcontig, b_ncontig, nprob, batch)                    \
 				  : launch_skinny<W, false, false>(args, a_mcontig, b_ncontig, nprob, batch)))
-	// Four wavefronts per tile: the time of a tile is set by the compute unit's vector memory pipeline (each load
-	// instruction touches 4 to 16 cache lines), not by how many wavefronts share the work, and small workgroups leave
-	// room for a second tile on the same unit.
-	*rc = CNET_SKINNY(4);
+	// Four wavefronts per tile, which leaves room for several tiles on a compute unit; eight (two per SIMD, each other's
+	// latency cover) when there are so few tiles that most units hold one at most (64 x 784 x 784: 9.0 -> 8.5 us; with
+	// three tiles per unit, 256 x 784 x 784: 19.8 -> 21.6 us, so not there).
+	static const int forced_w = [] {
+		const char *e = getenv("CNET_CGEMM_SKINNY_W");  // tuning override: 4, 8 or 16 wavefronts per tile
+		return e ? atoi(e) : 0;
+	}();
+	const long wgs = (long) args.tiles_m * args.tiles_n * nprob * batch * args.splits;
+	const int w = forced_w ? forced_w : (args.splits == 1 && 2 * wgs <= 3 * cnet::rt().prop.multiProcessorCount && args.K >= 256) ? 8 : 4;
+	*rc = w == 16 ? CNET_SKINNY(16) : w == 8 ? CNET_SKINNY(8) : CNET_SKINNY(4);
 #undef CNET_SKINNY
 	return true;
 }
