@@ -367,6 +367,8 @@ protected:
 		float *g(int plane) const { return grad + (size_t) plane * rows * len; }
 	};
 	std::vector<Slot> slots_;
+	bool trainable_ = true;   // input functions: stepped by the update (CNet::setInputTrainable)
+	bool wants_grad_ = true;  // a trainable input function lies below this node: gradients have to flow through it
 	int rows_ = 0;           // batch rows of this node's output (1 for parameter nodes)
 	float *out_ = NULL;      // 2 planes [rows][out_size]: what consumers read
 	float *out_re() const { return out_; }
@@ -1039,6 +1041,7 @@ private:
 			ck(cnet_l2out_bwd(zre(f, 0), zim(f, 0), s.len, s.g(0), s.g(1), s.g(2), s.g(3), s.len, rows, s.len, 0), "cnet_l2out_bwd");
 			return;
 		}
+		if ((t == isInput || t == isEmbedding) && !f->trainable_) return;  // nothing steps it: nothing to gather
 		if (t == isInput) {  // impl/cinput.h:54-65: gathers dzs only, and keeps adding until the next update
 			// Both dz* planes of a consumer's slot are adjacent and dense, as they are in the node's own block: one array per
 			// consumer.  Nothing in the backward pass reads what an input function gathers, so the gathers of all of them
@@ -1067,6 +1070,9 @@ private:
 			for (auto &s : f->slots_) ck(cnet_memset_zero(s.grad, 4 * (size_t) s.rows * s.len * sizeof(float)), "zero");
 			return;
 		}
+		// Gradients flow only towards input functions that are stepped: a layer none of whose operands leads to one is
+		// skipped (all input functions are trainable unless CNet::setInputTrainable said otherwise, as upstream has it).
+		if (!f->wants_grad_) return;
 		for (int c = 0; c < f->no_outputs(); ++c) {
 			CFunc::Slot &u = upstream(f, c);
 			const int acc = c > 0;
@@ -1075,17 +1081,22 @@ private:
 			case isLinear: {
 				CFunc::Slot &w = f->slots_[1];
 				const int K = a.len, N = f->out_size_;
+				const bool to_data = a.producer->wants_grad_, to_weight = w.producer->wants_grad_;
 				if (conjugate_gradients_) {  // dz* = conj(dz): one product each, written to both pairs of planes
-					ck(cnet_clinear_bwd_input_sym(u.g(0), u.g(1), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K, rows, K, N,
-							acc), "cnet_clinear_bwd_input_sym");
-					ck(cnet_clinear_bwd_weight_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K, rows, K, N,
-							acc), "cnet_clinear_bwd_weight_sym");
+					if (to_data)
+						ck(cnet_clinear_bwd_input_sym(u.g(0), u.g(1), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K, rows, K,
+								N, acc), "cnet_clinear_bwd_input_sym");
+					if (to_weight)
+						ck(cnet_clinear_bwd_weight_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K, rows, K,
+								N, acc), "cnet_clinear_bwd_weight_sym");
 					break;
 				}
-				ck(cnet_clinear_bwd_input(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K,
-						rows, K, N, acc), "cnet_clinear_bwd_input");
-				ck(cnet_clinear_bwd_weight(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K,
-						rows, K, N, acc), "cnet_clinear_bwd_weight");
+				if (to_data)
+					ck(cnet_clinear_bwd_input(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K,
+							rows, K, N, acc), "cnet_clinear_bwd_input");
+				if (to_weight)
+					ck(cnet_clinear_bwd_weight(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K,
+							rows, K, N, acc), "cnet_clinear_bwd_weight");
 				break;
 			}
 			case isFourier:
@@ -1144,6 +1155,20 @@ private:
 				break;
 			default: throw std::logic_error(f->getName() + ": no device implementation");
 			}
+		}
+	}
+
+	// wants_grad_ of every function: input functions say it themselves, a layer wants gradients when one of its operands
+	// does (func_list_ is in insertion order, producers first)
+	void planGradients() {
+		for (auto f : func_list_) {
+			if (f->is_input_) {
+				f->wants_grad_ = f->trainable_;
+				continue;
+			}
+			f->wants_grad_ = false;
+			for (auto &sl : f->slots_)
+				if (sl.producer && sl.producer->wants_grad_) f->wants_grad_ = true;
 		}
 	}
 
@@ -1404,6 +1429,7 @@ public:
 	}
 	bool gpuBackward() {
 		requireAllocated("gpuBackward");
+		planGradients();
 		runPhase(1, graphs_[active_].bwd, [&] {
 			gather_src_.clear();  // nothing is left over from a pass that threw
 			gather_dst_.clear();
@@ -1434,6 +1460,7 @@ public:
 			std::vector<float *> zr, zi, dr, di;
 			std::vector<int64_t> len;
 			for (auto f : inputs_) {
+				if (!f->trainable_) continue;
 				CFunc::Slot &s = f->slots_[0];
 				const size_t n = (size_t) s.rows * s.len;
 				zr.push_back(s.z);
@@ -1443,6 +1470,7 @@ public:
 				len.push_back((int64_t) n);
 				if (input_dz_dirty_) ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
 			}
+			if (zr.empty()) return;
 			ck(cnet_sgd_update_multi((int) zr.size(), zr.data(), zi.data(), dr.data(), di.data(), len.data(), l_rate, 1),
 					"cnet_sgd_update_multi");
 		});
@@ -1468,11 +1496,23 @@ public:
 		conjugate_gradients_ = on;
 	}
 	bool conjugateGradients() const { return conjugate_gradients_; }
+	// Upstream steps every input function, the data input included (impl/cnet.h:413-421), and therefore runs the backward
+	// pass all the way down to it.  An input function marked not trainable is left alone by gpuUpdateInputs /
+	// gpuAdamUpdate, gathers nothing, and the backward products that would only serve it are not computed (for the
+	// 784 -> 10 net: the whole backward pass of the FourierTrans).  Losses and the steps of the other input functions are
+	// unchanged to the bit.  Recordings are dropped.
+	void setInputTrainable(InputFunc *inp, bool on) {
+		CFunc *f = dynamic_cast<CFunc *>(inp);
+		if (!f || !f->is_input_) throw std::invalid_argument("setInputTrainable: not an input function of this net");
+		if (f->trainable_ != on && batch_) dropGraphs();
+		f->trainable_ = on;
+	}
 	// The Adam-style step of upstream GpuNet::adamUpdate (gpu/gpu_func.h:503-510, gpu/kernels.cpp:494-514) on every input
 	// function: the first moment lives in the node's dz planes, dz* is cleared, dz is kept.
 	void gpuAdamUpdate(float l_rate, float beta, int t) {
 		requireAllocated("gpuAdamUpdate");
 		for (auto f : inputs_) {
+			if (!f->trainable_) continue;
 			CFunc::Slot &s = f->slots_[0];
 			const size_t n = (size_t) s.rows * s.len;
 			float *z = s.z;

@@ -868,15 +868,16 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 	// 4: prefetch + gpuTrainStep (the whole step as one recorded graph); 5: prefetch with both halves of every gradient
 	// pair computed by matrix products (conjugateGradients(false), what upstream does)
 	// 6: prefetch, the loss of a step read one step later (gpuQueueLoss / getLoss(pending)); 7: the same with gpuTrainStep
-	constexpr int MODES = 8;
+	// 8: as 6 with the data input marked not trainable (CNet::setInputTrainable: no step on it, no backward pass into it)
+	constexpr int MODES = 9;
 	std::vector<float> losses[MODES];
 	std::vector<float> weights[MODES];
-	double ms[MODES] = {0, 0, 0, 0, 0, 0, 0, 0};
+	double ms[MODES] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
 	for (int mode = 0; mode < MODES; ++mode) {
 		if (!with_graphs && ((mode >= 2 && mode <= 4) || mode == 7)) continue;
 		if (mode == 5 && timing_only && !both_halves) continue;
 		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4 || mode == 7;
-		const bool late_loss = mode == 6 || mode == 7;
+		const bool late_loss = mode == 6 || mode == 7 || mode == 8;
 		CNet::PendingLoss pending;
 		CNet net;
 		int inp, outp;
@@ -889,6 +890,7 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 		if (mode == 0 && !timing_only) expect("batches built after cnet_init are page-locked", ring[0].isPinned());
 		if (graphs) net.useGraphs(true);
 		if (mode == 5) net.conjugateGradients(false);
+		if (mode == 8) net.setInputTrainable(cin, false);
 		net.sync();
 		auto t0 = std::chrono::steady_clock::now();
 		// With prefetch the host runs two batches ahead: while the device computes step s, batch s+1 (assembled during
@@ -975,6 +977,7 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 		expect("losses identical when each is read one step late (gpuQueueLoss)", losses[0] == losses[6]);
 		expect("weights identical when each loss is read one step late", weights[0] == weights[6]);
 		expect("losses and weights identical with gpuTrainStep and the late read together", losses[0] == losses[7] && weights[0] == weights[7]);
+		expect("losses and weights identical with the data input not trainable", losses[0] == losses[8] && weights[0] == weights[8]);
 		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
 		// dz* planes written as the conjugate of the dz product against dz* planes computed by a product of their own
 		double worst = 0, num = 0, den = 0;
@@ -994,9 +997,64 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 		   "\"samples_per_sec_prefetch_graphs\": %.1f, \"ms_per_step_train_step_graph\": %.3f, \"samples_per_sec_train_step_graph\": %.1f, "
 		   "\"ms_per_step_prefetch_two_products_per_gradient_pair\": %.3f, \"ms_per_step_prefetch_loss_read_one_step_late\": %.3f, "
 		   "\"samples_per_sec_prefetch_loss_read_one_step_late\": %.1f, \"ms_per_step_train_step_graph_loss_read_one_step_late\": %.3f, "
+		   "\"ms_per_step_data_input_not_trainable\": %.3f, \"samples_per_sec_data_input_not_trainable\": %.1f, "
 		   "\"upload_bytes_per_step\": %zu}\n",
 			B, steps, ms[0], ms[1], ms[2], ms[3], B / ms[0] * 1e3, B / ms[1] * 1e3, ms[2] > 0 ? B / ms[2] * 1e3 : 0.0, ms[4],
-			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, ms[5], ms[6], B / ms[6] * 1e3, ms[7], (size_t) 2 * B * n * sizeof(float));
+			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, ms[5], ms[6], B / ms[6] * 1e3, ms[7], ms[8], B / ms[8] * 1e3, (size_t) 2 * B * n * sizeof(float));
+}
+
+// ------------------------------------------------------------------------------------------------- frozen data input
+// The data input marked not trainable: the update leaves it alone and the backward pass stops where only it would be
+// served (the FourierTrans of this net).  Losses and every other input function must come out the same to the bit.
+static void test_frozen_input() {
+	const int n = 96, classes = 7, B = 24, steps = 5;
+	if (cnet_init(0) != CNET_OK) {
+		expect("cnet_init", false);
+		return;
+	}
+	SyntheticReader data(n, 3 * B, classes);
+	std::vector<float> losses[2], weights[2], fed, left_on_device[2];
+	for (int frozen = 0; frozen < 2; ++frozen) {
+		CNet net;
+		int inp, outp;
+		build_readme(net, n, classes, &inp, &outp);
+		net.allocateOnGpu(B);
+		CInput *cin = (CInput *) net[inp];
+		CrossEntropy *cen = (CrossEntropy *) net[outp];
+		if (frozen) net.setInputTrainable(cin, false);
+		SyntheticReader reader = data;
+		InputBatch batch(B, n);
+		for (int s = 0; s < steps; ++s) {
+			reader.nextBatch(batch);
+			net.gpuForward(cin, cen, batch);
+			net.gpuBackward();
+			net.gpuUpdateInputs(0.05f / B);
+			losses[frozen].push_back(net.getLoss(cen, NULL));
+		}
+		net.getInputsFromGpu();  // row 0 of every input function
+		for (auto f : net.inputs()) {
+			std::vector<float> &dst = f == cin ? left_on_device[frozen] : weights[frozen];
+			dst.insert(dst.end(), f->input().real_, f->input().real_ + 2 * f->input().length_);
+		}
+		if (frozen) {
+			fed.assign(batch.realDataPtr(0), batch.realDataPtr(0) + n);
+			fed.insert(fed.end(), batch.imagDataPtr(0), batch.imagDataPtr(0) + n);
+		}
+	}
+	expect("losses identical with the data input not trainable", losses[0] == losses[1]);
+	expect("weights identical with the data input not trainable", weights[0] == weights[1] && !weights[0].empty());
+	expect("a data input that is not trainable keeps what was fed", left_on_device[1] == fed);
+	expect("a trainable data input is stepped like a parameter (upstream's behaviour)", left_on_device[0] != left_on_device[1]);
+	bool threw = false;
+	try {
+		CNet other;
+		int a, b;
+		build_readme(other, n, classes, &a, &b);
+		other.setInputTrainable(NULL, false);
+	} catch (const std::invalid_argument &) {
+		threw = true;
+	}
+	expect("setInputTrainable refuses what is not an input function", threw);
 }
 
 // ------------------------------------------------------------------------------------------------- upstream's test nets
@@ -1271,6 +1329,7 @@ int main(int argc, char **argv) {
 		if (what == "pipeline_timing")
 			test_pipeline(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, true, argc > 4 && std::string(argv[4]) == "graphs",
 					argc > 4 && std::string(argv[4]) == "both_halves");
+		if (what == "frozen_input" || what == "all") test_frozen_input();
 		if (what == "upstream_nets" || what == "all") test_upstream_nets();
 		if (what == "errors" || what == "all") test_errors();
 		if (what == "c4")

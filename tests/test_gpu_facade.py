@@ -73,6 +73,12 @@ def test_host_batch_pipeline_prefetch_and_graph_replay_give_the_same_bits():
     assert "FAIL" not in out and out.count("PASS") >= 11 and "samples_per_sec_prefetch" in out
 
 
+def test_data_input_marked_not_trainable():
+    """CNet::setInputTrainable(inp, false): same losses and weights to the bit, the data input keeps what was fed."""
+    out = _run("frozen_input")
+    assert "PASS" in out and "FAIL" not in out
+
+
 def test_nets_of_the_upstream_gpu_tests():
     out = _run("upstream_nets")
     assert "FAIL" not in out and out.count("PASS") >= 25
