@@ -857,7 +857,7 @@ struct SyntheticReader : public BatchedDataReader {
 
 // with_graphs: also run the two modes that replay recorded graphs (left out of plain timing runs: they are not faster, and
 // the profiler's kernel trace has been seen to crash inside hipGraphLaunch on them)
-static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, bool both_halves = false) {
+static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, bool both_halves = false, bool frozen_input = false) {
 	const int n = 784, classes = 10;
 	const float lr = 0.01f;
 	if (cnet_init(0) != CNET_OK) {
@@ -876,6 +876,7 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 	for (int mode = 0; mode < MODES; ++mode) {
 		if (!with_graphs && ((mode >= 2 && mode <= 4) || mode == 7)) continue;
 		if (mode == 5 && timing_only && !both_halves) continue;
+		if (mode == 8 && timing_only && !frozen_input) continue;
 		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4 || mode == 7;
 		const bool late_loss = mode == 6 || mode == 7 || mode == 8;
 		CNet::PendingLoss pending;
@@ -1000,7 +1001,7 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 		   "\"ms_per_step_data_input_not_trainable\": %.3f, \"samples_per_sec_data_input_not_trainable\": %.1f, "
 		   "\"upload_bytes_per_step\": %zu}\n",
 			B, steps, ms[0], ms[1], ms[2], ms[3], B / ms[0] * 1e3, B / ms[1] * 1e3, ms[2] > 0 ? B / ms[2] * 1e3 : 0.0, ms[4],
-			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, ms[5], ms[6], B / ms[6] * 1e3, ms[7], ms[8], B / ms[8] * 1e3, (size_t) 2 * B * n * sizeof(float));
+			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, ms[5], ms[6], B / ms[6] * 1e3, ms[7], ms[8], ms[8] > 0 ? B / ms[8] * 1e3 : 0.0, (size_t) 2 * B * n * sizeof(float));
 }
 
 // ------------------------------------------------------------------------------------------------- frozen data input
@@ -1328,7 +1329,7 @@ int main(int argc, char **argv) {
 		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12, false, true);
 		if (what == "pipeline_timing")
 			test_pipeline(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, true, argc > 4 && std::string(argv[4]) == "graphs",
-					argc > 4 && std::string(argv[4]) == "both_halves");
+					argc > 4 && std::string(argv[4]) == "both_halves", argc > 4 && std::string(argv[4]) == "frozen_input");
 		if (what == "frozen_input" || what == "all") test_frozen_input();
 		if (what == "upstream_nets" || what == "all") test_upstream_nets();
 		if (what == "errors" || what == "all") test_errors();
