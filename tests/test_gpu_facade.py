@@ -73,6 +73,13 @@ def test_host_batch_pipeline_prefetch_and_graph_replay_give_the_same_bits():
     assert "FAIL" not in out and out.count("PASS") >= 11 and "samples_per_sec_prefetch" in out
 
 
+def test_host_batch_pipeline_variants_at_batch_1024():
+    """The same loop variants at a batch where the products take the block kernels (columns split off, K cut): losses and
+    weights must still agree to the bit between all of them."""
+    out = _run("pipeline", "1024", "4")
+    assert "PASS" in out and "FAIL" not in out
+
+
 def test_data_input_marked_not_trainable():
     """CNet::setInputTrainable(inp, false): same losses and weights to the bit, the data input keeps what was fed."""
     out = _run("frozen_input")
