@@ -211,14 +211,16 @@ def test_cgemm_conjugate_combinations(gpu, port, M, N, K, nb):
 
 
 def test_cgemm_random_shapes(gpu, port):
-    """Eighty seeded random problems across the paths of the GEMM: aligned and odd shapes, K with and without a whole
+    """About a hundred seeded random problems across the paths of the GEMM: aligned and odd shapes, K with and without a whole
     number of chunks, every layout, conj(B), accumulation, leading dimensions wider than the matrix, against numpy in
     complex128."""
     rs = np.random.RandomState(20240)
-    for case in range(80):
-        M = int(rs.choice([1, 3, 4, 7, 16, 60, 64, 68, 100, 128, 132, 200, 257, 384, 520]))
-        N = int(rs.choice([1, 2, 4, 10, 16, 36, 64, 72, 128, 196, 260, 512, 784]))
-        K = int(rs.choice([1, 2, 5, 16, 32, 48, 33, 64, 100, 128, 160, 784, 1024]))
+    for case in range(110):
+        M = int(rs.choice([1, 3, 4, 7, 16, 60, 64, 68, 100, 128, 132, 200, 257, 384, 520, 1000, 2048, 4100]))
+        N = int(rs.choice([1, 2, 4, 10, 16, 36, 64, 72, 128, 196, 260, 512, 784, 1040, 1300]))
+        K = int(rs.choice([1, 2, 5, 16, 32, 48, 33, 64, 100, 128, 160, 784, 1024, 2048, 4096]))
+        if M * N * K > 3e9:
+            continue  # the larger ones are there for the paths that only many blocks take (columns split off, K cuts)
         a_km, b_km, cj, acc = int(rs.randint(2)), int(rs.randint(2)), int(rs.randint(2)), int(rs.randint(2))
         pad_a, pad_b, pad_c = (int(rs.choice([0, 4, 8, 3])) for _ in range(3))
         A = rs.randn(M, K) + 1j * rs.randn(M, K)
