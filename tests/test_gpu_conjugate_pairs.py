@@ -42,7 +42,7 @@ def _prefilled(port, seed, rows, cols):
 
 # B, K (in), N (out)
 LINEAR = [(4096, 1024, 1024), (512, 784, 256), (64, 784, 10), (300, 100, 37), (4096, 832, 784), (2048, 544, 544), (4096, 784, 10),
-          (16, 16, 16)]
+          (16, 16, 16), (2048, 550, 549)]   # the last: odd sizes, scalar-load kernel cut along K
 
 
 @pytest.mark.parametrize("B,K,N", LINEAR)
