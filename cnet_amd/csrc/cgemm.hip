@@ -1389,10 +1389,37 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 		}
 	}
 	// float4 path: every contiguous run starts 16-byte aligned and has a length that is a multiple of 4
-	bool vec = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (a.stride_a % 4 == 0) && (a.stride_b % 4 == 0);
-	vec = vec && (a_mcontig ? a.M % 4 == 0 : a.K % 4 == 0) && (b_ncontig ? a.N % 4 == 0 : a.K % 4 == 0);
-	for (int q = 0; q < nprob; ++q)
-		vec = vec && aligned16(a.p[q].a_re) && aligned16(a.p[q].a_im) && aligned16(a.p[q].b_re) && aligned16(a.p[q].b_im);
+	auto vec_ok = [&](int K) {
+		bool v = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (a.stride_a % 4 == 0) && (a.stride_b % 4 == 0);
+		v = v && (a_mcontig ? a.M % 4 == 0 : K % 4 == 0) && (b_ncontig ? a.N % 4 == 0 : K % 4 == 0);
+		for (int q = 0; q < nprob; ++q)
+			v = v && aligned16(a.p[q].a_re) && aligned16(a.p[q].a_im) && aligned16(a.p[q].b_re) && aligned16(a.p[q].b_im);
+		return v;
+	};
+	// A K that is not a whole number of chunks (a batch of 1000 in a weight gradient, a layer 1000 wide) would send the
+	// whole product to the register-staged kernel (109-124 against 135-148 TFLOP/s on such shapes).  Instead the whole
+	// chunks go to the fast kernel and the last 1..15 values of k are added by a second, short launch.
+	static const bool split_k_rest = [] {
+		const char *e = getenv("CNET_CGEMM_KREST");  // tuning override: 0 never splits off the rest of K
+		return !e || atoi(e) != 0;
+	}();
+	const int k_rest = a.K % KC, k_whole = a.K - k_rest;
+	if (split_k_rest && k_rest != 0 && k_whole >= 8 * KC && !a.tri && batch == 1 && vec_ok(k_whole) && (long) a.M * a.N >= 256 * 256) {
+		CgemmArgs head = a, rest = a;
+		head.K = k_whole;
+		rest.K = k_rest;
+		rest.accumulate = 1;  // onto what the first launch has written (its mirror planes too)
+		for (int q = 0; q < nprob; ++q) {
+			const long sa = a_mcontig ? (long) k_whole * a.lda : k_whole, sb = b_ncontig ? (long) k_whole * a.ldb : k_whole;
+			rest.p[q].a_re += sa;
+			rest.p[q].a_im += sa;
+			rest.p[q].b_re += sb;
+			rest.p[q].b_im += sb;
+		}
+		rc = cgemm_dispatch(a_mcontig, b_ncontig, head, nprob, batch);
+		return rc != CNET_OK ? rc : cgemm_dispatch(a_mcontig, b_ncontig, rest, nprob, batch);
+	}
+	const bool vec = vec_ok(a.K);
 	if (vec) {
 		if (!a_mcontig && !b_ncontig) return pick_tile<false, false, 4>(a, nprob, batch);
 		if (!a_mcontig && b_ncontig) return pick_tile<false, true, 4>(a, nprob, batch);

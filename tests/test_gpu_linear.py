@@ -130,11 +130,13 @@ def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(4, 4, 16), (132, 200, 64), (260, 68, 48), (700, 388, 32), (1028, 516, 80), (68, 1300, 160),
-                                   (4100, 1028, 16), (61, 67, 64), (4096, 784, 256)])
+                                   (4100, 1028, 16), (61, 67, 64), (4096, 784, 256), (1028, 516, 1000), (520, 772, 4092)])
 def test_cgemm_blocks_on_the_edge_of_c(gpu, port, M, N, K):
     """K a multiple of 16 with M and N that are not multiples of any block shape: blocks that hang over the edge of C
     read the last valid rows again and must store nothing outside C.  The last shape (784 = 12 x 64 + 16 columns) is one
-    the library computes as two products, columns 0..767 by the block kernel and the 16 left over by the small-C kernel."""
+    the library computes as two products, columns 0..767 by the block kernel and the 16 left over by the small-C kernel;
+    the two after it have a K that is not a whole number of 16-long chunks: the whole chunks go to the fast kernel and the
+    last 8 / 12 values of k are added by a second launch."""
     _check_all_layouts(port, M, N, K)
 
 
@@ -218,7 +220,7 @@ def test_cgemm_random_shapes(gpu, port):
     for case in range(110):
         M = int(rs.choice([1, 3, 4, 7, 16, 60, 64, 68, 100, 128, 132, 200, 257, 384, 520, 1000, 2048, 4100]))
         N = int(rs.choice([1, 2, 4, 10, 16, 36, 64, 72, 128, 196, 260, 512, 784, 1040, 1300]))
-        K = int(rs.choice([1, 2, 5, 16, 32, 48, 33, 64, 100, 128, 160, 784, 1024, 2048, 4096]))
+        K = int(rs.choice([1, 2, 5, 16, 32, 48, 33, 64, 100, 128, 160, 784, 1000, 1024, 2044, 2048, 4096]))
         if M * N * K > 3e9:
             continue  # the larger ones are there for the paths that only many blocks take (columns split off, K cuts)
         a_km, b_km, cj, acc = int(rs.randint(2)), int(rs.randint(2)), int(rs.randint(2)), int(rs.randint(2))
