@@ -42,7 +42,9 @@ def _prefilled(port, seed, rows, cols):
 
 # B, K (in), N (out)
 LINEAR = [(4096, 1024, 1024), (512, 784, 256), (64, 784, 10), (300, 100, 37), (4096, 832, 784), (2048, 544, 544), (4096, 784, 10),
-          (16, 16, 16), (2048, 550, 549)]   # the last: odd sizes, scalar-load kernel cut along K
+          (16, 16, 16), (2048, 550, 549), (1000, 512, 1000)]
+# (2048, 550, 549): odd sizes, scalar-load kernel cut along K; (1000, 512, 1000): both reductions (over out = 1000 and over
+# B = 1000) are not a whole number of chunks, so each product is two launches and the second adds to both halves
 
 
 @pytest.mark.parametrize("B,K,N", LINEAR)
