@@ -235,8 +235,11 @@ def train_lines(steps):
     if not os.path.exists(exe):
         return None
     out = []
-    for batch in (64, 4096):
-        r = subprocess.run([exe, "pipeline_timing", str(batch), str(steps)], capture_output=True, text=True, timeout=600)
+    for batch in (64, 1024, 4096):
+        # "frozen_input" adds the mode in which the data input is marked not trainable (no step on it, no backward pass
+        # into it; off by default in the facade, as upstream steps every input function)
+        r = subprocess.run([exe, "pipeline_timing", str(batch), str(steps), "frozen_input"], capture_output=True, text=True,
+                           timeout=600)
         lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
         if r.returncode != 0 or not lines:
             sys.stderr.write("bench.py: facade_test pipeline_timing failed:\n" + r.stdout[-2000:] + r.stderr[-2000:])
@@ -404,6 +407,7 @@ def main():
                              "ms_per_step": t["ms_per_step_prefetch_loss_read_one_step_late"],
                              "samples_per_sec": t["samples_per_sec_prefetch_loss_read_one_step_late"],
                              "samples_per_sec_loss_read_before_next_step": t["samples_per_sec_prefetch"],
+                             "samples_per_sec_data_input_not_trainable": t["samples_per_sec_data_input_not_trainable"],
                              "samples_per_sec_copy_inside_forward": t["samples_per_sec_copy_in_forward"]} for t in train]
     print(json.dumps(out))
 
