@@ -39,6 +39,16 @@ def test_invalid_arguments_are_reported_not_fatal(gpu, port):
     assert _status("cnet_cgelu_fwd", *x.p(), 8, *y.p(), 8, 0, 8) == 0
     after = y.host()
     assert np.array_equal(before[0], after[0])
+    # the entry points for conjugate gradient pairs check their operands like the two-product ones
+    g = ops.Grad.empty(4, 8)
+    w = ops.CMat.from_host(seeded(port, 3, (8, 8)), seeded(port, 4, (8, 8)))
+    dx = ops.Grad.empty(4, 8)
+    assert _status("cnet_clinear_bwd_input_sym", g.p()[0], None, 8, *w.p(), 8, *dx.p(), 8, 4, 8, 8, 0) == INVALID
+    assert _status("cnet_clinear_bwd_input_sym", *g.p()[:2], 4, *w.p(), 8, *dx.p(), 8, 4, 8, 8, 0) == INVALID      # ldg < N
+    assert _status("cnet_clinear_bwd_weight_sym", *g.p()[:2], 8, *x.p(), 8, dx.p()[0], dx.p()[1], dx.p()[2], None, 8, 4, 8, 8, 0) == INVALID
+    assert _status("cnet_cdft_bwd_sym", *g.p()[:2], 8, *dx.p(), 4, 4, 8, 0) == INVALID                               # lddx < n
+    assert _status("cnet_ctriang_dft_bwd_sym", *g.p()[:2], 8, *dx.p(), 8, 4, 50000, 0) == INVALID
+    assert _status("cnet_cdft_bwd_sym", *g.p()[:2], 8, *dx.p(), 8, 0, 8, 0) == 0                                     # no rows: nothing to do
     # DFT length beyond the int exponent range of the reference, Adam with a negative step, unknown marker
     assert _status("cnet_cdft_plan", 50000) == INVALID
     assert _status("cnet_adam_update", x.re.ptr, x.im.ptr, y.re.ptr, y.im.ptr, y.re.ptr, y.im.ptr, 32, 0.1, 0.9, -1, 1) == INVALID
