@@ -1152,7 +1152,17 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 		}
 	}
 	dim3 grid(args.tiles_m * grid_tiles_n(args), nprob, batch * args.splits);
-	if (tail_splits >= 2 && VEC == 4 && args.K % KC == 0 && !args.tri && batch == 1 && args.splits == 1) {
+	// The fast kernel addresses a lane's 16 bytes inside the operand tile of a chunk with an unsigned 32-bit byte offset:
+	// (row * ld + k) * 4 for rows < min(block edge, rows of the operand), or (k * ld + row) * 4 for k < KC.  A leading
+	// dimension beyond that (8.4 M floats for a K-contiguous operand under a 128-row block) goes to cgemm_kernel, whose
+	// offsets are 64-bit.
+	auto offsets_fit = [](long ld, bool rows_contig, int block_rows, int rows) {
+		const long last = rows_contig ? (long) (KC - 1) * ld + block_rows : (long) (std::min(block_rows, rows) - 1) * ld + KC;
+		return last * 4 < (1L << 32);
+	};
+	const bool fast_ok = VEC == 4 && args.K % KC == 0 && offsets_fit(args.lda, A_MCONTIG, BM, args.M) &&
+			offsets_fit(args.ldb, B_NCONTIG, BN, args.N);
+	if (tail_splits >= 2 && fast_ok && !args.tri && batch == 1 && args.splits == 1) {
 		const long cus = cnet::rt().prop.multiProcessorCount;
 		const long all = (long) args.tiles_m * args.tiles_n * nprob;
 		const int nchunks = args.K / KC;
@@ -1179,7 +1189,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 		return CNET_OK;
 	};
 	if constexpr (VEC == 4) {
-		if (args.K % KC == 0) {  // any M and N: edge blocks re-read the last valid rows and store only what is inside C
+		if (fast_ok) {  // any M and N: edge blocks re-read the last valid rows and store only what is inside C
 			constexpr int NST = (BM == 128 && BN == 128) ? 2 : 3;
 			constexpr size_t fast_smem = (size_t) NST * 2 * KC * (BM + BN) * sizeof(float);
 			static bool fast_attr_set = false;

@@ -37,7 +37,13 @@ struct Runtime {
 	size_t workspace_bytes = 0;
 	// A recorded graph holds the workspace address it was recorded with: while any recording exists, a workspace that
 	// has to grow is retired (kept until shutdown) instead of freed.
+	// Each live recording is kept as (executable, the graph it was instantiated from): the template graph lives as long
+	// as its executable, so that nothing that still walks its nodes (a tracing tool) finds them gone, and shutdown can
+	// destroy what the caller left behind.
 	int graphs_alive = 0;
+	static constexpr int kGraphs = 256;
+	hipGraphExec_t graph_exec[kGraphs] = {};
+	hipGraph_t graph_template[kGraphs] = {};
 	static constexpr int kRetired = 16;
 	void *retired[kRetired] = {};
 	int retired_count = 0;

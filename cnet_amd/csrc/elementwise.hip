@@ -900,7 +900,7 @@ int cnet_sgd_update_multi(int count, float *const *z_re, float *const *z_im, flo
 		SgdMulti t;
 		int used = 0;
 		long longest = 0;
-		for (int k = first; k < count && used < SGD_MULTI_MAX; ++k) {
+		for (int k = first; k < count && k < first + SGD_MULTI_MAX; ++k) {
 			if (!n[k]) continue;
 			t.z_re[used] = z_re[k];
 			t.z_im[used] = z_im[k];

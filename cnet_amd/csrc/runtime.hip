@@ -127,7 +127,23 @@ int cnet_init(int device) {
 int cnet_shutdown(void) {
 	Runtime &r = rt();
 	if (!r.ready) return CNET_OK;
-	hipStreamSynchronize(r.stream);
+	int rc = CNET_OK;
+	if (r.capturing) {  // an open recording is ended and dropped: the stream cannot be waited for while it records
+		hipGraph_t open_graph = nullptr;
+		(void) hipStreamEndCapture(r.stream, &open_graph);
+		if (open_graph) (void) hipGraphDestroy(open_graph);
+		(void) hipGetLastError();
+		r.capturing = false;
+	}
+	hipError_t sync_err = hipStreamSynchronize(r.stream);
+	if (sync_err != hipSuccess) rc = hip_fail(sync_err, "cnet_shutdown: hipStreamSynchronize");
+	// recordings the caller did not destroy: their handles die with the library's buffers
+	for (int k = 0; k < Runtime::kGraphs; ++k) {
+		if (r.graph_exec[k]) (void) hipGraphExecDestroy(r.graph_exec[k]);
+		if (r.graph_template[k]) (void) hipGraphDestroy(r.graph_template[k]);
+		r.graph_exec[k] = nullptr;
+		r.graph_template[k] = nullptr;
+	}
 	release_twiddles();
 	if (r.workspace) hipFree(r.workspace);
 	r.workspace = nullptr;
@@ -136,10 +152,9 @@ int cnet_shutdown(void) {
 	r.retired_count = 0;
 	r.graphs_alive = 0;
 	destroy_streams(r);
-	r.capturing = false;
 	r.ready = false;
 	r.device = -1;
-	return CNET_OK;
+	return rc;
 }
 
 int cnet_get_device_info(cnet_device_info *out) {
@@ -353,29 +368,59 @@ int cnet_graph_end(void **graph_exec) {
 		(void) hipGraphDestroy(graph);
 		return CNET_OK;
 	}
+	*graph_exec = nullptr;
+	int slot = 0;
+	while (slot < Runtime::kGraphs && r.graph_exec[slot]) ++slot;
+	if (slot == Runtime::kGraphs) {
+		(void) hipGraphDestroy(graph);
+		return fail(CNET_ERR_UNSUPPORTED, "cnet_graph_end: %d recordings exist already: destroy some first", Runtime::kGraphs);
+	}
 	hipGraphExec_t exec = nullptr;
 	e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-	(void) hipGraphDestroy(graph);
-	if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+	if (e != hipSuccess) {
+		(void) hipGraphDestroy(graph);
+		return hip_fail(e, "hipGraphInstantiate");
+	}
+	// the graph the executable was made from is kept until cnet_graph_destroy
+	r.graph_exec[slot] = exec;
+	r.graph_template[slot] = graph;
 	*graph_exec = exec;
 	r.graphs_alive++;
 	return CNET_OK;
+}
+
+// slot of a live recording, -1 for a handle this library did not hand out (or has destroyed already)
+static int graph_slot(void *graph_exec) {
+	Runtime &r = rt();
+	for (int k = 0; k < Runtime::kGraphs; ++k)
+		if (r.graph_exec[k] && (void *) r.graph_exec[k] == graph_exec) return k;
+	return -1;
 }
 
 int cnet_graph_launch(void *graph_exec) {
 	CNET_REQUIRE_INIT();
 	CNET_NOT_IN_CAPTURE();
 	CNET_CHECK_ARG(graph_exec != nullptr);
+	if (graph_slot(graph_exec) < 0) return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_graph_launch: not a live recording of this library");
 	CNET_HIP(hipGraphLaunch((hipGraphExec_t) graph_exec, rt().stream));
 	return CNET_OK;
 }
 
 int cnet_graph_destroy(void *graph_exec) {
 	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // waits for the stream, which would break the recording
 	if (!graph_exec) return CNET_OK;
-	CNET_HIP(hipStreamSynchronize(rt().stream));
-	CNET_HIP(hipGraphExecDestroy((hipGraphExec_t) graph_exec));
-	if (rt().graphs_alive > 0) rt().graphs_alive--;
+	Runtime &r = rt();
+	const int slot = graph_slot(graph_exec);
+	if (slot < 0) return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_graph_destroy: not a live recording of this library");
+	CNET_HIP(hipStreamSynchronize(r.stream));
+	const hipError_t e1 = hipGraphExecDestroy(r.graph_exec[slot]);
+	const hipError_t e2 = hipGraphDestroy(r.graph_template[slot]);
+	r.graph_exec[slot] = nullptr;
+	r.graph_template[slot] = nullptr;
+	if (r.graphs_alive > 0) r.graphs_alive--;
+	if (e1 != hipSuccess) return hip_fail(e1, "hipGraphExecDestroy");
+	if (e2 != hipSuccess) return hip_fail(e2, "hipGraphDestroy");
 	return CNET_OK;
 }
 

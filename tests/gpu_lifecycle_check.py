@@ -40,6 +40,27 @@ def main():
         print("FAIL: a second cnet_shutdown is not a no-op")
         return 1
     capi.init(0)
+    # a shutdown with a recording left alive and another one still open: the open one is dropped, the live one destroyed
+    # with the library's buffers, and the next initialisation starts clean
+    import ctypes as C
+    x = ops.CMat.from_host(np.ones((4, 8), np.float32), np.ones((4, 8), np.float32))
+    y = ops.CMat.empty(4, 8)
+    ops.gelu_fwd(x, y)
+    capi.call("cnet_graph_begin")
+    ops.gelu_fwd(x, y)
+    exe = C.c_void_p()
+    capi.call("cnet_graph_end", C.byref(exe))
+    capi.call("cnet_graph_launch", exe)
+    capi.call("cnet_graph_begin")
+    ops.gelu_fwd(x, y)
+    if lib.cnet_shutdown() != 0:
+        print("FAIL: cnet_shutdown with a live and an open recording: " + lib.cnet_last_error().decode())
+        return 1
+    capi.init(0)
+    del x, y   # the device allocations outlive the library's own state
+    if lib.cnet_graph_launch(exe) != -2:
+        print("FAIL: a recording from before the shutdown was accepted")
+        return 1
     second = work()
     for a, b in zip(first, second):
         if not np.array_equal(a, b):

@@ -110,8 +110,69 @@ def test_graph_recording_rules_and_replay(gpu, port):
         assert h[0] == 1 and not h[1:501].any() and h[501] == 1
         ops.residual_fwd(y, y, z)  # unrelated eager work between replays
         capi.sync()
+    # a recording cannot be destroyed while another one is being recorded (the call waits for the stream)
+    capi.call("cnet_graph_begin")
+    assert _status("cnet_graph_destroy", exe) == UNSUPPORTED and "cnet_graph_begin" in _msg()
+    capi.call("cnet_graph_end", None)
+    capi.call("cnet_graph_launch", exe)   # ... and is still whole
+    capi.sync()
     capi.call("cnet_graph_destroy", exe)
     capi.call("cnet_graph_destroy", None)
+    # a handle that is not a live recording is refused, not handed to the runtime
+    assert _status("cnet_graph_launch", exe) == INVALID and _status("cnet_graph_destroy", exe) == INVALID
+
+
+def test_sgd_update_of_more_tensors_than_one_launch_takes_steps_each_once(gpu, port):
+    """Ten tensors, one of them empty, gradients kept (zero_grad = 0): every tensor is stepped exactly once (a launch takes
+    eight table entries; the empty one must not shift the next launch's window)."""
+    sizes = [16, 12, 0, 8, 5, 64, 7, 9, 33, 4]
+    zs, ds, want = [], [], []
+    for k, n in enumerate(sizes):
+        m = max(n, 1)
+        zr, zi, dr, di = [seeded(port, 100 + 4 * k + j, (1, m)) for j in range(4)]
+        zs.append(ops.CMat.from_host(zr, zi)); ds.append((ops.Plane.from_host(dr), ops.Plane.from_host(di)))
+        a, b = zr.copy(), zi.copy()
+        if n:
+            port.sgd_update(a, b, dr.copy(), di.copy(), 0.5)
+        want.append((a, b, dr, di))
+    arr = lambda ptrs: (C.c_void_p * len(ptrs))(*ptrs)
+    lens = (C.c_int64 * len(sizes))(*sizes)
+    capi.call("cnet_sgd_update_multi", len(sizes), arr([z.re.ptr for z in zs]), arr([z.im.ptr for z in zs]),
+              arr([d[0].ptr for d in ds]), arr([d[1].ptr for d in ds]), lens, 0.5, 0)
+    for n, z, d, (a, b, dr, di) in zip(sizes, zs, ds, want):
+        h = z.host()
+        assert np.array_equal(h[0], a) and np.array_equal(h[1], b), n
+        assert np.array_equal(d[0].host(), dr) and np.array_equal(d[1].host(), di), n
+
+
+def test_operand_rows_further_apart_than_32_bit_offsets_reach(gpu):
+    """A K-contiguous operand whose rows lie 8.4 M floats apart: inside a 128-row block the byte offset of the last rows
+    passes 2^32, which the kernel that moves tiles straight into LDS cannot address.  Such a product must take the kernel
+    with 64-bit offsets and give the same result (4.3 GB of device memory per plane, written row by row)."""
+    M, N, K = 128, 64, 32
+    ld = (1 << 32) // 4 // 127 + 8        # 127 * ld * 4 > 2^32
+    assert ld % 4 == 0 and 127 * ld * 4 >= 1 << 32
+    rng = np.random.default_rng(11)
+    ar, ai = rng.standard_normal((M, K), dtype=np.float32), rng.standard_normal((M, K), dtype=np.float32)
+    br, bi = rng.standard_normal((N, K), dtype=np.float32), rng.standard_normal((N, K), dtype=np.float32)
+    bytes_plane = ((M - 1) * ld + K) * 4
+    pa = [C.c_void_p(), C.c_void_p()]
+    for p in pa:
+        capi.call("cnet_alloc", bytes_plane, C.byref(p))
+    try:
+        for p, host in zip(pa, (ar, ai)):
+            for r in range(M):
+                row = np.ascontiguousarray(host[r])
+                capi.call("cnet_memcpy_h2d", C.c_void_p(p.value + 4 * r * ld), row.ctypes.data_as(C.c_void_p), 4 * K)
+        Bm, c = ops.CMat.from_host(br, bi), ops.CMat.empty(M, N)
+        capi.call("cnet_cgemm", 0, 0, 0, M, N, K, pa[0], pa[1], ld, *Bm.p(), Bm.ld, *c.p(), c.ld, 0)
+        want = (ar.astype(np.float64) + 1j * ai) @ (br.astype(np.float64) + 1j * bi).T
+        got = c.host()
+        err = np.linalg.norm(got[0] + 1j * got[1] - want) / np.linalg.norm(want)
+        assert err < 1e-6, err
+    finally:
+        for p in pa:
+            capi.call("cnet_free", p)
 
 
 def test_out_of_range_labels_and_token_ids_touch_nothing_outside_their_operands(gpu, port):

@@ -68,20 +68,37 @@ def test_l2out(gpu, port, B, n):
         assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("B,n", [(1, 1), (3, 6), (7, 97), (5, 1024), (4, 3000)])
-def test_softmax_l2_normalisation(gpu, port, B, n):
+# (B, n, ld): the row lengths walk every kernel the dispatcher can pick: rows held in registers (128-bit path up to 8192
+# columns forward / 4096 backward), the two-pass kernels beyond that with one or four wavefronts per row, their scalar
+# twins for lengths that are not a multiple of 4, and rows inside a wider buffer (ld > n).
+SOFTMAX_CASES = [(1, 1, 0), (3, 6, 0), (7, 97, 0), (5, 1024, 0), (3, 2048, 0), (4, 3000, 0), (2, 4100, 0), (2, 5001, 0),
+                 (2, 8196, 0), (3, 32768, 0), (2, 32772, 32780), (2, 1030, 1033)]
+
+
+@pytest.mark.parametrize("B,n,ld", SOFTMAX_CASES)
+def test_softmax_l2_normalisation(gpu, port, B, n, ld):
+    ld = ld or n
     zr, zi = seeded(port, 1, (B, n)), seeded(port, 2, (B, n))
     g4 = [seeded(port, 5 + p, (B, n)) for p in range(4)]
     yr, yi, S = port.softmax_fwd(zr, zi)
-    z, g = ops.CMat.from_host(zr, zi), ops.Grad.from_host(g4)
-    y, s, dz = ops.CMat.empty(B, n), capi.empty(B), ops.Grad.empty(B, n)
+
+    def padded(a):   # the rows inside a buffer ld wide; the padding must come back untouched
+        w = np.full((B, ld), 7.0, np.float32)
+        w[:, :n] = a
+        return ops.Plane.from_host(w).sub(0, n)
+
+    z, g = ops.CMat(padded(zr), padded(zi)), ops.Grad([padded(a) for a in g4])
+    y, s = ops.CMat(padded(0 * zr), padded(0 * zr)), capi.empty(B)
+    dz = ops.Grad([padded(0 * zr) for _ in range(4)])
     ops.l2norm_fwd(z, y, s)
     ops.l2norm_bwd(z, s, g, dz)
     assert rel_c(y.host(), (yr, yi)) < 1e-6 and rel(s.download(), S) < 1e-6
     h = dz.host()
-    if n <= 1024:   # the oracle's chain rule is O(n^2)
-        dzo = port.softmax_bwd(zr, zi, g4)
-        assert rel_c(h[0:2], dzo[0:2]) < 2e-5 and rel_c(h[2:4], dzo[2:4]) < 2e-5
+    # the oracle's chain rule is O(n^2) per row (6 s for two rows of 32768): the longest rows compare their first row
+    # only
+    rows = slice(0, B) if n <= 8196 else slice(0, 1)
+    dzo = port.softmax_bwd(zr[rows], zi[rows], [a[rows] for a in g4])
+    assert rel_c([a[rows] for a in h[0:2]], dzo[0:2]) < TOL and rel_c([a[rows] for a in h[2:4]], dzo[2:4]) < TOL
     Z = zr.astype(np.float64) + 1j * zi
     G, Gs = g4[0].astype(np.float64) + 1j * g4[1], g4[2].astype(np.float64) + 1j * g4[3]
     Sd = (abs(Z) ** 2).sum(1, keepdims=True)
@@ -89,3 +106,11 @@ def test_softmax_l2_normalisation(gpu, port, B, n):
     e1 = G / np.sqrt(Sd) - Z.conj() * A / (2 * Sd ** 1.5)
     e2 = Gs / np.sqrt(Sd) - Z * A / (2 * Sd ** 1.5)
     assert rel_c(h[0:2], (e1.real, e1.imag)) < 1e-5 and rel_c(h[2:4], (e2.real, e2.imag)) < 1e-5
+    # accumulate adds a second copy onto what the planes hold
+    ops.l2norm_bwd(z, s, g, dz, accumulate=1)
+    h2 = dz.host()
+    for p in range(4):
+        assert rel(h2[p], 2.0 * h[p]) < 1e-6
+    if ld > n:
+        for pl in [y.re, y.im] + dz.planes:
+            assert np.all(pl.owner.download().reshape(B, ld)[:, n:] == 7.0)
