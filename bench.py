@@ -21,9 +21,26 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X published dense fp32 matrix peak
 # Bytes the eight L2s exchanged with the fabric per launch (FETCH_SIZE + WRITE_SIZE of `rocprofv3 --pmc`, each scaled by
-# what the same counter reads for a 256 MiB copy kernel: x2.000 and x1.000); an upper bound on HBM traffic, since hits
-# in the memory-side cache are included.  Source: profiles/cgemm_linear_b4096_1024x1024_counters.md.
-MEASURED_TRAFFIC_BYTES = {"linear_fwd": 197399783, "linear_bwd_input": 235300390, "linear_bwd_weight": 417957585}
+# what the same counter reads for a 256 MiB copy kernel); an upper bound on HBM traffic, since hits in the memory-side
+# cache are included.  Counters cannot be read inside this run: the figures come from the committed summary of a counter
+# run of this same command (`--counter-pass`), which names the commit it was measured at.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "cgemm_linear_b4096_1024x1024_traffic.txt")
+
+
+def measured_traffic():
+    """{launch: bytes} and the commit the counters were collected at, from profiles/ (None, None when absent)."""
+    if not os.path.exists(TRAFFIC_FILE):
+        return None, None
+    table, at = {}, None
+    for line in open(TRAFFIC_FILE):
+        f = line.split()
+        if len(f) >= 2 and f[0] == "measured_at":
+            at = f[1]
+        elif len(f) >= 2 and not line.startswith("#") and f[1].isdigit():
+            table[f[0]] = int(f[1])
+    return table, at
+
+
 B, K, N = 4096, 1024, 1024      # BASELINE.json configs[1]
 
 
@@ -186,23 +203,25 @@ def kernel_suite(steps):
     hbm("cross_entropy_fwd (loss, argmax; no normalised output)", [R, Cc], 8, n,
         lambda: ops.cross_entropy_fwd(z, labels, s_, l_, am, None), extra_bytes=4 * R)
     hbm("cross_entropy_bwd", [R, Cc], 24, n, lambda: ops.cross_entropy_bwd(z, s_, labels, dz))
-    for ln in lines:
-        print(json.dumps(ln))
+    return lines
 
 
 def token_model_suite(steps):
     """Fifth configuration at full size: batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096; forward + backward."""
     from cnet_amd import capi
     from cnet_amd.workloads import TokenModel
-    from oracle import binding as ob
     capi.init(0)
-    gen = ob.load_port()
+    rng = np.random.default_rng(0)
     Bq, S, D, H, V = 16, 512, 1024, 4096, 32768
-    P = {"table": gen.normal(1, (2, V, D)), "gate": gen.normal(2, (2, D), 0, 0.05),
-         "w1": gen.normal(3, (2, H, D), 0, D ** -0.5), "w2": gen.normal(4, (2, D, H), 0, H ** -0.5),
-         "w3": gen.normal(5, (2, V, D), 0, D ** -0.5)}
-    ids = gen.randint(6, (Bq, S), V)
+
+    def normal(shape, sig=1.0):
+        return (sig * rng.standard_normal(shape, dtype=np.float32)).astype(np.float32)
+
+    P = {"table": normal((2, V, D)), "gate": normal((2, D), 0.05), "w1": normal((2, H, D), D ** -0.5),
+         "w2": normal((2, D, H), H ** -0.5), "w3": normal((2, V, D), D ** -0.5)}
+    ids = rng.integers(0, V, (Bq, S)).astype(np.int32)
     ev = HipEvents(capi.load().cnet_stream())
+    out = []
     # first with every product computed (what upstream's backward pass does), then with the dz* halves of the gradient
     # pairs written as conjugates of the dz products (the loss is real); one model at a time on the device
     for conjugate_pairs in (False, True):
@@ -217,42 +236,67 @@ def token_model_suite(steps):
         ev.record(b)
         ms = ev.elapsed_ms(a, b) / steps
         loss = float(model.loss.download().mean())
-        print(json.dumps({"workload": "configs[4]: complex token model fwd+bwd, batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096",
-                          "gradient_pairs": "dz* written as conj(dz)" if conjugate_pairs else "both halves computed",
-                          "ms_per_step": round(ms, 3), "tokens_per_sec": round(Bq * S / ms * 1e3, 1),
-                          "gemm_tflops_executed": round(model.gemm_flops() / ms / 1e9, 2), "mean_loss": round(loss, 4),
-                          "loss_of_uniform_guess": round(float(np.log(V)), 4)}), flush=True)
+        out.append({"workload": "configs[4]: complex token model fwd+bwd, batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096",
+                    "gradient_pairs": "dz* written as conj(dz)" if conjugate_pairs else "both halves computed",
+                    "ms_per_step": round(ms, 3), "tokens_per_sec": round(Bq * S / ms * 1e3, 1),
+                    "gemm_tflops_executed": round(model.gemm_flops() / ms / 1e9, 2), "mean_loss": round(loss, 4),
+                    "loss_of_uniform_guess": round(float(np.log(V)), 4)})
         del model
+    return out
+
+
+TRAIN_BENCH = os.path.join(ROOT, "cnet_amd", "bin", "train_bench")
+
+
+def _train_bench(*args):
+    """One run of the C++ timing driver (cnet_amd/host/train_bench.cpp) in a process of its own; its JSON line or None."""
+    import subprocess
+    if not os.path.exists(TRAIN_BENCH):
+        return None
+    r = subprocess.run([TRAIN_BENCH] + [str(a) for a in args], capture_output=True, text=True, timeout=600)
+    lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
+    if r.returncode != 0 or not lines:
+        sys.stderr.write("bench.py: train_bench %s failed:\n" % " ".join(map(str, args)) + r.stdout[-2000:] + r.stderr[-2000:])
+        return None
+    return json.loads(lines[-1])
 
 
 def train_lines(steps):
     """Training steps (upload of the batch, forward, loss read-back, backward, SGD) of the FourierTrans -> Hadamard ->
-    CGelu -> Linear -> CrossEntropy net on 784-long samples, run by the C++ facade's own driver in a process of its own;
-    one dict per batch size with the time per step of each input mode (copy inside forward / prefetch / recorded
-    graphs).  None when the driver is not built or fails."""
-    import subprocess
-    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "bin", "facade_test")
-    if not os.path.exists(exe):
-        return None
+    CGelu -> Linear -> CrossEntropy net on 784-long samples through the C++ facade; one dict per batch size with the
+    time per step of each input mode.  None when the driver is not built or fails."""
     out = []
     for batch in (64, 1024, 4096):
         # "frozen_input" adds the mode in which the data input is marked not trainable (no step on it, no backward pass
         # into it; off by default in the facade, as upstream steps every input function)
-        r = subprocess.run([exe, "pipeline_timing", str(batch), str(steps), "frozen_input"], capture_output=True, text=True,
-                           timeout=600)
-        lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
-        if r.returncode != 0 or not lines:
-            sys.stderr.write("bench.py: facade_test pipeline_timing failed:\n" + r.stdout[-2000:] + r.stderr[-2000:])
+        line = _train_bench("readme", batch, steps, "frozen_input")
+        if line is None:
             return None
-        out.append(json.loads(lines[-1]))
+        out.append(line)
+    return out
+
+
+STACK_LR = 3e-6   # configs[3] names 0.01, at which fp32 overflows in the first update on the CPU path as well; 1e-5 still diverges
+
+
+def stack_lines(steps=10):
+    """configs[3]: 8 x (Linear 2048 -> 2048, CGelu, Residual), L2Out, batch 2048, `steps` SGD steps through the C++ facade,
+    both data inputs uploaded and the loss read back every step; first with the dz* halves of the gradient pairs written
+    as conjugates (the facade's default), then with both halves computed as upstream does."""
+    out = []
+    for mode in ((), ("both_halves",)):
+        line = _train_bench("stack", 2048, 8, 2048, steps, STACK_LR, *mode)
+        if line is None:
+            return None
+        out.append(line)
     return out
 
 
 def train_suite(steps):
     lines = train_lines(steps)
     if lines is None:
-        sys.exit("bench.py: tests/bin/facade_test is missing or failed; run __graft_entry__.build() first")
-    for l in lines:
+        sys.exit("bench.py: cnet_amd/bin/train_bench is missing or failed; run __graft_entry__.build() first")
+    for l in lines + (stack_lines() or []):
         print(json.dumps(l))
 
 
@@ -275,10 +319,12 @@ def main():
                  "supported. Run with --gpus 1." % args.gpus)
 
     if args.suite == "kernels":
-        kernel_suite(max(args.steps // 5, 10))
+        for ln in kernel_suite(max(args.steps // 5, 10)):
+            print(json.dumps(ln))
         return
     if args.suite == "token_model":
-        token_model_suite(max(args.steps // 20, 3))
+        for ln in token_model_suite(max(args.steps // 20, 3)):
+            print(json.dumps(ln), flush=True)
         return
     if args.suite == "train":
         train_suite(max(args.steps, 30))
@@ -294,11 +340,14 @@ def main():
     except Exception:  # torch is only used for the contract's device-wide synchronize
         tsync = lambda: None
 
-    from oracle import binding as ob   # seeded generator only (identical arrays for every backend)
-    gen = ob.load_port()
-    x = ops.CMat.from_host(gen.normal(1, (B, K)), gen.normal(2, (B, K)))
-    w = ops.CMat.from_host(gen.normal(3, (N, K), 0, K ** -0.5), gen.normal(4, (N, K), 0, K ** -0.5))
-    g = ops.Grad.from_host([gen.normal(5 + p, (B, N)) for p in range(4)])
+    rng = np.random.default_rng(0)
+
+    def normal(shape, sig=1.0):
+        return (sig * rng.standard_normal(shape, dtype=np.float32)).astype(np.float32)
+
+    x = ops.CMat.from_host(normal((B, K)), normal((B, K)))
+    w = ops.CMat.from_host(normal((N, K), K ** -0.5), normal((N, K), K ** -0.5))
+    g = ops.Grad.from_host([normal((B, N)) for _ in range(4)])
     y, dx, dw = ops.CMat.empty(B, N), ops.Grad.empty(B, K), ops.Grad.empty(N, K)
 
     launches = {
@@ -350,10 +399,12 @@ def main():
         fl = 8.0 * B * N * K * ngemm
         kern[name] = {"ms": round(ms, 4), "flops": fl, "tflops": round(fl / ms / 1e9, 2)}
     dom = max(kern, key=lambda k: kern[k]["ms"])
-    traffic = MEASURED_TRAFFIC_BYTES.get(dom)
+    traffic_table, traffic_at = measured_traffic()
+    traffic = traffic_table.get(dom) if traffic_table else None
     roofline = {"bound": "mfma", "kernel": "cgemm_fast_kernel (%s)" % dom, "achieved": kern[dom]["tflops"],
                 "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(kern[dom]["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": traffic,
+                "traffic_measured_at": traffic_at,
                 "flops_per_launch": kern[dom]["flops"], "avg_launch_ms": kern[dom]["ms"],
                 "all_launches": kern, "device_clock_khz": info.clock_khz, "compute_units": info.compute_units}
 
@@ -361,7 +412,8 @@ def main():
         # Beside the headline (all five products computed, whatever the gradient planes hold): the same layer step through the
         # entry points for a conjugate gradient pair (dz* = conj(dz), as under every real loss), which compute three products
         # and write the other two as conjugates.  Its rate counts the three products that are executed.
-        gc = ops.Grad.from_host([gen.normal(5, (B, N)), gen.normal(6, (B, N)), gen.normal(5, (B, N)), -gen.normal(6, (B, N))])
+        gr, gi = normal((B, N)), normal((B, N))
+        gc = ops.Grad.from_host([gr, gi, gr, -gi])
 
         def step_sym():
             ops.linear_fwd(x, w, y)
@@ -409,6 +461,13 @@ def main():
                              "samples_per_sec_loss_read_before_next_step": t["samples_per_sec_prefetch"],
                              "samples_per_sec_data_input_not_trainable": t["samples_per_sec_data_input_not_trainable"],
                              "samples_per_sec_copy_inside_forward": t["samples_per_sec_copy_in_forward"]} for t in train]
+        # the other configurations and kernels of the hot path, each bounded to a few seconds
+        del x, w, g, y, dx, dw
+        stack = stack_lines(10)
+        if stack:
+            out["configs3_residual_stack"] = stack
+        out["kernels"] = kernel_suite(20)
+        out["configs4_token_model"] = token_model_suite(3)
     print(json.dumps(out))
 
 

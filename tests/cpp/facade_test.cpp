@@ -10,10 +10,10 @@
 //   facade_test adam               TriangFourier / CRelu net trained with the Adam-style step, batched and per sample
 //   facade_test saved_model <golden dir> <scratch dir>   upstream-written .mod files restored and run on the device
 //   facade_test pipeline [B steps]  reader -> page-locked batches -> device, with and without gpuPrefetch (same bits)
-//   facade_test pipeline_timing B steps [graphs]   the same, timing only (JSON line); `graphs` adds the graph-replay modes
 //   facade_test upstream_nets      the nets of upstream's own GPU tests (E2E chain, fan-out into one consumer, ...)
 //   facade_test errors             error behaviour
-//   facade_test c4 n blocks B steps lr   throughput of the residual stack (no oracle), JSON line
+//   facade_test stack8 n blocks B steps lr rows overflow|finite [learn]   residual stack of `blocks` blocks against the
+//                                  oracle on `rows` rows of the batch (0: all rows, every step)
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -855,9 +855,7 @@ struct SyntheticReader : public BatchedDataReader {
 	bool readData() override { return true; }
 };
 
-// with_graphs: also run the two modes that replay recorded graphs (left out of plain timing runs: they are not faster, and
-// the profiler's kernel trace has been seen to crash inside hipGraphLaunch on them)
-static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, bool both_halves = false, bool frozen_input = false) {
+static void test_pipeline(int B, int steps) {
 	const int n = 784, classes = 10;
 	const float lr = 0.01f;
 	if (cnet_init(0) != CNET_OK) {
@@ -874,9 +872,6 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 	std::vector<float> weights[MODES];
 	double ms[MODES] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
 	for (int mode = 0; mode < MODES; ++mode) {
-		if (!with_graphs && ((mode >= 2 && mode <= 4) || mode == 7)) continue;
-		if (mode == 5 && timing_only && !both_halves) continue;
-		if (mode == 8 && timing_only && !frozen_input) continue;
 		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4 || mode == 7;
 		const bool late_loss = mode == 6 || mode == 7 || mode == 8;
 		CNet::PendingLoss pending;
@@ -888,7 +883,7 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 		CrossEntropy *cen = (CrossEntropy *) net[outp];
 		SyntheticReader reader = data;  // same order for both modes
 		InputBatch ring[3] = {InputBatch(B, n), InputBatch(B, n), InputBatch(B, n)};
-		if (mode == 0 && !timing_only) expect("batches built after cnet_init are page-locked", ring[0].isPinned());
+		if (mode == 0) expect("batches built after cnet_init are page-locked", ring[0].isPinned());
 		if (graphs) net.useGraphs(true);
 		if (mode == 5) net.conjugateGradients(false);
 		if (mode == 8) net.setInputTrainable(cin, false);
@@ -938,7 +933,7 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 			if (f == cin) continue;
 			weights[mode].insert(weights[mode].end(), f->input().real_, f->input().real_ + 2 * f->input().length_);
 		}
-		if (mode == 1 && !timing_only) {
+		if (mode == 1) {
 			// error behaviour of the staging
 			InputBatch a(B, n), b(B, n);
 			reader.nextBatch(a);
@@ -966,7 +961,7 @@ static void test_pipeline(int B, int steps, bool timing_only, bool with_graphs, 
 			expect("a batch of the wrong shape is refused", threw);
 		}
 	}
-	if (!timing_only) {
+	{
 		expect("losses identical with and without prefetch (" + std::to_string(steps) + " steps)", losses[0] == losses[1]);
 		expect("weights identical after training with and without prefetch", weights[0] == weights[1] && !weights[0].empty());
 		expect("losses identical with graph replay (prefetch)", losses[0] == losses[2]);
@@ -1253,64 +1248,144 @@ static void test_errors() {
 	expect("error text names the call", std::string(cnet_last_error()).find("cnet_cgemm") != std::string::npos);
 }
 
-// ------------------------------------------------------------------------------------------------- throughput
-static void run_c4(int n, int blocks, int B, int steps, float lr, bool both_halves) {
+// ------------------------------------------------------------------------------------------------- residual stack, 8 blocks
+// The residual-stack workload (8 x (Linear n -> n, CGelu, Residual), L2Out against targets, SGD) against the oracle run
+// sample by sample, over `rows_checked` rows of the batch (all rows when 0): per-sample losses, the dz* that reaches the
+// data input through all blocks, and - when every row is checked - the batch-summed weight gradients and the weights
+// after each step.  Eight un-normalised blocks amplify the input about 4000 times, so the configured rate of 0.01
+// overflows fp32 in the first update on the CPU path itself: `expect_overflow` asserts that the device leaves the finite
+// numbers at the same step as the oracle, with the same losses before it.
+struct OracleStack {
+	orc::Net on;
+	int ox, ot, ol2;
+	std::vector<int> ow;
+};
+
+static void build_oracle_stack(OracleStack &o, int n, int blocks) {
+	o.ox = o.on.add(orc::kInput, n, 0, 0, NULL, 0);
+	int cur = o.ox;
+	for (int b = 0; b < blocks; ++b) {
+		int w = o.on.add(orc::kInput, n * n, 0, 0, NULL, 0);
+		o.ow.push_back(w);
+		int two[2] = {cur, w};
+		int lin = o.on.add(orc::kLinear, n, n * n, 0, two, 2);
+		int ge = o.on.add(orc::kGelu, n, 0, 0, &lin, 1);
+		int two2[2] = {cur, ge};
+		cur = o.on.add(orc::kResidual, n, 0, 0, two2, 2);
+	}
+	o.ot = o.on.add(orc::kInput, n, 0, 0, NULL, 0);
+	int two[2] = {cur, o.ot};
+	int odiff = o.on.add(orc::kResidual, n, 0, 0, two, 2);
+	o.ol2 = o.on.add(orc::kL2Out, n, 0, 0, &odiff, 1);
+}
+
+static void test_stack8(int n, int blocks, int B, int steps, float lr, int rows_checked, bool expect_overflow, bool must_learn) {
 	orc::Rng rng(4);
 	ResStack r;
 	build_stack(r, n, blocks);
-	if (both_halves) r.net.conjugateGradients(false);  // dz* products computed as upstream does, not written as conjugates
-	for (int b = 0; b < blocks; ++b) fill_normal(rng, r.net[r.w[b]]->mutable_input()->real_, (size_t) 2 * n * n, 1.0 / std::sqrt((double) n));
+	OracleStack o;
+	build_oracle_stack(o, n, blocks);
+	for (int b = 0; b < blocks; ++b) {
+		float *w = r.net[r.w[b]]->mutable_input()->real_;
+		fill_normal(rng, w, (size_t) 2 * n * n, 1.0 / std::sqrt((double) n));
+		std::copy(w, w + (size_t) 2 * n * n, o.on.at(o.ow[b])->in.re);
+	}
 	r.net.allocateOnGpu(B);
 	std::vector<float> xs((size_t) 2 * B * n), ts((size_t) 2 * B * n);
 	fill_normal(rng, xs.data(), xs.size(), 1.0);
 	fill_normal(rng, ts.data(), ts.size(), 1.0);
-	InputBatch bx(B, n), bt(B, n);
-	for (int b = 0; b < B; ++b) {
-		bx.add(xs.data() + (size_t) b * n, xs.data() + (size_t) (B + b) * n, n, 0);
-		bt.add(ts.data() + (size_t) b * n, ts.data() + (size_t) (B + b) * n, n, 0);
+	const bool all_rows = rows_checked <= 0 || rows_checked >= B;
+	std::vector<int> rows;
+	if (all_rows) {
+		for (int b = 0; b < B; ++b) rows.push_back(b);
+	} else {
+		for (int k = 0; k < rows_checked; ++k) rows.push_back((int) ((long) k * (B - 1) / std::max(1, rows_checked - 1)));
 	}
 	CInput *cx = (CInput *) r.net[r.x], *ct = (CInput *) r.net[r.t];
 	L2Out *l2 = (L2Out *) r.net[r.l2];
-	std::vector<float> losses;
-	// Both data inputs are sent again every step: the update also steps them (impl/cnet.h:413-421 upstream).  The batch of
-	// the main input travels on the upload stream under the previous step; the targets are queued on the compute stream.
-	// The host queues the whole step and reads the loss last.
-	auto one = [&]() {
-		r.net.gpuSetInput(ct, bt);
+	std::vector<float> means;
+	int dev_overflow = -1, cpu_overflow = -1;
+	for (int step = 0; step < steps; ++step) {
+		InputBatch bx(B, n), bt(B, n);
+		for (int b = 0; b < B; ++b) {
+			bx.add(xs.data() + (size_t) b * n, xs.data() + (size_t) (B + b) * n, n, 0);
+			bt.add(ts.data() + (size_t) b * n, ts.data() + (size_t) (B + b) * n, n, 0);
+		}
+		r.net.gpuSetInput(ct, bt);  // inputs are re-set every step: the update steps the data inputs too
 		r.net.gpuForward(cx, l2, bx);
+		const float mean = r.net.getLoss(l2, &bx);
+		means.push_back(mean);
 		r.net.gpuBackward();
-		r.net.gpuUpdateInputs(lr / B);  // upstream GPU loop: l_rate / batch.size() (cnet.cpp:147 upstream)
-		r.net.gpuPrefetch(cx, bx);
-		losses.push_back(r.net.getLoss(l2, NULL));
-	};
-	// timed region = the `steps` training steps from the initial weights (the first call also pays the one-off
-	// workspace growth; it is part of the job)
-	r.net.sync();
-	auto t0 = std::chrono::steady_clock::now();
-	r.net.gpuPrefetch(cx, bx);
-	auto t1 = t0;
-	for (int s = 0; s < steps; ++s) {
-		one();
-		if (s == 0) t1 = std::chrono::steady_clock::now();  // getLoss has waited for step 0
+		const std::string s = " step " + std::to_string(step);
+		// the oracle runs where it can say something: over the checked rows while it is in step with the device (with a
+		// subsample of rows its weights cannot follow the device past the first update)
+		if (all_rows || step == 0) {
+			double loss_sum = 0, loss_err = 0;
+			bool cpu_finite = true;
+			ErrAcc gx;
+			for (int b : rows) {
+				orc::Planes &px = o.on.at(o.ox)->in, &pt = o.on.at(o.ot)->in;
+				std::copy(xs.data() + (size_t) b * n, xs.data() + (size_t) (b + 1) * n, px.re);
+				std::copy(xs.data() + (size_t) (B + b) * n, xs.data() + (size_t) (B + b + 1) * n, px.im);
+				std::copy(ts.data() + (size_t) b * n, ts.data() + (size_t) (b + 1) * n, pt.re);
+				std::copy(ts.data() + (size_t) (B + b) * n, ts.data() + (size_t) (B + b + 1) * n, pt.im);
+				px.zero_gradients();
+				pt.zero_gradients();
+				o.on.forward();
+				const float l = o.on.loss(o.ol2, 0);
+				if (!std::isfinite(l)) cpu_finite = false;
+				loss_sum += l;
+				loss_err = std::max(loss_err, (double) std::fabs(l - bx.loss(b)) / l);
+				o.on.backward(-1);
+				r.net.fetch(cx, b);
+				gx.add(cx->input().dz_star_real_, px.dzs_re, 2 * n);
+			}
+			if (!cpu_finite && cpu_overflow < 0) cpu_overflow = step;
+			if (!std::isfinite(mean) && dev_overflow < 0) dev_overflow = step;
+			if (cpu_finite && std::isfinite(mean)) {
+				report("L2 loss per sample (" + std::to_string(rows.size()) + " rows)" + s, loss_err, TOL);
+				if (all_rows) report("mean loss" + s, std::fabs(mean - loss_sum / B) / (loss_sum / B), TOL);
+				report("data input dz* through all blocks" + s, gx.value());
+				if (all_rows) {
+					ErrAcc gw;
+					for (int b = 0; b < blocks; ++b) {
+						r.net.fetch(r.net[r.w[b]], 0);
+						gw.add(r.net[r.w[b]]->input().dz_star_real_, o.on.at(o.ow[b])->in.dzs_re, 2 * n * n);
+					}
+					report("weight dz* of all blocks (batch sum)" + s, gw.value());
+				}
+			}
+		} else if (!std::isfinite(mean) && dev_overflow < 0) {
+			dev_overflow = step;
+		}
+		r.net.gpuUpdateInputs(lr / B);
+		if (all_rows) {
+			o.on.update(lr, B);
+			if (cpu_overflow < 0 && dev_overflow < 0) {
+				ErrAcc ww;
+				bool finite = true;
+				for (int b = 0; b < blocks; ++b) {
+					r.net.fetch(r.net[r.w[b]], 0);
+					const float *got = r.net[r.w[b]]->input().real_, *want = o.on.at(o.ow[b])->in.re;
+					for (size_t k = 0; k < (size_t) 2 * n * n; ++k) finite = finite && std::isfinite(got[k]) && std::isfinite(want[k]);
+					ww.add(got, want, 2 * n * n);
+				}
+				if (finite) report("weights after update" + s, ww.value(), TOL);
+			}
+		}
+		printf("     step %d mean loss %.6g\n", step, mean);
+		if (cpu_overflow >= 0 || dev_overflow >= 0) break;
 	}
-	r.net.sync();
-	double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
-	double sec_later = std::chrono::duration<double>(std::chrono::steady_clock::now() - t1).count();
-	printf("losses:");
-	for (float l : losses) printf(" %.4f", l);
-	printf("\n");
-	// matrix products executed per Linear and step: forward, and per gradient pair one product (the other half written as
-	// its conjugate) or two (both computed), for the input and for the weight
-	const int products = both_halves ? 5 : 3;
-	double flops = 8.0 * products * B * (double) n * n * blocks;
-	printf("{\"workload\": \"residual stack: %d x (Linear %d->%d, CGelu, Residual), L2Out, SGD\", \"batch\": %d, \"steps\": %d, "
-		   "\"ms_per_step\": %.3f, \"ms_per_step_after_the_first\": %.3f, \"samples_per_sec\": %.1f, "
-		   "\"complex_products_per_linear\": %d, \"gemm_tflops_executed\": %.2f, \"first_loss\": %.4f, \"last_loss\": %.4f}\n",
-			blocks, n, n, B, steps, 1e3 * sec / steps, steps > 1 ? 1e3 * sec_later / (steps - 1) : 0.0, B * steps / sec, products,
-			flops * steps / sec / 1e12, losses.front(), losses.back());
-	if (!(losses.back() < losses.front())) {
-		printf("FAIL loss did not decrease\n");
-		g_fail++;
+	if (expect_overflow) {
+		expect("the CPU path leaves the finite numbers at this rate (step " + std::to_string(cpu_overflow) + ")", cpu_overflow >= 1);
+		expect("the device leaves them at the same step (" + std::to_string(dev_overflow) + ")", dev_overflow == cpu_overflow);
+	} else {
+		expect("every loss finite", dev_overflow < 0 && cpu_overflow < 0);
+	}
+	if (must_learn) {
+		bool falls = true;
+		for (size_t k = 1; k < means.size(); ++k) falls = falls && means[k] < means[k - 1];
+		expect("the mean loss falls at every one of the " + std::to_string(means.size()) + " steps", falls && means.size() == (size_t) steps);
 	}
 }
 
@@ -1326,16 +1401,15 @@ int main(int argc, char **argv) {
 		if (what == "adam" || what == "all") test_adam();
 		if (what == "loss_map" || what == "all") test_loss_map_and_sampling();
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
-		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12, false, true);
-		if (what == "pipeline_timing")
-			test_pipeline(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, true, argc > 4 && std::string(argv[4]) == "graphs",
-					argc > 4 && std::string(argv[4]) == "both_halves", argc > 4 && std::string(argv[4]) == "frozen_input");
+		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12);
 		if (what == "frozen_input" || what == "all") test_frozen_input();
 		if (what == "upstream_nets" || what == "all") test_upstream_nets();
 		if (what == "errors" || what == "all") test_errors();
-		if (what == "c4")
-			run_c4(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048, argc > 5 ? atoi(argv[5]) : 10,
-					argc > 6 ? (float) atof(argv[6]) : 0.01f, argc > 7 && std::string(argv[7]) == "both_halves");
+		// stack8 n blocks B steps lr rows_checked overflow|finite [learn]
+		if (what == "stack8")
+			test_stack8(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 16, argc > 5 ? atoi(argv[5]) : 4,
+					argc > 6 ? (float) atof(argv[6]) : 0.01f, argc > 7 ? atoi(argv[7]) : 0, argc > 8 && std::string(argv[8]) == "overflow",
+					argc > 9 && std::string(argv[9]) == "learn");
 	} catch (const std::exception &e) {
 		printf("FAIL uncaught exception: %s\n", e.what());
 		return 2;
