@@ -81,6 +81,7 @@ SIGNATURES = {
     "cnet_add2d": [c_fp, _l, c_fp, _l, _i, _i],
     "cnet_add_multi": [_i, C.c_void_p, C.c_void_p, C.c_void_p],
     "cnet_batch_sum": [c_fp, _l, c_fp, _i, _i, _i],
+    "cnet_batch_sum_noalloc": [c_fp, _l, c_fp, _i, _i, _i],
     "cnet_sgd_update": [c_fp, c_fp, c_fp, c_fp, _l, C.c_float, _i],
     "cnet_sgd_update_multi": [_i, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, _i],
     "cnet_adam_update": [c_fp] * 6 + [_l, C.c_float, C.c_float, _i, _i],

@@ -587,7 +587,46 @@ __global__ __launch_bounds__(TPB) void colsum_final_kernel(const float *__restri
 
 inline bool mult4(long a, long b = 0, long c = 0, long d = 0) { return !(a % 4) && !(b % 4) && !(c % 4) && !(d % 4); }
 
+// Slabs of rows for the two-stage column sum: enough workgroups to cover the chip about four times, at most 256 slabs.
+struct ColsumPlan {
+	int V, nslabs, rows_per_slab;
+	long col_blocks;
+};
+inline ColsumPlan plan_colsum(int rows, int cols, bool vec) {
+	ColsumPlan p;
+	p.V = vec ? 4 : 1;
+	p.col_blocks = ((long) cols / p.V + CS_X - 1) / CS_X;
+	int nslabs = (int) std::max(1L, std::min(256L, 4L * cnet::rt().prop.multiProcessorCount / p.col_blocks));
+	nslabs = std::min(nslabs, (rows + CS_Y - 1) / CS_Y);
+	p.rows_per_slab = (rows + nslabs - 1) / nslabs;
+	p.nslabs = (rows + p.rows_per_slab - 1) / p.rows_per_slab;
+	return p;
+}
+
+// Partial sums of cnet_batch_sum_noalloc: part of the library's image on every device it is loaded on, so the call
+// needs no allocation.  In host code the array's name is only a handle for hipGetSymbolAddress: kernels get the device
+// address that was looked up once per device (g_static_partial).
+constexpr long kStaticPartialFloats = 512 * 1024;  // 2 MiB
+__device__ __align__(256) float static_partial[kStaticPartialFloats];
+constexpr int kMaxDevices = 64;
+float *g_static_partial[kMaxDevices] = {};
+
 }  // namespace
+
+namespace cnet {
+
+// Called by cnet_init with `device` current: looks up this device's copy of the static partial-sum array.
+int init_static_scratch(int device) {
+	if (device < 0 || device >= kMaxDevices) return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_init: device %d beyond the %d the library keeps state for", device, kMaxDevices);
+	if (g_static_partial[device]) return CNET_OK;
+	float *ptr = nullptr;
+	CNET_HIP(hipGetSymbolAddress((void **) &ptr, HIP_SYMBOL(static_partial)));
+	if (!ptr) return fail(CNET_ERR_HIP, "cnet_init: hipGetSymbolAddress returned no address for the static scratch array");
+	g_static_partial[device] = ptr;
+	return CNET_OK;
+}
+
+}  // namespace cnet
 
 using namespace cnet;
 
@@ -692,30 +731,46 @@ int cnet_l2norm_bwd(const float *z_re, const float *z_im, int64_t ldz, const flo
 	return CNET_OK;
 }
 
+static int batch_sum_launch(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate, bool vec,
+		const ColsumPlan &p, float *partial) {
+	dim3 grid((unsigned) p.col_blocks, (unsigned) p.nslabs);
+	if (vec)
+		hipLaunchKernelGGL(colsum_partial_kernel<4>, grid, dim3(TPB), 0, rt().stream, src, (long) lds, partial, rows, cols, p.rows_per_slab);
+	else
+		hipLaunchKernelGGL(colsum_partial_kernel<1>, grid, dim3(TPB), 0, rt().stream, src, (long) lds, partial, rows, cols, p.rows_per_slab);
+	CNET_LAUNCH_CHECK();
+	hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned) ((cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, p.nslabs, cols, dst,
+			accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
 int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate) {
 	CNET_REQUIRE_INIT();
 	CNET_CHECK_ARG(rows > 0 && cols >= 0);
 	if (!cols) return CNET_OK;
 	CNET_CHECK_ARG(src && dst && lds >= cols);
 	const bool vec = mult4(cols, lds) && aligned16(src);
-	const int V = vec ? 4 : 1;
-	const long col_blocks = ((long) cols / V + CS_X - 1) / CS_X;
-	int nslabs = (int) std::max(1L, std::min(256L, 4L * rt().prop.multiProcessorCount / col_blocks));
-	nslabs = std::min(nslabs, (rows + CS_Y - 1) / CS_Y);
-	const int rows_per_slab = (rows + nslabs - 1) / nslabs;
-	nslabs = (rows + rows_per_slab - 1) / rows_per_slab;
-	float *partial = (float *) workspace((size_t) nslabs * cols * sizeof(float));
+	const ColsumPlan p = plan_colsum(rows, cols, vec);
+	float *partial = (float *) workspace((size_t) p.nslabs * cols * sizeof(float));
 	if (!partial) return CNET_ERR_OUT_OF_MEMORY;
-	dim3 grid((unsigned) col_blocks, (unsigned) nslabs);
-	if (vec)
-		hipLaunchKernelGGL(colsum_partial_kernel<4>, grid, dim3(TPB), 0, rt().stream, src, (long) lds, partial, rows, cols, rows_per_slab);
-	else
-		hipLaunchKernelGGL(colsum_partial_kernel<1>, grid, dim3(TPB), 0, rt().stream, src, (long) lds, partial, rows, cols, rows_per_slab);
-	CNET_LAUNCH_CHECK();
-	hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned) ((cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, nslabs, cols, dst,
-			accumulate);
-	CNET_LAUNCH_CHECK();
-	return CNET_OK;
+	return batch_sum_launch(src, lds, dst, rows, cols, accumulate, vec, p, partial);
+}
+
+int cnet_batch_sum_noalloc(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows > 0 && cols >= 0);
+	if (!cols) return CNET_OK;
+	CNET_CHECK_ARG(src && dst && lds >= cols);
+	const bool vec = mult4(cols, lds) && aligned16(src);
+	const ColsumPlan p = plan_colsum(rows, cols, vec);  // the same slabs as cnet_batch_sum: the same sums in the same order
+	if ((long) p.nslabs * cols > kStaticPartialFloats)
+		return fail(CNET_ERR_UNSUPPORTED, "cnet_batch_sum_noalloc: %d slabs x %d columns of partial sums exceed the static scratch of %ld floats; use cnet_batch_sum",
+				p.nslabs, cols, kStaticPartialFloats);
+	float *partial = g_static_partial[rt().device];
+	if (!partial) return fail(CNET_ERR_NOT_INITIALIZED, "cnet_batch_sum_noalloc: the static scratch of device %d was not looked up", rt().device);
+	// every partial sum the second kernel reads is written by the first one of this call: nothing to clear
+	return batch_sum_launch(src, lds, dst, rows, cols, accumulate, vec, p, partial);
 }
 
 }  // extern "C"

@@ -59,6 +59,7 @@ void *workspace(size_t bytes) {
 }
 
 void release_twiddles();  // cdft.hip
+int init_static_scratch(int device);  // reduce.hip
 
 // destroys whatever streams and events exist (also the leftovers of an initialisation that failed half-way)
 static void destroy_streams(Runtime &r) {
@@ -118,6 +119,11 @@ int cnet_init(int device) {
 	if (rc != CNET_OK) {
 		destroy_streams(r);
 		return rc;
+	}
+	const int rc_scratch = init_static_scratch(device);
+	if (rc_scratch != CNET_OK) {
+		destroy_streams(r);
+		return rc_scratch;
 	}
 	r.device = device;
 	r.ready = true;

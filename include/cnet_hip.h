@@ -272,6 +272,14 @@ int cnet_l2out_bwd(const float *z_re, const float *z_im, int64_t ldz,
 int cnet_copy2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols);       /* one plane */
 int cnet_add2d(const float *src, int64_t lds, float *dst, int64_t ldd, int rows, int cols);        /* dst += src */
 int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate); /* dst[c] (+)= sum_r src[r][c] */
+/* cnet_batch_sum for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc); it has no counterpart upstream.  Same arguments, same kernels and bit-identical
+ * results; the partial sums of its first stage go to a 2 MiB array that is part of the library's image on each device
+ * instead of the library workspace, so the call never allocates or frees.  Limit: slabs x cols <= 524288 floats, which
+ * holds for every cols <= 524288 (slabs = min(256, 4 x compute units / ceil(cols / 256)), at most rows / 4); beyond it
+ * the call returns CNET_ERR_UNSUPPORTED.  All calls on one device share the array: calls that overlap in time (two
+ * streams, two host threads) race. */
+int cnet_batch_sum_noalloc(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate);
 /* dst[k][0..n[k]) += src[k][0..n[k]) for `count` dense arrays in one launch: what the loop over the input functions in
  * GpuNet::GpuBackward becomes (each CInput gathers the dz* of its consumer, impl/cinput.h:54-65, gpu/kernels.cpp:118-143).
  * The destinations of one call must not overlap (the additions of a call run concurrently). */
