@@ -173,19 +173,26 @@ def kernel_suite(steps):
     hbm("plain copy of one plane (practical HBM ceiling)", [R, Cc], 8, n, lambda: ops.copy2d(u.re, yy.re))
     hbm("cgelu_fwd", [R, Cc], 16, n, lambda: ops.gelu_fwd(u, yy))
     hbm("cgelu_bwd", [R, Cc], 40, n, lambda: ops.gelu_bwd(u, g, du))
+    # the same pass for a conjugate gradient pair (real loss): g.dz read, dx.dz written, the dz* halves neither read nor written
+    hbm("cgelu_bwd, conjugate pair (dz only)", [R, Cc], 24, n, lambda: ops.gelu_bwd_sym(u, g, du, mirror=False))
     hbm("crelu_fwd", [R, Cc], 16, n, lambda: ops.crelu_fwd(u, yy))
     hbm("crelu_bwd", [R, Cc], 40, n, lambda: ops.crelu_bwd(u, g, du))
     hbm("residual_fwd", [R, Cc], 24, n, lambda: ops.residual_fwd(u, v, yy))
     hbm("residual_bwd", [R, Cc], 48, n, lambda: ops.residual_bwd(g, du, dv))
+    hbm("residual_bwd, conjugate pair (dz only)", [R, Cc], 24, n, lambda: ops.residual_bwd_sym(g, du, dv, mirror=False))
     hbm("hadamard_fwd (shared weights)", [R, Cc], 16, n, lambda: ops.hadamard_fwd(u, w1, yy, True))
     hbm("hadamard_bwd (shared weights, batch-summed dW)", [R, Cc], 40, n, lambda: ops.hadamard_bwd(u, w1, g, du, dw1, True),
         extra_bytes=16 * Cc)
+    hbm("hadamard_bwd, conjugate pair (shared weights, dz only)", [R, Cc], 24, n,
+        lambda: ops.hadamard_bwd_sym(u, w1, g, du, dw1, True, mirror=False), extra_bytes=8 * Cc)
     loss = capi.empty(R)
     hbm("l2out_fwd", [R, Cc], 8, n, lambda: ops.l2out_fwd(u, loss))
     hbm("l2out_bwd", [R, Cc], 24, n, lambda: ops.l2out_bwd(u, du))
+    hbm("l2out_bwd, conjugate pair (dz only)", [R, Cc], 16, n, lambda: ops.l2out_bwd_sym(u, du, mirror=False))
     s_ = capi.empty(R)
     hbm("l2norm_fwd (SoftMax)", [R, Cc], 16, n, lambda: ops.l2norm_fwd(u, yy, s_))
     hbm("l2norm_bwd (SoftMax)", [R, Cc], 40, n, lambda: ops.l2norm_bwd(u, s_, g, du))
+    hbm("l2norm_bwd (SoftMax), conjugate pair (dz only)", [R, Cc], 24, n, lambda: ops.l2norm_bwd_sym(u, s_, g, du, mirror=False))
     hbm("sgd_update", [n], 32, n, lambda: ops.sgd_update(u, du.planes[2], du.planes[3], 1e-9))
     hbm("adam_update", [n], 48, n, lambda: ops.adam_update(u, du.planes[0], du.planes[1], du.planes[2], du.planes[3], 1e-9, 0.9, 3))
     hbm("zero 4 gradient planes", [R, Cc], 16, n, lambda: [p.owner.zero() for p in du.planes])
@@ -203,6 +210,7 @@ def kernel_suite(steps):
     hbm("cross_entropy_fwd (loss, argmax; no normalised output)", [R, Cc], 8, n,
         lambda: ops.cross_entropy_fwd(z, labels, s_, l_, am, None), extra_bytes=4 * R)
     hbm("cross_entropy_bwd", [R, Cc], 24, n, lambda: ops.cross_entropy_bwd(z, s_, labels, dz))
+    hbm("cross_entropy_bwd, conjugate pair (dz only)", [R, Cc], 16, n, lambda: ops.cross_entropy_bwd_sym(z, s_, labels, dz, mirror=False))
     return lines
 
 

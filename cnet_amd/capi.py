@@ -77,6 +77,13 @@ SIGNATURES = {
     "cnet_cross_entropy_bwd": [c_fp, c_fp, _l, c_fp, c_fp] + [c_fp] * 4 + [_l, _i, _i],
     "cnet_l2out_fwd": [c_fp, c_fp, _l, c_fp, _i, _i],
     "cnet_l2out_bwd": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_hadamard_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_cgelu_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_crelu_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_residual_bwd_sym": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_l2norm_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_l2out_bwd_sym": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_cross_entropy_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp] + [c_fp] * 4 + [_l, _i, _i],
     "cnet_copy2d": [c_fp, _l, c_fp, _l, _i, _i],
     "cnet_add2d": [c_fp, _l, c_fp, _l, _i, _i],
     "cnet_add_multi": [_i, C.c_void_p, C.c_void_p, C.c_void_p],

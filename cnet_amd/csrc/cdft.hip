@@ -209,7 +209,7 @@ int cnet_cdft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, f
 	CNET_REQUIRE_INIT();
 	CNET_CHECK_ARG(B >= 0 && n > 0 && n <= 46340);
 	if (B == 0) return CNET_OK;
-	CNET_CHECK_ARG(g_dz_re && g_dz_im && dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && dx_dz_re && dx_dz_im && ((dx_dzs_re == nullptr) == (dx_dzs_im == nullptr)));
 	CNET_CHECK_ARG(ldg >= n && lddx >= n);
 	Twiddle t;
 	int rc = get_plan(n, &t, true);
@@ -218,7 +218,7 @@ int cnet_cdft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, f
 	const float *ar[2] = {g_dz_re, g_dz_re}, *ai[2] = {g_dz_im, g_dz_im}, *br[2] = {t.re, t.re}, *bi[2] = {t.im, t.im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 0, true);
+	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 0, dx_dzs_re != nullptr);
 }
 
 int cnet_ctriang_dft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, float *dx_dz_re, float *dx_dz_im,
@@ -226,7 +226,7 @@ int cnet_ctriang_dft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t
 	CNET_REQUIRE_INIT();
 	CNET_CHECK_ARG(B >= 0 && n > 0 && n <= 46340);
 	if (B == 0) return CNET_OK;
-	CNET_CHECK_ARG(g_dz_re && g_dz_im && dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && dx_dz_re && dx_dz_im && ((dx_dzs_re == nullptr) == (dx_dzs_im == nullptr)));
 	CNET_CHECK_ARG(ldg >= n && lddx >= n);
 	Twiddle t;
 	int rc = get_triangular(n, &t);
@@ -234,7 +234,7 @@ int cnet_ctriang_dft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t
 	const float *ar[2] = {g_dz_re, g_dz_re}, *ai[2] = {g_dz_im, g_dz_im}, *br[2] = {t.tri_re, t.tri_re}, *bi[2] = {t.tri_im, t.tri_im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(false, false, 1, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 2, true);
+	return cgemm_pair(false, false, 1, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 2, dx_dzs_re != nullptr);
 }
 
 int cnet_ctriang_dft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,

@@ -1581,14 +1581,14 @@ int cnet_clinear_bwd_input_sym(const float *g_dz_re, const float *g_dz_im, int64
 	CNET_REQUIRE_INIT();
 	CNET_CHECK_ARG(B >= 0 && K >= 0 && N > 0);
 	if (B == 0 || K == 0) return CNET_OK;
-	CNET_CHECK_ARG(g_dz_re && g_dz_im && w_re && w_im && dx_dz_re && dx_dz_im && dx_dzs_re && dx_dzs_im);
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && w_re && w_im && dx_dz_re && dx_dz_im && ((dx_dzs_re == nullptr) == (dx_dzs_im == nullptr)));
 	CNET_CHECK_ARG(ldg >= N && ldw >= K && lddx >= K);
 	// dx = g * w as in cnet_clinear_bwd_input; dx* = conj(g) * conj(w) is its conjugate and is written, not computed
 	const float *ar[2] = {g_dz_re, g_dz_re}, *ai[2] = {g_dz_im, g_dz_im};
 	const float *br[2] = {w_re, w_re}, *bi[2] = {w_im, w_im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(false, true, 1, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0, true);
+	return cgemm_pair(false, true, 1, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0, dx_dzs_re != nullptr);
 }
 
 int cnet_clinear_bwd_weight_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *x_re, const float *x_im,
@@ -1597,13 +1597,13 @@ int cnet_clinear_bwd_weight_sym(const float *g_dz_re, const float *g_dz_im, int6
 	CNET_REQUIRE_INIT();
 	CNET_CHECK_ARG(B > 0 && K >= 0 && N >= 0);
 	if (N == 0 || K == 0) return CNET_OK;
-	CNET_CHECK_ARG(g_dz_re && g_dz_im && x_re && x_im && dw_dz_re && dw_dz_im && dw_dzs_re && dw_dzs_im);
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && x_re && x_im && dw_dz_re && dw_dz_im && ((dw_dzs_re == nullptr) == (dw_dzs_im == nullptr)));
 	CNET_CHECK_ARG(ldg >= N && ldx >= K && lddw >= K);
 	const float *ar[2] = {g_dz_re, g_dz_re}, *ai[2] = {g_dz_im, g_dz_im};
 	const float *br[2] = {x_re, x_re}, *bi[2] = {x_im, x_im};
 	float *cr[2] = {dw_dz_re, dw_dzs_re}, *ci[2] = {dw_dz_im, dw_dzs_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(true, true, 1, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0, true);
+	return cgemm_pair(true, true, 1, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0, dw_dzs_re != nullptr);
 }
 
 }  // extern "C"

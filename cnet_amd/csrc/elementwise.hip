@@ -422,6 +422,227 @@ __global__ __launch_bounds__(TPB) void crossent_bwd_kernel(const float *__restri
 	stv<V, NT>(dz.dz_im + off, n_i);
 }
 
+// ------------------------------------------------------------------------------------------------ conjugate gradient pairs
+// Under a real-valued loss the gradient pair of every value is conjugate: dL/dz* = conj(dL/dz).  The kernels below are
+// the backward passes above for such a pair: they read the dz planes of the incoming gradient only, form the dz planes of
+// the result with the arithmetic of the general kernel (operation for operation, so the bits agree with it on an exactly
+// conjugate pair), and write the dz* planes as the conjugate only where the caller passes them (non-NULL): a consumer
+// that is itself one of these kernels, or a conjugate-pair matrix product, never reads them.  24 bytes per complex
+// element instead of 40 (CGelu, CRelu, Hadamard, SoftMax), 24 instead of 48 (Residual), 16 instead of 24 (the losses).
+struct Pair2 {  // dz planes, and optionally the planes that receive the conjugate
+	float *dz_re, *dz_im, *dzs_re, *dzs_im;
+};
+
+// (o_r, o_i) to the dz planes and, conjugated, to the dz* planes when they are wanted
+template <int V, bool NT>
+__device__ __forceinline__ void out_pair(const Pair2 &d, long off, const float (&o_r)[V], const float (&o_i)[V], int accumulate) {
+	outv<V, NT>(d.dz_re + off, o_r, accumulate);
+	outv<V, NT>(d.dz_im + off, o_i, accumulate);
+	if (d.dzs_re) {
+		float n_i[V];
+#pragma unroll
+		for (int k = 0; k < V; ++k) n_i[k] = -o_i[k];
+		outv<V, NT>(d.dzs_re + off, o_r, accumulate);
+		outv<V, NT>(d.dzs_im + off, n_i, accumulate);
+	}
+}
+
+template <int V, bool NT>
+__global__ __launch_bounds__(TPB) void gelu_bwd_sym_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
+		const float *__restrict__ g_re, const float *__restrict__ g_im, long ldg, Pair2 dx, long lddx, int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], gr[V], gi[V], o_r[V], o_i[V];
+	ldv<V, NT>(a, xr + row * ldx + col);
+	ldv<V, NT>(b, xi + row * ldx + col);
+	ldv<V, NT>(gr, g_re + row * ldg + col);
+	ldv<V, NT>(gi, g_im + row * ldg + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		const float px = 0.5f * gelu_slope(a[k]), py = 0.5f * gelu_slope(b[k]);
+		const float s = px + py, d = px - py;
+		o_r[k] = gr[k] * s + gr[k] * d;      // G s + conj(G) d
+		o_i[k] = gi[k] * s + (-gi[k]) * d;
+	}
+	out_pair<V, NT>(dx, row * lddx + col, o_r, o_i, accumulate);
+}
+
+template <int V, bool NT>
+__global__ __launch_bounds__(TPB) void crelu_bwd_sym_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
+		const float *__restrict__ g_re, const float *__restrict__ g_im, long ldg, Pair2 dx, long lddx, int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], o_r[V], o_i[V];
+	ldv<V, NT>(a, xr + row * ldx + col);
+	ldv<V, NT>(b, xi + row * ldx + col);
+	ldv<V, NT>(o_r, g_re + row * ldg + col);
+	ldv<V, NT>(o_i, g_im + row * ldg + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		const bool on = a[k] > 0.f && b[k] > 0.f;
+		o_r[k] = on ? o_r[k] : 0.f;
+		o_i[k] = on ? o_i[k] : 0.f;
+	}
+	out_pair<V, NT>(dx, row * lddx + col, o_r, o_i, accumulate);
+}
+
+template <int V, bool NT>
+__global__ __launch_bounds__(TPB) void residual_bwd_sym_kernel(const float *__restrict__ g_re, const float *__restrict__ g_im, long ldg,
+		Pair2 du, long lddu, Pair2 dv, long lddv, int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float o_r[V], o_i[V];
+	ldv<V, NT>(o_r, g_re + row * ldg + col);
+	ldv<V, NT>(o_i, g_im + row * ldg + col);
+	out_pair<V, NT>(du, row * lddu + col, o_r, o_i, accumulate);
+	out_pair<V, NT>(dv, row * lddv + col, o_r, o_i, accumulate);
+}
+
+// du = G v, dv = G u (per-row operands)
+template <int V, bool NT>
+__global__ __launch_bounds__(TPB) void hadamard_bwd_sym_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
+		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, const float *__restrict__ g_re,
+		const float *__restrict__ g_im, long ldg, Pair2 du, long lddu, Pair2 dv, long lddv, int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], c[V], d[V], gr[V], gi[V], o_r[V], o_i[V];
+	ldv<V, NT>(a, ur + row * ldu + col);
+	ldv<V, NT>(b, ui + row * ldu + col);
+	ldv<V, NT>(c, vr + row * ldv_ + col);
+	ldv<V, NT>(d, vi + row * ldv_ + col);
+	ldv<V, NT>(gr, g_re + row * ldg + col);
+	ldv<V, NT>(gi, g_im + row * ldg + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		o_r[k] = gr[k] * c[k] - gi[k] * d[k];
+		o_i[k] = gr[k] * d[k] + gi[k] * c[k];
+	}
+	out_pair<V, NT>(du, row * lddu + col, o_r, o_i, accumulate);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		o_r[k] = gr[k] * a[k] - gi[k] * b[k];
+		o_i[k] = gr[k] * b[k] + gi[k] * a[k];
+	}
+	out_pair<V, NT>(dv, row * lddv + col, o_r, o_i, accumulate);
+}
+
+// v is one shared parameter row: as hadamard_bwd_shared_kernel, two partial planes per slab
+template <int V, bool NT>
+__global__ __launch_bounds__(TPB) void hadamard_bwd_shared_sym_kernel(const float *__restrict__ ur, const float *__restrict__ ui,
+		long ldu, const float *__restrict__ vr, const float *__restrict__ vi, const float *__restrict__ g_re,
+		const float *__restrict__ g_im, long ldg, Pair2 du, long lddu, float *__restrict__ partial, int rows, int cols,
+		int rows_per_slab, int accumulate) {
+	__shared__ float red[CS_Y][2][CS_X * V];
+	const int tx = threadIdx.x % CS_X, ty = threadIdx.x / CS_X;
+	const long col = ((long) blockIdx.x * CS_X + tx) * V;
+	const bool live = col < cols;
+	const int slab = blockIdx.y;
+	const int r0 = slab * rows_per_slab;
+	const int r1 = min(rows, r0 + rows_per_slab);
+	float acc[2][V];
+#pragma unroll
+	for (int p = 0; p < 2; ++p)
+#pragma unroll
+		for (int k = 0; k < V; ++k) acc[p][k] = 0.f;
+	if (live) {
+		float c[V], d[V];
+		ldv<V, false>(c, vr + col);
+		ldv<V, false>(d, vi + col);
+		for (int row = r0 + ty; row < r1; row += CS_Y) {
+			float a[V], b[V], gr[V], gi[V], o_r[V], o_i[V];
+			ldv<V, NT>(a, ur + (long) row * ldu + col);
+			ldv<V, NT>(b, ui + (long) row * ldu + col);
+			ldv<V, NT>(gr, g_re + (long) row * ldg + col);
+			ldv<V, NT>(gi, g_im + (long) row * ldg + col);
+#pragma unroll
+			for (int k = 0; k < V; ++k) {
+				o_r[k] = gr[k] * c[k] - gi[k] * d[k];
+				o_i[k] = gr[k] * d[k] + gi[k] * c[k];
+			}
+			out_pair<V, NT>(du, (long) row * lddu + col, o_r, o_i, accumulate);
+#pragma unroll
+			for (int k = 0; k < V; ++k) {
+				acc[0][k] += gr[k] * a[k] - gi[k] * b[k];
+				acc[1][k] += gr[k] * b[k] + gi[k] * a[k];
+			}
+		}
+	}
+#pragma unroll
+	for (int p = 0; p < 2; ++p)
+#pragma unroll
+		for (int k = 0; k < V; ++k) red[ty][p][tx * V + k] = acc[p][k];
+	__syncthreads();
+	if (ty == 0 && live) {
+#pragma unroll
+		for (int p = 0; p < 2; ++p) {
+			float t[V];
+#pragma unroll
+			for (int k = 0; k < V; ++k) t[k] = ((red[0][p][tx * V + k] + red[1][p][tx * V + k]) + red[2][p][tx * V + k]) + red[3][p][tx * V + k];
+			stv<V, NT>(partial + ((long) slab * 2 + p) * cols + col, t);
+		}
+	}
+}
+
+// dst.dz (+)= sum over slabs of partial[slab][re, im][c], slabs added in index order; the conjugate goes to dst.dzs when
+// those planes are given
+__global__ __launch_bounds__(TPB) void slab_sum_sym_kernel(const float *__restrict__ partial, int nslabs, int cols, Pair2 dst, int accumulate) {
+	__shared__ float red[4][64];
+	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+	const long idx = (long) blockIdx.x * 64 + tx;
+	const bool live = idx < 2L * cols;
+	const int p = live ? (int) (idx / cols) : 0;
+	const int c = live ? (int) (idx - (long) p * cols) : 0;
+	const int per = (nslabs + 3) / 4, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
+	red[ty][tx] = live ? cnet::ordered_sum(partial + ((long) k0 * 2 + p) * cols + c, 2L * cols, k1 - k0) : 0.f;
+	__syncthreads();
+	if (ty == 0 && live) {
+		const float s = ((red[0][tx] + red[1][tx]) + red[2][tx]) + red[3][tx];
+		float *out = p == 0 ? dst.dz_re : dst.dz_im;
+		out[c] = accumulate ? out[c] + s : s;
+		if (dst.dzs_re) {
+			float *m = p == 0 ? dst.dzs_re : dst.dzs_im;
+			const float mv = p == 0 ? s : -s;
+			m[c] = accumulate ? m[c] + mv : mv;
+		}
+	}
+}
+
+// L2Out: dz = conj z (and dz* = z)
+template <int V, bool NT>
+__global__ __launch_bounds__(TPB) void l2out_bwd_sym_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		Pair2 dz, long lddz, int rows, int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], nb[V];
+	ldv<V, NT>(a, zr + row * ldz + col);
+	ldv<V, NT>(b, zi + row * ldz + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) nb[k] = -b[k];
+	out_pair<V, NT>(dz, row * lddz + col, a, nb, accumulate);
+}
+
+// CrossEntropy: dz* as in crossent_bwd_kernel, dz = conj(dz*); assigns
+template <int V, bool NT>
+__global__ __launch_bounds__(TPB) void crossent_bwd_sym_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		const float *__restrict__ s, const int *__restrict__ labels, Pair2 dz, long lddz, int rows, int cols) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], o_r[V], n_i[V];
+	ldv<V, NT>(a, zr + row * ldz + col);
+	ldv<V, NT>(b, zi + row * ldz + col);
+	const float S = s[row];
+	const int label = labels[row];
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		float o_i;
+		if (col + k == label) {
+			float m = (float) ((double) a[k] * (double) a[k] + (double) b[k] * (double) b[k]);
+			m = (m < 1e-15f ? 1e-15f : m);
+			o_r[k] = -a[k] * (S - m) / (m * S);
+			o_i = -b[k] * (S - m) / (m * S);
+		} else {
+			o_r[k] = a[k] / S;
+			o_i = b[k] / S;
+		}
+		n_i[k] = -o_i;
+	}
+	out_pair<V, NT>(dz, row * lddz + col, o_r, n_i, 0);
+}
+
 // ------------------------------------------------------------------------------------------------ plumbing
 template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void copy2d_kernel(const float *__restrict__ src, long lds, float *__restrict__ dst, long ldd,
@@ -933,6 +1154,149 @@ int cnet_adam_update(float *z_re, float *z_im, float *m_re, float *m_im, float *
 	else
 		hipLaunchKernelGGL((adam_kernel<1, false>), dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
 				(long) n, lr, beta, denom, zero_grad);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+// ---- backward passes for a conjugate gradient pair (g.dzs == conj(g.dz)); the dz* planes of the results are optional
+static inline Pair2 pair_of(float *dz_re, float *dz_im, float *dzs_re, float *dzs_im) { return Pair2{dz_re, dz_im, dzs_re, dzs_im}; }
+#define CNET_CHECK_PAIR(p) CNET_CHECK_ARG((p).dz_re && (p).dz_im && (((p).dzs_re == nullptr) == ((p).dzs_im == nullptr)))
+static inline int pair_planes(const Pair2 &p) { return p.dzs_re ? 4 : 2; }
+
+int cnet_cgelu_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const float *g_dz_re, const float *g_dz_im, int64_t ldg,
+		float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	const Pair2 dx = pair_of(dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im);
+	CNET_CHECK_ARG(x_re && x_im && g_dz_re && g_dz_im);
+	CNET_CHECK_PAIR(dx);
+	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
+	const bool nt = streaming(4 + pair_planes(dx), (long) rows * cols);
+	if (all_mult4({cols, ldx, ldg, lddx}) && all_aligned({x_re, x_im, g_dz_re, g_dz_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
+		CNET_LAUNCH_V4(gelu_bwd_sym_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
+	else
+		hipLaunchKernelGGL((gelu_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_crelu_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const float *g_dz_re, const float *g_dz_im, int64_t ldg,
+		float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	const Pair2 dx = pair_of(dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im);
+	CNET_CHECK_ARG(x_re && x_im && g_dz_re && g_dz_im);
+	CNET_CHECK_PAIR(dx);
+	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
+	const bool nt = streaming(4 + pair_planes(dx), (long) rows * cols);
+	if (all_mult4({cols, ldx, ldg, lddx}) && all_aligned({x_re, x_im, g_dz_re, g_dz_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
+		CNET_LAUNCH_V4(crelu_bwd_sym_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
+	else
+		hipLaunchKernelGGL((crelu_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_residual_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, float *du_dz_re, float *du_dz_im, float *du_dzs_re,
+		float *du_dzs_im, int64_t lddu, float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv, int rows,
+		int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	const Pair2 du = pair_of(du_dz_re, du_dz_im, du_dzs_re, du_dzs_im), dv = pair_of(dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im);
+	CNET_CHECK_ARG(g_dz_re && g_dz_im);
+	CNET_CHECK_PAIR(du);
+	CNET_CHECK_PAIR(dv);
+	CNET_CHECK_ARG(ldg >= cols && lddu >= cols && lddv >= cols);
+	const bool nt = streaming(2 + pair_planes(du) + pair_planes(dv), (long) rows * cols);
+	if (all_mult4({cols, ldg, lddu, lddv}) &&
+			all_aligned({g_dz_re, g_dz_im, du_dz_re, du_dz_im, du_dzs_re, du_dzs_im, dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im}))
+		CNET_LAUNCH_V4(residual_bwd_sym_kernel, nt, CNET_GRID_2D(4), g_dz_re, g_dz_im, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
+	else
+		hipLaunchKernelGGL((residual_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), g_dz_re, g_dz_im, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_hadamard_bwd_sym(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+		const float *g_dz_re, const float *g_dz_im, int64_t ldg, float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im,
+		int64_t lddu, float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv, int rows, int cols,
+		int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	const Pair2 du = pair_of(du_dz_re, du_dz_im, du_dzs_re, du_dzs_im), dv = pair_of(dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im);
+	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && g_dz_re && g_dz_im);
+	CNET_CHECK_PAIR(du);
+	CNET_CHECK_PAIR(dv);
+	CNET_CHECK_ARG(ldu >= cols && ldg >= cols && lddu >= cols && (ldv == 0 || (ldv >= cols && lddv >= cols)));
+	const bool vec = all_mult4({cols, ldu, ldv, ldg, lddu, ldv ? lddv : 0}) &&
+			all_aligned({u_re, u_im, v_re, v_im, g_dz_re, g_dz_im, du_dz_re, du_dz_im, du_dzs_re, du_dzs_im, dv_dz_re, dv_dz_im, dv_dzs_re,
+					dv_dzs_im});
+	const bool nt = streaming(4 + pair_planes(du) + (ldv ? 2 + pair_planes(dv) : 0), (long) rows * cols);
+	if (ldv != 0) {
+		if (vec)
+			CNET_LAUNCH_V4(hadamard_bwd_sym_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg, du, lddu, dv,
+					lddv, rows, cols, accumulate);
+		else
+			hipLaunchKernelGGL((hadamard_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg, du,
+					lddu, dv, lddv, rows, cols, accumulate);
+		CNET_LAUNCH_CHECK();
+		return CNET_OK;
+	}
+	const int V = vec ? 4 : 1;
+	const long col_blocks = ((long) cols / V + CS_X - 1) / CS_X;
+	int nslabs = (int) std::max(1L, std::min(256L, 4L * rt().prop.multiProcessorCount / col_blocks));
+	nslabs = std::min(nslabs, (rows + CS_Y - 1) / CS_Y);
+	const int rows_per_slab = (rows + nslabs - 1) / nslabs;
+	nslabs = (rows + rows_per_slab - 1) / rows_per_slab;
+	float *partial = (float *) workspace((size_t) nslabs * 2 * cols * sizeof(float));
+	if (!partial) return CNET_ERR_OUT_OF_MEMORY;
+	dim3 grid((unsigned) col_blocks, (unsigned) nslabs);
+	if (vec)
+		CNET_LAUNCH_V4(hadamard_bwd_shared_sym_kernel, nt, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g_dz_re, g_dz_im, ldg,
+				du, lddu, partial, rows, cols, rows_per_slab, accumulate);
+	else
+		hipLaunchKernelGGL((hadamard_bwd_shared_sym_kernel<1, false>), grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g_dz_re,
+				g_dz_im, ldg, du, lddu, partial, rows, cols, rows_per_slab, accumulate);
+	CNET_LAUNCH_CHECK();
+	hipLaunchKernelGGL(slab_sum_sym_kernel, dim3((unsigned) ((2L * cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, nslabs, cols, dv, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_l2out_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re,
+		float *dz_dzs_im, int64_t lddz, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	const Pair2 dz = pair_of(dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im);
+	CNET_CHECK_ARG(z_re && z_im && ldz >= cols && lddz >= cols);
+	CNET_CHECK_PAIR(dz);
+	const bool nt = streaming(2 + pair_planes(dz), (long) rows * cols);
+	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
+		CNET_LAUNCH_V4(l2out_bwd_sym_kernel, nt, CNET_GRID_2D(4), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
+	else
+		hipLaunchKernelGGL((l2out_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_cross_entropy_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, const float *s, const int32_t *labels, float *dz_dz_re,
+		float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	const Pair2 dz = pair_of(dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im);
+	CNET_CHECK_ARG(z_re && z_im && s && labels && ldz >= cols && lddz >= cols);
+	CNET_CHECK_PAIR(dz);
+	const bool nt = streaming(2 + pair_planes(dz), (long) rows * cols);
+	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
+		CNET_LAUNCH_V4(crossent_bwd_sym_kernel, nt, CNET_GRID_2D(4), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
+	else
+		hipLaunchKernelGGL((crossent_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }

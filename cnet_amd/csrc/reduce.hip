@@ -308,7 +308,9 @@ __global__ __launch_bounds__(TPB) void l2norm_fwd_kernel(const float *__restrict
 //   A = sum_j G_j z_j + sum_j Gs_j conj(z_j)
 //   dz_i  = G_i /sqrt(S) - conj(z_i) A / (2 S^1.5)
 //   dzs_i = Gs_i/sqrt(S) - z_i       A / (2 S^1.5)
-template <int V, int G>
+// SYM: the incoming pair is conjugate (gs = conj(g)): the gs planes are not read, and the dz* planes of the result are
+// written only when given (ds_re != nullptr).  Same arithmetic otherwise, so the bits agree with the general kernel.
+template <int V, int G, bool SYM>
 __global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		const float *__restrict__ s, const float *__restrict__ g_re, const float *__restrict__ g_im,
 		const float *__restrict__ gs_re, const float *__restrict__ gs_im, long ldg, float *__restrict__ d_re,
@@ -318,8 +320,10 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict
 	CNET_ROW_SETUP();
 	const float *pzr = zr + (long) row * ldz, *pzi = zi + (long) row * ldz;
 	const float *pgr = g_re + (long) row * ldg, *pgi = g_im + (long) row * ldg;
-	const float *psr = gs_re + (long) row * ldg, *psi = gs_im + (long) row * ldg;
-	float *q0 = d_re + (long) row * ldd, *q1 = d_im + (long) row * ldd, *q2 = ds_re + (long) row * ldd, *q3 = ds_im + (long) row * ldd;
+	const float *psr = SYM ? pgr : gs_re + (long) row * ldg, *psi = SYM ? pgi : gs_im + (long) row * ldg;
+	const bool stars = !SYM || ds_re != nullptr;
+	float *q0 = d_re + (long) row * ldd, *q1 = d_im + (long) row * ldd;
+	float *q2 = stars ? ds_re + (long) row * ldd : nullptr, *q3 = stars ? ds_im + (long) row * ldd : nullptr;
 	constexpr int W = V;  // columns per thread and step
 	Cplx4 acc = {0.f, 0.f, 0.f, 0.f};  // a,b: G z   c,d: Gs conj z
 	for (int c = t * W; c < cols; c += STRIDE * W) {
@@ -329,10 +333,22 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict
 			*reinterpret_cast<float4 *>(b) = *reinterpret_cast<const float4 *>(pzi + c);
 			*reinterpret_cast<float4 *>(gr) = *reinterpret_cast<const float4 *>(pgr + c);
 			*reinterpret_cast<float4 *>(gi) = *reinterpret_cast<const float4 *>(pgi + c);
-			*reinterpret_cast<float4 *>(sr) = *reinterpret_cast<const float4 *>(psr + c);
-			*reinterpret_cast<float4 *>(si) = *reinterpret_cast<const float4 *>(psi + c);
+			if (!SYM) {
+				*reinterpret_cast<float4 *>(sr) = *reinterpret_cast<const float4 *>(psr + c);
+				*reinterpret_cast<float4 *>(si) = *reinterpret_cast<const float4 *>(psi + c);
+			}
 		} else {
-			a[0] = pzr[c]; b[0] = pzi[c]; gr[0] = pgr[c]; gi[0] = pgi[c]; sr[0] = psr[c]; si[0] = psi[c];
+			a[0] = pzr[c]; b[0] = pzi[c]; gr[0] = pgr[c]; gi[0] = pgi[c];
+			if (!SYM) {
+				sr[0] = psr[c]; si[0] = psi[c];
+			}
+		}
+		if (SYM) {
+#pragma unroll
+			for (int k = 0; k < W; ++k) {
+				sr[k] = gr[k];
+				si[k] = -gi[k];
+			}
 		}
 #pragma unroll
 		for (int k = 0; k < W; ++k) {
@@ -357,10 +373,22 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict
 			*reinterpret_cast<float4 *>(b) = *reinterpret_cast<const float4 *>(pzi + c);
 			*reinterpret_cast<float4 *>(gr) = *reinterpret_cast<const float4 *>(pgr + c);
 			*reinterpret_cast<float4 *>(gi) = *reinterpret_cast<const float4 *>(pgi + c);
-			*reinterpret_cast<float4 *>(sr) = *reinterpret_cast<const float4 *>(psr + c);
-			*reinterpret_cast<float4 *>(si) = *reinterpret_cast<const float4 *>(psi + c);
+			if (!SYM) {
+				*reinterpret_cast<float4 *>(sr) = *reinterpret_cast<const float4 *>(psr + c);
+				*reinterpret_cast<float4 *>(si) = *reinterpret_cast<const float4 *>(psi + c);
+			}
 		} else {
-			a[0] = pzr[c]; b[0] = pzi[c]; gr[0] = pgr[c]; gi[0] = pgi[c]; sr[0] = psr[c]; si[0] = psi[c];
+			a[0] = pzr[c]; b[0] = pzi[c]; gr[0] = pgr[c]; gi[0] = pgi[c];
+			if (!SYM) {
+				sr[0] = psr[c]; si[0] = psi[c];
+			}
+		}
+		if (SYM) {
+#pragma unroll
+			for (int k = 0; k < W; ++k) {
+				sr[k] = gr[k];
+				si[k] = -gi[k];
+			}
 		}
 #pragma unroll
 		for (int k = 0; k < W; ++k) {
@@ -372,17 +400,24 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict
 			if (accumulate) {
 				o0[k] += q0[c + k];
 				o1[k] += q1[c + k];
-				o2[k] += q2[c + k];
-				o3[k] += q3[c + k];
+				if (stars) {
+					o2[k] += q2[c + k];
+					o3[k] += q3[c + k];
+				}
 			}
 		}
 		if (W == 4) {
 			*reinterpret_cast<float4 *>(q0 + c) = *reinterpret_cast<float4 *>(o0);
 			*reinterpret_cast<float4 *>(q1 + c) = *reinterpret_cast<float4 *>(o1);
-			*reinterpret_cast<float4 *>(q2 + c) = *reinterpret_cast<float4 *>(o2);
-			*reinterpret_cast<float4 *>(q3 + c) = *reinterpret_cast<float4 *>(o3);
+			if (stars) {
+				*reinterpret_cast<float4 *>(q2 + c) = *reinterpret_cast<float4 *>(o2);
+				*reinterpret_cast<float4 *>(q3 + c) = *reinterpret_cast<float4 *>(o3);
+			}
 		} else {
-			q0[c] = o0[0]; q1[c] = o1[0]; q2[c] = o2[0]; q3[c] = o3[0];
+			q0[c] = o0[0]; q1[c] = o1[0];
+			if (stars) {
+				q2[c] = o2[0]; q3[c] = o3[0];
+			}
 		}
 	}
 }
@@ -437,7 +472,7 @@ __global__ __launch_bounds__(TPB) void l2norm_fwd_reg_kernel(const float *__rest
 	if (t == 0 && s) s[row] = (float) sum;
 }
 
-template <int G, int NIT>
+template <int G, int NIT, bool SYM>
 __global__ __launch_bounds__(TPB) void l2norm_bwd_reg_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		const float *__restrict__ s, const float *__restrict__ g_re, const float *__restrict__ g_im,
 		const float *__restrict__ gs_re, const float *__restrict__ gs_im, long ldg, float *__restrict__ d_re,
@@ -446,20 +481,30 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_reg_kernel(const float *__rest
 	__shared__ Cplx4 lds_c[TPB / 64];
 	CNET_ROW_SETUP();
 	const float *src[6] = {zr + (long) row * ldz, zi + (long) row * ldz, g_re + (long) row * ldg, g_im + (long) row * ldg,
-			gs_re + (long) row * ldg, gs_im + (long) row * ldg};
-	float *dst[4] = {d_re + (long) row * ldd, d_im + (long) row * ldd, ds_re + (long) row * ldd, ds_im + (long) row * ldd};
+			SYM ? nullptr : gs_re + (long) row * ldg, SYM ? nullptr : gs_im + (long) row * ldg};
+	const bool stars = !SYM || ds_re != nullptr;
+	float *dst[4] = {d_re + (long) row * ldd, d_im + (long) row * ldd, stars ? ds_re + (long) row * ldd : nullptr,
+			stars ? ds_im + (long) row * ldd : nullptr};
+	constexpr int NSRC = SYM ? 4 : 6;
 	float v[NIT][6][4];  // [chunk][z_re, z_im, g_re, g_im, gs_re, gs_im][column]
 #pragma unroll
 	for (int k = 0; k < NIT; ++k) {
 		const int c = (t + k * STRIDE) * 4;
 #pragma unroll
-		for (int p = 0; p < 6; ++p) {
+		for (int p = 0; p < NSRC; ++p) {
 			float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
 			if (c < cols) x = *reinterpret_cast<const float4 *>(src[p] + c);
 			v[k][p][0] = x.x;
 			v[k][p][1] = x.y;
 			v[k][p][2] = x.z;
 			v[k][p][3] = x.w;
+		}
+		if (SYM) {
+#pragma unroll
+			for (int q = 0; q < 4; ++q) {
+				v[k][4][q] = v[k][2][q];
+				v[k][5][q] = -v[k][3][q];
+			}
 		}
 	}
 	Cplx4 acc = {0.f, 0.f, 0.f, 0.f};  // a,b: G z   c,d: Gs conj z
@@ -499,6 +544,7 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_reg_kernel(const float *__rest
 			}
 #pragma unroll
 			for (int p = 0; p < 4; ++p) {
+				if (p >= 2 && !stars) continue;
 				float4 w = make_float4(o[p][0], o[p][1], o[p][2], o[p][3]);
 				if (accumulate) {
 					const float4 old = *reinterpret_cast<const float4 *>(dst[p] + c);
@@ -660,6 +706,38 @@ using namespace cnet;
 // chunks of 4 columns each thread must hold so that its group (64 lanes, x4 wavefronts for wide rows) covers a row
 static inline int chunks_per_thread(int cols) { return (cols + (cols > 2048 ? 1024 : 256) - 1) / (cols > 2048 ? 1024 : 256); }
 
+template <bool SYM>
+static int l2norm_bwd_dispatch(const float *z_re, const float *z_im, int64_t ldz, const float *s, const float *g_dz_re,
+		const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg, float *dz_dz_re, float *dz_dz_im,
+		float *dz_dzs_re, float *dz_dzs_im, int64_t lddz, int rows, int cols, int accumulate) {
+	const bool vec = mult4(cols, ldz, ldg, lddz) && aligned16(z_re) && aligned16(z_im) && aligned16(g_dz_re) && aligned16(g_dz_im) &&
+			aligned16(g_dzs_re) && aligned16(g_dzs_im) && aligned16(dz_dz_re) && aligned16(dz_dz_im) && aligned16(dz_dzs_re) &&
+			aligned16(dz_dzs_im);
+	const int nit = chunks_per_thread(cols);
+	const bool wide = cols > 2048;
+	const int rpb = wide ? 1 : TPB / 64;
+	dim3 grid((unsigned) ((rows + rpb - 1) / rpb));
+#define CNET_L2N_ARGS z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate
+	if (vec && nit <= 4) {
+		if (nit <= 2) {
+			if (wide) hipLaunchKernelGGL((l2norm_bwd_reg_kernel<4, 2, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+			else hipLaunchKernelGGL((l2norm_bwd_reg_kernel<1, 2, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+		} else {
+			if (wide) hipLaunchKernelGGL((l2norm_bwd_reg_kernel<4, 4, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+			else hipLaunchKernelGGL((l2norm_bwd_reg_kernel<1, 4, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+		}
+	} else if (vec) {
+		if (wide) hipLaunchKernelGGL((l2norm_bwd_kernel<4, 4, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+		else hipLaunchKernelGGL((l2norm_bwd_kernel<4, 1, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+	} else {
+		if (wide) hipLaunchKernelGGL((l2norm_bwd_kernel<1, 4, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+		else hipLaunchKernelGGL((l2norm_bwd_kernel<1, 1, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+	}
+#undef CNET_L2N_ARGS
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
 extern "C" {
 
 int cnet_l2out_fwd(const float *z_re, const float *z_im, int64_t ldz, float *loss, int rows, int cols) {
@@ -713,22 +791,21 @@ int cnet_l2norm_bwd(const float *z_re, const float *z_im, int64_t ldz, const flo
 	if (!rows) return CNET_OK;
 	CNET_CHECK_ARG(z_re && z_im && s && g_dz_re && g_dz_im && g_dzs_re && g_dzs_im);
 	CNET_CHECK_ARG(dz_dz_re && dz_dz_im && dz_dzs_re && dz_dzs_im && ldz >= cols && ldg >= cols && lddz >= cols);
-	const bool vec = mult4(cols, ldz, ldg, lddz) && aligned16(z_re) && aligned16(z_im) && aligned16(g_dz_re) && aligned16(g_dz_im) &&
-			aligned16(g_dzs_re) && aligned16(g_dzs_im) && aligned16(dz_dz_re) && aligned16(dz_dz_im) && aligned16(dz_dzs_re) &&
-			aligned16(dz_dzs_im);
-	const int nit = chunks_per_thread(cols);
-	if (vec && nit <= 4) {
-		if (nit <= 2)
-			CNET_ROW_LAUNCH_REG(l2norm_bwd_reg_kernel, 2, z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg,
-					dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate);
-		else
-			CNET_ROW_LAUNCH_REG(l2norm_bwd_reg_kernel, 4, z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg,
-					dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate);
-		return CNET_OK;
-	}
-	CNET_ROW_LAUNCH(l2norm_bwd_kernel, vec, z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg, dz_dz_re,
-			dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate);
-	return CNET_OK;
+	return l2norm_bwd_dispatch<false>(z_re, z_im, ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, ldg, dz_dz_re, dz_dz_im, dz_dzs_re,
+			dz_dzs_im, lddz, rows, cols, accumulate);
+}
+
+int cnet_l2norm_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, const float *s, const float *g_dz_re, const float *g_dz_im,
+		int64_t ldg, float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz, int rows, int cols,
+		int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols > 0);
+	if (!rows) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && s && g_dz_re && g_dz_im && dz_dz_re && dz_dz_im);
+	CNET_CHECK_ARG((dz_dzs_re == nullptr) == (dz_dzs_im == nullptr));
+	CNET_CHECK_ARG(ldz >= cols && ldg >= cols && lddz >= cols);
+	return l2norm_bwd_dispatch<true>(z_re, z_im, ldz, s, g_dz_re, g_dz_im, nullptr, nullptr, ldg, dz_dz_re, dz_dz_im, dz_dzs_re,
+			dz_dzs_im, lddz, rows, cols, accumulate);
 }
 
 static int batch_sum_launch(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate, bool vec,

@@ -365,6 +365,11 @@ protected:
 		float *grad = NULL;  // 4 planes [rows][len]
 		float *z = NULL;     // input functions only: their own 2 value planes [rows][len] (the parameter, the data batch, the table)
 		float *g(int plane) const { return grad + (size_t) plane * rows * len; }
+		// Under conjugate gradient pairs (CNet::conjugateGradients) the dz* planes of a slot are written on the device only
+		// where something reads them there: input functions and the embedding table gather dz*.  Elsewhere they are the
+		// conjugate of the dz planes by construction and fetch() forms them on the host.
+		bool star_on_device = true;
+		float *gs(int plane) const { return star_on_device ? g(plane) : NULL; }
 	};
 	std::vector<Slot> slots_;
 	bool trainable_ = true;   // input functions: stepped by the update (CNet::setInputTrainable)
@@ -938,6 +943,16 @@ private:
 			if (t != isInput && t != isEmbedding && f->slots_.empty())
 				throw std::invalid_argument(f->getName() + ": has no inputs");
 		}
+		// who reads the dz* planes of a slot on the device: the backward pass of its producer, when that is an input function
+		// or the embedding table (they gather dz*), or a Residual that sums one of its operands over the batch
+		for (auto f : func_list_)
+			for (auto &sl : f->slots_) {
+				CFunc *p = sl.producer;
+				bool reads = !p || p->typeId() == isInput || p->typeId() == isEmbedding;
+				if (p && p->typeId() == isResidual)
+					for (auto q : p->prev_func_) reads = reads || q->rows_ != p->rows_;
+				sl.star_on_device = reads;
+			}
 		d_labels_ = dalloc<int32_t>(batch_);
 		ck(cnet_memset_zero(d_labels_, batch_ * sizeof(int32_t)), "zero");
 		if (main_input_->typeId() == isInput) {
@@ -1032,13 +1047,20 @@ private:
 			if (!with_labels) return;  // upstream: CrossEntropy::backward() without a label does nothing
 			CrossEntropy *c = (CrossEntropy *) f;
 			CFunc::Slot &s = f->slots_[0];
-			ck(cnet_cross_entropy_bwd(zre(f, 0), zim(f, 0), s.len, c->d_s_, d_labels_, s.g(0), s.g(1), s.g(2), s.g(3), s.len, rows, s.len),
-					"cnet_cross_entropy_bwd");
+			if (conjugate_gradients_)
+				ck(cnet_cross_entropy_bwd_sym(zre(f, 0), zim(f, 0), s.len, c->d_s_, d_labels_, s.g(0), s.g(1), s.gs(2), s.gs(3), s.len, rows,
+						s.len), "cnet_cross_entropy_bwd_sym");
+			else
+				ck(cnet_cross_entropy_bwd(zre(f, 0), zim(f, 0), s.len, c->d_s_, d_labels_, s.g(0), s.g(1), s.g(2), s.g(3), s.len, rows, s.len),
+						"cnet_cross_entropy_bwd");
 			return;
 		}
 		if (t == isL2Out) {
 			CFunc::Slot &s = f->slots_[0];
-			ck(cnet_l2out_bwd(zre(f, 0), zim(f, 0), s.len, s.g(0), s.g(1), s.g(2), s.g(3), s.len, rows, s.len, 0), "cnet_l2out_bwd");
+			if (conjugate_gradients_)
+				ck(cnet_l2out_bwd_sym(zre(f, 0), zim(f, 0), s.len, s.g(0), s.g(1), s.gs(2), s.gs(3), s.len, rows, s.len, 0), "cnet_l2out_bwd_sym");
+			else
+				ck(cnet_l2out_bwd(zre(f, 0), zim(f, 0), s.len, s.g(0), s.g(1), s.g(2), s.g(3), s.len, rows, s.len, 0), "cnet_l2out_bwd");
 			return;
 		}
 		if ((t == isInput || t == isEmbedding) && !f->trainable_) return;  // nothing steps it: nothing to gather
@@ -1084,10 +1106,10 @@ private:
 				const bool to_data = a.producer->wants_grad_, to_weight = w.producer->wants_grad_;
 				if (conjugate_gradients_) {  // dz* = conj(dz): one product each, written to both pairs of planes
 					if (to_data)
-						ck(cnet_clinear_bwd_input_sym(u.g(0), u.g(1), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K, rows, K,
+						ck(cnet_clinear_bwd_input_sym(u.g(0), u.g(1), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.gs(2), a.gs(3), K, rows, K,
 								N, acc), "cnet_clinear_bwd_input_sym");
 					if (to_weight)
-						ck(cnet_clinear_bwd_weight_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K, rows, K,
+						ck(cnet_clinear_bwd_weight_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.gs(2), w.gs(3), K, rows, K,
 								N, acc), "cnet_clinear_bwd_weight_sym");
 					break;
 				}
@@ -1101,37 +1123,57 @@ private:
 			}
 			case isFourier:
 				if (conjugate_gradients_)
-					ck(cnet_cdft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc), "cnet_cdft_bwd_sym");
+					ck(cnet_cdft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len, acc), "cnet_cdft_bwd_sym");
 				else
 					ck(cnet_cdft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
 							"cnet_cdft_bwd");
 				break;
 			case isTrianFourier:
 				if (conjugate_gradients_)
-					ck(cnet_ctriang_dft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
+					ck(cnet_ctriang_dft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len, acc),
 							"cnet_ctriang_dft_bwd_sym");
 				else
 					ck(cnet_ctriang_dft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
 							"cnet_ctriang_dft_bwd");
 				break;
 			case isCrelu:
+				if (conjugate_gradients_) {
+					ck(cnet_crelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,
+							acc), "cnet_crelu_bwd_sym");
+					break;
+				}
 				ck(cnet_crelu_bwd(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len,
 						rows, a.len, acc), "cnet_crelu_bwd");
 				break;
 			case isHadamard: {
 				CFunc::Slot &v = f->slots_[1];
 				const int n = f->out_size_;
+				if (conjugate_gradients_) {
+					ck(cnet_hadamard_bwd_sym(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, u.g(0), u.g(1), u.len, a.g(0),
+							a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows, n, acc), "cnet_hadamard_bwd_sym");
+					break;
+				}
 				ck(cnet_hadamard_bwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, u.g(0), u.g(1), u.g(2), u.g(3),
 						u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3), n, rows, n, acc), "cnet_hadamard_bwd");
 				break;
 			}
 			case isGelu:
+				if (conjugate_gradients_) {
+					ck(cnet_cgelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,
+							acc), "cnet_cgelu_bwd_sym");
+					break;
+				}
 				ck(cnet_cgelu_bwd(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len,
 						rows, a.len, acc), "cnet_cgelu_bwd");
 				break;
 			case isResidual: {
 				CFunc::Slot &v = f->slots_[1];
 				const int n = f->out_size_;
+				if (a.rows == rows && v.rows == rows && conjugate_gradients_) {
+					ck(cnet_residual_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows,
+							n, acc), "cnet_residual_bwd_sym");
+					break;
+				}
 				if (a.rows == rows && v.rows == rows) {
 					ck(cnet_residual_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3),
 							n, rows, n, acc), "cnet_residual_bwd");
@@ -1150,6 +1192,11 @@ private:
 				break;
 			}
 			case isSoftMax:
+				if (conjugate_gradients_) {
+					ck(cnet_l2norm_bwd_sym(zre(f, 0), zim(f, 0), a.len, ((SoftMax *) f)->d_s_, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2),
+							a.gs(3), a.len, rows, a.len, acc), "cnet_l2norm_bwd_sym");
+					break;
+				}
 				ck(cnet_l2norm_bwd(zre(f, 0), zim(f, 0), a.len, ((SoftMax *) f)->d_s_, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1),
 						a.g(2), a.g(3), a.len, rows, a.len, acc), "cnet_l2norm_bwd");
 				break;
@@ -1226,6 +1273,15 @@ public:
 			ck(cnet_memcpy_d2h(v->imag_ + s.offset, z_im, s.len * sizeof(float)), "cnet_memcpy_d2h");
 			for (int p = 0; p < 4; ++p)
 				ck(cnet_memcpy_d2h(v->plane(2 + p) + s.offset, s.g(p) + (size_t) row * s.len, s.len * sizeof(float)), "cnet_memcpy_d2h");
+			if (conjugate_gradients_ && !s.star_on_device) {
+				// the pair is conjugate and nothing on the device reads its dz* half: it is formed here
+				const float *dz_re = v->plane(2) + s.offset, *dz_im = v->plane(3) + s.offset;
+				float *dzs_re = v->plane(4) + s.offset, *dzs_im = v->plane(5) + s.offset;
+				for (int k = 0; k < s.len; ++k) {
+					dzs_re[k] = dz_re[k];
+					dzs_im[k] = -dz_im[k];
+				}
+			}
 		}
 		if (f->typeId() == isCrossEntropy) {
 			CrossEntropy *c = (CrossEntropy *) f;

@@ -116,13 +116,21 @@ def linear_bwd_weight(g, x, dw, accumulate=0):
     call("cnet_clinear_bwd_weight", *g.p(), g.ld, *x.p(), x.ld, *dw.p(), dw.ld, g.rows, x.cols, g.cols, accumulate)
 
 
-def linear_bwd_input_sym(g, w, dx, accumulate=0):
-    """g is a Grad whose dz* planes are the conjugate of its dz planes; only the dz planes are read."""
-    call("cnet_clinear_bwd_input_sym", *g.p()[:2], g.ld, *w.p(), w.ld, *dx.p(), dx.ld, g.rows, w.cols, w.rows, accumulate)
+def _mirrored(d, mirror):
+    p = d.p()
+    return (p[0], p[1], p[2] if mirror else None, p[3] if mirror else None)
 
 
-def linear_bwd_weight_sym(g, x, dw, accumulate=0):
-    call("cnet_clinear_bwd_weight_sym", *g.p()[:2], g.ld, *x.p(), x.ld, *dw.p(), dw.ld, g.rows, x.cols, g.cols, accumulate)
+def linear_bwd_input_sym(g, w, dx, accumulate=0, mirror=True):
+    """g is a Grad whose dz* planes are the conjugate of its dz planes; only the dz planes are read.  mirror=False: the
+    dz* planes of the result are not written."""
+    call("cnet_clinear_bwd_input_sym", *g.p()[:2], g.ld, *w.p(), w.ld, *_mirrored(dx, mirror), dx.ld, g.rows, w.cols, w.rows,
+         accumulate)
+
+
+def linear_bwd_weight_sym(g, x, dw, accumulate=0, mirror=True):
+    call("cnet_clinear_bwd_weight_sym", *g.p()[:2], g.ld, *x.p(), x.ld, *_mirrored(dw, mirror), dw.ld, g.rows, x.cols, g.cols,
+         accumulate)
 
 
 def dft_fwd(x, y, accumulate=0):
@@ -133,12 +141,12 @@ def dft_bwd(g, dx, accumulate=0):
     call("cnet_cdft_bwd", *g.p(), g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
 
 
-def dft_bwd_sym(g, dx, accumulate=0):
-    call("cnet_cdft_bwd_sym", *g.p()[:2], g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
+def dft_bwd_sym(g, dx, accumulate=0, mirror=True):
+    call("cnet_cdft_bwd_sym", *g.p()[:2], g.ld, *_mirrored(dx, mirror), dx.ld, g.rows, g.cols, accumulate)
 
 
-def triang_dft_bwd_sym(g, dx, accumulate=0):
-    call("cnet_ctriang_dft_bwd_sym", *g.p()[:2], g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
+def triang_dft_bwd_sym(g, dx, accumulate=0, mirror=True):
+    call("cnet_ctriang_dft_bwd_sym", *g.p()[:2], g.ld, *_mirrored(dx, mirror), dx.ld, g.rows, g.cols, accumulate)
 
 
 def triang_dft_fwd(x, y, accumulate=0):
@@ -207,6 +215,43 @@ def l2out_fwd(z, loss):
 
 def l2out_bwd(z, dz, accumulate=0):
     call("cnet_l2out_bwd", *z.p(), z.ld, *dz.p(), dz.ld, z.rows, z.cols, accumulate)
+
+
+# Backward passes for a conjugate gradient pair: `g` is a Grad whose dz* planes are the conjugate of its dz planes (only the
+# dz planes are read); mirror=False leaves the dz* planes of the results untouched (NULL pointers at the C ABI).
+def _pair(d, mirror):
+    p = d.p()
+    return (p[0], p[1], p[2] if mirror else None, p[3] if mirror else None)
+
+
+def hadamard_bwd_sym(u, v, g, du, dv, shared=False, accumulate=0, mirror=True):
+    call("cnet_hadamard_bwd_sym", *u.p(), u.ld, *v.p(), 0 if shared else v.ld, *g.p()[:2], g.ld, *_pair(du, mirror), du.ld,
+         *_pair(dv, mirror), dv.ld, u.rows, u.cols, accumulate)
+
+
+def gelu_bwd_sym(x, g, dx, accumulate=0, mirror=True):
+    call("cnet_cgelu_bwd_sym", *x.p(), x.ld, *g.p()[:2], g.ld, *_pair(dx, mirror), dx.ld, x.rows, x.cols, accumulate)
+
+
+def crelu_bwd_sym(x, g, dx, accumulate=0, mirror=True):
+    call("cnet_crelu_bwd_sym", *x.p(), x.ld, *g.p()[:2], g.ld, *_pair(dx, mirror), dx.ld, x.rows, x.cols, accumulate)
+
+
+def residual_bwd_sym(g, du, dv, accumulate=0, mirror=True):
+    call("cnet_residual_bwd_sym", *g.p()[:2], g.ld, *_pair(du, mirror), du.ld, *_pair(dv, mirror), dv.ld, g.rows, g.cols,
+         accumulate)
+
+
+def l2norm_bwd_sym(z, s, g, dz, accumulate=0, mirror=True):
+    call("cnet_l2norm_bwd_sym", *z.p(), z.ld, s.ptr, *g.p()[:2], g.ld, *_pair(dz, mirror), dz.ld, z.rows, z.cols, accumulate)
+
+
+def l2out_bwd_sym(z, dz, accumulate=0, mirror=True):
+    call("cnet_l2out_bwd_sym", *z.p(), z.ld, *_pair(dz, mirror), dz.ld, z.rows, z.cols, accumulate)
+
+
+def cross_entropy_bwd_sym(z, s, labels, dz, mirror=True):
+    call("cnet_cross_entropy_bwd_sym", *z.p(), z.ld, s.ptr, labels.ptr, *_pair(dz, mirror), dz.ld, z.rows, z.cols)
 
 
 def copy2d(src, dst):

@@ -61,17 +61,28 @@ class TokenModel:
 
     def backward(self):
         B, S, D = self.B, self.S, self.D
-        bwd_input = ops.linear_bwd_input_sym if self.conjugate_pairs else ops.linear_bwd_input
-        bwd_weight = ops.linear_bwd_weight_sym if self.conjugate_pairs else ops.linear_bwd_weight
-        ops.cross_entropy_bwd(self.logits, self.s, self.labels, self.d_logits)
-        bwd_input(self.d_logits, self.w3, self.d_o)
-        bwd_weight(self.d_logits, self.o, self.d_w3)
-        bwd_input(self.d_o, self.w2, self.d_a)
-        bwd_weight(self.d_o, self.a, self.d_w2)
-        ops.gelu_bwd(self.u, self.d_a, self.d_u)
-        bwd_input(self.d_u, self.w1, self.d_h)
-        bwd_weight(self.d_u, self.h, self.d_w1)
-        ops.hadamard_bwd(self.m, self.gate, self.d_h, self.d_m, self.d_gate, shared=True)
+        if self.conjugate_pairs:
+            # one gradient per value: every pass reads the dz planes only; the dz* planes are written where something reads
+            # them (parameter gradients, and d_m, whose dz* half feeds the sequence transform)
+            ops.cross_entropy_bwd_sym(self.logits, self.s, self.labels, self.d_logits, mirror=False)
+            ops.linear_bwd_input_sym(self.d_logits, self.w3, self.d_o, mirror=False)
+            ops.linear_bwd_weight_sym(self.d_logits, self.o, self.d_w3)
+            ops.linear_bwd_input_sym(self.d_o, self.w2, self.d_a, mirror=False)
+            ops.linear_bwd_weight_sym(self.d_o, self.a, self.d_w2)
+            ops.gelu_bwd_sym(self.u, self.d_a, self.d_u, mirror=False)
+            ops.linear_bwd_input_sym(self.d_u, self.w1, self.d_h, mirror=False)
+            ops.linear_bwd_weight_sym(self.d_u, self.h, self.d_w1)
+            ops.hadamard_bwd_sym(self.m, self.gate, self.d_h, self.d_m, self.d_gate, shared=True)
+        else:
+            ops.cross_entropy_bwd(self.logits, self.s, self.labels, self.d_logits)
+            ops.linear_bwd_input(self.d_logits, self.w3, self.d_o)
+            ops.linear_bwd_weight(self.d_logits, self.o, self.d_w3)
+            ops.linear_bwd_input(self.d_o, self.w2, self.d_a)
+            ops.linear_bwd_weight(self.d_o, self.a, self.d_w2)
+            ops.gelu_bwd(self.u, self.d_a, self.d_u)
+            ops.linear_bwd_input(self.d_u, self.w1, self.d_h)
+            ops.linear_bwd_weight(self.d_u, self.h, self.d_w1)
+            ops.hadamard_bwd(self.m, self.gate, self.d_h, self.d_m, self.d_gate, shared=True)
         # dz_b = F dM_b.dz ; dz*_b = conj(F) dM_b.dz*   (F symmetric)
         gdz = ops.CMat(self.d_m.planes[0], self.d_m.planes[1])
         gds = ops.CMat(self.d_m.planes[2], self.d_m.planes[3])

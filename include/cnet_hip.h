@@ -154,7 +154,9 @@ int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const fl
  * g.dzs * conj(w) == conj(g.dz * w), in floating point as well (same sums, signs applied exactly), so one product is
  * computed and written twice, once conjugated.  Same results as cnet_clinear_bwd_input / _bwd_weight on such a pair (to
  * rounding: half as many blocks may take another block shape) at half the matrix work.  Replace the same upstream
- * functions (gpu/reduce.cpp:532-604, gpu/reducegrad.cpp:288-322); the caller vouches for the pair. */
+ * functions (gpu/reduce.cpp:532-604, gpu/reducegrad.cpp:288-322); the caller vouches for the pair.  The dzs planes of the
+ * result may both be NULL (here and in cnet_cdft_bwd_sym / cnet_ctriang_dft_bwd_sym): then only the dz planes are written,
+ * which is all a consumer needs that is itself a conjugate-pair entry point. */
 int cnet_clinear_bwd_input_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *w_re, const float *w_im,
                                int64_t ldw, float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im,
                                int64_t lddx, int B, int K, int N, int accumulate);
@@ -296,6 +298,39 @@ int cnet_sgd_update_multi(int count, float *const *z_re, float *const *z_im, flo
  * m_re / m_im are the first-moment planes (upstream keeps them in the node's dz planes, impl/cfunc.h:341-349). */
 int cnet_adam_update(float *z_re, float *z_im, float *m_re, float *m_im, float *dzs_re, float *dzs_im, int64_t n,
                      float lr, float beta, int t, int zero_grad);
+
+/* ---- The elementwise and loss backward passes for a conjugate gradient pair (see cnet_clinear_bwd_input_sym): g.dzs ==
+ *      conj(g.dz) is not read, the dz planes of the result are formed with the arithmetic of the general entry point
+ *      (same bits on an exactly conjugate pair), and its dzs planes receive the conjugate when they are given; both may be
+ *      NULL, which leaves them untouched: 24 bytes per complex element instead of 40 (CGelu, CRelu, Hadamard, SoftMax),
+ *      24 instead of 48 (Residual), 16 instead of 24 (the losses).  They replace the same upstream kernels as the general
+ *      entry points: gpu/kernels.cpp:204-360, 145-202; gpu/reducegrad.cpp:268-286; gpu/reduce.cpp:408-446, 609-655. */
+int cnet_hadamard_bwd_sym(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+                          const float *g_dz_re, const float *g_dz_im, int64_t ldg,
+                          float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
+                          float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
+                          int rows, int cols, int accumulate);
+int cnet_cgelu_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const float *g_dz_re, const float *g_dz_im, int64_t ldg,
+                       float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
+                       int rows, int cols, int accumulate);
+int cnet_crelu_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const float *g_dz_re, const float *g_dz_im, int64_t ldg,
+                       float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
+                       int rows, int cols, int accumulate);
+int cnet_residual_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg,
+                          float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
+                          float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
+                          int rows, int cols, int accumulate);
+int cnet_l2norm_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, const float *s,
+                        const float *g_dz_re, const float *g_dz_im, int64_t ldg,
+                        float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,
+                        int rows, int cols, int accumulate);
+/* the two losses produce the pair themselves: dz = conj(dzs) */
+int cnet_l2out_bwd_sym(const float *z_re, const float *z_im, int64_t ldz,
+                       float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,
+                       int rows, int cols, int accumulate);
+int cnet_cross_entropy_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, const float *s, const int32_t *labels,
+                               float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,
+                               int rows, int cols);
 
 /* ---- CEmbedding: replaces gpu_embedding_forward / _backward (gpu/kernels.cpp:362-442), CPU twin impl/embed.h:109-148.
  * tokens[rows][slots] int32, -1 = padding (zero row); an id >= vocab is treated as padding too (upstream asserts on

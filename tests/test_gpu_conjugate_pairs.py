@@ -83,6 +83,122 @@ def test_triangular_dft_backward_of_a_conjugate_pair(gpu, port, B, n):
         _same(full, sym, ("triangular dft", accumulate))
 
 
+def _exact(full, sym, what):
+    """Elementwise passes use the arithmetic of the general kernel operation for operation: equal bits, not just close."""
+    f, s = full.host(), sym.host()
+    for p in range(4):
+        assert np.array_equal(f[p], s[p]), (what, "plane", p)
+
+
+def _dz_only(port, call, rows, cols, want, what):
+    """The same pass with the dz* planes withheld (NULL): dz as before, the dz* planes of the destination untouched."""
+    keep = _pair(port, 99, (rows, cols))
+    d = ops.Grad.from_host(keep)
+    call(d)
+    h, w = d.host(), want.host()
+    assert np.array_equal(h[0], w[0]) and np.array_equal(h[1], w[1]), (what, "dz")
+    assert np.array_equal(h[2], keep[2]) and np.array_equal(h[3], keep[3]), (what, "dz* was written")
+
+
+ELEMENTWISE = [(1, 1), (3, 7), (64, 784), (130, 36), (512, 2048), (33, 1028)]
+
+
+@pytest.mark.parametrize("B,n", ELEMENTWISE)
+def test_elementwise_backward_of_a_conjugate_pair(gpu, port, B, n):
+    """CGelu, CRelu, Residual and Hadamard (per-row and shared weights): the one-gradient entry points against the general
+    ones on an exactly conjugate pair, with and without accumulation, with and without the dz* planes."""
+    g = ops.Grad.from_host(_pair(port, 5 * B + n, (B, n)))
+    x = ops.CMat.from_host(seeded(port, 1, (B, n), 2.0), seeded(port, 2, (B, n), 2.0))
+    v = ops.CMat.from_host(seeded(port, 3, (B, n), 0.05), seeded(port, 4, (B, n), 0.05))
+    v1 = ops.CMat.from_host(seeded(port, 5, (1, n), 0.05), seeded(port, 6, (1, n), 0.05))
+    for accumulate in (0, 1):
+        for name, general, sym in (("gelu", ops.gelu_bwd, ops.gelu_bwd_sym), ("crelu", ops.crelu_bwd, ops.crelu_bwd_sym)):
+            full, one = _prefilled(port, 50, B, n)
+            general(x, g, full, accumulate=accumulate)
+            sym(x, g, one, accumulate=accumulate)
+            _exact(full, one, (name, accumulate))
+            if not accumulate:
+                _dz_only(port, lambda d: sym(x, g, d, mirror=False), B, n, full, name)
+        fu, su = _prefilled(port, 60, B, n)
+        fv, sv = _prefilled(port, 61, B, n)
+        ops.residual_bwd(g, fu, fv, accumulate=accumulate)
+        ops.residual_bwd_sym(g, su, sv, accumulate=accumulate)
+        _exact(fu, su, ("residual du", accumulate)); _exact(fv, sv, ("residual dv", accumulate))
+        for shared, vv in ((False, v), (True, v1)):
+            fu, su = _prefilled(port, 70, B, n)
+            fv, sv = _prefilled(port, 71, 1 if shared else B, n)
+            ops.hadamard_bwd(x, vv, g, fu, fv, shared, accumulate=accumulate)
+            ops.hadamard_bwd_sym(x, vv, g, su, sv, shared, accumulate=accumulate)
+            _exact(fu, su, ("hadamard du", shared, accumulate)); _exact(fv, sv, ("hadamard dv", shared, accumulate))
+            if not accumulate:
+                keep = ops.Grad.from_host(_pair(port, 98, (1 if shared else B, n)))
+                _dz_only(port, lambda d: ops.hadamard_bwd_sym(x, vv, g, d, keep, shared, mirror=False), B, n, fu, "hadamard")
+                hk = keep.host()
+                assert np.array_equal(hk[0], fv.host()[0]) and np.array_equal(hk[1], fv.host()[1])
+
+
+@pytest.mark.parametrize("B,n", [(3, 6), (64, 10), (5, 1024), (3, 2048), (4, 3000), (2, 4100), (2, 5001), (2, 32768)])
+def test_loss_and_softmax_backward_of_a_conjugate_pair(gpu, port, B, n):
+    """SoftMax (every row kernel: registers, two-pass, scalar), L2Out and CrossEntropy: one-gradient entry points against
+    the general ones, equal bits."""
+    g = ops.Grad.from_host(_pair(port, 9 * B + n, (B, n)))
+    zr, zi = seeded(port, 1, (B, n)), seeded(port, 2, (B, n))
+    z = ops.CMat.from_host(zr, zi)
+    y, s = ops.CMat.empty(B, n), ops.Plane.empty(1, B)
+    ops.l2norm_fwd(z, y, s)
+    for accumulate in (0, 1):
+        full, one = _prefilled(port, 80, B, n)
+        ops.l2norm_bwd(z, s, g, full, accumulate=accumulate)
+        ops.l2norm_bwd_sym(z, s, g, one, accumulate=accumulate)
+        _exact(full, one, ("softmax", accumulate))
+        if not accumulate:
+            _dz_only(port, lambda d: ops.l2norm_bwd_sym(z, s, g, d, mirror=False), B, n, full, "softmax")
+        full, one = _prefilled(port, 81, B, n)
+        ops.l2out_bwd(z, full, accumulate=accumulate)
+        ops.l2out_bwd_sym(z, one, accumulate=accumulate)
+        _exact(full, one, ("l2out", accumulate))
+    _dz_only(port, lambda d: ops.l2out_bwd_sym(z, d, mirror=False), B, n, _l2(z, B, n), "l2out")
+    labels = ops.ints(port.randint(3, (B,), n))
+    from cnet_amd import capi
+    S, loss, am = capi.empty(B), capi.empty(B), capi.empty(B, np.int32)
+    ops.cross_entropy_fwd(z, labels, S, loss, am, None)
+    full, one = ops.Grad.empty(B, n), ops.Grad.empty(B, n)
+    ops.cross_entropy_bwd(z, S, labels, full)
+    ops.cross_entropy_bwd_sym(z, S, labels, one)
+    _exact(full, one, "cross entropy")
+    _dz_only(port, lambda d: ops.cross_entropy_bwd_sym(z, S, labels, d, mirror=False), B, n, full, "cross entropy")
+
+
+def _l2(z, B, n):
+    d = ops.Grad.empty(B, n)
+    ops.l2out_bwd(z, d)
+    return d
+
+
+def test_matrix_products_of_a_conjugate_pair_without_the_mirror_planes(gpu, port):
+    """The conjugate-pair products with the dz* planes withheld: dz as with them, nothing else written (block kernel, K
+    cut, small-C kernel, DFT and triangular DFT)."""
+    for B, K, N in [(512, 256, 256), (64, 784, 10), (4096, 784, 16), (300, 100, 37)]:
+        g = ops.Grad.from_host(_pair(port, B + K + N, (B, N)))
+        x = ops.CMat.from_host(seeded(port, 1, (B, K)), seeded(port, 2, (B, K)))
+        w = ops.CMat.from_host(seeded(port, 3, (N, K)), seeded(port, 4, (N, K)))
+        for accumulate in (0, 1):
+            with_m, _ = _prefilled(port, 10, B, K)
+            ops.linear_bwd_input_sym(g, w, with_m, accumulate=accumulate)
+            if not accumulate:
+                _dz_only(port, lambda d: ops.linear_bwd_input_sym(g, w, d, mirror=False), B, K, with_m, ("dx", B, K, N))
+            with_m, _ = _prefilled(port, 20, N, K)
+            ops.linear_bwd_weight_sym(g, x, with_m, accumulate=accumulate)
+            if not accumulate:
+                _dz_only(port, lambda d: ops.linear_bwd_weight_sym(g, x, d, mirror=False), N, K, with_m, ("dw", B, K, N))
+    B, n = 100, 320
+    g = ops.Grad.from_host(_pair(port, 5, (B, n)))
+    for sym in (ops.dft_bwd_sym, ops.triang_dft_bwd_sym):
+        with_m = ops.Grad.empty(B, n)
+        sym(g, with_m)
+        _dz_only(port, lambda d: sym(g, d, mirror=False), B, n, with_m, sym.__name__)
+
+
 @pytest.mark.parametrize("overrides", [
     {"CNET_CGEMM_SKINNY": "0"},                            # small products on the block kernels (cut along K)
     {"CNET_CGEMM_TILE": "0", "CNET_CGEMM_COLSPLIT": "0"},  # 128 x 128 blocks (two accumulator sets, negated operand)
