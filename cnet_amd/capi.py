@@ -36,6 +36,8 @@ SIGNATURES = {
     "cnet_mark_compute": [_i],
     "cnet_upload_wait_marker": [_i],
     "cnet_compute_wait_upload": [],
+    "cnet_mark_upload": [_i],
+    "cnet_compute_wait_upload_marker": [_i],
     "cnet_upload_sync": [],
     "cnet_copy_ticket": [_i, C.POINTER(C.c_int64)],
     "cnet_copy_wait": [C.c_int64],

@@ -23,6 +23,7 @@ struct Runtime {
 	hipEvent_t upload_done = nullptr, compute_done = nullptr;
 	static constexpr int kMarkers = 8;
 	hipEvent_t marker[kMarkers] = {};  // caller-numbered points of the compute stream
+	hipEvent_t upload_marker[kMarkers] = {};  // caller-numbered points of the upload stream
 	// tickets: points of either stream the HOST can wait for one by one (has this copy left its page-locked source?).
 	// A ring of events per stream; a slot that was reused stands for a later point of the same stream, so waiting on it
 	// can only wait longer, never too short.

@@ -73,6 +73,10 @@ static void destroy_streams(Runtime &r) {
 		if (m) hipEventDestroy(m);
 		m = nullptr;
 	}
+	for (auto &m : r.upload_marker) {
+		if (m) hipEventDestroy(m);
+		m = nullptr;
+	}
 	for (auto &ring : r.ticket_event)
 		for (auto &e : ring) {
 			if (e) hipEventDestroy(e);
@@ -91,6 +95,7 @@ static int create_streams(Runtime &r) {
 	CNET_HIP(hipEventCreateWithFlags(&r.upload_done, hipEventDisableTiming));
 	CNET_HIP(hipEventCreateWithFlags(&r.compute_done, hipEventDisableTiming));
 	for (auto &m : r.marker) CNET_HIP(hipEventCreateWithFlags(&m, hipEventDisableTiming));
+	for (auto &m : r.upload_marker) CNET_HIP(hipEventCreateWithFlags(&m, hipEventDisableTiming));
 	for (auto &ring : r.ticket_event)
 		for (auto &e : ring) CNET_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
 	return CNET_OK;
@@ -297,6 +302,23 @@ int cnet_upload_wait_marker(int marker) {
 	CNET_CHECK_ARG(marker >= 0 && marker < Runtime::kMarkers);
 	// a marker that was never set does not hold anything back
 	CNET_HIP(hipStreamWaitEvent(rt().upload_stream, rt().marker[marker], 0));
+	return CNET_OK;
+}
+
+int cnet_mark_upload(int marker) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();
+	CNET_CHECK_ARG(marker >= 0 && marker < Runtime::kMarkers);
+	CNET_HIP(hipEventRecord(rt().upload_marker[marker], rt().upload_stream));
+	return CNET_OK;
+}
+
+int cnet_compute_wait_upload_marker(int marker) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // would pull the upload stream into the recording
+	CNET_CHECK_ARG(marker >= 0 && marker < Runtime::kMarkers);
+	// a marker that was never set does not hold anything back
+	CNET_HIP(hipStreamWaitEvent(rt().stream, rt().upload_marker[marker], 0));
 	return CNET_OK;
 }
 

@@ -647,6 +647,21 @@ class CNet {
 	}
 	SimpleRand rand_{(uint64_t) clock()};  // upstream ComplexNet::rand_ (impl/cnet.h:56): the coin of sample()
 	bool input_dz_dirty_ = false;  // the dz planes of the input functions hold a first moment
+	// data inputs whose batch is still travelling on the upload stream (gpuSetInput): the compute stream waits for the
+	// upload stream before the first kernel that touches one of them
+	std::vector<CFunc *> in_flight_;
+	void settleUploads() {
+		if (in_flight_.empty()) return;
+		in_flight_.clear();
+		ck(cnet_compute_wait_upload(), "cnet_compute_wait_upload");
+	}
+	bool readsInFlight(CFunc *f) const {
+		if (in_flight_.empty()) return false;
+		for (auto &sl : f->slots_)
+			for (auto g : in_flight_)
+				if (sl.producer == g || f == g) return true;
+		return false;
+	}
 	bool warmed_[3] = {false, false, false};  // phase has run once since useGraphs(true)
 
 	void dropGraphs() {
@@ -835,6 +850,7 @@ public:
 		}
 		batch_ = 0;
 		d_labels_ = NULL;
+		in_flight_.clear();
 		dropGraphs();
 		use_graphs_ = false;
 		input_dz_dirty_ = false;
@@ -1256,6 +1272,7 @@ public:
 	void fetch(CFunc *f, int b) {
 		requireAllocated("fetch");
 		if (b < 0 || b >= batch_) throw std::out_of_range("fetch: batch index");
+		settleUploads();
 		ck(cnet_sync(), "cnet_sync");
 		Vars *v = f->mutable_input();
 		for (auto &s : f->slots_) {
@@ -1315,6 +1332,7 @@ public:
 	void gpuTrainStep(InputFunc *inp, OutputFunc *outp, InputBatch &batch, float l_rate) {
 		if (use_graphs_) throw std::logic_error("gpuTrainStep records the whole step itself: call useGraphs(false) first");
 		feedBatch(inp, outp, batch);
+		settleUploads();  // the recording below cannot hold a wait for the upload stream
 		StepGraphs &g = graphs_[active_];
 		auto eager = [&] {
 			const bool was = use_graphs_;
@@ -1368,7 +1386,7 @@ private:
 			// the batch was sent ahead by gpuPrefetch(): switch the data input to the buffer it landed in.  Everything
 			// queued so far may still read the buffer in use, so its retirement point is remembered for the next refill.
 			checkLabels(batch.labelsPtr(), batch_);
-			ck(cnet_compute_wait_upload(), "cnet_compute_wait_upload");
+			ck(cnet_compute_wait_upload_marker(1 - active_), "cnet_compute_wait_upload_marker");  // this batch's copies, nothing later
 			ck(cnet_mark_compute(active_), "cnet_mark_compute");
 			active_ = 1 - active_;
 			staged.holds = NULL;
@@ -1426,6 +1444,7 @@ public:
 		ck(cnet_upload_async(st.z, batch.realDataPtr(), plane * sizeof(float)), "cnet_upload_async");
 		ck(cnet_upload_async(st.z + plane, batch.imagDataPtr(), plane * sizeof(float)), "cnet_upload_async");
 		ck(cnet_upload_async(st.labels, st.host_labels, batch_ * sizeof(int32_t)), "cnet_upload_async");
+		ck(cnet_mark_upload(other), "cnet_mark_upload");
 		ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
 		st.labels_ticket = batch.ticket_;
 		st.holds = &batch;
@@ -1437,7 +1456,16 @@ public:
 			throw std::invalid_argument("gpuSetInput: " + cin->getName() + " is not a data input of this batch shape");
 		CFunc::Slot &s = cin->slots_[0];
 		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
-		if (batch.isPinned()) {  // queued behind the kernels that still read the previous contents; the host does not wait
+		if (batch.isPinned() && !use_graphs_) {
+			// On the upload stream, behind everything queued on the compute stream so far (the kernels that still use the
+			// previous contents); the compute stream waits for it only in front of the first kernel that touches this
+			// input, so the copy travels under the layers of the forward pass that come before it.
+			ck(cnet_upload_wait_compute(), "cnet_upload_wait_compute");
+			ck(cnet_upload_async(s.z, batch.realDataPtr(), plane), "cnet_upload_async");
+			ck(cnet_upload_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_upload_async");
+			ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
+			in_flight_.push_back(cin);
+		} else if (batch.isPinned()) {  // queued behind the kernels that still read the previous contents; the host does not wait
 			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d_async");
 			ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
 			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
@@ -1459,9 +1487,14 @@ public:
 	}
 	bool GpuForward() {
 		requireAllocated("GpuForward");
+		if (use_graphs_) settleUploads();  // a recording cannot hold the wait
 		runPhase(0, graphs_[active_].fwd, [&] {
-			for (auto f : func_list_) nodeForward(f);
+			for (auto f : func_list_) {
+				if (readsInFlight(f)) settleUploads();
+				nodeForward(f);
+			}
 		});
+		settleUploads();
 		return true;
 	}
 	// spellings of upstream GpuNet (gpu/gpu_func.h:645-681).  GpuInfer is upstream's forward pass without the clearing of
@@ -1485,6 +1518,7 @@ public:
 	}
 	bool gpuBackward() {
 		requireAllocated("gpuBackward");
+		settleUploads();
 		planGradients();
 		runPhase(1, graphs_[active_].bwd, [&] {
 			gather_src_.clear();  // nothing is left over from a pass that threw
@@ -1498,6 +1532,7 @@ public:
 	// z -= l_rate * dzs on every input function (the data input too, impl/cnet.h:413-421), then its gradients are cleared
 	void gpuUpdateInputs(float l_rate) {
 		requireAllocated("gpuUpdateInputs");
+		settleUploads();
 		StepGraphs &g = graphs_[active_];
 		if (g.upd && g.upd_lr != l_rate) {  // the rate is frozen into a recording
 			ck(cnet_graph_destroy(g.upd), "cnet_graph_destroy");

@@ -76,6 +76,9 @@ int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes);   /* *_copy_
  *      compute stream under number m now, make later uploads wait for that point when a buffer is about to be refilled
  *      (double buffering: the marker is set when a buffer is retired, the wait is issued when it is reused).
  * cnet_compute_wait_upload: kernels queued after this call start only when every upload queued so far has landed.
+ * cnet_mark_upload(m) / cnet_compute_wait_upload_marker(m), m = 0..7: the same in two halves - remember the current tail
+ *      of the upload stream under number m (right after the copies of one batch were queued), make later kernels wait for
+ *      that point and for nothing queued on the upload stream after it (another batch may already be travelling).
  * cnet_upload_sync: host waits for the upload stream (before reusing a page-locked source buffer).
  * cnet_copy_ticket(upload_stream, &t) / cnet_copy_wait(t): the host-side twin of the markers - t names the current tail of
  *      the compute stream (upload_stream = 0) or of the upload stream (1); cnet_copy_wait(t) blocks the host until that
@@ -90,6 +93,8 @@ int cnet_upload_wait_compute(void);
 int cnet_mark_compute(int marker);
 int cnet_upload_wait_marker(int marker);
 int cnet_compute_wait_upload(void);
+int cnet_mark_upload(int marker);
+int cnet_compute_wait_upload_marker(int marker);
 int cnet_upload_sync(void);
 int cnet_copy_ticket(int upload_stream, int64_t *ticket);
 int cnet_copy_wait(int64_t ticket);

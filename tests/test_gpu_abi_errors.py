@@ -53,6 +53,9 @@ def test_invalid_arguments_are_reported_not_fatal(gpu, port):
     assert _status("cnet_cdft_plan", 50000) == INVALID
     assert _status("cnet_adam_update", x.re.ptr, x.im.ptr, y.re.ptr, y.im.ptr, y.re.ptr, y.im.ptr, 32, 0.1, 0.9, -1, 1) == INVALID
     assert _status("cnet_mark_compute", 8) == INVALID and _status("cnet_upload_wait_marker", -1) == INVALID
+    assert _status("cnet_mark_upload", 8) == INVALID and _status("cnet_compute_wait_upload_marker", -1) == INVALID
+    assert _status("cnet_mark_upload", 3) == 0 and _status("cnet_compute_wait_upload_marker", 3) == 0
+    assert _status("cnet_compute_wait_upload_marker", 5) == 0   # never set: holds nothing back
     # copy tickets: one per stream, waited for one by one; a ticket that was never issued is refused
     t0, t1 = C.c_int64(-1), C.c_int64(-1)
     assert _status("cnet_copy_ticket", 0, C.byref(t0)) == 0 and _status("cnet_copy_ticket", 1, C.byref(t1)) == 0
@@ -87,6 +90,7 @@ def test_graph_recording_rules_and_replay(gpu, port):
     assert _status("cnet_cdft_plan", 96) == UNSUPPORTED  # a new transform length needs memory
     assert _status("cnet_graph_begin") == UNSUPPORTED
     assert _status("cnet_mark_compute", 0) == UNSUPPORTED and _status("cnet_compute_wait_upload") == UNSUPPORTED
+    assert _status("cnet_mark_upload", 0) == UNSUPPORTED and _status("cnet_compute_wait_upload_marker", 0) == UNSUPPORTED
     t = C.c_int64(-1)
     assert _status("cnet_copy_ticket", 0, C.byref(t)) == UNSUPPORTED
     capi.call("cnet_graph_end", None)
