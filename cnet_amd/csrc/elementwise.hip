@@ -495,6 +495,58 @@ __global__ __launch_bounds__(TPB) void residual_bwd_sym_kernel(const float *__re
 	out_pair<V, NT>(dv, row * lddv + col, o_r, o_i, accumulate);
 }
 
+// A Residual whose result feeds two consumers: the two incoming gradients are added here (g1 first, as two passes with
+// accumulation would), so du and dv are written once instead of written, read and written again
+template <int V, bool NT>
+__global__ __launch_bounds__(TPB) void residual_bwd_sym2_kernel(const float *__restrict__ g1_re, const float *__restrict__ g1_im, long ldg1,
+		const float *__restrict__ g2_re, const float *__restrict__ g2_im, long ldg2, Pair2 du, long lddu, Pair2 dv, long lddv, int rows,
+		int cols, int accumulate) {
+	CNET_ELEM_INDEX();
+	float o_r[V], o_i[V], p_r[V], p_i[V];
+	ldv<V, NT>(o_r, g1_re + row * ldg1 + col);
+	ldv<V, NT>(o_i, g1_im + row * ldg1 + col);
+	ldv<V, NT>(p_r, g2_re + row * ldg2 + col);
+	ldv<V, NT>(p_i, g2_im + row * ldg2 + col);
+	if (accumulate) {
+		// the order of two accumulating passes: (old + g1) + g2, for each destination
+		const Pair2 *dst[2] = {&du, &dv};
+		const long off[2] = {row * lddu + col, row * lddv + col};
+#pragma unroll
+		for (int d = 0; d < 2; ++d) {
+			float a_r[V], a_i[V];
+			ldv<V, NT>(a_r, dst[d]->dz_re + off[d]);
+			ldv<V, NT>(a_i, dst[d]->dz_im + off[d]);
+#pragma unroll
+			for (int k = 0; k < V; ++k) {
+				a_r[k] = (a_r[k] + o_r[k]) + p_r[k];
+				a_i[k] = (a_i[k] + o_i[k]) + p_i[k];
+			}
+			stv<V, NT>(dst[d]->dz_re + off[d], a_r);
+			stv<V, NT>(dst[d]->dz_im + off[d], a_i);
+			if (dst[d]->dzs_re) {
+				float b_r[V], b_i[V];
+				ldv<V, NT>(b_r, dst[d]->dzs_re + off[d]);
+				ldv<V, NT>(b_i, dst[d]->dzs_im + off[d]);
+#pragma unroll
+				for (int k = 0; k < V; ++k) {
+					b_r[k] = (b_r[k] + o_r[k]) + p_r[k];
+					b_i[k] = (b_i[k] + (-o_i[k])) + (-p_i[k]);
+				}
+				stv<V, NT>(dst[d]->dzs_re + off[d], b_r);
+				stv<V, NT>(dst[d]->dzs_im + off[d], b_i);
+			}
+		}
+		return;
+	}
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		o_r[k] += p_r[k];
+		o_i[k] += p_i[k];
+	}
+	out_pair<V, NT>(du, row * lddu + col, o_r, o_i, 0);
+	out_pair<V, NT>(dv, row * lddv + col, o_r, o_i, 0);
+}
+
 // du = G v, dv = G u (per-row operands)
 template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_sym_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
@@ -1216,6 +1268,29 @@ int cnet_residual_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ld
 		CNET_LAUNCH_V4(residual_bwd_sym_kernel, nt, CNET_GRID_2D(4), g_dz_re, g_dz_im, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
 	else
 		hipLaunchKernelGGL((residual_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), g_dz_re, g_dz_im, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_residual_bwd_sym2(const float *g1_dz_re, const float *g1_dz_im, int64_t ldg1, const float *g2_dz_re, const float *g2_dz_im,
+		int64_t ldg2, float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu, float *dv_dz_re, float *dv_dz_im,
+		float *dv_dzs_re, float *dv_dzs_im, int64_t lddv, int rows, int cols, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	const Pair2 du = pair_of(du_dz_re, du_dz_im, du_dzs_re, du_dzs_im), dv = pair_of(dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im);
+	CNET_CHECK_ARG(g1_dz_re && g1_dz_im && g2_dz_re && g2_dz_im);
+	CNET_CHECK_PAIR(du);
+	CNET_CHECK_PAIR(dv);
+	CNET_CHECK_ARG(ldg1 >= cols && ldg2 >= cols && lddu >= cols && lddv >= cols);
+	const bool nt = streaming(4 + pair_planes(du) + pair_planes(dv), (long) rows * cols);
+	if (all_mult4({cols, ldg1, ldg2, lddu, lddv}) && all_aligned({g1_dz_re, g1_dz_im, g2_dz_re, g2_dz_im, du_dz_re, du_dz_im, du_dzs_re,
+			du_dzs_im, dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im}))
+		CNET_LAUNCH_V4(residual_bwd_sym2_kernel, nt, CNET_GRID_2D(4), g1_dz_re, g1_dz_im, ldg1, g2_dz_re, g2_dz_im, ldg2, du, lddu, dv, lddv,
+				rows, cols, accumulate);
+	else
+		hipLaunchKernelGGL((residual_bwd_sym2_kernel<1, false>), CNET_GRID_2D(1), g1_dz_re, g1_dz_im, ldg1, g2_dz_re, g2_dz_im, ldg2, du, lddu,
+				dv, lddv, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }

@@ -1111,6 +1111,14 @@ private:
 		// Gradients flow only towards input functions that are stepped: a layer none of whose operands leads to one is
 		// skipped (all input functions are trainable unless CNet::setInputTrainable said otherwise, as upstream has it).
 		if (!f->wants_grad_) return;
+		if (t == isResidual && conjugate_gradients_ && f->no_outputs() == 2 && f->slots_[0].rows == rows && f->slots_[1].rows == rows) {
+			// a Residual feeding two consumers (the usual skip connection): both incoming gradients in one pass
+			CFunc::Slot &u0 = upstream(f, 0), &u1 = upstream(f, 1), &a = f->slots_[0], &v = f->slots_[1];
+			const int n = f->out_size_;
+			ck(cnet_residual_bwd_sym2(u0.g(0), u0.g(1), u0.len, u1.g(0), u1.g(1), u1.len, a.g(0), a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1),
+					v.gs(2), v.gs(3), n, rows, n, 0), "cnet_residual_bwd_sym2");
+			return;
+		}
 		for (int c = 0; c < f->no_outputs(); ++c) {
 			CFunc::Slot &u = upstream(f, c);
 			const int acc = c > 0;

@@ -242,6 +242,11 @@ def residual_bwd_sym(g, du, dv, accumulate=0, mirror=True):
          accumulate)
 
 
+def residual_bwd_sym2(g1, g2, du, dv, accumulate=0, mirror=True):
+    call("cnet_residual_bwd_sym2", *g1.p()[:2], g1.ld, *g2.p()[:2], g2.ld, *_pair(du, mirror), du.ld, *_pair(dv, mirror), dv.ld,
+         g1.rows, g1.cols, accumulate)
+
+
 def l2norm_bwd_sym(z, s, g, dz, accumulate=0, mirror=True):
     call("cnet_l2norm_bwd_sym", *z.p(), z.ld, s.ptr, *g.p()[:2], g.ld, *_pair(dz, mirror), dz.ld, z.rows, z.cols, accumulate)
 

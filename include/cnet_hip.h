@@ -325,6 +325,13 @@ int cnet_residual_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ld
                           float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
                           float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
                           int rows, int cols, int accumulate);
+/* the same for a Residual whose result feeds two consumers: their two gradients are added in the kernel (g1 first: the
+ * bits of two cnet_residual_bwd_sym calls, the second accumulating), and du, dv are written once */
+int cnet_residual_bwd_sym2(const float *g1_dz_re, const float *g1_dz_im, int64_t ldg1,
+                           const float *g2_dz_re, const float *g2_dz_im, int64_t ldg2,
+                           float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
+                           float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
+                           int rows, int cols, int accumulate);
 int cnet_l2norm_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, const float *s,
                         const float *g_dz_re, const float *g_dz_im, int64_t ldg,
                         float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,

@@ -124,6 +124,14 @@ def test_elementwise_backward_of_a_conjugate_pair(gpu, port, B, n):
         ops.residual_bwd(g, fu, fv, accumulate=accumulate)
         ops.residual_bwd_sym(g, su, sv, accumulate=accumulate)
         _exact(fu, su, ("residual du", accumulate)); _exact(fv, sv, ("residual dv", accumulate))
+        # two incoming gradients added in the kernel against two passes, the second accumulating
+        g2 = ops.Grad.from_host(_pair(port, 7 * B + n, (B, n)))
+        fu, su = _prefilled(port, 62, B, n)
+        fv, sv = _prefilled(port, 63, B, n)
+        ops.residual_bwd_sym(g, fu, fv, accumulate=accumulate)
+        ops.residual_bwd_sym(g2, fu, fv, accumulate=1)
+        ops.residual_bwd_sym2(g, g2, su, sv, accumulate=accumulate)
+        _exact(fu, su, ("residual, two consumers, du", accumulate)); _exact(fv, sv, ("residual, two consumers, dv", accumulate))
         for shared, vv in ((False, v), (True, v1)):
             fu, su = _prefilled(port, 70, B, n)
             fv, sv = _prefilled(port, 71, 1 if shared else B, n)
