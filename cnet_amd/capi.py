@@ -81,6 +81,8 @@ SIGNATURES = {
     "cnet_l2out_bwd": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_hadamard_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_cgelu_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_hadamard_cgelu_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i],
+    "cnet_hadamard_cgelu_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l] + ([c_fp] * 4 + [_l]) * 3 + [_i, _i, _i],
     "cnet_crelu_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_residual_bwd_sym": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_residual_bwd_sym2": [c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],

@@ -295,6 +295,34 @@ __global__ __launch_bounds__(TPB) void gelu_bwd_kernel(const float *__restrict__
 	outv<V, NT>(dx.dzs_im + off, o, accumulate);
 }
 
+// Hadamard followed by CGelu in one pass: h = u .* v and a = gelu(h) are both written (the backward pass needs h), u and v
+// are read once and h is not read back: 24 bytes per complex element instead of 16 + 16.
+template <int V, bool NT>
+__global__ __launch_bounds__(TPB) void hadamard_gelu_fwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
+		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, float *__restrict__ hr, float *__restrict__ hi, long ldh,
+		float *__restrict__ yr, float *__restrict__ yi, long ldy, int rows, int cols) {
+	CNET_ELEM_INDEX();
+	float a[V], b[V], c[V], d[V], pr[V], pi[V];
+	ldv<V, NT>(a, ur + row * ldu + col);
+	ldv<V, NT>(b, ui + row * ldu + col);
+	ldv<V, false>(c, vr + row * ldv_ + col);
+	ldv<V, false>(d, vi + row * ldv_ + col);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		pr[k] = a[k] * c[k] - b[k] * d[k];
+		pi[k] = a[k] * d[k] + b[k] * c[k];
+	}
+	stv<V, NT>(hr + row * ldh + col, pr);
+	stv<V, NT>(hi + row * ldh + col, pi);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		pr[k] = gelu_value(pr[k]);
+		pi[k] = gelu_value(pi[k]);
+	}
+	stv<V, NT>(yr + row * ldy + col, pr);
+	stv<V, NT>(yi + row * ldy + col, pi);
+}
+
 // ------------------------------------------------------------------------------------------------ CRelu
 // y = z where Re z > 0 and Im z > 0, else 0 (impl/relu.h:32-46 upstream); the gradients pass under the same test
 // (impl/relu.h:48-63).
@@ -547,11 +575,30 @@ __global__ __launch_bounds__(TPB) void residual_bwd_sym2_kernel(const float *__r
 	out_pair<V, NT>(dv, row * lddv + col, o_r, o_i, 0);
 }
 
-// du = G v, dv = G u (per-row operands)
+// The gradient that reaches a Hadamard through a CGelu on its result, formed in place: h = u .* v is recomputed (the bits
+// of the forward pass), g becomes the CGelu backward of g at h (the arithmetic of gelu_bwd_sym_kernel), and is stored to
+// dh, the gradient planes of the CGelu's operand, which stay readable (skipped when dh.dz_re is NULL).
 template <int V, bool NT>
+__device__ __forceinline__ void through_gelu(const float (&a)[V], const float (&b)[V], const float (&c)[V], const float (&d)[V],
+		float (&gr)[V], float (&gi)[V], const Pair2 &dh, long off) {
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		const float hr = a[k] * c[k] - b[k] * d[k], hi = a[k] * d[k] + b[k] * c[k];
+		const float px = 0.5f * gelu_slope(hr), py = 0.5f * gelu_slope(hi);
+		const float sm = px + py, df = px - py;
+		const float o_r = gr[k] * sm + gr[k] * df, o_i = gi[k] * sm + (-gi[k]) * df;
+		gr[k] = o_r;
+		gi[k] = o_i;
+	}
+	if (dh.dz_re) out_pair<V, NT>(dh, off, gr, gi, 0);
+}
+
+// du = G v, dv = G u (per-row operands).  GELU: G is first taken through a CGelu that sits on the Hadamard's result.
+template <int V, bool NT, bool GELU>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_sym_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
 		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, const float *__restrict__ g_re,
-		const float *__restrict__ g_im, long ldg, Pair2 du, long lddu, Pair2 dv, long lddv, int rows, int cols, int accumulate) {
+		const float *__restrict__ g_im, long ldg, Pair2 dh, long lddh, Pair2 du, long lddu, Pair2 dv, long lddv, int rows, int cols,
+		int accumulate) {
 	CNET_ELEM_INDEX();
 	float a[V], b[V], c[V], d[V], gr[V], gi[V], o_r[V], o_i[V];
 	ldv<V, NT>(a, ur + row * ldu + col);
@@ -560,6 +607,7 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_sym_kernel(const float *__re
 	ldv<V, NT>(d, vi + row * ldv_ + col);
 	ldv<V, NT>(gr, g_re + row * ldg + col);
 	ldv<V, NT>(gi, g_im + row * ldg + col);
+	if (GELU) through_gelu<V, NT>(a, b, c, d, gr, gi, dh, row * lddh + col);
 #pragma unroll
 	for (int k = 0; k < V; ++k) {
 		o_r[k] = gr[k] * c[k] - gi[k] * d[k];
@@ -575,11 +623,11 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_sym_kernel(const float *__re
 }
 
 // v is one shared parameter row: as hadamard_bwd_shared_kernel, two partial planes per slab
-template <int V, bool NT>
+template <int V, bool NT, bool GELU>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_sym_kernel(const float *__restrict__ ur, const float *__restrict__ ui,
 		long ldu, const float *__restrict__ vr, const float *__restrict__ vi, const float *__restrict__ g_re,
-		const float *__restrict__ g_im, long ldg, Pair2 du, long lddu, float *__restrict__ partial, int rows, int cols,
-		int rows_per_slab, int accumulate) {
+		const float *__restrict__ g_im, long ldg, Pair2 dh, long lddh, Pair2 du, long lddu, float *__restrict__ partial, int rows,
+		int cols, int rows_per_slab, int accumulate) {
 	__shared__ float red[CS_Y][2][CS_X * V];
 	const int tx = threadIdx.x % CS_X, ty = threadIdx.x / CS_X;
 	const long col = ((long) blockIdx.x * CS_X + tx) * V;
@@ -602,6 +650,7 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_sym_kernel(const floa
 			ldv<V, NT>(b, ui + (long) row * ldu + col);
 			ldv<V, NT>(gr, g_re + (long) row * ldg + col);
 			ldv<V, NT>(gi, g_im + (long) row * ldg + col);
+			if (GELU) through_gelu<V, NT>(a, b, c, d, gr, gi, dh, (long) row * lddh + col);
 #pragma unroll
 			for (int k = 0; k < V; ++k) {
 				o_r[k] = gr[k] * c[k] - gi[k] * d[k];
@@ -1295,28 +1344,47 @@ int cnet_residual_bwd_sym2(const float *g1_dz_re, const float *g1_dz_im, int64_t
 	return CNET_OK;
 }
 
-int cnet_hadamard_bwd_sym(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
-		const float *g_dz_re, const float *g_dz_im, int64_t ldg, float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im,
-		int64_t lddu, float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv, int rows, int cols,
-		int accumulate) {
-	CNET_REQUIRE_INIT();
-	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+// the launch macro for kernels with a third template flag
+#define CNET_LAUNCH_V4G(kernel, nt, gelu, ...)                                   \
+	do {                                                                         \
+		if (nt) {                                                                \
+			if (gelu) hipLaunchKernelGGL((kernel<4, true, true>), __VA_ARGS__);   \
+			else hipLaunchKernelGGL((kernel<4, true, false>), __VA_ARGS__);      \
+		} else {                                                                 \
+			if (gelu) hipLaunchKernelGGL((kernel<4, false, true>), __VA_ARGS__);  \
+			else hipLaunchKernelGGL((kernel<4, false, false>), __VA_ARGS__);     \
+		}                                                                        \
+	} while (0)
+#define CNET_LAUNCH_V1G(kernel, gelu, ...)                                   \
+	do {                                                                     \
+		if (gelu) hipLaunchKernelGGL((kernel<1, false, true>), __VA_ARGS__);  \
+		else hipLaunchKernelGGL((kernel<1, false, false>), __VA_ARGS__);     \
+	} while (0)
+
+// gelu: the incoming gradient belongs to a CGelu applied to the Hadamard's result; dh receives the gradient of that CGelu's
+// operand
+static int hadamard_bwd_sym_impl(const char *who, bool gelu, const float *u_re, const float *u_im, int64_t ldu, const float *v_re,
+		const float *v_im, int64_t ldv, const float *g_dz_re, const float *g_dz_im, int64_t ldg, Pair2 dh, int64_t lddh, Pair2 du,
+		int64_t lddu, Pair2 dv, int64_t lddv, int rows, int cols, int accumulate) {
+	if (!rt().ready) return fail(CNET_ERR_NOT_INITIALIZED, "%s: cnet_init() has not been called", who);
+	if (rows < 0 || cols < 0) return fail(CNET_ERR_INVALID_ARGUMENT, "%s: negative shape", who);
 	if (!rows || !cols) return CNET_OK;
-	const Pair2 du = pair_of(du_dz_re, du_dz_im, du_dzs_re, du_dzs_im), dv = pair_of(dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im);
-	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && g_dz_re && g_dz_im);
-	CNET_CHECK_PAIR(du);
-	CNET_CHECK_PAIR(dv);
-	CNET_CHECK_ARG(ldu >= cols && ldg >= cols && lddu >= cols && (ldv == 0 || (ldv >= cols && lddv >= cols)));
-	const bool vec = all_mult4({cols, ldu, ldv, ldg, lddu, ldv ? lddv : 0}) &&
-			all_aligned({u_re, u_im, v_re, v_im, g_dz_re, g_dz_im, du_dz_re, du_dz_im, du_dzs_re, du_dzs_im, dv_dz_re, dv_dz_im, dv_dzs_re,
-					dv_dzs_im});
-	const bool nt = streaming(4 + pair_planes(du) + (ldv ? 2 + pair_planes(dv) : 0), (long) rows * cols);
+	auto pair_ok = [](const Pair2 &p) { return p.dz_re && p.dz_im && ((p.dzs_re == nullptr) == (p.dzs_im == nullptr)); };
+	if (!(u_re && u_im && v_re && v_im && g_dz_re && g_dz_im && pair_ok(du) && pair_ok(dv) &&
+			(!gelu || pair_ok(dh) || !(dh.dz_re || dh.dz_im || dh.dzs_re || dh.dzs_im))))
+		return fail(CNET_ERR_INVALID_ARGUMENT, "%s: a required plane is NULL (the dz* planes of a result are optional, in pairs)", who);
+	if (!(ldu >= cols && ldg >= cols && lddu >= cols && (ldv == 0 || (ldv >= cols && lddv >= cols)) && (!gelu || !dh.dz_re || lddh >= cols)))
+		return fail(CNET_ERR_INVALID_ARGUMENT, "%s: a leading dimension is shorter than the row", who);
+	const bool vec = all_mult4({cols, ldu, ldv, ldg, lddu, ldv ? lddv : 0, gelu && dh.dz_re ? lddh : 0}) &&
+			all_aligned({u_re, u_im, v_re, v_im, g_dz_re, g_dz_im, du.dz_re, du.dz_im, du.dzs_re, du.dzs_im, dv.dz_re, dv.dz_im, dv.dzs_re,
+					dv.dzs_im, gelu ? dh.dz_re : nullptr, gelu ? dh.dz_im : nullptr, gelu ? dh.dzs_re : nullptr, gelu ? dh.dzs_im : nullptr});
+	const bool nt = streaming(4 + pair_planes(du) + (ldv ? 2 + pair_planes(dv) : 0) + (gelu && dh.dz_re ? pair_planes(dh) : 0), (long) rows * cols);
 	if (ldv != 0) {
 		if (vec)
-			CNET_LAUNCH_V4(hadamard_bwd_sym_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg, du, lddu, dv,
-					lddv, rows, cols, accumulate);
+			CNET_LAUNCH_V4G(hadamard_bwd_sym_kernel, nt, gelu, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg, dh, lddh,
+					du, lddu, dv, lddv, rows, cols, accumulate);
 		else
-			hipLaunchKernelGGL((hadamard_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg, du,
+			CNET_LAUNCH_V1G(hadamard_bwd_sym_kernel, gelu, CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg, dh, lddh, du,
 					lddu, dv, lddv, rows, cols, accumulate);
 		CNET_LAUNCH_CHECK();
 		return CNET_OK;
@@ -1331,13 +1399,49 @@ int cnet_hadamard_bwd_sym(const float *u_re, const float *u_im, int64_t ldu, con
 	if (!partial) return CNET_ERR_OUT_OF_MEMORY;
 	dim3 grid((unsigned) col_blocks, (unsigned) nslabs);
 	if (vec)
-		CNET_LAUNCH_V4(hadamard_bwd_shared_sym_kernel, nt, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g_dz_re, g_dz_im, ldg,
-				du, lddu, partial, rows, cols, rows_per_slab, accumulate);
+		CNET_LAUNCH_V4G(hadamard_bwd_shared_sym_kernel, nt, gelu, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g_dz_re, g_dz_im,
+				ldg, dh, lddh, du, lddu, partial, rows, cols, rows_per_slab, accumulate);
 	else
-		hipLaunchKernelGGL((hadamard_bwd_shared_sym_kernel<1, false>), grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g_dz_re,
-				g_dz_im, ldg, du, lddu, partial, rows, cols, rows_per_slab, accumulate);
+		CNET_LAUNCH_V1G(hadamard_bwd_shared_sym_kernel, gelu, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g_dz_re, g_dz_im, ldg,
+				dh, lddh, du, lddu, partial, rows, cols, rows_per_slab, accumulate);
 	CNET_LAUNCH_CHECK();
 	hipLaunchKernelGGL(slab_sum_sym_kernel, dim3((unsigned) ((2L * cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, nslabs, cols, dv, accumulate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+int cnet_hadamard_bwd_sym(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+		const float *g_dz_re, const float *g_dz_im, int64_t ldg, float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im,
+		int64_t lddu, float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv, int rows, int cols,
+		int accumulate) {
+	return hadamard_bwd_sym_impl(__func__, false, u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg, Pair2{nullptr, nullptr, nullptr, nullptr}, 0,
+			pair_of(du_dz_re, du_dz_im, du_dzs_re, du_dzs_im), lddu, pair_of(dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im), lddv, rows, cols,
+			accumulate);
+}
+
+int cnet_hadamard_cgelu_bwd_sym(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+		const float *g_dz_re, const float *g_dz_im, int64_t ldg, float *dh_dz_re, float *dh_dz_im, float *dh_dzs_re, float *dh_dzs_im,
+		int64_t lddh, float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu, float *dv_dz_re, float *dv_dz_im,
+		float *dv_dzs_re, float *dv_dzs_im, int64_t lddv, int rows, int cols, int accumulate) {
+	return hadamard_bwd_sym_impl(__func__, true, u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg,
+			pair_of(dh_dz_re, dh_dz_im, dh_dzs_re, dh_dzs_im), lddh, pair_of(du_dz_re, du_dz_im, du_dzs_re, du_dzs_im), lddu,
+			pair_of(dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im), lddv, rows, cols, accumulate);
+}
+
+int cnet_hadamard_cgelu_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+		float *h_re, float *h_im, int64_t ldh, float *y_re, float *y_im, int64_t ldy, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && h_re && h_im && y_re && y_im);
+	CNET_CHECK_ARG(ldu >= cols && ldh >= cols && ldy >= cols && (ldv == 0 || ldv >= cols));
+	const bool nt = streaming(6, (long) rows * cols);
+	if (all_mult4({cols, ldu, ldv, ldh, ldy}) && all_aligned({u_re, u_im, v_re, v_im, h_re, h_im, y_re, y_im}))
+		CNET_LAUNCH_V4(hadamard_gelu_fwd_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, h_re, h_im, ldh, y_re, y_im, ldy, rows,
+				cols);
+	else
+		hipLaunchKernelGGL((hadamard_gelu_fwd_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, h_re, h_im, ldh, y_re, y_im,
+				ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }

@@ -374,6 +374,10 @@ protected:
 	std::vector<Slot> slots_;
 	bool trainable_ = true;   // input functions: stepped by the update (CNet::setInputTrainable)
 	bool wants_grad_ = true;  // a trainable input function lies below this node: gradients have to flow through it
+	// A Hadamard whose only consumer is a CGelu that feeds one consumer itself runs with it as one pass each way
+	// (cnet_hadamard_cgelu_*): fused_next_ of the Hadamard names the CGelu, fused_prev_ of the CGelu is set.
+	CFunc *fused_next_ = NULL;
+	bool fused_prev_ = false;
 	int rows_ = 0;           // batch rows of this node's output (1 for parameter nodes)
 	float *out_ = NULL;      // 2 planes [rows][out_size]: what consumers read
 	float *out_re() const { return out_; }
@@ -632,6 +636,7 @@ class CNet {
 	StepGraphs graphs_[2];
 	bool use_graphs_ = false;
 	bool conjugate_gradients_ = true;
+	bool fuse_layers_ = true;
 	float *loss_ring_ = NULL;  // page-locked [kLossSlots][batch]: losses on their way to the host (gpuQueueLoss)
 	int64_t loss_queued_ = 0;
 	std::vector<const float *> gather_src_;  // pending dz* gathers of the input functions (see nodeBackward)
@@ -969,6 +974,7 @@ private:
 					for (auto q : p->prev_func_) reads = reads || q->rows_ != p->rows_;
 				sl.star_on_device = reads;
 			}
+		planFusion();
 		d_labels_ = dalloc<int32_t>(batch_);
 		ck(cnet_memset_zero(d_labels_, batch_ * sizeof(int32_t)), "zero");
 		if (main_input_->typeId() == isInput) {
@@ -976,6 +982,23 @@ private:
 			stage_[0].labels = d_labels_;
 		}
 		copyInputsToGpu();
+	}
+
+	void planFusion() {
+		for (auto f : func_list_) {
+			f->fused_next_ = NULL;
+			f->fused_prev_ = false;
+		}
+		if (!fuse_layers_) return;
+		for (auto f : func_list_) {
+			if (f->typeId() != isHadamard || f->no_outputs() != 1 || f->slots_[0].rows != f->rows_) continue;
+			CFunc *g = f->next_func_[0];
+			if (g->typeId() != isGelu || g->no_outputs() != 1 || g->rows_ != f->rows_ || g->slots_.size() != 1 ||
+					g->slots_[0].len != f->out_size_ || g->out_size_ != f->out_size_)
+				continue;
+			f->fused_next_ = g;
+			g->fused_prev_ = true;
+		}
 	}
 
 	// z planes of slot k of node f (read in place from the producer)
@@ -1020,11 +1043,17 @@ private:
 			break;
 		case isHadamard: {
 			const int n = f->out_size_;
+			if (CFunc *g = f->fused_next_) {  // the CGelu on its result in the same pass
+				ck(cnet_hadamard_cgelu_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), f->slots_[1].rows == rows ? n : 0, f->out_re(),
+						f->out_im(), n, g->out_re(), g->out_im(), n, rows, n), "cnet_hadamard_cgelu_fwd");
+				break;
+			}
 			ck(cnet_hadamard_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), f->slots_[1].rows == rows ? n : 0, f->out_re(),
 					f->out_im(), n, rows, n), "cnet_hadamard_fwd");
 			break;
 		}
 		case isGelu:
+			if (f->fused_prev_) break;  // written by the Hadamard below it
 			ck(cnet_cgelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_),
 					"cnet_cgelu_fwd");
 			break;
@@ -1172,6 +1201,14 @@ private:
 			case isHadamard: {
 				CFunc::Slot &v = f->slots_[1];
 				const int n = f->out_size_;
+				if (conjugate_gradients_ && f->fused_next_) {  // the backward pass of the CGelu above it in the same pass
+					CFunc *g = f->fused_next_;
+					CFunc::Slot &ug = upstream(g, 0), &h = g->slots_[0];
+					ck(cnet_hadamard_cgelu_bwd_sym(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, ug.g(0), ug.g(1), ug.len,
+							h.g(0), h.g(1), h.gs(2), h.gs(3), n, a.g(0), a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows, n,
+							acc), "cnet_hadamard_cgelu_bwd_sym");
+					break;
+				}
 				if (conjugate_gradients_) {
 					ck(cnet_hadamard_bwd_sym(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, u.g(0), u.g(1), u.len, a.g(0),
 							a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows, n, acc), "cnet_hadamard_bwd_sym");
@@ -1182,6 +1219,7 @@ private:
 				break;
 			}
 			case isGelu:
+				if (conjugate_gradients_ && f->fused_prev_) break;  // done by the Hadamard below it
 				if (conjugate_gradients_) {
 					ck(cnet_cgelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,
 							acc), "cnet_cgelu_bwd_sym");
@@ -1595,6 +1633,18 @@ public:
 		conjugate_gradients_ = on;
 	}
 	bool conjugateGradients() const { return conjugate_gradients_; }
+	// Neighbouring layers that run as one kernel where the device layer has one (Hadamard followed by CGelu): same bits,
+	// fewer passes over memory and fewer launches.  Off: one launch per layer.  Takes effect at the next allocateOnGpu,
+	// or at once when the net is allocated (recordings are dropped).
+	void fuseLayers(bool on) {
+		if (on == fuse_layers_) return;
+		fuse_layers_ = on;
+		if (batch_) {
+			dropGraphs();
+			planFusion();
+		}
+	}
+	bool fusingLayers() const { return fuse_layers_; }
 	// Upstream steps every input function, the data input included (impl/cnet.h:413-421), and therefore runs the backward
 	// pass all the way down to it.  An input function marked not trainable is left alone by gpuUpdateInputs /
 	// gpuAdamUpdate, gathers nothing, and the backward products that would only serve it are not computed (for the

@@ -233,6 +233,17 @@ def gelu_bwd_sym(x, g, dx, accumulate=0, mirror=True):
     call("cnet_cgelu_bwd_sym", *x.p(), x.ld, *g.p()[:2], g.ld, *_pair(dx, mirror), dx.ld, x.rows, x.cols, accumulate)
 
 
+def hadamard_gelu_fwd(u, v, h, y, shared=False):
+    call("cnet_hadamard_cgelu_fwd", *u.p(), u.ld, *v.p(), 0 if shared else v.ld, *h.p(), h.ld, *y.p(), y.ld, u.rows, u.cols)
+
+
+def hadamard_gelu_bwd_sym(u, v, g, dh, du, dv, shared=False, accumulate=0, mirror=True):
+    """g: the gradient pair that reaches the CGelu; dh (a Grad or None) receives the CGelu's gradient."""
+    ph = _pair(dh, mirror) if dh is not None else (None,) * 4
+    call("cnet_hadamard_cgelu_bwd_sym", *u.p(), u.ld, *v.p(), 0 if shared else v.ld, *g.p()[:2], g.ld, *ph,
+         dh.ld if dh is not None else 0, *_pair(du, mirror), du.ld, *_pair(dv, mirror), dv.ld, u.rows, u.cols, accumulate)
+
+
 def crelu_bwd_sym(x, g, dx, accumulate=0, mirror=True):
     call("cnet_crelu_bwd_sym", *x.p(), x.ld, *g.p()[:2], g.ld, *_pair(dx, mirror), dx.ld, x.rows, x.cols, accumulate)
 

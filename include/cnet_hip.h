@@ -318,6 +318,21 @@ int cnet_hadamard_bwd_sym(const float *u_re, const float *u_im, int64_t ldu, con
 int cnet_cgelu_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const float *g_dz_re, const float *g_dz_im, int64_t ldg,
                        float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
                        int rows, int cols, int accumulate);
+/* Hadamard followed by CGelu as one pass each way (the pair gpu_hadamard_forward + gpu_gelu_forward and
+ * gpu_gelu_backward + gpu_hadamard_backward, gpu/kernels.cpp:204-360; CPU twins impl/hadamard.h:34-68, impl/relu.h:119-168).
+ * Forward: h = u .* v and y = gelu(h) are both written, u and v read once: with a shared v 24 bytes per complex element
+ * instead of 16 + 16.  Backward: g is the gradient pair that reaches the CGelu; h is recomputed from u and v (the bits of
+ * the forward pass), dh = the CGelu's gradient (assigned, never accumulated; its dzs planes optional, and all four NULL
+ * when nobody reads it), du and dv as cnet_hadamard_bwd_sym from dh: with a shared v 24 (32 with dh) bytes per complex
+ * element instead of 24 + 24.  Every result has the bits of the two separate calls. */
+int cnet_hadamard_cgelu_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+                            float *h_re, float *h_im, int64_t ldh, float *y_re, float *y_im, int64_t ldy, int rows, int cols);
+int cnet_hadamard_cgelu_bwd_sym(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+                                const float *g_dz_re, const float *g_dz_im, int64_t ldg,
+                                float *dh_dz_re, float *dh_dz_im, float *dh_dzs_re, float *dh_dzs_im, int64_t lddh,
+                                float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
+                                float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
+                                int rows, int cols, int accumulate);
 int cnet_crelu_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const float *g_dz_re, const float *g_dz_im, int64_t ldg,
                        float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
                        int rows, int cols, int accumulate);

@@ -867,10 +867,11 @@ static void test_pipeline(int B, int steps) {
 	// pair computed by matrix products (conjugateGradients(false), what upstream does)
 	// 6: prefetch, the loss of a step read one step later (gpuQueueLoss / getLoss(pending)); 7: the same with gpuTrainStep
 	// 8: as 6 with the data input marked not trainable (CNet::setInputTrainable: no step on it, no backward pass into it)
-	constexpr int MODES = 9;
+	// 9: prefetch, one launch per layer (CNet::fuseLayers(false): Hadamard and CGelu as separate passes)
+	constexpr int MODES = 10;
 	std::vector<float> losses[MODES];
 	std::vector<float> weights[MODES];
-	double ms[MODES] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+	double ms[MODES] = {0};
 	for (int mode = 0; mode < MODES; ++mode) {
 		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4 || mode == 7;
 		const bool late_loss = mode == 6 || mode == 7 || mode == 8;
@@ -887,6 +888,7 @@ static void test_pipeline(int B, int steps) {
 		if (graphs) net.useGraphs(true);
 		if (mode == 5) net.conjugateGradients(false);
 		if (mode == 8) net.setInputTrainable(cin, false);
+		if (mode == 9) net.fuseLayers(false);
 		net.sync();
 		auto t0 = std::chrono::steady_clock::now();
 		// With prefetch the host runs two batches ahead: while the device computes step s, batch s+1 (assembled during
@@ -974,6 +976,7 @@ static void test_pipeline(int B, int steps) {
 		expect("weights identical when each loss is read one step late", weights[0] == weights[6]);
 		expect("losses and weights identical with gpuTrainStep and the late read together", losses[0] == losses[7] && weights[0] == weights[7]);
 		expect("losses and weights identical with the data input not trainable", losses[0] == losses[8] && weights[0] == weights[8]);
+		expect("losses and weights identical with one launch per layer (no fused Hadamard + CGelu)", losses[0] == losses[9] && weights[0] == weights[9]);
 		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
 		// dz* planes written as the conjugate of the dz product against dz* planes computed by a product of their own
 		double worst = 0, num = 0, den = 0;

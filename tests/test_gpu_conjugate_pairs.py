@@ -145,6 +145,46 @@ def test_elementwise_backward_of_a_conjugate_pair(gpu, port, B, n):
                 assert np.array_equal(hk[0], fv.host()[0]) and np.array_equal(hk[1], fv.host()[1])
 
 
+@pytest.mark.parametrize("B,n", ELEMENTWISE + [(4096, 784)])
+def test_hadamard_followed_by_cgelu_in_one_pass(gpu, port, B, n):
+    """cnet_hadamard_cgelu_fwd / _bwd_sym against the two separate calls each way (equal bits: h, y, dh, du, dv), per-row and
+    shared weights, with and without accumulation into du / dv, with and without the planes of dh; and against the oracle."""
+    from tests.gpu_util import rel_c, TOL
+    g = ops.Grad.from_host(_pair(port, 11 * B + n, (B, n)))
+    xr, xi = seeded(port, 1, (B, n), 2.0), seeded(port, 2, (B, n), 2.0)
+    x = ops.CMat.from_host(xr, xi)
+    for shared in (False, True):
+        rows_v = 1 if shared else B
+        vr, vi = seeded(port, 3, (rows_v, n), 0.7), seeded(port, 4, (rows_v, n), 0.7)
+        v = ops.CMat.from_host(vr, vi)
+        h0, y0, h1, y1 = (ops.CMat.empty(B, n) for _ in range(4))
+        ops.hadamard_fwd(x, v, h0, shared)
+        ops.gelu_fwd(h0, y0)
+        ops.hadamard_gelu_fwd(x, v, h1, y1, shared)
+        for a, b in ((h0, h1), (y0, y1)):
+            assert np.array_equal(a.host()[0], b.host()[0]) and np.array_equal(a.host()[1], b.host()[1]), ("forward", shared)
+        if B * n <= 1 << 17:  # the oracle, sample by sample
+            hr, hi = port.hadamard_fwd(xr, xi, vr if not shared else vr[0], vi if not shared else vi[0])
+            assert rel_c(y1.host(), port.gelu_fwd(hr, hi)) < TOL
+        for accumulate in (0, 1):
+            dh0 = ops.Grad.empty(B, n)
+            ops.gelu_bwd_sym(h0, g, dh0)
+            fu, su = _prefilled(port, 70, B, n)
+            fv, sv = _prefilled(port, 71, rows_v, n)
+            ops.hadamard_bwd_sym(x, v, dh0, fu, fv, shared, accumulate=accumulate)
+            dh1 = ops.Grad.from_host(_pair(port, 97, (B, n)))
+            ops.hadamard_gelu_bwd_sym(x, v, g, dh1, su, sv, shared, accumulate=accumulate)
+            _exact(dh0, dh1, ("dh", shared, accumulate))
+            _exact(fu, su, ("du", shared, accumulate)); _exact(fv, sv, ("dv", shared, accumulate))
+            # without the planes of dh, and without the dz* planes of du and dv
+            nu, nv = _prefilled(port, 70, B, n)[0], _prefilled(port, 71, rows_v, n)[0]
+            ops.hadamard_gelu_bwd_sym(x, v, g, None, nu, nv, shared, accumulate=accumulate, mirror=False)
+            for got, want, keep_seed, r in ((nu, fu, 70, B), (nv, fv, 71, rows_v)):
+                hg, hw, keep = got.host(), want.host(), _pair(port, keep_seed, (r, n))
+                assert np.array_equal(hg[0], hw[0]) and np.array_equal(hg[1], hw[1]), ("dz", shared, accumulate)
+                assert np.array_equal(hg[2], keep[2]) and np.array_equal(hg[3], keep[3]), ("dz* was written", shared)
+
+
 @pytest.mark.parametrize("B,n", [(3, 6), (64, 10), (5, 1024), (3, 2048), (4, 3000), (2, 4100), (2, 5001), (2, 32768)])
 def test_loss_and_softmax_backward_of_a_conjugate_pair(gpu, port, B, n):
     """SoftMax (every row kernel: registers, two-pass, scalar), L2Out and CrossEntropy: one-gradient entry points against
