@@ -51,6 +51,7 @@ SIGNATURES = {
     "cnet_cgemm": [_i, _i, _i, _i, _i, _i, c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, _i],
     "cnet_cgemm_batched": [_i, _i, _i, _i, _i, _i, _i, c_fp, c_fp, _l, _l, c_fp, c_fp, _l, _l, c_fp, c_fp, _l, _l, _i, _i],
     "cnet_clinear_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i, _i, _i],
+    "cnet_clinear_cgelu_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, c_fp, c_fp, _l, _i, _i, _i, _i],
     "cnet_clinear_bwd_input": [c_fp] * 4 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
     "cnet_clinear_bwd_weight": [c_fp] * 4 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
     "cnet_clinear_bwd_input_sym": [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],

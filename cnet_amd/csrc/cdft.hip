@@ -11,7 +11,7 @@ namespace cnet {
 
 int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
 		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
-		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri, bool mirror);
+		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri, int mirror);
 
 struct Twiddle {
 	float *re = nullptr;
@@ -159,7 +159,7 @@ int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re
 	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {f_re, f_re}, *bi[2] = {f_im, f_im};
 	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate, 0, false);
+	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate, 0, 0);
 }
 
 int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
@@ -176,7 +176,7 @@ int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs
 	const float *ar[2] = {g_dz_re, g_dzs_re}, *ai[2] = {g_dz_im, g_dzs_im}, *br[2] = {t.re, t.re}, *bi[2] = {t.im, t.im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, true};
-	return cgemm_pair(false, true, 2, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 0, false);
+	return cgemm_pair(false, true, 2, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 0, 0);
 }
 
 int cnet_ctriang_dft_plan(int n) {
@@ -199,7 +199,7 @@ int cnet_ctriang_dft_fwd(const float *x_re, const float *x_im, int64_t ldx, floa
 	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {t.tri_re, t.tri_re}, *bi[2] = {t.tri_im, t.tri_im};
 	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate, 1, false);
+	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate, 1, 0);
 }
 
 // dz_i = sum_{o >= i} G_o T[i][o], dzs_i = sum_{o >= i} Gs_o conj(T[i][o])  (impl/ft.h:163-189 upstream): the same
@@ -218,7 +218,7 @@ int cnet_cdft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, f
 	const float *ar[2] = {g_dz_re, g_dz_re}, *ai[2] = {g_dz_im, g_dz_im}, *br[2] = {t.re, t.re}, *bi[2] = {t.im, t.im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 0, dx_dzs_re != nullptr);
+	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 0, dx_dzs_re != nullptr ? 1 : 0);
 }
 
 int cnet_ctriang_dft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, float *dx_dz_re, float *dx_dz_im,
@@ -234,7 +234,7 @@ int cnet_ctriang_dft_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t
 	const float *ar[2] = {g_dz_re, g_dz_re}, *ai[2] = {g_dz_im, g_dz_im}, *br[2] = {t.tri_re, t.tri_re}, *bi[2] = {t.tri_im, t.tri_im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(false, false, 1, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 2, dx_dzs_re != nullptr);
+	return cgemm_pair(false, false, 1, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 2, dx_dzs_re != nullptr ? 1 : 0);
 }
 
 int cnet_ctriang_dft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
@@ -250,7 +250,7 @@ int cnet_ctriang_dft_bwd(const float *g_dz_re, const float *g_dz_im, const float
 	const float *ar[2] = {g_dz_re, g_dzs_re}, *ai[2] = {g_dz_im, g_dzs_im}, *br[2] = {t.tri_re, t.tri_re}, *bi[2] = {t.tri_im, t.tri_im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, true};
-	return cgemm_pair(false, false, 2, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 2, false);
+	return cgemm_pair(false, false, 2, B, n, n, ar, ai, ldg, br, bi, t.ld, cj, cr, ci, lddx, accumulate, 2, 0);
 }
 
 }  // extern "C"

@@ -72,11 +72,15 @@ struct CgemmArgs {
 	// `accumulate` there as well).  The backward passes use it when the incoming dz* gradient is the conjugate of the dz
 	// gradient, as it is under every real-valued loss: the dz* product is then the conjugate of the dz product (the same
 	// sums with signs applied exactly) and need not be computed.  Not combined with a strided batch.
+	// mirror == 2 (MIRROR_GELU): the C planes of p[1] receive the CGelu of the final value of C instead (a Linear followed by
+	// a CGelu in one launch: the pre-activation and the activation are both written, neither is read back); always assigned.
 	int mirror;
 };
+constexpr int MIRROR_CONJ = 1, MIRROR_GELU = 2;
 
 // the conjugate of (vr, vi) into element `off` of the mirror planes
 __device__ __forceinline__ void mirror_store(const CgemmArgs &args, long off, float vr, float vi) {
+	if (args.mirror != MIRROR_CONJ) return;
 	float mr = vr, mi = -vi;
 	if (args.accumulate) {
 		mr += args.p[1].c_re[off];
@@ -84,6 +88,13 @@ __device__ __forceinline__ void mirror_store(const CgemmArgs &args, long off, fl
 	}
 	args.p[1].c_re[off] = mr;
 	args.p[1].c_im[off] = mi;
+}
+
+// the CGelu of the final value (vr, vi) of element `off` into the planes of p[1]
+__device__ __forceinline__ void gelu_store(const CgemmArgs &args, long off, float vr, float vi) {
+	if (args.mirror != MIRROR_GELU) return;
+	args.p[1].c_re[off] = cnet::gelu_value(vr);
+	args.p[1].c_im[off] = cnet::gelu_value(vi);
 }
 
 // Which block of C (per problem) a linear block number stands for: walks groups of 8 block rows column by column, after
@@ -384,6 +395,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 					}
 					pb.c_re[off] = vr;
 					pb.c_im[off] = vi;
+					if (args.mirror && args.splits == 1) gelu_store(args, (long) row * args.ldc + col, vr, vi);
 				}
 			}
 		}
@@ -805,6 +817,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 					}
 					pb.c_re[off] = vr;
 					pb.c_im[off] = vi;
+					if (mirror_now) gelu_store(args, (long) row * args.ldc + col, vr, vi);
 				}
 			}
 		}
@@ -823,11 +836,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(CgemmArgs args, int 
 	const float *first = args.partial + (((long) prob * nbatch + b) * 2 + part) * plane + e;
 	float v = cnet::ordered_sum(first, (long) nprob * nbatch * 2 * plane, args.splits);
 	float *c = (part ? args.p[prob].c_im : args.p[prob].c_re) + (long) b * args.stride_c + row * args.ldc + col;
-	*c = args.accumulate ? *c + v : v;
-	if (args.mirror) {
+	const float fin = args.accumulate ? *c + v : v;
+	*c = fin;
+	if (args.mirror == MIRROR_CONJ) {
 		float *m = (part ? args.p[1].c_im : args.p[1].c_re) + row * args.ldc + col;
 		const float mv = part ? -v : v;
 		*m = args.accumulate ? *m + mv : mv;
+	} else if (args.mirror == MIRROR_GELU) {
+		(part ? args.p[1].c_im : args.p[1].c_re)[row * args.ldc + col] = cnet::gelu_value(fin);
 	}
 }
 
@@ -850,11 +866,14 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(CgemmArgs args) {
 		if (row >= args.M || col >= args.N) continue;
 		const float v = cnet::ordered_sum(first + idx, 2L * BM * BN, args.tail_splits);
 		float *c = (part ? args.p[prob].c_im : args.p[prob].c_re) + (long) row * args.ldc + col;
-		*c = args.accumulate ? *c + v : v;
-		if (args.mirror) {
+		const float fin = args.accumulate ? *c + v : v;
+		*c = fin;
+		if (args.mirror == MIRROR_CONJ) {
 			float *m = (part ? args.p[1].c_im : args.p[1].c_re) + (long) row * args.ldc + col;
 			const float mv = part ? -v : v;
 			*m = args.accumulate ? *m + mv : mv;
+		} else if (args.mirror == MIRROR_GELU) {
+			(part ? args.p[1].c_im : args.p[1].c_re)[(long) row * args.ldc + col] = cnet::gelu_value(fin);
 		}
 	}
 }
@@ -1001,11 +1020,14 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 		const int row = m0 + 4 * q + e;
 		if (row < args.M && col < args.N) {
 			float *dst = (part ? pb.c_im : pb.c_re) + (long) row * ldc + col;
-			*dst = accumulate ? *dst + v : v;
-			if (args.mirror && args.splits == 1) {
+			const float fin = accumulate ? *dst + v : v;
+			*dst = fin;
+			if (args.mirror == MIRROR_CONJ && args.splits == 1) {
 				float *m = (part ? args.p[1].c_im : args.p[1].c_re) + (long) row * args.ldc + col;
 				const float mv = part ? -v : v;
 				*m = args.accumulate ? *m + mv : mv;
+			} else if (args.mirror == MIRROR_GELU && args.splits == 1) {
+				(part ? args.p[1].c_im : args.p[1].c_re)[(long) row * args.ldc + col] = cnet::gelu_value(fin);
 			}
 		}
 	}
@@ -1445,12 +1467,12 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 // Used by cdft.hip
 int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
 		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
-		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri, bool mirror) {
+		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri, int mirror) {
 	if (tri && N != K) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: a triangular operand must be square");
 	if (mirror && nprob != 1) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: a mirrored product is one problem");
 	CgemmArgs a;
 	a.tri = tri;
-	a.mirror = mirror ? 1 : 0;
+	a.mirror = mirror;
 	for (int q = 0; q < nprob; ++q) {
 		a.p[q].a_re = a_re[q];
 		a.p[q].a_im = a_im[q];
@@ -1463,7 +1485,7 @@ int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, c
 	}
 	if (nprob == 1) {
 		a.p[1] = a.p[0];
-		if (mirror) {  // the planes that receive the conjugate of the product
+		if (mirror) {  // the planes that receive the conjugate of the product, or its CGelu
 			a.p[1].c_re = c_re[1];
 			a.p[1].c_im = c_im[1];
 		}
@@ -1497,7 +1519,7 @@ int cnet_cgemm(int a_kmajor, int b_kmajor, int conj_b, int M, int N, int K, cons
 	const float *ar[2] = {a_re, a_re}, *ai[2] = {a_im, a_im}, *br[2] = {b_re, b_re}, *bi[2] = {b_im, b_im};
 	float *cr[2] = {c_re, c_re}, *ci[2] = {c_im, c_im};
 	bool cj[2] = {conj_b != 0, conj_b != 0};
-	return cgemm_pair(a_kmajor != 0, b_kmajor != 0, 1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, accumulate, 0, false);
+	return cgemm_pair(a_kmajor != 0, b_kmajor != 0, 1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, accumulate, 0, 0);
 }
 
 int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M, int N, int K, const float *a_re,
@@ -1541,6 +1563,19 @@ int cnet_clinear_fwd(const float *x_re, const float *x_im, int64_t ldx, const fl
 	return cnet_cgemm(0, 0, 0, B, N, K, x_re, x_im, ldx, w_re, w_im, ldw, y_re, y_im, ldy, accumulate);
 }
 
+int cnet_clinear_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx, const float *w_re, const float *w_im, int64_t ldw,
+		float *h_re, float *h_im, float *y_re, float *y_im, int64_t ldy, int B, int K, int N, int accumulate) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && N >= 0 && K > 0);
+	if (B == 0 || N == 0) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && w_re && w_im && h_re && h_im && y_re && y_im);
+	CNET_CHECK_ARG(ldx >= K && ldw >= K && ldy >= N);
+	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {w_re, w_re}, *bi[2] = {w_im, w_im};
+	float *cr[2] = {h_re, y_re}, *ci[2] = {h_im, y_im};
+	bool cj[2] = {false, false};
+	return cgemm_pair(false, false, 1, B, N, K, ar, ai, ldx, br, bi, ldw, cj, cr, ci, ldy, accumulate, 0, MIRROR_GELU);
+}
+
 int cnet_clinear_bwd_input(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,
 		int64_t ldg, const float *w_re, const float *w_im, int64_t ldw, float *dx_dz_re, float *dx_dz_im,
 		float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int B, int K, int N, int accumulate) {
@@ -1555,7 +1590,7 @@ int cnet_clinear_bwd_input(const float *g_dz_re, const float *g_dz_im, const flo
 	const float *br[2] = {w_re, w_re}, *bi[2] = {w_im, w_im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, true};
-	return cgemm_pair(false, true, 2, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0, false);
+	return cgemm_pair(false, true, 2, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0, 0);
 }
 
 int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,
@@ -1572,7 +1607,7 @@ int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const fl
 	const float *br[2] = {x_re, x_re}, *bi[2] = {x_im, x_im};
 	float *cr[2] = {dw_dz_re, dw_dzs_re}, *ci[2] = {dw_dz_im, dw_dzs_im};
 	bool cj[2] = {false, true};
-	return cgemm_pair(true, true, 2, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0, false);
+	return cgemm_pair(true, true, 2, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0, 0);
 }
 
 int cnet_clinear_bwd_input_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *w_re, const float *w_im,
@@ -1588,7 +1623,7 @@ int cnet_clinear_bwd_input_sym(const float *g_dz_re, const float *g_dz_im, int64
 	const float *br[2] = {w_re, w_re}, *bi[2] = {w_im, w_im};
 	float *cr[2] = {dx_dz_re, dx_dzs_re}, *ci[2] = {dx_dz_im, dx_dzs_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(false, true, 1, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0, dx_dzs_re != nullptr);
+	return cgemm_pair(false, true, 1, B, K, N, ar, ai, ldg, br, bi, ldw, cj, cr, ci, lddx, accumulate, 0, dx_dzs_re != nullptr ? MIRROR_CONJ : 0);
 }
 
 int cnet_clinear_bwd_weight_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *x_re, const float *x_im,
@@ -1603,7 +1638,7 @@ int cnet_clinear_bwd_weight_sym(const float *g_dz_re, const float *g_dz_im, int6
 	const float *br[2] = {x_re, x_re}, *bi[2] = {x_im, x_im};
 	float *cr[2] = {dw_dz_re, dw_dzs_re}, *ci[2] = {dw_dz_im, dw_dzs_im};
 	bool cj[2] = {false, false};
-	return cgemm_pair(true, true, 1, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0, dw_dzs_re != nullptr);
+	return cgemm_pair(true, true, 1, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0, dw_dzs_re != nullptr ? MIRROR_CONJ : 0);
 }
 
 }  // extern "C"

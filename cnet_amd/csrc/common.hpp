@@ -100,6 +100,22 @@ __device__ __forceinline__ float ordered_sum(const float *__restrict__ first, lo
 	return s;
 }
 
+// tanh-GELU of one real plane value and its derivative (impl/relu.h:119-131, 144-166 upstream); shared by the elementwise
+// kernels and the matrix-product epilogue that applies the CGelu of a Linear's result, so both give the same bits
+__device__ __forceinline__ float gelu_value(float t) {
+	const float c = 0.7978845608028654f;  // sqrt(2/pi)
+	float arg = c * (t + 0.044715f * t * t * t);
+	return 0.5f * t * (1.0f + tanhf(arg));
+}
+
+__device__ __forceinline__ float gelu_slope(float t) {
+	const float c = 0.7978845608028654f;
+	float arg = c * (t + 0.044715f * t * t * t);
+	float th = tanhf(arg);
+	float sech2 = 1.0f - th * th;  // = 1/cosh^2
+	return 0.5f * (1.0f + th) + t * 0.5f * sech2 * c * (1.0f + 3.0f * 0.044715f * t * t);
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace cnet

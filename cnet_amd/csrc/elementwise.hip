@@ -11,6 +11,9 @@
 
 namespace {
 
+using cnet::gelu_slope;
+using cnet::gelu_value;
+
 constexpr int TPB = 256;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -232,20 +235,6 @@ __global__ __launch_bounds__(TPB) void slab_sum_kernel(const float *__restrict__
 
 // ------------------------------------------------------------------------------------------------ CGelu
 // tanh-GELU on each real plane (impl/relu.h:119-131 upstream).
-__device__ __forceinline__ float gelu_value(float t) {
-	const float c = 0.7978845608028654f;  // sqrt(2/pi)
-	float arg = c * (t + 0.044715f * t * t * t);
-	return 0.5f * t * (1.0f + tanhf(arg));
-}
-
-__device__ __forceinline__ float gelu_slope(float t) {
-	const float c = 0.7978845608028654f;
-	float arg = c * (t + 0.044715f * t * t * t);
-	float th = tanhf(arg);
-	float sech2 = 1.0f - th * th;  // = 1/cosh^2
-	return 0.5f * (1.0f + th) + t * 0.5f * sech2 * c * (1.0f + 3.0f * 0.044715f * t * t);
-}
-
 template <int V, bool NT>
 __global__ __launch_bounds__(TPB) void gelu_fwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		float *__restrict__ yr, float *__restrict__ yi, long ldy, int rows, int cols) {

@@ -375,9 +375,11 @@ protected:
 	bool trainable_ = true;   // input functions: stepped by the update (CNet::setInputTrainable)
 	bool wants_grad_ = true;  // a trainable input function lies below this node: gradients have to flow through it
 	// A Hadamard whose only consumer is a CGelu that feeds one consumer itself runs with it as one pass each way
-	// (cnet_hadamard_cgelu_*): fused_next_ of the Hadamard names the CGelu, fused_prev_ of the CGelu is set.
+	// (cnet_hadamard_cgelu_*): fused_next_ of the Hadamard names the CGelu, fused_prev_ of the CGelu is 2.  A Linear whose
+	// only consumer is a CGelu applies it when it stores its product (cnet_clinear_cgelu_fwd): fused_prev_ of the CGelu is
+	// 1, its backward pass runs as usual.
 	CFunc *fused_next_ = NULL;
-	bool fused_prev_ = false;
+	int fused_prev_ = 0;
 	int rows_ = 0;           // batch rows of this node's output (1 for parameter nodes)
 	float *out_ = NULL;      // 2 planes [rows][out_size]: what consumers read
 	float *out_re() const { return out_; }
@@ -987,17 +989,19 @@ private:
 	void planFusion() {
 		for (auto f : func_list_) {
 			f->fused_next_ = NULL;
-			f->fused_prev_ = false;
+			f->fused_prev_ = 0;
 		}
 		if (!fuse_layers_) return;
 		for (auto f : func_list_) {
-			if (f->typeId() != isHadamard || f->no_outputs() != 1 || f->slots_[0].rows != f->rows_) continue;
+			const int t = f->typeId();
+			if ((t != isHadamard && t != isLinear) || f->no_outputs() != 1 || f->slots_[0].rows != f->rows_) continue;
 			CFunc *g = f->next_func_[0];
-			if (g->typeId() != isGelu || g->no_outputs() != 1 || g->rows_ != f->rows_ || g->slots_.size() != 1 ||
-					g->slots_[0].len != f->out_size_ || g->out_size_ != f->out_size_)
+			if (g->typeId() != isGelu || g->rows_ != f->rows_ || g->slots_.size() != 1 || g->slots_[0].len != f->out_size_ ||
+					g->out_size_ != f->out_size_)
 				continue;
+			if (t == isHadamard && g->no_outputs() != 1) continue;
 			f->fused_next_ = g;
-			g->fused_prev_ = true;
+			g->fused_prev_ = t == isHadamard ? 2 : 1;
 		}
 	}
 
@@ -1025,6 +1029,11 @@ private:
 		}
 		case isLinear: {
 			const int K = f->slots_[0].len, N = f->out_size_;
+			if (CFunc *g = f->fused_next_) {  // the CGelu on its result is applied as the product is stored
+				ck(cnet_clinear_cgelu_fwd(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), g->out_re(), g->out_im(),
+						N, rows, K, N, 0), "cnet_clinear_cgelu_fwd");
+				break;
+			}
 			ck(cnet_clinear_fwd(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), N, rows, K, N, 0),
 					"cnet_clinear_fwd");
 			break;
@@ -1053,7 +1062,7 @@ private:
 			break;
 		}
 		case isGelu:
-			if (f->fused_prev_) break;  // written by the Hadamard below it
+			if (f->fused_prev_) break;  // written by the Hadamard or the Linear below it
 			ck(cnet_cgelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_),
 					"cnet_cgelu_fwd");
 			break;
@@ -1219,7 +1228,7 @@ private:
 				break;
 			}
 			case isGelu:
-				if (conjugate_gradients_ && f->fused_prev_) break;  // done by the Hadamard below it
+				if (conjugate_gradients_ && f->fused_prev_ == 2) break;  // done by the Hadamard below it
 				if (conjugate_gradients_) {
 					ck(cnet_cgelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,
 							acc), "cnet_cgelu_bwd_sym");
@@ -1633,7 +1642,7 @@ public:
 		conjugate_gradients_ = on;
 	}
 	bool conjugateGradients() const { return conjugate_gradients_; }
-	// Neighbouring layers that run as one kernel where the device layer has one (Hadamard followed by CGelu): same bits,
+	// Neighbouring layers that run as one kernel where the device layer has one (Hadamard or Linear followed by CGelu): same bits,
 	// fewer passes over memory and fewer launches.  Off: one launch per layer.  Takes effect at the next allocateOnGpu,
 	// or at once when the net is allocated (recordings are dropped).
 	void fuseLayers(bool on) {

@@ -108,6 +108,11 @@ def linear_fwd(x, w, y, accumulate=0):
     call("cnet_clinear_fwd", *x.p(), x.ld, *w.p(), w.ld, *y.p(), y.ld, x.rows, x.cols, w.rows, accumulate)
 
 
+def linear_gelu_fwd(x, w, h, y, accumulate=0):
+    assert h.ld == y.ld
+    call("cnet_clinear_cgelu_fwd", *x.p(), x.ld, *w.p(), w.ld, *h.p(), *y.p(), y.ld, x.rows, x.cols, w.rows, accumulate)
+
+
 def linear_bwd_input(g, w, dx, accumulate=0):
     call("cnet_clinear_bwd_input", *g.p(), g.ld, *w.p(), w.ld, *dx.p(), dx.ld, g.rows, w.cols, w.rows, accumulate)
 

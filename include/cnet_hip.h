@@ -142,6 +142,15 @@ int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M
 int cnet_clinear_fwd(const float *x_re, const float *x_im, int64_t ldx,
                      const float *w_re, const float *w_im, int64_t ldw,
                      float *y_re, float *y_im, int64_t ldy, int B, int K, int N, int accumulate);
+/* Linear followed by CGelu in one launch (gpu_linear_forward + gpu_gelu_forward, gpu/reduce.cpp:56-77 and
+ * gpu/kernels.cpp:276-300; CPU twins impl/linear.h:51-69, impl/relu.h:119-131): h = x * w^T (the pre-activation, which
+ * the backward pass of the CGelu reads) and y = gelu(h), applied to the accumulators when they are stored, so h is not
+ * read back.  h and y share the leading dimension ldy.  With accumulate != 0 the product is added to h and y = gelu of
+ * the sum.  y has the bits of cnet_cgelu_fwd applied to h. */
+int cnet_clinear_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx,
+                           const float *w_re, const float *w_im, int64_t ldw,
+                           float *h_re, float *h_im, float *y_re, float *y_im, int64_t ldy,
+                           int B, int K, int N, int accumulate);
 /* dx.dz = g.dz * w ; dx.dzs = g.dzs * conj(w)            (both products in one launch) */
 int cnet_clinear_bwd_input(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,
                            int64_t ldg, const float *w_re, const float *w_im, int64_t ldw,

@@ -334,6 +334,32 @@ static void test_resblock() {
 		report("weights after update" + s, ww.value(), 1e-5);
 		printf("     step %d mean loss %.6f\n", step, mean);
 	}
+	// the same training with one launch per layer (no CGelu applied in the Linear's store): equal bits
+	auto train = [&](bool fuse) {
+		ResStack q;
+		build_stack(q, n, blocks);
+		for (int b = 0; b < blocks; ++b) std::copy(w0[b].begin(), w0[b].end(), q.net[q.w[b]]->mutable_input()->real_);
+		q.net.fuseLayers(fuse);
+		q.net.allocateOnGpu(B);
+		std::vector<float> out;
+		for (int step = 0; step < steps; ++step) {
+			InputBatch bx(B, n), bt(B, n);
+			for (int b = 0; b < B; ++b) {
+				bx.add(xs.data() + (size_t) b * n, xs.data() + (size_t) (B + b) * n, n, 0);
+				bt.add(ts.data() + (size_t) b * n, ts.data() + (size_t) (B + b) * n, n, 0);
+			}
+			q.net.gpuSetInput((CInput *) q.net[q.t], bt);
+			q.net.gpuForward((CInput *) q.net[q.x], (L2Out *) q.net[q.l2], bx);
+			out.push_back(q.net.getLoss((L2Out *) q.net[q.l2], &bx));
+			q.net.gpuBackward();
+			q.net.gpuUpdateInputs(lr / B);
+		}
+		q.net.getInputsFromGpu();
+		for (int b = 0; b < blocks; ++b)
+			out.insert(out.end(), q.net[q.w[b]]->input().real_, q.net[q.w[b]]->input().real_ + 2 * n * n);
+		return out;
+	};
+	expect("losses and weights identical with Linear + CGelu as one launch and as two", train(true) == train(false));
 }
 
 // ------------------------------------------------------------------------------------------------- per-sample API

@@ -1,0 +1,76 @@
+"""Layers that run as one launch: Linear followed by CGelu (the activation applied to the accumulators of the matrix product
+when they are stored).  The fused entry point must give the bits of the two separate calls, whichever kernel the shape takes
+(block kernels of each shape, the register-staged kernel for odd sizes, a K that is not a whole number of chunks, the
+small-C kernel with and without slices of K, blocks cut along K, tail blocks, columns split off), and agree with the CPU
+oracle."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from cnet_amd import ops
+from tests.gpu_util import gpu, rel_c, seeded, TOL  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+# B, K (in), N (out)
+LINEAR = [(4096, 1024, 1024), (2048, 2048, 2048), (512, 784, 256), (64, 784, 10), (64, 784, 784), (300, 100, 37), (4096, 784, 784),
+          (2048, 544, 544), (4096, 784, 10), (16, 16, 16), (257, 33, 7), (2048, 550, 549), (1000, 1000, 512), (256, 4096, 64)]
+
+
+@pytest.mark.parametrize("B,K,N", LINEAR)
+def test_linear_followed_by_cgelu_in_one_launch(gpu, port, B, K, N):
+    xr, xi = seeded(port, B + K, (B, K)), seeded(port, B + K + 1, (B, K))
+    wr, wi = seeded(port, N + 2, (N, K), K ** -0.5), seeded(port, N + 3, (N, K), K ** -0.5)
+    x, w = ops.CMat.from_host(xr, xi), ops.CMat.from_host(wr, wi)
+    base = (seeded(port, 5, (B, N)), seeded(port, 6, (B, N)))
+    for accumulate in (0, 1):
+        h0, h1 = ops.CMat.from_host(*base), ops.CMat.from_host(*base)
+        y0, y1 = ops.CMat.empty(B, N), ops.CMat.from_host(*base)
+        ops.linear_fwd(x, w, h0, accumulate=accumulate)
+        ops.gelu_fwd(h0, y0)
+        ops.linear_gelu_fwd(x, w, h1, y1, accumulate=accumulate)
+        for a, b, what in ((h0, h1, "pre-activation"), (y0, y1, "activation")):
+            ha, hb = a.host(), b.host()
+            assert np.array_equal(ha[0], hb[0]) and np.array_equal(ha[1], hb[1]), (what, accumulate)
+    if B * K * N <= 1 << 26:   # the CPU path, sample by sample
+        hr, hi = port.linear_fwd(xr, xi, wr, wi)
+        ops.linear_gelu_fwd(x, w, h1, y1)
+        assert rel_c(h1.host(), (hr, hi)) < TOL / 5
+        assert rel_c(y1.host(), port.gelu_fwd(hr, hi)) < TOL / 5
+
+
+def test_linear_cgelu_into_a_column_window(gpu, port):
+    """Both results land in column windows of wider buffers (shared leading dimension) and leave the rest alone."""
+    B, K, N, W = 70, 48, 40, 64
+    x = ops.CMat.from_host(seeded(port, 1, (B, K)), seeded(port, 2, (B, K)))
+    w = ops.CMat.from_host(seeded(port, 3, (N, K)), seeded(port, 4, (N, K)))
+    base = seeded(port, 9, (B, W))
+    hw = ops.CMat(ops.Plane.from_host(base), ops.Plane.from_host(base))
+    yw = ops.CMat(ops.Plane.from_host(base), ops.Plane.from_host(base))
+    ops.linear_gelu_fwd(x, w, hw.sub(8, N), yw.sub(8, N))
+    h0, y0 = ops.CMat.empty(B, N), ops.CMat.empty(B, N)
+    ops.linear_fwd(x, w, h0)
+    ops.gelu_fwd(h0, y0)
+    mask = np.ones(W, bool); mask[8:8 + N] = False
+    for wide, want in ((hw, h0), (yw, y0)):
+        for plane, ref in zip((wide.re.owner.download(), wide.im.owner.download()), want.host()):
+            assert np.array_equal(plane[:, 8:8 + N], ref) and np.array_equal(plane[:, mask], base[:, mask])
+
+
+@pytest.mark.parametrize("overrides", [
+    {"CNET_CGEMM_SKINNY": "0"},                            # small products on the block kernels (cut along K)
+    {"CNET_CGEMM_TILE": "0", "CNET_CGEMM_COLSPLIT": "0"},  # 128 x 128 blocks
+    {"CNET_CGEMM_TILE": "3", "CNET_CGEMM_TAIL": "1"},      # 64 x 64 blocks, tail blocks cut along K whenever possible
+])
+def test_fused_layers_under_other_kernel_choices(gpu, overrides):
+    """The tests of this file again in a process whose tuning overrides (read once per process) send the same shapes to
+    other kernels: every epilogue and both partial-sum kernels apply the activation."""
+    if os.environ.get("CNET_TEST_INNER"):
+        pytest.skip("already the inner run")
+    env = dict(os.environ, CNET_TEST_INNER="1", **overrides)
+    r = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-m", "gpu"], env=env,
+                       capture_output=True, text=True, timeout=280, cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-2000:]
