@@ -87,6 +87,7 @@ SIGNATURES = {
     "cnet_crelu_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_residual_bwd_sym": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_residual_bwd_sym2": [c_fp, c_fp, _l, c_fp, c_fp, _l] + [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
+    "cnet_residual_cgelu_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l] + ([c_fp] * 4 + [_l]) * 3 + [_i, _i],
     "cnet_l2norm_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_l2out_bwd_sym": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_cross_entropy_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp] + [c_fp] * 4 + [_l, _i, _i],

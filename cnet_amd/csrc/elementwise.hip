@@ -564,6 +564,43 @@ __global__ __launch_bounds__(TPB) void residual_bwd_sym2_kernel(const float *__r
 	out_pair<V, NT>(dv, row * lddv + col, o_r, o_i, 0);
 }
 
+// A Residual one of whose operands is the result of a CGelu: the gradient of the Residual (g1, plus g2 when it feeds two
+// consumers, added as residual_bwd_sym2_kernel adds them) goes to the other operand (du) and, optionally, to the CGelu's
+// result (dv); its CGelu backward at h, the CGelu's operand, goes to dh with the arithmetic of gelu_bwd_sym_kernel.  The
+// gradient of the CGelu's result is not read back: 40 bytes per complex element (32 with one consumer) against 32 + 24.
+template <int V, bool NT, bool TWO>
+__global__ __launch_bounds__(TPB) void residual_gelu_bwd_sym_kernel(const float *__restrict__ g1_re, const float *__restrict__ g1_im,
+		long ldg1, const float *__restrict__ g2_re, const float *__restrict__ g2_im, long ldg2, const float *__restrict__ hr,
+		const float *__restrict__ hi, long ldh, Pair2 du, long lddu, Pair2 dv, long lddv, Pair2 dh, long lddh, int rows, int cols) {
+	CNET_ELEM_INDEX();
+	float o_r[V], o_i[V], a[V], b[V];
+	ldv<V, NT>(o_r, g1_re + row * ldg1 + col);
+	ldv<V, NT>(o_i, g1_im + row * ldg1 + col);
+	if (TWO) {
+		float p_r[V], p_i[V];
+		ldv<V, NT>(p_r, g2_re + row * ldg2 + col);
+		ldv<V, NT>(p_i, g2_im + row * ldg2 + col);
+#pragma unroll
+		for (int k = 0; k < V; ++k) {
+			o_r[k] += p_r[k];
+			o_i[k] += p_i[k];
+		}
+	}
+	ldv<V, NT>(a, hr + row * ldh + col);
+	ldv<V, NT>(b, hi + row * ldh + col);
+	out_pair<V, NT>(du, row * lddu + col, o_r, o_i, 0);
+	if (dv.dz_re) out_pair<V, NT>(dv, row * lddv + col, o_r, o_i, 0);
+#pragma unroll
+	for (int k = 0; k < V; ++k) {
+		const float px = 0.5f * gelu_slope(a[k]), py = 0.5f * gelu_slope(b[k]);
+		const float sm = px + py, df = px - py;
+		const float q_r = o_r[k] * sm + o_r[k] * df, q_i = o_i[k] * sm + (-o_i[k]) * df;
+		o_r[k] = q_r;
+		o_i[k] = q_i;
+	}
+	out_pair<V, NT>(dh, row * lddh + col, o_r, o_i, 0);
+}
+
 // The gradient that reaches a Hadamard through a CGelu on its result, formed in place: h = u .* v is recomputed (the bits
 // of the forward pass), g becomes the CGelu backward of g at h (the arithmetic of gelu_bwd_sym_kernel), and is stored to
 // dh, the gradient planes of the CGelu's operand, which stay readable (skipped when dh.dz_re is NULL).
@@ -1349,6 +1386,35 @@ int cnet_residual_bwd_sym2(const float *g1_dz_re, const float *g1_dz_im, int64_t
 		if (gelu) hipLaunchKernelGGL((kernel<1, false, true>), __VA_ARGS__);  \
 		else hipLaunchKernelGGL((kernel<1, false, false>), __VA_ARGS__);     \
 	} while (0)
+
+int cnet_residual_cgelu_bwd_sym(const float *g1_dz_re, const float *g1_dz_im, int64_t ldg1, const float *g2_dz_re, const float *g2_dz_im,
+		int64_t ldg2, const float *h_re, const float *h_im, int64_t ldh, float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im,
+		int64_t lddu, float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv, float *dh_dz_re, float *dh_dz_im,
+		float *dh_dzs_re, float *dh_dzs_im, int64_t lddh, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
+	if (!rows || !cols) return CNET_OK;
+	const Pair2 du = pair_of(du_dz_re, du_dz_im, du_dzs_re, du_dzs_im), dv = pair_of(dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im),
+			dh = pair_of(dh_dz_re, dh_dz_im, dh_dzs_re, dh_dzs_im);
+	const bool two = g2_dz_re != nullptr, with_dv = dv_dz_re != nullptr;
+	CNET_CHECK_ARG(g1_dz_re && g1_dz_im && h_re && h_im && (g2_dz_re == nullptr) == (g2_dz_im == nullptr));
+	CNET_CHECK_PAIR(du);
+	CNET_CHECK_PAIR(dh);
+	if (with_dv) CNET_CHECK_PAIR(dv);
+	else CNET_CHECK_ARG(!dv_dz_im && !dv_dzs_re && !dv_dzs_im);
+	CNET_CHECK_ARG(ldg1 >= cols && (!two || ldg2 >= cols) && ldh >= cols && lddu >= cols && (!with_dv || lddv >= cols) && lddh >= cols);
+	const bool nt = streaming(4 + (two ? 2 : 0) + pair_planes(du) + (with_dv ? pair_planes(dv) : 0) + pair_planes(dh), (long) rows * cols);
+	if (all_mult4({cols, ldg1, two ? ldg2 : 0, ldh, lddu, with_dv ? lddv : 0, lddh}) &&
+			all_aligned({g1_dz_re, g1_dz_im, g2_dz_re, g2_dz_im, h_re, h_im, du_dz_re, du_dz_im, du_dzs_re, du_dzs_im, dv_dz_re, dv_dz_im,
+					dv_dzs_re, dv_dzs_im, dh_dz_re, dh_dz_im, dh_dzs_re, dh_dzs_im}))
+		CNET_LAUNCH_V4G(residual_gelu_bwd_sym_kernel, nt, two, CNET_GRID_2D(4), g1_dz_re, g1_dz_im, ldg1, g2_dz_re, g2_dz_im, ldg2, h_re, h_im,
+				ldh, du, lddu, dv, lddv, dh, lddh, rows, cols);
+	else
+		CNET_LAUNCH_V1G(residual_gelu_bwd_sym_kernel, two, CNET_GRID_2D(1), g1_dz_re, g1_dz_im, ldg1, g2_dz_re, g2_dz_im, ldg2, h_re, h_im, ldh,
+				du, lddu, dv, lddv, dh, lddh, rows, cols);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
 
 // gelu: the incoming gradient belongs to a CGelu applied to the Hadamard's result; dh receives the gradient of that CGelu's
 // operand

@@ -380,6 +380,12 @@ protected:
 	// 1, its backward pass runs as usual.
 	CFunc *fused_next_ = NULL;
 	int fused_prev_ = 0;
+	// A Residual one of whose operands (slot fused_gelu_slot_) is a CGelu that feeds nothing else runs the CGelu's backward
+	// pass inside its own (cnet_residual_cgelu_bwd_sym) under conjugate gradient pairs; bwd_by_consumer_ of the CGelu is
+	// set.  The gradient of that operand equals the gradient of the other one and is not stored a second time: fetch()
+	// reads it from there.
+	int fused_gelu_slot_ = -1;
+	bool bwd_by_consumer_ = false;
 	int rows_ = 0;           // batch rows of this node's output (1 for parameter nodes)
 	float *out_ = NULL;      // 2 planes [rows][out_size]: what consumers read
 	float *out_re() const { return out_; }
@@ -990,6 +996,8 @@ private:
 		for (auto f : func_list_) {
 			f->fused_next_ = NULL;
 			f->fused_prev_ = 0;
+			f->fused_gelu_slot_ = -1;
+			f->bwd_by_consumer_ = false;
 		}
 		if (!fuse_layers_) return;
 		for (auto f : func_list_) {
@@ -1002,6 +1010,18 @@ private:
 			if (t == isHadamard && g->no_outputs() != 1) continue;
 			f->fused_next_ = g;
 			g->fused_prev_ = t == isHadamard ? 2 : 1;
+		}
+		for (auto f : func_list_) {
+			if (f->typeId() != isResidual || f->no_outputs() < 1 || f->no_outputs() > 2) continue;
+			if (f->slots_[0].rows != f->rows_ || f->slots_[1].rows != f->rows_) continue;
+			for (int k = 0; k < 2 && f->fused_gelu_slot_ < 0; ++k) {
+				CFunc *g = f->slots_[k].producer;
+				if (!g || g->typeId() != isGelu || g->no_outputs() != 1 || g->fused_prev_ == 2 || g->rows_ != f->rows_ ||
+						f->slots_[1 - k].producer == g || f->slots_[k].offset != 0 || g->out_size_ != f->out_size_)
+					continue;
+				f->fused_gelu_slot_ = k;
+				g->bwd_by_consumer_ = true;
+			}
 		}
 	}
 
@@ -1149,6 +1169,18 @@ private:
 		// Gradients flow only towards input functions that are stepped: a layer none of whose operands leads to one is
 		// skipped (all input functions are trainable unless CNet::setInputTrainable said otherwise, as upstream has it).
 		if (!f->wants_grad_) return;
+		if (t == isResidual && conjugate_gradients_ && f->fused_gelu_slot_ >= 0) {
+			// one operand is a CGelu that feeds nothing else: its backward pass in the same kernel
+			const int k = f->fused_gelu_slot_;
+			CFunc *g = f->slots_[k].producer;
+			CFunc::Slot &u0 = upstream(f, 0), &a = f->slots_[1 - k], &h = g->slots_[0];
+			CFunc::Slot *u1 = f->no_outputs() == 2 ? &upstream(f, 1) : NULL;
+			const int n = f->out_size_;
+			ck(cnet_residual_cgelu_bwd_sym(u0.g(0), u0.g(1), u0.len, u1 ? u1->g(0) : NULL, u1 ? u1->g(1) : NULL, u1 ? u1->len : 0, zre(g, 0),
+					zim(g, 0), n, a.g(0), a.g(1), a.gs(2), a.gs(3), n, NULL, NULL, NULL, NULL, 0, h.g(0), h.g(1), h.gs(2), h.gs(3), n, rows, n),
+					"cnet_residual_cgelu_bwd_sym");
+			return;
+		}
 		if (t == isResidual && conjugate_gradients_ && f->no_outputs() == 2 && f->slots_[0].rows == rows && f->slots_[1].rows == rows) {
 			// a Residual feeding two consumers (the usual skip connection): both incoming gradients in one pass
 			CFunc::Slot &u0 = upstream(f, 0), &u1 = upstream(f, 1), &a = f->slots_[0], &v = f->slots_[1];
@@ -1228,7 +1260,7 @@ private:
 				break;
 			}
 			case isGelu:
-				if (conjugate_gradients_ && f->fused_prev_ == 2) break;  // done by the Hadamard below it
+				if (conjugate_gradients_ && (f->fused_prev_ == 2 || f->bwd_by_consumer_)) break;  // done by the Hadamard below it or the Residual above it
 				if (conjugate_gradients_) {
 					ck(cnet_cgelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,
 							acc), "cnet_cgelu_bwd_sym");
@@ -1343,9 +1375,12 @@ public:
 			}
 			ck(cnet_memcpy_d2h(v->real_ + s.offset, z_re, s.len * sizeof(float)), "cnet_memcpy_d2h");
 			ck(cnet_memcpy_d2h(v->imag_ + s.offset, z_im, s.len * sizeof(float)), "cnet_memcpy_d2h");
+			// the gradient of a Residual's CGelu operand is kept once, in the planes of the other operand (see fused_gelu_slot_)
+			const bool alias = conjugate_gradients_ && f->fused_gelu_slot_ >= 0 && &s == &f->slots_[f->fused_gelu_slot_];
+			const CFunc::Slot &gsrc = alias ? f->slots_[1 - f->fused_gelu_slot_] : s;
 			for (int p = 0; p < 4; ++p)
-				ck(cnet_memcpy_d2h(v->plane(2 + p) + s.offset, s.g(p) + (size_t) row * s.len, s.len * sizeof(float)), "cnet_memcpy_d2h");
-			if (conjugate_gradients_ && !s.star_on_device) {
+				ck(cnet_memcpy_d2h(v->plane(2 + p) + s.offset, gsrc.g(p) + (size_t) row * s.len, s.len * sizeof(float)), "cnet_memcpy_d2h");
+			if (conjugate_gradients_ && !gsrc.star_on_device) {
 				// the pair is conjugate and nothing on the device reads its dz* half: it is formed here
 				const float *dz_re = v->plane(2) + s.offset, *dz_im = v->plane(3) + s.offset;
 				float *dzs_re = v->plane(4) + s.offset, *dzs_im = v->plane(5) + s.offset;

@@ -263,6 +263,14 @@ def residual_bwd_sym2(g1, g2, du, dv, accumulate=0, mirror=True):
          g1.rows, g1.cols, accumulate)
 
 
+def residual_gelu_bwd_sym(g1, g2, h, du, dv, dh, mirror=True):
+    """g2 and dv may be None (one consumer; the gradient of the CGelu's result not wanted)."""
+    p2 = g2.p()[:2] if g2 is not None else (None, None)
+    pv = _pair(dv, mirror) if dv is not None else (None,) * 4
+    call("cnet_residual_cgelu_bwd_sym", *g1.p()[:2], g1.ld, *p2, g2.ld if g2 is not None else 0, *h.p(), h.ld, *_pair(du, mirror),
+         du.ld, *pv, dv.ld if dv is not None else 0, *_pair(dh, mirror), dh.ld, g1.rows, g1.cols)
+
+
 def l2norm_bwd_sym(z, s, g, dz, accumulate=0, mirror=True):
     call("cnet_l2norm_bwd_sym", *z.p(), z.ld, s.ptr, *g.p()[:2], g.ld, *_pair(dz, mirror), dz.ld, z.rows, z.cols, accumulate)
 

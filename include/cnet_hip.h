@@ -356,6 +356,20 @@ int cnet_residual_bwd_sym2(const float *g1_dz_re, const float *g1_dz_im, int64_t
                            float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
                            float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
                            int rows, int cols, int accumulate);
+/* A Residual one of whose operands is the result of a CGelu, both backward passes in one (gpu_residual_backward +
+ * gpu_gelu_backward, gpu/kernels.cpp:170-202, 302-360; CPU twins impl/residual.h:56-77, impl/relu.h:144-166).  g1 (and g2,
+ * or NULL for both of its planes: the Residual then feeds one consumer) is the gradient pair that reaches the Residual;
+ * du, the gradient of its other operand, receives g1 + g2; dv, the gradient of the CGelu's result, receives the same when
+ * its planes are given (all four NULL: nobody reads it); dh, the gradient of the CGelu's operand h, receives the CGelu
+ * backward of g1 + g2 at h.  All assigned.  The bits of cnet_residual_bwd_sym2 (or _sym) followed by cnet_cgelu_bwd_sym;
+ * 40 bytes per complex element (32 with one consumer) instead of 56 (48). */
+int cnet_residual_cgelu_bwd_sym(const float *g1_dz_re, const float *g1_dz_im, int64_t ldg1,
+                                const float *g2_dz_re, const float *g2_dz_im, int64_t ldg2,
+                                const float *h_re, const float *h_im, int64_t ldh,
+                                float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
+                                float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
+                                float *dh_dz_re, float *dh_dz_im, float *dh_dzs_re, float *dh_dzs_im, int64_t lddh,
+                                int rows, int cols);
 int cnet_l2norm_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, const float *s,
                         const float *g_dz_re, const float *g_dz_im, int64_t ldg,
                         float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,

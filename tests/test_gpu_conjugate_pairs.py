@@ -185,6 +185,32 @@ def test_hadamard_followed_by_cgelu_in_one_pass(gpu, port, B, n):
                 assert np.array_equal(hg[2], keep[2]) and np.array_equal(hg[3], keep[3]), ("dz* was written", shared)
 
 
+@pytest.mark.parametrize("B,n", ELEMENTWISE + [(2048, 2048)])
+def test_residual_and_cgelu_backward_in_one_pass(gpu, port, B, n):
+    """cnet_residual_cgelu_bwd_sym against cnet_residual_bwd_sym2 (or _sym) followed by cnet_cgelu_bwd_sym: equal bits in du, dv
+    and dh, with one and two consumers, with and without the planes of dv and the dz* planes."""
+    g1 = ops.Grad.from_host(_pair(port, 13 * B + n, (B, n)))
+    g2 = ops.Grad.from_host(_pair(port, 17 * B + n, (B, n)))
+    h = ops.CMat.from_host(seeded(port, 1, (B, n), 2.0), seeded(port, 2, (B, n), 2.0))
+    for two in (True, False):
+        fu, fv, fh = (ops.Grad.empty(B, n) for _ in range(3))
+        if two:
+            ops.residual_bwd_sym2(g1, g2, fu, fv)
+        else:
+            ops.residual_bwd_sym(g1, fu, fv)
+        ops.gelu_bwd_sym(h, fv, fh)
+        su, sv, sh = (ops.Grad.from_host(_pair(port, 90 + k, (B, n))) for k in range(3))
+        ops.residual_gelu_bwd_sym(g1, g2 if two else None, h, su, sv, sh)
+        _exact(fu, su, ("du", two)); _exact(fv, sv, ("dv", two)); _exact(fh, sh, ("dh", two))
+        keep = _pair(port, 91, (B, n))
+        nu, nh = ops.Grad.from_host(keep), ops.Grad.from_host(keep)
+        ops.residual_gelu_bwd_sym(g1, g2 if two else None, h, nu, None, nh, mirror=False)
+        for got, want in ((nu, fu), (nh, fh)):
+            hg, hw = got.host(), want.host()
+            assert np.array_equal(hg[0], hw[0]) and np.array_equal(hg[1], hw[1]), ("dz", two)
+            assert np.array_equal(hg[2], keep[2]) and np.array_equal(hg[3], keep[3]), ("dz* was written", two)
+
+
 @pytest.mark.parametrize("B,n", [(3, 6), (64, 10), (5, 1024), (3, 2048), (4, 3000), (2, 4100), (2, 5001), (2, 32768)])
 def test_loss_and_softmax_backward_of_a_conjugate_pair(gpu, port, B, n):
     """SoftMax (every row kernel: registers, two-pass, scalar), L2Out and CrossEntropy: one-gradient entry points against
