@@ -100,20 +100,29 @@ __device__ __forceinline__ float ordered_sum(const float *__restrict__ first, lo
 	return s;
 }
 
-// tanh-GELU of one real plane value and its derivative (impl/relu.h:119-131, 144-166 upstream); shared by the elementwise
-// kernels and the matrix-product epilogue that applies the CGelu of a Linear's result, so both give the same bits
-__device__ __forceinline__ float gelu_value(float t) {
+// tanh-GELU of one real plane value and its derivative (impl/relu.h:119-131 upstream); shared by the elementwise kernels
+// and the matrix-product epilogue that applies the CGelu of a Linear's result, so both give the same bits.
+// With a = sqrt(2/pi) (t + 0.044715 t^3) and e = exp(-2a): (1 + tanh a)/2 = 1/(1 + e) and 1/(2 cosh^2 a) = 2e/(1 + e)^2,
+// so one hardware exponential and one reciprocal (about 1 ulp each) stand in for tanhf and coshf of the CPU path, without
+// the cancellation of 1 + tanh a for negative a.  a is kept above -43 so that e stays finite (e = inf would give inf * 0).
+__device__ __forceinline__ float gelu_gate(float t, float &e) {
 	const float c = 0.7978845608028654f;  // sqrt(2/pi)
-	float arg = c * (t + 0.044715f * t * t * t);
-	return 0.5f * t * (1.0f + tanhf(arg));
+	const float arg = fmaxf(c * (t + 0.044715f * t * t * t), -43.0f);
+	e = __builtin_amdgcn_exp2f(-2.8853900817779268f * arg);  // exp(-2 arg) = 2^(-2 log2(e) arg)
+	return __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+__device__ __forceinline__ float gelu_value(float t) {
+	float e;
+	return t * gelu_gate(t, e);
 }
 
 __device__ __forceinline__ float gelu_slope(float t) {
 	const float c = 0.7978845608028654f;
-	float arg = c * (t + 0.044715f * t * t * t);
-	float th = tanhf(arg);
-	float sech2 = 1.0f - th * th;  // = 1/cosh^2
-	return 0.5f * (1.0f + th) + t * 0.5f * sech2 * c * (1.0f + 3.0f * 0.044715f * t * t);
+	float e;
+	const float sig = gelu_gate(t, e);
+	const float half_sech2 = 2.0f * ((e * sig) * sig);
+	return sig + t * half_sech2 * c * (1.0f + 3.0f * 0.044715f * t * t);
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
