@@ -386,6 +386,14 @@ protected:
 	// reads it from there.
 	int fused_gelu_slot_ = -1;
 	bool bwd_by_consumer_ = false;
+	// Input functions with one consumer: the dz* of a backward pass is not added to the node's own planes at once.  While
+	// those planes are clear (grad_clean_: nothing gathered since the last update) the gradient stays where the consumer's
+	// backward pass wrote it (pending_), and the update reads it from there, which saves a pass that adds it to zeros and
+	// the pass that clears it again.  Anything that looks at the node's planes or overwrites the consumer's first brings
+	// them up to date (CNet::flushPending).  defer_now_ is the decision for the pass that is being queued.
+	Slot *pending_ = NULL;
+	bool grad_clean_ = false;
+	bool defer_now_ = false;
 	int rows_ = 0;           // batch rows of this node's output (1 for parameter nodes)
 	float *out_ = NULL;      // 2 planes [rows][out_size]: what consumers read
 	float *out_re() const { return out_; }
@@ -658,6 +666,53 @@ class CNet {
 		gather_len_.clear();
 		ck(rc, "cnet_add_multi");
 	}
+	// ---- deferred gathers of the input functions (see CFunc::pending_) ----
+	bool defer_gathers_ = true;
+	static bool deferrable(CFunc *f) { return f->typeId() == isInput && f->trainable_ && f->no_outputs() == 1; }
+	// adds every gradient that is still with a consumer to its input function's own planes, as the backward pass would have
+	void flushPending() {
+		std::vector<const float *> src;
+		std::vector<float *> dst;
+		std::vector<int64_t> len;
+		for (auto f : inputs_) {
+			if (!f->pending_) continue;
+			CFunc::Slot &own = f->slots_[0];
+			src.push_back(f->pending_->g(2));
+			dst.push_back(own.g(2));
+			len.push_back(2 * (int64_t) own.rows * own.len);
+			f->pending_ = NULL;
+			f->grad_clean_ = false;
+		}
+		if (!src.empty()) ck(cnet_add_multi((int) src.size(), src.data(), dst.data(), len.data()), "cnet_add_multi");
+	}
+	// decides, for the backward pass about to be queued, which input functions leave their gradient with the consumer;
+	// true when every candidate does (the state a recorded backward pass stands for)
+	bool planDeferral(bool allow) {
+		bool all = true;
+		for (auto f : inputs_) {
+			f->defer_now_ = allow && defer_gathers_ && deferrable(f) && f->grad_clean_ && !f->pending_;
+			if (deferrable(f) && !f->defer_now_) all = false;
+		}
+		return all;
+	}
+	// after the pass has been queued (or replayed): note where the gradients are
+	void noteDeferred() {
+		for (auto f : inputs_) {
+			if (f->defer_now_) f->pending_ = &upstream(f, 0);
+			else if (f->trainable_ && f->no_outputs() > 0) f->grad_clean_ = false;
+			f->defer_now_ = false;
+		}
+	}
+	bool allPending() const {
+		for (auto f : inputs_)
+			if (deferrable(f) && !f->pending_) return false;
+		return true;
+	}
+	bool allCleanNonePending() const {
+		for (auto f : inputs_)
+			if (deferrable(f) && (!f->grad_clean_ || f->pending_)) return false;
+		return true;
+	}
 	SimpleRand rand_{(uint64_t) clock()};  // upstream ComplexNet::rand_ (impl/cnet.h:56): the coin of sample()
 	bool input_dz_dirty_ = false;  // the dz planes of the input functions hold a first moment
 	// data inputs whose batch is still travelling on the upload stream (gpuSetInput): the compute stream waits for the
@@ -860,6 +915,8 @@ public:
 			f->slots_.clear();
 			f->out_ = NULL;
 			f->rows_ = 0;
+			f->pending_ = NULL;
+			f->grad_clean_ = false;
 		}
 		batch_ = 0;
 		d_labels_ = NULL;
@@ -983,6 +1040,10 @@ private:
 				sl.star_on_device = reads;
 			}
 		planFusion();
+		for (auto f : inputs_) {  // the gradient planes were cleared above
+			f->pending_ = NULL;
+			f->grad_clean_ = true;
+		}
 		d_labels_ = dalloc<int32_t>(batch_);
 		ck(cnet_memset_zero(d_labels_, batch_ * sizeof(int32_t)), "zero");
 		if (main_input_->typeId() == isInput) {
@@ -1148,6 +1209,7 @@ private:
 			// consumer.  Nothing in the backward pass reads what an input function gathers, so the gathers of all of them
 			// wait for the end of the pass and go out as one launch (flushGathers).
 			CFunc::Slot &own = f->slots_[0];
+			if (f->defer_now_) return;  // the update will read the consumer's planes (see pending_)
 			for (int c = 0; c < f->no_outputs(); ++c) {
 				CFunc::Slot &u = upstream(f, c);
 				if (c) flushGathers();  // one launch must not hold two additions into the same planes
@@ -1364,6 +1426,7 @@ public:
 	void fetch(CFunc *f, int b) {
 		requireAllocated("fetch");
 		if (b < 0 || b >= batch_) throw std::out_of_range("fetch: batch index");
+		if (f->pending_) flushPending();
 		settleUploads();
 		ck(cnet_sync(), "cnet_sync");
 		Vars *v = f->mutable_input();
@@ -1442,7 +1505,9 @@ public:
 			}
 			use_graphs_ = was;
 		};
-		if (input_dz_dirty_ || !g.step_warm) {  // an update that also clears a first moment is not what a recording replays
+		// an update that also clears a first moment is not what a recording replays, nor is a step that finds gradients of
+		// an earlier backward pass waiting for their update
+		if (input_dz_dirty_ || !g.step_warm || !allCleanNonePending()) {
 			eager();
 			g.step_warm = true;
 			return;
@@ -1615,13 +1680,19 @@ public:
 		requireAllocated("gpuBackward");
 		settleUploads();
 		planGradients();
-		runPhase(1, graphs_[active_].bwd, [&] {
+		flushPending();  // this pass overwrites the planes a deferred gradient sits in
+		const bool nominal = planDeferral(true);
+		auto body = [&] {
 			gather_src_.clear();  // nothing is left over from a pass that threw
 			gather_dst_.clear();
 			gather_len_.clear();
 			for (int k = (int) func_list_.size() - 1; k >= 0; --k) nodeBackward(func_list_[k], true);
 			flushGathers();
-		});
+		};
+		// a recording stands for the usual state (every gradient deferred); a second pass before an update runs as it is
+		if (nominal) runPhase(1, graphs_[active_].bwd, body);
+		else body();
+		noteDeferred();
 		return true;
 	}
 	// z -= l_rate * dzs on every input function (the data input too, impl/cnet.h:413-421), then its gradients are cleared
@@ -1640,26 +1711,38 @@ public:
 					ck(cnet_graph_destroy(sg.upd), "cnet_graph_destroy");
 					sg.upd = NULL;
 				}
-		runPhase(2, g.upd, [&] {
-			// every input function in one launch; their dz planes only hold something after an Adam-style step (its
-			// first moment), so they are cleared only then
-			std::vector<float *> zr, zi, dr, di;
-			std::vector<int64_t> len;
-			for (auto f : inputs_) {
-				if (!f->trainable_) continue;
-				CFunc::Slot &s = f->slots_[0];
-				const size_t n = (size_t) s.rows * s.len;
-				zr.push_back(s.z);
-				zi.push_back(s.z + n);
-				dr.push_back(s.g(2));
-				di.push_back(s.g(3));
-				len.push_back((int64_t) n);
-				if (input_dz_dirty_) ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
+		auto body = [&] {
+			// every input function in one launch (two when some gradients are still with their consumers: those are read
+			// there and nothing has to be cleared); the dz planes only hold something after an Adam-style step (its first
+			// moment), so they are cleared only then
+			for (int deferred = 0; deferred < 2; ++deferred) {
+				std::vector<float *> zr, zi, dr, di;
+				std::vector<int64_t> len;
+				for (auto f : inputs_) {
+					if (!f->trainable_ || (f->pending_ != NULL) != (deferred != 0)) continue;
+					CFunc::Slot &s = f->slots_[0];
+					const CFunc::Slot &gsrc = deferred ? *f->pending_ : s;
+					const size_t n = (size_t) s.rows * s.len;
+					zr.push_back(s.z);
+					zi.push_back(s.z + n);
+					dr.push_back(gsrc.g(2));
+					di.push_back(gsrc.g(3));
+					len.push_back((int64_t) n);
+					if (input_dz_dirty_) ck(cnet_memset_zero(s.g(0), 2 * n * sizeof(float)), "zero");
+				}
+				if (zr.empty()) continue;
+				ck(cnet_sgd_update_multi((int) zr.size(), zr.data(), zi.data(), dr.data(), di.data(), len.data(), l_rate, deferred ? 0 : 1),
+						"cnet_sgd_update_multi");
 			}
-			if (zr.empty()) return;
-			ck(cnet_sgd_update_multi((int) zr.size(), zr.data(), zi.data(), dr.data(), di.data(), len.data(), l_rate, 1),
-					"cnet_sgd_update_multi");
-		});
+		};
+		// a recording stands for the usual state: every gradient that can be is still with its consumer
+		if (allPending()) runPhase(2, g.upd, body);
+		else body();
+		for (auto f : inputs_) {
+			if (!f->trainable_) continue;
+			f->pending_ = NULL;
+			f->grad_clean_ = true;
+		}
 		input_dz_dirty_ = false;
 	}
 	// Replay the kernels of GpuForward / gpuBackward / gpuUpdateInputs from recorded graphs instead of launching them
@@ -1694,6 +1777,17 @@ public:
 		}
 	}
 	bool fusingLayers() const { return fuse_layers_; }
+	// An input function with one consumer leaves the gradient of a backward pass in that consumer's planes until the update
+	// reads it there (nothing is added to cleared planes and cleared again).  Off: every backward pass adds it to the input
+	// function's own planes at once, as upstream does.  Same weights to the bit either way.
+	void deferGathers(bool on) {
+		if (on == defer_gathers_) return;
+		if (batch_) {
+			dropGraphs();
+			flushPending();
+		}
+		defer_gathers_ = on;
+	}
 	// Upstream steps every input function, the data input included (impl/cnet.h:413-421), and therefore runs the backward
 	// pass all the way down to it.  An input function marked not trainable is left alone by gpuUpdateInputs /
 	// gpuAdamUpdate, gathers nothing, and the backward products that would only serve it are not computed (for the
@@ -1702,7 +1796,10 @@ public:
 	void setInputTrainable(InputFunc *inp, bool on) {
 		CFunc *f = dynamic_cast<CFunc *>(inp);
 		if (!f || !f->is_input_) throw std::invalid_argument("setInputTrainable: not an input function of this net");
-		if (f->trainable_ != on && batch_) dropGraphs();
+		if (f->trainable_ != on && batch_) {
+			dropGraphs();
+			flushPending();
+		}
 		f->trainable_ = on;
 	}
 	// The Adam-style step of upstream GpuNet::adamUpdate (gpu/gpu_func.h:503-510, gpu/kernels.cpp:494-514) on every input
@@ -1714,7 +1811,11 @@ public:
 			CFunc::Slot &s = f->slots_[0];
 			const size_t n = (size_t) s.rows * s.len;
 			float *z = s.z;
-			ck(cnet_adam_update(z, z + n, s.g(0), s.g(1), s.g(2), s.g(3), (int64_t) n, l_rate, beta, t, 1), "cnet_adam_update");
+			const CFunc::Slot &gsrc = f->pending_ ? *f->pending_ : s;  // a gradient still with its consumer is read there
+			ck(cnet_adam_update(z, z + n, s.g(0), s.g(1), gsrc.g(2), gsrc.g(3), (int64_t) n, l_rate, beta, t, f->pending_ ? 0 : 1),
+					"cnet_adam_update");
+			f->pending_ = NULL;
+			f->grad_clean_ = true;
 		}
 		input_dz_dirty_ = true;
 	}
@@ -1866,6 +1967,7 @@ public:
 		copyInputsToGpu();
 		// upstream forward() clears the gradients of every non-input function (impl/cnet.h:372-374); the batched path
 		// never needs that (first contribution overwrites), the per-sample views do
+		flushPending();  // before the planes a deferred gradient sits in are cleared
 		for (auto f : func_list_)
 			if (!f->is_input_)
 				for (auto &s : f->slots_) ck(cnet_memset_zero(s.grad, 4 * (size_t) s.rows * s.len * sizeof(float)), "zero");
@@ -1879,11 +1981,14 @@ public:
 		// the device-side loss, which is refreshed here so getLoss() matches the label in use
 		for (auto f : outputs_)
 			if (f->typeId() == isCrossEntropy) nodeForward(f);
+		flushPending();
+		planDeferral(false);  // every host view is read right after the pass: nothing to gain from deferring
 		gather_src_.clear();
 		gather_dst_.clear();
 		gather_len_.clear();
 		for (int k = (int) func_list_.size() - 1; k >= 0; --k) nodeBackward(func_list_[k], label >= 0);
 		flushGathers();
+		noteDeferred();
 		fetchAll(0);
 	}
 	void backward() { backward(-1); }

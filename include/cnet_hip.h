@@ -292,7 +292,7 @@ int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols
  * harnesses that forbid hipMalloc); it has no counterpart upstream.  Same arguments, same kernels and bit-identical
  * results; the partial sums of its first stage go to a 2 MiB array that is part of the library's image on each device
  * instead of the library workspace, so the call never allocates or frees.  Limit: slabs x cols <= 524288 floats, which
- * holds for every cols <= 524288 (slabs = min(256, 4 x compute units / ceil(cols / 256)), at most rows / 4); beyond it
+ * holds for every cols <= 524288 (slabs = min(256, w x compute units / ceil(cols / 256)), w = 8 for planes of 2^24 elements and more, else 4; at most rows / 4); beyond it
  * the call returns CNET_ERR_UNSUPPORTED.  All calls on one device share the array: calls that overlap in time (two
  * streams, two host threads) race. */
 int cnet_batch_sum_noalloc(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate);

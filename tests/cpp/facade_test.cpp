@@ -10,6 +10,7 @@
 //   facade_test adam               TriangFourier / CRelu net trained with the Adam-style step, batched and per sample
 //   facade_test saved_model <golden dir> <scratch dir>   upstream-written .mod files restored and run on the device
 //   facade_test pipeline [B steps]  reader -> page-locked batches -> device, with and without gpuPrefetch (same bits)
+//   facade_test deferred           gradients of the input functions left with their consumers until the update (same bits)
 //   facade_test upstream_nets      the nets of upstream's own GPU tests (E2E chain, fan-out into one consumer, ...)
 //   facade_test errors             error behaviour
 //   facade_test stack8 n blocks B steps lr rows overflow|finite [learn]   residual stack of `blocks` blocks against the
@@ -894,7 +895,8 @@ static void test_pipeline(int B, int steps) {
 	// 6: prefetch, the loss of a step read one step later (gpuQueueLoss / getLoss(pending)); 7: the same with gpuTrainStep
 	// 8: as 6 with the data input marked not trainable (CNet::setInputTrainable: no step on it, no backward pass into it)
 	// 9: prefetch, one launch per layer (CNet::fuseLayers(false): Hadamard and CGelu as separate passes)
-	constexpr int MODES = 10;
+	// 10: prefetch, every backward pass adds the gradients to the input functions' own planes at once (CNet::deferGathers(false))
+	constexpr int MODES = 11;
 	std::vector<float> losses[MODES];
 	std::vector<float> weights[MODES];
 	double ms[MODES] = {0};
@@ -915,6 +917,7 @@ static void test_pipeline(int B, int steps) {
 		if (mode == 5) net.conjugateGradients(false);
 		if (mode == 8) net.setInputTrainable(cin, false);
 		if (mode == 9) net.fuseLayers(false);
+		if (mode == 10) net.deferGathers(false);
 		net.sync();
 		auto t0 = std::chrono::steady_clock::now();
 		// With prefetch the host runs two batches ahead: while the device computes step s, batch s+1 (assembled during
@@ -1003,6 +1006,7 @@ static void test_pipeline(int B, int steps) {
 		expect("losses and weights identical with gpuTrainStep and the late read together", losses[0] == losses[7] && weights[0] == weights[7]);
 		expect("losses and weights identical with the data input not trainable", losses[0] == losses[8] && weights[0] == weights[8]);
 		expect("losses and weights identical with one launch per layer (no fused Hadamard + CGelu)", losses[0] == losses[9] && weights[0] == weights[9]);
+		expect("losses and weights identical with the gradients of the input functions gathered at once", losses[0] == losses[10] && weights[0] == weights[10]);
 		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
 		// dz* planes written as the conjugate of the dz product against dz* planes computed by a product of their own
 		double worst = 0, num = 0, den = 0;
@@ -1026,6 +1030,79 @@ static void test_pipeline(int B, int steps) {
 		   "\"upload_bytes_per_step\": %zu}\n",
 			B, steps, ms[0], ms[1], ms[2], ms[3], B / ms[0] * 1e3, B / ms[1] * 1e3, ms[2] > 0 ? B / ms[2] * 1e3 : 0.0, ms[4],
 			ms[4] > 0 ? B / ms[4] * 1e3 : 0.0, ms[5], ms[6], B / ms[6] * 1e3, ms[7], ms[8], ms[8] > 0 ? B / ms[8] * 1e3 : 0.0, (size_t) 2 * B * n * sizeof(float));
+}
+
+// ------------------------------------------------------------------------------------------------- deferred gathers
+// An input function with one consumer leaves its gradient with the consumer until the update.  Everything that could tell
+// the difference must not: two backward passes before one update (the input keeps adding, impl/cinput.h:54-65), a look at
+// the gradient between backward pass and update, an Adam-style step, recorded phases, a whole recorded step after a
+// backward pass that was never followed by an update.
+static void test_deferred_gathers() {
+	const int n = 96, classes = 10, B = 32;
+	if (cnet_init(0) != CNET_OK) {
+		expect("cnet_init", false);
+		return;
+	}
+	SyntheticReader data(n, 8 * B, classes);
+	std::vector<float> trace[4];
+	for (int variant = 0; variant < 4; ++variant) {  // 0: deferred, 1: gathered at once, 2: deferred + recorded phases, 3: gathered + recorded phases
+		CNet net;
+		int inp, outp;
+		build_readme(net, n, classes, &inp, &outp);
+		net.allocateOnGpu(B);
+		net.deferGathers(variant % 2 == 0);
+		if (variant >= 2) net.useGraphs(true);
+		CInput *cin = (CInput *) net[inp];
+		CrossEntropy *cen = (CrossEntropy *) net[outp];
+		SyntheticReader reader = data;
+		InputBatch batch(B, n);
+		std::vector<float> &out = trace[variant];
+		auto weights = [&] {
+			net.getInputsFromGpu();
+			for (auto f : net.inputs())
+				if (f != cin) out.insert(out.end(), f->input().real_, f->input().real_ + 2 * f->input().length_);
+		};
+		auto gradients = [&] {
+			for (auto f : net.inputs()) {
+				net.fetch(f, 1);
+				out.insert(out.end(), f->input().dz_star_real_, f->input().dz_star_real_ + 2 * f->input().length_);
+			}
+		};
+		auto step = [&](bool update) {
+			reader.nextBatch(batch);
+			net.gpuForward(cin, cen, batch);
+			net.gpuBackward();
+			if (update) net.gpuUpdateInputs(0.05f / B);
+			out.push_back(net.getLoss(cen, NULL));
+		};
+		for (int k = 0; k < 3; ++k) step(true);       // the usual loop (recorded from the second step on)
+		step(false);                                   // two backward passes ...
+		step(true);                                    // ... before one update
+		step(false);
+		gradients();                                   // a look at the gradients before the update
+		net.gpuUpdateInputs(0.05f / B);
+		gradients();                                   // cleared by the update
+		weights();
+		step(false);
+		net.gpuAdamUpdate(0.01f / B, 0.9f, 0);         // an Adam-style step takes the gradient from where it is
+		step(true);                                    // (this update also clears the first moment)
+		weights();
+		if (variant < 2) {                             // a whole recorded step, also right after a pass without update
+			reader.nextBatch(batch);
+			for (int k = 0; k < 3; ++k) net.gpuTrainStep(cin, cen, batch, 0.05f / B);
+			step(false);
+			net.gpuTrainStep(cin, cen, batch, 0.05f / B);
+			net.gpuTrainStep(cin, cen, batch, 0.05f / B);
+			out.push_back(net.getLoss(cen, NULL));
+			weights();
+		}
+	}
+	expect("deferred and immediate gathers: same losses, gradients and weights", trace[0] == trace[1] && trace[0].size() > 1000);
+	expect("the same with recorded phases", trace[2] == trace[3] && !trace[2].empty());
+	expect("recorded phases agree with launches one by one", std::equal(trace[2].begin(), trace[2].end(), trace[0].begin()));
+	bool finite = true;
+	for (float v : trace[0]) finite = finite && std::isfinite(v);
+	expect("all finite", finite);
 }
 
 // ------------------------------------------------------------------------------------------------- frozen data input
@@ -1432,6 +1509,7 @@ int main(int argc, char **argv) {
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
 		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12);
 		if (what == "frozen_input" || what == "all") test_frozen_input();
+		if (what == "deferred" || what == "all") test_deferred_gathers();
 		if (what == "upstream_nets" || what == "all") test_upstream_nets();
 		if (what == "errors" || what == "all") test_errors();
 		// stack8 n blocks B steps lr rows_checked overflow|finite [learn]

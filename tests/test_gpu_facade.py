@@ -86,6 +86,13 @@ def test_data_input_marked_not_trainable():
     assert "PASS" in out and "FAIL" not in out
 
 
+def test_gradients_of_input_functions_left_with_their_consumers_until_the_update():
+    """CNet::deferGathers: two backward passes before an update, a look at the gradients in between, an Adam-style step,
+    recorded phases and whole recorded steps give the bits of gathering at once."""
+    out = _run("deferred")
+    assert "FAIL" not in out and out.count("PASS") >= 4
+
+
 def test_nets_of_the_upstream_gpu_tests():
     out = _run("upstream_nets")
     assert "FAIL" not in out and out.count("PASS") >= 25
