@@ -185,6 +185,13 @@ def kernel_suite(steps):
         extra_bytes=16 * Cc)
     hbm("hadamard_bwd, conjugate pair (shared weights, dz only)", [R, Cc], 24, n,
         lambda: ops.hadamard_bwd_sym(u, w1, g, du, dw1, True, mirror=False), extra_bytes=8 * Cc)
+    # fused pairs of layers: one pass where two were, the intermediate values written but not read back
+    hbm("hadamard + cgelu fwd, one pass (shared weights; h and gelu(h) written)", [R, Cc], 24, n,
+        lambda: ops.hadamard_gelu_fwd(u, w1, yy, v, True), extra_bytes=8 * Cc)
+    hbm("cgelu_bwd + hadamard_bwd, one pass, conjugate pair (shared weights, dz only, dh not kept)", [R, Cc], 24, n,
+        lambda: ops.hadamard_gelu_bwd_sym(u, w1, g, None, du, dw1, True, mirror=False), extra_bytes=8 * Cc)
+    hbm("residual_bwd (two consumers) + cgelu_bwd, one pass, conjugate pair (dz only)", [R, Cc], 40, n,
+        lambda: ops.residual_gelu_bwd_sym(g, dv, u, du, None, ops.Grad([yy.re, yy.im, yy.re, yy.im]), mirror=False))
     loss = capi.empty(R)
     hbm("l2out_fwd", [R, Cc], 8, n, lambda: ops.l2out_fwd(u, loss))
     hbm("l2out_bwd", [R, Cc], 24, n, lambda: ops.l2out_bwd(u, du))
