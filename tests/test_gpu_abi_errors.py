@@ -49,6 +49,24 @@ def test_invalid_arguments_are_reported_not_fatal(gpu, port):
     assert _status("cnet_cdft_bwd_sym", *g.p()[:2], 8, *dx.p(), 4, 4, 8, 0) == INVALID                               # lddx < n
     assert _status("cnet_ctriang_dft_bwd_sym", *g.p()[:2], 8, *dx.p(), 8, 4, 50000, 0) == INVALID
     assert _status("cnet_cdft_bwd_sym", *g.p()[:2], 8, *dx.p(), 8, 0, 8, 0) == 0                                     # no rows: nothing to do
+    # the fused pairs of layers check theirs too
+    h = ops.CMat.empty(4, 8)
+    assert _status("cnet_hadamard_cgelu_fwd", *x.p(), 8, *x.p(), 8, h.re.ptr, None, 8, *y.p(), 8, 4, 8) == INVALID        # a plane of h missing
+    assert _status("cnet_hadamard_cgelu_fwd", *x.p(), 8, *x.p(), 8, *h.p(), 4, *y.p(), 8, 4, 8) == INVALID                # ldh < cols
+    assert _status("cnet_hadamard_cgelu_fwd", *x.p(), 8, *x.p(), 8, *h.p(), 8, *y.p(), 8, 0, 8) == 0
+    none4 = (None,) * 4
+    assert _status("cnet_hadamard_cgelu_bwd_sym", *x.p(), 8, *x.p(), 8, *g.p()[:2], 8, *none4, 0, *dx.p(), 8, *dx.p(), 8, 4, 8, 0) == 0   # dh not wanted
+    assert _status("cnet_hadamard_cgelu_bwd_sym", *x.p(), 8, *x.p(), 8, *g.p()[:2], 8, g.p()[0], None, None, None, 8, *dx.p(), 8, *dx.p(), 8,
+                   4, 8, 0) == INVALID                                                                                    # half a dh
+    assert _status("cnet_hadamard_cgelu_bwd_sym", *x.p(), 8, *x.p(), 8, *g.p()[:2], 8, *g.p(), 4, *dx.p(), 8, *dx.p(), 8, 4, 8, 0) == INVALID  # lddh < cols
+    assert _status("cnet_residual_cgelu_bwd_sym", *g.p()[:2], 8, g.p()[0], None, 8, *x.p(), 8, *dx.p(), 8, *none4, 0, *dx.p(), 8, 4, 8) == INVALID  # half a g2
+    assert _status("cnet_residual_cgelu_bwd_sym", *g.p()[:2], 8, None, None, 0, *x.p(), 8, *dx.p(), 8, None, dx.p()[1], None, None, 8,
+                   *dx.p(), 8, 4, 8) == INVALID                                                                           # half a dv
+    assert _status("cnet_residual_cgelu_bwd_sym", *g.p()[:2], 8, None, None, 0, *x.p(), 8, *dx.p(), 8, *none4, 0, *none4, 8, 4, 8) == INVALID  # no dh
+    assert _status("cnet_residual_cgelu_bwd_sym", *g.p()[:2], 8, None, None, 0, *x.p(), 4, *dx.p(), 8, *none4, 0, *dx.p(), 8, 4, 8) == INVALID  # ldh < cols
+    assert _status("cnet_clinear_cgelu_fwd", *x.p(), 8, *w.p(), 8, *h.p(), y.re.ptr, None, 8, 4, 8, 8, 0) == INVALID      # a plane of y missing
+    assert _status("cnet_clinear_cgelu_fwd", *x.p(), 8, *w.p(), 8, *h.p(), *y.p(), 4, 4, 8, 8, 0) == INVALID              # ldy < N
+    assert _status("cnet_clinear_cgelu_fwd", *x.p(), 8, *w.p(), 8, *h.p(), *y.p(), 8, 0, 8, 8, 0) == 0
     # DFT length beyond the int exponent range of the reference, Adam with a negative step, unknown marker
     assert _status("cnet_cdft_plan", 50000) == INVALID
     assert _status("cnet_adam_update", x.re.ptr, x.im.ptr, y.re.ptr, y.im.ptr, y.re.ptr, y.im.ptr, 32, 0.1, 0.9, -1, 1) == INVALID
