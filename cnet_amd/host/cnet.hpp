@@ -1069,11 +1069,6 @@ private:
 					g->out_size_ != f->out_size_)
 				continue;
 			if (t == isHadamard && g->no_outputs() != 1) continue;
-			// The activation in the store of the product saves a launch and the read of the pre-activation, but the second
-			// pair of planes leaves the product's kernel at its very end, when nothing is left to overlap it with: at
-			// 2048 x 2048 the fused launch took 17 us longer than the product alone, the separate CGelu 13 us.  It pays
-			// where a launch costs more than the bytes (small batches).
-			if (t == isLinear && (size_t) f->rows_ * f->out_size_ > ((size_t) 1 << 20)) continue;
 			f->fused_next_ = g;
 			g->fused_prev_ = t == isHadamard ? 2 : 1;
 		}
