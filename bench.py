@@ -287,6 +287,12 @@ def train_lines(steps):
         line = _train_bench("readme", batch, steps, "frozen_input")
         if line is None:
             return None
+        # configs[0] states real samples (imaginary parts 0), whose imaginary plane is cleared on the device instead of
+        # sent; beside it the same loop on samples with uniform imaginary parts, both planes travelling
+        both = _train_bench("readme", batch, steps, "complex_samples")
+        if both is not None:
+            line["samples_per_sec_complex_samples"] = both["samples_per_sec_prefetch_loss_read_one_step_late"]
+            line["upload_bytes_per_step_complex_samples"] = both["upload_bytes_per_step"]
         out.append(line)
     return out
 
@@ -475,7 +481,9 @@ def main():
                              "samples_per_sec": t["samples_per_sec_prefetch_loss_read_one_step_late"],
                              "samples_per_sec_loss_read_before_next_step": t["samples_per_sec_prefetch"],
                              "samples_per_sec_data_input_not_trainable": t["samples_per_sec_data_input_not_trainable"],
-                             "samples_per_sec_copy_inside_forward": t["samples_per_sec_copy_in_forward"]} for t in train]
+                             "samples_per_sec_copy_inside_forward": t["samples_per_sec_copy_in_forward"],
+                             "samples": t.get("samples"), "upload_bytes_per_step": t.get("upload_bytes_per_step"),
+                             "samples_per_sec_complex_samples": t.get("samples_per_sec_complex_samples")} for t in train]
         # the other configurations and kernels of the hot path, each bounded to a few seconds
         del x, w, g, y, dx, dw
         stack = stack_lines(10)

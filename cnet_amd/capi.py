@@ -32,6 +32,7 @@ SIGNATURES = {
     "cnet_memcpy_h2d_async": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_memcpy_d2h_async": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_upload_async": [C.c_void_p, C.c_void_p, C.c_size_t],
+    "cnet_upload_zero": [C.c_void_p, C.c_size_t],
     "cnet_upload_wait_compute": [],
     "cnet_mark_compute": [_i],
     "cnet_upload_wait_marker": [_i],

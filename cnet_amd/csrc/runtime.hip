@@ -280,6 +280,15 @@ int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes) {
 	return CNET_OK;
 }
 
+int cnet_upload_zero(void *dst, size_t bytes) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // a fill on the upload stream: never part of a recording
+	if (!bytes) return CNET_OK;
+	CNET_CHECK_ARG(dst != nullptr);
+	CNET_HIP(hipMemsetAsync(dst, 0, bytes, rt().upload_stream));
+	return CNET_OK;
+}
+
 int cnet_upload_wait_compute(void) {
 	CNET_REQUIRE_INIT();
 	CNET_NOT_IN_CAPTURE();  // would pull the upload stream into the recording

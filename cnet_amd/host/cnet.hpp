@@ -177,6 +177,18 @@ class InputBatch : public Batch {
 	float *real_data_ = NULL, *imag_data_ = NULL;  // [batch][dim] each, one allocation
 	bool pinned_ = false;
 	int64_t ticket_ = -1;     // >= 0: a copy queued from these planes may not have finished; what the host waits for
+	// Some sample added since the last clear() has an imaginary part that is not +0: while this is false the imaginary plane
+	// holds nothing but zeros and need not travel to the device (real-valued data such as images: half the upload).
+	bool imag_nonzero_ = false;
+	static bool anyBitSet(const float *p, size_t n) {
+		uint32_t acc = 0;
+		for (size_t k = 0; k < n; ++k) {
+			uint32_t w;
+			std::memcpy(&w, p + k, sizeof(w));
+			acc |= w;
+		}
+		return acc != 0;
+	}
 
 	void allocate() {
 		const size_t bytes = 2 * (size_t) batch_size_ * sample_dim_ * sizeof(float);
@@ -222,9 +234,10 @@ public:
 	InputBatch(const InputBatch &o) : Batch(o) {
 		allocate();
 		if (o.real_data_) std::copy(o.real_data_, o.real_data_ + 2 * (size_t) batch_size_ * sample_dim_, real_data_);
+		imag_nonzero_ = o.imag_nonzero_;
 	}
 	InputBatch(InputBatch &&o) noexcept : Batch(std::move(o)), real_data_(o.real_data_), imag_data_(o.imag_data_), pinned_(o.pinned_),
-			ticket_(o.ticket_) {
+			ticket_(o.ticket_), imag_nonzero_(o.imag_nonzero_) {
 		o.real_data_ = o.imag_data_ = NULL;
 	}
 	InputBatch &operator=(InputBatch &&o) noexcept {
@@ -235,6 +248,7 @@ public:
 			imag_data_ = o.imag_data_;
 			pinned_ = o.pinned_;
 			ticket_ = o.ticket_;
+			imag_nonzero_ = o.imag_nonzero_;
 			o.real_data_ = o.imag_data_ = NULL;
 		}
 		return *this;
@@ -250,7 +264,10 @@ public:
 		labels_.clear();
 		sizes_.clear();
 		current_pos_ = 0;
+		imag_nonzero_ = false;
 	}
+	// every imaginary part added so far is +0: the samples are real
+	bool imagIsZero() const { return !imag_nonzero_; }
 	void add(const std::vector<std::complex<float> > &sample, int label) {
 		assert(current_pos_ < batch_size_ && (int) sample.size() <= sample_dim_);
 		settle();
@@ -259,6 +276,7 @@ public:
 			re[k] = sample[k].real();
 			im[k] = sample[k].imag();
 		}
+		imag_nonzero_ = imag_nonzero_ || anyBitSet(im, sample.size());
 		finishRow((int) sample.size(), label);
 	}
 	void add(std::initializer_list<std::complex<float> > list, int label) {
@@ -270,6 +288,7 @@ public:
 		settle();
 		std::copy(re, re + n, rowRe());
 		std::copy(im, im + n, rowIm());
+		imag_nonzero_ = imag_nonzero_ || anyBitSet(im, (size_t) n);
 		finishRow(n, label);
 	}
 	// Fill the next `count` rows from planar sample storage ([sample][dim] re and im): row k takes sample index[k] and
@@ -280,11 +299,14 @@ public:
 		settle();
 		const size_t dim = (size_t) sample_dim_;
 		float *dst_re = rowRe(), *dst_im = rowIm();
-#pragma omp parallel for schedule(static) if ((size_t) count * dim >= (1u << 18))
+		int nonzero = imag_nonzero_ ? 1 : 0;
+#pragma omp parallel for schedule(static) reduction(| : nonzero) if ((size_t) count * dim >= (1u << 18))
 		for (int k = 0; k < count; ++k) {
 			std::memcpy(dst_re + k * dim, re + index[k] * dim, dim * sizeof(float));
 			std::memcpy(dst_im + k * dim, im + index[k] * dim, dim * sizeof(float));
+			nonzero |= anyBitSet(dst_im + k * dim, dim) ? 1 : 0;
 		}
+		imag_nonzero_ = nonzero != 0;
 		for (int k = 0; k < count; ++k) {
 			labels_.push_back(labels[index[k]]);
 			sizes_.push_back(sample_dim_);
@@ -653,6 +675,7 @@ class CNet {
 	bool use_graphs_ = false;
 	bool conjugate_gradients_ = true;
 	bool fuse_layers_ = true;
+	bool send_zero_planes_ = false;
 	float *loss_ring_ = NULL;  // page-locked [kLossSlots][batch]: losses on their way to the host (gpuQueueLoss)
 	int64_t loss_queued_ = 0;
 	std::vector<const float *> gather_src_;  // pending dz* gathers of the input functions (see nodeBackward)
@@ -1554,13 +1577,17 @@ private:
 		}
 		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
 		// one copy per plane (upstream: two small copies per sample, gpu/gpu_func.h:403-419)
+		// (a batch of real samples sends its real plane only; the imaginary plane is cleared on the device)
+		const bool real_only = batch.imagIsZero() && !send_zero_planes_;
 		if (batch.isPinned()) {
 			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d_async");
-			ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
+			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
+			else ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
 			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
 		} else {
 			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d");
-			ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
+			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
+			else ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
 		}
 		setLabels(batch.labelsPtr(), batch_);
 	}
@@ -1597,7 +1624,8 @@ public:
 		std::copy(batch.labelsPtr(), batch.labelsPtr() + batch_, st.host_labels);
 		ck(cnet_upload_wait_marker(other), "cnet_upload_wait_marker");  // kernels of the step that last used this buffer
 		ck(cnet_upload_async(st.z, batch.realDataPtr(), plane * sizeof(float)), "cnet_upload_async");
-		ck(cnet_upload_async(st.z + plane, batch.imagDataPtr(), plane * sizeof(float)), "cnet_upload_async");
+		if (batch.imagIsZero() && !send_zero_planes_) ck(cnet_upload_zero(st.z + plane, plane * sizeof(float)), "cnet_upload_zero");
+		else ck(cnet_upload_async(st.z + plane, batch.imagDataPtr(), plane * sizeof(float)), "cnet_upload_async");
 		ck(cnet_upload_async(st.labels, st.host_labels, batch_ * sizeof(int32_t)), "cnet_upload_async");
 		ck(cnet_mark_upload(other), "cnet_mark_upload");
 		ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
@@ -1611,22 +1639,26 @@ public:
 			throw std::invalid_argument("gpuSetInput: " + cin->getName() + " is not a data input of this batch shape");
 		CFunc::Slot &s = cin->slots_[0];
 		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
+		const bool real_only = batch.imagIsZero() && !send_zero_planes_;
 		if (batch.isPinned() && !use_graphs_) {
 			// On the upload stream, behind everything queued on the compute stream so far (the kernels that still use the
 			// previous contents); the compute stream waits for it only in front of the first kernel that touches this
 			// input, so the copy travels under the layers of the forward pass that come before it.
 			ck(cnet_upload_wait_compute(), "cnet_upload_wait_compute");
 			ck(cnet_upload_async(s.z, batch.realDataPtr(), plane), "cnet_upload_async");
-			ck(cnet_upload_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_upload_async");
+			if (real_only) ck(cnet_upload_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_upload_zero");
+			else ck(cnet_upload_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_upload_async");
 			ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
 			in_flight_.push_back(cin);
 		} else if (batch.isPinned()) {  // queued behind the kernels that still read the previous contents; the host does not wait
 			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d_async");
-			ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
+			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
+			else ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
 			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
 		} else {
 			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d");
-			ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
+			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
+			else ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
 		}
 	}
 	bool gpuForward(InputFunc *inp, OutputFunc *outp, EmbeddingBatch &batch) {
@@ -1772,6 +1804,10 @@ public:
 		}
 	}
 	bool fusingLayers() const { return fuse_layers_; }
+	// A batch all of whose samples are real (InputBatch::imagIsZero: images, for instance) sends its real plane only and
+	// the imaginary plane of the data input is cleared on the device: half the bytes over the link, the same values on
+	// the device.  On: the plane of zeros travels like any other.
+	void sendZeroPlanes(bool on) { send_zero_planes_ = on; }
 	// An input function with one consumer leaves the gradient of a backward pass in that consumer's planes until the update
 	// reads it there (nothing is added to cleared planes and cleared again).  Off: every backward pass adds it to the input
 	// function's own planes at once, as upstream does.  Same weights to the bit either way.

@@ -2,7 +2,7 @@
 // bench.py runs for the "train samples/sec" half of the metric.  Synthetic, seeded data from its own generator; no
 // comparison with anything (the parity tests do that), one JSON line per run on stdout.
 //
-//   train_bench readme B steps [graphs] [both_halves] [frozen_input]
+//   train_bench readme B steps [graphs] [both_halves] [frozen_input] [complex_samples]
 //       FourierTrans(784) -> Hadamard -> CGelu -> Linear 784 -> 10 -> CrossEntropy, SGD, batches from a
 //       BatchedDataReader; the loop of upstream cnet.cpp:119-150 in several input / read-back modes.
 //   train_bench stack n blocks B steps lr [both_halves]
@@ -54,14 +54,14 @@ void build_readme(CNet &net, int n, int classes, int *inp, int *outp) {
 }
 
 struct SyntheticReader : public BatchedDataReader {
-	SyntheticReader(int dim, int count, int classes) : BatchedDataReader(dim) {
+	SyntheticReader(int dim, int count, int classes, bool complex_samples) : BatchedDataReader(dim) {
 		Gen rng(123);
 		std::vector<float> re(dim), im(dim);
 		reserve(count);
 		for (int s = 0; s < count; ++s) {
 			for (int k = 0; k < dim; ++k) {
-				re[k] = (float) rng.uniform();
-				im[k] = (float) rng.uniform();
+				re[k] = (float) rng.uniform();  // real parts uniform in [0, 1], imaginary parts 0: image-like samples
+				im[k] = complex_samples ? (float) rng.uniform() : 0.f;
 			}
 			addPlanes(re.data(), im.data(), (int) (rng.next() % classes));
 		}
@@ -81,14 +81,14 @@ bool has(int argc, char **argv, int from, const char *word) {
 //   4 as 1 with gpuTrainStep (one recorded graph)      5 as 1 with both halves of every gradient pair computed
 //   6 as 1, the loss of a step read one step later     7 as 6 with gpuTrainStep
 //   8 as 6 with the data input marked not trainable
-int run_readme(int B, int steps, bool with_graphs, bool both_halves, bool frozen_input) {
+int run_readme(int B, int steps, bool with_graphs, bool both_halves, bool frozen_input, bool complex_samples) {
 	const int n = 784, classes = 10;
 	const float lr = 0.01f;
 	if (cnet_init(0) != CNET_OK) {
 		fprintf(stderr, "train_bench: cnet_init failed: %s\n", cnet_last_error());
 		return 2;
 	}
-	SyntheticReader data(n, 3 * B + 7, classes);
+	SyntheticReader data(n, 3 * B + 7, classes, complex_samples);
 	constexpr int MODES = 9;
 	double ms[MODES] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
 	float last_loss[MODES] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -156,9 +156,10 @@ int run_readme(int B, int steps, bool with_graphs, bool both_halves, bool frozen
 		   "\"ms_per_step_prefetch_two_products_per_gradient_pair\": %.3f, \"ms_per_step_prefetch_loss_read_one_step_late\": %.3f, "
 		   "\"samples_per_sec_prefetch_loss_read_one_step_late\": %.1f, \"ms_per_step_train_step_graph_loss_read_one_step_late\": %.3f, "
 		   "\"ms_per_step_data_input_not_trainable\": %.3f, \"samples_per_sec_data_input_not_trainable\": %.1f, "
-		   "\"last_loss\": %.5f, \"upload_bytes_per_step\": %zu}\n",
+		   "\"last_loss\": %.5f, \"samples\": \"%s\", \"upload_bytes_per_step\": %zu}\n",
 			B, steps, ms[0], ms[1], ms[2], ms[3], rate(0), rate(1), rate(2), ms[4], rate(4), ms[5], ms[6], rate(6), ms[7], ms[8], rate(8),
-			last_loss[6], (size_t) 2 * B * n * sizeof(float));
+			last_loss[6], complex_samples ? "complex: real and imaginary parts uniform in [0, 1]" : "real parts uniform in [0, 1], imaginary parts 0 (the imaginary plane is cleared on the device, not sent)",
+			(size_t) (complex_samples ? 2 : 1) * B * n * sizeof(float));
 	return std::isfinite(last_loss[6]) ? 0 : 1;
 }
 
@@ -243,7 +244,7 @@ int main(int argc, char **argv) {
 	try {
 		if (what == "readme")
 			return run_readme(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, has(argc, argv, 4, "graphs"),
-					has(argc, argv, 4, "both_halves"), has(argc, argv, 4, "frozen_input"));
+					has(argc, argv, 4, "both_halves"), has(argc, argv, 4, "frozen_input"), has(argc, argv, 4, "complex_samples"));
 		if (what == "stack")
 			return run_stack(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048,
 					argc > 5 ? atoi(argv[5]) : 10, argc > 6 ? (float) atof(argv[6]) : 0.01f, has(argc, argv, 7, "both_halves"));
@@ -251,6 +252,6 @@ int main(int argc, char **argv) {
 		fprintf(stderr, "train_bench: %s\n", e.what());
 		return 2;
 	}
-	fprintf(stderr, "usage: train_bench readme B steps [graphs] [both_halves] [frozen_input] | stack n blocks B steps lr [both_halves]\n");
+	fprintf(stderr, "usage: train_bench readme B steps [graphs] [both_halves] [frozen_input] [complex_samples] | stack n blocks B steps lr [both_halves]\n");
 	return 64;
 }

@@ -70,6 +70,8 @@ int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes);   /* *_copy_
  *      read of CNet::getLoss, impl/cnet.h / gpu/gpu_func.h:928-969 upstream); the page-locked destination is valid once a
  *      ticket taken after the call has been waited for.
  * cnet_upload_async: the same on the library's upload stream, so it overlaps kernels of the compute stream.
+ * cnet_upload_zero: clears device memory on the upload stream, in order with the copies queued there (the imaginary plane
+ *      of a batch of real samples is cleared on the device instead of travelling as zeros).
  * cnet_upload_wait_compute: uploads queued after this call start only when everything queued on the compute stream so
  *      far has finished (call before overwriting a device buffer that kernels may still read).
  * cnet_mark_compute(m) / cnet_upload_wait_marker(m), m = 0..7: the same in two halves - remember the current tail of the
@@ -89,6 +91,7 @@ int cnet_host_free(void *host_ptr);
 int cnet_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
 int cnet_memcpy_d2h_async(void *pinned_dst, const void *src, size_t bytes);
 int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes);
+int cnet_upload_zero(void *dst, size_t bytes);
 int cnet_upload_wait_compute(void);
 int cnet_mark_compute(int marker);
 int cnet_upload_wait_marker(int marker);

@@ -11,6 +11,7 @@
 //   facade_test saved_model <golden dir> <scratch dir>   upstream-written .mod files restored and run on the device
 //   facade_test pipeline [B steps]  reader -> page-locked batches -> device, with and without gpuPrefetch (same bits)
 //   facade_test deferred           gradients of the input functions left with their consumers until the update (same bits)
+//   facade_test real_batches       batches of real samples send their real plane only (same bits)
 //   facade_test upstream_nets      the nets of upstream's own GPU tests (E2E chain, fan-out into one consumer, ...)
 //   facade_test errors             error behaviour
 //   facade_test stack8 n blocks B steps lr rows overflow|finite [learn]   residual stack of `blocks` blocks against the
@@ -867,14 +868,14 @@ static void build_readme(CNet &net, int n, int classes, int *inp, int *outp) {
 }
 
 struct SyntheticReader : public BatchedDataReader {
-	SyntheticReader(int dim, int count, int classes) : BatchedDataReader(dim) {
+	SyntheticReader(int dim, int count, int classes, bool real_samples = false) : BatchedDataReader(dim) {
 		orc::Rng rng(123);
 		std::vector<float> re(dim), im(dim);
 		reserve(count);
 		for (int s = 0; s < count; ++s) {
 			for (int k = 0; k < dim; ++k) {
 				re[k] = (float) rng.uniform();
-				im[k] = (float) rng.uniform();
+				im[k] = real_samples ? 0.f : (float) rng.uniform();
 			}
 			addPlanes(re.data(), im.data(), (int) (rng.next() % classes));
 		}
@@ -1103,6 +1104,57 @@ static void test_deferred_gathers() {
 	bool finite = true;
 	for (float v : trace[0]) finite = finite && std::isfinite(v);
 	expect("all finite", finite);
+}
+
+// ------------------------------------------------------------------------------------------------- real-valued batches
+// A batch whose samples are all real sends its real plane only; the imaginary plane of the data input is cleared on the
+// device (the update steps the data input, so it is not zero any more after a step).  Same bits as sending the zeros, with
+// the copy inside gpuForward and with gpuPrefetch; a batch with one imaginary part set takes the usual path.
+static void test_real_batches() {
+	const int n = 784, classes = 10, B = 48, steps = 5;
+	if (cnet_init(0) != CNET_OK) {
+		expect("cnet_init", false);
+		return;
+	}
+	SyntheticReader data(n, 4 * B, classes, true);
+	std::vector<float> trace[4];
+	for (int variant = 0; variant < 4; ++variant) {  // bit 0: send the zeros, bit 1: prefetch
+		CNet net;
+		int inp, outp;
+		build_readme(net, n, classes, &inp, &outp);
+		net.allocateOnGpu(B);
+		net.sendZeroPlanes((variant & 1) != 0);
+		CInput *cin = (CInput *) net[inp];
+		CrossEntropy *cen = (CrossEntropy *) net[outp];
+		SyntheticReader reader = data;
+		InputBatch ring[2] = {InputBatch(B, n), InputBatch(B, n)};
+		const bool prefetch = (variant & 2) != 0;
+		reader.nextBatch(ring[0]);
+		if (variant == 0) expect("a batch of real samples knows it", ring[0].imagIsZero());
+		if (prefetch) net.gpuPrefetch(cin, ring[0]);
+		for (int s = 0; s < steps; ++s) {
+			InputBatch &cur = ring[s % 2];
+			net.gpuForward(cin, cen, cur);
+			net.gpuBackward();
+			net.gpuUpdateInputs(0.05f / B);
+			if (s + 1 < steps) {
+				reader.nextBatch(ring[(s + 1) % 2]);
+				if (prefetch) net.gpuPrefetch(cin, ring[(s + 1) % 2]);
+			}
+			trace[variant].push_back(net.getLoss(cen, NULL));
+		}
+		net.getInputsFromGpu();
+		for (auto f : net.inputs()) trace[variant].insert(trace[variant].end(), f->input().real_, f->input().real_ + 2 * f->input().length_);
+	}
+	expect("real plane only, copy inside gpuForward: same losses, weights and data input as with the zeros sent", trace[0] == trace[1] && trace[0].size() > 100);
+	expect("real plane only, gpuPrefetch: the same", trace[2] == trace[3] && trace[0] == trace[2]);
+	InputBatch mixed(2, 3);
+	mixed.add({{1.f, 0.f}, {2.f, 0.f}}, 0);
+	expect("real samples so far", mixed.imagIsZero());
+	mixed.add({{1.f, 0.f}, {2.f, -0.f}}, 1);
+	expect("an imaginary part of -0 is not +0: the plane travels", !mixed.imagIsZero());
+	mixed.clear();
+	expect("clear() starts over", mixed.imagIsZero());
 }
 
 // ------------------------------------------------------------------------------------------------- frozen data input
@@ -1510,6 +1562,7 @@ int main(int argc, char **argv) {
 		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12);
 		if (what == "frozen_input" || what == "all") test_frozen_input();
 		if (what == "deferred" || what == "all") test_deferred_gathers();
+		if (what == "real_batches" || what == "all") test_real_batches();
 		if (what == "upstream_nets" || what == "all") test_upstream_nets();
 		if (what == "errors" || what == "all") test_errors();
 		// stack8 n blocks B steps lr rows_checked overflow|finite [learn]

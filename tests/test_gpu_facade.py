@@ -93,6 +93,13 @@ def test_gradients_of_input_functions_left_with_their_consumers_until_the_update
     assert "FAIL" not in out and out.count("PASS") >= 4
 
 
+def test_batches_of_real_samples_send_their_real_plane_only():
+    """InputBatch::imagIsZero / CNet::sendZeroPlanes: the imaginary plane of real data is cleared on the device instead of
+    travelling; losses, weights and the stepped data input agree to the bit with the zeros sent."""
+    out = _run("real_batches")
+    assert "FAIL" not in out and out.count("PASS") >= 6
+
+
 def test_nets_of_the_upstream_gpu_tests():
     out = _run("upstream_nets")
     assert "FAIL" not in out and out.count("PASS") >= 25
