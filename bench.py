@@ -472,7 +472,7 @@ def main():
     if not args.no_cpu_baseline:   # the flag leaves the headline alone (profiled runs)
         out["conjugate_gradient_pair"] = conjugate_pair_step()
         out["cpu_baseline"] = cpu_baseline()
-        train = train_lines(100)
+        train = train_lines(300)
         if train:   # the other half of the metric: training steps of the configs[0] net through the C++ facade
             # ms_per_step: batches staged on the upload stream, every step's loss read on the host one step later;
             # ..._loss_read_before_next_step: the same with the host waiting for each loss before it queues the next step

@@ -1576,18 +1576,17 @@ private:
 			return;
 		}
 		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
-		// one copy per plane (upstream: two small copies per sample, gpu/gpu_func.h:403-419)
+		// one copy for both planes, which are one array here and there (upstream: two small copies per sample,
+		// gpu/gpu_func.h:403-419)
 		// (a batch of real samples sends its real plane only; the imaginary plane is cleared on the device)
 		const bool real_only = batch.imagIsZero() && !send_zero_planes_;
 		if (batch.isPinned()) {
-			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d_async");
+			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), real_only ? plane : 2 * plane), "cnet_memcpy_h2d_async");
 			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
-			else ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
 			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
 		} else {
-			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d");
+			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), real_only ? plane : 2 * plane), "cnet_memcpy_h2d");
 			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
-			else ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
 		}
 		setLabels(batch.labelsPtr(), batch_);
 	}
@@ -1623,9 +1622,13 @@ public:
 		if (st.labels_ticket >= 0) ck(cnet_copy_wait(st.labels_ticket), "cnet_copy_wait");  // the previous copy has left host_labels
 		std::copy(batch.labelsPtr(), batch.labelsPtr() + batch_, st.host_labels);
 		ck(cnet_upload_wait_marker(other), "cnet_upload_wait_marker");  // kernels of the step that last used this buffer
-		ck(cnet_upload_async(st.z, batch.realDataPtr(), plane * sizeof(float)), "cnet_upload_async");
-		if (batch.imagIsZero() && !send_zero_planes_) ck(cnet_upload_zero(st.z + plane, plane * sizeof(float)), "cnet_upload_zero");
-		else ck(cnet_upload_async(st.z + plane, batch.imagDataPtr(), plane * sizeof(float)), "cnet_upload_async");
+		// the two planes of a batch are one array on the host and on the device: one copy for both
+		if (batch.imagIsZero() && !send_zero_planes_) {
+			ck(cnet_upload_async(st.z, batch.realDataPtr(), plane * sizeof(float)), "cnet_upload_async");
+			ck(cnet_upload_zero(st.z + plane, plane * sizeof(float)), "cnet_upload_zero");
+		} else {
+			ck(cnet_upload_async(st.z, batch.realDataPtr(), 2 * plane * sizeof(float)), "cnet_upload_async");
+		}
 		ck(cnet_upload_async(st.labels, st.host_labels, batch_ * sizeof(int32_t)), "cnet_upload_async");
 		ck(cnet_mark_upload(other), "cnet_mark_upload");
 		ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
@@ -1645,20 +1648,17 @@ public:
 			// previous contents); the compute stream waits for it only in front of the first kernel that touches this
 			// input, so the copy travels under the layers of the forward pass that come before it.
 			ck(cnet_upload_wait_compute(), "cnet_upload_wait_compute");
-			ck(cnet_upload_async(s.z, batch.realDataPtr(), plane), "cnet_upload_async");
+			ck(cnet_upload_async(s.z, batch.realDataPtr(), real_only ? plane : 2 * plane), "cnet_upload_async");
 			if (real_only) ck(cnet_upload_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_upload_zero");
-			else ck(cnet_upload_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_upload_async");
 			ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
 			in_flight_.push_back(cin);
 		} else if (batch.isPinned()) {  // queued behind the kernels that still read the previous contents; the host does not wait
-			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d_async");
+			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), real_only ? plane : 2 * plane), "cnet_memcpy_h2d_async");
 			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
-			else ck(cnet_memcpy_h2d_async(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d_async");
 			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
 		} else {
-			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), plane), "cnet_memcpy_h2d");
+			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), real_only ? plane : 2 * plane), "cnet_memcpy_h2d");
 			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
-			else ck(cnet_memcpy_h2d(s.z + (size_t) batch_ * s.len, batch.imagDataPtr(), plane), "cnet_memcpy_h2d");
 		}
 	}
 	bool gpuForward(InputFunc *inp, OutputFunc *outp, EmbeddingBatch &batch) {
