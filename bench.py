@@ -127,8 +127,19 @@ def kernel_suite(steps):
         return ops.Grad.from_host([rs.randn(r, c).astype(np.float32) for _ in range(4)])
 
     def timed(fn, warm=3):
-        for _ in range(warm):
-            fn()
+        # warm-up: groups of `warm` calls until two groups in a row agree to 2 % (at most 0.2 s): the device may have
+        # gone idle while the host prepared the operands of this line, and comes back to its clocks over some 30 ms
+        last, t0 = None, time.perf_counter()
+        while time.perf_counter() - t0 < 0.2:
+            a, b = ev.event(), ev.event()
+            ev.record(a)
+            for _ in range(warm):
+                fn()
+            ev.record(b)
+            cur = ev.elapsed_ms(a, b)
+            if last is not None and abs(cur - last) <= 0.02 * last:
+                break
+            last = cur
         capi.sync()
         a, b = ev.event(), ev.event()
         ev.record(a)
@@ -391,6 +402,22 @@ def main():
         print(json.dumps({"counter_pass": True, "copy_bytes_read": rows * cols * 4, "copy_bytes_written": rows * cols * 4}))
         return
 
+    # Out of idle first: a device that has just been handed over runs its first ~25 steps (30 ms) of this workload up to 25 %
+    # slower while its clocks come up (1.45 -> 1.18 ms per step, measured step by step with events).  Groups of 10 steps are
+    # run until two in a row agree to 1 % (at most 0.5 s in all); the W warm-up steps and the K timed steps follow.
+    preroll, last = 0, None
+    t_pre = time.perf_counter()
+    while time.perf_counter() - t_pre < 0.5:
+        a, b = ev.event(), ev.event()
+        ev.record(a)
+        for _ in range(10):
+            step()
+        ev.record(b)
+        cur = ev.elapsed_ms(a, b)
+        preroll += 10
+        if last is not None and abs(cur - last) <= 0.01 * last:
+            break
+        last = cur
     for _ in range(args.warmup):
         step()
     capi.sync(); tsync()
@@ -459,7 +486,7 @@ def main():
     out = {
         "metric": "complex-Linear fwd+bwd TFLOP/s (% fp32 MFMA peak); train samples/sec",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "preroll_steps": preroll, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: isolated complex Linear fwd + Wirtinger bwd (dx, dx*, dW, dW*), "
                                "complex64 split-plane", "batch": B, "in": K, "out": N,
