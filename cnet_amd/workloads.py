@@ -53,8 +53,7 @@ class TokenModel:
         # M_b = F X_b for every sequence b: one strided-batched launch, F shared (stride 0)
         ops.cgemm_batched(self.F, 0, self.x, S * D, self.m, S * D, S, D, S, B, a_kmajor=0, b_kmajor=1)
         ops.hadamard_fwd(self.m, self.gate, self.h, shared=True)
-        ops.linear_fwd(self.h, self.w1, self.u)
-        ops.gelu_fwd(self.u, self.a)
+        ops.linear_gelu_fwd(self.h, self.w1, self.u, self.a)   # the CGelu applied where the product is stored
         ops.linear_fwd(self.a, self.w2, self.o)
         ops.linear_fwd(self.o, self.w3, self.logits)
         ops.cross_entropy_fwd(self.logits, self.labels, self.s, self.loss, self.argmax, None)
