@@ -61,6 +61,7 @@ SIGNATURES = {
     "cnet_cdft_twiddle": [_i, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)],
     "cnet_cdft_set_forward_matrix": [_i, C.c_void_p, C.c_void_p],
     "cnet_cdft_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i, _i],
+    "cnet_cdft_fwd_real_input": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i],
     "cnet_cdft_bwd": [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_cdft_bwd_sym": [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_ctriang_dft_bwd_sym": [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],

@@ -4,6 +4,7 @@
 // entry is the correctly rounded fp32 value of the exact root of unity; F is symmetric, so y = x * F.
 #include "common.hpp"
 
+#include <algorithm>
 #include <map>
 #include <vector>
 
@@ -48,6 +49,19 @@ __global__ void twiddle_kernel(float *__restrict__ fre, float *__restrict__ fim,
 	const double scale = (upper_only && p > q) ? 0.0 : 1.0 / sqrt((double) n);
 	fre[(long) p * ld + q] = (float) (c * scale);
 	fim[(long) p * ld + q] = (float) (s * scale);
+}
+
+// The transform of real samples is conjugate-symmetric, y[n - q] = conj(y[q]): the columns beyond n/2 are written from
+// the ones below it.  One thread per (row, q), q = 1 .. half.
+__global__ __launch_bounds__(256) void hermitian_mirror_kernel(float *__restrict__ y_re, float *__restrict__ y_im, long ldy, int rows, int n,
+		int half) {
+	const long idx = (long) blockIdx.x * 256 + threadIdx.x;
+	if (idx >= (long) rows * half) return;
+	const long row = idx / half;
+	const int q = (int) (idx - row * half) + 1;
+	const long src = row * ldy + q, dst = row * ldy + (n - q);
+	y_re[dst] = y_re[src];
+	y_im[dst] = -y_im[src];
 }
 
 static int get_plan(int n, Twiddle *out, bool create) {
@@ -160,6 +174,35 @@ int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re
 	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
 	bool cj[2] = {false, false};
 	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate, 0, 0);
+}
+
+int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy, int B, int n) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && n > 0 && n <= 46340);
+	if (B == 0) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= n && ldy >= n);
+	Twiddle t;
+	int rc = get_plan(n, &t, true);
+	if (rc) return rc;
+	// a caller-supplied forward operator need not be symmetric under q -> n - q: the whole product then
+	if (t.fwd_re) return cnet_cdft_fwd(x_re, x_im, ldx, y_re, y_im, ldy, B, n, 0);
+	// columns 0 .. n/2 by the matrix product (x_im is read and holds zeros), the others as conjugates of those
+	// (rounded up to a multiple of four columns, which keeps the product on the kernels with 128-bit loads; the few
+	// extra columns are correct values that the mirror pass writes again)
+	const int cols = std::min(n, (n / 2 + 1 + 3) / 4 * 4);
+	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {t.re, t.re}, *bi[2] = {t.im, t.im};
+	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
+	bool cj[2] = {false, false};
+	rc = cgemm_pair(false, true, 1, B, cols, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, 0, 0, 0);
+	if (rc) return rc;
+	const int half = (n - 1) / 2;  // columns 1 .. half have a partner n - q of their own
+	if (half > 0) {
+		const long total = (long) B * half;
+		hipLaunchKernelGGL(hermitian_mirror_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, rt().stream, y_re, y_im, (long) ldy, B, n,
+				half);
+		CNET_LAUNCH_CHECK();
+	}
+	return CNET_OK;
 }
 
 int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,

@@ -142,6 +142,11 @@ def dft_fwd(x, y, accumulate=0):
     call("cnet_cdft_fwd", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols, accumulate)
 
 
+def dft_fwd_real_input(x, y):
+    """x holds real samples: its imaginary plane is all +0."""
+    call("cnet_cdft_fwd_real_input", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols)
+
+
 def dft_bwd(g, dx, accumulate=0):
     call("cnet_cdft_bwd", *g.p(), g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
 

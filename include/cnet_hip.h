@@ -195,6 +195,13 @@ int cnet_cdft_twiddle(int n, const float **f_re, const float **f_im);  /* the pl
 int cnet_cdft_set_forward_matrix(int n, const float *host_f_re, const float *host_f_im);
 int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
                   int B, int n, int accumulate);      /* y = x * F */
+/* The same transform for REAL samples (upstream's FourierTrans forward, impl/ft.h:37-55, transforms them like any
+ * others, and so does gpu_fft_forward, gpu/reduce.cpp:160-187).  The caller vouches that every x_im is +0
+ * (the plane is still read).  The result is conjugate-symmetric, y[n - q] = conj(y[q]), so only columns 0 .. n/2 go
+ * through the matrix product and the rest are written as conjugates: half the matrix work.  Agrees with cnet_cdft_fwd on
+ * such samples to rounding (the stored twiddles are symmetric under q -> n - q up to their last bit); assigns. */
+int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
+                             int B, int n);
 int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
                   float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
                   int B, int n, int accumulate);      /* dx.dz = g.dz * F ; dx.dzs = g.dzs * conj(F) */

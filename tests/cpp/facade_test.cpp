@@ -1111,32 +1111,40 @@ static void test_deferred_gathers() {
 // device (the update steps the data input, so it is not zero any more after a step).  Same bits as sending the zeros, with
 // the copy inside gpuForward and with gpuPrefetch; a batch with one imaginary part set takes the usual path.
 static void test_real_batches() {
-	const int n = 784, classes = 10, B = 48, steps = 5;
+	const int n = 784, classes = 10, B = 512, steps = 6;  // large enough for the transform of real samples to take half its columns
 	if (cnet_init(0) != CNET_OK) {
 		expect("cnet_init", false);
 		return;
 	}
 	SyntheticReader data(n, 4 * B, classes, true);
-	std::vector<float> trace[4];
-	for (int variant = 0; variant < 4; ++variant) {  // bit 0: send the zeros, bit 1: prefetch
+	std::vector<float> trace[7];
+	// bit 0: send the zeros, bit 1: prefetch; 4: the whole transform whatever the samples; 5: whole recorded steps;
+	// 6: recorded phases
+	for (int variant = 0; variant < 7; ++variant) {
 		CNet net;
 		int inp, outp;
 		build_readme(net, n, classes, &inp, &outp);
 		net.allocateOnGpu(B);
-		net.sendZeroPlanes((variant & 1) != 0);
+		net.sendZeroPlanes((variant & 1) != 0 && variant < 4);
+		if (variant == 4) net.realTransforms(false);
+		if (variant == 6) net.useGraphs(true);
 		CInput *cin = (CInput *) net[inp];
 		CrossEntropy *cen = (CrossEntropy *) net[outp];
 		SyntheticReader reader = data;
 		InputBatch ring[2] = {InputBatch(B, n), InputBatch(B, n)};
-		const bool prefetch = (variant & 2) != 0;
+		const bool prefetch = (variant & 2) != 0 || variant >= 4;
 		reader.nextBatch(ring[0]);
 		if (variant == 0) expect("a batch of real samples knows it", ring[0].imagIsZero());
 		if (prefetch) net.gpuPrefetch(cin, ring[0]);
 		for (int s = 0; s < steps; ++s) {
 			InputBatch &cur = ring[s % 2];
-			net.gpuForward(cin, cen, cur);
-			net.gpuBackward();
-			net.gpuUpdateInputs(0.05f / B);
+			if (variant == 5) {
+				net.gpuTrainStep(cin, cen, cur, 0.05f / B);
+			} else {
+				net.gpuForward(cin, cen, cur);
+				net.gpuBackward();
+				net.gpuUpdateInputs(0.05f / B);
+			}
 			if (s + 1 < steps) {
 				reader.nextBatch(ring[(s + 1) % 2]);
 				if (prefetch) net.gpuPrefetch(cin, ring[(s + 1) % 2]);
@@ -1148,6 +1156,17 @@ static void test_real_batches() {
 	}
 	expect("real plane only, copy inside gpuForward: same losses, weights and data input as with the zeros sent", trace[0] == trace[1] && trace[0].size() > 100);
 	expect("real plane only, gpuPrefetch: the same", trace[2] == trace[3] && trace[0] == trace[2]);
+	expect("whole recorded steps and recorded phases: the same", trace[5] == trace[2] && trace[6] == trace[2]);
+	{
+		// half the columns of the first FourierTrans computed and the rest written as conjugates, against the whole product
+		double num = 0, den = 0;
+		for (size_t k = 0; k < trace[2].size(); ++k) {
+			num += ((double) trace[2][k] - trace[4][k]) * ((double) trace[2][k] - trace[4][k]);
+			den += (double) trace[4][k] * trace[4][k];
+		}
+		report("transform of real samples through half its columns: losses, weights and data input (relative Frobenius)", std::sqrt(num / den), 1e-5);
+		expect("the two are different computations", trace[2].size() == trace[4].size());
+	}
 	InputBatch mixed(2, 3);
 	mixed.add({{1.f, 0.f}, {2.f, 0.f}}, 0);
 	expect("real samples so far", mixed.imagIsZero());

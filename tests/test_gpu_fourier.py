@@ -109,3 +109,23 @@ def test_cpu_forward_operator_can_be_installed(gpu, port):
     assert installed_err < 2e-6, installed_err
     assert 2e-5 < exact_err < TOL, exact_err
     assert abs(rel_c(y.host(), (yr, yi)) - exact_err) < 1e-9
+
+
+@pytest.mark.parametrize("B,n", [(1, 1), (3, 2), (5, 7), (64, 784), (33, 97), (300, 1024), (4096, 784)])
+def test_transform_of_real_samples_through_half_the_columns(gpu, port, B, n):
+    """cnet_cdft_fwd_real_input: columns 0 .. n/2 by the matrix product, the rest as conjugates.  Against the full transform of
+    the same samples (to rounding: the stored twiddles are symmetric under q -> n - q up to their last bit), against the CPU
+    path, and the symmetry itself to the bit."""
+    xr = seeded(port, 7 * B + n, (B, n))
+    x = ops.CMat.from_host(xr, np.zeros_like(xr))
+    full, half = ops.CMat.empty(B, n), ops.CMat.from_host(seeded(port, 1, (B, n)), seeded(port, 2, (B, n)))
+    ops.dft_fwd(x, full)
+    ops.dft_fwd_real_input(x, half)
+    fr, fi = full.host()
+    hr, hi = half.host()
+    assert rel_c((hr, hi), (fr, fi)) < 1e-6   # two roundings of the same sums
+    for q in range(1, (n - 1) // 2 + 1):
+        assert np.array_equal(hr[:, n - q], hr[:, q]) and np.array_equal(hi[:, n - q], -hi[:, q])
+    if B * n * n <= 1 << 27:
+        yr, yi = port.dft_fwd(xr, np.zeros_like(xr))
+        assert rel_c((hr, hi), (yr, yi)) < TOL
