@@ -406,6 +406,10 @@ def main():
         print(json.dumps({"counter_pass": True, "copy_bytes_read": rows * cols * 4, "copy_bytes_written": rows * cols * 4}))
         return
 
+    # no collector pauses inside the timed loops (one of 20 ms was seen to drain the queue in the middle of a loop)
+    import gc
+    gc.collect()
+    gc.disable()
     # Out of idle first: a device that has just been handed over runs its first ~25 steps (30 ms) of this workload up to 25 %
     # slower while its clocks come up (1.45 -> 1.18 ms per step, measured step by step with events).  Groups of 10 steps are
     # run until two in a row agree to 1 % (at most 0.5 s in all); the W warm-up steps and the K timed steps follow.
@@ -441,15 +445,19 @@ def main():
     # per-launch durations (HIP events around back-to-back launches of one kernel on the library's stream)
     kern = {}
     for name, (fn, ngemm) in launches.items():
-        a, b = ev.event(), ev.event()
         fn(); capi.sync()
-        ev.record(a)
-        for _ in range(args.steps):
-            fn()
-        ev.record(b)
-        ms = ev.elapsed_ms(a, b) / args.steps
+        groups = []   # five groups of K launches, the median group: one disturbed group does not decide the figure
+        for _ in range(5):
+            a, b = ev.event(), ev.event()
+            ev.record(a)
+            for _ in range(args.steps):
+                fn()
+            ev.record(b)
+            groups.append(ev.elapsed_ms(a, b) / args.steps)
+        ms = sorted(groups)[2]
         fl = 8.0 * B * N * K * ngemm
         kern[name] = {"ms": round(ms, 4), "flops": fl, "tflops": round(fl / ms / 1e9, 2)}
+    gc.enable()
     dom = max(kern, key=lambda k: kern[k]["ms"])
     traffic_table, traffic_at = measured_traffic()
     traffic = traffic_table.get(dom) if traffic_table else None
