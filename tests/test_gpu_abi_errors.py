@@ -331,6 +331,16 @@ def test_device_copy_caller_stream_and_upload_ordering(gpu, port):
     assert _status("cnet_memcpy_d2h_async", None, b.ptr, 16) == INVALID
     capi.call("cnet_graph_begin")
     assert _status("cnet_memcpy_d2h_async", host, b.ptr, 4 * n) == UNSUPPORTED
+    assert _status("cnet_upload_zero", b.ptr, 16) == UNSUPPORTED
     capi.call("cnet_graph_end", None)
+    # clearing on the upload stream, in order with the copies queued there: copy 7s, clear the first half, copy 7s to the end
+    assert _status("cnet_upload_zero", None, 16) == INVALID and _status("cnet_upload_zero", None, 0) == 0
+    pinned[:] = 7.0
+    capi.call("cnet_upload_async", a.ptr, host, 4 * n)
+    capi.call("cnet_upload_zero", a.ptr, 2 * n)
+    capi.call("cnet_upload_async", a.ptr + 3 * n, host, n)
+    capi.call("cnet_upload_sync")
+    got = a.download()
+    assert (got[: n // 2] == 0.0).all() and (got[n // 2:] == 7.0).all()
     del pinned
     capi.call("cnet_host_free", host)
