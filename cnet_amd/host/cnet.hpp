@@ -419,6 +419,13 @@ protected:
 	// input functions: the imaginary plane on the device is known to hold +0 only (a batch of real samples was fed and
 	// nothing has stepped or overwritten the values since); a FourierTrans on it then takes cnet_cdft_fwd_real_input
 	bool z_imag_zero_ = false;
+	// Data inputs (one row per sample) whose only consumer is a FourierTrans / TriangFourier: the backward pass of that
+	// transform, the gather and the update of the input are work whose results the next batch overwrites.  They are left
+	// out (lazy_bwd_: a backward pass has skipped them; lazy_upd_: an update at rate lazy_lr_ has skipped them too) and
+	// done later, from the gradients the transform's consumers left, if anything looks before the next batch arrives
+	// (CNet::materializeLazy).  lazy_now_ / lazy_skip_now_ are the decisions for the pass that is being queued.
+	bool lazy_bwd_ = false, lazy_upd_ = false, lazy_now_ = false, lazy_skip_now_ = false;
+	float lazy_lr_ = 0.f;
 	int rows_ = 0;           // batch rows of this node's output (1 for parameter nodes)
 	float *out_ = NULL;      // 2 planes [rows][out_size]: what consumers read
 	float *out_re() const { return out_; }
@@ -714,32 +721,96 @@ class CNet {
 		}
 		if (!src.empty()) ck(cnet_add_multi((int) src.size(), src.data(), dst.data(), len.data()), "cnet_add_multi");
 	}
-	// decides, for the backward pass about to be queued, which input functions leave their gradient with the consumer;
-	// true when every candidate does (the state a recorded backward pass stands for)
+	// ---- lazy data inputs (see CFunc::lazy_bwd_) ----
+	bool lazy_inputs_ = true;
+	// the transform on a data input whose backward pass can wait, or NULL
+	CFunc *lazyHead(CFunc *d) const {
+		if (!lazy_inputs_ || d->typeId() != isInput || !d->trainable_ || isParameter(d) || d->no_outputs() != 1) return NULL;
+		CFunc *f = d->next_func_[0];
+		if ((f->typeId() != isFourier && f->typeId() != isTrianFourier) || f->rows_ != d->rows_ || f->slots_.size() != 1 ||
+				f->slots_[0].producer != d || f->no_outputs() == 0)
+			return NULL;
+		return f;
+	}
+	// does now what was left out: the transform's backward pass from the gradients its consumers left (they stay where they
+	// are until the next backward pass), then the gather or, when an update was asked for in the meantime, that update
+	void materializeLazy() {
+		for (auto d : inputs_) {
+			if (!d->lazy_bwd_) {
+				d->lazy_upd_ = false;
+				continue;
+			}
+			CFunc *f = d->next_func_[0];
+			CFunc::Slot &own = d->slots_[0], &u = upstream(d, 0);
+			f->lazy_skip_now_ = false;
+			nodeBackward(f, true);
+			d->lazy_bwd_ = false;
+			const int64_t n = (int64_t) own.rows * own.len;
+			if (d->lazy_upd_) {  // the node's own planes are clear: the step reads the gradient where it is, nothing to clear
+				ck(cnet_sgd_update(own.z, own.z + n, u.g(2), u.g(3), n, d->lazy_lr_, 0), "cnet_sgd_update");
+				d->lazy_upd_ = false;
+			} else if (defer_gathers_ && d->grad_clean_ && !d->pending_) {
+				d->pending_ = &u;
+			} else {
+				const float *src = u.g(2);
+				float *dst = own.g(2);
+				const int64_t len = 2 * n;
+				ck(cnet_add_multi(1, &src, &dst, &len), "cnet_add_multi");
+				d->grad_clean_ = false;
+			}
+		}
+	}
+	// a new batch is about to overwrite the values of `d`: work that was left out for it and whose result would be
+	// overwritten is dropped; a backward pass without an update still owes its gradient
+	void beforeFeed(CFunc *d) {
+		if (d->lazy_bwd_ && d->lazy_upd_) d->lazy_bwd_ = d->lazy_upd_ = false;
+		else if (d->lazy_bwd_) materializeLazy();
+	}
+	// decides, for the backward pass about to be queued, which input functions leave their gradient with the consumer and
+	// which data inputs are left out altogether; true when every candidate does (the state a recorded backward pass stands
+	// for)
 	bool planDeferral(bool allow) {
 		bool all = true;
 		for (auto f : inputs_) {
-			f->defer_now_ = allow && defer_gathers_ && deferrable(f) && f->grad_clean_ && !f->pending_;
-			if (deferrable(f) && !f->defer_now_) all = false;
+			CFunc *head = allow ? lazyHead(f) : NULL;
+			f->lazy_now_ = head && f->grad_clean_ && !f->pending_ && !f->lazy_bwd_ && !f->lazy_upd_;
+			if (head) head->lazy_skip_now_ = f->lazy_now_;
+			f->defer_now_ = !f->lazy_now_ && allow && defer_gathers_ && deferrable(f) && f->grad_clean_ && !f->pending_;
+			if (lazyHead(f) ? !f->lazy_now_ : (deferrable(f) && !f->defer_now_)) all = false;
 		}
 		return all;
 	}
 	// after the pass has been queued (or replayed): note where the gradients are
 	void noteDeferred() {
 		for (auto f : inputs_) {
-			if (f->defer_now_) f->pending_ = &upstream(f, 0);
-			else if (f->trainable_ && f->no_outputs() > 0) f->grad_clean_ = false;
-			f->defer_now_ = false;
+			if (f->lazy_now_) {
+				f->lazy_bwd_ = true;
+				f->next_func_[0]->lazy_skip_now_ = false;
+			} else if (f->defer_now_) {
+				f->pending_ = &upstream(f, 0);
+			} else if (f->trainable_ && f->no_outputs() > 0) {
+				f->grad_clean_ = false;
+			}
+			f->defer_now_ = f->lazy_now_ = false;
 		}
 	}
+	// the state a recorded update stands for: every gradient that can be is still with its consumer, every data input that
+	// can be is waiting for its backward pass
 	bool allPending() const {
-		for (auto f : inputs_)
-			if (deferrable(f) && !f->pending_) return false;
+		for (auto f : inputs_) {
+			if (lazyHead(f)) {
+				if (!f->lazy_bwd_ || f->lazy_upd_) return false;
+			} else if (deferrable(f) && !f->pending_) {
+				return false;
+			}
+		}
 		return true;
 	}
 	bool allCleanNonePending() const {
-		for (auto f : inputs_)
+		for (auto f : inputs_) {
+			if (f->lazy_bwd_ || f->lazy_upd_) return false;
 			if (deferrable(f) && (!f->grad_clean_ || f->pending_)) return false;
+		}
 		return true;
 	}
 	SimpleRand rand_{(uint64_t) clock()};  // upstream ComplexNet::rand_ (impl/cnet.h:56): the coin of sample()
@@ -946,6 +1017,7 @@ public:
 			f->rows_ = 0;
 			f->pending_ = NULL;
 			f->grad_clean_ = false;
+			f->lazy_bwd_ = f->lazy_upd_ = f->lazy_now_ = f->lazy_skip_now_ = false;
 		}
 		batch_ = 0;
 		d_labels_ = NULL;
@@ -1247,6 +1319,7 @@ private:
 			return;
 		}
 		if ((t == isInput || t == isEmbedding) && !f->trainable_) return;  // nothing steps it: nothing to gather
+		if (f->lazy_now_ || f->lazy_skip_now_) return;  // left out for now (see CFunc::lazy_bwd_)
 		if (t == isInput) {  // impl/cinput.h:54-65: gathers dzs only, and keeps adding until the next update
 			// Both dz* planes of a consumer's slot are adjacent and dense, as they are in the node's own block: one array per
 			// consumer.  Nothing in the backward pass reads what an input function gathers, so the gathers of all of them
@@ -1470,6 +1543,7 @@ public:
 	void fetch(CFunc *f, int b) {
 		requireAllocated("fetch");
 		if (b < 0 || b >= batch_) throw std::out_of_range("fetch: batch index");
+		materializeLazy();
 		if (f->pending_) flushPending();
 		settleUploads();
 		ck(cnet_sync(), "cnet_sync");
@@ -1574,8 +1648,14 @@ public:
 			g.step_lr = l_rate;
 		}
 		ck(cnet_graph_launch(g.step), "cnet_graph_launch");
-		for (auto f : inputs_)  // what the update inside the recording does to the host's picture of the inputs
-			if (f->trainable_) f->z_imag_zero_ = false;
+		for (auto f : inputs_) {  // what the steps inside the recording do to the host's picture of the inputs
+			if (!f->trainable_) continue;
+			f->z_imag_zero_ = false;
+			if (lazyHead(f)) {  // the recording was made in the usual state: its backward pass and update left these out
+				f->lazy_bwd_ = f->lazy_upd_ = true;
+				f->lazy_lr_ = l_rate;
+			}
+		}
 	}
 
 private:
@@ -1588,6 +1668,7 @@ private:
 		if (batch.size() != batch_ || batch.noOfLabels() != batch_) throw std::invalid_argument("gpuForward: batch size differs from allocateOnGpu");
 		if (batch.sampleDim() != cin->input().length_) throw std::invalid_argument("gpuForward: sample dimension differs from the input length");
 		(void) outp;
+		beforeFeed(cin);
 		CFunc::Slot &s = cin->slots_[0];
 		Stage &staged = stage_[1 - active_];
 		if (staged.holds == &batch) {
@@ -1673,6 +1754,7 @@ public:
 		requireAllocated("gpuSetInput");
 		if (cin->rows_ != batch_ || batch.size() != batch_ || batch.sampleDim() != cin->input().length_)
 			throw std::invalid_argument("gpuSetInput: " + cin->getName() + " is not a data input of this batch shape");
+		beforeFeed(cin);
 		CFunc::Slot &s = cin->slots_[0];
 		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
 		const bool real_only = batch.imagIsZero() && !send_zero_planes_;
@@ -1708,6 +1790,7 @@ public:
 	}
 	bool GpuForward() {
 		requireAllocated("GpuForward");
+		materializeLazy();  // a forward pass on values that were not replaced reads what the update made of them
 		if (use_graphs_) settleUploads();  // a recording cannot hold the wait
 		{
 			StepGraphs &g = graphs_[active_];  // a recording holds one of the two transforms of a data input
@@ -1750,7 +1833,8 @@ public:
 		requireAllocated("gpuBackward");
 		settleUploads();
 		planGradients();
-		flushPending();  // this pass overwrites the planes a deferred gradient sits in
+		materializeLazy();  // this pass overwrites the gradients a transform left out would start from
+		flushPending();     // ... and the planes a deferred gradient sits in
 		const bool nominal = planDeferral(true);
 		auto body = [&] {
 			gather_src_.clear();  // nothing is left over from a pass that threw
@@ -1775,6 +1859,7 @@ public:
 			g.upd = NULL;
 		}
 		g.upd_lr = l_rate;
+		if (input_dz_dirty_) materializeLazy();  // the first moment of every input function is cleared here: all of them take part
 		if (input_dz_dirty_)  // this update also clears the first moment: not what a recording made without it does
 			for (auto &sg : graphs_)
 				if (sg.upd) {
@@ -1789,7 +1874,7 @@ public:
 				std::vector<float *> zr, zi, dr, di;
 				std::vector<int64_t> len;
 				for (auto f : inputs_) {
-					if (!f->trainable_ || (f->pending_ != NULL) != (deferred != 0)) continue;
+					if (!f->trainable_ || f->lazy_bwd_ || (f->pending_ != NULL) != (deferred != 0)) continue;
 					CFunc::Slot &s = f->slots_[0];
 					const CFunc::Slot &gsrc = deferred ? *f->pending_ : s;
 					const size_t n = (size_t) s.rows * s.len;
@@ -1810,6 +1895,10 @@ public:
 		else body();
 		for (auto f : inputs_) {
 			if (!f->trainable_) continue;
+			if (f->lazy_bwd_ && !f->lazy_upd_) {  // its step waits with its backward pass
+				f->lazy_upd_ = true;
+				f->lazy_lr_ = l_rate;
+			}
 			f->pending_ = NULL;
 			f->grad_clean_ = true;
 			f->z_imag_zero_ = false;  // stepped: complex from here on
@@ -1832,7 +1921,10 @@ public:
 	// pass; same results to rounding).  Off: both halves are computed, as upstream does.  Recordings are dropped, since
 	// they hold the kernels of the other setting.
 	void conjugateGradients(bool on) {
-		if (on != conjugate_gradients_ && batch_) dropGraphs();
+		if (on != conjugate_gradients_ && batch_) {
+			dropGraphs();
+			materializeLazy();  // with the kernels of the setting the backward pass ran under
+		}
 		conjugate_gradients_ = on;
 	}
 	bool conjugateGradients() const { return conjugate_gradients_; }
@@ -1865,9 +1957,24 @@ public:
 		if (on == defer_gathers_) return;
 		if (batch_) {
 			dropGraphs();
+			materializeLazy();
 			flushPending();
 		}
 		defer_gathers_ = on;
+	}
+	// A data input that feeds a FourierTrans or TriangFourier and nothing else: the backward pass of the transform and the
+	// gather and step of the input (upstream steps data inputs like parameters, impl/cnet.h:413-421) produce values that
+	// the next batch overwrites.  By default they are left out and done only if something looks first (fetch,
+	// getInputsFromGpu, a forward pass on the same values, a second backward pass, an Adam-style step, the per-sample
+	// calls), from the gradients the transform's consumers left; a new batch drops them.  Off: done at once, as upstream
+	// does.  Same observable values either way.
+	void lazyDataInputs(bool on) {
+		if (on == lazy_inputs_) return;
+		if (batch_) {
+			dropGraphs();
+			materializeLazy();
+		}
+		lazy_inputs_ = on;
 	}
 	// Upstream steps every input function, the data input included (impl/cnet.h:413-421), and therefore runs the backward
 	// pass all the way down to it.  An input function marked not trainable is left alone by gpuUpdateInputs /
@@ -1879,6 +1986,7 @@ public:
 		if (!f || !f->is_input_) throw std::invalid_argument("setInputTrainable: not an input function of this net");
 		if (f->trainable_ != on && batch_) {
 			dropGraphs();
+			materializeLazy();
 			flushPending();
 		}
 		f->trainable_ = on;
@@ -1887,6 +1995,7 @@ public:
 	// function: the first moment lives in the node's dz planes, dz* is cleared, dz is kept.
 	void gpuAdamUpdate(float l_rate, float beta, int t) {
 		requireAllocated("gpuAdamUpdate");
+		materializeLazy();
 		for (auto f : inputs_) {
 			if (!f->trainable_) continue;
 			CFunc::Slot &s = f->slots_[0];
@@ -2049,6 +2158,7 @@ public:
 		copyInputsToGpu();
 		// upstream forward() clears the gradients of every non-input function (impl/cnet.h:372-374); the batched path
 		// never needs that (first contribution overwrites), the per-sample views do
+		materializeLazy();
 		flushPending();  // before the planes a deferred gradient sits in are cleared
 		for (auto f : func_list_)
 			if (!f->is_input_)
@@ -2063,6 +2173,7 @@ public:
 		// the device-side loss, which is refreshed here so getLoss() matches the label in use
 		for (auto f : outputs_)
 			if (f->typeId() == isCrossEntropy) nodeForward(f);
+		materializeLazy();
 		flushPending();
 		planDeferral(false);  // every host view is read right after the pass: nothing to gain from deferring
 		gather_src_.clear();

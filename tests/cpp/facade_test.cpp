@@ -1045,14 +1045,17 @@ static void test_deferred_gathers() {
 		return;
 	}
 	SyntheticReader data(n, 8 * B, classes);
-	std::vector<float> trace[4];
-	for (int variant = 0; variant < 4; ++variant) {  // 0: deferred, 1: gathered at once, 2: deferred + recorded phases, 3: gathered + recorded phases
+	std::vector<float> trace[6];
+	// 0: deferred, 1: gathered at once, 2: deferred + recorded phases, 3: gathered + recorded phases; 4, 5: as 0, 1 with the
+	// backward pass and step of the data input done at once as well (CNet::lazyDataInputs(false))
+	for (int variant = 0; variant < 6; ++variant) {
 		CNet net;
 		int inp, outp;
 		build_readme(net, n, classes, &inp, &outp);
 		net.allocateOnGpu(B);
 		net.deferGathers(variant % 2 == 0);
-		if (variant >= 2) net.useGraphs(true);
+		if (variant == 2 || variant == 3) net.useGraphs(true);
+		if (variant >= 4) net.lazyDataInputs(false);
 		CInput *cin = (CInput *) net[inp];
 		CrossEntropy *cen = (CrossEntropy *) net[outp];
 		SyntheticReader reader = data;
@@ -1084,11 +1087,24 @@ static void test_deferred_gathers() {
 		net.gpuUpdateInputs(0.05f / B);
 		gradients();                                   // cleared by the update
 		weights();
+		step(true);
+		net.GpuForward();                              // a forward pass on the values the update left (no new batch)
+		out.push_back(net.getLoss(cen, NULL));
+		net.fetch(cin, 2);                             // the stepped data input itself
+		out.insert(out.end(), cin->input().real_, cin->input().real_ + 2 * n);
+		step(true);
+		step(false);
+		reader.nextBatch(batch);                       // a new batch after a backward pass that no update followed:
+		net.gpuForward(cin, cen, batch);               // the gradient of the old one is still owed
+		net.gpuBackward();
+		net.gpuUpdateInputs(0.05f / B);
+		out.push_back(net.getLoss(cen, NULL));
+		weights();
 		step(false);
 		net.gpuAdamUpdate(0.01f / B, 0.9f, 0);         // an Adam-style step takes the gradient from where it is
 		step(true);                                    // (this update also clears the first moment)
 		weights();
-		if (variant < 2) {                             // a whole recorded step, also right after a pass without update
+		if (variant < 2 || variant >= 4) {             // a whole recorded step, also right after a pass without update
 			reader.nextBatch(batch);
 			for (int k = 0; k < 3; ++k) net.gpuTrainStep(cin, cen, batch, 0.05f / B);
 			step(false);
@@ -1096,9 +1112,13 @@ static void test_deferred_gathers() {
 			net.gpuTrainStep(cin, cen, batch, 0.05f / B);
 			out.push_back(net.getLoss(cen, NULL));
 			weights();
+			net.fetch(cin, 0);                         // what the last recorded step left in the data input
+			out.insert(out.end(), cin->input().real_, cin->input().real_ + 2 * n);
+			gradients();
 		}
 	}
 	expect("deferred and immediate gathers: same losses, gradients and weights", trace[0] == trace[1] && trace[0].size() > 1000);
+	expect("the data input's backward pass and step left out until something looks, against done at once", trace[0] == trace[4] && trace[1] == trace[5]);
 	expect("the same with recorded phases", trace[2] == trace[3] && !trace[2].empty());
 	expect("recorded phases agree with launches one by one", std::equal(trace[2].begin(), trace[2].end(), trace[0].begin()));
 	bool finite = true;
