@@ -1514,6 +1514,7 @@ public:
 	bool copyInputsToGpu() {
 		requireAllocated("copyInputsToGpu");
 		for (auto f : inputs_) {
+			beforeFeed(f);
 			f->z_imag_zero_ = false;
 			CFunc::Slot &s = f->slots_[0];
 			float *z = s.z;
