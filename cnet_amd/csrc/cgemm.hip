@@ -917,10 +917,16 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t plane_rsrc(const float *p, uns
 	return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p), 0, bytes, 0x00020000);
 }
 
+// how the lanes of cgemm_skinny_kernel step through the two operands (elements), and the length of each plane (bytes)
+struct SkinnyStrides {
+	unsigned a_kstride, a_mstride, b_kstride, b_nstride, a_bytes, b_bytes;
+};
+
+// the tile numbered `bx` of the product `args`; red = W x 2 x 4 x 64 floats of LDS ([W][re, im][4][64])
 template <int W, bool A_V4, bool B_V4>
-__global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs args, unsigned a_kstride, unsigned a_mstride,
-		unsigned b_kstride, unsigned b_nstride, unsigned a_bytes, unsigned b_bytes) {
-	__shared__ float red[W * 2 * 4 * 64];  // [W][re, im][4][64]
+__device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyStrides &st, const int bx, float *red) {
+	const unsigned a_kstride = st.a_kstride, a_mstride = st.a_mstride, b_kstride = st.b_kstride, b_nstride = st.b_nstride;
+	const unsigned a_bytes = st.a_bytes, b_bytes = st.b_bytes;
 	constexpr int DEPTH = 3;
 	// the wavefront number as a scalar: the K range, the loop over it and its branches then run on the scalar unit
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -929,8 +935,8 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 	batch_offset(pb, args);
 	// Consecutive workgroup numbers go round-robin to the XCDs: give each XCD a contiguous run of tiles, row tiles
 	// fastest, so that the tiles sharing columns of B meet in one L2 and each XCD reads its own part of B only.
-	const int total = args.tiles_m * args.tiles_n, xcd = blockIdx.x % NUM_XCD, share = total / NUM_XCD, extra = total % NUM_XCD;
-	const int tile = xcd * share + min(xcd, extra) + blockIdx.x / NUM_XCD;
+	const int total = args.tiles_m * args.tiles_n, xcd = bx % NUM_XCD, share = total / NUM_XCD, extra = total % NUM_XCD;
+	const int tile = xcd * share + min(xcd, extra) + bx / NUM_XCD;
 	const int tile_n = tile / args.tiles_m, tile_m = tile - tile_n * args.tiles_m;
 	const int m0 = tile_m * 16, n0 = tile_n * 16;
 	// lanes beyond the edge of C read the last valid row / column again; their results are not stored
@@ -1034,14 +1040,36 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs ar
 }
 
 template <int W, bool A_V4, bool B_V4>
-int launch_skinny(const CgemmArgs &args, bool a_mcontig, bool b_ncontig, int nprob, int batch) {
+__global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs args, const SkinnyStrides st) {
+	__shared__ float red[W * 2 * 4 * 64];
+	skinny_tile<W, A_V4, B_V4>(args, st, blockIdx.x, red);
+}
+
+// Two unrelated small products in one launch (the input gradient and the weight gradient of a narrow Linear layer, each
+// a few microseconds of work behind a launch that costs as much): workgroups [0, tiles0) take the tiles of the first,
+// the others those of the second.  Neither is cut along K or batched (blockIdx.z = 0); blockIdx.y is the problem of
+// a pair, as in the plain kernel.
+template <int W, bool A_V4, bool B_V4>
+__global__ __launch_bounds__(64 * W) void cgemm_skinny_two_kernel(const CgemmArgs args0, const SkinnyStrides st0, const int tiles0,
+		const CgemmArgs args1, const SkinnyStrides st1) {
+	__shared__ float red[W * 2 * 4 * 64];
+	if ((int) blockIdx.x < tiles0) skinny_tile<W, A_V4, B_V4>(args0, st0, blockIdx.x, red);
+	else skinny_tile<W, A_V4, B_V4>(args1, st1, blockIdx.x - tiles0, red);
+}
+
+SkinnyStrides skinny_strides(const CgemmArgs &args, bool a_mcontig, bool b_ncontig) {
 	// elements from the first to one past the last of an operand plane
 	const long span_a = a_mcontig ? (args.K - 1) * args.lda + args.M : (args.M - 1) * args.lda + args.K;
 	const long span_b = b_ncontig ? (args.K - 1) * args.ldb + args.N : (args.N - 1) * args.ldb + args.K;
+	return SkinnyStrides{a_mcontig ? (unsigned) args.lda : 1u, a_mcontig ? 1u : (unsigned) args.lda, b_ncontig ? (unsigned) args.ldb : 1u,
+			b_ncontig ? 1u : (unsigned) args.ldb, (unsigned) (4 * span_a), (unsigned) (4 * span_b)};
+}
+
+template <int W, bool A_V4, bool B_V4>
+int launch_skinny(const CgemmArgs &args, bool a_mcontig, bool b_ncontig, int nprob, int batch) {
 	auto kern = cgemm_skinny_kernel<W, A_V4, B_V4>;
 	hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, nprob, batch * args.splits), dim3(64 * W), 0, cnet::rt().stream, args,
-			a_mcontig ? (unsigned) args.lda : 1u, a_mcontig ? 1u : (unsigned) args.lda, b_ncontig ? (unsigned) args.ldb : 1u,
-			b_ncontig ? 1u : (unsigned) args.ldb, (unsigned) (4 * span_a), (unsigned) (4 * span_b));
+			skinny_strides(args, a_mcontig, b_ncontig));
 	CNET_LAUNCH_CHECK();
 	if (args.splits > 1) {
 		dim3 rgrid((unsigned) ((2L * args.M * args.N + 255) / 256), nprob, batch);
@@ -1105,6 +1133,41 @@ double skinny_us(const CgemmArgs &args, int nprob, int batch) {
 	return (3.0 + 0.0075 * k_slice) * std::max(1.0, wgs / (2.0 * cus)) + (args.splits > 1 ? 6.0 : 0.0);
 }
 
+// which instantiation of cgemm_skinny_kernel a planned product takes: float4 loads along K per operand, wavefronts per tile
+struct SkinnyVariant {
+	bool a_v4, b_v4;
+	int w;
+	bool operator==(const SkinnyVariant &o) const { return a_v4 == o.a_v4 && b_v4 == o.b_v4 && w == o.w; }
+};
+
+SkinnyVariant skinny_variant(bool a_mcontig, bool b_ncontig, const CgemmArgs &args, int nprob, int batch) {
+	SkinnyVariant v;
+	v.a_v4 = !a_mcontig && args.lda % 4 == 0 && args.stride_a % 4 == 0 && args.K % 4 == 0;
+	v.b_v4 = !b_ncontig && args.ldb % 4 == 0 && args.stride_b % 4 == 0 && args.K % 4 == 0;
+	for (int q = 0; q < nprob; ++q) {
+		v.a_v4 = v.a_v4 && cnet::aligned16(args.p[q].a_re) && cnet::aligned16(args.p[q].a_im);
+		v.b_v4 = v.b_v4 && cnet::aligned16(args.p[q].b_re) && cnet::aligned16(args.p[q].b_im);
+	}
+	// Four wavefronts per tile, which leaves room for several tiles on a compute unit; eight (two per SIMD, each other's
+	// latency cover) when there are so few tiles that most units hold one at most (64 x 784 x 784: 9.0 -> 8.5 us; with
+	// three tiles per unit, 256 x 784 x 784: 19.8 -> 21.6 us, so not there).
+	static const int forced_w = [] {
+		const char *e = getenv("CNET_CGEMM_SKINNY_W");  // tuning override: 4, 8 or 16 wavefronts per tile
+		return e ? atoi(e) : 0;
+	}();
+	const long wgs = (long) args.tiles_m * args.tiles_n * nprob * batch * args.splits;
+	v.w = forced_w == 4 || forced_w == 8 || forced_w == 16 ? forced_w
+			: (args.splits == 1 && 2 * wgs <= 3 * cnet::rt().prop.multiProcessorCount && args.K >= 256) ? 8 : 4;
+	return v;
+}
+
+// expands to CALL<W, A_V4, B_V4> ARGS for the variant v
+#define CNET_SKINNY_PICK(v, CALL, ARGS)                                                                                          \
+	((v).w == 16 ? CNET_SKINNY_PICK_W(v, 16, CALL, ARGS) : (v).w == 8 ? CNET_SKINNY_PICK_W(v, 8, CALL, ARGS) : CNET_SKINNY_PICK_W(v, 4, CALL, ARGS))
+#define CNET_SKINNY_PICK_W(v, W, CALL, ARGS)                                                                                     \
+	((v).a_v4 ? ((v).b_v4 ? CALL<W, true, true> ARGS : CALL<W, true, false> ARGS)                                                \
+			  : ((v).b_v4 ? CALL<W, false, true> ARGS : CALL<W, false, false> ARGS))
+
 // true and *rc set when the product was small enough for cgemm_skinny_kernel
 bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int nprob, int batch, int *rc) {
 	CgemmArgs args;
@@ -1116,28 +1179,40 @@ bool try_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int npro
 			return true;
 		}
 	}
-	bool a_v4 = !a_mcontig && args.lda % 4 == 0 && args.stride_a % 4 == 0 && args.K % 4 == 0;
-	bool b_v4 = !b_ncontig && args.ldb % 4 == 0 && args.stride_b % 4 == 0 && args.K % 4 == 0;
-	for (int q = 0; q < nprob; ++q) {
-		a_v4 = a_v4 && cnet::aligned16(args.p[q].a_re) && cnet::aligned16(args.p[q].a_im);
-		b_v4 = b_v4 && cnet::aligned16(args.p[q].b_re) && cnet::aligned16(args.p[q].b_im);
-	}
-#define CNET_SKINNY(W)                                                                                         \
-	(a_v4 ? (b_v4 ? launch_skinny<W, true, true>(args, a_mcontig, b_ncontig, nprob, batch)                     \
-				  : launch_skinny<W, true, false>(args, a_mcontig, b_ncontig, nprob, batch))                   \
-		  : (b_v4 ? launch_skinny<W, false, true>(args, a_mcontig, b_ncontig, nprob, batch)                    \
-				  : launch_skinny<W, false, false>(args, a_mcontig, b_ncontig, nprob, batch)))
-	// Four wavefronts per tile, which leaves room for several tiles on a compute unit; eight (two per SIMD, each other's
-	// latency cover) when there are so few tiles that most units hold one at most (64 x 784 x 784: 9.0 -> 8.5 us; with
-	// three tiles per unit, 256 x 784 x 784: 19.8 -> 21.6 us, so not there).
-	static const int forced_w = [] {
-		const char *e = getenv("CNET_CGEMM_SKINNY_W");  // tuning override: 4, 8 or 16 wavefronts per tile
-		return e ? atoi(e) : 0;
+	const SkinnyVariant v = skinny_variant(a_mcontig, b_ncontig, args, nprob, batch);
+	*rc = CNET_SKINNY_PICK(v, launch_skinny, (args, a_mcontig, b_ncontig, nprob, batch));
+	return true;
+}
+
+template <int W, bool A_V4, bool B_V4>
+int launch_skinny_two(const CgemmArgs &args0, const SkinnyStrides &st0, const CgemmArgs &args1, const SkinnyStrides &st1, int nprob) {
+	const int tiles0 = args0.tiles_m * args0.tiles_n, tiles1 = args1.tiles_m * args1.tiles_n;
+	auto kern = cgemm_skinny_two_kernel<W, A_V4, B_V4>;
+	hipLaunchKernelGGL(kern, dim3(tiles0 + tiles1, nprob, 1), dim3(64 * W), 0, cnet::rt().stream, args0, st0, tiles0, args1, st1);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
+// Two products that are both small enough for cgemm_skinny_kernel, neither cut along K, and that take the same
+// instantiation of it, go out as one launch: true and *rc set.  Otherwise nothing is launched.
+bool try_skinny_two(bool a_mcontig0, bool b_ncontig0, const CgemmArgs &proto0, bool a_mcontig1, bool b_ncontig1, const CgemmArgs &proto1,
+		int nprob, int *rc) {
+	static const bool enabled = [] {
+		const char *e = getenv("CNET_CGEMM_SKINNY_TWO");  // tuning override: 0 launches the two products one after the other
+		return !e || atoi(e) != 0;
 	}();
-	const long wgs = (long) args.tiles_m * args.tiles_n * nprob * batch * args.splits;
-	const int w = forced_w ? forced_w : (args.splits == 1 && 2 * wgs <= 3 * cnet::rt().prop.multiProcessorCount && args.K >= 256) ? 8 : 4;
-	*rc = w == 16 ? CNET_SKINNY(16) : w == 8 ? CNET_SKINNY(8) : CNET_SKINNY(4);
-#undef CNET_SKINNY
+	if (!enabled || proto0.M <= 0 || proto0.N <= 0 || proto0.K <= 0 || proto1.M <= 0 || proto1.N <= 0 || proto1.K <= 0) return false;
+	CgemmArgs args0, args1;
+	if (!plan_skinny(a_mcontig0, b_ncontig0, proto0, nprob, 1, args0) || !plan_skinny(a_mcontig1, b_ncontig1, proto1, nprob, 1, args1))
+		return false;
+	if (args0.splits != 1 || args1.splits != 1) return false;
+	// together they must still be a small launch
+	if (((long) args0.tiles_m * args0.tiles_n + (long) args1.tiles_m * args1.tiles_n) * nprob > 4L * cnet::rt().prop.multiProcessorCount)
+		return false;
+	const SkinnyVariant v0 = skinny_variant(a_mcontig0, b_ncontig0, args0, nprob, 1), v1 = skinny_variant(a_mcontig1, b_ncontig1, args1, nprob, 1);
+	if (!(v0 == v1)) return false;
+	const SkinnyStrides st0 = skinny_strides(args0, a_mcontig0, b_ncontig0), st1 = skinny_strides(args1, a_mcontig1, b_ncontig1);
+	*rc = CNET_SKINNY_PICK(v0, launch_skinny_two, (args0, st0, args1, st1, nprob));
 	return true;
 }
 
@@ -1464,12 +1539,23 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 	return pick_tile<true, false, 1>(a, nprob, batch);
 }
 
+static CgemmArgs pair_args(int nprob, int M, int N, int K, const float *const a_re[2], const float *const a_im[2], long lda,
+		const float *const b_re[2], const float *const b_im[2], long ldb, const bool conj_b[2], float *const c_re[2], float *const c_im[2],
+		long ldc, int accumulate, int tri, int mirror);
+
 // Used by cdft.hip
 int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
 		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
 		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri, int mirror) {
 	if (tri && N != K) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: a triangular operand must be square");
 	if (mirror && nprob != 1) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: a mirrored product is one problem");
+	CgemmArgs a = pair_args(nprob, M, N, K, a_re, a_im, lda, b_re, b_im, ldb, conj_b, c_re, c_im, ldc, accumulate, tri, mirror);
+	return cgemm_dispatch(a_mcontig, b_ncontig, a, nprob, 1);
+}
+
+static CgemmArgs pair_args(int nprob, int M, int N, int K, const float *const a_re[2], const float *const a_im[2], long lda,
+		const float *const b_re[2], const float *const b_im[2], long ldb, const bool conj_b[2], float *const c_re[2], float *const c_im[2],
+		long ldc, int accumulate, int tri, int mirror) {
 	CgemmArgs a;
 	a.tri = tri;
 	a.mirror = mirror;
@@ -1499,7 +1585,7 @@ int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, c
 	a.accumulate = accumulate;
 	a.tiles_m = a.tiles_n = 0;
 	a.stride_a = a.stride_b = a.stride_c = 0;
-	return cgemm_dispatch(a_mcontig, b_ncontig, a, nprob, 1);
+	return a;
 }
 
 }  // namespace cnet
@@ -1639,6 +1725,29 @@ int cnet_clinear_bwd_weight_sym(const float *g_dz_re, const float *g_dz_im, int6
 	float *cr[2] = {dw_dz_re, dw_dzs_re}, *ci[2] = {dw_dz_im, dw_dzs_im};
 	bool cj[2] = {false, false};
 	return cgemm_pair(true, true, 1, N, K, B, ar, ai, ldg, br, bi, ldx, cj, cr, ci, lddw, accumulate, 0, dw_dzs_re != nullptr ? MIRROR_CONJ : 0);
+}
+
+int cnet_clinear_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *x_re, const float *x_im, int64_t ldx,
+		const float *w_re, const float *w_im, int64_t ldw, float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
+		int accumulate_dx, float *dw_dz_re, float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im, int64_t lddw, int accumulate_dw, int B,
+		int K, int N) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B > 0 && K > 0 && N > 0);
+	CNET_CHECK_ARG(g_dz_re && g_dz_im && x_re && x_im && w_re && w_im);
+	CNET_CHECK_ARG(dx_dz_re && dx_dz_im && ((dx_dzs_re == nullptr) == (dx_dzs_im == nullptr)));
+	CNET_CHECK_ARG(dw_dz_re && dw_dz_im && ((dw_dzs_re == nullptr) == (dw_dzs_im == nullptr)));
+	CNET_CHECK_ARG(ldg >= N && ldx >= K && ldw >= K && lddx >= K && lddw >= K);
+	// the two products as cnet_clinear_bwd_input_sym and cnet_clinear_bwd_weight_sym set them up
+	const float *gr[2] = {g_dz_re, g_dz_re}, *gi[2] = {g_dz_im, g_dz_im};
+	const float *wr[2] = {w_re, w_re}, *wi[2] = {w_im, w_im}, *xr[2] = {x_re, x_re}, *xi[2] = {x_im, x_im};
+	float *dxr[2] = {dx_dz_re, dx_dzs_re}, *dxi[2] = {dx_dz_im, dx_dzs_im}, *dwr[2] = {dw_dz_re, dw_dzs_re}, *dwi[2] = {dw_dz_im, dw_dzs_im};
+	const bool cj[2] = {false, false};
+	CgemmArgs to_input = pair_args(1, B, K, N, gr, gi, ldg, wr, wi, ldw, cj, dxr, dxi, lddx, accumulate_dx, 0, dx_dzs_re ? MIRROR_CONJ : 0);
+	CgemmArgs to_weight = pair_args(1, N, K, B, gr, gi, ldg, xr, xi, ldx, cj, dwr, dwi, lddw, accumulate_dw, 0, dw_dzs_re ? MIRROR_CONJ : 0);
+	int rc = CNET_OK;
+	if (try_skinny_two(false, true, to_input, true, true, to_weight, 1, &rc)) return rc;
+	rc = cgemm_dispatch(false, true, to_input, 1, 1);
+	return rc != CNET_OK ? rc : cgemm_dispatch(true, true, to_weight, 1, 1);
 }
 
 }  // extern "C"

@@ -1381,6 +1381,11 @@ private:
 				CFunc::Slot &w = f->slots_[1];
 				const int K = a.len, N = f->out_size_;
 				const bool to_data = a.producer->wants_grad_, to_weight = w.producer->wants_grad_;
+				if (conjugate_gradients_ && to_data && to_weight) {  // both gradients in one call (one launch when both products are small)
+					ck(cnet_clinear_bwd_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.gs(2),
+							a.gs(3), K, acc, w.g(0), w.g(1), w.gs(2), w.gs(3), K, acc, rows, K, N), "cnet_clinear_bwd_sym");
+					break;
+				}
 				if (conjugate_gradients_) {  // dz* = conj(dz): one product each, written to both pairs of planes
 					if (to_data)
 						ck(cnet_clinear_bwd_input_sym(u.g(0), u.g(1), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.gs(2), a.gs(3), K, rows, K,

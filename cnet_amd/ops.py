@@ -138,6 +138,12 @@ def linear_bwd_weight_sym(g, x, dw, accumulate=0, mirror=True):
          accumulate)
 
 
+def linear_bwd_sym(g, x, w, dx, dw, accumulate_dx=0, accumulate_dw=0, mirror_dx=True, mirror_dw=True):
+    """Both gradients of a Linear in one call (one launch when both products are small)."""
+    call("cnet_clinear_bwd_sym", *g.p()[:2], g.ld, *x.p(), x.ld, *w.p(), w.ld, *_mirrored(dx, mirror_dx), dx.ld, accumulate_dx,
+         *_mirrored(dw, mirror_dw), dw.ld, accumulate_dw, g.rows, w.cols, w.rows)
+
+
 def dft_fwd(x, y, accumulate=0):
     call("cnet_cdft_fwd", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols, accumulate)
 

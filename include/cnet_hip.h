@@ -180,6 +180,16 @@ int cnet_clinear_bwd_input_sym(const float *g_dz_re, const float *g_dz_im, int64
 int cnet_clinear_bwd_weight_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *x_re, const float *x_im,
                                 int64_t ldx, float *dw_dz_re, float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im,
                                 int64_t lddw, int B, int K, int N, int accumulate);
+/* Both of them in one call, as upstream's LinearGpu::gpu_linear_backward forms every gradient of the layer in one call
+ * (gpu/reducegrad.cpp:309-322): dx (+)= g w and dw (+)= g^T x with the bits of the two calls above, each with its own
+ * accumulate flag.  When both products are small (a narrow layer at a small batch, 64 x 784 -> 10: each a few microseconds of
+ * work behind a launch that costs as much) and take the same kernel they go out as ONE launch; otherwise as the launches
+ * of the two calls above, one after the other. */
+int cnet_clinear_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *x_re, const float *x_im,
+                         int64_t ldx, const float *w_re, const float *w_im, int64_t ldw, float *dx_dz_re, float *dx_dz_im,
+                         float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int accumulate_dx, float *dw_dz_re,
+                         float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im, int64_t lddw, int accumulate_dw, int B, int K,
+                         int N);
 
 /* ---- FourierTrans as dense complex GEMM: replaces FourierGpu::gpu_fft_forward / gpu_fft_backward
  *      (gpu/reduce.cpp:25-35,160-187,382-393; gpu/reducegrad.cpp:45-48,324-336) and the root-table upload

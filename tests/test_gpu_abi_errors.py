@@ -46,6 +46,11 @@ def test_invalid_arguments_are_reported_not_fatal(gpu, port):
     assert _status("cnet_clinear_bwd_input_sym", g.p()[0], None, 8, *w.p(), 8, *dx.p(), 8, 4, 8, 8, 0) == INVALID
     assert _status("cnet_clinear_bwd_input_sym", *g.p()[:2], 4, *w.p(), 8, *dx.p(), 8, 4, 8, 8, 0) == INVALID      # ldg < N
     assert _status("cnet_clinear_bwd_weight_sym", *g.p()[:2], 8, *x.p(), 8, dx.p()[0], dx.p()[1], dx.p()[2], None, 8, 4, 8, 8, 0) == INVALID
+    dw = ops.Grad.empty(8, 8)
+    assert _status("cnet_clinear_bwd_sym", *g.p()[:2], 8, *x.p(), 8, *w.p(), 8, *dx.p(), 8, 0, dw.p()[0], dw.p()[1], None, dw.p()[3], 8, 0,
+                   4, 8, 8) == INVALID                                                                                # half a pair of dz* planes
+    assert _status("cnet_clinear_bwd_sym", *g.p()[:2], 8, *x.p(), 4, *w.p(), 8, *dx.p(), 8, 0, *dw.p(), 8, 0, 4, 8, 8) == INVALID   # ldx < K
+    assert _status("cnet_clinear_bwd_sym", *g.p()[:2], 8, *x.p(), 8, *w.p(), 8, *dx.p(), 8, 0, *dw.p(), 8, 0, 0, 8, 8) == INVALID   # no rows
     assert _status("cnet_cdft_bwd_sym", *g.p()[:2], 8, *dx.p(), 4, 4, 8, 0) == INVALID                               # lddx < n
     assert _status("cnet_ctriang_dft_bwd_sym", *g.p()[:2], 8, *dx.p(), 8, 4, 50000, 0) == INVALID
     assert _status("cnet_cdft_bwd_sym", *g.p()[:2], 8, *dx.p(), 8, 0, 8, 0) == 0                                     # no rows: nothing to do

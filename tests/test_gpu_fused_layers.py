@@ -60,6 +60,34 @@ def test_linear_cgelu_into_a_column_window(gpu, port):
             assert np.array_equal(plane[:, 8:8 + N], ref) and np.array_equal(plane[:, mask], base[:, mask])
 
 
+@pytest.mark.parametrize("B,K,N", [(64, 784, 10), (64, 16, 16), (33, 7, 5), (16, 64, 12), (1, 3, 2), (200, 40, 24), (64, 784, 784),
+                                   (1024, 256, 256)])
+def test_both_gradients_of_a_linear_in_one_call(gpu, port, B, K, N):
+    """cnet_clinear_bwd_sym against cnet_clinear_bwd_input_sym + cnet_clinear_bwd_weight_sym: same bits, whether the two
+    products share a launch (both small and on the same kernel: the first cases) or not, with each accumulate flag and with
+    the dz* planes of either result left out."""
+    gr, gi = seeded(port, B + 11, (B, N)), seeded(port, B + 12, (B, N))
+    g = ops.Grad.from_host([gr, gi, gr, -gi])
+    x = ops.CMat.from_host(seeded(port, K + 1, (B, K)), seeded(port, K + 2, (B, K)))
+    w = ops.CMat.from_host(seeded(port, N + 3, (N, K)), seeded(port, N + 4, (N, K)))
+    bx, bw = [seeded(port, 20 + p, (B, K)) for p in range(4)], [seeded(port, 30 + p, (N, K)) for p in range(4)]
+    for acc_x, acc_w, mir_x, mir_w in ((0, 0, True, True), (1, 0, True, False), (0, 1, False, True), (1, 1, True, True)):
+        dx0, dw0, dx1, dw1 = ops.Grad.from_host(bx), ops.Grad.from_host(bw), ops.Grad.from_host(bx), ops.Grad.from_host(bw)
+        ops.linear_bwd_input_sym(g, w, dx0, accumulate=acc_x, mirror=mir_x)
+        ops.linear_bwd_weight_sym(g, x, dw0, accumulate=acc_w, mirror=mir_w)
+        ops.linear_bwd_sym(g, x, w, dx1, dw1, accumulate_dx=acc_x, accumulate_dw=acc_w, mirror_dx=mir_x, mirror_dw=mir_w)
+        for a, b in ((dx0, dx1), (dw0, dw1)):
+            for pa, pb in zip(a.host(), b.host()):
+                assert np.array_equal(pa, pb), (acc_x, acc_w, mir_x, mir_w)
+    if B * K * N <= 1 << 24:   # the CPU path on the same pair
+        (xr, xi), (wr, wi) = x.host(), w.host()
+        dxo, dwo = port.linear_bwd(xr, xi, wr, wi, [gr, gi, gr, -gi])
+        dx1, dw1 = ops.Grad.empty(B, K), ops.Grad.empty(N, K)
+        ops.linear_bwd_sym(g, x, w, dx1, dw1)
+        assert rel_c(dx1.host()[0:2], dxo[0:2]) < TOL / 5 and rel_c(dx1.host()[2:4], dxo[2:4]) < TOL / 5
+        assert rel_c(dw1.host()[0:2], dwo[0:2]) < TOL / 5 and rel_c(dw1.host()[2:4], dwo[2:4]) < TOL / 5
+
+
 @pytest.mark.parametrize("overrides", [
     {"CNET_CGEMM_SKINNY": "0"},                            # small products on the block kernels (cut along K)
     {"CNET_CGEMM_TILE": "0", "CNET_CGEMM_COLSPLIT": "0"},  # 128 x 128 blocks
