@@ -180,6 +180,8 @@ class InputBatch : public Batch {
 	// Some sample added since the last clear() has an imaginary part that is not +0: while this is false the imaginary plane
 	// holds nothing but zeros and need not travel to the device (real-valued data such as images: half the upload).
 	bool imag_nonzero_ = false;
+	// every element of the imaginary plane, filled rows or not, holds +0: rows of real samples then need no write at all
+	bool imag_clean_ = false;
 	static bool anyBitSet(const float *p, size_t n) {
 		uint32_t acc = 0;
 		for (size_t k = 0; k < n; ++k) {
@@ -202,6 +204,8 @@ class InputBatch : public Batch {
 		}
 		real_data_ = (float *) p;
 		imag_data_ = real_data_ + (size_t) batch_size_ * sample_dim_;
+		std::fill(imag_data_, imag_data_ + (size_t) batch_size_ * sample_dim_, 0.f);
+		imag_clean_ = true;
 	}
 	void release() {
 		if (!real_data_) return;
@@ -217,6 +221,11 @@ class InputBatch : public Batch {
 			}
 			ticket_ = -1;
 		}
+	}
+	void noteImag(bool some_bit_set) {
+		if (!some_bit_set) return;
+		imag_nonzero_ = true;
+		imag_clean_ = false;
 	}
 	float *rowRe() { return real_data_ + (size_t) current_pos_ * sample_dim_; }
 	float *rowIm() { return imag_data_ + (size_t) current_pos_ * sample_dim_; }
@@ -235,9 +244,10 @@ public:
 		allocate();
 		if (o.real_data_) std::copy(o.real_data_, o.real_data_ + 2 * (size_t) batch_size_ * sample_dim_, real_data_);
 		imag_nonzero_ = o.imag_nonzero_;
+		imag_clean_ = o.imag_clean_;
 	}
 	InputBatch(InputBatch &&o) noexcept : Batch(std::move(o)), real_data_(o.real_data_), imag_data_(o.imag_data_), pinned_(o.pinned_),
-			ticket_(o.ticket_), imag_nonzero_(o.imag_nonzero_) {
+			ticket_(o.ticket_), imag_nonzero_(o.imag_nonzero_), imag_clean_(o.imag_clean_) {
 		o.real_data_ = o.imag_data_ = NULL;
 	}
 	InputBatch &operator=(InputBatch &&o) noexcept {
@@ -249,6 +259,7 @@ public:
 			pinned_ = o.pinned_;
 			ticket_ = o.ticket_;
 			imag_nonzero_ = o.imag_nonzero_;
+			imag_clean_ = o.imag_clean_;
 			o.real_data_ = o.imag_data_ = NULL;
 		}
 		return *this;
@@ -276,7 +287,7 @@ public:
 			re[k] = sample[k].real();
 			im[k] = sample[k].imag();
 		}
-		imag_nonzero_ = imag_nonzero_ || anyBitSet(im, sample.size());
+		noteImag(anyBitSet(im, sample.size()));
 		finishRow((int) sample.size(), label);
 	}
 	void add(std::initializer_list<std::complex<float> > list, int label) {
@@ -288,25 +299,33 @@ public:
 		settle();
 		std::copy(re, re + n, rowRe());
 		std::copy(im, im + n, rowIm());
-		imag_nonzero_ = imag_nonzero_ || anyBitSet(im, (size_t) n);
+		noteImag(anyBitSet(im, (size_t) n));
 		finishRow(n, label);
 	}
 	// Fill the next `count` rows from planar sample storage ([sample][dim] re and im): row k takes sample index[k] and
 	// label labels[index[k]].  The rows are independent copies, spread over the host threads when built with OpenMP (a
 	// batch of 4096 x 784 is 25 MB; one thread assembles it no faster than the device trains on it).
+	// im == NULL: every sample is real (the reader knows); the imaginary rows then only need clearing if something else
+	// than +0 has been in the plane since it was last all zeros.
 	void gather(const float *re, const float *im, const int *labels, const int *index, int count) {
 		assert(current_pos_ + count <= batch_size_);
 		settle();
 		const size_t dim = (size_t) sample_dim_;
 		float *dst_re = rowRe(), *dst_im = rowIm();
-		int nonzero = imag_nonzero_ ? 1 : 0;
+		const bool clear_im = !im && !imag_clean_;
+		int nonzero = 0;
 #pragma omp parallel for schedule(static) reduction(| : nonzero) if ((size_t) count * dim >= (1u << 18))
 		for (int k = 0; k < count; ++k) {
 			std::memcpy(dst_re + k * dim, re + index[k] * dim, dim * sizeof(float));
-			std::memcpy(dst_im + k * dim, im + index[k] * dim, dim * sizeof(float));
-			nonzero |= anyBitSet(dst_im + k * dim, dim) ? 1 : 0;
+			if (im) {
+				std::memcpy(dst_im + k * dim, im + index[k] * dim, dim * sizeof(float));
+				nonzero |= anyBitSet(dst_im + k * dim, dim) ? 1 : 0;
+			} else if (clear_im) {
+				std::memset(dst_im + k * dim, 0, dim * sizeof(float));
+			}
 		}
-		imag_nonzero_ = nonzero != 0;
+		noteImag(nonzero != 0);
+		if (clear_im && current_pos_ == 0 && count == batch_size_) imag_clean_ = true;  // every row of the plane was cleared just now
 		for (int k = 0; k < count; ++k) {
 			labels_.push_back(labels[index[k]]);
 			sizes_.push_back(sample_dim_);
@@ -568,11 +587,25 @@ public:
 	int typeId() const override { return isSoftMax; }
 };
 
+// Where the per-row losses of an output function go.  A forward pass that is launched kernel by kernel writes them straight
+// into page-locked host memory (a ring of slots, one per forward pass: the kernel's stores travel over the link, no copy
+// is queued); a forward pass inside a recording writes to the device buffer, since a replay cannot move to the next slot.
+struct OutLoss {
+	static constexpr int kSlots = 4;
+	float *dev = NULL;        // device: [rows]
+	float *host = NULL;       // page-locked: [kSlots][rows]
+	int rows = 0;
+	int64_t serial = -1;      // forward passes that have written to the ring so far, minus one
+	const float *cur = NULL;  // where the last forward pass wrote
+	bool cur_on_host = false;
+};
+
 class CrossEntropy : public CFunc, public OutputFunc {
 	friend class CNet;
 	Vars output_;
 	int prediction_ = 0;                    // argmax of the fetched sample, computed on the device
-	float *d_s_ = NULL, *d_loss_ = NULL;    // device: [rows]
+	float *d_s_ = NULL;                     // device: [rows]
+	OutLoss loss_;
 	int32_t *d_argmax_ = NULL;
 	float *d_norm_ = NULL;                  // device: normalised z, 2 planes [rows][n]
 public:
@@ -597,7 +630,7 @@ public:
 class L2Out : public CFunc, public OutputFunc {
 	friend class CNet;
 	Vars output_;
-	float *d_loss_ = NULL;  // device: [rows]
+	OutLoss loss_;
 public:
 	L2Out(Uid uid, InSize n) : CFunc(uid, n, OutSize(1)), output_(1) { is_output_ = true; }
 	L2Out(InSize n) : CFunc(n, OutSize(1)), output_(1) { is_output_ = true; }
@@ -875,6 +908,50 @@ class CNet {
 		allocations_.push_back(p);
 		return (T *) p;
 	}
+	// ---- per-row losses of the output functions (see OutLoss) ----
+	bool host_losses_ = true;
+	bool in_train_step_ = false;  // gpuTrainStep is queueing or recording: its forward pass writes to the device buffer
+	std::vector<void *> host_allocations_;
+	void planLoss(OutLoss &l, int rows) {
+		l = OutLoss();
+		l.rows = rows;
+		l.dev = dalloc<float>(rows);
+		ck(cnet_memset_zero(l.dev, rows * sizeof(float)), "zero");
+		void *h = NULL;
+		if (cnet_host_alloc((size_t) OutLoss::kSlots * rows * sizeof(float), &h) == CNET_OK && h) {
+			host_allocations_.push_back(h);
+			l.host = (float *) h;
+			std::fill(l.host, l.host + (size_t) OutLoss::kSlots * rows, 0.f);
+		}
+		l.cur = l.dev;
+	}
+	static OutLoss *lossOf(CFunc *f) {
+		if (!f) return NULL;
+		if (f->typeId() == isCrossEntropy) return &((CrossEntropy *) f)->loss_;
+		if (f->typeId() == isL2Out) return &((L2Out *) f)->loss_;
+		return NULL;
+	}
+	// where the forward pass that is being queued writes its losses
+	float *lossTarget(OutLoss &l) {
+		if (host_losses_ && !use_graphs_ && !in_train_step_ && l.host) {
+			l.serial++;
+			l.cur = l.host + (size_t) (l.serial % OutLoss::kSlots) * l.rows;
+			l.cur_on_host = true;
+		} else {
+			l.cur = l.dev;
+			l.cur_on_host = false;
+		}
+		return const_cast<float *>(l.cur);
+	}
+	// `count` losses of the last forward pass from row `first` on, for the host (waits for the device)
+	void readLoss(OutLoss &l, float *dst, int first, int count) {
+		if (l.cur_on_host) {
+			ck(cnet_sync(), "cnet_sync");
+			std::copy(l.cur + first, l.cur + first + count, dst);
+		} else {
+			ck(cnet_memcpy_d2h(dst, l.dev + first, (size_t) count * sizeof(float)), "cnet_memcpy_d2h");
+		}
+	}
 	static bool isParameter(CFunc *f) {  // stored once: every CInput that carries no per-sample data
 		if (f->typeId() != isInput) return false;
 		CInput *c = (CInput *) f;
@@ -1011,6 +1088,10 @@ public:
 		if (!batch_ && allocations_.empty()) return;
 		for (void *p : allocations_) cnet_free(p);
 		allocations_.clear();
+		for (void *p : host_allocations_) cnet_host_free(p);
+		host_allocations_.clear();
+		for (auto f : outputs_)
+			if (OutLoss *l = lossOf(f)) *l = OutLoss();
 		for (auto f : func_list_) {
 			f->slots_.clear();
 			f->out_ = NULL;
@@ -1117,13 +1198,13 @@ private:
 			case isCrossEntropy: {
 				CrossEntropy *c = (CrossEntropy *) f;
 				c->d_s_ = dalloc<float>(rows);
-				c->d_loss_ = dalloc<float>(rows);
+				planLoss(c->loss_, (int) rows);
 				c->d_argmax_ = dalloc<int32_t>(rows);
 				c->d_norm_ = dalloc<float>(2 * rows * f->input().length_);
 				break;
 			}
 			case isL2Out:
-				((L2Out *) f)->d_loss_ = dalloc<float>(rows);
+				planLoss(((L2Out *) f)->loss_, (int) rows);
 				break;
 			default: break;
 			}
@@ -1282,11 +1363,11 @@ private:
 			CrossEntropy *c = (CrossEntropy *) f;
 			const int n = f->input().length_;
 			ck(cnet_cross_entropy_fwd(zre(f, 0), zim(f, 0), n, d_labels_, c->d_norm_, c->d_norm_ + (size_t) rows * n, n, c->d_s_,
-					c->d_loss_, c->d_argmax_, rows, n), "cnet_cross_entropy_fwd");
+					lossTarget(c->loss_), c->d_argmax_, rows, n), "cnet_cross_entropy_fwd");
 			break;
 		}
 		case isL2Out:
-			ck(cnet_l2out_fwd(zre(f, 0), zim(f, 0), f->input().length_, ((L2Out *) f)->d_loss_, rows, f->input().length_),
+			ck(cnet_l2out_fwd(zre(f, 0), zim(f, 0), f->input().length_, lossTarget(((L2Out *) f)->loss_), rows, f->input().length_),
 					"cnet_l2out_fwd");
 			break;
 		default: throw std::logic_error(f->getName() + ": no device implementation");
@@ -1592,7 +1673,7 @@ public:
 			ck(cnet_memcpy_d2h(&am, c->d_argmax_ + rb, sizeof(am)), "cnet_memcpy_d2h");
 			c->prediction_ = am;
 		} else if (f->typeId() == isL2Out) {
-			ck(cnet_memcpy_d2h(((L2Out *) f)->output_.real_, ((L2Out *) f)->d_loss_ + (f->rows_ == 1 ? 0 : b), sizeof(float)), "cnet_memcpy_d2h");
+			readLoss(((L2Out *) f)->loss_, ((L2Out *) f)->output_.real_, f->rows_ == 1 ? 0 : b, 1);
 		}
 	}
 	void fetchAll(int b) {
@@ -1619,15 +1700,18 @@ public:
 		auto eager = [&] {
 			const bool was = use_graphs_;
 			use_graphs_ = false;  // the phases launch (or record) their kernels themselves
+			in_train_step_ = true;  // every step of this loop leaves its losses where a replay does: in the device buffer
 			try {
 				GpuForward();
 				gpuBackward();
 				gpuUpdateInputs(l_rate);
 			} catch (...) {
 				use_graphs_ = was;
+				in_train_step_ = false;
 				throw;
 			}
 			use_graphs_ = was;
+			in_train_step_ = false;
 		};
 		// an update that also clears a first moment is not what a recording replays, nor is a step that finds gradients of
 		// an earlier backward pass waiting for their update
@@ -1950,6 +2034,10 @@ public:
 	// the imaginary plane of the data input is cleared on the device: half the bytes over the link, the same values on
 	// the device.  On: the plane of zeros travels like any other.
 	void sendZeroPlanes(bool on) { send_zero_planes_ = on; }
+	// The loss kernels of a forward pass that is launched kernel by kernel store the per-row losses straight into page-locked
+	// host memory (see OutLoss): getLoss and gpuQueueLoss then queue no copy.  Off: the losses stay in a device buffer and are
+	// copied when asked for, as in a recorded forward pass.  Same values either way.
+	void hostLosses(bool on) { host_losses_ = on; }
 	// A FourierTrans applied to a data input that was fed real samples computes half of its columns and writes the others
 	// as their conjugates (cnet_cdft_fwd_real_input); off: the whole product, whatever the samples.  Same values to rounding.
 	void realTransforms(bool on) {
@@ -2019,12 +2107,10 @@ public:
 	float getLoss(OutputFunc *outp, Batch *batch) {
 		requireAllocated("getLoss");
 		CFunc *f = dynamic_cast<CFunc *>(outp);
-		float *d = NULL;
-		if (CrossEntropy *c = dynamic_cast<CrossEntropy *>(f)) d = c->d_loss_;
-		else if (L2Out *l = dynamic_cast<L2Out *>(f)) d = l->d_loss_;
-		else throw std::invalid_argument("getLoss: not supported for this output");
+		OutLoss *l = lossOf(f);
+		if (!l) throw std::invalid_argument("getLoss: not supported for this output");
 		std::vector<float> tmp(f->rows_);
-		ck(cnet_memcpy_d2h(tmp.data(), d, tmp.size() * sizeof(float)), "cnet_memcpy_d2h");
+		readLoss(*l, tmp.data(), 0, f->rows_);
 		float loss = 0.f;
 		for (float v : tmp) {
 			loss += v;
@@ -2037,36 +2123,43 @@ public:
 	// waits for that copy alone, typically one step later, when it has long arrived.  The host can then queue step k+1
 	// before it looks at the loss of step k, and the device never runs dry between steps.  Up to kLossSlots reads may be
 	// pending; an older one is overwritten.
-	static constexpr int kLossSlots = 4;
+	static constexpr int kLossSlots = OutLoss::kSlots;
 	struct PendingLoss {
 		int64_t ticket = -1, serial = -1;
 		int rows = 0;
+		const OutLoss *direct = NULL;  // the forward pass wrote to that output's own ring (serial counts its forward passes)
 	};
 	PendingLoss gpuQueueLoss(OutputFunc *outp) {
 		requireAllocated("gpuQueueLoss");
 		CFunc *f = dynamic_cast<CFunc *>(outp);
-		float *d = NULL;
-		if (CrossEntropy *c = dynamic_cast<CrossEntropy *>(f)) d = c->d_loss_;
-		else if (L2Out *l = dynamic_cast<L2Out *>(f)) d = l->d_loss_;
-		else throw std::invalid_argument("gpuQueueLoss: not supported for this output");
+		OutLoss *l = lossOf(f);
+		if (!l) throw std::invalid_argument("gpuQueueLoss: not supported for this output");
+		PendingLoss p;
+		p.rows = f->rows_;
+		if (l->cur_on_host) {  // already on its way: the kernel stores into page-locked memory; only the point in the stream is marked
+			p.serial = l->serial;
+			p.direct = l;
+			ck(cnet_copy_ticket(0, &p.ticket), "cnet_copy_ticket");
+			return p;
+		}
 		if (!loss_ring_) {
 			void *h = NULL;
 			ck(cnet_host_alloc((size_t) kLossSlots * batch_ * sizeof(float), &h), "cnet_host_alloc");
 			loss_ring_ = (float *) h;
 		}
-		PendingLoss p;
 		p.serial = loss_queued_++;
-		p.rows = f->rows_;
-		ck(cnet_memcpy_d2h_async(loss_ring_ + (size_t) (p.serial % kLossSlots) * batch_, d, (size_t) p.rows * sizeof(float)),
+		ck(cnet_memcpy_d2h_async(loss_ring_ + (size_t) (p.serial % kLossSlots) * batch_, l->dev, (size_t) p.rows * sizeof(float)),
 				"cnet_memcpy_d2h_async");
 		ck(cnet_copy_ticket(0, &p.ticket), "cnet_copy_ticket");
 		return p;
 	}
 	float getLoss(const PendingLoss &p, Batch *batch) {
-		if (p.serial < 0 || !loss_ring_) throw std::logic_error("getLoss: nothing was queued under this handle");
-		if (loss_queued_ - p.serial > kLossSlots) throw std::logic_error("getLoss: the queued losses were overwritten by later ones");
+		if (p.serial < 0 || (!p.direct && !loss_ring_)) throw std::logic_error("getLoss: nothing was queued under this handle");
+		if ((p.direct ? p.direct->serial - p.serial + 1 : loss_queued_ - p.serial) > kLossSlots)
+			throw std::logic_error("getLoss: the queued losses were overwritten by later ones");
 		ck(cnet_copy_wait(p.ticket), "cnet_copy_wait");
-		const float *v = loss_ring_ + (size_t) (p.serial % kLossSlots) * batch_;
+		const float *v = p.direct ? p.direct->host + (size_t) (p.serial % kLossSlots) * p.direct->rows
+								  : loss_ring_ + (size_t) (p.serial % kLossSlots) * batch_;
 		float loss = 0.f;
 		for (int b = 0; b < p.rows; ++b) {
 			loss += v[b];
@@ -2085,7 +2178,7 @@ public:
 		for (auto f : outputs_) {
 			if (f->typeId() == isL2Out) {
 				float v = 0.f;
-				ck(cnet_memcpy_d2h(&v, ((L2Out *) f)->d_loss_, sizeof(float)), "cnet_memcpy_d2h");
+				readLoss(((L2Out *) f)->loss_, &v, 0, 1);
 				ret[f->uid()] = v;
 			} else if (f->typeId() == isCrossEntropy) {
 				const int lab = batch_labels_ ? labels_[0] : label;

@@ -22,6 +22,16 @@ class BatchedDataReader {
 	std::vector<int> labels_;
 	std::vector<int> order_;      // position -> sample
 	std::vector<int> pick_;       // samples of the batch being assembled
+	bool imag_all_zero_ = true;   // no sample added so far has an imaginary part other than +0 (images): batches skip that plane
+	void noteImag(const float *im, size_t n) {
+		uint32_t acc = 0;
+		for (size_t k = 0; k < n; ++k) {
+			uint32_t w;
+			std::memcpy(&w, im + k, sizeof(w));
+			acc |= w;
+		}
+		if (acc) imag_all_zero_ = false;
+	}
 
 protected:
 	int sample_dim_ = 0;
@@ -59,7 +69,7 @@ public:
 			pick_[i] = order_[current_];
 			current_ = (current_ + 1) % (int) labels_.size();
 		}
-		batch.gather(re_.data(), im_.data(), labels_.data(), pick_.data(), batch.size());
+		batch.gather(re_.data(), imag_all_zero_ ? NULL : im_.data(), labels_.data(), pick_.data(), batch.size());
 	}
 
 	void add(const std::vector<std::complex<float> > &data, int label) {
@@ -71,12 +81,14 @@ public:
 			re_[at + k] = data[k].real();
 			im_[at + k] = data[k].imag();
 		}
+		noteImag(&im_[at], data.size());
 		order_.push_back((int) labels_.size());
 		labels_.push_back(label);
 	}
 	void addPlanes(const float *re, const float *im, int label) {
 		re_.insert(re_.end(), re, re + sample_dim_);
 		im_.insert(im_.end(), im, im + sample_dim_);
+		noteImag(im, (size_t) sample_dim_);
 		order_.push_back((int) labels_.size());
 		labels_.push_back(label);
 	}

@@ -897,13 +897,15 @@ static void test_pipeline(int B, int steps) {
 	// 8: as 6 with the data input marked not trainable (CNet::setInputTrainable: no step on it, no backward pass into it)
 	// 9: prefetch, one launch per layer (CNet::fuseLayers(false): Hadamard and CGelu as separate passes)
 	// 10: prefetch, every backward pass adds the gradients to the input functions' own planes at once (CNet::deferGathers(false))
-	constexpr int MODES = 11;
+	// 11 / 12: as 1 / 6 with the losses kept in a device buffer and copied when asked for (CNet::hostLosses(false)) instead of
+	//          stored into page-locked memory by the loss kernel
+	constexpr int MODES = 13;
 	std::vector<float> losses[MODES];
 	std::vector<float> weights[MODES];
 	double ms[MODES] = {0};
 	for (int mode = 0; mode < MODES; ++mode) {
 		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4 || mode == 7;
-		const bool late_loss = mode == 6 || mode == 7 || mode == 8;
+		const bool late_loss = mode == 6 || mode == 7 || mode == 8 || mode == 12;
 		CNet::PendingLoss pending;
 		CNet net;
 		int inp, outp;
@@ -911,6 +913,7 @@ static void test_pipeline(int B, int steps) {
 		net.allocateOnGpu(B);
 		CInput *cin = (CInput *) net[inp];
 		CrossEntropy *cen = (CrossEntropy *) net[outp];
+		if (mode >= 11) net.hostLosses(false);
 		SyntheticReader reader = data;  // same order for both modes
 		InputBatch ring[3] = {InputBatch(B, n), InputBatch(B, n), InputBatch(B, n)};
 		if (mode == 0) expect("batches built after cnet_init are page-locked", ring[0].isPinned());
@@ -1008,6 +1011,8 @@ static void test_pipeline(int B, int steps) {
 		expect("losses and weights identical with the data input not trainable", losses[0] == losses[8] && weights[0] == weights[8]);
 		expect("losses and weights identical with one launch per layer (no fused Hadamard + CGelu)", losses[0] == losses[9] && weights[0] == weights[9]);
 		expect("losses and weights identical with the gradients of the input functions gathered at once", losses[0] == losses[10] && weights[0] == weights[10]);
+		expect("losses and weights identical with the losses copied from a device buffer", losses[0] == losses[11] && weights[0] == weights[11]);
+		expect("losses and weights identical with the losses copied from a device buffer, read one step late", losses[0] == losses[12] && weights[0] == weights[12]);
 		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
 		// dz* planes written as the conjugate of the dz product against dz* planes computed by a product of their own
 		double worst = 0, num = 0, den = 0;
