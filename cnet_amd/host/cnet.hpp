@@ -704,6 +704,9 @@ class CNet {
 		int64_t labels_ticket = -1;   // the last copy out of host_labels
 		const InputBatch *holds = NULL;
 		bool imag_zero = false;       // the staged batch held real samples: its imaginary plane on the device is all +0
+		// Every element of the imaginary plane of this buffer on the device is +0 (it was cleared and nothing has written to it
+		// since): the next batch of real samples that lands here need not clear it again.
+		bool imag_dev_zero = false;
 	};
 	Stage stage_[2];
 	int active_ = 0;
@@ -754,6 +757,10 @@ class CNet {
 		}
 		if (!src.empty()) ck(cnet_add_multi((int) src.size(), src.data(), dst.data(), len.data()), "cnet_add_multi");
 	}
+	// a kernel or a copy other than a batch upload has written (or is about to write) the value planes of `f`
+	void dataValuesWritten(CFunc *f) {
+		if (f == main_input_) stage_[active_].imag_dev_zero = false;
+	}
 	// ---- lazy data inputs (see CFunc::lazy_bwd_) ----
 	bool lazy_inputs_ = true;
 	// the transform on a data input whose backward pass can wait, or NULL
@@ -781,6 +788,7 @@ class CNet {
 			const int64_t n = (int64_t) own.rows * own.len;
 			if (d->lazy_upd_) {  // the node's own planes are clear: the step reads the gradient where it is, nothing to clear
 				ck(cnet_sgd_update(own.z, own.z + n, u.g(2), u.g(3), n, d->lazy_lr_, 0), "cnet_sgd_update");
+				dataValuesWritten(d);
 				d->lazy_upd_ = false;
 			} else if (defer_gathers_ && d->grad_clean_ && !d->pending_) {
 				d->pending_ = &u;
@@ -1602,6 +1610,7 @@ public:
 		for (auto f : inputs_) {
 			beforeFeed(f);
 			f->z_imag_zero_ = false;
+			dataValuesWritten(f);
 			CFunc::Slot &s = f->slots_[0];
 			float *z = s.z;
 			if (s.rows == 1) {
@@ -1741,6 +1750,7 @@ public:
 		for (auto f : inputs_) {  // what the steps inside the recording do to the host's picture of the inputs
 			if (!f->trainable_) continue;
 			f->z_imag_zero_ = false;
+			if (!lazyHead(f)) dataValuesWritten(f);  // stepped inside the recording
 			if (lazyHead(f)) {  // the recording was made in the usual state: its backward pass and update left these out
 				f->lazy_bwd_ = f->lazy_upd_ = true;
 				f->lazy_lr_ = l_rate;
@@ -1782,15 +1792,18 @@ private:
 		// gpu/gpu_func.h:403-419)
 		// (a batch of real samples sends its real plane only; the imaginary plane is cleared on the device)
 		const bool real_only = batch.imagIsZero() && !send_zero_planes_;
+		Stage &here = stage_[active_];
+		const bool clear_imag = real_only && !here.imag_dev_zero;  // unless the plane is still clear from the last batch
 		if (batch.isPinned()) {
 			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), real_only ? plane : 2 * plane), "cnet_memcpy_h2d_async");
-			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
+			if (clear_imag) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
 			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
 		} else {
 			ck(cnet_memcpy_h2d(s.z, batch.realDataPtr(), real_only ? plane : 2 * plane), "cnet_memcpy_h2d");
-			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
+			if (clear_imag) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
 		}
-		cin->z_imag_zero_ = batch.imagIsZero();  // zeros on the device, sent or cleared there
+		here.imag_dev_zero = batch.imagIsZero();  // zeros on the device, cleared there (now or earlier) or sent
+		cin->z_imag_zero_ = batch.imagIsZero();
 		setLabels(batch.labelsPtr(), batch_);
 	}
 
@@ -1829,10 +1842,12 @@ public:
 		st.imag_zero = batch.imagIsZero();
 		if (st.imag_zero && !send_zero_planes_) {
 			ck(cnet_upload_async(st.z, batch.realDataPtr(), plane * sizeof(float)), "cnet_upload_async");
-			ck(cnet_upload_zero(st.z + plane, plane * sizeof(float)), "cnet_upload_zero");
+			// the plane is still clear when the last batch that landed here was real and nothing has stepped the values since
+			if (!st.imag_dev_zero) ck(cnet_upload_zero(st.z + plane, plane * sizeof(float)), "cnet_upload_zero");
 		} else {
 			ck(cnet_upload_async(st.z, batch.realDataPtr(), 2 * plane * sizeof(float)), "cnet_upload_async");
 		}
+		st.imag_dev_zero = st.imag_zero;
 		ck(cnet_upload_async(st.labels, st.host_labels, batch_ * sizeof(int32_t)), "cnet_upload_async");
 		ck(cnet_mark_upload(other), "cnet_mark_upload");
 		ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
@@ -1866,6 +1881,7 @@ public:
 			if (real_only) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
 		}
 		cin->z_imag_zero_ = batch.imagIsZero();
+		if (cin == main_input_) stage_[active_].imag_dev_zero = batch.imagIsZero();  // cleared or sent just now
 	}
 	bool gpuForward(InputFunc *inp, OutputFunc *outp, EmbeddingBatch &batch) {
 		requireAllocated("gpuForward");
@@ -1985,6 +2001,7 @@ public:
 		else body();
 		for (auto f : inputs_) {
 			if (!f->trainable_) continue;
+			if (!f->lazy_bwd_) dataValuesWritten(f);  // stepped by the launch above (or by its replay)
 			if (f->lazy_bwd_ && !f->lazy_upd_) {  // its step waits with its backward pass
 				f->lazy_upd_ = true;
 				f->lazy_lr_ = l_rate;
@@ -2098,6 +2115,7 @@ public:
 			const CFunc::Slot &gsrc = f->pending_ ? *f->pending_ : s;  // a gradient still with its consumer is read there
 			ck(cnet_adam_update(z, z + n, s.g(0), s.g(1), gsrc.g(2), gsrc.g(3), (int64_t) n, l_rate, beta, t, f->pending_ ? 0 : 1),
 					"cnet_adam_update");
+			dataValuesWritten(f);
 			f->pending_ = NULL;
 			f->grad_clean_ = true;
 			f->z_imag_zero_ = false;

@@ -937,10 +937,14 @@ static void test_pipeline(int B, int steps) {
 			// the whole step is queued first; only then does the host turn to the next batches, and last of all it waits
 			// for this step's losses (backward and update do not touch them)
 			const float rate = (s < steps / 2 ? lr : 0.5f * lr) / B;
+			// modes 6 and 12 send the next batch off between the forward and the backward pass of this one (the order of the
+			// timing driver), the others after the update
+			const bool early = (mode == 6 || mode == 12) && s + 1 < steps;
 			if (one_graph) {
 				net.gpuTrainStep(cin, cen, cur, rate);
 			} else {
 				net.gpuForward(cin, cen, cur);
+				if (early) net.gpuPrefetch(cin, ring[(s + 1) % 3]);
 				net.gpuBackward();
 				net.gpuUpdateInputs(rate);
 			}
@@ -948,7 +952,7 @@ static void test_pipeline(int B, int steps) {
 				// the loss of this step starts its way to the host; the one of the step before is read (into its batch,
 				// which is the buffer of the ring that is refilled next)
 				CNet::PendingLoss now = net.gpuQueueLoss(cen);
-				if (s + 1 < steps) net.gpuPrefetch(cin, ring[(s + 1) % 3]);
+				if (s + 1 < steps && !early) net.gpuPrefetch(cin, ring[(s + 1) % 3]);
 				if (s > 0) losses[mode].push_back(net.getLoss(pending, &ring[(s + 2) % 3]));
 				if (s + 2 < steps) reader.nextBatch(ring[(s + 2) % 3]);
 				pending = now;
@@ -1142,22 +1146,26 @@ static void test_real_batches() {
 		return;
 	}
 	SyntheticReader data(n, 4 * B, classes, true);
-	std::vector<float> trace[7];
+	std::vector<float> trace[13];
 	// bit 0: send the zeros, bit 1: prefetch; 4: the whole transform whatever the samples; 5: whole recorded steps;
-	// 6: recorded phases
-	for (int variant = 0; variant < 7; ++variant) {
+	// 6: recorded phases.  The imaginary plane of a buffer is cleared once and then left alone while only real batches land
+	// in it and nothing steps the values; the cases in which something does, each against the same loop with the zeros sent:
+	// 7 / 8: every update steps the data input (lazyDataInputs(false)), prefetch; 9 / 10: the step of the data input is made
+	// up for by a look at the inputs after every update; 11 / 12: as 7 / 8 with the copy inside gpuForward
+	for (int variant = 0; variant < 13; ++variant) {
 		CNet net;
 		int inp, outp;
 		build_readme(net, n, classes, &inp, &outp);
 		net.allocateOnGpu(B);
-		net.sendZeroPlanes((variant & 1) != 0 && variant < 4);
+		net.sendZeroPlanes(((variant & 1) != 0 && variant < 4) || variant == 8 || variant == 10 || variant == 12);
+		if (variant == 7 || variant == 8 || variant >= 11) net.lazyDataInputs(false);
 		if (variant == 4) net.realTransforms(false);
 		if (variant == 6) net.useGraphs(true);
 		CInput *cin = (CInput *) net[inp];
 		CrossEntropy *cen = (CrossEntropy *) net[outp];
 		SyntheticReader reader = data;
 		InputBatch ring[2] = {InputBatch(B, n), InputBatch(B, n)};
-		const bool prefetch = (variant & 2) != 0 || variant >= 4;
+		const bool prefetch = ((variant & 2) != 0 || variant >= 4) && variant < 11;
 		reader.nextBatch(ring[0]);
 		if (variant == 0) expect("a batch of real samples knows it", ring[0].imagIsZero());
 		if (prefetch) net.gpuPrefetch(cin, ring[0]);
@@ -1169,6 +1177,10 @@ static void test_real_batches() {
 				net.gpuForward(cin, cen, cur);
 				net.gpuBackward();
 				net.gpuUpdateInputs(0.05f / B);
+			}
+			if (variant == 9 || variant == 10) {
+				net.getInputsFromGpu();
+				trace[variant].push_back(cin->input().imag_[3]);
 			}
 			if (s + 1 < steps) {
 				reader.nextBatch(ring[(s + 1) % 2]);
@@ -1182,6 +1194,9 @@ static void test_real_batches() {
 	expect("real plane only, copy inside gpuForward: same losses, weights and data input as with the zeros sent", trace[0] == trace[1] && trace[0].size() > 100);
 	expect("real plane only, gpuPrefetch: the same", trace[2] == trace[3] && trace[0] == trace[2]);
 	expect("whole recorded steps and recorded phases: the same", trace[5] == trace[2] && trace[6] == trace[2]);
+	expect("a data input that every update steps: its imaginary plane is cleared again for the next real batch", trace[7] == trace[8] && trace[7] == trace[2]);
+	expect("the same when the step is made up for by a look at the inputs", trace[9] == trace[10] && trace[9].size() == trace[2].size() + 6);
+	expect("the same with the copy inside gpuForward", trace[11] == trace[12] && trace[11] == trace[2]);
 	{
 		// half the columns of the first FourierTrans computed and the rest written as conjugates, against the whole product
 		double num = 0, den = 0;
