@@ -94,6 +94,7 @@ SIGNATURES = {
     "cnet_l2norm_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_l2out_bwd_sym": [c_fp, c_fp, _l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_cross_entropy_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp] + [c_fp] * 4 + [_l, _i, _i],
+    "cnet_cross_entropy_fwd_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, c_fp, _l, c_fp, c_fp, c_fp] + [c_fp] * 4 + [_l, _i, _i],
     "cnet_copy2d": [c_fp, _l, c_fp, _l, _i, _i],
     "cnet_add2d": [c_fp, _l, c_fp, _l, _i, _i],
     "cnet_add_multi": [_i, C.c_void_p, C.c_void_p, C.c_void_p],

@@ -175,10 +175,30 @@ __device__ __forceinline__ float label_loss(const float *__restrict__ pr, const 
 
 // impl/crossent.h:50-80, 117-130 upstream: S in double, clamped; out = z / sqrt(S); p_k = out_r^2 + out_i^2 evaluated
 // in double and rounded to float; argmax = first strict maximum of p; loss = -log(max(p_label, 1e-15)).
+// The four planes that receive the gradient of the row's loss in the same launch (all null: the forward pass alone).  The
+// values are the ones of crossent_bwd_sym_kernel, formed by the same operations from the same S: dz* = z / S, at the label
+// -z (S - m) / (m S) with m = max(|z_label|^2, 1e-15); dz = conj(dz*) (impl/crossent.h:82-104 upstream).
+struct GradPlanes {
+	float *dz_re, *dz_im, *dzs_re, *dzs_im;
+	long ld;
+};
+
+__device__ __forceinline__ void crossent_grad(float a, float b, bool at_label, float S, float &g_re, float &g_im) {
+	if (at_label) {
+		float m = (float) ((double) a * (double) a + (double) b * (double) b);
+		m = (m < 1e-15f ? 1e-15f : m);
+		g_re = -a * (S - m) / (m * S);
+		g_im = -b * (S - m) / (m * S);
+	} else {
+		g_re = a / S;
+		g_im = b / S;
+	}
+}
+
 template <int V, int G>
 __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		const int *__restrict__ labels, float *__restrict__ outr, float *__restrict__ outi, long ldo, float *__restrict__ s,
-		float *__restrict__ loss, int *__restrict__ argmax, int rows, int cols) {
+		float *__restrict__ loss, int *__restrict__ argmax, int rows, int cols, GradPlanes grad) {
 	__shared__ double lds_d[TPB / 64];
 	__shared__ ArgMax lds_a[TPB / 64];
 	__shared__ Top2 lds_t[TPB / 64];
@@ -222,7 +242,8 @@ __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restri
 	// ulp.  When the runner-up is more than 1e-5 (relative) below the maximum the winner is already decided; otherwise,
 	// or when the normalised planes are wanted, a second pass evaluates p_k exactly as the reference does.
 	const bool clear_cut = top.q2 < top.q1 * (1.0 - 1.0e-5);
-	if (!want_out && clear_cut) {
+	const bool want_grad = (grad.dz_re != nullptr);
+	if (!want_out && !want_grad && clear_cut) {
 		if (live && t == 0) {
 			s[row] = S;
 			loss[row] = label_loss(pr, pi, labels[row], cols, inv);
@@ -234,6 +255,8 @@ __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restri
 	ArgMax best = {-1.0f, 0x7fffffff};
 	float *qr = want_out ? outr + (long) row * ldo : nullptr;
 	float *qi = want_out ? outi + (long) row * ldo : nullptr;
+	const int label = want_grad ? labels[row] : -1;
+	const long goff = (long) row * grad.ld;
 	if (V == 4) {
 		for (int c = t * 4; c < cols; c += STRIDE * 4) {
 			float4 a = *reinterpret_cast<const float4 *>(pr + c);
@@ -249,6 +272,18 @@ __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restri
 				*reinterpret_cast<float4 *>(qr + c) = make_float4(o_r[0], o_r[1], o_r[2], o_r[3]);
 				*reinterpret_cast<float4 *>(qi + c) = make_float4(o_i[0], o_i[1], o_i[2], o_i[3]);
 			}
+			if (want_grad && live) {
+				const float za[4] = {a.x, a.y, a.z, a.w}, zb[4] = {b.x, b.y, b.z, b.w};
+				float g_r[4], g_i[4];
+#pragma unroll
+				for (int k = 0; k < 4; ++k) crossent_grad(za[k], zb[k], c + k == label, S, g_r[k], g_i[k]);
+				*reinterpret_cast<float4 *>(grad.dz_re + goff + c) = make_float4(g_r[0], g_r[1], g_r[2], g_r[3]);
+				*reinterpret_cast<float4 *>(grad.dz_im + goff + c) = make_float4(-g_i[0], -g_i[1], -g_i[2], -g_i[3]);
+				if (grad.dzs_re) {
+					*reinterpret_cast<float4 *>(grad.dzs_re + goff + c) = make_float4(g_r[0], g_r[1], g_r[2], g_r[3]);
+					*reinterpret_cast<float4 *>(grad.dzs_im + goff + c) = make_float4(g_i[0], g_i[1], g_i[2], g_i[3]);
+				}
+			}
 		}
 	} else {
 		for (int c = t; c < cols; c += STRIDE) {
@@ -258,6 +293,16 @@ __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restri
 			if (want_out && live) {
 				qr[c] = o_r;
 				qi[c] = o_i;
+			}
+			if (want_grad && live) {
+				float g_r, g_i;
+				crossent_grad(pr[c], pi[c], c == label, S, g_r, g_i);
+				grad.dz_re[goff + c] = g_r;
+				grad.dz_im[goff + c] = -g_i;
+				if (grad.dzs_re) {
+					grad.dzs_re[goff + c] = g_r;
+					grad.dzs_im[goff + c] = g_i;
+				}
 			}
 		}
 	}
@@ -765,7 +810,24 @@ int cnet_cross_entropy_fwd(const float *z_re, const float *z_im, int64_t ldz, co
 	const bool vec = mult4(cols, ldz, out_re ? ldo : 0) && aligned16(z_re) && aligned16(z_im) && aligned16(out_re) &&
 			aligned16(out_im);
 	CNET_ROW_LAUNCH(crossent_fwd_kernel, vec, z_re, z_im, (long) ldz, labels, out_re, out_im, (long) ldo, s, loss, argmax, rows,
-			cols);
+			cols, GradPlanes{nullptr, nullptr, nullptr, nullptr, 0});
+	return CNET_OK;
+}
+
+int cnet_cross_entropy_fwd_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, const int32_t *labels, float *out_re,
+		float *out_im, int64_t ldo, float *s, float *loss, int32_t *argmax, float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re,
+		float *dz_dzs_im, int64_t lddz, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(rows >= 0 && cols > 0);
+	if (!rows) return CNET_OK;
+	CNET_CHECK_ARG(z_re && z_im && labels && s && loss && argmax && ldz >= cols);
+	CNET_CHECK_ARG((out_re == nullptr) == (out_im == nullptr));
+	CNET_CHECK_ARG(out_re == nullptr || ldo >= cols);
+	CNET_CHECK_ARG(dz_dz_re && dz_dz_im && ((dz_dzs_re == nullptr) == (dz_dzs_im == nullptr)) && lddz >= cols);
+	const bool vec = mult4(cols, ldz, out_re ? ldo : 0, lddz) && aligned16(z_re) && aligned16(z_im) && aligned16(out_re) &&
+			aligned16(out_im) && aligned16(dz_dz_re) && aligned16(dz_dz_im) && aligned16(dz_dzs_re) && aligned16(dz_dzs_im);
+	CNET_ROW_LAUNCH(crossent_fwd_kernel, vec, z_re, z_im, (long) ldz, labels, out_re, out_im, (long) ldo, s, loss, argmax, rows,
+			cols, GradPlanes{dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz});
 	return CNET_OK;
 }
 

@@ -606,6 +606,9 @@ class CrossEntropy : public CFunc, public OutputFunc {
 	int prediction_ = 0;                    // argmax of the fetched sample, computed on the device
 	float *d_s_ = NULL;                     // device: [rows]
 	OutLoss loss_;
+	// The gradient planes hold what a backward pass with the current labels would write: the forward pass wrote it in the
+	// same launch (cnet_cross_entropy_fwd_bwd_sym), and the backward pass of this node then has nothing to do.
+	bool grad_from_forward_ = false;
 	int32_t *d_argmax_ = NULL;
 	float *d_norm_ = NULL;                  // device: normalised z, 2 planes [rows][n]
 public:
@@ -916,6 +919,12 @@ class CNet {
 		allocations_.push_back(p);
 		return (T *) p;
 	}
+	bool per_sample_call_ = false;  // forward() / backward() of the per-sample API are running
+	// the labels, the gradient planes or the kind of gradient pair changed: what a forward pass wrote ahead no longer stands
+	void lossGradientsStale() {
+		for (auto f : outputs_)
+			if (f->typeId() == isCrossEntropy) ((CrossEntropy *) f)->grad_from_forward_ = false;
+	}
 	// ---- per-row losses of the output functions (see OutLoss) ----
 	bool host_losses_ = true;
 	bool in_train_step_ = false;  // gpuTrainStep is queueing or recording: its forward pass writes to the device buffer
@@ -1100,6 +1109,7 @@ public:
 		host_allocations_.clear();
 		for (auto f : outputs_)
 			if (OutLoss *l = lossOf(f)) *l = OutLoss();
+		lossGradientsStale();
 		for (auto f : func_list_) {
 			f->slots_.clear();
 			f->out_ = NULL;
@@ -1370,8 +1380,19 @@ private:
 		case isCrossEntropy: {
 			CrossEntropy *c = (CrossEntropy *) f;
 			const int n = f->input().length_;
+			// A short-rowed loss (a classifier head) costs less than the launch it rides on: forward pass and gradient go out as
+			// one launch.  Not inside the recorded phases (the labels may change between a recorded forward and a recorded
+			// backward pass) and not in the per-sample calls (upstream shows cleared gradients after forward()).
+			if (fuse_layers_ && conjugate_gradients_ && !use_graphs_ && !per_sample_call_ && (long) rows * n <= (1L << 18)) {
+				CFunc::Slot &sl = f->slots_[0];
+				ck(cnet_cross_entropy_fwd_bwd_sym(zre(f, 0), zim(f, 0), n, d_labels_, c->d_norm_, c->d_norm_ + (size_t) rows * n, n, c->d_s_,
+						lossTarget(c->loss_), c->d_argmax_, sl.g(0), sl.g(1), sl.gs(2), sl.gs(3), sl.len, rows, n), "cnet_cross_entropy_fwd_bwd_sym");
+				c->grad_from_forward_ = true;
+				break;
+			}
 			ck(cnet_cross_entropy_fwd(zre(f, 0), zim(f, 0), n, d_labels_, c->d_norm_, c->d_norm_ + (size_t) rows * n, n, c->d_s_,
 					lossTarget(c->loss_), c->d_argmax_, rows, n), "cnet_cross_entropy_fwd");
+			c->grad_from_forward_ = false;
 			break;
 		}
 		case isL2Out:
@@ -1391,6 +1412,7 @@ private:
 			if (!with_labels) return;  // upstream: CrossEntropy::backward() without a label does nothing
 			CrossEntropy *c = (CrossEntropy *) f;
 			CFunc::Slot &s = f->slots_[0];
+			if (conjugate_gradients_ && c->grad_from_forward_) return;  // written by the forward pass, with these labels
 			if (conjugate_gradients_)
 				ck(cnet_cross_entropy_bwd_sym(zre(f, 0), zim(f, 0), s.len, c->d_s_, d_labels_, s.g(0), s.g(1), s.gs(2), s.gs(3), s.len, rows,
 						s.len), "cnet_cross_entropy_bwd_sym");
@@ -1785,6 +1807,7 @@ private:
 			d_labels_ = staged.labels;
 			labels_.assign(batch.labelsPtr(), batch.labelsPtr() + batch_);
 			batch_labels_ = true;
+			lossGradientsStale();
 			return;
 		}
 		const size_t plane = (size_t) batch_ * s.len * sizeof(float);
@@ -2019,6 +2042,7 @@ public:
 	void useGraphs(bool on) {
 		requireAllocated("useGraphs");
 		if (!on) dropGraphs();
+		lossGradientsStale();  // a recorded backward pass holds the loss's own backward kernel
 		use_graphs_ = on;
 	}
 	bool usingGraphs() const { return use_graphs_; }
@@ -2031,6 +2055,7 @@ public:
 		if (on != conjugate_gradients_ && batch_) {
 			dropGraphs();
 			materializeLazy();  // with the kernels of the setting the backward pass ran under
+			lossGradientsStale();
 		}
 		conjugate_gradients_ = on;
 	}
@@ -2259,6 +2284,7 @@ public:
 		checkLabels(labels, count);
 		labels_.assign(labels, labels + count);
 		batch_labels_ = from_batch;
+		lossGradientsStale();
 		ck(cnet_memcpy_h2d(d_labels_, labels, count * sizeof(int32_t)), "cnet_memcpy_h2d");
 	}
 	void sync() { ck(cnet_sync(), "cnet_sync"); }
@@ -2280,7 +2306,15 @@ public:
 		for (auto f : func_list_)
 			if (!f->is_input_)
 				for (auto &s : f->slots_) ck(cnet_memset_zero(s.grad, 4 * (size_t) s.rows * s.len * sizeof(float)), "zero");
-		GpuForward();
+		lossGradientsStale();
+		per_sample_call_ = true;
+		try {
+			GpuForward();
+		} catch (...) {
+			per_sample_call_ = false;
+			throw;
+		}
+		per_sample_call_ = false;
 		fetchAll(0);
 	}
 	void backward(int label) {
@@ -2288,8 +2322,15 @@ public:
 		if (label >= 0) setLabels(&label, 1, false);
 		// the label only enters the backward pass of CrossEntropy; its forward outputs do not depend on it except
 		// the device-side loss, which is refreshed here so getLoss() matches the label in use
-		for (auto f : outputs_)
-			if (f->typeId() == isCrossEntropy) nodeForward(f);
+		per_sample_call_ = true;
+		try {
+			for (auto f : outputs_)
+				if (f->typeId() == isCrossEntropy) nodeForward(f);
+		} catch (...) {
+			per_sample_call_ = false;
+			throw;
+		}
+		per_sample_call_ = false;
 		materializeLazy();
 		flushPending();
 		planDeferral(false);  // every host view is read right after the pass: nothing to gain from deferring

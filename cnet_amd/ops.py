@@ -321,3 +321,10 @@ def embedding_fwd(table, tokens, y, slots):
 def embedding_bwd(tokens, gs_re, gs_im, dtab_re, dtab_im, dim, vocab, rows, slots, accumulate=0):
     call("cnet_embedding_bwd", tokens.ptr, gs_re.ptr, gs_im.ptr, gs_re.ld, dtab_re.ptr, dtab_im.ptr, dim, vocab, rows,
          slots, accumulate)
+
+
+def cross_entropy_fwd_bwd_sym(z, labels, s, loss, argmax, dz, out=None, mirror=True):
+    """Forward pass and gradient of the loss in one launch."""
+    o = out.p() if out is not None else (None, None)
+    call("cnet_cross_entropy_fwd_bwd_sym", *z.p(), z.ld, labels.ptr, o[0], o[1], out.ld if out is not None else 0, s.ptr,
+         loss.ptr, argmax.ptr, *_pair(dz, mirror), dz.ld, z.rows, z.cols)

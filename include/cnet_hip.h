@@ -401,6 +401,15 @@ int cnet_l2out_bwd_sym(const float *z_re, const float *z_im, int64_t ldz,
 int cnet_cross_entropy_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, const float *s, const int32_t *labels,
                                float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,
                                int rows, int cols);
+/* cnet_cross_entropy_fwd and cnet_cross_entropy_bwd_sym in one launch (upstream: gpu_cross_ent_forward and
+ * gpu_cross_ent_backward, gpu/reduce.cpp:469-530, 609-655, which a training step always runs one after the other with the
+ * same labels): every result of the forward call, and the gradient of each row's loss in the dz planes (its conjugate in
+ * the dz* planes when those are given), with the bits of the two separate calls.  For rows short enough that a launch
+ * costs more than the pass itself (a classifier head: 10 columns). */
+int cnet_cross_entropy_fwd_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, const int32_t *labels,
+                                   float *out_re, float *out_im, int64_t ldo, float *s, float *loss, int32_t *argmax,
+                                   float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,
+                                   int rows, int cols);
 
 /* ---- CEmbedding: replaces gpu_embedding_forward / _backward (gpu/kernels.cpp:362-442), CPU twin impl/embed.h:109-148.
  * tokens[rows][slots] int32, -1 = padding (zero row); an id >= vocab is treated as padding too (upstream asserts on

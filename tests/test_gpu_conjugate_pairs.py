@@ -241,6 +241,21 @@ def test_loss_and_softmax_backward_of_a_conjugate_pair(gpu, port, B, n):
     ops.cross_entropy_bwd_sym(z, S, labels, one)
     _exact(full, one, "cross entropy")
     _dz_only(port, lambda d: ops.cross_entropy_bwd_sym(z, S, labels, d, mirror=False), B, n, full, "cross entropy")
+    # forward pass and gradient in one launch: every result of the two calls, to the bit, with and without the normalised
+    # planes and the dz* planes
+    norm = ops.CMat.empty(B, n)
+    ops.cross_entropy_fwd(z, labels, S, loss, am, norm)
+    want = [S.download(), loss.download(), am.download()] + list(norm.host())
+    for with_out in (True, False):
+        S2, loss2, am2 = capi.empty(B), capi.empty(B), capi.empty(B, np.int32)
+        norm2, both = ops.CMat.empty(B, n), ops.Grad.from_host(_pair(port, 98, (B, n)))
+        ops.cross_entropy_fwd_bwd_sym(z, labels, S2, loss2, am2, both, out=norm2 if with_out else None)
+        _exact(full, both, ("cross entropy, one launch", with_out))
+        got = [S2.download(), loss2.download(), am2.download()] + (list(norm2.host()) if with_out else [])
+        for a, b in zip(got, want):
+            assert np.array_equal(a, b), ("cross entropy forward results, one launch", with_out)
+        _dz_only(port, lambda d: ops.cross_entropy_fwd_bwd_sym(z, labels, S2, loss2, am2, d, out=norm2 if with_out else None, mirror=False),
+                 B, n, full, "cross entropy, one launch")
 
 
 def _l2(z, B, n):
