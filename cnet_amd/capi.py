@@ -33,6 +33,7 @@ SIGNATURES = {
     "cnet_memcpy_d2h_async": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_upload_async": [C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_upload_zero": [C.c_void_p, C.c_size_t],
+    "cnet_upload_pair": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_upload_wait_compute": [],
     "cnet_mark_compute": [_i],
     "cnet_upload_wait_marker": [_i],
@@ -42,6 +43,7 @@ SIGNATURES = {
     "cnet_upload_sync": [],
     "cnet_copy_ticket": [_i, C.POINTER(C.c_int64)],
     "cnet_copy_wait": [C.c_int64],
+    "cnet_compute_wait_ticket": [C.c_int64],
     "cnet_graph_begin": [],
     "cnet_graph_end": [C.POINTER(C.c_void_p)],
     "cnet_graph_launch": [C.c_void_p],

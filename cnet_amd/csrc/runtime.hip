@@ -280,6 +280,40 @@ int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes) {
 	return CNET_OK;
 }
 
+// two regions of page-locked host memory to the device in one launch: the lanes read the host memory over the link
+__global__ __launch_bounds__(256) void upload_pair_kernel(uint32_t *__restrict__ d0, const uint32_t *__restrict__ s0, long words0,
+		long vec0, uint32_t *__restrict__ d1, const uint32_t *__restrict__ s1, long words1) {
+	const long i = (long) blockIdx.x * blockDim.x + threadIdx.x, stride = (long) gridDim.x * blockDim.x;
+	for (long k = i; k < vec0; k += stride) reinterpret_cast<uint4 *>(d0)[k] = reinterpret_cast<const uint4 *>(s0)[k];
+	for (long k = 4 * vec0 + i; k < words0; k += stride) d0[k] = s0[k];
+	for (long k = i; k < words1; k += stride) d1[k] = s1[k];
+}
+
+int cnet_upload_pair(void *dst0, const void *pinned_src0, size_t bytes0, void *dst1, const void *pinned_src1, size_t bytes1) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // work on the upload stream: never part of a recording
+	CNET_CHECK_ARG((bytes0 == 0 || (dst0 && pinned_src0)) && (bytes1 == 0 || (dst1 && pinned_src1)));
+	CNET_CHECK_ARG(bytes0 % 4 == 0 && bytes1 % 4 == 0);
+	if (!bytes0 && !bytes1) return CNET_OK;
+	Runtime &r = rt();
+	// Small batches: a copy queued through the runtime costs the host 3-5 us each and takes the copy engine's start-up time
+	// to arrive; one kernel launch that reads the page-locked memory directly does both regions.  Large ones stay with the
+	// copy engine, which moves them without occupying compute units.
+	if (bytes0 + bytes1 <= (1u << 20)) {
+		const long words0 = (long) (bytes0 / 4), words1 = (long) (bytes1 / 4);
+		const long vec0 = aligned16(dst0) && aligned16(pinned_src0) ? words0 / 4 : 0;
+		const long threads = std::max(vec0 + (words0 - 4 * vec0), words1);
+		const unsigned blocks = (unsigned) std::min<long>((threads + 255) / 256, 1024);
+		hipLaunchKernelGGL(upload_pair_kernel, dim3(blocks), dim3(256), 0, r.upload_stream, (uint32_t *) dst0, (const uint32_t *) pinned_src0,
+				words0, vec0, (uint32_t *) dst1, (const uint32_t *) pinned_src1, words1);
+		CNET_LAUNCH_CHECK();
+		return CNET_OK;
+	}
+	if (bytes0) CNET_HIP(hipMemcpyAsync(dst0, pinned_src0, bytes0, hipMemcpyHostToDevice, r.upload_stream));
+	if (bytes1) CNET_HIP(hipMemcpyAsync(dst1, pinned_src1, bytes1, hipMemcpyHostToDevice, r.upload_stream));
+	return CNET_OK;
+}
+
 int cnet_upload_zero(void *dst, size_t bytes) {
 	CNET_REQUIRE_INIT();
 	CNET_NOT_IN_CAPTURE();  // a fill on the upload stream: never part of a recording
@@ -360,6 +394,18 @@ int cnet_copy_wait(int64_t ticket) {
 	const int64_t n = ticket >> 1;
 	CNET_CHECK_ARG(ticket >= 0 && n < r.tickets_issued[which]);
 	CNET_HIP(hipEventSynchronize(r.ticket_event[which][n % Runtime::kTickets]));
+	return CNET_OK;
+}
+
+int cnet_compute_wait_ticket(int64_t ticket) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // would pull the upload stream into the recording
+	Runtime &r = rt();
+	const int which = (int) (ticket & 1);
+	const int64_t n = ticket >> 1;
+	CNET_CHECK_ARG(ticket >= 0 && which == 1 && n < r.tickets_issued[which]);
+	// a ticket whose event has been handed out again since stands for a later point of the same stream: the wait still covers it
+	CNET_HIP(hipStreamWaitEvent(r.stream, r.ticket_event[which][n % Runtime::kTickets], 0));
 	return CNET_OK;
 }
 

@@ -710,6 +710,7 @@ class CNet {
 		// Every element of the imaginary plane of this buffer on the device is +0 (it was cleared and nothing has written to it
 		// since): the next batch of real samples that lands here need not clear it again.
 		bool imag_dev_zero = false;
+		int64_t upload_ticket = -1;   // the point of the upload stream at which the staged batch and its labels have landed
 	};
 	Stage stage_[2];
 	int active_ = 0;
@@ -1797,7 +1798,7 @@ private:
 			// the batch was sent ahead by gpuPrefetch(): switch the data input to the buffer it landed in.  Everything
 			// queued so far may still read the buffer in use, so its retirement point is remembered for the next refill.
 			checkLabels(batch.labelsPtr(), batch_);
-			ck(cnet_compute_wait_upload_marker(1 - active_), "cnet_compute_wait_upload_marker");  // this batch's copies, nothing later
+			ck(cnet_compute_wait_ticket(staged.upload_ticket), "cnet_compute_wait_ticket");  // this batch's copies, nothing later
 			ck(cnet_mark_compute(active_), "cnet_mark_compute");
 			active_ = 1 - active_;
 			staged.holds = NULL;
@@ -1863,17 +1864,17 @@ public:
 		ck(cnet_upload_wait_marker(other), "cnet_upload_wait_marker");  // kernels of the step that last used this buffer
 		// the two planes of a batch are one array on the host and on the device: one copy for both
 		st.imag_zero = batch.imagIsZero();
-		if (st.imag_zero && !send_zero_planes_) {
-			ck(cnet_upload_async(st.z, batch.realDataPtr(), plane * sizeof(float)), "cnet_upload_async");
-			// the plane is still clear when the last batch that landed here was real and nothing has stepped the values since
-			if (!st.imag_dev_zero) ck(cnet_upload_zero(st.z + plane, plane * sizeof(float)), "cnet_upload_zero");
-		} else {
-			ck(cnet_upload_async(st.z, batch.realDataPtr(), 2 * plane * sizeof(float)), "cnet_upload_async");
-		}
+		const bool real_only = st.imag_zero && !send_zero_planes_;
+		// the plane is still clear when the last batch that landed here was real and nothing has stepped the values since
+		if (real_only && !st.imag_dev_zero) ck(cnet_upload_zero(st.z + plane, plane * sizeof(float)), "cnet_upload_zero");
+		// the samples and their labels: one launch for a small batch, two queued copies for a large one
+		ck(cnet_upload_pair(st.z, batch.realDataPtr(), (real_only ? 1 : 2) * plane * sizeof(float), st.labels, st.host_labels,
+				batch_ * sizeof(int32_t)), "cnet_upload_pair");
 		st.imag_dev_zero = st.imag_zero;
-		ck(cnet_upload_async(st.labels, st.host_labels, batch_ * sizeof(int32_t)), "cnet_upload_async");
-		ck(cnet_mark_upload(other), "cnet_mark_upload");
+		// one recorded point serves the host (the batch may be refilled, the staging of the labels reused) and the compute
+		// stream (the forward pass of this batch)
 		ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
+		st.upload_ticket = batch.ticket_;
 		st.labels_ticket = batch.ticket_;
 		st.holds = &batch;
 	}

@@ -92,6 +92,10 @@ int cnet_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
 int cnet_memcpy_d2h_async(void *pinned_dst, const void *src, size_t bytes);
 int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes);
 int cnet_upload_zero(void *dst, size_t bytes);
+/* two regions (a batch and its labels) from page-locked memory to the device on the upload stream, sizes in bytes, multiples
+ * of 4; up to 1 MiB in all they travel in ONE kernel launch whose lanes read the host memory over the link (half the
+ * host time of two queued copies and none of the copy engine's start-up time), beyond that as two cnet_upload_async */
+int cnet_upload_pair(void *dst0, const void *pinned_src0, size_t bytes0, void *dst1, const void *pinned_src1, size_t bytes1);
 int cnet_upload_wait_compute(void);
 int cnet_mark_compute(int marker);
 int cnet_upload_wait_marker(int marker);
@@ -101,6 +105,9 @@ int cnet_compute_wait_upload_marker(int marker);
 int cnet_upload_sync(void);
 int cnet_copy_ticket(int upload_stream, int64_t *ticket);
 int cnet_copy_wait(int64_t ticket);
+/* kernels queued after this call start only when the point of the upload stream that ticket t names has been reached: one
+ * recorded point then serves the host (cnet_copy_wait) and the compute stream, instead of a ticket and a marker */
+int cnet_compute_wait_ticket(int64_t ticket);
 
 /* ---- Graphs: a training step at small batch sizes is bound by launch overhead (upstream pays a cudaDeviceSynchronize
  *      per layer on top, gpu/kernels.cpp:104-105).  Between cnet_graph_begin and cnet_graph_end the layer entry points

@@ -347,5 +347,35 @@ def test_device_copy_caller_stream_and_upload_ordering(gpu, port):
     capi.call("cnet_upload_sync")
     got = a.download()
     assert (got[: n // 2] == 0.0).all() and (got[n // 2:] == 7.0).all()
+    # two regions in one call: a small pair travels in one kernel launch that reads the page-locked memory, a large one as two
+    # queued copies; either way the compute stream can wait for the ticket taken behind them
+    pinned[:] = np.arange(n, dtype=np.float32)
+    for words0, words1, off in ((50176, 64, 0), (50176, 64, 1), (3, 0, 0), (0, 5, 0), (n - 1024, 512, 0)):
+        capi.call("cnet_memset_zero", a.ptr, 4 * n)
+        capi.call("cnet_memset_zero", b.ptr, 4 * n)
+        capi.call("cnet_upload_wait_compute")                    # the upload starts behind the clearing
+        capi.call("cnet_upload_pair", a.ptr + 4 * off, host.value + 4 * off, 4 * words0, b.ptr, host.value + 4 * (n - 1024), 4 * words1)
+        t = C.c_int64(-1)
+        capi.call("cnet_copy_ticket", 1, C.byref(t))
+        capi.call("cnet_compute_wait_ticket", t)
+        c = capi.zeros((n,))
+        capi.call("cnet_copy2d", a.ptr, n, c.ptr, n, 1, n)       # on the compute stream, behind the wait
+        capi.sync()
+        want = np.zeros(n, np.float32)
+        want[off:off + words0] = np.arange(off, off + words0)
+        assert np.array_equal(c.download(), want), (words0, words1, off)
+        got1 = b.download()
+        assert np.array_equal(got1[:words1], np.arange(n - 1024, n - 1024 + words1)) and (got1[words1:] == 0).all()
+    assert _status("cnet_upload_pair", a.ptr, host, 6, b.ptr, host, 4) == INVALID        # not whole words
+    assert _status("cnet_upload_pair", None, host, 8, b.ptr, host, 4) == INVALID
+    assert _status("cnet_upload_pair", None, None, 0, None, None, 0) == 0
+    t0 = C.c_int64(-1)
+    capi.call("cnet_copy_ticket", 0, C.byref(t0))
+    assert _status("cnet_compute_wait_ticket", t0.value) == INVALID                      # a point of the compute stream itself
+    assert _status("cnet_compute_wait_ticket", t.value + 2) == INVALID and _status("cnet_compute_wait_ticket", -1) == INVALID
+    capi.call("cnet_graph_begin")
+    assert _status("cnet_upload_pair", a.ptr, host, 8, b.ptr, host, 4) == UNSUPPORTED
+    assert _status("cnet_compute_wait_ticket", t.value) == UNSUPPORTED
+    capi.call("cnet_graph_end", None)
     del pinned
     capi.call("cnet_host_free", host)
