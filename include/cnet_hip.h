@@ -292,7 +292,10 @@ int cnet_l2norm_bwd(const float *z_re, const float *z_im, int64_t ldz, const flo
  *      and the loss read-back of CNet::getLoss (gpu/gpu_func.h:906-926).  CPU twin impl/crossent.h:50-130.
  * labels[rows] int32.  s = clamped sum |z|^2, loss = -log(max(|z_label|^2/s, 1e-15)), argmax = first index of the
  * strict maximum of |z_k/sqrt(s)|^2.  out_re/out_im (normalised z) may be NULL.  A label outside [0, cols) gives a NaN
- * loss for its row (upstream reads out of bounds); the backward pass then treats every entry as a non-label entry. */
+ * loss for its row (upstream reads out of bounds); the backward pass then treats every entry as a non-label entry.
+ * `loss` (here and in cnet_l2out_fwd) may point into page-locked host memory from cnet_host_alloc: the kernel then stores
+ * the per-row losses there itself and no copy has to be queued to read them (a point taken with cnet_copy_ticket behind the
+ * call tells the host when they have arrived). */
 int cnet_cross_entropy_fwd(const float *z_re, const float *z_im, int64_t ldz, const int32_t *labels,
                            float *out_re, float *out_im, int64_t ldo, float *s, float *loss, int32_t *argmax,
                            int rows, int cols);

@@ -50,6 +50,36 @@ def test_cross_entropy_batch_case_of_upstream_test(gpu, port):
     assert np.allclose(got[:2], np.log(2), rtol=1e-6) and np.allclose(got, loss, rtol=1e-6)
 
 
+@pytest.mark.parametrize("B,n", [(64, 10), (5, 3000), (300, 64)])
+def test_loss_kernels_store_into_page_locked_memory(gpu, port, B, n):
+    """The `loss` argument of cnet_cross_entropy_fwd, cnet_cross_entropy_fwd_bwd_sym and cnet_l2out_fwd may point into
+    page-locked host memory: the same values arrive there, readable once a ticket taken behind the call has been waited for."""
+    import ctypes as C
+    zr, zi = seeded(port, n, (B, n)), seeded(port, n + 1, (B, n))
+    z, lab = ops.CMat.from_host(zr, zi), ops.ints(port.randint(n + 2, (B,), n))
+    s, l, am = capi.empty(B), capi.empty(B), capi.empty(B, np.int32)
+    ops.cross_entropy_fwd(z, lab, s, l, am, None)
+    l2 = capi.empty(B)
+    ops.l2out_fwd(z, l2)
+    host = C.c_void_p()
+    capi.call("cnet_host_alloc", 4 * 3 * B, C.byref(host))
+    pinned = np.ctypeslib.as_array((C.c_float * (3 * B)).from_address(host.value))
+    pinned[:] = -1.0
+    dz = ops.Grad.empty(B, n)
+    none = C.c_void_p(None)
+    capi.call("cnet_cross_entropy_fwd", *z.p(), z.ld, lab.ptr, none, none, 0, s.ptr, host.value, am.ptr, B, n)
+    capi.call("cnet_cross_entropy_fwd_bwd_sym", *z.p(), z.ld, lab.ptr, none, none, 0, s.ptr, host.value + 4 * B, am.ptr, *dz.p(), dz.ld, B, n)
+    capi.call("cnet_l2out_fwd", *z.p(), z.ld, host.value + 8 * B, B, n)
+    t = C.c_int64(-1)
+    capi.call("cnet_copy_ticket", 0, C.byref(t))
+    capi.call("cnet_copy_wait", t)
+    want = l.download()
+    assert np.array_equal(pinned[:B], want) and np.array_equal(pinned[B:2 * B], want)
+    assert np.array_equal(pinned[2 * B:], l2.download())
+    del pinned
+    capi.call("cnet_host_free", host)
+
+
 @pytest.mark.parametrize("B,n", [(2, 6), (64, 10), (2048, 2048), (3, 5001)])
 def test_l2out(gpu, port, B, n):
     zr, zi = seeded(port, 1, (B, n)), seeded(port, 2, (B, n))
