@@ -195,10 +195,10 @@ __device__ __forceinline__ void crossent_grad(float a, float b, bool at_label, f
 	}
 }
 
-template <int V, int G>
-__global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+template <int V, int G, bool GRAD>
+__device__ __forceinline__ void crossent_fwd_row(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		const int *__restrict__ labels, float *__restrict__ outr, float *__restrict__ outi, long ldo, float *__restrict__ s,
-		float *__restrict__ loss, int *__restrict__ argmax, int rows, int cols, GradPlanes grad) {
+		float *__restrict__ loss, int *__restrict__ argmax, int rows, int cols, const GradPlanes &grad) {
 	__shared__ double lds_d[TPB / 64];
 	__shared__ ArgMax lds_a[TPB / 64];
 	__shared__ Top2 lds_t[TPB / 64];
@@ -242,7 +242,7 @@ __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restri
 	// ulp.  When the runner-up is more than 1e-5 (relative) below the maximum the winner is already decided; otherwise,
 	// or when the normalised planes are wanted, a second pass evaluates p_k exactly as the reference does.
 	const bool clear_cut = top.q2 < top.q1 * (1.0 - 1.0e-5);
-	const bool want_grad = (grad.dz_re != nullptr);
+	constexpr bool want_grad = GRAD;
 	if (!want_out && !want_grad && clear_cut) {
 		if (live && t == 0) {
 			s[row] = S;
@@ -312,6 +312,21 @@ __global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restri
 		loss[row] = label_loss(pr, pi, labels[row], cols, inv);
 		argmax[row] = best.i;
 	}
+}
+
+template <int V, int G>
+__global__ __launch_bounds__(TPB) void crossent_fwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		const int *__restrict__ labels, float *__restrict__ outr, float *__restrict__ outi, long ldo, float *__restrict__ s,
+		float *__restrict__ loss, int *__restrict__ argmax, int rows, int cols) {
+	crossent_fwd_row<V, G, false>(zr, zi, ldz, labels, outr, outi, ldo, s, loss, argmax, rows, cols, GradPlanes{nullptr, nullptr, nullptr, nullptr, 0});
+}
+
+// the same pass with the gradient of each row's loss written as well
+template <int V, int G>
+__global__ __launch_bounds__(TPB) void crossent_fwd_grad_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
+		const int *__restrict__ labels, float *__restrict__ outr, float *__restrict__ outi, long ldo, float *__restrict__ s,
+		float *__restrict__ loss, int *__restrict__ argmax, int rows, int cols, GradPlanes grad) {
+	crossent_fwd_row<V, G, true>(zr, zi, ldz, labels, outr, outi, ldo, s, loss, argmax, rows, cols, grad);
 }
 
 // ---------------------------------------------------------------------------------------------- SoftMax (L2 normalise)
@@ -810,7 +825,7 @@ int cnet_cross_entropy_fwd(const float *z_re, const float *z_im, int64_t ldz, co
 	const bool vec = mult4(cols, ldz, out_re ? ldo : 0) && aligned16(z_re) && aligned16(z_im) && aligned16(out_re) &&
 			aligned16(out_im);
 	CNET_ROW_LAUNCH(crossent_fwd_kernel, vec, z_re, z_im, (long) ldz, labels, out_re, out_im, (long) ldo, s, loss, argmax, rows,
-			cols, GradPlanes{nullptr, nullptr, nullptr, nullptr, 0});
+			cols);
 	return CNET_OK;
 }
 
@@ -826,7 +841,7 @@ int cnet_cross_entropy_fwd_bwd_sym(const float *z_re, const float *z_im, int64_t
 	CNET_CHECK_ARG(dz_dz_re && dz_dz_im && ((dz_dzs_re == nullptr) == (dz_dzs_im == nullptr)) && lddz >= cols);
 	const bool vec = mult4(cols, ldz, out_re ? ldo : 0, lddz) && aligned16(z_re) && aligned16(z_im) && aligned16(out_re) &&
 			aligned16(out_im) && aligned16(dz_dz_re) && aligned16(dz_dz_im) && aligned16(dz_dzs_re) && aligned16(dz_dzs_im);
-	CNET_ROW_LAUNCH(crossent_fwd_kernel, vec, z_re, z_im, (long) ldz, labels, out_re, out_im, (long) ldo, s, loss, argmax, rows,
+	CNET_ROW_LAUNCH(crossent_fwd_grad_kernel, vec, z_re, z_im, (long) ldz, labels, out_re, out_im, (long) ldo, s, loss, argmax, rows,
 			cols, GradPlanes{dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz});
 	return CNET_OK;
 }
