@@ -438,13 +438,18 @@ protected:
 	// input functions: the imaginary plane on the device is known to hold +0 only (a batch of real samples was fed and
 	// nothing has stepped or overwritten the values since); a FourierTrans on it then takes cnet_cdft_fwd_real_input
 	bool z_imag_zero_ = false;
-	// Data inputs (one row per sample) whose only consumer is a FourierTrans / TriangFourier: the backward pass of that
-	// transform, the gather and the update of the input are work whose results the next batch overwrites.  They are left
-	// out (lazy_bwd_: a backward pass has skipped them; lazy_upd_: an update at rate lazy_lr_ has skipped them too) and
-	// done later, from the gradients the transform's consumers left, if anything looks before the next batch arrives
-	// (CNet::materializeLazy).  lazy_now_ / lazy_skip_now_ are the decisions for the pass that is being queued.
-	bool lazy_bwd_ = false, lazy_upd_ = false, lazy_now_ = false, lazy_skip_now_ = false;
+	// Data inputs (one row per sample) that feed a FourierTrans / TriangFourier or the data operand of a Linear: the part
+	// of that consumer's backward pass that only serves the data input (the whole backward pass of a transform, the
+	// input-gradient product of a Linear), the gather and the update of the input are work whose results the next batch
+	// overwrites.  They are left out (lazy_bwd_: a backward pass has skipped them; lazy_upd_: an update at rate lazy_lr_
+	// has skipped them too) and done later, from the gradients the consumer's consumers left, if anything looks before the
+	// next batch arrives (CNet::materializeLazy).  lazy_now_ (on the input) / lazy_skip_now_ (on the consumer) are the
+	// decisions for the pass that is being queued; lazy_owed_ (on the consumer) says that a pass has skipped its share.
+	// A Linear whose weights an update changes in the meantime keeps their old values in w_saved_ (w_saved_valid_).
+	bool lazy_bwd_ = false, lazy_upd_ = false, lazy_now_ = false, lazy_skip_now_ = false, lazy_owed_ = false;
 	float lazy_lr_ = 0.f;
+	float *w_saved_ = NULL;
+	bool w_saved_valid_ = false;
 	int rows_ = 0;           // batch rows of this node's output (1 for parameter nodes)
 	float *out_ = NULL;      // 2 planes [rows][out_size]: what consumers read
 	float *out_re() const { return out_; }
@@ -767,40 +772,88 @@ class CNet {
 	}
 	// ---- lazy data inputs (see CFunc::lazy_bwd_) ----
 	bool lazy_inputs_ = true;
-	// the transform on a data input whose backward pass can wait, or NULL
-	CFunc *lazyHead(CFunc *d) const {
-		if (!lazy_inputs_ || d->typeId() != isInput || !d->trainable_ || isParameter(d) || d->no_outputs() != 1) return NULL;
-		CFunc *f = d->next_func_[0];
-		if ((f->typeId() != isFourier && f->typeId() != isTrianFourier) || f->rows_ != d->rows_ || f->slots_.size() != 1 ||
-				f->slots_[0].producer != d || f->no_outputs() == 0)
-			return NULL;
-		return f;
+	// what of the backward pass of consumer c only serves the data input d: 0 nothing, 1 all of it (a transform of d),
+	// 2 its input-gradient product (a Linear with d as its data operand).  The second kind needs a copy of the weights when
+	// an update comes first, which a recording would have to hold: launch-by-launch passes only.
+	int lazyKind(CFunc *d, CFunc *c) const {
+		if (c->rows_ != d->rows_ || c->no_outputs() == 0) return 0;
+		const int t = c->typeId();
+		if ((t == isFourier || t == isTrianFourier) && c->slots_.size() == 1 && c->slots_[0].producer == d) return 1;
+		if (t == isLinear && !use_graphs_ && !in_train_step_ && c->slots_.size() == 2 && c->slots_[0].producer == d &&
+				c->slots_[1].producer != d)
+			return 2;
+		return 0;
 	}
-	// does now what was left out: the transform's backward pass from the gradients its consumers left (they stay where they
-	// are until the next backward pass), then the gather or, when an update was asked for in the meantime, that update
+	// a data input some of whose consumers have work that can wait
+	bool lazyEligible(CFunc *d) const {
+		if (!lazy_inputs_ || d->typeId() != isInput || !d->trainable_ || isParameter(d)) return false;
+		for (auto c : d->next_func_)
+			if (lazyKind(d, c)) return true;
+		return false;
+	}
+	// does now what was left out: the consumers' skipped shares from the gradients their own consumers left (they stay where
+	// they are until the next backward pass), then the gather or, when an update was asked for in the meantime, that update
 	void materializeLazy() {
 		for (auto d : inputs_) {
 			if (!d->lazy_bwd_) {
 				d->lazy_upd_ = false;
 				continue;
 			}
-			CFunc *f = d->next_func_[0];
-			CFunc::Slot &own = d->slots_[0], &u = upstream(d, 0);
-			f->lazy_skip_now_ = false;
-			nodeBackward(f, true);
+			for (auto f : d->next_func_) {
+				if (!f->lazy_owed_) continue;
+				f->lazy_owed_ = f->lazy_skip_now_ = false;
+				if (f->typeId() != isLinear) {
+					nodeBackward(f, true);
+					continue;
+				}
+				// dx = g w with the weights the skipped pass would have read
+				const float *w_re = f->w_saved_valid_ ? f->w_saved_ : zre(f, 1);
+				const float *w_im = f->w_saved_valid_ ? f->w_saved_ + f->slots_[1].len : zim(f, 1);
+				CFunc::Slot &a = f->slots_[0];
+				const int K = a.len, N = f->out_size_;
+				for (int c = 0; c < f->no_outputs(); ++c) {
+					CFunc::Slot &u = upstream(f, c);
+					if (conjugate_gradients_)
+						ck(cnet_clinear_bwd_input_sym(u.g(0), u.g(1), u.len, w_re, w_im, K, a.g(0), a.g(1), a.gs(2), a.gs(3), K, f->rows_, K, N,
+								c > 0), "cnet_clinear_bwd_input_sym");
+					else
+						ck(cnet_clinear_bwd_input(u.g(0), u.g(1), u.g(2), u.g(3), u.len, w_re, w_im, K, a.g(0), a.g(1), a.g(2), a.g(3), K,
+								f->rows_, K, N, c > 0), "cnet_clinear_bwd_input");
+				}
+				f->w_saved_valid_ = false;
+			}
 			d->lazy_bwd_ = false;
+			CFunc::Slot &own = d->slots_[0];
 			const int64_t n = (int64_t) own.rows * own.len;
-			if (d->lazy_upd_) {  // the node's own planes are clear: the step reads the gradient where it is, nothing to clear
-				ck(cnet_sgd_update(own.z, own.z + n, u.g(2), u.g(3), n, d->lazy_lr_, 0), "cnet_sgd_update");
-				dataValuesWritten(d);
-				d->lazy_upd_ = false;
-			} else if (defer_gathers_ && d->grad_clean_ && !d->pending_) {
-				d->pending_ = &u;
-			} else {
-				const float *src = u.g(2);
+			if (d->no_outputs() == 1) {
+				CFunc::Slot &u = upstream(d, 0);
+				if (d->lazy_upd_) {  // the node's own planes are clear: the step reads the gradient where it is, nothing to clear
+					ck(cnet_sgd_update(own.z, own.z + n, u.g(2), u.g(3), n, d->lazy_lr_, 0), "cnet_sgd_update");
+					dataValuesWritten(d);
+					d->lazy_upd_ = false;
+				} else if (defer_gathers_ && d->grad_clean_ && !d->pending_) {
+					d->pending_ = &u;
+				} else {
+					const float *src = u.g(2);
+					float *dst = own.g(2);
+					const int64_t len = 2 * n;
+					ck(cnet_add_multi(1, &src, &dst, &len), "cnet_add_multi");
+					d->grad_clean_ = false;
+				}
+				continue;
+			}
+			// several consumers: their contributions are added to the node's own planes as the backward pass would have done
+			for (int c = 0; c < d->no_outputs(); ++c) {
+				const float *src = upstream(d, c).g(2);
 				float *dst = own.g(2);
 				const int64_t len = 2 * n;
 				ck(cnet_add_multi(1, &src, &dst, &len), "cnet_add_multi");
+			}
+			if (d->lazy_upd_) {
+				ck(cnet_sgd_update(own.z, own.z + n, own.g(2), own.g(3), n, d->lazy_lr_, 1), "cnet_sgd_update");
+				dataValuesWritten(d);
+				d->lazy_upd_ = false;
+			} else {
 				d->grad_clean_ = false;
 			}
 		}
@@ -808,8 +861,26 @@ class CNet {
 	// a new batch is about to overwrite the values of `d`: work that was left out for it and whose result would be
 	// overwritten is dropped; a backward pass without an update still owes its gradient
 	void beforeFeed(CFunc *d) {
-		if (d->lazy_bwd_ && d->lazy_upd_) d->lazy_bwd_ = d->lazy_upd_ = false;
-		else if (d->lazy_bwd_) materializeLazy();
+		if (d->lazy_bwd_ && d->lazy_upd_) {
+			d->lazy_bwd_ = d->lazy_upd_ = false;
+			for (auto f : d->next_func_) f->lazy_owed_ = f->w_saved_valid_ = false;
+		} else if (d->lazy_bwd_) {
+			materializeLazy();
+		}
+	}
+	// an update is about to change the weights: a Linear that still owes the input gradient of a data input keeps the
+	// values that product has to read
+	void saveWeightsOwed() {
+		for (auto d : inputs_) {
+			if (!d->lazy_bwd_ || d->lazy_upd_) continue;
+			for (auto f : d->next_func_) {
+				if (!f->lazy_owed_ || f->typeId() != isLinear || !f->slots_[1].producer->trainable_) continue;
+				const size_t count = 2 * (size_t) f->slots_[1].len;
+				if (!f->w_saved_) f->w_saved_ = dalloc<float>(count);
+				ck(cnet_memcpy_d2d(f->w_saved_, zre(f, 1), count * sizeof(float)), "cnet_memcpy_d2d");
+				f->w_saved_valid_ = true;
+			}
+		}
 	}
 	// decides, for the backward pass about to be queued, which input functions leave their gradient with the consumer and
 	// which data inputs are left out altogether; true when every candidate does (the state a recorded backward pass stands
@@ -817,11 +888,13 @@ class CNet {
 	bool planDeferral(bool allow) {
 		bool all = true;
 		for (auto f : inputs_) {
-			CFunc *head = allow ? lazyHead(f) : NULL;
-			f->lazy_now_ = head && f->grad_clean_ && !f->pending_ && !f->lazy_bwd_ && !f->lazy_upd_;
-			if (head) head->lazy_skip_now_ = f->lazy_now_;
+			const bool eligible = lazyEligible(f);
+			f->lazy_now_ = allow && eligible && f->grad_clean_ && !f->pending_ && !f->lazy_bwd_ && !f->lazy_upd_;
+			if (eligible)
+				for (auto c : f->next_func_)
+					if (lazyKind(f, c)) c->lazy_skip_now_ = f->lazy_now_;
 			f->defer_now_ = !f->lazy_now_ && allow && defer_gathers_ && deferrable(f) && f->grad_clean_ && !f->pending_;
-			if (lazyHead(f) ? !f->lazy_now_ : (deferrable(f) && !f->defer_now_)) all = false;
+			if (eligible ? !f->lazy_now_ : (deferrable(f) && !f->defer_now_)) all = false;
 		}
 		return all;
 	}
@@ -830,7 +903,10 @@ class CNet {
 		for (auto f : inputs_) {
 			if (f->lazy_now_) {
 				f->lazy_bwd_ = true;
-				f->next_func_[0]->lazy_skip_now_ = false;
+				for (auto c : f->next_func_) {
+					if (c->lazy_skip_now_) c->lazy_owed_ = true;
+					c->lazy_skip_now_ = false;
+				}
 			} else if (f->defer_now_) {
 				f->pending_ = &upstream(f, 0);
 			} else if (f->trainable_ && f->no_outputs() > 0) {
@@ -843,7 +919,7 @@ class CNet {
 	// can be is waiting for its backward pass
 	bool allPending() const {
 		for (auto f : inputs_) {
-			if (lazyHead(f)) {
+			if (lazyEligible(f)) {
 				if (!f->lazy_bwd_ || f->lazy_upd_) return false;
 			} else if (deferrable(f) && !f->pending_) {
 				return false;
@@ -1117,7 +1193,8 @@ public:
 			f->rows_ = 0;
 			f->pending_ = NULL;
 			f->grad_clean_ = false;
-			f->lazy_bwd_ = f->lazy_upd_ = f->lazy_now_ = f->lazy_skip_now_ = false;
+			f->lazy_bwd_ = f->lazy_upd_ = f->lazy_now_ = f->lazy_skip_now_ = f->lazy_owed_ = f->w_saved_valid_ = false;
+			f->w_saved_ = NULL;
 		}
 		batch_ = 0;
 		d_labels_ = NULL;
@@ -1431,7 +1508,7 @@ private:
 			return;
 		}
 		if ((t == isInput || t == isEmbedding) && !f->trainable_) return;  // nothing steps it: nothing to gather
-		if (f->lazy_now_ || f->lazy_skip_now_) return;  // left out for now (see CFunc::lazy_bwd_)
+		if (f->lazy_now_ || (f->lazy_skip_now_ && t != isLinear)) return;  // left out for now (see CFunc::lazy_bwd_)
 		if (t == isInput) {  // impl/cinput.h:54-65: gathers dzs only, and keeps adding until the next update
 			// Both dz* planes of a consumer's slot are adjacent and dense, as they are in the node's own block: one array per
 			// consumer.  Nothing in the backward pass reads what an input function gathers, so the gathers of all of them
@@ -1492,7 +1569,8 @@ private:
 			case isLinear: {
 				CFunc::Slot &w = f->slots_[1];
 				const int K = a.len, N = f->out_size_;
-				const bool to_data = a.producer->wants_grad_, to_weight = w.producer->wants_grad_;
+				// (the input gradient of a lazy data input waits: see CFunc::lazy_bwd_)
+				const bool to_data = a.producer->wants_grad_ && !f->lazy_skip_now_, to_weight = w.producer->wants_grad_;
 				if (conjugate_gradients_ && to_data && to_weight) {  // both gradients in one call (one launch when both products are small)
 					ck(cnet_clinear_bwd_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.gs(2),
 							a.gs(3), K, acc, w.g(0), w.g(1), w.gs(2), w.gs(3), K, acc, rows, K, N), "cnet_clinear_bwd_sym");
@@ -1630,8 +1708,8 @@ public:
 	// ---- host <-> device (upstream copyInputsToGpu / getInputsFromGpu, gpu/gpu_func.h:512-527, 543-574) ----
 	bool copyInputsToGpu() {
 		requireAllocated("copyInputsToGpu");
+		for (auto f : inputs_) beforeFeed(f);  // first of all: work that was left out may still read weights that are replaced below
 		for (auto f : inputs_) {
-			beforeFeed(f);
 			f->z_imag_zero_ = false;
 			dataValuesWritten(f);
 			CFunc::Slot &s = f->slots_[0];
@@ -1729,21 +1807,25 @@ public:
 		feedBatch(inp, outp, batch);
 		settleUploads();  // the recording below cannot hold a wait for the upload stream
 		StepGraphs &g = graphs_[active_];
+		// every step of this loop, queued or replayed, leaves its losses in the device buffer and decides what can wait the
+		// way a recording does
+		struct InStep {
+			bool &flag;
+			explicit InStep(bool &f) : flag(f) { flag = true; }
+			~InStep() { flag = false; }
+		} in_step(in_train_step_);
 		auto eager = [&] {
 			const bool was = use_graphs_;
 			use_graphs_ = false;  // the phases launch (or record) their kernels themselves
-			in_train_step_ = true;  // every step of this loop leaves its losses where a replay does: in the device buffer
 			try {
 				GpuForward();
 				gpuBackward();
 				gpuUpdateInputs(l_rate);
 			} catch (...) {
 				use_graphs_ = was;
-				in_train_step_ = false;
 				throw;
 			}
 			use_graphs_ = was;
-			in_train_step_ = false;
 		};
 		// an update that also clears a first moment is not what a recording replays, nor is a step that finds gradients of
 		// an earlier backward pass waiting for their update
@@ -1773,8 +1855,10 @@ public:
 		for (auto f : inputs_) {  // what the steps inside the recording do to the host's picture of the inputs
 			if (!f->trainable_) continue;
 			f->z_imag_zero_ = false;
-			if (!lazyHead(f)) dataValuesWritten(f);  // stepped inside the recording
-			if (lazyHead(f)) {  // the recording was made in the usual state: its backward pass and update left these out
+			if (!lazyEligible(f)) dataValuesWritten(f);  // stepped inside the recording
+			if (lazyEligible(f)) {  // the recording was made in the usual state: its backward pass and update left these out
+				for (auto c : f->next_func_)
+					if (lazyKind(f, c)) c->lazy_owed_ = true;
 				f->lazy_bwd_ = f->lazy_upd_ = true;
 				f->lazy_lr_ = l_rate;
 			}
@@ -1990,6 +2074,7 @@ public:
 		}
 		g.upd_lr = l_rate;
 		if (input_dz_dirty_) materializeLazy();  // the first moment of every input function is cleared here: all of them take part
+		saveWeightsOwed();  // before the launch below changes them
 		if (input_dz_dirty_)  // this update also clears the first moment: not what a recording made without it does
 			for (auto &sg : graphs_)
 				if (sg.upd) {
@@ -2044,6 +2129,7 @@ public:
 		requireAllocated("useGraphs");
 		if (!on) dropGraphs();
 		lossGradientsStale();  // a recorded backward pass holds the loss's own backward kernel
+		if (on != use_graphs_) materializeLazy();  // what may wait differs between the two ways of running a pass
 		use_graphs_ = on;
 	}
 	bool usingGraphs() const { return use_graphs_; }

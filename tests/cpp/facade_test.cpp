@@ -867,6 +867,29 @@ static void build_readme(CNet &net, int n, int classes, int *inp, int *outp) {
 	net.init_inputs(11);
 }
 
+// A net whose data input feeds a Linear and, as a skip connection, the Residual above it: Linear, CGelu, Residual(x, .),
+// Linear to the classes, CrossEntropy.  Only the input-gradient product of the first Linear can wait for a look at the data
+// input; the Residual's backward pass writes its share of that gradient as a by-product.
+static void build_linear_head(CNet &net, int n, int classes, int *inp, int *outp) {
+	*inp = net.add(new CInput(OutSize(n)));
+	auto w1 = net.add(new CInput(OutSize(n * n)));
+	auto lin1 = net.add(new Linear(InSize(n), InSize(n * n)), {*inp, w1});
+	auto gelu = net.add(new CGelu(InSize(n)), {lin1});
+	auto res = net.add(new Residual(InSize(n)), {*inp, gelu});
+	auto w2 = net.add(new CInput(OutSize(n * classes)));
+	auto lin2 = net.add(new Linear(InSize(n), InSize(n * classes)), {res, w2});
+	*outp = net.add(new CrossEntropy(InSize(classes)), {lin2});
+	net.init_inputs(11);
+	// weights of the usual size for a layer n wide (init_inputs scales by the number of weights, which leaves them tiny)
+	for (int uid : {w1, w2}) {
+		Vars *v = net[uid]->mutable_input();
+		for (int k = 0; k < v->length_; ++k) {
+			v->real_[k] *= (float) n * 0.5f;
+			v->imag_[k] *= (float) n * 0.5f;
+		}
+	}
+}
+
 struct SyntheticReader : public BatchedDataReader {
 	SyntheticReader(int dim, int count, int classes, bool real_samples = false) : BatchedDataReader(dim) {
 		orc::Rng rng(123);
@@ -1047,7 +1070,7 @@ static void test_pipeline(int B, int steps) {
 // the difference must not: two backward passes before one update (the input keeps adding, impl/cinput.h:54-65), a look at
 // the gradient between backward pass and update, an Adam-style step, recorded phases, a whole recorded step after a
 // backward pass that was never followed by an update.
-static void test_deferred_gathers() {
+static void test_deferred_gathers(void (*build)(CNet &, int, int, int *, int *), const std::string &which) {
 	const int n = 96, classes = 10, B = 32;
 	if (cnet_init(0) != CNET_OK) {
 		expect("cnet_init", false);
@@ -1060,7 +1083,7 @@ static void test_deferred_gathers() {
 	for (int variant = 0; variant < 6; ++variant) {
 		CNet net;
 		int inp, outp;
-		build_readme(net, n, classes, &inp, &outp);
+		build(net, n, classes, &inp, &outp);
 		net.allocateOnGpu(B);
 		net.deferGathers(variant % 2 == 0);
 		if (variant == 2 || variant == 3) net.useGraphs(true);
@@ -1126,13 +1149,16 @@ static void test_deferred_gathers() {
 			gradients();
 		}
 	}
-	expect("deferred and immediate gathers: same losses, gradients and weights", trace[0] == trace[1] && trace[0].size() > 1000);
-	expect("the data input's backward pass and step left out until something looks, against done at once", trace[0] == trace[4] && trace[1] == trace[5]);
-	expect("the same with recorded phases", trace[2] == trace[3] && !trace[2].empty());
-	expect("recorded phases agree with launches one by one", std::equal(trace[2].begin(), trace[2].end(), trace[0].begin()));
+	expect(which + ": deferred and immediate gathers: same losses, gradients and weights", trace[0] == trace[1] && trace[0].size() > 1000);
+	expect(which + ": the data input's backward pass and step left out until something looks, against done at once", trace[0] == trace[4] && trace[1] == trace[5]);
+	expect(which + ": the same with recorded phases", trace[2] == trace[3] && !trace[2].empty());
+	expect(which + ": recorded phases agree with launches one by one", std::equal(trace[2].begin(), trace[2].end(), trace[0].begin()));
 	bool finite = true;
 	for (float v : trace[0]) finite = finite && std::isfinite(v);
-	expect("all finite", finite);
+	expect(which + ": all finite", finite);
+	bool moved = false;  // the trace must depend on what the steps did
+	for (size_t k = 1; k < 3; ++k) moved = moved || trace[0][k] != trace[0][0];
+	expect(which + ": the losses of the first steps differ", moved);
 }
 
 // ------------------------------------------------------------------------------------------------- real-valued batches
@@ -1620,7 +1646,10 @@ int main(int argc, char **argv) {
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
 		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12);
 		if (what == "frozen_input" || what == "all") test_frozen_input();
-		if (what == "deferred" || what == "all") test_deferred_gathers();
+		if (what == "deferred" || what == "all") {
+			test_deferred_gathers(build_readme, "transform on the data input");
+			test_deferred_gathers(build_linear_head, "Linear and Residual on the data input");
+		}
 		if (what == "real_batches" || what == "all") test_real_batches();
 		if (what == "upstream_nets" || what == "all") test_upstream_nets();
 		if (what == "errors" || what == "all") test_errors();
