@@ -6,6 +6,7 @@
 
 #include <cstdarg>
 #include <cstdint>
+#include <cstdlib>
 #include <cstdio>
 
 #include "cnet_hip.h"
@@ -126,6 +127,32 @@ __device__ __forceinline__ float gelu_slope(float t) {
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// The cache policy of a launch that touches `planes` fp32 planes of `elems` elements each.  Operands that fit the 256 MB
+// memory-side cache together are left there for the next kernel (plain accesses: with hints the next kernel no longer
+// finds them and loses up to 20 %).  Beyond that everything streams from and to HBM, and which side carries the streaming
+// hint decides up to 30 % of the rate.  Measured kernel by kernel at [8192 x 4096] (the same ranking on three machines,
+// with the operands in other buffers and at other offsets), ms under: the hint on loads and stores (1) / plain loads,
+// streaming stores (2) / streaming loads, device-scope stores (3) / no hints:
+//   two planes read:    CGelu forward .086 / .074 / .076 / .097; Hadamard + CGelu forward (four written) .137 / .113 / .138 / .149;
+//                       Residual backward of a pair (four written) .144 / .113 / .147 / .155; L2Out backward .142 / .113 / .148 / .162
+//   four read, two written: CGelu backward of a pair .129 / .152 / .116 / .152; shared-weight Hadamard backward of a pair
+//                       .132 / .146 / .121 / .158; SoftMax backward of a pair .129 / .141 / .115 / .148; but Residual forward
+//                       .109 / .144 / .136 / .150
+//   six read, four written: CGelu backward .221 / .251 / .249 / .257; Residual + CGelu backward of a pair .222 / .245 / .228 / .239
+//   four read and written (the SGD step) .179 / .187 / .178 / .195; six (the Adam-style step) .279 / .318 / .304 / .315
+// A probe kernel that only moves R planes to W planes ranks the three the same way.  `when_streaming` is the caller's entry
+// of that table.
+constexpr int ST_BOTH = 1, ST_STORES = 2, ST_LOADS = 3;
+inline int stream_policy(int when_streaming, int planes, long elems) {
+	static const int forced = [] {
+		const char *e = getenv("CNET_STREAM_POLICY");  // tuning override: 0..3 for every launch beyond the cache size
+		return e ? atoi(e) : -1;
+	}();
+	if ((long) planes * elems * 4 <= (256L << 20)) return 0;
+	return forced >= 0 && forced <= 3 ? forced : when_streaming;
+}
+
 
 }  // namespace cnet
 

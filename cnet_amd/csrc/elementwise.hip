@@ -18,15 +18,17 @@ constexpr int TPB = 256;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// NT: the access carries the streaming (non-temporal) hint.  Launches whose operands together exceed the 256 MB
-// memory-side cache set it: nothing they touch can be found there again, and without the hint the lines they leave
-// behind cost ~8 % of the achievable rate; smaller launches keep normal accesses, because the next kernel does find
-// their results in that cache.
-template <int V, bool NT>
+// NT: the cache policy of the 128-bit accesses of a launch (see stream_policy below for how it is chosen).
+//   0  plain loads and stores: launches whose operands fit the 256 MB memory-side cache, where the next kernel finds them
+//   1  loads and stores carry the streaming (non-temporal) hint
+//   2  plain loads, streaming stores
+//   3  streaming loads, stores at device scope (sc1) without the hint
+constexpr bool nt_loads(int policy) { return policy == 1 || policy == 3; }
+template <int V, int NT>
 __device__ __forceinline__ void ldv(float (&d)[V], const float *__restrict__ p) {
 	if (V == 4) {
 		const f32x4 *q = reinterpret_cast<const f32x4 *>(p);
-		f32x4 t = NT ? __builtin_nontemporal_load(q) : *q;
+		f32x4 t = nt_loads(NT) ? __builtin_nontemporal_load(q) : *q;
 		d[0] = t.x;
 		d[1 % V] = t.y;
 		d[2 % V] = t.z;
@@ -36,12 +38,18 @@ __device__ __forceinline__ void ldv(float (&d)[V], const float *__restrict__ p) 
 	}
 }
 
-template <int V, bool NT>
+template <int V, int NT>
 __device__ __forceinline__ void stv(float *__restrict__ p, const float (&d)[V]) {
 	if (V == 4) {
 		f32x4 t = {d[0], d[1 % V], d[2 % V], d[3 % V]};
-		if (NT)
-			__builtin_nontemporal_store(t, reinterpret_cast<f32x4 *>(p));
+		// The hinted stores are written out: when the two arms of an `accumulate` branch end in the same store the compiler
+		// merges them and the merged store loses the non-temporal mark (seen in the listing of every kernel that goes through
+		// outv), so the builtin gave plain stores exactly where the hint was wanted.  The s_nop covers the wait state between
+		// a 128-bit store and a vector instruction that overwrites its data registers, which the compiler cannot see here.
+		if (NT == 1 || NT == 2)
+			asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(p), "v"(t) : "memory");
+		else if (NT == 3)
+			asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(t) : "memory");
 		else
 			*reinterpret_cast<f32x4 *>(p) = t;
 	} else {
@@ -50,7 +58,7 @@ __device__ __forceinline__ void stv(float *__restrict__ p, const float (&d)[V]) 
 }
 
 // store or accumulate
-template <int V, bool NT>
+template <int V, int NT>
 __device__ __forceinline__ void outv(float *__restrict__ p, const float (&d)[V], int accumulate) {
 	if (accumulate) {
 		float o[V];
@@ -79,7 +87,7 @@ struct CGrad4 {
 	const long col = (idx - row * cv) * V;
 
 // ------------------------------------------------------------------------------------------------ Hadamard
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void hadamard_fwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
 		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, float *__restrict__ yr,
 		float *__restrict__ yi, long ldy, int rows, int cols) {
@@ -99,7 +107,7 @@ __global__ __launch_bounds__(TPB) void hadamard_fwd_kernel(const float *__restri
 }
 
 // Both operands per-row: du = (G v, Gs conj v), dv = (G u, Gs conj u).
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
 		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, CGrad4 g, long ldg, Grad4 du, long lddu,
 		Grad4 dv, long lddv, int rows, int cols, int accumulate) {
@@ -146,7 +154,7 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_kernel(const float *__restri
 // the slabs in slab order.  Deterministic: no atomics, fixed summation tree.
 constexpr int CS_X = 64, CS_Y = 4;
 
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *__restrict__ ur, const float *__restrict__ ui,
 		long ldu, const float *__restrict__ vr, const float *__restrict__ vi, CGrad4 g, long ldg, Grad4 du, long lddu,
 		float *__restrict__ partial, int rows, int cols, int rows_per_slab, int accumulate) {
@@ -235,7 +243,7 @@ __global__ __launch_bounds__(TPB) void slab_sum_kernel(const float *__restrict__
 
 // ------------------------------------------------------------------------------------------------ CGelu
 // tanh-GELU on each real plane (impl/relu.h:119-131 upstream).
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void gelu_fwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		float *__restrict__ yr, float *__restrict__ yi, long ldy, int rows, int cols) {
 	CNET_ELEM_INDEX();
@@ -252,7 +260,7 @@ __global__ __launch_bounds__(TPB) void gelu_fwd_kernel(const float *__restrict__
 }
 
 // dz = G s + Gs d ; dzs = G d + Gs s ; s = (g'(x)+g'(y))/2, d = (g'(x)-g'(y))/2   (impl/relu.h:144-166 upstream)
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void gelu_bwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		CGrad4 g, long ldg, Grad4 dx, long lddx, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
@@ -286,7 +294,7 @@ __global__ __launch_bounds__(TPB) void gelu_bwd_kernel(const float *__restrict__
 
 // Hadamard followed by CGelu in one pass: h = u .* v and a = gelu(h) are both written (the backward pass needs h), u and v
 // are read once and h is not read back: 24 bytes per complex element instead of 16 + 16.
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void hadamard_gelu_fwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
 		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, float *__restrict__ hr, float *__restrict__ hi, long ldh,
 		float *__restrict__ yr, float *__restrict__ yi, long ldy, int rows, int cols) {
@@ -315,7 +323,7 @@ __global__ __launch_bounds__(TPB) void hadamard_gelu_fwd_kernel(const float *__r
 // ------------------------------------------------------------------------------------------------ CRelu
 // y = z where Re z > 0 and Im z > 0, else 0 (impl/relu.h:32-46 upstream); the gradients pass under the same test
 // (impl/relu.h:48-63).
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void crelu_fwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		float *__restrict__ yr, float *__restrict__ yi, long ldy, int rows, int cols) {
 	CNET_ELEM_INDEX();
@@ -332,7 +340,7 @@ __global__ __launch_bounds__(TPB) void crelu_fwd_kernel(const float *__restrict_
 	stv<V, NT>(yi + row * ldy + col, b);
 }
 
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void crelu_bwd_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		CGrad4 g, long ldg, Grad4 dx, long lddx, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
@@ -351,7 +359,7 @@ __global__ __launch_bounds__(TPB) void crelu_bwd_kernel(const float *__restrict_
 }
 
 // ------------------------------------------------------------------------------------------------ Residual
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void residual_fwd_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
 		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, float *__restrict__ yr,
 		float *__restrict__ yi, long ldy, int rows, int cols) {
@@ -370,7 +378,7 @@ __global__ __launch_bounds__(TPB) void residual_fwd_kernel(const float *__restri
 	stv<V, NT>(yi + row * ldy + col, b);
 }
 
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void residual_bwd_kernel(CGrad4 g, long ldg, Grad4 du, long lddu, Grad4 dv, long lddv,
 		int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
@@ -392,7 +400,7 @@ __global__ __launch_bounds__(TPB) void residual_bwd_kernel(CGrad4 g, long ldg, G
 
 // ------------------------------------------------------------------------------------------------ loss backward
 // L2Out: dz = conj z, dzs = z  (impl/l2out.h:44-58 upstream)
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void l2out_bwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		Grad4 dz, long lddz, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
@@ -410,7 +418,7 @@ __global__ __launch_bounds__(TPB) void l2out_bwd_kernel(const float *__restrict_
 
 // CrossEntropy (impl/crossent.h:82-104 upstream): assigns.  label: dzs = -z (S-m)/(m S), m = max(|z_l|^2, 1e-15);
 // other entries: dzs = z/S; dz = conj(dzs).
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void crossent_bwd_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		const float *__restrict__ s, const int *__restrict__ labels, Grad4 dz, long lddz, int rows, int cols) {
 	CNET_ELEM_INDEX();
@@ -451,7 +459,7 @@ struct Pair2 {  // dz planes, and optionally the planes that receive the conjuga
 };
 
 // (o_r, o_i) to the dz planes and, conjugated, to the dz* planes when they are wanted
-template <int V, bool NT>
+template <int V, int NT>
 __device__ __forceinline__ void out_pair(const Pair2 &d, long off, const float (&o_r)[V], const float (&o_i)[V], int accumulate) {
 	outv<V, NT>(d.dz_re + off, o_r, accumulate);
 	outv<V, NT>(d.dz_im + off, o_i, accumulate);
@@ -464,7 +472,7 @@ __device__ __forceinline__ void out_pair(const Pair2 &d, long off, const float (
 	}
 }
 
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void gelu_bwd_sym_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		const float *__restrict__ g_re, const float *__restrict__ g_im, long ldg, Pair2 dx, long lddx, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
@@ -483,7 +491,7 @@ __global__ __launch_bounds__(TPB) void gelu_bwd_sym_kernel(const float *__restri
 	out_pair<V, NT>(dx, row * lddx + col, o_r, o_i, accumulate);
 }
 
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void crelu_bwd_sym_kernel(const float *__restrict__ xr, const float *__restrict__ xi, long ldx,
 		const float *__restrict__ g_re, const float *__restrict__ g_im, long ldg, Pair2 dx, long lddx, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
@@ -501,7 +509,7 @@ __global__ __launch_bounds__(TPB) void crelu_bwd_sym_kernel(const float *__restr
 	out_pair<V, NT>(dx, row * lddx + col, o_r, o_i, accumulate);
 }
 
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void residual_bwd_sym_kernel(const float *__restrict__ g_re, const float *__restrict__ g_im, long ldg,
 		Pair2 du, long lddu, Pair2 dv, long lddv, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
@@ -514,7 +522,7 @@ __global__ __launch_bounds__(TPB) void residual_bwd_sym_kernel(const float *__re
 
 // A Residual whose result feeds two consumers: the two incoming gradients are added here (g1 first, as two passes with
 // accumulation would), so du and dv are written once instead of written, read and written again
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void residual_bwd_sym2_kernel(const float *__restrict__ g1_re, const float *__restrict__ g1_im, long ldg1,
 		const float *__restrict__ g2_re, const float *__restrict__ g2_im, long ldg2, Pair2 du, long lddu, Pair2 dv, long lddv, int rows,
 		int cols, int accumulate) {
@@ -568,7 +576,7 @@ __global__ __launch_bounds__(TPB) void residual_bwd_sym2_kernel(const float *__r
 // consumers, added as residual_bwd_sym2_kernel adds them) goes to the other operand (du) and, optionally, to the CGelu's
 // result (dv); its CGelu backward at h, the CGelu's operand, goes to dh with the arithmetic of gelu_bwd_sym_kernel.  The
 // gradient of the CGelu's result is not read back: 40 bytes per complex element (32 with one consumer) against 32 + 24.
-template <int V, bool NT, bool TWO>
+template <int V, int NT, bool TWO>
 __global__ __launch_bounds__(TPB) void residual_gelu_bwd_sym_kernel(const float *__restrict__ g1_re, const float *__restrict__ g1_im,
 		long ldg1, const float *__restrict__ g2_re, const float *__restrict__ g2_im, long ldg2, const float *__restrict__ hr,
 		const float *__restrict__ hi, long ldh, Pair2 du, long lddu, Pair2 dv, long lddv, Pair2 dh, long lddh, int rows, int cols) {
@@ -604,7 +612,7 @@ __global__ __launch_bounds__(TPB) void residual_gelu_bwd_sym_kernel(const float 
 // The gradient that reaches a Hadamard through a CGelu on its result, formed in place: h = u .* v is recomputed (the bits
 // of the forward pass), g becomes the CGelu backward of g at h (the arithmetic of gelu_bwd_sym_kernel), and is stored to
 // dh, the gradient planes of the CGelu's operand, which stay readable (skipped when dh.dz_re is NULL).
-template <int V, bool NT>
+template <int V, int NT>
 __device__ __forceinline__ void through_gelu(const float (&a)[V], const float (&b)[V], const float (&c)[V], const float (&d)[V],
 		float (&gr)[V], float (&gi)[V], const Pair2 &dh, long off) {
 #pragma unroll
@@ -620,7 +628,7 @@ __device__ __forceinline__ void through_gelu(const float (&a)[V], const float (&
 }
 
 // du = G v, dv = G u (per-row operands).  GELU: G is first taken through a CGelu that sits on the Hadamard's result.
-template <int V, bool NT, bool GELU>
+template <int V, int NT, bool GELU>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_sym_kernel(const float *__restrict__ ur, const float *__restrict__ ui, long ldu,
 		const float *__restrict__ vr, const float *__restrict__ vi, long ldv_, const float *__restrict__ g_re,
 		const float *__restrict__ g_im, long ldg, Pair2 dh, long lddh, Pair2 du, long lddu, Pair2 dv, long lddv, int rows, int cols,
@@ -649,7 +657,7 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_sym_kernel(const float *__re
 }
 
 // v is one shared parameter row: as hadamard_bwd_shared_kernel, two partial planes per slab
-template <int V, bool NT, bool GELU>
+template <int V, int NT, bool GELU>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_sym_kernel(const float *__restrict__ ur, const float *__restrict__ ui,
 		long ldu, const float *__restrict__ vr, const float *__restrict__ vi, const float *__restrict__ g_re,
 		const float *__restrict__ g_im, long ldg, Pair2 dh, long lddh, Pair2 du, long lddu, float *__restrict__ partial, int rows,
@@ -731,7 +739,7 @@ __global__ __launch_bounds__(TPB) void slab_sum_sym_kernel(const float *__restri
 }
 
 // L2Out: dz = conj z (and dz* = z)
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void l2out_bwd_sym_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		Pair2 dz, long lddz, int rows, int cols, int accumulate) {
 	CNET_ELEM_INDEX();
@@ -744,7 +752,7 @@ __global__ __launch_bounds__(TPB) void l2out_bwd_sym_kernel(const float *__restr
 }
 
 // CrossEntropy: dz* as in crossent_bwd_kernel, dz = conj(dz*); assigns
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void crossent_bwd_sym_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
 		const float *__restrict__ s, const int *__restrict__ labels, Pair2 dz, long lddz, int rows, int cols) {
 	CNET_ELEM_INDEX();
@@ -771,7 +779,7 @@ __global__ __launch_bounds__(TPB) void crossent_bwd_sym_kernel(const float *__re
 }
 
 // ------------------------------------------------------------------------------------------------ plumbing
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void copy2d_kernel(const float *__restrict__ src, long lds, float *__restrict__ dst, long ldd,
 		int rows, int cols, int add) {
 	CNET_ELEM_INDEX();
@@ -781,7 +789,7 @@ __global__ __launch_bounds__(TPB) void copy2d_kernel(const float *__restrict__ s
 }
 
 // z -= lr * dzs ; dzs = 0   (impl/cfunc.h:147-152, impl/cnet.h:413-421 upstream)
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void sgd_kernel(float *__restrict__ zr, float *__restrict__ zi, float *__restrict__ dr,
 		float *__restrict__ di, long n, float lr, int zero_grad) {
 	const long i = ((long) blockIdx.x * TPB + threadIdx.x) * V;
@@ -808,7 +816,7 @@ __global__ __launch_bounds__(TPB) void sgd_kernel(float *__restrict__ zr, float 
 // m = beta m + (1 - beta) dzs ; z -= lr m / denom ; dzs = 0   (impl/cfunc.h:273-287, gpu/kernels.cpp:494-514 upstream).
 // denom = 1 - beta^(t+1) arrives as a double and the quotient is formed in double, as the CPU loop does
 // (pow(float, int) promotes), so the parameter gets one rounding per step.
-template <int V, bool NT>
+template <int V, int NT>
 __global__ __launch_bounds__(TPB) void adam_kernel(float *__restrict__ zr, float *__restrict__ zi, float *__restrict__ mr,
 		float *__restrict__ mi, float *__restrict__ dr, float *__restrict__ di, long n, float lr, float beta, double denom,
 		int zero_grad) {
@@ -931,17 +939,16 @@ inline bool all_mult4(std::initializer_list<long> v) {
 
 using namespace cnet;
 
-// the 128-bit variant of a kernel, with or without the streaming hint
-#define CNET_LAUNCH_V4(kernel, nt, ...)                          \
-	do {                                                         \
-		if (nt)                                                  \
-			hipLaunchKernelGGL((kernel<4, true>), __VA_ARGS__);  \
-		else                                                     \
-			hipLaunchKernelGGL((kernel<4, false>), __VA_ARGS__); \
+// the 128-bit variant of a kernel under cache policy `pol` (0..3)
+#define CNET_LAUNCH_V4(kernel, pol, ...)                                    \
+	do {                                                                    \
+		switch (pol) {                                                      \
+		case 1: hipLaunchKernelGGL((kernel<4, 1>), __VA_ARGS__); break;     \
+		case 2: hipLaunchKernelGGL((kernel<4, 2>), __VA_ARGS__); break;     \
+		case 3: hipLaunchKernelGGL((kernel<4, 3>), __VA_ARGS__); break;     \
+		default: hipLaunchKernelGGL((kernel<4, 0>), __VA_ARGS__); break;    \
+		}                                                                   \
 	} while (0)
-
-// planes: fp32 planes of [rows x cols] the launch reads or writes
-static inline bool streaming(int planes, long elems) { return (long) planes * elems * 4 > (256L << 20); }
 
 #define CNET_GRID_2D(V) dim3(nblocks((long) rows * (cols / (V)))), dim3(TPB), 0, rt().stream
 
@@ -978,11 +985,11 @@ int cnet_hadamard_fwd(const float *u_re, const float *u_im, int64_t ldu, const f
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && y_re && y_im);
 	CNET_CHECK_ARG(ldu >= cols && ldy >= cols && (ldv == 0 || ldv >= cols));
-	const bool nt = streaming(4, (long) rows * cols);
+	const int nt = stream_policy(ST_STORES, 4 + (ldv ? 2 : 0), (long) rows * cols);
 	if (all_mult4({cols, ldu, ldv, ldy}) && all_aligned({u_re, u_im, v_re, v_im, y_re, y_im}))
 		CNET_LAUNCH_V4(hadamard_fwd_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
 	else
-		hipLaunchKernelGGL((hadamard_fwd_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+		hipLaunchKernelGGL((hadamard_fwd_kernel<1, 0>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1003,13 +1010,13 @@ int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const f
 	bool vec = all_mult4({cols, ldu, ldv, ldg, lddu, ldv ? lddv : 0}) &&
 			all_aligned({u_re, u_im, v_re, v_im, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, du_dz_re, du_dz_im, du_dzs_re,
 					du_dzs_im, dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im});
-	const bool nt = streaming(10, (long) rows * cols);
+	const int nt = stream_policy(ST_BOTH, 10 + (ldv ? 6 : 0), (long) rows * cols);
 	if (ldv != 0) {
 		if (vec)
 			CNET_LAUNCH_V4(hadamard_bwd_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, g, ldg, du, lddu, dv, lddv,
 					rows, cols, accumulate);
 		else
-			hipLaunchKernelGGL((hadamard_bwd_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, g, ldg, du, lddu, dv, lddv,
+			hipLaunchKernelGGL((hadamard_bwd_kernel<1, 0>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, g, ldg, du, lddu, dv, lddv,
 					rows, cols, accumulate);
 		CNET_LAUNCH_CHECK();
 		return CNET_OK;
@@ -1028,7 +1035,7 @@ int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const f
 		CNET_LAUNCH_V4(hadamard_bwd_shared_kernel, nt, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
 				lddu, partial, rows, cols, rows_per_slab, accumulate);
 	else
-		hipLaunchKernelGGL((hadamard_bwd_shared_kernel<1, false>), grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
+		hipLaunchKernelGGL((hadamard_bwd_shared_kernel<1, 0>), grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
 				lddu, partial, rows, cols, rows_per_slab, accumulate);
 	CNET_LAUNCH_CHECK();
 	hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned) ((4L * cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
@@ -1041,11 +1048,11 @@ int cnet_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_r
 	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= cols && ldy >= cols);
-	const bool nt = streaming(4, (long) rows * cols);
+	const int nt = stream_policy(ST_STORES, 4, (long) rows * cols);
 	if (all_mult4({cols, ldx, ldy}) && all_aligned({x_re, x_im, y_re, y_im}))
 		CNET_LAUNCH_V4(gelu_fwd_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
 	else
-		hipLaunchKernelGGL((gelu_fwd_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+		hipLaunchKernelGGL((gelu_fwd_kernel<1, 0>), CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1060,12 +1067,12 @@ int cnet_cgelu_bwd(const float *x_re, const float *x_im, int64_t ldx, const floa
 	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
 	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
 	Grad4 dx = {dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im};
-	const bool nt = streaming(10, (long) rows * cols);
+	const int nt = stream_policy(ST_BOTH, 10, (long) rows * cols);
 	if (all_mult4({cols, ldx, ldg, lddx}) &&
 			all_aligned({x_re, x_im, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
 		CNET_LAUNCH_V4(gelu_bwd_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL((gelu_bwd_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+		hipLaunchKernelGGL((gelu_bwd_kernel<1, 0>), CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1075,11 +1082,11 @@ int cnet_crelu_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_r
 	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(x_re && x_im && y_re && y_im && ldx >= cols && ldy >= cols);
-	const bool nt = streaming(4, (long) rows * cols);
+	const int nt = stream_policy(ST_STORES, 4, (long) rows * cols);
 	if (all_mult4({cols, ldx, ldy}) && all_aligned({x_re, x_im, y_re, y_im}))
 		CNET_LAUNCH_V4(crelu_fwd_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
 	else
-		hipLaunchKernelGGL((crelu_fwd_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
+		hipLaunchKernelGGL((crelu_fwd_kernel<1, 0>), CNET_GRID_2D(1), x_re, x_im, ldx, y_re, y_im, ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1094,12 +1101,12 @@ int cnet_crelu_bwd(const float *x_re, const float *x_im, int64_t ldx, const floa
 	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
 	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
 	Grad4 dx = {dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im};
-	const bool nt = streaming(10, (long) rows * cols);
+	const int nt = stream_policy(ST_BOTH, 10, (long) rows * cols);
 	if (all_mult4({cols, ldx, ldg, lddx}) &&
 			all_aligned({x_re, x_im, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
 		CNET_LAUNCH_V4(crelu_bwd_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL((crelu_bwd_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
+		hipLaunchKernelGGL((crelu_bwd_kernel<1, 0>), CNET_GRID_2D(1), x_re, x_im, ldx, g, ldg, dx, lddx, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1111,11 +1118,11 @@ int cnet_residual_fwd(const float *u_re, const float *u_im, int64_t ldu, const f
 	if (!rows || !cols) return CNET_OK;
 	// a leading dimension of 0 makes that operand one row shared by all rows (a parameter added to every sample)
 	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && y_re && y_im && (ldu >= cols || ldu == 0) && (ldv >= cols || ldv == 0) && ldy >= cols);
-	const bool nt = streaming(6, (long) rows * cols);
+	const int nt = stream_policy(ST_BOTH, 2 + (ldu ? 2 : 0) + (ldv ? 2 : 0), (long) rows * cols);
 	if (all_mult4({cols, ldu, ldv, ldy}) && all_aligned({u_re, u_im, v_re, v_im, y_re, y_im}))
 		CNET_LAUNCH_V4(residual_fwd_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
 	else
-		hipLaunchKernelGGL((residual_fwd_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
+		hipLaunchKernelGGL((residual_fwd_kernel<1, 0>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, y_re, y_im, ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1132,13 +1139,13 @@ int cnet_residual_bwd(const float *g_dz_re, const float *g_dz_im, const float *g
 	CGrad4 g = {g_dz_re, g_dz_im, g_dzs_re, g_dzs_im};
 	Grad4 du = {du_dz_re, du_dz_im, du_dzs_re, du_dzs_im};
 	Grad4 dv = {dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im};
-	const bool nt = streaming(12, (long) rows * cols);
+	const int nt = stream_policy(ST_LOADS, 12, (long) rows * cols);
 	if (all_mult4({cols, ldg, lddu, lddv}) &&
 			all_aligned({g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, du_dz_re, du_dz_im, du_dzs_re, du_dzs_im, dv_dz_re, dv_dz_im,
 					dv_dzs_re, dv_dzs_im}))
 		CNET_LAUNCH_V4(residual_bwd_kernel, nt, CNET_GRID_2D(4), g, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL((residual_bwd_kernel<1, false>), CNET_GRID_2D(1), g, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
+		hipLaunchKernelGGL((residual_bwd_kernel<1, 0>), CNET_GRID_2D(1), g, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1150,11 +1157,11 @@ int cnet_l2out_bwd(const float *z_re, const float *z_im, int64_t ldz, float *dz_
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(z_re && z_im && dz_dz_re && dz_dz_im && dz_dzs_re && dz_dzs_im && ldz >= cols && lddz >= cols);
 	Grad4 dz = {dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im};
-	const bool nt = streaming(6, (long) rows * cols);
+	const int nt = stream_policy(ST_STORES, 6, (long) rows * cols);
 	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
 		CNET_LAUNCH_V4(l2out_bwd_kernel, nt, CNET_GRID_2D(4), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL((l2out_bwd_kernel<1, false>), CNET_GRID_2D(1), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
+		hipLaunchKernelGGL((l2out_bwd_kernel<1, 0>), CNET_GRID_2D(1), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1166,11 +1173,11 @@ int cnet_cross_entropy_bwd(const float *z_re, const float *z_im, int64_t ldz, co
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(z_re && z_im && s && labels && dz_dz_re && dz_dz_im && dz_dzs_re && dz_dzs_im && ldz >= cols && lddz >= cols);
 	Grad4 dz = {dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im};
-	const bool nt = streaming(6, (long) rows * cols);
+	const int nt = stream_policy(ST_BOTH, 6, (long) rows * cols);
 	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
 		CNET_LAUNCH_V4(crossent_bwd_kernel, nt, CNET_GRID_2D(4), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
 	else
-		hipLaunchKernelGGL((crossent_bwd_kernel<1, false>), CNET_GRID_2D(1), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
+		hipLaunchKernelGGL((crossent_bwd_kernel<1, 0>), CNET_GRID_2D(1), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1180,11 +1187,11 @@ static int copy_or_add(const float *src, int64_t lds, float *dst, int64_t ldd, i
 	CNET_CHECK_ARG(rows >= 0 && cols >= 0);
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(src && dst && lds >= cols && ldd >= cols);
-	const bool nt = streaming(2, (long) rows * cols);
+	const int nt = stream_policy(ST_LOADS, 2, (long) rows * cols);
 	if (all_mult4({cols, lds, ldd}) && all_aligned({src, dst}))
 		CNET_LAUNCH_V4(copy2d_kernel, nt, CNET_GRID_2D(4), src, lds, dst, ldd, rows, cols, add);
 	else
-		hipLaunchKernelGGL((copy2d_kernel<1, false>), CNET_GRID_2D(1), src, lds, dst, ldd, rows, cols, add);
+		hipLaunchKernelGGL((copy2d_kernel<1, 0>), CNET_GRID_2D(1), src, lds, dst, ldd, rows, cols, add);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1228,11 +1235,11 @@ int cnet_sgd_update(float *z_re, float *z_im, float *dzs_re, float *dzs_im, int6
 	CNET_CHECK_ARG(n >= 0);
 	if (!n) return CNET_OK;
 	CNET_CHECK_ARG(z_re && z_im && dzs_re && dzs_im);
-	const bool nt = streaming(4, (long) n);
+	const int nt = stream_policy(ST_LOADS, 4, (long) n);
 	if (n % 4 == 0 && all_aligned({z_re, z_im, dzs_re, dzs_im}))
 		CNET_LAUNCH_V4(sgd_kernel, nt, dim3(nblocks(n / 4)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
 	else
-		hipLaunchKernelGGL((sgd_kernel<1, false>), dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
+		hipLaunchKernelGGL((sgd_kernel<1, 0>), dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, dzs_re, dzs_im, (long) n, lr, zero_grad);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1274,12 +1281,12 @@ int cnet_adam_update(float *z_re, float *z_im, float *m_re, float *m_im, float *
 	CNET_CHECK_ARG(z_re && z_im && m_re && m_im && dzs_re && dzs_im);
 	const double denom = 1 - std::pow((double) beta, (double) (t + 1));
 	CNET_CHECK_ARG(denom != 0.0);
-	const bool nt = streaming(6, (long) n);
+	const int nt = stream_policy(ST_BOTH, 6, (long) n);
 	if (n % 4 == 0 && all_aligned({z_re, z_im, m_re, m_im, dzs_re, dzs_im}))
 		CNET_LAUNCH_V4(adam_kernel, nt, dim3(nblocks(n / 4)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
 				(long) n, lr, beta, denom, zero_grad);
 	else
-		hipLaunchKernelGGL((adam_kernel<1, false>), dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
+		hipLaunchKernelGGL((adam_kernel<1, 0>), dim3(nblocks(n)), dim3(TPB), 0, rt().stream, z_re, z_im, m_re, m_im, dzs_re, dzs_im,
 				(long) n, lr, beta, denom, zero_grad);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
@@ -1299,11 +1306,11 @@ int cnet_cgelu_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const 
 	CNET_CHECK_ARG(x_re && x_im && g_dz_re && g_dz_im);
 	CNET_CHECK_PAIR(dx);
 	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
-	const bool nt = streaming(4 + pair_planes(dx), (long) rows * cols);
+	const int nt = stream_policy(ST_LOADS, 4 + pair_planes(dx), (long) rows * cols);
 	if (all_mult4({cols, ldx, ldg, lddx}) && all_aligned({x_re, x_im, g_dz_re, g_dz_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
 		CNET_LAUNCH_V4(gelu_bwd_sym_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL((gelu_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
+		hipLaunchKernelGGL((gelu_bwd_sym_kernel<1, 0>), CNET_GRID_2D(1), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1317,11 +1324,11 @@ int cnet_crelu_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const 
 	CNET_CHECK_ARG(x_re && x_im && g_dz_re && g_dz_im);
 	CNET_CHECK_PAIR(dx);
 	CNET_CHECK_ARG(ldx >= cols && ldg >= cols && lddx >= cols);
-	const bool nt = streaming(4 + pair_planes(dx), (long) rows * cols);
+	const int nt = stream_policy(ST_LOADS, 4 + pair_planes(dx), (long) rows * cols);
 	if (all_mult4({cols, ldx, ldg, lddx}) && all_aligned({x_re, x_im, g_dz_re, g_dz_im, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im}))
 		CNET_LAUNCH_V4(crelu_bwd_sym_kernel, nt, CNET_GRID_2D(4), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL((crelu_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
+		hipLaunchKernelGGL((crelu_bwd_sym_kernel<1, 0>), CNET_GRID_2D(1), x_re, x_im, ldx, g_dz_re, g_dz_im, ldg, dx, lddx, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1337,12 +1344,12 @@ int cnet_residual_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ld
 	CNET_CHECK_PAIR(du);
 	CNET_CHECK_PAIR(dv);
 	CNET_CHECK_ARG(ldg >= cols && lddu >= cols && lddv >= cols);
-	const bool nt = streaming(2 + pair_planes(du) + pair_planes(dv), (long) rows * cols);
+	const int nt = stream_policy(ST_STORES, 2 + pair_planes(du) + pair_planes(dv), (long) rows * cols);
 	if (all_mult4({cols, ldg, lddu, lddv}) &&
 			all_aligned({g_dz_re, g_dz_im, du_dz_re, du_dz_im, du_dzs_re, du_dzs_im, dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im}))
 		CNET_LAUNCH_V4(residual_bwd_sym_kernel, nt, CNET_GRID_2D(4), g_dz_re, g_dz_im, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL((residual_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), g_dz_re, g_dz_im, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
+		hipLaunchKernelGGL((residual_bwd_sym_kernel<1, 0>), CNET_GRID_2D(1), g_dz_re, g_dz_im, ldg, du, lddu, dv, lddv, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1358,33 +1365,37 @@ int cnet_residual_bwd_sym2(const float *g1_dz_re, const float *g1_dz_im, int64_t
 	CNET_CHECK_PAIR(du);
 	CNET_CHECK_PAIR(dv);
 	CNET_CHECK_ARG(ldg1 >= cols && ldg2 >= cols && lddu >= cols && lddv >= cols);
-	const bool nt = streaming(4 + pair_planes(du) + pair_planes(dv), (long) rows * cols);
+	const int nt = stream_policy(ST_LOADS, 4 + pair_planes(du) + pair_planes(dv), (long) rows * cols);
 	if (all_mult4({cols, ldg1, ldg2, lddu, lddv}) && all_aligned({g1_dz_re, g1_dz_im, g2_dz_re, g2_dz_im, du_dz_re, du_dz_im, du_dzs_re,
 			du_dzs_im, dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im}))
 		CNET_LAUNCH_V4(residual_bwd_sym2_kernel, nt, CNET_GRID_2D(4), g1_dz_re, g1_dz_im, ldg1, g2_dz_re, g2_dz_im, ldg2, du, lddu, dv, lddv,
 				rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL((residual_bwd_sym2_kernel<1, false>), CNET_GRID_2D(1), g1_dz_re, g1_dz_im, ldg1, g2_dz_re, g2_dz_im, ldg2, du, lddu,
+		hipLaunchKernelGGL((residual_bwd_sym2_kernel<1, 0>), CNET_GRID_2D(1), g1_dz_re, g1_dz_im, ldg1, g2_dz_re, g2_dz_im, ldg2, du, lddu,
 				dv, lddv, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
 
 // the launch macro for kernels with a third template flag
-#define CNET_LAUNCH_V4G(kernel, nt, gelu, ...)                                   \
-	do {                                                                         \
-		if (nt) {                                                                \
-			if (gelu) hipLaunchKernelGGL((kernel<4, true, true>), __VA_ARGS__);   \
-			else hipLaunchKernelGGL((kernel<4, true, false>), __VA_ARGS__);      \
-		} else {                                                                 \
-			if (gelu) hipLaunchKernelGGL((kernel<4, false, true>), __VA_ARGS__);  \
-			else hipLaunchKernelGGL((kernel<4, false, false>), __VA_ARGS__);     \
-		}                                                                        \
+#define CNET_LAUNCH_V4G_P(kernel, P, gelu, ...)                              \
+	do {                                                                     \
+		if (gelu) hipLaunchKernelGGL((kernel<4, P, true>), __VA_ARGS__);      \
+		else hipLaunchKernelGGL((kernel<4, P, false>), __VA_ARGS__);         \
+	} while (0)
+#define CNET_LAUNCH_V4G(kernel, pol, gelu, ...)                              \
+	do {                                                                     \
+		switch (pol) {                                                       \
+		case 1: CNET_LAUNCH_V4G_P(kernel, 1, gelu, __VA_ARGS__); break;      \
+		case 2: CNET_LAUNCH_V4G_P(kernel, 2, gelu, __VA_ARGS__); break;      \
+		case 3: CNET_LAUNCH_V4G_P(kernel, 3, gelu, __VA_ARGS__); break;      \
+		default: CNET_LAUNCH_V4G_P(kernel, 0, gelu, __VA_ARGS__); break;     \
+		}                                                                    \
 	} while (0)
 #define CNET_LAUNCH_V1G(kernel, gelu, ...)                                   \
 	do {                                                                     \
-		if (gelu) hipLaunchKernelGGL((kernel<1, false, true>), __VA_ARGS__);  \
-		else hipLaunchKernelGGL((kernel<1, false, false>), __VA_ARGS__);     \
+		if (gelu) hipLaunchKernelGGL((kernel<1, 0, true>), __VA_ARGS__);  \
+		else hipLaunchKernelGGL((kernel<1, 0, false>), __VA_ARGS__);     \
 	} while (0)
 
 int cnet_residual_cgelu_bwd_sym(const float *g1_dz_re, const float *g1_dz_im, int64_t ldg1, const float *g2_dz_re, const float *g2_dz_im,
@@ -1403,7 +1414,7 @@ int cnet_residual_cgelu_bwd_sym(const float *g1_dz_re, const float *g1_dz_im, in
 	if (with_dv) CNET_CHECK_PAIR(dv);
 	else CNET_CHECK_ARG(!dv_dz_im && !dv_dzs_re && !dv_dzs_im);
 	CNET_CHECK_ARG(ldg1 >= cols && (!two || ldg2 >= cols) && ldh >= cols && lddu >= cols && (!with_dv || lddv >= cols) && lddh >= cols);
-	const bool nt = streaming(4 + (two ? 2 : 0) + pair_planes(du) + (with_dv ? pair_planes(dv) : 0) + pair_planes(dh), (long) rows * cols);
+	const int nt = stream_policy(ST_BOTH, 4 + (two ? 2 : 0) + pair_planes(du) + (with_dv ? pair_planes(dv) : 0) + pair_planes(dh), (long) rows * cols);
 	if (all_mult4({cols, ldg1, two ? ldg2 : 0, ldh, lddu, with_dv ? lddv : 0, lddh}) &&
 			all_aligned({g1_dz_re, g1_dz_im, g2_dz_re, g2_dz_im, h_re, h_im, du_dz_re, du_dz_im, du_dzs_re, du_dzs_im, dv_dz_re, dv_dz_im,
 					dv_dzs_re, dv_dzs_im, dh_dz_re, dh_dz_im, dh_dzs_re, dh_dzs_im}))
@@ -1433,7 +1444,7 @@ static int hadamard_bwd_sym_impl(const char *who, bool gelu, const float *u_re, 
 	const bool vec = all_mult4({cols, ldu, ldv, ldg, lddu, ldv ? lddv : 0, gelu && dh.dz_re ? lddh : 0}) &&
 			all_aligned({u_re, u_im, v_re, v_im, g_dz_re, g_dz_im, du.dz_re, du.dz_im, du.dzs_re, du.dzs_im, dv.dz_re, dv.dz_im, dv.dzs_re,
 					dv.dzs_im, gelu ? dh.dz_re : nullptr, gelu ? dh.dz_im : nullptr, gelu ? dh.dzs_re : nullptr, gelu ? dh.dzs_im : nullptr});
-	const bool nt = streaming(4 + pair_planes(du) + (ldv ? 2 + pair_planes(dv) : 0) + (gelu && dh.dz_re ? pair_planes(dh) : 0), (long) rows * cols);
+	const int nt = stream_policy(ST_LOADS, 4 + pair_planes(du) + (ldv ? 2 + pair_planes(dv) : 0) + (gelu && dh.dz_re ? pair_planes(dh) : 0), (long) rows * cols);
 	if (ldv != 0) {
 		if (vec)
 			CNET_LAUNCH_V4G(hadamard_bwd_sym_kernel, nt, gelu, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg, dh, lddh,
@@ -1490,12 +1501,12 @@ int cnet_hadamard_cgelu_fwd(const float *u_re, const float *u_im, int64_t ldu, c
 	if (!rows || !cols) return CNET_OK;
 	CNET_CHECK_ARG(u_re && u_im && v_re && v_im && h_re && h_im && y_re && y_im);
 	CNET_CHECK_ARG(ldu >= cols && ldh >= cols && ldy >= cols && (ldv == 0 || ldv >= cols));
-	const bool nt = streaming(6, (long) rows * cols);
+	const int nt = stream_policy(ST_STORES, 6 + (ldv ? 2 : 0), (long) rows * cols);
 	if (all_mult4({cols, ldu, ldv, ldh, ldy}) && all_aligned({u_re, u_im, v_re, v_im, h_re, h_im, y_re, y_im}))
 		CNET_LAUNCH_V4(hadamard_gelu_fwd_kernel, nt, CNET_GRID_2D(4), u_re, u_im, ldu, v_re, v_im, ldv, h_re, h_im, ldh, y_re, y_im, ldy, rows,
 				cols);
 	else
-		hipLaunchKernelGGL((hadamard_gelu_fwd_kernel<1, false>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, h_re, h_im, ldh, y_re, y_im,
+		hipLaunchKernelGGL((hadamard_gelu_fwd_kernel<1, 0>), CNET_GRID_2D(1), u_re, u_im, ldu, v_re, v_im, ldv, h_re, h_im, ldh, y_re, y_im,
 				ldy, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
@@ -1509,11 +1520,11 @@ int cnet_l2out_bwd_sym(const float *z_re, const float *z_im, int64_t ldz, float 
 	const Pair2 dz = pair_of(dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im);
 	CNET_CHECK_ARG(z_re && z_im && ldz >= cols && lddz >= cols);
 	CNET_CHECK_PAIR(dz);
-	const bool nt = streaming(2 + pair_planes(dz), (long) rows * cols);
+	const int nt = stream_policy(ST_LOADS, 2 + pair_planes(dz), (long) rows * cols);
 	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
 		CNET_LAUNCH_V4(l2out_bwd_sym_kernel, nt, CNET_GRID_2D(4), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
 	else
-		hipLaunchKernelGGL((l2out_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
+		hipLaunchKernelGGL((l2out_bwd_sym_kernel<1, 0>), CNET_GRID_2D(1), z_re, z_im, ldz, dz, lddz, rows, cols, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1526,11 +1537,11 @@ int cnet_cross_entropy_bwd_sym(const float *z_re, const float *z_im, int64_t ldz
 	const Pair2 dz = pair_of(dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im);
 	CNET_CHECK_ARG(z_re && z_im && s && labels && ldz >= cols && lddz >= cols);
 	CNET_CHECK_PAIR(dz);
-	const bool nt = streaming(2 + pair_planes(dz), (long) rows * cols);
+	const int nt = stream_policy(ST_BOTH, 2 + pair_planes(dz), (long) rows * cols);
 	if (all_mult4({cols, ldz, lddz}) && all_aligned({z_re, z_im, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im}))
 		CNET_LAUNCH_V4(crossent_bwd_sym_kernel, nt, CNET_GRID_2D(4), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
 	else
-		hipLaunchKernelGGL((crossent_bwd_sym_kernel<1, false>), CNET_GRID_2D(1), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
+		hipLaunchKernelGGL((crossent_bwd_sym_kernel<1, 0>), CNET_GRID_2D(1), z_re, z_im, ldz, s, labels, dz, lddz, rows, cols);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }

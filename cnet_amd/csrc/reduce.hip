@@ -485,9 +485,30 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_kernel(const float *__restrict
 // Register-resident variants for rows of at most 64 * G * 4 * NIT columns (128-bit path): the row is read from memory
 // once, held in registers across the reduction and written back normalised, so the traffic is the algorithmic one
 // (the two-pass kernels above read every operand twice).  Same per-thread summation order as the two-pass kernels.
+// 128-bit accesses under a cache policy chosen at launch (cnet::stream_policy; uniform over the launch)
+__device__ __forceinline__ float4 ld4(const float *p, int policy) {
+	typedef float f32x4 __attribute__((ext_vector_type(4)));
+	if (policy == cnet::ST_BOTH || policy == cnet::ST_LOADS) {
+		const f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+		return make_float4(t.x, t.y, t.z, t.w);
+	}
+	return *reinterpret_cast<const float4 *>(p);
+}
+__device__ __forceinline__ void st4(float *p, float4 v, int policy) {
+	typedef float f32x4 __attribute__((ext_vector_type(4)));
+	const f32x4 t = {v.x, v.y, v.z, v.w};
+	// (written out: see stv in elementwise.hip)
+	if (policy == cnet::ST_BOTH || policy == cnet::ST_STORES)
+		asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(p), "v"(t) : "memory");
+	else if (policy == cnet::ST_LOADS)
+		asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(t) : "memory");
+	else
+		*reinterpret_cast<float4 *>(p) = v;
+}
+
 template <int G, int NIT>
 __global__ __launch_bounds__(TPB) void l2norm_fwd_reg_kernel(const float *__restrict__ zr, const float *__restrict__ zi, long ldz,
-		float *__restrict__ yr, float *__restrict__ yi, long ldy, float *__restrict__ s, int rows, int cols) {
+		float *__restrict__ yr, float *__restrict__ yi, long ldy, float *__restrict__ s, int rows, int cols, int policy) {
 	__shared__ double lds_d[TPB / 64];
 	CNET_ROW_SETUP();
 	const float *pr = zr + (long) row * ldz, *pi = zi + (long) row * ldz;
@@ -497,8 +518,8 @@ __global__ __launch_bounds__(TPB) void l2norm_fwd_reg_kernel(const float *__rest
 		const int c = (t + k * STRIDE) * 4;
 		a[k] = b[k] = make_float4(0.f, 0.f, 0.f, 0.f);
 		if (c < cols) {
-			a[k] = *reinterpret_cast<const float4 *>(pr + c);
-			b[k] = *reinterpret_cast<const float4 *>(pi + c);
+			a[k] = ld4(pr + c, policy);
+			b[k] = ld4(pi + c, policy);
 		}
 	}
 	double sum = 0.0;
@@ -523,10 +544,8 @@ __global__ __launch_bounds__(TPB) void l2norm_fwd_reg_kernel(const float *__rest
 	for (int k = 0; k < NIT; ++k) {
 		const int c = (t + k * STRIDE) * 4;
 		if (c < cols) {
-			*reinterpret_cast<float4 *>(qr + c) =
-					make_float4((float) (a[k].x * inv), (float) (a[k].y * inv), (float) (a[k].z * inv), (float) (a[k].w * inv));
-			*reinterpret_cast<float4 *>(qi + c) =
-					make_float4((float) (b[k].x * inv), (float) (b[k].y * inv), (float) (b[k].z * inv), (float) (b[k].w * inv));
+			st4(qr + c, make_float4((float) (a[k].x * inv), (float) (a[k].y * inv), (float) (a[k].z * inv), (float) (a[k].w * inv)), policy);
+			st4(qi + c, make_float4((float) (b[k].x * inv), (float) (b[k].y * inv), (float) (b[k].z * inv), (float) (b[k].w * inv)), policy);
 		}
 	}
 	if (t == 0 && s) s[row] = (float) sum;
@@ -537,7 +556,7 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_reg_kernel(const float *__rest
 		const float *__restrict__ s, const float *__restrict__ g_re, const float *__restrict__ g_im,
 		const float *__restrict__ gs_re, const float *__restrict__ gs_im, long ldg, float *__restrict__ d_re,
 		float *__restrict__ d_im, float *__restrict__ ds_re, float *__restrict__ ds_im, long ldd, int rows, int cols,
-		int accumulate) {
+		int accumulate, int policy) {
 	__shared__ Cplx4 lds_c[TPB / 64];
 	CNET_ROW_SETUP();
 	const float *src[6] = {zr + (long) row * ldz, zi + (long) row * ldz, g_re + (long) row * ldg, g_im + (long) row * ldg,
@@ -553,7 +572,7 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_reg_kernel(const float *__rest
 #pragma unroll
 		for (int p = 0; p < NSRC; ++p) {
 			float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-			if (c < cols) x = *reinterpret_cast<const float4 *>(src[p] + c);
+			if (c < cols) x = ld4(src[p] + c, policy);
 			v[k][p][0] = x.x;
 			v[k][p][1] = x.y;
 			v[k][p][2] = x.z;
@@ -613,7 +632,7 @@ __global__ __launch_bounds__(TPB) void l2norm_bwd_reg_kernel(const float *__rest
 					w.z += old.z;
 					w.w += old.w;
 				}
-				*reinterpret_cast<float4 *>(dst[p] + c) = w;
+				st4(dst[p] + c, w, policy);
 			}
 		}
 	}
@@ -781,14 +800,16 @@ static int l2norm_bwd_dispatch(const float *z_re, const float *z_im, int64_t ldz
 	const bool wide = cols > 2048;
 	const int rpb = wide ? 1 : TPB / 64;
 	dim3 grid((unsigned) ((rows + rpb - 1) / rpb));
+	// z, g (both halves unless the pair is conjugate) and the planes of the result
+	const int policy = stream_policy(SYM ? ST_LOADS : ST_BOTH, (SYM ? 4 : 6) + (SYM && !dz_dzs_re ? 2 : 4), (long) rows * cols);
 #define CNET_L2N_ARGS z_re, z_im, (long) ldz, s, g_dz_re, g_dz_im, g_dzs_re, g_dzs_im, (long) ldg, dz_dz_re, dz_dz_im, dz_dzs_re, dz_dzs_im, (long) lddz, rows, cols, accumulate
 	if (vec && nit <= 4) {
 		if (nit <= 2) {
-			if (wide) hipLaunchKernelGGL((l2norm_bwd_reg_kernel<4, 2, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
-			else hipLaunchKernelGGL((l2norm_bwd_reg_kernel<1, 2, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+			if (wide) hipLaunchKernelGGL((l2norm_bwd_reg_kernel<4, 2, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS, policy);
+			else hipLaunchKernelGGL((l2norm_bwd_reg_kernel<1, 2, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS, policy);
 		} else {
-			if (wide) hipLaunchKernelGGL((l2norm_bwd_reg_kernel<4, 4, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
-			else hipLaunchKernelGGL((l2norm_bwd_reg_kernel<1, 4, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
+			if (wide) hipLaunchKernelGGL((l2norm_bwd_reg_kernel<4, 4, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS, policy);
+			else hipLaunchKernelGGL((l2norm_bwd_reg_kernel<1, 4, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS, policy);
 		}
 	} else if (vec) {
 		if (wide) hipLaunchKernelGGL((l2norm_bwd_kernel<4, 4, SYM>), grid, dim3(TPB), 0, rt().stream, CNET_L2N_ARGS);
@@ -855,9 +876,10 @@ int cnet_l2norm_fwd(const float *z_re, const float *z_im, int64_t ldz, float *y_
 	const bool vec = mult4(cols, ldz, ldy) && aligned16(z_re) && aligned16(z_im) && aligned16(y_re) && aligned16(y_im);
 	const int nit = chunks_per_thread(cols);
 	if (vec && nit <= 8) {
-		if (nit <= 2) CNET_ROW_LAUNCH_REG(l2norm_fwd_reg_kernel, 2, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols);
-		else if (nit <= 4) CNET_ROW_LAUNCH_REG(l2norm_fwd_reg_kernel, 4, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols);
-		else CNET_ROW_LAUNCH_REG(l2norm_fwd_reg_kernel, 8, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols);
+		const int policy = stream_policy(ST_STORES, 4, (long) rows * cols);
+		if (nit <= 2) CNET_ROW_LAUNCH_REG(l2norm_fwd_reg_kernel, 2, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols, policy);
+		else if (nit <= 4) CNET_ROW_LAUNCH_REG(l2norm_fwd_reg_kernel, 4, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols, policy);
+		else CNET_ROW_LAUNCH_REG(l2norm_fwd_reg_kernel, 8, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols, policy);
 		return CNET_OK;
 	}
 	CNET_ROW_LAUNCH(l2norm_fwd_kernel, vec, z_re, z_im, (long) ldz, y_re, y_im, (long) ldy, s, rows, cols);
