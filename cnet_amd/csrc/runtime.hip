@@ -234,6 +234,21 @@ int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes) {
 	return CNET_OK;
 }
 
+// page-locked ranges handed out by cnet_host_alloc: only these may be read by a kernel directly (cnet_upload_pair); a
+// pointer into pageable memory there would be a memory fault on the device instead of an error code
+static std::map<uintptr_t, size_t> &pinned_ranges() {
+	static std::map<uintptr_t, size_t> ranges;
+	return ranges;
+}
+static bool in_pinned_range(const void *p, size_t bytes) {
+	if (!bytes) return true;
+	auto &ranges = pinned_ranges();
+	auto it = ranges.upper_bound((uintptr_t) p);
+	if (it == ranges.begin()) return false;
+	--it;
+	return (uintptr_t) p + bytes <= it->first + it->second;
+}
+
 int cnet_host_alloc(size_t bytes, void **out) {
 	CNET_REQUIRE_INIT();
 	CNET_NOT_IN_CAPTURE();
@@ -241,6 +256,7 @@ int cnet_host_alloc(size_t bytes, void **out) {
 	*out = nullptr;
 	if (bytes == 0) return CNET_OK;
 	CNET_HIP(hipHostMalloc(out, bytes, hipHostMallocDefault));
+	pinned_ranges()[(uintptr_t) *out] = bytes;
 	return CNET_OK;
 }
 
@@ -251,6 +267,7 @@ int cnet_host_free(void *ptr) {
 	// copies queued from this buffer must have left it
 	CNET_HIP(hipStreamSynchronize(rt().stream));
 	CNET_HIP(hipStreamSynchronize(rt().upload_stream));
+	pinned_ranges().erase((uintptr_t) ptr);
 	CNET_HIP(hipHostFree(ptr));
 	return CNET_OK;
 }
@@ -299,7 +316,7 @@ int cnet_upload_pair(void *dst0, const void *pinned_src0, size_t bytes0, void *d
 	// Small batches: a copy queued through the runtime costs the host 3-5 us each and takes the copy engine's start-up time
 	// to arrive; one kernel launch that reads the page-locked memory directly does both regions.  Large ones stay with the
 	// copy engine, which moves them without occupying compute units.
-	if (bytes0 + bytes1 <= (1u << 20)) {
+	if (bytes0 + bytes1 <= (1u << 20) && in_pinned_range(pinned_src0, bytes0) && in_pinned_range(pinned_src1, bytes1)) {
 		const long words0 = (long) (bytes0 / 4), words1 = (long) (bytes1 / 4);
 		const long vec0 = aligned16(dst0) && aligned16(pinned_src0) ? words0 / 4 : 0;
 		const long threads = std::max(vec0 + (words0 - 4 * vec0), words1);

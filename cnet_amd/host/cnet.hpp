@@ -2284,7 +2284,7 @@ public:
 		return p;
 	}
 	float getLoss(const PendingLoss &p, Batch *batch) {
-		if (p.serial < 0 || (!p.direct && !loss_ring_)) throw std::logic_error("getLoss: nothing was queued under this handle");
+		if (p.serial < 0 || (p.direct ? !p.direct->host : !loss_ring_)) throw std::logic_error("getLoss: nothing was queued under this handle");
 		if ((p.direct ? p.direct->serial - p.serial + 1 : loss_queued_ - p.serial) > kLossSlots)
 			throw std::logic_error("getLoss: the queued losses were overwritten by later ones");
 		ck(cnet_copy_wait(p.ticket), "cnet_copy_wait");

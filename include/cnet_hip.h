@@ -94,7 +94,8 @@ int cnet_upload_async(void *dst, const void *pinned_src, size_t bytes);
 int cnet_upload_zero(void *dst, size_t bytes);
 /* two regions (a batch and its labels) from page-locked memory to the device on the upload stream, sizes in bytes, multiples
  * of 4; up to 1 MiB in all they travel in ONE kernel launch whose lanes read the host memory over the link (half the
- * host time of two queued copies and none of the copy engine's start-up time), beyond that as two cnet_upload_async */
+ * host time of two queued copies and none of the copy engine's start-up time), beyond that, or when a source does not lie
+ * in memory from cnet_host_alloc, as two cnet_upload_async */
 int cnet_upload_pair(void *dst0, const void *pinned_src0, size_t bytes0, void *dst1, const void *pinned_src1, size_t bytes1);
 int cnet_upload_wait_compute(void);
 int cnet_mark_compute(int marker);

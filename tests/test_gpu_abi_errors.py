@@ -366,6 +366,12 @@ def test_device_copy_caller_stream_and_upload_ordering(gpu, port):
         assert np.array_equal(c.download(), want), (words0, words1, off)
         got1 = b.download()
         assert np.array_equal(got1[:words1], np.arange(n - 1024, n - 1024 + words1)) and (got1[words1:] == 0).all()
+    # a source that does not come from cnet_host_alloc (pageable memory) is not handed to a kernel: it goes through the runtime's copy
+    pageable = np.arange(1000, 1512, dtype=np.float32)
+    capi.call("cnet_upload_wait_compute")
+    capi.call("cnet_upload_pair", a.ptr, pageable.ctypes.data, pageable.nbytes, b.ptr, host.value, 16)
+    capi.call("cnet_upload_sync")
+    assert np.array_equal(a.download()[:512], pageable) and np.array_equal(b.download()[:4], pinned[:4])
     assert _status("cnet_upload_pair", a.ptr, host, 6, b.ptr, host, 4) == INVALID        # not whole words
     assert _status("cnet_upload_pair", None, host, 8, b.ptr, host, 4) == INVALID
     assert _status("cnet_upload_pair", None, None, 0, None, None, 0) == 0
