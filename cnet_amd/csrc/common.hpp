@@ -149,7 +149,11 @@ inline int stream_policy(int when_streaming, int planes, long elems) {
 		const char *e = getenv("CNET_STREAM_POLICY");  // tuning override: 0..3 for every launch beyond the cache size
 		return e ? atoi(e) : -1;
 	}();
-	if ((long) planes * elems * 4 <= (256L << 20)) return 0;
+	static const long cache_bytes = [] {
+		const char *e = getenv("CNET_STREAM_MIN_MB");  // tuning override of the footprint from which a launch counts as streaming
+		return (e ? atol(e) : 256L) << 20;
+	}();
+	if ((long) planes * elems * 4 <= cache_bytes) return 0;
 	return forced >= 0 && forced <= 3 ? forced : when_streaming;
 }
 
