@@ -297,14 +297,16 @@ def train_lines(steps):
     time per step of each input mode.  None when the driver is not built or fails."""
     out = []
     for batch in (64, 1024, 4096):
+        # the same number of samples at every batch size (a loop of 300 steps at batch 64 lasts 17 ms: too short to time)
+        n = min(3000, steps * (4096 // batch))
         # "frozen_input" adds the mode in which the data input is marked not trainable (no step on it, no backward pass
         # into it; off by default in the facade, as upstream steps every input function)
-        line = _train_bench("readme", batch, steps, "frozen_input")
+        line = _train_bench("readme", batch, n, "frozen_input")
         if line is None:
             return None
         # configs[0] states real samples (imaginary parts 0), whose imaginary plane is cleared on the device instead of
         # sent; beside it the same loop on samples with uniform imaginary parts, both planes travelling
-        both = _train_bench("readme", batch, steps, "complex_samples")
+        both = _train_bench("readme", batch, n, "complex_samples")
         if both is not None:
             line["samples_per_sec_complex_samples"] = both["samples_per_sec_prefetch_loss_read_one_step_late"]
             line["upload_bytes_per_step_complex_samples"] = both["upload_bytes_per_step"]
