@@ -236,11 +236,14 @@ def kernel_suite(steps):
     return lines
 
 
-def token_model_suite(steps):
-    """Fifth configuration at full size: batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096; forward + backward."""
+def token_model_suite(steps, products=4):
+    """Fifth configuration at full size: batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096; forward + backward.
+    products = 3: the block kernels form a complex product from three real ones (cnet_cgemm_set_products), conjugate
+    gradient pairs only."""
     from cnet_amd import capi
     from cnet_amd.workloads import TokenModel
     capi.init(0)
+    capi.call("cnet_cgemm_set_products", products)
     rng = np.random.default_rng(0)
     Bq, S, D, H, V = 16, 512, 1024, 4096, 32768
 
@@ -254,7 +257,7 @@ def token_model_suite(steps):
     out = []
     # first with every product computed (what upstream's backward pass does), then with the dz* halves of the gradient
     # pairs written as conjugates of the dz products (the loss is real); one model at a time on the device
-    for conjugate_pairs in (False, True):
+    for conjugate_pairs in ((False, True) if products == 4 else (True,)):
         model = TokenModel(Bq, S, D, H, V, P, conjugate_pairs=conjugate_pairs).set_tokens(ids)
         for _ in range(2):
             model.forward(); model.backward()
@@ -269,21 +272,25 @@ def token_model_suite(steps):
         out.append({"workload": "configs[4]: complex token model fwd+bwd, batch 16 x seq 512, vocab 32768, dim 1024, hidden 4096",
                     "gradient_pairs": "dz* written as conj(dz)" if conjugate_pairs else "both halves computed",
                     "ms_per_step": round(ms, 3), "tokens_per_sec": round(Bq * S / ms * 1e3, 1),
+                    "real_products_per_complex_product": products,
+                    # complex products executed, each counted as 8 M N K
                     "gemm_tflops_executed": round(model.gemm_flops() / ms / 1e9, 2), "mean_loss": round(loss, 4),
                     "loss_of_uniform_guess": round(float(np.log(V)), 4)})
         del model
+    capi.call("cnet_cgemm_set_products", 4)
     return out
 
 
 TRAIN_BENCH = os.path.join(ROOT, "cnet_amd", "bin", "train_bench")
 
 
-def _train_bench(*args):
+def _train_bench(*args, env=None):
     """One run of the C++ timing driver (cnet_amd/host/train_bench.cpp) in a process of its own; its JSON line or None."""
     import subprocess
     if not os.path.exists(TRAIN_BENCH):
         return None
-    r = subprocess.run([TRAIN_BENCH] + [str(a) for a in args], capture_output=True, text=True, timeout=600)
+    r = subprocess.run([TRAIN_BENCH] + [str(a) for a in args], capture_output=True, text=True, timeout=600,
+                       env=dict(os.environ, **env) if env else None)
     lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
     if r.returncode != 0 or not lines:
         sys.stderr.write("bench.py: train_bench %s failed:\n" % " ".join(map(str, args)) + r.stdout[-2000:] + r.stderr[-2000:])
@@ -317,15 +324,17 @@ def train_lines(steps):
 STACK_LR = 3e-6   # configs[3] names 0.01, at which fp32 overflows in the first update on the CPU path as well; 1e-5 still diverges
 
 
-def stack_lines(steps=10):
+def stack_lines(steps=10, products=4):
     """configs[3]: 8 x (Linear 2048 -> 2048, CGelu, Residual), L2Out, batch 2048, `steps` SGD steps through the C++ facade,
     both data inputs uploaded and the loss read back every step; first with the dz* halves of the gradient pairs written
-    as conjugates (the facade's default), then with both halves computed as upstream does."""
+    as conjugates (the facade's default), then with both halves computed as upstream does.  products = 3: the first of the
+    two only, with the block kernels forming a complex product from three real ones (CNET_CGEMM_3M=1)."""
     out = []
-    for mode in ((), ("both_halves",)):
-        line = _train_bench("stack", 2048, 8, 2048, steps, STACK_LR, *mode)
+    for mode in ((), ("both_halves",)) if products == 4 else ((),):
+        line = _train_bench("stack", 2048, 8, 2048, steps, STACK_LR, *mode, env={"CNET_CGEMM_3M": "1" if products == 3 else "0"})
         if line is None:
             return None
+        line["real_products_per_complex_product"] = products
         out.append(line)
     return out
 
@@ -497,6 +506,41 @@ def main():
 
         return conjugate_pair
 
+    def three_products_step():
+        # Beside the headline (four real matrix products per complex one, as the metric's 8 M N K counts them): the same five
+        # products with the block kernels forming each from three real ones (cnet_cgemm_set_products(3): 6 M N K executed).
+        capi.call("cnet_cgemm_set_products", 3)
+        for _ in range(args.warmup):
+            step()
+        capi.sync()
+        a, b = ev.event(), ev.event()
+        ev.record(a)
+        for _ in range(args.steps):
+            step()
+        ev.record(b)
+        ms3 = ev.elapsed_ms(a, b) / args.steps
+        per = {}
+        for name, (fn, ngemm) in launches.items():
+            groups = []
+            for _ in range(3):
+                a, b = ev.event(), ev.event()
+                ev.record(a)
+                for _ in range(args.steps):
+                    fn()
+                ev.record(b)
+                groups.append(ev.elapsed_ms(a, b) / args.steps)
+            ms = sorted(groups)[1]
+            per[name] = {"ms": round(ms, 4), "tflops_counted_as_8mnk": round(8.0 * B * N * K * ngemm / ms / 1e9, 2),
+                         "tflops_executed": round(6.0 * B * N * K * ngemm / ms / 1e9, 2)}
+        res = {"option": "cnet_cgemm_set_products(3) / CNET_CGEMM_3M=1; not the default",
+               "ms_per_step": round(ms3, 4), "tflops_counted_as_8mnk": round(flops_step / ms3 / 1e9, 2),
+               "tflops_executed": round(0.75 * flops_step / ms3 / 1e9, 2),
+               "frac_of_fp32_mfma_peak_executed": round(0.75 * flops_step / ms3 / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),
+               "samples_per_sec": round(B / ms3 * 1e3, 1), "all_launches": per,
+               "conjugate_gradient_pair": conjugate_pair_step()}
+        capi.call("cnet_cgemm_set_products", 4)
+        return res
+
     out = {
         "metric": "complex-Linear fwd+bwd TFLOP/s (% fp32 MFMA peak); train samples/sec",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -512,6 +556,7 @@ def main():
     }
     if not args.no_cpu_baseline:   # the flag leaves the headline alone (profiled runs)
         out["conjugate_gradient_pair"] = conjugate_pair_step()
+        three = three_products_step()
         out["cpu_baseline"] = cpu_baseline()
         train = train_lines(300)
         if train:   # the other half of the metric: training steps of the configs[0] net through the C++ facade
@@ -532,6 +577,11 @@ def main():
             out["configs3_residual_stack"] = stack
         out["kernels"] = kernel_suite(20)
         out["configs4_token_model"] = token_model_suite(3)
+        stack3 = stack_lines(10, products=3)
+        if stack3:
+            three["configs3_residual_stack"] = stack3[0]
+        three["configs4_token_model"] = token_model_suite(3, products=3)[0]
+        out["three_real_products_per_complex_product"] = three
     print(json.dumps(out))
 
 

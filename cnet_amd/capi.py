@@ -63,6 +63,8 @@ SIGNATURES = {
     "cnet_cdft_plan": [_i],
     "cnet_cdft_twiddle": [_i, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)],
     "cnet_cdft_set_forward_matrix": [_i, C.c_void_p, C.c_void_p],
+    "cnet_cgemm_set_products": [_i],
+    "cnet_cgemm_get_products": [],
     "cnet_cdft_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i, _i],
     "cnet_cdft_fwd_real_input": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i],
     "cnet_cdft_bwd": [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],

@@ -529,7 +529,11 @@ struct DlStage {
 // shorter than a memory round trip, use three; 128 x 128 has room for two).
 // waves_per_eu(2, 4): LDS allows at most four workgroups per compute unit anyway, so the register allocator need not
 // squeeze the small blocks for an occupancy that cannot materialise.
-template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int NST>
+// GAUSS: three real products per complex one instead of four (P = Ar Br, Q = Ai Bi, T = (Ar + sa Ai)(Br + sb Bi) with
+// sa, sb the signs of the imaginary parts: re = P - sa sb Q, im = T - P - sa sb Q).  A quarter of the matrix work less,
+// for one addition per operand fragment and k pair; the imaginary part then carries the rounding of all three products
+// (normwise as accurate as four products, not componentwise).
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int NST, bool GAUSS = false>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))) void cgemm_fast_kernel(const CgemmArgs args) {
 	static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per workgroup");
 	constexpr int TM = WM / 32, TN = WN / 32;
@@ -568,7 +572,8 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	// all; with four tiles there are only registers for two sets, re = P -+ Q and im = +-R +- S, and one operand of the
 	// second product is negated per k pair (see the modes below).
 	constexpr bool ACC4 = TM * TN <= 2;
-	floatx16 acc_re[TM][TN], acc_im[TM][TN], acc_q[ACC4 ? TM : 1][ACC4 ? TN : 1], acc_s[ACC4 ? TM : 1][ACC4 ? TN : 1];
+	constexpr bool ACC_Q = ACC4 || GAUSS, ACC_S = ACC4 && !GAUSS;
+	floatx16 acc_re[TM][TN], acc_im[TM][TN], acc_q[ACC_Q ? TM : 1][ACC_Q ? TN : 1], acc_s[ACC_S ? TM : 1][ACC_S ? TN : 1];
 	for (int pass = 0; pass < npass; ++pass) {
 	int prob = blockIdx.y, tile_m = tile_m_first, tile_n = pass ? args.tiles_n - 1 - tile_n_first : tile_n_first;
 	int piece = -1, tail_block = 0;  // piece >= 0: this pass computes one K piece of a tail block
@@ -597,10 +602,8 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			for (int e = 0; e < 16; ++e) {
 				acc_re[i][j][e] = 0.f;
 				acc_im[i][j][e] = 0.f;
-				if (ACC4) {
-					acc_q[i][j][e] = 0.f;
-					acc_s[i][j][e] = 0.f;
-				}
+				if (ACC_Q) acc_q[i][j][e] = 0.f;
+				if (ACC_S) acc_s[i][j][e] = 0.f;
 			}
 
 	StageA sa;
@@ -646,6 +649,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	//   mode 2 (conj A):   re += Ar Br + Ai Bi      im += Ar Bi + (-Ai) Br
 	//   mode 3 (both):     re += Ar Br + (-Ai) Bi   im += Ar Bi + Ai Br, negated when it is stored
 	const int mode = (pb.a_im_sign < 0.f ? 2 : 0) | (pb.b_im_sign < 0.f ? 1 : 0);
+	const float sign_a = pb.a_im_sign < 0.f ? -1.f : 1.f, sign_b = pb.b_im_sign < 0.f ? -1.f : 1.f;  // uniform: scalar registers
 
 	constexpr int LOADS_PER_CHUNK = 2 * (UA + UB);  // transfers one wavefront issues per chunk
 	static_assert(NST == 2 || NST == 3, "two or three stages");
@@ -700,14 +704,28 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			for (int i = 0; i < TM; ++i) {
 				are[i] = fa.re(ks, i);
 				aim[i] = fa.im(ks, i);
-				if (!ACC4) neg[i] = MODE == 1 ? -are[i] : -aim[i];
+				if (!ACC4 && !GAUSS) neg[i] = MODE == 1 ? -are[i] : -aim[i];
 			}
 #pragma unroll
 			for (int j = 0; j < TN; ++j) {
 				bre[j] = fb.re(ks, j);
 				bim[j] = fb.im(ks, j);
 			}
-			if constexpr (ACC4) {
+			if constexpr (GAUSS) {
+				float asum[TM], bsum[TN];
+#pragma unroll
+				for (int i = 0; i < TM; ++i) asum[i] = fmaf(sign_a, aim[i], are[i]);
+#pragma unroll
+				for (int j = 0; j < TN; ++j) bsum[j] = fmaf(sign_b, bim[j], bre[j]);
+#pragma unroll
+				for (int i = 0; i < TM; ++i)
+#pragma unroll
+					for (int j = 0; j < TN; ++j) {
+						acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bre[j], acc_re[i][j], 0, 0, 0);    // P
+						acc_q[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aim[i], bim[j], acc_q[i][j], 0, 0, 0);      // Q
+						acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(asum[i], bsum[j], acc_im[i][j], 0, 0, 0);  // T
+					}
+			} else if constexpr (ACC4) {
 #pragma unroll
 				for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -742,7 +760,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				// scheduling recipe for this k pair: after each MFMA let a few of the pending VALU / LDS / global
 				// instructions issue, so they run in the shadow of the matrix pipe
 #pragma unroll
-				for (int q = 0; q < 4 * TM * TN; ++q) {
+				for (int q = 0; q < (GAUSS ? 3 : 4) * TM * TN; ++q) {
 					__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
 					__builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // <= 2 VALU
 					__builtin_amdgcn_sched_group_barrier(0x080, 1, 0);  // <= 1 LDS
@@ -773,7 +791,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			if (c + 1 < c_hi) chunk(1, mode_c, c + 1);
 		}
 	};
-	if constexpr (ACC4) {
+	if constexpr (ACC4 || GAUSS) {
 		kloop(std::integral_constant<int, 0>());  // the signs wait for the store
 	} else {
 		switch (mode) {
@@ -802,7 +820,11 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				if (row < args.M) {
 					const long off = (long) (row - row_org) * ldc + (col - col_org);
 					float vr, vi;
-					if constexpr (ACC4) {
+					if constexpr (GAUSS) {
+						const float p = acc_re[i][j][e], q = q_minus ? acc_q[i][j][e] : -acc_q[i][j][e];  // q_minus: sa sb = +1
+						vr = p - q;
+						vi = (acc_im[i][j][e] - p) - q;
+					} else if constexpr (ACC4) {
 						const float q = acc_q[i][j][e], rr = acc_im[i][j][e], ss = acc_s[i][j][e];
 						vr = q_minus ? acc_re[i][j][e] - q : acc_re[i][j][e] + q;
 						vi = (r_minus ? -rr : rr) + (s_minus ? -ss : ss);
@@ -1217,6 +1239,17 @@ bool try_skinny_two(bool a_mcontig0, bool b_ncontig0, const CgemmArgs &proto0, b
 }
 
 // tail_splits >= 2: cut the blocks of the last, partly filled round into that many pieces along K (see CgemmArgs)
+// Whether the block kernels of one or two tiles per wavefront form a complex product from three real ones
+// (cgemm_fast_kernel<.., GAUSS>); the cost model then prices those shapes at three quarters of their matrix work.
+int g_three_products = -1;
+inline bool three_products() {
+	if (g_three_products < 0) {
+		const char *e = getenv("CNET_CGEMM_3M");
+		g_three_products = e ? (atoi(e) != 0) : 0;
+	}
+	return g_three_products != 0;
+}
+
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
 int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, int k_cuts = -1) {
 	CgemmArgs args = proto;
@@ -1289,6 +1322,22 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 		if (fast_ok) {  // any M and N: edge blocks re-read the last valid rows and store only what is inside C
 			constexpr int NST = (BM == 128 && BN == 128) ? 2 : 3;
 			constexpr size_t fast_smem = (size_t) NST * 2 * KC * (BM + BN) * sizeof(float);
+			// Three accumulator sets of four tiles (192 registers) leave too few for the fragments of two k-contiguous
+			// operands (float4 each): that one layout of the 128 x 128 block spills and keeps four products.
+			if constexpr ((WM / 32) * (WN / 32) <= 2 || A_MCONTIG || B_NCONTIG) {
+				if (three_products()) {
+					static bool gauss_attr_set = false;
+					if (!gauss_attr_set) {
+						CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, true>),
+								hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem));
+						gauss_attr_set = true;
+					}
+					hipLaunchKernelGGL((cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, true>), grid, dim3(NTHREADS), fast_smem,
+							cnet::rt().stream, args);
+					CNET_LAUNCH_CHECK();
+					return finish();
+				}
+			}
 			static bool fast_attr_set = false;
 			if (!fast_attr_set) {
 				CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST>),
@@ -1315,7 +1364,9 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 
 // Block shape for the fast kernel (0: 128 x 128, 1: 64 x 128, 2: 128 x 64, 3: 64 x 64), whether the blocks of a partly
 // filled last round are cut along K (*tail = number of pieces, 0 = no), and the expected duration of the launch in us.
-double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *tail_pieces, int *k_cuts) {
+// k_contig_operands: both operands are stored with k contiguous (the one layout whose 128 x 128 kernel has no
+// three-product form).
+double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_operands, int *shape, int *tail_pieces, int *k_cuts) {
 	const long cus = cnet::rt().prop.multiProcessorCount;
 	auto blocks = [&](int bm, int bn) {
 		long tn = (a.N + bn - 1) / bn;
@@ -1379,7 +1430,9 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 		if (forced >= 0 && forced != k) continue;
 		const long nb = blocks(shapes[k].bm, shapes[k].bn);
 		const long per_unit = (nb + cus - 1) / cus;
-		const double block_us = 8.0 * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
+		// three real products per complex one in the shapes that have the registers for it (fast kernel only: K in whole chunks)
+		const double work = (three_products() && a.K % KC == 0 && !(k == 0 && k_contig_operands)) ? 6.0 : 8.0;
+		const double block_us = work * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
 		// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
 		const double bonus = 1.0 - 0.000001 * shapes[k].bm * shapes[k].bn;
 		double us = per_unit * block_us / eff(k, per_unit, a.K) * bonus;
@@ -1411,7 +1464,7 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int *shape, int *ta
 				if (s < 2 || nchunks / s < 4 || (long) batch * s > 65535) continue;
 				const int k_slice = (int) ((nchunks + s - 1) / s) * KC;
 				const long p = (nb * s + cus - 1) / cus;
-				const double slice_us = 8.0 * shapes[k].bm * shapes[k].bn * k_slice / flop_per_us_per_unit;
+				const double slice_us = work * shapes[k].bm * shapes[k].bn * k_slice / flop_per_us_per_unit;
 				const double pass_us = 6.0 + (s + 1.0 + (a.accumulate ? 1.0 : 0.0)) * 8.0 * a.M * a.N * nprob * batch / 4.0e6;
 				const double cut_us = p * slice_us / eff(k, p, k_slice) * bonus + pass_us;
 				if (cut_us < us) {
@@ -1441,7 +1494,7 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 	} else {
 		int best, best_tail, cuts;
-		plan_blocks(a, nprob, batch, &best, &best_tail, &cuts);
+		plan_blocks(a, nprob, batch, !A_MCONTIG && !B_NCONTIG, &best, &best_tail, &cuts);
 		if (best == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
 		if (best == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
 		if (best == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
@@ -1484,8 +1537,8 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 		}
 		if (plan_skinny(a_mcontig, b_ncontig, right, nprob, batch, planned)) {
 			int shape, tail, cuts;
-			const double whole = plan_blocks(a, nprob, batch, &shape, &tail, &cuts);
-			const double parts = plan_blocks(left, nprob, batch, &shape, &tail, &cuts) + skinny_us(planned, nprob, batch);
+			const double whole = plan_blocks(a, nprob, batch, !a_mcontig && !b_ncontig, &shape, &tail, &cuts);
+			const double parts = plan_blocks(left, nprob, batch, !a_mcontig && !b_ncontig, &shape, &tail, &cuts) + skinny_us(planned, nprob, batch);
 			if (parts < whole) {
 				// one after the other on the compute stream: run side by side on two streams the narrow part's
 				// workgroups took slots from the first round of the block kernel and the pair got slower (842 against
@@ -1642,6 +1695,14 @@ int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M
 	a.stride_c = stride_c;
 	return cgemm_dispatch(a_kmajor != 0, b_kmajor != 0, a, 1, batch);
 }
+
+int cnet_cgemm_set_products(int n) {
+	CNET_CHECK_ARG(n == 3 || n == 4);
+	g_three_products = n == 3;
+	return CNET_OK;
+}
+
+int cnet_cgemm_get_products(void) { return three_products() ? 3 : 4; }
 
 int cnet_clinear_fwd(const float *x_re, const float *x_im, int64_t ldx, const float *w_re, const float *w_im,
 		int64_t ldw, float *y_re, float *y_im, int64_t ldy, int B, int K, int N, int accumulate) {

@@ -176,9 +176,10 @@ int cnet_clinear_bwd_weight(const float *g_dz_re, const float *g_dz_im, const fl
 
 /* The same two backward passes for a gradient pair that is conjugate, g.dzs == conj(g.dz), as the loss layers produce it
  * (CrossEntropy impl/crossent.h, L2Out impl/l2out.h: the loss is real) and every layer's backward pass hands it on: then
- * g.dzs * conj(w) == conj(g.dz * w), in floating point as well (same sums, signs applied exactly), so one product is
- * computed and written twice, once conjugated.  Same results as cnet_clinear_bwd_input / _bwd_weight on such a pair (to
- * rounding: half as many blocks may take another block shape) at half the matrix work.  Replace the same upstream
+ * g.dzs * conj(w) == conj(g.dz * w), so one product is computed and written twice, once conjugated.  Same results as
+ * cnet_clinear_bwd_input / _bwd_weight on such a pair to rounding (with four real products per complex one the sums are
+ * the same and the signs exact, but half as many blocks may take another block shape; with three, see
+ * cnet_cgemm_set_products, the imaginary parts of the two halves are rounded differently) at half the matrix work.  Replace the same upstream
  * functions (gpu/reduce.cpp:532-604, gpu/reducegrad.cpp:288-322); the caller vouches for the pair.  The dzs planes of the
  * result may both be NULL (here and in cnet_cdft_bwd_sym / cnet_ctriang_dft_bwd_sym): then only the dz planes are written,
  * which is all a consumer needs that is itself a conjugate-pair entry point. */
@@ -198,6 +199,26 @@ int cnet_clinear_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg
                          float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int accumulate_dx, float *dw_dz_re,
                          float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im, int64_t lddw, int accumulate_dw, int B, int K,
                          int N);
+
+/* How many real matrix products the block kernels of every complex product above and below (Linear, FourierTrans,
+ * TriangFourier; forward and backward) form one complex product from.  No counterpart upstream, whose kernels multiply
+ * complex numbers one by one with four real multiplications (gpu/reduce.cpp:56-77, impl/linear.h:51-69).
+ *   4 (default): Cr = Ar Br - Ai Bi, Ci = Ar Bi + Ai Br, the four real products of the complex multiplication.
+ *   3: P = Ar Br, Q = Ai Bi, T = (Ar + Ai)(Br + Bi); Cr = P - Q, Ci = T - P - Q (signs of a conjugated operand
+ *      applied to its imaginary part in the sums): a quarter of the matrix work less.  The real part is formed as with
+ *      4; the imaginary part carries the rounding of all three products, so its error is bounded against the size
+ *      of the whole complex entry, not of the imaginary part alone (measured against double precision on normal operands, relative
+ *      Frobenius error of C with 3 against 4: 8.1e-7 against 5.8e-7 at K = 1024, 1.6e-6 against 1.1e-6 at K = 4096; of the
+ *      imaginary plane alone 1.7 times that of 4, of the real plane the same).  An operand pair
+ *      with both imaginary planes zero still gives an imaginary plane of exact zeros (T and P are then the same sums).
+ *      Applies to the block kernels for 16-byte aligned operands with K a multiple of 16 (the ones every large product
+ *      runs on), except the 128 x 128 block when both operands are stored with k contiguous (no registers for a third
+ *      set of accumulators there: the cost model then weighs that block shape at its four products); the small-C
+ *      kernel and the kernel for unaligned operands always use 4.
+ * Process-wide; takes effect with the next product.  The environment variable CNET_CGEMM_3M=0 / 1 sets the initial value.
+ * Returns CNET_ERR_INVALID_ARGUMENT for any other n. */
+int cnet_cgemm_set_products(int n);
+int cnet_cgemm_get_products(void);
 
 /* ---- FourierTrans as dense complex GEMM: replaces FourierGpu::gpu_fft_forward / gpu_fft_backward
  *      (gpu/reduce.cpp:25-35,160-187,382-393; gpu/reducegrad.cpp:45-48,324-336) and the root-table upload

@@ -15,9 +15,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BIN = os.path.join(ROOT, "tests", "bin", "facade_test")
 
 
-def _run(*args, timeout=240):
+def _run(*args, timeout=240, env=None):
     assert os.path.exists(BIN), "tests/bin/facade_test is not built (make -C cnet_amd/host)"
-    res = subprocess.run([BIN] + list(args), capture_output=True, text=True, timeout=timeout)
+    res = subprocess.run([BIN] + list(args), capture_output=True, text=True, timeout=timeout,
+                         env=dict(os.environ, **env) if env else None)
     print(res.stdout[-6000:])
     print(res.stderr[-2000:])
     assert res.returncode == 0, "facade_test %s failed:\n%s" % (" ".join(args), "\n".join(
@@ -131,3 +132,14 @@ def test_residual_stack_full_size_against_the_oracle_and_ten_steps():
     that trains, the loss falling at every step."""
     out = _run("stack8", "2048", "8", "2048", "10", "0.000003", "4", "finite", "learn", timeout=600)
     assert "FAIL" not in out and out.count("PASS") >= 4
+
+
+@pytest.mark.parametrize("scenario", [("pipeline", "1024", "4"), ("resblock",), ("adam",), ("upstream_nets",),
+                                      ("stack8", "64", "8", "16", "6", "0.0001", "0", "finite", "learn"),
+                                      ("stack8", "2048", "8", "2048", "10", "0.000003", "4", "finite", "learn")],
+                         ids=lambda s: "_".join(s[:3]))
+def test_scenarios_with_three_real_products_per_complex_product(scenario):
+    """The block kernels of the matrix products forming a complex product from three real ones (CNET_CGEMM_3M=1,
+    cnet_cgemm_set_products(3)): the same comparisons with the oracle, at the same bounds, as with four."""
+    out = _run(*scenario, timeout=600, env={"CNET_CGEMM_3M": "1"})
+    assert "FAIL" not in out and "PASS" in out

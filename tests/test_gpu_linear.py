@@ -16,6 +16,16 @@ SHAPES = [  # B, K, N
 ]
 
 
+@pytest.fixture(params=[3, 4], ids=["three_products", "four_products"])
+def products(request, gpu):
+    """Runs a test with the block kernels forming a complex product from three real ones (the default) and from four."""
+    lib = capi.load()
+    before = lib.cnet_cgemm_get_products()
+    capi.call("cnet_cgemm_set_products", request.param)
+    yield request.param
+    capi.call("cnet_cgemm_set_products", before)
+
+
 def _case(port, B, K, N, seed):
     xr, xi = seeded(port, seed, (B, K)), seeded(port, seed + 1, (B, K))
     wr, wi = seeded(port, seed + 2, (N, K), 1 / np.sqrt(K)), seeded(port, seed + 3, (N, K), 1 / np.sqrt(K))
@@ -23,6 +33,7 @@ def _case(port, B, K, N, seed):
     return xr, xi, wr, wi, g4
 
 
+@pytest.mark.usefixtures("products")
 @pytest.mark.parametrize("B,K,N", SHAPES)
 def test_linear_forward_and_backward(gpu, port, B, K, N):
     xr, xi, wr, wi, g4 = _case(port, B, K, N, seed=B + K + N)
@@ -68,6 +79,7 @@ def test_linear_accumulate_and_leading_dimensions(gpu, port):
     assert rel_c(dx.host()[0:2], dx_o[0:2]) < 1e-5
 
 
+@pytest.mark.usefixtures("products")
 def test_cgemm_all_layouts(gpu, port):
     """C = op(A) op(B) for the four storage combinations, with and without conj(B), against numpy complex128."""
     M, N, K = 72, 40, 52
@@ -119,6 +131,7 @@ def _check_all_layouts(port, M, N, K):
             assert np.array_equal(hr, base) and np.array_equal(hi, base)
 
 
+@pytest.mark.usefixtures("products")
 @pytest.mark.parametrize("M,N,K", [(8, 24, 1000), (64, 64, 4096), (40, 100, 333), (64, 784, 784), (3, 5, 2049), (784, 784, 4096),
                                    (64, 64, 100000), (520, 516, 2048)])
 def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
@@ -129,6 +142,7 @@ def test_cgemm_short_grid_long_reduction(gpu, port, M, N, K):
     _check_all_layouts(port, M, N, K)
 
 
+@pytest.mark.usefixtures("products")
 @pytest.mark.parametrize("M,N,K", [(4, 4, 16), (132, 200, 64), (260, 68, 48), (700, 388, 32), (1028, 516, 80), (68, 1300, 160),
                                    (4100, 1028, 16), (61, 67, 64), (4096, 784, 256), (1028, 516, 1000), (520, 772, 4092)])
 def test_cgemm_blocks_on_the_edge_of_c(gpu, port, M, N, K):
@@ -191,6 +205,7 @@ def test_linear_headline_shape_rows_against_oracle(gpu, port):
     assert rel_c(full[0:2], parts[0:2]) < 1e-5 and rel_c(full[2:4], parts[2:4]) < 1e-5
 
 
+@pytest.mark.usefixtures("products")
 @pytest.mark.parametrize("M,N,K,nb", [(8192, 1024, 64, 1), (192, 256, 48, 2), (4096, 512, 32, 1), (1024, 2048, 32, 1),
                                       (40, 52, 200, 2), (64, 10, 784, 1)])
 def test_cgemm_conjugate_combinations(gpu, port, M, N, K, nb):
@@ -212,6 +227,7 @@ def test_cgemm_conjugate_combinations(gpu, port, M, N, K, nb):
             assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-5, (conj_a, conj_b)
 
 
+@pytest.mark.usefixtures("products")
 def test_cgemm_random_shapes(gpu, port):
     """About a hundred seeded random problems across the paths of the GEMM: aligned and odd shapes, K with and without a whole
     number of chunks, every layout, conj(B), accumulation, leading dimensions wider than the matrix, against numpy in
@@ -260,3 +276,53 @@ def test_cgemm_tail_blocks_cut_along_k(gpu, tile):
     script = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gpu_tail_blocks_check.py")
     r = subprocess.run([sys.executable, script], env=env, capture_output=True, text=True, timeout=280)
     assert r.returncode == 0 and "OK" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
+def test_three_real_products_per_complex_product(gpu):
+    """cnet_cgemm_set_products: the same products with three and with four real products per complex one against complex128,
+    on rows of the headline shape and of a long reduction.  Three products stay normwise as accurate (the bound below is
+    what they are allowed over four; both are two orders below the parity bar), a product of real operands keeps an
+    imaginary plane of exact zeros, and any other count is refused."""
+    lib = capi.load()
+    before = lib.cnet_cgemm_get_products()
+    rs = np.random.RandomState(7)
+    try:
+        for B, K, N in [(4096, 1024, 1024), (1024, 4096, 2048)]:
+            X = (rs.randn(B, K) + 1j * rs.randn(B, K)).astype(np.complex64)
+            W = ((rs.randn(N, K) + 1j * rs.randn(N, K)) / np.sqrt(K)).astype(np.complex64)
+            x = ops.CMat.from_host(np.ascontiguousarray(X.real), np.ascontiguousarray(X.imag))
+            w = ops.CMat.from_host(np.ascontiguousarray(W.real), np.ascontiguousarray(W.imag))
+            rows = rs.choice(B, 48, replace=False)
+            want = X[rows].astype(np.complex128) @ W.astype(np.complex128).T
+            err = {}
+            for n in (4, 3):
+                capi.call("cnet_cgemm_set_products", n)
+                assert lib.cnet_cgemm_get_products() == n
+                y = ops.CMat.empty(B, N)
+                ops.linear_fwd(x, w, y)
+                yr, yi = y.host()
+                got = (yr + 1j * yi)[rows]
+                err[n] = np.linalg.norm(got - want) / np.linalg.norm(want)
+                # each plane on its own as well: neither is traded for the other
+                err[n, "re"] = np.linalg.norm(got.real - want.real) / np.linalg.norm(want.real)
+                err[n, "im"] = np.linalg.norm(got.imag - want.imag) / np.linalg.norm(want.imag)
+            print("B, K, N = %s: relative error against complex128, four products %.2e (re %.2e, im %.2e), three %.2e (re %.2e, im %.2e)"
+                  % ((B, K, N), err[4], err[4, "re"], err[4, "im"], err[3], err[3, "re"], err[3, "im"]))
+            assert err[4] < 5e-6 and err[3] < 5e-6
+            assert err[3] < 3 * err[4] and err[3, "im"] < 4 * err[4, "im"]
+        # real operands: T and P are the same sums, Q is zero
+        capi.call("cnet_cgemm_set_products", 3)
+        B, K, N = 512, 256, 384
+        xr, wr = rs.randn(B, K).astype(np.float32), rs.randn(N, K).astype(np.float32)
+        x = ops.CMat.from_host(xr, np.zeros_like(xr))
+        w = ops.CMat.from_host(wr, np.zeros_like(wr))
+        y = ops.CMat.empty(B, N)
+        ops.linear_fwd(x, w, y)
+        yr, yi = y.host()
+        assert not yi.any()
+        assert np.linalg.norm(yr - xr.astype(np.float64) @ wr.astype(np.float64).T) / np.linalg.norm(yr) < 1e-6
+        for bad in (0, 2, 5, -3):
+            assert lib.cnet_cgemm_set_products(bad) == -2  # CNET_ERR_INVALID_ARGUMENT
+        assert lib.cnet_cgemm_get_products() == 3
+    finally:
+        capi.call("cnet_cgemm_set_products", before)
