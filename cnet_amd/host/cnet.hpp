@@ -2147,6 +2147,19 @@ public:
 		conjugate_gradients_ = on;
 	}
 	bool conjugateGradients() const { return conjugate_gradients_; }
+	// The block kernels of the matrix products (Linear, FourierTrans, TriangFourier; forward and backward) form a complex
+	// product from three real ones instead of four (cnet_cgemm_set_products): a quarter of the matrix work less, the
+	// imaginary parts rounded against the size of the whole entry instead of their own.  A setting of the device library,
+	// shared by every net of the process; off unless CNET_CGEMM_3M=1 is in the environment.  Recordings of this net are
+	// dropped, since they hold the kernels of the other setting.
+	void threeProductGemm(bool on) {
+		if (on != threeProductGemm() && batch_) {
+			dropGraphs();
+			materializeLazy();  // with the kernels of the setting the backward pass ran under
+		}
+		ck(cnet_cgemm_set_products(on ? 3 : 4), "cnet_cgemm_set_products");
+	}
+	bool threeProductGemm() const { return cnet_cgemm_get_products() == 3; }
 	// Neighbouring layers that run as one kernel where the device layer has one (Hadamard or Linear followed by CGelu): same bits,
 	// fewer passes over memory and fewer launches.  Off: one launch per layer.  Takes effect at the next allocateOnGpu,
 	// or at once when the net is allocated (recordings are dropped).

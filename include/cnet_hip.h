@@ -215,7 +215,8 @@ int cnet_clinear_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg
  *      runs on), except the 128 x 128 block when both operands are stored with k contiguous (no registers for a third
  *      set of accumulators there: the cost model then weighs that block shape at its four products); the small-C
  *      kernel and the kernel for unaligned operands always use 4.
- * Process-wide; takes effect with the next product.  The environment variable CNET_CGEMM_3M=0 / 1 sets the initial value.
+ * Process-wide; takes effect with the next product that is queued (a recorded graph keeps the kernels it was recorded
+ * with).  The environment variable CNET_CGEMM_3M=0 / 1 sets the initial value.
  * Returns CNET_ERR_INVALID_ARGUMENT for any other n. */
 int cnet_cgemm_set_products(int n);
 int cnet_cgemm_get_products(void);

@@ -1632,6 +1632,58 @@ static void test_stack8(int n, int blocks, int B, int steps, float lr, int rows_
 	}
 }
 
+// CNet::threeProductGemm: the same training from the same weights with four and with three real products per complex one, at
+// a size whose products run on the block kernels: the results differ in their last bits (the switch reached the kernels)
+// and agree far inside the parity bound.
+static void test_three_products() {
+	const int n = 512, blocks = 2, B = 1024, steps = 3;  // forward and input-gradient products of 2048 tiles of 16 x 16: block kernels
+	const float lr = 1e-4f;
+	orc::Rng rng(11);
+	std::vector<float> xs((size_t) 2 * B * n), ts((size_t) 2 * B * n);
+	fill_normal(rng, xs.data(), xs.size(), 1.0);
+	fill_normal(rng, ts.data(), ts.size(), 1.0);
+	std::vector<std::vector<float> > w0(blocks, std::vector<float>((size_t) 2 * n * n));
+	for (auto &w : w0) fill_normal(rng, w.data(), w.size(), 1.0 / std::sqrt((double) n));
+	bool initial = false;
+	auto train = [&](bool three, bool switch_after_allocation) {
+		ResStack q;
+		build_stack(q, n, blocks);
+		for (int b = 0; b < blocks; ++b) std::copy(w0[b].begin(), w0[b].end(), q.net[q.w[b]]->mutable_input()->real_);
+		initial = q.net.threeProductGemm();
+		if (!switch_after_allocation) q.net.threeProductGemm(three);
+		q.net.allocateOnGpu(B);
+		if (switch_after_allocation) q.net.threeProductGemm(three);
+		expect(std::string("the setting reads back as ") + (three ? "three" : "four"), q.net.threeProductGemm() == three);
+		std::vector<float> out;
+		for (int step = 0; step < steps; ++step) {
+			InputBatch bx(B, n), bt(B, n);
+			for (int b = 0; b < B; ++b) {
+				bx.add(xs.data() + (size_t) b * n, xs.data() + (size_t) (B + b) * n, n, 0);
+				bt.add(ts.data() + (size_t) b * n, ts.data() + (size_t) (B + b) * n, n, 0);
+			}
+			q.net.gpuSetInput((CInput *) q.net[q.t], bt);
+			q.net.gpuForward((CInput *) q.net[q.x], (L2Out *) q.net[q.l2], bx);
+			out.push_back(q.net.getLoss((L2Out *) q.net[q.l2], &bx));
+			q.net.gpuBackward();
+			q.net.gpuUpdateInputs(lr / B);
+		}
+		q.net.getInputsFromGpu();
+		for (int b = 0; b < blocks; ++b)
+			out.insert(out.end(), q.net[q.w[b]]->input().real_, q.net[q.w[b]]->input().real_ + 2 * n * n);
+		q.net.threeProductGemm(initial);
+		return out;
+	};
+	const std::vector<float> four = train(false, false), three = train(true, false), late = train(true, true);
+	ErrAcc losses, weights;
+	losses.add(three.data(), four.data(), steps);
+	weights.add(three.data() + steps, four.data() + steps, blocks * 2 * n * n);
+	report("losses of three steps, three products against four", losses.value(), 1e-5);
+	report("weights after three steps, three products against four", weights.value(), 1e-5);
+	expect("the two forms do not give the same bits", three != four);
+	expect("switched after allocateOnGpu: the bits of switching before", late == three);
+	expect("the loss falls", four[steps - 1] < four[0] && three[steps - 1] < three[0]);
+}
+
 int main(int argc, char **argv) {
 	std::string what = argc > 1 ? argv[1] : "all";
 	setvbuf(stdout, NULL, _IOLBF, 0);  // keep the log complete if a scenario dies
@@ -1653,6 +1705,7 @@ int main(int argc, char **argv) {
 		if (what == "real_batches" || what == "all") test_real_batches();
 		if (what == "upstream_nets" || what == "all") test_upstream_nets();
 		if (what == "errors" || what == "all") test_errors();
+		if (what == "three_products" || what == "all") test_three_products();
 		// stack8 n blocks B steps lr rows_checked overflow|finite [learn]
 		if (what == "stack8")
 			test_stack8(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 16, argc > 5 ? atoi(argv[5]) : 4,

@@ -134,6 +134,13 @@ def test_residual_stack_full_size_against_the_oracle_and_ten_steps():
     assert "FAIL" not in out and out.count("PASS") >= 4
 
 
+def test_three_product_switch_of_the_facade():
+    """CNet::threeProductGemm(bool): reaches the kernels (other bits), agrees with four products to 1e-5 over three SGD steps,
+    and may be flipped on an allocated net."""
+    out = _run("three_products")
+    assert "FAIL" not in out and out.count("PASS") >= 8
+
+
 @pytest.mark.parametrize("scenario", [("pipeline", "1024", "4"), ("resblock",), ("adam",), ("upstream_nets",),
                                       ("stack8", "64", "8", "16", "6", "0.0001", "0", "finite", "learn"),
                                       ("stack8", "2048", "8", "2048", "10", "0.000003", "4", "finite", "learn")],
