@@ -92,9 +92,10 @@ struct ArgMaxOp {
 		return a;
 	}
 };
-// the largest |z|^2 of a row with its first index, and the runner-up value (to detect near ties)
+// the largest |z|^2 of a row with its first index, and the runner-up value (to detect near ties); single precision is
+// enough for both: they only decide whether the exact second pass is needed (a margin of 1e-5 against 1e-7 of rounding)
 struct Top2 {
-	double q1, q2;
+	float q1, q2;
 	int i1, pad;
 };
 struct Top2Op {
@@ -104,7 +105,7 @@ struct Top2Op {
 		const Top2 &w = b_wins ? b : a, &l = b_wins ? a : b;
 		r.q1 = w.q1;
 		r.i1 = w.i1;
-		r.q2 = fmax(w.q2, l.q1);
+		r.q2 = fmaxf(w.q2, l.q1);
 		r.pad = 0;
 		return r;
 	}
@@ -204,12 +205,13 @@ __device__ __forceinline__ void crossent_fwd_row(const float *__restrict__ zr, c
 	__shared__ Top2 lds_t[TPB / 64];
 	CNET_ROW_SETUP();
 	const float *pr = zr + (long) row * ldz, *pi = zi + (long) row * ldz;
-	// pass 1 (the only pass in the common case): sum |z|^2 in double, and the two largest |z_k|^2 of the row
+	// pass 1 (the only pass in the common case): sum |z|^2 in double (two fused multiply-adds per element: the squares of
+	// floats are exact in double), and the two largest |z_k|^2 of the row in single precision
 	double sum = 0.0;
-	Top2 top = {-1.0, -1.0, 0x7fffffff, 0};
+	Top2 top = {-1.0f, -1.0f, 0x7fffffff, 0};
 	auto visit = [&](float a, float b, int k) {
-		const double q = (double) a * (double) a + (double) b * (double) b;
-		sum += q;
+		sum = fma((double) b, (double) b, fma((double) a, (double) a, sum));
+		const float q = fmaf(a, a, b * b);
 		if (q > top.q1) {
 			top.q2 = top.q1;
 			top.q1 = q;
@@ -241,7 +243,7 @@ __device__ __forceinline__ void crossent_fwd_row(const float *__restrict__ zr, c
 	// The reference argmax is taken over p_k = fl(|fl(z_k / sqrt S)|^2), which orders like |z_k|^2 except within a few
 	// ulp.  When the runner-up is more than 1e-5 (relative) below the maximum the winner is already decided; otherwise,
 	// or when the normalised planes are wanted, a second pass evaluates p_k exactly as the reference does.
-	const bool clear_cut = top.q2 < top.q1 * (1.0 - 1.0e-5);
+	const bool clear_cut = top.q2 < top.q1 * (1.0f - 1.0e-5f);
 	constexpr bool want_grad = GRAD;
 	if (!want_out && !want_grad && clear_cut) {
 		if (live && t == 0) {
