@@ -308,7 +308,8 @@ def train_lines(steps):
         n = min(3000, steps * (4096 // batch))
         # "frozen_input" adds the mode in which the data input is marked not trainable (no step on it, no backward pass
         # into it; off by default in the facade, as upstream steps every input function)
-        line = _train_bench("readme", batch, n, "frozen_input")
+        # "on_device" adds the loop whose reader keeps its samples in device memory (BatchedDataReader::storeOnDevice)
+        line = _train_bench("readme", batch, n, "frozen_input", "on_device")
         if line is None:
             return None
         # configs[0] states real samples (imaginary parts 0), whose imaginary plane is cleared on the device instead of
@@ -576,6 +577,8 @@ def main():
                              "samples_per_sec": t["samples_per_sec_prefetch_loss_read_one_step_late"],
                              "samples_per_sec_loss_read_before_next_step": t["samples_per_sec_prefetch"],
                              "samples_per_sec_data_input_not_trainable": t["samples_per_sec_data_input_not_trainable"],
+                             # the reader's samples kept in device memory: a batch travels as 4 bytes per sample
+                             "samples_per_sec_samples_stored_on_device": t.get("samples_per_sec_samples_stored_on_device"),
                              "samples_per_sec_copy_inside_forward": t["samples_per_sec_copy_in_forward"],
                              "samples": t.get("samples"), "upload_bytes_per_step": t.get("upload_bytes_per_step"),
                              "samples_per_sec_complex_samples": t.get("samples_per_sec_complex_samples")} for t in train]

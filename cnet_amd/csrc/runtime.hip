@@ -331,6 +331,48 @@ int cnet_upload_pair(void *dst0, const void *pinned_src0, size_t bytes0, void *d
 	return CNET_OK;
 }
 
+// rows of a table on the device into a batch buffer, with their labels: workgroup (r, p) copies row idx[r] of plane p
+__global__ __launch_bounds__(256) void gather_rows_kernel(float *__restrict__ dst, long ldd, long dst_plane, const float *__restrict__ src,
+		long lds, long src_plane, int src_rows, const int32_t *__restrict__ idx, int32_t *__restrict__ dst_labels,
+		const int32_t *__restrict__ src_labels, int cols, int vec) {
+	__shared__ int which;
+	if (threadIdx.x == 0) which = min(max(idx[blockIdx.x], 0), src_rows - 1);  // one read over the link per workgroup
+	__syncthreads();
+	const int i = which;
+	const float *s = src + (long) blockIdx.y * src_plane + (long) i * lds;
+	float *d = dst + (long) blockIdx.y * dst_plane + (long) blockIdx.x * ldd;
+	if (vec) {
+		for (int c = threadIdx.x * 4; c < cols; c += 1024) *reinterpret_cast<float4 *>(d + c) = *reinterpret_cast<const float4 *>(s + c);
+	} else {
+		for (int c = threadIdx.x; c < cols; c += 256) d[c] = s[c];
+	}
+	if (blockIdx.y == 0 && threadIdx.x == 0 && dst_labels) dst_labels[blockIdx.x] = src_labels[i];
+}
+
+int cnet_upload_gather_rows(float *dst, int64_t ldd, int64_t dst_plane_stride, const float *src, int64_t lds, int64_t src_plane_stride,
+		int planes, int src_rows, const int32_t *pinned_idx, int32_t *dst_labels, const int32_t *src_labels, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // work on the upload stream: never part of a recording
+	CNET_CHECK_ARG(rows >= 0 && rows <= 65535 * 32 && cols > 0 && src_rows > 0 && (planes == 1 || planes == 2));
+	if (!rows) return CNET_OK;
+	CNET_CHECK_ARG(dst && src && pinned_idx && ldd >= cols && lds >= cols);
+	CNET_CHECK_ARG((dst_labels == nullptr) == (src_labels == nullptr));
+	CNET_CHECK_ARG(planes == 1 || (dst_plane_stride >= (int64_t) (rows - 1) * ldd + cols && src_plane_stride >= (int64_t) (src_rows - 1) * lds + cols));
+	// the kernel reads the indices where they are: anything but memory from cnet_host_alloc would be a fault on the device
+	if (!in_pinned_range(pinned_idx, (size_t) rows * sizeof(int32_t)))
+		return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_upload_gather_rows: the indices do not lie in memory from cnet_host_alloc");
+	for (int r = 0; r < rows; ++r)
+		if (pinned_idx[r] < 0 || pinned_idx[r] >= src_rows)
+			return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_upload_gather_rows: index %d of row %d outside the table of %d rows", pinned_idx[r], r, src_rows);
+	const bool vec = cols % 4 == 0 && ldd % 4 == 0 && lds % 4 == 0 && dst_plane_stride % 4 == 0 && src_plane_stride % 4 == 0 && aligned16(dst) &&
+			aligned16(src);
+	dim3 grid((unsigned) rows, (unsigned) planes);
+	hipLaunchKernelGGL(gather_rows_kernel, grid, dim3(256), 0, rt().upload_stream, dst, (long) ldd, (long) dst_plane_stride, src, (long) lds,
+			(long) src_plane_stride, src_rows, pinned_idx, dst_labels, src_labels, cols, vec ? 1 : 0);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
+}
+
 int cnet_upload_zero(void *dst, size_t bytes) {
 	CNET_REQUIRE_INIT();
 	CNET_NOT_IN_CAPTURE();  // a fill on the upload stream: never part of a recording

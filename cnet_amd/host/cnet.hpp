@@ -169,6 +169,63 @@ public:
 	int label(int i) { return labels_[i]; }
 };
 
+// A data set kept on the device: the samples as planes [count][dim] (the imaginary plane only if some sample has an imaginary
+// part other than +0) and their labels.  A batch assembled out of it (InputBatch::gatherResident, BatchedDataReader::
+// storeOnDevice) names its samples by index; gpuForward / gpuPrefetch then send the indices, 4 bytes per sample, and the
+// device copies the rows out of its own memory (cnet_upload_gather_rows) instead of receiving them over the link again in
+// every epoch.  No counterpart upstream, whose batches always travel from host memory (gpu/gpu_func.h:403-419).  Must outlive
+// every batch that refers to it and every step that such a batch was fed to.
+class DeviceDataset {
+	friend class CNet;
+	friend class InputBatch;
+	float *z_ = NULL;             // device: planes_ x [count][dim]
+	int32_t *labels_dev_ = NULL;  // device: [count]
+	std::vector<int> labels_;
+	int count_ = 0, dim_ = 0, planes_ = 1;
+	static void must(int rc, const char *what) {
+		if (rc != CNET_OK) throw std::runtime_error(std::string(what) + " failed (" + std::to_string(rc) + "): " + cnet_last_error());
+	}
+
+public:
+	// re, im: [count][dim] on the host (im may be NULL: real samples); labels: [count]
+	DeviceDataset(const float *re, const float *im, const int *labels, int count, int dim) : labels_(labels, labels + count), count_(count), dim_(dim) {
+		if (count <= 0 || dim <= 0) throw std::invalid_argument("DeviceDataset: no samples");
+		const size_t plane = (size_t) count * dim;
+		bool complex_samples = false;
+		if (im) {
+			uint32_t acc = 0;
+			for (size_t k = 0; k < plane; ++k) {
+				uint32_t w;
+				std::memcpy(&w, im + k, sizeof(w));
+				acc |= w;
+			}
+			complex_samples = acc != 0;
+		}
+		planes_ = complex_samples ? 2 : 1;
+		void *p = NULL;
+		must(cnet_alloc((size_t) planes_ * plane * sizeof(float), &p), "cnet_alloc");
+		z_ = (float *) p;
+		must(cnet_alloc((size_t) count * sizeof(int32_t), &p), "cnet_alloc");
+		labels_dev_ = (int32_t *) p;
+		must(cnet_memcpy_h2d(z_, re, plane * sizeof(float)), "cnet_memcpy_h2d");
+		if (complex_samples) must(cnet_memcpy_h2d(z_ + plane, im, plane * sizeof(float)), "cnet_memcpy_h2d");
+		std::vector<int32_t> l32(labels, labels + count);
+		must(cnet_memcpy_h2d(labels_dev_, l32.data(), (size_t) count * sizeof(int32_t)), "cnet_memcpy_h2d");
+	}
+	DeviceDataset(const DeviceDataset &) = delete;
+	DeviceDataset &operator=(const DeviceDataset &) = delete;
+	~DeviceDataset() {
+		cnet_upload_sync();  // a batch may still be on its way out of these planes
+		cnet_sync();
+		cnet_free(z_);
+		cnet_free(labels_dev_);
+	}
+	int size() const { return count_; }
+	int sampleDim() const { return dim_; }
+	int label(int i) const { return labels_[i]; }
+	bool imagIsZero() const { return planes_ == 1; }  // every sample is real
+};
+
 // Two [batch x dim] planes in page-locked host memory when the device library is initialised (pageable otherwise), so
 // a batch goes to the device as one asynchronous copy per plane (upstream: two pageable copies per sample,
 // gpu/gpu_func.h:403-419).  Movable and reusable: clear() empties it for the next fill without giving the memory back.
@@ -182,6 +239,10 @@ class InputBatch : public Batch {
 	bool imag_nonzero_ = false;
 	// every element of the imaginary plane, filled rows or not, holds +0: rows of real samples then need no write at all
 	bool imag_clean_ = false;
+	// The samples of this batch are rows of a data set on the device (gatherResident): indices_[k] names the row of sample k,
+	// the planes above are not filled.
+	const DeviceDataset *resident_ = NULL;
+	int32_t *indices_ = NULL;  // [batch], page-locked, allocated at the first gatherResident
 	static bool anyBitSet(const float *p, size_t n) {
 		uint32_t acc = 0;
 		for (size_t k = 0; k < n; ++k) {
@@ -212,6 +273,8 @@ class InputBatch : public Batch {
 		if (pinned_) cnet_host_free(real_data_);  // waits for copies still reading it
 		else ::operator delete(real_data_);
 		real_data_ = imag_data_ = NULL;
+		if (indices_) cnet_host_free(indices_);
+		indices_ = NULL;
 	}
 	void settle() {  // before the host writes the planes again
 		if (ticket_ >= 0) {  // waits for that copy only: a copy out of another batch may still be running
@@ -230,6 +293,7 @@ class InputBatch : public Batch {
 	float *rowRe() { return real_data_ + (size_t) current_pos_ * sample_dim_; }
 	float *rowIm() { return imag_data_ + (size_t) current_pos_ * sample_dim_; }
 	void finishRow(int filled, int label) {
+		if (resident_) throw std::logic_error("InputBatch: the batch holds samples of a data set on the device; clear() it first");
 		std::fill(rowRe() + filled, rowRe() + sample_dim_, 0.f);  // padding with 0s
 		std::fill(rowIm() + filled, rowIm() + sample_dim_, 0.f);
 		labels_.push_back(label);
@@ -245,10 +309,20 @@ public:
 		if (o.real_data_) std::copy(o.real_data_, o.real_data_ + 2 * (size_t) batch_size_ * sample_dim_, real_data_);
 		imag_nonzero_ = o.imag_nonzero_;
 		imag_clean_ = o.imag_clean_;
+		if (o.resident_ && o.indices_) {
+			void *p = NULL;
+			if (cnet_host_alloc((size_t) batch_size_ * sizeof(int32_t), &p) == CNET_OK && p) {
+				indices_ = (int32_t *) p;
+				std::copy(o.indices_, o.indices_ + batch_size_, indices_);
+				resident_ = o.resident_;
+			}
+		}
 	}
 	InputBatch(InputBatch &&o) noexcept : Batch(std::move(o)), real_data_(o.real_data_), imag_data_(o.imag_data_), pinned_(o.pinned_),
-			ticket_(o.ticket_), imag_nonzero_(o.imag_nonzero_), imag_clean_(o.imag_clean_) {
+			ticket_(o.ticket_), imag_nonzero_(o.imag_nonzero_), imag_clean_(o.imag_clean_), resident_(o.resident_), indices_(o.indices_) {
 		o.real_data_ = o.imag_data_ = NULL;
+		o.indices_ = NULL;
+		o.resident_ = NULL;
 	}
 	InputBatch &operator=(InputBatch &&o) noexcept {
 		if (this != &o) {
@@ -260,7 +334,11 @@ public:
 			ticket_ = o.ticket_;
 			imag_nonzero_ = o.imag_nonzero_;
 			imag_clean_ = o.imag_clean_;
+			resident_ = o.resident_;
+			indices_ = o.indices_;
 			o.real_data_ = o.imag_data_ = NULL;
+			o.indices_ = NULL;
+			o.resident_ = NULL;
 		}
 		return *this;
 	}
@@ -276,6 +354,7 @@ public:
 		sizes_.clear();
 		current_pos_ = 0;
 		imag_nonzero_ = false;
+		resident_ = NULL;
 	}
 	// every imaginary part added so far is +0: the samples are real
 	bool imagIsZero() const { return !imag_nonzero_; }
@@ -309,6 +388,7 @@ public:
 	// than +0 has been in the plane since it was last all zeros.
 	void gather(const float *re, const float *im, const int *labels, const int *index, int count) {
 		assert(current_pos_ + count <= batch_size_);
+		if (resident_) throw std::logic_error("InputBatch: the batch holds samples of a data set on the device; clear() it first");
 		settle();
 		const size_t dim = (size_t) sample_dim_;
 		float *dst_re = rowRe(), *dst_im = rowIm();
@@ -332,6 +412,32 @@ public:
 		}
 		current_pos_ += count;
 	}
+	// The next `count` samples of the batch are rows index[0 .. count) of a data set on the device: only the indices and the
+	// labels are noted here, the planes of this batch stay as they are.  A batch is filled either this way, from one data
+	// set, or with add() / gather(), not both.
+	void gatherResident(const DeviceDataset &ds, const int *index, int count) {
+		assert(current_pos_ + count <= batch_size_);
+		if (ds.sampleDim() != sample_dim_) throw std::invalid_argument("InputBatch::gatherResident: sample dimension differs from the data set");
+		if ((current_pos_ > 0 && resident_ != &ds) || (resident_ && resident_ != &ds))
+			throw std::logic_error("InputBatch::gatherResident: the batch already holds samples from elsewhere");
+		settle();  // the indices of the last fill may still be read
+		if (!indices_) {
+			void *p = NULL;
+			if (cnet_host_alloc((size_t) batch_size_ * sizeof(int32_t), &p) != CNET_OK || !p)
+				throw std::runtime_error("InputBatch::gatherResident: no page-locked memory for the indices (is the device library initialised?)");
+			indices_ = (int32_t *) p;
+		}
+		resident_ = &ds;
+		for (int k = 0; k < count; ++k) {
+			if (index[k] < 0 || index[k] >= ds.size()) throw std::out_of_range("InputBatch::gatherResident: no such sample in the data set");
+			indices_[current_pos_ + k] = index[k];
+			labels_.push_back(ds.label(index[k]));
+			sizes_.push_back(sample_dim_);
+		}
+		if (!ds.imagIsZero()) imag_nonzero_ = true;
+		current_pos_ += count;
+	}
+	bool isResident() const { return resident_ != NULL; }
 	const float *realDataPtr() const { return real_data_; }
 	const float *imagDataPtr() const { return imag_data_; }
 	const float *realDataPtr(int b) const { return real_data_ + (size_t) b * sample_dim_; }
@@ -1902,7 +2008,20 @@ private:
 		const bool real_only = batch.imagIsZero() && !send_zero_planes_;
 		Stage &here = stage_[active_];
 		const bool clear_imag = real_only && !here.imag_dev_zero;  // unless the plane is still clear from the last batch
-		if (batch.isPinned()) {
+		if (batch.resident_) {
+			// The samples are on the device already: the upload stream, behind everything queued on the compute stream so far
+			// (which may still read this buffer), copies the rows named by the indices; the compute stream waits for that.
+			const DeviceDataset &ds = *batch.resident_;
+			const size_t floats = (size_t) batch_ * s.len;
+			ck(cnet_upload_wait_compute(), "cnet_upload_wait_compute");
+			if (clear_imag) ck(cnet_upload_zero(s.z + floats, plane), "cnet_upload_zero");
+			ck(cnet_upload_gather_rows(s.z, s.len, (int64_t) floats, ds.z_, ds.dim_, (int64_t) ds.count_ * ds.dim_, ds.planes_, ds.count_, batch.indices_,
+					NULL, NULL, batch_, s.len), "cnet_upload_gather_rows");
+			// a data set of real samples fills the real plane only; sendZeroPlanes has nothing to send here
+			if (!real_only && ds.planes_ == 1) ck(cnet_upload_zero(s.z + floats, plane), "cnet_upload_zero");
+			ck(cnet_copy_ticket(1, &batch.ticket_), "cnet_copy_ticket");
+			ck(cnet_compute_wait_ticket(batch.ticket_), "cnet_compute_wait_ticket");
+		} else if (batch.isPinned()) {
 			ck(cnet_memcpy_h2d_async(s.z, batch.realDataPtr(), real_only ? plane : 2 * plane), "cnet_memcpy_h2d_async");
 			if (clear_imag) ck(cnet_memset_zero(s.z + (size_t) batch_ * s.len, plane), "cnet_memset_zero");
 			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
@@ -1927,7 +2046,7 @@ public:
 		if (!cin || cin != main_input_) throw std::invalid_argument("gpuPrefetch: not the main input of the allocated net");
 		if (batch.size() != batch_ || batch.noOfLabels() != batch_ || batch.sampleDim() != cin->input().length_)
 			throw std::invalid_argument("gpuPrefetch: batch shape differs from the allocated net");
-		if (!batch.isPinned()) throw std::invalid_argument("gpuPrefetch: the batch is not in page-locked memory");
+		if (!batch.isPinned() && !batch.resident_) throw std::invalid_argument("gpuPrefetch: the batch is not in page-locked memory");
 		checkLabels(batch.labelsPtr(), batch_);
 		const int other = 1 - active_;
 		Stage &st = stage_[other];
@@ -1938,22 +2057,32 @@ public:
 			st.z = dalloc<float>(2 * plane);
 			st.labels = dalloc<int32_t>(batch_);
 		}
-		if (!st.host_labels) {
-			void *h = NULL;
-			ck(cnet_host_alloc(batch_ * sizeof(int32_t), &h), "cnet_host_alloc");
-			st.host_labels = (int32_t *) h;
+		if (!batch.resident_) {
+			if (!st.host_labels) {
+				void *h = NULL;
+				ck(cnet_host_alloc(batch_ * sizeof(int32_t), &h), "cnet_host_alloc");
+				st.host_labels = (int32_t *) h;
+			}
+			if (st.labels_ticket >= 0) ck(cnet_copy_wait(st.labels_ticket), "cnet_copy_wait");  // the previous copy has left host_labels
+			std::copy(batch.labelsPtr(), batch.labelsPtr() + batch_, st.host_labels);
 		}
-		if (st.labels_ticket >= 0) ck(cnet_copy_wait(st.labels_ticket), "cnet_copy_wait");  // the previous copy has left host_labels
-		std::copy(batch.labelsPtr(), batch.labelsPtr() + batch_, st.host_labels);
 		ck(cnet_upload_wait_marker(other), "cnet_upload_wait_marker");  // kernels of the step that last used this buffer
 		// the two planes of a batch are one array on the host and on the device: one copy for both
 		st.imag_zero = batch.imagIsZero();
 		const bool real_only = st.imag_zero && !send_zero_planes_;
 		// the plane is still clear when the last batch that landed here was real and nothing has stepped the values since
 		if (real_only && !st.imag_dev_zero) ck(cnet_upload_zero(st.z + plane, plane * sizeof(float)), "cnet_upload_zero");
-		// the samples and their labels: one launch for a small batch, two queued copies for a large one
-		ck(cnet_upload_pair(st.z, batch.realDataPtr(), (real_only ? 1 : 2) * plane * sizeof(float), st.labels, st.host_labels,
-				batch_ * sizeof(int32_t)), "cnet_upload_pair");
+		if (batch.resident_) {
+			// the samples and their labels are on the device already: one launch copies the rows that the indices name
+			const DeviceDataset &ds = *batch.resident_;
+			ck(cnet_upload_gather_rows(st.z, s.len, (int64_t) plane, ds.z_, ds.dim_, (int64_t) ds.count_ * ds.dim_, ds.planes_, ds.count_, batch.indices_,
+					st.labels, ds.labels_dev_, batch_, s.len), "cnet_upload_gather_rows");
+			if (!real_only && ds.planes_ == 1) ck(cnet_upload_zero(st.z + plane, plane * sizeof(float)), "cnet_upload_zero");
+		} else {
+			// the samples and their labels: one launch for a small batch, two queued copies for a large one
+			ck(cnet_upload_pair(st.z, batch.realDataPtr(), (real_only ? 1 : 2) * plane * sizeof(float), st.labels, st.host_labels,
+					batch_ * sizeof(int32_t)), "cnet_upload_pair");
+		}
 		st.imag_dev_zero = st.imag_zero;
 		// one recorded point serves the host (the batch may be refilled, the staging of the labels reused) and the compute
 		// stream (the forward pass of this batch)

@@ -10,6 +10,7 @@
 
 #include <algorithm>
 #include <fstream>
+#include <memory>
 #include <random>
 #include <string>
 #include <vector>
@@ -23,6 +24,7 @@ class BatchedDataReader {
 	std::vector<int> order_;      // position -> sample
 	std::vector<int> pick_;       // samples of the batch being assembled
 	bool imag_all_zero_ = true;   // no sample added so far has an imaginary part other than +0 (images): batches skip that plane
+	std::shared_ptr<DeviceDataset> on_device_;  // the samples as they were at storeOnDevice(), kept in device memory (copies of the reader share it)
 	void noteImag(const float *im, size_t n) {
 		uint32_t acc = 0;
 		for (size_t k = 0; k < n; ++k) {
@@ -69,8 +71,24 @@ public:
 			pick_[i] = order_[current_];
 			current_ = (current_ + 1) % (int) labels_.size();
 		}
-		batch.gather(re_.data(), imag_all_zero_ ? NULL : im_.data(), labels_.data(), pick_.data(), batch.size());
+		if (on_device_)
+			batch.gatherResident(*on_device_, pick_.data(), batch.size());
+		else
+			batch.gather(re_.data(), imag_all_zero_ ? NULL : im_.data(), labels_.data(), pick_.data(), batch.size());
 	}
+
+	// Keep a copy of all samples and labels in device memory (the device library must be initialised): the batches of
+	// nextBatch() then only name their samples, and CNet::gpuForward / gpuPrefetch copy them on the device instead of
+	// sending them over the link again in every epoch.  Same samples, same order, same results.  Samples added afterwards
+	// are not part of the copy until the next call; releaseDevice() goes back to batches that carry their samples.  The
+	// reader must outlive the steps its batches were fed to.
+	void storeOnDevice() {
+		assert(labels_.size());
+		on_device_.reset();
+		on_device_.reset(new DeviceDataset(re_.data(), imag_all_zero_ ? NULL : im_.data(), labels_.data(), (int) labels_.size(), sample_dim_));
+	}
+	void releaseDevice() { on_device_.reset(); }
+	bool storedOnDevice() const { return on_device_ != NULL; }
 
 	void add(const std::vector<std::complex<float> > &data, int label) {
 		assert((int) data.size() <= sample_dim_);

@@ -2,7 +2,7 @@
 // bench.py runs for the "train samples/sec" half of the metric.  Synthetic, seeded data from its own generator; no
 // comparison with anything (the parity tests do that), one JSON line per run on stdout.
 //
-//   train_bench readme B steps [graphs] [both_halves] [frozen_input] [complex_samples]
+//   train_bench readme B steps [graphs] [both_halves] [frozen_input] [complex_samples] [on_device]
 //       FourierTrans(784) -> Hadamard -> CGelu -> Linear 784 -> 10 -> CrossEntropy, SGD, batches from a
 //       BatchedDataReader; the loop of upstream cnet.cpp:119-150 in several input / read-back modes.
 //   train_bench stack n blocks B steps lr [both_halves]
@@ -92,8 +92,8 @@ bool has(int argc, char **argv, int from, const char *word) {
 //   2 as 1, phases replayed from recorded graphs       3 as 0 with recorded graphs
 //   4 as 1 with gpuTrainStep (one recorded graph)      5 as 1 with both halves of every gradient pair computed
 //   6 as 1, the loss of a step read one step later     7 as 6 with gpuTrainStep
-//   8 as 6 with the data input marked not trainable
-int run_readme(int B, int steps, bool with_graphs, bool both_halves, bool frozen_input, bool complex_samples) {
+//   8 as 6 with the data input marked not trainable     9 as 6 with the reader's samples stored on the device
+int run_readme(int B, int steps, bool with_graphs, bool both_halves, bool frozen_input, bool complex_samples, bool on_device) {
 	const int n = 784, classes = 10;
 	const float lr = 0.01f;
 	if (cnet_init(0) != CNET_OK) {
@@ -101,15 +101,16 @@ int run_readme(int B, int steps, bool with_graphs, bool both_halves, bool frozen
 		return 2;
 	}
 	SyntheticReader data(n, 3 * B + 7, classes, complex_samples);
-	constexpr int MODES = 9;
-	double ms[MODES] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
-	float last_loss[MODES] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+	constexpr int MODES = 10;
+	double ms[MODES] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+	float last_loss[MODES] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 	for (int mode = 0; mode < MODES; ++mode) {
 		if (!with_graphs && ((mode >= 2 && mode <= 4) || mode == 7)) continue;
 		if (mode == 5 && !both_halves) continue;
 		if (mode == 8 && !frozen_input) continue;
+		if (mode == 9 && !on_device) continue;
 		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4 || mode == 7;
-		const bool late_loss = mode == 6 || mode == 7 || mode == 8;
+		const bool late_loss = mode == 6 || mode == 7 || mode == 8 || mode == 9;
 		CNet::PendingLoss pending;
 		CNet net;
 		int inp, outp;
@@ -118,6 +119,7 @@ int run_readme(int B, int steps, bool with_graphs, bool both_halves, bool frozen
 		CInput *cin = (CInput *) net[inp];
 		CrossEntropy *cen = (CrossEntropy *) net[outp];
 		SyntheticReader reader = data;
+		if (mode == 9) reader.storeOnDevice();  // before the clock starts: the samples are in device memory when the loop begins
 		InputBatch ring[3] = {InputBatch(B, n), InputBatch(B, n), InputBatch(B, n)};
 		if (graphs) net.useGraphs(true);
 		if (mode == 5) net.conjugateGradients(false);
@@ -176,9 +178,10 @@ int run_readme(int B, int steps, bool with_graphs, bool both_halves, bool frozen
 		   "\"ms_per_step_prefetch_two_products_per_gradient_pair\": %.3f, \"ms_per_step_prefetch_loss_read_one_step_late\": %.3f, "
 		   "\"samples_per_sec_prefetch_loss_read_one_step_late\": %.1f, \"ms_per_step_train_step_graph_loss_read_one_step_late\": %.3f, "
 		   "\"ms_per_step_data_input_not_trainable\": %.3f, \"samples_per_sec_data_input_not_trainable\": %.1f, "
-		   "\"last_loss\": %.5f, \"samples\": \"%s\", \"upload_bytes_per_step\": %zu}\n",
+		   "\"ms_per_step_samples_stored_on_device\": %.3f, \"samples_per_sec_samples_stored_on_device\": %.1f, "
+		   "\"last_loss\": %.5f, \"last_loss_samples_stored_on_device\": %.5f, \"samples\": \"%s\", \"upload_bytes_per_step\": %zu}\n",
 			B, steps, ms[0], ms[1], ms[2], ms[3], rate(0), rate(1), rate(2), ms[4], rate(4), ms[5], ms[6], rate(6), ms[7], ms[8], rate(8),
-			last_loss[6], complex_samples ? "complex: real and imaginary parts uniform in [0, 1]" : "real parts uniform in [0, 1], imaginary parts 0 (the imaginary plane is cleared on the device, not sent)",
+			ms[9], rate(9), last_loss[6], last_loss[9], complex_samples ? "complex: real and imaginary parts uniform in [0, 1]" : "real parts uniform in [0, 1], imaginary parts 0 (the imaginary plane is cleared on the device, not sent)",
 			(size_t) (complex_samples ? 2 : 1) * B * n * sizeof(float));
 	return std::isfinite(last_loss[6]) ? 0 : 1;
 }
@@ -266,7 +269,7 @@ int main(int argc, char **argv) {
 	try {
 		if (what == "readme")
 			return run_readme(argc > 2 ? atoi(argv[2]) : 4096, argc > 3 ? atoi(argv[3]) : 30, has(argc, argv, 4, "graphs"),
-					has(argc, argv, 4, "both_halves"), has(argc, argv, 4, "frozen_input"), has(argc, argv, 4, "complex_samples"));
+					has(argc, argv, 4, "both_halves"), has(argc, argv, 4, "frozen_input"), has(argc, argv, 4, "complex_samples"), has(argc, argv, 4, "on_device"));
 		if (what == "stack")
 			return run_stack(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048,
 					argc > 5 ? atoi(argv[5]) : 10, argc > 6 ? (float) atof(argv[6]) : 0.01f, has(argc, argv, 7, "both_halves"));
@@ -274,6 +277,6 @@ int main(int argc, char **argv) {
 		fprintf(stderr, "train_bench: %s\n", e.what());
 		return 2;
 	}
-	fprintf(stderr, "usage: train_bench readme B steps [graphs] [both_halves] [frozen_input] [complex_samples] | stack n blocks B steps lr [both_halves]\n");
+	fprintf(stderr, "usage: train_bench readme B steps [graphs] [both_halves] [frozen_input] [complex_samples] [on_device] | stack n blocks B steps lr [both_halves]\n");
 	return 64;
 }

@@ -97,6 +97,15 @@ int cnet_upload_zero(void *dst, size_t bytes);
  * host time of two queued copies and none of the copy engine's start-up time), beyond that, or when a source does not lie
  * in memory from cnet_host_alloc, as two cnet_upload_async */
 int cnet_upload_pair(void *dst0, const void *pinned_src0, size_t bytes0, void *dst1, const void *pinned_src1, size_t bytes1);
+/* A batch out of a data set that is kept on the device, on the upload stream, in one launch:
+ *   dst[p][r][0 .. cols) = src[p][idx[r]][0 .. cols)  for p < planes (1 or 2; plane p starts p * plane_stride floats in),
+ *   dst_labels[r] = src_labels[idx[r]]                 when both label arrays are given (both NULL: samples only).
+ * idx: `rows` int32 in memory from cnet_host_alloc, each in [0, src_rows) (checked on the host; the kernel reads them over
+ * the link, 4 bytes per sample instead of the sample).  No counterpart upstream, which copies every sample of every batch
+ * from host memory (gpu/gpu_func.h:403-419): with the samples resident, a batch moves at the speed of device memory. */
+int cnet_upload_gather_rows(float *dst, int64_t ldd, int64_t dst_plane_stride, const float *src, int64_t lds,
+                            int64_t src_plane_stride, int planes, int src_rows, const int32_t *pinned_idx,
+                            int32_t *dst_labels, const int32_t *src_labels, int rows, int cols);
 int cnet_upload_wait_compute(void);
 int cnet_mark_compute(int marker);
 int cnet_upload_wait_marker(int marker);

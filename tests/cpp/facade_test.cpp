@@ -922,11 +922,15 @@ static void test_pipeline(int B, int steps) {
 	// 10: prefetch, every backward pass adds the gradients to the input functions' own planes at once (CNet::deferGathers(false))
 	// 11 / 12: as 1 / 6 with the losses kept in a device buffer and copied when asked for (CNet::hostLosses(false)) instead of
 	//          stored into page-locked memory by the loss kernel
-	constexpr int MODES = 13;
+	// 13 / 14 / 15: as 0 / 6 / 4 with the reader's samples stored on the device (BatchedDataReader::storeOnDevice): the batches
+	//          name their samples and the device copies them out of its own memory
+	constexpr int MODES = 16;
 	std::vector<float> losses[MODES];
 	std::vector<float> weights[MODES];
 	double ms[MODES] = {0};
-	for (int mode = 0; mode < MODES; ++mode) {
+	for (int slot = 0; slot < MODES; ++slot) {
+		const bool resident = slot >= 13;
+		const int mode = slot == 13 ? 0 : slot == 14 ? 6 : slot == 15 ? 4 : slot;  // what the loop does; `slot` is where its results go
 		const bool prefetch = mode == 1 || mode == 2 || mode >= 4, graphs = mode == 2 || mode == 3, one_graph = mode == 4 || mode == 7;
 		const bool late_loss = mode == 6 || mode == 7 || mode == 8 || mode == 12;
 		CNet::PendingLoss pending;
@@ -938,8 +942,9 @@ static void test_pipeline(int B, int steps) {
 		CrossEntropy *cen = (CrossEntropy *) net[outp];
 		if (mode >= 11) net.hostLosses(false);
 		SyntheticReader reader = data;  // same order for both modes
+		if (resident) reader.storeOnDevice();
 		InputBatch ring[3] = {InputBatch(B, n), InputBatch(B, n), InputBatch(B, n)};
-		if (mode == 0) expect("batches built after cnet_init are page-locked", ring[0].isPinned());
+		if (slot == 0) expect("batches built after cnet_init are page-locked", ring[0].isPinned());
 		if (graphs) net.useGraphs(true);
 		if (mode == 5) net.conjugateGradients(false);
 		if (mode == 8) net.setInputTrainable(cin, false);
@@ -976,7 +981,7 @@ static void test_pipeline(int B, int steps) {
 				// which is the buffer of the ring that is refilled next)
 				CNet::PendingLoss now = net.gpuQueueLoss(cen);
 				if (s + 1 < steps && !early) net.gpuPrefetch(cin, ring[(s + 1) % 3]);
-				if (s > 0) losses[mode].push_back(net.getLoss(pending, &ring[(s + 2) % 3]));
+				if (s > 0) losses[slot].push_back(net.getLoss(pending, &ring[(s + 2) % 3]));
 				if (s + 2 < steps) reader.nextBatch(ring[(s + 2) % 3]);
 				pending = now;
 				continue;
@@ -985,17 +990,18 @@ static void test_pipeline(int B, int steps) {
 				if (s + 1 < steps) net.gpuPrefetch(cin, ring[(s + 1) % 3]);
 				if (s + 2 < steps) reader.nextBatch(ring[(s + 2) % 3]);
 			}
-			losses[mode].push_back(net.getLoss(cen, &cur));
+			losses[slot].push_back(net.getLoss(cen, &cur));
 		}
-		if (late_loss) losses[mode].push_back(net.getLoss(pending, NULL));
+		if (late_loss) losses[slot].push_back(net.getLoss(pending, NULL));
 		net.sync();
-		ms[mode] = 1e3 * std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / steps;
+		ms[slot] = 1e3 * std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / steps;
 		net.getInputsFromGpu();
 		for (auto f : net.inputs()) {
 			if (f == cin) continue;
-			weights[mode].insert(weights[mode].end(), f->input().real_, f->input().real_ + 2 * f->input().length_);
+			weights[slot].insert(weights[slot].end(), f->input().real_, f->input().real_ + 2 * f->input().length_);
 		}
-		if (mode == 1) {
+		if (slot == 14) expect("a batch of a stored reader names its samples", ring[0].isResident());
+		if (slot == 1) {
 			// error behaviour of the staging
 			InputBatch a(B, n), b(B, n);
 			reader.nextBatch(a);
@@ -1040,6 +1046,9 @@ static void test_pipeline(int B, int steps) {
 		expect("losses and weights identical with the gradients of the input functions gathered at once", losses[0] == losses[10] && weights[0] == weights[10]);
 		expect("losses and weights identical with the losses copied from a device buffer", losses[0] == losses[11] && weights[0] == weights[11]);
 		expect("losses and weights identical with the losses copied from a device buffer, read one step late", losses[0] == losses[12] && weights[0] == weights[12]);
+		expect("losses and weights identical with the samples stored on the device, copied in the forward pass", losses[0] == losses[13] && weights[0] == weights[13]);
+		expect("losses and weights identical with the samples stored on the device, staged ahead, losses read late", losses[0] == losses[14] && weights[0] == weights[14]);
+		expect("losses and weights identical with the samples stored on the device and gpuTrainStep", losses[0] == losses[15] && weights[0] == weights[15]);
 		expect("training moved the loss", losses[0].front() != losses[0].back() && std::isfinite(losses[0].back()));
 		// dz* planes written as the conjugate of the dz product against dz* planes computed by a product of their own
 		double worst = 0, num = 0, den = 0;

@@ -14,7 +14,7 @@ def generate(header_path, out_path):
     decls = re.findall(r'\n((?:int|void \*|const char \*)\s*cnet_\w+\s*\([^;]*?\));', text)
     special = {'cnet_graph_end', 'cnet_graph_launch', 'cnet_graph_destroy', 'cnet_graph_begin', 'cnet_alloc', 'cnet_host_alloc',
                'cnet_free', 'cnet_host_free', 'cnet_memcpy_h2d', 'cnet_memcpy_d2h', 'cnet_memcpy_d2d', 'cnet_memcpy_h2d_async',
-               'cnet_memcpy_d2h_async', 'cnet_upload_async', 'cnet_upload_zero', 'cnet_upload_pair', 'cnet_memset_zero', 'cnet_last_error', 'cnet_stream',
+               'cnet_memcpy_d2h_async', 'cnet_upload_async', 'cnet_upload_zero', 'cnet_upload_pair', 'cnet_upload_gather_rows', 'cnet_memset_zero', 'cnet_last_error', 'cnet_stream',
                'cnet_get_device_info'}
     out = ['#include "cnet_hip.h"\n#include <cstdio>\n#include <cstdlib>\n#include <cstring>\n#include <set>\nextern "C" {\n']
     seen = set()
@@ -43,6 +43,16 @@ int cnet_memcpy_d2h_async(void *d, const void *s, size_t b) { memcpy(d, s, b); r
 int cnet_upload_async(void *d, const void *s, size_t b) { memcpy(d, s, b); return 0; }
 int cnet_upload_zero(void *d, size_t b) { memset(d, 0, b); return 0; }
 int cnet_upload_pair(void *d0, const void *s0, size_t b0, void *d1, const void *s1, size_t b1) { if (b0) memcpy(d0, s0, b0); if (b1) memcpy(d1, s1, b1); return 0; }
+int cnet_upload_gather_rows(float *d, int64_t ldd, int64_t dps, const float *s, int64_t lds, int64_t sps, int planes, int src_rows,
+		const int32_t *idx, int32_t *dl, const int32_t *sl, int rows, int cols) {
+	for (int p = 0; p < planes; ++p)
+		for (int r = 0; r < rows; ++r) {
+			if (idx[r] < 0 || idx[r] >= src_rows) { fprintf(stderr, "stub: gather index outside the table\\n"); abort(); }
+			memcpy(d + p * dps + (int64_t) r * ldd, s + p * sps + (int64_t) idx[r] * lds, cols * sizeof(float));
+		}
+	if (dl) for (int r = 0; r < rows; ++r) dl[r] = sl[idx[r]];
+	return 0;
+}
 int cnet_memset_zero(void *d, size_t b) { memset(d, 0, b); return 0; }
 const char *cnet_last_error(void) { return "stub"; }
 void *cnet_stream(void) { return 0; }

@@ -385,3 +385,49 @@ def test_device_copy_caller_stream_and_upload_ordering(gpu, port):
     capi.call("cnet_graph_end", None)
     del pinned
     capi.call("cnet_host_free", host)
+
+
+def test_rows_of_a_table_on_the_device_into_a_batch_buffer(gpu):
+    """cnet_upload_gather_rows: rows and labels named by indices in page-locked memory, one and two planes, aligned and odd
+    widths, a window of a wider buffer; indices outside the table, in pageable memory, or a label array without its twin are
+    refused with an error code."""
+    import ctypes as C
+    lib = capi.load()
+    rs = np.random.RandomState(3)
+    for count, dim, rows, planes, pad in [(50, 784, 64, 1, 0), (37, 33, 8, 2, 3), (4, 4, 1, 2, 0), (300, 128, 4096, 2, 4)]:
+        table = rs.randn(planes, count, dim).astype(np.float32)
+        labels = rs.randint(0, 10, count).astype(np.int32)
+        d_table, d_labels = capi.to_device(table), capi.to_device(labels)
+        ld = dim + pad
+        d_out = capi.to_device(np.full((planes, rows, ld), -7.0, np.float32))
+        d_lab = capi.to_device(np.full(rows, -1, np.int32))
+        hp = C.c_void_p()
+        capi.call("cnet_host_alloc", rows * 4, C.byref(hp))
+        idx = np.ctypeslib.as_array(C.cast(hp, C.POINTER(C.c_int32)), shape=(rows,))
+        idx[:] = rs.randint(0, count, rows)
+        capi.call("cnet_upload_wait_compute")   # the fills above ran on the compute stream
+        capi.call("cnet_upload_gather_rows", d_out.ptr, ld, rows * ld, d_table.ptr, dim, count * dim, planes, count, hp, d_lab.ptr,
+                  d_labels.ptr, rows, dim)
+        capi.call("cnet_upload_sync")
+        out = d_out.download()
+        assert np.array_equal(out[:, :, :dim], table[:, idx, :])
+        assert (out[:, :, dim:] == -7.0).all()
+        assert np.array_equal(d_lab.download(), labels[idx])
+        # samples only
+        capi.call("cnet_upload_gather_rows", d_out.ptr, ld, rows * ld, d_table.ptr, dim, count * dim, 1, count, hp, None, None, rows, dim)
+        capi.call("cnet_upload_sync")
+        # refused: an index outside the table, a lone label array, indices in pageable memory
+        keep = int(idx[0])
+        idx[0] = count
+        assert lib.cnet_upload_gather_rows(d_out.ptr, ld, rows * ld, d_table.ptr, dim, count * dim, planes, count, hp, d_lab.ptr, d_labels.ptr, rows, dim) == -2
+        idx[0] = -1
+        assert lib.cnet_upload_gather_rows(d_out.ptr, ld, rows * ld, d_table.ptr, dim, count * dim, planes, count, hp, d_lab.ptr, d_labels.ptr, rows, dim) == -2
+        idx[0] = keep
+        assert lib.cnet_upload_gather_rows(d_out.ptr, ld, rows * ld, d_table.ptr, dim, count * dim, planes, count, hp, d_lab.ptr, None, rows, dim) == -2
+        pageable = np.zeros(rows, np.int32)
+        assert lib.cnet_upload_gather_rows(d_out.ptr, ld, rows * ld, d_table.ptr, dim, count * dim, planes, count, pageable.ctypes.data, d_lab.ptr,
+                                           d_labels.ptr, rows, dim) == -2
+        assert lib.cnet_upload_gather_rows(d_out.ptr, dim - 1, rows * ld, d_table.ptr, dim, count * dim, planes, count, hp, d_lab.ptr, d_labels.ptr, rows, dim) == -2
+        assert "cnet_upload_gather_rows" in _msg()
+        capi.call("cnet_upload_sync")
+        capi.call("cnet_host_free", hp)
