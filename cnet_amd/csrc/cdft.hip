@@ -10,6 +10,8 @@
 
 namespace cnet {
 
+int cgemm_real_a(int M, int N, int K, const float *a_re, const float *a_im, long lda, const float *b_re, const float *b_im, long ldb, float *c_re,
+		float *c_im, long ldc);
 int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
 		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
 		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri, int mirror);
@@ -190,10 +192,7 @@ int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, 
 	// (rounded up to a multiple of four columns, which keeps the product on the kernels with 128-bit loads; the few
 	// extra columns are correct values that the mirror pass writes again)
 	const int cols = std::min(n, (n / 2 + 1 + 3) / 4 * 4);
-	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {t.re, t.re}, *bi[2] = {t.im, t.im};
-	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
-	bool cj[2] = {false, false};
-	rc = cgemm_pair(false, true, 1, B, cols, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, 0, 0, 0);
+	rc = cgemm_real_a(B, cols, n, x_re, x_im, ldx, t.re, t.im, t.ld, y_re, y_im, ldy);  // x_im is not read by the block kernels
 	if (rc) return rc;
 	const int half = (n - 1) / 2;  // columns 1 .. half have a partner n - q of their own
 	if (half > 0) {

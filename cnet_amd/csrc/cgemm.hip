@@ -75,6 +75,10 @@ struct CgemmArgs {
 	// mirror == 2 (MIRROR_GELU): the C planes of p[1] receive the CGelu of the final value of C instead (a Linear followed by
 	// a CGelu in one launch: the pre-activation and the activation are both written, neither is read back); always assigned.
 	int mirror;
+	// The imaginary plane of A holds nothing but +0 (the caller vouches: real samples in front of a transform) and is not read:
+	// two real products per complex one, re = Ar Br, im = +-Ar Bi, the bits of the four products on such an A.  Honoured by the
+	// block kernels for a row-major A against a k-major B (the layout of the transform); ignored elsewhere.
+	int a_real = 0;
 };
 constexpr int MIRROR_CONJ = 1, MIRROR_GELU = 2;
 
@@ -429,7 +433,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 // Operand fragments of one wavefront: T tiles of 32 rows, both planes.
 //   MCONTIG ([k][row] in LDS): one float per tile, plane and k step, double buffered per step.
 //   otherwise ([row][k] swizzled): one float4 per tile, plane and half chunk (set 0: steps 0..3, set 1: steps 4..7).
-template <int T, bool MCONTIG, int PITCH, int PLANE>
+template <int T, bool MCONTIG, int PITCH, int PLANE, bool REAL = false>
 struct Frag {
 	float s_re[2][T], s_im[2][T];
 	float4 q_re[2][T], q_im[2][T];
@@ -457,7 +461,7 @@ struct Frag {
 #pragma unroll
 			for (int i = 0; i < T; ++i) {
 				s_re[s & 1][i] = row_base[i][stage_off + line];
-				s_im[s & 1][i] = row_base[i][stage_off + PLANE + line];
+				if (!REAL) s_im[s & 1][i] = row_base[i][stage_off + PLANE + line];
 			}
 		}
 	}
@@ -468,13 +472,13 @@ struct Frag {
 #pragma unroll
 			for (int i = 0; i < T; ++i) {
 				q_re[set][i] = *reinterpret_cast<const float4 *>(b + i * 32 * KC);
-				q_im[set][i] = *reinterpret_cast<const float4 *>(b + PLANE + i * 32 * KC);
+				if (!REAL) q_im[set][i] = *reinterpret_cast<const float4 *>(b + PLANE + i * 32 * KC);
 			}
 		}
 	}
 	static __device__ __forceinline__ float comp(const float4 &v, int c) { return c == 0 ? v.x : (c == 1 ? v.y : (c == 2 ? v.z : v.w)); }
 	__device__ __forceinline__ float re(int s, int i) const { return MCONTIG ? s_re[s & 1][i] : comp(q_re[s >> 2][i], s & 3); }
-	__device__ __forceinline__ float im(int s, int i) const { return MCONTIG ? s_im[s & 1][i] : comp(q_im[s >> 2][i], s & 3); }
+	__device__ __forceinline__ float im(int s, int i) const { return REAL ? 0.f : (MCONTIG ? s_im[s & 1][i] : comp(q_im[s >> 2][i], s & 3)); }
 };
 
 // One operand (both planes) of one K chunk, loaded straight into LDS.  A unit is one wave-wide instruction: lane l
@@ -522,6 +526,14 @@ struct DlStage {
 		asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(goff[u]), "s"(tile_im), "s"(lim) : "memory", "m0");
 #endif
 	}
+	// the real plane only (an operand whose imaginary plane is not read)
+	__device__ __forceinline__ void issue_re(int u, const float *tile_re, float *sre) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+		const unsigned dst = (unsigned) ((u * 4 + wave_s) * 1024);
+		const unsigned lre = (unsigned) (size_t) sre + dst;
+		asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(goff[u]), "s"(tile_re), "s"(lre) : "memory", "m0");
+#endif
+	}
 };
 
 // Signs (conj) are applied to the fragments.  NST stages of LDS: chunk c + NST - 1 is requested while chunk c is
@@ -533,9 +545,11 @@ struct DlStage {
 // sa, sb the signs of the imaginary parts: re = P - sa sb Q, im = T - P - sa sb Q).  A quarter of the matrix work less,
 // for one addition per operand fragment and k pair; the imaginary part then carries the rounding of all three products
 // (normwise as accurate as four products, not componentwise).
-template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int NST, bool GAUSS = false>
+// A_REAL: the imaginary plane of A is all +0 and is neither fetched nor multiplied (CgemmArgs::a_real): two real products.
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int NST, bool GAUSS = false, bool A_REAL = false>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))) void cgemm_fast_kernel(const CgemmArgs args) {
 	static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per workgroup");
+	static_assert(!(GAUSS && A_REAL), "a real operand leaves two products: nothing for the three-product form to save");
 	constexpr int TM = WM / 32, TN = WN / 32;
 	typedef DlStage<BM, A_MCONTIG> StageA;
 	typedef DlStage<BN, B_NCONTIG> StageB;
@@ -571,7 +585,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	// S = Ai Br) and combines them with their signs when it stores, so its K loop has no vector-ALU instruction for signs at
 	// all; with four tiles there are only registers for two sets, re = P -+ Q and im = +-R +- S, and one operand of the
 	// second product is negated per k pair (see the modes below).
-	constexpr bool ACC4 = TM * TN <= 2;
+	constexpr bool ACC4 = TM * TN <= 2 && !A_REAL;
 	constexpr bool ACC_Q = ACC4 || GAUSS, ACC_S = ACC4 && !GAUSS;
 	floatx16 acc_re[TM][TN], acc_im[TM][TN], acc_q[ACC_Q ? TM : 1][ACC_Q ? TN : 1], acc_s[ACC_S ? TM : 1][ACC_S ? TN : 1];
 	for (int pass = 0; pass < npass; ++pass) {
@@ -634,8 +648,12 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	// all units of one chunk of both operands into the stage at `stage`
 	auto issue_chunk = [&](int chunk, float *stage) {
 #pragma unroll
-		for (int u = 0; u < UA; ++u)
-			sa.issue(u, pb.a_re + a_tile0 + chunk * a_step, pb.a_im + a_tile0 + chunk * a_step, stage, stage + A_PLANE);
+		for (int u = 0; u < UA; ++u) {
+			if (A_REAL)
+				sa.issue_re(u, pb.a_re + a_tile0 + chunk * a_step, stage);
+			else
+				sa.issue(u, pb.a_re + a_tile0 + chunk * a_step, pb.a_im + a_tile0 + chunk * a_step, stage, stage + A_PLANE);
+		}
 #pragma unroll
 		for (int u = 0; u < UB; ++u)
 			sb.issue(u, pb.b_re + b_tile0 + chunk * b_step, pb.b_im + b_tile0 + chunk * b_step, stage + 2 * A_PLANE,
@@ -651,7 +669,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	const int mode = (pb.a_im_sign < 0.f ? 2 : 0) | (pb.b_im_sign < 0.f ? 1 : 0);
 	const float sign_a = pb.a_im_sign < 0.f ? -1.f : 1.f, sign_b = pb.b_im_sign < 0.f ? -1.f : 1.f;  // uniform: scalar registers
 
-	constexpr int LOADS_PER_CHUNK = 2 * (UA + UB);  // transfers one wavefront issues per chunk
+	constexpr int LOADS_PER_CHUNK = (A_REAL ? 1 : 2) * UA + 2 * UB;  // transfers one wavefront issues per chunk
 	static_assert(NST == 2 || NST == 3, "two or three stages");
 	static_assert(LOADS_PER_CHUNK < 16, "fits the low bits of the vmcnt field");
 #pragma unroll
@@ -660,7 +678,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	__builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the tiles have landed in LDS
 	__syncthreads();
 
-	Frag<TM, A_MCONTIG, StageA::PITCH, A_PLANE> fa;
+	Frag<TM, A_MCONTIG, StageA::PITCH, A_PLANE, A_REAL> fa;
 	Frag<TN, B_NCONTIG, StageB::PITCH, B_PLANE> fb;
 	fa.init(smem, wm0, r, h);
 	fb.init(smem + 2 * A_PLANE, wn0, r, h);
@@ -704,14 +722,22 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			for (int i = 0; i < TM; ++i) {
 				are[i] = fa.re(ks, i);
 				aim[i] = fa.im(ks, i);
-				if (!ACC4 && !GAUSS) neg[i] = MODE == 1 ? -are[i] : -aim[i];
+				if (!ACC4 && !GAUSS && !A_REAL) neg[i] = MODE == 1 ? -are[i] : -aim[i];
 			}
 #pragma unroll
 			for (int j = 0; j < TN; ++j) {
 				bre[j] = fb.re(ks, j);
 				bim[j] = fb.im(ks, j);
 			}
-			if constexpr (GAUSS) {
+			if constexpr (A_REAL) {
+#pragma unroll
+				for (int i = 0; i < TM; ++i)
+#pragma unroll
+					for (int j = 0; j < TN; ++j) {
+						acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bre[j], acc_re[i][j], 0, 0, 0);
+						acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bim[j], acc_im[i][j], 0, 0, 0);
+					}
+			} else if constexpr (GAUSS) {
 				float asum[TM], bsum[TN];
 #pragma unroll
 				for (int i = 0; i < TM; ++i) asum[i] = fmaf(sign_a, aim[i], are[i]);
@@ -760,7 +786,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				// scheduling recipe for this k pair: after each MFMA let a few of the pending VALU / LDS / global
 				// instructions issue, so they run in the shadow of the matrix pipe
 #pragma unroll
-				for (int q = 0; q < (GAUSS ? 3 : 4) * TM * TN; ++q) {
+				for (int q = 0; q < (A_REAL ? 2 : GAUSS ? 3 : 4) * TM * TN; ++q) {
 					__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
 					__builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // <= 2 VALU
 					__builtin_amdgcn_sched_group_barrier(0x080, 1, 0);  // <= 1 LDS
@@ -791,7 +817,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			if (c + 1 < c_hi) chunk(1, mode_c, c + 1);
 		}
 	};
-	if constexpr (ACC4 || GAUSS) {
+	if constexpr (ACC4 || GAUSS || A_REAL) {
 		kloop(std::integral_constant<int, 0>());  // the signs wait for the store
 	} else {
 		switch (mode) {
@@ -820,7 +846,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				if (row < args.M) {
 					const long off = (long) (row - row_org) * ldc + (col - col_org);
 					float vr, vi;
-					if constexpr (GAUSS) {
+					if constexpr (A_REAL) {
+						vr = acc_re[i][j][e];
+						vi = r_minus ? -acc_im[i][j][e] : acc_im[i][j][e];
+					} else if constexpr (GAUSS) {
 						const float p = acc_re[i][j][e], q = q_minus ? acc_q[i][j][e] : -acc_q[i][j][e];  // q_minus: sa sb = +1
 						vr = p - q;
 						vi = (acc_im[i][j][e] - p) - q;
@@ -1322,6 +1351,20 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 		if (fast_ok) {  // any M and N: edge blocks re-read the last valid rows and store only what is inside C
 			constexpr int NST = (BM == 128 && BN == 128) ? 2 : 3;
 			constexpr size_t fast_smem = (size_t) NST * 2 * KC * (BM + BN) * sizeof(float);
+			if constexpr (!A_MCONTIG && B_NCONTIG) {
+				if (args.a_real) {
+					static bool real_attr_set = false;
+					if (!real_attr_set) {
+						CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, true>),
+								hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem));
+						real_attr_set = true;
+					}
+					hipLaunchKernelGGL((cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, true>), grid, dim3(NTHREADS), fast_smem,
+							cnet::rt().stream, args);
+					CNET_LAUNCH_CHECK();
+					return finish();
+				}
+			}
 			// Three accumulator sets of four tiles (192 registers) leave too few for the fragments of two k-contiguous
 			// operands (float4 each): that one layout of the 128 x 128 block spills and keeps four products.
 			if constexpr ((WM / 32) * (WN / 32) <= 2 || A_MCONTIG || B_NCONTIG) {
@@ -1431,7 +1474,8 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_opera
 		const long nb = blocks(shapes[k].bm, shapes[k].bn);
 		const long per_unit = (nb + cus - 1) / cus;
 		// three real products per complex one in the shapes that have the registers for it (fast kernel only: K in whole chunks)
-		const double work = (three_products() && a.K % KC == 0 && !(k == 0 && k_contig_operands)) ? 6.0 : 8.0;
+		// an A without imaginary parts: two real products (fast kernel only: K in whole chunks)
+		const double work = (a.a_real && a.K % KC == 0) ? 4.0 : (three_products() && a.K % KC == 0 && !(k == 0 && k_contig_operands)) ? 6.0 : 8.0;
 		const double block_us = work * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
 		// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
 		const double bonus = 1.0 - 0.000001 * shapes[k].bm * shapes[k].bn;
@@ -1510,6 +1554,7 @@ namespace cnet {
 static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int nprob, int batch) {
 	if (a.M <= 0 || a.N <= 0) return CNET_OK;
 	if (a.K <= 0) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: K must be positive");
+	if (a_mcontig || !b_ncontig) a.a_real = 0;  // only that layout has the kernels (the imaginary plane holds zeros: reading it is right too)
 	int rc = CNET_OK;
 	if (try_skinny(a_mcontig, b_ncontig, a, nprob, batch, &rc)) return rc;
 	// A C that is a few columns wider than a multiple of the block width (784 = 12 x 64 + 16) costs a whole extra column
@@ -1604,6 +1649,17 @@ int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, c
 	if (mirror && nprob != 1) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: a mirrored product is one problem");
 	CgemmArgs a = pair_args(nprob, M, N, K, a_re, a_im, lda, b_re, b_im, ldb, conj_b, c_re, c_im, ldc, accumulate, tri, mirror);
 	return cgemm_dispatch(a_mcontig, b_ncontig, a, nprob, 1);
+}
+
+// One product whose A (row-major) has an imaginary plane of nothing but +0, against a k-major B (used by cdft.hip)
+int cgemm_real_a(int M, int N, int K, const float *a_re, const float *a_im, long lda, const float *b_re, const float *b_im, long ldb, float *c_re,
+		float *c_im, long ldc) {
+	const float *ar[2] = {a_re, a_re}, *ai[2] = {a_im, a_im}, *br[2] = {b_re, b_re}, *bi[2] = {b_im, b_im};
+	float *cr[2] = {c_re, c_re}, *ci[2] = {c_im, c_im};
+	const bool cj[2] = {false, false};
+	CgemmArgs a = pair_args(1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, 0, 0, 0);
+	a.a_real = 1;
+	return cgemm_dispatch(false, true, a, 1, 1);
 }
 
 static CgemmArgs pair_args(int nprob, int M, int N, int K, const float *const a_re[2], const float *const a_im[2], long lda,
