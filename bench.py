@@ -170,8 +170,10 @@ def kernel_suite(steps):
     mfma("cdft_fwd", [Bf, nf], 8.0 * Bf * nf * nf, lambda: ops.dft_fwd(x, y))
     mfma("cdft_bwd", [Bf, nf], 16.0 * Bf * nf * nf, lambda: ops.dft_bwd(g, dx))
     xr = ops.CMat.from_host(rs.randn(Bf, nf).astype(np.float32), np.zeros((Bf, nf), np.float32))
-    mfma("cdft_fwd of real samples (columns 0..n/2 by the product, the rest as conjugates; flops of the product executed)", [Bf, nf],
-         8.0 * Bf * nf * (nf // 2 + 4), lambda: ops.dft_fwd_real_input(xr, y))
+    # a quarter of the full transform's flops: columns 0..n/2 only, and two real products per complex one (the imaginary
+    # plane of the samples is neither read nor multiplied)
+    mfma("cdft_fwd of real samples (columns 0..n/2 by the product, the rest as conjugates; two real products per complex one; flops executed)",
+         [Bf, nf], 4.0 * Bf * nf * (nf // 2 + 4), lambda: ops.dft_fwd_real_input(xr, y))
     del xr
     # TriangFourier: only the pairs in <= out contribute, n (n + 1) / 2 complex multiply-adds per row
     tri = nf * (nf + 1) / 2.0

@@ -1441,10 +1441,12 @@ private:
 	bool realInputNow(CFunc *f) const {
 		if (!real_transforms_ || f->typeId() != isFourier) return false;
 		CFunc *p = f->slots_[0].producer;
-		// Half the product is saved and one short launch (the conjugate columns) added: it pays from about 15 us of
-		// product on (batch 64 x 784: 10 us either way and a launch more; batch 4096: 146 -> 95 + 7 us).
+		// Three quarters of the product are saved (half of the columns, and of the rest the two real products with the
+		// imaginary plane) and one short launch (the conjugate columns) added: it pays once the product runs on the block
+		// kernels (784 long: 10.7 against 13.2 us at batch 128, 22 against 34 at 512, 60 against 147 at 4096; at batch 64 both
+		// take the small-C kernel, 10 us either way and a launch more).
 		const double n = f->out_size_;
-		return p && p->typeId() == isInput && p->z_imag_zero_ && p->rows_ == f->rows_ && f->rows_ * n * n >= 3e8;
+		return p && p->typeId() == isInput && p->z_imag_zero_ && p->rows_ == f->rows_ && f->rows_ * n * n >= 7.5e7;
 	}
 	bool anyRealTransformNow() const {
 		for (auto f : func_list_)
