@@ -618,6 +618,7 @@ public:
 	int typeId() const override { return ::isInput; }
 	void setInput(InputBatch &batch, int b) {
 		assert(batch.sampleDim() == input().length_);
+		if (batch.isResident()) throw std::logic_error("CInput::setInput: the samples of this batch are on the device, not in the batch");
 		std::copy(batch.realDataPtr(b), batch.realDataPtr(b) + input().length_, mutable_input()->real_);
 		std::copy(batch.imagDataPtr(b), batch.imagDataPtr(b) + input().length_, mutable_input()->imag_);
 	}
@@ -2098,6 +2099,8 @@ public:
 		requireAllocated("gpuSetInput");
 		if (cin->rows_ != batch_ || batch.size() != batch_ || batch.sampleDim() != cin->input().length_)
 			throw std::invalid_argument("gpuSetInput: " + cin->getName() + " is not a data input of this batch shape");
+		if (batch.isResident())
+			throw std::invalid_argument("gpuSetInput: a batch that names samples of a data set on the device feeds the main data input only (gpuForward / gpuPrefetch)");
 		beforeFeed(cin);
 		CFunc::Slot &s = cin->slots_[0];
 		const size_t plane = (size_t) batch_ * s.len * sizeof(float);

@@ -1495,6 +1495,41 @@ static void test_errors() {
 	expect("token id outside the table throws", throws<std::out_of_range>([&] {
 		net4.gpuForward((CEmbedding *) net4[emb], (L2Out *) net4[out4], ids);
 	}));
+	{  // batches that name samples of a data set on the device
+		const float re[3 * 8] = {1, 2, 3}, im[3 * 8] = {0};
+		const int labels[3] = {0, 1, 2};
+		DeviceDataset ds(re, im, labels, 3, 8);
+		expect("a data set whose imaginary parts are all +0 keeps the real plane only", ds.imagIsZero() && ds.size() == 3 && ds.label(2) == 2);
+		InputBatch rb(4, 8);
+		const int pick[4] = {2, 0, 1, 2}, bad[1] = {3};
+		expect("a sample index outside the data set throws", throws<std::out_of_range>([&] { rb.gatherResident(ds, bad, 1); }));
+		rb.clear();
+		rb.gatherResident(ds, pick, 4);
+		expect("labels of a resident batch come from the data set", rb.isResident() && rb.noOfLabels() == 4 && rb.label(0) == 2 && rb.label(1) == 0);
+		InputBatch part(4, 8);
+		part.gatherResident(ds, pick, 2);
+		expect("add() into a resident batch throws", throws<std::logic_error>([&] { part.add({{1.f, 0.f}}, 0); }));
+		InputBatch other(4, 7);
+		expect("a data set of another sample length throws", throws<std::invalid_argument>([&] { other.gatherResident(ds, pick, 4); }));
+		CNet net5;
+		auto x5 = net5.add(new CInput(OutSize(8)));
+		CInput *t5 = new CInput(OutSize(8));
+		t5->setIsBatched(true);
+		auto tt5 = net5.add(t5);
+		auto r5 = net5.add(new Residual(InSize(8)), {x5, tt5});
+		auto o5 = net5.add(new L2Out(InSize(8)), {r5});
+		net5.allocateOnGpu(4);
+		expect("a resident batch for a second data input is refused", throws<std::invalid_argument>([&] { net5.gpuSetInput(t5, rb); }));
+		InputBatch tb(4, 8);
+		for (int b = 0; b < 4; ++b) tb.add({{0.5f, 0.f}}, 0);
+		net5.gpuSetInput(t5, tb);
+		net5.gpuForward((CInput *) net5[x5], (L2Out *) net5[o5], rb);  // rows 2, 0, 1, 2 of the data set
+		net5.getLoss((L2Out *) net5[o5], &rb);
+		// |x + t|^2 summed, t = (0.5, 0, ...): row 0 of the set is (1, 2, 3, 0, ...), the other rows are zeros
+		const float row0 = 1.5f * 1.5f + 2.f * 2.f + 3.f * 3.f, rest = 0.5f * 0.5f;
+		expect("the forward pass saw the rows that the indices name", std::fabs(rb.loss(1) - row0) < 1e-5f && std::fabs(rb.loss(0) - rest) < 1e-6f && std::fabs(rb.loss(3) - rest) < 1e-6f);
+		net5.sync();
+	}
 	// device layer status codes
 	expect("invalid argument gives a status, not an exit", cnet_cgemm(0, 0, 0, 4, 4, 0, NULL, NULL, 0, NULL, NULL, 0, NULL, NULL, 0, 0) == CNET_ERR_INVALID_ARGUMENT);
 	expect("error text names the call", std::string(cnet_last_error()).find("cnet_cgemm") != std::string::npos);
