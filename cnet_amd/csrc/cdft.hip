@@ -11,7 +11,7 @@
 namespace cnet {
 
 int cgemm_real_a(int M, int N, int K, const float *a_re, const float *a_im, long lda, const float *b_re, const float *b_im, long ldb, float *c_re,
-		float *c_im, long ldc);
+		float *c_im, long ldc, int herm_n);
 int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],
 		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
 		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri, int mirror);
@@ -51,19 +51,6 @@ __global__ void twiddle_kernel(float *__restrict__ fre, float *__restrict__ fim,
 	const double scale = (upper_only && p > q) ? 0.0 : 1.0 / sqrt((double) n);
 	fre[(long) p * ld + q] = (float) (c * scale);
 	fim[(long) p * ld + q] = (float) (s * scale);
-}
-
-// The transform of real samples is conjugate-symmetric, y[n - q] = conj(y[q]): the columns beyond n/2 are written from
-// the ones below it.  One thread per (row, q), q = 1 .. half.
-__global__ __launch_bounds__(256) void hermitian_mirror_kernel(float *__restrict__ y_re, float *__restrict__ y_im, long ldy, int rows, int n,
-		int half) {
-	const long idx = (long) blockIdx.x * 256 + threadIdx.x;
-	if (idx >= (long) rows * half) return;
-	const long row = idx / half;
-	const int q = (int) (idx - row * half) + 1;
-	const long src = row * ldy + q, dst = row * ldy + (n - q);
-	y_re[dst] = y_re[src];
-	y_im[dst] = -y_im[src];
 }
 
 static int get_plan(int n, Twiddle *out, bool create) {
@@ -188,20 +175,12 @@ int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, 
 	if (rc) return rc;
 	// a caller-supplied forward operator need not be symmetric under q -> n - q: the whole product then
 	if (t.fwd_re) return cnet_cdft_fwd(x_re, x_im, ldx, y_re, y_im, ldy, B, n, 0);
-	// columns 0 .. n/2 by the matrix product (x_im is read and holds zeros), the others as conjugates of those
-	// (rounded up to a multiple of four columns, which keeps the product on the kernels with 128-bit loads; the few
-	// extra columns are correct values that the mirror pass writes again)
+	// Columns 0 .. n/2 by the matrix product, rounded up to a multiple of four columns, which keeps the product on the
+	// kernels with 128-bit loads (x_im holds zeros: the block kernels do not read it, the others do).  Columns cols .. n - 1
+	// are the partners n - q of columns 1 .. n - cols (cols > n / 2: each of those has its partner outside the product): the
+	// product writes them, conjugated, as it stores their partners.
 	const int cols = std::min(n, (n / 2 + 1 + 3) / 4 * 4);
-	rc = cgemm_real_a(B, cols, n, x_re, x_im, ldx, t.re, t.im, t.ld, y_re, y_im, ldy);  // x_im is not read by the block kernels
-	if (rc) return rc;
-	const int half = (n - 1) / 2;  // columns 1 .. half have a partner n - q of their own
-	if (half > 0) {
-		const long total = (long) B * half;
-		hipLaunchKernelGGL(hermitian_mirror_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, rt().stream, y_re, y_im, (long) ldy, B, n,
-				half);
-		CNET_LAUNCH_CHECK();
-	}
-	return CNET_OK;
+	return cgemm_real_a(B, cols, n, x_re, x_im, ldx, t.re, t.im, t.ld, y_re, y_im, ldy, n);
 }
 
 int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,

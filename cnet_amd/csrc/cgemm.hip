@@ -79,8 +79,12 @@ struct CgemmArgs {
 	// two real products per complex one, re = Ar Br, im = +-Ar Bi, the bits of the four products on such an A.  Honoured by the
 	// block kernels for a row-major A against a k-major B (the layout of the transform); ignored elsewhere.
 	int a_real = 0;
+	// mirror == 3 (MIRROR_HERM): element (row, col) with herm_lo <= col <= herm_hi also goes, conjugated, to column herm_n - col
+	// of the same row of C (honouring `accumulate`): the transform of real samples computes columns 0 .. n/2 and fills the others
+	// as it stores those.  One problem; the columns written this way must lie outside the product's own.
+	int herm_n = 0, herm_lo = 1, herm_hi = 0;
 };
-constexpr int MIRROR_CONJ = 1, MIRROR_GELU = 2;
+constexpr int MIRROR_CONJ = 1, MIRROR_GELU = 2, MIRROR_HERM = 3;
 
 // the conjugate of (vr, vi) into element `off` of the mirror planes
 __device__ __forceinline__ void mirror_store(const CgemmArgs &args, long off, float vr, float vi) {
@@ -92,6 +96,18 @@ __device__ __forceinline__ void mirror_store(const CgemmArgs &args, long off, fl
 	}
 	args.p[1].c_re[off] = mr;
 	args.p[1].c_im[off] = mi;
+}
+
+// one plane (part 0: real, 1: imaginary) of the product's value at (row, col) to the Hermitian partner of that element
+__device__ __forceinline__ void herm_store_part(const CgemmArgs &args, int part, int row, int col, float v) {
+	if (args.mirror != MIRROR_HERM || col < args.herm_lo || col > args.herm_hi) return;
+	float *m = (part ? args.p[0].c_im : args.p[0].c_re) + (long) row * args.ldc + (args.herm_n - col);
+	const float mv = part ? -v : v;
+	*m = args.accumulate ? *m + mv : mv;
+}
+__device__ __forceinline__ void herm_store(const CgemmArgs &args, int row, int col, float vr, float vi) {
+	herm_store_part(args, 0, row, col, vr);
+	herm_store_part(args, 1, row, col, vi);
 }
 
 // the CGelu of the final value (vr, vi) of element `off` into the planes of p[1]
@@ -392,7 +408,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void cgemm_kernel(const CgemmArgs args
 				if (row < M) {
 					const long off = (long) row * ldc + col;
 					float vr = acc_re[i][j][e], vi = acc_im[i][j][e];
-					if (args.mirror && args.splits == 1) mirror_store(args, (long) row * args.ldc + col, vr, vi);
+					if (args.mirror && args.splits == 1) {
+						mirror_store(args, (long) row * args.ldc + col, vr, vi);
+						herm_store(args, row, col, vr, vi);
+					}
 					if (accumulate) {
 						vr += pb.c_re[off];
 						vi += pb.c_im[off];
@@ -861,7 +880,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 						vr = acc_re[i][j][e];
 						vi = mode == 3 ? -acc_im[i][j][e] : acc_im[i][j][e];
 					}
-					if (mirror_now) mirror_store(args, (long) row * args.ldc + col, vr, vi);
+					if (mirror_now) {
+						mirror_store(args, (long) row * args.ldc + col, vr, vi);
+						herm_store(args, row, col, vr, vi);
+					}
 					if (accumulate) {
 						vr += pb.c_re[off];
 						vi += pb.c_im[off];
@@ -889,6 +911,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(CgemmArgs args, int 
 	float *c = (part ? args.p[prob].c_im : args.p[prob].c_re) + (long) b * args.stride_c + row * args.ldc + col;
 	const float fin = args.accumulate ? *c + v : v;
 	*c = fin;
+	herm_store_part(args, part, (int) row, (int) col, v);
 	if (args.mirror == MIRROR_CONJ) {
 		float *m = (part ? args.p[1].c_im : args.p[1].c_re) + row * args.ldc + col;
 		const float mv = part ? -v : v;
@@ -919,6 +942,7 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(CgemmArgs args) {
 		float *c = (part ? args.p[prob].c_im : args.p[prob].c_re) + (long) row * args.ldc + col;
 		const float fin = args.accumulate ? *c + v : v;
 		*c = fin;
+		herm_store_part(args, part, row, col, v);
 		if (args.mirror == MIRROR_CONJ) {
 			float *m = (part ? args.p[1].c_im : args.p[1].c_re) + (long) row * args.ldc + col;
 			const float mv = part ? -v : v;
@@ -1079,6 +1103,7 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 			float *dst = (part ? pb.c_im : pb.c_re) + (long) row * ldc + col;
 			const float fin = accumulate ? *dst + v : v;
 			*dst = fin;
+			if (args.splits == 1) herm_store_part(args, part, row, col, v);
 			if (args.mirror == MIRROR_CONJ && args.splits == 1) {
 				float *m = (part ? args.p[1].c_im : args.p[1].c_re) + (long) row * args.ldc + col;
 				const float mv = part ? -v : v;
@@ -1580,6 +1605,11 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 				right.p[q].c_im += left.N;
 			}
 		}
+		if (a.mirror == MIRROR_HERM) {  // columns of the right part count from its own first column
+			right.herm_n = a.herm_n - 2 * left.N;
+			right.herm_lo = a.herm_lo - left.N;
+			right.herm_hi = a.herm_hi - left.N;
+		}
 		if (plan_skinny(a_mcontig, b_ncontig, right, nprob, batch, planned)) {
 			int shape, tail, cuts;
 			const double whole = plan_blocks(a, nprob, batch, !a_mcontig && !b_ncontig, &shape, &tail, &cuts);
@@ -1652,13 +1682,20 @@ int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, c
 }
 
 // One product whose A (row-major) has an imaginary plane of nothing but +0, against a k-major B (used by cdft.hip)
+// herm_n > 0: the conjugate of column c, 1 <= c <= herm_n - N, is also written to column herm_n - c (the columns from N on)
 int cgemm_real_a(int M, int N, int K, const float *a_re, const float *a_im, long lda, const float *b_re, const float *b_im, long ldb, float *c_re,
-		float *c_im, long ldc) {
+		float *c_im, long ldc, int herm_n) {
 	const float *ar[2] = {a_re, a_re}, *ai[2] = {a_im, a_im}, *br[2] = {b_re, b_re}, *bi[2] = {b_im, b_im};
 	float *cr[2] = {c_re, c_re}, *ci[2] = {c_im, c_im};
 	const bool cj[2] = {false, false};
 	CgemmArgs a = pair_args(1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, 0, 0, 0);
 	a.a_real = 1;
+	if (herm_n > N) {
+		a.mirror = MIRROR_HERM;
+		a.herm_n = herm_n;
+		a.herm_lo = 1;
+		a.herm_hi = herm_n - N;
+	}
 	return cgemm_dispatch(false, true, a, 1, 1);
 }
 

@@ -1443,9 +1443,8 @@ private:
 		if (!real_transforms_ || f->typeId() != isFourier) return false;
 		CFunc *p = f->slots_[0].producer;
 		// Three quarters of the product are saved (half of the columns, and of the rest the two real products with the
-		// imaginary plane) and one short launch (the conjugate columns) added: it pays once the product runs on the block
-		// kernels (784 long: 10.7 against 13.2 us at batch 128, 22 against 34 at 512, 60 against 147 at 4096; at batch 64 both
-		// take the small-C kernel, 10 us either way and a launch more).
+		// imaginary plane), which pays once the product runs on the block kernels (784 long: 8.7 against 13.3 us at batch
+		// 128, 21 against 35 at 512, 56 against 148 at 4096; at batch 64 both take the small-C kernel, 10 us either way).
 		const double n = f->out_size_;
 		return p && p->typeId() == isInput && p->z_imag_zero_ && p->rows_ == f->rows_ && f->rows_ * n * n >= 7.5e7;
 	}

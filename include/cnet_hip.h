@@ -247,8 +247,10 @@ int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re
 /* The same transform for REAL samples (upstream's FourierTrans forward, impl/ft.h:37-55, transforms them like any
  * others, and so does gpu_fft_forward, gpu/reduce.cpp:160-187).  The caller vouches that every x_im is +0 (the plane must
  * exist and hold the zeros: the kernels for small and for unaligned shapes read it; the block kernels do not).  The result is
- * conjugate-symmetric, y[n - q] = conj(y[q]), so only columns 0 .. n/2 go through the matrix product and the rest are
- * written as conjugates, and of the four real products of a complex one the two with x_im are left out: a quarter of the
+ * conjugate-symmetric, y[n - q] = conj(y[q]), so only columns 0 .. n/2 (rounded up to a multiple of four) go through the
+ * matrix product and the rest are written as conjugates by the same kernels as they store their partners (exact conjugates;
+ * the up to three columns next to n/2 whose partners the product computes as well agree with them to rounding), and of the
+ * four real products of a complex one the two with x_im are left out: a quarter of the
  * matrix work of cnet_cdft_fwd.  Agrees with cnet_cdft_fwd on such samples to rounding (the stored twiddles are symmetric
  * under q -> n - q up to their last bit; the products that are left out add exact zeros); assigns. */
 int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
