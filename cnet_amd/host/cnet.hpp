@@ -1444,9 +1444,10 @@ private:
 		CFunc *p = f->slots_[0].producer;
 		// Three quarters of the product are saved (half of the columns, and of the rest the two real products with the
 		// imaginary plane), which pays once the product runs on the block kernels (784 long: 8.7 against 13.3 us at batch
-		// 128, 21 against 35 at 512, 56 against 148 at 4096; at batch 64 both take the small-C kernel, 10 us either way).
+		// 128, 21 against 35 at 512, 56 against 148 at 4096; 8.2 against 12.3 at batch 96; up to batch 64 both take the small-C
+		// kernel and 8 us either way).
 		const double n = f->out_size_;
-		return p && p->typeId() == isInput && p->z_imag_zero_ && p->rows_ == f->rows_ && f->rows_ * n * n >= 7.5e7;
+		return p && p->typeId() == isInput && p->z_imag_zero_ && p->rows_ == f->rows_ && f->rows_ * n * n >= 5e7;
 	}
 	bool anyRealTransformNow() const {
 		for (auto f : func_list_)
