@@ -35,6 +35,7 @@ SIGNATURES = {
     "cnet_upload_zero": [C.c_void_p, C.c_size_t],
     "cnet_upload_pair": [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t],
     "cnet_upload_gather_rows": [c_fp, _l, _l, c_fp, _l, _l, _i, _i, C.c_void_p, c_fp, c_fp, _i, _i],
+    "cnet_gather_rows": [c_fp, _l, _l, c_fp, _l, _l, _i, _i, C.c_void_p, c_fp, c_fp, _i, _i],
     "cnet_upload_wait_compute": [],
     "cnet_mark_compute": [_i],
     "cnet_upload_wait_marker": [_i],

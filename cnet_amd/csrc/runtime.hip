@@ -349,25 +349,46 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(float *__restrict__ ds
 	if (blockIdx.y == 0 && threadIdx.x == 0 && dst_labels) dst_labels[blockIdx.x] = src_labels[i];
 }
 
+static int gather_rows_on(hipStream_t stream, const char *who, float *dst, int64_t ldd, int64_t dst_plane_stride, const float *src, int64_t lds,
+		int64_t src_plane_stride, int planes, int src_rows, const int32_t *pinned_idx, int32_t *dst_labels, const int32_t *src_labels, int rows,
+		int cols);
+
 int cnet_upload_gather_rows(float *dst, int64_t ldd, int64_t dst_plane_stride, const float *src, int64_t lds, int64_t src_plane_stride,
 		int planes, int src_rows, const int32_t *pinned_idx, int32_t *dst_labels, const int32_t *src_labels, int rows, int cols) {
 	CNET_REQUIRE_INIT();
 	CNET_NOT_IN_CAPTURE();  // work on the upload stream: never part of a recording
-	CNET_CHECK_ARG(rows >= 0 && rows <= 65535 * 32 && cols > 0 && src_rows > 0 && (planes == 1 || planes == 2));
-	if (!rows) return CNET_OK;
-	CNET_CHECK_ARG(dst && src && pinned_idx && ldd >= cols && lds >= cols);
-	CNET_CHECK_ARG((dst_labels == nullptr) == (src_labels == nullptr));
-	CNET_CHECK_ARG(planes == 1 || (dst_plane_stride >= (int64_t) (rows - 1) * ldd + cols && src_plane_stride >= (int64_t) (src_rows - 1) * lds + cols));
+	return gather_rows_on(rt().upload_stream, "cnet_upload_gather_rows", dst, ldd, dst_plane_stride, src, lds, src_plane_stride, planes, src_rows,
+			pinned_idx, dst_labels, src_labels, rows, cols);
+}
+
+int cnet_gather_rows(float *dst, int64_t ldd, int64_t dst_plane_stride, const float *src, int64_t lds, int64_t src_plane_stride, int planes,
+		int src_rows, const int32_t *pinned_idx, int32_t *dst_labels, const int32_t *src_labels, int rows, int cols) {
+	CNET_REQUIRE_INIT();
+	CNET_NOT_IN_CAPTURE();  // the indices are read when the kernel runs: a replay would read whatever the buffer holds then
+	return gather_rows_on(rt().stream, "cnet_gather_rows", dst, ldd, dst_plane_stride, src, lds, src_plane_stride, planes, src_rows, pinned_idx,
+			dst_labels, src_labels, rows, cols);
+}
+
+static int gather_rows_on(hipStream_t stream, const char *who, float *dst, int64_t ldd, int64_t dst_plane_stride, const float *src, int64_t lds,
+		int64_t src_plane_stride, int planes, int src_rows, const int32_t *pinned_idx, int32_t *dst_labels, const int32_t *src_labels, int rows,
+		int cols) {
+	const bool shape_ok = rows >= 0 && rows <= 65535 * 32 && cols > 0 && src_rows > 0 && (planes == 1 || planes == 2);
+	if (shape_ok && !rows) return CNET_OK;
+	const bool args_ok = shape_ok && dst && src && pinned_idx && ldd >= cols && lds >= cols && (dst_labels == nullptr) == (src_labels == nullptr) &&
+			(planes == 1 || (dst_plane_stride >= (int64_t) (rows - 1) * ldd + cols && src_plane_stride >= (int64_t) (src_rows - 1) * lds + cols));
+	if (!args_ok)
+		return fail(CNET_ERR_INVALID_ARGUMENT, "%s: rows, cols, table rows > 0, 1 or 2 planes, pointers given, leading dimensions >= cols, planes that "
+				"do not overlap, and both label arrays or neither", who);
 	// the kernel reads the indices where they are: anything but memory from cnet_host_alloc would be a fault on the device
 	if (!in_pinned_range(pinned_idx, (size_t) rows * sizeof(int32_t)))
-		return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_upload_gather_rows: the indices do not lie in memory from cnet_host_alloc");
+		return fail(CNET_ERR_INVALID_ARGUMENT, "%s: the indices do not lie in memory from cnet_host_alloc", who);
 	for (int r = 0; r < rows; ++r)
 		if (pinned_idx[r] < 0 || pinned_idx[r] >= src_rows)
-			return fail(CNET_ERR_INVALID_ARGUMENT, "cnet_upload_gather_rows: index %d of row %d outside the table of %d rows", pinned_idx[r], r, src_rows);
+			return fail(CNET_ERR_INVALID_ARGUMENT, "%s: index %d of row %d outside the table of %d rows", who, pinned_idx[r], r, src_rows);
 	const bool vec = cols % 4 == 0 && ldd % 4 == 0 && lds % 4 == 0 && dst_plane_stride % 4 == 0 && src_plane_stride % 4 == 0 && aligned16(dst) &&
 			aligned16(src);
 	dim3 grid((unsigned) rows, (unsigned) planes);
-	hipLaunchKernelGGL(gather_rows_kernel, grid, dim3(256), 0, rt().upload_stream, dst, (long) ldd, (long) dst_plane_stride, src, (long) lds,
+	hipLaunchKernelGGL(gather_rows_kernel, grid, dim3(256), 0, stream, dst, (long) ldd, (long) dst_plane_stride, src, (long) lds,
 			(long) src_plane_stride, src_rows, pinned_idx, dst_labels, src_labels, cols, vec ? 1 : 0);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;

@@ -823,7 +823,14 @@ class CNet {
 		// since): the next batch of real samples that lands here need not clear it again.
 		bool imag_dev_zero = false;
 		int64_t upload_ticket = -1;   // the point of the upload stream at which the staged batch and its labels have landed
+		// The staged batch names samples on the device and is small: nothing was queued for it; its rows are copied on the
+		// compute stream when it is fed (see gatherOnCompute).
+		bool deferred = false;
 	};
+	// A batch whose samples are on the device and whose copy is a few microseconds of kernel (up to 1 MiB) skips the upload
+	// stream: the hand-over between the streams (two waits and two recorded points per step) costs the host more than the
+	// copy costs the device in front of the forward pass.
+	bool gatherOnCompute(const InputBatch &batch, size_t plane_bytes) const { return batch.resident_ && 2 * plane_bytes <= ((size_t) 1 << 20); }
 	Stage stage_[2];
 	int active_ = 0;
 	// recorded phases of a step, one set per buffer of the data input (device pointers are frozen into a recording)
@@ -1987,6 +1994,10 @@ private:
 		beforeFeed(cin);
 		CFunc::Slot &s = cin->slots_[0];
 		Stage &staged = stage_[1 - active_];
+		if (staged.holds == &batch && staged.deferred) {  // nothing was sent ahead: the direct path below copies it on the compute stream
+			staged.holds = NULL;
+			staged.deferred = false;
+		}
 		if (staged.holds == &batch) {
 			// the batch was sent ahead by gpuPrefetch(): switch the data input to the buffer it landed in.  Everything
 			// queued so far may still read the buffer in use, so its retirement point is remembered for the next refill.
@@ -2011,7 +2022,22 @@ private:
 		const bool real_only = batch.imagIsZero() && !send_zero_planes_;
 		Stage &here = stage_[active_];
 		const bool clear_imag = real_only && !here.imag_dev_zero;  // unless the plane is still clear from the last batch
-		if (batch.resident_) {
+		bool labels_set = false;
+		if (gatherOnCompute(batch, plane)) {
+			// the rows and their labels by one short kernel on the compute stream, behind the kernels that still read this buffer
+			const DeviceDataset &ds = *batch.resident_;
+			const size_t floats = (size_t) batch_ * s.len;
+			checkLabels(batch.labelsPtr(), batch_);
+			if (clear_imag) ck(cnet_memset_zero(s.z + floats, plane), "cnet_memset_zero");
+			ck(cnet_gather_rows(s.z, s.len, (int64_t) floats, ds.z_, ds.dim_, (int64_t) ds.count_ * ds.dim_, ds.planes_, ds.count_, batch.indices_, d_labels_,
+					ds.labels_dev_, batch_, s.len), "cnet_gather_rows");
+			if (!real_only && ds.planes_ == 1) ck(cnet_memset_zero(s.z + floats, plane), "cnet_memset_zero");
+			ck(cnet_copy_ticket(0, &batch.ticket_), "cnet_copy_ticket");
+			labels_.assign(batch.labelsPtr(), batch.labelsPtr() + batch_);
+			batch_labels_ = true;
+			lossGradientsStale();
+			labels_set = true;
+		} else if (batch.resident_) {
 			// The samples are on the device already: the upload stream, behind everything queued on the compute stream so far
 			// (which may still read this buffer), copies the rows named by the indices; the compute stream waits for that.
 			const DeviceDataset &ds = *batch.resident_;
@@ -2034,7 +2060,7 @@ private:
 		}
 		here.imag_dev_zero = batch.imagIsZero();  // zeros on the device, cleared there (now or earlier) or sent
 		cin->z_imag_zero_ = batch.imagIsZero();
-		setLabels(batch.labelsPtr(), batch_);
+		if (!labels_set) setLabels(batch.labelsPtr(), batch_);
 	}
 
 public:
@@ -2056,6 +2082,11 @@ public:
 		if (st.holds) throw std::logic_error("gpuPrefetch: a staged batch is still waiting for its gpuForward");
 		CFunc::Slot &s = cin->slots_[0];
 		const size_t plane = (size_t) batch_ * s.len;
+		if (gatherOnCompute(batch, plane * sizeof(float))) {  // nothing to send ahead: gpuForward copies the rows itself
+			st.holds = &batch;
+			st.deferred = true;
+			return;
+		}
 		if (!st.z) {
 			st.z = dalloc<float>(2 * plane);
 			st.labels = dalloc<int32_t>(batch_);

@@ -106,6 +106,11 @@ int cnet_upload_pair(void *dst0, const void *pinned_src0, size_t bytes0, void *d
 int cnet_upload_gather_rows(float *dst, int64_t ldd, int64_t dst_plane_stride, const float *src, int64_t lds,
                             int64_t src_plane_stride, int planes, int src_rows, const int32_t *pinned_idx,
                             int32_t *dst_labels, const int32_t *src_labels, int rows, int cols);
+/* The same on the compute stream, in front of the kernels that read the batch (no hand-over between the streams: what a small
+ * batch wants, whose copy is shorter than the hand-over).  Not while recording: the indices are read when the kernel runs. */
+int cnet_gather_rows(float *dst, int64_t ldd, int64_t dst_plane_stride, const float *src, int64_t lds,
+                     int64_t src_plane_stride, int planes, int src_rows, const int32_t *pinned_idx,
+                     int32_t *dst_labels, const int32_t *src_labels, int rows, int cols);
 int cnet_upload_wait_compute(void);
 int cnet_mark_compute(int marker);
 int cnet_upload_wait_marker(int marker);

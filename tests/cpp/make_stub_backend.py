@@ -14,7 +14,7 @@ def generate(header_path, out_path):
     decls = re.findall(r'\n((?:int|void \*|const char \*)\s*cnet_\w+\s*\([^;]*?\));', text)
     special = {'cnet_graph_end', 'cnet_graph_launch', 'cnet_graph_destroy', 'cnet_graph_begin', 'cnet_alloc', 'cnet_host_alloc',
                'cnet_free', 'cnet_host_free', 'cnet_memcpy_h2d', 'cnet_memcpy_d2h', 'cnet_memcpy_d2d', 'cnet_memcpy_h2d_async',
-               'cnet_memcpy_d2h_async', 'cnet_upload_async', 'cnet_upload_zero', 'cnet_upload_pair', 'cnet_upload_gather_rows', 'cnet_memset_zero', 'cnet_last_error', 'cnet_stream',
+               'cnet_memcpy_d2h_async', 'cnet_upload_async', 'cnet_upload_zero', 'cnet_upload_pair', 'cnet_upload_gather_rows', 'cnet_gather_rows', 'cnet_memset_zero', 'cnet_last_error', 'cnet_stream',
                'cnet_get_device_info'}
     out = ['#include "cnet_hip.h"\n#include <cstdio>\n#include <cstdlib>\n#include <cstring>\n#include <set>\nextern "C" {\n']
     seen = set()
@@ -52,6 +52,10 @@ int cnet_upload_gather_rows(float *d, int64_t ldd, int64_t dps, const float *s, 
 		}
 	if (dl) for (int r = 0; r < rows; ++r) dl[r] = sl[idx[r]];
 	return 0;
+}
+int cnet_gather_rows(float *d, int64_t ldd, int64_t dps, const float *s, int64_t lds, int64_t sps, int planes, int src_rows,
+		const int32_t *idx, int32_t *dl, const int32_t *sl, int rows, int cols) {
+	return cnet_upload_gather_rows(d, ldd, dps, s, lds, sps, planes, src_rows, idx, dl, sl, rows, cols);
 }
 int cnet_memset_zero(void *d, size_t b) { memset(d, 0, b); return 0; }
 const char *cnet_last_error(void) { return "stub"; }
