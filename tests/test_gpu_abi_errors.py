@@ -416,6 +416,13 @@ def test_rows_of_a_table_on_the_device_into_a_batch_buffer(gpu):
         # samples only
         capi.call("cnet_upload_gather_rows", d_out.ptr, ld, rows * ld, d_table.ptr, dim, count * dim, 1, count, hp, None, None, rows, dim)
         capi.call("cnet_upload_sync")
+        # the twin on the compute stream
+        d_out2 = capi.to_device(np.full((planes, rows, ld), -7.0, np.float32))
+        d_lab2 = capi.to_device(np.full(rows, -1, np.int32))
+        capi.call("cnet_gather_rows", d_out2.ptr, ld, rows * ld, d_table.ptr, dim, count * dim, planes, count, hp, d_lab2.ptr, d_labels.ptr, rows, dim)
+        assert np.array_equal(d_out2.download(), out) and np.array_equal(d_lab2.download(), labels[idx])
+        assert lib.cnet_gather_rows(d_out2.ptr, ld, rows * ld, d_table.ptr, dim, count * dim, 3, count, hp, d_lab2.ptr, d_labels.ptr, rows, dim) == -2
+        assert "cnet_gather_rows" in _msg()
         # refused: an index outside the table, a lone label array, indices in pageable memory
         keep = int(idx[0])
         idx[0] = count
