@@ -61,11 +61,13 @@ def test_linear_cgelu_into_a_column_window(gpu, port):
 
 
 @pytest.mark.parametrize("B,K,N", [(64, 784, 10), (64, 16, 16), (33, 7, 5), (16, 64, 12), (1, 3, 2), (200, 40, 24), (64, 784, 784),
-                                   (1024, 256, 256)])
+                                   (1024, 256, 256), (4096, 784, 10), (1000, 100, 16), (300, 5, 1), (256, 1030, 3), (513, 260, 7),
+                                   (257, 33, 12)])
 def test_both_gradients_of_a_linear_in_one_call(gpu, port, B, K, N):
     """cnet_clinear_bwd_sym against cnet_clinear_bwd_input_sym + cnet_clinear_bwd_weight_sym: same bits, whether the two
     products share a launch (both small and on the same kernel: the first cases) or not, with each accumulate flag and with
-    the dz* planes of either result left out."""
+    the dz* planes of either result left out.  The cases from (4096, 784, 10) on are narrow layers (few outputs) at batches
+    beyond the small-C kernel: a K of 1 .. 16 for the input gradient, a reduction over the whole batch for the weights."""
     gr, gi = seeded(port, B + 11, (B, N)), seeded(port, B + 12, (B, N))
     g = ops.Grad.from_host([gr, gi, gr, -gi])
     x = ops.CMat.from_host(seeded(port, K + 1, (B, K)), seeded(port, K + 2, (B, K)))
@@ -79,13 +81,46 @@ def test_both_gradients_of_a_linear_in_one_call(gpu, port, B, K, N):
         for a, b in ((dx0, dx1), (dw0, dw1)):
             for pa, pb in zip(a.host(), b.host()):
                 assert np.array_equal(pa, pb), (acc_x, acc_w, mir_x, mir_w)
-    if B * K * N <= 1 << 24:   # the CPU path on the same pair
+    if B * K * N <= 1 << 26:   # the CPU path on the same pair
         (xr, xi), (wr, wi) = x.host(), w.host()
         dxo, dwo = port.linear_bwd(xr, xi, wr, wi, [gr, gi, gr, -gi])
         dx1, dw1 = ops.Grad.empty(B, K), ops.Grad.empty(N, K)
         ops.linear_bwd_sym(g, x, w, dx1, dw1)
         assert rel_c(dx1.host()[0:2], dxo[0:2]) < TOL / 5 and rel_c(dx1.host()[2:4], dxo[2:4]) < TOL / 5
         assert rel_c(dw1.host()[0:2], dwo[0:2]) < TOL / 5 and rel_c(dw1.host()[2:4], dwo[2:4]) < TOL / 5
+
+
+def test_backward_pass_of_a_narrow_linear_in_windows_of_wider_buffers(gpu):
+    """Both gradients of a narrow layer (few outputs, many rows) with every operand a column window of a wider buffer, against
+    numpy in complex128; what lies beside the windows stays untouched, and accumulation adds to what the windows held."""
+    rs = np.random.RandomState(5)
+    for B, K, N in [(700, 300, 10), (256, 7, 16), (1200, 1025, 2)]:
+        def wide(rows, cols, pad_l, pad_r):
+            buf = rs.randn(rows, pad_l + cols + pad_r).astype(np.float32)
+            bufi = rs.randn(rows, pad_l + cols + pad_r).astype(np.float32)
+            full = ops.CMat.from_host(buf, bufi)
+            return full, full.sub(pad_l, cols), (buf + 1j * bufi)[:, pad_l:pad_l + cols].astype(np.complex128), buf, bufi
+        _, g, G, _, _ = wide(B, N, 3, 2)
+        _, x, X, _, _ = wide(B, K, 1, 4)
+        _, w, W, _, _ = wide(N, K, 5, 0)
+        gg = ops.Grad([g.re, g.im, g.re, g.im])   # only the dz planes are read
+        for acc in (0, 1):
+            dxf, dx, DX0, dxb, dxbi = wide(B, K, 2, 3)
+            dwf, dw, DW0, dwb, dwbi = wide(N, K, 4, 1)
+            dxs, dws = ops.CMat.empty(B, K, ld=K + 5, zero=True), ops.CMat.empty(N, K, ld=K + 5, zero=True)   # the leading dimension of the windows
+            ops.linear_bwd_sym(gg, x, w, ops.Grad([dx.re, dx.im, dxs.re, dxs.im]), ops.Grad([dw.re, dw.im, dws.re, dws.im]),
+                               accumulate_dx=acc, accumulate_dw=acc)
+            want_dx, want_dw = G @ W + (DX0 if acc else 0), G.T @ X + (DW0 if acc else 0)
+            for full, window, want, b_re, b_im, pad_l, cols in ((dxf, dx, want_dx, dxb, dxbi, 2, K), (dwf, dw, want_dw, dwb, dwbi, 4, K)):
+                hr, hi = full.re.owner.download(), full.im.owner.download()
+                got = (hr + 1j * hi)[:, pad_l:pad_l + cols]
+                assert np.linalg.norm(got - want) / np.linalg.norm(want) < 2e-6, (B, K, N, acc)
+                mask = np.ones(hr.shape[1], bool); mask[pad_l:pad_l + cols] = False
+                assert np.array_equal(hr[:, mask], b_re[:, mask]) and np.array_equal(hi[:, mask], b_im[:, mask])
+            # the dz* planes: conjugates of what was added
+            (sr, si), (tr, ti) = dxs.host(), dws.host()
+            assert np.linalg.norm((sr + 1j * si) - np.conj(G @ W)) / np.linalg.norm(G @ W) < 2e-6
+            assert np.linalg.norm((tr + 1j * ti) - np.conj(G.T @ X)) / np.linalg.norm(G.T @ X) < 2e-6
 
 
 @pytest.mark.parametrize("overrides", [
