@@ -129,7 +129,9 @@ def test_transform_of_real_samples_through_half_the_columns(gpu, port, B, n):
     ops.dft_fwd_real_input(x, half)
     fr, fi = full.host()
     hr, hi = half.host()
-    assert rel_c((hr, hi), (fr, fi)) < 1e-6   # two roundings of the same sums
+    # two roundings of the same sums; the full transform rounds more where the process forms a complex product from three real
+    # ones (CNET_CGEMM_3M=1: 1.6e-6 from double precision at n = 4096), which the transform of real samples never does
+    assert rel_c((hr, hi), (fr, fi)) < (1e-6 if capi.load().cnet_cgemm_get_products() == 4 else 3e-6)
     cols = min(n, (n // 2 + 1 + 3) // 4 * 4)   # what the product computes; the columns from there on are written as conjugates
     for q in range(1, (n - 1) // 2 + 1):
         if q <= n - cols:
