@@ -215,8 +215,9 @@ int cnet_clinear_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg
                          int N);
 
 /* How many real matrix products the block kernels of every complex product above and below (Linear, FourierTrans,
- * TriangFourier; forward and backward) form one complex product from.  No counterpart upstream, whose kernels multiply
- * complex numbers one by one with four real multiplications (gpu/reduce.cpp:56-77, impl/linear.h:51-69).
+ * TriangFourier; forward and backward) form one complex product from.  Upstream's CPU path, the parity reference, multiplies
+ * complex numbers with four real multiplications (std::complex, impl/linear.h:51-69); its device code with three, number by
+ * number (cmplx_::operator*=, gpu/compl.h:57-63: (a - b) d + a (c - d) and (a + b) c - a (c - d)).
  *   4 (default): Cr = Ar Br - Ai Bi, Ci = Ar Bi + Ai Br, the four real products of the complex multiplication.
  *   3: P = Ar Br, Q = Ai Bi, T = (Ar + Ai)(Br + Bi); Cr = P - Q, Ci = T - P - Q (signs of a conjugated operand
  *      applied to its imaginary part in the sums): a quarter of the matrix work less.  The real part is formed as with
