@@ -221,21 +221,27 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *_
 }
 
 // dst[p][c] (+)= sum over slabs of partial[slab][p][c], slabs added in index order.
-__global__ __launch_bounds__(TPB) void slab_sum_kernel(const float *__restrict__ partial, int nslabs, int nplanes, int cols,
+// SLAB_LANES: lanes that share the slabs of one (plane, column) pair: 16 for many slabs, 4 for few (a workgroup of 1024
+// threads takes longer to start than the few loads of a small sum take)
+template <int SLAB_LANES>
+__global__ __launch_bounds__(64 * SLAB_LANES) void slab_sum_kernel(const float *__restrict__ partial, int nslabs, int nplanes, int cols,
 		Grad4 dst, int accumulate) {
-	// 64 (plane, column) pairs per workgroup x 4 lanes that each add one contiguous quarter of the slabs in order; the
-	// four quarter sums are then added in lane order
-	__shared__ float red[4][64];
+	// 64 (plane, column) pairs per workgroup x SLAB_LANES lanes that each add one contiguous part of the slabs in order (128
+	// slabs on 16 lanes: a batch of eight loads per lane, not four batches one after the other); the lanes' sums are then added
+	// in lane order
+	__shared__ float red[SLAB_LANES][64];
 	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
 	const long idx = (long) blockIdx.x * 64 + tx;
 	const bool live = idx < (long) nplanes * cols;
 	const int p = live ? (int) (idx / cols) : 0;
 	const int c = live ? (int) (idx - (long) p * cols) : 0;
-	const int per = (nslabs + 3) / 4, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
+	const int per = (nslabs + SLAB_LANES - 1) / SLAB_LANES, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
 	red[ty][tx] = live ? cnet::ordered_sum(partial + ((long) k0 * nplanes + p) * cols + c, (long) nplanes * cols, k1 - k0) : 0.f;
 	__syncthreads();
 	if (ty == 0 && live) {
-		const float s = ((red[0][tx] + red[1][tx]) + red[2][tx]) + red[3][tx];
+		float s = red[0][tx];
+#pragma unroll
+		for (int l = 1; l < SLAB_LANES; ++l) s += red[l][tx];
 		float *out = p == 0 ? dst.dz_re : (p == 1 ? dst.dz_im : (p == 2 ? dst.dzs_re : dst.dzs_im));
 		out[c] = accumulate ? out[c] + s : s;
 	}
@@ -716,18 +722,21 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_sym_kernel(const floa
 
 // dst.dz (+)= sum over slabs of partial[slab][re, im][c], slabs added in index order; the conjugate goes to dst.dzs when
 // those planes are given
-__global__ __launch_bounds__(TPB) void slab_sum_sym_kernel(const float *__restrict__ partial, int nslabs, int cols, Pair2 dst, int accumulate) {
-	__shared__ float red[4][64];
+template <int SLAB_LANES>
+__global__ __launch_bounds__(64 * SLAB_LANES) void slab_sum_sym_kernel(const float *__restrict__ partial, int nslabs, int cols, Pair2 dst, int accumulate) {
+	__shared__ float red[SLAB_LANES][64];
 	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
 	const long idx = (long) blockIdx.x * 64 + tx;
 	const bool live = idx < 2L * cols;
 	const int p = live ? (int) (idx / cols) : 0;
 	const int c = live ? (int) (idx - (long) p * cols) : 0;
-	const int per = (nslabs + 3) / 4, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
+	const int per = (nslabs + SLAB_LANES - 1) / SLAB_LANES, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
 	red[ty][tx] = live ? cnet::ordered_sum(partial + ((long) k0 * 2 + p) * cols + c, 2L * cols, k1 - k0) : 0.f;
 	__syncthreads();
 	if (ty == 0 && live) {
-		const float s = ((red[0][tx] + red[1][tx]) + red[2][tx]) + red[3][tx];
+		float s = red[0][tx];
+#pragma unroll
+		for (int l = 1; l < SLAB_LANES; ++l) s += red[l][tx];
 		float *out = p == 0 ? dst.dz_re : dst.dz_im;
 		out[c] = accumulate ? out[c] + s : s;
 		if (dst.dzs_re) {
@@ -1038,7 +1047,10 @@ int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const f
 		hipLaunchKernelGGL((hadamard_bwd_shared_kernel<1, 0>), grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g, ldg, du,
 				lddu, partial, rows, cols, rows_per_slab, accumulate);
 	CNET_LAUNCH_CHECK();
-	hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned) ((4L * cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
+	if (nslabs > 32)
+		hipLaunchKernelGGL(slab_sum_kernel<16>, dim3((unsigned) ((4L * cols + 63) / 64)), dim3(64 * 16), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
+	else
+		hipLaunchKernelGGL(slab_sum_kernel<4>, dim3((unsigned) ((4L * cols + 63) / 64)), dim3(64 * 4), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1473,7 +1485,10 @@ static int hadamard_bwd_sym_impl(const char *who, bool gelu, const float *u_re, 
 		CNET_LAUNCH_V1G(hadamard_bwd_shared_sym_kernel, gelu, grid, dim3(TPB), 0, rt().stream, u_re, u_im, ldu, v_re, v_im, g_dz_re, g_dz_im, ldg,
 				dh, lddh, du, lddu, partial, rows, cols, rows_per_slab, accumulate);
 	CNET_LAUNCH_CHECK();
-	hipLaunchKernelGGL(slab_sum_sym_kernel, dim3((unsigned) ((2L * cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, nslabs, cols, dv, accumulate);
+	if (nslabs > 32)
+		hipLaunchKernelGGL(slab_sum_sym_kernel<16>, dim3((unsigned) ((2L * cols + 63) / 64)), dim3(64 * 16), 0, rt().stream, partial, nslabs, cols, dv, accumulate);
+	else
+		hipLaunchKernelGGL(slab_sum_sym_kernel<4>, dim3((unsigned) ((2L * cols + 63) / 64)), dim3(64 * 4), 0, rt().stream, partial, nslabs, cols, dv, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }

@@ -696,19 +696,25 @@ __global__ __launch_bounds__(TPB) void colsum_partial_kernel(const float *__rest
 	}
 }
 
-__global__ __launch_bounds__(TPB) void colsum_final_kernel(const float *__restrict__ partial, int nslabs, int cols,
+// FINAL_LANES: lanes that share the slabs of one column in the second stage: 16 for many slabs, 4 for few (a workgroup of
+// 1024 threads takes longer to start than the few loads of a small sum take)
+template <int FINAL_LANES>
+__global__ __launch_bounds__(64 * FINAL_LANES) void colsum_final_kernel(const float *__restrict__ partial, int nslabs, int cols,
 		float *__restrict__ dst, int accumulate) {
-	// 64 columns per workgroup x 4 lanes that each add one contiguous quarter of the slabs in order; the four quarter
-	// sums are then added in lane order
-	__shared__ float red[4][64];
+	// 64 columns per workgroup x FINAL_LANES lanes that each add one contiguous part of the slabs in order (128 slabs on 16
+	// lanes: one batch of eight loads per lane instead of four batches one after the other on four lanes); the lanes' sums
+	// are then added in lane order
+	__shared__ float red[FINAL_LANES][64];
 	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
 	const int c = blockIdx.x * 64 + tx;
 	const bool live = c < cols;
-	const int per = (nslabs + 3) / 4, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
+	const int per = (nslabs + FINAL_LANES - 1) / FINAL_LANES, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
 	red[ty][tx] = live ? cnet::ordered_sum(partial + (long) k0 * cols + c, cols, k1 - k0) : 0.f;
 	__syncthreads();
 	if (ty == 0 && live) {
-		const float s = ((red[0][tx] + red[1][tx]) + red[2][tx]) + red[3][tx];
+		float s = red[0][tx];
+#pragma unroll
+		for (int l = 1; l < FINAL_LANES; ++l) s += red[l][tx];
 		dst[c] = accumulate ? dst[c] + s : s;
 	}
 }
@@ -921,8 +927,12 @@ static int batch_sum_launch(const float *src, int64_t lds, float *dst, int rows,
 	else
 		hipLaunchKernelGGL(colsum_partial_kernel<1>, grid, dim3(TPB), 0, rt().stream, src, (long) lds, partial, rows, cols, p.rows_per_slab);
 	CNET_LAUNCH_CHECK();
-	hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned) ((cols + 63) / 64)), dim3(TPB), 0, rt().stream, partial, p.nslabs, cols, dst,
-			accumulate);
+	if (p.nslabs > 32)
+		hipLaunchKernelGGL(colsum_final_kernel<16>, dim3((unsigned) ((cols + 63) / 64)), dim3(64 * 16), 0, rt().stream, partial, p.nslabs, cols, dst,
+				accumulate);
+	else
+		hipLaunchKernelGGL(colsum_final_kernel<4>, dim3((unsigned) ((cols + 63) / 64)), dim3(64 * 4), 0, rt().stream, partial, p.nslabs, cols, dst,
+				accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
