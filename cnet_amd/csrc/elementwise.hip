@@ -221,17 +221,15 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *_
 }
 
 // dst[p][c] (+)= sum over slabs of partial[slab][p][c], slabs added in index order.
-// SLAB_LANES: lanes that share the slabs of one (plane, column) pair: 16 for many slabs, 4 for few (a workgroup of 1024
-// threads takes longer to start than the few loads of a small sum take)
-template <int SLAB_LANES>
-__global__ __launch_bounds__(64 * SLAB_LANES) void slab_sum_kernel(const float *__restrict__ partial, int nslabs, int nplanes, int cols,
+// SLAB_COLS (plane, column) pairs per workgroup x SLAB_LANES lanes that each add one contiguous part of the slabs in order; the
+// lanes' sums are then added in lane order.  Few slabs: 64 pairs x 4 lanes; more than 32: 16 pairs x 64 lanes (two loads
+// per lane for 128 slabs, four times as many workgroups: the kernel is all latency).
+template <int SLAB_LANES, int SLAB_COLS>
+__global__ __launch_bounds__(SLAB_LANES * SLAB_COLS) void slab_sum_kernel(const float *__restrict__ partial, int nslabs, int nplanes, int cols,
 		Grad4 dst, int accumulate) {
-	// 64 (plane, column) pairs per workgroup x SLAB_LANES lanes that each add one contiguous part of the slabs in order (128
-	// slabs on 16 lanes: a batch of eight loads per lane, not four batches one after the other); the lanes' sums are then added
-	// in lane order
-	__shared__ float red[SLAB_LANES][64];
-	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-	const long idx = (long) blockIdx.x * 64 + tx;
+	__shared__ float red[SLAB_LANES][SLAB_COLS];
+	const int tx = threadIdx.x % SLAB_COLS, ty = threadIdx.x / SLAB_COLS;
+	const long idx = (long) blockIdx.x * SLAB_COLS + tx;
 	const bool live = idx < (long) nplanes * cols;
 	const int p = live ? (int) (idx / cols) : 0;
 	const int c = live ? (int) (idx - (long) p * cols) : 0;
@@ -240,7 +238,7 @@ __global__ __launch_bounds__(64 * SLAB_LANES) void slab_sum_kernel(const float *
 	__syncthreads();
 	if (ty == 0 && live) {
 		float s = red[0][tx];
-#pragma unroll
+#pragma unroll 8
 		for (int l = 1; l < SLAB_LANES; ++l) s += red[l][tx];
 		float *out = p == 0 ? dst.dz_re : (p == 1 ? dst.dz_im : (p == 2 ? dst.dzs_re : dst.dzs_im));
 		out[c] = accumulate ? out[c] + s : s;
@@ -722,11 +720,11 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_sym_kernel(const floa
 
 // dst.dz (+)= sum over slabs of partial[slab][re, im][c], slabs added in index order; the conjugate goes to dst.dzs when
 // those planes are given
-template <int SLAB_LANES>
-__global__ __launch_bounds__(64 * SLAB_LANES) void slab_sum_sym_kernel(const float *__restrict__ partial, int nslabs, int cols, Pair2 dst, int accumulate) {
-	__shared__ float red[SLAB_LANES][64];
-	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-	const long idx = (long) blockIdx.x * 64 + tx;
+template <int SLAB_LANES, int SLAB_COLS>
+__global__ __launch_bounds__(SLAB_LANES * SLAB_COLS) void slab_sum_sym_kernel(const float *__restrict__ partial, int nslabs, int cols, Pair2 dst, int accumulate) {
+	__shared__ float red[SLAB_LANES][SLAB_COLS];
+	const int tx = threadIdx.x % SLAB_COLS, ty = threadIdx.x / SLAB_COLS;
+	const long idx = (long) blockIdx.x * SLAB_COLS + tx;
 	const bool live = idx < 2L * cols;
 	const int p = live ? (int) (idx / cols) : 0;
 	const int c = live ? (int) (idx - (long) p * cols) : 0;
@@ -735,7 +733,7 @@ __global__ __launch_bounds__(64 * SLAB_LANES) void slab_sum_sym_kernel(const flo
 	__syncthreads();
 	if (ty == 0 && live) {
 		float s = red[0][tx];
-#pragma unroll
+#pragma unroll 8
 		for (int l = 1; l < SLAB_LANES; ++l) s += red[l][tx];
 		float *out = p == 0 ? dst.dz_re : dst.dz_im;
 		out[c] = accumulate ? out[c] + s : s;
@@ -1048,9 +1046,9 @@ int cnet_hadamard_bwd(const float *u_re, const float *u_im, int64_t ldu, const f
 				lddu, partial, rows, cols, rows_per_slab, accumulate);
 	CNET_LAUNCH_CHECK();
 	if (nslabs > 32)
-		hipLaunchKernelGGL(slab_sum_kernel<16>, dim3((unsigned) ((4L * cols + 63) / 64)), dim3(64 * 16), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
+		hipLaunchKernelGGL((slab_sum_kernel<64, 16>), dim3((unsigned) ((4L * cols + 15) / 16)), dim3(1024), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
 	else
-		hipLaunchKernelGGL(slab_sum_kernel<4>, dim3((unsigned) ((4L * cols + 63) / 64)), dim3(64 * 4), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
+		hipLaunchKernelGGL((slab_sum_kernel<4, 64>), dim3((unsigned) ((4L * cols + 63) / 64)), dim3(256), 0, rt().stream, partial, nslabs, 4, cols, dv, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
@@ -1486,9 +1484,9 @@ static int hadamard_bwd_sym_impl(const char *who, bool gelu, const float *u_re, 
 				dh, lddh, du, lddu, partial, rows, cols, rows_per_slab, accumulate);
 	CNET_LAUNCH_CHECK();
 	if (nslabs > 32)
-		hipLaunchKernelGGL(slab_sum_sym_kernel<16>, dim3((unsigned) ((2L * cols + 63) / 64)), dim3(64 * 16), 0, rt().stream, partial, nslabs, cols, dv, accumulate);
+		hipLaunchKernelGGL((slab_sum_sym_kernel<64, 16>), dim3((unsigned) ((2L * cols + 15) / 16)), dim3(1024), 0, rt().stream, partial, nslabs, cols, dv, accumulate);
 	else
-		hipLaunchKernelGGL(slab_sum_sym_kernel<4>, dim3((unsigned) ((2L * cols + 63) / 64)), dim3(64 * 4), 0, rt().stream, partial, nslabs, cols, dv, accumulate);
+		hipLaunchKernelGGL((slab_sum_sym_kernel<4, 64>), dim3((unsigned) ((2L * cols + 63) / 64)), dim3(256), 0, rt().stream, partial, nslabs, cols, dv, accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }

@@ -696,24 +696,23 @@ __global__ __launch_bounds__(TPB) void colsum_partial_kernel(const float *__rest
 	}
 }
 
-// FINAL_LANES: lanes that share the slabs of one column in the second stage: 16 for many slabs, 4 for few (a workgroup of
-// 1024 threads takes longer to start than the few loads of a small sum take)
-template <int FINAL_LANES>
-__global__ __launch_bounds__(64 * FINAL_LANES) void colsum_final_kernel(const float *__restrict__ partial, int nslabs, int cols,
+// Second stage: FINAL_COLS columns per workgroup x FINAL_LANES lanes that each add one contiguous part of the slabs in order;
+// the lanes' sums are then added in lane order.  Few slabs: 64 columns x 4 lanes.  Many (more than 32): 16 columns x 64
+// lanes, which for 128 slabs is two loads per lane and, at 4096 columns, 256 workgroups instead of 64 (the kernel is all
+// latency: 2 MiB to read behind a launch).
+template <int FINAL_LANES, int FINAL_COLS>
+__global__ __launch_bounds__(FINAL_LANES * FINAL_COLS) void colsum_final_kernel(const float *__restrict__ partial, int nslabs, int cols,
 		float *__restrict__ dst, int accumulate) {
-	// 64 columns per workgroup x FINAL_LANES lanes that each add one contiguous part of the slabs in order (128 slabs on 16
-	// lanes: one batch of eight loads per lane instead of four batches one after the other on four lanes); the lanes' sums
-	// are then added in lane order
-	__shared__ float red[FINAL_LANES][64];
-	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-	const int c = blockIdx.x * 64 + tx;
+	__shared__ float red[FINAL_LANES][FINAL_COLS];
+	const int tx = threadIdx.x % FINAL_COLS, ty = threadIdx.x / FINAL_COLS;
+	const int c = blockIdx.x * FINAL_COLS + tx;
 	const bool live = c < cols;
 	const int per = (nslabs + FINAL_LANES - 1) / FINAL_LANES, k0 = min(nslabs, ty * per), k1 = min(nslabs, k0 + per);
 	red[ty][tx] = live ? cnet::ordered_sum(partial + (long) k0 * cols + c, cols, k1 - k0) : 0.f;
 	__syncthreads();
 	if (ty == 0 && live) {
 		float s = red[0][tx];
-#pragma unroll
+#pragma unroll 8
 		for (int l = 1; l < FINAL_LANES; ++l) s += red[l][tx];
 		dst[c] = accumulate ? dst[c] + s : s;
 	}
@@ -928,10 +927,10 @@ static int batch_sum_launch(const float *src, int64_t lds, float *dst, int rows,
 		hipLaunchKernelGGL(colsum_partial_kernel<1>, grid, dim3(TPB), 0, rt().stream, src, (long) lds, partial, rows, cols, p.rows_per_slab);
 	CNET_LAUNCH_CHECK();
 	if (p.nslabs > 32)
-		hipLaunchKernelGGL(colsum_final_kernel<16>, dim3((unsigned) ((cols + 63) / 64)), dim3(64 * 16), 0, rt().stream, partial, p.nslabs, cols, dst,
+		hipLaunchKernelGGL((colsum_final_kernel<64, 16>), dim3((unsigned) ((cols + 15) / 16)), dim3(1024), 0, rt().stream, partial, p.nslabs, cols, dst,
 				accumulate);
 	else
-		hipLaunchKernelGGL(colsum_final_kernel<4>, dim3((unsigned) ((cols + 63) / 64)), dim3(64 * 4), 0, rt().stream, partial, p.nslabs, cols, dst,
+		hipLaunchKernelGGL((colsum_final_kernel<4, 64>), dim3((unsigned) ((cols + 63) / 64)), dim3(256), 0, rt().stream, partial, p.nslabs, cols, dst,
 				accumulate);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
