@@ -1528,6 +1528,31 @@ static void test_errors() {
 		// |x + t|^2 summed, t = (0.5, 0, ...): row 0 of the set is (1, 2, 3, 0, ...), the other rows are zeros
 		const float row0 = 1.5f * 1.5f + 2.f * 2.f + 3.f * 3.f, rest = 0.5f * 0.5f;
 		expect("the forward pass saw the rows that the indices name", std::fabs(rb.loss(1) - row0) < 1e-5f && std::fabs(rb.loss(0) - rest) < 1e-6f && std::fabs(rb.loss(3) - rest) < 1e-6f);
+		// complex samples: both planes live on the device and both are copied; the same batch sent from the host gives the same losses
+		float cre[3 * 8], cim[3 * 8];
+		for (int k = 0; k < 24; ++k) {
+			cre[k] = 0.25f * (float) (k % 7) - 0.5f;
+			cim[k] = 0.125f * (float) (k % 5) + 0.0625f;
+		}
+		DeviceDataset cds(cre, cim, labels, 3, 8);
+		expect("a data set with imaginary parts keeps both planes", !cds.imagIsZero());
+		InputBatch cb(4, 8), hb(4, 8);
+		cb.gatherResident(cds, pick, 4);
+		hb.gather(cre, cim, labels, pick, 4);
+		net5.gpuSetInput(t5, tb);
+		net5.gpuForward((CInput *) net5[x5], (L2Out *) net5[o5], cb);
+		net5.getLoss((L2Out *) net5[o5], &cb);
+		net5.gpuSetInput(t5, tb);
+		net5.gpuForward((CInput *) net5[x5], (L2Out *) net5[o5], hb);
+		net5.getLoss((L2Out *) net5[o5], &hb);
+		bool same = true;
+		for (int b = 0; b < 4; ++b) same = same && cb.loss(b) == hb.loss(b) && cb.loss(b) > 0.f;
+		expect("complex samples copied on the device give the losses of the same samples sent from the host", same && !cb.imagIsZero());
+		// and back to real samples in the same buffer: its imaginary plane is cleared again
+		net5.gpuSetInput(t5, tb);
+		net5.gpuForward((CInput *) net5[x5], (L2Out *) net5[o5], rb);
+		net5.getLoss((L2Out *) net5[o5], &rb);
+		expect("real samples after complex ones find a cleared imaginary plane", std::fabs(rb.loss(1) - row0) < 1e-5f && std::fabs(rb.loss(0) - rest) < 1e-6f);
 		net5.sync();
 	}
 	// device layer status codes
