@@ -331,22 +331,22 @@ int cnet_upload_pair(void *dst0, const void *pinned_src0, size_t bytes0, void *d
 	return CNET_OK;
 }
 
-// rows of a table on the device into a batch buffer, with their labels: workgroup (r, p) copies row idx[r] of plane p
+// rows of a table on the device into a batch buffer, with their labels: each wavefront of workgroup (x, p) copies one row,
+// idx[4 x + wavefront], of plane p (its lanes read the index over the link in one request)
 __global__ __launch_bounds__(256) void gather_rows_kernel(float *__restrict__ dst, long ldd, long dst_plane, const float *__restrict__ src,
 		long lds, long src_plane, int src_rows, const int32_t *__restrict__ idx, int32_t *__restrict__ dst_labels,
-		const int32_t *__restrict__ src_labels, int cols, int vec) {
-	__shared__ int which;
-	if (threadIdx.x == 0) which = min(max(idx[blockIdx.x], 0), src_rows - 1);  // one read over the link per workgroup
-	__syncthreads();
-	const int i = which;
+		const int32_t *__restrict__ src_labels, int rows, int cols, int vec) {
+	const int r = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+	if (r >= rows) return;
+	const int i = min(max(idx[r], 0), src_rows - 1);
 	const float *s = src + (long) blockIdx.y * src_plane + (long) i * lds;
-	float *d = dst + (long) blockIdx.y * dst_plane + (long) blockIdx.x * ldd;
+	float *d = dst + (long) blockIdx.y * dst_plane + (long) r * ldd;
 	if (vec) {
-		for (int c = threadIdx.x * 4; c < cols; c += 1024) *reinterpret_cast<float4 *>(d + c) = *reinterpret_cast<const float4 *>(s + c);
+		for (int c = lane * 4; c < cols; c += 256) *reinterpret_cast<float4 *>(d + c) = *reinterpret_cast<const float4 *>(s + c);
 	} else {
-		for (int c = threadIdx.x; c < cols; c += 256) d[c] = s[c];
+		for (int c = lane; c < cols; c += 64) d[c] = s[c];
 	}
-	if (blockIdx.y == 0 && threadIdx.x == 0 && dst_labels) dst_labels[blockIdx.x] = src_labels[i];
+	if (blockIdx.y == 0 && lane == 0 && dst_labels) dst_labels[r] = src_labels[i];
 }
 
 static int gather_rows_on(hipStream_t stream, const char *who, float *dst, int64_t ldd, int64_t dst_plane_stride, const float *src, int64_t lds,
@@ -387,9 +387,9 @@ static int gather_rows_on(hipStream_t stream, const char *who, float *dst, int64
 			return fail(CNET_ERR_INVALID_ARGUMENT, "%s: index %d of row %d outside the table of %d rows", who, pinned_idx[r], r, src_rows);
 	const bool vec = cols % 4 == 0 && ldd % 4 == 0 && lds % 4 == 0 && dst_plane_stride % 4 == 0 && src_plane_stride % 4 == 0 && aligned16(dst) &&
 			aligned16(src);
-	dim3 grid((unsigned) rows, (unsigned) planes);
+	dim3 grid((unsigned) ((rows + 3) / 4), (unsigned) planes);
 	hipLaunchKernelGGL(gather_rows_kernel, grid, dim3(256), 0, stream, dst, (long) ldd, (long) dst_plane_stride, src, (long) lds,
-			(long) src_plane_stride, src_rows, pinned_idx, dst_labels, src_labels, cols, vec ? 1 : 0);
+			(long) src_plane_stride, src_rows, pinned_idx, dst_labels, src_labels, rows, cols, vec ? 1 : 0);
 	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
