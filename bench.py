@@ -150,35 +150,35 @@ def kernel_suite(steps):
 
     lines = []
 
-    def hbm(name, shape, bytes_per_elem, elems, fn, extra_bytes=0):
+    def hbm(kid, name, shape, bytes_per_elem, elems, fn, extra_bytes=0):
         ms = timed(fn)
         gbs = (bytes_per_elem * elems + extra_bytes) / ms / 1e6
-        lines.append({"kernel": name, "shape": shape, "ms": round(ms, 4), "roofline": {
+        lines.append({"id": kid, "kernel": name, "shape": shape, "ms": round(ms, 4), "roofline": {
             "bound": "hbm", "achieved": round(gbs, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(gbs / 8000.0, 4),
             "bytes_per_complex_element": bytes_per_elem}})
 
-    def mfma(name, shape, flops, fn):
+    def mfma(kid, name, shape, flops, fn):
         ms = timed(fn, warm=20)  # millisecond launches: the clocks settle within a few of them
         tf = flops / ms / 1e9
-        lines.append({"kernel": name, "shape": shape, "ms": round(ms, 4), "roofline": {
+        lines.append({"id": kid, "kernel": name, "shape": shape, "ms": round(ms, 4), "roofline": {
             "bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}})
 
     # config 3: FourierTrans n = 4096, batch 1024 (3 complex GEMMs against the twiddle matrix)
     Bf, nf = 1024, 4096
     x, y, g, dx = cmat(Bf, nf), ops.CMat.empty(Bf, nf), grad(Bf, nf), ops.Grad.empty(Bf, nf)
-    mfma("cdft_fwd", [Bf, nf], 8.0 * Bf * nf * nf, lambda: ops.dft_fwd(x, y))
-    mfma("cdft_bwd", [Bf, nf], 16.0 * Bf * nf * nf, lambda: ops.dft_bwd(g, dx))
+    mfma("cdft_fwd", "cdft_fwd", [Bf, nf], 8.0 * Bf * nf * nf, lambda: ops.dft_fwd(x, y))
+    mfma("cdft_bwd", "cdft_bwd", [Bf, nf], 16.0 * Bf * nf * nf, lambda: ops.dft_bwd(g, dx))
     xr = ops.CMat.from_host(rs.randn(Bf, nf).astype(np.float32), np.zeros((Bf, nf), np.float32))
     # a quarter of the full transform's flops: columns 0..n/2 only, and two real products per complex one (the imaginary
     # plane of the samples is neither read nor multiplied)
-    mfma("cdft_fwd of real samples (columns 0..n/2 by the product, the rest as conjugates; two real products per complex one; flops executed)",
+    mfma("cdft_fwd_real", "cdft_fwd of real samples (columns 0..n/2 by the product, the rest as conjugates; two real products per complex one; flops executed)",
          [Bf, nf], 4.0 * Bf * nf * (nf // 2 + 4), lambda: ops.dft_fwd_real_input(xr, y))
     del xr
     # TriangFourier: only the pairs in <= out contribute, n (n + 1) / 2 complex multiply-adds per row
     tri = nf * (nf + 1) / 2.0
-    mfma("ctriang_dft_fwd (useful flops: upper triangle only)", [Bf, nf], 8.0 * Bf * tri, lambda: ops.triang_dft_fwd(x, y))
-    mfma("ctriang_dft_bwd (useful flops: upper triangle only)", [Bf, nf], 16.0 * Bf * tri, lambda: ops.triang_dft_bwd(g, dx))
+    mfma("ctriang_fwd", "ctriang_dft_fwd (useful flops: upper triangle only)", [Bf, nf], 8.0 * Bf * tri, lambda: ops.triang_dft_fwd(x, y))
+    mfma("ctriang_bwd", "ctriang_dft_bwd (useful flops: upper triangle only)", [Bf, nf], 16.0 * Bf * tri, lambda: ops.triang_dft_bwd(g, dx))
     del x, y, g, dx
 
     # config 5 activation shape [8192 x 4096]: 256 MiB per complex matrix, so every operand streams from HBM
@@ -187,41 +187,41 @@ def kernel_suite(steps):
     n = R * Cc
     u, v, w1 = cmat(R, Cc), cmat(R, Cc), cmat(1, Cc)
     yy, g, du, dv, dw1 = ops.CMat.empty(R, Cc), grad(R, Cc), ops.Grad.empty(R, Cc), ops.Grad.empty(R, Cc), ops.Grad.empty(1, Cc)
-    hbm("plain copy of one plane (practical HBM ceiling)", [R, Cc], 8, n, lambda: ops.copy2d(u.re, yy.re))
-    hbm("cgelu_fwd", [R, Cc], 16, n, lambda: ops.gelu_fwd(u, yy))
-    hbm("cgelu_bwd", [R, Cc], 40, n, lambda: ops.gelu_bwd(u, g, du))
+    hbm("copy", "plain copy of one plane (practical HBM ceiling)", [R, Cc], 8, n, lambda: ops.copy2d(u.re, yy.re))
+    hbm("cgelu_fwd", "cgelu_fwd", [R, Cc], 16, n, lambda: ops.gelu_fwd(u, yy))
+    hbm("cgelu_bwd", "cgelu_bwd", [R, Cc], 40, n, lambda: ops.gelu_bwd(u, g, du))
     # the same pass for a conjugate gradient pair (real loss): g.dz read, dx.dz written, the dz* halves neither read nor written
-    hbm("cgelu_bwd, conjugate pair (dz only)", [R, Cc], 24, n, lambda: ops.gelu_bwd_sym(u, g, du, mirror=False))
-    hbm("crelu_fwd", [R, Cc], 16, n, lambda: ops.crelu_fwd(u, yy))
-    hbm("crelu_bwd", [R, Cc], 40, n, lambda: ops.crelu_bwd(u, g, du))
-    hbm("residual_fwd", [R, Cc], 24, n, lambda: ops.residual_fwd(u, v, yy))
-    hbm("residual_bwd", [R, Cc], 48, n, lambda: ops.residual_bwd(g, du, dv))
-    hbm("residual_bwd, conjugate pair (dz only)", [R, Cc], 24, n, lambda: ops.residual_bwd_sym(g, du, dv, mirror=False))
-    hbm("hadamard_fwd (shared weights)", [R, Cc], 16, n, lambda: ops.hadamard_fwd(u, w1, yy, True))
-    hbm("hadamard_bwd (shared weights, batch-summed dW)", [R, Cc], 40, n, lambda: ops.hadamard_bwd(u, w1, g, du, dw1, True),
+    hbm("cgelu_bwd_sym", "cgelu_bwd, conjugate pair (dz only)", [R, Cc], 24, n, lambda: ops.gelu_bwd_sym(u, g, du, mirror=False))
+    hbm("crelu_fwd", "crelu_fwd", [R, Cc], 16, n, lambda: ops.crelu_fwd(u, yy))
+    hbm("crelu_bwd", "crelu_bwd", [R, Cc], 40, n, lambda: ops.crelu_bwd(u, g, du))
+    hbm("residual_fwd", "residual_fwd", [R, Cc], 24, n, lambda: ops.residual_fwd(u, v, yy))
+    hbm("residual_bwd", "residual_bwd", [R, Cc], 48, n, lambda: ops.residual_bwd(g, du, dv))
+    hbm("residual_bwd_sym", "residual_bwd, conjugate pair (dz only)", [R, Cc], 24, n, lambda: ops.residual_bwd_sym(g, du, dv, mirror=False))
+    hbm("hadamard_fwd", "hadamard_fwd (shared weights)", [R, Cc], 16, n, lambda: ops.hadamard_fwd(u, w1, yy, True))
+    hbm("hadamard_bwd", "hadamard_bwd (shared weights, batch-summed dW)", [R, Cc], 40, n, lambda: ops.hadamard_bwd(u, w1, g, du, dw1, True),
         extra_bytes=16 * Cc)
-    hbm("hadamard_bwd, conjugate pair (shared weights, dz only)", [R, Cc], 24, n,
+    hbm("hadamard_bwd_sym", "hadamard_bwd, conjugate pair (shared weights, dz only)", [R, Cc], 24, n,
         lambda: ops.hadamard_bwd_sym(u, w1, g, du, dw1, True, mirror=False), extra_bytes=8 * Cc)
     # fused pairs of layers: one pass where two were, the intermediate values written but not read back
-    hbm("hadamard + cgelu fwd, one pass (shared weights; h and gelu(h) written)", [R, Cc], 24, n,
+    hbm("hadamard_cgelu_fwd", "hadamard + cgelu fwd, one pass (shared weights; h and gelu(h) written)", [R, Cc], 24, n,
         lambda: ops.hadamard_gelu_fwd(u, w1, yy, v, True), extra_bytes=8 * Cc)
-    hbm("cgelu_bwd + hadamard_bwd, one pass, conjugate pair (shared weights, dz only, dh not kept)", [R, Cc], 24, n,
+    hbm("hadamard_cgelu_bwd_sym", "cgelu_bwd + hadamard_bwd, one pass, conjugate pair (shared weights, dz only, dh not kept)", [R, Cc], 24, n,
         lambda: ops.hadamard_gelu_bwd_sym(u, w1, g, None, du, dw1, True, mirror=False), extra_bytes=8 * Cc)
-    hbm("residual_bwd (two consumers) + cgelu_bwd, one pass, conjugate pair (dz only)", [R, Cc], 40, n,
+    hbm("residual_cgelu_bwd_sym", "residual_bwd (two consumers) + cgelu_bwd, one pass, conjugate pair (dz only)", [R, Cc], 40, n,
         lambda: ops.residual_gelu_bwd_sym(g, dv, u, du, None, ops.Grad([yy.re, yy.im, yy.re, yy.im]), mirror=False))
     loss = capi.empty(R)
-    hbm("l2out_fwd", [R, Cc], 8, n, lambda: ops.l2out_fwd(u, loss))
-    hbm("l2out_bwd", [R, Cc], 24, n, lambda: ops.l2out_bwd(u, du))
-    hbm("l2out_bwd, conjugate pair (dz only)", [R, Cc], 16, n, lambda: ops.l2out_bwd_sym(u, du, mirror=False))
+    hbm("l2out_fwd", "l2out_fwd", [R, Cc], 8, n, lambda: ops.l2out_fwd(u, loss))
+    hbm("l2out_bwd", "l2out_bwd", [R, Cc], 24, n, lambda: ops.l2out_bwd(u, du))
+    hbm("l2out_bwd_sym", "l2out_bwd, conjugate pair (dz only)", [R, Cc], 16, n, lambda: ops.l2out_bwd_sym(u, du, mirror=False))
     s_ = capi.empty(R)
-    hbm("l2norm_fwd (SoftMax)", [R, Cc], 16, n, lambda: ops.l2norm_fwd(u, yy, s_))
-    hbm("l2norm_bwd (SoftMax)", [R, Cc], 40, n, lambda: ops.l2norm_bwd(u, s_, g, du))
-    hbm("l2norm_bwd (SoftMax), conjugate pair (dz only)", [R, Cc], 24, n, lambda: ops.l2norm_bwd_sym(u, s_, g, du, mirror=False))
-    hbm("sgd_update", [n], 32, n, lambda: ops.sgd_update(u, du.planes[2], du.planes[3], 1e-9))
-    hbm("adam_update", [n], 48, n, lambda: ops.adam_update(u, du.planes[0], du.planes[1], du.planes[2], du.planes[3], 1e-9, 0.9, 3))
-    hbm("zero 4 gradient planes", [R, Cc], 16, n, lambda: [p.owner.zero() for p in du.planes])
+    hbm("l2norm_fwd", "l2norm_fwd (SoftMax)", [R, Cc], 16, n, lambda: ops.l2norm_fwd(u, yy, s_))
+    hbm("l2norm_bwd", "l2norm_bwd (SoftMax)", [R, Cc], 40, n, lambda: ops.l2norm_bwd(u, s_, g, du))
+    hbm("l2norm_bwd_sym", "l2norm_bwd (SoftMax), conjugate pair (dz only)", [R, Cc], 24, n, lambda: ops.l2norm_bwd_sym(u, s_, g, du, mirror=False))
+    hbm("sgd_update", "sgd_update", [n], 32, n, lambda: ops.sgd_update(u, du.planes[2], du.planes[3], 1e-9))
+    hbm("adam_update", "adam_update", [n], 48, n, lambda: ops.adam_update(u, du.planes[0], du.planes[1], du.planes[2], du.planes[3], 1e-9, 0.9, 3))
+    hbm("zero4", "zero 4 gradient planes", [R, Cc], 16, n, lambda: [p.owner.zero() for p in du.planes])
     out1 = ops.Plane.empty(1, Cc)
-    hbm("batch_sum (one plane)", [R, Cc], 4, n, lambda: ops.batch_sum(u.re, out1))
+    hbm("batch_sum", "batch_sum (one plane)", [R, Cc], 4, n, lambda: ops.batch_sum(u.re, out1))
     del u, v, yy, g, du, dv
 
     # config 5: CrossEntropy over 32768 logits (rows reduced from 8192 to 2048 to keep the suite short)
@@ -231,10 +231,10 @@ def kernel_suite(steps):
     labels = ops.ints(rs.randint(0, Cc, R))
     s_, l_, am = capi.empty(R), capi.empty(R), capi.empty(R, np.int32)
     dz = ops.Grad.empty(R, Cc)
-    hbm("cross_entropy_fwd (loss, argmax; no normalised output)", [R, Cc], 8, n,
+    hbm("ce_fwd", "cross_entropy_fwd (loss, argmax; no normalised output)", [R, Cc], 8, n,
         lambda: ops.cross_entropy_fwd(z, labels, s_, l_, am, None), extra_bytes=4 * R)
-    hbm("cross_entropy_bwd", [R, Cc], 24, n, lambda: ops.cross_entropy_bwd(z, s_, labels, dz))
-    hbm("cross_entropy_bwd, conjugate pair (dz only)", [R, Cc], 16, n, lambda: ops.cross_entropy_bwd_sym(z, s_, labels, dz, mirror=False))
+    hbm("ce_bwd", "cross_entropy_bwd", [R, Cc], 24, n, lambda: ops.cross_entropy_bwd(z, s_, labels, dz))
+    hbm("ce_bwd_sym", "cross_entropy_bwd, conjugate pair (dz only)", [R, Cc], 16, n, lambda: ops.cross_entropy_bwd_sym(z, s_, labels, dz, mirror=False))
     return lines
 
 
@@ -314,13 +314,14 @@ def train_lines(steps):
         line = _train_bench("readme", batch, n, "frozen_input", "on_device")
         if line is None:
             return None
-        # the faster of two runs: the loop at batch 4096 is bound by the host's link, which other devices of the host share
-        # (one run in a dozen reads twice the time of the others)
+        # two runs, both reported (`ms_per_step_runs`), the faster one kept as the figure: the loop at batch 4096 is bound by
+        # the host's link, which other devices of the host share (one run in a dozen reads twice the time of the others)
         again = _train_bench("readme", batch, n, "frozen_input", "on_device")
         key = "ms_per_step_prefetch_loss_read_one_step_late"
+        both_runs = [line[key]] + ([again[key]] if again is not None else [])
         if again is not None and again[key] < line[key]:
             line = again
-        line["runs"] = 2
+        line["ms_per_step_runs"] = both_runs
         # configs[0] states real samples (imaginary parts 0), whose imaginary plane is cleared on the device instead of
         # sent; beside it the same loop on samples with uniform imaginary parts, both planes travelling
         both = _train_bench("readme", batch, n, "complex_samples")
@@ -558,6 +559,12 @@ def main():
         capi.call("cnet_cgemm_set_products", 4)
         return res
 
+    def sig(v, digits=3):
+        """three significant digits: the line has to fit the 8 kB of output the driver's record keeps"""
+        return float("%.*g" % (digits, v)) if isinstance(v, float) else v
+
+    short = {"linear_fwd": "fwd", "linear_bwd_input": "bwd_input", "linear_bwd_weight": "bwd_weight"}
+    roofline["launches"] = {short[k]: {"ms": v["ms"], "tflops": v["tflops"]} for k, v in roofline.pop("all_launches").items()}
     out = {
         "metric": "complex-Linear fwd+bwd TFLOP/s (% fp32 MFMA peak); train samples/sec",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -573,36 +580,64 @@ def main():
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:   # the flag leaves the headline alone (profiled runs)
-        out["conjugate_gradient_pair"] = conjugate_pair_step()
+        # Everything below is rounded to three significant digits and keyed tersely; `python bench.py --suite kernels |
+        # token_model | train` print the same measurements one verbose line each.
+        pair = conjugate_pair_step()
         three = three_products_step()
         capi.call("cnet_cgemm_set_products", args.products)
         out["cpu_baseline"] = cpu_baseline()
+        # the step through the entry points for a conjugate gradient pair: 3 complex products executed instead of 5
+        out["conjugate_gradient_pair"] = {"ms": sig(pair["ms_per_step"]), "products": 3, "tflops_executed": sig(pair["tflops_executed"])}
         train = train_lines(300)
-        if train:   # the other half of the metric: training steps of the configs[0] net through the C++ facade
-            # ms_per_step: batches staged on the upload stream, every step's loss read on the host one step later;
-            # ..._loss_read_before_next_step: the same with the host waiting for each loss before it queues the next step
-            out["train"] = [{"workload": t["workload"], "batch": t["batch"],
-                             "ms_per_step": t["ms_per_step_prefetch_loss_read_one_step_late"],
-                             "samples_per_sec": t["samples_per_sec_prefetch_loss_read_one_step_late"],
-                             "samples_per_sec_loss_read_before_next_step": t["samples_per_sec_prefetch"],
-                             "samples_per_sec_data_input_not_trainable": t["samples_per_sec_data_input_not_trainable"],
-                             # the reader's samples kept in device memory: a batch travels as 4 bytes per sample
-                             "samples_per_sec_samples_stored_on_device": t.get("samples_per_sec_samples_stored_on_device"),
-                             "samples_per_sec_copy_inside_forward": t["samples_per_sec_copy_in_forward"],
-                             "samples": t.get("samples"), "upload_bytes_per_step": t.get("upload_bytes_per_step"),
-                             "samples_per_sec_complex_samples": t.get("samples_per_sec_complex_samples")} for t in train]
+        if train:
+            # The other half of the metric: training steps of the configs[0] net (FourierTrans 784, Hadamard, CGelu, Linear
+            # 784 -> 10, CrossEntropy; SGD) through the C++ facade, upload of every batch and read-back of every loss included.
+            # ms / sps: real samples fed from the host, the next batch travelling under the current step, each loss read one
+            # step late; ms_runs: that figure in each of the two runs (the faster is reported); sps_wait: the host waits for
+            # each loss before the next step; sps_sync: copy inside gpuForward; sps_dev: the reader's samples stored on the
+            # device (a batch travels as indices); sps_cplx: complex samples (both planes travel); up_B: bytes sent per step
+            out["train"] = [{"batch": t["batch"], "ms": sig(t["ms_per_step_prefetch_loss_read_one_step_late"]),
+                             "ms_runs": [sig(v) for v in t["ms_per_step_runs"]],
+                             "sps": sig(t["samples_per_sec_prefetch_loss_read_one_step_late"]),
+                             "sps_wait": sig(t["samples_per_sec_prefetch"]),
+                             "sps_sync": sig(t["samples_per_sec_copy_in_forward"]),
+                             "sps_dev": sig(t.get("samples_per_sec_samples_stored_on_device")),
+                             "sps_cplx": sig(t.get("samples_per_sec_complex_samples")),
+                             "up_B": t.get("upload_bytes_per_step")} for t in train]
         # the other configurations and kernels of the hot path, each bounded to a few seconds
         del x, w, g, y, dx, dw
+
+        def stack_brief(t):
+            # configs[3] through the C++ facade: 10 SGD steps, data and targets uploaded and the loss read back every step
+            return {"products_per_linear": t["complex_products_per_linear"], "ms": sig(t["ms_per_step"]),
+                    "ms_after_first": sig(t["ms_per_step_after_the_first"]), "sps": sig(t["samples_per_sec"]),
+                    "tflops_executed": sig(t["gemm_tflops_executed"]),
+                    "loss_first_last": [sig(t["mean_loss_per_step"][0], 5), sig(t["mean_loss_per_step"][-1], 5)]}
+
+        def token_brief(t):
+            return {"pairs": "conj" if t["gradient_pairs"].startswith("dz*") else "both", "ms": sig(t["ms_per_step"]),
+                    "tok_s": sig(t["tokens_per_sec"]), "tflops_executed": sig(t["gemm_tflops_executed"]), "loss": sig(t["mean_loss"], 5)}
+
         stack = stack_lines(10)
         if stack:
-            out["configs3_residual_stack"] = stack
-        out["kernels"] = kernel_suite(20)
-        out["configs4_token_model"] = token_model_suite(3)
+            out["configs3_residual_stack"] = {"batch": 2048, "lr": STACK_LR, "runs": [stack_brief(t) for t in stack]}
+        # id: see kernel_suite; frac: of 157.3 TFLOP/s (cdft_*, ctriang_*: flops executed) or of 8 TB/s (algorithmic bytes)
+        out["kernels"] = [{"id": k["id"], "ms": sig(k["ms"]), "frac": sig(k["roofline"]["frac"])} for k in kernel_suite(20)]
+        out["configs4_token_model"] = [token_brief(t) for t in token_model_suite(3)]
+        # option, not the default: cnet_cgemm_set_products(3), three real products per complex one (6 M N K executed)
+        three_brief = {"ms": sig(three["ms_per_step"]), "tflops_as_8mnk": sig(three["tflops_counted_as_8mnk"]),
+                       "tflops_executed": sig(three["tflops_executed"]),
+                       "launch_ms": {short[k]: sig(v["ms"]) for k, v in three["all_launches"].items()},
+                       "conjugate_gradient_pair_ms": sig(three["conjugate_gradient_pair"]["ms_per_step"])}
         stack3 = stack_lines(10, products=3)
         if stack3:
-            three["configs3_residual_stack"] = stack3[0]
-        three["configs4_token_model"] = token_model_suite(3, products=3)[0]
-        out["three_real_products_per_complex_product"] = three
+            three_brief["configs3_residual_stack"] = stack_brief(stack3[0])
+        three_brief["configs4_token_model"] = token_brief(token_model_suite(3, products=3)[0])
+        out["three_real_products"] = three_brief
+    line = json.dumps(out, separators=(",", ":"))
+    if len(line) > 7000:
+        sys.stderr.write("bench.py: the line is %d bytes long; the driver's record keeps 8 kB\n" % len(line))
+    print(line)
     print(json.dumps(out))
 
 

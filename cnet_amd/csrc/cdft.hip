@@ -67,7 +67,13 @@ static int get_plan(int n, Twiddle *out, bool create) {
 	size_t plane = (size_t) n * t.ld;
 	CNET_HIP(hipMalloc((void **) &t.re, 2 * plane * sizeof(float)));
 	t.im = t.re + plane;
-	if (t.ld != n) CNET_HIP(hipMemsetAsync(t.re, 0, 2 * plane * sizeof(float), rt().stream));
+	if (t.ld != n) {
+		const hipError_t e = hipMemsetAsync(t.re, 0, 2 * plane * sizeof(float), rt().stream);
+		if (e != hipSuccess) {
+			hipFree(t.re);  // not in the table yet: nothing else would free the planes
+			return hip_fail(e, "hipMemsetAsync(twiddle planes)");
+		}
+	}
 	const long total = (long) n * n;
 	hipLaunchKernelGGL(twiddle_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, rt().stream, t.re, t.im, n, t.ld, 0);
 	g_twiddles[n] = t;  // owned by the table from here on, whatever the launch reports
@@ -85,7 +91,14 @@ static int get_triangular(int n, Twiddle *out) {
 	const size_t plane = (size_t) n * slot.ld;
 	CNET_HIP(hipMalloc((void **) &slot.tri_re, 2 * plane * sizeof(float)));
 	slot.tri_im = slot.tri_re + plane;
-	if (slot.ld != n) CNET_HIP(hipMemsetAsync(slot.tri_re, 0, 2 * plane * sizeof(float), rt().stream));
+	if (slot.ld != n) {
+		const hipError_t e = hipMemsetAsync(slot.tri_re, 0, 2 * plane * sizeof(float), rt().stream);
+		if (e != hipSuccess) {
+			hipFree(slot.tri_re);  // the slot must not keep planes that were never filled
+			slot.tri_re = slot.tri_im = nullptr;
+			return hip_fail(e, "hipMemsetAsync(triangular twiddle planes)");
+		}
+	}
 	const long total = (long) n * n;
 	hipLaunchKernelGGL(twiddle_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, rt().stream, slot.tri_re, slot.tri_im, n,
 			slot.ld, 1);

@@ -1489,7 +1489,10 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_opera
 		// efficiency above that of the large ones
 		return 1.0 / (inv2048 + slope * std::max(0.0, 1.0 / K - 1.0 / 2048));
 	};
-	const double flop_per_us_per_unit = 256.0 * 2.4e3;  // 256 flop per clock at 2.4 GHz
+	// 256 flop per clock and compute unit at the device's engine clock (kHz -> cycles per microsecond), as cnet_get_device_info
+	// reports it; 2.4 GHz when the driver gives none
+	const int khz = cnet::rt().prop.clockRate;
+	const double flop_per_us_per_unit = 256.0 * (khz > 0 ? khz * 1e-3 : 2.4e3);
 	const int nchunks = (a.K + KC - 1) / KC;
 	const bool tail_possible = forced_tail != 0 && a.K % KC == 0 && !a.tri && batch == 1;
 	int best = 3, best_tail = 0, best_cuts = 1;
@@ -1791,6 +1794,8 @@ int cnet_cgemm_batched(int a_kmajor, int b_kmajor, int conj_a, int conj_b, int M
 
 int cnet_cgemm_set_products(int n) {
 	CNET_CHECK_ARG(n == 3 || n == 4);
+	if (cnet::rt().capturing && (n == 3) != three_products())
+		return cnet::fail(CNET_ERR_UNSUPPORTED, "cnet_cgemm_set_products: not between cnet_graph_begin and cnet_graph_end");
 	g_three_products = n == 3;
 	return CNET_OK;
 }

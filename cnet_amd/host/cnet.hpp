@@ -269,12 +269,12 @@ class InputBatch : public Batch {
 		imag_clean_ = true;
 	}
 	void release() {
+		if (indices_) cnet_host_free(indices_);  // (a batch of dimension 0 has indices and no planes)
+		indices_ = NULL;
 		if (!real_data_) return;
 		if (pinned_) cnet_host_free(real_data_);  // waits for copies still reading it
 		else ::operator delete(real_data_);
 		real_data_ = imag_data_ = NULL;
-		if (indices_) cnet_host_free(indices_);
-		indices_ = NULL;
 	}
 	void settle() {  // before the host writes the planes again
 		if (ticket_ >= 0) {  // waits for that copy only: a copy out of another batch may still be running
@@ -313,7 +313,7 @@ public:
 			void *p = NULL;
 			if (cnet_host_alloc((size_t) batch_size_ * sizeof(int32_t), &p) == CNET_OK && p) {
 				indices_ = (int32_t *) p;
-				std::copy(o.indices_, o.indices_ + batch_size_, indices_);
+				std::copy(o.indices_, o.indices_ + current_pos_, indices_);  // only the filled entries hold values
 				resident_ = o.resident_;
 			}
 		}

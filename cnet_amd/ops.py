@@ -35,9 +35,15 @@ class Plane:
     def sub(self, col0, cols):
         return Plane(self.ptr + 4 * col0, self.rows, cols, self.ld, self.owner)
 
+    def rows_from(self, row0, rows):
+        """rows row0 .. row0 + rows of the same columns, without copying"""
+        return Plane(self.ptr + 4 * row0 * self.ld, rows, self.cols, self.ld, self.owner)
+
     def host(self):
         full = self.owner.download().reshape(-1)
         base = (self.ptr - self.owner.ptr) // 4
+        if self.ld == self.cols:
+            return full[base:base + self.rows * self.cols].reshape(self.rows, self.cols)
         idx = base + np.arange(self.rows)[:, None] * self.ld + np.arange(self.cols)[None, :]
         return full[idx]
 
@@ -58,6 +64,9 @@ class CMat:
 
     def sub(self, col0, cols):
         return CMat(self.re.sub(col0, cols), self.im.sub(col0, cols))
+
+    def rows_from(self, row0, rows):
+        return CMat(self.re.rows_from(row0, rows), self.im.rows_from(row0, rows))
 
     def host(self):
         return self.re.host(), self.im.host()
@@ -81,6 +90,9 @@ class Grad:
 
     def sub(self, col0, cols):
         return Grad([p.sub(col0, cols) for p in self.planes])
+
+    def rows_from(self, row0, rows):
+        return Grad([p.rows_from(row0, rows) for p in self.planes])
 
     def host(self):
         return [p.host() for p in self.planes]

@@ -232,7 +232,8 @@ int cnet_clinear_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg
  *      kernel and the kernel for unaligned operands always use 4.
  * Process-wide; takes effect with the next product that is queued (a recorded graph keeps the kernels it was recorded
  * with).  The environment variable CNET_CGEMM_3M=0 / 1 sets the initial value.
- * Returns CNET_ERR_INVALID_ARGUMENT for any other n. */
+ * Returns CNET_ERR_INVALID_ARGUMENT for any other n, and CNET_ERR_UNSUPPORTED for a change between cnet_graph_begin and
+ * cnet_graph_end (one recording would otherwise hold products of both kinds). */
 int cnet_cgemm_set_products(int n);
 int cnet_cgemm_get_products(void);
 
@@ -363,9 +364,10 @@ int cnet_batch_sum(const float *src, int64_t lds, float *dst, int rows, int cols
 /* cnet_batch_sum for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc); it has no counterpart upstream.  Same arguments, same kernels and bit-identical
  * results; the partial sums of its first stage go to a 2 MiB array that is part of the library's image on each device
- * instead of the library workspace, so the call never allocates or frees.  Limit: slabs x cols <= 524288 floats, which
- * holds for every cols <= 524288 (slabs = min(256, w x compute units / ceil(cols / 256)), w = 8 for planes of 2^24 elements and more, else 4; at most rows / 4); beyond it
- * the call returns CNET_ERR_UNSUPPORTED.  All calls on one device share the array: calls that overlap in time (two
+ * instead of the library workspace, so the call never allocates or frees.  Limit: slabs x cols <= 524288 floats, with
+ * slabs = max(1, min(256, w x compute units / ceil(cols / 256))), w = 8 for planes of 2^24 elements and more, else 4, and at
+ * most ceil(rows / 4).  On a device with up to 256 compute units that holds for every cols <= 524288; a device with more
+ * units refuses some of the widest planes.  Beyond the limit the call returns CNET_ERR_UNSUPPORTED.  All calls on one device share the array: calls that overlap in time (two
  * streams, two host threads) race. */
 int cnet_batch_sum_noalloc(const float *src, int64_t lds, float *dst, int rows, int cols, int accumulate);
 /* dst[k][0..n[k]) += src[k][0..n[k]) for `count` dense arrays in one launch: what the loop over the input functions in
@@ -471,6 +473,26 @@ int cnet_embedding_fwd(const float *table_re, const float *table_im, int dim, in
                        float *y_re, float *y_im, int64_t ldy, int rows, int slots);
 int cnet_embedding_bwd(const int32_t *tokens, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
                        float *table_dzs_re, float *table_dzs_im, int dim, int vocab, int rows, int slots, int accumulate);
+
+/* ---- Tuning overrides (environment variables).  None is needed for correct results or for the figures this library is
+ *      measured with; they exist so that tests and sweeps can send a shape to every kernel that could take it.  Each is
+ *      read ONCE per process, when the first launch that consults it is queued; results do not depend on them beyond
+ *      rounding (another block shape or cut groups the sums differently), and every path they select is deterministic.
+ *   CNET_CGEMM_TILE = 0..3       block shape of the matrix kernels: 128x128, 64x128, 128x64, 64x64 (default: cost model)
+ *   CNET_CGEMM_TAIL = 0 | 1      never / whenever possible cut the blocks of a partly filled last round along K
+ *   CNET_CGEMM_KCUT = 0          cut a product along K only when half of the compute units would idle
+ *   CNET_CGEMM_KMODEL = 0        price every K with the efficiency table measured at K = 2048
+ *   CNET_CGEMM_COLSPLIT = 0      never split the last few columns of C off into a launch of their own
+ *   CNET_CGEMM_KREST = 0         never split the last K % 16 values of k off (the whole product takes the general kernel)
+ *   CNET_CGEMM_SKINNY = 0        small products on the block kernels instead of the small-C kernel
+ *   CNET_CGEMM_SKINNY_TILES = n  largest number of 16x16 tiles of C the small-C kernel takes (default 4 per compute unit)
+ *   CNET_CGEMM_SKINNY_W = 4|8|16 wavefronts per tile of the small-C kernel
+ *   CNET_CGEMM_SKINNY_TWO = 0    two small products of one call as two launches
+ *   CNET_CGEMM_3M = 0 | 1        initial value of cnet_cgemm_set_products (1: three real products per complex one)
+ *   CNET_STREAM_MIN_MB = n       footprint (MiB) from which an elementwise / row launch counts as streaming (default 256)
+ *   CNET_STREAM_POLICY = 0..3    cache policy of every streaming launch: plain, hint on loads and stores, hinted stores,
+ *                                hinted loads + device-scope stores (default: per kernel)
+ */
 
 #ifdef __cplusplus
 }

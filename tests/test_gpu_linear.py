@@ -18,7 +18,7 @@ SHAPES = [  # B, K, N
 
 @pytest.fixture(params=[3, 4], ids=["three_products", "four_products"])
 def products(request, gpu):
-    """Runs a test with the block kernels forming a complex product from three real ones (the default) and from four."""
+    """Runs a test with the block kernels forming a complex product from four real ones (the default) and from three."""
     lib = capi.load()
     before = lib.cnet_cgemm_get_products()
     capi.call("cnet_cgemm_set_products", request.param)

@@ -94,10 +94,13 @@ def test_token_model_reduced(gpu, port, conjugate_pairs):
     assert rel_c((model.d_table_re.host(), model.d_table_im.host()), (dt_r, dt_i)) < TOL
 
 
-def test_token_model_full_size_properties(gpu, port):
+@pytest.mark.parametrize("conjugate_pairs", [False, True])
+def test_token_model_full_size_properties(gpu, port, conjugate_pairs):
     """The fifth configuration at its full size (16 x 512 tokens, vocab 32768, dim 1024, hidden 4096), checked through
     what does not need the CPU path on all of it: the oracle on a subsample of logit rows, bit-identical repetition,
-    and a directional finite difference of the total loss along the gradient of the shared gate weights."""
+    rows of a weight gradient against complex128 sums over the whole batch, and a directional finite difference of the
+    total loss along the gradient of the shared gate weights.  Once with both halves of every gradient pair computed (as
+    upstream does) and once with the one-gradient entry points, whose elementwise kernels stream at this size."""
     B, S, D, H, V = 16, 512, 1024, 4096, 32768
     rs = np.random.RandomState(5)
 
@@ -107,7 +110,7 @@ def test_token_model_full_size_properties(gpu, port):
     P = {"table": nrm((2, V, D), 1.0), "gate": nrm((2, D), 0.05), "w1": nrm((2, H, D), D ** -0.5),
          "w2": nrm((2, D, H), H ** -0.5), "w3": nrm((2, V, D), D ** -0.5)}
     ids = rs.randint(0, V, (B, S)).astype(np.int32)
-    model = TokenModel(B, S, D, H, V, P).set_tokens(ids)
+    model = TokenModel(B, S, D, H, V, P, conjugate_pairs=conjugate_pairs).set_tokens(ids)
     model.forward()
     model.backward()
     loss0 = model.loss.download().copy()
@@ -125,6 +128,18 @@ def test_token_model_full_size_properties(gpu, port):
     assert np.allclose(loss0[rows], loss_o, rtol=2e-4, atol=2e-5)
     assert np.array_equal(model.argmax.download()[rows], pred_o)
     del lg, o
+
+    # rows of the first layer's weight gradient over the whole batch: dW[j] = sum_b G[b, j] x[b], dW*[j] = sum_b G*[b, j] conj(x[b])
+    # (impl/linear.h:76-107 upstream); with one gradient per value the dz* planes of G are not written and G* = conj(G)
+    picked = [0, 1, 2047, 4095]
+    du, hh = model.d_u.host(), model.h.host()
+    xh = hh[0].astype(np.float64) + 1j * hh[1]
+    gz = du[0][:, picked].astype(np.float64) + 1j * du[1][:, picked]
+    gs = np.conj(gz) if conjugate_pairs else du[2][:, picked].astype(np.float64) + 1j * du[3][:, picked]
+    dw = model.d_w1.host()
+    assert rel_c((dw[0][picked], dw[1][picked]), ((gz.T @ xh).real, (gz.T @ xh).imag)) < TOL / 10
+    assert rel_c((dw[2][picked], dw[3][picked]), ((gs.T @ np.conj(xh)).real, (gs.T @ np.conj(xh)).imag)) < TOL / 10
+    del du, hh, xh, dw
 
     # same bits on repetition
     model.forward()
