@@ -367,6 +367,8 @@ def main():
     ap.add_argument("--counter-pass", action="store_true",
                     help="short run for `rocprofv3 --pmc`: 3 launches of each GEMM kernel plus a plain copy kernel of "
                          "known size (256 MiB read, 256 MiB written) that calibrates FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--counter-launches", type=int, default=24,
+                    help="with --counter-pass: launches in a row of each GEMM kernel after the three calibration rounds")
     ap.add_argument("--products", type=int, choices=[3, 4], default=4,
                     help="real matrix products per complex one in the block kernels (cnet_cgemm_set_products) for the "
                          "headline step of this run; 4 is the library's default and what the driver's line is measured with")
@@ -428,8 +430,15 @@ def main():
         for _ in range(3):
             ops.copy2d(src, dst)
             step()
+        # then each launch `--counter-launches` times in a row: the collector reads its counters between dispatches, so a
+        # lone dispatch starts on a drained device (cold caches, first wavefronts placed one by one); the median of a run of
+        # equal dispatches is the kernel as the timed loop runs it
+        for fn, _ in launches.values():
+            for _ in range(args.counter_launches):
+                fn()
         capi.sync()
-        print(json.dumps({"counter_pass": True, "copy_bytes_read": rows * cols * 4, "copy_bytes_written": rows * cols * 4}))
+        print(json.dumps({"counter_pass": True, "copy_bytes_read": rows * cols * 4, "copy_bytes_written": rows * cols * 4,
+                          "launches_in_a_row": args.counter_launches}))
         return
 
     # no collector pauses inside the timed loops (one of 20 ms was seen to drain the queue in the middle of a loop)
@@ -439,19 +448,23 @@ def main():
     # Out of idle first: a device that has just been handed over runs its first ~25 steps (30 ms) of this workload up to 25 %
     # slower while its clocks come up (1.45 -> 1.18 ms per step, measured step by step with events).  Groups of 10 steps are
     # run until two in a row agree to 1 % (at most 0.5 s in all); the W warm-up steps and the K timed steps follow.
-    preroll, last = 0, None
-    t_pre = time.perf_counter()
-    while time.perf_counter() - t_pre < 0.5:
-        a, b = ev.event(), ev.event()
-        ev.record(a)
-        for _ in range(10):
-            step()
-        ev.record(b)
-        cur = ev.elapsed_ms(a, b)
-        preroll += 10
-        if last is not None and abs(cur - last) <= 0.01 * last:
-            break
-        last = cur
+    def settle(fn):
+        done, last = 0, None
+        t_pre = time.perf_counter()
+        while time.perf_counter() - t_pre < 0.5:
+            a, b = ev.event(), ev.event()
+            ev.record(a)
+            for _ in range(10):
+                fn()
+            ev.record(b)
+            cur = ev.elapsed_ms(a, b)
+            done += 10
+            if last is not None and abs(cur - last) <= 0.01 * last:
+                break
+            last = cur
+        return done
+
+    preroll = settle(step)
     for _ in range(args.warmup):
         step()
     capi.sync(); tsync()
@@ -509,6 +522,7 @@ def main():
             ops.linear_bwd_input_sym(gc, w, dx)
             ops.linear_bwd_weight_sym(gc, x, dw)
 
+        settle(step_sym)   # the host has just spent a while generating the pair: the device has gone idle
         for _ in range(args.warmup):
             step_sym()
         capi.sync()
@@ -528,6 +542,7 @@ def main():
         # Beside the headline (four real matrix products per complex one, as the metric's 8 M N K counts them): the same five
         # products with the block kernels forming each from three real ones (cnet_cgemm_set_products(3): 6 M N K executed).
         capi.call("cnet_cgemm_set_products", 3)
+        settle(step)
         for _ in range(args.warmup):
             step()
         capi.sync()
@@ -638,7 +653,6 @@ def main():
     if len(line) > 7000:
         sys.stderr.write("bench.py: the line is %d bytes long; the driver's record keeps 8 kB\n" % len(line))
     print(line)
-    print(json.dumps(out))
 
 
 if __name__ == "__main__":
