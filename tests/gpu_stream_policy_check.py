@@ -119,6 +119,9 @@ def results(shapes=SHAPES):
         S, loss, am = capi.empty(B), capi.empty(B), capi.empty(B, np.int32)
         norm = ops.CMat.empty(B, n)
         ops.cross_entropy_fwd(x, labels, S, loss, am, norm); keep(tag + " cross_entropy_fwd", S, loss, am, norm)
+        S1, loss1, am1 = capi.empty(B), capi.empty(B), capi.empty(B, np.int32)   # the pass that only reads
+        ops.cross_entropy_fwd(x, labels, S1, loss1, am1, None); keep(tag + " cross_entropy_fwd, no planes", S1, loss1, am1)
+        ops.l2out_fwd(x, loss1); keep(tag + " l2out_fwd", loss1)
         d = dest(); ops.cross_entropy_bwd(x, S, labels, d); keep(tag + " cross_entropy_bwd", d)
         for mirror in (True, False):
             d = dest(); ops.cross_entropy_bwd_sym(x, S, labels, d, mirror=mirror); keep(tag + " cross_entropy_bwd_sym mirror=%d" % mirror, d)
