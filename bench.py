@@ -284,6 +284,7 @@ def token_model_suite(steps, products=4):
 
 
 TRAIN_BENCH = os.path.join(ROOT, "cnet_amd", "bin", "train_bench")
+TOKEN_LR = 0.05
 
 
 def _train_bench(*args, env=None):
@@ -350,11 +351,24 @@ def stack_lines(steps=10, products=4):
     return out
 
 
+def token_facade_lines(steps=5):
+    """configs[4] through the C++ facade (one token per sample, SeqFourierTrans along the sequence): training steps, i.e.
+    upload of tokens and labels, forward, backward, SGD on the table and every weight, mean loss read back; with one
+    gradient per value (the facade's default) and with both halves of every pair."""
+    out = []
+    for mode in ((), ("both_halves",)):
+        line = _train_bench("token", 16, 512, 1024, 4096, 32768, steps, TOKEN_LR, *mode)
+        if line is None:
+            return None
+        out.append(line)
+    return out
+
+
 def train_suite(steps):
     lines = train_lines(steps)
     if lines is None:
         sys.exit("bench.py: cnet_amd/bin/train_bench is missing or failed; run __graft_entry__.build() first")
-    for l in lines + (stack_lines() or []):
+    for l in lines + (stack_lines() or []) + (token_facade_lines() or []):
         print(json.dumps(l))
 
 
@@ -638,7 +652,14 @@ def main():
             out["configs3_residual_stack"] = {"batch": 2048, "lr": STACK_LR, "runs": [stack_brief(t) for t in stack]}
         # id: see kernel_suite; frac: of 157.3 TFLOP/s (cdft_*, ctriang_*: flops executed) or of 8 TB/s (algorithmic bytes)
         out["kernels"] = [{"id": k["id"], "ms": sig(k["ms"]), "frac": sig(k["roofline"]["frac"])} for k in kernel_suite(20)]
-        out["configs4_token_model"] = [token_brief(t) for t in token_model_suite(3)]
+        # api "c": forward + backward as a sequence of C-ABI calls; api "facade": training steps (SGD included) through the
+        # C++ facade with one token per sample
+        out["configs4_token_model"] = [dict(token_brief(t), api="c") for t in token_model_suite(3)]
+        for t in token_facade_lines() or []:
+            out["configs4_token_model"].append({"api": "facade", "pairs": "conj" if t["gradient_pairs"].startswith("dz*") else "both",
+                                                "ms": sig(t["ms_per_step"]), "tok_s": sig(t["tokens_per_sec"]),
+                                                "tflops_executed": sig(t["gemm_tflops_executed"]),
+                                                "loss_first_last": [sig(t["mean_loss_per_step"][0], 5), sig(t["mean_loss_per_step"][-1], 5)]})
         # option, not the default: cnet_cgemm_set_products(3), three real products per complex one (6 M N K executed)
         three_brief = {"ms": sig(three["ms_per_step"]), "tflops_as_8mnk": sig(three["tflops_counted_as_8mnk"]),
                        "tflops_executed": sig(three["tflops_executed"]),

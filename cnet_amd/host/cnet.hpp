@@ -491,6 +491,8 @@ public:
 // node type ids of impl/cnet.h:31-44
 const int isHadamard = 1, isEmbedding = 2, isLinear = 3, isFourier = 4, isCrossEntropy = 5, isResidual = 6, isSoftMax = 7,
 		isInput = 8, isCrelu = 9, isGelu = 10, isL2Out = 11, isTrianFourier = 12;
+// not an upstream type (and not part of its .mod format): SeqFourierTrans below
+const int isSeqFourier = 64;
 
 class CFunc {
 	friend class CNet;
@@ -643,6 +645,31 @@ public:
 	FourierTrans(InSize n) : CFunc(n, OutSize(n.value())) {}
 	std::string getName() override { return "FourierTrans_" + std::to_string(uid_); }
 	int typeId() const override { return isFourier; }
+};
+
+// Not an upstream layer: a FourierTrans along an axis upstream's API cannot address.  Upstream transforms the flat vector
+// of ONE sample (impl/ft.h:37-80), and a Linear there acts on the whole flattened sample; a model that treats the positions
+// of a sequence alike (the same Linear for every token) has no spelling.  With one token per sample it has: an
+// EmbeddingBatch of batch x seq one-token samples, CEmbedding(dim, 1, vocab), and Hadamard / Linear / CGelu /
+// CrossEntropy as they are, row by row.  What is then missing is the one layer that mixes the tokens of a sequence, and
+// that is this one: the batch rows are taken in groups of `seq` consecutive rows (the positions of one sequence), and
+// each of the n channels is transformed along its group,
+//     y[g seq + p][c] = (1 / sqrt(seq)) sum_q x[g seq + q][c] e^{-2 pi i p q / seq},
+// FourierTrans(seq) applied to every (sequence, channel) column; backward dz = F g.dz, dz* = conj(F) g.dz* along the same
+// axis (impl/ft.h:57-79).  On the device one strided-batched matrix product against the seq x seq twiddle planes.
+// The batch must hold whole sequences (allocateOnGpu(B) with B a multiple of seq); the per-sample calls, which see one
+// row, refuse a net that contains it.  ModelSaver refuses it as well (upstream's file format has no such record).
+class SeqFourierTrans : public CFunc {
+	friend class CNet;
+	int seq_;
+	const float *f_re_ = NULL, *f_im_ = NULL;  // device: the twiddle planes of length seq (owned by the device library)
+	int f_ld_ = 0;
+public:
+	SeqFourierTrans(Uid uid, InSize n, int seq) : CFunc(uid, n, OutSize(n.value())), seq_(seq) { assert(seq > 0); }
+	SeqFourierTrans(InSize n, int seq) : CFunc(n, OutSize(n.value())), seq_(seq) { assert(seq > 0); }
+	int seq() const { return seq_; }
+	std::string getName() override { return "SeqFourierTrans_" + std::to_string(uid_); }
+	int typeId() const override { return isSeqFourier; }
 };
 
 class Hadamard : public CFunc {
@@ -1402,6 +1429,17 @@ private:
 			case isTrianFourier:
 				ck(cnet_ctriang_dft_plan(f->out_size_), "cnet_ctriang_dft_plan");
 				break;
+			case isSeqFourier: {
+				SeqFourierTrans *q = (SeqFourierTrans *) f;
+				if (f->slots_.size() != 1 || (int) rows != batch_ || batch_ % q->seq_ != 0)
+					throw std::invalid_argument(f->getName() + ": transforms along groups of " + std::to_string(q->seq_) +
+							" batch rows; the batch of " + std::to_string(batch_) + " must hold whole sequences of a batched operand");
+				if (batch_ / q->seq_ > 65535) throw std::invalid_argument(f->getName() + ": more than 65535 sequences in a batch");
+				ck(cnet_cdft_plan(q->seq_), "cnet_cdft_plan");
+				ck(cnet_cdft_twiddle(q->seq_, &q->f_re_, &q->f_im_), "cnet_cdft_twiddle");
+				q->f_ld_ = (q->seq_ + 3) / 4 * 4;
+				break;
+			}
 			case isSoftMax:
 				((SoftMax *) f)->d_s_ = dalloc<float>(rows);
 				break;
@@ -1540,6 +1578,13 @@ private:
 			ck(cnet_ctriang_dft_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_, 0),
 					"cnet_ctriang_dft_fwd");
 			break;
+		case isSeqFourier: {  // Y_g = F X_g for every sequence g: one strided-batched product, F shared (stride 0)
+			SeqFourierTrans *q = (SeqFourierTrans *) f;
+			const int S = q->seq_, n = f->out_size_;
+			ck(cnet_cgemm_batched(0, 1, 0, 0, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, zre(f, 0), zim(f, 0), n, (int64_t) S * n, f->out_re(),
+					f->out_im(), n, (int64_t) S * n, rows / S, 0), "cnet_cgemm_batched");
+			break;
+		}
 		case isCrelu:
 			ck(cnet_crelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_),
 					"cnet_crelu_fwd");
@@ -1724,6 +1769,23 @@ private:
 					ck(cnet_ctriang_dft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
 							"cnet_ctriang_dft_bwd");
 				break;
+			case isSeqFourier: {
+				// dX_g.dz = F G_g.dz and dX_g.dz* = conj(F) G_g.dz* (F is symmetric).  Of a conjugate pair only the dz planes of G
+				// hold values: dz* = conj(F) conj(G.dz), formed where something reads it on the device.
+				SeqFourierTrans *q = (SeqFourierTrans *) f;
+				const int S = q->seq_, n = f->out_size_;
+				ck(cnet_cgemm_batched(0, 1, 0, 0, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, u.g(0), u.g(1), u.len, (int64_t) S * u.len, a.g(0), a.g(1),
+						a.len, (int64_t) S * a.len, rows / S, acc), "cnet_cgemm_batched");
+				if (conjugate_gradients_) {
+					if (a.gs(2))
+						ck(cnet_cgemm_batched(0, 1, 1, 1, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, u.g(0), u.g(1), u.len, (int64_t) S * u.len,
+								a.g(2), a.g(3), a.len, (int64_t) S * a.len, rows / S, acc), "cnet_cgemm_batched");
+				} else {
+					ck(cnet_cgemm_batched(0, 1, 1, 0, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, u.g(2), u.g(3), u.len, (int64_t) S * u.len, a.g(2),
+							a.g(3), a.len, (int64_t) S * a.len, rows / S, acc), "cnet_cgemm_batched");
+				}
+				break;
+			}
 			case isCrelu:
 				if (conjugate_gradients_) {
 					ck(cnet_crelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,

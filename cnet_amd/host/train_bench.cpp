@@ -7,6 +7,9 @@
 //       BatchedDataReader; the loop of upstream cnet.cpp:119-150 in several input / read-back modes.
 //   train_bench stack n blocks B steps lr [both_halves]
 //       blocks x (Linear n -> n, CGelu, Residual), L2Out against targets, SGD (the residual stack workload).
+//   train_bench token batch seq dim hidden vocab steps lr [both_halves]
+//       the complex token model, one token per sample: CEmbedding -> SeqFourierTrans -> Hadamard gate -> Linear, CGelu,
+//       Linear -> Linear to the vocabulary -> CrossEntropy on the next token, SGD.
 #include <chrono>
 #include <cmath>
 #include <cstdio>
@@ -261,6 +264,73 @@ int run_stack(int n, int blocks, int B, int steps, float lr, bool both_halves) {
 	return 0;
 }
 
+// The complex token model with one token per sample: an EmbeddingBatch of batch x seq one-token samples, CEmbedding, the
+// transform along the sequence (SeqFourierTrans), a Hadamard gate with shared weights, Linear dim -> hidden, CGelu, Linear
+// hidden -> dim, Linear dim -> vocab, CrossEntropy on the next token (the last position of a sequence is labelled with its
+// first token).  One step = upload of the tokens and labels, forward, backward, SGD on the table and every weight, and the
+// read-back of the mean loss.
+int run_token(int Bq, int S, int D, int H, int V, int steps, float lr, bool both_halves) {
+	Gen rng(7);
+	const int R = Bq * S;
+	CNet net;
+	int emb = net.add(new CEmbedding(D, 1, V));
+	int mix = net.add(new SeqFourierTrans(InSize(D), S), {emb});
+	int gd = net.add(new CInput(OutSize(D)));
+	int had = net.add(new Hadamard(InSize(D), InSize(D)), {mix, gd});
+	int w1 = net.add(new CInput(OutSize(H * D)));
+	int l1 = net.add(new Linear(InSize(D), InSize(H * D)), {had, w1});
+	int ge = net.add(new CGelu(InSize(H)), {l1});
+	int w2 = net.add(new CInput(OutSize(D * H)));
+	int l2 = net.add(new Linear(InSize(H), InSize(D * H)), {ge, w2});
+	int w3 = net.add(new CInput(OutSize(V * D)));
+	int l3 = net.add(new Linear(InSize(D), InSize(V * D)), {l2, w3});
+	int ce = net.add(new CrossEntropy(InSize(V)), {l3});
+	if (both_halves) net.conjugateGradients(false);
+	rng.fill_normal(net[emb]->mutable_input()->real_, (size_t) 2 * V * D, 1.0);
+	rng.fill_normal(net[gd]->mutable_input()->real_, (size_t) 2 * D, 0.05);
+	rng.fill_normal(net[w1]->mutable_input()->real_, (size_t) 2 * H * D, 1.0 / std::sqrt((double) D));
+	rng.fill_normal(net[w2]->mutable_input()->real_, (size_t) 2 * D * H, 1.0 / std::sqrt((double) H));
+	rng.fill_normal(net[w3]->mutable_input()->real_, (size_t) 2 * V * D, 1.0 / std::sqrt((double) D));
+	((CEmbedding *) net[emb])->setInput({0});
+	net.allocateOnGpu(R);
+	std::vector<int> ids(R);
+	for (auto &t : ids) t = (int) (rng.next() % (uint64_t) V);
+	EmbeddingBatch batch(R, 1);
+	for (int r = 0; r < R; ++r) batch.add(std::vector<int>(1, ids[r]), ids[r / S * S + (r % S + 1) % S]);
+	CEmbedding *e = (CEmbedding *) net[emb];
+	CrossEntropy *c = (CrossEntropy *) net[ce];
+	std::vector<float> losses;
+	auto one = [&]() {
+		net.gpuForward(e, c, batch);
+		net.gpuBackward();
+		net.gpuUpdateInputs(lr / R);
+		losses.push_back(net.getLoss(c, NULL));
+	};
+	one();  // the first step pays the one-off growth of the library workspace and the twiddle planes
+	net.sync();
+	auto t0 = std::chrono::steady_clock::now();
+	for (int s = 0; s < steps; ++s) one();
+	net.sync();
+	const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+	std::string all;
+	for (float l : losses) {
+		char buf[64];
+		snprintf(buf, sizeof(buf), "%s%.6g", all.empty() ? "" : ", ", l);
+		all += buf;
+	}
+	// complex products executed per step: each Linear forward + one (conjugate pairs) or two per gradient; the transform
+	// forward + two backward
+	const double lin = 8.0 * R * ((double) D * H + (double) H * D + (double) D * V), dft = 8.0 * Bq * (double) S * S * D;
+	const double flops = (both_halves ? 5 : 3) * lin + 3 * dft;
+	printf("{\"workload\": \"configs[4] through the C++ facade: complex token model, one token per sample, fwd + bwd + SGD\", "
+		   "\"batch\": %d, \"seq\": %d, \"dim\": %d, \"hidden\": %d, \"vocab\": %d, \"steps\": %d, \"lr\": %g, "
+		   "\"gradient_pairs\": \"%s\", \"ms_per_step\": %.3f, \"tokens_per_sec\": %.1f, \"gemm_tflops_executed\": %.2f, "
+		   "\"mean_loss_per_step\": [%s], \"loss_of_uniform_guess\": %.4f}\n",
+			Bq, S, D, H, V, steps, (double) lr, both_halves ? "both halves computed" : "dz* written as conj(dz)", 1e3 * sec / steps,
+			R * steps / sec, flops * steps / sec / 1e12, all.c_str(), std::log((double) V));
+	return std::isfinite(losses.back()) ? 0 : 1;
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
@@ -273,10 +343,14 @@ int main(int argc, char **argv) {
 		if (what == "stack")
 			return run_stack(argc > 2 ? atoi(argv[2]) : 2048, argc > 3 ? atoi(argv[3]) : 8, argc > 4 ? atoi(argv[4]) : 2048,
 					argc > 5 ? atoi(argv[5]) : 10, argc > 6 ? (float) atof(argv[6]) : 0.01f, has(argc, argv, 7, "both_halves"));
+		if (what == "token")
+			return run_token(argc > 2 ? atoi(argv[2]) : 16, argc > 3 ? atoi(argv[3]) : 512, argc > 4 ? atoi(argv[4]) : 1024,
+					argc > 5 ? atoi(argv[5]) : 4096, argc > 6 ? atoi(argv[6]) : 32768, argc > 7 ? atoi(argv[7]) : 5,
+					argc > 8 ? (float) atof(argv[8]) : 0.05f, has(argc, argv, 9, "both_halves"));
 	} catch (const std::exception &e) {
 		fprintf(stderr, "train_bench: %s\n", e.what());
 		return 2;
 	}
-	fprintf(stderr, "usage: train_bench readme B steps [graphs] [both_halves] [frozen_input] [complex_samples] [on_device] | stack n blocks B steps lr [both_halves]\n");
+	fprintf(stderr, "usage: train_bench readme B steps [graphs] [both_halves] [frozen_input] [complex_samples] [on_device] | stack n blocks B steps lr [both_halves] | token batch seq dim hidden vocab steps lr [both_halves]\n");
 	return 64;
 }

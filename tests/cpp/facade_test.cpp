@@ -7,6 +7,7 @@
 //   facade_test resblock           residual stack with a second data input (L2 target), several SGD steps
 //   facade_test persample          the per-sample API (forward / backward(label) / updateInputs) on the device
 //   facade_test embedding          CEmbedding -> Linear -> CrossEntropy with an EmbeddingBatch
+//   facade_test token_model        one token per sample: CEmbedding -> SeqFourierTrans -> gate -> MLP -> logits -> CrossEntropy, with an SGD step
 //   facade_test adam               TriangFourier / CRelu net trained with the Adam-style step, batched and per sample
 //   facade_test saved_model <golden dir> <scratch dir>   upstream-written .mod files restored and run on the device
 //   facade_test pipeline [B steps]  reader -> page-locked batches -> device, with and without gpuPrefetch (same bits)
@@ -581,6 +582,223 @@ static void test_embedding() {
 	ErrAcc gt;
 	gt.add(net[emb]->input().dz_star_real_, on.at(oe)->in.dzs_re, 2 * vocab * dim);
 	report("embedding table dz* (scatter-add over the batch)", gt.value());
+}
+
+// ------------------------------------------------------------------------------------------------- complex token model
+// The fifth configuration at reduced size through the facade: one token per sample (EmbeddingBatch of batch x seq rows),
+// CEmbedding -> SeqFourierTrans (mixing along the sequence) -> Hadamard gate -> Linear, CGelu, Linear -> Linear to vocabulary
+// logits -> CrossEntropy on the next token; forward, backward, one SGD step, forward again.  The oracle is composed of the
+// upstream layers: FourierTrans(seq) applied to every (sequence, channel) column for the mixing layer (impl/ft.h:37-80),
+// one net run token by token for the rest (parameter gradients accumulate over the tokens as upstream's do over samples).
+static void test_token_model() {
+	const int Bq = 3, S = 8, D = 12, H = 20, V = 29, R = Bq * S;
+	const float lr = 0.05f;
+	orc::Rng rng(33);
+	std::vector<float> table((size_t) 2 * V * D), gate(2 * D), w1((size_t) 2 * H * D), w2((size_t) 2 * D * H), w3((size_t) 2 * V * D);
+	fill_normal(rng, table.data(), table.size(), 1.0);
+	fill_normal(rng, gate.data(), gate.size(), 0.7);
+	fill_normal(rng, w1.data(), w1.size(), 1.0 / std::sqrt((double) D));
+	fill_normal(rng, w2.data(), w2.size(), 1.0 / std::sqrt((double) H));
+	fill_normal(rng, w3.data(), w3.size(), 1.0 / std::sqrt((double) D));
+	std::vector<int> ids(R), labels(R);
+	for (auto &t : ids) t = (int) (rng.next() % V);
+	ids[5] = ids[2];  // a token that occurs twice in a sequence, and in two sequences
+	ids[S + 1] = ids[2];
+	for (int g = 0; g < Bq; ++g)
+		for (int q = 0; q < S; ++q) labels[g * S + q] = ids[g * S + (q + 1) % S];  // next token, wrapping within the sequence
+
+	for (int mode = 0; mode < 2; ++mode) {
+		const std::string tag = mode ? "both halves: " : "conjugate pairs: ";
+		CNet net;
+		auto emb = net.add(new CEmbedding(D, 1, V));
+		auto mix = net.add(new SeqFourierTrans(InSize(D), S), {emb});
+		auto gd = net.add(new CInput(OutSize(D)));
+		auto had = net.add(new Hadamard(InSize(D), InSize(D)), {mix, gd});
+		auto w1d = net.add(new CInput(OutSize(H * D)));
+		auto l1 = net.add(new Linear(InSize(D), InSize(H * D)), {had, w1d});
+		auto ge = net.add(new CGelu(InSize(H)), {l1});
+		auto w2d = net.add(new CInput(OutSize(D * H)));
+		auto l2 = net.add(new Linear(InSize(H), InSize(D * H)), {ge, w2d});
+		auto w3d = net.add(new CInput(OutSize(V * D)));
+		auto l3 = net.add(new Linear(InSize(D), InSize(V * D)), {l2, w3d});
+		auto ce = net.add(new CrossEntropy(InSize(V)), {l3});
+		std::copy(table.begin(), table.end(), net[emb]->mutable_input()->real_);
+		std::copy(gate.begin(), gate.end(), net[gd]->mutable_input()->real_);
+		std::copy(w1.begin(), w1.end(), net[w1d]->mutable_input()->real_);
+		std::copy(w2.begin(), w2.end(), net[w2d]->mutable_input()->real_);
+		std::copy(w3.begin(), w3.end(), net[w3d]->mutable_input()->real_);
+		((CEmbedding *) net[emb])->setInput({0});
+		if (mode) net.conjugateGradients(false);
+		if (mode == 0) {
+			expect("a batch that does not hold whole sequences is refused", throws<std::invalid_argument>([&] { net.allocateOnGpu(R + 1); }));
+		}
+		net.allocateOnGpu(R);
+
+		// ---- the oracle: the layers after the mixing, one token at a time
+		orc::Net ot;
+		int om = ot.add(orc::kInput, D, 0, 0, NULL, 0), og = ot.add(orc::kInput, D, 0, 0, NULL, 0);
+		int in2[2] = {om, og};
+		int oh = ot.add(orc::kHadamard, D, 0, 0, in2, 2);
+		int ow1 = ot.add(orc::kInput, H * D, 0, 0, NULL, 0);
+		in2[0] = oh; in2[1] = ow1;
+		int ol1 = ot.add(orc::kLinear, D, H * D, 0, in2, 2);
+		int oge = ot.add(orc::kGelu, H, 0, 0, &ol1, 1);
+		int ow2 = ot.add(orc::kInput, D * H, 0, 0, NULL, 0);
+		in2[0] = oge; in2[1] = ow2;
+		int ol2 = ot.add(orc::kLinear, H, D * H, 0, in2, 2);
+		int ow3 = ot.add(orc::kInput, V * D, 0, 0, NULL, 0);
+		in2[0] = ol2; in2[1] = ow3;
+		int ol3 = ot.add(orc::kLinear, D, V * D, 0, in2, 2);
+		int oc = ot.add(orc::kCrossEntropy, V, 0, 0, &ol3, 1);
+		std::copy(gate.begin(), gate.end(), ot.at(og)->in.re);
+		std::copy(w1.begin(), w1.end(), ot.at(ow1)->in.re);
+		std::copy(w2.begin(), w2.end(), ot.at(ow2)->in.re);
+		std::copy(w3.begin(), w3.end(), ot.at(ow3)->in.re);
+		std::vector<float> tab = table;  // the oracle's table: re plane, im plane
+		const std::vector<orc::cf> roots = orc::unity_roots(S);
+
+		EmbeddingBatch batch(R, 1);
+		for (int r = 0; r < R; ++r) batch.add(std::vector<int>(1, ids[r]), labels[r]);
+		CrossEntropy *cen = (CrossEntropy *) net[ce];
+		double first_loss[2] = {0, 0};
+		for (int step = 0; step < 2; ++step) {
+			net.gpuForward((CEmbedding *) net[emb], cen, batch);
+			const float mean = net.getLoss(cen, &batch);
+			// oracle forward: gather, transform every column, then the per-token net
+			std::vector<float> xr((size_t) R * D), xi((size_t) R * D), mr((size_t) R * D), mi((size_t) R * D);
+			for (int r = 0; r < R; ++r)
+				for (int c = 0; c < D; ++c) {
+					xr[(size_t) r * D + c] = tab[(size_t) ids[r] * D + c];
+					xi[(size_t) r * D + c] = tab[(size_t) V * D + (size_t) ids[r] * D + c];
+				}
+			std::vector<float> cr(S), ci(S), yr(S), yi(S);
+			for (int g = 0; g < Bq; ++g)
+				for (int c = 0; c < D; ++c) {
+					for (int q = 0; q < S; ++q) {
+						cr[q] = xr[(size_t) (g * S + q) * D + c];
+						ci[q] = xi[(size_t) (g * S + q) * D + c];
+					}
+					orc::dft_forward(S, cr.data(), ci.data(), yr.data(), yi.data());
+					for (int q = 0; q < S; ++q) {
+						mr[(size_t) (g * S + q) * D + c] = yr[q];
+						mi[(size_t) (g * S + q) * D + c] = yi[q];
+					}
+				}
+			if (step == 1) {  // after the update: the loss of the stepped model, row by row
+				double worst = 0, sum = 0;
+				for (int r = 0; r < R; ++r) {
+					std::copy(mr.begin() + (size_t) r * D, mr.begin() + (size_t) (r + 1) * D, ot.at(om)->in.re);
+					std::copy(mi.begin() + (size_t) r * D, mi.begin() + (size_t) (r + 1) * D, ot.at(om)->in.im);
+					ot.forward();
+					const double l = ot.loss(oc, labels[r]);
+					sum += l;
+					// (a batch keeps appending the losses it is handed, as upstream's does, impl/batch.h: the second pass follows the first)
+					worst = std::max(worst, std::fabs(l - batch.loss(R + r)) / std::max(1.0, std::fabs(l)));
+				}
+				report(tag + "loss per token after the SGD step", worst, 2e-4);
+				expect(tag + "the step lowered the mean loss", sum / R < first_loss[0] && mean < first_loss[1]);
+				break;
+			}
+			net.gpuBackward();
+			ErrAcc zm, gm, gx, lz;
+			double loss_err = 0, loss_sum = 0;
+			bool same_argmax = true;
+			std::vector<float> dm((size_t) 4 * R * D, 0.f);  // dz_re, dz_im, dzs_re, dzs_im of the mixing layer's result
+			std::vector<int> pred = net.getPredictions(cen);
+			for (int r = 0; r < R; ++r) {
+				std::copy(mr.begin() + (size_t) r * D, mr.begin() + (size_t) (r + 1) * D, ot.at(om)->in.re);
+				std::copy(mi.begin() + (size_t) r * D, mi.begin() + (size_t) (r + 1) * D, ot.at(om)->in.im);
+				ot.forward();
+				const double l = ot.loss(oc, labels[r]);
+				loss_sum += l;
+				loss_err = std::max(loss_err, std::fabs(l - batch.loss(r)));
+				same_argmax = same_argmax && ot.prediction(oc) == pred[r];
+				ot.backward(labels[r]);
+				const orc::Planes &hin = ot.at(oh)->in;
+				for (int p = 0; p < 4; ++p) {
+					const float *src = p == 0 ? hin.dz_re : p == 1 ? hin.dz_im : p == 2 ? hin.dzs_re : hin.dzs_im;
+					std::copy(src, src + D, dm.begin() + ((size_t) p * R + r) * D);
+				}
+				net.fetch(net[had], r);
+				zm.add(net[had]->input().real_, mr.data() + (size_t) r * D, D);   // the mixed row
+				zm.add(net[had]->input().imag_, mi.data() + (size_t) r * D, D);
+				gm.add(net[had]->input().dz_real_, hin.dz_re, D);
+				gm.add(net[had]->input().dz_imag_, hin.dz_im, D);
+				gm.add(net[had]->input().dz_star_real_, hin.dzs_re, D);
+				gm.add(net[had]->input().dz_star_imag_, hin.dzs_im, D);
+				net.fetch(net[ce], r);
+				lz.add(net[ce]->input().real_, ot.at(oc)->in.re, V);
+				lz.add(net[ce]->input().imag_, ot.at(oc)->in.im, V);
+			}
+			first_loss[0] = loss_sum / R;
+			first_loss[1] = mean;
+			report(tag + "rows mixed along the sequence", zm.value());
+			report(tag + "logits", lz.value());
+			report(tag + "loss per token", loss_err, 1e-4);
+			report(tag + "mean loss", std::fabs(mean - loss_sum / R), 1e-4);
+			expect(tag + "predicted tokens equal", same_argmax);
+			report(tag + "gradient that reaches the mixing layer", gm.value());
+			// oracle backward of the mixing layer, column by column; then the scatter-add into the table
+			std::vector<float> dx((size_t) 4 * R * D, 0.f), dtab((size_t) 2 * V * D, 0.f);
+			std::vector<float> up(4 * S), own(4 * S);
+			for (int g = 0; g < Bq; ++g)
+				for (int c = 0; c < D; ++c) {
+					for (int p = 0; p < 4; ++p)
+						for (int q = 0; q < S; ++q) up[p * S + q] = dm[((size_t) p * R + g * S + q) * D + c];
+					std::fill(own.begin(), own.end(), 0.f);
+					orc::GradIn gi;
+					gi.dz_re = up.data(); gi.dz_im = up.data() + S; gi.dzs_re = up.data() + 2 * S; gi.dzs_im = up.data() + 3 * S;
+					orc::GradOut go;
+					go.dz_re = own.data(); go.dz_im = own.data() + S; go.dzs_re = own.data() + 2 * S; go.dzs_im = own.data() + 3 * S;
+					orc::dft_backward(S, roots, gi, go);
+					for (int p = 0; p < 4; ++p)
+						for (int q = 0; q < S; ++q) dx[((size_t) p * R + g * S + q) * D + c] = own[p * S + q];
+				}
+			for (int r = 0; r < R; ++r) {
+				net.fetch(net[mix], r);
+				gx.add(net[mix]->input().dz_real_, dx.data() + ((size_t) 0 * R + r) * D, D);
+				gx.add(net[mix]->input().dz_imag_, dx.data() + ((size_t) 1 * R + r) * D, D);
+				gx.add(net[mix]->input().dz_star_real_, dx.data() + ((size_t) 2 * R + r) * D, D);
+				gx.add(net[mix]->input().dz_star_imag_, dx.data() + ((size_t) 3 * R + r) * D, D);
+				for (int c = 0; c < D; ++c) {
+					dtab[(size_t) ids[r] * D + c] += dx[((size_t) 2 * R + r) * D + c];
+					dtab[(size_t) V * D + (size_t) ids[r] * D + c] += dx[((size_t) 3 * R + r) * D + c];
+				}
+			}
+			report(tag + "gradient below the mixing layer (dz and dz*)", gx.value());
+			net.fetch(net[emb], 0);
+			ErrAcc gt, gp;
+			gt.add(net[emb]->input().dz_star_real_, dtab.data(), 2 * V * D);
+			report(tag + "embedding table dz* (tokens repeated within and across sequences)", gt.value());
+			const int fac[4] = {gd, w1d, w2d, w3d}, orc_id[4] = {og, ow1, ow2, ow3};
+			for (int k = 0; k < 4; ++k) {
+				net.fetch(net[fac[k]], 0);
+				gp.add(net[fac[k]]->input().dz_star_real_, ot.at(orc_id[k])->in.dzs_re, 2 * net[fac[k]]->input().length_);
+			}
+			report(tag + "parameter dz* summed over all tokens (gate, three weights)", gp.value());
+			// one SGD step on both sides (upstream's GPU loop passes l_rate / batch size, cnet.cpp:147)
+			net.gpuUpdateInputs(lr / R);
+			ot.update(lr, R);
+			for (size_t k = 0; k < tab.size(); ++k) tab[k] -= lr / R * dtab[k];
+			ErrAcc zp;
+			for (int k = 0; k < 4; ++k) {
+				net.fetch(net[fac[k]], 0);
+				zp.add(net[fac[k]]->input().real_, ot.at(orc_id[k])->in.re, 2 * net[fac[k]]->input().length_);
+			}
+			net.fetch(net[emb], 0);
+			zp.add(net[emb]->input().real_, tab.data(), 2 * V * D);
+			report(tag + "parameters and table after the SGD step", zp.value(), 1e-6);
+		}
+		expect(tag + "the per-sample calls refuse the net", throws<std::invalid_argument>([&] {
+			CNet one;
+			auto e = one.add(new CEmbedding(D, 1, V));
+			auto m = one.add(new SeqFourierTrans(InSize(D), S), {e});
+			auto o = one.add(new L2Out(InSize(D)), {m});
+			(void) o;
+			((CEmbedding *) one[e])->setInput({0});
+			one.forward();
+		}));
+	}
 }
 
 // ------------------------------------------------------------------------------------------------- Adam, TriangFourier, CRelu
@@ -1762,6 +1980,7 @@ int main(int argc, char **argv) {
 		if (what == "resblock" || what == "all") test_resblock();
 		if (what == "persample" || what == "all") test_persample();
 		if (what == "embedding" || what == "all") test_embedding();
+		if (what == "token_model" || what == "all") test_token_model();
 		if (what == "adam" || what == "all") test_adam();
 		if (what == "loss_map" || what == "all") test_loss_map_and_sampling();
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");

@@ -53,6 +53,14 @@ def test_embedding_batch():
     assert "FAIL" not in out
 
 
+def test_token_model_with_one_token_per_sample():
+    """The fifth configuration's model at reduced size through the facade: an EmbeddingBatch of batch x seq one-token samples,
+    SeqFourierTrans mixing along the sequence, per-token layers, CrossEntropy on the next token, one SGD step; with one
+    gradient per value and with both halves of every pair."""
+    out = _run("token_model")
+    assert "FAIL" not in out and out.count("PASS") >= 26
+
+
 def test_triang_fourier_crelu_net_with_adam_steps():
     out = _run("adam")
     assert "FAIL" not in out and out.count("PASS") > 30
