@@ -69,6 +69,7 @@ SIGNATURES = {
     "cnet_cgemm_get_products": [],
     "cnet_cdft_fwd": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i, _i],
     "cnet_cdft_fwd_real_input": [c_fp, c_fp, _l, c_fp, c_fp, _l, _i, _i],
+    "cnet_cdft_hadamard_cgelu_fwd": [c_fp, c_fp, _l] + [c_fp] * 8 + [_l, _i, _i],
     "cnet_cdft_bwd": [c_fp] * 4 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_cdft_bwd_sym": [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_ctriang_dft_bwd_sym": [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i],

@@ -16,6 +16,10 @@ int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, c
 		const float *const a_im[2], long lda, const float *const b_re[2], const float *const b_im[2], long ldb,
 		const bool conj_b[2], float *const c_re[2], float *const c_im[2], long ldc, int accumulate, int tri, int mirror);
 
+int cgemm_dft_hgelu(int M, int n, const float *x_re, const float *x_im, long ldx, const float *f_re, const float *f_im, long ldf,
+		const float *hv_re, const float *hv_im, float *y_re, float *y_im, float *h_re, float *h_im, float *g_re, float *g_im, long ld,
+		bool *launched);
+
 struct Twiddle {
 	float *re = nullptr;
 	float *im = nullptr;
@@ -176,6 +180,24 @@ int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re
 	float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
 	bool cj[2] = {false, false};
 	return cgemm_pair(false, true, 1, B, n, n, ar, ai, ldx, br, bi, t.ld, cj, cr, ci, ldy, accumulate, 0, 0);
+}
+
+int cnet_cdft_hadamard_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx, const float *v_re, const float *v_im, float *y_re,
+		float *y_im, float *h_re, float *h_im, float *a_re, float *a_im, int64_t ld, int B, int n) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && n > 0 && n <= 46340);
+	if (B == 0) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && v_re && v_im && y_re && y_im && h_re && h_im && a_re && a_im && ldx >= n && ld >= n);
+	Twiddle t;
+	int rc = get_plan(n, &t, true);
+	if (rc) return rc;
+	const float *f_re = t.fwd_re ? t.fwd_re : t.re, *f_im = t.fwd_re ? t.fwd_im : t.im;
+	bool launched = false;
+	rc = cgemm_dft_hgelu(B, n, x_re, x_im, ldx, f_re, f_im, t.ld, v_re, v_im, y_re, y_im, h_re, h_im, a_re, a_im, ld, &launched);
+	if (rc || launched) return rc;
+	// a product for the block kernels, or one cut along K: the transform, then gate and activation in one pass over its result
+	rc = cnet_cdft_fwd(x_re, x_im, ldx, y_re, y_im, ld, B, n, 0);
+	return rc ? rc : cnet_hadamard_cgelu_fwd(y_re, y_im, ld, v_re, v_im, 0, h_re, h_im, ld, a_re, a_im, ld, B, n);
 }
 
 int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy, int B, int n) {

@@ -83,8 +83,14 @@ struct CgemmArgs {
 	// of the same row of C (honouring `accumulate`): the transform of real samples computes columns 0 .. n/2 and fills the others
 	// as it stores those.  One problem; the columns written this way must lie outside the product's own.
 	int herm_n = 0, herm_lo = 1, herm_hi = 0;
+	// mirror == 4 (MIRROR_HGELU): the value y of C at (row, col) is multiplied by the shared row hv[col], h = y hv goes to the C
+	// planes of p[1] and its CGelu to (g_re, g_im), all with leading dimension ldc: a transform followed by a Hadamard gate with
+	// shared weights and a CGelu in one launch, with the arithmetic of hadamard_gelu_fwd_kernel on the stored y.  Honoured by the
+	// small-C kernel without slices of K only (the caller checks); always assigned.
+	const float *hv_re = nullptr, *hv_im = nullptr;
+	float *g_re = nullptr, *g_im = nullptr;
 };
-constexpr int MIRROR_CONJ = 1, MIRROR_GELU = 2, MIRROR_HERM = 3;
+constexpr int MIRROR_CONJ = 1, MIRROR_GELU = 2, MIRROR_HERM = 3, MIRROR_HGELU = 4;
 
 // the conjugate of (vr, vi) into element `off` of the mirror planes
 __device__ __forceinline__ void mirror_store(const CgemmArgs &args, long off, float vr, float vi) {
@@ -1002,7 +1008,7 @@ template <int W, bool A_V4, bool B_V4>
 __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyStrides &st, const int bx, float *red) {
 	const unsigned a_kstride = st.a_kstride, a_mstride = st.a_mstride, b_kstride = st.b_kstride, b_nstride = st.b_nstride;
 	const unsigned a_bytes = st.a_bytes, b_bytes = st.b_bytes;
-	constexpr int DEPTH = 3;
+	constexpr int DEPTH = 3;  // (5 and 8 groups in flight measured 4 to 20 % slower: the loop is not waiting for memory)
 	// the wavefront number as a scalar: the K range, the loop over it and its branches then run on the scalar unit
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 	const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
@@ -1091,8 +1097,33 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 		red[((wave * 2 + 1) * 4 + e) * 64 + lane] = sb * acc_r[e] + sa * acc_s[e];
 	}
 	__syncthreads();
-	// the 8 (plane, accumulator register) pairs are added and stored by the first wavefronts, one or two pairs each
 	const int col = n0 + r;
+	if (args.mirror == MIRROR_HGELU) {
+		// both planes of an element by one lane (the gate needs the complex value): the 4 accumulator registers go to the first
+		// four wavefronts; each plane is added in wavefront order, as below
+		for (int e = wave; e < 4; e += W) {
+			float vr = 0.f, vi = 0.f;
+#pragma unroll
+			for (int w = 0; w < W; ++w) {
+				vr += red[((w * 2 + 0) * 4 + e) * 64 + lane];
+				vi += red[((w * 2 + 1) * 4 + e) * 64 + lane];
+			}
+			const int row = m0 + 4 * q + e;
+			if (row < args.M && col < args.N) {
+				const long off = (long) row * ldc + col;
+				pb.c_re[off] = vr;
+				pb.c_im[off] = vi;
+				const float wr = args.hv_re[col], wi = args.hv_im[col];
+				const float hr = vr * wr - vi * wi, hi = vr * wi + vi * wr;
+				args.p[1].c_re[off] = hr;
+				args.p[1].c_im[off] = hi;
+				args.g_re[off] = cnet::gelu_value(hr);
+				args.g_im[off] = cnet::gelu_value(hi);
+			}
+		}
+		return;
+	}
+	// the 8 (plane, accumulator register) pairs are added and stored by the first wavefronts, one or two pairs each
 	for (int c = wave; c < 8; c += W) {
 		const int part = c >> 2, e = c & 3;
 		float v = 0.f;
@@ -1682,6 +1713,32 @@ int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, c
 	if (mirror && nprob != 1) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: a mirrored product is one problem");
 	CgemmArgs a = pair_args(nprob, M, N, K, a_re, a_im, lda, b_re, b_im, ldb, conj_b, c_re, c_im, ldc, accumulate, tri, mirror);
 	return cgemm_dispatch(a_mcontig, b_ncontig, a, nprob, 1);
+}
+
+// y = x F, h = y .* hv (hv one shared row), g = gelu(h) in one launch of the small-C kernel, when the product is small enough
+// for it and is not cut along K: *launched says whether it went out (used by cdft.hip; otherwise the caller runs the two passes)
+int cgemm_dft_hgelu(int M, int n, const float *x_re, const float *x_im, long ldx, const float *f_re, const float *f_im, long ldf,
+		const float *hv_re, const float *hv_im, float *y_re, float *y_im, float *h_re, float *h_im, float *g_re, float *g_im, long ld,
+		bool *launched) {
+	const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {f_re, f_re}, *bi[2] = {f_im, f_im};
+	float *cr[2] = {y_re, h_re}, *ci[2] = {y_im, h_im};
+	const bool cj[2] = {false, false};
+	CgemmArgs a = pair_args(1, M, n, n, ar, ai, ldx, br, bi, ldf, cj, cr, ci, ld, 0, 0, MIRROR_HGELU);
+	a.hv_re = hv_re;
+	a.hv_im = hv_im;
+	a.g_re = g_re;
+	a.g_im = g_im;
+	a.splits = 1;
+	a.chunks_per_split = 0;
+	a.partial = nullptr;
+	a.tail_tiles = a.tail_splits = a.tail_chunks = 0;
+	a.nprob = 1;
+	*launched = false;
+	CgemmArgs planned;
+	if (!plan_skinny(false, true, a, 1, 1, planned) || planned.splits != 1) return CNET_OK;
+	const SkinnyVariant v = skinny_variant(false, true, planned, 1, 1);
+	*launched = true;
+	return CNET_SKINNY_PICK(v, launch_skinny, (planned, false, true, 1, 1));
 }
 
 // One product whose A (row-major) has an imaginary plane of nothing but +0, against a k-major B (used by cdft.hip)

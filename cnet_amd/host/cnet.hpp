@@ -529,6 +529,10 @@ protected:
 	// 1, its backward pass runs as usual.
 	CFunc *fused_next_ = NULL;
 	int fused_prev_ = 0;
+	// A FourierTrans whose only consumer is such a Hadamard with a shared weight row hands all three layers to one call
+	// (cnet_cdft_hadamard_cgelu_fwd: one launch at small batches): fused_next_ of the transform names the Hadamard, and
+	// fwd_by_producer_ of the Hadamard says that the transform of this forward pass has written its planes and the CGelu's.
+	bool fwd_by_producer_ = false;
 	// A Residual one of whose operands (slot fused_gelu_slot_) is a CGelu that feeds nothing else runs the CGelu's backward
 	// pass inside its own (cnet_residual_cgelu_bwd_sym) under conjugate gradient pairs; bwd_by_consumer_ of the CGelu is
 	// set.  The gradient of that operand equals the gradient of the other one and is not stored a second time: fetch()
@@ -1502,6 +1506,7 @@ private:
 	void planFusion() {
 		for (auto f : func_list_) {
 			f->fused_next_ = NULL;
+			f->fwd_by_producer_ = false;
 			f->fused_prev_ = 0;
 			f->fused_gelu_slot_ = -1;
 			f->bwd_by_consumer_ = false;
@@ -1517,6 +1522,14 @@ private:
 			if (t == isHadamard && g->no_outputs() != 1) continue;
 			f->fused_next_ = g;
 			g->fused_prev_ = t == isHadamard ? 2 : 1;
+		}
+		for (auto f : func_list_) {  // FourierTrans -> Hadamard (shared row) -> CGelu
+			if (f->typeId() != isFourier || f->no_outputs() != 1) continue;
+			CFunc *h = f->next_func_[0];
+			if (h->typeId() != isHadamard || !h->fused_next_ || h->rows_ != f->rows_ || h->slots_.size() != 2 || h->slots_[0].producer != f ||
+					h->slots_[0].len != f->out_size_ || h->slots_[1].rows != 1 || h->out_size_ != f->out_size_)
+				continue;
+			f->fused_next_ = h;
 		}
 		for (auto f : func_list_) {
 			if (f->typeId() != isResidual || f->no_outputs() < 1 || f->no_outputs() > 2) continue;
@@ -1571,6 +1584,13 @@ private:
 						"cnet_cdft_fwd_real_input");
 				break;
 			}
+			if (CFunc *h = f->fused_next_) {  // the gate and the activation above it where the transform is stored
+				CFunc *g = h->fused_next_;
+				ck(cnet_cdft_hadamard_cgelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, zre(h, 1), zim(h, 1), f->out_re(), f->out_im(), h->out_re(),
+						h->out_im(), g->out_re(), g->out_im(), f->out_size_, rows, f->out_size_), "cnet_cdft_hadamard_cgelu_fwd");
+				h->fwd_by_producer_ = true;
+				break;
+			}
 			ck(cnet_cdft_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_, 0),
 					"cnet_cdft_fwd");
 			break;
@@ -1591,6 +1611,10 @@ private:
 			break;
 		case isHadamard: {
 			const int n = f->out_size_;
+			if (f->fwd_by_producer_) {  // written by the transform below it in this pass
+				f->fwd_by_producer_ = false;
+				break;
+			}
 			if (CFunc *g = f->fused_next_) {  // the CGelu on its result in the same pass
 				ck(cnet_hadamard_cgelu_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), f->slots_[1].rows == rows ? n : 0, f->out_re(),
 						f->out_im(), n, g->out_re(), g->out_im(), n, rows, n), "cnet_hadamard_cgelu_fwd");

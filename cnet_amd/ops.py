@@ -165,6 +165,12 @@ def dft_fwd_real_input(x, y):
     call("cnet_cdft_fwd_real_input", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols)
 
 
+def dft_hadamard_gelu_fwd(x, v, y, h, a):
+    """y = x F, h = y .* v (v: one shared row), a = gelu(h); y, h and a share a leading dimension."""
+    assert y.ld == h.ld == a.ld
+    call("cnet_cdft_hadamard_cgelu_fwd", *x.p(), x.ld, *v.p(), *y.p(), *h.p(), *a.p(), y.ld, x.rows, x.cols)
+
+
 def dft_bwd(g, dx, accumulate=0):
     call("cnet_cdft_bwd", *g.p(), g.ld, *dx.p(), dx.ld, g.rows, g.cols, accumulate)
 

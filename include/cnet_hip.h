@@ -251,6 +251,15 @@ int cnet_cdft_twiddle(int n, const float **f_re, const float **f_im);  /* the pl
 int cnet_cdft_set_forward_matrix(int n, const float *host_f_re, const float *host_f_im);
 int cnet_cdft_fwd(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
                   int B, int n, int accumulate);      /* y = x * F */
+/* FourierTrans followed by a Hadamard gate with one shared weight row and a CGelu, the first three layers of upstream's README
+ * net (README.md:19-30; FourierGpu::gpu_fft_forward gpu/reduce.cpp:382-393, gpu_hadamard_forward gpu/kernels.cpp:204-232,
+ * gpu_gelu_forward gpu/kernels.cpp:292-315): y = x F, h = y .* v (v one row of n weights), a = gelu(h), all three written
+ * (leading dimension ld each), with the bits of cnet_cdft_fwd followed by cnet_hadamard_cgelu_fwd.  One launch when the
+ * product is small enough for the small-C kernel (a small batch: the step is then bound by its launches), else those two
+ * calls. */
+int cnet_cdft_hadamard_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx, const float *v_re, const float *v_im,
+                                 float *y_re, float *y_im, float *h_re, float *h_im, float *a_re, float *a_im, int64_t ld,
+                                 int B, int n);
 /* The same transform for REAL samples (upstream's FourierTrans forward, impl/ft.h:37-55, transforms them like any
  * others, and so does gpu_fft_forward, gpu/reduce.cpp:160-187).  The caller vouches that every x_im is +0 (the plane must
  * exist and hold the zeros: the kernels for small and for unaligned shapes read it; the block kernels do not).  The result is

@@ -137,3 +137,37 @@ def test_fused_layers_under_other_kernel_choices(gpu, overrides):
     r = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-m", "gpu"], env=env,
                        capture_output=True, text=True, timeout=280, cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-2000:]
+
+
+# B, n: small batches take the small-C kernel and one launch; 50 x 2048 (K cut into slices), 4096 x 784 and 1024 x 1024 (block
+# kernels) two launches
+TRANSFORM_GATE = [(64, 784), (16, 96), (1, 4), (100, 333), (256, 784), (50, 2048), (4096, 784), (1024, 1024)]
+
+
+@pytest.mark.parametrize("B,n", TRANSFORM_GATE)
+def test_transform_gate_and_activation_in_one_call(gpu, port, B, n):
+    """cnet_cdft_hadamard_cgelu_fwd (FourierTrans -> Hadamard with a shared weight row -> CGelu, the first three layers of
+    upstream's README net) against cnet_cdft_fwd followed by cnet_hadamard_cgelu_fwd: equal bits in all three results, in
+    column windows of wider buffers as well; and against the CPU oracle layer by layer (upstream testFfft / testHadamard /
+    testGelu, tests/gputests.h:91, 464, 517)."""
+    xr, xi = seeded(port, 3 * B + n, (B, n)), seeded(port, 3 * B + n + 1, (B, n))
+    vr, vi = seeded(port, n + 7, (1, n), 0.7), seeded(port, n + 8, (1, n), 0.7)
+    x, v = ops.CMat.from_host(xr, xi), ops.CMat.from_host(vr, vi)
+    y0, h0, a0 = (ops.CMat.empty(B, n) for _ in range(3))
+    ops.dft_fwd(x, y0)
+    ops.hadamard_gelu_fwd(y0, v, h0, a0, shared=True)
+    W = n + 12   # wider buffers: the results land in a window that starts at column 8
+    base = seeded(port, 5, (B, W))
+    wide = [ops.CMat(ops.Plane.from_host(base), ops.Plane.from_host(base)) for _ in range(3)]
+    y1, h1, a1 = (w.sub(8, n) for w in wide)
+    ops.dft_hadamard_gelu_fwd(x, v, y1, h1, a1)
+    mask = np.ones(W, bool); mask[8:8 + n] = False
+    for w, want, what in zip(wide, (y0, h0, a0), ("transform", "gated", "activation")):
+        for plane, ref in zip((w.re.owner.download(), w.im.owner.download()), want.host()):
+            assert np.array_equal(plane[:, 8:8 + n], ref), (what, B, n)
+            assert np.array_equal(plane[:, mask], base[:, mask]), (what, "outside the window")
+    if B * n * n <= 1 << 27:
+        yr, yi = port.dft_fwd(xr, xi)
+        hr, hi = port.hadamard_fwd(yr, yi, vr[0], vi[0])
+        assert rel_c(y0.host(), (yr, yi)) < TOL and rel_c(h0.host(), (hr, hi)) < TOL
+        assert rel_c(a0.host(), port.gelu_fwd(hr, hi)) < TOL
