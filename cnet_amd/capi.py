@@ -62,6 +62,8 @@ SIGNATURES = {
     "cnet_clinear_bwd_input_sym": [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
     "cnet_clinear_bwd_weight_sym": [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
     "cnet_clinear_bwd_sym": [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
+    "cnet_clinear_cross_entropy_fwd_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, c_fp, _l, c_fp, c_fp, c_fp] +
+                                              [c_fp] * 4 + [_l, _i, _i, _i],
     "cnet_cdft_plan": [_i],
     "cnet_cdft_twiddle": [_i, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)],
     "cnet_cdft_set_forward_matrix": [_i, C.c_void_p, C.c_void_p],

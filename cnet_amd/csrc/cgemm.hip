@@ -26,6 +26,7 @@
 // and cgemm_skinny_kernel (a C of few 16 x 16 tiles: one tile per workgroup, K shared among its wavefronts).
 // cgemm_dispatch picks among them and pick_tile picks the block shape.
 #include "common.hpp"
+#include "rows.hpp"
 
 #include <algorithm>
 #include <cstdlib>
@@ -89,8 +90,18 @@ struct CgemmArgs {
 	// small-C kernel without slices of K only (the caller checks); always assigned.
 	const float *hv_re = nullptr, *hv_im = nullptr;
 	float *g_re = nullptr, *g_im = nullptr;
+	// mirror == 5 (MIRROR_CE): C is a block of logits whose columns all lie in one tile (N <= 16).  The workgroup that has formed
+	// 16 rows of it also runs the forward pass of CrossEntropy and the gradient of the loss over them (crossent_fwd_row_at on the
+	// tile in LDS, the routine and the instantiation the separate launch would run: the same bits): a narrow Linear head and its
+	// loss in one launch.  Small-C kernel without slices of K (the caller checks); C is assigned.
+	const int *ce_labels = nullptr;
+	float *ce_out_re = nullptr, *ce_out_im = nullptr, *ce_s = nullptr, *ce_loss = nullptr;
+	int *ce_argmax = nullptr;
+	float *ce_dz_re = nullptr, *ce_dz_im = nullptr, *ce_dzs_re = nullptr, *ce_dzs_im = nullptr;
+	long ce_ldo = 0, ce_lddz = 0;
+	int ce_vec = 0;  // the 128-bit instantiation of the row routine (what the separate launch would pick for these operands)
 };
-constexpr int MIRROR_CONJ = 1, MIRROR_GELU = 2, MIRROR_HERM = 3, MIRROR_HGELU = 4;
+constexpr int MIRROR_CONJ = 1, MIRROR_GELU = 2, MIRROR_HERM = 3, MIRROR_HGELU = 4, MIRROR_CE = 5;
 
 // the conjugate of (vr, vi) into element `off` of the mirror planes
 __device__ __forceinline__ void mirror_store(const CgemmArgs &args, long off, float vr, float vi) {
@@ -1004,7 +1015,7 @@ struct SkinnyStrides {
 };
 
 // the tile numbered `bx` of the product `args`; red = W x 2 x 4 x 64 floats of LDS ([W][re, im][4][64])
-template <int W, bool A_V4, bool B_V4>
+template <int W, bool A_V4, bool B_V4, bool CE = false>
 __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyStrides &st, const int bx, float *red) {
 	const unsigned a_kstride = st.a_kstride, a_mstride = st.a_mstride, b_kstride = st.b_kstride, b_nstride = st.b_nstride;
 	const unsigned a_bytes = st.a_bytes, b_bytes = st.b_bytes;
@@ -1124,12 +1135,14 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 		return;
 	}
 	// the 8 (plane, accumulator register) pairs are added and stored by the first wavefronts, one or two pairs each
+	__shared__ float logits[CE ? 2 * 16 * 16 : 1];  // CE: the finished tile, [re, im][row][col]
 	for (int c = wave; c < 8; c += W) {
 		const int part = c >> 2, e = c & 3;
 		float v = 0.f;
 #pragma unroll
 		for (int w = 0; w < W; ++w) v += red[((w * 2 + part) * 4 + e) * 64 + lane];
 		const int row = m0 + 4 * q + e;
+		if (CE) logits[(part * 16 + 4 * q + e) * 16 + r] = v;
 		if (row < args.M && col < args.N) {
 			float *dst = (part ? pb.c_im : pb.c_re) + (long) row * ldc + col;
 			const float fin = accumulate ? *dst + v : v;
@@ -1144,12 +1157,26 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 			}
 		}
 	}
+	if constexpr (CE) {
+		// the 16 rows of logits of this tile, one wavefront per row at a time: loss, argmax, normalised row and gradient
+		__syncthreads();
+		const cnet::rows::GradPlanes grad = {args.ce_dz_re, args.ce_dz_im, args.ce_dzs_re, args.ce_dzs_im, args.ce_lddz};
+		for (int rr = wave; rr < 16 && m0 + rr < args.M; rr += W) {
+			const float *pr = logits + rr * 16, *pi = logits + (16 + rr) * 16;
+			if (args.ce_vec)
+				cnet::rows::crossent_fwd_row_at<4, 1, true>(pr, pi, m0 + rr, true, lane, lane, 0, 0, nullptr, nullptr, nullptr, args.ce_labels,
+						args.ce_out_re, args.ce_out_im, args.ce_ldo, args.ce_s, args.ce_loss, args.ce_argmax, args.N, grad, 0);
+			else
+				cnet::rows::crossent_fwd_row_at<1, 1, true>(pr, pi, m0 + rr, true, lane, lane, 0, 0, nullptr, nullptr, nullptr, args.ce_labels,
+						args.ce_out_re, args.ce_out_im, args.ce_ldo, args.ce_s, args.ce_loss, args.ce_argmax, args.N, grad, 0);
+		}
+	}
 }
 
-template <int W, bool A_V4, bool B_V4>
+template <int W, bool A_V4, bool B_V4, bool CE = false>
 __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs args, const SkinnyStrides st) {
 	__shared__ float red[W * 2 * 4 * 64];
-	skinny_tile<W, A_V4, B_V4>(args, st, blockIdx.x, red);
+	skinny_tile<W, A_V4, B_V4, CE>(args, st, blockIdx.x, red);
 }
 
 // Two unrelated small products in one launch (the input gradient and the weight gradient of a narrow Linear layer, each
@@ -1183,6 +1210,15 @@ int launch_skinny(const CgemmArgs &args, bool a_mcontig, bool b_ncontig, int npr
 		hipLaunchKernelGGL(splitk_reduce_kernel, rgrid, dim3(256), 0, cnet::rt().stream, args, nprob, batch);
 		CNET_LAUNCH_CHECK();
 	}
+	return CNET_OK;
+}
+
+// the launch whose workgroups go on to the CrossEntropy of their rows of logits (CgemmArgs::ce_*; one column of tiles, no slices)
+template <int W, bool A_V4, bool B_V4>
+int launch_skinny_ce(const CgemmArgs &args, bool a_mcontig, bool b_ncontig) {
+	auto kern = cgemm_skinny_kernel<W, A_V4, B_V4, true>;
+	hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, 1), dim3(64 * W), 0, cnet::rt().stream, args, skinny_strides(args, a_mcontig, b_ncontig));
+	CNET_LAUNCH_CHECK();
 	return CNET_OK;
 }
 
@@ -1876,6 +1912,48 @@ int cnet_clinear_cgelu_fwd(const float *x_re, const float *x_im, int64_t ldx, co
 	float *cr[2] = {h_re, y_re}, *ci[2] = {h_im, y_im};
 	bool cj[2] = {false, false};
 	return cgemm_pair(false, false, 1, B, N, K, ar, ai, ldx, br, bi, ldw, cj, cr, ci, ldy, accumulate, 0, MIRROR_GELU);
+}
+
+int cnet_clinear_cross_entropy_fwd_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const float *w_re, const float *w_im, int64_t ldw,
+		float *y_re, float *y_im, int64_t ldy, const int32_t *labels, float *out_re, float *out_im, int64_t ldo, float *s, float *loss,
+		int32_t *argmax, float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz, int B, int K, int N) {
+	CNET_REQUIRE_INIT();
+	CNET_CHECK_ARG(B >= 0 && N > 0 && K > 0);
+	if (B == 0) return CNET_OK;
+	CNET_CHECK_ARG(x_re && x_im && w_re && w_im && y_re && y_im && labels && s && loss && argmax);
+	CNET_CHECK_ARG(ldx >= K && ldw >= K && ldy >= N);
+	CNET_CHECK_ARG((out_re == nullptr) == (out_im == nullptr) && (out_re == nullptr || ldo >= N));
+	CNET_CHECK_ARG(dz_dz_re && dz_dz_im && ((dz_dzs_re == nullptr) == (dz_dzs_im == nullptr)) && lddz >= N);
+	if (N <= 16) {
+		const float *ar[2] = {x_re, x_re}, *ai[2] = {x_im, x_im}, *br[2] = {w_re, w_re}, *bi[2] = {w_im, w_im};
+		float *cr[2] = {y_re, y_re}, *ci[2] = {y_im, y_im};
+		const bool cj[2] = {false, false};
+		CgemmArgs a = pair_args(1, B, N, K, ar, ai, ldx, br, bi, ldw, cj, cr, ci, ldy, 0, 0, MIRROR_CE), planned;
+		if (plan_skinny(false, false, a, 1, 1, planned) && planned.splits == 1 && planned.tiles_n == 1) {
+			planned.ce_labels = labels;
+			planned.ce_out_re = out_re;
+			planned.ce_out_im = out_im;
+			planned.ce_ldo = ldo;
+			planned.ce_s = s;
+			planned.ce_loss = loss;
+			planned.ce_argmax = argmax;
+			planned.ce_dz_re = dz_dz_re;
+			planned.ce_dz_im = dz_dz_im;
+			planned.ce_dzs_re = dz_dzs_re;
+			planned.ce_dzs_im = dz_dzs_im;
+			planned.ce_lddz = lddz;
+			// the instantiation cnet_cross_entropy_fwd_bwd_sym would run on these planes
+			auto m4 = [](long v) { return v % 4 == 0; };
+			planned.ce_vec = m4(N) && m4(ldy) && (!out_re || m4(ldo)) && m4(lddz) && aligned16(y_re) && aligned16(y_im) && aligned16(out_re) &&
+					aligned16(out_im) && aligned16(dz_dz_re) && aligned16(dz_dz_im) && aligned16(dz_dzs_re) && aligned16(dz_dzs_im);
+			const SkinnyVariant v = skinny_variant(false, false, planned, 1, 1);
+			return CNET_SKINNY_PICK(v, launch_skinny_ce, (planned, false, false));
+		}
+	}
+	// a head too wide or too tall for that kernel: the product, then the pass over its rows
+	const int rc = cnet_clinear_fwd(x_re, x_im, ldx, w_re, w_im, ldw, y_re, y_im, ldy, B, K, N, 0);
+	return rc ? rc : cnet_cross_entropy_fwd_bwd_sym(y_re, y_im, ldy, labels, out_re, out_im, ldo, s, loss, argmax, dz_dz_re, dz_dz_im, dz_dzs_re,
+			dz_dzs_im, lddz, B, N);
 }
 
 int cnet_clinear_bwd_input(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im,

@@ -533,6 +533,10 @@ protected:
 	// (cnet_cdft_hadamard_cgelu_fwd: one launch at small batches): fused_next_ of the transform names the Hadamard, and
 	// fwd_by_producer_ of the Hadamard says that the transform of this forward pass has written its planes and the CGelu's.
 	bool fwd_by_producer_ = false;
+	// A Linear that feeds nothing but a CrossEntropy hands its product and the loss (forward pass and gradient) to one call
+	// (cnet_clinear_cross_entropy_fwd_bwd_sym: one launch for a narrow head) whenever the loss would write its gradient from
+	// its forward pass anyway: loss_next_ of the Linear names the CrossEntropy, whose fwd_by_producer_ is then set per pass.
+	CFunc *loss_next_ = NULL;
 	// A Residual one of whose operands (slot fused_gelu_slot_) is a CGelu that feeds nothing else runs the CGelu's backward
 	// pass inside its own (cnet_residual_cgelu_bwd_sym) under conjugate gradient pairs; bwd_by_consumer_ of the CGelu is
 	// set.  The gradient of that operand equals the gradient of the other one and is not stored a second time: fetch()
@@ -1506,6 +1510,7 @@ private:
 	void planFusion() {
 		for (auto f : func_list_) {
 			f->fused_next_ = NULL;
+			f->loss_next_ = NULL;
 			f->fwd_by_producer_ = false;
 			f->fused_prev_ = 0;
 			f->fused_gelu_slot_ = -1;
@@ -1522,6 +1527,14 @@ private:
 			if (t == isHadamard && g->no_outputs() != 1) continue;
 			f->fused_next_ = g;
 			g->fused_prev_ = t == isHadamard ? 2 : 1;
+		}
+		for (auto f : func_list_) {  // Linear -> CrossEntropy
+			if (f->typeId() != isLinear || f->fused_next_ || f->no_outputs() != 1 || f->slots_[0].rows != f->rows_) continue;
+			CFunc *c = f->next_func_[0];
+			if (c->typeId() != isCrossEntropy || c->rows_ != f->rows_ || c->slots_.size() != 1 || c->slots_[0].producer != f ||
+					c->slots_[0].len != f->out_size_)
+				continue;
+			f->loss_next_ = c;
 		}
 		for (auto f : func_list_) {  // FourierTrans -> Hadamard (shared row) -> CGelu
 			if (f->typeId() != isFourier || f->no_outputs() != 1) continue;
@@ -1556,6 +1569,13 @@ private:
 		throw std::logic_error("broken wiring at " + f->getName());
 	}
 
+	// A short-rowed loss (a classifier head) costs less than the launch it rides on: forward pass and gradient go out as one
+	// launch.  Not inside the recorded phases (the labels may change between a recorded forward and a recorded backward pass)
+	// and not in the per-sample calls (upstream shows cleared gradients after forward()).
+	bool lossFromForward(CFunc *c) const {
+		return fuse_layers_ && conjugate_gradients_ && !use_graphs_ && !per_sample_call_ && (long) c->rows_ * c->input().length_ <= (1L << 18);
+	}
+
 	void nodeForward(CFunc *f) {
 		const int rows = f->rows_;
 		switch (f->typeId()) {
@@ -1572,6 +1592,16 @@ private:
 			if (CFunc *g = f->fused_next_) {  // the CGelu on its result is applied as the product is stored
 				ck(cnet_clinear_cgelu_fwd(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), g->out_re(), g->out_im(),
 						N, rows, K, N, 0), "cnet_clinear_cgelu_fwd");
+				break;
+			}
+			if (f->loss_next_ && lossFromForward(f->loss_next_)) {  // the loss on its rows where the product is stored
+				CrossEntropy *c = (CrossEntropy *) f->loss_next_;
+				CFunc::Slot &sl = c->slots_[0];
+				ck(cnet_clinear_cross_entropy_fwd_bwd_sym(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), N, d_labels_,
+						c->d_norm_, c->d_norm_ + (size_t) rows * N, N, c->d_s_, lossTarget(c->loss_), c->d_argmax_, sl.g(0), sl.g(1), sl.gs(2),
+						sl.gs(3), sl.len, rows, K, N), "cnet_clinear_cross_entropy_fwd_bwd_sym");
+				c->grad_from_forward_ = true;
+				c->fwd_by_producer_ = true;
 				break;
 			}
 			ck(cnet_clinear_fwd(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), N, rows, K, N, 0),
@@ -1643,10 +1673,11 @@ private:
 		case isCrossEntropy: {
 			CrossEntropy *c = (CrossEntropy *) f;
 			const int n = f->input().length_;
-			// A short-rowed loss (a classifier head) costs less than the launch it rides on: forward pass and gradient go out as
-			// one launch.  Not inside the recorded phases (the labels may change between a recorded forward and a recorded
-			// backward pass) and not in the per-sample calls (upstream shows cleared gradients after forward()).
-			if (fuse_layers_ && conjugate_gradients_ && !use_graphs_ && !per_sample_call_ && (long) rows * n <= (1L << 18)) {
+			if (f->fwd_by_producer_) {  // written by the Linear below it in this pass
+				f->fwd_by_producer_ = false;
+				break;
+			}
+			if (lossFromForward(f)) {
 				CFunc::Slot &sl = f->slots_[0];
 				ck(cnet_cross_entropy_fwd_bwd_sym(zre(f, 0), zim(f, 0), n, d_labels_, c->d_norm_, c->d_norm_ + (size_t) rows * n, n, c->d_s_,
 						lossTarget(c->loss_), c->d_argmax_, sl.g(0), sl.g(1), sl.gs(2), sl.gs(3), sl.len, rows, n), "cnet_cross_entropy_fwd_bwd_sym");

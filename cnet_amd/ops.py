@@ -346,3 +346,10 @@ def cross_entropy_fwd_bwd_sym(z, labels, s, loss, argmax, dz, out=None, mirror=T
     o = out.p() if out is not None else (None, None)
     call("cnet_cross_entropy_fwd_bwd_sym", *z.p(), z.ld, labels.ptr, o[0], o[1], out.ld if out is not None else 0, s.ptr,
          loss.ptr, argmax.ptr, *_pair(dz, mirror), dz.ld, z.rows, z.cols)
+
+
+def linear_cross_entropy_fwd_bwd_sym(x, w, y, labels, s, loss, argmax, dz, out=None, mirror=True):
+    """y = x w^T, then the loss over the rows of y and its gradient (one launch for a narrow head)."""
+    o = out.p() if out is not None else (None, None)
+    call("cnet_clinear_cross_entropy_fwd_bwd_sym", *x.p(), x.ld, *w.p(), w.ld, *y.p(), y.ld, labels.ptr, o[0], o[1],
+         out.ld if out is not None else 0, s.ptr, loss.ptr, argmax.ptr, *_pair(dz, mirror), dz.ld, x.rows, x.cols, w.rows)

@@ -237,6 +237,18 @@ int cnet_clinear_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg
 int cnet_cgemm_set_products(int n);
 int cnet_cgemm_get_products(void);
 
+/* A Linear layer that feeds a CrossEntropy (a classifier head): y = x w^T, then the forward pass of the loss over the rows of y
+ * and its gradient, with the arguments and the bits of cnet_clinear_fwd followed by cnet_cross_entropy_fwd_bwd_sym (y takes the
+ * place of z there).  Upstream runs LinearGpu::forward and CrossEntGpu::forward / backward one after the other
+ * (gpu/reduce.cpp:581-604, 609-655).  One launch when the head is narrow (N <= 16) and the product small enough for the
+ * small-C kernel without slices of K: the workgroup that has formed 16 rows of logits goes on to their loss.  Otherwise those
+ * two calls. */
+int cnet_clinear_cross_entropy_fwd_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const float *w_re, const float *w_im,
+                                           int64_t ldw, float *y_re, float *y_im, int64_t ldy, const int32_t *labels,
+                                           float *out_re, float *out_im, int64_t ldo, float *s, float *loss, int32_t *argmax,
+                                           float *dz_dz_re, float *dz_dz_im, float *dz_dzs_re, float *dz_dzs_im, int64_t lddz,
+                                           int B, int K, int N);
+
 /* ---- FourierTrans as dense complex GEMM: replaces FourierGpu::gpu_fft_forward / gpu_fft_backward
  *      (gpu/reduce.cpp:25-35,160-187,382-393; gpu/reducegrad.cpp:45-48,324-336) and the root-table upload
  *      u_roots_allocate_and_copy_on_gpu (gpu/allocator.h:389-407).  CPU twin impl/ft.h:37-80.

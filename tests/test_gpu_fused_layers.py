@@ -171,3 +171,49 @@ def test_transform_gate_and_activation_in_one_call(gpu, port, B, n):
         hr, hi = port.hadamard_fwd(yr, yi, vr[0], vi[0])
         assert rel_c(y0.host(), (yr, yi)) < TOL and rel_c(h0.host(), (hr, hi)) < TOL
         assert rel_c(a0.host(), port.gelu_fwd(hr, hi)) < TOL
+
+
+# B, K, N: narrow heads on the small-C kernel (one launch), a head of 16 logits (the 128-bit row routine), a head that is too
+# wide (N = 20) and one whose product is cut along K (K = 4096): two launches
+HEADS = [(64, 784, 10), (1, 8, 1), (100, 96, 3), (4096, 784, 10), (64, 64, 16), (50, 300, 12), (64, 128, 20), (32, 4096, 10)]
+
+
+@pytest.mark.parametrize("B,K,N", HEADS)
+def test_linear_head_and_its_loss_in_one_call(gpu, port, B, K, N):
+    """cnet_clinear_cross_entropy_fwd_bwd_sym against cnet_clinear_fwd followed by cnet_cross_entropy_fwd_bwd_sym: equal bits
+    in the logits, S, loss, argmax, the normalised rows and the gradient, with and without the normalised planes and the dz*
+    planes; and against the CPU oracle (upstream testLinear / testCE, tests/gputests.h:317, 266)."""
+    from cnet_amd import capi
+    xr, xi = seeded(port, B + K, (B, K)), seeded(port, B + K + 1, (B, K))
+    wr, wi = seeded(port, N + 2, (N, K), K ** -0.5), seeded(port, N + 3, (N, K), K ** -0.5)
+    labels_h = port.randint(B + N, (B,), N)
+    x, w, labels = ops.CMat.from_host(xr, xi), ops.CMat.from_host(wr, wi), ops.ints(labels_h)
+    keep = [seeded(port, 40 + p, (B, N)) for p in range(4)]
+    for with_out in (True, False):
+        for mirror in (True, False):
+            y0, y1 = ops.CMat.empty(B, N), ops.CMat.empty(B, N)
+            n0, n1 = ops.CMat.empty(B, N, zero=True), ops.CMat.empty(B, N, zero=True)
+            d0, d1 = ops.Grad.from_host(keep), ops.Grad.from_host(keep)
+            r0 = [capi.empty(B), capi.empty(B), capi.empty(B, np.int32)]
+            r1 = [capi.empty(B), capi.empty(B), capi.empty(B, np.int32)]
+            ops.linear_fwd(x, w, y0)
+            ops.cross_entropy_fwd_bwd_sym(y0, labels, r0[0], r0[1], r0[2], d0, out=n0 if with_out else None, mirror=mirror)
+            ops.linear_cross_entropy_fwd_bwd_sym(x, w, y1, labels, r1[0], r1[1], r1[2], d1, out=n1 if with_out else None, mirror=mirror)
+            what = (B, K, N, with_out, mirror)
+            for a, b in zip(list(y0.host()) + list(n0.host()) + d0.host(), list(y1.host()) + list(n1.host()) + d1.host()):
+                assert np.array_equal(a, b), what
+            for a, b in zip(r0, r1):
+                assert np.array_equal(a.download(), b.download()), what
+            if not mirror:
+                assert np.array_equal(d1.host()[2], keep[2]) and np.array_equal(d1.host()[3], keep[3]), (what, "dz* was written")
+    if B * K * N <= 1 << 24:
+        zr, zi = port.linear_fwd(xr, xi, wr, wi)
+        _, _, S, loss, pred = port.crossent_fwd(zr, zi, labels_h)
+        assert rel_c(y1.host(), (zr, zi)) < TOL / 5
+        assert np.array_equal(r1[2].download(), pred) and np.allclose(r1[1].download(), loss, rtol=2e-5, atol=2e-6)
+        want = port.crossent_bwd(zr, zi, labels_h)
+        d = ops.Grad.empty(B, N)
+        ops.linear_cross_entropy_fwd_bwd_sym(x, w, y1, labels, r1[0], r1[1], r1[2], d)
+        h = d.host()
+        # (the gradient at a label whose logit is small is large and as ill conditioned as 1 / |z_label|: the bar itself)
+        assert rel_c(h[0:2], want[0:2]) < TOL and rel_c(h[2:4], want[2:4]) < TOL
