@@ -1371,6 +1371,48 @@ inline bool three_products() {
 	return g_three_products != 0;
 }
 
+// The block kernels ask for more dynamic LDS than the default limit, which takes one hipFuncSetAttribute per instantiation.
+// launch() makes that call at the first launch of each; a first launch inside a stream capture would make it while the capture
+// is open, so cnet_graph_begin has all of them made beforehand (cgemm_prime_attributes) and launch() skips its own.
+bool g_attrs_primed = false;
+
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
+hipError_t prime_attributes() {
+	constexpr size_t smem = 2 * (size_t) (2 * KC * (BM + 4) + 2 * KC * (BN + 4)) * sizeof(float);
+	hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, VEC>),
+			hipFuncAttributeMaxDynamicSharedMemorySize, (int) smem);
+	if constexpr (VEC == 4) {
+		constexpr int NST = (BM == 128 && BN == 128) ? 2 : 3;
+		constexpr size_t fast_smem = (size_t) NST * 2 * KC * (BM + BN) * sizeof(float);
+		if (e == hipSuccess)
+			e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST>),
+					hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem);
+		if constexpr (!A_MCONTIG && B_NCONTIG) {
+			if (e == hipSuccess)
+				e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, true>),
+						hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem);
+		}
+		if constexpr ((WM / 32) * (WN / 32) <= 2 || A_MCONTIG || B_NCONTIG) {
+			if (e == hipSuccess)
+				e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, true>),
+						hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem);
+		}
+	}
+	return e;
+}
+
+// (the shapes pick_tile can choose: the scalar-load fallback keeps to the small block)
+template <bool A_MCONTIG, bool B_NCONTIG, int VEC>
+hipError_t prime_shapes() {
+	hipError_t e = prime_attributes<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>();
+	if constexpr (VEC == 4) {
+		if (e == hipSuccess) e = prime_attributes<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>();
+		if (e == hipSuccess) e = prime_attributes<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>();
+		if (e == hipSuccess) e = prime_attributes<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>();
+	}
+	return e;
+}
+
 template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
 int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, int k_cuts = -1) {
 	CgemmArgs args = proto;
@@ -1446,7 +1488,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 			if constexpr (!A_MCONTIG && B_NCONTIG) {
 				if (args.a_real) {
 					static bool real_attr_set = false;
-					if (!real_attr_set) {
+					if (!real_attr_set && !g_attrs_primed) {
 						CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, true>),
 								hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem));
 						real_attr_set = true;
@@ -1462,7 +1504,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 			if constexpr ((WM / 32) * (WN / 32) <= 2 || A_MCONTIG || B_NCONTIG) {
 				if (three_products()) {
 					static bool gauss_attr_set = false;
-					if (!gauss_attr_set) {
+					if (!gauss_attr_set && !g_attrs_primed) {
 						CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, true>),
 								hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem));
 						gauss_attr_set = true;
@@ -1474,7 +1516,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 				}
 			}
 			static bool fast_attr_set = false;
-			if (!fast_attr_set) {
+			if (!fast_attr_set && !g_attrs_primed) {
 				CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST>),
 						hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem));
 				fast_attr_set = true;
@@ -1487,7 +1529,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 	}
 	auto kern = cgemm_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, VEC>;
 	static bool attr_set = false;  // per instantiation
-	if (!attr_set) {
+	if (!attr_set && !g_attrs_primed) {
 		CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
 				(int) smem));
 		attr_set = true;
@@ -1740,6 +1782,22 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 static CgemmArgs pair_args(int nprob, int M, int N, int K, const float *const a_re[2], const float *const a_im[2], long lda,
 		const float *const b_re[2], const float *const b_im[2], long ldb, const bool conj_b[2], float *const c_re[2], float *const c_im[2],
 		long ldc, int accumulate, int tri, int mirror);
+
+// Called by cnet_graph_begin before the capture opens (see g_attrs_primed)
+int cgemm_prime_attributes() {
+	if (g_attrs_primed) return CNET_OK;
+	hipError_t e = prime_shapes<false, false, 4>();
+	if (e == hipSuccess) e = prime_shapes<false, true, 4>();
+	if (e == hipSuccess) e = prime_shapes<true, true, 4>();
+	if (e == hipSuccess) e = prime_shapes<true, false, 4>();
+	if (e == hipSuccess) e = prime_shapes<false, false, 1>();
+	if (e == hipSuccess) e = prime_shapes<false, true, 1>();
+	if (e == hipSuccess) e = prime_shapes<true, true, 1>();
+	if (e == hipSuccess) e = prime_shapes<true, false, 1>();
+	if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute (dynamic LDS of the matrix kernels)");
+	g_attrs_primed = true;
+	return CNET_OK;
+}
 
 // Used by cdft.hip
 int cgemm_pair(bool a_mcontig, bool b_ncontig, int nprob, int M, int N, int K, const float *const a_re[2],

@@ -56,6 +56,8 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int hip_fail(hipError_t e, const char *what);
 // returns nullptr (and records the error) when the allocation fails
 void *workspace(size_t bytes);
+// every hipFuncSetAttribute the matrix kernels need, made once, outside any stream capture (cgemm.hip)
+int cgemm_prime_attributes();
 
 #define CNET_REQUIRE_INIT()                                                              \
 	do {                                                                                 \

@@ -510,6 +510,9 @@ int cnet_memcpy_d2h(void *host_dst, const void *src, size_t bytes) {
 int cnet_graph_begin(void) {
 	CNET_REQUIRE_INIT();
 	CNET_NOT_IN_CAPTURE();
+	// no first-use set-up call of a kernel may fall inside the recording
+	const int primed = cgemm_prime_attributes();
+	if (primed != CNET_OK) return primed;
 	CNET_HIP(hipStreamBeginCapture(rt().stream, hipStreamCaptureModeThreadLocal));
 	rt().capturing = true;
 	return CNET_OK;
