@@ -111,7 +111,7 @@ def cpu_baseline(budget_s=15.0):
                       "%.2f ms/row (%.1f samples/s)" % (rows, B, dt, 1e3 * dt / rows, rows / dt)}
 
 
-def kernel_suite(steps):
+def kernel_suite(steps, rows=8192, parts=("mfma", "hbm", "ce")):
     """Per-kernel lines for the other rows of the hot path: the DFT-as-GEMM at config-3 shape (MFMA bound) and the
     elementwise / reduction kernels at config-4/5 shapes (HBM bound).  Bytes are the algorithmic (compulsory) traffic
     per complex element: every operand read once, every result written once, parameters amortised over the batch."""
@@ -119,12 +119,13 @@ def kernel_suite(steps):
     capi.init(0)
     ev = HipEvents(capi.load().cnet_stream())
     rs = np.random.RandomState(0)
+    rng = np.random.default_rng(0)
 
     def cmat(r, c):
-        return ops.CMat.from_host(rs.randn(r, c).astype(np.float32), rs.randn(r, c).astype(np.float32))
+        return ops.CMat.from_host(rng.standard_normal((r, c), dtype=np.float32), rng.standard_normal((r, c), dtype=np.float32))
 
     def grad(r, c):
-        return ops.Grad.from_host([rs.randn(r, c).astype(np.float32) for _ in range(4)])
+        return ops.Grad.from_host([rng.standard_normal((r, c), dtype=np.float32) for _ in range(4)])
 
     def timed(fn, warm=3):
         # warm-up: groups of `warm` calls until two groups in a row agree to 2 % (at most 0.2 s): the device may have
@@ -164,6 +165,17 @@ def kernel_suite(steps):
             "bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}})
 
+    if "mfma" in parts:
+        dft_lines(mfma, cmat, grad, rs)
+    if "hbm" in parts:
+        hbm_lines(hbm, cmat, grad, rows)
+    if "ce" in parts:
+        ce_lines(hbm, cmat, rs)
+    return lines
+
+
+def dft_lines(mfma, cmat, grad, rs):
+    from cnet_amd import ops
     # config 3: FourierTrans n = 4096, batch 1024 (3 complex GEMMs against the twiddle matrix)
     Bf, nf = 1024, 4096
     x, y, g, dx = cmat(Bf, nf), ops.CMat.empty(Bf, nf), grad(Bf, nf), ops.Grad.empty(Bf, nf)
@@ -181,9 +193,14 @@ def kernel_suite(steps):
     mfma("ctriang_bwd", "ctriang_dft_bwd (useful flops: upper triangle only)", [Bf, nf], 16.0 * Bf * tri, lambda: ops.triang_dft_bwd(g, dx))
     del x, y, g, dx
 
-    # config 5 activation shape [8192 x 4096]: 256 MiB per complex matrix, so every operand streams from HBM
-    # (config 4's [2048 x 2048] planes would sit in the 256 MB memory-side cache and overstate the rate)
-    R, Cc = 8192, 4096
+
+
+def hbm_lines(hbm, cmat, grad, rows):
+    from cnet_amd import capi, ops
+    # config 5 activation shape [8192 x 4096]: 128 MiB per plane (config 4's [2048 x 2048] planes would sit in the 256 MB
+    # memory-side cache and overstate the rate).  Even so a kernel that reads two planes of this size still finds part of them
+    # in that cache from one call to the next; with rows = 32768 (512 MiB per plane) nothing is served by it.
+    R, Cc = rows, 4096
     n = R * Cc
     u, v, w1 = cmat(R, Cc), cmat(R, Cc), cmat(1, Cc)
     yy, g, du, dv, dw1 = ops.CMat.empty(R, Cc), grad(R, Cc), ops.Grad.empty(R, Cc), ops.Grad.empty(R, Cc), ops.Grad.empty(1, Cc)
@@ -224,6 +241,10 @@ def kernel_suite(steps):
     hbm("batch_sum", "batch_sum (one plane)", [R, Cc], 4, n, lambda: ops.batch_sum(u.re, out1))
     del u, v, yy, g, du, dv
 
+
+
+def ce_lines(hbm, cmat, rs):
+    from cnet_amd import capi, ops
     # config 5: CrossEntropy over 32768 logits (rows reduced from 8192 to 2048 to keep the suite short)
     R, Cc = 2048, 32768
     n = R * Cc
@@ -235,7 +256,6 @@ def kernel_suite(steps):
         lambda: ops.cross_entropy_fwd(z, labels, s_, l_, am, None), extra_bytes=4 * R)
     hbm("ce_bwd", "cross_entropy_bwd", [R, Cc], 24, n, lambda: ops.cross_entropy_bwd(z, s_, labels, dz))
     hbm("ce_bwd_sym", "cross_entropy_bwd, conjugate pair (dz only)", [R, Cc], 16, n, lambda: ops.cross_entropy_bwd_sym(z, s_, labels, dz, mirror=False))
-    return lines
 
 
 def token_model_suite(steps, products=4):
@@ -383,6 +403,8 @@ def main():
                          "known size (256 MiB read, 256 MiB written) that calibrates FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--counter-launches", type=int, default=24,
                     help="with --counter-pass: launches in a row of each GEMM kernel after the three calibration rounds")
+    ap.add_argument("--rows", type=int, default=8192,
+                    help="with --suite kernels: rows of the [rows x 4096] planes the HBM-bound kernels run on (8192: 128 MiB per plane)")
     ap.add_argument("--products", type=int, choices=[3, 4], default=4,
                     help="real matrix products per complex one in the block kernels (cnet_cgemm_set_products) for the "
                          "headline step of this run; 4 is the library's default and what the driver's line is measured with")
@@ -396,7 +418,7 @@ def main():
                  "supported. Run with --gpus 1." % args.gpus)
 
     if args.suite == "kernels":
-        for ln in kernel_suite(max(args.steps // 5, 10)):
+        for ln in kernel_suite(max(args.steps // 5, 10), rows=args.rows):
             print(json.dumps(ln))
         return
     if args.suite == "token_model":
@@ -651,7 +673,12 @@ def main():
         if stack:
             out["configs3_residual_stack"] = {"batch": 2048, "lr": STACK_LR, "runs": [stack_brief(t) for t in stack]}
         # id: see kernel_suite; frac: of 157.3 TFLOP/s (cdft_*, ctriang_*: flops executed) or of 8 TB/s (algorithmic bytes)
-        out["kernels"] = [{"id": k["id"], "ms": sig(k["ms"]), "frac": sig(k["roofline"]["frac"])} for k in kernel_suite(20)]
+        # frac4x: the same HBM-bound kernel on planes four times as large ([32768 x 4096], 512 MiB each): at [8192 x 4096] (the
+        # activation shape of configs[4]) a kernel that reads two planes still finds part of them in the 256 MB memory-side cache
+        # from one call to the next; at four times the size every byte comes from and goes to HBM
+        big = {k["id"]: k["roofline"]["frac"] for k in kernel_suite(10, rows=32768, parts=("hbm",))}
+        out["kernels"] = [dict({"id": k["id"], "ms": sig(k["ms"]), "frac": sig(k["roofline"]["frac"])},
+                               **({"frac4x": sig(big[k["id"]])} if k["id"] in big else {})) for k in kernel_suite(20)]
         # api "c": forward + backward as a sequence of C-ABI calls; api "facade": training steps (SGD included) through the
         # C++ facade with one token per sample
         out["configs4_token_model"] = [dict(token_brief(t), api="c") for t in token_model_suite(3)]
