@@ -61,6 +61,8 @@ SIGNATURES = {
     "cnet_clinear_bwd_weight": [c_fp] * 4 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
     "cnet_clinear_bwd_input_sym": [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
     "cnet_clinear_bwd_weight_sym": [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
+    "cnet_clinear_hadamard_cgelu_bwd_sym": [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + ([c_fp] * 4 + [_l, _i]) * 2 +
+                                           [c_fp] * 2 + [_l] + [c_fp] * 2 + ([c_fp] * 4 + [_l]) * 2 + [c_fp] * 4 + [_i, _i, _i, _i],
     "cnet_clinear_bwd_sym": [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 2 + [_l] + [c_fp] * 4 + [_l, _i] + [c_fp] * 4 + [_l, _i, _i, _i, _i],
     "cnet_clinear_cross_entropy_fwd_bwd_sym": [c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, _l, c_fp, c_fp, c_fp, _l, c_fp, c_fp, c_fp] +
                                               [c_fp] * 4 + [_l, _i, _i, _i],

@@ -26,6 +26,7 @@
 // and cgemm_skinny_kernel (a C of few 16 x 16 tiles: one tile per workgroup, K shared among its wavefronts).
 // cgemm_dispatch picks among them and pick_tile picks the block shape.
 #include "common.hpp"
+#include "gate.hpp"
 #include "rows.hpp"
 
 #include <algorithm>
@@ -1014,22 +1015,23 @@ struct SkinnyStrides {
 	unsigned a_kstride, a_mstride, b_kstride, b_nstride, a_bytes, b_bytes;
 };
 
-// the tile numbered `bx` of the product `args`; red = W x 2 x 4 x 64 floats of LDS ([W][re, im][4][64])
-template <int W, bool A_V4, bool B_V4, bool CE = false>
-__device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyStrides &st, const int bx, float *red) {
+// the tile (tile_m, tile_n) of the product `args`; red = W x 2 x 4 x 64 floats of LDS ([W][re, im][4][64]).  KEEP: the finished
+// values (what the planes of C hold afterwards) also go to keep[re, im][row of C][16] in LDS, for a workgroup that goes on
+// with them.  SOLO: the calling wavefront forms the tile alone, for a K of one group (K <= 16), where the other wavefronts
+// of a workgroup would only add zeros: no LDS, no barrier, the same bits; the wavefronts of a workgroup can then take
+// different tiles at the same time.
+template <int W, bool A_V4, bool B_V4, bool CE = false, bool KEEP = false, bool SOLO = false>
+__device__ __forceinline__ void skinny_tile_at(const CgemmArgs &args, const SkinnyStrides &st, const int tile_m, const int tile_n, float *red,
+		float *keep = nullptr) {
+	constexpr int WS = SOLO ? 1 : W;  // wavefronts that share K
 	const unsigned a_kstride = st.a_kstride, a_mstride = st.a_mstride, b_kstride = st.b_kstride, b_nstride = st.b_nstride;
 	const unsigned a_bytes = st.a_bytes, b_bytes = st.b_bytes;
 	constexpr int DEPTH = 3;  // (5 and 8 groups in flight measured 4 to 20 % slower: the loop is not waiting for memory)
 	// the wavefront number as a scalar: the K range, the loop over it and its branches then run on the scalar unit
-	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int wave = SOLO ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 	const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
 	CgemmProblem pb = args.p[blockIdx.y];
 	batch_offset(pb, args);
-	// Consecutive workgroup numbers go round-robin to the XCDs: give each XCD a contiguous run of tiles, row tiles
-	// fastest, so that the tiles sharing columns of B meet in one L2 and each XCD reads its own part of B only.
-	const int total = args.tiles_m * args.tiles_n, xcd = bx % NUM_XCD, share = total / NUM_XCD, extra = total % NUM_XCD;
-	const int tile = xcd * share + min(xcd, extra) + bx / NUM_XCD;
-	const int tile_n = tile / args.tiles_m, tile_m = tile - tile_n * args.tiles_m;
 	const int m0 = tile_m * 16, n0 = tile_n * 16;
 	// lanes beyond the edge of C read the last valid row / column again; their results are not stored
 	const unsigned a_off = 4u * min(m0 + r, args.M - 1) * a_mstride, b_off = 4u * min(n0 + r, args.N - 1) * b_nstride;  // bytes
@@ -1042,7 +1044,7 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 		first = (blockIdx.z % args.splits) * args.chunks_per_split;
 		last = min(last, first + args.chunks_per_split);
 	}
-	const int per = (last - first + W - 1) / W;
+	const int per = (last - first + WS - 1) / WS;
 	const int g_lo = first + wave * per, g_hi = min(last, g_lo + per);
 	long ldc;
 	int accumulate;
@@ -1063,8 +1065,12 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 	const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
 	floatx4 acc_p = zero, acc_r = zero, acc_q = zero, acc_s = zero;
 	Group buf[DEPTH];
+	if constexpr (SOLO) {
+		fetch(buf[0], g_lo);  // the one group there is
+	} else {
 #pragma unroll
-	for (int d = 0; d < DEPTH; ++d) fetch(buf[d], g_lo + d);
+		for (int d = 0; d < DEPTH; ++d) fetch(buf[d], g_lo + d);
+	}
 	// One group: what lies past the end of K is zeroed first (an operand stored along K has its next row or padding
 	// there; four selects per plane, nothing next to 16 MFMAs), then P, R, Q, S advance by four k values per step.
 	auto use = [&](Group &t, int g) __attribute__((always_inline)) {
@@ -1089,27 +1095,38 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 	// stay in the registers they arrived in).  The loop body is one round over the slots without a branch, which lets
 	// the compiler count the loads in flight instead of waiting for all of them; the refill is unconditional (beyond
 	// this wavefront's range it is not used), and what is left after the last full round follows the loop.
-	int g = g_lo;
-	for (; g + DEPTH <= g_hi; g += DEPTH) {
+	if constexpr (SOLO) {
+		if (g_lo < g_hi) use(buf[0], g_lo);
+	} else {
+		int g = g_lo;
+		for (; g + DEPTH <= g_hi; g += DEPTH) {
 #pragma unroll
-		for (int d = 0; d < DEPTH; ++d) {
-			use(buf[d], g + d);
-			fetch(buf[d], g + d + DEPTH);
+			for (int d = 0; d < DEPTH; ++d) {
+				use(buf[d], g + d);
+				fetch(buf[d], g + d + DEPTH);
+			}
 		}
-	}
 #pragma unroll
-	for (int d = 0; d < DEPTH - 1; ++d)
-		if (g + d < g_hi) use(buf[d], g + d);
+		for (int d = 0; d < DEPTH - 1; ++d)
+			if (g + d < g_hi) use(buf[d], g + d);
+	}
 	// re = Ar Br - (sa Ai)(sb Bi), im = Ar (sb Bi) + (sa Ai) Br
 	const float sa = pb.a_im_sign, sb = pb.b_im_sign, sq = -sa * sb;
+	float solo[2][4];
 #pragma unroll
 	for (int e = 0; e < 4; ++e) {
-		red[((wave * 2 + 0) * 4 + e) * 64 + lane] = acc_p[e] + sq * acc_q[e];
-		red[((wave * 2 + 1) * 4 + e) * 64 + lane] = sb * acc_r[e] + sa * acc_s[e];
+		const float fr = acc_p[e] + sq * acc_q[e], fi = sb * acc_r[e] + sa * acc_s[e];
+		if (SOLO) {
+			solo[0][e] = fr;
+			solo[1][e] = fi;
+		} else {
+			red[((wave * 2 + 0) * 4 + e) * 64 + lane] = fr;
+			red[((wave * 2 + 1) * 4 + e) * 64 + lane] = fi;
+		}
 	}
-	__syncthreads();
+	if (!SOLO) __syncthreads();
 	const int col = n0 + r;
-	if (args.mirror == MIRROR_HGELU) {
+	if (!SOLO && args.mirror == MIRROR_HGELU) {
 		// both planes of an element by one lane (the gate needs the complex value): the 4 accumulator registers go to the first
 		// four wavefronts; each plane is added in wavefront order, as below
 		for (int e = wave; e < 4; e += W) {
@@ -1136,17 +1153,14 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 	}
 	// the 8 (plane, accumulator register) pairs are added and stored by the first wavefronts, one or two pairs each
 	__shared__ float logits[CE ? 2 * 16 * 16 : 1];  // CE: the finished tile, [re, im][row][col]
-	for (int c = wave; c < 8; c += W) {
-		const int part = c >> 2, e = c & 3;
-		float v = 0.f;
-#pragma unroll
-		for (int w = 0; w < W; ++w) v += red[((w * 2 + part) * 4 + e) * 64 + lane];
+	auto finish = [&](const int part, const int e, const float v) __attribute__((always_inline)) {
 		const int row = m0 + 4 * q + e;
 		if (CE) logits[(part * 16 + 4 * q + e) * 16 + r] = v;
 		if (row < args.M && col < args.N) {
 			float *dst = (part ? pb.c_im : pb.c_re) + (long) row * ldc + col;
 			const float fin = accumulate ? *dst + v : v;
 			*dst = fin;
+			if (KEEP) keep[(part * cnet::GATE_MAX_ROWS + row) * 16 + r] = fin;
 			if (args.splits == 1) herm_store_part(args, part, row, col, v);
 			if (args.mirror == MIRROR_CONJ && args.splits == 1) {
 				float *m = (part ? args.p[1].c_im : args.p[1].c_re) + (long) row * args.ldc + col;
@@ -1155,6 +1169,19 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 			} else if (args.mirror == MIRROR_GELU && args.splits == 1) {
 				(part ? args.p[1].c_im : args.p[1].c_re)[(long) row * args.ldc + col] = cnet::gelu_value(fin);
 			}
+		}
+	};
+	if constexpr (SOLO) {
+		// (0 + x, as the sum over the wavefronts starts: a zero result is +0 either way)
+#pragma unroll
+		for (int c = 0; c < 8; ++c) finish(c >> 2, c & 3, 0.f + solo[c >> 2][c & 3]);
+	} else {
+		for (int c = wave; c < 8; c += W) {
+			const int part = c >> 2, e = c & 3;
+			float v = 0.f;
+#pragma unroll
+			for (int w = 0; w < W; ++w) v += red[((w * 2 + part) * 4 + e) * 64 + lane];
+			finish(part, e, v);
 		}
 	}
 	if constexpr (CE) {
@@ -1173,6 +1200,17 @@ __device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyS
 	}
 }
 
+// the tile that workgroup number `bx` of a launch over all tiles of `args` takes
+template <int W, bool A_V4, bool B_V4, bool CE = false>
+__device__ __forceinline__ void skinny_tile(const CgemmArgs &args, const SkinnyStrides &st, const int bx, float *red) {
+	// Consecutive workgroup numbers go round-robin to the XCDs: give each XCD a contiguous run of tiles, row tiles
+	// fastest, so that the tiles sharing columns of B meet in one L2 and each XCD reads its own part of B only.
+	const int total = args.tiles_m * args.tiles_n, xcd = bx % NUM_XCD, share = total / NUM_XCD, extra = total % NUM_XCD;
+	const int tile = xcd * share + min(xcd, extra) + bx / NUM_XCD;
+	const int tile_n = tile / args.tiles_m;
+	skinny_tile_at<W, A_V4, B_V4, CE>(args, st, tile - tile_n * args.tiles_m, tile_n, red);
+}
+
 template <int W, bool A_V4, bool B_V4, bool CE = false>
 __global__ __launch_bounds__(64 * W) void cgemm_skinny_kernel(const CgemmArgs args, const SkinnyStrides st) {
 	__shared__ float red[W * 2 * 4 * 64];
@@ -1189,6 +1227,125 @@ __global__ __launch_bounds__(64 * W) void cgemm_skinny_two_kernel(const CgemmArg
 	__shared__ float red[W * 2 * 4 * 64];
 	if ((int) blockIdx.x < tiles0) skinny_tile<W, A_V4, B_V4>(args0, st0, blockIdx.x, red);
 	else skinny_tile<W, A_V4, B_V4>(args1, st1, blockIdx.x - tiles0, red);
+}
+
+// The two backward products of a narrow Linear (args0: dx = g w, all rows of the batch, K <= 16; args1: dw = g^T x) and, behind
+// them, the backward pass of the Hadamard gate with a shared row of weights whose CGelu produced x.  Workgroup n < tiles_n of
+// dx forms columns 16 n .. 16 n + 15 of dx (a row tile per wavefront), keeps them in LDS, takes them through the CGelu and
+// the gate (the arithmetic of hadamard_bwd_shared_sym_kernel, operation for operation) and adds the rows of the batch into
+// dv in the order of that kernel and of slab_sum_sym_kernel<4, 64>; the workgroups after those take the tiles of dw, which
+// the gate does not read.  The bits of the three launches it replaces, without their partial planes.  The gate's operands
+// are fetched before the product starts.
+template <int W, bool A_V4, bool B_V4>
+__global__ __launch_bounds__(64 * W) void cgemm_skinny_gate_bwd_kernel(const CgemmArgs args0, const SkinnyStrides st0, const CgemmArgs args1,
+		const SkinnyStrides st1, const cnet::GateBwd ga) {
+	__shared__ float red[W * 2 * 4 * 64];  // the sums over the wavefronts of a tile of dw, or the slab sums of dv, [slab][re, im][16]
+	__shared__ float keep[2 * cnet::GATE_MAX_ROWS * 16];  // [re, im][row][column of the tile]: dx, then the terms of dv
+	if ((int) blockIdx.x >= args0.tiles_n) {
+		skinny_tile<W, A_V4, B_V4>(args1, st1, blockIdx.x - args0.tiles_n, red);
+		return;
+	}
+	constexpr int PER = cnet::GATE_MAX_ROWS * 16 / (64 * W);  // elements of the column block per thread, at most
+	const int tn = blockIdx.x, n0 = tn * 16, rows = args0.M, cols = args0.N;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int c = threadIdx.x & 15, col = n0 + c;
+	const bool live = col < cols;
+	float ua[PER], ub[PER], vc = 0.f, vd = 0.f;
+	if (live) {
+		vc = ga.v_re[col];
+		vd = ga.v_im[col];
+	}
+#pragma unroll
+	for (int j = 0; j < PER; ++j) {
+		const int row = (threadIdx.x >> 4) + j * (4 * W);
+		ua[j] = ub[j] = 0.f;
+		if (live && row < rows) {
+			ua[j] = ga.u_re[(long) row * ga.ldu + col];
+			ub[j] = ga.u_im[(long) row * ga.ldu + col];
+		}
+	}
+	for (int tm = wave; tm < args0.tiles_m; tm += W) skinny_tile_at<W, A_V4, B_V4, false, true, true>(args0, st0, tm, tn, red, keep);
+	__syncthreads();  // keep holds the column block of dx
+#pragma unroll
+	for (int j = 0; j < PER; ++j) {
+		const int row = (threadIdx.x >> 4) + j * (4 * W);
+		if (!live || row >= rows) continue;
+		const float a = ua[j], b = ub[j];
+		float gr = keep[row * 16 + c], gi = keep[(cnet::GATE_MAX_ROWS + row) * 16 + c];
+		{  // through the CGelu at h = u v, recomputed with the bits of the forward pass
+			const float hr = a * vc - b * vd, hi = a * vd + b * vc;
+			const float px = 0.5f * cnet::gelu_slope(hr), py = 0.5f * cnet::gelu_slope(hi);
+			const float sm = px + py, df = px - py;
+			const float o_r = gr * sm + gr * df, o_i = gi * sm + (-gi) * df;
+			gr = o_r;
+			gi = o_i;
+		}
+		if (ga.dh.dz_re) {
+			const long off = (long) row * ga.lddh + col;
+			ga.dh.dz_re[off] = gr;
+			ga.dh.dz_im[off] = gi;
+			if (ga.dh.dzs_re) {
+				ga.dh.dzs_re[off] = gr;
+				ga.dh.dzs_im[off] = -gi;
+			}
+		}
+		{
+			const float o_r = gr * vc - gi * vd, o_i = gr * vd + gi * vc;
+			const long off = (long) row * ga.lddu + col;
+			if (ga.accumulate) {
+				ga.du.dz_re[off] = ga.du.dz_re[off] + o_r;
+				ga.du.dz_im[off] = ga.du.dz_im[off] + o_i;
+				if (ga.du.dzs_re) {
+					ga.du.dzs_re[off] = ga.du.dzs_re[off] + o_r;
+					ga.du.dzs_im[off] = ga.du.dzs_im[off] + (-o_i);
+				}
+			} else {
+				ga.du.dz_re[off] = o_r;
+				ga.du.dz_im[off] = o_i;
+				if (ga.du.dzs_re) {
+					ga.du.dzs_re[off] = o_r;
+					ga.du.dzs_im[off] = -o_i;
+				}
+			}
+		}
+		keep[row * 16 + c] = gr * a - gi * b;
+		keep[(cnet::GATE_MAX_ROWS + row) * 16 + c] = gr * b + gi * a;
+	}
+	__syncthreads();
+	// dv: the sum of each slab of rows (at most 32 slabs: the host checks), then the slabs
+	const int nslabs = ga.nslabs;
+	for (int idx = threadIdx.x; idx < 32 * nslabs; idx += 64 * W) {
+		const int k = idx >> 5, part = (idx >> 4) & 1;
+		const float *term = keep + part * cnet::GATE_MAX_ROWS * 16 + c;
+		const int r0 = k * ga.rows_per_slab, r1 = min(rows, r0 + ga.rows_per_slab);
+		float acc[cnet::GATE_CS_Y];
+#pragma unroll
+		for (int ty = 0; ty < cnet::GATE_CS_Y; ++ty) {
+			acc[ty] = 0.f;
+			for (int row = r0 + ty; row < r1; row += cnet::GATE_CS_Y) acc[ty] += term[row * 16];
+		}
+		red[idx] = ((acc[0] + acc[1]) + acc[2]) + acc[3];
+	}
+	__syncthreads();
+	if (threadIdx.x < 32 && live) {
+		const int part = threadIdx.x >> 4;
+		const int per = (nslabs + 3) / 4;
+		float s = 0.f;
+#pragma unroll
+		for (int l = 0; l < 4; ++l) {
+			const int k0 = min(nslabs, l * per), k1 = min(nslabs, k0 + per);
+			float run = 0.f;  // the slabs of lane l, in order
+			for (int k = k0; k < k1; ++k) run += red[k * 32 + threadIdx.x];
+			s = l == 0 ? run : s + run;
+		}
+		float *out = part == 0 ? ga.dv.dz_re : ga.dv.dz_im;
+		out[col] = ga.accumulate ? out[col] + s : s;
+		if (ga.dv.dzs_re) {
+			float *m = part == 0 ? ga.dv.dzs_re : ga.dv.dzs_im;
+			const float mv = part == 0 ? s : -s;
+			m[col] = ga.accumulate ? m[col] + mv : mv;
+		}
+	}
 }
 
 SkinnyStrides skinny_strides(const CgemmArgs &args, bool a_mcontig, bool b_ncontig) {
@@ -1336,27 +1493,44 @@ int launch_skinny_two(const CgemmArgs &args0, const SkinnyStrides &st0, const Cg
 	return CNET_OK;
 }
 
-// Two products that are both small enough for cgemm_skinny_kernel, neither cut along K, and that take the same
-// instantiation of it, go out as one launch: true and *rc set.  Otherwise nothing is launched.
-bool try_skinny_two(bool a_mcontig0, bool b_ncontig0, const CgemmArgs &proto0, bool a_mcontig1, bool b_ncontig1, const CgemmArgs &proto1,
-		int nprob, int *rc) {
+// Whether two products are both small enough for cgemm_skinny_kernel, neither cut along K, and take the same
+// instantiation `v` of it, so that they can go out as one launch.
+bool plan_skinny_two(bool a_mcontig0, bool b_ncontig0, const CgemmArgs &proto0, bool a_mcontig1, bool b_ncontig1, const CgemmArgs &proto1,
+		int nprob, CgemmArgs &args0, CgemmArgs &args1, SkinnyVariant &v) {
 	static const bool enabled = [] {
 		const char *e = getenv("CNET_CGEMM_SKINNY_TWO");  // tuning override: 0 launches the two products one after the other
 		return !e || atoi(e) != 0;
 	}();
 	if (!enabled || proto0.M <= 0 || proto0.N <= 0 || proto0.K <= 0 || proto1.M <= 0 || proto1.N <= 0 || proto1.K <= 0) return false;
-	CgemmArgs args0, args1;
 	if (!plan_skinny(a_mcontig0, b_ncontig0, proto0, nprob, 1, args0) || !plan_skinny(a_mcontig1, b_ncontig1, proto1, nprob, 1, args1))
 		return false;
 	if (args0.splits != 1 || args1.splits != 1) return false;
 	// together they must still be a small launch
 	if (((long) args0.tiles_m * args0.tiles_n + (long) args1.tiles_m * args1.tiles_n) * nprob > 4L * cnet::rt().prop.multiProcessorCount)
 		return false;
-	const SkinnyVariant v0 = skinny_variant(a_mcontig0, b_ncontig0, args0, nprob, 1), v1 = skinny_variant(a_mcontig1, b_ncontig1, args1, nprob, 1);
-	if (!(v0 == v1)) return false;
+	v = skinny_variant(a_mcontig0, b_ncontig0, args0, nprob, 1);
+	return v == skinny_variant(a_mcontig1, b_ncontig1, args1, nprob, 1);
+}
+
+// Two such products as one launch: true and *rc set.  Otherwise nothing is launched.
+bool try_skinny_two(bool a_mcontig0, bool b_ncontig0, const CgemmArgs &proto0, bool a_mcontig1, bool b_ncontig1, const CgemmArgs &proto1,
+		int nprob, int *rc) {
+	CgemmArgs args0, args1;
+	SkinnyVariant v0;
+	if (!plan_skinny_two(a_mcontig0, b_ncontig0, proto0, a_mcontig1, b_ncontig1, proto1, nprob, args0, args1, v0)) return false;
 	const SkinnyStrides st0 = skinny_strides(args0, a_mcontig0, b_ncontig0), st1 = skinny_strides(args1, a_mcontig1, b_ncontig1);
 	*rc = CNET_SKINNY_PICK(v0, launch_skinny_two, (args0, st0, args1, st1, nprob));
 	return true;
+}
+
+template <int W, bool A_V4, bool B_V4>
+int launch_skinny_gate_bwd(const CgemmArgs &args0, const SkinnyStrides &st0, const CgemmArgs &args1, const SkinnyStrides &st1,
+		const cnet::GateBwd &gate) {
+	auto kern = cgemm_skinny_gate_bwd_kernel<W, A_V4, B_V4>;
+	hipLaunchKernelGGL(kern, dim3(args0.tiles_n + args1.tiles_m * args1.tiles_n, 1, 1), dim3(64 * W), 0, cnet::rt().stream, args0, st0, args1, st1,
+			gate);
+	CNET_LAUNCH_CHECK();
+	return CNET_OK;
 }
 
 // tail_splits >= 2: cut the blocks of the last, partly filled round into that many pieces along K (see CgemmArgs)
@@ -1837,6 +2011,27 @@ int cgemm_dft_hgelu(int M, int n, const float *x_re, const float *x_im, long ldx
 
 // One product whose A (row-major) has an imaginary plane of nothing but +0, against a k-major B (used by cdft.hip)
 // herm_n > 0: the conjugate of column c, 1 <= c <= herm_n - N, is also written to column herm_n - c (the columns from N on)
+bool cgemm_linear_bwd_gate(const float *g_re, const float *g_im, long ldg, const float *x_re, const float *x_im, long ldx, const float *w_re,
+		const float *w_im, long ldw, const Pair2 &dx, long lddx, int accumulate_dx, const Pair2 &dw, long lddw, int accumulate_dw, int B, int K,
+		int N, const GateBwd &gate, int *rc) {
+	if (B > GATE_MAX_ROWS) return false;
+	// the two products as cnet_clinear_bwd_sym sets them up
+	const float *gr[2] = {g_re, g_re}, *gi[2] = {g_im, g_im};
+	const float *wr[2] = {w_re, w_re}, *wi[2] = {w_im, w_im}, *xr[2] = {x_re, x_re}, *xi[2] = {x_im, x_im};
+	float *dxr[2] = {dx.dz_re, dx.dzs_re}, *dxi[2] = {dx.dz_im, dx.dzs_im}, *dwr[2] = {dw.dz_re, dw.dzs_re}, *dwi[2] = {dw.dz_im, dw.dzs_im};
+	const bool cj[2] = {false, false};
+	const CgemmArgs to_input = pair_args(1, B, K, N, gr, gi, ldg, wr, wi, ldw, cj, dxr, dxi, lddx, accumulate_dx, 0, dx.dzs_re ? MIRROR_CONJ : 0);
+	const CgemmArgs to_weight = pair_args(1, N, K, B, gr, gi, ldg, xr, xi, ldx, cj, dwr, dwi, lddw, accumulate_dw, 0, dw.dzs_re ? MIRROR_CONJ : 0);
+	CgemmArgs args0, args1;
+	SkinnyVariant v;
+	if (!plan_skinny_two(false, true, to_input, true, true, to_weight, 1, args0, args1, v)) return false;
+	// one group of K per tile of dx (a wavefront forms it alone), the slab sums in LDS, one column block per workgroup
+	if (args0.K > 16 || gate.nslabs > 32 || v.w * 64 * 2 * 4 < 32 * gate.nslabs) return false;
+	const SkinnyStrides st0 = skinny_strides(args0, false, true), st1 = skinny_strides(args1, true, true);
+	*rc = CNET_SKINNY_PICK(v, launch_skinny_gate_bwd, (args0, st0, args1, st1, gate));
+	return true;
+}
+
 int cgemm_real_a(int M, int N, int K, const float *a_re, const float *a_im, long lda, const float *b_re, const float *b_im, long ldb, float *c_re,
 		float *c_im, long ldc, int herm_n) {
 	const float *ar[2] = {a_re, a_re}, *ai[2] = {a_im, a_im}, *br[2] = {b_re, b_re}, *bi[2] = {b_im, b_im};

@@ -5,6 +5,7 @@
 // handles one group of V consecutive columns (V = 4 -> 128-bit loads and stores; V = 1 for odd shapes), so a
 // wavefront touches 1 KiB of each plane per access and every byte is read and written exactly once.
 #include "common.hpp"
+#include "gate.hpp"
 
 #include <algorithm>
 #include <cmath>
@@ -152,7 +153,7 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_kernel(const float *__restri
 // of rows.  Each thread writes du for its rows and keeps the four dv sums of those rows in registers; the four row
 // lanes are added through LDS in lane order and partial[slab][plane][cols] goes to the workspace; a second kernel adds
 // the slabs in slab order.  Deterministic: no atomics, fixed summation tree.
-constexpr int CS_X = 64, CS_Y = 4;
+constexpr int CS_X = cnet::GATE_CS_X, CS_Y = cnet::GATE_CS_Y;
 
 template <int V, int NT>
 __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *__restrict__ ur, const float *__restrict__ ui,
@@ -458,9 +459,7 @@ __global__ __launch_bounds__(TPB) void crossent_bwd_kernel(const float *__restri
 // conjugate pair), and write the dz* planes as the conjugate only where the caller passes them (non-NULL): a consumer
 // that is itself one of these kernels, or a conjugate-pair matrix product, never reads them.  24 bytes per complex
 // element instead of 40 (CGelu, CRelu, Hadamard, SoftMax), 24 instead of 48 (Residual), 16 instead of 24 (the losses).
-struct Pair2 {  // dz planes, and optionally the planes that receive the conjugate
-	float *dz_re, *dz_im, *dzs_re, *dzs_im;
-};
+using cnet::Pair2;  // dz planes, and optionally the planes that receive the conjugate (gate.hpp)
 
 // (o_r, o_i) to the dz planes and, conjugated, to the dz* planes when they are wanted
 template <int V, int NT>
@@ -1437,6 +1436,15 @@ int cnet_residual_cgelu_bwd_sym(const float *g1_dz_re, const float *g1_dz_im, in
 	return CNET_OK;
 }
 
+// whether the backward pass of a Hadamard for a conjugate pair runs on 128-bit accesses
+static bool hadamard_sym_vec(bool gelu, const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,
+		const float *g_dz_re, const float *g_dz_im, int64_t ldg, const Pair2 &dh, int64_t lddh, const Pair2 &du, int64_t lddu, const Pair2 &dv,
+		int64_t lddv, int cols) {
+	return all_mult4({cols, ldu, ldv, ldg, lddu, ldv ? lddv : 0, gelu && dh.dz_re ? lddh : 0}) &&
+			all_aligned({u_re, u_im, v_re, v_im, g_dz_re, g_dz_im, du.dz_re, du.dz_im, du.dzs_re, du.dzs_im, dv.dz_re, dv.dz_im, dv.dzs_re,
+					dv.dzs_im, gelu ? dh.dz_re : nullptr, gelu ? dh.dz_im : nullptr, gelu ? dh.dzs_re : nullptr, gelu ? dh.dzs_im : nullptr});
+}
+
 // gelu: the incoming gradient belongs to a CGelu applied to the Hadamard's result; dh receives the gradient of that CGelu's
 // operand
 static int hadamard_bwd_sym_impl(const char *who, bool gelu, const float *u_re, const float *u_im, int64_t ldu, const float *v_re,
@@ -1451,9 +1459,7 @@ static int hadamard_bwd_sym_impl(const char *who, bool gelu, const float *u_re, 
 		return fail(CNET_ERR_INVALID_ARGUMENT, "%s: a required plane is NULL (the dz* planes of a result are optional, in pairs)", who);
 	if (!(ldu >= cols && ldg >= cols && lddu >= cols && (ldv == 0 || (ldv >= cols && lddv >= cols)) && (!gelu || !dh.dz_re || lddh >= cols)))
 		return fail(CNET_ERR_INVALID_ARGUMENT, "%s: a leading dimension is shorter than the row", who);
-	const bool vec = all_mult4({cols, ldu, ldv, ldg, lddu, ldv ? lddv : 0, gelu && dh.dz_re ? lddh : 0}) &&
-			all_aligned({u_re, u_im, v_re, v_im, g_dz_re, g_dz_im, du.dz_re, du.dz_im, du.dzs_re, du.dzs_im, dv.dz_re, dv.dz_im, dv.dzs_re,
-					dv.dzs_im, gelu ? dh.dz_re : nullptr, gelu ? dh.dz_im : nullptr, gelu ? dh.dzs_re : nullptr, gelu ? dh.dzs_im : nullptr});
+	const bool vec = hadamard_sym_vec(gelu, u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg, dh, lddh, du, lddu, dv, lddv, cols);
 	const int nt = stream_policy(ST_LOADS, 4 + pair_planes(du) + (ldv ? 2 + pair_planes(dv) : 0) + (gelu && dh.dz_re ? pair_planes(dh) : 0), (long) rows * cols);
 	if (ldv != 0) {
 		if (vec)
@@ -1467,12 +1473,8 @@ static int hadamard_bwd_sym_impl(const char *who, bool gelu, const float *u_re, 
 	}
 	const int V = vec ? 4 : 1;
 	const long col_blocks = ((long) cols / V + CS_X - 1) / CS_X;
-	// two workgroups per compute unit: against four, 129 instead of 138 us at 8192 x 4096 and 10.0 instead of 11.4 us at
-	// 1024 x 784 (half as many slabs for the second kernel to add); one per unit is slower everywhere
-	int nslabs = (int) std::max(1L, std::min(256L, 2L * rt().prop.multiProcessorCount / col_blocks));
-	nslabs = std::min(nslabs, (rows + CS_Y - 1) / CS_Y);
-	const int rows_per_slab = (rows + nslabs - 1) / nslabs;
-	nslabs = (rows + rows_per_slab - 1) / rows_per_slab;
+	int nslabs, rows_per_slab;
+	cnet::gate_slabs(rows, cols, V, rt().prop.multiProcessorCount, &nslabs, &rows_per_slab);
 	float *partial = (float *) workspace((size_t) nslabs * 2 * cols * sizeof(float));
 	if (!partial) return CNET_ERR_OUT_OF_MEMORY;
 	dim3 grid((unsigned) col_blocks, (unsigned) nslabs);
@@ -1507,6 +1509,38 @@ int cnet_hadamard_cgelu_bwd_sym(const float *u_re, const float *u_im, int64_t ld
 	return hadamard_bwd_sym_impl(__func__, true, u_re, u_im, ldu, v_re, v_im, ldv, g_dz_re, g_dz_im, ldg,
 			pair_of(dh_dz_re, dh_dz_im, dh_dzs_re, dh_dzs_im), lddh, pair_of(du_dz_re, du_dz_im, du_dzs_re, du_dzs_im), lddu,
 			pair_of(dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im), lddv, rows, cols, accumulate);
+}
+
+int cnet_clinear_hadamard_cgelu_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg, const float *x_re, const float *x_im,
+		int64_t ldx, const float *w_re, const float *w_im, int64_t ldw, float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im,
+		int64_t lddx, int accumulate_dx, float *dw_dz_re, float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im, int64_t lddw, int accumulate_dw,
+		const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, float *dh_dz_re, float *dh_dz_im,
+		float *dh_dzs_re, float *dh_dzs_im, int64_t lddh, float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
+		float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int accumulate_gate, int B, int K, int N) {
+	CNET_REQUIRE_INIT();
+	const Pair2 dx = pair_of(dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im), dw = pair_of(dw_dz_re, dw_dz_im, dw_dzs_re, dw_dzs_im);
+	const Pair2 dh = pair_of(dh_dz_re, dh_dz_im, dh_dzs_re, dh_dzs_im), du = pair_of(du_dz_re, du_dz_im, du_dzs_re, du_dzs_im);
+	const Pair2 dv = pair_of(dv_dz_re, dv_dz_im, dv_dzs_re, dv_dzs_im);
+	auto pair_ok = [](const Pair2 &p) { return p.dz_re && p.dz_im && ((p.dzs_re == nullptr) == (p.dzs_im == nullptr)); };
+	// One launch when every argument is in order and both products are small (the workgroup that owns 16 columns of dx goes
+	// on to the gate's backward pass of those columns); whatever is not goes to the two calls, which name what is wrong.
+	const bool plain = B > 0 && K > 0 && N > 0 && g_dz_re && g_dz_im && x_re && x_im && w_re && w_im && u_re && u_im && v_re && v_im &&
+			pair_ok(dx) && pair_ok(dw) && pair_ok(du) && pair_ok(dv) && (pair_ok(dh) || !(dh.dz_re || dh.dz_im || dh.dzs_re || dh.dzs_im)) &&
+			ldg >= N && ldx >= K && ldw >= K && lddx >= K && lddw >= K && ldu >= K && lddu >= K && (!dh.dz_re || lddh >= K);
+	if (plain) {
+		cnet::GateBwd gate{u_re, u_im, ldu, v_re, v_im, dh, lddh, du, lddu, dv, accumulate_gate, 0, 0};
+		const bool vec = hadamard_sym_vec(true, u_re, u_im, ldu, v_re, v_im, 0, dx_dz_re, dx_dz_im, lddx, dh, lddh, du, lddu, dv, K, K);
+		cnet::gate_slabs(B, K, vec ? 4 : 1, rt().prop.multiProcessorCount, &gate.nslabs, &gate.rows_per_slab);
+		int rc = CNET_OK;
+		if (cnet::cgemm_linear_bwd_gate(g_dz_re, g_dz_im, ldg, x_re, x_im, ldx, w_re, w_im, ldw, dx, lddx, accumulate_dx, dw, lddw,
+					accumulate_dw, B, K, N, gate, &rc))
+			return rc;
+	}
+	const int rc = cnet_clinear_bwd_sym(g_dz_re, g_dz_im, ldg, x_re, x_im, ldx, w_re, w_im, ldw, dx_dz_re, dx_dz_im, dx_dzs_re, dx_dzs_im, lddx,
+			accumulate_dx, dw_dz_re, dw_dz_im, dw_dzs_re, dw_dzs_im, lddw, accumulate_dw, B, K, N);
+	if (rc != CNET_OK) return rc;
+	return hadamard_bwd_sym_impl(__func__, true, u_re, u_im, ldu, v_re, v_im, 0, dx_dz_re, dx_dz_im, lddx, dh, lddh, du, lddu, dv, K, B, K,
+			accumulate_gate);
 }
 
 int cnet_hadamard_cgelu_fwd(const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im, int64_t ldv,

@@ -533,6 +533,9 @@ protected:
 	// (cnet_cdft_hadamard_cgelu_fwd: one launch at small batches): fused_next_ of the transform names the Hadamard, and
 	// fwd_by_producer_ of the Hadamard says that the transform of this forward pass has written its planes and the CGelu's.
 	bool fwd_by_producer_ = false;
+	// A narrow Linear whose operand is the CGelu of a Hadamard gate with a shared row takes the backward pass of that pair
+	// into its own call (cnet_clinear_hadamard_cgelu_bwd_sym): bwd_by_consumer_now_ of the Hadamard is then set for the pass.
+	bool bwd_by_consumer_now_ = false;
 	// A Linear that feeds nothing but a CrossEntropy hands its product and the loss (forward pass and gradient) to one call
 	// (cnet_clinear_cross_entropy_fwd_bwd_sym: one launch for a narrow head) whenever the loss would write its gradient from
 	// its forward pass anyway: loss_next_ of the Linear names the CrossEntropy, whose fwd_by_producer_ is then set per pass.
@@ -1512,6 +1515,7 @@ private:
 			f->fused_next_ = NULL;
 			f->loss_next_ = NULL;
 			f->fwd_by_producer_ = false;
+			f->bwd_by_consumer_now_ = false;
 			f->fused_prev_ = 0;
 			f->fused_gelu_slot_ = -1;
 			f->bwd_by_consumer_ = false;
@@ -1556,6 +1560,16 @@ private:
 				g->bwd_by_consumer_ = true;
 			}
 		}
+	}
+
+	// Whether the operand of the Linear f is the CGelu of a Hadamard gate with one shared row of weights that runs its backward
+	// pass with that CGelu's (fused_prev_ == 2: the CGelu feeds f only) in this pass, on rows of the same count.
+	bool gateBelow(CFunc *f) const {
+		CFunc *g = f->slots_[0].producer;
+		if (!g || g->typeId() != isGelu || g->fused_prev_ != 2 || g->rows_ != f->rows_ || f->slots_[0].len != g->out_size_) return false;
+		CFunc *h = g->slots_[0].producer;
+		return h && h->typeId() == isHadamard && h->fused_next_ == g && h->rows_ == f->rows_ && h->slots_.size() == 2 &&
+				h->slots_[1].rows == 1 && h->slots_[0].rows == f->rows_ && !h->lazy_now_ && !h->lazy_skip_now_;
 	}
 
 	// z planes of slot k of node f (read in place from the producer)
@@ -1787,6 +1801,18 @@ private:
 				const int K = a.len, N = f->out_size_;
 				// (the input gradient of a lazy data input waits: see CFunc::lazy_bwd_)
 				const bool to_data = a.producer->wants_grad_ && !f->lazy_skip_now_, to_weight = w.producer->wants_grad_;
+				if (conjugate_gradients_ && to_data && to_weight && f->no_outputs() == 1 && gateBelow(f)) {
+					// the operand is the CGelu of a Hadamard gate with a shared row: the gate's backward pass in the same call (one
+					// launch at small batches: the workgroup that forms 16 columns of dx goes on to the gate)
+					CFunc *g = a.producer, *h = g->slots_[0].producer;
+					CFunc::Slot &hs = g->slots_[0], &hu = h->slots_[0], &hv = h->slots_[1];
+					ck(cnet_clinear_hadamard_cgelu_bwd_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1),
+							a.gs(2), a.gs(3), K, acc, w.g(0), w.g(1), w.gs(2), w.gs(3), K, acc, zre(h, 0), zim(h, 0), K, zre(h, 1), zim(h, 1), hs.g(0),
+							hs.g(1), hs.gs(2), hs.gs(3), K, hu.g(0), hu.g(1), hu.gs(2), hu.gs(3), K, hv.g(0), hv.g(1), hv.gs(2), hv.gs(3), 0, rows, K, N),
+							"cnet_clinear_hadamard_cgelu_bwd_sym");
+					h->bwd_by_consumer_now_ = true;
+					break;
+				}
 				if (conjugate_gradients_ && to_data && to_weight) {  // both gradients in one call (one launch when both products are small)
 					ck(cnet_clinear_bwd_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.gs(2),
 							a.gs(3), K, acc, w.g(0), w.g(1), w.gs(2), w.gs(3), K, acc, rows, K, N), "cnet_clinear_bwd_sym");
@@ -1853,6 +1879,10 @@ private:
 			case isHadamard: {
 				CFunc::Slot &v = f->slots_[1];
 				const int n = f->out_size_;
+				if (f->bwd_by_consumer_now_) {  // done by the Linear above its CGelu in this pass
+					f->bwd_by_consumer_now_ = false;
+					break;
+				}
 				if (conjugate_gradients_ && f->fused_next_) {  // the backward pass of the CGelu above it in the same pass
 					CFunc *g = f->fused_next_;
 					CFunc::Slot &ug = upstream(g, 0), &h = g->slots_[0];

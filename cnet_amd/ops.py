@@ -156,6 +156,14 @@ def linear_bwd_sym(g, x, w, dx, dw, accumulate_dx=0, accumulate_dw=0, mirror_dx=
          *_mirrored(dw, mirror_dw), dw.ld, accumulate_dw, g.rows, w.cols, w.rows)
 
 
+def linear_hadamard_gelu_bwd_sym(g, x, w, dx, dw, u, v, dh, du, dv, accumulate_dx=0, accumulate_dw=0, accumulate_gate=0, mirror=True):
+    """linear_bwd_sym, then hadamard_gelu_bwd_sym with a shared row v on dx, in one call (one launch at small batches)."""
+    ph = _pair(dh, mirror) if dh is not None else (None,) * 4
+    call("cnet_clinear_hadamard_cgelu_bwd_sym", *g.p()[:2], g.ld, *x.p(), x.ld, *w.p(), w.ld, *_mirrored(dx, mirror), dx.ld, accumulate_dx,
+         *_mirrored(dw, mirror), dw.ld, accumulate_dw, *u.p(), u.ld, *v.p(), *ph, dh.ld if dh is not None else 0, *_pair(du, mirror), du.ld,
+         *_pair(dv, mirror), accumulate_gate, g.rows, w.cols, w.rows)
+
+
 def dft_fwd(x, y, accumulate=0):
     call("cnet_cdft_fwd", *x.p(), x.ld, *y.p(), y.ld, x.rows, x.cols, accumulate)
 

@@ -437,6 +437,24 @@ int cnet_hadamard_cgelu_bwd_sym(const float *u_re, const float *u_im, int64_t ld
                                 float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
                                 float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int64_t lddv,
                                 int rows, int cols, int accumulate);
+/* The backward pass of a narrow Linear whose operand x = gelu(u .* v) came from a Hadamard gate with one shared row of weights
+ * v under a CGelu: cnet_clinear_bwd_sym (dx, dw from the gradient g at the Linear's result) followed by
+ * cnet_hadamard_cgelu_bwd_sym with ldv = 0 on dx (dh at the CGelu's operand, du, and dv summed over the batch), with the
+ * arguments and the bits of those two calls.  Upstream runs LinearGpu::backward, gpu_gelu_backward and
+ * gpu_hadamard_backward one after the other (gpu/reducegrad.cpp:324-336, gpu/kernels.cpp:204-360).  One launch when the batch
+ * has at most 128 rows and both products fit the small-C kernel without slices of K: the workgroup that has formed 16 columns
+ * of dx (all rows) and of dw goes on to the gate's backward pass of those columns and adds their rows into dv in the order of
+ * the separate launches.  Otherwise those two calls (three to four launches). */
+int cnet_clinear_hadamard_cgelu_bwd_sym(const float *g_dz_re, const float *g_dz_im, int64_t ldg,
+                                        const float *x_re, const float *x_im, int64_t ldx,
+                                        const float *w_re, const float *w_im, int64_t ldw,
+                                        float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx, int accumulate_dx,
+                                        float *dw_dz_re, float *dw_dz_im, float *dw_dzs_re, float *dw_dzs_im, int64_t lddw, int accumulate_dw,
+                                        const float *u_re, const float *u_im, int64_t ldu, const float *v_re, const float *v_im,
+                                        float *dh_dz_re, float *dh_dz_im, float *dh_dzs_re, float *dh_dzs_im, int64_t lddh,
+                                        float *du_dz_re, float *du_dz_im, float *du_dzs_re, float *du_dzs_im, int64_t lddu,
+                                        float *dv_dz_re, float *dv_dz_im, float *dv_dzs_re, float *dv_dzs_im, int accumulate_gate,
+                                        int B, int K, int N);
 int cnet_crelu_bwd_sym(const float *x_re, const float *x_im, int64_t ldx, const float *g_dz_re, const float *g_dz_im, int64_t ldg,
                        float *dx_dz_re, float *dx_dz_im, float *dx_dzs_re, float *dx_dzs_im, int64_t lddx,
                        int rows, int cols, int accumulate);

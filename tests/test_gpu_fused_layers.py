@@ -217,3 +217,49 @@ def test_linear_head_and_its_loss_in_one_call(gpu, port, B, K, N):
         h = d.host()
         # (the gradient at a label whose logit is small is large and as ill conditioned as 1 / |z_label|: the bar itself)
         assert rel_c(h[0:2], want[0:2]) < TOL and rel_c(h[2:4], want[2:4]) < TOL
+
+
+# B, K (hidden width = columns of the gate), N (outputs of the Linear): up to 128 rows with small products take one launch;
+# 129 and 200 rows, and 784 outputs (products beyond the small-C kernel) the separate launches
+GATED_HEADS = [(64, 784, 10), (1, 4, 1), (3, 20, 2), (16, 96, 16), (100, 333, 12), (128, 784, 10), (127, 130, 5), (129, 784, 10),
+               (200, 64, 7), (64, 784, 784), (60, 2052, 10)]
+
+
+@pytest.mark.parametrize("B,K,N", GATED_HEADS)
+def test_backward_pass_of_a_linear_and_the_gate_below_it_in_one_call(gpu, port, B, K, N):
+    """cnet_clinear_hadamard_cgelu_bwd_sym against cnet_clinear_bwd_sym followed by cnet_hadamard_cgelu_bwd_sym (shared row):
+    same bits in dx, dw, dh, du and dv, with each accumulate flag, with and without the dz* planes, with and without dh; and
+    the gradients against the CPU path (Linear, CGelu and Hadamard backward of the oracle on the same conjugate pair)."""
+    u = ops.CMat.from_host(seeded(port, K + 1, (B, K)), seeded(port, K + 2, (B, K)))
+    v = ops.CMat.from_host(seeded(port, K + 3, (1, K)), seeded(port, K + 4, (1, K)))
+    h, x = ops.CMat.empty(B, K), ops.CMat.empty(B, K)
+    ops.hadamard_gelu_fwd(u, v, h, x, shared=True)
+    w = ops.CMat.from_host(seeded(port, N + 5, (N, K)), seeded(port, N + 6, (N, K)))
+    gr, gi = seeded(port, B + 7, (B, N)), seeded(port, B + 8, (B, N))
+    g = ops.Grad.from_host([gr, gi, gr, -gi])
+    bx, bw, bv = ([seeded(port, s + p, shape) for p in range(4)] for s, shape in ((20, (B, K)), (30, (N, K)), (40, (1, K))))
+    cases = ((0, 0, 0, True, True), (1, 0, 1, True, True), (0, 1, 0, False, True), (1, 1, 1, True, False), (0, 0, 1, False, False))
+    for acc_x, acc_w, acc_g, mirror, with_dh in cases:
+        def planes():
+            return (ops.Grad.from_host(bx), ops.Grad.from_host(bw), ops.Grad.from_host(bx) if with_dh else None, ops.Grad.from_host(bx),
+                    ops.Grad.from_host(bv))
+        dx0, dw0, dh0, du0, dv0 = planes()
+        ops.linear_bwd_sym(g, x, w, dx0, dw0, accumulate_dx=acc_x, accumulate_dw=acc_w, mirror_dx=mirror, mirror_dw=mirror)
+        ops.hadamard_gelu_bwd_sym(u, v, dx0, dh0, du0, dv0, shared=True, accumulate=acc_g, mirror=mirror)
+        dx1, dw1, dh1, du1, dv1 = planes()
+        ops.linear_hadamard_gelu_bwd_sym(g, x, w, dx1, dw1, u, v, dh1, du1, dv1, accumulate_dx=acc_x, accumulate_dw=acc_w,
+                                         accumulate_gate=acc_g, mirror=mirror)
+        for name, a, b in (("dx", dx0, dx1), ("dw", dw0, dw1), ("dh", dh0, dh1), ("du", du0, du1), ("dv", dv0, dv1)):
+            if a is None:
+                continue
+            for pa, pb in zip(a.host(), b.host()):
+                assert np.array_equal(pa, pb), (name, acc_x, acc_w, acc_g, mirror, with_dh)
+    # the CPU path on the same pair
+    (ur, ui), (vr, vi), (hr, hi), (xr, xi), (wr, wi) = u.host(), v.host(), h.host(), x.host(), w.host()
+    dxo, dwo = port.linear_bwd(xr, xi, wr, wi, [gr, gi, gr, -gi])
+    dho = port.gelu_bwd(hr, hi, dxo)
+    duo, dvo = port.hadamard_bwd(ur, ui, np.ascontiguousarray(vr[0]), np.ascontiguousarray(vi[0]), dho)   # shared row: dv summed over the batch
+    dx1, dw1, dh1, du1, dv1 = ops.Grad.empty(B, K), ops.Grad.empty(N, K), ops.Grad.empty(B, K), ops.Grad.empty(B, K), ops.Grad.empty(1, K)
+    ops.linear_hadamard_gelu_bwd_sym(g, x, w, dx1, dw1, u, v, dh1, du1, dv1)
+    for got, want in ((dx1, dxo), (dw1, dwo), (dh1, dho), (du1, duo), (dv1, [p[None, :] for p in dvo])):
+        assert rel_c(got.host()[0:2], want[0:2]) < TOL / 5 and rel_c(got.host()[2:4], want[2:4]) < TOL / 5
