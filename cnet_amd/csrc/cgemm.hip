@@ -2009,8 +2009,6 @@ int cgemm_dft_hgelu(int M, int n, const float *x_re, const float *x_im, long ldx
 	return CNET_SKINNY_PICK(v, launch_skinny, (planned, false, true, 1, 1));
 }
 
-// One product whose A (row-major) has an imaginary plane of nothing but +0, against a k-major B (used by cdft.hip)
-// herm_n > 0: the conjugate of column c, 1 <= c <= herm_n - N, is also written to column herm_n - c (the columns from N on)
 bool cgemm_linear_bwd_gate(const float *g_re, const float *g_im, long ldg, const float *x_re, const float *x_im, long ldx, const float *w_re,
 		const float *w_im, long ldw, const Pair2 &dx, long lddx, int accumulate_dx, const Pair2 &dw, long lddw, int accumulate_dw, int B, int K,
 		int N, const GateBwd &gate, int *rc) {
@@ -2032,6 +2030,8 @@ bool cgemm_linear_bwd_gate(const float *g_re, const float *g_im, long ldg, const
 	return true;
 }
 
+// One product whose A (row-major) has an imaginary plane of nothing but +0, against a k-major B (used by cdft.hip)
+// herm_n > 0: the conjugate of column c, 1 <= c <= herm_n - N, is also written to column herm_n - c (the columns from N on)
 int cgemm_real_a(int M, int N, int K, const float *a_re, const float *a_im, long lda, const float *b_re, const float *b_im, long ldb, float *c_re,
 		float *c_im, long ldc, int herm_n) {
 	const float *ar[2] = {a_re, a_re}, *ai[2] = {a_im, a_im}, *br[2] = {b_re, b_re}, *bi[2] = {b_im, b_im};
