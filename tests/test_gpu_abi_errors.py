@@ -72,6 +72,31 @@ def test_invalid_arguments_are_reported_not_fatal(gpu, port):
     assert _status("cnet_clinear_cgelu_fwd", *x.p(), 8, *w.p(), 8, *h.p(), y.re.ptr, None, 8, 4, 8, 8, 0) == INVALID      # a plane of y missing
     assert _status("cnet_clinear_cgelu_fwd", *x.p(), 8, *w.p(), 8, *h.p(), *y.p(), 4, 4, 8, 8, 0) == INVALID              # ldy < N
     assert _status("cnet_clinear_cgelu_fwd", *x.p(), 8, *w.p(), 8, *h.p(), *y.p(), 8, 0, 8, 8, 0) == 0
+    # the calls that carry a layer and what follows it in one launch at small batches hand a bad argument to the separate calls,
+    # which name it
+    v1 = ops.CMat.from_host(seeded(port, 5, (1, 8)), seeded(port, 6, (1, 8)))
+    a8 = ops.CMat.empty(4, 8)
+    du, dv, dh = ops.Grad.empty(4, 8), ops.Grad.empty(1, 8), ops.Grad.empty(4, 8)
+
+    def gated(g_im=g.p()[1], ldx=8, dw_dzs_im=dw.p()[3], u_im=x.im.ptr, lddu=8, dh4=dh.p(), B=4):
+        return _status("cnet_clinear_hadamard_cgelu_bwd_sym", g.p()[0], g_im, 8, *a8.p(), ldx, *w.p(), 8, *dx.p(), 8, 0, *dw.p()[:3], dw_dzs_im,
+                       8, 0, x.re.ptr, u_im, 8, *v1.p(), *dh4, 8, *du.p(), lddu, *dv.p(), 0, B, 8, 8)
+    assert gated() == 0 and gated(dh4=none4) == 0
+    assert gated(g_im=None) == INVALID and gated(ldx=4) == INVALID and gated(dw_dzs_im=None) == INVALID
+    assert gated(u_im=None) == INVALID and gated(lddu=4) == INVALID and gated(dh4=(dh.p()[0], None, None, None)) == INVALID
+    assert gated(B=0) == INVALID   # as cnet_clinear_bwd_sym: no rows
+    assert _status("cnet_cdft_plan", 8) == 0
+    assert _status("cnet_cdft_hadamard_cgelu_fwd", *x.p(), 8, *v1.p(), *y.p(), *h.p(), *a8.p(), 8, 4, 8) == 0
+    assert _status("cnet_cdft_hadamard_cgelu_fwd", *x.p(), 8, v1.re.ptr, None, *y.p(), *h.p(), *a8.p(), 8, 4, 8) == INVALID   # half a gate
+    assert _status("cnet_cdft_hadamard_cgelu_fwd", *x.p(), 8, *v1.p(), *y.p(), *h.p(), *a8.p(), 4, 4, 8) == INVALID           # ld < n
+    lab = ops.ints(np.zeros(4, np.int32))
+    s4, l4, am4 = capi.empty(4), capi.empty(4), capi.empty(4, np.int32)
+
+    def head(w_im=w.im.ptr, ldy=8, labels=lab.ptr, dz_im=dx.p()[1]):
+        return _status("cnet_clinear_cross_entropy_fwd_bwd_sym", *x.p(), 8, w.re.ptr, w_im, 8, *y.p(), ldy, labels, None, None, 0, s4.ptr,
+                       l4.ptr, am4.ptr, dx.p()[0], dz_im, None, None, 8, 4, 8, 8)
+    assert head() == 0
+    assert head(w_im=None) == INVALID and head(ldy=4) == INVALID and head(labels=None) == INVALID and head(dz_im=None) == INVALID
     # DFT length beyond the int exponent range of the reference, Adam with a negative step, unknown marker
     assert _status("cnet_cdft_plan", 50000) == INVALID
     assert _status("cnet_adam_update", x.re.ptr, x.im.ptr, y.re.ptr, y.im.ptr, y.re.ptr, y.im.ptr, 32, 0.1, 0.9, -1, 1) == INVALID
