@@ -41,7 +41,7 @@ def measured_traffic():
     return table, at
 
 
-B, K, N = 4096, 1024, 1024      # BASELINE.json configs[1]
+B, K, N = 4096, 1024, 1024      # the configuration the metric is quoted on: batched complex Linear, 4096 samples, 1024 -> 1024
 
 
 class HipEvents:
