@@ -526,7 +526,7 @@ int cnet_embedding_bwd(const int32_t *tokens, const float *g_dzs_re, const float
  *   CNET_CGEMM_SKINNY = 0        small products on the block kernels instead of the small-C kernel
  *   CNET_CGEMM_SKINNY_TILES = n  largest number of 16x16 tiles of C the small-C kernel takes (default 4 per compute unit)
  *   CNET_CGEMM_SKINNY_W = 4|8|16 wavefronts per tile of the small-C kernel
- *   CNET_CGEMM_SKINNY_TWO = 0    two small products of one call as two launches
+ *   CNET_CGEMM_SKINNY_TWO = 0    two small products of one call as two launches (and the gate behind them as launches of its own)
  *   CNET_CGEMM_3M = 0 | 1        initial value of cnet_cgemm_set_products (1: three real products per complex one)
  *   CNET_STREAM_MIN_MB = n       footprint (MiB) from which an elementwise / row launch counts as streaming (default 256)
  *   CNET_STREAM_POLICY = 0..3    cache policy of every streaming launch: plain, hint on loads and stores, hinted stores,
