@@ -301,6 +301,11 @@ class CrossEntropy : public CFunc, public OutputFunc {
 	bool grad_from_forward_ = false;
 	int32_t *d_argmax_ = NULL;
 	float *d_norm_ = NULL;                  // device: normalised z, 2 planes [rows][n]
+	// Nothing on the device reads the normalised rows: the loss, the prediction and the gradient come from z and its row
+	// sums.  A forward pass launched kernel by kernel therefore leaves them out (a pass that only reads, a quarter of the time
+	// on long rows) and notes it here; they are written when something looks (CNet::fetch), from the same z, by the same
+	// kernel.  d_norm_ itself is allocated then.
+	bool norm_current_ = false;
 public:
 	CrossEntropy(Uid uid, InSize n) : CFunc(uid, n, OutSize(1)), output_(n.value()) { is_output_ = true; }
 	CrossEntropy(InSize n) : CFunc(n, OutSize(1)), output_(n.value()) { is_output_ = true; }

@@ -466,6 +466,46 @@ static void test_loss_map_and_sampling() {
 	expect("findFirstOfType", net.findFirstOfType(isCrossEntropy) == net[id[3]] && net.findFirstOfType(isLinear) == net[id[2]] &&
 			net.findFirstOfType(isFourier) == NULL);
 
+	// The normalised rows of the loss (its output values upstream): the forward pass leaves them out by default and fetch
+	// writes them when asked; with lazyLossRows(false) every forward pass writes them.  Same bits and predictions either
+	// way, before and after a backward pass and an update, and -log |row[label]|^2 is the loss the device reported.
+	{
+		CNet lazy, eager;
+		int ld[5], kd[5];
+		build(lazy, ld);
+		build(eager, kd);
+		eager.lazyLossRows(false);
+		lazy.allocateOnGpu(B);
+		eager.allocateOnGpu(B);
+		CrossEntropy *cl = (CrossEntropy *) lazy[ld[3]], *ce = (CrossEntropy *) eager[kd[3]];
+		bool same = true;
+		double worst = 0;
+		for (int pass = 0; pass < 2; ++pass) {
+			InputBatch b2(B, n);
+			for (int b = 0; b < B; ++b) b2.add(x.data() + (size_t) b * n, x.data() + (size_t) (B + b) * n, n, labels[b]);
+			lazy.gpuForward((CInput *) lazy[ld[0]], cl, b2);
+			eager.gpuForward((CInput *) eager[kd[0]], ce, b2);
+			std::vector<float> dev_loss(B);
+			eager.getLoss(ce, &b2);  // appends the loss of every row to the batch
+			for (int b = 0; b < B; ++b) dev_loss[b] = b2.loss(b);
+			if (pass == 0) {  // the first pass looks after the step, the second before it
+				lazy.gpuBackward();
+				lazy.gpuUpdateInputs(0.01f);
+				eager.gpuBackward();
+				eager.gpuUpdateInputs(0.01f);
+			}
+			for (int b = 0; b < B; ++b) {
+				lazy.fetch(cl, b);
+				eager.fetch(ce, b);
+				same = same && std::memcmp(cl->mutableOutput()->real_, ce->mutableOutput()->real_, 2 * classes * sizeof(float)) == 0 &&
+						cl->get_prediction() == ce->get_prediction();
+				worst = std::max(worst, (double) std::fabs(cl->loss(labels[b]) - dev_loss[b]) / dev_loss[b]);
+			}
+		}
+		expect("normalised rows of the loss: written on demand = written by every forward pass (bits, predictions)", same);
+		report("-log |row[label]|^2 of the fetched rows against the losses the device reported", worst, 1e-5);
+	}
+
 	// sample(): frequencies follow p_k = |z_k|^2 / S of row 0; a seed repeats the draws
 	std::vector<double> p(classes);
 	{
