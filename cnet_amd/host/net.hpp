@@ -799,6 +799,87 @@ private:
 		c->norm_current_ = true;
 	}
 
+	// ---- the forward pass of the layers that have more than one way to run ----
+	// y = x w^T, with the CGelu or the loss on its rows in the same call where the plan says so
+	void forwardLinear(CFunc *f) {
+		const int rows = f->rows_;
+		const int K = f->slots_[0].len, N = f->out_size_;
+		if (CFunc *g = f->fused_next_) {  // the CGelu on its result is applied as the product is stored
+			ck(cnet_clinear_cgelu_fwd(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), g->out_re(), g->out_im(),
+					N, rows, K, N, 0), "cnet_clinear_cgelu_fwd");
+			return;
+		}
+		if (f->loss_next_ && lossFromForward(f->loss_next_)) {  // the loss on its rows where the product is stored
+			CrossEntropy *c = (CrossEntropy *) f->loss_next_;
+			CFunc::Slot &sl = c->slots_[0];
+			float *nr = normPlanes(c);
+			ck(cnet_clinear_cross_entropy_fwd_bwd_sym(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), N, d_labels_,
+					nr, nr ? nr + (size_t) rows * N : NULL, N, c->d_s_, lossTarget(c->loss_), c->d_argmax_, sl.g(0), sl.g(1), sl.gs(2),
+					sl.gs(3), sl.len, rows, K, N), "cnet_clinear_cross_entropy_fwd_bwd_sym");
+			c->grad_from_forward_ = true;
+			c->fwd_by_producer_ = true;
+			return;
+		}
+		ck(cnet_clinear_fwd(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), N, rows, K, N, 0),
+				"cnet_clinear_fwd");
+	}
+
+	// y = x F: half the work on real samples, with the gate and activation above it in the same call where the plan says so
+	void forwardFourier(CFunc *f) {
+		const int rows = f->rows_;
+		if (realInputNow(f)) {  // real samples: half the columns by the matrix product, the rest are their conjugates
+			ck(cnet_cdft_fwd_real_input(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_),
+					"cnet_cdft_fwd_real_input");
+			return;
+		}
+		if (CFunc *h = f->fused_next_) {  // the gate and the activation above it where the transform is stored
+			CFunc *g = h->fused_next_;
+			ck(cnet_cdft_hadamard_cgelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, zre(h, 1), zim(h, 1), f->out_re(), f->out_im(), h->out_re(),
+					h->out_im(), g->out_re(), g->out_im(), f->out_size_, rows, f->out_size_), "cnet_cdft_hadamard_cgelu_fwd");
+			h->fwd_by_producer_ = true;
+			return;
+		}
+		ck(cnet_cdft_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_, 0),
+				"cnet_cdft_fwd");
+	}
+
+	void forwardHadamard(CFunc *f) {
+		const int rows = f->rows_;
+		const int n = f->out_size_;
+		if (f->fwd_by_producer_) {  // written by the transform below it in this pass
+			f->fwd_by_producer_ = false;
+			return;
+		}
+		if (CFunc *g = f->fused_next_) {  // the CGelu on its result in the same pass
+			ck(cnet_hadamard_cgelu_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), f->slots_[1].rows == rows ? n : 0, f->out_re(),
+					f->out_im(), n, g->out_re(), g->out_im(), n, rows, n), "cnet_hadamard_cgelu_fwd");
+			return;
+		}
+		ck(cnet_hadamard_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), f->slots_[1].rows == rows ? n : 0, f->out_re(),
+				f->out_im(), n, rows, n), "cnet_hadamard_fwd");
+	}
+
+	void forwardCrossEntropy(CFunc *f) {
+		const int rows = f->rows_;
+		CrossEntropy *c = (CrossEntropy *) f;
+		const int n = f->input().length_;
+		if (f->fwd_by_producer_) {  // written by the Linear below it in this pass
+			f->fwd_by_producer_ = false;
+			return;
+		}
+		float *nr = normPlanes(c);
+		if (lossFromForward(f)) {
+			CFunc::Slot &sl = f->slots_[0];
+			ck(cnet_cross_entropy_fwd_bwd_sym(zre(f, 0), zim(f, 0), n, d_labels_, nr, nr ? nr + (size_t) rows * n : NULL, n, c->d_s_,
+					lossTarget(c->loss_), c->d_argmax_, sl.g(0), sl.g(1), sl.gs(2), sl.gs(3), sl.len, rows, n), "cnet_cross_entropy_fwd_bwd_sym");
+			c->grad_from_forward_ = true;
+			return;
+		}
+		ck(cnet_cross_entropy_fwd(zre(f, 0), zim(f, 0), n, d_labels_, nr, nr ? nr + (size_t) rows * n : NULL, n, c->d_s_,
+				lossTarget(c->loss_), c->d_argmax_, rows, n), "cnet_cross_entropy_fwd");
+		c->grad_from_forward_ = false;
+	}
+
 	void nodeForward(CFunc *f) {
 		const int rows = f->rows_;
 		switch (f->typeId()) {
@@ -810,44 +891,8 @@ private:
 					f->out_im(), f->out_size_, rows, e->no_out_tokens_), "cnet_embedding_fwd");
 			break;
 		}
-		case isLinear: {
-			const int K = f->slots_[0].len, N = f->out_size_;
-			if (CFunc *g = f->fused_next_) {  // the CGelu on its result is applied as the product is stored
-				ck(cnet_clinear_cgelu_fwd(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), g->out_re(), g->out_im(),
-						N, rows, K, N, 0), "cnet_clinear_cgelu_fwd");
-				break;
-			}
-			if (f->loss_next_ && lossFromForward(f->loss_next_)) {  // the loss on its rows where the product is stored
-				CrossEntropy *c = (CrossEntropy *) f->loss_next_;
-				CFunc::Slot &sl = c->slots_[0];
-				float *nr = normPlanes(c);
-				ck(cnet_clinear_cross_entropy_fwd_bwd_sym(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), N, d_labels_,
-						nr, nr ? nr + (size_t) rows * N : NULL, N, c->d_s_, lossTarget(c->loss_), c->d_argmax_, sl.g(0), sl.g(1), sl.gs(2),
-						sl.gs(3), sl.len, rows, K, N), "cnet_clinear_cross_entropy_fwd_bwd_sym");
-				c->grad_from_forward_ = true;
-				c->fwd_by_producer_ = true;
-				break;
-			}
-			ck(cnet_clinear_fwd(zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, f->out_re(), f->out_im(), N, rows, K, N, 0),
-					"cnet_clinear_fwd");
-			break;
-		}
-		case isFourier:
-			if (realInputNow(f)) {  // real samples: half the columns by the matrix product, the rest are their conjugates
-				ck(cnet_cdft_fwd_real_input(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_),
-						"cnet_cdft_fwd_real_input");
-				break;
-			}
-			if (CFunc *h = f->fused_next_) {  // the gate and the activation above it where the transform is stored
-				CFunc *g = h->fused_next_;
-				ck(cnet_cdft_hadamard_cgelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, zre(h, 1), zim(h, 1), f->out_re(), f->out_im(), h->out_re(),
-						h->out_im(), g->out_re(), g->out_im(), f->out_size_, rows, f->out_size_), "cnet_cdft_hadamard_cgelu_fwd");
-				h->fwd_by_producer_ = true;
-				break;
-			}
-			ck(cnet_cdft_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_, 0),
-					"cnet_cdft_fwd");
-			break;
+		case isLinear: forwardLinear(f); break;
+		case isFourier: forwardFourier(f); break;
 		case isTrianFourier:
 			ck(cnet_ctriang_dft_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_, 0),
 					"cnet_ctriang_dft_fwd");
@@ -863,21 +908,7 @@ private:
 			ck(cnet_crelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_),
 					"cnet_crelu_fwd");
 			break;
-		case isHadamard: {
-			const int n = f->out_size_;
-			if (f->fwd_by_producer_) {  // written by the transform below it in this pass
-				f->fwd_by_producer_ = false;
-				break;
-			}
-			if (CFunc *g = f->fused_next_) {  // the CGelu on its result in the same pass
-				ck(cnet_hadamard_cgelu_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), f->slots_[1].rows == rows ? n : 0, f->out_re(),
-						f->out_im(), n, g->out_re(), g->out_im(), n, rows, n), "cnet_hadamard_cgelu_fwd");
-				break;
-			}
-			ck(cnet_hadamard_fwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), f->slots_[1].rows == rows ? n : 0, f->out_re(),
-					f->out_im(), n, rows, n), "cnet_hadamard_fwd");
-			break;
-		}
+		case isHadamard: forwardHadamard(f); break;
 		case isGelu:
 			if (f->fused_prev_) break;  // written by the Hadamard or the Linear below it
 			ck(cnet_cgelu_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, rows, f->out_size_),
@@ -894,26 +925,7 @@ private:
 			ck(cnet_l2norm_fwd(zre(f, 0), zim(f, 0), f->out_size_, f->out_re(), f->out_im(), f->out_size_, ((SoftMax *) f)->d_s_, rows,
 					f->out_size_), "cnet_l2norm_fwd");
 			break;
-		case isCrossEntropy: {
-			CrossEntropy *c = (CrossEntropy *) f;
-			const int n = f->input().length_;
-			if (f->fwd_by_producer_) {  // written by the Linear below it in this pass
-				f->fwd_by_producer_ = false;
-				break;
-			}
-			float *nr = normPlanes(c);
-			if (lossFromForward(f)) {
-				CFunc::Slot &sl = f->slots_[0];
-				ck(cnet_cross_entropy_fwd_bwd_sym(zre(f, 0), zim(f, 0), n, d_labels_, nr, nr ? nr + (size_t) rows * n : NULL, n, c->d_s_,
-						lossTarget(c->loss_), c->d_argmax_, sl.g(0), sl.g(1), sl.gs(2), sl.gs(3), sl.len, rows, n), "cnet_cross_entropy_fwd_bwd_sym");
-				c->grad_from_forward_ = true;
-				break;
-			}
-			ck(cnet_cross_entropy_fwd(zre(f, 0), zim(f, 0), n, d_labels_, nr, nr ? nr + (size_t) rows * n : NULL, n, c->d_s_,
-					lossTarget(c->loss_), c->d_argmax_, rows, n), "cnet_cross_entropy_fwd");
-			c->grad_from_forward_ = false;
-			break;
-		}
+		case isCrossEntropy: forwardCrossEntropy(f); break;
 		case isL2Out:
 			ck(cnet_l2out_fwd(zre(f, 0), zim(f, 0), f->input().length_, lossTarget(((L2Out *) f)->loss_), rows, f->input().length_),
 					"cnet_l2out_fwd");
@@ -922,15 +934,189 @@ private:
 		}
 	}
 
-	// Each consumer's contribution is added in turn (the per-consumer loops of the upstream layers); the first one
-	// overwrites, so the planes never need zeroing between steps.  Nodes without consumers get zeros.
-	void nodeBackward(CFunc *f, bool with_labels) {
+	// ---- the backward pass of one layer for the gradient u of one consumer (acc: added to what an earlier consumer left) ----
+	// dx = g w and dw = g^T x of a Linear (upstream gpu_linear_backward), with what the plan lets ride on the same call
+	void backwardLinear(CFunc *f, CFunc::Slot &u, const int acc) {
 		const int rows = f->rows_;
-		const int t = f->typeId();
-		if (t == isCrossEntropy) {
+		CFunc::Slot &a = f->slots_[0];
+		CFunc::Slot &w = f->slots_[1];
+		const int K = a.len, N = f->out_size_;
+		// (the input gradient of a lazy data input waits: see CFunc::lazy_bwd_)
+		const bool to_data = a.producer->wants_grad_ && !f->lazy_skip_now_, to_weight = w.producer->wants_grad_;
+		if (conjugate_gradients_ && to_data && to_weight && f->no_outputs() == 1 && gateBelow(f)) {
+			// the operand is the CGelu of a Hadamard gate with a shared row: the gate's backward pass in the same call (one
+			// launch at small batches: the workgroup that forms 16 columns of dx goes on to the gate)
+			CFunc *g = a.producer, *h = g->slots_[0].producer;
+			CFunc::Slot &hs = g->slots_[0], &hu = h->slots_[0], &hv = h->slots_[1];
+			ck(cnet_clinear_hadamard_cgelu_bwd_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1),
+					a.gs(2), a.gs(3), K, acc, w.g(0), w.g(1), w.gs(2), w.gs(3), K, acc, zre(h, 0), zim(h, 0), K, zre(h, 1), zim(h, 1), hs.g(0),
+					hs.g(1), hs.gs(2), hs.gs(3), K, hu.g(0), hu.g(1), hu.gs(2), hu.gs(3), K, hv.g(0), hv.g(1), hv.gs(2), hv.gs(3), 0, rows, K, N),
+					"cnet_clinear_hadamard_cgelu_bwd_sym");
+			h->bwd_by_consumer_now_ = true;
+			return;
+		}
+		if (conjugate_gradients_ && to_data && to_weight) {  // both gradients in one call (one launch when both products are small)
+			ck(cnet_clinear_bwd_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.gs(2),
+					a.gs(3), K, acc, w.g(0), w.g(1), w.gs(2), w.gs(3), K, acc, rows, K, N), "cnet_clinear_bwd_sym");
+			return;
+		}
+		if (conjugate_gradients_) {  // dz* = conj(dz): one product each, written to both pairs of planes
+			if (to_data)
+				ck(cnet_clinear_bwd_input_sym(u.g(0), u.g(1), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.gs(2), a.gs(3), K, rows, K,
+						N, acc), "cnet_clinear_bwd_input_sym");
+			if (to_weight)
+				ck(cnet_clinear_bwd_weight_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.gs(2), w.gs(3), K, rows, K,
+						N, acc), "cnet_clinear_bwd_weight_sym");
+			return;
+		}
+		if (to_data)
+			ck(cnet_clinear_bwd_input(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K,
+					rows, K, N, acc), "cnet_clinear_bwd_input");
+		if (to_weight)
+			ck(cnet_clinear_bwd_weight(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K,
+					rows, K, N, acc), "cnet_clinear_bwd_weight");
+	}
+
+	// the backward pass of the transform is the transform of the gradients
+	void backwardFourier(CFunc *f, CFunc::Slot &u, const int acc) {
+		const int rows = f->rows_;
+		CFunc::Slot &a = f->slots_[0];
+		if (conjugate_gradients_)
+			ck(cnet_cdft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len, acc), "cnet_cdft_bwd_sym");
+		else
+			ck(cnet_cdft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
+					"cnet_cdft_bwd");
+	}
+
+	void backwardTrianFourier(CFunc *f, CFunc::Slot &u, const int acc) {
+		const int rows = f->rows_;
+		CFunc::Slot &a = f->slots_[0];
+		if (conjugate_gradients_)
+			ck(cnet_ctriang_dft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len, acc),
+					"cnet_ctriang_dft_bwd_sym");
+		else
+			ck(cnet_ctriang_dft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
+					"cnet_ctriang_dft_bwd");
+	}
+
+	void backwardSeqFourier(CFunc *f, CFunc::Slot &u, const int acc) {
+		const int rows = f->rows_;
+		CFunc::Slot &a = f->slots_[0];
+		// dX_g.dz = F G_g.dz and dX_g.dz* = conj(F) G_g.dz* (F is symmetric).  Of a conjugate pair only the dz planes of G
+		// hold values: dz* = conj(F) conj(G.dz), formed where something reads it on the device.
+		SeqFourierTrans *q = (SeqFourierTrans *) f;
+		const int S = q->seq_, n = f->out_size_;
+		ck(cnet_cgemm_batched(0, 1, 0, 0, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, u.g(0), u.g(1), u.len, (int64_t) S * u.len, a.g(0), a.g(1),
+				a.len, (int64_t) S * a.len, rows / S, acc), "cnet_cgemm_batched");
+		if (conjugate_gradients_) {
+			if (a.gs(2))
+				ck(cnet_cgemm_batched(0, 1, 1, 1, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, u.g(0), u.g(1), u.len, (int64_t) S * u.len,
+						a.g(2), a.g(3), a.len, (int64_t) S * a.len, rows / S, acc), "cnet_cgemm_batched");
+		} else {
+			ck(cnet_cgemm_batched(0, 1, 1, 0, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, u.g(2), u.g(3), u.len, (int64_t) S * u.len, a.g(2),
+					a.g(3), a.len, (int64_t) S * a.len, rows / S, acc), "cnet_cgemm_batched");
+		}
+	}
+
+	void backwardCrelu(CFunc *f, CFunc::Slot &u, const int acc) {
+		const int rows = f->rows_;
+		CFunc::Slot &a = f->slots_[0];
+		if (conjugate_gradients_) {
+			ck(cnet_crelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,
+					acc), "cnet_crelu_bwd_sym");
+			return;
+		}
+		ck(cnet_crelu_bwd(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len,
+				rows, a.len, acc), "cnet_crelu_bwd");
+	}
+
+	// du = G v, dv = G u; with the CGelu above it in the same pass where the plan says so
+	void backwardHadamard(CFunc *f, CFunc::Slot &u, const int acc) {
+		const int rows = f->rows_;
+		CFunc::Slot &a = f->slots_[0];
+		CFunc::Slot &v = f->slots_[1];
+		const int n = f->out_size_;
+		if (f->bwd_by_consumer_now_) {  // done by the Linear above its CGelu in this pass
+			f->bwd_by_consumer_now_ = false;
+			return;
+		}
+		if (conjugate_gradients_ && f->fused_next_) {  // the backward pass of the CGelu above it in the same pass
+			CFunc *g = f->fused_next_;
+			CFunc::Slot &ug = upstream(g, 0), &h = g->slots_[0];
+			ck(cnet_hadamard_cgelu_bwd_sym(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, ug.g(0), ug.g(1), ug.len,
+					h.g(0), h.g(1), h.gs(2), h.gs(3), n, a.g(0), a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows, n,
+					acc), "cnet_hadamard_cgelu_bwd_sym");
+			return;
+		}
+		if (conjugate_gradients_) {
+			ck(cnet_hadamard_bwd_sym(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, u.g(0), u.g(1), u.len, a.g(0),
+					a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows, n, acc), "cnet_hadamard_bwd_sym");
+			return;
+		}
+		ck(cnet_hadamard_bwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, u.g(0), u.g(1), u.g(2), u.g(3),
+				u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3), n, rows, n, acc), "cnet_hadamard_bwd");
+	}
+
+	void backwardGelu(CFunc *f, CFunc::Slot &u, const int acc) {
+		const int rows = f->rows_;
+		CFunc::Slot &a = f->slots_[0];
+		if (conjugate_gradients_ && (f->fused_prev_ == 2 || f->bwd_by_consumer_)) return;  // done by the Hadamard below it or the Residual above it
+		if (conjugate_gradients_) {
+			ck(cnet_cgelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,
+					acc), "cnet_cgelu_bwd_sym");
+			return;
+		}
+		ck(cnet_cgelu_bwd(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len,
+				rows, a.len, acc), "cnet_cgelu_bwd");
+	}
+
+	// the incoming gradient goes to both operands
+	void backwardResidual(CFunc *f, CFunc::Slot &u, const int acc) {
+		const int rows = f->rows_;
+		CFunc::Slot &a = f->slots_[0];
+		CFunc::Slot &v = f->slots_[1];
+		const int n = f->out_size_;
+		if (a.rows == rows && v.rows == rows && conjugate_gradients_) {
+			ck(cnet_residual_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows,
+					n, acc), "cnet_residual_bwd_sym");
+			return;
+		}
+		if (a.rows == rows && v.rows == rows) {
+			ck(cnet_residual_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3),
+					n, rows, n, acc), "cnet_residual_bwd");
+			return;
+		}
+		// a parameter operand receives the sum over the batch rows, a batched one a copy
+		for (CFunc::Slot *s : {&a, &v})
+			for (int p = 0; p < 4; ++p) {
+				if (s->rows == 1 && rows > 1)
+					ck(cnet_batch_sum(u.g(p), u.len, s->g(p), rows, n, acc), "cnet_batch_sum");
+				else if (acc)
+					ck(cnet_add2d(u.g(p), u.len, s->g(p), n, s->rows, n), "cnet_add2d");
+				else
+					ck(cnet_copy2d(u.g(p), u.len, s->g(p), n, s->rows, n), "cnet_copy2d");
+			}
+	}
+
+	void backwardSoftMax(CFunc *f, CFunc::Slot &u, const int acc) {
+		const int rows = f->rows_;
+		CFunc::Slot &a = f->slots_[0];
+		if (conjugate_gradients_) {
+			ck(cnet_l2norm_bwd_sym(zre(f, 0), zim(f, 0), a.len, ((SoftMax *) f)->d_s_, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2),
+					a.gs(3), a.len, rows, a.len, acc), "cnet_l2norm_bwd_sym");
+			return;
+		}
+		ck(cnet_l2norm_bwd(zre(f, 0), zim(f, 0), a.len, ((SoftMax *) f)->d_s_, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1),
+				a.g(2), a.g(3), a.len, rows, a.len, acc), "cnet_l2norm_bwd");
+	}
+
+	// the gradient of a loss at its operand (upstream CrossEntropy::backward / L2Out::backward)
+	void backwardLoss(CFunc *f, bool with_labels) {
+		const int rows = f->rows_;
+		CFunc::Slot &s = f->slots_[0];
+		if (f->typeId() == isCrossEntropy) {
 			if (!with_labels) return;  // upstream: CrossEntropy::backward() without a label does nothing
 			CrossEntropy *c = (CrossEntropy *) f;
-			CFunc::Slot &s = f->slots_[0];
 			if (conjugate_gradients_ && c->grad_from_forward_) return;  // written by the forward pass, with these labels
 			if (conjugate_gradients_)
 				ck(cnet_cross_entropy_bwd_sym(zre(f, 0), zim(f, 0), s.len, c->d_s_, d_labels_, s.g(0), s.g(1), s.gs(2), s.gs(3), s.len, rows,
@@ -940,41 +1126,71 @@ private:
 						"cnet_cross_entropy_bwd");
 			return;
 		}
-		if (t == isL2Out) {
-			CFunc::Slot &s = f->slots_[0];
-			if (conjugate_gradients_)
-				ck(cnet_l2out_bwd_sym(zre(f, 0), zim(f, 0), s.len, s.g(0), s.g(1), s.gs(2), s.gs(3), s.len, rows, s.len, 0), "cnet_l2out_bwd_sym");
-			else
-				ck(cnet_l2out_bwd(zre(f, 0), zim(f, 0), s.len, s.g(0), s.g(1), s.g(2), s.g(3), s.len, rows, s.len, 0), "cnet_l2out_bwd");
-			return;
+		if (conjugate_gradients_)
+			ck(cnet_l2out_bwd_sym(zre(f, 0), zim(f, 0), s.len, s.g(0), s.g(1), s.gs(2), s.gs(3), s.len, rows, s.len, 0), "cnet_l2out_bwd_sym");
+		else
+			ck(cnet_l2out_bwd(zre(f, 0), zim(f, 0), s.len, s.g(0), s.g(1), s.g(2), s.g(3), s.len, rows, s.len, 0), "cnet_l2out_bwd");
+	}
+
+	// An input function gathers the dz* of its consumers (impl/cinput.h:54-65), and keeps adding until the next update.
+	// Both dz* planes of a consumer's slot are adjacent and dense, as they are in the node's own block: one array per
+	// consumer.  Nothing in the backward pass reads what an input function gathers, so the gathers of all of them
+	// wait for the end of the pass and go out as one launch (flushGathers).
+	void backwardInput(CFunc *f) {
+		CFunc::Slot &own = f->slots_[0];
+		if (f->defer_now_) return;  // the update will read the consumer's planes (see pending_)
+		for (int c = 0; c < f->no_outputs(); ++c) {
+			CFunc::Slot &u = upstream(f, c);
+			if (c) flushGathers();  // one launch must not hold two additions into the same planes
+			gather_src_.push_back(u.g(2));
+			gather_dst_.push_back(own.g(2));
+			gather_len_.push_back(2 * (int64_t) own.rows * own.len);
 		}
+	}
+
+	void backwardEmbedding(CFunc *f) {
+		CEmbedding *e = (CEmbedding *) f;
+		CFunc::Slot &own = f->slots_[0];
+		for (int c = 0; c < f->no_outputs(); ++c) {
+			CFunc::Slot &u = upstream(f, c);
+			ck(cnet_embedding_bwd(e->d_tokens_, u.g(2), u.g(3), u.len, own.g(2), own.g(3), e->embedding_dim_, e->no_embeddings_, f->rows_,
+					e->no_out_tokens_, 1), "cnet_embedding_bwd");
+		}
+	}
+
+	// a Residual that takes all its incoming gradients in one kernel: true when it did
+	bool backwardResidualInOnePass(CFunc *f) {
+		const int rows = f->rows_, n = f->out_size_;
+		if (!conjugate_gradients_) return false;
+		if (f->fused_gelu_slot_ >= 0) {  // one operand is a CGelu that feeds nothing else: its backward pass in the same kernel
+			const int k = f->fused_gelu_slot_;
+			CFunc *g = f->slots_[k].producer;
+			CFunc::Slot &u0 = upstream(f, 0), &a = f->slots_[1 - k], &h = g->slots_[0];
+			CFunc::Slot *u1 = f->no_outputs() == 2 ? &upstream(f, 1) : NULL;
+			ck(cnet_residual_cgelu_bwd_sym(u0.g(0), u0.g(1), u0.len, u1 ? u1->g(0) : NULL, u1 ? u1->g(1) : NULL, u1 ? u1->len : 0, zre(g, 0),
+					zim(g, 0), n, a.g(0), a.g(1), a.gs(2), a.gs(3), n, NULL, NULL, NULL, NULL, 0, h.g(0), h.g(1), h.gs(2), h.gs(3), n, rows, n),
+					"cnet_residual_cgelu_bwd_sym");
+			return true;
+		}
+		if (f->no_outputs() == 2 && f->slots_[0].rows == rows && f->slots_[1].rows == rows) {
+			// a Residual feeding two consumers (the usual skip connection): both incoming gradients in one pass
+			CFunc::Slot &u0 = upstream(f, 0), &u1 = upstream(f, 1), &a = f->slots_[0], &v = f->slots_[1];
+			ck(cnet_residual_bwd_sym2(u0.g(0), u0.g(1), u0.len, u1.g(0), u1.g(1), u1.len, a.g(0), a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1),
+					v.gs(2), v.gs(3), n, rows, n, 0), "cnet_residual_bwd_sym2");
+			return true;
+		}
+		return false;
+	}
+
+	// Each consumer's contribution is added in turn (the per-consumer loops of the upstream layers); the first one
+	// overwrites, so the planes never need zeroing between steps.  Nodes without consumers get zeros.
+	void nodeBackward(CFunc *f, bool with_labels) {
+		const int t = f->typeId();
+		if (t == isCrossEntropy || t == isL2Out) return backwardLoss(f, with_labels);
 		if ((t == isInput || t == isEmbedding) && !f->trainable_) return;  // nothing steps it: nothing to gather
 		if (f->lazy_now_ || (f->lazy_skip_now_ && t != isLinear)) return;  // left out for now (see CFunc::lazy_bwd_)
-		if (t == isInput) {  // impl/cinput.h:54-65: gathers dzs only, and keeps adding until the next update
-			// Both dz* planes of a consumer's slot are adjacent and dense, as they are in the node's own block: one array per
-			// consumer.  Nothing in the backward pass reads what an input function gathers, so the gathers of all of them
-			// wait for the end of the pass and go out as one launch (flushGathers).
-			CFunc::Slot &own = f->slots_[0];
-			if (f->defer_now_) return;  // the update will read the consumer's planes (see pending_)
-			for (int c = 0; c < f->no_outputs(); ++c) {
-				CFunc::Slot &u = upstream(f, c);
-				if (c) flushGathers();  // one launch must not hold two additions into the same planes
-				gather_src_.push_back(u.g(2));
-				gather_dst_.push_back(own.g(2));
-				gather_len_.push_back(2 * (int64_t) own.rows * own.len);
-			}
-			return;
-		}
-		if (t == isEmbedding) {
-			CEmbedding *e = (CEmbedding *) f;
-			CFunc::Slot &own = f->slots_[0];
-			for (int c = 0; c < f->no_outputs(); ++c) {
-				CFunc::Slot &u = upstream(f, c);
-				ck(cnet_embedding_bwd(e->d_tokens_, u.g(2), u.g(3), u.len, own.g(2), own.g(3), e->embedding_dim_, e->no_embeddings_,
-						rows, e->no_out_tokens_, 1), "cnet_embedding_bwd");
-			}
-			return;
-		}
+		if (t == isInput) return backwardInput(f);
+		if (t == isEmbedding) return backwardEmbedding(f);
 		if (f->no_outputs() == 0) {
 			for (auto &s : f->slots_) ck(cnet_memset_zero(s.grad, 4 * (size_t) s.rows * s.len * sizeof(float)), "zero");
 			return;
@@ -982,179 +1198,20 @@ private:
 		// Gradients flow only towards input functions that are stepped: a layer none of whose operands leads to one is
 		// skipped (all input functions are trainable unless CNet::setInputTrainable said otherwise, as upstream has it).
 		if (!f->wants_grad_) return;
-		if (t == isResidual && conjugate_gradients_ && f->fused_gelu_slot_ >= 0) {
-			// one operand is a CGelu that feeds nothing else: its backward pass in the same kernel
-			const int k = f->fused_gelu_slot_;
-			CFunc *g = f->slots_[k].producer;
-			CFunc::Slot &u0 = upstream(f, 0), &a = f->slots_[1 - k], &h = g->slots_[0];
-			CFunc::Slot *u1 = f->no_outputs() == 2 ? &upstream(f, 1) : NULL;
-			const int n = f->out_size_;
-			ck(cnet_residual_cgelu_bwd_sym(u0.g(0), u0.g(1), u0.len, u1 ? u1->g(0) : NULL, u1 ? u1->g(1) : NULL, u1 ? u1->len : 0, zre(g, 0),
-					zim(g, 0), n, a.g(0), a.g(1), a.gs(2), a.gs(3), n, NULL, NULL, NULL, NULL, 0, h.g(0), h.g(1), h.gs(2), h.gs(3), n, rows, n),
-					"cnet_residual_cgelu_bwd_sym");
-			return;
-		}
-		if (t == isResidual && conjugate_gradients_ && f->no_outputs() == 2 && f->slots_[0].rows == rows && f->slots_[1].rows == rows) {
-			// a Residual feeding two consumers (the usual skip connection): both incoming gradients in one pass
-			CFunc::Slot &u0 = upstream(f, 0), &u1 = upstream(f, 1), &a = f->slots_[0], &v = f->slots_[1];
-			const int n = f->out_size_;
-			ck(cnet_residual_bwd_sym2(u0.g(0), u0.g(1), u0.len, u1.g(0), u1.g(1), u1.len, a.g(0), a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1),
-					v.gs(2), v.gs(3), n, rows, n, 0), "cnet_residual_bwd_sym2");
-			return;
-		}
+		if (t == isResidual && backwardResidualInOnePass(f)) return;
 		for (int c = 0; c < f->no_outputs(); ++c) {
-			CFunc::Slot &u = upstream(f, c);
+			CFunc::Slot &u = upstream(f, c);  // the gradient that consumer c left for this node
 			const int acc = c > 0;
-			CFunc::Slot &a = f->slots_[0];
 			switch (t) {
-			case isLinear: {
-				CFunc::Slot &w = f->slots_[1];
-				const int K = a.len, N = f->out_size_;
-				// (the input gradient of a lazy data input waits: see CFunc::lazy_bwd_)
-				const bool to_data = a.producer->wants_grad_ && !f->lazy_skip_now_, to_weight = w.producer->wants_grad_;
-				if (conjugate_gradients_ && to_data && to_weight && f->no_outputs() == 1 && gateBelow(f)) {
-					// the operand is the CGelu of a Hadamard gate with a shared row: the gate's backward pass in the same call (one
-					// launch at small batches: the workgroup that forms 16 columns of dx goes on to the gate)
-					CFunc *g = a.producer, *h = g->slots_[0].producer;
-					CFunc::Slot &hs = g->slots_[0], &hu = h->slots_[0], &hv = h->slots_[1];
-					ck(cnet_clinear_hadamard_cgelu_bwd_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1),
-							a.gs(2), a.gs(3), K, acc, w.g(0), w.g(1), w.gs(2), w.gs(3), K, acc, zre(h, 0), zim(h, 0), K, zre(h, 1), zim(h, 1), hs.g(0),
-							hs.g(1), hs.gs(2), hs.gs(3), K, hu.g(0), hu.g(1), hu.gs(2), hu.gs(3), K, hv.g(0), hv.g(1), hv.gs(2), hv.gs(3), 0, rows, K, N),
-							"cnet_clinear_hadamard_cgelu_bwd_sym");
-					h->bwd_by_consumer_now_ = true;
-					break;
-				}
-				if (conjugate_gradients_ && to_data && to_weight) {  // both gradients in one call (one launch when both products are small)
-					ck(cnet_clinear_bwd_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.gs(2),
-							a.gs(3), K, acc, w.g(0), w.g(1), w.gs(2), w.gs(3), K, acc, rows, K, N), "cnet_clinear_bwd_sym");
-					break;
-				}
-				if (conjugate_gradients_) {  // dz* = conj(dz): one product each, written to both pairs of planes
-					if (to_data)
-						ck(cnet_clinear_bwd_input_sym(u.g(0), u.g(1), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.gs(2), a.gs(3), K, rows, K,
-								N, acc), "cnet_clinear_bwd_input_sym");
-					if (to_weight)
-						ck(cnet_clinear_bwd_weight_sym(u.g(0), u.g(1), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.gs(2), w.gs(3), K, rows, K,
-								N, acc), "cnet_clinear_bwd_weight_sym");
-					break;
-				}
-				if (to_data)
-					ck(cnet_clinear_bwd_input(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 1), zim(f, 1), K, a.g(0), a.g(1), a.g(2), a.g(3), K,
-							rows, K, N, acc), "cnet_clinear_bwd_input");
-				if (to_weight)
-					ck(cnet_clinear_bwd_weight(u.g(0), u.g(1), u.g(2), u.g(3), u.len, zre(f, 0), zim(f, 0), K, w.g(0), w.g(1), w.g(2), w.g(3), K,
-							rows, K, N, acc), "cnet_clinear_bwd_weight");
-				break;
-			}
-			case isFourier:
-				if (conjugate_gradients_)
-					ck(cnet_cdft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len, acc), "cnet_cdft_bwd_sym");
-				else
-					ck(cnet_cdft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
-							"cnet_cdft_bwd");
-				break;
-			case isTrianFourier:
-				if (conjugate_gradients_)
-					ck(cnet_ctriang_dft_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len, acc),
-							"cnet_ctriang_dft_bwd_sym");
-				else
-					ck(cnet_ctriang_dft_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len, rows, a.len, acc),
-							"cnet_ctriang_dft_bwd");
-				break;
-			case isSeqFourier: {
-				// dX_g.dz = F G_g.dz and dX_g.dz* = conj(F) G_g.dz* (F is symmetric).  Of a conjugate pair only the dz planes of G
-				// hold values: dz* = conj(F) conj(G.dz), formed where something reads it on the device.
-				SeqFourierTrans *q = (SeqFourierTrans *) f;
-				const int S = q->seq_, n = f->out_size_;
-				ck(cnet_cgemm_batched(0, 1, 0, 0, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, u.g(0), u.g(1), u.len, (int64_t) S * u.len, a.g(0), a.g(1),
-						a.len, (int64_t) S * a.len, rows / S, acc), "cnet_cgemm_batched");
-				if (conjugate_gradients_) {
-					if (a.gs(2))
-						ck(cnet_cgemm_batched(0, 1, 1, 1, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, u.g(0), u.g(1), u.len, (int64_t) S * u.len,
-								a.g(2), a.g(3), a.len, (int64_t) S * a.len, rows / S, acc), "cnet_cgemm_batched");
-				} else {
-					ck(cnet_cgemm_batched(0, 1, 1, 0, S, n, S, q->f_re_, q->f_im_, q->f_ld_, 0, u.g(2), u.g(3), u.len, (int64_t) S * u.len, a.g(2),
-							a.g(3), a.len, (int64_t) S * a.len, rows / S, acc), "cnet_cgemm_batched");
-				}
-				break;
-			}
-			case isCrelu:
-				if (conjugate_gradients_) {
-					ck(cnet_crelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,
-							acc), "cnet_crelu_bwd_sym");
-					break;
-				}
-				ck(cnet_crelu_bwd(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len,
-						rows, a.len, acc), "cnet_crelu_bwd");
-				break;
-			case isHadamard: {
-				CFunc::Slot &v = f->slots_[1];
-				const int n = f->out_size_;
-				if (f->bwd_by_consumer_now_) {  // done by the Linear above its CGelu in this pass
-					f->bwd_by_consumer_now_ = false;
-					break;
-				}
-				if (conjugate_gradients_ && f->fused_next_) {  // the backward pass of the CGelu above it in the same pass
-					CFunc *g = f->fused_next_;
-					CFunc::Slot &ug = upstream(g, 0), &h = g->slots_[0];
-					ck(cnet_hadamard_cgelu_bwd_sym(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, ug.g(0), ug.g(1), ug.len,
-							h.g(0), h.g(1), h.gs(2), h.gs(3), n, a.g(0), a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows, n,
-							acc), "cnet_hadamard_cgelu_bwd_sym");
-					break;
-				}
-				if (conjugate_gradients_) {
-					ck(cnet_hadamard_bwd_sym(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, u.g(0), u.g(1), u.len, a.g(0),
-							a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows, n, acc), "cnet_hadamard_bwd_sym");
-					break;
-				}
-				ck(cnet_hadamard_bwd(zre(f, 0), zim(f, 0), n, zre(f, 1), zim(f, 1), v.rows == rows ? n : 0, u.g(0), u.g(1), u.g(2), u.g(3),
-						u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3), n, rows, n, acc), "cnet_hadamard_bwd");
-				break;
-			}
-			case isGelu:
-				if (conjugate_gradients_ && (f->fused_prev_ == 2 || f->bwd_by_consumer_)) break;  // done by the Hadamard below it or the Residual above it
-				if (conjugate_gradients_) {
-					ck(cnet_cgelu_bwd_sym(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), a.len, rows, a.len,
-							acc), "cnet_cgelu_bwd_sym");
-					break;
-				}
-				ck(cnet_cgelu_bwd(zre(f, 0), zim(f, 0), a.len, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), a.len,
-						rows, a.len, acc), "cnet_cgelu_bwd");
-				break;
-			case isResidual: {
-				CFunc::Slot &v = f->slots_[1];
-				const int n = f->out_size_;
-				if (a.rows == rows && v.rows == rows && conjugate_gradients_) {
-					ck(cnet_residual_bwd_sym(u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2), a.gs(3), n, v.g(0), v.g(1), v.gs(2), v.gs(3), n, rows,
-							n, acc), "cnet_residual_bwd_sym");
-					break;
-				}
-				if (a.rows == rows && v.rows == rows) {
-					ck(cnet_residual_bwd(u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1), a.g(2), a.g(3), n, v.g(0), v.g(1), v.g(2), v.g(3),
-							n, rows, n, acc), "cnet_residual_bwd");
-					break;
-				}
-				// a parameter operand receives the sum over the batch rows, a batched one a copy
-				for (CFunc::Slot *s : {&a, &v})
-					for (int p = 0; p < 4; ++p) {
-						if (s->rows == 1 && rows > 1)
-							ck(cnet_batch_sum(u.g(p), u.len, s->g(p), rows, n, acc), "cnet_batch_sum");
-						else if (acc)
-							ck(cnet_add2d(u.g(p), u.len, s->g(p), n, s->rows, n), "cnet_add2d");
-						else
-							ck(cnet_copy2d(u.g(p), u.len, s->g(p), n, s->rows, n), "cnet_copy2d");
-					}
-				break;
-			}
-			case isSoftMax:
-				if (conjugate_gradients_) {
-					ck(cnet_l2norm_bwd_sym(zre(f, 0), zim(f, 0), a.len, ((SoftMax *) f)->d_s_, u.g(0), u.g(1), u.len, a.g(0), a.g(1), a.gs(2),
-							a.gs(3), a.len, rows, a.len, acc), "cnet_l2norm_bwd_sym");
-					break;
-				}
-				ck(cnet_l2norm_bwd(zre(f, 0), zim(f, 0), a.len, ((SoftMax *) f)->d_s_, u.g(0), u.g(1), u.g(2), u.g(3), u.len, a.g(0), a.g(1),
-						a.g(2), a.g(3), a.len, rows, a.len, acc), "cnet_l2norm_bwd");
-				break;
+			case isLinear: backwardLinear(f, u, acc); break;
+			case isFourier: backwardFourier(f, u, acc); break;
+			case isTrianFourier: backwardTrianFourier(f, u, acc); break;
+			case isSeqFourier: backwardSeqFourier(f, u, acc); break;
+			case isCrelu: backwardCrelu(f, u, acc); break;
+			case isHadamard: backwardHadamard(f, u, acc); break;
+			case isGelu: backwardGelu(f, u, acc); break;
+			case isResidual: backwardResidual(f, u, acc); break;
+			case isSoftMax: backwardSoftMax(f, u, acc); break;
 			default: throw std::logic_error(f->getName() + ": no device implementation");
 			}
 		}
