@@ -419,13 +419,24 @@ int cnet_mark_compute(int marker) {
 	return CNET_OK;
 }
 
+// `stream` waits for the point that `ev` stands for.  A point that has been reached already needs no wait, and asking
+// costs the host a tenth of what queueing a wait across streams does (0.5 against 5-8 us); in a training loop that is
+// the usual case for both directions (the buffer about to be refilled was retired two steps ago, the batch about to be
+// used landed a step ago).
+static int wait_unless_reached(hipStream_t stream, hipEvent_t ev) {
+	const hipError_t q = hipEventQuery(ev);
+	if (q == hipSuccess) return CNET_OK;
+	(void) hipGetLastError();  // "not ready" is an answer, not a failure to carry into the next call
+	CNET_HIP(hipStreamWaitEvent(stream, ev, 0));
+	return CNET_OK;
+}
+
 int cnet_upload_wait_marker(int marker) {
 	CNET_REQUIRE_INIT();
 	CNET_NOT_IN_CAPTURE();
 	CNET_CHECK_ARG(marker >= 0 && marker < Runtime::kMarkers);
 	// a marker that was never set does not hold anything back
-	CNET_HIP(hipStreamWaitEvent(rt().upload_stream, rt().marker[marker], 0));
-	return CNET_OK;
+	return wait_unless_reached(rt().upload_stream, rt().marker[marker]);
 }
 
 int cnet_mark_upload(int marker) {
@@ -441,8 +452,7 @@ int cnet_compute_wait_upload_marker(int marker) {
 	CNET_NOT_IN_CAPTURE();  // would pull the upload stream into the recording
 	CNET_CHECK_ARG(marker >= 0 && marker < Runtime::kMarkers);
 	// a marker that was never set does not hold anything back
-	CNET_HIP(hipStreamWaitEvent(rt().stream, rt().upload_marker[marker], 0));
-	return CNET_OK;
+	return wait_unless_reached(rt().stream, rt().upload_marker[marker]);
 }
 
 int cnet_compute_wait_upload(void) {
@@ -485,8 +495,7 @@ int cnet_compute_wait_ticket(int64_t ticket) {
 	const int64_t n = ticket >> 1;
 	CNET_CHECK_ARG(ticket >= 0 && which == 1 && n < r.tickets_issued[which]);
 	// a ticket whose event has been handed out again since stands for a later point of the same stream: the wait still covers it
-	CNET_HIP(hipStreamWaitEvent(r.stream, r.ticket_event[which][n % Runtime::kTickets], 0));
-	return CNET_OK;
+	return wait_unless_reached(r.stream, r.ticket_event[which][n % Runtime::kTickets]);
 }
 
 int cnet_upload_sync(void) {

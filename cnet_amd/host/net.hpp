@@ -21,8 +21,11 @@ class CNet {
 	int32_t *d_labels_ = NULL;
 	std::vector<int> labels_;
 	bool batch_labels_ = false;       // labels_ came with a batch (they then win over a label argument, as upstream)
-	// device double buffer of the data input: stage_[active_] is what the kernels read, the other one can be filled by
-	// gpuPrefetch() meanwhile
+	// Device buffers of the data input, used in turn: stage_[active_] is what the kernels read, the next one can be filled by
+	// gpuPrefetch() meanwhile.  Three rather than two: the buffer about to be refilled was then last read two steps ago, and
+	// the point of the compute stream at which it was retired has been reached by the time the upload stream is told to wait
+	// for it (with two buffers that point is the end of the step that is still running when the next batch is sent off).
+	static constexpr int kStages = 3;
 	struct Stage {
 		float *z = NULL;            // 2 planes [batch][len]
 		int32_t *labels = NULL;     // [batch]
@@ -42,8 +45,9 @@ class CNet {
 	// stream: the hand-over between the streams (two waits and two recorded points per step) costs the host more than the
 	// copy costs the device in front of the forward pass.
 	bool gatherOnCompute(const InputBatch &batch, size_t plane_bytes) const { return batch.resident_ && 2 * plane_bytes <= ((size_t) 1 << 20); }
-	Stage stage_[2];
+	Stage stage_[kStages];
 	int active_ = 0;
+	int nextStage() const { return (active_ + 1) % kStages; }
 	// recorded phases of a step, one set per buffer of the data input (device pointers are frozen into a recording)
 	struct StepGraphs {
 		void *fwd = NULL, *bwd = NULL, *upd = NULL;
@@ -53,7 +57,7 @@ class CNet {
 		float step_lr = 0.f;
 		bool step_warm = false;  // the three phases have run once with this buffer since the last change of the plan
 	};
-	StepGraphs graphs_[2];
+	StepGraphs graphs_[kStages];
 	bool use_graphs_ = false;
 	bool conjugate_gradients_ = true;
 	bool fuse_layers_ = true;
@@ -1409,7 +1413,7 @@ private:
 		(void) outp;
 		beforeFeed(cin);
 		CFunc::Slot &s = cin->slots_[0];
-		Stage &staged = stage_[1 - active_];
+		Stage &staged = stage_[nextStage()];
 		if (staged.holds == &batch && staged.deferred) {  // nothing was sent ahead: the direct path below copies it on the compute stream
 			staged.holds = NULL;
 			staged.deferred = false;
@@ -1420,7 +1424,7 @@ private:
 			checkLabels(batch.labelsPtr(), batch_);
 			ck(cnet_compute_wait_ticket(staged.upload_ticket), "cnet_compute_wait_ticket");  // this batch's copies, nothing later
 			ck(cnet_mark_compute(active_), "cnet_mark_compute");
-			active_ = 1 - active_;
+			active_ = nextStage();
 			staged.holds = NULL;
 			cin->out_ = staged.z;
 			s.z = staged.z;
@@ -1493,7 +1497,7 @@ public:
 			throw std::invalid_argument("gpuPrefetch: batch shape differs from the allocated net");
 		if (!batch.isPinned() && !batch.resident_) throw std::invalid_argument("gpuPrefetch: the batch is not in page-locked memory");
 		checkLabels(batch.labelsPtr(), batch_);
-		const int other = 1 - active_;
+		const int other = nextStage();
 		Stage &st = stage_[other];
 		if (st.holds) throw std::logic_error("gpuPrefetch: a staged batch is still waiting for its gpuForward");
 		CFunc::Slot &s = cin->slots_[0];

@@ -76,7 +76,8 @@ int cnet_memcpy_h2d(void *dst, const void *host_src, size_t bytes);   /* *_copy_
  *      far has finished (call before overwriting a device buffer that kernels may still read).
  * cnet_mark_compute(m) / cnet_upload_wait_marker(m), m = 0..7: the same in two halves - remember the current tail of the
  *      compute stream under number m now, make later uploads wait for that point when a buffer is about to be refilled
- *      (double buffering: the marker is set when a buffer is retired, the wait is issued when it is reused).
+ *      (buffers used in turn: the marker is set when a buffer is retired, the wait is issued when it is reused; a wait for a
+ *      point that has been reached already is not queued at all).
  * cnet_compute_wait_upload: kernels queued after this call start only when every upload queued so far has landed.
  * cnet_mark_upload(m) / cnet_compute_wait_upload_marker(m), m = 0..7: the same in two halves - remember the current tail
  *      of the upload stream under number m (right after the copies of one batch were queued), make later kernels wait for
