@@ -80,6 +80,9 @@ struct CgemmArgs {
 	// The imaginary plane of A holds nothing but +0 (the caller vouches: real samples in front of a transform) and is not read:
 	// two real products per complex one, re = Ar Br, im = +-Ar Bi, the bits of the four products on such an A.  Honoured by the
 	// block kernels for a row-major A against a k-major B (the layout of the transform); ignored elsewhere.
+	// a_real == 2: the two planes of A are two real operands of their own and C = (Ar Br) + i (Ai Bi): the transform of
+	// real samples folded about n/2 (cos is even and sin odd under k -> n - k: Ar holds x[k] + x[n - k], Ai holds
+	// x[k] - x[n - k], and K is half as long).  Block kernels of that layout only; the caller sees to it that they take it.
 	int a_real = 0;
 	// mirror == 3 (MIRROR_HERM): element (row, col) with herm_lo <= col <= herm_hi also goes, conjugated, to column herm_n - col
 	// of the same row of C (honouring `accumulate`): the transform of real samples computes columns 0 .. n/2 and fills the others
@@ -583,10 +586,12 @@ struct DlStage {
 // for one addition per operand fragment and k pair; the imaginary part then carries the rounding of all three products
 // (normwise as accurate as four products, not componentwise).
 // A_REAL: the imaginary plane of A is all +0 and is neither fetched nor multiplied (CgemmArgs::a_real): two real products.
-template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int NST, bool GAUSS = false, bool A_REAL = false>
+// A_FOLD: the planes of A are two real operands, C = (Ar Br) + i (Ai Bi) (CgemmArgs::a_real == 2): two real products.
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int NST, bool GAUSS = false, bool A_REAL = false, bool A_FOLD = false>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))) void cgemm_fast_kernel(const CgemmArgs args) {
 	static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per workgroup");
 	static_assert(!(GAUSS && A_REAL), "a real operand leaves two products: nothing for the three-product form to save");
+	static_assert(!(A_FOLD && (GAUSS || A_REAL)), "the folded form has its own two products");
 	constexpr int TM = WM / 32, TN = WN / 32;
 	typedef DlStage<BM, A_MCONTIG> StageA;
 	typedef DlStage<BN, B_NCONTIG> StageB;
@@ -622,7 +627,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 	// S = Ai Br) and combines them with their signs when it stores, so its K loop has no vector-ALU instruction for signs at
 	// all; with four tiles there are only registers for two sets, re = P -+ Q and im = +-R +- S, and one operand of the
 	// second product is negated per k pair (see the modes below).
-	constexpr bool ACC4 = TM * TN <= 2 && !A_REAL;
+	constexpr bool ACC4 = TM * TN <= 2 && !A_REAL && !A_FOLD;
 	constexpr bool ACC_Q = ACC4 || GAUSS, ACC_S = ACC4 && !GAUSS;
 	floatx16 acc_re[TM][TN], acc_im[TM][TN], acc_q[ACC_Q ? TM : 1][ACC_Q ? TN : 1], acc_s[ACC_S ? TM : 1][ACC_S ? TN : 1];
 	for (int pass = 0; pass < npass; ++pass) {
@@ -759,14 +764,22 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			for (int i = 0; i < TM; ++i) {
 				are[i] = fa.re(ks, i);
 				aim[i] = fa.im(ks, i);
-				if (!ACC4 && !GAUSS && !A_REAL) neg[i] = MODE == 1 ? -are[i] : -aim[i];
+				if (!ACC4 && !GAUSS && !A_REAL && !A_FOLD) neg[i] = MODE == 1 ? -are[i] : -aim[i];
 			}
 #pragma unroll
 			for (int j = 0; j < TN; ++j) {
 				bre[j] = fb.re(ks, j);
 				bim[j] = fb.im(ks, j);
 			}
-			if constexpr (A_REAL) {
+			if constexpr (A_FOLD) {
+#pragma unroll
+				for (int i = 0; i < TM; ++i)
+#pragma unroll
+					for (int j = 0; j < TN; ++j) {
+						acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(are[i], bre[j], acc_re[i][j], 0, 0, 0);
+						acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aim[i], bim[j], acc_im[i][j], 0, 0, 0);
+					}
+			} else if constexpr (A_REAL) {
 #pragma unroll
 				for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -823,7 +836,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				// scheduling recipe for this k pair: after each MFMA let a few of the pending VALU / LDS / global
 				// instructions issue, so they run in the shadow of the matrix pipe
 #pragma unroll
-				for (int q = 0; q < (A_REAL ? 2 : GAUSS ? 3 : 4) * TM * TN; ++q) {
+				for (int q = 0; q < ((A_REAL || A_FOLD) ? 2 : GAUSS ? 3 : 4) * TM * TN; ++q) {
 					__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
 					__builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // <= 2 VALU
 					__builtin_amdgcn_sched_group_barrier(0x080, 1, 0);  // <= 1 LDS
@@ -854,7 +867,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 			if (c + 1 < c_hi) chunk(1, mode_c, c + 1);
 		}
 	};
-	if constexpr (ACC4 || GAUSS || A_REAL) {
+	if constexpr (ACC4 || GAUSS || A_REAL || A_FOLD) {
 		kloop(std::integral_constant<int, 0>());  // the signs wait for the store
 	} else {
 		switch (mode) {
@@ -883,7 +896,10 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))
 				if (row < args.M) {
 					const long off = (long) (row - row_org) * ldc + (col - col_org);
 					float vr, vi;
-					if constexpr (A_REAL) {
+					if constexpr (A_FOLD) {
+						vr = acc_re[i][j][e];
+						vi = acc_im[i][j][e];
+					} else if constexpr (A_REAL) {
 						vr = acc_re[i][j][e];
 						vi = r_minus ? -acc_im[i][j][e] : acc_im[i][j][e];
 					} else if constexpr (GAUSS) {
@@ -1565,6 +1581,9 @@ hipError_t prime_attributes() {
 			if (e == hipSuccess)
 				e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, true>),
 						hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem);
+			if (e == hipSuccess)
+				e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, false, true>),
+						hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem);
 		}
 		if constexpr ((WM / 32) * (WN / 32) <= 2 || A_MCONTIG || B_NCONTIG) {
 			if (e == hipSuccess)
@@ -1660,6 +1679,18 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 			constexpr int NST = (BM == 128 && BN == 128) ? 2 : 3;
 			constexpr size_t fast_smem = (size_t) NST * 2 * KC * (BM + BN) * sizeof(float);
 			if constexpr (!A_MCONTIG && B_NCONTIG) {
+				if (args.a_real == 2) {
+					static bool fold_attr_set = false;
+					if (!fold_attr_set && !g_attrs_primed) {
+						CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, false, true>),
+								hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem));
+						fold_attr_set = true;
+					}
+					hipLaunchKernelGGL((cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, false, true>), grid, dim3(NTHREADS), fast_smem,
+							cnet::rt().stream, args);
+					CNET_LAUNCH_CHECK();
+					return finish();
+				}
 				if (args.a_real) {
 					static bool real_attr_set = false;
 					if (!real_attr_set && !g_attrs_primed) {
@@ -1701,6 +1732,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 			return finish();
 		}
 	}
+	if (args.a_real == 2) return cnet::fail(CNET_ERR_UNSUPPORTED, "cgemm: the folded form of a real operand has block kernels for aligned operands only");
 	auto kern = cgemm_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, VEC>;
 	static bool attr_set = false;  // per instantiation
 	if (!attr_set && !g_attrs_primed) {
@@ -1865,6 +1897,11 @@ namespace cnet {
 static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int nprob, int batch) {
 	if (a.M <= 0 || a.N <= 0) return CNET_OK;
 	if (a.K <= 0) return fail(CNET_ERR_INVALID_ARGUMENT, "cgemm: K must be positive");
+	if (a.a_real == 2) {  // (cgemm_folded has checked that the block kernels of this layout take it: nothing is split off)
+		if (a_mcontig || !b_ncontig || nprob != 1 || batch != 1 || a.K % KC != 0)
+			return fail(CNET_ERR_UNSUPPORTED, "cgemm: the folded form of a real operand is a row-major A against a k-major B, K in whole chunks");
+		return pick_tile<false, true, 4>(a, nprob, batch);
+	}
 	if (a_mcontig || !b_ncontig) a.a_real = 0;  // only that layout has the kernels (the imaginary plane holds zeros: reading it is right too)
 	int rc = CNET_OK;
 	if (try_skinny(a_mcontig, b_ncontig, a, nprob, batch, &rc)) return rc;
@@ -2028,6 +2065,29 @@ bool cgemm_linear_bwd_gate(const float *g_re, const float *g_im, long ldg, const
 	const SkinnyStrides st0 = skinny_strides(args0, false, true), st1 = skinny_strides(args1, true, true);
 	*rc = CNET_SKINNY_PICK(v, launch_skinny_gate_bwd, (args0, st0, args1, st1, gate));
 	return true;
+}
+
+// Whether a product of this size would go to the block kernels (and not to the small-C kernel), as the folded form needs
+bool cgemm_block_sized(int M, int N) {
+	return ((long) (M + 15) / 16) * ((N + 15) / 16) > 4L * rt().prop.multiProcessorCount;
+}
+
+// C = (Ae B_re) + i (Ao B_im) for two real operands Ae, Ao [M][K] (K a multiple of 16, planes 16-byte aligned) against a
+// k-major B, with the mirrored columns of cgemm_real_a (used by cdft.hip for the folded transform of real samples)
+int cgemm_folded(int M, int N, int K, const float *ae, const float *ao, long lda, const float *b_re, const float *b_im, long ldb, float *c_re,
+		float *c_im, long ldc, int herm_n) {
+	const float *ar[2] = {ae, ae}, *ai[2] = {ao, ao}, *br[2] = {b_re, b_re}, *bi[2] = {b_im, b_im};
+	float *cr[2] = {c_re, c_re}, *ci[2] = {c_im, c_im};
+	const bool cj[2] = {false, false};
+	CgemmArgs a = pair_args(1, M, N, K, ar, ai, lda, br, bi, ldb, cj, cr, ci, ldc, 0, 0, 0);
+	a.a_real = 2;
+	if (herm_n > N) {
+		a.mirror = MIRROR_HERM;
+		a.herm_n = herm_n;
+		a.herm_lo = 1;
+		a.herm_hi = herm_n - N;
+	}
+	return cgemm_dispatch(false, true, a, 1, 1);
 }
 
 // One product whose A (row-major) has an imaginary plane of nothing but +0, against a k-major B (used by cdft.hip)

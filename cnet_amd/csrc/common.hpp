@@ -37,6 +37,10 @@ struct Runtime {
 	// for the same size)
 	void *workspace = nullptr;
 	size_t workspace_bytes = 0;
+	// a second buffer of the same kind, for an operand that a product reads while it may itself use the workspace for partial
+	// sums (the folded samples of the transform of real input)
+	void *operand_workspace = nullptr;
+	size_t operand_workspace_bytes = 0;
 	// A recorded graph holds the workspace address it was recorded with: while any recording exists, a workspace that
 	// has to grow is retired (kept until shutdown) instead of freed.
 	// Each live recording is kept as (executable, the graph it was instantiated from): the template graph lives as long
@@ -56,6 +60,7 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int hip_fail(hipError_t e, const char *what);
 // returns nullptr (and records the error) when the allocation fails
 void *workspace(size_t bytes);
+void *operand_workspace(size_t bytes);  // the second buffer (Runtime::operand_workspace); same rules
 // every hipFuncSetAttribute the matrix kernels need, made once, outside any stream capture (cgemm.hip)
 int cgemm_prime_attributes();
 

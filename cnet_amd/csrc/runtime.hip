@@ -25,38 +25,43 @@ int hip_fail(hipError_t e, const char *what) {
 	return e == hipErrorOutOfMemory ? CNET_ERR_OUT_OF_MEMORY : CNET_ERR_HIP;
 }
 
-void *workspace(size_t bytes) {
+// one grow-only buffer (see Runtime::workspace): at least `bytes` long, or nullptr with the error recorded
+static void *grown(void *&buf, size_t &have, size_t bytes) {
 	Runtime &r = rt();
-	if (bytes <= r.workspace_bytes) return r.workspace;
+	if (bytes <= have) return buf;
 	if (r.capturing) {
 		fail(CNET_ERR_UNSUPPORTED, "the workspace would have to grow while a graph is being recorded: run the same calls once before recording");
 		return nullptr;
 	}
-	if (r.workspace) {
+	if (buf) {
 		if (r.graphs_alive > 0) {  // a recording may replay kernels that use the old buffer
 			if (r.retired_count == Runtime::kRetired) {
 				fail(CNET_ERR_UNSUPPORTED, "the workspace had to grow %d times while recorded graphs exist: destroy the graphs first", Runtime::kRetired);
 				return nullptr;
 			}
-			r.retired[r.retired_count++] = r.workspace;
+			r.retired[r.retired_count++] = buf;
 		} else {
 			// queued kernels may still read the old buffer
 			hipStreamSynchronize(r.stream);
-			hipFree(r.workspace);
+			hipFree(buf);
 		}
-		r.workspace = nullptr;
-		r.workspace_bytes = 0;
+		buf = nullptr;
+		have = 0;
 	}
 	size_t want = bytes + bytes / 2;
-	hipError_t e = hipMalloc(&r.workspace, want);
+	hipError_t e = hipMalloc(&buf, want);
 	if (e != hipSuccess) {
 		hip_fail(e, "workspace hipMalloc");
-		r.workspace = nullptr;
+		buf = nullptr;
 		return nullptr;
 	}
-	r.workspace_bytes = want;
-	return r.workspace;
+	have = want;
+	return buf;
 }
+
+void *workspace(size_t bytes) { return grown(rt().workspace, rt().workspace_bytes, bytes); }
+
+void *operand_workspace(size_t bytes) { return grown(rt().operand_workspace, rt().operand_workspace_bytes, bytes); }
 
 void release_twiddles();  // cdft.hip
 int init_static_scratch(int device);  // reduce.hip
@@ -159,6 +164,9 @@ int cnet_shutdown(void) {
 	if (r.workspace) hipFree(r.workspace);
 	r.workspace = nullptr;
 	r.workspace_bytes = 0;
+	if (r.operand_workspace) hipFree(r.operand_workspace);
+	r.operand_workspace = nullptr;
+	r.operand_workspace_bytes = 0;
 	for (int k = 0; k < r.retired_count; ++k) hipFree(r.retired[k]);
 	r.retired_count = 0;
 	r.graphs_alive = 0;

@@ -280,8 +280,12 @@ int cnet_cdft_hadamard_cgelu_fwd(const float *x_re, const float *x_im, int64_t l
  * matrix product and the rest are written as conjugates by the same kernels as they store their partners (exact conjugates;
  * the up to three columns next to n/2 whose partners the product computes as well agree with them to rounding), and of the
  * four real products of a complex one the two with x_im are left out: a quarter of the
- * matrix work of cnet_cdft_fwd.  Agrees with cnet_cdft_fwd on such samples to rounding (the stored twiddles are symmetric
- * under q -> n - q up to their last bit; the products that are left out add exact zeros); assigns. */
+ * matrix work of cnet_cdft_fwd.  Where the block kernels run the product (an even n at a batch beyond the small-C kernel)
+ * the samples are folded about n/2 first, e[k] = x[k] + x[n - k] and o[k] = x[k] - x[n - k] (cos is even and sin odd under
+ * k -> n - k), so that Re y = e F_re and Im y = o F_im are sums over k = 0 .. n/2 only: an eighth of the matrix work
+ * (4096 x 784: 46 us with the pass that folds, 59 without; 1024 x 4096: 165 against 257; against double precision 8.0e-7
+ * where the full product has 1.1e-6 at n = 4096).  Agrees with cnet_cdft_fwd on such samples to rounding (the stored
+ * twiddles are symmetric under q -> n - q up to their last bit; the products that are left out add exact zeros); assigns. */
 int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
                              int B, int n);
 int cnet_cdft_bwd(const float *g_dz_re, const float *g_dz_im, const float *g_dzs_re, const float *g_dzs_im, int64_t ldg,
@@ -529,6 +533,7 @@ int cnet_embedding_bwd(const int32_t *tokens, const float *g_dzs_re, const float
  *   CNET_CGEMM_SKINNY_W = 4|8|16 wavefronts per tile of the small-C kernel
  *   CNET_CGEMM_SKINNY_TWO = 0    two small products of one call as two launches (and the gate behind them as launches of its own)
  *   CNET_CGEMM_3M = 0 | 1        initial value of cnet_cgemm_set_products (1: three real products per complex one)
+ *   CNET_DFT_FOLD = 0            the transform of real samples without folding them about n/2 first
  *   CNET_STREAM_MIN_MB = n       footprint (MiB) from which an elementwise / row launch counts as streaming (default 256)
  *   CNET_STREAM_POLICY = 0..3    cache policy of every streaming launch: plain, hint on loads and stores, hinted stores,
  *                                hinted loads + device-scope stores (default: per kernel)

@@ -112,13 +112,14 @@ def test_cpu_forward_operator_can_be_installed(gpu, port):
 
 
 @pytest.mark.parametrize("B,n", [(1, 1), (3, 2), (5, 7), (64, 784), (33, 97), (300, 1024), (4096, 784), (1024, 784), (128, 784),
-                                 (8, 100), (300, 1000), (130, 36), (700, 516), (1024, 4096)])
+                                 (8, 100), (300, 1000), (130, 36), (700, 516), (1024, 4096), (700, 2000), (2000, 786)])
 def test_transform_of_real_samples_through_half_the_columns(gpu, port, B, n):
     """cnet_cdft_fwd_real_input: columns 0 .. n/2 by the matrix product (without the real products that the zero imaginary
     plane of the samples would feed), the rest as conjugates, written by the same kernels as they store their partners.  The
     shapes take every kernel that writes them: the small-C kernel (64 x 784), the block kernels with the columns beyond a
     multiple of 64 split off and K cut (1024 x 784), with blocks on the edge (700 x 516), the kernel for unaligned shapes (odd
-    n), a K that is not a whole number of chunks (n = 100, 1000: the rest of K is added by a second launch, to the mirrored
+    n), the samples folded about n/2 first and a product half as long (an even n at batches beyond the small-C kernel:
+    1024 and 4096 x 784, 1024 x 4096, 700 x 2000), a K that is not a whole number of chunks (n = 100, 1000: the rest of K is added by a second launch, to the mirrored
     columns as well).  Against the full transform of the same samples (to rounding: the stored twiddles are symmetric under
     q -> n - q up to their last bit), against the CPU path, and the symmetry itself: to the bit for every column that is written as
     a conjugate, to rounding for the up to three columns next to n/2 that the product computes together with their partners."""
@@ -129,9 +130,17 @@ def test_transform_of_real_samples_through_half_the_columns(gpu, port, B, n):
     ops.dft_fwd_real_input(x, half)
     fr, fi = full.host()
     hr, hi = half.host()
-    # two roundings of the same sums; the full transform rounds more where the process forms a complex product from three real
-    # ones (CNET_CGEMM_3M=1: 1.6e-6 from double precision at n = 4096), which the transform of real samples never does
-    assert rel_c((hr, hi), (fr, fi)) < (1e-6 if capi.load().cnet_cgemm_get_products() == 4 else 3e-6)
+    # two roundings of the same sums, in another order where the samples are folded about n/2 first (an even n at a batch that
+    # takes the block kernels: half as many terms per sum; against double precision 8.0e-7 where the full product has 1.14e-6
+    # at n = 4096, 3.6e-7 against 5.0e-7 at n = 784); the full transform rounds more where the process forms a complex product
+    # from three real ones (CNET_CGEMM_3M=1: 1.6e-6 from double precision at n = 4096), which the transform of real samples
+    # never does
+    assert rel_c((hr, hi), (fr, fi)) < (2e-6 if capi.load().cnet_cgemm_get_products() == 4 else 3e-6)
+    if B * n <= 1 << 22:   # against double precision: no worse than the full product
+        ref = np.fft.fft(xr.astype(np.float64), axis=1) / np.sqrt(n)
+        def err(re, im):
+            return np.linalg.norm((re.astype(np.float64) + 1j * im.astype(np.float64)) - ref) / np.linalg.norm(ref)
+        assert err(hr, hi) < max(1.2 * err(fr, fi), 2e-7), (err(hr, hi), err(fr, fi))
     cols = min(n, (n // 2 + 1 + 3) // 4 * 4)   # what the product computes; the columns from there on are written as conjugates
     for q in range(1, (n - 1) // 2 + 1):
         if q <= n - cols:
