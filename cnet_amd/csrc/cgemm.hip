@@ -585,13 +585,17 @@ struct DlStage {
 // sa, sb the signs of the imaginary parts: re = P - sa sb Q, im = T - P - sa sb Q).  A quarter of the matrix work less,
 // for one addition per operand fragment and k pair; the imaginary part then carries the rounding of all three products
 // (normwise as accurate as four products, not componentwise).
-// A_REAL: the imaginary plane of A is all +0 and is neither fetched nor multiplied (CgemmArgs::a_real): two real products.
-// A_FOLD: the planes of A are two real operands, C = (Ar Br) + i (Ai Bi) (CgemmArgs::a_real == 2): two real products.
-template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int NST, bool GAUSS = false, bool A_REAL = false, bool A_FOLD = false>
+// The last two template arguments name the form of the complex product:
+//   THREE, REAL_A = false, false  four real products (or two sets of accumulators with signs, see below)
+//   true, false                   three real products (Gauss; CgemmArgs via cnet_cgemm_set_products)
+//   false, true                   the imaginary plane of A is all +0 and is neither fetched nor multiplied
+//                                 (CgemmArgs::a_real == 1): two real products, re = Ar Br, im = Ar Bi
+//   true, true                    the planes of A are two real operands of their own, C = (Ar Br) + i (Ai Bi)
+//                                 (CgemmArgs::a_real == 2, the folded samples of a transform): two real products
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int NST, bool THREE = false, bool REAL_A = false>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 4))) void cgemm_fast_kernel(const CgemmArgs args) {
 	static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per workgroup");
-	static_assert(!(GAUSS && A_REAL), "a real operand leaves two products: nothing for the three-product form to save");
-	static_assert(!(A_FOLD && (GAUSS || A_REAL)), "the folded form has its own two products");
+	constexpr bool A_FOLD = THREE && REAL_A, GAUSS = THREE && !REAL_A, A_REAL = REAL_A && !THREE;
 	constexpr int TM = WM / 32, TN = WN / 32;
 	typedef DlStage<BM, A_MCONTIG> StageA;
 	typedef DlStage<BN, B_NCONTIG> StageB;
@@ -1582,7 +1586,7 @@ hipError_t prime_attributes() {
 				e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, true>),
 						hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem);
 			if (e == hipSuccess)
-				e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, false, true>),
+				e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, true, true>),
 						hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem);
 		}
 		if constexpr ((WM / 32) * (WN / 32) <= 2 || A_MCONTIG || B_NCONTIG) {
@@ -1682,11 +1686,11 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 				if (args.a_real == 2) {
 					static bool fold_attr_set = false;
 					if (!fold_attr_set && !g_attrs_primed) {
-						CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, false, true>),
+						CNET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, true, true>),
 								hipFuncAttributeMaxDynamicSharedMemorySize, (int) fast_smem));
 						fold_attr_set = true;
 					}
-					hipLaunchKernelGGL((cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, false, false, true>), grid, dim3(NTHREADS), fast_smem,
+					hipLaunchKernelGGL((cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST, true, true>), grid, dim3(NTHREADS), fast_smem,
 							cnet::rt().stream, args);
 					CNET_LAUNCH_CHECK();
 					return finish();
