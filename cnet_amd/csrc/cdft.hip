@@ -249,9 +249,9 @@ int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, 
 	// product writes them, conjugated, as it stores their partners.
 	const int cols = std::min(n, (n / 2 + 1 + 3) / 4 * 4);
 	// Folded about n/2 (fold_kernel), the product is half as long: where the block kernels run it (an even n, a batch
-	// beyond the small-C kernel), 4096 x 784: 59 -> 46 us with the pass that folds.  The folded samples live in a buffer of the library's own that only
-	// grows (not the workspace, where the product may keep partial sums); while a graph is being recorded it cannot, and
-	// the unfolded product runs.
+	// beyond the small-C kernel), 4096 x 784: 59 -> 46 us with the pass that folds.  The folded samples live in a buffer of
+	// the library's own that only grows (not the workspace, where the product may keep partial sums); while a graph is
+	// being recorded it cannot, and a batch larger than any before runs the unfolded product.
 	const int kp = (n / 2 + 1 + 15) / 16 * 16;
 	static const bool fold = [] {
 		const char *e = getenv("CNET_DFT_FOLD");  // tuning override: 0 keeps the unfolded product
