@@ -151,3 +151,24 @@ def test_transform_of_real_samples_through_half_the_columns(gpu, port, B, n):
     if B * n * n <= 1 << 27:
         yr, yi = port.dft_fwd(xr, np.zeros_like(xr))
         assert rel_c((hr, hi), (yr, yi)) < TOL
+
+
+def test_folded_transform_of_real_samples_in_windows_of_wider_buffers(gpu, port):
+    """The transform of real samples at a batch that folds them about n/2 first, with the samples and the result each a column
+    window of a wider buffer (leading dimensions beyond n, first columns at multiples of four): against double precision, and
+    what lies beside the result's window stays untouched."""
+    rs = np.random.RandomState(11)
+    B, n = 1500, 784
+    xw = rs.randn(B, n + 16).astype(np.float32)
+    x_full = ops.CMat.from_host(xw, np.zeros_like(xw))
+    x = x_full.sub(8, n)
+    yb_re, yb_im = rs.randn(B, n + 24).astype(np.float32), rs.randn(B, n + 24).astype(np.float32)
+    y_full = ops.CMat.from_host(yb_re, yb_im)
+    y = y_full.sub(12, n)
+    ops.dft_fwd_real_input(x, y)
+    gr, gi = y_full.re.owner.download(), y_full.im.owner.download()
+    ref = np.fft.fft(xw[:, 8:8 + n].astype(np.float64), axis=1) / np.sqrt(n)
+    got = gr[:, 12:12 + n].astype(np.float64) + 1j * gi[:, 12:12 + n].astype(np.float64)
+    assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 6e-7
+    mask = np.ones(n + 24, bool); mask[12:12 + n] = False
+    assert np.array_equal(gr[:, mask], yb_re[:, mask]) and np.array_equal(gi[:, mask], yb_im[:, mask])
