@@ -65,6 +65,7 @@ __global__ void twiddle_kernel(float *__restrict__ fre, float *__restrict__ fim,
 // with e[0] = x[0], e[n/2] = x[n/2], e[k] = x[k] + x[n - k] and o[k] = x[k] - x[n - k] in between (o[0] = o[n/2] = 0): two
 // real products over half the k.  This kernel writes e and o as planes [rows][kp], kp = n/2 + 1 rounded up to a multiple
 // of 16 (the chunk of the block kernels), zeros beyond n/2; one thread per four k.
+template <bool V4>
 __global__ __launch_bounds__(256) void fold_kernel(const float *__restrict__ x, long ldx, float *__restrict__ e, float *__restrict__ o, int rows,
 		int n, int kp) {
 	const long idx = (long) blockIdx.x * 256 + threadIdx.x;
@@ -73,17 +74,29 @@ __global__ __launch_bounds__(256) void fold_kernel(const float *__restrict__ x, 
 	const long row = idx / groups;
 	const int k0 = (int) (idx - row * groups) * 4;
 	const float *xr = x + row * ldx;
+	float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};  // x[k0 + s] and its partner x[n - k0 - s]
+	if (V4 && k0 + 3 < n / 2 && k0 > 0) {
+		// (n and ldx multiples of four, x 16-byte aligned: x[k0 .. k0 + 3] is one aligned group, and the partners are the last
+		// three values of the aligned group that ends at n - k0, and the first value of the next one)
+		const float4 f = *reinterpret_cast<const float4 *>(xr + k0), g = *reinterpret_cast<const float4 *>(xr + n - k0 - 4);
+		a[0] = f.x, a[1] = f.y, a[2] = f.z, a[3] = f.w;
+		b[0] = xr[n - k0], b[1] = g.w, b[2] = g.z, b[3] = g.y;
+	} else {
+#pragma unroll
+		for (int s = 0; s < 4; ++s) {
+			const int k = k0 + s;
+			if (k <= n / 2) {
+				a[s] = xr[k];
+				if (k > 0 && k < n / 2) b[s] = xr[n - k];
+			}
+		}
+	}
 	float ev[4], ov[4];
 #pragma unroll
 	for (int s = 0; s < 4; ++s) {
 		const int k = k0 + s;
-		float a = 0.f, b = 0.f;
-		if (k <= n / 2) {
-			a = xr[k];
-			if (k > 0 && k < n / 2) b = xr[n - k];
-		}
-		ev[s] = a + b;
-		ov[s] = (k > 0 && k < n / 2) ? a - b : 0.f;
+		ev[s] = a[s] + b[s];
+		ov[s] = (k > 0 && k < n / 2) ? a[s] - b[s] : 0.f;
 	}
 	float4 *pe = reinterpret_cast<float4 *>(e + row * kp + k0), *po = reinterpret_cast<float4 *>(o + row * kp + k0);
 	*pe = make_float4(ev[0], ev[1], ev[2], ev[3]);
@@ -264,7 +277,10 @@ int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, 
 			if (!e) return CNET_ERR_OUT_OF_MEMORY;
 			float *o = e + (size_t) B * kp;
 			const long threads = (long) B * (kp / 4);
-			hipLaunchKernelGGL(fold_kernel, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, rt().stream, x_re, (long) ldx, e, o, B, n, kp);
+			if (n % 4 == 0 && ldx % 4 == 0 && aligned16(x_re))
+				hipLaunchKernelGGL(fold_kernel<true>, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, rt().stream, x_re, (long) ldx, e, o, B, n, kp);
+			else
+				hipLaunchKernelGGL(fold_kernel<false>, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, rt().stream, x_re, (long) ldx, e, o, B, n, kp);
 			CNET_LAUNCH_CHECK();
 			return cgemm_folded(B, cols, kp, e, o, kp, t.re, t.im, t.ld, y_re, y_im, ldy, n);
 		}
