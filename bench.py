@@ -184,10 +184,11 @@ def dft_lines(mfma, cmat, grad, rs):
     xr = ops.CMat.from_host(rs.randn(Bf, nf).astype(np.float32), np.zeros((Bf, nf), np.float32))
     # an eighth of the full transform's flops: columns 0..n/2 only, two real products per complex one (the imaginary plane of
     # the samples is neither read nor multiplied), and the samples folded about n/2 first (cos is even, sin odd), which
-    # halves the length of every sum: n/2 + 1 terms, rounded up to whole chunks of 16
+    # halves the length of every sum: n/2 + 1 terms, rounded up to whole chunks of 16; the pass that folds forms column n/2
+    # itself (n/2 is a multiple of 64 here), so the product has n/2 columns
     kp = (nf // 2 + 1 + 15) // 16 * 16
     mfma("cdft_fwd_real", "cdft_fwd of real samples (columns 0..n/2 by the product, the rest as conjugates; the samples folded about n/2, two real products over half the terms; flops executed, the pass that folds included in the time)",
-         [Bf, nf], 4.0 * Bf * kp * (nf // 2 + 4), lambda: ops.dft_fwd_real_input(xr, y))
+         [Bf, nf], 4.0 * Bf * kp * (nf // 2), lambda: ops.dft_fwd_real_input(xr, y))
     del xr
     # TriangFourier: only the pairs in <= out contribute, n (n + 1) / 2 complex multiply-adds per row
     tri = nf * (nf + 1) / 2.0

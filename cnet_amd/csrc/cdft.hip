@@ -66,14 +66,7 @@ __global__ void twiddle_kernel(float *__restrict__ fre, float *__restrict__ fim,
 // real products over half the k.  This kernel writes e and o as planes [rows][kp], kp = n/2 + 1 rounded up to a multiple
 // of 16 (the chunk of the block kernels), zeros beyond n/2; one thread per four k.
 template <bool V4>
-__global__ __launch_bounds__(256) void fold_kernel(const float *__restrict__ x, long ldx, float *__restrict__ e, float *__restrict__ o, int rows,
-		int n, int kp) {
-	const long idx = (long) blockIdx.x * 256 + threadIdx.x;
-	const int groups = kp / 4;
-	if (idx >= (long) rows * groups) return;
-	const long row = idx / groups;
-	const int k0 = (int) (idx - row * groups) * 4;
-	const float *xr = x + row * ldx;
+__device__ __forceinline__ void fold_group(const float *__restrict__ xr, int n, int k0, float ev[4], float ov[4]) {
 	float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};  // x[k0 + s] and its partner x[n - k0 - s]
 	if (V4 && k0 + 3 < n / 2 && k0 > 0) {
 		// (n and ldx multiples of four, x 16-byte aligned: x[k0 .. k0 + 3] is one aligned group, and the partners are the last
@@ -91,16 +84,55 @@ __global__ __launch_bounds__(256) void fold_kernel(const float *__restrict__ x, 
 			}
 		}
 	}
-	float ev[4], ov[4];
 #pragma unroll
 	for (int s = 0; s < 4; ++s) {
 		const int k = k0 + s;
 		ev[s] = a[s] + b[s];
 		ov[s] = (k > 0 && k < n / 2) ? a[s] - b[s] : 0.f;
 	}
+}
+
+template <bool V4>
+__global__ __launch_bounds__(256) void fold_kernel(const float *__restrict__ x, long ldx, float *__restrict__ e, float *__restrict__ o, int rows,
+		int n, int kp) {
+	const long idx = (long) blockIdx.x * 256 + threadIdx.x;
+	const int groups = kp / 4;
+	if (idx >= (long) rows * groups) return;
+	const long row = idx / groups;
+	const int k0 = (int) (idx - row * groups) * 4;
+	float ev[4], ov[4];
+	fold_group<V4>(x + row * ldx, n, k0, ev, ov);
 	float4 *pe = reinterpret_cast<float4 *>(e + row * kp + k0), *po = reinterpret_cast<float4 *>(o + row * kp + k0);
 	*pe = make_float4(ev[0], ev[1], ev[2], ev[3]);
 	*po = make_float4(ov[0], ov[1], ov[2], ov[3]);
+}
+
+// The same pass with one wavefront per row, which also forms column n/2 of the transform: F[k][n/2] = (-1)^k / sqrt n, so
+// Re X[n/2] = (e[0] - e[1] + e[2] - ...) / sqrt n and Im X[n/2] = 0.  The product then stops at column n/2 - 1; where n/2
+// is a multiple of the blocks' width that spares it a round of blocks that hold this one column.  The lanes' sums are
+// added in a fixed order.
+template <bool V4>
+__global__ __launch_bounds__(256) void fold_nyquist_kernel(const float *__restrict__ x, long ldx, float *__restrict__ e, float *__restrict__ o,
+		int rows, int n, int kp, float *__restrict__ y_re, float *__restrict__ y_im, long ldy, float scale) {
+	const long row = (long) blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (row >= rows) return;  // (a whole wavefront: nothing below is shared between wavefronts)
+	const int lane = threadIdx.x & 63, groups = kp / 4;
+	const float *xr = x + row * ldx;
+	float alt = 0.f;
+	for (int g = lane; g < groups; g += 64) {
+		float ev[4], ov[4];
+		fold_group<V4>(xr, n, g * 4, ev, ov);
+		float4 *pe = reinterpret_cast<float4 *>(e + row * kp + g * 4), *po = reinterpret_cast<float4 *>(o + row * kp + g * 4);
+		*pe = make_float4(ev[0], ev[1], ev[2], ev[3]);
+		*po = make_float4(ov[0], ov[1], ov[2], ov[3]);
+		alt += (ev[0] - ev[1]) + (ev[2] - ev[3]);
+	}
+#pragma unroll
+	for (int d = 32; d >= 1; d >>= 1) alt += __shfl_xor(alt, d, 64);
+	if (lane == 0) {
+		y_re[row * ldy + n / 2] = alt * scale;
+		y_im[row * ldy + n / 2] = 0.f;
+	}
 }
 
 static int get_plan(int n, Twiddle *out, bool create) {
@@ -276,8 +308,20 @@ int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, 
 			float *e = (float *) operand_workspace(need);
 			if (!e) return CNET_ERR_OUT_OF_MEMORY;
 			float *o = e + (size_t) B * kp;
+			const bool v4 = n % 4 == 0 && ldx % 4 == 0 && aligned16(x_re);
+			// n/2 a multiple of 64, the narrowest block: column n/2 would take a round of blocks of its own
+			if (n % 128 == 0 && cgemm_block_sized(B, n / 2)) {
+				const float scale = (float) (1.0 / sqrt((double) n));
+				const dim3 grid((unsigned) ((B + 3) / 4));
+				if (v4)
+					hipLaunchKernelGGL(fold_nyquist_kernel<true>, grid, dim3(256), 0, rt().stream, x_re, (long) ldx, e, o, B, n, kp, y_re, y_im, (long) ldy, scale);
+				else
+					hipLaunchKernelGGL(fold_nyquist_kernel<false>, grid, dim3(256), 0, rt().stream, x_re, (long) ldx, e, o, B, n, kp, y_re, y_im, (long) ldy, scale);
+				CNET_LAUNCH_CHECK();
+				return cgemm_folded(B, n / 2, kp, e, o, kp, t.re, t.im, t.ld, y_re, y_im, ldy, n);
+			}
 			const long threads = (long) B * (kp / 4);
-			if (n % 4 == 0 && ldx % 4 == 0 && aligned16(x_re))
+			if (v4)
 				hipLaunchKernelGGL(fold_kernel<true>, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, rt().stream, x_re, (long) ldx, e, o, B, n, kp);
 			else
 				hipLaunchKernelGGL(fold_kernel<false>, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, rt().stream, x_re, (long) ldx, e, o, B, n, kp);

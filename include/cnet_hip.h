@@ -283,8 +283,9 @@ int cnet_cdft_hadamard_cgelu_fwd(const float *x_re, const float *x_im, int64_t l
  * matrix work of cnet_cdft_fwd.  Where the block kernels run the product (an even n at a batch beyond the small-C kernel)
  * the samples are folded about n/2 first, e[k] = x[k] + x[n - k] and o[k] = x[k] - x[n - k] (cos is even and sin odd under
  * k -> n - k), so that Re y = e F_re and Im y = o F_im are sums over k = 0 .. n/2 only: an eighth of the matrix work
- * (4096 x 784: 46 us with the pass that folds, 59 without; 1024 x 4096: 165 against 257; against double precision 8.0e-7
- * where the full product has 1.1e-6 at n = 4096).  Agrees with cnet_cdft_fwd on such samples to rounding (the stored
+ * (4096 x 784: 46 us with the pass that folds, 59 without; 1024 x 4096: 150 against 257; against double precision 8.0e-7
+ * where the full product has 1.1e-6 at n = 4096); where n/2 is a multiple of 64 that pass also forms column n/2, the
+ * alternating sum of the samples over sqrt n, and the product stops before it.  Agrees with cnet_cdft_fwd on such samples to rounding (the stored
  * twiddles are symmetric under q -> n - q up to their last bit; the products that are left out add exact zeros); assigns. */
 int cnet_cdft_fwd_real_input(const float *x_re, const float *x_im, int64_t ldx, float *y_re, float *y_im, int64_t ldy,
                              int B, int n);

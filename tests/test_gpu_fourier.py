@@ -112,14 +112,16 @@ def test_cpu_forward_operator_can_be_installed(gpu, port):
 
 
 @pytest.mark.parametrize("B,n", [(1, 1), (3, 2), (5, 7), (64, 784), (33, 97), (300, 1024), (4096, 784), (1024, 784), (128, 784),
-                                 (8, 100), (300, 1000), (130, 36), (700, 516), (1024, 4096), (700, 2000), (2000, 786)])
+                                 (8, 100), (300, 1000), (130, 36), (700, 516), (1024, 4096), (700, 2000), (2000, 786), (600, 1024),
+                                 (2100, 256)])
 def test_transform_of_real_samples_through_half_the_columns(gpu, port, B, n):
     """cnet_cdft_fwd_real_input: columns 0 .. n/2 by the matrix product (without the real products that the zero imaginary
     plane of the samples would feed), the rest as conjugates, written by the same kernels as they store their partners.  The
     shapes take every kernel that writes them: the small-C kernel (64 x 784), the block kernels with the columns beyond a
     multiple of 64 split off and K cut (1024 x 784), with blocks on the edge (700 x 516), the kernel for unaligned shapes (odd
     n), the samples folded about n/2 first and a product half as long (an even n at batches beyond the small-C kernel:
-    1024 and 4096 x 784, 1024 x 4096, 700 x 2000), a K that is not a whole number of chunks (n = 100, 1000: the rest of K is added by a second launch, to the mirrored
+    1024 and 4096 x 784, 1024 x 4096, 700 x 2000; with n/2 a multiple of 64 the pass that folds also forms column n/2, as an
+    alternating sum, and the product stops before it: 1024 x 4096, 600 x 1024, 2100 x 256), a K that is not a whole number of chunks (n = 100, 1000: the rest of K is added by a second launch, to the mirrored
     columns as well).  Against the full transform of the same samples (to rounding: the stored twiddles are symmetric under
     q -> n - q up to their last bit), against the CPU path, and the symmetry itself: to the bit for every column that is written as
     a conjugate, to rounding for the up to three columns next to n/2 that the product computes together with their partners."""
@@ -141,6 +143,9 @@ def test_transform_of_real_samples_through_half_the_columns(gpu, port, B, n):
         def err(re, im):
             return np.linalg.norm((re.astype(np.float64) + 1j * im.astype(np.float64)) - ref) / np.linalg.norm(ref)
         assert err(hr, hi) < max(1.2 * err(fr, fi), 2e-7), (err(hr, hi), err(fr, fi))
+        if n % 2 == 0:   # column n/2 alone: the alternating sum of the samples, a real number
+            assert np.abs(hr[:, n // 2] - ref[:, n // 2].real).max() < 2e-6 * np.abs(xr).sum(axis=1).max() / np.sqrt(n)
+            assert np.abs(hi[:, n // 2]).max() < 2e-6 * np.abs(xr).sum(axis=1).max() / np.sqrt(n)
     cols = min(n, (n // 2 + 1 + 3) // 4 * 4)   # what the product computes; the columns from there on are written as conjugates
     for q in range(1, (n - 1) // 2 + 1):
         if q <= n - cols:
@@ -153,22 +158,24 @@ def test_transform_of_real_samples_through_half_the_columns(gpu, port, B, n):
         assert rel_c((hr, hi), (yr, yi)) < TOL
 
 
-def test_folded_transform_of_real_samples_in_windows_of_wider_buffers(gpu, port):
+@pytest.mark.parametrize("B,n,x_pad,x_off", [(1500, 784, 16, 8), (1200, 1024, 16, 8), (1200, 1024, 18, 5)])
+def test_folded_transform_of_real_samples_in_windows_of_wider_buffers(gpu, port, B, n, x_pad, x_off):
     """The transform of real samples at a batch that folds them about n/2 first, with the samples and the result each a column
-    window of a wider buffer (leading dimensions beyond n, first columns at multiples of four): against double precision, and
-    what lies beside the result's window stays untouched."""
+    window of a wider buffer (leading dimensions beyond n; the samples' first column at a multiple of four or not, which
+    decides between 128-bit and single loads in the pass that folds; n = 1024 has that pass form column n/2 as well): against
+    double precision, and what lies beside the result's window stays untouched."""
     rs = np.random.RandomState(11)
-    B, n = 1500, 784
-    xw = rs.randn(B, n + 16).astype(np.float32)
+    xw = rs.randn(B, n + x_pad).astype(np.float32)
     x_full = ops.CMat.from_host(xw, np.zeros_like(xw))
-    x = x_full.sub(8, n)
+    x = x_full.sub(x_off, n)
     yb_re, yb_im = rs.randn(B, n + 24).astype(np.float32), rs.randn(B, n + 24).astype(np.float32)
     y_full = ops.CMat.from_host(yb_re, yb_im)
     y = y_full.sub(12, n)
     ops.dft_fwd_real_input(x, y)
     gr, gi = y_full.re.owner.download(), y_full.im.owner.download()
-    ref = np.fft.fft(xw[:, 8:8 + n].astype(np.float64), axis=1) / np.sqrt(n)
+    ref = np.fft.fft(xw[:, x_off:x_off + n].astype(np.float64), axis=1) / np.sqrt(n)
     got = gr[:, 12:12 + n].astype(np.float64) + 1j * gi[:, 12:12 + n].astype(np.float64)
     assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 6e-7
+    assert np.abs(got[:, n // 2] - ref[:, n // 2]).max() < 1e-5
     mask = np.ones(n + 24, bool); mask[12:12 + n] = False
     assert np.array_equal(gr[:, mask], yb_re[:, mask]) and np.array_equal(gi[:, mask], yb_im[:, mask])
