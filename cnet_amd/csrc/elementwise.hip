@@ -161,8 +161,11 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_kernel(const float *_
 		float *__restrict__ partial, int rows, int cols, int rows_per_slab, int accumulate) {
 	__shared__ float red[CS_Y][4][CS_X * V];
 	const int tx = threadIdx.x % CS_X, ty = threadIdx.x / CS_X;
-	const long col = ((long) blockIdx.x * CS_X + tx) * V;
-	const bool live = col < cols;
+	// the groups of V columns are dealt evenly to the column blocks of the launch (n = 784: four blocks of 49 groups, not
+	// three of 64 and one of 4, whose workgroups would sit idle beside full ones)
+	const int per_block = ((cols + V - 1) / V + (int) gridDim.x - 1) / (int) gridDim.x;
+	const long col = ((long) blockIdx.x * per_block + tx) * V;
+	const bool live = tx < per_block && col < cols;
 	const int slab = blockIdx.y;
 	const int r0 = slab * rows_per_slab;
 	const int r1 = min(rows, r0 + rows_per_slab);
@@ -667,8 +670,11 @@ __global__ __launch_bounds__(TPB) void hadamard_bwd_shared_sym_kernel(const floa
 		int cols, int rows_per_slab, int accumulate) {
 	__shared__ float red[CS_Y][2][CS_X * V];
 	const int tx = threadIdx.x % CS_X, ty = threadIdx.x / CS_X;
-	const long col = ((long) blockIdx.x * CS_X + tx) * V;
-	const bool live = col < cols;
+	// the groups of V columns are dealt evenly to the column blocks of the launch (n = 784: four blocks of 49 groups, not
+	// three of 64 and one of 4, whose workgroups would sit idle beside full ones)
+	const int per_block = ((cols + V - 1) / V + (int) gridDim.x - 1) / (int) gridDim.x;
+	const long col = ((long) blockIdx.x * per_block + tx) * V;
+	const bool live = tx < per_block && col < cols;
 	const int slab = blockIdx.y;
 	const int r0 = slab * rows_per_slab;
 	const int r1 = min(rows, r0 + rows_per_slab);

@@ -392,8 +392,11 @@ __global__ __launch_bounds__(TPB) void colsum_partial_kernel(const float *__rest
 		int rows, int cols, int rows_per_slab, int policy) {
 	__shared__ float red[CS_Y][CS_X * V];
 	const int tx = threadIdx.x % CS_X, ty = threadIdx.x / CS_X;
-	const long col = ((long) blockIdx.x * CS_X + tx) * V;
-	const bool live = col < cols;
+	// the groups of V columns are dealt evenly to the column blocks of the launch (n = 784: four blocks of 49 groups, not
+	// three of 64 and one of 4, whose workgroups would sit idle beside full ones)
+	const int per_block = ((cols + V - 1) / V + (int) gridDim.x - 1) / (int) gridDim.x;
+	const long col = ((long) blockIdx.x * per_block + tx) * V;
+	const bool live = tx < per_block && col < cols;
 	const int r0 = blockIdx.y * rows_per_slab, r1 = min(rows, r0 + rows_per_slab);
 	float acc[V];
 #pragma unroll
