@@ -135,6 +135,20 @@ public:
 	int no_previous_func() const { return (int) prev_func_.size(); }
 	CFunc *previous(int i) { return prev_func_[i]; }
 	virtual int sizeInBytes() const { return (int) input_.size_in_bytes(); }
+	// upstream's per-class operator== (impl/linear.h:135-151, impl/cinput.h:90-114 and the like): the same kind of function
+	// with the same uid, sizes and consumers; input functions also hold the same values
+	virtual bool operator==(const CFunc &rhs) const {
+		if (typeId() != rhs.typeId() || uid_ != rhs.uid_ || input_.length_ != rhs.input_.length_ || out_size_ != rhs.out_size_ ||
+				no_outputs() != rhs.no_outputs())
+			return false;
+		for (int i = 0; i < no_outputs(); ++i)
+			if (next(i)->uid_ != rhs.next(i)->uid_) return false;
+		if (is_input_)
+			for (int i = 0; i < input_.length_; ++i)
+				if (input_.real_[i] != rhs.input_.real_[i] || input_.imag_[i] != rhs.input_.imag_[i]) return false;
+		return true;
+	}
+	bool operator!=(const CFunc &rhs) const { return !(*this == rhs); }
 	virtual std::string getName() = 0;
 	virtual int typeId() const = 0;
 
@@ -358,6 +372,11 @@ public:
 	int noOutTokens() { return no_out_tokens_; }
 	std::string getName() override { return "Embedding " + std::to_string(uid_); }
 	int typeId() const override { return isEmbedding; }
+	bool operator==(const CFunc &rhs) const override {  // impl/embed.h:161-197: also the shape of the table and the token list
+		const CEmbedding *e = dynamic_cast<const CEmbedding *>(&rhs);
+		return e && CFunc::operator==(rhs) && embedding_dim_ == e->embedding_dim_ && no_embeddings_ == e->no_embeddings_ &&
+				no_out_tokens_ == e->no_out_tokens_ && tokens_ == e->tokens_;
+	}
 	void setInput(const std::vector<int> &list) {
 		tokens_.clear();
 		for (auto id : list) {

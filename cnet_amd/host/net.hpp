@@ -13,6 +13,7 @@ class CNet {
 	std::vector<CFunc *> inputs_, outputs_;
 	int next_uid_ = 0;
 	bool graph_ready_ = false;
+	std::vector<std::vector<CFunc *>> func_at_depth_;  // filled by init_exec_graph()
 
 	// device plan
 	int batch_ = 0;                   // 0: nothing allocated
@@ -465,12 +466,94 @@ public:
 			f->init_inputs();
 		}
 	}
+	// impl/cnet.h:156-198: the functions of every depth, within a depth by type (descending) and size (ascending); the
+	// executor here walks func_list_ (insertion order is a topological order), the lists serve callers that ask by depth
 	void init_exec_graph(bool print_status = false) {
 		graph_ready_ = true;
-		if (print_status) std::cout << toString();
+		int deepest = 0;
+		for (auto f : func_list_) deepest = std::max(deepest, f->depth());
+		func_at_depth_.assign(func_list_.empty() ? 0 : deepest + 1, std::vector<CFunc *>());
+		for (auto f : func_list_) {
+			if (!(f->isOutput() || f->no_outputs())) throw std::logic_error("init_exec_graph: " + f->getName() + " feeds nothing and is no output");
+			func_at_depth_[f->depth()].push_back(f);
+		}
+		for (auto &level : func_at_depth_)
+			std::stable_sort(level.begin(), level.end(), [](const CFunc *a, const CFunc *b) {
+				return a->typeId() == b->typeId() ? a->sizeInBytes() < b->sizeInBytes() : a->typeId() > b->typeId();
+			});
+		if (print_status)
+			for (size_t d = 0; d < func_at_depth_.size(); ++d) {
+				std::cout << "Depth " << d << ": ";
+				for (auto f : func_at_depth_[d]) std::cout << f->getName() << " " << f->sizeInBytes() << ", ";
+				std::cout << std::endl;
+			}
+	}
+	// ---- the small accessors of upstream's ComplexNet (impl/cnet.h:77-83, 201-226, 252-254, 312-357), which CNet::cpuNet()
+	//      hands out there; here the net and its device plan are one object ----
+	CNet &cpuNet() { return *this; }
+	int noClones() { return 0; }  // the batch is rows of one graph, not copies of it
+	int maxDepth() { return (int) func_at_depth_.size(); }  // 0 before init_exec_graph()
+	std::vector<CFunc *> &getFuncAtDepth(int depth) {
+		if (depth < 0 || depth >= maxDepth()) throw std::out_of_range("getFuncAtDepth: depth " + std::to_string(depth) + " of " + std::to_string(maxDepth()));
+		return func_at_depth_[depth];
+	}
+	void print_func_at_depth(int depth) {
+		if (maxDepth() == 0) {
+			std::cout << "init_exec_graph() not called yet." << std::endl;
+			return;
+		}
+		if (depth < 0 || depth >= maxDepth()) {
+			std::cout << "print_func_at_depth called with wrong depth: " << depth << std::endl;
+			return;
+		}
+		std::cout << func_at_depth_[depth].size() << " functions: ";
+		for (auto f : func_at_depth_[depth]) std::cout << f->getName() << ", ";
+		std::cout << std::endl;
+	}
+	unsigned long long getTotalSizeBytes() {  // six planes per function input, as one sample takes them
+		unsigned long long sum = 0;
+		for (auto f : func_list_) sum += f->sizeInBytes();
+		return sum;
+	}
+	int getNoVars() {
+		int sum = 0;
+		for (auto f : inputs_) sum += f->input().length_;
+		return sum;
+	}
+	void print_inputs() {
+		for (auto f : inputs_) {
+			std::cout << f->getName();
+			for (int i = 0; i < f->input().length_; ++i) std::cout << " " << f->input().z(i) << ",";
+			std::cout << std::endl;
+		}
+	}
+	CFunc *layer_at(int indx) {
+		if (indx < 0 || indx >= (int) func_list_.size()) throw std::out_of_range("layer_at: index " + std::to_string(indx));
+		return func_list_[indx];
+	}
+	CFunc *front() {
+		if (func_list_.empty()) throw std::logic_error("front: empty net");
+		return func_list_.front();
+	}
+	CFunc *back() {
+		if (func_list_.empty()) throw std::logic_error("back: empty net");
+		return func_list_.back();
+	}
+	// impl/cnet.h:437-484 (upstream asserts; here the first function that differs is named): same functions in the same
+	// order, each with the same uid, sizes and consumers, input functions with the same values
+	bool testEqual(CNet &other, std::string *why = NULL) {
+		auto differs = [&](const std::string &what) {
+			if (why) *why = what;
+			return false;
+		};
+		if (func_list_.size() != other.func_list_.size()) return differs("number of functions");
+		for (size_t k = 0; k < func_list_.size(); ++k)
+			if (*func_list_[k] != *other.func_list_[k]) return differs(func_list_[k]->getName());
+		return true;
 	}
 	std::string toString() {
 		std::ostringstream oss;
+		oss << func_list_.size() << " functions: " << " vars: " << getNoVars() << std::endl;
 		for (auto f : func_list_) {
 			oss << "depth: " << f->depth() << ": " << f->getName() << ": from C^" << f->input().length_ << " to C^" << f->out_size_;
 			for (int i = 0; i < f->no_outputs(); ++i) oss << " into " << f->next(i)->getName() << " at offset " << f->offset(i);
@@ -1984,7 +2067,12 @@ public:
 
 	// ---- per-sample API of upstream (CNet::forward / backward / updateInputs, gpu/gpu_func.h:1046-1056, 497-501):
 	//      host views are the state, the arithmetic runs on the device with a batch of one ----
-	void forward() {
+	void forward() { forwardOneSample(true); }
+	// ComplexNet::infer (impl/cnet.h:379-389): the forward pass alone, the gradients stay as they are
+	void infer() { forwardOneSample(false); }
+	// ComplexNet::update (impl/cnet.h:413-421): a step at learning_rate / batch_size that also clears the inputs' gradients
+	void update(float learning_rate, int batch_size) { updateInputs(learning_rate / batch_size); }
+	void forwardOneSample(bool clear_gradients) {
 		if (!batch_) allocateOnGpu(1);
 		if (batch_ != 1) throw std::logic_error("forward(): the per-sample API needs allocateOnGpu(1); use gpuForward for batches");
 		copyInputsToGpu();
@@ -1992,9 +2080,10 @@ public:
 		// never needs that (first contribution overwrites), the per-sample views do
 		materializeLazy();
 		flushPending();  // before the planes a deferred gradient sits in are cleared
-		for (auto f : func_list_)
-			if (!f->is_input_)
-				for (auto &s : f->slots_) ck(cnet_memset_zero(s.grad, 4 * (size_t) s.rows * s.len * sizeof(float)), "zero");
+		if (clear_gradients)
+			for (auto f : func_list_)
+				if (!f->is_input_)
+					for (auto &s : f->slots_) ck(cnet_memset_zero(s.grad, 4 * (size_t) s.rows * s.len * sizeof(float)), "zero");
 		lossGradientsStale();
 		per_sample_call_ = true;
 		try {

@@ -15,6 +15,7 @@
 //   facade_test real_batches       batches of real samples send their real plane only (same bits)
 //   facade_test upstream_nets      the nets of upstream's own GPU tests (E2E chain, fan-out into one consumer, ...)
 //   facade_test errors             error behaviour
+//   facade_test accessors          ComplexNet's small members (depth lists, sizes, testEqual), infer() and update()
 //   facade_test stack8 n blocks B steps lr rows overflow|finite [learn]   residual stack of `blocks` blocks against the
 //                                  oracle on `rows` rows of the batch (0: all rows, every step)
 #include <chrono>
@@ -420,6 +421,94 @@ static void test_persample() {
 		on.update(0.3f, 1);
 	}
 	expect("loss decreases under Wirtinger gradient descent (" + std::to_string(first) + " -> " + std::to_string(last) + ")", last < first);
+}
+
+// ------------------------------------------------------------------------------------------------- accessors
+// The small members of upstream's ComplexNet that code written against CNet::cpuNet() uses (impl/cnet.h:77-83, 201-226,
+// 252-254, 312-357, 379-389, 413-421, 437-484; tests/gputests.h:342, 1431): depth lists, sizes, layer_at / front / back,
+// testEqual, infer and update.
+static void test_accessors() {
+	const int n = 48, classes = 6;
+	orc::Rng rng(21);
+	std::vector<float> x(2 * n), hw(2 * n), w((size_t) 2 * n * classes);
+	fill_normal(rng, x.data(), x.size(), 1.0);
+	fill_normal(rng, hw.data(), hw.size(), 0.5);
+	fill_normal(rng, w.data(), w.size(), 0.2);
+	int ids[7];
+	auto build = [&](CNet &net) {
+		ids[0] = net.add(new CInput(OutSize(n)));
+		ids[1] = net.add(new FourierTrans(InSize(n)), {ids[0]});
+		ids[2] = net.add(new CInput(OutSize(n)));
+		ids[3] = net.add(new Hadamard(InSize(n), InSize(n)), {ids[1], ids[2]});
+		ids[4] = net.add(new CInput(OutSize(n * classes)));
+		ids[5] = net.add(new Linear(InSize(n), InSize(n * classes)), {ids[3], ids[4]});
+		ids[6] = net.add(new CrossEntropy(InSize(classes)), {ids[5]});
+		std::copy(x.begin(), x.end(), net[ids[0]]->mutable_input()->real_);
+		std::copy(hw.begin(), hw.end(), net[ids[2]]->mutable_input()->real_);
+		std::copy(w.begin(), w.end(), net[ids[4]]->mutable_input()->real_);
+	};
+	CNet net, twin;
+	build(net);
+	expect("maxDepth is 0 before init_exec_graph", net.maxDepth() == 0);
+	net.init_exec_graph(false);
+	build(twin);
+	twin.init_exec_graph(false);
+	// depths: inputs 0, transform 1, gate 2, Linear 3, loss 4
+	expect("maxDepth counts the levels", net.maxDepth() == 5);
+	bool levels = net.getFuncAtDepth(0).size() == 3 && net.getFuncAtDepth(1).size() == 1 && net.getFuncAtDepth(4).size() == 1 &&
+			net.getFuncAtDepth(4)[0] == net[ids[6]] && net.getFuncAtDepth(3)[0] == net[ids[5]];
+	// within a level by size: the two inputs of n values before the weights of the Linear
+	levels = levels && net.getFuncAtDepth(0)[2] == net[ids[4]] && net.getFuncAtDepth(0)[0]->input().length_ == n;
+	expect("getFuncAtDepth lists every level, smaller functions first", levels);
+	expect("getFuncAtDepth refuses a depth beyond the last", throws<std::out_of_range>([&] { net.getFuncAtDepth(5); }));
+	// function inputs: inputs of n, n and n * classes; transform n; gate 2n; Linear n + n * classes; loss classes, and its
+	// normalised output of as many again (impl/crossent.h sizeInBytes)
+	const unsigned long long values = 2ULL * n + (unsigned long long) n * classes + n + 2 * n + n + (unsigned long long) n * classes + 2 * classes;
+	expect("getTotalSizeBytes is six float planes per input value", net.getTotalSizeBytes() == 6ULL * sizeof(float) * values);
+	expect("getNoVars counts the values of the input functions", net.getNoVars() == 2 * n + n * classes);
+	expect("layer_at / front / back", net.layer_at(0) == net.front() && net.front() == net[ids[0]] && net.back() == net[ids[6]] &&
+			net.layer_at(5) == net[ids[5]] && throws<std::out_of_range>([&] { net.layer_at(7); }));
+	expect("cpuNet is the net itself, without clones", &net.cpuNet() == &net && net.noClones() == 0);
+	expect("toString starts with the counts", net.toString().rfind("7 functions:  vars: " + std::to_string(net.getNoVars()), 0) == 0);
+	std::string why;
+	expect("testEqual: two nets built alike", net.testEqual(twin, &why) && why.empty());
+	twin[ids[2]]->mutable_input()->imag_[7] += 1e-3f;
+	expect("testEqual names the input function whose values differ", !net.testEqual(twin, &why) && why == twin[ids[2]]->getName());
+	twin[ids[2]]->mutable_input()->imag_[7] = net[ids[2]]->input().imag_[7];
+	expect("testEqual: equal again", net.testEqual(twin));
+	CNet other;
+	other.add(new CInput(OutSize(n)));
+	expect("testEqual: another number of functions", !net.testEqual(other, &why) && why == "number of functions");
+
+	// infer() is forward() without the clearing of the gradients; update(rate, batch) is updateInputs(rate / batch)
+	const int label = 3;
+	net.forward();
+	net.backward(label);
+	twin.forward();
+	twin.backward(label);
+	const Vars &lin_in = net[ids[5]]->input();
+	std::vector<float> grads(lin_in.dz_real_, lin_in.dz_real_ + 4 * lin_in.length_), values_before(net[ids[6]]->input().real_, net[ids[6]]->input().real_ + 2 * classes);
+	double gnorm = 0;
+	for (float g : grads) gnorm += (double) g * g;
+	net.infer();
+	bool kept = gnorm > 0, same_values = true;
+	for (int k = 0; k < 4 * lin_in.length_; ++k) kept = kept && lin_in.dz_real_[k] == grads[k];
+	for (int k = 0; k < 2 * classes; ++k) same_values = same_values && net[ids[6]]->input().real_[k] == values_before[k];
+	expect("infer leaves the gradients of the functions alone", kept);
+	expect("infer gives the values of forward", same_values);
+	net.update(0.6f, 4);
+	twin.updateInputs(0.6f / 4);
+	bool same_step = true, moved = false;
+	for (int id : {ids[2], ids[4]})
+		for (int k = 0; k < 2 * net[id]->input().length_; ++k) {
+			same_step = same_step && net[id]->input().real_[k] == twin[id]->input().real_[k];
+			moved = moved || net[id]->input().real_[k] != (id == ids[2] ? hw[k] : w[k]);
+		}
+	expect("update(rate, batch) steps as updateInputs(rate / batch)", same_step && moved);
+	net.forward();
+	bool cleared = true;
+	for (int k = 0; k < 4 * lin_in.length_; ++k) cleared = cleared && lin_in.dz_real_[k] == 0.f;
+	expect("forward clears them", cleared);
 }
 
 // ------------------------------------------------------------------------------------------------- loss map, sampling
@@ -2023,6 +2112,7 @@ int main(int argc, char **argv) {
 		if (what == "token_model" || what == "all") test_token_model();
 		if (what == "adam" || what == "all") test_adam();
 		if (what == "loss_map" || what == "all") test_loss_map_and_sampling();
+		if (what == "accessors" || what == "all") test_accessors();
 		if (what == "saved_model") test_saved_model(argc > 2 ? argv[2] : "tests/golden", argc > 3 ? argv[3] : "/tmp");
 		if (what == "pipeline" || what == "all") test_pipeline(argc > 2 ? atoi(argv[2]) : 64, argc > 3 ? atoi(argv[3]) : 12);
 		if (what == "frozen_input" || what == "all") test_frozen_input();

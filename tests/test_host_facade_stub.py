@@ -12,7 +12,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SCENARIOS = ["mnist", "resblock", "persample", "loss_map", "embedding", "adam", "pipeline", "frozen_input", "deferred", "real_batches",
-             "upstream_nets", "three_products", "errors", "token_model"]
+             "upstream_nets", "three_products", "errors", "token_model", "accessors"]
 
 
 @pytest.fixture(scope="module")
