@@ -1327,24 +1327,34 @@ public:
 	bool copyInputsToGpu() {
 		requireAllocated("copyInputsToGpu");
 		for (auto f : inputs_) beforeFeed(f);  // first of all: work that was left out may still read weights that are replaced below
-		for (auto f : inputs_) {
-			f->z_imag_zero_ = false;
-			dataValuesWritten(f);
-			CFunc::Slot &s = f->slots_[0];
-			float *z = s.z;
-			if (s.rows == 1) {
-				ck(cnet_memcpy_h2d(z, f->mutable_input()->real_, 2 * (size_t) s.len * sizeof(float)), "cnet_memcpy_h2d");
-			} else {  // the data input: the host view holds one sample, replicate it to every row (one copy for both planes)
-				std::vector<float> rows(2 * (size_t) s.rows * s.len);
-				for (int b = 0; b < s.rows; ++b) {
-					std::copy(f->input().real_, f->input().real_ + s.len, rows.begin() + (size_t) b * s.len);
-					std::copy(f->input().imag_, f->input().imag_ + s.len, rows.begin() + (size_t) (s.rows + b) * s.len);
-				}
-				ck(cnet_memcpy_h2d(z, rows.data(), rows.size() * sizeof(float)), "cnet_memcpy_h2d");
-			}
-			if (f->typeId() == isEmbedding) uploadTokens((CEmbedding *) f, NULL);
-		}
+		for (auto f : inputs_) sendInputValues(f);
 		return true;
+	}
+	// upstream inputToGpu (gpu/gpu_func.h:470-487): the host values (or token list) of ONE input function to the device
+	bool inputToGpu(CFunc *input) {
+		requireAllocated("inputToGpu");
+		if (!input || !input->is_input_ || std::find(inputs_.begin(), inputs_.end(), input) == inputs_.end())
+			throw std::invalid_argument("inputToGpu: not an input function of this net");
+		for (auto f : inputs_) beforeFeed(f);
+		sendInputValues(input);
+		return true;
+	}
+	void sendInputValues(CFunc *f) {
+		f->z_imag_zero_ = false;
+		dataValuesWritten(f);
+		CFunc::Slot &s = f->slots_[0];
+		float *z = s.z;
+		if (s.rows == 1) {
+			ck(cnet_memcpy_h2d(z, f->mutable_input()->real_, 2 * (size_t) s.len * sizeof(float)), "cnet_memcpy_h2d");
+		} else {  // the data input: the host view holds one sample, replicate it to every row (one copy for both planes)
+			std::vector<float> rows(2 * (size_t) s.rows * s.len);
+			for (int b = 0; b < s.rows; ++b) {
+				std::copy(f->input().real_, f->input().real_ + s.len, rows.begin() + (size_t) b * s.len);
+				std::copy(f->input().imag_, f->input().imag_ + s.len, rows.begin() + (size_t) (s.rows + b) * s.len);
+			}
+			ck(cnet_memcpy_h2d(z, rows.data(), rows.size() * sizeof(float)), "cnet_memcpy_h2d");
+		}
+		if (f->typeId() == isEmbedding) uploadTokens((CEmbedding *) f, NULL);
 	}
 
 	bool getInputsFromGpu() {
@@ -1414,6 +1424,33 @@ public:
 	bool gpuForward(InputFunc *inp, OutputFunc *outp, InputBatch &batch) {
 		feedBatch(inp, outp, batch);
 		return GpuForward();
+	}
+	// The steps upstream's gpuForward / gpuBackward / allocateOnGpu are made of, under their names, for code that calls
+	// them one by one as upstream's GPU tests do (gpu/gpu_func.h:368-425, 532-541, 576-643): a batch and its labels to the
+	// device without the pass; the two copies between a function and its clones, of which there are none here; the
+	// allocation for `no_batches` samples side by side.
+	void batchToGpu(InputFunc *inp, OutputFunc *outp, Batch *batch) {
+		if (InputBatch *ib = dynamic_cast<InputBatch *>(batch)) {
+			feedBatch(inp, outp, *ib);
+		} else if (EmbeddingBatch *eb = dynamic_cast<EmbeddingBatch *>(batch)) {
+			feedTokens(inp, outp, *eb);
+		} else {
+			throw std::invalid_argument("batchToGpu: needs an InputBatch or an EmbeddingBatch");
+		}
+	}
+	void copyInputsToClones() {}
+	void updateGradientsFromClones() {}
+	std::string AllocateNet(int no_batches, bool &was_failure, bool print_graph = false) {
+		was_failure = true;
+		if (func_list_.empty()) return "AllocateNet error: 0 depth net.";
+		if (batch_) return "Net already initialised on GPU.";
+		if (print_graph) std::cout << toString();
+		try {
+			was_failure = !allocateOnGpu(no_batches);
+		} catch (const std::exception &e) {
+			return std::string("AllocateNet error: ") + e.what();
+		}
+		return was_failure ? "AllocateNet error" : "Allocated";
 	}
 	// forward + backward + update of one batch, replayed from ONE recorded graph: a step at small batch sizes is bound by
 	// the cost of launching ~20 kernels one by one, not by the kernels.  The first call with each buffer of the data input
@@ -1660,6 +1697,10 @@ public:
 		if (cin == main_input_) stage_[active_].imag_dev_zero = batch.imagIsZero();  // cleared or sent just now
 	}
 	bool gpuForward(InputFunc *inp, OutputFunc *outp, EmbeddingBatch &batch) {
+		feedTokens(inp, outp, batch);
+		return GpuForward();
+	}
+	void feedTokens(InputFunc *inp, OutputFunc *outp, EmbeddingBatch &batch) {
 		requireAllocated("gpuForward");
 		CEmbedding *emb = dynamic_cast<CEmbedding *>(inp);
 		if (!emb || emb != main_input_) throw std::invalid_argument("gpuForward: the EmbeddingBatch needs the main CEmbedding input");
@@ -1668,7 +1709,6 @@ public:
 		(void) outp;
 		uploadTokens(emb, batch.tokensPtr());
 		setLabels(batch.labelsPtr(), batch_);
-		return GpuForward();
 	}
 	bool GpuForward() {
 		requireAllocated("GpuForward");

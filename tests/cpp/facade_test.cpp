@@ -509,6 +509,58 @@ static void test_accessors() {
 	bool cleared = true;
 	for (int k = 0; k < 4 * lin_in.length_; ++k) cleared = cleared && lin_in.dz_real_[k] == 0.f;
 	expect("forward clears them", cleared);
+
+	// the steps of upstream's gpuForward under their own names (tests/gputests.h:50-71 pattern): AllocateNet, batchToGpu,
+	// copyInputsToClones, GpuForward(was_failure), ..., inputToGpu; against gpuForward on a twin
+	const int B = 4;
+	CNet one, two;
+	build(one);
+	build(two);
+	one.init_exec_graph(false);
+	two.init_exec_graph(false);
+	bool failed = false;
+	CNet empty;
+	expect("AllocateNet refuses an empty net by message", empty.AllocateNet(1, failed) == "AllocateNet error: 0 depth net." && failed);
+	one.AllocateNet(B, failed);
+	expect("AllocateNet allocates", !failed);
+	expect("AllocateNet refuses a second allocation by message", one.AllocateNet(B, failed) == "Net already initialised on GPU." && failed);
+	two.allocateOnGpu(B);
+	InputBatch batch(B, n);
+	std::vector<float> sample(2 * n);
+	for (int b = 0; b < B; ++b) {
+		fill_normal(rng, sample.data(), sample.size(), 1.0);
+		batch.add(sample.data(), sample.data() + n, n, b % classes);
+	}
+	CInput *in1 = (CInput *) one[ids[0]], *in2 = (CInput *) two[ids[0]];
+	CrossEntropy *ce1 = (CrossEntropy *) one[ids[6]], *ce2 = (CrossEntropy *) two[ids[6]];
+	one.copyInputsToClones();
+	one.batchToGpu(in1, ce1, &batch);
+	one.GpuForward(failed);
+	two.gpuForward(in2, ce2, batch);
+	expect("batchToGpu + GpuForward give the loss of gpuForward", !failed && one.getLoss(ce1, &batch) == two.getLoss(ce2, &batch));
+	one.GpuBackward(0, failed);
+	one.updateGradientsFromClones();
+	two.gpuBackward();
+	one.gpuUpdateInputs(0.1f);
+	two.gpuUpdateInputs(0.1f);
+	one.getInputsFromGpu();
+	two.getInputsFromGpu();
+	expect("... and the same weights after a step", !failed && one.testEqual(two, &why));
+	// inputToGpu sends one input function: new weights for the Linear change the loss, the gate's stay
+	for (int k = 0; k < 2 * n * classes; ++k) one[ids[4]]->mutable_input()->real_[k] = w[k];
+	one[ids[2]]->mutable_input()->real_[0] += 5.f;  // changed on the host only: not sent
+	one.inputToGpu(one[ids[4]]);
+	one.batchToGpu(in1, ce1, &batch);
+	one.GpuForward(failed);
+	CNet three;
+	build(three);
+	three.init_exec_graph(false);
+	three.allocateOnGpu(B);
+	for (int k = 0; k < 2 * n; ++k) three[ids[2]]->mutable_input()->real_[k] = two[ids[2]]->input().real_[k];
+	three.copyInputsToGpu();
+	three.gpuForward((CInput *) three[ids[0]], (CrossEntropy *) three[ids[6]], batch);
+	expect("inputToGpu sends the one input function it is given", one.getLoss(ce1, &batch) == three.getLoss((CrossEntropy *) three[ids[6]], &batch));
+	expect("inputToGpu refuses a function that is no input", throws<std::invalid_argument>([&] { one.inputToGpu(one[ids[5]]); }));
 }
 
 // ------------------------------------------------------------------------------------------------- loss map, sampling
