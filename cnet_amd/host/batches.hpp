@@ -302,6 +302,9 @@ public:
 	const float *imagDataPtr() const { return imag_data_; }
 	const float *realDataPtr(int b) const { return real_data_ + (size_t) b * sample_dim_; }
 	const float *imagDataPtr(int b) const { return imag_data_ + (size_t) b * sample_dim_; }
+	// one sample's planes as vectors (impl/batch.h:171-183)
+	std::vector<float> realData(int b) const { return std::vector<float>(realDataPtr(b), realDataPtr(b) + sample_dim_); }
+	std::vector<float> imagData(int b) const { return std::vector<float>(imagDataPtr(b), imagDataPtr(b) + sample_dim_); }
 };
 
 class EmbeddingBatch : public Batch {
@@ -321,6 +324,12 @@ public:
 		counter_ += (int) sample.size();
 	}
 	int noOfTokens() const { return (int) token_.size(); }
+	// impl/batch.h:112-122: tokens (padding aside) and labels folded into 0 .. mod - 1
+	void scale(int mod) {
+		for (auto &t : token_)
+			if (t >= 0) t %= mod;
+		for (auto &l : labels_) l %= mod;
+	}
 	const int *tokensPtr() const { return &token_[0]; }
 	int tokenCount() { return counter_; }
 };

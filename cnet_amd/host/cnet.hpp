@@ -29,6 +29,7 @@
 #include <cstring>
 #include <ctime>
 #include <initializer_list>
+#include <iomanip>
 #include <iostream>
 #include <map>
 #include <memory>

@@ -127,6 +127,8 @@ public:
 	Vars *mutable_input() { return &input_; }
 	const Vars &output() { assert(next_func_.size()); return next_func_[0]->input(); }
 	const Vars &output(int i) { return next_func_[i]->input(); }
+	Vars *mutable_output() { assert(next_func_.size()); return next_func_[0]->mutable_input(); }
+	Vars *mutable_output(int i) { assert(i >= 0 && i < (int) next_func_.size()); return next_func_[i]->mutable_input(); }
 	int uid() { return uid_; }
 	int depth() { return depth_; }
 	CFunc *next(int i) const { return next_func_[i]; }
@@ -159,6 +161,29 @@ public:
 			input_.real_[i] = re / input_.length_;
 			input_.imag_[i] = sqrt(1 - re * re) / input_.length_;
 		}
+	}
+	// the host view as text (impl/cfunc.h:158-209): values, values in rows of in_len, both gradients
+	virtual void printInput() {
+		std::cout << getName() << ": ";
+		for (int i = 0; i < input_.length_; ++i) std::cout << i << ": " << input_.z(i) << ", ";
+		std::cout << std::endl;
+	}
+	virtual void printInput2D(int in_len) { printInput2D(in_len, 0, input_.length_); }
+	virtual void printInput2D(int in_len, int offset, int len) {
+		assert(in_len > 0 && offset >= 0 && offset + len <= input_.length_);
+		std::cout << getName() << ": " << std::endl;
+		for (int i = 0; i < len; ++i) {
+			std::cout << (offset + i) << ": " << input_.z(offset + i) << ", ";
+			if (i % in_len == in_len - 1) std::cout << std::endl;
+		}
+		std::cout << std::endl;
+	}
+	virtual void printGradient() {
+		std::cout << getName() << ": ";
+		for (int i = 0; i < input_.length_; ++i) std::cout << i << "\tdz: " << input_.dz(i) << ", ";
+		std::cout << std::endl << getName() << ": ";
+		for (int i = 0; i < input_.length_; ++i) std::cout << i << "\tdz_star: " << input_.dz_star(i) << ", ";
+		std::cout << std::endl;
 	}
 	// impl/cfunc.h:211-224
 	void addOutput(CFunc *next, int offset) {
@@ -334,6 +359,10 @@ public:
 		return -std::log(v);
 	}
 	int get_prediction() { return prediction_; }
+	void printProbabilities() {  // impl/crossent.h:43-48
+		for (int k = 0; k < input().length_; ++k) std::cout << std::setprecision(9) << k << ": " << getProbability(k) << ", ";
+		std::cout << std::endl;
+	}
 	int sizeInBytes() const override { return (int) (input().size_in_bytes() + output_.size_in_bytes()); }
 	int outputLength() override { return output_.length_; }
 	Vars *mutableOutput() override { return &output_; }
@@ -386,6 +415,26 @@ public:
 		assert(tokens_.size() && (int) tokens_.size() <= no_out_tokens_);
 	}
 	void setInput(std::initializer_list<int> list) { setInput(std::vector<int>(list)); }
+	// impl/embed.h:56-74, 208-222: the table row by row, the token list, and both in short
+	void printEmbedding() {
+		for (int t = 0; t < no_embeddings_; ++t) {
+			std::cout << t << ":\t";
+			for (int i = 0; i < embedding_dim_; ++i) std::cout << input().z(t * embedding_dim_ + i) << ", ";
+			std::cout << std::endl;
+		}
+	}
+	void printTokens() {
+		std::cout << "Tokens:\t";
+		for (auto t : tokens_) std::cout << t << ", ";
+		std::cout << std::endl;
+	}
+	void printInput() override {
+		std::cout << getName() << " on CPU:\n\t tokens: ";
+		for (auto t : tokens_) std::cout << t << ",";
+		std::cout << std::endl << "\t embeddings: ";
+		for (int i = 0; i < std::min(16, input().length_); ++i) std::cout << i / embedding_dim_ << ": " << input().z(i) << ", ";
+		std::cout << std::endl;
+	}
 	void init_inputs() override {  // impl/embed.h:101-107
 		for (int i = 0; i < input().length_; ++i) {
 			float re = (float) rand_.randDouble() - 0.5;

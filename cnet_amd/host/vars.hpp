@@ -97,9 +97,22 @@ public:
 	std::complex<float> dz(int i) const { return std::complex<float>(dz_real_[i], dz_imag_[i]); }
 	std::complex<float> dz_star(int i) const { return std::complex<float>(dz_star_real_[i], dz_star_imag_[i]); }
 	void zSetValue(int i, std::complex<float> v) { real_[i] = v.real(); imag_[i] = v.imag(); }
+	void dzSetValue(int i, std::complex<float> v) { dz_real_[i] = v.real(); dz_imag_[i] = v.imag(); }
+	void dz_starSetValue(int i, std::complex<float> v) { dz_star_real_[i] = v.real(); dz_star_imag_[i] = v.imag(); }
+	void zero_dZ() { std::fill(dz_real_, dz_real_ + (size_t) length_ * 2, 0.0f); }
+	void zero_dZ_star() { std::fill(dz_star_real_, dz_star_real_ + (size_t) length_ * 2, 0.0f); }
+	// the first max_len values / gradients as text (impl/vars.h:123-145)
+	std::string zToString(int max_len) const { return listed(real_, max_len); }
+	std::string dzToString(int max_len) const { return listed(dz_real_, max_len); }
+	std::string dz_starToString(int max_len) const { return listed(dz_star_real_, max_len); }
 	unsigned long long size_in_bytes() const { return 6ULL * length_ * sizeof(float); }
 	float *plane(int p) { return real_ + (size_t) p * length_; }
 private:
+	std::string listed(const float *re, int max_len) const {  // re and the plane after it: one complex value per index
+		std::ostringstream oss;
+		for (int i = 0; i < std::min(length_, max_len); ++i) oss << std::complex<float>(re[i], re[length_ + i]) << ", ";
+		return oss.str();
+	}
 	void bind() {
 		imag_ = real_ + length_;
 		dz_real_ = imag_ + length_;
@@ -108,5 +121,13 @@ private:
 		dz_star_imag_ = dz_star_real_ + length_;
 	}
 };
+
+// impl/vars.h:165-177: sum of |z|^2 over the values, and its root
+inline float norm(const Vars &v) {
+	float sum = 0;
+	for (int i = 0; i < v.length_; ++i) sum += v.real_[i] * v.real_[i] + v.imag_[i] * v.imag_[i];
+	return sum;
+}
+inline float abs(const Vars &v) { return std::sqrt(norm(v)); }
 
 #endif  // CNET_AMD_HOST_VARS_HPP_

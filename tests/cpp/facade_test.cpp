@@ -510,6 +510,55 @@ static void test_accessors() {
 	for (int k = 0; k < 4 * lin_in.length_; ++k) cleared = cleared && lin_in.dz_real_[k] == 0.f;
 	expect("forward clears them", cleared);
 
+	// the host views as text and the small members of Vars and the batches (impl/vars.h:63-177, impl/cfunc.h:122-209,
+	// impl/crossent.h:43-48, impl/embed.h:56-74, impl/batch.h:112-122, 171-183)
+	{
+		Vars v(3);
+		v.zSetValue(0, {3.f, 4.f});
+		v.dzSetValue(1, {1.f, -2.f});
+		v.dz_starSetValue(2, {0.5f, 0.25f});
+		expect("Vars: setters reach their planes", v.dz(1) == std::complex<float>(1.f, -2.f) && v.dz_star(2) == std::complex<float>(0.5f, 0.25f));
+		expect("Vars: norm and abs of the values", norm(v) == 25.f && abs(v) == 5.f);
+		expect("Vars: values and gradients as text", v.zToString(2) == "(3,4), (0,0), " && v.dzToString(8) == "(0,0), (1,-2), (0,0), " &&
+				v.dz_starToString(3) == "(0,0), (0,0), (0.5,0.25), ");
+		v.zero_dZ();
+		expect("Vars: zero_dZ clears dz alone", v.dz(1) == std::complex<float>(0.f, 0.f) && v.dz_star(2) == std::complex<float>(0.5f, 0.25f));
+		v.zero_dZ_star();
+		expect("Vars: zero_dZ_star clears dz*", v.dz_star(2) == std::complex<float>(0.f, 0.f) && v.z(0) == std::complex<float>(3.f, 4.f));
+		std::ostringstream text;
+		std::streambuf *console = std::cout.rdbuf(text.rdbuf());
+		CFunc *lin = net[ids[5]];
+		lin->printInput2D(2, 0, 4);
+		net[ids[6]]->printGradient();
+		((CrossEntropy *) net[ids[6]])->printProbabilities();
+		CEmbedding table(2, 3, 4);
+		table.setInput({1, 3});
+		table.printTokens();
+		table.printEmbedding();
+		table.printInput();
+		std::cout.rdbuf(console);
+		const std::string out = text.str();
+		expect("printInput2D / printGradient / printProbabilities / printTokens / printEmbedding write the host views",
+				out.find(lin->getName() + ": \n0: ") == 0 && out.find("\tdz_star: ") != std::string::npos && out.find("Tokens:\t1, 3, ") != std::string::npos &&
+						out.find("3:\t(0,0), (0,0), ") != std::string::npos && out.find(" on CPU:") != std::string::npos &&
+						out.find(std::to_string(classes - 1) + ": ") != std::string::npos);
+		expect("mutable_output is the consumer's input", net[ids[5]]->mutable_output() == net[ids[6]]->mutable_input() &&
+				net[ids[1]]->mutable_output(0) == net[ids[3]]->mutable_input());
+		EmbeddingBatch tokens(2, 3);
+		tokens.add({7, 12}, 9);
+		tokens.add({5, 6, 11}, 4);
+		tokens.scale(5);
+		const int want[6] = {2, 2, NO_TOKEN, 0, 1, 1};
+		bool scaled = tokens.labelsPtr()[0] == 4 && tokens.labelsPtr()[1] == 4;
+		for (int k = 0; k < 6; ++k) scaled = scaled && tokens.tokensPtr()[k] == want[k];
+		expect("EmbeddingBatch::scale folds tokens and labels, not the padding", scaled);
+		InputBatch two_samples(2, 3);
+		two_samples.add({{1.f, 2.f}, {3.f, 4.f}, {5.f, 6.f}}, 0);
+		two_samples.add({{7.f, 8.f}, {9.f, 10.f}, {11.f, 12.f}}, 1);
+		expect("InputBatch::realData / imagData of one sample", two_samples.realData(1) == std::vector<float>({7.f, 9.f, 11.f}) &&
+				two_samples.imagData(0) == std::vector<float>({2.f, 4.f, 6.f}));
+	}
+
 	// the steps of upstream's gpuForward under their own names (tests/gputests.h:50-71 pattern): AllocateNet, batchToGpu,
 	// copyInputsToClones, GpuForward(was_failure), ..., inputToGpu; against gpuForward on a twin
 	const int B = 4;
