@@ -1438,7 +1438,14 @@ bool plan_skinny(bool a_mcontig, bool b_ncontig, const CgemmArgs &proto, int npr
 		const long splits = std::min<long>(2 * cus / tiles, groups / 16);
 		if (splits < 2 || (long) batch * splits > 65535) return false;
 		args.chunks_per_split = (int) ((groups + splits - 1) / splits);
-		if (args.chunks_per_split > 64) return false;  // still longer than 1024 per slice: the block kernels do better
+		if (args.chunks_per_split > 64) {
+			// still longer than 1024 per slice: the block kernels do better, unless C is so small (the weight gradient of a
+			// 784 -> 10 layer over a batch of 16384: 49 tiles) that they would run a handful of blocks; then slices of 1024,
+			// several workgroups to a compute unit (16384 x 784 x 10: 90 -> 25 us)
+			const long more = (groups + 63) / 64;
+			if (2 * tiles > cus || more > 128 || (long) batch * more > 65535) return false;
+			args.chunks_per_split = (int) ((groups + more - 1) / more);
+		}
 		args.splits = (groups + args.chunks_per_split - 1) / args.chunks_per_split;  // no empty slice
 	}
 	return true;

@@ -62,12 +62,13 @@ def test_linear_cgelu_into_a_column_window(gpu, port):
 
 @pytest.mark.parametrize("B,K,N", [(64, 784, 10), (64, 16, 16), (33, 7, 5), (16, 64, 12), (1, 3, 2), (200, 40, 24), (64, 784, 784),
                                    (1024, 256, 256), (4096, 784, 10), (1000, 100, 16), (300, 5, 1), (256, 1030, 3), (513, 260, 7),
-                                   (257, 33, 12)])
+                                   (257, 33, 12), (16384, 784, 10)])
 def test_both_gradients_of_a_linear_in_one_call(gpu, port, B, K, N):
     """cnet_clinear_bwd_sym against cnet_clinear_bwd_input_sym + cnet_clinear_bwd_weight_sym: same bits, whether the two
     products share a launch (both small and on the same kernel: the first cases) or not, with each accumulate flag and with
     the dz* planes of either result left out.  The cases from (4096, 784, 10) on are narrow layers (few outputs) at batches
-    beyond the small-C kernel: a K of 1 .. 16 for the input gradient, a reduction over the whole batch for the weights."""
+    beyond the small-C kernel: a K of 1 .. 16 for the input gradient, a reduction over the whole batch for the weights (at
+    16384 rows in slices of 1024, more than two workgroups to a compute unit)."""
     gr, gi = seeded(port, B + 11, (B, N)), seeded(port, B + 12, (B, N))
     g = ops.Grad.from_host([gr, gi, gr, -gi])
     x = ops.CMat.from_host(seeded(port, K + 1, (B, K)), seeded(port, K + 2, (B, K)))
@@ -81,7 +82,7 @@ def test_both_gradients_of_a_linear_in_one_call(gpu, port, B, K, N):
         for a, b in ((dx0, dx1), (dw0, dw1)):
             for pa, pb in zip(a.host(), b.host()):
                 assert np.array_equal(pa, pb), (acc_x, acc_w, mir_x, mir_w)
-    if B * K * N <= 1 << 26:   # the CPU path on the same pair
+    if B * K * N <= 1 << 27:   # the CPU path on the same pair
         (xr, xi), (wr, wi) = x.host(), w.host()
         dxo, dwo = port.linear_bwd(xr, xi, wr, wi, [gr, gi, gr, -gi])
         dx1, dw1 = ops.Grad.empty(B, K), ops.Grad.empty(N, K)
