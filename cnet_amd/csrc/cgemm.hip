@@ -1577,13 +1577,20 @@ inline bool three_products() {
 // is open, so cnet_graph_begin has all of them made beforehand (cgemm_prime_attributes) and launch() skips its own.
 bool g_attrs_primed = false;
 
-template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
+// STAGES: LDS stages of the fast kernel; 0 = three, two for the 128 x 128 block (whose two stages fill the LDS of two
+// workgroups per compute unit).  The 64 x 64 block also runs with two: four workgroups to a unit instead of three.
+template <int BM, int BN, int STAGES>
+constexpr int fast_stages() {
+	return STAGES ? STAGES : (BM == 128 && BN == 128) ? 2 : 3;
+}
+
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC, int STAGES = 0>
 hipError_t prime_attributes() {
 	constexpr size_t smem = 2 * (size_t) (2 * KC * (BM + 4) + 2 * KC * (BN + 4)) * sizeof(float);
 	hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, VEC>),
 			hipFuncAttributeMaxDynamicSharedMemorySize, (int) smem);
 	if constexpr (VEC == 4) {
-		constexpr int NST = (BM == 128 && BN == 128) ? 2 : 3;
+		constexpr int NST = fast_stages<BM, BN, STAGES>();
 		constexpr size_t fast_smem = (size_t) NST * 2 * KC * (BM + BN) * sizeof(float);
 		if (e == hipSuccess)
 			e = hipFuncSetAttribute(reinterpret_cast<const void *>(&cgemm_fast_kernel<BM, BN, WM, WN, A_MCONTIG, B_NCONTIG, NST>),
@@ -1613,11 +1620,12 @@ hipError_t prime_shapes() {
 		if (e == hipSuccess) e = prime_attributes<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>();
 		if (e == hipSuccess) e = prime_attributes<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>();
 		if (e == hipSuccess) e = prime_attributes<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>();
+		if (e == hipSuccess) e = prime_attributes<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC, 2>();
 	}
 	return e;
 }
 
-template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC>
+template <int BM, int BN, int WM, int WN, bool A_MCONTIG, bool B_NCONTIG, int VEC, int STAGES = 0>
 int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, int k_cuts = -1) {
 	CgemmArgs args = proto;
 	args.tiles_m = (args.M + BM - 1) / BM;
@@ -1687,7 +1695,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 	};
 	if constexpr (VEC == 4) {
 		if (fast_ok) {  // any M and N: edge blocks re-read the last valid rows and store only what is inside C
-			constexpr int NST = (BM == 128 && BN == 128) ? 2 : 3;
+			constexpr int NST = fast_stages<BM, BN, STAGES>();
 			constexpr size_t fast_smem = (size_t) NST * 2 * KC * (BM + BN) * sizeof(float);
 			if constexpr (!A_MCONTIG && B_NCONTIG) {
 				if (args.a_real == 2) {
@@ -1756,7 +1764,7 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 	return finish();
 }
 
-// Block shape for the fast kernel (0: 128 x 128, 1: 64 x 128, 2: 128 x 64, 3: 64 x 64), whether the blocks of a partly
+// Block shape for the fast kernel (0: 128 x 128, 1: 64 x 128, 2: 128 x 64, 3: 64 x 64, 4: 64 x 64 with two LDS stages), whether the blocks of a partly
 // filled last round are cut along K (*tail = number of pieces, 0 = no), and the expected duration of the launch in us.
 // k_contig_operands: both operands are stored with k contiguous (the one layout whose 128 x 128 kernel has no
 // three-product form).
@@ -1767,7 +1775,7 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_opera
 		if (a.tri) tn = (tn + 1) / 2;  // one workgroup per mirrored pair of column blocks
 		return (long) ((a.M + bm - 1) / bm) * tn * nprob * batch;
 	};
-	// tuning override: CNET_CGEMM_TILE = 0 (128x128), 1 (64x128), 2 (128x64), 3 (64x64)
+	// tuning override: CNET_CGEMM_TILE = 0 (128x128), 1 (64x128), 2 (128x64), 3 (64x64), 4 (64x64, two LDS stages)
 	static const int forced = [] {
 		const char *e = getenv("CNET_CGEMM_TILE");
 		return e ? atoi(e) : -1;
@@ -1793,7 +1801,7 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_opera
 		int bm, bn;
 		float eff_k512[8], eff_k2048[8];  // p = 1 .. 8 (8 stands for everything above)
 	};
-	static const Shape shapes[4] = {
+	static const Shape shapes[5] = {
 			{128, 128, {0.834f, 0.911f, 0.743f, 0.918f, 0.777f, 0.917f, 0.785f, 0.918f},
 					{0.887f, 0.946f, 0.713f, 0.941f, 0.794f, 0.946f, 0.800f, 0.948f}},
 			{64, 128, {0.786f, 0.868f, 0.876f, 0.890f, 0.894f, 0.899f, 0.901f, 0.903f},
@@ -1801,7 +1809,11 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_opera
 			{128, 64, {0.786f, 0.861f, 0.883f, 0.888f, 0.898f, 0.900f, 0.902f, 0.905f},
 					{0.892f, 0.940f, 0.936f, 0.945f, 0.945f, 0.948f, 0.949f, 0.950f}},
 			{64, 64, {0.768f, 0.840f, 0.873f, 0.723f, 0.884f, 0.866f, 0.870f, 0.874f},
-					{0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}}};
+					{0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}},
+			// 64 x 64 with two LDS stages (four workgroups to a unit: the uneven round is the fifth, not the fourth)
+			// (beyond seven per unit the layout with both operands K-contiguous falls off: .84 - .93 where the others hold .96)
+			{64, 64, {0.746f, 0.828f, 0.856f, 0.866f, 0.749f, 0.891f, 0.901f, 0.839f},
+					{0.869f, 0.929f, 0.941f, 0.947f, 0.801f, 0.945f, 0.960f, 0.875f}}};
 	static const bool k_dependent = [] {
 		const char *e = getenv("CNET_CGEMM_KMODEL");  // tuning override: 0 uses the K = 2048 table for every K
 		return !e || atoi(e) != 0;
@@ -1823,8 +1835,9 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_opera
 	const bool tail_possible = forced_tail != 0 && a.K % KC == 0 && !a.tri && batch == 1;
 	int best = 3, best_tail = 0, best_cuts = 1;
 	double best_us = 1e30;
-	for (int k = 0; k < 4; ++k) {
+	for (int k = 0; k < 5; ++k) {
 		if (forced >= 0 && forced != k) continue;
+		if (k == 4 && (forced != 4 && a.K % KC != 0)) continue;  // only the fast kernel has the two-stage form: shape 3 there
 		const long nb = blocks(shapes[k].bm, shapes[k].bn);
 		const long per_unit = (nb + cus - 1) / cus;
 		// three real products per complex one in the shapes that have the registers for it (fast kernel only: K in whole chunks)
@@ -1896,6 +1909,7 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 		if (best == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
 		if (best == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
 		if (best == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
+		if (best == 4) return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC, 2>(a, nprob, batch, best_tail, cuts);
 		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
 	}
 }

@@ -523,7 +523,8 @@ int cnet_embedding_bwd(const int32_t *tokens, const float *g_dzs_re, const float
  *      measured with; they exist so that tests and sweeps can send a shape to every kernel that could take it.  Each is
  *      read ONCE per process, when the first launch that consults it is queued; results do not depend on them beyond
  *      rounding (another block shape or cut groups the sums differently), and every path they select is deterministic.
- *   CNET_CGEMM_TILE = 0..3       block shape of the matrix kernels: 128x128, 64x128, 128x64, 64x64 (default: cost model)
+ *   CNET_CGEMM_TILE = 0..4       block shape of the matrix kernels: 128x128, 64x128, 128x64, 64x64, 64x64 with two LDS
+ *                                stages (default: cost model)
  *   CNET_CGEMM_TAIL = 0 | 1      never / whenever possible cut the blocks of a partly filled last round along K
  *   CNET_CGEMM_KCUT = 0          cut a product along K only when half of the compute units would idle
  *   CNET_CGEMM_KMODEL = 0        price every K with the efficiency table measured at K = 2048

@@ -292,6 +292,7 @@ def test_matrix_products_of_a_conjugate_pair_without_the_mirror_planes(gpu, port
     {"CNET_CGEMM_SKINNY": "0"},                            # small products on the block kernels (cut along K)
     {"CNET_CGEMM_TILE": "0", "CNET_CGEMM_COLSPLIT": "0"},  # 128 x 128 blocks (two accumulator sets, negated operand)
     {"CNET_CGEMM_TILE": "3", "CNET_CGEMM_TAIL": "1"},      # 64 x 64 blocks, tail blocks cut along K whenever possible
+    {"CNET_CGEMM_TILE": "4"},                              # 64 x 64 blocks with two LDS stages
 ])
 def test_conjugate_pairs_under_other_kernel_choices(gpu, overrides):
     """The tests of this file again, in a process whose tuning overrides (read once per process) send the same shapes to

@@ -138,11 +138,11 @@ def test_transform_of_real_samples_through_half_the_columns(gpu, port, B, n):
     # from three real ones (CNET_CGEMM_3M=1: 1.6e-6 from double precision at n = 4096), which the transform of real samples
     # never does
     assert rel_c((hr, hi), (fr, fi)) < (2e-6 if capi.load().cnet_cgemm_get_products() == 4 else 3e-6)
-    if B * n <= 1 << 22:   # against double precision: no worse than the full product
+    if B * n <= 1 << 22:   # against double precision: about as close as the full product (either may be cut along K, which shortens its sums)
         ref = np.fft.fft(xr.astype(np.float64), axis=1) / np.sqrt(n)
         def err(re, im):
             return np.linalg.norm((re.astype(np.float64) + 1j * im.astype(np.float64)) - ref) / np.linalg.norm(ref)
-        assert err(hr, hi) < max(1.2 * err(fr, fi), 2e-7), (err(hr, hi), err(fr, fi))
+        assert err(hr, hi) < max(1.5 * err(fr, fi), 2e-7), (err(hr, hi), err(fr, fi))
         if n % 2 == 0:   # column n/2 alone: the alternating sum of the samples, a real number
             assert np.abs(hr[:, n // 2] - ref[:, n // 2].real).max() < 2e-6 * np.abs(xr).sum(axis=1).max() / np.sqrt(n)
             assert np.abs(hi[:, n // 2]).max() < 2e-6 * np.abs(xr).sum(axis=1).max() / np.sqrt(n)
@@ -179,3 +179,22 @@ def test_folded_transform_of_real_samples_in_windows_of_wider_buffers(gpu, port,
     assert np.abs(got[:, n // 2] - ref[:, n // 2]).max() < 1e-5
     mask = np.ones(n + 24, bool); mask[12:12 + n] = False
     assert np.array_equal(gr[:, mask], yb_re[:, mask]) and np.array_equal(gi[:, mask], yb_im[:, mask])
+
+
+@pytest.mark.parametrize("overrides", [
+    {"CNET_CGEMM_TILE": "4"},                          # 64 x 64 blocks with two LDS stages: full, real-operand and folded forms
+    {"CNET_CGEMM_TILE": "4", "CNET_CGEMM_3M": "1"},    # and three real products per complex one
+    {"CNET_CGEMM_TILE": "0", "CNET_DFT_FOLD": "0"},    # 128 x 128 blocks, the transform of real samples unfolded
+])
+def test_transforms_under_other_kernel_choices(gpu, overrides):
+    """The tests of this file again in a process whose tuning overrides (read once per process) send the transforms to other
+    block shapes and forms of the product."""
+    import os
+    import subprocess
+    import sys
+    if os.environ.get("CNET_TEST_INNER"):
+        pytest.skip("already the inner run")
+    env = dict(os.environ, CNET_TEST_INNER="1", **overrides)
+    r = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-m", "gpu"], env=env,
+                       capture_output=True, text=True, timeout=280, cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-2000:]

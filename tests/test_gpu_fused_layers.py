@@ -128,6 +128,7 @@ def test_backward_pass_of_a_narrow_linear_in_windows_of_wider_buffers(gpu):
     {"CNET_CGEMM_SKINNY": "0"},                            # small products on the block kernels (cut along K)
     {"CNET_CGEMM_TILE": "0", "CNET_CGEMM_COLSPLIT": "0"},  # 128 x 128 blocks
     {"CNET_CGEMM_TILE": "3", "CNET_CGEMM_TAIL": "1"},      # 64 x 64 blocks, tail blocks cut along K whenever possible
+    {"CNET_CGEMM_TILE": "4", "CNET_CGEMM_TAIL": "1"},      # the same blocks with two LDS stages
     {"CNET_CGEMM_SKINNY_W": "16"},                         # sixteen wavefronts per tile of the small-C kernel (1024 threads a workgroup)
 ])
 def test_fused_layers_under_other_kernel_choices(gpu, overrides):

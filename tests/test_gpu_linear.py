@@ -263,10 +263,11 @@ def test_cgemm_random_shapes(gpu, port):
         assert np.array_equal(got[:, N:], c0[:, N:]), (case, "columns beside C were touched")
 
 
-@pytest.mark.parametrize("tile", ["0", "1", "2", "3", ""])
+@pytest.mark.parametrize("tile", ["0", "1", "2", "3", "4", ""])
 def test_cgemm_tail_blocks_cut_along_k(gpu, tile):
     """Products whose blocks do not fill a whole number of rounds over the compute units, with the cut of the last round's
-    blocks along K switched on for every such launch and each block shape in turn (and the library's own choice)."""
+    blocks along K switched on for every such launch and each block shape in turn (4: the 64 x 64 block with two LDS stages; and
+    the library's own choice)."""
     import os
     import subprocess
     import sys
