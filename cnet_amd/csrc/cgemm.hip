@@ -1766,9 +1766,12 @@ int launch(const CgemmArgs &proto, int nprob, int batch, int tail_splits = 0, in
 
 // Block shape for the fast kernel (0: 128 x 128, 1: 64 x 128, 2: 128 x 64, 3: 64 x 64, 4: 64 x 64 with two LDS stages), whether the blocks of a partly
 // filled last round are cut along K (*tail = number of pieces, 0 = no), and the expected duration of the launch in us.
-// k_contig_operands: both operands are stored with k contiguous (the one layout whose 128 x 128 kernel has no
-// three-product form).
-double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_operands, int *shape, int *tail_pieces, int *k_cuts) {
+// layout (block_layout): 0 = A row-major and B k-major, 1 = both operands with k contiguous (the one layout whose
+// 128 x 128 kernel has no three-product form), 2 = both with their rows contiguous (and the fourth combination).
+inline int block_layout(bool a_mcontig, bool b_ncontig) {
+	return (!a_mcontig && b_ncontig) ? 0 : (!a_mcontig && !b_ncontig) ? 1 : 2;
+}
+double plan_blocks(const CgemmArgs &a, int nprob, int batch, int layout, int *shape, int *tail_pieces, int *k_cuts) {
 	const long cus = cnet::rt().prop.multiProcessorCount;
 	auto blocks = [&](int bm, int bn) {
 		long tn = (a.N + bn - 1) / bn;
@@ -1788,44 +1791,96 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_opera
 	// Expected duration of the launch with each block shape.  The busiest compute unit works through p = ceil(blocks /
 	// units) blocks, so the launch takes p block-times, whether or not all units have that many and whether or not a
 	// block on the edge of C is full, divided by the efficiency measured for the shape at p blocks per unit on full
-	// blocks (fraction of the fp32 MFMA peak, lowest of three operand layouts), at K = 512 and at K = 2048; in between
-	// and below, 1 / efficiency is taken as linear in 1 / K (a loop part and a fixed part per block: first loads and
-	// the write-out of C weigh more on a short K, and more on the small shapes).  The tables carry what a formula would
-	// miss: a unit holds two workgroups of the larger shapes and three of 64 x 64, a lone workgroup cannot keep the
-	// matrix pipe busy, and with 3 or 5 blocks of 128 x 128 per unit, or 4 of 64 x 64, the hardware dispatcher leaves
-	// some units with one block more than the others.
+	// blocks (fraction of the fp32 MFMA peak on operands of random values; the layout with both operands K-contiguous has
+	// tables of its own), at K = 512, 1024 and 2048; in between and below, 1 / efficiency follows a broken line in 1 / K (a
+	// loop part and a fixed part per block: first loads and the write-out of C weigh more on a short K, and more on the
+	// small shapes).  The tables carry what a formula would miss: a unit holds two workgroups of the larger shapes, three
+	// of 64 x 64 and four of 64 x 64 with two LDS stages, a lone workgroup cannot keep the matrix pipe busy, and with 3 or 5
+	// blocks of 128 x 128 per unit, 4 of 64 x 64 or 5 of its two-stage form, the hardware dispatcher leaves some units with
+	// one block more than the others.
 	// Alternative for a partly filled last round (q full rounds, r blocks left over): cut those r blocks into s pieces
 	// along K, one piece for each workgroup of the full rounds.  Then the launch takes q block-times plus 1/s of one,
 	// plus the fixed cost of a short piece and of the kernel that adds the pieces.
 	struct Shape {
 		int bm, bn;
-		float eff_k512[8], eff_k2048[8];  // p = 1 .. 8 (8 stands for everything above)
+		// [layout: 0 A row-major and B k-major, 1 both K-contiguous, 2 both with their rows contiguous][K = 512, 1024, 2048]
+		// [p = 1 .. 8 (8 stands for everything above)], operands of random values
+		float eff[3][3][8];
 	};
 	static const Shape shapes[5] = {
-			{128, 128, {0.834f, 0.911f, 0.743f, 0.918f, 0.777f, 0.917f, 0.785f, 0.918f},
-					{0.887f, 0.946f, 0.713f, 0.941f, 0.794f, 0.946f, 0.800f, 0.948f}},
-			{64, 128, {0.786f, 0.868f, 0.876f, 0.890f, 0.894f, 0.899f, 0.901f, 0.903f},
-					{0.883f, 0.935f, 0.931f, 0.943f, 0.938f, 0.943f, 0.943f, 0.944f}},
-			{128, 64, {0.786f, 0.861f, 0.883f, 0.888f, 0.898f, 0.900f, 0.902f, 0.905f},
-					{0.892f, 0.940f, 0.936f, 0.945f, 0.945f, 0.948f, 0.949f, 0.950f}},
-			{64, 64, {0.768f, 0.840f, 0.873f, 0.723f, 0.884f, 0.866f, 0.870f, 0.874f},
-					{0.882f, 0.933f, 0.946f, 0.769f, 0.956f, 0.900f, 0.950f, 0.945f}},
-			// 64 x 64 with two LDS stages (four workgroups to a unit: the uneven round is the fifth, not the fourth)
-			// (beyond seven per unit the layout with both operands K-contiguous falls off: .84 - .93 where the others hold .96)
-			{64, 64, {0.746f, 0.828f, 0.856f, 0.866f, 0.749f, 0.891f, 0.901f, 0.839f},
-					{0.869f, 0.929f, 0.941f, 0.947f, 0.801f, 0.945f, 0.960f, 0.875f}}};
+			{128, 128,
+					{{{0.808f, 0.897f, 0.686f, 0.903f, 0.760f, 0.902f, 0.796f, 0.905f},
+							{0.848f, 0.922f, 0.702f, 0.925f, 0.778f, 0.923f, 0.814f, 0.924f},
+							{0.873f, 0.936f, 0.707f, 0.934f, 0.782f, 0.937f, 0.822f, 0.936f}},
+					{{0.821f, 0.899f, 0.689f, 0.907f, 0.763f, 0.908f, 0.806f, 0.909f},
+							{0.864f, 0.928f, 0.912f, 0.932f, 0.921f, 0.931f, 0.901f, 0.930f},
+							{0.892f, 0.943f, 0.933f, 0.946f, 0.939f, 0.947f, 0.944f, 0.947f}},
+					{{0.815f, 0.897f, 0.686f, 0.906f, 0.763f, 0.907f, 0.799f, 0.908f},
+							{0.856f, 0.927f, 0.702f, 0.929f, 0.783f, 0.929f, 0.819f, 0.931f},
+							{0.881f, 0.943f, 0.710f, 0.944f, 0.791f, 0.945f, 0.828f, 0.946f}}}},
+			{64, 128,
+					{{{0.775f, 0.864f, 0.857f, 0.879f, 0.873f, 0.883f, 0.881f, 0.887f},
+							{0.842f, 0.904f, 0.897f, 0.912f, 0.909f, 0.915f, 0.913f, 0.917f},
+							{0.875f, 0.924f, 0.917f, 0.929f, 0.927f, 0.931f, 0.930f, 0.933f}},
+					{{0.794f, 0.858f, 0.867f, 0.879f, 0.879f, 0.886f, 0.887f, 0.891f},
+							{0.865f, 0.903f, 0.910f, 0.915f, 0.918f, 0.920f, 0.921f, 0.922f},
+							{0.903f, 0.930f, 0.936f, 0.940f, 0.942f, 0.943f, 0.944f, 0.945f}},
+					{{0.780f, 0.870f, 0.865f, 0.884f, 0.879f, 0.888f, 0.887f, 0.891f},
+							{0.846f, 0.907f, 0.904f, 0.917f, 0.915f, 0.920f, 0.920f, 0.922f},
+							{0.879f, 0.931f, 0.927f, 0.936f, 0.936f, 0.938f, 0.939f, 0.940f}}}},
+			{128, 64,
+					{{{0.792f, 0.862f, 0.866f, 0.881f, 0.879f, 0.885f, 0.884f, 0.888f},
+							{0.857f, 0.906f, 0.913f, 0.918f, 0.921f, 0.921f, 0.921f, 0.921f},
+							{0.894f, 0.932f, 0.937f, 0.939f, 0.939f, 0.942f, 0.941f, 0.943f}},
+					{{0.795f, 0.859f, 0.863f, 0.878f, 0.876f, 0.883f, 0.882f, 0.887f},
+							{0.862f, 0.903f, 0.911f, 0.916f, 0.918f, 0.918f, 0.918f, 0.919f},
+							{0.898f, 0.928f, 0.935f, 0.939f, 0.941f, 0.943f, 0.942f, 0.942f}},
+					{{0.781f, 0.865f, 0.861f, 0.880f, 0.877f, 0.883f, 0.882f, 0.885f},
+							{0.846f, 0.906f, 0.902f, 0.917f, 0.913f, 0.917f, 0.917f, 0.918f},
+							{0.881f, 0.927f, 0.923f, 0.932f, 0.932f, 0.936f, 0.936f, 0.936f}}}},
+			{64, 64,
+					{{{0.756f, 0.833f, 0.868f, 0.713f, 0.880f, 0.887f, 0.888f, 0.894f},
+							{0.835f, 0.891f, 0.914f, 0.743f, 0.923f, 0.925f, 0.925f, 0.926f},
+							{0.880f, 0.919f, 0.936f, 0.758f, 0.942f, 0.942f, 0.946f, 0.949f}},
+					{{0.764f, 0.831f, 0.867f, 0.711f, 0.880f, 0.884f, 0.886f, 0.888f},
+							{0.850f, 0.894f, 0.913f, 0.744f, 0.923f, 0.921f, 0.924f, 0.923f},
+							{0.899f, 0.929f, 0.941f, 0.761f, 0.945f, 0.946f, 0.947f, 0.950f}},
+					{{0.752f, 0.829f, 0.866f, 0.712f, 0.880f, 0.886f, 0.888f, 0.891f},
+							{0.834f, 0.886f, 0.912f, 0.744f, 0.921f, 0.921f, 0.925f, 0.928f},
+							{0.878f, 0.921f, 0.934f, 0.761f, 0.943f, 0.945f, 0.949f, 0.948f}}}},
+			{64, 64,
+					{{{0.767f, 0.843f, 0.873f, 0.889f, 0.756f, 0.902f, 0.905f, 0.909f},
+							{0.846f, 0.899f, 0.917f, 0.924f, 0.785f, 0.933f, 0.935f, 0.934f},
+							{0.890f, 0.926f, 0.939f, 0.944f, 0.798f, 0.950f, 0.951f, 0.948f}},
+					{{0.770f, 0.845f, 0.866f, 0.888f, 0.754f, 0.894f, 0.896f, 0.873f},
+							{0.852f, 0.900f, 0.915f, 0.924f, 0.784f, 0.928f, 0.934f, 0.875f},
+							{0.901f, 0.929f, 0.939f, 0.948f, 0.798f, 0.939f, 0.951f, 0.888f}},
+					{{0.754f, 0.839f, 0.870f, 0.886f, 0.754f, 0.900f, 0.904f, 0.904f},
+							{0.834f, 0.894f, 0.914f, 0.923f, 0.784f, 0.930f, 0.933f, 0.932f},
+							{0.878f, 0.921f, 0.934f, 0.944f, 0.797f, 0.951f, 0.951f, 0.950f}}}}};
 	static const bool k_dependent = [] {
 		const char *e = getenv("CNET_CGEMM_KMODEL");  // tuning override: 0 uses the K = 2048 table for every K
 		return !e || atoi(e) != 0;
 	}();
 	auto eff = [&](int k, long p, int K) {
 		const int i = p < 8 ? (int) p - 1 : 7;
-		if (!k_dependent) return (double) shapes[k].eff_k2048[i];
-		const double inv512 = 1.0 / shapes[k].eff_k512[i], inv2048 = 1.0 / shapes[k].eff_k2048[i];
-		const double slope = (inv512 - inv2048) / (1.0 / 512 - 1.0 / 2048);  // per 1 / K
-		// beyond K = 2048 the K = 2048 table stands: the straight line would credit the small shapes with a loop
-		// efficiency above that of the large ones
-		return 1.0 / (inv2048 + slope * std::max(0.0, 1.0 / K - 1.0 / 2048));
+		const float(*t)[8] = shapes[k].eff[layout];
+		if (!k_dependent) return (double) t[2][i];
+		// 1 / efficiency as a broken line in 1 / K through the three tables; the piece between 512 and 1024 also serves below
+		// 512; beyond K = 2048 the K = 2048 table stands (a straight line would credit the small shapes with a loop efficiency
+		// above that of the large ones)
+		const double inv512 = 1.0 / t[0][i], inv1024 = 1.0 / t[1][i], inv2048 = 1.0 / t[2][i], x = 1.0 / K;
+		double e;
+		if (x <= 1.0 / 2048)
+			e = 1.0 / inv2048;
+		else if (x <= 1.0 / 1024)
+			e = 1.0 / (inv2048 + (inv1024 - inv2048) * (x - 1.0 / 2048) / (1.0 / 1024 - 1.0 / 2048));
+		else
+			e = 1.0 / (inv1024 + (inv512 - inv1024) * (x - 1.0 / 1024) / (1.0 / 512 - 1.0 / 1024));
+		// A row-major A against a k-major B with rows of A beyond 4096 values: the 64 x 64 blocks lose 1.9 % per doubling of K
+		// (8192 x 1024 of C: .960 at K = 4096, .941, .925, .904 at 32768, where the larger shapes hold .95 - .97)
+		if (layout == 0 && shapes[k].bm == 64 && shapes[k].bn == 64 && K > 4096) e *= 1.0 - 0.019 * std::log2(K / 4096.0);
+		return e;
 	};
 	// 256 flop per clock and compute unit at the device's engine clock (kHz -> cycles per microsecond), as cnet_get_device_info
 	// reports it; 2.4 GHz when the driver gives none
@@ -1838,14 +1893,17 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, bool k_contig_opera
 	for (int k = 0; k < 5; ++k) {
 		if (forced >= 0 && forced != k) continue;
 		if (k == 4 && (forced != 4 && a.K % KC != 0)) continue;  // only the fast kernel has the two-stage form: shape 3 there
+		// beyond seven blocks per unit the two-stage form is erratic on a long K (8192 x 1024 of C: .95 at K = 2048, .83 - .97
+		// from 4096 on, layout by layout)
+		if (k == 4 && forced != 4 && a.K > 2048 && blocks(64, 64) > 7 * cus) continue;
 		const long nb = blocks(shapes[k].bm, shapes[k].bn);
 		const long per_unit = (nb + cus - 1) / cus;
 		// three real products per complex one in the shapes that have the registers for it (fast kernel only: K in whole chunks)
 		// an A without imaginary parts: two real products (fast kernel only: K in whole chunks)
-		const double work = (a.a_real && a.K % KC == 0) ? 4.0 : (three_products() && a.K % KC == 0 && !(k == 0 && k_contig_operands)) ? 6.0 : 8.0;
+		const double work = (a.a_real && a.K % KC == 0) ? 4.0 : (three_products() && a.K % KC == 0 && !(k == 0 && layout == 1)) ? 6.0 : 8.0;
 		const double block_us = work * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
 		// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
-		const double bonus = 1.0 - 0.000001 * shapes[k].bm * shapes[k].bn;
+		const double bonus = 1.0 - 0.0000005 * shapes[k].bm * shapes[k].bn;
 		double us = per_unit * block_us / eff(k, per_unit, a.K) * bonus;
 		int tail = 0, cuts = 1;
 		const long q = nb / cus, r = nb % cus;
@@ -1905,7 +1963,7 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 		return launch<64, 64, 32, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch);
 	} else {
 		int best, best_tail, cuts;
-		plan_blocks(a, nprob, batch, !A_MCONTIG && !B_NCONTIG, &best, &best_tail, &cuts);
+		plan_blocks(a, nprob, batch, block_layout(A_MCONTIG, B_NCONTIG), &best, &best_tail, &cuts);
 		if (best == 0) return launch<128, 128, 64, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
 		if (best == 1) return launch<64, 128, 32, 64, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
 		if (best == 2) return launch<128, 64, 64, 32, A_MCONTIG, B_NCONTIG, VEC>(a, nprob, batch, best_tail, cuts);
@@ -1960,8 +2018,8 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 		}
 		if (plan_skinny(a_mcontig, b_ncontig, right, nprob, batch, planned)) {
 			int shape, tail, cuts;
-			const double whole = plan_blocks(a, nprob, batch, !a_mcontig && !b_ncontig, &shape, &tail, &cuts);
-			const double parts = plan_blocks(left, nprob, batch, !a_mcontig && !b_ncontig, &shape, &tail, &cuts) + skinny_us(planned, nprob, batch);
+			const double whole = plan_blocks(a, nprob, batch, block_layout(a_mcontig, b_ncontig), &shape, &tail, &cuts);
+			const double parts = plan_blocks(left, nprob, batch, block_layout(a_mcontig, b_ncontig), &shape, &tail, &cuts) + skinny_us(planned, nprob, batch);
 			if (parts < whole) {
 				// one after the other on the compute stream: run side by side on two streams the narrow part's
 				// workgroups took slots from the first round of the block kernel and the pair got slower (842 against
