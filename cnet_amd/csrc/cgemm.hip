@@ -1858,6 +1858,9 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int layout, int *sh
 					{{0.754f, 0.839f, 0.870f, 0.886f, 0.754f, 0.900f, 0.904f, 0.904f},
 							{0.834f, 0.894f, 0.914f, 0.923f, 0.784f, 0.930f, 0.933f, 0.932f},
 							{0.878f, 0.921f, 0.934f, 0.944f, 0.797f, 0.951f, 0.951f, 0.950f}}}}};
+	// what a very long K adds to the K = 2048 figures (8192 x 1024 of C, K up to 32768: 1 / efficiency stays linear in 1 / K)
+	static const float long_k_gain[5][3] = {{0.007f, 0.016f, 0.019f}, {0.018f, 0.032f, 0.027f}, {0.030f, 0.027f, 0.032f},
+			{0.021f, 0.025f, 0.024f}, {0.021f, 0.025f, 0.024f}};
 	static const bool k_dependent = [] {
 		const char *e = getenv("CNET_CGEMM_KMODEL");  // tuning override: 0 uses the K = 2048 table for every K
 		return !e || atoi(e) != 0;
@@ -1867,12 +1870,11 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int layout, int *sh
 		const float(*t)[8] = shapes[k].eff[layout];
 		if (!k_dependent) return (double) t[2][i];
 		// 1 / efficiency as a broken line in 1 / K through the three tables; the piece between 512 and 1024 also serves below
-		// 512; beyond K = 2048 the K = 2048 table stands (a straight line would credit the small shapes with a loop efficiency
-		// above that of the large ones)
+		// 512; beyond K = 2048 the line runs on to the figure for an endless K (long_k_gain)
 		const double inv512 = 1.0 / t[0][i], inv1024 = 1.0 / t[1][i], inv2048 = 1.0 / t[2][i], x = 1.0 / K;
 		double e;
 		if (x <= 1.0 / 2048)
-			e = 1.0 / inv2048;
+			e = (1.0 + long_k_gain[k][layout] * (1.0 - 2048.0 * x)) / inv2048;
 		else if (x <= 1.0 / 1024)
 			e = 1.0 / (inv2048 + (inv1024 - inv2048) * (x - 1.0 / 2048) / (1.0 / 1024 - 1.0 / 2048));
 		else
@@ -1903,7 +1905,7 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int layout, int *sh
 		const double work = (a.a_real && a.K % KC == 0) ? 4.0 : (three_products() && a.K % KC == 0 && !(k == 0 && layout == 1)) ? 6.0 : 8.0;
 		const double block_us = work * shapes[k].bm * shapes[k].bn * a.K / flop_per_us_per_unit;
 		// between shapes that are equally fast the larger block wins: it moves half as many operand bytes through L2
-		const double bonus = 1.0 - 0.0000005 * shapes[k].bm * shapes[k].bn;
+		const double bonus = 1.0 - 0.00000025 * shapes[k].bm * shapes[k].bn;
 		double us = per_unit * block_us / eff(k, per_unit, a.K) * bonus;
 		int tail = 0, cuts = 1;
 		const long q = nb / cus, r = nb % cus;
