@@ -234,14 +234,27 @@ int run_stack(int n, int blocks, int B, int steps, float lr, bool both_halves) {
 	// timed region = the `steps` training steps from the initial weights (the first call also pays the one-off
 	// workspace growth of the backward pass; it is part of the job)
 	net.gpuSetInput(ct, bt);
-	wake_device(net, [&] { net.gpuForward(cx, l2, bx); });
+	// (the warm-up sends its batch ahead as the loop does, so that every device buffer of the data input has been the target
+	// of a copy before the clock starts: the first copy into a buffer while kernels run stalls host and device for 7 ms, once
+	// per buffer, which a loop of 10 steps would carry as 6 % of its time)
+	wake_device(net, [&] {
+		net.gpuPrefetch(cx, bx);
+		net.gpuForward(cx, l2, bx);
+	});
 	net.sync();
 	auto t0 = std::chrono::steady_clock::now();
 	net.gpuPrefetch(cx, bx);
 	auto t1 = t0;
+	std::string each;  // every step ends with its loss on the host, so the host's clock sees the steps one by one
+	auto last = t0;
 	for (int s = 0; s < steps; ++s) {
 		one();
-		if (s == 0) t1 = std::chrono::steady_clock::now();  // getLoss has waited for step 0
+		const auto now = std::chrono::steady_clock::now();
+		if (s == 0) t1 = now;  // getLoss has waited for step 0
+		char buf[32];
+		snprintf(buf, sizeof(buf), "%s%.2f", s ? ", " : "", 1e3 * std::chrono::duration<double>(now - last).count());
+		each += buf;
+		last = now;
 	}
 	net.sync();
 	const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
@@ -258,9 +271,9 @@ int run_stack(int n, int blocks, int B, int steps, float lr, bool both_halves) {
 	const double flops = 8.0 * products * B * (double) n * n * blocks;
 	printf("{\"workload\": \"residual stack: %d x (Linear %d->%d, CGelu, Residual), L2Out, SGD\", \"batch\": %d, \"steps\": %d, "
 		   "\"lr\": %g, \"ms_per_step\": %.3f, \"ms_per_step_after_the_first\": %.3f, \"samples_per_sec\": %.1f, "
-		   "\"complex_products_per_linear\": %d, \"gemm_tflops_executed\": %.2f, \"mean_loss_per_step\": [%s]}\n",
+		   "\"complex_products_per_linear\": %d, \"gemm_tflops_executed\": %.2f, \"ms_of_each_step\": [%s], \"mean_loss_per_step\": [%s]}\n",
 			blocks, n, n, B, steps, (double) lr, 1e3 * sec / steps, steps > 1 ? 1e3 * sec_later / (steps - 1) : 0.0, B * steps / sec, products,
-			flops * steps / sec / 1e12, all.c_str());
+			flops * steps / sec / 1e12, each.c_str(), all.c_str());
 	return 0;
 }
 
