@@ -1791,8 +1791,8 @@ double plan_blocks(const CgemmArgs &a, int nprob, int batch, int layout, int *sh
 	// Expected duration of the launch with each block shape.  The busiest compute unit works through p = ceil(blocks /
 	// units) blocks, so the launch takes p block-times, whether or not all units have that many and whether or not a
 	// block on the edge of C is full, divided by the efficiency measured for the shape at p blocks per unit on full
-	// blocks (fraction of the fp32 MFMA peak on operands of random values; the layout with both operands K-contiguous has
-	// tables of its own), at K = 512, 1024 and 2048; in between and below, 1 / efficiency follows a broken line in 1 / K (a
+	// blocks (fraction of the fp32 MFMA peak on operands of random values, a set of tables per operand layout), at K = 512,
+	// 1024 and 2048; in between and below, 1 / efficiency follows a broken line in 1 / K (a
 	// loop part and a fixed part per block: first loads and the write-out of C weigh more on a short K, and more on the
 	// small shapes).  The tables carry what a formula would miss: a unit holds two workgroups of the larger shapes, three
 	// of 64 x 64 and four of 64 x 64 with two LDS stages, a lone workgroup cannot keep the matrix pipe busy, and with 3 or 5
