@@ -1976,7 +1976,91 @@ int pick_tile(const CgemmArgs &a, int nprob, int batch) {
 
 }  // namespace
 
+namespace {
+
+// dst[plane][r][c] = src_plane[r][c] inside rows x cols and zero outside, for the two planes (blockIdx.y) of an operand;
+// dst has rows_d rows of ldd floats per plane, ldd a multiple of four.  One thread per four columns of dst.
+__global__ __launch_bounds__(256) void pack_planes_kernel(const float *__restrict__ s_re, const float *__restrict__ s_im, long lds, int rows,
+		int cols, float *__restrict__ dst, int rows_d, int ldd) {
+	const int groups = ldd / 4;
+	const long idx = (long) blockIdx.x * 256 + threadIdx.x;
+	if (idx >= (long) rows_d * groups) return;
+	const int r = (int) (idx / groups), c0 = (int) (idx - (long) r * groups) * 4;
+	const float *s = (blockIdx.y ? s_im : s_re) + (long) r * lds;
+	float v[4] = {0.f, 0.f, 0.f, 0.f};
+	if (r < rows) {
+#pragma unroll
+		for (int k = 0; k < 4; ++k)
+			if (c0 + k < cols) v[k] = s[c0 + k];
+	}
+	*reinterpret_cast<float4 *>(dst + ((long) blockIdx.y * rows_d + r) * ldd + c0) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+}  // namespace
+
 namespace cnet {
+
+static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int nprob, int batch);
+
+// Operands that the 128-bit transfers of the fast kernel cannot take (a leading dimension that is no multiple of four, a
+// plane that does not start on 16 bytes): a large product first copies them into aligned planes of the library's operand
+// buffer, K padded with zeros to whole chunks, and runs on those (2048^3 with every plane one float off its alignment:
+// 0.67 -> 0.49 ms; the register-staged kernel that takes such operands directly runs at 102-106 TFLOP/s).  True when the
+// product has been handed on that way (*rc set); false when it is not such a product or the buffer cannot be had.
+static bool cgemm_packed(bool a_mcontig, bool b_ncontig, const CgemmArgs &a, int nprob, int batch, int *rc) {
+	static const bool enabled = [] {
+		const char *e = getenv("CNET_CGEMM_PACK");  // tuning override: 0 leaves misaligned operands to the register-staged kernel
+		return !e || atoi(e) != 0;
+	}();
+	if (!enabled || batch != 1 || a.tri || a.a_real == 2) return false;
+	auto misaligned = [&](const float *re, const float *im, long ld) { return ld % 4 != 0 || !aligned16(re) || !aligned16(im); };
+	bool any = false;
+	for (int q = 0; q < nprob; ++q)
+		any = any || misaligned(a.p[q].a_re, a.p[q].a_im, a.lda) || misaligned(a.p[q].b_re, a.p[q].b_im, a.ldb);
+	// (a run along M or N that is no multiple of four cannot be padded: the product would write rows or columns C does not have)
+	if (!any || (a_mcontig && a.M % 4 != 0) || (b_ncontig && a.N % 4 != 0)) return false;
+	if ((double) a.M * a.N * a.K < (double) (1L << 27) || (long) a.M * a.N < 256L * 256) return false;
+	const int kp = (a.K + KC - 1) / KC * KC;
+	const int a_rows = a_mcontig ? kp : a.M, a_ld = a_mcontig ? a.M : kp, b_rows = b_ncontig ? kp : a.N, b_ld = b_ncontig ? a.N : kp;
+	const size_t a_floats = 2 * (size_t) a_rows * a_ld, b_floats = 2 * (size_t) b_rows * b_ld;
+	// the distinct operands of the one or two problems (a pair of gradients shares one of them)
+	const bool same_a = nprob == 2 && a.p[0].a_re == a.p[1].a_re && a.p[0].a_im == a.p[1].a_im;
+	const bool same_b = nprob == 2 && a.p[0].b_re == a.p[1].b_re && a.p[0].b_im == a.p[1].b_im;
+	const int na = (nprob == 2 && !same_a) ? 2 : 1, nb = (nprob == 2 && !same_b) ? 2 : 1;
+	const size_t bytes = (na * a_floats + nb * b_floats) * sizeof(float);
+	if (bytes > ((size_t) 2 << 30)) return false;
+	if (rt().capturing && bytes > rt().operand_workspace_bytes) return false;  // the buffer cannot grow inside a recording
+	float *buf = (float *) operand_workspace(bytes);
+	if (!buf) {
+		*rc = CNET_ERR_OUT_OF_MEMORY;
+		return true;
+	}
+	CgemmArgs pk = a;
+	pk.K = kp;
+	pk.lda = a_ld;
+	pk.ldb = b_ld;
+	auto pack = [&](const float *re, const float *im, long ld, int rows, int cols, float *dst, int rows_d, int ldd) {
+		const long threads = (long) rows_d * (ldd / 4);
+		hipLaunchKernelGGL(pack_planes_kernel, dim3((unsigned) ((threads + 255) / 256), 2), dim3(256), 0, rt().stream, re, im, ld, rows, cols, dst,
+				rows_d, ldd);
+	};
+	for (int q = 0; q < nprob; ++q) {
+		float *pa = buf + (size_t) ((q == 1 && !same_a) ? 1 : 0) * a_floats;
+		float *pb = buf + na * a_floats + (size_t) ((q == 1 && !same_b) ? 1 : 0) * b_floats;
+		if (q == 0 || !same_a) pack(a.p[q].a_re, a.p[q].a_im, a.lda, a_mcontig ? a.K : a.M, a_mcontig ? a.M : a.K, pa, a_rows, a_ld);
+		if (q == 0 || !same_b) pack(a.p[q].b_re, a.p[q].b_im, a.ldb, b_ncontig ? a.K : a.N, b_ncontig ? a.N : a.K, pb, b_rows, b_ld);
+		pk.p[q].a_re = pa;
+		pk.p[q].a_im = pa + (size_t) a_rows * a_ld;
+		pk.p[q].b_re = pb;
+		pk.p[q].b_im = pb + (size_t) b_rows * b_ld;
+	}
+	if (hipGetLastError() != hipSuccess) {
+		*rc = fail(CNET_ERR_HIP, "cgemm: launch of the pass that aligns the operands failed");
+		return true;
+	}
+	*rc = cgemm_dispatch(a_mcontig, b_ncontig, pk, nprob, batch);
+	return true;
+}
 
 // nprob = 1 or 2 problems of identical shape.
 static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int nprob, int batch) {
@@ -1990,6 +2074,7 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 	if (a_mcontig || !b_ncontig) a.a_real = 0;  // only that layout has the kernels (the imaginary plane holds zeros: reading it is right too)
 	int rc = CNET_OK;
 	if (try_skinny(a_mcontig, b_ncontig, a, nprob, batch, &rc)) return rc;
+	if (cgemm_packed(a_mcontig, b_ncontig, a, nprob, batch, &rc)) return rc;
 	// A C that is a few columns wider than a multiple of the block width (784 = 12 x 64 + 16) costs a whole extra column
 	// of blocks.  If the cost model says so, the product is done as two: the columns up to that multiple by the block
 	// kernels, the narrow rest by the small-C kernel.  The two write disjoint columns of C.

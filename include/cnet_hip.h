@@ -535,6 +535,7 @@ int cnet_embedding_bwd(const int32_t *tokens, const float *g_dzs_re, const float
  *   CNET_CGEMM_SKINNY_W = 4|8|16 wavefronts per tile of the small-C kernel
  *   CNET_CGEMM_SKINNY_TWO = 0    two small products of one call as two launches (and the gate behind them as launches of its own)
  *   CNET_CGEMM_3M = 0 | 1        initial value of cnet_cgemm_set_products (1: three real products per complex one)
+ *   CNET_CGEMM_PACK = 0          large products of misaligned operands on the operands as they are (no aligned copies)
  *   CNET_DFT_FOLD = 0            the transform of real samples without folding them about n/2 first
  *   CNET_STREAM_MIN_MB = n       footprint (MiB) from which an elementwise / row launch counts as streaming (default 256)
  *   CNET_STREAM_POLICY = 0..3    cache policy of every streaming launch: plain, hint on loads and stores, hinted stores,

@@ -263,6 +263,61 @@ def test_cgemm_random_shapes(gpu, port):
         assert np.array_equal(got[:, N:], c0[:, N:]), (case, "columns beside C were touched")
 
 
+@pytest.mark.usefixtures("products")
+@pytest.mark.parametrize("M,N,K,a_km,b_km,off_a,off_b", [(640, 512, 1000, 0, 1, 1, 0), (640, 512, 1024, 0, 0, 3, 2), (512, 768, 1000, 1, 1, 0, 1),
+                                                        (1024, 520, 2040, 0, 1, 2, 3), (516, 600, 1024, 1, 0, 1, 1)])
+def test_cgemm_large_products_of_misaligned_operands(gpu, port, M, N, K, a_km, b_km, off_a, off_b):
+    """Operands whose planes start one to three floats off a 16-byte boundary (column windows of wider buffers, leading
+    dimensions that are no multiple of four) in products large enough for the pass that first copies them into aligned
+    planes, K with and without a whole number of chunks, every layout: against numpy in complex128, with and without
+    accumulation and conj(B); what lies beside C stays untouched, and CNET_CGEMM_PACK=0 (the register-staged kernel on the
+    operands as they are) is checked by the random shapes above at smaller sizes."""
+    rs = np.random.RandomState(M + N + K)
+    A = (rs.randn(M, K) + 1j * rs.randn(M, K)).astype(np.complex64)
+    Bm = (rs.randn(K, N) + 1j * rs.randn(K, N)).astype(np.complex64)
+    def window(h, off):   # the matrix sits `off` columns into a buffer 5 columns wider (an odd leading dimension)
+        buf = np.zeros((h.shape[0], h.shape[1] + 5), np.complex64)
+        buf[:, off:off + h.shape[1]] = h
+        return ops.CMat.from_host(np.ascontiguousarray(buf.real), np.ascontiguousarray(buf.imag)).sub(off, h.shape[1])
+    a, b = window(A.T if a_km else A, off_a), window(Bm if b_km else Bm.T, off_b)
+    for cj, acc in ((0, 0), (1, 1)):
+        c0 = (rs.randn(M, N + 4) + 1j * rs.randn(M, N + 4)).astype(np.complex64)
+        cfull = ops.CMat.from_host(np.ascontiguousarray(c0.real), np.ascontiguousarray(c0.imag))
+        ops.cgemm(a, b, cfull.sub(0, N), M, N, K, a_km, b_km, cj, accumulate=acc)
+        got = cfull.re.owner.download() + 1j * cfull.im.owner.download()
+        want = A.astype(np.complex128) @ (Bm.conj() if cj else Bm).astype(np.complex128) + (c0[:, :N] if acc else 0)
+        assert np.linalg.norm(got[:, :N] - want) / np.linalg.norm(want) < 2e-5, (cj, acc)
+        assert np.array_equal(got[:, N:], c0[:, N:])
+
+
+def test_gradient_pairs_of_a_linear_with_misaligned_operands(gpu, port):
+    """Both halves of the input gradient and of the weight gradient (two problems per launch that share one operand) with
+    every operand a misaligned column window: against the same calls on aligned copies of the operands."""
+    rs = np.random.RandomState(5)
+    B, K, N = 1024, 520, 512
+    def both(h, off):
+        buf = np.zeros((h.shape[0], h.shape[1] + 5), np.float32)
+        buf[:, off:off + h.shape[1]] = h
+        return buf
+    planes = {name: [rs.randn(*shape).astype(np.float32) for _ in range(count)]
+              for name, shape, count in (("x", (B, K), 2), ("w", (N, K), 2), ("g", (B, N), 4))}
+    def run(off):
+        if off is None:
+            x, w = ops.CMat.from_host(*planes["x"]), ops.CMat.from_host(*planes["w"])
+            g = ops.Grad.from_host(planes["g"])
+        else:
+            x = ops.CMat.from_host(both(planes["x"][0], off), both(planes["x"][1], off)).sub(off, K)
+            w = ops.CMat.from_host(both(planes["w"][0], off), both(planes["w"][1], off)).sub(off, K)
+            g = ops.Grad.from_host([both(p, off) for p in planes["g"]]).sub(off, N)
+        dx, dw = ops.Grad.empty(B, K), ops.Grad.empty(N, K)
+        ops.linear_bwd_input(g, w, dx)
+        ops.linear_bwd_weight(g, x, dw)
+        return dx.host(), dw.host()
+    (dx0, dw0), (dx1, dw1) = run(None), run(3)
+    for p in range(0, 4, 2):
+        assert rel_c(dx1[p:p + 2], dx0[p:p + 2]) < 2e-6 and rel_c(dw1[p:p + 2], dw0[p:p + 2]) < 2e-6
+
+
 @pytest.mark.parametrize("tile", ["0", "1", "2", "3", "4", ""])
 def test_cgemm_tail_blocks_cut_along_k(gpu, tile):
     """Products whose blocks do not fill a whole number of rounds over the compute units, with the cut of the last round's
