@@ -534,9 +534,11 @@ struct DlStage {
 	unsigned goff[UNITS];  // byte offset of this lane's 16 bytes inside the operand tile of a chunk
 	int wave_s;            // wavefront number, held in a scalar register
 
-	// rows_valid: rows of the operand that exist from the first row of this block on (>= ROWS inside the matrix; a
-	// multiple of 4 when MCONTIG).  Rows past the end are fetched from the last valid ones instead: what they produce
-	// lies outside C and is never stored.
+	// rows_valid: rows of the operand that exist from the first row of this block on (>= ROWS inside the matrix).  Rows
+	// past the end are fetched from the last valid ones instead: what they produce lies outside C and is never stored.
+	// When MCONTIG a line of k is fetched in groups of four rows, so the last group may reach up to three floats past the
+	// rows that exist: they lie inside the line (the leading dimension is a multiple of four) and feed only rows of C that
+	// do not exist either.
 	__device__ __forceinline__ void init(long ld, int rows_valid) {
 		const int wave = threadIdx.x >> 6;
 		wave_s = __builtin_amdgcn_readfirstlane(wave);
@@ -545,7 +547,7 @@ struct DlStage {
 		for (int u = 0; u < UNITS; ++u) {
 			const int pos = ((u * 4 + wave) * 64 + lane) * 4;  // float offset inside the LDS plane
 			if (MCONTIG) {
-				const int k = pos / ROWS, row = min(pos % ROWS, rows_valid - 4);
+				const int k = pos / ROWS, row = min(pos % ROWS, ((rows_valid + 3) & ~3) - 4);
 				goff[u] = (unsigned) (((long) k * ld + row) * 4);
 			} else {
 				const int row = pos / KC, q = (pos % KC) / 4;
@@ -2017,11 +2019,12 @@ static bool cgemm_packed(bool a_mcontig, bool b_ncontig, const CgemmArgs &a, int
 	bool any = false;
 	for (int q = 0; q < nprob; ++q)
 		any = any || misaligned(a.p[q].a_re, a.p[q].a_im, a.lda) || misaligned(a.p[q].b_re, a.p[q].b_im, a.ldb);
-	// (a run along M or N that is no multiple of four cannot be padded: the product would write rows or columns C does not have)
-	if (!any || (a_mcontig && a.M % 4 != 0) || (b_ncontig && a.N % 4 != 0)) return false;
+	if (!any) return false;
 	if ((double) a.M * a.N * a.K < (double) (1L << 27) || (long) a.M * a.N < 256L * 256) return false;
 	const int kp = (a.K + KC - 1) / KC * KC;
-	const int a_rows = a_mcontig ? kp : a.M, a_ld = a_mcontig ? a.M : kp, b_rows = b_ncontig ? kp : a.N, b_ld = b_ncontig ? a.N : kp;
+	// (a run along M or N is padded to a multiple of four floats; the product itself keeps its M and N)
+	const int a_rows = a_mcontig ? kp : a.M, a_ld = a_mcontig ? (a.M + 3) / 4 * 4 : kp;
+	const int b_rows = b_ncontig ? kp : a.N, b_ld = b_ncontig ? (a.N + 3) / 4 * 4 : kp;
 	const size_t a_floats = 2 * (size_t) a_rows * a_ld, b_floats = 2 * (size_t) b_rows * b_ld;
 	// the distinct operands of the one or two problems (a pair of gradients shares one of them)
 	const bool same_a = nprob == 2 && a.p[0].a_re == a.p[1].a_re && a.p[0].a_im == a.p[1].a_im;
@@ -2116,10 +2119,13 @@ static int cgemm_dispatch(bool a_mcontig, bool b_ncontig, CgemmArgs &a, int npro
 			}
 		}
 	}
-	// float4 path: every contiguous run starts 16-byte aligned and has a length that is a multiple of 4
+	// float4 path: every contiguous run starts 16-byte aligned and has a length that is a multiple of 4; a run along M or N
+	// may also end inside its last group of four where the fast kernel takes the product (K in whole chunks, offsets that
+	// fit): the leading dimension, a multiple of four, covers the group, and what the extra values feed is never stored
 	auto vec_ok = [&](int K) {
 		bool v = (a.lda % 4 == 0) && (a.ldb % 4 == 0) && (a.stride_a % 4 == 0) && (a.stride_b % 4 == 0);
-		v = v && (a_mcontig ? a.M % 4 == 0 : K % 4 == 0) && (b_ncontig ? a.N % 4 == 0 : K % 4 == 0);
+		const bool ragged = K % KC == 0 && a.lda < (1L << 22) && a.ldb < (1L << 22);
+		v = v && (a_mcontig ? (a.M % 4 == 0 || ragged) : K % 4 == 0) && (b_ncontig ? (a.N % 4 == 0 || ragged) : K % 4 == 0);
 		for (int q = 0; q < nprob; ++q)
 			v = v && aligned16(a.p[q].a_re) && aligned16(a.p[q].a_im) && aligned16(a.p[q].b_re) && aligned16(a.p[q].b_im);
 		return v;

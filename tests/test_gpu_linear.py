@@ -265,11 +265,14 @@ def test_cgemm_random_shapes(gpu, port):
 
 @pytest.mark.usefixtures("products")
 @pytest.mark.parametrize("M,N,K,a_km,b_km,off_a,off_b", [(640, 512, 1000, 0, 1, 1, 0), (640, 512, 1024, 0, 0, 3, 2), (512, 768, 1000, 1, 1, 0, 1),
-                                                        (1024, 520, 2040, 0, 1, 2, 3), (516, 600, 1024, 1, 0, 1, 1)])
+                                                        (1024, 520, 2040, 0, 1, 2, 3), (516, 600, 1024, 1, 0, 1, 1), (1001, 1001, 1001, 1, 1, 0, 0),
+                                                        (1001, 1001, 1008, 0, 1, 0, 0), (2050, 514, 1024, 1, 0, 0, 2)])
 def test_cgemm_large_products_of_misaligned_operands(gpu, port, M, N, K, a_km, b_km, off_a, off_b):
     """Operands whose planes start one to three floats off a 16-byte boundary (column windows of wider buffers, leading
     dimensions that are no multiple of four) in products large enough for the pass that first copies them into aligned
-    planes, K with and without a whole number of chunks, every layout: against numpy in complex128, with and without
+    planes, K with and without a whole number of chunks, every layout, also with M or N that end inside a group of four
+    floats (1001, 2050, 514: such a run is padded, or taken as it is where its leading dimension covers the group): against
+    numpy in complex128, with and without
     accumulation and conj(B); what lies beside C stays untouched, and CNET_CGEMM_PACK=0 (the register-staged kernel on the
     operands as they are) is checked by the random shapes above at smaller sizes."""
     rs = np.random.RandomState(M + N + K)
